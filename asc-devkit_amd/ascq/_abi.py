@@ -1,0 +1,127 @@
+"""ctypes view of include/ascq.h: enums, descriptor structs and the library loader.
+
+The shared library is the product; this module only binds it.  Loading fails
+loudly when the library has not been built: there is no CPU fallback.
+"""
+import ctypes as C
+import os
+
+# ascq_status
+OK, EINVAL, EUNSUPPORTED, EALIGN, EHIP, ENULL = range(6)
+# ascq_dtype
+F16, BF16, F32, I8, I4, I32, U64 = range(7)
+# ascq_policy
+PER_TENSOR, PER_CHANNEL, PER_TOKEN, PER_GROUP = range(4)
+# ascq_round_mode (values of the reference's RoundMode enum)
+CAST_NONE, CAST_RINT, CAST_FLOOR, CAST_CEIL, CAST_ROUND, CAST_TRUNC = range(6)
+# ascq_quant_compute
+COMPUTE_F16, COMPUTE_SCALE_T, COMPUTE_F32 = range(3)
+# ascq_offset_kind
+OFFSET_NONE, OFFSET_SCALAR, OFFSET_TENSOR = range(3)
+# ascq_dequant_mode
+DEQUANT_WITH_SINGLE_ROW, DEQUANT_WITH_MULTI_ROW = range(2)
+# ascq_mm_*
+MM_QUANT_NONE, MM_QUANT_SCALAR, MM_QUANT_VECTOR = range(3)
+MM_SCALE_U64, MM_SCALE_F32 = range(2)
+MM_BIAS_NONE, MM_BIAS_I32_PRE, MM_BIAS_F32_POST, MM_BIAS_BF16_POST = range(4)
+MM_ACT_NONE, MM_ACT_FASTER_GELU = range(2)
+GROUP_LIST_COUNTS, GROUP_LIST_PREFIX_SUM = range(2)
+
+STATUS_NAMES = {OK: "ASCQ_OK", EINVAL: "ASCQ_EINVAL", EUNSUPPORTED: "ASCQ_EUNSUPPORTED", EALIGN: "ASCQ_EALIGN",
+                EHIP: "ASCQ_EHIP", ENULL: "ASCQ_ENULL"}
+
+
+class QuantDesc(C.Structure):
+    _fields_ = [("policy", C.c_int32), ("src_dtype", C.c_int32), ("scale_dtype", C.c_int32), ("compute", C.c_int32),
+                ("round_mode", C.c_int32), ("offset_kind", C.c_int32), ("k_dim", C.c_int32), ("scale", C.c_float),
+                ("offset", C.c_float), ("m", C.c_uint32), ("n", C.c_uint32), ("cal_count", C.c_uint32),
+                ("group_size", C.c_uint32)]
+
+
+class DequantDesc(C.Structure):
+    _fields_ = [("policy", C.c_int32), ("src_dtype", C.c_int32), ("scale_dtype", C.c_int32), ("dst_dtype", C.c_int32),
+                ("mode", C.c_int32), ("k_dim", C.c_int32), ("scale", C.c_float), ("m", C.c_uint32), ("n", C.c_uint32),
+                ("cal_count", C.c_uint32), ("group_size", C.c_uint32)]
+
+
+class AntiQuantDesc(C.Structure):
+    _fields_ = [("src_dtype", C.c_int32), ("dst_dtype", C.c_int32), ("is_transpose", C.c_int32),
+                ("has_offset", C.c_int32), ("per_tensor", C.c_int32), ("scale", C.c_float), ("offset", C.c_float),
+                ("k", C.c_uint32), ("n", C.c_uint32), ("offset_height", C.c_uint32), ("offset_width", C.c_uint32),
+                ("scale_height", C.c_uint32), ("scale_width", C.c_uint32)]
+
+
+class MatmulDesc(C.Structure):
+    _fields_ = [("m", C.c_uint32), ("n", C.c_uint32), ("k", C.c_uint32), ("trans_a", C.c_int32),
+                ("trans_b", C.c_int32), ("out_dtype", C.c_int32), ("quant_mode", C.c_int32),
+                ("scale_format", C.c_int32), ("bias_kind", C.c_int32), ("has_tok_scale", C.c_int32),
+                ("activation", C.c_int32), ("quant_scalar", C.c_uint64)]
+
+
+class GroupMatmulDesc(C.Structure):
+    _fields_ = [("mm", MatmulDesc), ("groups", C.c_uint32), ("group_list_kind", C.c_int32)]
+
+
+class W4A16Desc(C.Structure):
+    _fields_ = [("m", C.c_uint32), ("n", C.c_uint32), ("k", C.c_uint32), ("group_size", C.c_uint32),
+                ("has_offset", C.c_int32)]
+
+
+_P = C.c_void_p
+# name -> (restype, argtypes): every symbol include/ascq.h declares
+SIGNATURES = {
+    "ascq_quant": (C.c_int, [C.POINTER(QuantDesc), _P, _P, _P, _P, _P]),
+    "ascq_dynamic_quant_per_token": (C.c_int, [C.c_int32, C.c_uint32, C.c_uint32, _P, _P, _P, _P]),
+    "ascq_dequant": (C.c_int, [C.POINTER(DequantDesc), _P, _P, _P, _P]),
+    "ascq_dequant_dst_stride": (C.c_uint32, [C.c_int32, C.c_uint32]),
+    "ascq_antiquant": (C.c_int, [C.POINTER(AntiQuantDesc), _P, _P, _P, _P, _P]),
+    "ascq_matmul_w8a8": (C.c_int, [C.POINTER(MatmulDesc), _P, _P, _P, _P, _P, _P, _P, C.c_size_t, _P]),
+    "ascq_matmul_w8a8_workspace_size": (C.c_int, [C.POINTER(MatmulDesc), C.POINTER(C.c_size_t)]),
+    "ascq_group_matmul_w8a8": (C.c_int, [C.POINTER(GroupMatmulDesc), _P, _P, _P, _P, _P, _P, _P, _P]),
+    "ascq_matmul_w4a16": (C.c_int, [C.POINTER(W4A16Desc), _P, _P, _P, _P, _P, _P, C.c_size_t, _P]),
+    "ascq_matmul_w4a16_workspace_size": (C.c_int, [C.POINTER(W4A16Desc), C.POINTER(C.c_size_t)]),
+    "ascq_get_ascend_quant_max_min_tmp_size": (C.c_int, [C.POINTER(C.c_uint32), C.c_uint32, C.c_uint32,
+                                                         C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
+    "ascq_get_ascend_dequant_max_min_tmp_size": (C.c_int, [C.POINTER(C.c_uint32), C.c_uint32, C.c_uint32,
+                                                           C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
+    "ascq_get_ascend_antiquant_max_min_tmp_size": (C.c_int, [C.POINTER(C.c_uint32), C.c_uint32,
+                                                             C.POINTER(C.c_uint32), C.c_uint32, C.c_int32, C.c_int32,
+                                                             C.c_int32, C.POINTER(C.c_uint32),
+                                                             C.POINTER(C.c_uint32)]),
+    "ascq_pack_quant_param": (C.c_uint64, [C.c_float, C.c_int32, C.c_int32]),
+    "ascq_zero_fill": (C.c_int, [_P, C.c_size_t, _P]),
+    "ascq_last_error": (C.c_char_p, []),
+    "ascq_version": (C.c_char_p, []),
+}
+
+LIB_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "lib", "libascq.so")
+_lib = None
+
+
+def load_library():
+    """Load libascq.so (built in-tree by `make -C asc-devkit_amd/csrc`) and bind every declared symbol."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(f"{LIB_PATH} is missing: build it first (python -c 'import __graft_entry__ as g; "
+                           f"g.build()'); there is no fallback path")
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if a declared symbol is not exported
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+class AscqError(RuntimeError):
+    def __init__(self, status, message):
+        super().__init__(f"{STATUS_NAMES.get(status, status)}: {message}")
+        self.status = status
+
+
+def check(status):
+    if status != OK:
+        msg = load_library().ascq_last_error()
+        raise AscqError(status, msg.decode() if msg else "")

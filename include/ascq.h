@@ -1,0 +1,307 @@
+/*
+ * ascq.h - C ABI of libascq: the quantized-inference operators of the Ascend C
+ * devkit (AscendQuant / AscendDequant / AscendAntiQuant, the int8 Matmul quant
+ * path, the quantized grouped matmul, W4A16) implemented for one AMD MI355X
+ * (gfx950).
+ *
+ * Every tensor argument is a DEVICE (HBM) pointer owned by the caller.  A call
+ * validates its descriptor on the host, enqueues HIP kernels on `stream`
+ * (a hipStream_t passed as void*; NULL = the default stream) and returns without
+ * synchronising.  The library allocates nothing and never writes an input.
+ * All entry points are thread-safe; the only state is a thread-local error
+ * string (ascq_last_error).  Validation happens before the first HIP call, so
+ * every error path can be exercised on a machine without a GPU.
+ *
+ * Citations "ref:" name files of the asc-devkit reference tree whose interface
+ * the entry point replaces.
+ */
+#ifndef ASCQ_H
+#define ASCQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------ status */
+typedef enum ascq_status {
+    ASCQ_OK = 0,
+    ASCQ_EINVAL = 1,       /* descriptor violates a shape / count rule           */
+    ASCQ_EUNSUPPORTED = 2, /* dtype / mode combination the operator does not have */
+    ASCQ_EALIGN = 3,       /* a 32-byte row rule or pointer alignment is violated */
+    ASCQ_EHIP = 4,         /* a HIP runtime call failed (launch, no device)       */
+    ASCQ_ENULL = 5         /* a required pointer is NULL                          */
+} ascq_status;
+
+/* -------------------------------------------------------------------- enums */
+typedef enum ascq_dtype {
+    ASCQ_F16 = 0,
+    ASCQ_BF16 = 1,
+    ASCQ_F32 = 2,
+    ASCQ_I8 = 3,
+    ASCQ_I4 = 4, /* two per byte, element 2j in the low nibble (ref: impl/utils/common_types.h:57-111) */
+    ASCQ_I32 = 5,
+    ASCQ_U64 = 6 /* fixpipe quant parameter word, fp32 scale in the low 32 bits */
+} ascq_dtype;
+
+/* ref: include/adv_api/quantization/ascend_quant_utils.h:73-80 (AscendQuantPolicy) */
+typedef enum ascq_policy {
+    ASCQ_PER_TENSOR = 0,
+    ASCQ_PER_CHANNEL = 1,
+    ASCQ_PER_TOKEN = 2,
+    ASCQ_PER_GROUP = 3
+} ascq_policy;
+
+/* ref: impl/basic_api/utils/kernel_utils_mode.h:94-109 (RoundMode), same values */
+typedef enum ascq_round_mode {
+    ASCQ_CAST_NONE = 0, /* == RINT whenever precision is lost */
+    ASCQ_CAST_RINT = 1, /* half to even */
+    ASCQ_CAST_FLOOR = 2,
+    ASCQ_CAST_CEIL = 3,
+    ASCQ_CAST_ROUND = 4, /* half away from zero */
+    ASCQ_CAST_TRUNC = 5
+} ascq_round_mode;
+
+/* Which arithmetic contract AscendQuant follows (the reference has three). */
+typedef enum ascq_quant_compute {
+    ASCQ_COMPUTE_F16 = 0,     /* AscendQuant per-tensor / per-channel: every intermediate is fp16
+                                 (ref: impl/.../quant/ascend_quant_pre_impl.h:101-164,320-397)      */
+    ASCQ_COMPUTE_SCALE_T = 1, /* AscendQuant PER_TOKEN / PER_GROUP: math in the scale dtype
+                                 (ref: impl/.../quant/ascend_quant_per_group_3510_impl.h:142-178)   */
+    ASCQ_COMPUTE_F32 = 2      /* Quantize: always fp32 (ref: impl/.../quantize/quantize_impl.h:641-968) */
+} ascq_quant_compute;
+
+typedef enum ascq_offset_kind { ASCQ_OFFSET_NONE = 0, ASCQ_OFFSET_SCALAR = 1, ASCQ_OFFSET_TENSOR = 2 } ascq_offset_kind;
+
+/* ref: impl/basic_api/utils/kernel_utils_mode.h:181-184 (DeQuantMode) */
+typedef enum ascq_dequant_mode { ASCQ_DEQUANT_WITH_SINGLE_ROW = 0, ASCQ_DEQUANT_WITH_MULTI_ROW = 1 } ascq_dequant_mode;
+
+/* ------------------------------------------------------------ AscendQuant */
+/*
+ * ref: include/adv_api/quantization/ascend_quant.h:63-762, quantize.h.
+ * dst int8 [cal_count]; src [cal_count] of src_dtype (F16|BF16|F32).
+ *   PER_TENSOR : scalar `scale`/`offset`; elements = cal_count.
+ *   PER_CHANNEL: scale tensor [scale_count] (= n); rows = cal_count / scale_count.
+ *   PER_TOKEN  : scale [m]; rows = cal_count / n.
+ *   PER_GROUP  : k_dim=1: scale [m, ceil(n/group_size)]; k_dim=0: scale [ceil(m/group_size), n].
+ * Offset follows the scale's indexing when offset_kind == TENSOR, is the scalar
+ * `offset` when SCALAR.  dst may alias src only for identical element offsets
+ * (the reference allows reuse for AscendQuant).
+ * COMPUTE_F16:  y = sat8(rint( f16( f16( f16(x) * f16(s) ) + f16(o) ) ))   (policy TENSOR | CHANNEL)
+ * COMPUTE_SCALE_T / F32: v = cvt(x) * s [+ o] with one rounding per operation in the compute
+ *               type, y = sat8(round_mode(v)).
+ * Tensor scale/offset dtype = scale_dtype (COMPUTE_F16: must equal src_dtype).
+ */
+typedef struct ascq_quant_desc {
+    int32_t policy;      /* ascq_policy */
+    int32_t src_dtype;   /* ASCQ_F16 | ASCQ_BF16 | ASCQ_F32 */
+    int32_t scale_dtype; /* dtype of the scale/offset tensors */
+    int32_t compute;     /* ascq_quant_compute */
+    int32_t round_mode;  /* ascq_round_mode (COMPUTE_F16 always rounds half-even) */
+    int32_t offset_kind; /* ascq_offset_kind */
+    int32_t k_dim;       /* PER_GROUP: 1 = groups along n, 0 = groups along m */
+    float scale;         /* PER_TENSOR scale */
+    float offset;        /* scalar offset */
+    uint32_t m, n;       /* PER_TOKEN / PER_GROUP row count and row length; PER_CHANNEL: n = scale_count */
+    uint32_t cal_count;  /* number of elements processed */
+    uint32_t group_size; /* PER_GROUP */
+} ascq_quant_desc;
+
+int ascq_quant(const ascq_quant_desc* desc, void* dst, const void* src, const void* scale, const void* offset,
+               void* stream);
+
+/*
+ * Dynamic per-token quantisation of an activation matrix (no single reference
+ * op: the reference composes it from ReduceMax/Abs and AscendQuant PER_TOKEN,
+ * ref: impl/.../quant/ascend_quant_per_group_3510_impl.h:142-178).
+ * x [m, n] F16|BF16|F32 row-major -> q int8 [m, n], tok_scale f32 [m]:
+ *   amax = max_j |f32(x[i,j])|;  tok_scale[i] = amax / 127.0f (1.0f when amax == 0);
+ *   q[i,j] = sat8(rint( f32(x[i,j]) * (127.0f / amax) ))      (0 when amax == 0).
+ */
+int ascq_dynamic_quant_per_token(int32_t src_dtype, uint32_t m, uint32_t n, void* q, void* tok_scale, const void* x,
+                                 void* stream);
+
+/* ---------------------------------------------------------- AscendDequant */
+/*
+ * ref: include/adv_api/quantization/ascend_dequant.h:58-305, ascend_dequant_utils.h:26-44.
+ * src int32 (or f32 for PER_TOKEN/PER_GROUP) [m, n]; dst [m, n_dst] where
+ * n_dst = n rounded up so that a dst row is a multiple of 32 bytes.
+ *   j <  cal_count: dst[i,j] = dstT( f32(src[i,j]) * f32(scale) )
+ *   cal_count <= j < n: dst[i,j] = dstT( f32(src[i,j]) )      (converted, not scaled)
+ *   n <= j < n_dst: not written.
+ * scale: PER_TENSOR scalar `scale`; PER_CHANNEL tensor [>=cal_count] of F32 | BF16 | U64
+ * (U64: the low 32 bits are the fp32 scale); PER_TOKEN [m]; PER_GROUP as for quant.
+ * SINGLE_ROW mode applies the reference's {1, m*n, n} -> {m, n, n} reshape rule.
+ */
+typedef struct ascq_dequant_desc {
+    int32_t policy;      /* ascq_policy */
+    int32_t src_dtype;   /* ASCQ_I32 (ASCQ_F32 allowed for PER_TOKEN / PER_GROUP) */
+    int32_t scale_dtype; /* ASCQ_F32 | ASCQ_BF16 | ASCQ_U64 (also F16 for PER_TOKEN / PER_GROUP) */
+    int32_t dst_dtype;   /* ASCQ_F16 | ASCQ_BF16 | ASCQ_F32 */
+    int32_t mode;        /* ascq_dequant_mode */
+    int32_t k_dim;       /* PER_GROUP axis */
+    float scale;         /* PER_TENSOR scalar */
+    uint32_t m, n, cal_count;
+    uint32_t group_size;
+} ascq_dequant_desc;
+
+int ascq_dequant(const ascq_dequant_desc* desc, void* dst, const void* src, const void* scale, void* stream);
+
+/* Number of dst elements per row (n rounded up to a 32-byte multiple of dst_dtype). */
+uint32_t ascq_dequant_dst_stride(int32_t dst_dtype, uint32_t n);
+
+/* -------------------------------------------------------- AscendAntiQuant */
+/*
+ * ref: include/adv_api/quantization/ascend_antiquant.h (10 overloads), ascend_antiquant_utils.h:27-32.
+ * Not transposed: src [k, n], params [G, n], group = k / G:  dst[i][j] = scale[i/group][j] * (src[i][j] + offset[i/group][j])
+ * Transposed    : src [n, k], params [n, G], group = k / G:  dst[i][j] = scale[i][j/group] * (src[i][j] + offset[i][j/group])
+ * G = shape_info scale height (not transposed) / scale width (transposed); 0 means 1.
+ * dst F16 : a = f16( f16(src) + off ), dst = f16( scale * a )           (fp16 math)
+ * dst BF16: dst = bf16( (f32(src) + f32(off)) * f32(scale) )             (fp32 math)
+ * src I8 or I4 (packed, low nibble first along the contiguous axis).
+ * per_tensor != 0: `scale` / `offset` scalars are used instead of tensors.
+ */
+typedef struct ascq_antiquant_desc {
+    int32_t src_dtype;    /* ASCQ_I8 | ASCQ_I4 */
+    int32_t dst_dtype;    /* ASCQ_F16 | ASCQ_BF16 (= dtype of scale / offset tensors) */
+    int32_t is_transpose; /* 0: src [k, n]; 1: src [n, k] */
+    int32_t has_offset;
+    int32_t per_tensor;
+    float scale, offset;  /* per_tensor scalars (rounded once to dst_dtype) */
+    uint32_t k, n;
+    uint32_t offset_height, offset_width, scale_height, scale_width; /* AntiQuantShapeInfo */
+} ascq_antiquant_desc;
+
+int ascq_antiquant(const ascq_antiquant_desc* desc, void* dst, const void* src, const void* offset, const void* scale,
+                   void* stream);
+
+/* ------------------------------------------------- Matmul int8 quant path */
+typedef enum ascq_mm_quant_mode {
+    ASCQ_MM_QUANT_NONE = 0,   /* int32 out */
+    ASCQ_MM_QUANT_SCALAR = 1, /* SetQuantScalar (ref: impl/adv_api/detail/matmul/matmul_impl_base.h:355-366) */
+    ASCQ_MM_QUANT_VECTOR = 2  /* SetQuantVector, one parameter per output channel (ref: :367-378) */
+} ascq_mm_quant_mode;
+
+typedef enum ascq_mm_scale_format {
+    ASCQ_MM_SCALE_U64 = 0, /* fixpipe word: scale = f32(bits[31:0] & 0xFFFFE000)  (1-8-10 float), REQ8: bits[45:37]
+                              offset, bit 46 sign (ref: examples/.../fixpipe_l0c2gm/scripts/gen_data_s322f16.py:37-66) */
+    ASCQ_MM_SCALE_F32 = 1  /* plain fp32, all 23 mantissa bits used */
+} ascq_mm_scale_format;
+
+typedef enum ascq_mm_bias_kind {
+    ASCQ_MM_BIAS_NONE = 0,
+    ASCQ_MM_BIAS_I32_PRE = 1,   /* int32 [n], initial value of the accumulator
+                                   (ref: impl/adv_api/detail/matmul/stage/compute/mmad_compute.h:40-82) */
+    ASCQ_MM_BIAS_F32_POST = 2,  /* fp32 [n] added after dequant */
+    ASCQ_MM_BIAS_BF16_POST = 3  /* bf16 [n] added after dequant (widened to fp32) */
+} ascq_mm_bias_kind;
+
+typedef enum ascq_mm_activation {
+    ASCQ_MM_ACT_NONE = 0,
+    ASCQ_MM_ACT_FASTER_GELU = 1 /* x*exp(0.851(x-|x|))/(1+exp(-1.702|x|)) (ref: examples/.../quant_group_matmul_high_performance/scripts/gen_data.py:19-23) */
+} ascq_mm_activation;
+
+/*
+ * ref: include/adv_api/matmul/matmul.h:175-185 (SetQuantScalar/SetQuantVector),
+ *      impl/adv_api/detail/matmul/stage/copy_cube_out/quant/quant_processor_fixpipe.h:74-222.
+ * A int8 [m, k] (trans_a: [k, m]); B int8 [k, n] (trans_b: [n, k]); row-major, dense.
+ *   acc[i,j] = sum_k A[i,k]*B[k,j] (+ bias_i32[j])                          exact int32
+ *   QUANT_NONE: C int32 = acc.
+ *   else v = f32(acc) * s_j  [* tok_scale[i]]  [+ bias_post[j]]  [act]      one fp32 rounding per op
+ *        C = F16: f16(v) saturated to +-65504;  BF16: bf16 rne;  F32: v;
+ *            I8 (U64 format only): sat( sat9(rint(v)) + offset9 ), offset9 = bits[45:37] taken as unsigned,
+ *            saturating to int8 when bit 46 is set and to uint8 otherwise.
+ */
+typedef struct ascq_matmul_desc {
+    uint32_t m, n, k;
+    int32_t trans_a, trans_b;
+    int32_t out_dtype;     /* ASCQ_I32 | ASCQ_F16 | ASCQ_BF16 | ASCQ_F32 | ASCQ_I8 */
+    int32_t quant_mode;    /* ascq_mm_quant_mode */
+    int32_t scale_format;  /* ascq_mm_scale_format */
+    int32_t bias_kind;     /* ascq_mm_bias_kind */
+    int32_t has_tok_scale; /* fp32 [m] multiplied after the channel scale */
+    int32_t activation;    /* ascq_mm_activation */
+    uint64_t quant_scalar; /* QUANT_SCALAR: U64 word, or fp32 bits in the low half for F32 format */
+} ascq_matmul_desc;
+
+int ascq_matmul_w8a8(const ascq_matmul_desc* desc, void* c, const void* a, const void* b, const void* bias,
+                     const void* quant_vector, const void* tok_scale, void* workspace, size_t workspace_bytes,
+                     void* stream);
+int ascq_matmul_w8a8_workspace_size(const ascq_matmul_desc* desc, size_t* bytes);
+
+/* ------------------------------------------------ quantized grouped matmul */
+typedef enum ascq_group_list_kind {
+    ASCQ_GROUP_LIST_COUNTS = 0,    /* rows per group (ref: examples/.../quant_group_matmul_custom.asc:264) */
+    ASCQ_GROUP_LIST_PREFIX_SUM = 1 /* inclusive prefix sums */
+} ascq_group_list_kind;
+
+/*
+ * ref: examples/01_simd_cpp_api/05_best_practices/03_fusion_compute/quant_group_matmul_high_performance/
+ *      quant_group_matmul_custom.asc:255-454.
+ * x int8 [m, k]; w int8 [groups, k, n]; scale fp32 [groups, n]; tok_scale fp32 [m] (optional);
+ * bias [groups, n] per mm.bias_kind; group_list int64 [groups] (device).  Rows of group g are
+ * [off_g, off_g + cnt_g); rows beyond the last group are not written; groups with cnt <= 0 are skipped.
+ *   y[i,j] = out( act( (f32(acc) * scale[g][j]) * tok_scale[i] + bias[g][j] ) )
+ * mm.m is the row capacity of x / y, mm.quant_mode must be QUANT_VECTOR, scale_format F32.
+ */
+typedef struct ascq_group_matmul_desc {
+    ascq_matmul_desc mm;
+    uint32_t groups;
+    int32_t group_list_kind; /* ascq_group_list_kind */
+} ascq_group_matmul_desc;
+
+int ascq_group_matmul_w8a8(const ascq_group_matmul_desc* desc, void* y, const void* x, const void* w,
+                           const void* bias, const void* scale, const void* tok_scale, const int64_t* group_list,
+                           void* stream);
+
+/* ------------------------------------------------------------------- W4A16 */
+/*
+ * W4A16 weight-only linear = AscendAntiQuant<int4b_t, half> (per-group along k,
+ * ref: include/adv_api/quantization/ascend_antiquant.h:50-54) feeding a half GEMV/GEMM.
+ * x f16 [m, k]; w int4 [k, n] packed along n (n even); scale, offset f16 [k/group_size, n].
+ *   wdq[k,j] = f16( scale[k/g][j] * f16( f16(w[k,j]) + offset[k/g][j] ) )     (offset optional)
+ *   y[i,j]   = f16( sum_k f32(x[i,k]) * f32(wdq[k,j]) )                       fp32 accumulation
+ * workspace: ascq_matmul_w4a16_workspace_size bytes, ZERO-FILLED before the first call
+ * (the library leaves it zero-filled on return); calls sharing a workspace must not overlap.
+ */
+typedef struct ascq_w4a16_desc {
+    uint32_t m, n, k;
+    uint32_t group_size;
+    int32_t has_offset;
+} ascq_w4a16_desc;
+
+int ascq_matmul_w4a16(const ascq_w4a16_desc* desc, void* y, const void* x, const void* w, const void* scale,
+                      const void* offset, void* workspace, size_t workspace_bytes, void* stream);
+int ascq_matmul_w4a16_workspace_size(const ascq_w4a16_desc* desc, size_t* bytes);
+
+/* --------------------------------------------- host "tiling" size queries */
+/*
+ * Scratch-size queries with the reference's answers, for callers that size a
+ * shared temporary buffer from them.  On the GPU the elementwise operators need
+ * no scratch; the values are the reference's so that existing host code keeps
+ * working.  ref: impl/adv_api/tiling/quantization/ascend_quant_tiling_impl.cpp:31-68,
+ * ascend_dequant_tiling_impl.cpp, ascend_antiquant_tiling_impl.cpp.
+ */
+int ascq_get_ascend_quant_max_min_tmp_size(const uint32_t* shape, uint32_t ndim, uint32_t type_size,
+                                           uint32_t* max_value, uint32_t* min_value);
+int ascq_get_ascend_dequant_max_min_tmp_size(const uint32_t* shape, uint32_t ndim, uint32_t type_size,
+                                             uint32_t* max_value, uint32_t* min_value);
+int ascq_get_ascend_antiquant_max_min_tmp_size(const uint32_t* src_shape, uint32_t src_ndim,
+                                               const uint32_t* scale_shape, uint32_t scale_ndim, int32_t is_transpose,
+                                               int32_t input_dtype, int32_t output_dtype, uint32_t* max_value,
+                                               uint32_t* min_value);
+
+/* -------------------------------------------------------------- utilities */
+/* Pack an fp32 scale (and optional REQ8 offset / sign) into the fixpipe uint64 word. Host-side, pure. */
+uint64_t ascq_pack_quant_param(float scale, int32_t offset9, int32_t is_signed);
+/* Fill `bytes` of device memory with zero using a kernel (safe inside stream capture). */
+int ascq_zero_fill(void* ptr, size_t bytes, void* stream);
+const char* ascq_last_error(void);
+const char* ascq_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ASCQ_H */

@@ -1,0 +1,712 @@
+/*
+ * ascq_oracle.c - CPU restatement of the asc-devkit quantized-inference operators.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This file is the checker that the HIP kernels are
+ * compared with; nothing in the shipped library links, loads or calls it, and
+ * it must never be used as a fallback for a missing GPU path.  It is also the
+ * program timed as the "CPU baseline" (kind "port": the reference's own CPU
+ * build needs the closed CANN `tikicpulib` model, which is not available).
+ *
+ * All floating-point formats narrower than fp32 are implemented in software
+ * (integer bit manipulation), so the oracle shares no arithmetic with the
+ * device code, which uses the hardware's fp16 / bf16 instructions.
+ *
+ * Each operator cites the reference file it restates (paths relative to the
+ * asc-devkit tree).  Pinning status of every function is listed in
+ * oracle/README.md.
+ */
+#include "ascq_oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+/* --------------------------------------------------------------- threads */
+static int g_threads = 1;
+void orc_set_threads(int n)
+{
+    g_threads = n > 0 ? n : 1;
+#ifdef _OPENMP
+    omp_set_num_threads(g_threads);
+#endif
+}
+int orc_get_threads(void) { return g_threads; }
+
+/* ------------------------------------------------------- scalar numerics */
+static inline uint32_t f32_bits(float f)
+{
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    return u;
+}
+static inline float bits_f32(uint32_t u)
+{
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+static inline uint64_t f64_bits(double d)
+{
+    uint64_t u;
+    memcpy(&u, &d, 8);
+    return u;
+}
+
+/* binary16 <- binary64, round to nearest even, IEEE overflow to infinity.
+ * Pins: docs/zh/api/SIMD-API/基础API/数据结构/precision_conversion.md:520-534 (float -> half examples). */
+uint16_t orc_f64_to_f16(double d)
+{
+    uint64_t u = f64_bits(d);
+    uint16_t sign = (uint16_t)((u >> 48) & 0x8000u);
+    int exp = (int)((u >> 52) & 0x7FF);
+    uint64_t mant = u & 0xFFFFFFFFFFFFFull;
+    if (exp == 0x7FF) {
+        return (uint16_t)(sign | (mant ? 0x7E00u : 0x7C00u));
+    }
+    if (exp == 0) {
+        return sign; /* zero or a binary64 subnormal, far below half the smallest binary16 subnormal */
+    }
+    int e = exp - 1023;
+    if (e > 15) {
+        return (uint16_t)(sign | 0x7C00u);
+    }
+    if (e >= -14) {
+        uint64_t m = mant >> 42;
+        uint64_t rem = mant & ((1ull << 42) - 1);
+        uint64_t half = 1ull << 41;
+        uint32_t r = (uint32_t)(((uint32_t)(e + 15) << 10) + m);
+        if (rem > half || (rem == half && (m & 1))) {
+            r += 1; /* a carry out of the mantissa increments the exponent, which is the right result */
+        }
+        if (r >= 0x7C00u) {
+            r = 0x7C00u;
+        }
+        return (uint16_t)(sign | r);
+    }
+    /* subnormal result: value / 2^-24 rounded to an integer */
+    int shift = 28 - e; /* (1.mant * 2^52) >> shift == value * 2^24 */
+    if (shift > 63) {
+        return sign;
+    }
+    uint64_t full = (1ull << 52) | mant;
+    uint64_t m = full >> shift;
+    uint64_t rem = full & ((1ull << shift) - 1);
+    uint64_t half = 1ull << (shift - 1);
+    if (rem > half || (rem == half && (m & 1))) {
+        m += 1;
+    }
+    return (uint16_t)(sign | (uint16_t)m);
+}
+
+uint16_t orc_f32_to_f16(float f) { return orc_f64_to_f16((double)f); }
+
+float orc_f16_to_f32(uint16_t h)
+{
+    uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1F;
+    uint32_t mant = h & 0x3FFu;
+    if (exp == 0x1F) {
+        return bits_f32(sign | 0x7F800000u | (mant << 13));
+    }
+    if (exp == 0) {
+        if (mant == 0) {
+            return bits_f32(sign);
+        }
+        float v = (float)mant * 5.9604644775390625e-08f; /* 2^-24 */
+        return sign ? -v : v;
+    }
+    return bits_f32(sign | ((exp + 112u) << 23) | (mant << 13));
+}
+
+/* bfloat16 <- binary32, round to nearest even.
+ * ref: impl/basic_api/kernel_type_conversion_utils.h:48-60 (IsBf16NeedRound truth table),
+ *      precision_conversion.md:541-553. */
+uint16_t orc_f32_to_bf16(float f)
+{
+    uint32_t u = f32_bits(f);
+    if ((u & 0x7F800000u) == 0x7F800000u) {
+        if (u & 0x007FFFFFu) {
+            return (uint16_t)((u >> 16) | 0x0040u);
+        }
+        return (uint16_t)(u >> 16);
+    }
+    uint32_t lsb = (u >> 16) & 1u;
+    u += 0x7FFFu + lsb;
+    return (uint16_t)(u >> 16);
+}
+
+float orc_bf16_to_f32(uint16_t b) { return bits_f32((uint32_t)b << 16); }
+
+/* One IEEE operation in binary16: the exact result rounded once. */
+uint16_t orc_f16_mul(uint16_t a, uint16_t b)
+{
+    /* 11-bit x 11-bit significands: the binary64 product is exact */
+    return orc_f64_to_f16((double)orc_f16_to_f32(a) * (double)orc_f16_to_f32(b));
+}
+uint16_t orc_f16_add(uint16_t a, uint16_t b)
+{
+    /* exponents span 2^-24 .. 2^15: the binary64 sum is exact */
+    return orc_f64_to_f16((double)orc_f16_to_f32(a) + (double)orc_f16_to_f32(b));
+}
+/* One operation in bfloat16 (8-bit significands: the binary32-range product is exact in binary64). */
+uint16_t orc_bf16_mul(uint16_t a, uint16_t b)
+{
+    double p = (double)orc_bf16_to_f32(a) * (double)orc_bf16_to_f32(b);
+    return orc_f32_to_bf16((float)p);
+}
+uint16_t orc_bf16_add(uint16_t a, uint16_t b)
+{
+    double s = (double)orc_bf16_to_f32(a) + (double)orc_bf16_to_f32(b);
+    return orc_f32_to_bf16((float)s);
+}
+
+/* float -> int8 with a round mode and saturation.
+ * ref: impl/basic_api/utils/kernel_utils_mode.h:94-109; precision_conversion.md:242-252 (half -> int8, saturating);
+ *      impl/adv_api/detail/quantization/quant/ascend_quant_3510_impl.h:969-990 (f32 -> s16 -> f16 -> s8 chain,
+ *      which equals a direct saturating conversion because every step saturates and s16 -> f16 is monotone). */
+int8_t orc_round_sat8(double v, int round_mode)
+{
+    double r;
+    if (v != v) {
+        return 0; /* NaN: outside the pinned domain */
+    }
+    switch (round_mode) {
+        case ASCQ_CAST_FLOOR: r = floor(v); break;
+        case ASCQ_CAST_CEIL: r = ceil(v); break;
+        case ASCQ_CAST_ROUND: r = round(v); break;
+        case ASCQ_CAST_TRUNC: r = trunc(v); break;
+        default: r = nearbyint(v); break; /* NONE / RINT: ties to even (default rounding direction) */
+    }
+    if (r > 127.0) {
+        return 127;
+    }
+    if (r < -128.0) {
+        return -128;
+    }
+    return (int8_t)r;
+}
+
+static inline float load_as_f32(const void* p, size_t i, int dtype)
+{
+    switch (dtype) {
+        case ASCQ_F16: return orc_f16_to_f32(((const uint16_t*)p)[i]);
+        case ASCQ_BF16: return orc_bf16_to_f32(((const uint16_t*)p)[i]);
+        case ASCQ_F32: return ((const float*)p)[i];
+        case ASCQ_U64: return bits_f32((uint32_t)(((const uint64_t*)p)[i] & 0xFFFFFFFFull));
+        default: return 0.0f;
+    }
+}
+
+static inline void store_from_f32(void* p, size_t i, int dtype, float v)
+{
+    switch (dtype) {
+        case ASCQ_F16: ((uint16_t*)p)[i] = orc_f32_to_f16(v); break;
+        case ASCQ_BF16: ((uint16_t*)p)[i] = orc_f32_to_bf16(v); break;
+        case ASCQ_F32: ((float*)p)[i] = v; break;
+        default: break;
+    }
+}
+
+/* int4 element i of a packed buffer: element 2j in the low nibble of byte j.
+ * ref: impl/utils/common_types.h:57-111; examples/.../matmul_int4/scripts/gen_data.py:32-42. */
+static inline int load_i4(const uint8_t* p, size_t i)
+{
+    uint8_t b = p[i >> 1];
+    int v = (i & 1) ? (b >> 4) : (b & 0xF);
+    return v >= 8 ? v - 16 : v;
+}
+
+/* ------------------------------------------------------------ AscendQuant */
+/* index of the scale / offset element that applies to (row i, col j) */
+static inline size_t quant_param_index(const ascq_quant_desc* d, size_t i, size_t j)
+{
+    switch (d->policy) {
+        case ASCQ_PER_CHANNEL: return j;
+        case ASCQ_PER_TOKEN: return i;
+        case ASCQ_PER_GROUP:
+            if (d->k_dim == 1) {
+                size_t per_row = (d->n + d->group_size - 1) / d->group_size;
+                return i * per_row + j / d->group_size;
+            }
+            return (i / d->group_size) * (size_t)d->n + j;
+        default: return 0;
+    }
+}
+
+/*
+ * COMPUTE_F16   ref: impl/adv_api/detail/quantization/quant/ascend_quant_pre_impl.h:101-164 (per channel),
+ *               :320-397 (per tensor), :439-483 (float scale/offset are cast to half first);
+ *               bf16 source is first cast to half: ascend_quant_3510_impl.h:51-54.
+ * COMPUTE_SCALE_T ref: .../quant/ascend_quant_per_group_3510_impl.h:142-178,498-538,1000-1044.
+ * COMPUTE_F32   ref: impl/adv_api/detail/quantization/quantize/quantize_impl.h:641-695,737-792,832-872.
+ */
+int orc_quant(const ascq_quant_desc* d, int8_t* dst, const void* src, const void* scale, const void* offset)
+{
+    size_t total = d->cal_count;
+    size_t n = (d->policy == ASCQ_PER_TENSOR) ? total : d->n;
+    if (n == 0) {
+        return 0;
+    }
+    size_t rows = total / n;
+    int comp = d->compute;
+    int ctype = (comp == ASCQ_COMPUTE_F16) ? ASCQ_F16 : (comp == ASCQ_COMPUTE_F32 ? ASCQ_F32 : d->scale_dtype);
+    int rmode = (comp == ASCQ_COMPUTE_F16) ? ASCQ_CAST_RINT : d->round_mode;
+
+#pragma omp parallel for schedule(static) if (rows * n > 65536)
+    for (size_t i = 0; i < rows; ++i) {
+        for (size_t j = 0; j < n; ++j) {
+            size_t e = i * n + j;
+            float s, o = 0.0f;
+            if (d->policy == ASCQ_PER_TENSOR) {
+                s = d->scale;
+            } else {
+                s = load_as_f32(scale, quant_param_index(d, i, j), d->scale_dtype);
+            }
+            if (d->offset_kind == ASCQ_OFFSET_SCALAR) {
+                o = d->offset;
+            } else if (d->offset_kind == ASCQ_OFFSET_TENSOR) {
+                o = load_as_f32(offset, quant_param_index(d, i, j), d->scale_dtype);
+            }
+            float x = load_as_f32(src, e, d->src_dtype);
+            double v;
+            if (ctype == ASCQ_F16) {
+                uint16_t xh = orc_f32_to_f16(x); /* exact for a half source */
+                uint16_t t = orc_f16_mul(xh, orc_f32_to_f16(s));
+                if (comp == ASCQ_COMPUTE_F16 || d->offset_kind != ASCQ_OFFSET_NONE) {
+                    t = orc_f16_add(t, orc_f32_to_f16(o)); /* the legacy op always executes Adds/Add */
+                }
+                v = (double)orc_f16_to_f32(t);
+            } else if (ctype == ASCQ_BF16) {
+                uint16_t t = orc_bf16_mul(orc_f32_to_bf16(x), orc_f32_to_bf16(s));
+                if (d->offset_kind != ASCQ_OFFSET_NONE) {
+                    t = orc_bf16_add(t, orc_f32_to_bf16(o));
+                }
+                v = (double)orc_bf16_to_f32(t);
+            } else {
+                volatile float t = x * s; /* one fp32 rounding, never fused with the add */
+                if (d->offset_kind != ASCQ_OFFSET_NONE) {
+                    volatile float t2 = t + o;
+                    t = t2;
+                }
+                v = (double)t;
+            }
+            dst[e] = orc_round_sat8(v, rmode);
+        }
+    }
+    return 0;
+}
+
+/* Dynamic per-token quantisation: the composition ReduceMax(|x|) -> AscendQuant PER_TOKEN (scaleT = float)
+ * ref: impl/adv_api/detail/quantization/quant/ascend_quant_per_group_3510_impl.h:142-178. */
+int orc_dynamic_quant_per_token(int src_dtype, uint32_t m, uint32_t n, int8_t* q, float* tok_scale, const void* x)
+{
+#pragma omp parallel for schedule(static) if ((size_t)m * n > 65536)
+    for (size_t i = 0; i < m; ++i) {
+        float amax = 0.0f;
+        for (size_t j = 0; j < n; ++j) {
+            float a = fabsf(load_as_f32(x, i * n + j, src_dtype));
+            if (a > amax) {
+                amax = a;
+            }
+        }
+        if (amax == 0.0f) {
+            tok_scale[i] = 1.0f;
+            memset(q + i * n, 0, n);
+            continue;
+        }
+        volatile float inv = 127.0f / amax;
+        tok_scale[i] = amax / 127.0f;
+        for (size_t j = 0; j < n; ++j) {
+            volatile float t = load_as_f32(x, i * n + j, src_dtype) * inv;
+            q[i * n + j] = orc_round_sat8((double)t, ASCQ_CAST_RINT);
+        }
+    }
+    return 0;
+}
+
+/* ---------------------------------------------------------- AscendDequant */
+uint32_t orc_dequant_dst_stride(int dst_dtype, uint32_t n)
+{
+    uint32_t per_blk = (dst_dtype == ASCQ_F32) ? 8u : 16u; /* 32 bytes of dstT */
+    return (n + per_blk - 1) / per_blk * per_blk;
+}
+
+/*
+ * ref: impl/adv_api/detail/quantization/dequant/ascend_dequant_common_impl.h:207-223 (single-row reshape),
+ *      :229-255 (scale -> fp32, uint64 keeps the low word), :260-267 (int32 -> fp32), :273-325 (Mul over the first
+ *      calCount columns only), :328-362 (cast out), :368-431 (dst row stride padded to 32 bytes);
+ *      per token / per group: .../dequant/ascend_dequant_3510_impl.h:227-307,337-380,449-537;
+ *      worked example docs/zh/api/SIMD-API/高阶API/量化操作/AscendDequant.md:385-401.
+ */
+int orc_dequant(const ascq_dequant_desc* d, void* dst, const void* src, const void* scale)
+{
+    uint32_t m = d->m, n = d->n, cal = d->cal_count;
+    if (d->mode == ASCQ_DEQUANT_WITH_SINGLE_ROW && d->policy <= ASCQ_PER_CHANNEL) {
+        uint32_t per_blk = (d->dst_dtype == ASCQ_F32) ? 8u : 16u;
+        if (m == 1 && cal != 0 && cal % per_blk == 0 && n % cal == 0) {
+            m = n / cal;
+            n = cal;
+        }
+    }
+    uint32_t stride = orc_dequant_dst_stride(d->dst_dtype, n);
+#pragma omp parallel for schedule(static) if ((size_t)m * n > 65536)
+    for (size_t i = 0; i < m; ++i) {
+        for (size_t j = 0; j < n; ++j) {
+            float x = (d->src_dtype == ASCQ_F32) ? ((const float*)src)[i * n + j]
+                                                  : (float)((const int32_t*)src)[i * n + j]; /* RNE */
+            float v = x;
+            if (j < cal) {
+                float s;
+                switch (d->policy) {
+                    case ASCQ_PER_TENSOR: s = d->scale; break;
+                    case ASCQ_PER_CHANNEL: s = load_as_f32(scale, j, d->scale_dtype); break;
+                    case ASCQ_PER_TOKEN: s = load_as_f32(scale, i, d->scale_dtype); break;
+                    default:
+                        if (d->k_dim == 1) {
+                            size_t per_row = (n + d->group_size - 1) / d->group_size;
+                            s = load_as_f32(scale, i * per_row + j / d->group_size, d->scale_dtype);
+                        } else {
+                            s = load_as_f32(scale, (i / d->group_size) * (size_t)n + j, d->scale_dtype);
+                        }
+                        break;
+                }
+                volatile float t = x * s;
+                v = t;
+            }
+            store_from_f32(dst, i * stride + j, d->dst_dtype, v);
+        }
+    }
+    return 0;
+}
+
+/* -------------------------------------------------------- AscendAntiQuant */
+/*
+ * ref: docs/zh/api/SIMD-API/高阶API/量化操作/AscendAntiQuant.md:36-50 (the contract),
+ *      impl/adv_api/detail/quantization/antiquant/ascend_antiquant_impl.h:47-135 (cast, add offset, mul scale in
+ *      half), .../ascend_antiquant_c220_impl.h:46-101 (bf16 output: fp32 add / mul, one rounding to bf16),
+ *      examples/.../03_quantization/antiquant/scripts/gen_data.py:27-49.
+ */
+int orc_antiquant(const ascq_antiquant_desc* d, void* dst, const void* src, const void* offset, const void* scale)
+{
+    size_t K = d->k, N = d->n;
+    size_t rows = d->is_transpose ? N : K;
+    size_t cols = d->is_transpose ? K : N;
+    uint32_t G;
+    if (d->is_transpose) {
+        G = d->scale_width ? d->scale_width : 1;
+    } else {
+        G = d->scale_height ? d->scale_height : 1;
+    }
+    size_t gs = K / G;
+    int pt = d->dst_dtype; /* parameter dtype == dst dtype */
+#pragma omp parallel for schedule(static) if (rows * cols > 65536)
+    for (size_t i = 0; i < rows; ++i) {
+        for (size_t j = 0; j < cols; ++j) {
+            size_t e = i * cols + j;
+            int w = (d->src_dtype == ASCQ_I4) ? load_i4((const uint8_t*)src, e) : ((const int8_t*)src)[e];
+            float s, o = 0.0f;
+            if (d->per_tensor) {
+                /* scalars arrive as dstT values */
+                s = (pt == ASCQ_F16) ? orc_f16_to_f32(orc_f32_to_f16(d->scale))
+                                     : orc_bf16_to_f32(orc_f32_to_bf16(d->scale));
+                o = (pt == ASCQ_F16) ? orc_f16_to_f32(orc_f32_to_f16(d->offset))
+                                     : orc_bf16_to_f32(orc_f32_to_bf16(d->offset));
+            } else {
+                size_t pi = d->is_transpose ? (i * G + j / gs) : ((i / gs) * N + j);
+                s = load_as_f32(scale, pi, pt);
+                if (d->has_offset) {
+                    o = load_as_f32(offset, pi, pt);
+                }
+            }
+            if (d->dst_dtype == ASCQ_F16) {
+                uint16_t h = orc_f32_to_f16((float)w); /* exact */
+                if (d->has_offset) {
+                    h = orc_f16_add(h, orc_f32_to_f16(o));
+                }
+                ((uint16_t*)dst)[e] = orc_f16_mul(orc_f32_to_f16(s), h);
+            } else {
+                volatile float t = (float)w;
+                if (d->has_offset) {
+                    volatile float t2 = t + o;
+                    t = t2;
+                }
+                volatile float r = t * s;
+                ((uint16_t*)dst)[e] = orc_f32_to_bf16(r);
+            }
+        }
+    }
+    return 0;
+}
+
+/* ------------------------------------------------- Matmul int8 quant path */
+/* ref: examples/01_simd_cpp_api/05_best_practices/03_fusion_compute/quant_group_matmul_high_performance/scripts/
+ *      gen_data.py:19-23 (FastGelu closed form), evaluated in fp32 with libm expf. */
+float orc_faster_gelu(float x)
+{
+    float ax = fabsf(x);
+    float x2 = expf(0.851f * (x - ax));
+    float x3 = 1.0f + expf(-1.702f * ax);
+    return x * x2 / x3;
+}
+
+/* The fp32 scale a quant parameter word carries.
+ * ref: examples/01_simd_cpp_api/03_basic_api/03_matrix_compute/fixpipe_l0c2gm/scripts/gen_data_s322f16.py:37-66
+ *      (bits [31:13] = sign, 8 exponent, 10 mantissa bits); matmul_quant/scripts/gen_data.py:36-40 (& 0xFFFFE000). */
+float orc_quant_word_scale(uint64_t w, int scale_format)
+{
+    uint32_t lo = (uint32_t)(w & 0xFFFFFFFFull);
+    if (scale_format == ASCQ_MM_SCALE_U64) {
+        lo &= 0xFFFFE000u;
+    }
+    return bits_f32(lo);
+}
+
+/* Epilogue applied to one int32 accumulator.
+ * ref: impl/adv_api/detail/matmul/stage/copy_cube_out/quant/quant_processor_fixpipe.h:89-117,197-222 (mode selection),
+ *      fixpipe_l0c2gm/scripts/gen_data_s322f16.py:76-102 (deqf16: fp32 multiply, saturate to the fp16 range),
+ *      gen_data_s322s8.py:76-97 (req8: round, saturate to 9 bits, add offset, saturate to 8 bits),
+ *      quant_group_matmul_custom.asc:433-452 (channel scale, then token scale, then activation). */
+static inline void mm_epilogue(const ascq_matmul_desc* d, void* c, size_t idx, int32_t acc, uint64_t qword,
+                               const float* tok_scale, size_t row, const void* bias, size_t bias_idx)
+{
+    if (d->quant_mode == ASCQ_MM_QUANT_NONE) {
+        ((int32_t*)c)[idx] = acc;
+        return;
+    }
+    float s = orc_quant_word_scale(qword, d->scale_format);
+    volatile float v = (float)acc * s;
+    if (d->has_tok_scale) {
+        volatile float t = v * tok_scale[row];
+        v = t;
+    }
+    if (d->bias_kind == ASCQ_MM_BIAS_F32_POST) {
+        volatile float t = v + ((const float*)bias)[bias_idx];
+        v = t;
+    } else if (d->bias_kind == ASCQ_MM_BIAS_BF16_POST) {
+        volatile float t = v + orc_bf16_to_f32(((const uint16_t*)bias)[bias_idx]);
+        v = t;
+    }
+    if (d->activation == ASCQ_MM_ACT_FASTER_GELU) {
+        v = orc_faster_gelu(v);
+    }
+    float r = v;
+    switch (d->out_dtype) {
+        case ASCQ_F16: {
+            if (r > 65504.0f) r = 65504.0f;
+            if (r < -65504.0f) r = -65504.0f;
+            uint16_t h = orc_f32_to_f16(r);
+            if ((h & 0x7FFFu) == 0x7C00u) {
+                h = (uint16_t)((h & 0x8000u) | 0x7BFFu);
+            }
+            ((uint16_t*)c)[idx] = h;
+            break;
+        }
+        case ASCQ_BF16: ((uint16_t*)c)[idx] = orc_f32_to_bf16(r); break;
+        case ASCQ_F32: ((float*)c)[idx] = r; break;
+        case ASCQ_I8: {
+            double q = nearbyint((double)r);
+            if (q > 255.0) q = 255.0;
+            if (q < -256.0) q = -256.0;
+            int off = (int)((qword >> 37) & 0x1FF); /* the spec script adds the 9 bits as an unsigned value */
+            int t = (int)q + off;
+            if ((qword >> 46) & 1) {
+                if (t > 127) t = 127;
+                if (t < -128) t = -128;
+            } else {
+                if (t > 255) t = 255;
+                if (t < 0) t = 0;
+            }
+            ((int8_t*)c)[idx] = (int8_t)t;
+            break;
+        }
+        default: break;
+    }
+}
+
+/* Exact int32 accumulation of rows [r0, r1) of A [.., k] with B [k, n] (or [n, k] when trans_b). */
+static void mm_rows(const ascq_matmul_desc* d, void* c, const int8_t* a, const int8_t* b, const void* bias,
+                    size_t bias_row_off, const uint64_t* qv, const float* qvf, const float* tok_scale, size_t r0,
+                    size_t r1)
+{
+    size_t n = d->n, k = d->k, lda = d->trans_a ? d->m : d->k;
+#pragma omp parallel
+    {
+        int32_t* acc = (int32_t*)malloc(n * sizeof(int32_t));
+#pragma omp for schedule(dynamic, 4)
+        for (size_t i = r0; i < r1; ++i) {
+            for (size_t j = 0; j < n; ++j) {
+                acc[j] = (d->bias_kind == ASCQ_MM_BIAS_I32_PRE) ? ((const int32_t*)bias)[bias_row_off + j] : 0;
+            }
+            if (!d->trans_b) {
+                for (size_t kk = 0; kk < k; ++kk) {
+                    int32_t av = d->trans_a ? a[kk * lda + i] : a[i * lda + kk];
+                    const int8_t* brow = b + kk * n;
+                    for (size_t j = 0; j < n; ++j) {
+                        acc[j] += av * (int32_t)brow[j];
+                    }
+                }
+            } else {
+                for (size_t j = 0; j < n; ++j) {
+                    const int8_t* bcol = b + j * k;
+                    int32_t s = 0;
+                    for (size_t kk = 0; kk < k; ++kk) {
+                        int32_t av = d->trans_a ? a[kk * lda + i] : a[i * lda + kk];
+                        s += av * (int32_t)bcol[kk];
+                    }
+                    acc[j] += s;
+                }
+            }
+            for (size_t j = 0; j < n; ++j) {
+                uint64_t w;
+                if (d->quant_mode == ASCQ_MM_QUANT_VECTOR) {
+                    w = (d->scale_format == ASCQ_MM_SCALE_U64) ? qv[bias_row_off + j]
+                                                                : (uint64_t)f32_bits(qvf[bias_row_off + j]);
+                } else {
+                    w = d->quant_scalar;
+                }
+                mm_epilogue(d, c, i * n + j, acc[j], w, tok_scale, i, bias, bias_row_off + j);
+            }
+        }
+        free(acc);
+    }
+}
+
+/* ref: include/adv_api/matmul/matmul.h:175-185; impl/adv_api/detail/matmul/matmul_impl_base.h:355-378;
+ *      stage/compute/mmad_compute.h:40-82 (an int32 bias is the accumulator's initial value);
+ *      examples/01_simd_cpp_api/04_advanced_api/00_matmul/matmul_quant/scripts/gen_data.py:20-51. */
+int orc_matmul_w8a8(const ascq_matmul_desc* d, void* c, const int8_t* a, const int8_t* b, const void* bias,
+                    const void* quant_vector, const float* tok_scale)
+{
+    mm_rows(d, c, a, b, bias, 0, (const uint64_t*)quant_vector, (const float*)quant_vector, tok_scale, 0, d->m);
+    return 0;
+}
+
+/* Same, restricted to rows [r0, r1): lets a benchmark time a bounded sample of a large problem. */
+int orc_matmul_w8a8_rows(const ascq_matmul_desc* d, void* c, const int8_t* a, const int8_t* b, const void* bias,
+                         const void* quant_vector, const float* tok_scale, uint32_t r0, uint32_t r1)
+{
+    mm_rows(d, c, a, b, bias, 0, (const uint64_t*)quant_vector, (const float*)quant_vector, tok_scale, r0, r1);
+    return 0;
+}
+
+/* ref: examples/.../quant_group_matmul_high_performance/quant_group_matmul_custom.asc:255-289 (group walk, groups
+ *      with a non-positive count are skipped), :425-454 (epilogue order); scripts/gen_data.py:31-57 (cumsum split). */
+int orc_group_matmul_w8a8(const ascq_group_matmul_desc* g, void* y, const int8_t* x, const int8_t* w,
+                          const void* bias, const float* scale, const float* tok_scale, const int64_t* group_list)
+{
+    const ascq_matmul_desc* d = &g->mm;
+    size_t n = d->n, k = d->k;
+    int64_t off = 0;
+    for (uint32_t gi = 0; gi < g->groups; ++gi) {
+        int64_t cnt;
+        if (g->group_list_kind == ASCQ_GROUP_LIST_PREFIX_SUM) {
+            cnt = group_list[gi] - off;
+        } else {
+            cnt = group_list[gi];
+        }
+        if (cnt <= 0) {
+            continue;
+        }
+        int64_t end = off + cnt;
+        if (end > (int64_t)d->m) {
+            end = d->m;
+        }
+        if (end > off) {
+            mm_rows(d, y, x, w + (size_t)gi * k * n, bias, (size_t)gi * n, NULL, scale, tok_scale, (size_t)off,
+                    (size_t)end);
+        }
+        off += cnt;
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------- W4A16 */
+/* Weight de-quantisation = AscendAntiQuant<int4b_t, half>, half math
+ * (ref: impl/adv_api/detail/quantization/antiquant/ascend_antiquant_impl.h:47-135), followed by an fp32-accumulated
+ * dot product in increasing k order and one rounding to half. */
+int orc_matmul_w4a16(const ascq_w4a16_desc* d, uint16_t* y, const uint16_t* x, const uint8_t* w,
+                     const uint16_t* scale, const uint16_t* offset)
+{
+    size_t M = d->m, N = d->n, K = d->k, gs = d->group_size;
+#pragma omp parallel
+    {
+        double* acc = (double*)malloc(N * sizeof(double));
+#pragma omp for schedule(static)
+        for (size_t i = 0; i < M; ++i) {
+            for (size_t j = 0; j < N; ++j) {
+                acc[j] = 0.0;
+            }
+            for (size_t kk = 0; kk < K; ++kk) {
+                float xv = orc_f16_to_f32(x[i * K + kk]);
+                size_t g = kk / gs;
+                for (size_t j = 0; j < N; ++j) {
+                    uint16_t h = orc_f32_to_f16((float)load_i4(w, kk * N + j));
+                    if (d->has_offset) {
+                        h = orc_f16_add(h, offset[g * N + j]);
+                    }
+                    uint16_t wd = orc_f16_mul(scale[g * N + j], h);
+                    acc[j] += (double)xv * (double)orc_f16_to_f32(wd);
+                }
+            }
+            for (size_t j = 0; j < N; ++j) {
+                y[i * N + j] = orc_f64_to_f16(acc[j]);
+            }
+        }
+        free(acc);
+    }
+    return 0;
+}
+
+/* Only the weight de-quantisation of output columns [j0, j1) for one activation row: bounded CPU timing sample. */
+int orc_matmul_w4a16_cols(const ascq_w4a16_desc* d, uint16_t* y, const uint16_t* x, const uint8_t* w,
+                          const uint16_t* scale, const uint16_t* offset, uint32_t j0, uint32_t j1)
+{
+    size_t N = d->n, K = d->k, gs = d->group_size;
+    for (size_t i = 0; i < d->m; ++i) {
+#pragma omp parallel for schedule(static)
+        for (size_t j = j0; j < j1; ++j) {
+            double acc = 0.0;
+            for (size_t kk = 0; kk < K; ++kk) {
+                size_t g = kk / gs;
+                uint16_t h = orc_f32_to_f16((float)load_i4(w, kk * N + j));
+                if (d->has_offset) {
+                    h = orc_f16_add(h, offset[g * N + j]);
+                }
+                uint16_t wd = orc_f16_mul(scale[g * N + j], h);
+                acc += (double)orc_f16_to_f32(x[i * K + kk]) * (double)orc_f16_to_f32(wd);
+            }
+            y[i * N + j] = orc_f64_to_f16(acc);
+        }
+    }
+    return 0;
+}
+
+/* ------------------------------------------------ vectorised array helpers */
+void orc_f32_to_f16_array(uint16_t* dst, const float* src, size_t n)
+{
+    for (size_t i = 0; i < n; ++i) dst[i] = orc_f32_to_f16(src[i]);
+}
+void orc_f16_to_f32_array(float* dst, const uint16_t* src, size_t n)
+{
+    for (size_t i = 0; i < n; ++i) dst[i] = orc_f16_to_f32(src[i]);
+}
+void orc_f32_to_bf16_array(uint16_t* dst, const float* src, size_t n)
+{
+    for (size_t i = 0; i < n; ++i) dst[i] = orc_f32_to_bf16(src[i]);
+}
+void orc_f16_mul_array(uint16_t* dst, const uint16_t* a, const uint16_t* b, size_t n)
+{
+    for (size_t i = 0; i < n; ++i) dst[i] = orc_f16_mul(a[i], b[i]);
+}
+void orc_f16_add_array(uint16_t* dst, const uint16_t* a, const uint16_t* b, size_t n)
+{
+    for (size_t i = 0; i < n; ++i) dst[i] = orc_f16_add(a[i], b[i]);
+}
+void orc_round_sat8_array(int8_t* dst, const float* src, size_t n, int round_mode)
+{
+    for (size_t i = 0; i < n; ++i) dst[i] = orc_round_sat8((double)src[i], round_mode);
+}

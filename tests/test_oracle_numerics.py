@@ -1,0 +1,112 @@
+"""Pins of the oracle's scalar numerics against independent implementations (numpy's float16, torch's bfloat16),
+closed forms, and the worked examples of the reference's precision-conversion document."""
+import numpy as np
+import pytest
+import torch
+
+import orc
+from ascq import _abi as abi
+
+
+def test_f16_to_f32_all_patterns():
+    bits = np.arange(65536, dtype=np.uint16)
+    got = orc.f16_bits_to_f32(bits)
+    want = bits.view(np.float16).astype(np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+    assert np.all(np.isnan(got[nan]))
+
+
+def test_f32_to_f16_roundtrip_and_random():
+    bits = np.arange(65536, dtype=np.uint16)
+    f = bits.view(np.float16).astype(np.float32)
+    ok = ~np.isnan(f)
+    assert np.array_equal(orc.f32_to_f16_bits(f)[ok], bits[ok])
+    rng = np.random.default_rng(1)
+    x = np.concatenate([
+        rng.standard_normal(2_000_000).astype(np.float32) * np.float32(100.0),
+        (rng.standard_normal(500_000) * 1e-6).astype(np.float32),           # subnormal results
+        rng.integers(0, 2**32, 2_000_000, dtype=np.uint64).astype(np.uint32).view(np.float32),  # any bit pattern
+    ])
+    x = x[~np.isnan(x)]
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    assert np.array_equal(orc.f32_to_f16_bits(x), want)
+
+
+def test_f64_to_f16_ties_go_to_even():
+    # the exact midpoint of two adjacent half values must round to the one with an even mantissa
+    bits = np.arange(0, 0x7BFF, dtype=np.uint16)
+    lo = bits.view(np.float16).astype(np.float64)
+    hi = (bits + 1).astype(np.uint16).view(np.float16).astype(np.float64)
+    mid = (lo + hi) / 2
+    L = orc.lib()
+    got = np.array([L.orc_f64_to_f16(float(v)) for v in mid[::7]], dtype=np.uint16)
+    b = bits[::7]
+    want = np.where(b % 2 == 0, b, b + 1).astype(np.uint16)
+    assert np.array_equal(got, want)
+    # doc example: 0.5 + 2^-12 -> 0.5 under RINT (precision_conversion.md:520-534)
+    assert L.orc_f32_to_f16(0.5 + 2.0**-12) == np.float16(0.5).view(np.uint16)
+    # overflow goes to infinity, 65520 is the first value that does
+    assert L.orc_f32_to_f16(65519.0) == 0x7BFF and L.orc_f32_to_f16(65520.0) == 0x7C00
+
+
+def test_f16_mul_add_against_numpy_half():
+    rng = np.random.default_rng(2)
+    n = 4_000_000
+    a = rng.integers(0, 65536, n).astype(np.uint16)
+    b = rng.integers(0, 65536, n).astype(np.uint16)
+    # concentrate half of the pairs where products / sums stay finite and hit subnormals and ties
+    a[: n // 2] = (rng.standard_normal(n // 2) * 8).astype(np.float16).view(np.uint16)
+    b[: n // 2] = (rng.standard_normal(n // 2) * 0.01).astype(np.float16).view(np.uint16)
+    af, bf = a.view(np.float16), b.view(np.float16)
+    with np.errstate(all="ignore"):
+        wm = (af * bf)
+        wa = (af + bf)
+    gm = orc.f16_mul_bits(a, b).view(np.float16)
+    ga = orc.f16_add_bits(a, b).view(np.float16)
+    for got, want in ((gm, wm), (ga, wa)):
+        ok = ~np.isnan(want)
+        assert np.array_equal(got[ok].view(np.uint16), want[ok].view(np.uint16))
+        assert np.all(np.isnan(got[~ok]))
+
+
+def test_bf16_against_torch():
+    rng = np.random.default_rng(3)
+    x = np.concatenate([
+        rng.standard_normal(1_000_000).astype(np.float32),
+        rng.integers(0, 2**32, 1_000_000, dtype=np.uint64).astype(np.uint32).view(np.float32),
+    ])
+    x = x[~np.isnan(x)]
+    want = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(orc.f32_to_bf16_bits(x), want)
+    # doc example precision_conversion.md:541-553: 0.5 + 2^-9 + 2^-11 -> 0.5 + 2^-8 under RINT
+    got = orc.f32_to_bf16_bits(np.array([0.5 + 2.0**-9 + 2.0**-11], dtype=np.float32))
+    assert orc.bf16_bits_to_f32(got)[0] == np.float32(0.5 + 2.0**-8)
+
+
+def test_int32_to_float_doc_example():
+    # precision_conversion.md:427-437: 2^25 + 3 -> 2^25 + 4 under RINT; the oracle uses the C cast (RNE)
+    d = abi.DequantDesc(policy=abi.PER_TENSOR, src_dtype=abi.I32, scale_dtype=abi.F32, dst_dtype=abi.F32,
+                        mode=abi.DEQUANT_WITH_MULTI_ROW, scale=1.0, m=1, n=8, cal_count=8)
+    src = np.full((1, 8), 2**25 + 3, dtype=np.int32)
+    assert orc.dequant(d, src)[0, 0] == np.float32(2**25 + 4)
+
+
+@pytest.mark.parametrize("mode,fn", [
+    (abi.CAST_RINT, np.rint), (abi.CAST_NONE, np.rint), (abi.CAST_FLOOR, np.floor), (abi.CAST_CEIL, np.ceil),
+    (abi.CAST_TRUNC, np.trunc), (abi.CAST_ROUND, lambda v: np.sign(v) * np.floor(np.abs(v) + 0.5)),
+])
+def test_round_sat8_modes(mode, fn):
+    x = np.concatenate([np.arange(-140, 140, 0.25), [127.5, 127.49, -128.5, -128.51, 1e9, -1e9, np.inf, -np.inf]])
+    x = x.astype(np.float32)
+    want = np.clip(fn(x.astype(np.float64)), -128, 127).astype(np.int8)
+    assert np.array_equal(orc.round_sat8(x, mode), want)
+
+
+def test_round_sat8_doc_example():
+    # precision_conversion.md:242-252: half 2^7 - 0.5 saturates to 2^7 - 1 in every mode
+    for mode in (abi.CAST_RINT, abi.CAST_FLOOR, abi.CAST_CEIL, abi.CAST_ROUND, abi.CAST_TRUNC):
+        assert orc.round_sat8(np.array([127.5], np.float32), mode)[0] == 127
+    # ties to even under RINT
+    assert list(orc.round_sat8(np.array([0.5, 1.5, 2.5, -0.5, -1.5, -2.5], np.float32))) == [0, 2, 2, 0, -2, -2]

@@ -1,0 +1,455 @@
+"""Pins of the oracle's operators: the reference's documented examples, its example golden formulas evaluated with
+numpy's own float16 arithmetic, brute-force integer matmul, and closed-form identities."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import orc
+from ascq import _abi as abi
+
+GOLD = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "doc_examples.json")))
+U16 = np.uint16
+
+
+def h(x):
+    return np.asarray(x, dtype=np.float16)
+
+
+# ------------------------------------------------------------------ AscendQuant
+def quant_desc(**kw):
+    d = abi.QuantDesc(policy=abi.PER_TENSOR, src_dtype=abi.F16, scale_dtype=abi.F16, compute=abi.COMPUTE_F16,
+                      round_mode=abi.CAST_RINT, offset_kind=abi.OFFSET_SCALAR, k_dim=1, scale=1.0, offset=0.0)
+    for k, v in kw.items():
+        setattr(d, k, v)
+    return d
+
+
+def test_quant_doc_example():
+    g = GOLD["ascend_quant_md_495_509"]
+    x = h(g["x"])
+    y = orc.quant(quant_desc(scale=g["scale"], offset=g["offset"], cal_count=x.size), x)
+    assert list(y[:3]) == g["y_head"] and y[3] == g["y_509"]
+
+
+def test_quant_per_tensor_matches_example_golden_formula_all_halves():
+    # examples/.../03_quantization/quant/scripts/gen_data.py:29 (dav-2201): np.round(src*2.0+0.9) on a half array
+    bits = np.arange(65536, dtype=U16)
+    x = bits.view(np.float16)
+    x = x[np.isfinite(x) & (np.abs(x.astype(np.float32)) <= 60)]
+    want = np.round(x * np.float16(2.0) + np.float16(0.9)).astype(np.int8)
+    got = orc.quant(quant_desc(scale=2.0, offset=0.9, cal_count=x.size), x)
+    assert np.array_equal(got, want)
+    # float source is cast to half first (ascend_quant_pre_impl.h:339-343)
+    got32 = orc.quant(quant_desc(src_dtype=abi.F32, scale=2.0, offset=0.9, cal_count=x.size), x.astype(np.float32))
+    assert np.array_equal(got32, want)
+
+
+def test_quant_per_channel_half_math_and_saturation():
+    rng = np.random.default_rng(5)
+    rows, n = 37, 64
+    x = h(rng.standard_normal((rows, n)) * 3)
+    s = h(rng.uniform(1, 60, n))
+    o = h(rng.uniform(-3, 3, n))
+    with np.errstate(over="ignore"):
+        want = np.clip(np.rint(((x * s) + o).astype(np.float64)), -128, 127).astype(np.int8)  # numpy half ops round once each
+    d = quant_desc(policy=abi.PER_CHANNEL, offset_kind=abi.OFFSET_TENSOR, n=n, cal_count=rows * n)
+    assert np.array_equal(orc.quant(d, x, s, o), want)
+    assert (want == 127).any() and (want == -128).any()
+    # invariants: scale 1, offset 0 is the identity on small integers; output is monotone in x
+    ints = h(np.arange(-128, 128))
+    assert np.array_equal(orc.quant(quant_desc(cal_count=256), ints), np.arange(-128, 128).astype(np.int8))
+    xs = np.sort(h(rng.standard_normal(4096) * 50))
+    ys = orc.quant(quant_desc(scale=1.7, offset=0.3, cal_count=xs.size), xs)
+    assert np.all(np.diff(ys.astype(np.int32)) >= 0)
+
+
+@pytest.mark.parametrize("rmode", [abi.CAST_RINT, abi.CAST_FLOOR, abi.CAST_CEIL, abi.CAST_ROUND, abi.CAST_TRUNC])
+def test_quant_per_token_fp32_and_quantize_agree(rmode):
+    rng = np.random.default_rng(6)
+    m, n = 10, 288
+    x = rng.standard_normal((m, n)).astype(np.float32)
+    xb = orc.f32_to_bf16_bits(x)
+    s = rng.uniform(5, 90, m).astype(np.float32)
+    o = rng.uniform(-2, 2, m).astype(np.float32)
+    base = dict(policy=abi.PER_TOKEN, src_dtype=abi.BF16, scale_dtype=abi.F32, round_mode=rmode,
+                offset_kind=abi.OFFSET_TENSOR, m=m, n=n, cal_count=m * n)
+    a3 = orc.quant(quant_desc(compute=abi.COMPUTE_SCALE_T, **base), xb, s, o)
+    a4 = orc.quant(quant_desc(compute=abi.COMPUTE_F32, **base), xb, s, o)
+    assert np.array_equal(a3, a4)
+    xf = orc.bf16_bits_to_f32(xb)
+    v = (xf * s[:, None] + o[:, None]).astype(np.float64)          # numpy fp32 ops: one rounding each
+    fn = {abi.CAST_RINT: np.rint, abi.CAST_FLOOR: np.floor, abi.CAST_CEIL: np.ceil, abi.CAST_TRUNC: np.trunc,
+          abi.CAST_ROUND: lambda t: np.sign(t) * np.floor(np.abs(t) + 0.5)}[rmode]
+    assert np.array_equal(a3, np.clip(fn(v), -128, 127).astype(np.int8).reshape(a3.shape))
+
+
+@pytest.mark.parametrize("k_dim", [0, 1])
+@pytest.mark.parametrize("gs", [32, 64, 128, 256])
+def test_quant_per_group_indexing(k_dim, gs):
+    rng = np.random.default_rng(7)
+    m, n = (10, 256) if k_dim == 1 else (256, 32)
+    x = rng.standard_normal((m, n)).astype(np.float32)
+    if k_dim == 1:
+        s = rng.uniform(5, 60, (m, -(-n // gs))).astype(np.float32)
+        sx = np.repeat(s, gs, axis=1)[:, :n]
+    else:
+        s = rng.uniform(5, 60, (-(-m // gs), n)).astype(np.float32)
+        sx = np.repeat(s, gs, axis=0)[:m]
+    d = quant_desc(policy=abi.PER_GROUP, src_dtype=abi.F32, scale_dtype=abi.F32, compute=abi.COMPUTE_F32,
+                   offset_kind=abi.OFFSET_NONE, k_dim=k_dim, m=m, n=n, cal_count=m * n, group_size=gs)
+    want = np.clip(np.rint((x * sx).astype(np.float64)), -128, 127).astype(np.int8)
+    assert np.array_equal(orc.quant(d, x, s), want)
+
+
+def test_quant_half_and_bf16_scale_type_math():
+    rng = np.random.default_rng(8)
+    m, n = 7, 288
+    x = h(rng.standard_normal((m, n)))
+    s = h(rng.uniform(5, 90, m))
+    d = quant_desc(policy=abi.PER_TOKEN, compute=abi.COMPUTE_SCALE_T, offset_kind=abi.OFFSET_NONE, m=m, n=n,
+                   cal_count=m * n)
+    want = np.clip(np.rint((x * s[:, None]).astype(np.float64)), -128, 127).astype(np.int8)
+    assert np.array_equal(orc.quant(d, x, s), want)
+    # bf16: product rounded to bf16 before the integer rounding (checked with torch's bf16 multiply)
+    import torch
+    xb = torch.randn(m, n, generator=torch.Generator().manual_seed(0)).to(torch.bfloat16)
+    sb = (torch.rand(m, generator=torch.Generator().manual_seed(1)) * 80 + 5).to(torch.bfloat16)
+    prod = (xb * sb[:, None]).float().numpy().astype(np.float64)
+    d = quant_desc(policy=abi.PER_TOKEN, src_dtype=abi.BF16, scale_dtype=abi.BF16, compute=abi.COMPUTE_SCALE_T,
+                   offset_kind=abi.OFFSET_NONE, m=m, n=n, cal_count=m * n)
+    got = orc.quant(d, xb.view(torch.int16).numpy().view(U16), sb.view(torch.int16).numpy().view(U16))
+    assert np.array_equal(got, np.clip(np.rint(prod), -128, 127).astype(np.int8))
+
+
+def test_dynamic_quant_per_token():
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((5, 4096)).astype(np.float32)
+    x[3] = 0
+    xb = orc.f32_to_bf16_bits(x)
+    xf = orc.bf16_bits_to_f32(xb)
+    q, ts = orc.dynamic_quant_per_token(abi.BF16, xb)
+    amax = np.abs(xf).max(axis=1)
+    assert ts[3] == 1.0 and not q[3].any()
+    ok = amax > 0
+    assert np.array_equal(ts[ok], (amax[ok] / np.float32(127.0)).astype(np.float32))
+    inv = (np.float32(127.0) / amax[ok]).astype(np.float32)
+    want = np.clip(np.rint((xf[ok] * inv[:, None]).astype(np.float64)), -128, 127).astype(np.int8)
+    assert np.array_equal(q[ok], want)
+    assert np.abs(q[ok]).max(axis=1).min() == 127  # the row maximum always maps to +-127
+
+
+# ------------------------------------------------------------------ AscendDequant
+def test_dequant_doc_example():
+    g = GOLD["ascend_dequant_md_385_401"]
+    src = np.array(g["src"], dtype=np.int32)
+    scale = np.array(g["scale"], dtype=np.float32)
+    d = abi.DequantDesc(policy=abi.PER_CHANNEL, src_dtype=abi.I32, scale_dtype=abi.F32, dst_dtype=abi.F32,
+                        mode=abi.DEQUANT_WITH_MULTI_ROW, m=g["m"], n=g["n"], cal_count=g["cal_count"])
+    got = orc.dequant(d, src, scale)
+    want = np.array(g["dst"], dtype=np.float32)
+    assert np.allclose(got, want, rtol=1e-6, atol=0) and np.array_equal(got[:, 6:], src[:, 6:].astype(np.float32))
+    # scalar form of the same example (columns >= calCount converted, not scaled)
+    d.policy, d.scale = abi.PER_TENSOR, 2.2
+    got = orc.dequant(d, src)
+    assert np.array_equal(got[:, :6], (src[:, :6].astype(np.float32) * np.float32(2.2)))
+    assert np.array_equal(got[:, 6:], src[:, 6:].astype(np.float32))
+
+
+@pytest.mark.parametrize("dst,scale_t", [(abi.F16, abi.U64), (abi.F32, abi.F32), (abi.F32, abi.BF16),
+                                         (abi.BF16, abi.BF16), (abi.BF16, abi.F32)])
+def test_dequant_type_table_and_row_padding(dst, scale_t):
+    # examples/.../03_quantization/dequant/scripts/gen_data.py:21-27: golden[j][i] = inp[j][i] * scale[i]
+    import torch
+    rng = np.random.default_rng(10)
+    m, n, cal = 6, 40, 24            # 40 bf16/half columns pad to 48; fp32 rows need no padding
+    src = rng.integers(-2**20, 2**20, (m, n), dtype=np.int32)
+    sf = rng.uniform(1e-5, 1e-3, n).astype(np.float32)
+    if scale_t == abi.BF16:
+        sc = orc.f32_to_bf16_bits(sf)
+        sf = orc.bf16_bits_to_f32(sc)
+    elif scale_t == abi.U64:
+        sc = sf.view(np.uint32).astype(np.uint64) | (np.uint64(0x1234) << np.uint64(32))  # the high word is ignored
+    else:
+        sc = sf
+    d = abi.DequantDesc(policy=abi.PER_CHANNEL, src_dtype=abi.I32, scale_dtype=scale_t, dst_dtype=dst,
+                        mode=abi.DEQUANT_WITH_MULTI_ROW, m=m, n=n, cal_count=cal)
+    fill = 0x7E7E if dst != abi.F32 else 0
+    got = orc.dequant(d, src, sc, fill=fill)
+    v = src.astype(np.float32)
+    v[:, :cal] = v[:, :cal] * sf[:cal]
+    if dst == abi.F32:
+        assert got.shape == (m, 40) and np.array_equal(got, v)
+    else:
+        assert got.shape == (m, 48)
+        t = torch.from_numpy(v)
+        want = (t.to(torch.bfloat16) if dst == abi.BF16 else t.to(torch.float16)).view(torch.int16).numpy().view(U16)
+        assert np.array_equal(got[:, :40].view(U16), want)
+        assert np.all(got[:, 40:].view(U16) == 0x7E7E)      # padding columns are never written
+
+
+def test_dequant_single_row_reshape_rule():
+    # ascend_dequant_common_impl.h:207-223: {1, 16, 8} + fp32 dst becomes {2, 8, 8}; + bf16 dst stays {1, 16, 8}
+    src = np.arange(16, dtype=np.int32).reshape(1, 16)
+    sc = np.arange(1, 9, dtype=np.float32)
+    d = abi.DequantDesc(policy=abi.PER_CHANNEL, src_dtype=abi.I32, scale_dtype=abi.F32, dst_dtype=abi.F32,
+                        mode=abi.DEQUANT_WITH_SINGLE_ROW, m=1, n=16, cal_count=8)
+    got = orc.dequant(d, src, sc)
+    assert got.shape == (2, 8) and np.array_equal(got, src.reshape(2, 8).astype(np.float32) * sc)
+    d.dst_dtype = abi.BF16
+    got = orc.bf16_bits_to_f32(orc.dequant(d, src, sc))
+    assert got.shape == (1, 16)
+    assert np.array_equal(got[0, :8], np.arange(8) * sc) and np.array_equal(got[0, 8:], np.arange(8, 16))
+    d.mode, d.dst_dtype = abi.DEQUANT_WITH_MULTI_ROW, abi.F32
+    assert orc.dequant(d, src, sc).shape == (1, 16)
+
+
+def test_dequant_per_token_and_group():
+    rng = np.random.default_rng(11)
+    m, n, gs = 10, 256, 64
+    src = rng.integers(-1000, 1000, (m, n), dtype=np.int32)
+    st = rng.uniform(0.01, 1, m).astype(np.float32)
+    d = abi.DequantDesc(policy=abi.PER_TOKEN, src_dtype=abi.I32, scale_dtype=abi.F32, dst_dtype=abi.F32,
+                        mode=abi.DEQUANT_WITH_MULTI_ROW, m=m, n=n, cal_count=n)
+    assert np.array_equal(orc.dequant(d, src, st), src.astype(np.float32) * st[:, None])
+    sg = rng.uniform(0.01, 1, (m, n // gs)).astype(np.float32)
+    d.policy, d.group_size, d.k_dim = abi.PER_GROUP, gs, 1
+    assert np.array_equal(orc.dequant(d, src, sg), src.astype(np.float32) * np.repeat(sg, gs, axis=1))
+    m2 = 128
+    src2 = rng.integers(-1000, 1000, (m2, 32), dtype=np.int32)
+    sg0 = rng.uniform(0.01, 1, (m2 // gs, 32)).astype(np.float32)
+    d2 = abi.DequantDesc(policy=abi.PER_GROUP, src_dtype=abi.I32, scale_dtype=abi.F32, dst_dtype=abi.F32,
+                         mode=abi.DEQUANT_WITH_MULTI_ROW, k_dim=0, m=m2, n=32, cal_count=32, group_size=gs)
+    assert np.array_equal(orc.dequant(d2, src2, sg0), src2.astype(np.float32) * np.repeat(sg0, gs, axis=0))
+
+
+# ------------------------------------------------------------------ AscendAntiQuant
+def aq_desc(**kw):
+    d = abi.AntiQuantDesc(src_dtype=abi.I8, dst_dtype=abi.F16, is_transpose=0, has_offset=1, per_tensor=0)
+    for k, v in kw.items():
+        setattr(d, k, v)
+    return d
+
+
+def test_antiquant_doc_example():
+    g = GOLD["ascend_antiquant_md_469_490"]
+    src = np.full((g["k"], g["n"]), g["src"], dtype=np.int8)
+    off = h(np.full((1, g["n"]), g["offset"]))
+    sc = h(np.full((1, g["n"]), g["scale"]))
+    got = orc.antiquant(aq_desc(k=g["k"], n=g["n"], scale_height=1, scale_width=g["n"], offset_height=1,
+                                offset_width=g["n"]), src, off, sc)
+    assert np.all(got == np.float16(g["dst"]))
+
+
+def test_antiquant_example_golden_formula():
+    # examples/.../03_quantization/antiquant/scripts/gen_data.py:27-39 (seed 10, dav-2201: half arithmetic)
+    np.random.seed(10)
+    src = np.random.uniform(-10, 10, [8, 128]).astype(np.int8)
+    offset = np.random.uniform(-10, 10, [1, 128]).astype(np.float16)
+    scale = np.random.uniform(-10, 10, [1, 128]).astype(np.float16)
+    want = (scale * (src.astype(np.float16) + offset)).astype(np.float16)
+    got = orc.antiquant(aq_desc(k=8, n=128, scale_height=1, scale_width=128), src, offset, scale)
+    assert np.array_equal(got.view(U16), want.view(U16))
+    # bf16 output: fp32 add and multiply, one rounding to bf16 (ascend_antiquant_c220_impl.h:58-75)
+    import torch
+    ob, sb = orc.f32_to_bf16_bits(offset.astype(np.float32)), orc.f32_to_bf16_bits(scale.astype(np.float32))
+    v = (src.astype(np.float32) + orc.bf16_bits_to_f32(ob)) * orc.bf16_bits_to_f32(sb)
+    wantb = torch.from_numpy(v).to(torch.bfloat16).view(torch.int16).numpy().view(U16)
+    gotb = orc.antiquant(aq_desc(dst_dtype=abi.BF16, k=8, n=128, scale_height=1, scale_width=128), src, ob, sb)
+    assert np.array_equal(gotb, wantb)
+
+
+@pytest.mark.parametrize("transpose", [0, 1])
+def test_antiquant_all_int8_and_int4_values_per_group(transpose):
+    rng = np.random.default_rng(12)
+    K, N, G = 256, 32, 4
+    gs = K // G
+    w8 = np.tile(np.arange(-128, 128, dtype=np.int8)[:, None], (1, N))          # every int8 value in every column
+    w4 = rng.integers(-8, 8, (K, N)).astype(np.int8)
+    w4[:16, :] = np.arange(-8, 8, dtype=np.int8)[:, None]
+    sc = h(rng.uniform(-2, 2, (G, N)))
+    of = h(rng.uniform(-9, 9, (G, N)))
+    for src, dt in ((w8, abi.I8), (w4, abi.I4)):
+        want = (np.repeat(sc, gs, 0) * (src.astype(np.float16) + np.repeat(of, gs, 0))).astype(np.float16)
+        s_in, sc_in, of_in = src, sc, of
+        if transpose:
+            s_in, sc_in, of_in = (np.ascontiguousarray(t.T) for t in (src, sc, of))
+            want = np.ascontiguousarray(want.T)
+        if dt == abi.I4:
+            flat = s_in.reshape(-1).astype(np.uint8) & 0xF
+            s_in = (flat[0::2] | (flat[1::2] << 4)).astype(np.uint8)           # even element in the low nibble
+        if transpose:
+            d = aq_desc(src_dtype=dt, is_transpose=1, k=K, n=N, scale_height=N, scale_width=G, offset_height=N,
+                        offset_width=G)
+        else:
+            d = aq_desc(src_dtype=dt, k=K, n=N, scale_height=G, scale_width=N, offset_height=G, offset_width=N)
+        got = orc.antiquant(d, s_in, of_in, sc_in)
+        assert np.array_equal(got.view(U16), want.view(U16))
+        d.has_offset = 0                                                         # scale-only overload
+        want0 = (np.repeat(sc, gs, 0) * src.astype(np.float16)).astype(np.float16)
+        got0 = orc.antiquant(d, s_in, None, sc_in)
+        assert np.array_equal(got0.view(U16), (want0.T if transpose else want0).copy().view(U16))
+
+
+def test_antiquant_per_tensor_scalar():
+    src = np.arange(-128, 128, dtype=np.int8).reshape(8, 32)
+    d = aq_desc(per_tensor=1, scale=0.37, offset=-3.25, k=8, n=32)
+    want = (np.float16(0.37) * (src.astype(np.float16) + np.float16(-3.25))).astype(np.float16)
+    assert np.array_equal(orc.antiquant(d, src).view(U16), want.view(U16))
+
+
+# ------------------------------------------------------------------ Matmul quant path
+def mm_desc(m, n, k, **kw):
+    d = abi.MatmulDesc(m=m, n=n, k=k, out_dtype=abi.I32, quant_mode=abi.MM_QUANT_NONE, scale_format=abi.MM_SCALE_F32)
+    for key, v in kw.items():
+        setattr(d, key, v)
+    return d
+
+
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_matmul_int32_brute_force_and_identities(ta, tb):
+    rng = np.random.default_rng(13)
+    m, n, k = 19, 23, 77
+    a = rng.integers(-128, 128, (m, k)).astype(np.int8)
+    b = rng.integers(-128, 128, (k, n)).astype(np.int8)
+    bias = rng.integers(-1000, 1000, n).astype(np.int32)
+    want = a.astype(np.int64) @ b.astype(np.int64) + bias
+    a_in = np.ascontiguousarray(a.T) if ta else a
+    b_in = np.ascontiguousarray(b.T) if tb else b
+    got = orc.matmul_w8a8(mm_desc(m, n, k, trans_a=ta, trans_b=tb, bias_kind=abi.MM_BIAS_I32_PRE), a_in, b_in, bias)
+    assert np.array_equal(got.astype(np.int64), want)
+    ones = np.ones((m, k), dtype=np.int8)
+    got = orc.matmul_w8a8(mm_desc(m, n, k, trans_b=tb), ones, b_in)
+    assert np.array_equal(got[0], b.astype(np.int64).sum(axis=0))           # A = 1 gives the column sums of B
+
+
+def spec_extract_scale(word):
+    # fixpipe_l0c2gm/scripts/gen_data_s322f16.py:37-66: bits [31:13] decoded as sign, 8 exponent, 10 mantissa bits
+    bits = (int(word) >> 13) & 0x7FFFF
+    sign, exponent, mantissa = (bits >> 18) & 1, (bits >> 10) & 0xFF, bits & 0x3FF
+    return (-1) ** sign * (1 + mantissa / 1024) * (2.0 ** (exponent - 127))
+
+
+def test_quant_word_scale_keeps_19_bits():
+    rng = np.random.default_rng(14)
+    s = np.concatenate([rng.uniform(1e-4, 2.0, 2000), -rng.uniform(1e-4, 2.0, 200)]).astype(np.float32)
+    L = orc.lib()
+    for v in s:
+        w = int(np.float32(v).view(np.uint32)) | (0x155 << 37) | (1 << 46)
+        assert L.orc_quant_word_scale(w, abi.MM_SCALE_U64) == np.float32(spec_extract_scale(w))
+        assert L.orc_quant_word_scale(w, abi.MM_SCALE_F32) == v
+
+
+def test_matmul_deqf16_vector_follows_fixpipe_spec():
+    rng = np.random.default_rng(15)
+    m, n, k = 16, 48, 64
+    a = rng.integers(-10, 10, (m, k)).astype(np.int8)
+    b = rng.integers(-10, 10, (k, n)).astype(np.int8)
+    bias = rng.integers(-2, 2, n).astype(np.int32)
+    qf = rng.uniform(0.1, 2.0, n).astype(np.float32)
+    qf[0], qf[1] = 3000.0, -3000.0                      # forces fp16 saturation on both sides
+    qv = qf.view(np.uint32).astype(np.uint64)
+    acc = a.astype(np.int64) @ b.astype(np.int64) + bias
+    acc[:, 0] = np.abs(acc[:, 0]) + 30
+    # deqf16 (gen_data_s322f16.py:76-102): fp32 multiply by the 19-bit scale, clip to the fp16 range, round to fp16
+    trunc = (qf.view(np.uint32) & np.uint32(0xFFFFE000)).view(np.float32)
+    d = mm_desc(m, n, k, out_dtype=abi.F16, quant_mode=abi.MM_QUANT_VECTOR, scale_format=abi.MM_SCALE_U64,
+                bias_kind=abi.MM_BIAS_I32_PRE)
+    got = orc.matmul_w8a8(d, a, b, bias, qv)
+    acc2 = a.astype(np.int64) @ b.astype(np.int64) + bias
+    want = np.clip(acc2.astype(np.float32) * trunc, -65504, 65504).astype(np.float16)
+    assert np.array_equal(got.view(U16), want.view(U16))
+    assert (np.abs(want.astype(np.float32)) == 65504).any()
+    # the matmul_quant example's own golden (gen_data.py:26-42 casts acc to half first) agrees within its gate
+    gold = (acc2.astype(np.float16).astype(np.float32) * trunc)
+    okc = np.abs(gold) < 60000
+    assert np.isclose(got.astype(np.float32)[okc], gold[okc], rtol=1e-3, atol=1e-3).mean() > 0.999
+    # scalar mode
+    d.quant_mode, d.quant_scalar = abi.MM_QUANT_SCALAR, int(np.float32(0.1).view(np.uint32))
+    got = orc.matmul_w8a8(d, a, b, bias)
+    s01 = (np.float32(0.1).view(np.uint32) & np.uint32(0xFFFFE000)).view(np.float32)
+    assert np.array_equal(got.view(U16), (acc2.astype(np.float32) * s01).astype(np.float16).view(U16))
+
+
+def test_matmul_req8_follows_spec():
+    # gen_data_s322s8.py:76-97: round, clip to [-256, 255], add the 9-bit offset, clip to int8 (sign = 1)
+    rng = np.random.default_rng(16)
+    m, n, k = 8, 32, 32
+    a = rng.integers(-20, 20, (m, k)).astype(np.int8)
+    b = rng.integers(-20, 20, (k, n)).astype(np.int8)
+    scale, off = np.float32(0.0625), 5
+    word = int(scale.view(np.uint32)) | (off << 37) | (1 << 46)
+    d = mm_desc(m, n, k, out_dtype=abi.I8, quant_mode=abi.MM_QUANT_SCALAR, scale_format=abi.MM_SCALE_U64,
+                quant_scalar=word)
+    acc = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
+    want = np.clip(np.clip(np.rint(acc * scale), -256, 255) + off, -128, 127).astype(np.int8)
+    assert np.array_equal(orc.matmul_w8a8(d, a, b), want)
+
+
+def test_matmul_bf16_epilogue_order_token_scale_and_bias():
+    import torch
+    rng = np.random.default_rng(17)
+    m, n, k = 9, 40, 128
+    a = rng.integers(-127, 128, (m, k)).astype(np.int8)
+    b = rng.integers(-127, 128, (k, n)).astype(np.int8)
+    cs = rng.uniform(1e-4, 1e-2, n).astype(np.float32)
+    ts = rng.uniform(1e-3, 1e-1, m).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    acc = (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
+    v = (acc * cs) * ts[:, None] + bias                     # numpy fp32: one rounding per operation, this order
+    want = torch.from_numpy(v).to(torch.bfloat16).view(torch.int16).numpy().view(U16)
+    d = mm_desc(m, n, k, out_dtype=abi.BF16, quant_mode=abi.MM_QUANT_VECTOR, bias_kind=abi.MM_BIAS_F32_POST,
+                has_tok_scale=1)
+    assert np.array_equal(orc.matmul_w8a8(d, a, b, bias, cs, ts), want)
+
+
+def fast_gelu(x):
+    # quant_group_matmul_high_performance/scripts/gen_data.py:19-23
+    ax = np.abs(x)
+    return x * np.exp(0.851 * (x - ax)) / (1 + np.exp(-1.702 * ax))
+
+
+@pytest.mark.parametrize("kind", [abi.GROUP_LIST_COUNTS, abi.GROUP_LIST_PREFIX_SUM])
+def test_group_matmul_against_example_golden(kind):
+    rng = np.random.default_rng(18)
+    G, m, k, n = 5, 96, 64, 48
+    counts = np.array([30, 0, 1, 45, 12], dtype=np.int64)      # an empty group, a one-row group, 8 unassigned rows
+    x = rng.integers(-10, 10, (m, k)).astype(np.int8)
+    w = rng.integers(-10, 10, (G, k, n)).astype(np.int8)
+    scale = rng.normal(0, 0.01, (G, n)).astype(np.float32)
+    tok = rng.normal(0, 0.01, m).astype(np.float32)
+    d = abi.GroupMatmulDesc(mm=mm_desc(m, n, k, out_dtype=abi.F16, quant_mode=abi.MM_QUANT_VECTOR, has_tok_scale=1,
+                                       activation=abi.MM_ACT_FASTER_GELU), groups=G, group_list_kind=kind)
+    gl = counts if kind == abi.GROUP_LIST_COUNTS else np.cumsum(counts)
+    got = orc.group_matmul_w8a8(d, x, w, None, scale, tok, gl, fill=np.float16(777).view(U16).item()
+                                if False else 0)
+    idx = np.concatenate([[0], np.cumsum(counts)])
+    gold = np.zeros((m, n), dtype=np.float64)
+    for g in range(G):
+        s, e = idx[g], idx[g + 1]
+        gold[s:e] = (x[s:e].astype(np.float64) @ w[g].astype(np.float64)) * scale[g].astype(np.float64) \
+            * tok[s:e, None].astype(np.float64)
+    gold = fast_gelu(gold)
+    rows = idx[-1]
+    # the example's gate: rtol = atol = 1e-3, at most 0.01 % mismatches (scripts/verify_result.py:19-21)
+    assert np.isclose(got[:rows].astype(np.float64), gold[:rows], rtol=1e-3, atol=1e-3).mean() >= 0.9999
+    assert not got[rows:].any()                                # rows past the last group are left alone
+
+
+def test_w4a16_against_numpy_half_dequant():
+    rng = np.random.default_rng(19)
+    M, K, N, gs = 3, 256, 64, 128
+    x = h(rng.standard_normal((M, K)))
+    wq = rng.integers(-8, 8, (K, N)).astype(np.int8)
+    flat = wq.reshape(-1).astype(np.uint8) & 0xF
+    packed = (flat[0::2] | (flat[1::2] << 4)).astype(np.uint8)
+    sc = h(rng.uniform(1e-3, 1e-2, (K // gs, N)))
+    of = h(rng.integers(-8, 8, (K // gs, N)))
+    wdq = (np.repeat(sc, gs, 0) * (wq.astype(np.float16) + np.repeat(of, gs, 0))).astype(np.float16)
+    want = (x.astype(np.float64) @ wdq.astype(np.float64)).astype(np.float16)
+    d = abi.W4A16Desc(m=M, n=N, k=K, group_size=gs, has_offset=1)
+    got = orc.matmul_w4a16(d, x, packed, sc, of)
+    assert np.array_equal(got.view(U16), want.view(U16))
+    sub = orc.matmul_w4a16(d, x, packed, sc, of, cols=(8, 24))
+    assert np.array_equal(sub[:, 8:24].view(U16), want[:, 8:24].view(U16))
