@@ -1,0 +1,320 @@
+"""Operator interface of the asc-devkit quantization path on torch device tensors, bound to libascq over its C ABI.
+
+Names and argument meaning follow the reference's `AscendC::` functions (citations below are files of the reference
+tree); a tensor argument is a CUDA/HIP torch tensor whose storage is handed to the library as a raw device pointer.
+torch only provides device memory and the current stream.  Every function raises `AscqError` when the library
+rejects the call; nothing here computes on the CPU.
+"""
+import ctypes as C
+from dataclasses import dataclass
+
+import torch
+
+from . import _abi as abi
+from ._abi import AscqError, check, load_library  # noqa: F401
+
+_DT = {torch.float16: abi.F16, torch.bfloat16: abi.BF16, torch.float32: abi.F32, torch.int8: abi.I8,
+       torch.int32: abi.I32, torch.int64: abi.U64, torch.uint8: abi.I4}
+if hasattr(torch, "uint64"):
+    _DT[torch.uint64] = abi.U64
+_TORCH = {abi.F16: torch.float16, abi.BF16: torch.bfloat16, abi.F32: torch.float32, abi.I8: torch.int8,
+          abi.I32: torch.int32}
+
+
+def _ptr(t):
+    if t is None:
+        return None
+    if not t.is_cuda:
+        raise ValueError("ascq operators take device tensors")
+    if not t.is_contiguous():
+        raise ValueError("ascq operators take contiguous tensors")
+    return C.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dt(t):
+    return _DT[t.dtype]
+
+
+# ------------------------------------------------------------------------------------------------ AscendQuant
+@dataclass
+class AscendQuantConfig:
+    """ref: include/adv_api/quantization/ascend_quant_utils.h:31-71"""
+    has_offset: bool = False
+    k_dim: int = 1
+    round_mode: int = abi.CAST_RINT
+
+
+@dataclass
+class AscendQuantParam:
+    """ref: include/adv_api/quantization/ascend_quant_utils.h:82-87"""
+    m: int
+    n: int
+    cal_count: int
+    group_size: int = 0
+
+
+def _quant(desc, dst, src, scale, offset):
+    check(load_library().ascq_quant(C.byref(desc), _ptr(dst), _ptr(src), _ptr(scale), _ptr(offset), _stream()))
+    return dst
+
+
+def ascend_quant(dst, src, scale, offset, cal_count=None, scale_count=None, offset_count=None):
+    """AscendQuant<T>(dst, src, scale, offset, [scaleCount, offsetCount,] calCount): per-tensor when `scale` is a
+    float, per-channel when it is a tensor (offset: float or tensor).  Every intermediate is fp16.
+    ref: include/adv_api/quantization/ascend_quant.h:63-347."""
+    cal = src.numel() if cal_count is None else cal_count
+    d = abi.QuantDesc(src_dtype=_dt(src), compute=abi.COMPUTE_F16, round_mode=abi.CAST_RINT, k_dim=1, cal_count=cal)
+    if torch.is_tensor(scale):
+        n = scale.numel() if scale_count is None else scale_count
+        d.policy, d.scale_dtype, d.n = abi.PER_CHANNEL, _dt(scale), n
+        if torch.is_tensor(offset):
+            oc = offset.numel() if offset_count is None else offset_count
+            if oc != n:
+                raise AscqError(abi.EINVAL, f"scaleCount {n} must equal offsetCount {oc}")
+            d.offset_kind = abi.OFFSET_TENSOR
+            return _quant(d, dst, src, scale, offset)
+        d.offset_kind, d.offset = abi.OFFSET_SCALAR, float(offset)
+        return _quant(d, dst, src, scale, None)
+    d.policy, d.scale_dtype = abi.PER_TENSOR, _dt(src)
+    d.scale, d.offset, d.offset_kind = float(scale), float(offset), abi.OFFSET_SCALAR
+    return _quant(d, dst, src, None, None)
+
+
+def _policy_quant(compute, dst, src, scale, offset, para, policy, config):
+    d = abi.QuantDesc(policy=policy, src_dtype=_dt(src), compute=compute, round_mode=config.round_mode,
+                      k_dim=config.k_dim, m=para.m, n=para.n, cal_count=para.cal_count, group_size=para.group_size)
+    if policy == abi.PER_TENSOR:
+        d.scale, d.scale_dtype = float(scale), _dt(src)
+        scale = None
+    else:
+        d.scale_dtype = _dt(scale)
+    if not config.has_offset:
+        d.offset_kind, offset = abi.OFFSET_NONE, None
+    elif torch.is_tensor(offset):
+        d.offset_kind = abi.OFFSET_TENSOR
+    else:
+        d.offset_kind, d.offset, offset = abi.OFFSET_SCALAR, float(offset), None
+    return _quant(d, dst, src, scale, offset)
+
+
+def ascend_quant_policy(dst, src, scale, offset, para, policy, config=AscendQuantConfig()):
+    """AscendQuant<dstT, srcT, scaleT, config, policy>(dst, src, scale, offset, para) for PER_TOKEN / PER_GROUP:
+    arithmetic in the scale's dtype.  ref: include/adv_api/quantization/ascend_quant.h:667-762."""
+    return _policy_quant(abi.COMPUTE_SCALE_T, dst, src, scale, offset, para, policy, config)
+
+
+def quantize(dst, src, scale, offset, para, policy, config=AscendQuantConfig()):
+    """Quantize<config>(dst, src, scale, offset, params): always fp32 arithmetic, any policy.
+    ref: include/adv_api/quantization/quantize.h, impl/adv_api/detail/quantization/quantize/quantize_impl.h:923-968."""
+    return _policy_quant(abi.COMPUTE_F32, dst, src, scale, offset, para, policy, config)
+
+
+def dynamic_quant_per_token(x, q=None, tok_scale=None):
+    """Row abs-max -> scale = amax/127 -> AscendQuant PER_TOKEN with 127/amax, in one kernel."""
+    m, n = x.shape
+    q = torch.empty((m, n), dtype=torch.int8, device=x.device) if q is None else q
+    tok_scale = torch.empty(m, dtype=torch.float32, device=x.device) if tok_scale is None else tok_scale
+    check(load_library().ascq_dynamic_quant_per_token(_dt(x), m, n, _ptr(q), _ptr(tok_scale), _ptr(x), _stream()))
+    return q, tok_scale
+
+
+# ---------------------------------------------------------------------------------------------- AscendDequant
+@dataclass
+class DequantParams:
+    """ref: include/adv_api/quantization/ascend_dequant_utils.h:26-30"""
+    m: int
+    n: int
+    cal_count: int
+
+
+def dequant_dst_stride(dst_dtype, n):
+    return load_library().ascq_dequant_dst_stride(_DT[dst_dtype], n)
+
+
+def ascend_dequant(dst, src, deq_scale, params, mode=abi.DEQUANT_WITH_SINGLE_ROW, scale_dtype=None):
+    """AscendDequant<dstT, scaleT, mode>(dst, src, deqScale, {m, n, calCount}); deqScale is a tensor (float32,
+    bfloat16, or uint64 passed as an int64 tensor) or a float.  ref: include/adv_api/quantization/ascend_dequant.h:58-281."""
+    d = abi.DequantDesc(src_dtype=_dt(src), dst_dtype=_dt(dst), mode=mode, m=params.m, n=params.n,
+                        cal_count=params.cal_count)
+    if torch.is_tensor(deq_scale):
+        d.policy = abi.PER_CHANNEL
+        d.scale_dtype = _dt(deq_scale) if scale_dtype is None else scale_dtype
+    else:
+        d.policy, d.scale, d.scale_dtype = abi.PER_TENSOR, float(deq_scale), abi.F32
+        deq_scale = None
+    check(load_library().ascq_dequant(C.byref(d), _ptr(dst), _ptr(src), _ptr(deq_scale), _stream()))
+    return dst
+
+
+def ascend_dequant_policy(dst, src, scale, para, policy, k_dim=1):
+    """AscendDequant<dstT, srcT, scaleT, config, policy> for PER_TOKEN / PER_GROUP.
+    ref: include/adv_api/quantization/ascend_dequant.h:284-305."""
+    d = abi.DequantDesc(policy=policy, src_dtype=_dt(src), scale_dtype=_dt(scale), dst_dtype=_dt(dst),
+                        mode=abi.DEQUANT_WITH_MULTI_ROW, k_dim=k_dim, m=para.m, n=para.n, cal_count=para.cal_count,
+                        group_size=para.group_size)
+    check(load_library().ascq_dequant(C.byref(d), _ptr(dst), _ptr(src), _ptr(scale), _stream()))
+    return dst
+
+
+# -------------------------------------------------------------------------------------------- AscendAntiQuant
+@dataclass
+class AntiQuantShapeInfo:
+    """ref: include/adv_api/quantization/ascend_antiquant_utils.h:27-32"""
+    offset_height: int = 0
+    offset_width: int = 0
+    scale_height: int = 0
+    scale_width: int = 0
+
+
+def ascend_antiquant(dst, src, offset, scale, k, shape_info=AntiQuantShapeInfo(), is_transpose=False, int4=False):
+    """AscendAntiQuant<SrcT, DstT, isTranspose>(dst, src, offset, scale, k, shapeInfo).  `offset` may be None (the
+    scale-only overloads); `scale` / `offset` floats select the per-tensor overloads.  `src` is int8, or uint8 holding
+    packed int4 when int4=True.  ref: include/adv_api/quantization/ascend_antiquant.h:50-199."""
+    elems = dst.numel()
+    d = abi.AntiQuantDesc(src_dtype=abi.I4 if int4 else abi.I8, dst_dtype=_dt(dst), is_transpose=int(is_transpose),
+                          has_offset=int(offset is not None), k=k, n=elems // k,
+                          offset_height=shape_info.offset_height, offset_width=shape_info.offset_width,
+                          scale_height=shape_info.scale_height, scale_width=shape_info.scale_width)
+    if not torch.is_tensor(scale):
+        d.per_tensor, d.scale, d.offset = 1, float(scale), float(offset or 0.0)
+        scale = offset = None
+    check(load_library().ascq_antiquant(C.byref(d), _ptr(dst), _ptr(src), _ptr(offset), _ptr(scale), _stream()))
+    return dst
+
+
+# ------------------------------------------------------------------------------------------ Matmul quant path
+class Matmul:
+    """Host-side mirror of `Matmul<A int8, B int8, C, Bias>` on the quant path: SetTensorA/B, SetBias,
+    SetQuantScalar / SetQuantVector, IterateAll.  ref: include/adv_api/matmul/matmul.h:73-398,
+    impl/adv_api/detail/matmul/matmul_impl_base.h:355-378."""
+
+    def __init__(self, m, n, k, trans_a=False, trans_b=False):
+        self.desc = abi.MatmulDesc(m=m, n=n, k=k, trans_a=int(trans_a), trans_b=int(trans_b), out_dtype=abi.I32,
+                                   quant_mode=abi.MM_QUANT_NONE, scale_format=abi.MM_SCALE_U64)
+        self.a = self.b = self.bias = self.quant = self.tok = None
+        self._ws = None
+
+    def set_tensor_a(self, a):
+        self.a = a
+
+    def set_tensor_b(self, b):
+        self.b = b
+
+    def set_bias(self, bias):
+        """int32 bias: initial value of the accumulator; float32 / bfloat16 bias: added after dequantisation."""
+        self.bias = bias
+        self.desc.bias_kind = {torch.int32: abi.MM_BIAS_I32_PRE, torch.float32: abi.MM_BIAS_F32_POST,
+                               torch.bfloat16: abi.MM_BIAS_BF16_POST}[bias.dtype]
+
+    def set_quant_scalar(self, quant_scalar):
+        """uint64 parameter word (ref: SetQuantScalar), or a Python float for a full-precision fp32 scale."""
+        self.desc.quant_mode = abi.MM_QUANT_SCALAR
+        if isinstance(quant_scalar, float):
+            self.desc.scale_format = abi.MM_SCALE_F32
+            self.desc.quant_scalar = int(torch.tensor(quant_scalar, dtype=torch.float32).view(torch.int32).item()) \
+                & 0xFFFFFFFF
+        else:
+            self.desc.scale_format, self.desc.quant_scalar = abi.MM_SCALE_U64, int(quant_scalar)
+
+    def set_quant_vector(self, quant_vector):
+        """uint64 parameter words (as an int64 / uint64 tensor; ref: SetQuantVector) or a float32 scale tensor."""
+        self.desc.quant_mode = abi.MM_QUANT_VECTOR
+        self.desc.scale_format = abi.MM_SCALE_F32 if quant_vector.dtype == torch.float32 else abi.MM_SCALE_U64
+        self.quant = quant_vector
+
+    def set_token_scale(self, tok_scale):
+        self.tok, self.desc.has_tok_scale = tok_scale, 1
+
+    def set_activation(self, activation):
+        self.desc.activation = activation
+
+    def iterate_all(self, c):
+        self.desc.out_dtype = _dt(c)
+        lib = load_library()
+        need = C.c_size_t(0)
+        check(lib.ascq_matmul_w8a8_workspace_size(C.byref(self.desc), C.byref(need)))
+        if need.value and (self._ws is None or self._ws.numel() * 4 < need.value):
+            self._ws = torch.empty((need.value + 3) // 4, dtype=torch.int32, device=c.device)
+        check(lib.ascq_matmul_w8a8(C.byref(self.desc), _ptr(c), _ptr(self.a), _ptr(self.b), _ptr(self.bias),
+                                   _ptr(self.quant), _ptr(self.tok), _ptr(self._ws) if need.value else None,
+                                   need.value, _stream()))
+        return c
+
+
+def quant_group_matmul(y, x, weight, group_list, scale, per_token_scale=None, bias=None,
+                       group_list_kind=abi.GROUP_LIST_COUNTS, activation=abi.MM_ACT_NONE):
+    """The quantized grouped matmul of the reference's MoE example: x int8 [m, k], weight int8 [g, k, n], scale
+    float32 [g, n], per_token_scale float32 [m], group_list int64 [g] (counts or prefix sums).
+    ref: examples/01_simd_cpp_api/05_best_practices/03_fusion_compute/quant_group_matmul_high_performance/
+    quant_group_matmul_custom.asc:255-454."""
+    g, k, n = weight.shape
+    mm = abi.MatmulDesc(m=x.shape[0], n=n, k=k, out_dtype=_dt(y), quant_mode=abi.MM_QUANT_VECTOR,
+                        scale_format=abi.MM_SCALE_F32, has_tok_scale=int(per_token_scale is not None),
+                        activation=activation)
+    if bias is not None:
+        mm.bias_kind = abi.MM_BIAS_F32_POST if bias.dtype == torch.float32 else abi.MM_BIAS_BF16_POST
+    d = abi.GroupMatmulDesc(mm=mm, groups=g, group_list_kind=group_list_kind)
+    check(load_library().ascq_group_matmul_w8a8(C.byref(d), _ptr(y), _ptr(x), _ptr(weight), _ptr(bias), _ptr(scale),
+                                                _ptr(per_token_scale), _ptr(group_list), _stream()))
+    return y
+
+
+# ------------------------------------------------------------------------------------------------------ W4A16
+_w4_ws = {}
+
+
+def matmul_w4a16(y, x, w_packed, scale, offset=None, group_size=128, workspace=None):
+    """y f16 [m, n] = x f16 [m, k] @ AscendAntiQuant<int4b_t, half>(w [k, n] packed two per byte, per-group params)."""
+    m, k = x.shape
+    n = y.shape[1]
+    d = abi.W4A16Desc(m=m, n=n, k=k, group_size=group_size, has_offset=int(offset is not None))
+    lib = load_library()
+    need = C.c_size_t(0)
+    check(lib.ascq_matmul_w4a16_workspace_size(C.byref(d), C.byref(need)))
+    if workspace is None:
+        key = (x.device, need.value)
+        if key not in _w4_ws:
+            _w4_ws[key] = torch.zeros(max(need.value // 4, 4), dtype=torch.float32, device=x.device)
+        workspace = _w4_ws[key]
+    check(lib.ascq_matmul_w4a16(C.byref(d), _ptr(y), _ptr(x), _ptr(w_packed), _ptr(scale), _ptr(offset),
+                                _ptr(workspace), workspace.numel() * workspace.element_size(), _stream()))
+    return y
+
+
+# ------------------------------------------------------------------------------------------- host size queries
+def _shape(shape):
+    return (C.c_uint32 * len(shape))(*shape), len(shape)
+
+
+def get_ascend_quant_max_min_tmp_size(shape, type_size):
+    """ref: impl/adv_api/tiling/quantization/ascend_quant_tiling_impl.cpp:60-68"""
+    mx, mn = C.c_uint32(0), C.c_uint32(0)
+    arr, nd = _shape(shape)
+    check(load_library().ascq_get_ascend_quant_max_min_tmp_size(arr, nd, type_size, C.byref(mx), C.byref(mn)))
+    return mx.value, mn.value
+
+
+def get_ascend_dequant_max_min_tmp_size(shape, type_size):
+    """ref: impl/adv_api/tiling/quantization/ascend_dequant_tiling_impl.cpp:95-118"""
+    mx, mn = C.c_uint32(0), C.c_uint32(0)
+    arr, nd = _shape(shape)
+    check(load_library().ascq_get_ascend_dequant_max_min_tmp_size(arr, nd, type_size, C.byref(mx), C.byref(mn)))
+    return mx.value, mn.value
+
+
+def get_ascend_antiquant_max_min_tmp_size(src_shape, scale_shape, is_transpose, input_dtype, output_dtype):
+    """ref: impl/adv_api/tiling/quantization/ascend_antiquant_tiling_impl.cpp:70-190"""
+    mx, mn = C.c_uint32(0), C.c_uint32(0)
+    a, na = _shape(src_shape)
+    b, nb = _shape(scale_shape)
+    check(load_library().ascq_get_ascend_antiquant_max_min_tmp_size(a, na, b, nb, int(is_transpose), input_dtype,
+                                                                    output_dtype, C.byref(mx), C.byref(mn)))
+    return mx.value, mn.value
+
+
+def pack_quant_param(scale, offset9=0, is_signed=True):
+    return int(load_library().ascq_pack_quant_param(float(scale), int(offset9), int(is_signed)))

@@ -1,0 +1,47 @@
+// Host-side helpers shared by the translation units of libascq: error string, argument checks, launch check.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "../../include/ascq.h"
+
+namespace ascq {
+
+// Records a message for ascq_last_error() and returns `code` so that `return fail(...)` reads naturally.
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+inline size_t dtype_size(int dt)
+{
+    switch (dt) {
+        case ASCQ_F16:
+        case ASCQ_BF16: return 2;
+        case ASCQ_F32:
+        case ASCQ_I32: return 4;
+        case ASCQ_I8: return 1;
+        case ASCQ_U64: return 8;
+        default: return 0;
+    }
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline int launch_status(const char* what)
+{
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        return fail(ASCQ_EHIP, "%s: %s", what, hipGetErrorString(e));
+    }
+    return ASCQ_OK;
+}
+
+#define ASCQ_REQUIRE(cond, code, ...)          \
+    do {                                       \
+        if (!(cond)) {                         \
+            return ::ascq::fail(code, __VA_ARGS__); \
+        }                                      \
+    } while (0)
+
+}  // namespace ascq

@@ -1,0 +1,224 @@
+// Device-side numeric primitives for gfx950.  Every operation rounds exactly once in the stated format; the
+// translation units are compiled with -ffp-contract=off so that a multiply and an add are never fused.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "../../include/ascq.h"
+
+namespace ascq {
+
+typedef _Float16 half_t;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
+typedef int32_t i32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+
+// fp32 -> bfloat16 bits, round to nearest even (NaN stays NaN).
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f)
+{
+    uint32_t u = __float_as_uint(f);
+    uint32_t r = (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+    return (f != f) ? ((u >> 16) | 0x40u) : r;
+}
+
+__device__ __forceinline__ float half_bits_to_f32(uint32_t h)
+{
+    union {
+        uint16_t u;
+        half_t h;
+    } c;
+    c.u = static_cast<uint16_t>(h);
+    return static_cast<float>(c.h);
+}
+
+__device__ __forceinline__ uint32_t f32_to_half_bits(float f)
+{
+    union {
+        uint16_t u;
+        half_t h;
+    } c;
+    c.h = static_cast<half_t>(f);  // v_cvt_f16_f32: round to nearest even, overflow to infinity
+    return c.u;
+}
+
+// fp32 -> fp16 bits with the fixpipe's saturation to +-65504 (NaN passes through).
+__device__ __forceinline__ uint32_t f32_to_half_bits_sat(float f)
+{
+    float c = fminf(fmaxf(f, -65504.0f), 65504.0f);
+    return f32_to_half_bits((f != f) ? f : c);
+}
+
+// Round a value (already exact in fp32) to an integer with the given mode and saturate to int8.
+template <bool kRint>
+__device__ __forceinline__ int round_sat8(float v, int round_mode)
+{
+    float r;
+    if (kRint) {
+        r = __builtin_rintf(v);
+    } else {
+        switch (round_mode) {
+            case ASCQ_CAST_FLOOR: r = __builtin_floorf(v); break;
+            case ASCQ_CAST_CEIL: r = __builtin_ceilf(v); break;
+            case ASCQ_CAST_ROUND: r = __builtin_roundf(v); break;
+            case ASCQ_CAST_TRUNC: r = __builtin_truncf(v); break;
+            default: r = __builtin_rintf(v); break;
+        }
+    }
+    r = fminf(fmaxf(r, -128.0f), 127.0f);
+    return (v != v) ? 0 : static_cast<int>(r);
+}
+
+// ---- arithmetic in a given compute format on values carried as fp32 (each op rounds once in the format) ----
+template <int kFmt>
+struct Fmt;
+
+template <>
+struct Fmt<ASCQ_F32> {
+    static __device__ __forceinline__ float cvt(float x) { return x; }
+    static __device__ __forceinline__ float mul(float a, float b) { return a * b; }
+    static __device__ __forceinline__ float add(float a, float b) { return a + b; }
+};
+template <>
+struct Fmt<ASCQ_F16> {
+    static __device__ __forceinline__ float cvt(float x) { return static_cast<float>(static_cast<half_t>(x)); }
+    static __device__ __forceinline__ float mul(float a, float b)
+    {
+        return static_cast<float>(static_cast<half_t>(a) * static_cast<half_t>(b));
+    }
+    static __device__ __forceinline__ float add(float a, float b)
+    {
+        return static_cast<float>(static_cast<half_t>(a) + static_cast<half_t>(b));
+    }
+};
+template <>
+struct Fmt<ASCQ_BF16> {
+    static __device__ __forceinline__ float cvt(float x) { return bf16_bits_to_f32(f32_to_bf16_bits(x)); }
+    // 8-bit significands: the fp32 product is exact, the fp32 sum is rounded to 24 >= 2*8+2 bits, so rounding
+    // the fp32 result to bfloat16 equals rounding the exact result once.
+    static __device__ __forceinline__ float mul(float a, float b) { return cvt(a * b); }
+    static __device__ __forceinline__ float add(float a, float b) { return cvt(a + b); }
+};
+
+// ---- typed element access (values widened to fp32, which is exact for every source type) ----
+template <int kDt>
+struct Elem;
+template <>
+struct Elem<ASCQ_F16> {
+    typedef uint16_t type;
+    static __device__ __forceinline__ float to_f32(uint16_t v) { return half_bits_to_f32(v); }
+};
+template <>
+struct Elem<ASCQ_BF16> {
+    typedef uint16_t type;
+    static __device__ __forceinline__ float to_f32(uint16_t v) { return bf16_bits_to_f32(v); }
+};
+template <>
+struct Elem<ASCQ_F32> {
+    typedef float type;
+    static __device__ __forceinline__ float to_f32(float v) { return v; }
+};
+template <>
+struct Elem<ASCQ_U64> {
+    typedef uint64_t type;
+    static __device__ __forceinline__ float to_f32(uint64_t v) { return __uint_as_float(static_cast<uint32_t>(v)); }
+};
+template <>
+struct Elem<ASCQ_I32> {
+    typedef int32_t type;
+    static __device__ __forceinline__ float to_f32(int32_t v) { return static_cast<float>(v); }  // RNE
+};
+
+// Load 8 consecutive elements (16-byte aligned group for 2-byte types) widened to fp32.
+template <int kDt>
+__device__ __forceinline__ void load8(const void* base, size_t idx, float (&out)[8])
+{
+    typedef typename Elem<kDt>::type T;
+    const T* p = static_cast<const T*>(base) + idx;
+    if constexpr (sizeof(T) == 2) {
+        u32x4 v = *reinterpret_cast<const u32x4*>(p);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            out[2 * i] = Elem<kDt>::to_f32(static_cast<uint16_t>(v[i] & 0xFFFFu));
+            out[2 * i + 1] = Elem<kDt>::to_f32(static_cast<uint16_t>(v[i] >> 16));
+        }
+    } else if constexpr (sizeof(T) == 4) {
+        u32x4 a = reinterpret_cast<const u32x4*>(p)[0];
+        u32x4 b = reinterpret_cast<const u32x4*>(p)[1];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t ua = a[i], ub = b[i];
+            T ta, tb;
+            __builtin_memcpy(&ta, &ua, 4);
+            __builtin_memcpy(&tb, &ub, 4);
+            out[i] = Elem<kDt>::to_f32(ta);
+            out[4 + i] = Elem<kDt>::to_f32(tb);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            u32x4 v = reinterpret_cast<const u32x4*>(p)[i];
+            out[2 * i] = __uint_as_float(v[0]);
+            out[2 * i + 1] = __uint_as_float(v[2]);
+        }
+    }
+}
+
+template <int kDt>
+__device__ __forceinline__ float load1(const void* base, size_t idx)
+{
+    typedef typename Elem<kDt>::type T;
+    return Elem<kDt>::to_f32(static_cast<const T*>(base)[idx]);
+}
+
+// Store 8 fp32 values as the destination type (rounded once).
+template <int kDt>
+__device__ __forceinline__ void store8(void* base, size_t idx, const float (&v)[8])
+{
+    if constexpr (kDt == ASCQ_F32) {
+        f32x4* p = reinterpret_cast<f32x4*>(static_cast<float*>(base) + idx);
+        p[0] = f32x4{v[0], v[1], v[2], v[3]};
+        p[1] = f32x4{v[4], v[5], v[6], v[7]};
+    } else {
+        u32x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint32_t lo, hi;
+            if constexpr (kDt == ASCQ_BF16) {
+                lo = f32_to_bf16_bits(v[2 * i]);
+                hi = f32_to_bf16_bits(v[2 * i + 1]);
+            } else {
+                lo = f32_to_half_bits(v[2 * i]);
+                hi = f32_to_half_bits(v[2 * i + 1]);
+            }
+            o[i] = lo | (hi << 16);
+        }
+        *reinterpret_cast<u32x4*>(static_cast<uint16_t*>(base) + idx) = o;
+    }
+}
+
+template <int kDt>
+__device__ __forceinline__ void store1(void* base, size_t idx, float v)
+{
+    if constexpr (kDt == ASCQ_F32) {
+        static_cast<float*>(base)[idx] = v;
+    } else if constexpr (kDt == ASCQ_BF16) {
+        static_cast<uint16_t*>(base)[idx] = static_cast<uint16_t>(f32_to_bf16_bits(v));
+    } else {
+        static_cast<uint16_t*>(base)[idx] = static_cast<uint16_t>(f32_to_half_bits(v));
+    }
+}
+
+__device__ __forceinline__ uint32_t pack4_i8(int a, int b, int c, int d)
+{
+    return (static_cast<uint32_t>(a) & 0xFFu) | ((static_cast<uint32_t>(b) & 0xFFu) << 8) |
+           ((static_cast<uint32_t>(c) & 0xFFu) << 16) | ((static_cast<uint32_t>(d) & 0xFFu) << 24);
+}
+
+}  // namespace ascq

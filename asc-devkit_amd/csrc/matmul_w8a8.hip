@@ -1,0 +1,770 @@
+// int8 x int8 -> int32 matmul with the fused dequant epilogue (Matmul + SetQuantScalar / SetQuantVector) and the
+// quantized grouped matmul, for gfx950.
+//
+// Design (one workgroup = 256 lanes = 4 wavefronts, one per SIMD):
+//   * v_mfma_i32_32x32x32_i8; a wavefront owns TM x TN accumulator blocks of 32x32 (4x4 -> 256 accumulator
+//     registers for the 256x256 tile), so every 16-byte operand fragment read from LDS feeds 4 MFMAs.
+//   * K is walked in steps of 128 bytes: one full 128-byte line per row of A per step.  Global loads of step t+1
+//     are issued into registers before the MFMAs of step t and written to the other LDS stage after them
+//     (double-buffered LDS, one barrier per step).
+//   * A [m, k] rows are K-contiguous, which is the MFMA operand order: 16-byte chunks go to LDS unchanged, with the
+//     chunk index XOR-swizzled by the row so that both the 16-byte writes and the 16-byte fragment reads of 16
+//     consecutive rows hit 16 different 16-byte bank groups.
+//   * B [k, n] is N-contiguous: each lane loads a 16(k) x 8(n) byte patch, transposes it in registers with
+//     v_perm_b32 (4x4 byte transposes) and writes one 16-byte K-chunk per column.  B rows in LDS are padded to
+//     144 bytes; with lanes ordered (k-block fastest) both these writes and the fragment reads are conflict-free.
+//     The MFMA sums over k, so any k order inside a chunk is fine as long as A and B agree (they do: byte b of
+//     chunk c is k = 16c + b for both).
+//   * Epilogue in registers: int32 -> fp32, x channel scale, x token scale, + bias, activation, one rounding to the
+//     output type.  No int32 round trip through memory (the reference hands the accumulator to the vector core
+//     through a global-memory workspace).
+//   * Tiles are numbered so that the 8 XCDs (workgroup id mod 8) each own a contiguous range of tiles, walking M
+//     fastest: the workgroups of one XCD share B column panels in that XCD's L2.
+//   * Small M is weight-bandwidth bound: 32-row tiles with split-K; partial sums are added with int32 atomics
+//     (exact and order-independent) into a caller workspace and a second kernel applies the epilogue.
+//   * Grouped matmul: same tile body; each workgroup finds its (group, row range) from the device-side group list,
+//     so no host synchronisation is needed and empty groups cost nothing.
+#include "ascq_common.h"
+#include "ascq_device.h"
+
+namespace ascq {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kBK = 128;          // bytes of K per pipeline step
+constexpr int kAStride = 128;     // LDS row stride of a K-contiguous operand (XOR swizzle)
+constexpr int kBStride = 144;     // LDS row stride of the transposed B operand (padding instead of swizzle)
+
+struct EpiParams {
+    void* c;
+    const void* bias;
+    const void* quant;  // uint64 words or fp32 scales, one per output channel (VECTOR mode)
+    const float* tok_scale;
+    uint32_t ldc;
+    int out_dtype, quant_mode, scale_format, bias_kind, has_tok, activation;
+    uint64_t quant_scalar;
+};
+
+struct GemmParams {
+    const int8_t* a;
+    const int8_t* b;
+    uint32_t m, n, k;
+    uint32_t tiles_m, tiles_n;
+    uint32_t k_splits, k_per_split;  // split-K: bytes of K per grid.z slice (multiple of kBK)
+    int32_t* partial;                // split-K int32 accumulator [m, n]
+    // grouped
+    const int64_t* group_list;
+    uint32_t groups;
+    int group_list_kind;
+    EpiParams epi;
+};
+
+struct ChannelQ {
+    float s;
+    int off9;
+    int sgn;
+};
+
+__device__ __forceinline__ ChannelQ load_channel_q(const EpiParams& e, size_t col)
+{
+    ChannelQ q{1.0f, 0, 1};
+    if (e.quant_mode == ASCQ_MM_QUANT_NONE) {
+        return q;
+    }
+    uint64_t w;
+    if (e.quant_mode == ASCQ_MM_QUANT_VECTOR) {
+        if (e.scale_format == ASCQ_MM_SCALE_U64) {
+            w = static_cast<const uint64_t*>(e.quant)[col];
+        } else {
+            w = __float_as_uint(static_cast<const float*>(e.quant)[col]);
+        }
+    } else {
+        w = e.quant_scalar;
+    }
+    uint32_t lo = static_cast<uint32_t>(w);
+    if (e.scale_format == ASCQ_MM_SCALE_U64) {
+        lo &= 0xFFFFE000u;  // the fixpipe reads sign, 8 exponent and 10 mantissa bits
+        q.off9 = static_cast<int>((w >> 37) & 0x1FF);
+        q.sgn = static_cast<int>((w >> 46) & 1);
+    }
+    q.s = __uint_as_float(lo);
+    return q;
+}
+
+__device__ __forceinline__ float faster_gelu(float x)
+{
+    const float ax = fabsf(x);
+    const float x2 = expf(0.851f * (x - ax));
+    const float x3 = 1.0f + expf(-1.702f * ax);
+    return x * x2 / x3;
+}
+
+// Everything after the int32 accumulator, for one output element.  `bias_post` is already widened to fp32.
+// kOut is the output dtype, or -1 for "no quantisation" (raw int32).
+template <int kOut>
+__device__ __forceinline__ void epilogue_store(const EpiParams& e, size_t row, size_t col, int32_t acc,
+                                               const ChannelQ& q, float tok, float bias_post)
+{
+    const size_t idx = row * e.ldc + col;
+    if constexpr (kOut < 0) {
+        static_cast<int32_t*>(e.c)[idx] = acc;
+    } else {
+        float v = static_cast<float>(acc) * q.s;
+        if (e.has_tok) {
+            v = v * tok;
+        }
+        if (e.bias_kind >= ASCQ_MM_BIAS_F32_POST) {
+            v = v + bias_post;
+        }
+        if (e.activation == ASCQ_MM_ACT_FASTER_GELU) {
+            v = faster_gelu(v);
+        }
+        if constexpr (kOut == ASCQ_BF16) {
+            static_cast<uint16_t*>(e.c)[idx] = static_cast<uint16_t>(f32_to_bf16_bits(v));
+        } else if constexpr (kOut == ASCQ_F16) {
+            static_cast<uint16_t*>(e.c)[idx] = static_cast<uint16_t>(f32_to_half_bits_sat(v));
+        } else if constexpr (kOut == ASCQ_F32) {
+            static_cast<float*>(e.c)[idx] = v;
+        } else {  // int8 / uint8 requantisation
+            float r = fminf(fmaxf(__builtin_rintf(v), -256.0f), 255.0f);
+            int t = ((v != v) ? 0 : static_cast<int>(r)) + q.off9;
+            t = q.sgn ? min(max(t, -128), 127) : min(max(t, 0), 255);
+            static_cast<uint8_t*>(e.c)[idx] = static_cast<uint8_t>(t);
+        }
+    }
+}
+
+// Calls f(tag) with the compile-time output kind selected by the (uniform) runtime descriptor.
+template <int k>
+struct OutTag {
+    static constexpr int value = k;
+};
+template <class F>
+__device__ __forceinline__ void dispatch_out(const EpiParams& e, F&& f)
+{
+    if (e.quant_mode == ASCQ_MM_QUANT_NONE) {
+        f(OutTag<-1>{});
+    } else if (e.out_dtype == ASCQ_BF16) {
+        f(OutTag<ASCQ_BF16>{});
+    } else if (e.out_dtype == ASCQ_F16) {
+        f(OutTag<ASCQ_F16>{});
+    } else if (e.out_dtype == ASCQ_F32) {
+        f(OutTag<ASCQ_F32>{});
+    } else {
+        f(OutTag<ASCQ_I8>{});
+    }
+}
+
+__device__ __forceinline__ float load_bias_post(const EpiParams& e, size_t col)
+{
+    if (e.bias_kind == ASCQ_MM_BIAS_F32_POST) {
+        return static_cast<const float*>(e.bias)[col];
+    }
+    if (e.bias_kind == ASCQ_MM_BIAS_BF16_POST) {
+        return bf16_bits_to_f32(static_cast<const uint16_t*>(e.bias)[col]);
+    }
+    return 0.0f;
+}
+
+// 4x4 byte transpose: r[i] holds bytes (n0..n3) of row i; c[j] receives (row0..row3) of column j.
+__device__ __forceinline__ void transpose4x4(uint32_t r0, uint32_t r1, uint32_t r2, uint32_t r3, uint32_t& c0,
+                                             uint32_t& c1, uint32_t& c2, uint32_t& c3)
+{
+    // v_perm_b32(s0, s1, sel): selector values 0-3 pick bytes of s1, 4-7 bytes of s0
+    const uint32_t lo01 = __builtin_amdgcn_perm(r1, r0, 0x05010400u);  // r0.b0 r1.b0 r0.b1 r1.b1
+    const uint32_t hi01 = __builtin_amdgcn_perm(r1, r0, 0x07030602u);  // r0.b2 r1.b2 r0.b3 r1.b3
+    const uint32_t lo23 = __builtin_amdgcn_perm(r3, r2, 0x05010400u);
+    const uint32_t hi23 = __builtin_amdgcn_perm(r3, r2, 0x07030602u);
+    c0 = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);
+    c1 = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
+    c2 = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);
+    c3 = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
+}
+
+__device__ __forceinline__ uint32_t swz_off(uint32_t row, uint32_t chunk)
+{
+    return row * kAStride + ((chunk ^ ((row >> 1) & 7u)) << 4);
+}
+
+// Maps a linear workgroup id to a tile id such that each XCD (id mod 8) gets a contiguous range of tiles.
+__device__ __forceinline__ uint32_t xcd_remap(uint32_t pid, uint32_t total)
+{
+    const uint32_t per = (total + 7u) / 8u;
+    uint32_t tall = total % 8u;
+    if (tall == 0) {
+        tall = 8;
+    }
+    const uint32_t xcd = pid & 7u, local = pid >> 3;
+    if (xcd < tall) {
+        return xcd * per + local;
+    }
+    if (local + 1u >= per) {
+        return 0xFFFFFFFFu;  // the short XCDs own one tile less: this workgroup has nothing to do
+    }
+    return tall * per + (xcd - tall) * (per - 1u) + local;
+}
+
+template <int TM, int TN, int WGM, int WGN, bool kTransB>
+struct Tile {
+    static constexpr int BM = WGM * TM * 32;
+    static constexpr int BN = WGN * TN * 32;
+    static constexpr int kWGM = WGM, kWGN = WGN, kWTM = TM, kWTN = TN;
+    static constexpr int kBRow = kTransB ? kAStride : kBStride;
+    static constexpr int kABytes = BM * kAStride;
+    static constexpr int kBBytes = BN * kBRow;
+    static constexpr int kStage = kABytes + kBBytes;
+    static constexpr int kLds = 2 * kStage;
+    static constexpr int kAChunks = BM * (kBK / 16) / kThreads;  // 16-byte chunks of A per lane per step
+    static constexpr int kBChunksT = BN * (kBK / 16) / kThreads; // same for a K-contiguous B
+    static constexpr int kCols = BN / 32;                        // columns per lane of an N-contiguous B (8 or 4)
+    static_assert(WGM * WGN == 4, "four wavefronts per workgroup");
+    static_assert(kCols == 8 || kCols == 4, "BN must be 256 or 128");
+};
+
+// One output tile: rows [row0, row_end) x columns [n0, n0 + BN), K range [k_begin, k_end).
+template <class T, bool kTransB, bool kSplitK>
+__device__ __forceinline__ void gemm_tile(const GemmParams& p, const int8_t* __restrict__ A,
+                                          const int8_t* __restrict__ B, const EpiParams& e, uint32_t row0,
+                                          uint32_t row_end, uint32_t n0, uint32_t k_begin, uint32_t k_end,
+                                          size_t chan_off, char* smem)
+{
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u;
+    const uint32_t wave = tid >> 6;
+    const uint32_t K = p.k, N = p.n;
+
+    // ---------------- staging registers
+    u32x4 areg[T::kAChunks];
+    u32x4 bregT[kTransB ? T::kBChunksT : 1];
+    uint32_t breg[kTransB ? 1 : 16][kTransB ? 1 : (T::kCols / 4)];
+
+    // lane -> patch of the N-contiguous B tile: k-block fastest so that LDS writes spread over all banks
+    const uint32_t kb = tid & 7u;
+    const uint32_t nb = tid >> 3;
+
+    auto load_global = [&](uint32_t k0) {
+#pragma unroll
+        for (int i = 0; i < T::kAChunks; ++i) {
+            const uint32_t c = tid + kThreads * i;
+            uint32_t row = row0 + (c >> 3);
+            row = row < row_end ? row : row_end - 1;  // rows past the end are never stored: any valid row will do
+            const uint32_t kk = k0 + ((c & 7u) << 4);
+            if (kk < k_end) {
+                areg[i] = *reinterpret_cast<const u32x4*>(A + static_cast<size_t>(row) * K + kk);
+            } else {
+                areg[i] = u32x4{0u, 0u, 0u, 0u};
+            }
+        }
+        if constexpr (kTransB) {
+#pragma unroll
+            for (int i = 0; i < T::kBChunksT; ++i) {
+                const uint32_t c = tid + kThreads * i;
+                uint32_t col = n0 + (c >> 3);
+                col = col < N ? col : N - 1;
+                const uint32_t kk = k0 + ((c & 7u) << 4);
+                if (kk < k_end) {
+                    bregT[i] = *reinterpret_cast<const u32x4*>(B + static_cast<size_t>(col) * K + kk);
+                } else {
+                    bregT[i] = u32x4{0u, 0u, 0u, 0u};
+                }
+            }
+        } else {
+            uint32_t col = n0 + nb * T::kCols;
+            col = col + T::kCols <= N ? col : N - T::kCols;  // columns past the end are never stored
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const uint32_t kk = k0 + kb * 16u + i;
+                const int8_t* src = B + static_cast<size_t>(kk) * N + col;
+                if (kk < k_end) {
+                    if constexpr (T::kCols == 8) {
+                        u32x2 v = *reinterpret_cast<const u32x2*>(src);
+                        breg[i][0] = v[0];
+                        breg[i][1] = v[1];
+                    } else {
+                        breg[i][0] = *reinterpret_cast<const uint32_t*>(src);
+                    }
+                } else {
+#pragma unroll
+                    for (int d = 0; d < T::kCols / 4; ++d) breg[i][d] = 0u;
+                }
+            }
+        }
+    };
+
+    auto store_lds = [&](char* stage) {
+        char* As = stage;
+        char* Bs = stage + T::kABytes;
+#pragma unroll
+        for (int i = 0; i < T::kAChunks; ++i) {
+            const uint32_t c = tid + kThreads * i;
+            *reinterpret_cast<u32x4*>(As + swz_off(c >> 3, c & 7u)) = areg[i];
+        }
+        if constexpr (kTransB) {
+#pragma unroll
+            for (int i = 0; i < T::kBChunksT; ++i) {
+                const uint32_t c = tid + kThreads * i;
+                *reinterpret_cast<u32x4*>(Bs + swz_off(c >> 3, c & 7u)) = bregT[i];
+            }
+        } else {
+#pragma unroll
+            for (int d = 0; d < T::kCols / 4; ++d) {
+                uint32_t t[4][4];  // t[q][c]: rows 4q..4q+3 of column 4d+c
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    transpose4x4(breg[4 * q][d], breg[4 * q + 1][d], breg[4 * q + 2][d], breg[4 * q + 3][d],
+                                 t[q][0], t[q][1], t[q][2], t[q][3]);
+                }
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const uint32_t col = nb * T::kCols + 4 * d + c;
+                    *reinterpret_cast<u32x4*>(Bs + col * kBStride + (kb << 4)) =
+                        u32x4{t[0][c], t[1][c], t[2][c], t[3][c]};
+                }
+            }
+        }
+    };
+
+    // ---------------- accumulators
+    constexpr int kWGN = T::kWGN;  // wavefront grid inside the tile
+    constexpr int kWTM = T::kWTM;  // 32x32 blocks per wavefront along M / N
+    constexpr int kWTN = T::kWTN;
+    const uint32_t wm = wave / kWGN, wn = wave % kWGN;
+
+    i32x16 acc[kWTM][kWTN];
+#pragma unroll
+    for (int i = 0; i < kWTM; ++i) {
+#pragma unroll
+        for (int j = 0; j < kWTN; ++j) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+        }
+    }
+
+    const uint32_t lrow = lane & 31u;
+    const uint32_t lgrp = lane >> 5;
+
+    auto compute = [&](const char* stage) {
+        const char* As = stage;
+        const char* Bs = stage + T::kABytes;
+#pragma unroll
+        for (int ks = 0; ks < kBK / 32; ++ks) {
+            const uint32_t chunk = 2u * ks + lgrp;
+            i32x4 af[kWTM], bf[kWTN];
+#pragma unroll
+            for (int i = 0; i < kWTM; ++i) {
+                const uint32_t row = (wm * kWTM + i) * 32u + lrow;
+                af[i] = *reinterpret_cast<const i32x4*>(As + swz_off(row, chunk));
+            }
+#pragma unroll
+            for (int j = 0; j < kWTN; ++j) {
+                const uint32_t col = (wn * kWTN + j) * 32u + lrow;
+                if constexpr (kTransB) {
+                    bf[j] = *reinterpret_cast<const i32x4*>(Bs + swz_off(col, chunk));
+                } else {
+                    bf[j] = *reinterpret_cast<const i32x4*>(Bs + col * kBStride + (chunk << 4));
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < kWTM; ++i) {
+#pragma unroll
+                for (int j = 0; j < kWTN; ++j) {
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
+                }
+            }
+        }
+    };
+
+    // ---------------- main loop
+    const uint32_t steps = (k_end - k_begin + kBK - 1) / kBK;
+    char* stage0 = smem;
+    char* stage1 = smem + T::kStage;
+    load_global(k_begin);
+    store_lds(stage0);
+    __syncthreads();
+    for (uint32_t t = 0; t < steps; ++t) {
+        char* cur = (t & 1u) ? stage1 : stage0;
+        char* nxt = (t & 1u) ? stage0 : stage1;
+        const bool more = t + 1 < steps;
+        if (more) {
+            load_global(k_begin + (t + 1) * kBK);
+        }
+        compute(cur);
+        if (more) {
+            store_lds(nxt);
+        }
+        __syncthreads();
+    }
+
+    // ---------------- epilogue (MFMA 32x32 layout: register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, col l%32)
+    ChannelQ qs[kWTN];
+    float bias_post[kWTN];
+    int32_t bias_pre[kWTN];
+    uint32_t cols[kWTN];
+#pragma unroll
+    for (int j = 0; j < kWTN; ++j) {
+        cols[j] = n0 + (wn * kWTN + j) * 32u + lrow;
+        qs[j] = ChannelQ{1.0f, 0, 1};
+        bias_post[j] = 0.0f;
+        bias_pre[j] = 0;
+        if constexpr (!kSplitK) {
+            if (cols[j] < N) {
+                qs[j] = load_channel_q(e, chan_off + cols[j]);
+                bias_post[j] = load_bias_post(e, chan_off + cols[j]);
+                if (e.bias_kind == ASCQ_MM_BIAS_I32_PRE) {
+                    bias_pre[j] = static_cast<const int32_t*>(e.bias)[chan_off + cols[j]];
+                }
+            }
+        }
+    }
+    auto run = [&](auto tag) {
+        constexpr int kOut = decltype(tag)::value;
+#pragma unroll
+        for (int i = 0; i < kWTM; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint32_t row = row0 + (wm * kWTM + i) * 32u + 8u * (r >> 2) + 4u * lgrp + (r & 3);
+                if (row < row_end) {
+                    float tok = 1.0f;
+                    if constexpr (!kSplitK) {
+                        if (e.has_tok) {
+                            tok = e.tok_scale[row];
+                        }
+                    }
+#pragma unroll
+                    for (int j = 0; j < kWTN; ++j) {
+                        if (cols[j] < N) {
+                            if constexpr (kSplitK) {
+                                atomicAdd(p.partial + static_cast<size_t>(row) * N + cols[j], acc[i][j][r]);
+                            } else {
+                                epilogue_store<kOut>(e, row, cols[j], acc[i][j][r] + bias_pre[j], qs[j], tok,
+                                                     bias_post[j]);
+                            }
+                        }
+                    }
+                }
+            }
+        }
+    };
+    if constexpr (kSplitK) {
+        run(OutTag<-1>{});
+    } else {
+        dispatch_out(e, run);
+    }
+}
+
+template <class T, bool kTransB, bool kSplitK>
+__global__ __launch_bounds__(kThreads) void gemm_kernel(GemmParams p)
+{
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const uint32_t total = p.tiles_m * p.tiles_n;
+    const uint32_t t = xcd_remap(blockIdx.x, total);
+    if (t >= total) {
+        return;
+    }
+    const uint32_t tm = t % p.tiles_m, tn = t / p.tiles_m;
+    uint32_t k_begin = 0, k_end = p.k;
+    if constexpr (kSplitK) {
+        k_begin = blockIdx.y * p.k_per_split;
+        k_end = min(p.k, k_begin + p.k_per_split);
+        if (k_begin >= k_end) {
+            return;
+        }
+    }
+    gemm_tile<T, kTransB, kSplitK>(p, p.a, p.b, p.epi, tm * T::BM, p.m, tn * T::BN, k_begin, k_end, 0, smem);
+}
+
+// Grouped: tile slot `ms` along M is resolved against the group list by every workgroup (groups is small).
+template <class T>
+__global__ __launch_bounds__(kThreads) void group_gemm_kernel(GemmParams p)
+{
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const uint32_t total = p.tiles_m * p.tiles_n;
+    const uint32_t t = xcd_remap(blockIdx.x, total);
+    if (t >= total) {
+        return;
+    }
+    const uint32_t ms = t % p.tiles_m, tn = t / p.tiles_m;
+    // walk the groups: group g owns tile slots [slot, slot + ceil(cnt / BM))
+    uint32_t slot = 0;
+    int64_t off = 0;
+    for (uint32_t g = 0; g < p.groups; ++g) {
+        const int64_t v = p.group_list[g];
+        const int64_t cnt = p.group_list_kind == ASCQ_GROUP_LIST_PREFIX_SUM ? v - off : v;
+        if (cnt <= 0) {
+            continue;
+        }
+        int64_t end = off + cnt;
+        if (end > static_cast<int64_t>(p.m)) {
+            end = p.m;
+        }
+        const uint32_t rows = end > off ? static_cast<uint32_t>(end - off) : 0u;
+        const uint32_t tiles = (rows + T::BM - 1) / T::BM;
+        if (ms < slot + tiles) {
+            const uint32_t row0 = static_cast<uint32_t>(off) + (ms - slot) * T::BM;
+            gemm_tile<T, false, false>(p, p.a, p.b + static_cast<size_t>(g) * p.k * p.n, p.epi, row0,
+                                       static_cast<uint32_t>(end), tn * T::BN, 0, p.k, static_cast<size_t>(g) * p.n,
+                                       smem);
+            return;
+        }
+        slot += tiles;
+        off += cnt;
+    }
+}
+
+// Second pass of the split-K path: workspace int32 [m, n] -> output, and leaves the workspace zeroed.
+__global__ __launch_bounds__(kThreads) void splitk_epilogue_kernel(GemmParams p)
+{
+    const size_t total = static_cast<size_t>(p.m) * p.n;
+    for (size_t idx = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x; idx < total;
+         idx += static_cast<size_t>(gridDim.x) * kThreads) {
+        const size_t row = idx / p.n, col = idx % p.n;
+        int32_t acc = p.partial[idx];
+        p.partial[idx] = 0;
+        if (p.epi.bias_kind == ASCQ_MM_BIAS_I32_PRE) {
+            acc += static_cast<const int32_t*>(p.epi.bias)[col];
+        }
+        const ChannelQ q = load_channel_q(p.epi, col);
+        const float tok = p.epi.has_tok ? p.epi.tok_scale[row] : 1.0f;
+        const float bp = load_bias_post(p.epi, col);
+        dispatch_out(p.epi, [&](auto tag) {
+            epilogue_store<decltype(tag)::value>(p.epi, row, col, acc, q, tok, bp);
+        });
+    }
+}
+
+// Shapes the MFMA kernels do not take (odd sizes, unaligned pointers, transposed A): one lane per output.
+__global__ __launch_bounds__(kThreads) void gemm_generic_kernel(GemmParams p, int trans_a, int trans_b)
+{
+    const size_t total = static_cast<size_t>(p.m) * p.n;
+    for (size_t idx = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x; idx < total;
+         idx += static_cast<size_t>(gridDim.x) * kThreads) {
+        const size_t row = idx / p.n, col = idx % p.n;
+        int32_t acc = 0;
+        for (uint32_t kk = 0; kk < p.k; ++kk) {
+            const int32_t av = trans_a ? p.a[static_cast<size_t>(kk) * p.m + row] : p.a[row * p.k + kk];
+            const int32_t bv = trans_b ? p.b[col * p.k + kk] : p.b[static_cast<size_t>(kk) * p.n + col];
+            acc += av * bv;
+        }
+        if (p.epi.bias_kind == ASCQ_MM_BIAS_I32_PRE) {
+            acc += static_cast<const int32_t*>(p.epi.bias)[col];
+        }
+        const ChannelQ q = load_channel_q(p.epi, col);
+        const float tok = p.epi.has_tok ? p.epi.tok_scale[row] : 1.0f;
+        const float bp = load_bias_post(p.epi, col);
+        dispatch_out(p.epi, [&](auto tag) {
+            epilogue_store<decltype(tag)::value>(p.epi, row, col, acc, q, tok, bp);
+        });
+    }
+}
+
+typedef Tile<4, 4, 2, 2, false> TileL;   // 256 x 256
+typedef Tile<4, 4, 2, 2, true> TileLT;
+typedef Tile<2, 4, 2, 2, false> TileM;   // 128 x 256
+typedef Tile<2, 4, 2, 2, true> TileMT;
+typedef Tile<1, 2, 1, 4, false> TileS;   // 32 x 256, split-K
+typedef Tile<1, 2, 1, 4, true> TileST;
+
+template <class K>
+int set_lds(K kernel, int bytes)
+{
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       bytes);
+    if (e != hipSuccess) {
+        return fail(ASCQ_EHIP, "hipFuncSetAttribute(%d bytes of LDS): %s", bytes, hipGetErrorString(e));
+    }
+    return ASCQ_OK;
+}
+
+template <class T, bool kTransB, bool kSplitK>
+int launch_gemm(GemmParams& p, hipStream_t st)
+{
+    p.tiles_m = (p.m + T::BM - 1) / T::BM;
+    p.tiles_n = (p.n + T::BN - 1) / T::BN;
+    auto kernel = gemm_kernel<T, kTransB, kSplitK>;
+    int rc = set_lds(kernel, T::kLds);
+    if (rc != ASCQ_OK) {
+        return rc;
+    }
+    const uint32_t total = p.tiles_m * p.tiles_n;
+    dim3 grid((total + 7u) / 8u * 8u, kSplitK ? p.k_splits : 1u);
+    kernel<<<grid, kThreads, T::kLds, st>>>(p);
+    return launch_status("ascq_matmul_w8a8");
+}
+
+int validate_mm(const ascq_matmul_desc* d, const char* who, const void* c, const void* a, const void* b,
+                const void* bias, const void* qv, const void* tok)
+{
+    ASCQ_REQUIRE(c && a && b, ASCQ_ENULL, "%s: c / a / b is NULL", who);
+    ASCQ_REQUIRE(d->m > 0 && d->n > 0 && d->k > 0, ASCQ_EINVAL, "%s: m, n, k must be greater than 0", who);
+    ASCQ_REQUIRE(d->quant_mode >= ASCQ_MM_QUANT_NONE && d->quant_mode <= ASCQ_MM_QUANT_VECTOR, ASCQ_EINVAL,
+                 "%s: unknown quant mode %d", who, d->quant_mode);
+    ASCQ_REQUIRE(d->scale_format == ASCQ_MM_SCALE_U64 || d->scale_format == ASCQ_MM_SCALE_F32, ASCQ_EINVAL,
+                 "%s: unknown scale format %d", who, d->scale_format);
+    ASCQ_REQUIRE(d->bias_kind >= ASCQ_MM_BIAS_NONE && d->bias_kind <= ASCQ_MM_BIAS_BF16_POST, ASCQ_EINVAL,
+                 "%s: unknown bias kind %d", who, d->bias_kind);
+    ASCQ_REQUIRE(d->activation == ASCQ_MM_ACT_NONE || d->activation == ASCQ_MM_ACT_FASTER_GELU, ASCQ_EINVAL,
+                 "%s: unknown activation %d", who, d->activation);
+    if (d->quant_mode == ASCQ_MM_QUANT_NONE) {
+        ASCQ_REQUIRE(d->out_dtype == ASCQ_I32, ASCQ_EUNSUPPORTED, "%s: without a quant mode the output is int32", who);
+        ASCQ_REQUIRE(d->bias_kind <= ASCQ_MM_BIAS_I32_PRE && !d->has_tok_scale && d->activation == ASCQ_MM_ACT_NONE,
+                     ASCQ_EUNSUPPORTED, "%s: int32 output takes no fp32 epilogue", who);
+    } else {
+        const int o = d->out_dtype;
+        ASCQ_REQUIRE(o == ASCQ_F16 || o == ASCQ_BF16 || o == ASCQ_F32 || o == ASCQ_I8, ASCQ_EUNSUPPORTED,
+                     "%s: output dtype %d is not half / bfloat16 / float / int8", who, o);
+        ASCQ_REQUIRE(o != ASCQ_I8 || d->scale_format == ASCQ_MM_SCALE_U64, ASCQ_EUNSUPPORTED,
+                     "%s: int8 output (requantisation) needs the uint64 quant parameter format", who);
+        if (d->quant_mode == ASCQ_MM_QUANT_VECTOR) {
+            ASCQ_REQUIRE(qv != nullptr, ASCQ_ENULL, "%s: quant vector is NULL", who);
+        }
+    }
+    ASCQ_REQUIRE(d->bias_kind == ASCQ_MM_BIAS_NONE || bias != nullptr, ASCQ_ENULL, "%s: bias is NULL", who);
+    ASCQ_REQUIRE(!d->has_tok_scale || tok != nullptr, ASCQ_ENULL, "%s: token scale is NULL", who);
+    return ASCQ_OK;
+}
+
+EpiParams make_epi(const ascq_matmul_desc* d, void* c, const void* bias, const void* qv, const void* tok)
+{
+    return EpiParams{c, bias, qv, static_cast<const float*>(tok), d->n, d->out_dtype, d->quant_mode, d->scale_format,
+                     d->bias_kind, d->has_tok_scale, d->activation, d->quant_scalar};
+}
+
+bool fast_path_ok(const ascq_matmul_desc* d, const void* a, const void* b)
+{
+    if (d->trans_a || d->k % 16 != 0 || !aligned16(a)) {
+        return false;
+    }
+    if (d->trans_b) {
+        return aligned16(b);
+    }
+    return d->n % 8 == 0 && d->n >= 8 && (reinterpret_cast<uintptr_t>(b) & 7u) == 0;
+}
+
+// split-K factor for the small-M kernel: enough workgroups to cover the chip ~3 times
+uint32_t pick_k_splits(uint32_t n, uint32_t k)
+{
+    const uint32_t tiles = (n + 255u) / 256u;
+    const uint32_t steps = (k + kBK - 1) / kBK;
+    uint32_t s = (768u + tiles - 1) / tiles;
+    if (s > steps) s = steps;
+    if (s > 32u) s = 32u;
+    return s ? s : 1u;
+}
+
+}  // namespace
+}  // namespace ascq
+
+using namespace ascq;
+
+extern "C" int ascq_matmul_w8a8_workspace_size(const ascq_matmul_desc* d, size_t* bytes)
+{
+    ASCQ_REQUIRE(d != nullptr && bytes != nullptr, ASCQ_ENULL, "ascq_matmul_w8a8_workspace_size: NULL argument");
+    *bytes = 0;
+    if (d->m <= 32 && !d->trans_a && pick_k_splits(d->n, d->k) > 1) {
+        *bytes = static_cast<size_t>(d->m) * d->n * sizeof(int32_t);
+    }
+    return ASCQ_OK;
+}
+
+// ref: include/adv_api/matmul/matmul.h:175-185 (SetQuantScalar / SetQuantVector), IterateAll: matmul_impl.h:65-92
+extern "C" int ascq_matmul_w8a8(const ascq_matmul_desc* d, void* c, const void* a, const void* b, const void* bias,
+                                const void* quant_vector, const void* tok_scale, void* workspace,
+                                size_t workspace_bytes, void* stream)
+{
+    ASCQ_REQUIRE(d != nullptr, ASCQ_ENULL, "ascq_matmul_w8a8: desc is NULL");
+    int rc = validate_mm(d, "ascq_matmul_w8a8", c, a, b, bias, quant_vector, tok_scale);
+    if (rc != ASCQ_OK) {
+        return rc;
+    }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    GemmParams p{};
+    p.a = static_cast<const int8_t*>(a);
+    p.b = static_cast<const int8_t*>(b);
+    p.m = d->m;
+    p.n = d->n;
+    p.k = d->k;
+    p.epi = make_epi(d, c, bias, quant_vector, tok_scale);
+    if (!fast_path_ok(d, a, b)) {
+        size_t total = static_cast<size_t>(d->m) * d->n;
+        size_t blocks = (total + kThreads - 1) / kThreads;
+        if (blocks > 65536) blocks = 65536;
+        gemm_generic_kernel<<<static_cast<uint32_t>(blocks), kThreads, 0, st>>>(p, d->trans_a, d->trans_b);
+        return launch_status("ascq_matmul_w8a8 (generic)");
+    }
+    if (d->m <= 32) {
+        const uint32_t splits = pick_k_splits(d->n, d->k);
+        size_t need = static_cast<size_t>(d->m) * d->n * sizeof(int32_t);
+        if (splits > 1 && workspace != nullptr && workspace_bytes >= need &&
+            (reinterpret_cast<uintptr_t>(workspace) & 3u) == 0) {
+            p.k_splits = splits;
+            const uint32_t steps = (d->k + kBK - 1) / kBK;
+            p.k_per_split = (steps + splits - 1) / splits * kBK;
+            p.partial = static_cast<int32_t*>(workspace);
+            rc = ascq_zero_fill(workspace, need, stream);
+            if (rc != ASCQ_OK) {
+                return rc;
+            }
+            rc = d->trans_b ? launch_gemm<TileST, true, true>(p, st) : launch_gemm<TileS, false, true>(p, st);
+            if (rc != ASCQ_OK) {
+                return rc;
+            }
+            size_t total = static_cast<size_t>(d->m) * d->n;
+            size_t blocks = (total + kThreads - 1) / kThreads;
+            if (blocks > 4096) blocks = 4096;
+            splitk_epilogue_kernel<<<static_cast<uint32_t>(blocks), kThreads, 0, st>>>(p);
+            return launch_status("ascq_matmul_w8a8 (split-K epilogue)");
+        }
+        return d->trans_b ? launch_gemm<TileST, true, false>(p, st) : launch_gemm<TileS, false, false>(p, st);
+    }
+    if (d->m <= 1024) {
+        return d->trans_b ? launch_gemm<TileMT, true, false>(p, st) : launch_gemm<TileM, false, false>(p, st);
+    }
+    return d->trans_b ? launch_gemm<TileLT, true, false>(p, st) : launch_gemm<TileL, false, false>(p, st);
+}
+
+// ref: examples/.../quant_group_matmul_high_performance/quant_group_matmul_custom.asc:255-454
+extern "C" int ascq_group_matmul_w8a8(const ascq_group_matmul_desc* g, void* y, const void* x, const void* w,
+                                      const void* bias, const void* scale, const void* tok_scale,
+                                      const int64_t* group_list, void* stream)
+{
+    ASCQ_REQUIRE(g != nullptr, ASCQ_ENULL, "ascq_group_matmul_w8a8: desc is NULL");
+    const ascq_matmul_desc* d = &g->mm;
+    int rc = validate_mm(d, "ascq_group_matmul_w8a8", y, x, w, bias, scale, tok_scale);
+    if (rc != ASCQ_OK) {
+        return rc;
+    }
+    ASCQ_REQUIRE(group_list != nullptr, ASCQ_ENULL, "ascq_group_matmul_w8a8: group list is NULL");
+    ASCQ_REQUIRE(g->groups > 0, ASCQ_EINVAL, "ascq_group_matmul_w8a8: groups must be greater than 0");
+    ASCQ_REQUIRE(g->group_list_kind == ASCQ_GROUP_LIST_COUNTS || g->group_list_kind == ASCQ_GROUP_LIST_PREFIX_SUM,
+                 ASCQ_EINVAL, "ascq_group_matmul_w8a8: unknown group list kind %d", g->group_list_kind);
+    ASCQ_REQUIRE(d->quant_mode == ASCQ_MM_QUANT_VECTOR && d->scale_format == ASCQ_MM_SCALE_F32, ASCQ_EUNSUPPORTED,
+                 "ascq_group_matmul_w8a8: the per-group channel scale is an fp32 vector");
+    ASCQ_REQUIRE(!d->trans_a && !d->trans_b, ASCQ_EUNSUPPORTED, "ascq_group_matmul_w8a8: transposed operands");
+    ASCQ_REQUIRE(d->bias_kind != ASCQ_MM_BIAS_I32_PRE, ASCQ_EUNSUPPORTED,
+                 "ascq_group_matmul_w8a8: bias is applied after dequantisation");
+    ASCQ_REQUIRE(d->k % 16 == 0 && d->n % 8 == 0 && aligned16(x) && aligned16(w), ASCQ_EALIGN,
+                 "ascq_group_matmul_w8a8: k must be a multiple of 16, n of 8, x and w 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    GemmParams p{};
+    p.a = static_cast<const int8_t*>(x);
+    p.b = static_cast<const int8_t*>(w);
+    p.m = d->m;
+    p.n = d->n;
+    p.k = d->k;
+    p.group_list = group_list;
+    p.groups = g->groups;
+    p.group_list_kind = g->group_list_kind;
+    p.epi = make_epi(d, y, bias, scale, tok_scale);
+    typedef TileL T;
+    // every group adds at most one partial tile along M
+    p.tiles_m = (d->m + T::BM - 1) / T::BM + g->groups;
+    p.tiles_n = (d->n + T::BN - 1) / T::BN;
+    auto kernel = group_gemm_kernel<T>;
+    rc = set_lds(kernel, T::kLds);
+    if (rc != ASCQ_OK) {
+        return rc;
+    }
+    const uint32_t total = p.tiles_m * p.tiles_n;
+    kernel<<<(total + 7u) / 8u * 8u, kThreads, T::kLds, st>>>(p);
+    return launch_status("ascq_group_matmul_w8a8");
+}

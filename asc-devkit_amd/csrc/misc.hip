@@ -1,0 +1,144 @@
+// Error string, version, host-side "tiling" size queries, quant-parameter packing and the zero-fill kernel.
+#include <algorithm>
+#include <cstring>
+
+#include "ascq_common.h"
+
+namespace ascq {
+
+static thread_local char g_error[512] = "";
+
+int fail(int code, const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+namespace {
+__global__ __launch_bounds__(256) void zero_fill_kernel(uint32_t* p, size_t words)
+{
+    for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < words;
+         i += static_cast<size_t>(gridDim.x) * 256) {
+        p[i] = 0u;
+    }
+}
+uint64_t shape_size(const uint32_t* shape, uint32_t ndim)
+{
+    uint64_t s = 1;
+    for (uint32_t i = 0; i < ndim; ++i) s *= shape[i];
+    return ndim ? s : 0;
+}
+}  // namespace
+}  // namespace ascq
+
+using namespace ascq;
+
+extern "C" const char* ascq_last_error(void) { return g_error; }
+extern "C" const char* ascq_version(void) { return "ascq 0.1 (gfx950)"; }
+
+extern "C" int ascq_zero_fill(void* ptr, size_t bytes, void* stream)
+{
+    ASCQ_REQUIRE(ptr != nullptr || bytes == 0, ASCQ_ENULL, "ascq_zero_fill: ptr is NULL");
+    ASCQ_REQUIRE(bytes % 4 == 0 && (reinterpret_cast<uintptr_t>(ptr) & 3u) == 0, ASCQ_EALIGN,
+                 "ascq_zero_fill: pointer and size must be multiples of 4 bytes");
+    if (bytes == 0) {
+        return ASCQ_OK;
+    }
+    size_t words = bytes / 4;
+    size_t blocks = std::min<size_t>((words + 255) / 256, 4096);
+    zero_fill_kernel<<<static_cast<uint32_t>(blocks), 256, 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<uint32_t*>(ptr), words);
+    return launch_status("ascq_zero_fill");
+}
+
+// Bit layout: docs/zh/api/SIMD-API/基础API/矩阵计算（ISASI）/矩阵计算的搬出/关键特性说明/随路量化.md (tables 1 and 2):
+// [31:0] fp32 scale (the hardware reads [31:13]), [45:37] offset, [46] signed result.
+extern "C" uint64_t ascq_pack_quant_param(float scale, int32_t offset9, int32_t is_signed)
+{
+    uint32_t bits;
+    std::memcpy(&bits, &scale, 4);
+    return static_cast<uint64_t>(bits) | (static_cast<uint64_t>(offset9 & 0x1FF) << 37) |
+           (static_cast<uint64_t>(is_signed ? 1 : 0) << 46);
+}
+
+// ref: impl/adv_api/tiling/quantization/ascend_quant_tiling_impl.cpp:31-68
+extern "C" int ascq_get_ascend_quant_max_min_tmp_size(const uint32_t* shape, uint32_t ndim, uint32_t type_size,
+                                                      uint32_t* max_value, uint32_t* min_value)
+{
+    ASCQ_REQUIRE(shape && max_value && min_value, ASCQ_ENULL, "GetAscendQuantMaxMinTmpSize: NULL argument");
+    // Like the reference, a failed check is reported but the sizes are still produced.
+    const uint64_t size = shape_size(shape, ndim);
+    const uint32_t two_repeats = 2u * 256u;
+    uint32_t mx = std::max<uint32_t>(static_cast<uint32_t>(size) * 2u, two_repeats);
+    *max_value = (mx + 31u) / 32u * 32u;
+    *min_value = two_repeats;
+    ASCQ_REQUIRE(size > 0, ASCQ_EINVAL, "[AscendQuant][GetAscendQuantMaxMinTmpSize] Input Shape size must be greater than 0.");
+    ASCQ_REQUIRE(size * type_size % 32 == 0, ASCQ_EALIGN,
+                 "[AscendQuant][GetAscendQuantMaxMinTmpSize] Input Shape size must be 32B aligned!.");
+    ASCQ_REQUIRE(type_size == 2 || type_size == 4, ASCQ_EUNSUPPORTED,
+                 "[AscendQuant][GetAscendQuantMaxMinTmpSize] Type size %u is unsupported!", type_size);
+    return ASCQ_OK;
+}
+
+// ref: impl/adv_api/tiling/quantization/ascend_dequant_tiling_impl.cpp:31-118
+extern "C" int ascq_get_ascend_dequant_max_min_tmp_size(const uint32_t* shape, uint32_t ndim, uint32_t type_size,
+                                                        uint32_t* max_value, uint32_t* min_value)
+{
+    ASCQ_REQUIRE(shape && max_value && min_value, ASCQ_ENULL, "GetAscendDequantMaxMinTmpSize: NULL argument");
+    ASCQ_REQUIRE(ndim == 1 || ndim == 2, ASCQ_EINVAL,
+                 "[AscendDequant][GetAscendDequantMaxMinTmpSize] SrcShape dim %u is unsupported, must be 1 or 2!", ndim);
+    const uint32_t outer = ndim == 2 ? shape[0] : 1u;
+    const uint32_t inner = ndim == 2 ? shape[1] : shape[0];
+    const uint32_t deq_scale = inner + 8u;  // covers a bf16 deqScale padded to 32 bytes
+    *max_value = (64u + outer * inner + deq_scale) * 4u;
+    *min_value = (64u + inner + deq_scale) * 4u;
+    // Like the reference, a failed check is reported but the sizes are still produced.
+    ASCQ_REQUIRE(shape_size(shape, ndim) > 0, ASCQ_EINVAL,
+                 "[AscendDequant][GetAscendDequantMaxMinTmpSize] Input Shape size must be greater than 0.");
+    ASCQ_REQUIRE(type_size == 4, ASCQ_EUNSUPPORTED,
+                 "[AscendDequant][GetAscendDequantMaxMinTmpSize] Type size %u is unsupported!", type_size);
+    return ASCQ_OK;
+}
+
+// ref: impl/adv_api/tiling/quantization/ascend_antiquant_tiling_impl.cpp:70-150 (int8 / int4 sources)
+extern "C" int ascq_get_ascend_antiquant_max_min_tmp_size(const uint32_t* src_shape, uint32_t src_ndim,
+                                                          const uint32_t* scale_shape, uint32_t scale_ndim,
+                                                          int32_t is_transpose, int32_t input_dtype,
+                                                          int32_t output_dtype, uint32_t* max_value,
+                                                          uint32_t* min_value)
+{
+    ASCQ_REQUIRE(src_shape && scale_shape && max_value && min_value, ASCQ_ENULL,
+                 "GetAscendAntiQuantMaxMinTmpSize: NULL argument");
+    ASCQ_REQUIRE(src_ndim == 2, ASCQ_EINVAL, "[AscendAntiQuant] srcShape must be 2-dimensional");
+    const uint64_t src_size = shape_size(src_shape, src_ndim);
+    ASCQ_REQUIRE(src_size > 0, ASCQ_EINVAL,
+                 "[AscendAntiQuant][GetAscendAntiQuantMaxMinTmpSize] Input Shape size must be greater than 0.");
+    ASCQ_REQUIRE(input_dtype == ASCQ_I8 || input_dtype == ASCQ_I4, ASCQ_EUNSUPPORTED,
+                 "[AscendAntiQuant] input dtype %d", input_dtype);
+    if (output_dtype == ASCQ_F16) {
+        *max_value = 0;
+        *min_value = 0;
+        return ASCQ_OK;
+    }
+    const uint32_t scale_size = static_cast<uint32_t>(std::max<uint64_t>(shape_size(scale_shape, scale_ndim), 1));
+    const bool per_channel = scale_size != 1;
+    const uint32_t k = src_shape[0];
+    const uint32_t transposed = 80u * scale_size * 4u;  // (8 + 8 + 64) * N fp32
+    const uint32_t not_transposed = scale_size * 2u * 4u + 64u * k * 4u;
+    if (is_transpose && per_channel) {
+        *max_value = transposed;
+    } else if (!is_transpose && per_channel) {
+        *max_value = not_transposed;
+    } else {
+        *max_value = static_cast<uint32_t>(src_size) * 4u;
+    }
+    if (!per_channel) {
+        *min_value = 1024u;
+    } else {
+        *min_value = is_transpose ? transposed : not_transposed;
+    }
+    return ASCQ_OK;
+}

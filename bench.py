@@ -1,0 +1,306 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-inference hot path on one MI355X.
+
+Headline (the `value` of the JSON line): the W8A8 LLM linear at M=2048, K=4096, N=11008 - one step = dynamic
+per-token quantisation of the bf16 activations + the int8 MFMA GEMM with the fused dequant epilogue to bf16 - reported
+as int8 TOPS (2*M*K*N per step).  The same line carries the roofline of the dominant kernel (the GEMM, timed alone with
+events on the launch stream), the CPU baseline (the oracle, timed on the host cores), the W4A16 decode GEMV as HBM GB/s
+and, unless --quick, the other BASELINE workloads (elementwise ops, small-M linears, W4A16 M=4/16, the MoE grouped
+matmul) under "others".
+
+Inputs are synthetic, seeded and resident in HBM before the timed region.  Memory-bound workloads rotate among
+several buffer sets larger than the 256 MB Infinity Cache so that their input is read from HBM every iteration.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (os.path.join(ROOT, "asc-devkit_amd"), os.path.join(ROOT, "oracle")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 matrix peak, TOP/s
+PEAK_HBM_GBS = 8000.0     # MI355X HBM3E peak, GB/s
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--quick", action="store_true", help="headline + W4A16 GEMV only")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", default="", help="run a single workload: w8a8 | w4a16 | quant | dequant | antiquant | group")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU; run it with --gpus 1 (the path shards without communication, "
+              "see DESIGN.md).", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from ascq import _abi as abi
+    from ascq import ops
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    abi.load_library()           # fail loudly if the HIP library is missing
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(0xA5C0)
+
+    def rand_i8(*shape):
+        return torch.randint(-127, 128, shape, dtype=torch.int8, device=dev, generator=gen)
+
+    def timed(fn, steps, warmup, inner=None):
+        """Times `steps` calls of fn(i) after `warmup`; returns (ms per step, ms per step of the `inner` section).
+        `inner` events are recorded by fn itself through the two lists it receives."""
+        starts, stops = [], []
+        for i in range(warmup):
+            fn(i, None, None)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            fn(warmup + i, starts, stops)
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+        kern_ms = None
+        if starts:
+            kern_ms = sum(a.elapsed_time(b) for a, b in zip(starts, stops)) / len(starts)
+        return wall_ms, kern_ms
+
+    def bracket(starts, stops, call):
+        if starts is None:
+            call()
+            return
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        call()
+        b.record()
+        starts.append(a)
+        stops.append(b)
+
+    results = {}
+
+    # ------------------------------------------------------------------ W8A8 linear (config 3)
+    def w8a8(M, steps, warmup):
+        K, N = 4096, 11008
+        x = torch.randn((M, K), device=dev, generator=gen).to(torch.bfloat16)
+        w = rand_i8(K, N)
+        cs = torch.rand(N, device=dev, generator=gen) * (1e-2 - 1e-4) + 1e-4
+        q = torch.empty((M, K), dtype=torch.int8, device=dev)
+        ts = torch.empty(M, dtype=torch.float32, device=dev)
+        c = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+        mm = ops.Matmul(M, N, K)
+        mm.set_tensor_a(q)
+        mm.set_tensor_b(w)
+        mm.set_quant_vector(cs)
+        mm.set_token_scale(ts)
+
+        def step(i, starts, stops):
+            ops.dynamic_quant_per_token(x, q, ts)
+            bracket(starts, stops, lambda: mm.iterate_all(c))
+
+        ms, kern_ms = timed(step, steps, warmup)
+        flops = 2.0 * M * K * N
+        bytes_ = M * K + K * N + 4 * N + 4 * M + 2 * M * N
+        return {"ms_per_step": ms, "gemm_kernel_ms": kern_ms, "tops": flops / (ms * 1e-3) / 1e12,
+                "gemm_tops": flops / (kern_ms * 1e-3) / 1e12, "gemm_gbs": bytes_ / (kern_ms * 1e-3) / 1e9,
+                "ops": flops, "bytes": bytes_, "tensors": (x, w, cs)}
+
+    # ------------------------------------------------------------------ W4A16 decode (config 4)
+    def w4a16(M, steps, warmup, sets=4):
+        K, N, gs = 8192, 28672, 128
+        xs = torch.randn((M, K), device=dev, generator=gen).to(torch.float16)
+        ws = [torch.randint(0, 256, (K, N // 2), dtype=torch.uint8, device=dev, generator=gen) for _ in range(sets)]
+        sc = [(torch.rand((K // gs, N), device=dev, generator=gen) * 9e-3 + 1e-3).to(torch.float16) for _ in range(sets)]
+        of = [torch.randint(-8, 8, (K // gs, N), device=dev, generator=gen).to(torch.float16) for _ in range(sets)]
+        y = torch.empty((M, N), dtype=torch.float16, device=dev)
+
+        def step(i, starts, stops):
+            j = i % sets
+            bracket(starts, stops, lambda: ops.matmul_w4a16(y, xs, ws[j], sc[j], of[j], gs))
+
+        ms, kern_ms = timed(step, steps, warmup)
+        bytes_ = K * N // 2 + 2 * (K // gs) * N * 2 + M * K * 2 + M * N * 2
+        return {"ms_per_step": ms, "kernel_ms": kern_ms, "gbs": bytes_ / (kern_ms * 1e-3) / 1e9, "bytes": bytes_,
+                "tops": 2.0 * M * K * N / (kern_ms * 1e-3) / 1e12, "tensors": (xs, ws[0], sc[0], of[0])}
+
+    # ------------------------------------------------------------------ elementwise (config 2)
+    def quant2a(steps, warmup, sets=3):
+        m, n = 8192, 4096
+        xs = [(torch.randn((m, n), device=dev, generator=gen) * 2).to(torch.float16) for _ in range(sets)]
+        ss = [(127.0 / x.float().abs().amax(dim=0)).to(torch.float16) for x in xs]
+        dst = [torch.empty((m, n), dtype=torch.int8, device=dev) for _ in range(sets)]
+
+        def step(i, starts, stops):
+            j = i % sets
+            bracket(starts, stops, lambda: ops.ascend_quant(dst[j], xs[j], ss[j], 0.0))
+
+        ms, kern_ms = timed(step, steps, warmup)
+        bytes_ = m * n * 3 + n * 2
+        return {"kernel_ms": kern_ms, "gbs": bytes_ / (kern_ms * 1e-3) / 1e9, "bytes": bytes_, "tensors": (xs[0], ss[0])}
+
+    def dequant2b(steps, warmup, sets=2):
+        m, n = 8192, 4096
+        src = [torch.randint(-2**20, 2**20 + 1, (m, n), dtype=torch.int32, device=dev, generator=gen) for _ in range(sets)]
+        sc = torch.rand(n, device=dev, generator=gen) * (1e-3 - 1e-5) + 1e-5
+        dst = [torch.empty((m, n), dtype=torch.bfloat16, device=dev) for _ in range(sets)]
+        prm = ops.DequantParams(m, n, n)
+
+        def step(i, starts, stops):
+            j = i % sets
+            bracket(starts, stops, lambda: ops.ascend_dequant(dst[j], src[j], sc, prm, abi.DEQUANT_WITH_MULTI_ROW))
+
+        ms, kern_ms = timed(step, steps, warmup)
+        bytes_ = m * n * 6 + n * 4
+        return {"kernel_ms": kern_ms, "gbs": bytes_ / (kern_ms * 1e-3) / 1e9, "bytes": bytes_}
+
+    def antiquant2c(steps, warmup, sets=3):
+        k, n = 4096, 11008
+        w = [rand_i8(k, n) for _ in range(sets)]
+        sc = (torch.rand((1, n), device=dev, generator=gen) * (1e-1 - 1e-3) + 1e-3).to(torch.float16)
+        of = torch.randint(-8, 9, (1, n), device=dev, generator=gen).to(torch.float16)
+        dst = [torch.empty((k, n), dtype=torch.float16, device=dev) for _ in range(sets)]
+        info = ops.AntiQuantShapeInfo(1, n, 1, n)
+
+        def step(i, starts, stops):
+            j = i % sets
+            bracket(starts, stops, lambda: ops.ascend_antiquant(dst[j], w[j], of, sc, k, info))
+
+        ms, kern_ms = timed(step, steps, warmup)
+        bytes_ = k * n * 3 + 2 * n * 2
+        return {"kernel_ms": kern_ms, "gbs": bytes_ / (kern_ms * 1e-3) / 1e9, "bytes": bytes_}
+
+    # ------------------------------------------------------------------ grouped matmul (config 5)
+    def group5(steps, warmup):
+        G, T, K, N = 8, 4096, 4096, 14336
+        rng = np.random.default_rng(0xC5)
+        counts = rng.multinomial(T, [1.0 / G] * G)
+        gl = torch.from_numpy(np.cumsum(counts).astype(np.int64)).to(dev)
+        x = rand_i8(T, K)
+        w = rand_i8(G, K, N)
+        cs = torch.rand((G, N), device=dev, generator=gen) * (1e-2 - 1e-4) + 1e-4
+        ts = torch.rand(T, device=dev, generator=gen) * (1e-1 - 1e-3) + 1e-3
+        bias = torch.randn((G, N), device=dev, generator=gen).to(torch.bfloat16)
+        y = torch.empty((T, N), dtype=torch.bfloat16, device=dev)
+
+        def step(i, starts, stops):
+            bracket(starts, stops, lambda: ops.quant_group_matmul(y, x, w, gl, cs, ts, bias, abi.GROUP_LIST_PREFIX_SUM))
+
+        ms, kern_ms = timed(step, steps, warmup)
+        flops = 2.0 * T * K * N
+        bytes_ = T * K + G * K * N + G * N * 4 + T * 4 + G * N * 2 + T * N * 2 + G * 8
+        return {"kernel_ms": kern_ms, "tops": flops / (kern_ms * 1e-3) / 1e12, "gbs": bytes_ / (kern_ms * 1e-3) / 1e9,
+                "ops": flops, "bytes": bytes_}
+
+    def strip(d):
+        return {k: v for k, v in d.items() if k != "tensors"}
+
+    only = args.only
+    if only and only != "w8a8":
+        fn = {"w4a16": lambda: w4a16(1, args.steps, args.warmup), "quant": lambda: quant2a(args.steps, args.warmup),
+              "dequant": lambda: dequant2b(args.steps, args.warmup),
+              "antiquant": lambda: antiquant2c(args.steps, args.warmup),
+              "group": lambda: group5(args.steps, args.warmup)}[only]
+        print(json.dumps({only: strip(fn())}))
+        return
+
+    head = w8a8(2048, args.steps, args.warmup)
+    out = {
+        "metric": "w8a8_linear_int8_tops_m2048_k4096_n11008",
+        "value": head["tops"],
+        "unit": "TOPS",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8",
+        "data": "synthetic",
+        "config": {"workload": "BASELINE configs[2] (W8A8 LLM linear) at M=2048: bf16 x [2048,4096] -> dynamic "
+                               "per-token int8 quant -> int8 GEMM with W [4096,11008] -> fused (channel x token) "
+                               "dequant to bf16; one step = quant kernel + GEMM kernel",
+                   "m": 2048, "k": 4096, "n": 11008, "ops_per_step": head["ops"]},
+        "roofline": {"bound": "mfma", "kernel": "gemm_kernel<Tile 256x256x128, B [k,n]>",
+                     "achieved": head["gemm_tops"], "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+                     "frac": head["gemm_tops"] / PEAK_INT8_TOPS, "traffic": None,
+                     "avg_kernel_ms": head["gemm_kernel_ms"]},
+    }
+    if only == "w8a8":
+        print(json.dumps(out))
+        return
+
+    gemv = w4a16(1, args.steps, args.warmup)
+    out["w4a16_gemv"] = {"metric": "w4a16_decode_gemv_hbm_gbs_m1_k8192_n28672", "value": gemv["gbs"], "unit": "GB/s",
+                         "workload": "BASELINE configs[3] at M=1, 4 rotating weight sets (500 MB > Infinity Cache)",
+                         "ms_per_step": gemv["ms_per_step"],
+                         "roofline": {"bound": "hbm", "kernel": "w4a16_partial_kernel<1> + w4a16_reduce_kernel",
+                                      "achieved": gemv["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                      "frac": gemv["gbs"] / PEAK_HBM_GBS, "traffic": None,
+                                      "avg_kernel_ms": gemv["kernel_ms"], "bytes_per_launch": gemv["bytes"]}}
+
+    if not args.quick:
+        others = {}
+        s2, w2 = max(10, args.steps // 2), max(3, args.warmup // 2)
+        for name, fn in (("quant_2a", lambda: quant2a(s2, w2)), ("dequant_2b", lambda: dequant2b(s2, w2)),
+                         ("antiquant_2c", lambda: antiquant2c(s2, w2))):
+            r = strip(fn())
+            r["hbm_frac"] = r["gbs"] / PEAK_HBM_GBS
+            others[name] = r
+            torch.cuda.empty_cache()
+        for M in (1, 16, 128):
+            r = strip(w8a8(M, s2, w2))
+            others[f"w8a8_m{M}"] = {"gemm_kernel_ms": r["gemm_kernel_ms"], "gemm_tops": r["gemm_tops"],
+                                    "gemm_gbs": r["gemm_gbs"], "hbm_frac": r["gemm_gbs"] / PEAK_HBM_GBS,
+                                    "mfma_frac": r["gemm_tops"] / PEAK_INT8_TOPS}
+        for M in (4, 16):
+            r = strip(w4a16(M, s2, w2))
+            others[f"w4a16_m{M}"] = {"kernel_ms": r["kernel_ms"], "gbs": r["gbs"], "hbm_frac": r["gbs"] / PEAK_HBM_GBS}
+            torch.cuda.empty_cache()
+        r = group5(max(5, args.steps // 5), 2)
+        r["mfma_frac"] = r["tops"] / PEAK_INT8_TOPS
+        r["hbm_frac"] = r["gbs"] / PEAK_HBM_GBS
+        others["group_matmul_config5"] = r
+        out["others"] = others
+
+    # ------------------------------------------------------------------ CPU baseline (the oracle; a checker being timed)
+    if not args.no_cpu:
+        import orc
+        cores = min(16, os.cpu_count() or 1)
+        orc.set_threads(cores)
+        x, w, cs = head["tensors"]
+        rows = 512                                    # bounded sample: the first 512 of the 2048 activation rows
+        xb = x[:rows].view(torch.int16).cpu().numpy().view(np.uint16)
+        wn, csn = w.cpu().numpy(), cs.cpu().numpy()
+        t0 = time.perf_counter()
+        qn, tsn = orc.dynamic_quant_per_token(abi.BF16, xb)
+        d = abi.MatmulDesc(m=rows, n=11008, k=4096, out_dtype=abi.BF16, quant_mode=abi.MM_QUANT_VECTOR,
+                           scale_format=abi.MM_SCALE_F32, has_tok_scale=1)
+        orc.matmul_w8a8(d, qn, wn, None, csn, tsn)
+        dt = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": 2.0 * rows * 4096 * 11008 / dt / 1e12, "unit": "TOPS", "cores": cores,
+                               "kind": "port",
+                               "sample": f"first {rows} of 2048 rows of the same workload (quant + GEMM + epilogue), "
+                                         f"{dt:.2f} s, OpenMP over rows"}
+        xs, w4, sc4, of4 = gemv["tensors"]
+        cols = 2048                                   # bounded sample: 2048 of the 28672 output columns
+        d4 = abi.W4A16Desc(m=1, n=28672, k=8192, group_size=128, has_offset=1)
+        t0 = time.perf_counter()
+        orc.matmul_w4a16(d4, xs.cpu().numpy(), w4.cpu().numpy(), sc4.cpu().numpy(), of4.cpu().numpy(), cols=(0, cols))
+        dt = time.perf_counter() - t0
+        out["w4a16_gemv"]["cpu_baseline"] = {"value": gemv["bytes"] * (cols / 28672) / dt / 1e9, "unit": "GB/s",
+                                             "cores": cores, "kind": "port",
+                                             "sample": f"{cols} of 28672 output columns, {dt:.2f} s"}
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

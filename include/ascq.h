@@ -99,7 +99,7 @@ typedef struct ascq_quant_desc {
     int32_t src_dtype;   /* ASCQ_F16 | ASCQ_BF16 | ASCQ_F32 */
     int32_t scale_dtype; /* dtype of the scale/offset tensors */
     int32_t compute;     /* ascq_quant_compute */
-    int32_t round_mode;  /* ascq_round_mode (COMPUTE_F16 always rounds half-even) */
+    int32_t round_mode;  /* an ascq_round_mode value; COMPUTE_F16 always rounds half-even */
     int32_t offset_kind; /* ascq_offset_kind */
     int32_t k_dim;       /* PER_GROUP: 1 = groups along n, 0 = groups along m */
     float scale;         /* PER_TENSOR scale */

@@ -631,57 +631,51 @@ int orc_group_matmul_w8a8(const ascq_group_matmul_desc* g, void* y, const int8_t
 int orc_matmul_w4a16(const ascq_w4a16_desc* d, uint16_t* y, const uint16_t* x, const uint8_t* w,
                      const uint16_t* scale, const uint16_t* offset)
 {
+    return orc_matmul_w4a16_cols(d, y, x, w, scale, offset, 0, d->n);
+}
+
+/* Output columns [j0, j1) only: lets a benchmark time a bounded sample of a large problem. */
+int orc_matmul_w4a16_cols(const ascq_w4a16_desc* d, uint16_t* y, const uint16_t* x, const uint8_t* w,
+                          const uint16_t* scale, const uint16_t* offset, uint32_t j0, uint32_t j1)
+{
     size_t M = d->m, N = d->n, K = d->k, gs = d->group_size;
+    const size_t blk = 64; /* columns per task: each weight is de-quantised once and used for all m rows */
+    size_t nblk = (j1 - j0 + blk - 1) / blk;
+    float* xf = (float*)malloc(M * K * sizeof(float));
+    for (size_t i = 0; i < M * K; ++i) {
+        xf[i] = orc_f16_to_f32(x[i]);
+    }
 #pragma omp parallel
     {
-        double* acc = (double*)malloc(N * sizeof(double));
-#pragma omp for schedule(static)
-        for (size_t i = 0; i < M; ++i) {
-            for (size_t j = 0; j < N; ++j) {
-                acc[j] = 0.0;
+        double* acc = (double*)malloc(M * blk * sizeof(double));
+#pragma omp for schedule(dynamic, 1)
+        for (size_t b = 0; b < nblk; ++b) {
+            size_t c0 = j0 + b * blk, c1 = c0 + blk < j1 ? c0 + blk : j1;
+            for (size_t t = 0; t < M * blk; ++t) {
+                acc[t] = 0.0;
             }
             for (size_t kk = 0; kk < K; ++kk) {
-                float xv = orc_f16_to_f32(x[i * K + kk]);
                 size_t g = kk / gs;
-                for (size_t j = 0; j < N; ++j) {
+                for (size_t j = c0; j < c1; ++j) {
                     uint16_t h = orc_f32_to_f16((float)load_i4(w, kk * N + j));
                     if (d->has_offset) {
                         h = orc_f16_add(h, offset[g * N + j]);
                     }
-                    uint16_t wd = orc_f16_mul(scale[g * N + j], h);
-                    acc[j] += (double)xv * (double)orc_f16_to_f32(wd);
+                    double wd = (double)orc_f16_to_f32(orc_f16_mul(scale[g * N + j], h));
+                    for (size_t i = 0; i < M; ++i) {
+                        acc[i * blk + (j - c0)] += (double)xf[i * K + kk] * wd;
+                    }
                 }
             }
-            for (size_t j = 0; j < N; ++j) {
-                y[i * N + j] = orc_f64_to_f16(acc[j]);
+            for (size_t i = 0; i < M; ++i) {
+                for (size_t j = c0; j < c1; ++j) {
+                    y[i * N + j] = orc_f64_to_f16(acc[i * blk + (j - c0)]);
+                }
             }
         }
         free(acc);
     }
-    return 0;
-}
-
-/* Only the weight de-quantisation of output columns [j0, j1) for one activation row: bounded CPU timing sample. */
-int orc_matmul_w4a16_cols(const ascq_w4a16_desc* d, uint16_t* y, const uint16_t* x, const uint8_t* w,
-                          const uint16_t* scale, const uint16_t* offset, uint32_t j0, uint32_t j1)
-{
-    size_t N = d->n, K = d->k, gs = d->group_size;
-    for (size_t i = 0; i < d->m; ++i) {
-#pragma omp parallel for schedule(static)
-        for (size_t j = j0; j < j1; ++j) {
-            double acc = 0.0;
-            for (size_t kk = 0; kk < K; ++kk) {
-                size_t g = kk / gs;
-                uint16_t h = orc_f32_to_f16((float)load_i4(w, kk * N + j));
-                if (d->has_offset) {
-                    h = orc_f16_add(h, offset[g * N + j]);
-                }
-                uint16_t wd = orc_f16_mul(scale[g * N + j], h);
-                acc += (double)orc_f16_to_f32(x[i * K + kk]) * (double)orc_f16_to_f32(wd);
-            }
-            y[i * N + j] = orc_f64_to_f16(acc);
-        }
-    }
+    free(xf);
     return 0;
 }
 

@@ -1,0 +1,184 @@
+"""No-GPU checks of the C ABI: the library loads, exports every symbol include/ascq.h declares, rejects bad
+descriptors with the documented status before touching the GPU, and answers the host tiling queries with the
+reference's known answers (tests/api/adv_api/tiling/test_tiling.cpp:6539-6703 of the reference)."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from ascq import _abi as abi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+L = abi.load_library()
+FAKE = C.c_void_p(0x1000)          # never dereferenced: validation fails first
+
+
+def err():
+    return L.ascq_last_error().decode()
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    header = open(os.path.join(ROOT, "include", "ascq.h")).read()
+    declared = set(re.findall(r"\b(ascq_[a-z0-9_]+)\s*\(", header))
+    assert declared == set(abi.SIGNATURES), declared ^ set(abi.SIGNATURES)
+    for name in declared:
+        assert hasattr(L, name)
+    assert b"gfx950" in L.ascq_version()
+
+
+def test_struct_sizes_match_the_header():
+    # field-by-field layout is 4-byte scalars; the matmul descriptor ends with an 8-byte word
+    assert C.sizeof(abi.QuantDesc) == 13 * 4
+    assert C.sizeof(abi.DequantDesc) == 11 * 4
+    assert C.sizeof(abi.AntiQuantDesc) == 13 * 4
+    assert C.sizeof(abi.MatmulDesc) == 11 * 4 + 4 + 8
+    assert C.sizeof(abi.GroupMatmulDesc) == C.sizeof(abi.MatmulDesc) + 8
+    assert C.sizeof(abi.W4A16Desc) == 5 * 4
+
+
+def q(**kw):
+    d = abi.QuantDesc(policy=abi.PER_CHANNEL, src_dtype=abi.F16, scale_dtype=abi.F16, compute=abi.COMPUTE_F16,
+                      round_mode=abi.CAST_RINT, offset_kind=abi.OFFSET_SCALAR, k_dim=1, n=64, cal_count=640)
+    for k, v in kw.items():
+        setattr(d, k, v)
+    return d
+
+
+def test_quant_rejections():
+    call = lambda d, dst=FAKE, src=C.c_void_p(0x100000), sc=FAKE, of=FAKE: L.ascq_quant(C.byref(d), dst, src, sc, of, None)
+    assert L.ascq_quant(None, FAKE, FAKE, FAKE, FAKE, None) == abi.ENULL
+    assert call(q(), dst=None) == abi.ENULL
+    assert call(q(), sc=None) == abi.ENULL
+    assert call(q(offset_kind=abi.OFFSET_TENSOR), of=None) == abi.ENULL
+    assert call(q(policy=9)) == abi.EINVAL
+    assert call(q(cal_count=650)) == abi.EINVAL and "integer multiple" in err()      # calCount % scaleCount != 0
+    assert call(q(n=0)) == abi.EINVAL
+    assert call(q(src_dtype=abi.I8)) == abi.EUNSUPPORTED
+    assert call(q(round_mode=6)) == abi.EUNSUPPORTED                                   # CAST_ODD has no int8 form
+    assert call(q(policy=abi.PER_TOKEN)) == abi.EUNSUPPORTED                           # fp16 compute is tensor/channel only
+    assert call(q(scale_dtype=abi.F32)) == abi.EUNSUPPORTED                            # legacy: scale dtype == src dtype
+    tok = dict(policy=abi.PER_TOKEN, compute=abi.COMPUTE_SCALE_T, m=10, n=288, cal_count=2880)
+    assert call(q(src_dtype=abi.F32, scale_dtype=abi.F16, **tok)) == abi.EUNSUPPORTED  # (float, half) is not a legal pair
+    assert call(q(**dict(tok, cal_count=2881))) == abi.EINVAL
+    assert call(q(**dict(tok, m=9))) == abi.EINVAL                                     # calCount > m*n
+    assert call(q(**dict(tok, n=24, cal_count=240))) == abi.EALIGN                     # 48-byte rows
+    grp = dict(tok, policy=abi.PER_GROUP, n=256, cal_count=2560)
+    assert call(q(group_size=48, **grp)) == abi.EINVAL and "multiple of 32" in err()
+    assert call(q(group_size=0, **grp)) == abi.EINVAL
+    assert call(q(group_size=64, k_dim=2, **grp)) == abi.EINVAL
+    assert call(q(), dst=C.c_void_p(0x100010)) == abi.EINVAL and "overlaps" in err()
+    assert call(q(cal_count=0)) == abi.OK                                              # nothing to do, nothing launched
+
+
+def test_dequant_rejections():
+    def d(**kw):
+        x = abi.DequantDesc(policy=abi.PER_CHANNEL, src_dtype=abi.I32, scale_dtype=abi.F32, dst_dtype=abi.BF16,
+                            mode=abi.DEQUANT_WITH_MULTI_ROW, m=4, n=64, cal_count=64)
+        for k, v in kw.items():
+            setattr(x, k, v)
+        return x
+    call = lambda x, sc=FAKE: L.ascq_dequant(C.byref(x), FAKE, C.c_void_p(0x100000), sc, None)
+    assert call(d(), sc=None) == abi.ENULL
+    assert call(d(n=60, cal_count=60)) == abi.EALIGN                                   # 240-byte rows
+    assert call(d(cal_count=65)) == abi.EINVAL
+    assert call(d(dst_dtype=abi.F16)) == abi.EUNSUPPORTED                              # half out needs uint64 scale
+    assert call(d(scale_dtype=abi.U64, dst_dtype=abi.BF16)) == abi.EUNSUPPORTED
+    assert call(d(policy=abi.PER_TENSOR, dst_dtype=abi.F16)) == abi.EUNSUPPORTED
+    assert call(d(src_dtype=abi.F32)) == abi.EUNSUPPORTED
+    assert call(d(policy=abi.PER_GROUP, group_size=40, k_dim=1)) == abi.EINVAL
+    assert call(d(m=0)) == abi.EINVAL
+    assert L.ascq_dequant_dst_stride(abi.BF16, 40) == 48 and L.ascq_dequant_dst_stride(abi.F32, 40) == 40
+
+
+def test_antiquant_rejections():
+    def d(**kw):
+        x = abi.AntiQuantDesc(src_dtype=abi.I8, dst_dtype=abi.F16, has_offset=1, k=64, n=128, scale_height=1,
+                              scale_width=128, offset_height=1, offset_width=128)
+        for k, v in kw.items():
+            setattr(x, k, v)
+        return x
+    call = lambda x, of=FAKE, sc=FAKE: L.ascq_antiquant(C.byref(x), FAKE, C.c_void_p(0x100000), of, sc, None)
+    assert call(d(), sc=None) == abi.ENULL
+    assert call(d(), of=None) == abi.ENULL
+    assert call(d(src_dtype=abi.F16)) == abi.EUNSUPPORTED
+    assert call(d(dst_dtype=abi.F32)) == abi.EUNSUPPORTED
+    assert call(d(scale_height=3)) == abi.EINVAL                                       # k % groups != 0
+    assert call(d(offset_height=2, scale_height=4)) == abi.EINVAL
+    assert call(d(is_transpose=1, k=48, scale_width=1, scale_height=128, offset_width=1, offset_height=128)) == abi.EALIGN  # k not 32-byte aligned
+    assert call(d(k=0)) == abi.EINVAL
+
+
+def test_matmul_rejections():
+    def d(**kw):
+        x = abi.MatmulDesc(m=32, n=64, k=64, out_dtype=abi.BF16, quant_mode=abi.MM_QUANT_VECTOR,
+                           scale_format=abi.MM_SCALE_F32)
+        for k, v in kw.items():
+            setattr(x, k, v)
+        return x
+    call = lambda x, bias=None, qv=FAKE, tok=None: L.ascq_matmul_w8a8(C.byref(x), FAKE, FAKE, FAKE, bias, qv, tok,
+                                                                     None, 0, None)
+    assert call(d(), qv=None) == abi.ENULL
+    assert call(d(bias_kind=abi.MM_BIAS_F32_POST)) == abi.ENULL
+    assert call(d(has_tok_scale=1)) == abi.ENULL
+    assert call(d(k=0)) == abi.EINVAL
+    assert call(d(out_dtype=abi.I32)) == abi.EUNSUPPORTED
+    assert call(d(out_dtype=abi.I8)) == abi.EUNSUPPORTED                               # requant needs the uint64 words
+    assert call(d(quant_mode=abi.MM_QUANT_NONE)) == abi.EUNSUPPORTED                   # int32 out only
+    assert call(d(quant_mode=abi.MM_QUANT_NONE, out_dtype=abi.I32, has_tok_scale=1), tok=FAKE) == abi.EUNSUPPORTED
+    g = abi.GroupMatmulDesc(mm=d(), groups=0, group_list_kind=abi.GROUP_LIST_COUNTS)
+    gcall = lambda x, gl=FAKE: L.ascq_group_matmul_w8a8(C.byref(x), FAKE, FAKE, FAKE, None, FAKE, None, gl, None)
+    assert gcall(g) == abi.EINVAL
+    g.groups = 4
+    assert gcall(g, gl=None) == abi.ENULL
+    g.mm.scale_format = abi.MM_SCALE_U64
+    assert gcall(g) == abi.EUNSUPPORTED
+    g.mm.scale_format, g.mm.k = abi.MM_SCALE_F32, 72
+    assert gcall(g) == abi.EALIGN
+
+
+def test_w4a16_rejections_and_workspace():
+    d = abi.W4A16Desc(m=1, n=1024, k=512, group_size=128, has_offset=1)
+    n = C.c_size_t(0)
+    assert L.ascq_matmul_w4a16_workspace_size(C.byref(d), C.byref(n)) == abi.OK and n.value % (1024 * 4) == 0
+    assert L.ascq_matmul_w4a16(C.byref(d), FAKE, FAKE, FAKE, FAKE, None, FAKE, 1 << 30, None) == abi.ENULL
+    assert L.ascq_matmul_w4a16(C.byref(d), FAKE, FAKE, FAKE, FAKE, FAKE, None, 0, None) == abi.EINVAL
+    assert "workspace" in err()
+    d.group_size = 96
+    assert L.ascq_matmul_w4a16_workspace_size(C.byref(d), C.byref(n)) == abi.EINVAL
+    d.group_size, d.n = 128, 1023
+    assert L.ascq_matmul_w4a16_workspace_size(C.byref(d), C.byref(n)) == abi.EINVAL
+
+
+def sizes(fn, *args):
+    mx, mn = C.c_uint32(0), C.c_uint32(0)
+    rc = fn(*args, C.byref(mx), C.byref(mn))
+    return rc, mx.value, mn.value
+
+
+def u32(*v):
+    return (C.c_uint32 * len(v))(*v)
+
+
+def test_tiling_known_answers():
+    # TestAscendQuantTiling: {512} x 2 bytes -> min 2*256, max 2*512
+    assert sizes(L.ascq_get_ascend_quant_max_min_tmp_size, u32(512), 1, 2) == (abi.OK, 1024, 512)
+    # TestAscendDequantTiling (the reference passes typeSize 2: reported, sizes still produced)
+    rc, mx, mn = sizes(L.ascq_get_ascend_dequant_max_min_tmp_size, u32(10, 32), 2, 2)
+    assert (mx, mn) == (4 * (64 + 32 * 10 + 40), 4 * (64 + 32 + 40)) and rc == abi.EUNSUPPORTED
+    assert sizes(L.ascq_get_ascend_dequant_max_min_tmp_size, u32(320), 1, 4) == (abi.OK, 4 * (64 + 320 + 328),
+                                                                                4 * (64 + 320 + 328))
+    aq = L.ascq_get_ascend_antiquant_max_min_tmp_size
+    # TestAntiquantTilingNoTransposePerChannelHalf / ...PerChannel / ...PerTensor / TransposePerChannel
+    assert sizes(aq, u32(640, 5120), 2, u32(1, 5120), 2, 0, abi.I8, abi.F16) == (abi.OK, 0, 0)
+    exp = 5120 * 2 * 4 + 64 * 640 * 4
+    assert sizes(aq, u32(640, 5120), 2, u32(1, 5120), 2, 0, abi.I8, abi.BF16) == (abi.OK, exp, exp)
+    assert sizes(aq, u32(640, 5120), 2, u32(1), 1, 0, abi.I8, abi.BF16) == (abi.OK, 640 * 5120 * 4, 1024)
+    assert sizes(aq, u32(64, 512), 2, u32(64, 1), 2, 1, abi.I8, abi.BF16) == (abi.OK, 80 * 64 * 4, 80 * 64 * 4)
+    assert sizes(aq, u32(640, 5120), 2, u32(1), 1, 1, abi.I8, abi.BF16) == (abi.OK, 640 * 5120 * 4, 1024)
+
+
+def test_pack_quant_param():
+    import numpy as np
+    w = L.ascq_pack_quant_param(0.1, 5, 1)
+    assert (w & 0xFFFFFFFF) == int(np.float32(0.1).view(np.uint32)) and (w >> 37) & 0x1FF == 5 and (w >> 46) & 1 == 1

@@ -1,0 +1,285 @@
+"""GPU parity of AscendQuant / AscendDequant / AscendAntiQuant / dynamic per-token quant against the CPU oracle,
+through the C ABI.  int8 outputs must be bit-exact; 16-bit float outputs are compared bit for bit as well (every
+operation of these operators rounds once, so there is no tolerance to grant)."""
+import numpy as np
+import pytest
+import torch
+
+import orc
+from ascq import _abi as abi
+from ascq import ops
+from gpu_util import DEV, announce, bits, pack_int4, src_array, src_array_uniform, to_dev
+
+pytestmark = pytest.mark.gpu
+TDT = {abi.F16: torch.float16, abi.BF16: torch.bfloat16, abi.F32: torch.float32}
+
+
+# ------------------------------------------------------------------ AscendQuant, fp16 contract
+@pytest.mark.parametrize("src_dt", [abi.F16, abi.F32, abi.BF16])
+@pytest.mark.parametrize("count", [256, 1022, 8192 * 3, 2048 * 37 + 8])
+def test_quant_per_tensor(src_dt, count):
+    announce("quant per-tensor", src_dt, count)
+    rng = np.random.default_rng(100 + count)
+    x, xd = src_array(rng, count, src_dt, 40.0)
+    dst = torch.zeros(count, dtype=torch.int8, device=DEV)
+    ops.ascend_quant(dst, xd, 2.0, 0.9)
+    d = abi.QuantDesc(policy=abi.PER_TENSOR, src_dtype=src_dt, scale_dtype=src_dt, compute=abi.COMPUTE_F16,
+                      round_mode=abi.CAST_RINT, offset_kind=abi.OFFSET_SCALAR, scale=2.0, offset=0.9, cal_count=count)
+    want = orc.quant(d, x)
+    assert np.array_equal(dst.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("src_dt", [abi.F16, abi.F32])
+@pytest.mark.parametrize("rows,n", [(37, 64), (8, 4096), (5, 36), (129, 2080)])
+@pytest.mark.parametrize("tensor_offset", [False, True])
+def test_quant_per_channel(src_dt, rows, n, tensor_offset):
+    announce("quant per-channel", src_dt, rows, n, tensor_offset)
+    rng = np.random.default_rng(7 * rows + n)
+    x, xd = src_array(rng, (rows, n), src_dt, 2.0)
+    amax = np.abs(x.astype(np.float32)).max(axis=0) + 1e-3
+    s, sd = (127.0 / amax).astype(np.float32), None
+    s = s.astype(np.float16) if src_dt == abi.F16 else s
+    sd = to_dev(s)
+    dst = torch.zeros((rows, n), dtype=torch.int8, device=DEV)
+    d = abi.QuantDesc(policy=abi.PER_CHANNEL, src_dtype=src_dt, scale_dtype=src_dt, compute=abi.COMPUTE_F16,
+                      round_mode=abi.CAST_RINT, n=n, cal_count=rows * n)
+    if tensor_offset:
+        o, od = src_array_uniform(rng, n, src_dt, -3, 3)
+        ops.ascend_quant(dst, xd, sd, od)
+        d.offset_kind = abi.OFFSET_TENSOR
+        want = orc.quant(d, x, s, o)
+    else:
+        ops.ascend_quant(dst, xd, sd, 0.0)
+        d.offset_kind, d.offset = abi.OFFSET_SCALAR, 0.0
+        want = orc.quant(d, x, s)
+    got = dst.cpu().numpy()
+    assert np.array_equal(got, want)
+    assert np.abs(got.astype(np.int32)).max() >= 126     # the column maxima reach the int8 range
+
+
+# ------------------------------------------------------------------ PER_TOKEN / PER_GROUP / Quantize
+SHAPES = [(10, 288, 1152), (7, 288, 864), (6, 288, 1440), (8, 512, 3584), (4, 256, 768)]   # {m, n, calCount}
+PAIRS = [(abi.F16, abi.F16), (abi.BF16, abi.BF16), (abi.F32, abi.F32), (abi.F16, abi.F32), (abi.BF16, abi.F32)]
+
+
+@pytest.mark.parametrize("compute", [abi.COMPUTE_SCALE_T, abi.COMPUTE_F32])
+@pytest.mark.parametrize("pair", PAIRS)
+@pytest.mark.parametrize("offset", ["tensor", "scalar", "none"])
+def test_quant_per_token_matrix(compute, pair, offset):
+    src_dt, sc_dt = pair
+    for (m, n, cal) in SHAPES:
+        for rmode in (abi.CAST_RINT, abi.CAST_FLOOR, abi.CAST_CEIL, abi.CAST_ROUND, abi.CAST_TRUNC):
+            announce("quant per-token", compute, pair, offset, m, n, cal, rmode)
+            rng = np.random.default_rng(m * 1000 + n + rmode)
+            x, xd = src_array(rng, (m, n), src_dt, 1.0)
+            s, sd = src_array_uniform(rng, m, sc_dt, 5, 60)
+            o, od = src_array_uniform(rng, m, sc_dt, -2, 2)
+            dst = torch.full((m, n), 99, dtype=torch.int8, device=DEV)
+            cfg = ops.AscendQuantConfig(has_offset=offset != "none", k_dim=1, round_mode=rmode)
+            para = ops.AscendQuantParam(m=m, n=n, cal_count=cal)
+            fn = ops.ascend_quant_policy if compute == abi.COMPUTE_SCALE_T else ops.quantize
+            d = abi.QuantDesc(policy=abi.PER_TOKEN, src_dtype=src_dt, scale_dtype=sc_dt, compute=compute,
+                              round_mode=rmode, k_dim=1, m=m, n=n, cal_count=cal)
+            if offset == "tensor":
+                fn(dst, xd, sd, od, para, abi.PER_TOKEN, cfg)
+                d.offset_kind = abi.OFFSET_TENSOR
+            elif offset == "scalar":
+                fn(dst, xd, sd, 0.75, para, abi.PER_TOKEN, cfg)
+                d.offset_kind, d.offset = abi.OFFSET_SCALAR, 0.75
+            else:
+                fn(dst, xd, sd, None, para, abi.PER_TOKEN, cfg)
+            want = orc.quant(d, x.reshape(-1)[:cal].copy(), s, o)
+            got = dst.cpu().numpy().reshape(-1)
+            assert np.array_equal(got[:cal], want)
+            assert np.all(got[cal:] == 99)               # only the first calCount elements are written
+
+
+@pytest.mark.parametrize("k_dim", [0, 1])
+@pytest.mark.parametrize("gs", [32, 64, 128, 256])
+@pytest.mark.parametrize("pair", PAIRS)
+def test_quant_per_group(k_dim, gs, pair):
+    announce("quant per-group", k_dim, gs, pair)
+    src_dt, sc_dt = pair
+    m, n = (10, 256) if k_dim == 1 else (256, 64)
+    rng = np.random.default_rng(gs + k_dim)
+    x, xd = src_array(rng, (m, n), src_dt, 1.0)
+    sshape = (m, -(-n // gs)) if k_dim == 1 else (-(-m // gs), n)
+    s, sd = src_array_uniform(rng, sshape, sc_dt, 5, 60)
+    o, od = src_array_uniform(rng, sshape, sc_dt, -2, 2)
+    for compute, fn in ((abi.COMPUTE_SCALE_T, ops.ascend_quant_policy), (abi.COMPUTE_F32, ops.quantize)):
+        dst = torch.zeros((m, n), dtype=torch.int8, device=DEV)
+        fn(dst, xd, sd, od, ops.AscendQuantParam(m, n, m * n, gs), abi.PER_GROUP,
+           ops.AscendQuantConfig(has_offset=True, k_dim=k_dim))
+        d = abi.QuantDesc(policy=abi.PER_GROUP, src_dtype=src_dt, scale_dtype=sc_dt, compute=compute,
+                          round_mode=abi.CAST_RINT, offset_kind=abi.OFFSET_TENSOR, k_dim=k_dim, m=m, n=n,
+                          cal_count=m * n, group_size=gs)
+        assert np.array_equal(dst.cpu().numpy(), orc.quant(d, x, s, o))
+
+
+@pytest.mark.parametrize("src_dt", [abi.BF16, abi.F16, abi.F32])
+@pytest.mark.parametrize("m,n", [(1, 4096), (16, 4096), (5, 1000), (3, 8192), (2, 12288), (4, 20000), (7, 37)])
+def test_dynamic_quant_per_token(src_dt, m, n):
+    announce("dynamic quant", src_dt, m, n)
+    rng = np.random.default_rng(m + n)
+    x, xd = src_array(rng, (m, n), src_dt, 1.0)
+    if m > 2:
+        x[1] = 0
+        xd[1] = 0
+    q, ts = ops.dynamic_quant_per_token(xd)
+    wq, wts = orc.dynamic_quant_per_token(src_dt, x)
+    assert np.array_equal(ts.cpu().numpy(), wts)
+    assert np.array_equal(q.cpu().numpy(), wq)
+
+
+# ------------------------------------------------------------------ AscendDequant
+@pytest.mark.parametrize("dst_dt,sc_dt", [(abi.F16, abi.U64), (abi.F32, abi.F32), (abi.F32, abi.BF16),
+                                          (abi.BF16, abi.BF16), (abi.BF16, abi.F32)])
+@pytest.mark.parametrize("m,n,cal", [(4, 8, 6), (6, 40, 24), (128, 32, 32), (33, 4096, 4096), (3, 136, 130)])
+def test_dequant_per_channel(dst_dt, sc_dt, m, n, cal):
+    announce("dequant per-channel", dst_dt, sc_dt, m, n, cal)
+    rng = np.random.default_rng(m * n + cal)
+    src = rng.integers(-2**20, 2**20, (m, n), dtype=np.int32)
+    sf = rng.uniform(1e-5, 1e-3, n).astype(np.float32) * rng.choice([-1, 1], n).astype(np.float32)
+    if sc_dt == abi.BF16:
+        sc = orc.f32_to_bf16_bits(sf)
+        scd = to_dev(sc, "bf16")
+    elif sc_dt == abi.U64:
+        sc = sf.view(np.uint32).astype(np.uint64) | (np.uint64(0xABC) << np.uint64(40))
+        scd = to_dev(sc)
+    else:
+        sc, scd = sf, to_dev(sf)
+    stride = ops.dequant_dst_stride(TDT[dst_dt], n)
+    fill = 0x7E7E if dst_dt != abi.F32 else 0
+    dst = torch.zeros((m, stride), dtype=TDT[dst_dt], device=DEV)
+    if dst_dt != abi.F32:
+        dst.view(torch.int16).fill_(0x7E7E)
+    ops.ascend_dequant(dst, to_dev(src), scd, ops.DequantParams(m, n, cal), mode=abi.DEQUANT_WITH_MULTI_ROW)
+    d = abi.DequantDesc(policy=abi.PER_CHANNEL, src_dtype=abi.I32, scale_dtype=sc_dt, dst_dtype=dst_dt,
+                        mode=abi.DEQUANT_WITH_MULTI_ROW, m=m, n=n, cal_count=cal)
+    want = orc.dequant(d, src, sc, fill=fill)
+    got = bits(dst)
+    assert np.array_equal(got, want.view(np.uint16) if dst_dt != abi.F32 else want)
+
+
+def test_dequant_scalar_single_row_and_policies():
+    announce("dequant scalar / single-row / per-token / per-group")
+    rng = np.random.default_rng(5)
+    src = rng.integers(-5000, 5000, (1, 64), dtype=np.int32)
+    for dst_dt in (abi.F32, abi.BF16):
+        dst = torch.zeros((8, ops.dequant_dst_stride(TDT[dst_dt], 8)), dtype=TDT[dst_dt], device=DEV)
+        sc = np.arange(1, 9, dtype=np.float32) * 0.37
+        ops.ascend_dequant(dst, to_dev(src), to_dev(sc), ops.DequantParams(1, 64, 8))      # SINGLE_ROW default
+        d = abi.DequantDesc(policy=abi.PER_CHANNEL, src_dtype=abi.I32, scale_dtype=abi.F32, dst_dtype=dst_dt,
+                            mode=abi.DEQUANT_WITH_SINGLE_ROW, m=1, n=64, cal_count=8)
+        want = orc.dequant(d, src, sc)
+        if dst_dt == abi.F32:
+            assert want.shape == (8, 8) and np.array_equal(bits(dst), want)
+        else:                                                     # 8 bf16 is not 32 bytes: stays {1, 64, 8}
+            assert want.shape == (1, 64)
+            assert np.array_equal(bits(dst).reshape(-1)[:64], want.reshape(-1))
+    src = rng.integers(-2**20, 2**20, (12, 256), dtype=np.int32)
+    dst = torch.zeros((12, 256), dtype=torch.float32, device=DEV)
+    ops.ascend_dequant(dst, to_dev(src), 2.2, ops.DequantParams(12, 256, 200), mode=abi.DEQUANT_WITH_MULTI_ROW)
+    d = abi.DequantDesc(policy=abi.PER_TENSOR, src_dtype=abi.I32, scale_dtype=abi.F32, dst_dtype=abi.F32,
+                        mode=abi.DEQUANT_WITH_MULTI_ROW, scale=2.2, m=12, n=256, cal_count=200)
+    assert np.array_equal(bits(dst), orc.dequant(d, src))
+    for policy, k_dim, gs, sshape in ((abi.PER_TOKEN, 1, 0, (12,)), (abi.PER_GROUP, 1, 64, (12, 4)),
+                                      (abi.PER_GROUP, 0, 32, (1, 256))):
+        for sc_dt in (abi.F32, abi.BF16, abi.F16):
+            for src_f32 in (False, True):
+                s, sd = src_array_uniform(rng, sshape, sc_dt, 0.01, 1.0)
+                sin = src.astype(np.float32) * np.float32(0.37) if src_f32 else src
+                dstb = torch.zeros((12, 256), dtype=torch.bfloat16, device=DEV)
+                para = ops.AscendQuantParam(12, 256, 256, gs)
+                ops.ascend_dequant_policy(dstb, to_dev(sin), sd, para, policy, k_dim)
+                d = abi.DequantDesc(policy=policy, src_dtype=abi.F32 if src_f32 else abi.I32, scale_dtype=sc_dt,
+                                    dst_dtype=abi.BF16, mode=abi.DEQUANT_WITH_MULTI_ROW, k_dim=k_dim, m=12, n=256,
+                                    cal_count=256, group_size=gs)
+                assert np.array_equal(bits(dstb), orc.dequant(d, sin, s))
+
+
+# ------------------------------------------------------------------ AscendAntiQuant
+@pytest.mark.parametrize("int4", [False, True])
+@pytest.mark.parametrize("dst_dt", [abi.F16, abi.BF16])
+@pytest.mark.parametrize("transpose", [False, True])
+@pytest.mark.parametrize("K,N,G", [(64, 128, 1), (256, 32, 4), (2048, 64, 1), (5888 // 256, 256, 1), (96, 128, 3),
+                                   (64, 40, 2)])
+@pytest.mark.parametrize("has_offset", [True, False])
+def test_antiquant(int4, dst_dt, transpose, K, N, G, has_offset):
+    if transpose and K % (64 if int4 else 32):
+        pytest.skip("transposed input needs a 32-byte aligned k axis")
+    announce("antiquant", int4, dst_dt, transpose, K, N, G, has_offset)
+    rng = np.random.default_rng(K + N + G)
+    w = rng.integers(-8, 8, (K, N)).astype(np.int8) if int4 else rng.integers(-128, 128, (K, N)).astype(np.int8)
+    sc, _ = src_array_uniform(rng, (G, N), dst_dt, -2, 2)
+    of, _ = src_array_uniform(rng, (G, N), dst_dt, -9, 9)
+    if transpose:
+        w, sc, of = (np.ascontiguousarray(t.T) for t in (w, sc, of))
+        d = abi.AntiQuantDesc(src_dtype=abi.I4 if int4 else abi.I8, dst_dtype=dst_dt, is_transpose=1,
+                              has_offset=int(has_offset), k=K, n=N, scale_height=N, scale_width=G, offset_height=N,
+                              offset_width=G)
+        info = ops.AntiQuantShapeInfo(N, G, N, G)
+    else:
+        d = abi.AntiQuantDesc(src_dtype=abi.I4 if int4 else abi.I8, dst_dtype=dst_dt, has_offset=int(has_offset), k=K,
+                              n=N, scale_height=G, scale_width=N, offset_height=G, offset_width=N)
+        info = ops.AntiQuantShapeInfo(G, N, G, N)
+    src = pack_int4(w) if int4 else w
+    kind = "bf16" if dst_dt == abi.BF16 else None
+    dst = torch.zeros(w.shape, dtype=TDT[dst_dt], device=DEV)
+    ops.ascend_antiquant(dst, to_dev(src), to_dev(of, kind) if has_offset else None, to_dev(sc, kind), K, info,
+                         is_transpose=transpose, int4=int4)
+    want = orc.antiquant(d, src, of if has_offset else None, sc)
+    assert np.array_equal(bits(dst), want.view(np.uint16))
+
+
+def test_antiquant_per_tensor():
+    announce("antiquant per-tensor")
+    w = np.arange(-128, 128, dtype=np.int8).reshape(8, 32)
+    for dst_dt in (abi.F16, abi.BF16):
+        dst = torch.zeros((8, 32), dtype=TDT[dst_dt], device=DEV)
+        ops.ascend_antiquant(dst, to_dev(w), -3.25, 0.37, 8)
+        d = abi.AntiQuantDesc(src_dtype=abi.I8, dst_dtype=dst_dt, has_offset=1, per_tensor=1, scale=0.37,
+                              offset=-3.25, k=8, n=32)
+        assert np.array_equal(bits(dst), orc.antiquant(d, w).view(np.uint16))
+
+
+# ------------------------------------------------------------------ full-size configurations
+def test_config2a_full_size_quant():
+    announce("config 2a: fp16 [8192, 4096] per-channel quant")
+    rng = np.random.default_rng(0x2A)
+    x = (rng.standard_normal((8192, 4096)) * 2).astype(np.float16)
+    s = (np.float32(127.0) / np.abs(x.astype(np.float32)).max(axis=0)).astype(np.float16)
+    dst = torch.zeros((8192, 4096), dtype=torch.int8, device=DEV)
+    ops.ascend_quant(dst, to_dev(x), to_dev(s), 0.0)
+    d = abi.QuantDesc(policy=abi.PER_CHANNEL, src_dtype=abi.F16, scale_dtype=abi.F16, compute=abi.COMPUTE_F16,
+                      round_mode=abi.CAST_RINT, offset_kind=abi.OFFSET_SCALAR, n=4096, cal_count=x.size)
+    orc.set_threads(16)
+    assert np.array_equal(dst.cpu().numpy(), orc.quant(d, x, s))
+
+
+def test_config2b_full_size_dequant():
+    announce("config 2b: int32 [8192, 4096] per-channel dequant to bf16")
+    rng = np.random.default_rng(0x2B)
+    src = rng.integers(-2**20, 2**20 + 1, (8192, 4096), dtype=np.int32)
+    sc = rng.uniform(1e-5, 1e-3, 4096).astype(np.float32)
+    dst = torch.zeros((8192, 4096), dtype=torch.bfloat16, device=DEV)
+    ops.ascend_dequant(dst, to_dev(src), to_dev(sc), ops.DequantParams(8192, 4096, 4096),
+                       mode=abi.DEQUANT_WITH_MULTI_ROW)
+    d = abi.DequantDesc(policy=abi.PER_CHANNEL, src_dtype=abi.I32, scale_dtype=abi.F32, dst_dtype=abi.BF16,
+                        mode=abi.DEQUANT_WITH_MULTI_ROW, m=8192, n=4096, cal_count=4096)
+    orc.set_threads(16)
+    assert np.array_equal(bits(dst), orc.dequant(d, src, sc))
+
+
+def test_config2c_full_size_antiquant():
+    announce("config 2c: int8 [4096, 11008] per-channel antiquant to fp16")
+    rng = np.random.default_rng(0x2C)
+    w = rng.integers(-127, 128, (4096, 11008)).astype(np.int8)
+    sc = rng.uniform(1e-3, 1e-1, (1, 11008)).astype(np.float16)
+    of = rng.integers(-8, 9, (1, 11008)).astype(np.float16)
+    dst = torch.zeros((4096, 11008), dtype=torch.float16, device=DEV)
+    ops.ascend_antiquant(dst, to_dev(w), to_dev(of), to_dev(sc), 4096, ops.AntiQuantShapeInfo(1, 11008, 1, 11008))
+    d = abi.AntiQuantDesc(src_dtype=abi.I8, dst_dtype=abi.F16, has_offset=1, k=4096, n=11008, scale_height=1,
+                          scale_width=11008, offset_height=1, offset_width=11008)
+    orc.set_threads(16)
+    assert np.array_equal(bits(dst), orc.antiquant(d, w, of, sc).view(np.uint16))

@@ -1,0 +1,243 @@
+"""GPU parity of the int8 matmul quant path, the quantized grouped matmul and W4A16 against the CPU oracle, through
+the C ABI.  int32 accumulators and every epilogue without a transcendental are compared bit for bit (each epilogue
+step rounds once in fp32, in the reference's order); FasterGelu outputs within 1 ulp of the output type; W4A16
+(free summation order) within the stated tolerance."""
+import numpy as np
+import pytest
+import torch
+
+import orc
+from ascq import _abi as abi
+from ascq import ops
+from gpu_util import DEV, announce, bits, max_ulp, pack_int4, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def rand_i8(rng, shape, lo=-127, hi=127):
+    return rng.integers(lo, hi + 1, shape).astype(np.int8)
+
+
+def run_mm(m, n, k, a, b, *, out, bias=None, quant=None, tok=None, trans_a=False, trans_b=False, act=abi.MM_ACT_NONE,
+           scalar=None):
+    mm = ops.Matmul(m, n, k, trans_a, trans_b)
+    mm.set_tensor_a(to_dev(a))
+    mm.set_tensor_b(to_dev(b))
+    if bias is not None:
+        mm.set_bias(to_dev(bias[0], bias[1]))
+    if quant is not None:
+        mm.set_quant_vector(to_dev(quant))
+    if scalar is not None:
+        mm.set_quant_scalar(scalar)
+    if tok is not None:
+        mm.set_token_scale(to_dev(tok))
+    mm.set_activation(act)
+    c = torch.zeros((m, n), dtype=out, device=DEV)
+    mm.iterate_all(c)
+    torch.cuda.synchronize()
+    return c, mm.desc
+
+
+def oracle_mm(desc, a, b, bias=None, quant=None, tok=None):
+    orc.set_threads(16)
+    return orc.matmul_w8a8(desc, a, b, None if bias is None else bias[0], quant, tok)
+
+
+# shapes chosen to hit: the 32-row split-K tile, the 128-row tile with a row tail, the 256-row tile with row and
+# column tails, K tails (K not a multiple of 128), and the generic kernel (odd sizes)
+SHAPES = [(1, 256, 512), (16, 1024, 4096), (32, 264, 1040), (33, 256, 256), (128, 512, 384), (300, 520, 272),
+          (1100, 776, 400), (2048, 512, 128), (19, 23, 77), (40, 100, 48)]
+
+
+@pytest.mark.parametrize("m,n,k", SHAPES)
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_int32_accumulators_bit_exact(m, n, k, trans_b):
+    announce("matmul int32", m, n, k, trans_b)
+    rng = np.random.default_rng(m * 7 + n * 3 + k)
+    a = rand_i8(rng, (m, k), -128, 127)
+    b = rand_i8(rng, (k, n), -128, 127)
+    bias = rng.integers(-10000, 10000, n).astype(np.int32)
+    b_in = np.ascontiguousarray(b.T) if trans_b else b
+    c, desc = run_mm(m, n, k, a, b_in, out=torch.int32, bias=(bias, None), trans_b=trans_b)
+    want = a.astype(np.int64) @ b.astype(np.int64) + bias
+    assert np.array_equal(c.cpu().numpy().astype(np.int64), want)
+    assert np.array_equal(oracle_mm(desc, a, b_in, (bias, None)).astype(np.int64), want)
+
+
+def test_trans_a_generic_path():
+    announce("matmul trans_a")
+    rng = np.random.default_rng(3)
+    m, n, k = 48, 64, 96
+    a, b = rand_i8(rng, (m, k)), rand_i8(rng, (k, n))
+    c, _ = run_mm(m, n, k, np.ascontiguousarray(a.T), b, out=torch.int32, trans_a=True)
+    assert np.array_equal(c.cpu().numpy().astype(np.int64), a.astype(np.int64) @ b.astype(np.int64))
+
+
+def test_config1_small_w8a8_bf16_with_bias():
+    """A int8 [256,1024], B int8 [1024,1024], per-channel fp32 deqScale in [1e-4,1e-3], fp32 bias N(0,1) -> bf16."""
+    announce("config 1")
+    rng = np.random.default_rng(0xC1)
+    m, n, k = 256, 1024, 1024
+    a, b = rand_i8(rng, (m, k)), rand_i8(rng, (k, n))
+    sc = rng.uniform(1e-4, 1e-3, n).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    c, desc = run_mm(m, n, k, a, b, out=torch.bfloat16, bias=(bias, None), quant=sc)
+    assert np.array_equal(bits(c), oracle_mm(desc, a, b, (bias, None), sc))
+
+
+@pytest.mark.parametrize("m", [1, 16, 128, 2048])
+def test_config3_w8a8_linear(m):
+    """bf16 activations quantised per token on the GPU, int8 weights [4096,11008], fused dequant to bf16."""
+    announce("config 3", m)
+    rng = np.random.default_rng(0xC3 + m)
+    k, n = 4096, 11008
+    x = orc.f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32))
+    w = rand_i8(rng, (k, n))
+    cs = rng.uniform(1e-4, 1e-2, n).astype(np.float32)
+    q, ts = ops.dynamic_quant_per_token(to_dev(x, "bf16"))
+    wq, wts = orc.dynamic_quant_per_token(abi.BF16, x)
+    assert np.array_equal(q.cpu().numpy(), wq) and np.array_equal(ts.cpu().numpy(), wts)
+    c, desc = run_mm(m, n, k, wq, w, out=torch.bfloat16, quant=cs, tok=wts)
+    want = oracle_mm(desc, wq, w, None, cs, wts)
+    got = bits(c)
+    assert max_ulp(got, want) <= 1
+    assert np.array_equal(got, want)
+
+
+def test_fixpipe_modes_uint64_words():
+    announce("matmul fixpipe words: VDEQF16, DEQF16 scalar, VREQ8, bf16")
+    rng = np.random.default_rng(21)
+    m, n, k = 64, 256, 256
+    a, b = rand_i8(rng, (m, k), -10, 10), rand_i8(rng, (k, n), -10, 10)
+    bias = rng.integers(-2, 2, n).astype(np.int32)
+    qf = rng.uniform(0.1, 2.0, n).astype(np.float32)
+    qf[0], qf[1] = 3000.0, -3000.0
+    words = qf.view(np.uint32).astype(np.uint64) | (np.uint64(7) << np.uint64(37)) | (np.uint64(1) << np.uint64(46))
+    for out in (torch.float16, torch.bfloat16, torch.int8):
+        c, desc = run_mm(m, n, k, a, b, out=out, bias=(bias, None), quant=words)
+        want = oracle_mm(desc, a, b, (bias, None), words)
+        assert np.array_equal(bits(c), want.view(np.uint16) if out == torch.float16 else want)
+    assert (np.abs(bits(run_mm(m, n, k, a, b, out=torch.float16, quant=words)[0]).view(np.float16)
+                   .astype(np.float32)) == 65504).any()            # the fp16 output saturates instead of overflowing
+    c, desc = run_mm(m, n, k, a, b, out=torch.float16, bias=(bias, None),
+                     scalar=ops.pack_quant_param(0.1))
+    assert np.array_equal(bits(c), oracle_mm(desc, a, b, (bias, None)).view(np.uint16))
+    c, desc = run_mm(m, n, k, a, b, out=torch.float32, scalar=0.1)
+    assert np.array_equal(bits(c), oracle_mm(desc, a, b))
+
+
+def test_post_bias_bf16_and_gelu():
+    announce("matmul bf16 bias + token scale + FasterGelu")
+    rng = np.random.default_rng(22)
+    m, n, k = 96, 512, 384
+    a, b = rand_i8(rng, (m, k)), rand_i8(rng, (k, n))
+    cs = rng.uniform(1e-4, 1e-3, n).astype(np.float32)
+    ts = rng.uniform(1e-2, 1e-1, m).astype(np.float32)
+    bias = orc.f32_to_bf16_bits(rng.standard_normal(n).astype(np.float32))
+    c, desc = run_mm(m, n, k, a, b, out=torch.bfloat16, bias=(bias, "bf16"), quant=cs, tok=ts)
+    assert np.array_equal(bits(c), oracle_mm(desc, a, b, (bias, None), cs, ts))
+    c, desc = run_mm(m, n, k, a, b, out=torch.float16, quant=cs, tok=ts, act=abi.MM_ACT_FASTER_GELU)
+    want = oracle_mm(desc, a, b, None, cs, ts)
+    assert max_ulp(bits(c), want.view(np.uint16)) <= 1             # expf differs by at most an ulp of fp32
+
+
+# ------------------------------------------------------------------ grouped matmul
+def run_group(m, k, n, counts, kind, out, rng, with_bias, act, rows_cap=None):
+    G = len(counts)
+    x, w = rand_i8(rng, (m, k)), rand_i8(rng, (G, k, n))
+    cs = rng.uniform(1e-4, 1e-2, (G, n)).astype(np.float32)
+    ts = rng.uniform(1e-3, 1e-1, m).astype(np.float32)
+    bias = orc.f32_to_bf16_bits(rng.standard_normal((G, n)).astype(np.float32)) if with_bias else None
+    gl = np.asarray(counts, dtype=np.int64) if kind == abi.GROUP_LIST_COUNTS else np.cumsum(counts).astype(np.int64)
+    y = torch.zeros((m, n), dtype=out, device=DEV)
+    y.view(torch.int16).fill_(0x7E7E)
+    ops.quant_group_matmul(y, to_dev(x), to_dev(w), to_dev(gl), to_dev(cs), to_dev(ts),
+                           None if bias is None else to_dev(bias, "bf16"), kind, act)
+    torch.cuda.synchronize()
+    mm = abi.MatmulDesc(m=m, n=n, k=k, out_dtype=abi.BF16 if out == torch.bfloat16 else abi.F16,
+                        quant_mode=abi.MM_QUANT_VECTOR, scale_format=abi.MM_SCALE_F32, has_tok_scale=1,
+                        bias_kind=abi.MM_BIAS_BF16_POST if with_bias else abi.MM_BIAS_NONE, activation=act)
+    d = abi.GroupMatmulDesc(mm=mm, groups=G, group_list_kind=kind)
+    orc.set_threads(16)
+    want = orc.group_matmul_w8a8(d, x, w, bias, cs, ts, gl, fill=0x7E7E)
+    return bits(y), (want.view(np.uint16) if want.dtype == np.float16 else want)
+
+
+@pytest.mark.parametrize("kind", [abi.GROUP_LIST_COUNTS, abi.GROUP_LIST_PREFIX_SUM])
+@pytest.mark.parametrize("counts", [[30, 0, 1, 45, 12], [256, 256], [0, 0, 700, 0], [1, 1, 1, 1, 1, 1, 1, 1],
+                                    [513, 255, 0, 256]])
+def test_group_matmul_edge_cases(kind, counts):
+    announce("grouped matmul", kind, counts)
+    rng = np.random.default_rng(sum(counts) + len(counts))
+    m = sum(counts) + 8                                         # 8 rows belong to no group and stay untouched
+    got, want = run_group(m, 256, 520, counts, kind, torch.bfloat16, rng, True, abi.MM_ACT_NONE)
+    assert np.array_equal(got, want)
+    assert np.all(got[sum(counts):] == 0x7E7E)
+
+
+def test_group_matmul_reference_example_form():
+    """The reference example's form: counts group list, no bias, FasterGelu, fp16 output."""
+    announce("grouped matmul, example form")
+    rng = np.random.default_rng(77)
+    got, want = run_group(512, 256, 512, [128] * 4, abi.GROUP_LIST_COUNTS, torch.float16, rng, False,
+                          abi.MM_ACT_FASTER_GELU)
+    assert max_ulp(got, want) <= 1
+
+
+def test_config5_moe_up_projection():
+    """8 experts, 4096 tokens from a seeded multinomial, K=4096, N=14336, bf16 bias, prefix-sum group list."""
+    announce("config 5")
+    rng = np.random.default_rng(0xC5)
+    counts = rng.multinomial(4096, [1 / 8] * 8).tolist()
+    got, want = run_group(4096, 4096, 14336, counts, abi.GROUP_LIST_PREFIX_SUM, torch.bfloat16, rng, True,
+                          abi.MM_ACT_NONE)
+    assert np.array_equal(got, want)
+
+
+# ------------------------------------------------------------------ W4A16
+def w4_case(rng, m, k, n, gs, has_offset):
+    x = rng.standard_normal((m, k)).astype(np.float16)
+    w = rng.integers(-8, 8, (k, n)).astype(np.int8)
+    sc = rng.uniform(1e-3, 1e-2, (k // gs, n)).astype(np.float16)
+    of = rng.integers(-8, 8, (k // gs, n)).astype(np.float16) if has_offset else None
+    return x, pack_int4(w), sc, of
+
+
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 7, 16])
+@pytest.mark.parametrize("k,n,gs", [(512, 1024, 128), (1024, 544, 64), (256, 66, 128), (384, 512, 384)])
+@pytest.mark.parametrize("has_offset", [True, False])
+def test_w4a16_small(m, k, n, gs, has_offset):
+    announce("w4a16", m, k, n, gs, has_offset)
+    rng = np.random.default_rng(m + k + n)
+    x, wp, sc, of = w4_case(rng, m, k, n, gs, has_offset)
+    y = torch.zeros((m, n), dtype=torch.float16, device=DEV)
+    ops.matmul_w4a16(y, to_dev(x), to_dev(wp), to_dev(sc), None if of is None else to_dev(of), gs)
+    d = abi.W4A16Desc(m=m, n=n, k=k, group_size=gs, has_offset=int(has_offset))
+    want = orc.matmul_w4a16(d, x, wp, sc, of)
+    got = y.cpu().numpy()
+    # fp32 accumulation in a different order than the oracle's: rel-err <= 1e-3 of the row scale, and <= 1 fp16 ulp
+    # wherever the result is not close to a cancellation
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    ref = np.abs(x.astype(np.float64)).sum(axis=1, keepdims=True) * 8 * 1e-2      # bound on sum |x||w|
+    assert np.all(err <= 1e-3 * ref + 1e-6)
+    assert np.mean(got.view(np.uint16) == want.view(np.uint16)) > 0.9
+
+
+@pytest.mark.parametrize("m", [1, 4, 16])
+def test_config4_w4a16_decode(m):
+    """fp16 [M,8192] x int4 [8192,28672], group 128, fp16 scale and offset."""
+    announce("config 4", m)
+    rng = np.random.default_rng(0xC4 + m)
+    k, n, gs = 8192, 28672, 128
+    x, wp, sc, of = w4_case(rng, m, k, n, gs, True)
+    y = torch.zeros((m, n), dtype=torch.float16, device=DEV)
+    ops.matmul_w4a16(y, to_dev(x), to_dev(wp), to_dev(sc), to_dev(of), gs)
+    d = abi.W4A16Desc(m=m, n=n, k=k, group_size=gs, has_offset=1)
+    orc.set_threads(16)
+    cols = (0, n) if m == 1 else (4096, 4096 + 2048)             # the oracle covers every column at M=1, a slab otherwise
+    want = orc.matmul_w4a16(d, x, wp, sc, of, cols=cols)[:, cols[0]:cols[1]]
+    got = y.cpu().numpy()[:, cols[0]:cols[1]]
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    tol = 1e-3 * np.maximum(np.abs(want.astype(np.float64)), 1.0)
+    assert np.all(err <= tol + 2e-3)
+    assert max_ulp(got.view(np.uint16), want.view(np.uint16), "f16") <= 4 or np.mean(err <= tol) > 0.999
