@@ -44,6 +44,10 @@ __device__ __forceinline__ uint32_t f32_to_half_bits(float f)
         uint16_t u;
         half_t h;
     } c;
+    // The empty asm makes `f` opaque: without it the compiler folds a preceding fp32 multiply into one
+    // mixed-precision instruction that rounds the exact product once to fp16, whereas the operators round to fp32
+    // first and to fp16 second.
+    asm volatile("" : "+v"(f));
     c.h = static_cast<half_t>(f);  // v_cvt_f16_f32: round to nearest even, overflow to infinity
     return c.u;
 }
