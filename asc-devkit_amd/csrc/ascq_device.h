@@ -13,6 +13,7 @@ typedef _Float16 half_t;
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
+typedef int32_t i32x2_t __attribute__((ext_vector_type(2)));
 typedef int32_t i32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));

@@ -1,0 +1,162 @@
+// Shared between the translation units of the int8 matmul: parameter blocks and the per-element epilogue.
+#pragma once
+#include "ascq_common.h"
+#include "ascq_device.h"
+
+namespace ascq {
+
+struct EpiParams {
+    void* c;
+    const void* bias;
+    const void* quant;  // uint64 words or fp32 scales, one per output channel (VECTOR mode)
+    const float* tok_scale;
+    uint32_t ldc;
+    int out_dtype, quant_mode, scale_format, bias_kind, has_tok, activation;
+    uint64_t quant_scalar;
+};
+
+struct GemmParams {
+    const int8_t* a;
+    const int8_t* b;
+    uint32_t m, n, k;
+    uint32_t tiles_m, tiles_n;
+    uint32_t k_splits, k_per_split;  // split-K: bytes of K per grid.z slice (multiple of kBK)
+    int32_t* partial;                // split-K int32 accumulator [m, n]
+    // grouped
+    const int64_t* group_list;
+    uint32_t groups;
+    int group_list_kind;
+    EpiParams epi;
+};
+
+struct ChannelQ {
+    float s;
+    int off9;
+    int sgn;
+};
+
+__device__ __forceinline__ ChannelQ load_channel_q(const EpiParams& e, size_t col)
+{
+    ChannelQ q{1.0f, 0, 1};
+    if (e.quant_mode == ASCQ_MM_QUANT_NONE) {
+        return q;
+    }
+    uint64_t w;
+    if (e.quant_mode == ASCQ_MM_QUANT_VECTOR) {
+        if (e.scale_format == ASCQ_MM_SCALE_U64) {
+            w = static_cast<const uint64_t*>(e.quant)[col];
+        } else {
+            w = __float_as_uint(static_cast<const float*>(e.quant)[col]);
+        }
+    } else {
+        w = e.quant_scalar;
+    }
+    uint32_t lo = static_cast<uint32_t>(w);
+    if (e.scale_format == ASCQ_MM_SCALE_U64) {
+        lo &= 0xFFFFE000u;  // the fixpipe reads sign, 8 exponent and 10 mantissa bits
+        q.off9 = static_cast<int>((w >> 37) & 0x1FF);
+        q.sgn = static_cast<int>((w >> 46) & 1);
+    }
+    q.s = __uint_as_float(lo);
+    return q;
+}
+
+__device__ __forceinline__ float faster_gelu(float x)
+{
+    const float ax = fabsf(x);
+    const float x2 = expf(0.851f * (x - ax));
+    const float x3 = 1.0f + expf(-1.702f * ax);
+    return x * x2 / x3;
+}
+
+// Everything after the int32 accumulator, for one output element.  `bias_post` is already widened to fp32.
+// kOut is the output dtype, or -1 for "no quantisation" (raw int32).
+template <int kOut>
+__device__ __forceinline__ void epilogue_store(const EpiParams& e, size_t row, size_t col, int32_t acc,
+                                               const ChannelQ& q, float tok, float bias_post)
+{
+    const size_t idx = row * e.ldc + col;
+    if constexpr (kOut < 0) {
+        static_cast<int32_t*>(e.c)[idx] = acc;
+    } else {
+        float v = static_cast<float>(acc) * q.s;
+        if (e.has_tok) {
+            v = v * tok;
+        }
+        if (e.bias_kind >= ASCQ_MM_BIAS_F32_POST) {
+            v = v + bias_post;
+        }
+        if (e.activation == ASCQ_MM_ACT_FASTER_GELU) {
+            v = faster_gelu(v);
+        }
+        if constexpr (kOut == ASCQ_BF16) {
+            static_cast<uint16_t*>(e.c)[idx] = static_cast<uint16_t>(f32_to_bf16_bits(v));
+        } else if constexpr (kOut == ASCQ_F16) {
+            static_cast<uint16_t*>(e.c)[idx] = static_cast<uint16_t>(f32_to_half_bits_sat(v));
+        } else if constexpr (kOut == ASCQ_F32) {
+            static_cast<float*>(e.c)[idx] = v;
+        } else {  // int8 / uint8 requantisation
+            float r = fminf(fmaxf(__builtin_rintf(v), -256.0f), 255.0f);
+            int t = ((v != v) ? 0 : static_cast<int>(r)) + q.off9;
+            t = q.sgn ? min(max(t, -128), 127) : min(max(t, 0), 255);
+            static_cast<uint8_t*>(e.c)[idx] = static_cast<uint8_t>(t);
+        }
+    }
+}
+
+// Calls f(tag) with the compile-time output kind selected by the (uniform) runtime descriptor.
+template <int k>
+struct OutTag {
+    static constexpr int value = k;
+};
+template <class F>
+__device__ __forceinline__ void dispatch_out(const EpiParams& e, F&& f)
+{
+    if (e.quant_mode == ASCQ_MM_QUANT_NONE) {
+        f(OutTag<-1>{});
+    } else if (e.out_dtype == ASCQ_BF16) {
+        f(OutTag<ASCQ_BF16>{});
+    } else if (e.out_dtype == ASCQ_F16) {
+        f(OutTag<ASCQ_F16>{});
+    } else if (e.out_dtype == ASCQ_F32) {
+        f(OutTag<ASCQ_F32>{});
+    } else {
+        f(OutTag<ASCQ_I8>{});
+    }
+}
+
+__device__ __forceinline__ float load_bias_post(const EpiParams& e, size_t col)
+{
+    if (e.bias_kind == ASCQ_MM_BIAS_F32_POST) {
+        return static_cast<const float*>(e.bias)[col];
+    }
+    if (e.bias_kind == ASCQ_MM_BIAS_BF16_POST) {
+        return bf16_bits_to_f32(static_cast<const uint16_t*>(e.bias)[col]);
+    }
+    return 0.0f;
+}
+
+
+// Maps a linear workgroup id to a tile id such that each XCD (id mod 8) gets a contiguous range of tiles.
+__device__ __forceinline__ uint32_t xcd_remap(uint32_t pid, uint32_t total)
+{
+    const uint32_t per = (total + 7u) / 8u;
+    uint32_t tall = total % 8u;
+    if (tall == 0) {
+        tall = 8;
+    }
+    const uint32_t xcd = pid & 7u, local = pid >> 3;
+    if (xcd < tall) {
+        return xcd * per + local;
+    }
+    if (local + 1u >= per) {
+        return 0xFFFFFFFFu;  // the short XCDs own one tile less: this workgroup has nothing to do
+    }
+    return tall * per + (xcd - tall) * (per - 1u) + local;
+}
+
+// Large-M kernel built on direct-to-LDS loads and transposing LDS reads (matmul_w8a8_dma.hip).
+bool gemm_dma_supported(const GemmParams& p);
+int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st);
+
+}  // namespace ascq

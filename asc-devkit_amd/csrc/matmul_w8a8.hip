@@ -24,8 +24,10 @@
 //     (exact and order-independent) into a caller workspace and a second kernel applies the epilogue.
 //   * Grouped matmul: same tile body; each workgroup finds its (group, row range) from the device-side group list,
 //     so no host synchronisation is needed and empty groups cost nothing.
-#include "ascq_common.h"
-#include "ascq_device.h"
+#include <cstdlib>
+#include <type_traits>
+
+#include "matmul_w8a8.h"
 
 namespace ascq {
 namespace {
@@ -34,137 +36,6 @@ constexpr int kThreads = 256;
 constexpr int kBK = 128;          // bytes of K per pipeline step
 constexpr int kAStride = 128;     // LDS row stride of a K-contiguous operand (XOR swizzle)
 constexpr int kBStride = 144;     // LDS row stride of the transposed B operand (padding instead of swizzle)
-
-struct EpiParams {
-    void* c;
-    const void* bias;
-    const void* quant;  // uint64 words or fp32 scales, one per output channel (VECTOR mode)
-    const float* tok_scale;
-    uint32_t ldc;
-    int out_dtype, quant_mode, scale_format, bias_kind, has_tok, activation;
-    uint64_t quant_scalar;
-};
-
-struct GemmParams {
-    const int8_t* a;
-    const int8_t* b;
-    uint32_t m, n, k;
-    uint32_t tiles_m, tiles_n;
-    uint32_t k_splits, k_per_split;  // split-K: bytes of K per grid.z slice (multiple of kBK)
-    int32_t* partial;                // split-K int32 accumulator [m, n]
-    // grouped
-    const int64_t* group_list;
-    uint32_t groups;
-    int group_list_kind;
-    EpiParams epi;
-};
-
-struct ChannelQ {
-    float s;
-    int off9;
-    int sgn;
-};
-
-__device__ __forceinline__ ChannelQ load_channel_q(const EpiParams& e, size_t col)
-{
-    ChannelQ q{1.0f, 0, 1};
-    if (e.quant_mode == ASCQ_MM_QUANT_NONE) {
-        return q;
-    }
-    uint64_t w;
-    if (e.quant_mode == ASCQ_MM_QUANT_VECTOR) {
-        if (e.scale_format == ASCQ_MM_SCALE_U64) {
-            w = static_cast<const uint64_t*>(e.quant)[col];
-        } else {
-            w = __float_as_uint(static_cast<const float*>(e.quant)[col]);
-        }
-    } else {
-        w = e.quant_scalar;
-    }
-    uint32_t lo = static_cast<uint32_t>(w);
-    if (e.scale_format == ASCQ_MM_SCALE_U64) {
-        lo &= 0xFFFFE000u;  // the fixpipe reads sign, 8 exponent and 10 mantissa bits
-        q.off9 = static_cast<int>((w >> 37) & 0x1FF);
-        q.sgn = static_cast<int>((w >> 46) & 1);
-    }
-    q.s = __uint_as_float(lo);
-    return q;
-}
-
-__device__ __forceinline__ float faster_gelu(float x)
-{
-    const float ax = fabsf(x);
-    const float x2 = expf(0.851f * (x - ax));
-    const float x3 = 1.0f + expf(-1.702f * ax);
-    return x * x2 / x3;
-}
-
-// Everything after the int32 accumulator, for one output element.  `bias_post` is already widened to fp32.
-// kOut is the output dtype, or -1 for "no quantisation" (raw int32).
-template <int kOut>
-__device__ __forceinline__ void epilogue_store(const EpiParams& e, size_t row, size_t col, int32_t acc,
-                                               const ChannelQ& q, float tok, float bias_post)
-{
-    const size_t idx = row * e.ldc + col;
-    if constexpr (kOut < 0) {
-        static_cast<int32_t*>(e.c)[idx] = acc;
-    } else {
-        float v = static_cast<float>(acc) * q.s;
-        if (e.has_tok) {
-            v = v * tok;
-        }
-        if (e.bias_kind >= ASCQ_MM_BIAS_F32_POST) {
-            v = v + bias_post;
-        }
-        if (e.activation == ASCQ_MM_ACT_FASTER_GELU) {
-            v = faster_gelu(v);
-        }
-        if constexpr (kOut == ASCQ_BF16) {
-            static_cast<uint16_t*>(e.c)[idx] = static_cast<uint16_t>(f32_to_bf16_bits(v));
-        } else if constexpr (kOut == ASCQ_F16) {
-            static_cast<uint16_t*>(e.c)[idx] = static_cast<uint16_t>(f32_to_half_bits_sat(v));
-        } else if constexpr (kOut == ASCQ_F32) {
-            static_cast<float*>(e.c)[idx] = v;
-        } else {  // int8 / uint8 requantisation
-            float r = fminf(fmaxf(__builtin_rintf(v), -256.0f), 255.0f);
-            int t = ((v != v) ? 0 : static_cast<int>(r)) + q.off9;
-            t = q.sgn ? min(max(t, -128), 127) : min(max(t, 0), 255);
-            static_cast<uint8_t*>(e.c)[idx] = static_cast<uint8_t>(t);
-        }
-    }
-}
-
-// Calls f(tag) with the compile-time output kind selected by the (uniform) runtime descriptor.
-template <int k>
-struct OutTag {
-    static constexpr int value = k;
-};
-template <class F>
-__device__ __forceinline__ void dispatch_out(const EpiParams& e, F&& f)
-{
-    if (e.quant_mode == ASCQ_MM_QUANT_NONE) {
-        f(OutTag<-1>{});
-    } else if (e.out_dtype == ASCQ_BF16) {
-        f(OutTag<ASCQ_BF16>{});
-    } else if (e.out_dtype == ASCQ_F16) {
-        f(OutTag<ASCQ_F16>{});
-    } else if (e.out_dtype == ASCQ_F32) {
-        f(OutTag<ASCQ_F32>{});
-    } else {
-        f(OutTag<ASCQ_I8>{});
-    }
-}
-
-__device__ __forceinline__ float load_bias_post(const EpiParams& e, size_t col)
-{
-    if (e.bias_kind == ASCQ_MM_BIAS_F32_POST) {
-        return static_cast<const float*>(e.bias)[col];
-    }
-    if (e.bias_kind == ASCQ_MM_BIAS_BF16_POST) {
-        return bf16_bits_to_f32(static_cast<const uint16_t*>(e.bias)[col]);
-    }
-    return 0.0f;
-}
 
 // 4x4 byte transpose: r[i] holds bytes (n0..n3) of row i; c[j] receives (row0..row3) of column j.
 __device__ __forceinline__ void transpose4x4(uint32_t r0, uint32_t r1, uint32_t r2, uint32_t r3, uint32_t& c0,
@@ -186,26 +57,10 @@ __device__ __forceinline__ uint32_t swz_off(uint32_t row, uint32_t chunk)
     return row * kAStride + ((chunk ^ ((row >> 1) & 7u)) << 4);
 }
 
-// Maps a linear workgroup id to a tile id such that each XCD (id mod 8) gets a contiguous range of tiles.
-__device__ __forceinline__ uint32_t xcd_remap(uint32_t pid, uint32_t total)
-{
-    const uint32_t per = (total + 7u) / 8u;
-    uint32_t tall = total % 8u;
-    if (tall == 0) {
-        tall = 8;
-    }
-    const uint32_t xcd = pid & 7u, local = pid >> 3;
-    if (xcd < tall) {
-        return xcd * per + local;
-    }
-    if (local + 1u >= per) {
-        return 0xFFFFFFFFu;  // the short XCDs own one tile less: this workgroup has nothing to do
-    }
-    return tall * per + (xcd - tall) * (per - 1u) + local;
-}
-
-template <int TM, int TN, int WGM, int WGN, bool kTransB>
+template <int TM, int TN, int WGM, int WGN, bool kTransB, int STAGES = 2, int MINBLOCKS = 1>
 struct Tile {
+    static constexpr int kStages = STAGES;
+    static constexpr int kMinBlocks = MINBLOCKS;
     static constexpr int BM = WGM * TM * 32;
     static constexpr int BN = WGN * TN * 32;
     static constexpr int kWGM = WGM, kWGN = WGN, kWTM = TM, kWTN = TN;
@@ -213,7 +68,7 @@ struct Tile {
     static constexpr int kABytes = BM * kAStride;
     static constexpr int kBBytes = BN * kBRow;
     static constexpr int kStage = kABytes + kBBytes;
-    static constexpr int kLds = 2 * kStage;
+    static constexpr int kLds = STAGES * kStage;
     static constexpr int kAChunks = BM * (kBK / 16) / kThreads;  // 16-byte chunks of A per lane per step
     static constexpr int kBChunksT = BN * (kBK / 16) / kThreads; // same for a K-contiguous B
     static constexpr int kCols = BN / 32;                        // columns per lane of an N-contiguous B (8 or 4)
@@ -242,52 +97,85 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int8_t* __r
     const uint32_t kb = tid & 7u;
     const uint32_t nb = tid >> 3;
 
-    auto load_global = [&](uint32_t k0) {
+    // Per-lane source pointers of the first K step (rows / columns past the end are clamped: they are never stored).
+    const int8_t* aptr[T::kAChunks];
+#pragma unroll
+    for (int i = 0; i < T::kAChunks; ++i) {
+        const uint32_t c = tid + kThreads * i;
+        uint32_t row = row0 + (c >> 3);
+        row = row < row_end ? row : row_end - 1;
+        aptr[i] = A + static_cast<size_t>(row) * K + ((c & 7u) << 4);
+    }
+    const int8_t* bptrT[kTransB ? T::kBChunksT : 1];
+    const int8_t* bptr = B;
+    if constexpr (kTransB) {
+#pragma unroll
+        for (int i = 0; i < T::kBChunksT; ++i) {
+            const uint32_t c = tid + kThreads * i;
+            uint32_t col = n0 + (c >> 3);
+            col = col < N ? col : N - 1;
+            bptrT[i] = B + static_cast<size_t>(col) * K + ((c & 7u) << 4);
+        }
+    } else {
+        uint32_t col = n0 + nb * T::kCols;
+        col = col + T::kCols <= N ? col : N - T::kCols;
+        bptr = B + static_cast<size_t>(kb * 16u) * N + col;
+    }
+
+    // kFull: the whole 128-byte K step is inside [k_begin, k_end): plain loads.  Otherwise loads are clamped to the
+    // last valid 16 bytes / row and the out-of-range part is replaced by zeros (selects, no branches).
+    auto load_global = [&](uint32_t k0, auto full_tag) {
+        constexpr bool kFull = decltype(full_tag)::value;
 #pragma unroll
         for (int i = 0; i < T::kAChunks; ++i) {
-            const uint32_t c = tid + kThreads * i;
-            uint32_t row = row0 + (c >> 3);
-            row = row < row_end ? row : row_end - 1;  // rows past the end are never stored: any valid row will do
-            const uint32_t kk = k0 + ((c & 7u) << 4);
-            if (kk < k_end) {
-                areg[i] = *reinterpret_cast<const u32x4*>(A + static_cast<size_t>(row) * K + kk);
+            const uint32_t kk = k0 + (((tid + kThreads * i) & 7u) << 4);
+            if constexpr (kFull) {
+                areg[i] = *reinterpret_cast<const u32x4*>(aptr[i] + k0);
             } else {
-                areg[i] = u32x4{0u, 0u, 0u, 0u};
+                const bool ok = kk < k_end;
+                u32x4 v = *reinterpret_cast<const u32x4*>(aptr[i] + (ok ? k0 : 0u));
+                areg[i] = ok ? v : u32x4{0u, 0u, 0u, 0u};
             }
         }
         if constexpr (kTransB) {
 #pragma unroll
             for (int i = 0; i < T::kBChunksT; ++i) {
-                const uint32_t c = tid + kThreads * i;
-                uint32_t col = n0 + (c >> 3);
-                col = col < N ? col : N - 1;
-                const uint32_t kk = k0 + ((c & 7u) << 4);
-                if (kk < k_end) {
-                    bregT[i] = *reinterpret_cast<const u32x4*>(B + static_cast<size_t>(col) * K + kk);
+                const uint32_t kk = k0 + (((tid + kThreads * i) & 7u) << 4);
+                if constexpr (kFull) {
+                    bregT[i] = *reinterpret_cast<const u32x4*>(bptrT[i] + k0);
                 } else {
-                    bregT[i] = u32x4{0u, 0u, 0u, 0u};
+                    const bool ok = kk < k_end;
+                    u32x4 v = *reinterpret_cast<const u32x4*>(bptrT[i] + (ok ? k0 : 0u));
+                    bregT[i] = ok ? v : u32x4{0u, 0u, 0u, 0u};
                 }
             }
         } else {
-            uint32_t col = n0 + nb * T::kCols;
-            col = col + T::kCols <= N ? col : N - T::kCols;  // columns past the end are never stored
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const uint32_t kk = k0 + kb * 16u + i;
-                const int8_t* src = B + static_cast<size_t>(kk) * N + col;
-                if (kk < k_end) {
-                    if constexpr (T::kCols == 8) {
-                        u32x2 v = *reinterpret_cast<const u32x2*>(src);
-                        breg[i][0] = v[0];
-                        breg[i][1] = v[1];
-                    } else {
-                        breg[i][0] = *reinterpret_cast<const uint32_t*>(src);
-                    }
+                bool ok = true;
+                size_t roff = static_cast<size_t>(k0 + i) * N;
+                if constexpr (!kFull) {
+                    ok = kk < k_end;
+                    roff = ok ? roff : 0;   // row kb*16 of the first step: always valid memory
+                }
+                const int8_t* src = bptr + roff;
+                if constexpr (T::kCols == 8) {
+                    u32x2 v = *reinterpret_cast<const u32x2*>(src);
+                    breg[i][0] = ok ? v[0] : 0u;
+                    breg[i][1] = ok ? v[1] : 0u;
                 } else {
-#pragma unroll
-                    for (int d = 0; d < T::kCols / 4; ++d) breg[i][d] = 0u;
+                    const uint32_t v = *reinterpret_cast<const uint32_t*>(src);
+                    breg[i][0] = ok ? v : 0u;
                 }
             }
+        }
+    };
+    auto load_step = [&](uint32_t k0) {
+        if (k0 + kBK <= k_end) {
+            load_global(k0, std::true_type{});
+        } else {
+            load_global(k0, std::false_type{});
         }
     };
 
@@ -377,8 +265,8 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int8_t* __r
     // ---------------- main loop
     const uint32_t steps = (k_end - k_begin + kBK - 1) / kBK;
     char* stage0 = smem;
-    char* stage1 = smem + T::kStage;
-    load_global(k_begin);
+    char* stage1 = smem + (T::kStages == 2 ? T::kStage : 0);
+    load_step(k_begin);
     store_lds(stage0);
     __syncthreads();
     for (uint32_t t = 0; t < steps; ++t) {
@@ -386,9 +274,12 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int8_t* __r
         char* nxt = (t & 1u) ? stage0 : stage1;
         const bool more = t + 1 < steps;
         if (more) {
-            load_global(k_begin + (t + 1) * kBK);
+            load_step(k_begin + (t + 1) * kBK);
         }
         compute(cur);
+        if constexpr (T::kStages == 1) {
+            __syncthreads();  // single LDS stage: every wavefront must have read it before it is overwritten
+        }
         if (more) {
             store_lds(nxt);
         }
@@ -453,7 +344,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int8_t* __r
 }
 
 template <class T, bool kTransB, bool kSplitK>
-__global__ __launch_bounds__(kThreads) void gemm_kernel(GemmParams p)
+__global__ __launch_bounds__(kThreads, T::kMinBlocks) void gemm_kernel(GemmParams p)
 {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const uint32_t total = p.tiles_m * p.tiles_n;
@@ -716,6 +607,9 @@ extern "C" int ascq_matmul_w8a8(const ascq_matmul_desc* d, void* c, const void* 
         }
         return d->trans_b ? launch_gemm<TileST, true, false>(p, st) : launch_gemm<TileS, false, false>(p, st);
     }
+    if (d->m > 128 && !d->trans_b && gemm_dma_supported(p)) {
+        return launch_gemm_dma(p, false, st);
+    }
     if (d->m <= 1024) {
         return d->trans_b ? launch_gemm<TileMT, true, false>(p, st) : launch_gemm<TileM, false, false>(p, st);
     }
@@ -755,6 +649,9 @@ extern "C" int ascq_group_matmul_w8a8(const ascq_group_matmul_desc* g, void* y, 
     p.groups = g->groups;
     p.group_list_kind = g->group_list_kind;
     p.epi = make_epi(d, y, bias, scale, tok_scale);
+    if (gemm_dma_supported(p)) {
+        return launch_gemm_dma(p, true, st);
+    }
     typedef TileL T;
     // every group adds at most one partial tile along M
     p.tiles_m = (d->m + T::BM - 1) / T::BM + g->groups;

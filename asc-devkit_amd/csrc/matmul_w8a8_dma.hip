@@ -1,0 +1,347 @@
+// Large-M int8 matmul for gfx950 built on the two CDNA4 data-movement instructions that remove all register staging:
+//
+//   * global_load_lds_dwordx4: every lane names a 16-byte global source, the data lands in LDS at
+//     (uniform base + lane * 16) without passing through registers and is tracked by vmcnt.  Because the global
+//     address is free per lane, the bank-conflict swizzles are applied on the *source* side: the lane that owns LDS
+//     slot s fetches the 16 bytes that belong in that slot.
+//   * ds_read_b64_tr_b8: a transposing LDS read.  Within 16 lanes, lane l receives byte (l & 7) of the eight 8-byte
+//     rows addressed by lanes 2b + (l >> 3), b = 0..7.  Pointing even lanes at columns [c, c+8) and odd lanes at
+//     [c+8, c+16) of eight consecutive k rows gives every lane the 8 consecutive k values of column c + l: exactly
+//     the MFMA B operand, read from a B tile that is stored in LDS as it is in memory ([k][n], n contiguous).
+//
+// So the main loop is: DMA loads for the next K step, LDS reads, MFMAs - no VALU work, no LDS writes, no staging
+// registers.  A workgroup is 512 lanes (8 wavefronts, two per SIMD, so that one wavefront's LDS / address
+// instructions issue under the other's MFMAs) and owns a 256 x 256 tile; a wavefront owns 128 x 64 (4 x 2 MFMA
+// blocks of 32x32x32, 128 accumulator registers).  Two LDS stages of 64 KiB (A 256 x 128 B, B 128 x 256 B) are
+// separate arrays so that the compiler can tell that LDS reads of one stage do not depend on DMA writes to the
+// other.
+//
+// LDS layouts (all reads and writes conflict-free, measured at ~220-250 B/clk/CU):
+//   A stage: row r = 128 bytes = 8 pieces of 16; piece c is stored at position c ^ ((r >> 1) & 7).
+//   B stage: row k = 256 bytes = 16 pieces of 16; piece q is stored at position q ^ (2 * (k & 7)).
+#include "matmul_w8a8.h"
+
+namespace ascq {
+namespace {
+
+constexpr int kThreads = 512;
+constexpr int BM = 256, BK = 128;
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef __attribute__((address_space(1))) const void* gptr_t;
+typedef i32x2_t __attribute__((address_space(3)))* lds_v2_t;
+
+// 16-bit output of two adjacent columns packed into one dword store.
+template <int kOut>
+__device__ __forceinline__ uint32_t to_bits16(float v)
+{
+    if constexpr (kOut == ASCQ_BF16) {
+        return f32_to_bf16_bits(v);
+    } else {
+        return f32_to_half_bits_sat(v);
+    }
+}
+
+__device__ __forceinline__ float epi_value(const EpiParams& e, int32_t acc, const ChannelQ& q, float tok,
+                                           float bias_post)
+{
+    float v = static_cast<float>(acc) * q.s;
+    v = v * tok;  // tok is 1.0f without a token scale: an exact identity
+    if (e.bias_kind >= ASCQ_MM_BIAS_F32_POST) {
+        v = v + bias_post;
+    }
+    if (e.activation == ASCQ_MM_ACT_FASTER_GELU) {
+        v = faster_gelu(v);
+    }
+    return v;
+}
+
+// BN = 256: wavefronts 2 (M) x 4 (N), 128 x 64 each.  BN = 128: wavefronts 4 (M) x 2 (N), 64 x 64 each (used for the
+// last, partially filled round of tiles: half-width tiles finish it in half the time).
+template <int BN>
+__global__ __launch_bounds__(kThreads) void gemm_dma_kernel(GemmParams p, int grouped, uint32_t col_begin)
+{
+    constexpr int kWN = BN / 64;            // wavefronts along N
+    constexpr int kWM = 8 / kWN;            // wavefronts along M
+    constexpr int TI = BM / 32 / kWM;       // 32x32 blocks per wavefront along M
+    constexpr int TJ = 2;                   // and along N
+    constexpr int kPieces = BN / 16;        // 16-byte pieces per B row
+    constexpr int kBInstr = BK * BN / 1024 / 8;  // B DMA instructions per wavefront and K step
+    constexpr int kKsB = 32 * BN;           // bytes of B per K sub-step of 32 rows
+    __shared__ __attribute__((aligned(1024))) char A0[BM * BK];
+    __shared__ __attribute__((aligned(1024))) char B0[BK * BN];
+    __shared__ __attribute__((aligned(1024))) char A1[BM * BK];
+    __shared__ __attribute__((aligned(1024))) char B1[BK * BN];
+
+    const uint32_t total = p.tiles_m * p.tiles_n;
+    const uint32_t t = xcd_remap(blockIdx.x, total);
+    if (t >= total) {
+        return;
+    }
+    const uint32_t ms = t % p.tiles_m, tn = t / p.tiles_m;
+    const uint32_t K = p.k, N = p.n;
+    uint32_t row0 = ms * BM, row_end = p.m;
+    const int8_t* Bmat = p.b;
+    size_t chan_off = 0;
+    if (grouped) {
+        // walk the groups: group g owns tile slots [slot, slot + ceil(rows / BM))
+        uint32_t slot = 0;
+        int64_t off = 0;
+        bool found = false;
+        for (uint32_t g = 0; g < p.groups; ++g) {
+            const int64_t v = p.group_list[g];
+            const int64_t cnt = p.group_list_kind == ASCQ_GROUP_LIST_PREFIX_SUM ? v - off : v;
+            if (cnt <= 0) {
+                continue;
+            }
+            int64_t end = off + cnt;
+            if (end > static_cast<int64_t>(p.m)) {
+                end = p.m;
+            }
+            const uint32_t rows = end > off ? static_cast<uint32_t>(end - off) : 0u;
+            const uint32_t tiles = (rows + BM - 1) / BM;
+            if (ms < slot + tiles) {
+                row0 = static_cast<uint32_t>(off) + (ms - slot) * BM;
+                row_end = static_cast<uint32_t>(end);
+                Bmat = p.b + static_cast<size_t>(g) * K * N;
+                chan_off = static_cast<size_t>(g) * N;
+                found = true;
+                break;
+            }
+            slot += tiles;
+            off += cnt;
+        }
+        if (!found) {
+            return;
+        }
+    }
+    const uint32_t n0 = col_begin + tn * BN;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t wm = wave / kWN, wn = wave % kWN;
+
+    // ---- DMA sources: 4 A and 4 B instructions per wavefront and K step; lane owns LDS slot (instr * 64 + lane)
+    uint32_t aoff[4], boff[kBInstr];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const uint32_t s = (wave * 4 + u) * 64 + lane;
+        const uint32_t r = s >> 3, c = (s & 7u) ^ ((r >> 1) & 7u);
+        uint32_t row = row0 + r;
+        row = row < row_end ? row : row_end - 1;  // rows past the end are never stored: any valid row will do
+        aoff[u] = (row - row0) * K + 16u * c;
+    }
+#pragma unroll
+    for (int u = 0; u < kBInstr; ++u) {
+        const uint32_t s = (wave * kBInstr + u) * 64 + lane;
+        const uint32_t kb = s / kPieces;
+        const uint32_t swz = BN == 256 ? 2u * (kb & 7u) : 2u * ((kb >> 1) & 3u);
+        const uint32_t q = (s % kPieces) ^ swz;
+        uint32_t col = n0 + 16u * q;
+        col = col + 16u <= N ? col : N - 16u;      // columns past the end are never stored
+        boff[u] = kb * N + (col - n0);
+    }
+    const int8_t* Abase = p.a + static_cast<size_t>(row0) * K;
+    const int8_t* Bbase = Bmat + n0;
+    auto issue = [&](uint32_t k0, char* As, char* Bs) {
+        const int8_t* ab = Abase + k0;
+        const int8_t* bb = Bbase + static_cast<size_t>(k0) * N;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            __builtin_amdgcn_global_load_lds((gptr_t)(ab + aoff[u]), (lds_ptr_t)(As + (wave * 4 + u) * 1024), 16, 0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < kBInstr; ++u) {
+            __builtin_amdgcn_global_load_lds((gptr_t)(bb + boff[u]), (lds_ptr_t)(Bs + (wave * kBInstr + u) * 1024), 16, 0,
+                                             0);
+        }
+    };
+
+    i32x16 acc[TI][TJ];
+#pragma unroll
+    for (int i = 0; i < TI; ++i) {
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+        }
+    }
+
+    // ---- fragment addresses: one base per K sub-step (A) / per column block (B), everything else is an immediate
+    const uint32_t lrow = lane & 31u, g = lane >> 5;
+    const uint32_t grp16 = (lane >> 4) & 1u, bsub = (lane & 15u) >> 1, psub = lane & 1u;
+    uint32_t a_base[4], b_base[2];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+        a_base[ks] = (wm * (TI * 32) + lrow) * 128 + (((2 * ks + g) ^ ((lrow >> 1) & 7u)) << 4);
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const uint32_t swz = BN == 256 ? 2u * bsub : 2u * ((bsub >> 1) & 3u);
+        b_base[j] = (16 * g + bsub) * BN + (((4 * wn + 2 * j + grp16) ^ swz) << 4) + 8 * psub;
+    }
+    auto load_frags = [&](const char* As, const char* Bs, int ks, i32x4 (&af)[TI], i32x4 (&bf)[TJ]) {
+#pragma unroll
+        for (int i = 0; i < TI; ++i) {
+            af[i] = *reinterpret_cast<const i32x4*>(As + a_base[ks] + i * 4096);
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const i32x2_t lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2_t)(Bs + b_base[j] + ks * kKsB));
+            const i32x2_t hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2_t)(Bs + b_base[j] + ks * kKsB + 8 * BN));
+            bf[j] = i32x4{lo[0], lo[1], hi[0], hi[1]};
+        }
+    };
+    auto compute = [&](const char* As, const char* Bs) {
+        i32x4 af[2][TI], bf[2][TJ];
+        // Re-materialise the bases inside the loop body: the constant parts of every address then fold into the
+        // 16-bit offset field of the DS instructions instead of being hoisted into dozens of registers.
+#pragma unroll
+        for (int q = 0; q < 4; ++q) asm volatile("" : "+v"(a_base[q]));
+#pragma unroll
+        for (int q = 0; q < 2; ++q) asm volatile("" : "+v"(b_base[q]));
+        load_frags(As, Bs, 0, af[0], bf[0]);
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            if (ks < 3) {
+                load_frags(As, Bs, ks + 1, af[(ks + 1) & 1], bf[(ks + 1) & 1]);
+            }
+#pragma unroll
+            for (int i = 0; i < TI; ++i) {
+#pragma unroll
+                for (int j = 0; j < TJ; ++j) {
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks & 1][i], bf[ks & 1][j], acc[i][j], 0, 0, 0);
+                }
+            }
+            if (ks < 3) {
+                // one LDS read of the next sub-step behind each MFMA of this one
+#pragma unroll
+                for (int n = 0; n < TI * TJ; ++n) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, (TI + 2 * TJ + TI * TJ - 1) / (TI * TJ), 0);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    const uint32_t steps = K / BK;
+    issue(0, A0, B0);
+    asm volatile("s_waitcnt vmcnt(0)");
+    __syncthreads();
+    uint32_t s = 0;
+    for (; s + 1 < steps; s += 2) {
+        issue((s + 1) * BK, A1, B1);
+        compute(A0, B0);
+        asm volatile("s_waitcnt vmcnt(0)");
+        __syncthreads();
+        if (s + 2 < steps) {
+            issue((s + 2) * BK, A0, B0);
+        }
+        compute(A1, B1);
+        asm volatile("s_waitcnt vmcnt(0)");
+        __syncthreads();
+    }
+    if (s < steps) {  // odd number of K steps: the last one sits in stage 0
+        compute(A0, B0);
+    }
+
+    // ---- epilogue: register r of lane l in a 32x32 block is row 8*(r/4) + 4*(l/32) + r%4, column l%32
+    const EpiParams& e = p.epi;
+    auto run = [&](auto tag) {
+        constexpr int kOut = decltype(tag)::value;
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) {
+            const uint32_t col = n0 + (wn * TJ + j) * 32u + lrow;
+            const bool cvalid = col < N;
+            ChannelQ q{1.0f, 0, 1};
+            float bias_post = 0.0f;
+            int32_t bias_pre = 0;
+            if (cvalid) {
+                q = load_channel_q(e, chan_off + col);
+                bias_post = load_bias_post(e, chan_off + col);
+                if (e.bias_kind == ASCQ_MM_BIAS_I32_PRE) {
+                    bias_pre = static_cast<const int32_t*>(e.bias)[chan_off + col];
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < TI; ++i) {
+                const uint32_t rbase = row0 + (wm * TI + i) * 32u + 4u * g;
+                if constexpr (kOut == ASCQ_BF16 || kOut == ASCQ_F16) {
+                    // two adjacent columns per dword store: even lanes keep row r, odd lanes row r + 1
+                    const bool odd = (lane & 1u) != 0;
+#pragma unroll
+                    for (int r = 0; r < 16; r += 2) {
+                        const uint32_t ra = rbase + 8u * (r >> 2) + (r & 3);
+                        const float ta = (e.has_tok && ra < row_end) ? e.tok_scale[ra] : 1.0f;
+                        const float tb = (e.has_tok && ra + 1 < row_end) ? e.tok_scale[ra + 1] : 1.0f;
+                        const uint32_t ha = to_bits16<kOut>(epi_value(e, acc[i][j][r] + bias_pre, q, ta, bias_post));
+                        const uint32_t hb = to_bits16<kOut>(epi_value(e, acc[i][j][r + 1] + bias_pre, q, tb, bias_post));
+                        const uint32_t send = odd ? ha : hb;
+                        const uint32_t recv = static_cast<uint32_t>(
+                            __builtin_amdgcn_mov_dpp(static_cast<int>(send), 0xB1, 0xF, 0xF, true));  // lane ^ 1
+                        const uint32_t word = odd ? (recv | (hb << 16)) : (ha | (recv << 16));
+                        const uint32_t row = odd ? ra + 1 : ra;
+                        if (cvalid && row < row_end) {
+                            *reinterpret_cast<uint32_t*>(static_cast<uint16_t*>(e.c) +
+                                                         static_cast<size_t>(row) * e.ldc + (col & ~1u)) = word;
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const uint32_t row = rbase + 8u * (r >> 2) + (r & 3);
+                        if (cvalid && row < row_end) {
+                            const float tok = e.has_tok ? e.tok_scale[row] : 1.0f;
+                            epilogue_store<kOut>(e, row, col, acc[i][j][r] + bias_pre, q, tok, bias_post);
+                        }
+                    }
+                }
+            }
+        }
+    };
+    dispatch_out(e, run);
+}
+
+}  // namespace
+
+bool gemm_dma_supported(const GemmParams& p)
+{
+    return p.k % BK == 0 && p.n % 16 == 0 && p.n >= 16 && aligned16(p.a) && aligned16(p.b);
+}
+
+int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st)
+{
+    p.tiles_m = (p.m + BM - 1) / BM + (grouped ? p.groups : 0u);  // every group adds at most one partial tile
+    uint32_t tiles_n = (p.n + 255u) / 256u;
+    // Tile quantisation: when the last round of 256-wide tiles would fill less than half of the 256 CUs, its
+    // columns are computed by a second launch with 128-wide tiles, which finishes that round in about half the time.
+    uint32_t narrow_cols = 0;  // number of 256-wide column tiles handed to the 128-wide kernel
+    const uint32_t total = p.tiles_m * tiles_n;
+    const uint32_t rem = total % 256u;
+    if (!grouped && total > 256u && rem != 0 && rem <= 128u) {
+        narrow_cols = (rem + p.tiles_m - 1) / p.tiles_m;
+        if (narrow_cols > tiles_n) {
+            narrow_cols = tiles_n;
+        }
+    }
+    const uint32_t wide_cols = tiles_n - narrow_cols;
+    if (wide_cols) {
+        p.tiles_n = wide_cols;
+        const uint32_t t = p.tiles_m * p.tiles_n;
+        // the wide launch must not touch the narrow region: clip n for its column masks
+        GemmParams q = p;
+        if (narrow_cols) {
+            q.n = p.n;  // row pitch stays n; columns >= wide_cols * 256 are simply not assigned to any tile
+        }
+        gemm_dma_kernel<256><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(q, grouped ? 1 : 0, 0u);
+    }
+    if (narrow_cols) {
+        const uint32_t col_begin = wide_cols * 256u;
+        p.tiles_n = (p.n - col_begin + 127u) / 128u;
+        const uint32_t t = p.tiles_m * p.tiles_n;
+        gemm_dma_kernel<128><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(p, 0, col_begin);
+    }
+    return launch_status(grouped ? "ascq_group_matmul_w8a8" : "ascq_matmul_w8a8");
+}
+
+}  // namespace ascq
