@@ -6,7 +6,7 @@
 //     columns (256 contiguous bytes) and the four quarters take four different k rows, so one load instruction of a
 //     wavefront reads 4 rows x 256 bytes; 8 such loads are in flight per lane;
 //   * the four wavefronts of a workgroup take different k ranges of the same 512 columns, K is further split over
-//     gridDim.y, so that about 900 workgroups stream the weights;
+//     gridDim.y, so that about 450 workgroups stream the weights;
 //   * de-quantisation follows AscendAntiQuant<int4b_t, half> exactly: the nibble becomes an exact half via the
 //     0x6400 exponent trick (1024 + u) - 1032, then one rounded half add of the offset and one rounded half
 //     multiply by the scale (packed v_pk_add_f16 / v_pk_mul_f16 on two columns at a time);
@@ -262,11 +262,13 @@ __global__ __launch_bounds__(kThreads) void w4a16_generic_kernel(W4Params p)
 
 uint32_t pick_splits(uint32_t n, uint32_t k, uint32_t group_size)
 {
-    // K range per workgroup: a multiple of 128 rows (32 per wavefront) and of the group size; aim at ~900 workgroups
+    // K range per workgroup: a multiple of 128 rows (32 per wavefront) and of the group size; aim at ~450 workgroups (measured best on 256 CUs)
     (void)group_size;
     const uint32_t blocks_n = (n + kColsPerBlock - 1) / kColsPerBlock;
     const uint32_t units = k / kRowsPerPass;
-    uint32_t want = (896u + blocks_n - 1) / blocks_n;
+    uint32_t target = 448u;
+    if (const char* e = std::getenv("ASCQ_W4_WGS")) target = static_cast<uint32_t>(std::atoi(e));
+    uint32_t want = (target + blocks_n - 1) / blocks_n;
     uint32_t splits = units < want ? units : want;
     if (splits == 0) splits = 1;
     while (units % splits != 0) --splits;
