@@ -18,15 +18,14 @@ typedef int32_t i32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef short s16x2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
 
-// fp32 -> bfloat16 bits, round to nearest even (NaN stays NaN).
+// fp32 -> bfloat16 bits, round to nearest even (v_cvt_pk_bf16_f32 on gfx950; NaN stays NaN).
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f)
 {
-    uint32_t u = __float_as_uint(f);
-    uint32_t r = (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
-    return (f != f) ? ((u >> 16) | 0x40u) : r;
+    return __builtin_bit_cast(unsigned short, static_cast<__bf16>(f));
 }
 
 __device__ __forceinline__ float half_bits_to_f32(uint32_t h)

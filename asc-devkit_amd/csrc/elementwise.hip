@@ -157,6 +157,85 @@ __global__ __launch_bounds__(kThreads) void quant_scalar_kernel(QuantArgs a)
     }
 }
 
+// Fast path of the fp16 contract for half sources (per tensor / per channel): the arithmetic stays in packed half
+// registers - v_pk_mul_f16, v_pk_add_f16 (one rounding each), v_rndne_f16, packed clamp, v_cvt_i16_f16 - about five
+// VALU operations per element instead of the generic path's conversions through fp32.  NaN inputs give an
+// unspecified int8 here (they are outside the operator's defined domain).
+__device__ __forceinline__ f16x2 h2_from_bits(uint32_t b)
+{
+    f16x2 r;
+    __builtin_memcpy(&r, &b, 4);
+    return r;
+}
+
+__device__ __forceinline__ uint32_t quant_h2x2_to_i8x4(f16x2 a, f16x2 b)
+{
+    const f16x2 lo = {static_cast<half_t>(-128.0f), static_cast<half_t>(-128.0f)};
+    const f16x2 hi = {static_cast<half_t>(127.0f), static_cast<half_t>(127.0f)};
+    a = __builtin_elementwise_min(__builtin_elementwise_max(__builtin_elementwise_rint(a), lo), hi);
+    b = __builtin_elementwise_min(__builtin_elementwise_max(__builtin_elementwise_rint(b), lo), hi);
+    const s16x2 ia = __builtin_convertvector(a, s16x2);
+    const s16x2 ib = __builtin_convertvector(b, s16x2);
+    uint32_t ua, ub;
+    __builtin_memcpy(&ua, &ia, 4);
+    __builtin_memcpy(&ub, &ib, 4);
+    return __builtin_amdgcn_perm(ub, ua, 0x06040200u);  // low bytes of the four 16-bit integers
+}
+
+__global__ __launch_bounds__(kThreads) void quant_f16_fast_kernel(QuantArgs a)
+{
+    const uint32_t j = (blockIdx.x * kThreads + threadIdx.x) * 8u;
+    if (j >= a.n) {
+        return;
+    }
+    f16x2 s[4], o[4];
+    if (a.policy == ASCQ_PER_CHANNEL) {
+        const u32x4 v = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(a.scale) + j);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) s[e] = h2_from_bits(v[e]);
+    } else {
+        const half_t hs = static_cast<half_t>(a.sscale);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) s[e] = f16x2{hs, hs};
+    }
+    if (a.offset_kind == ASCQ_OFFSET_TENSOR) {
+        const u32x4 v = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(a.offset) + j);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = h2_from_bits(v[e]);
+    } else {
+        // no offset: adding +0 changes nothing that survives the conversion to int8
+        const half_t ho = static_cast<half_t>(a.offset_kind == ASCQ_OFFSET_NONE ? 0.0f : a.soffset);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = f16x2{ho, ho};
+    }
+    const uint16_t* src = static_cast<const uint16_t*>(a.src);
+    for (uint32_t r0 = blockIdx.y * kRowsInFlight; r0 < a.rows; r0 += gridDim.y * kRowsInFlight) {
+        u32x4 x[kRowsInFlight];
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; ++u) {
+            if (r0 + u < a.rows) {
+                x[u] = __builtin_nontemporal_load(
+                    reinterpret_cast<const u32x4*>(src + static_cast<size_t>(r0 + u) * a.n + j));
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; ++u) {
+            if (r0 + u < a.rows) {
+                f16x2 t[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    t[e] = h2_from_bits(x[u][e]) * s[e];  // one rounding
+                    t[e] = t[e] + o[e];                    // one rounding
+                }
+                u32x2 out;
+                out[0] = quant_h2x2_to_i8x4(t[0], t[1]);
+                out[1] = quant_h2x2_to_i8x4(t[2], t[3]);
+                __builtin_nontemporal_store(out, reinterpret_cast<u32x2*>(a.dst + static_cast<size_t>(r0 + u) * a.n + j));
+            }
+        }
+    }
+}
+
 template <int kSrc, int kPar, int kCt>
 int launch_quant(const QuantArgs& a, bool vec, hipStream_t st)
 {
@@ -168,6 +247,13 @@ int launch_quant(const QuantArgs& a, bool vec, hipStream_t st)
         grid.y = row_groups < want ? row_groups : want;
         if (grid.y > 65535u) grid.y = 65535u;
         const bool rint = a.round_mode == ASCQ_CAST_RINT || a.round_mode == ASCQ_CAST_NONE;
+        if constexpr (kSrc == ASCQ_F16 && kCt == ASCQ_F16) {
+            // fp16 contract on a half source: scale / offset are half tensors or scalars
+            if (rint && (a.policy == ASCQ_PER_TENSOR || (a.policy == ASCQ_PER_CHANNEL && kPar == ASCQ_F16))) {
+                quant_f16_fast_kernel<<<grid, kThreads, 0, st>>>(a);
+                return launch_status("ascq_quant");
+            }
+        }
         if (rint) {
             quant_vec_kernel<kSrc, kPar, kCt, true><<<grid, kThreads, 0, st>>>(a);
         } else {
@@ -560,6 +646,97 @@ __global__ __launch_bounds__(kThreads) void antiquant_scalar_kernel(AntiQuantArg
     }
 }
 
+// Fast path int8 -> half, [k, n] layout: bytes become halves through the exponent trick (0x6400 | (b ^ 0x80) is
+// 1024 + b + 128, minus 1152 is b, both exact), then one rounded packed add of the offset and one rounded packed
+// multiply by the scale: about 2.5 VALU operations per element.
+template <bool kHasOffset>
+__global__ __launch_bounds__(kThreads) void antiquant_i8_f16_fast_kernel(AntiQuantArgs a)
+{
+    const uint32_t j = (blockIdx.x * kThreads + threadIdx.x) * 16u;
+    if (j >= a.cols) {
+        return;
+    }
+    const f16x2 k1152 = {static_cast<half_t>(1152.0f), static_cast<half_t>(1152.0f)};
+    f16x2 s[8], o[8];
+    uint32_t cached_group = 0xFFFFFFFFu;
+    const int8_t* src = static_cast<const int8_t*>(a.src);
+    uint16_t* dst = static_cast<uint16_t*>(a.dst);
+    for (uint32_t r0 = blockIdx.y * kRowsInFlight; r0 < a.rows; r0 += gridDim.y * kRowsInFlight) {
+        u32x4 raw[kRowsInFlight];
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; ++u) {
+            if (r0 + u < a.rows) {
+                raw[u] = __builtin_nontemporal_load(
+                    reinterpret_cast<const u32x4*>(src + static_cast<size_t>(r0 + u) * a.cols + j));
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; ++u) {
+            const uint32_t r = r0 + u;
+            if (r >= a.rows) {
+                break;
+            }
+            const uint32_t g = a.per_tensor ? 0u : r / a.group_size;
+            if (g != cached_group) {
+                cached_group = g;
+                if (a.per_tensor) {
+                    const half_t hs = static_cast<half_t>(a.sscale), ho = static_cast<half_t>(a.soffset);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        s[e] = f16x2{hs, hs};
+                        o[e] = f16x2{ho, ho};
+                    }
+                } else {
+                    const size_t pi = static_cast<size_t>(g) * a.cols + j;
+                    const u32x4 s0 = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(a.scale) + pi);
+                    const u32x4 s1 = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(a.scale) + pi + 8);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        s[e] = h2_from_bits(s0[e]);
+                        s[4 + e] = h2_from_bits(s1[e]);
+                    }
+                    if constexpr (kHasOffset) {
+                        const u32x4 o0 = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(a.offset) + pi);
+                        const u32x4 o1 =
+                            *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(a.offset) + pi + 8);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            o[e] = h2_from_bits(o0[e]);
+                            o[4 + e] = h2_from_bits(o1[e]);
+                        }
+                    }
+                }
+            }
+            u32x4 y0, y1;
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                const uint32_t x = raw[u][d] ^ 0x80808080u;
+                f16x2 lo = h2_from_bits(__builtin_amdgcn_perm(0x64646464u, x, 0x04010400u)) - k1152;  // bytes 0, 1
+                f16x2 hi = h2_from_bits(__builtin_amdgcn_perm(0x64646464u, x, 0x04030402u)) - k1152;  // bytes 2, 3
+                if constexpr (kHasOffset) {
+                    lo = lo + o[2 * d];
+                    hi = hi + o[2 * d + 1];
+                }
+                lo = s[2 * d] * lo;
+                hi = s[2 * d + 1] * hi;
+                uint32_t blo, bhi;
+                __builtin_memcpy(&blo, &lo, 4);
+                __builtin_memcpy(&bhi, &hi, 4);
+                if (d < 2) {
+                    y0[2 * d] = blo;
+                    y0[2 * d + 1] = bhi;
+                } else {
+                    y1[2 * (d - 2)] = blo;
+                    y1[2 * (d - 2) + 1] = bhi;
+                }
+            }
+            const size_t oe = static_cast<size_t>(r) * a.cols + j;
+            __builtin_nontemporal_store(y0, reinterpret_cast<u32x4*>(dst + oe));
+            __builtin_nontemporal_store(y1, reinterpret_cast<u32x4*>(dst + oe + 8));
+        }
+    }
+}
+
 template <int kSrc, int kDst>
 int launch_antiquant(const AntiQuantArgs& a, bool vec, hipStream_t st)
 {
@@ -570,6 +747,16 @@ int launch_antiquant(const AntiQuantArgs& a, bool vec, hipStream_t st)
         uint32_t want = (8192u + grid.x - 1) / grid.x;
         grid.y = row_groups < want ? row_groups : want;
         if (grid.y > 65535u) grid.y = 65535u;
+        if constexpr (kSrc == ASCQ_I8 && kDst == ASCQ_F16) {
+            if (!a.transpose) {
+                if (a.has_offset) {
+                    antiquant_i8_f16_fast_kernel<true><<<grid, kThreads, 0, st>>>(a);
+                } else {
+                    antiquant_i8_f16_fast_kernel<false><<<grid, kThreads, 0, st>>>(a);
+                }
+                return launch_status("ascq_antiquant");
+            }
+        }
         antiquant_vec_kernel<kSrc, kDst><<<grid, kThreads, 0, st>>>(a);
     } else {
         size_t total = static_cast<size_t>(a.rows) * a.cols;
