@@ -106,6 +106,10 @@ def load_library():
     if not os.path.exists(LIB_PATH):
         raise RuntimeError(f"{LIB_PATH} is missing: build it first (python -c 'import __graft_entry__ as g; "
                            f"g.build()'); there is no fallback path")
+    # One HIP runtime per process: torch bundles its own libamdhip64 and this package keeps its tensors in torch's
+    # allocations, so torch's copy has to be the one already mapped when libascq.so resolves its dependency;
+    # loading libascq.so first would bind it to a second runtime instance that cannot launch on torch's context.
+    import torch  # noqa: F401
     lib = C.CDLL(LIB_PATH)
     for name, (res, args) in SIGNATURES.items():
         fn = getattr(lib, name)  # AttributeError if a declared symbol is not exported

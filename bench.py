@@ -24,6 +24,12 @@ for _p in (os.path.join(ROOT, "asc-devkit_amd"), os.path.join(ROOT, "oracle")):
 
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 matrix peak, TOP/s
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E peak, GB/s
+# Bytes that left / entered the L2 caches per launch, from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs of
+# `bench.py --quick --no-cpu --copy-probe`; each counter is scaled by its reading for the 1 GiB copy of the same run
+# (FETCH_SIZE reads 0.5 per KiB there, WRITE_SIZE 1.0 per KiB).  Measured offline and recorded here; a run of this
+# file does not re-measure them.
+GEMM_TRAFFIC_BYTES = 249316454   # M=2048 GEMM, both launches: 191.7 MB fetched + 57.6 MB written
+GEMV_TRAFFIC_BYTES = 127087616   # W4A16 M=1 GEMV, partial + reduce kernels: 126.1 MB fetched + 1.0 MB written
 
 
 def main():
@@ -34,6 +40,9 @@ def main():
     ap.add_argument("--quick", action="store_true", help="headline + W4A16 GEMV only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="run a single workload: w8a8 | w4a16 | quant | dequant | antiquant | group")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also launch one device-to-device copy of 1 GiB: the known-size kernel that calibrates the "
+                         "FETCH_SIZE / WRITE_SIZE counters when this command runs under rocprofv3 --pmc")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU; run it with --gpus 1 (the path shards without communication, "
@@ -85,7 +94,13 @@ def main():
         starts.append(a)
         stops.append(b)
 
-    results = {}
+    if args.copy_probe:
+        a = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        b = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        b.copy_(a)
+        torch.cuda.synchronize()
+        del a, b
+        torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------ W8A8 linear (config 3)
     def w8a8(M, steps, warmup):
@@ -229,10 +244,16 @@ def main():
                                "per-token int8 quant -> int8 GEMM with W [4096,11008] -> fused (channel x token) "
                                "dequant to bf16; one step = quant kernel + GEMM kernel",
                    "m": 2048, "k": 4096, "n": 11008, "ops_per_step": head["ops"]},
-        "roofline": {"bound": "mfma", "kernel": "gemm_kernel<Tile 256x256x128, B [k,n]>",
+        # The GEMM is two launches of one kernel template back to back: 256x256 tiles for the full rounds of 256
+        # workgroups and 256x128 tiles for the last partial round; the events bracket both, so `achieved` is the
+        # 2*M*K*N operations over the sum of the two durations.  `traffic` is HBM bytes per GEMM (both launches) from
+        # rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of `bench.py --only w8a8 --copy-probe`, each counter scaled by
+        # its reading for the 1 GiB copy; it is a constant measured offline, not re-measured by this run.
+        "roofline": {"bound": "mfma", "kernel": "gemm_dma_kernel<256> + gemm_dma_kernel<128> (last partial round)",
                      "achieved": head["gemm_tops"], "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
-                     "frac": head["gemm_tops"] / PEAK_INT8_TOPS, "traffic": None,
-                     "avg_kernel_ms": head["gemm_kernel_ms"]},
+                     "frac": head["gemm_tops"] / PEAK_INT8_TOPS, "traffic": GEMM_TRAFFIC_BYTES,
+                     "avg_kernel_ms": head["gemm_kernel_ms"], "ops_per_launch": head["ops"],
+                     "algorithmic_bytes": head["bytes"]},
     }
     if only == "w8a8":
         print(json.dumps(out))
@@ -242,9 +263,9 @@ def main():
     out["w4a16_gemv"] = {"metric": "w4a16_decode_gemv_hbm_gbs_m1_k8192_n28672", "value": gemv["gbs"], "unit": "GB/s",
                          "workload": "BASELINE configs[3] at M=1, 4 rotating weight sets (500 MB > Infinity Cache)",
                          "ms_per_step": gemv["ms_per_step"],
-                         "roofline": {"bound": "hbm", "kernel": "w4a16_partial_kernel<1> + w4a16_reduce_kernel",
+                         "roofline": {"bound": "hbm", "kernel": "w4a16_mfma_kernel<1, offset> + w4a16_reduce_kernel",
                                       "achieved": gemv["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                      "frac": gemv["gbs"] / PEAK_HBM_GBS, "traffic": None,
+                                      "frac": gemv["gbs"] / PEAK_HBM_GBS, "traffic": GEMV_TRAFFIC_BYTES,
                                       "avg_kernel_ms": gemv["kernel_ms"], "bytes_per_launch": gemv["bytes"]}}
 
     if not args.quick:
@@ -277,28 +298,35 @@ def main():
         cores = min(16, os.cpu_count() or 1)
         orc.set_threads(cores)
         x, w, cs = head["tensors"]
-        rows = 512                                    # bounded sample: the first 512 of the 2048 activation rows
-        xb = x[:rows].view(torch.int16).cpu().numpy().view(np.uint16)
+        xb = x.view(torch.int16).cpu().numpy().view(np.uint16)
         wn, csn = w.cpu().numpy(), cs.cpu().numpy()
-        t0 = time.perf_counter()
-        qn, tsn = orc.dynamic_quant_per_token(abi.BF16, xb)
-        d = abi.MatmulDesc(m=rows, n=11008, k=4096, out_dtype=abi.BF16, quant_mode=abi.MM_QUANT_VECTOR,
+        d = abi.MatmulDesc(m=2048, n=11008, k=4096, out_dtype=abi.BF16, quant_mode=abi.MM_QUANT_VECTOR,
                            scale_format=abi.MM_SCALE_F32, has_tok_scale=1)
-        orc.matmul_w8a8(d, qn, wn, None, csn, tsn)
-        dt = time.perf_counter() - t0
-        out["cpu_baseline"] = {"value": 2.0 * rows * 4096 * 11008 / dt / 1e12, "unit": "TOPS", "cores": cores,
+        reps, t0 = 0, time.perf_counter()
+        while True:                                   # bounded sample: whole steps until about 12 s have passed
+            qn, tsn = orc.dynamic_quant_per_token(abi.BF16, xb)
+            orc.matmul_w8a8(d, qn, wn, None, csn, tsn)
+            reps += 1
+            dt = time.perf_counter() - t0
+            if dt >= 12.0 or reps >= 64:
+                break
+        out["cpu_baseline"] = {"value": reps * 2.0 * 2048 * 4096 * 11008 / dt / 1e12, "unit": "TOPS", "cores": cores,
                                "kind": "port",
-                               "sample": f"first {rows} of 2048 rows of the same workload (quant + GEMM + epilogue), "
-                                         f"{dt:.2f} s, OpenMP over rows"}
+                               "sample": f"{reps} whole steps of the same workload (per-token quant + int8 GEMM + "
+                                         f"epilogue, all 2048 rows) in {dt:.2f} s, OpenMP over rows"}
         xs, w4, sc4, of4 = gemv["tensors"]
-        cols = 2048                                   # bounded sample: 2048 of the 28672 output columns
         d4 = abi.W4A16Desc(m=1, n=28672, k=8192, group_size=128, has_offset=1)
-        t0 = time.perf_counter()
-        orc.matmul_w4a16(d4, xs.cpu().numpy(), w4.cpu().numpy(), sc4.cpu().numpy(), of4.cpu().numpy(), cols=(0, cols))
-        dt = time.perf_counter() - t0
-        out["w4a16_gemv"]["cpu_baseline"] = {"value": gemv["bytes"] * (cols / 28672) / dt / 1e9, "unit": "GB/s",
+        a4 = (xs.cpu().numpy(), w4.cpu().numpy(), sc4.cpu().numpy(), of4.cpu().numpy())
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            orc.matmul_w4a16(d4, *a4)
+            reps += 1
+            dt = time.perf_counter() - t0
+            if dt >= 6.0 or reps >= 64:
+                break
+        out["w4a16_gemv"]["cpu_baseline"] = {"value": reps * gemv["bytes"] / dt / 1e9, "unit": "GB/s",
                                              "cores": cores, "kind": "port",
-                                             "sample": f"{cols} of 28672 output columns, {dt:.2f} s"}
+                                             "sample": f"{reps} whole GEMVs (all 28672 columns) in {dt:.2f} s"}
     print(json.dumps(out))
 
 
