@@ -1,0 +1,416 @@
+// C++ host-side mirror of the reference's operator surface for the quantized-inference path, on top of the C ABI in
+// ascq.h.  The reference's operators are `AscendC::` function templates called inside a device kernel on on-chip
+// `LocalTensor<T>` views; here the same names, template parameters and argument order act on `DeviceTensor<T>` views
+// of HBM buffers and enqueue the fused gfx950 kernel on a HIP stream.
+//
+//   reference (include/adv_api/quantization/ascend_quant.h:63-762)       this header
+//   AscendC::AscendQuant<T>(dst, src, tmp, scale, offset, calCount)      ascq::AscendQuant<T>(dst, src, scale, offset, calCount, stream)
+//   AscendC::AscendDequant<dstT, scaleT, mode>(dst, src, deqScale, tmp, params)   ascq::AscendDequant<dstT, scaleT, mode>(dst, src, deqScale, params, stream)
+//   AscendC::AscendAntiQuant<In, Out, isTranspose>(dst, src, offset, scale, tmp, k, shapeInfo)   ascq::AscendAntiQuant<...>(dst, src, offset, scale, k, shapeInfo, stream)
+//   AscendC::Matmul<...> mm; mm.SetTensorA/B, SetBias, SetQuantScalar/Vector, IterateAll (include/adv_api/matmul/matmul.h:175-185)   ascq::Matmul
+//
+// Differences a caller sees: there is no `sharedTmpBuffer` argument (the kernels need none); a trailing `stream`
+// argument (a hipStream_t as void*, nullptr = default stream) is added; failed argument checks throw `ascq::Error`
+// carrying the C ABI's status code and message instead of the reference's log-and-abort in CPU-debug builds.
+#ifndef ASCQ_ASCENDC_HPP
+#define ASCQ_ASCENDC_HPP
+
+#include <cstddef>
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+
+#include "ascq.h"
+
+namespace ascq {
+
+class Error : public std::runtime_error {
+public:
+    Error(int status, const char* what) : std::runtime_error(what ? what : ""), status_(status) {}
+    int status() const { return status_; }
+
+private:
+    int status_;
+};
+
+inline void Check(int status)
+{
+    if (status != ASCQ_OK) {
+        throw Error(status, ascq_last_error());
+    }
+}
+
+// Storage-only element types: the host never does arithmetic on them.
+struct half {
+    uint16_t bits;
+};
+struct bfloat16_t {
+    uint16_t bits;
+};
+struct int4b_t {  // two values per byte, even element in the low nibble
+    uint8_t pair;
+};
+
+template <typename T>
+struct DTypeOf;
+template <>
+struct DTypeOf<half> {
+    static constexpr int32_t value = ASCQ_F16;
+};
+template <>
+struct DTypeOf<bfloat16_t> {
+    static constexpr int32_t value = ASCQ_BF16;
+};
+template <>
+struct DTypeOf<float> {
+    static constexpr int32_t value = ASCQ_F32;
+};
+template <>
+struct DTypeOf<int8_t> {
+    static constexpr int32_t value = ASCQ_I8;
+};
+template <>
+struct DTypeOf<int4b_t> {
+    static constexpr int32_t value = ASCQ_I4;
+};
+template <>
+struct DTypeOf<int32_t> {
+    static constexpr int32_t value = ASCQ_I32;
+};
+template <>
+struct DTypeOf<uint64_t> {
+    static constexpr int32_t value = ASCQ_U64;
+};
+
+// View of a caller-owned device buffer: the counterpart of LocalTensor / GlobalTensor.  `size` counts elements
+// (for int4b_t: values, two per byte).
+template <typename T>
+class DeviceTensor {
+public:
+    DeviceTensor() = default;
+    DeviceTensor(T* data, uint32_t size) : data_(data), size_(size) {}
+    T* GetPhyAddr() const { return data_; }
+    uint32_t GetSize() const { return size_; }
+
+private:
+    T* data_ = nullptr;
+    uint32_t size_ = 0;
+};
+
+// ref: include/adv_api/quantization/ascend_quant_utils.h:31-87
+enum class RoundMode : int32_t { CAST_NONE = 0, CAST_RINT, CAST_FLOOR, CAST_CEIL, CAST_ROUND, CAST_TRUNC };
+enum class AscendQuantPolicy : int32_t { PER_TENSOR, PER_CHANNEL, PER_TOKEN, PER_GROUP };
+struct AscendQuantConfig {
+    bool hasOffset = false;
+    int32_t kDim = 1;
+    RoundMode roundMode = RoundMode::CAST_RINT;
+};
+struct AscendQuantParam {
+    uint32_t m;
+    uint32_t n;
+    uint32_t calCount;
+    uint32_t groupSize = 0;
+};
+
+// Per tensor (ref: ascend_quant.h:63-139).
+template <typename T>
+void AscendQuant(const DeviceTensor<int8_t>& dstTensor, const DeviceTensor<T>& srcTensor, float scale, float offset,
+                 uint32_t calCount, void* stream = nullptr)
+{
+    ascq_quant_desc d{};
+    d.policy = ASCQ_PER_TENSOR;
+    d.src_dtype = d.scale_dtype = DTypeOf<T>::value;
+    d.compute = ASCQ_COMPUTE_F16;
+    d.round_mode = ASCQ_CAST_RINT;
+    d.offset_kind = ASCQ_OFFSET_SCALAR;
+    d.scale = scale;
+    d.offset = offset;
+    d.m = 1;
+    d.n = d.cal_count = calCount;
+    Check(ascq_quant(&d, dstTensor.GetPhyAddr(), srcTensor.GetPhyAddr(), nullptr, nullptr, stream));
+}
+
+template <typename T>
+void AscendQuant(const DeviceTensor<int8_t>& dstTensor, const DeviceTensor<T>& srcTensor, float scale, float offset,
+                 void* stream = nullptr)
+{
+    AscendQuant<T>(dstTensor, srcTensor, scale, offset, srcTensor.GetSize(), stream);
+}
+
+// Per channel, scalar offset (ref: ascend_quant.h:159-232); `offset` is given as float and rounded once to T.
+template <typename T>
+void AscendQuant(const DeviceTensor<int8_t>& dstTensor, const DeviceTensor<T>& srcTensor,
+                 const DeviceTensor<T>& scaleTensor, float offset, uint32_t scaleCount, uint32_t calCount,
+                 void* stream = nullptr)
+{
+    ascq_quant_desc d{};
+    d.policy = ASCQ_PER_CHANNEL;
+    d.src_dtype = d.scale_dtype = DTypeOf<T>::value;
+    d.compute = ASCQ_COMPUTE_F16;
+    d.round_mode = ASCQ_CAST_RINT;
+    d.offset_kind = ASCQ_OFFSET_SCALAR;
+    d.offset = offset;
+    d.n = scaleCount;
+    d.m = scaleCount ? calCount / scaleCount : 0;
+    d.cal_count = calCount;
+    Check(ascq_quant(&d, dstTensor.GetPhyAddr(), srcTensor.GetPhyAddr(), scaleTensor.GetPhyAddr(), nullptr, stream));
+}
+
+// Per channel, offset tensor (ref: ascend_quant.h:234-347).
+template <typename T>
+void AscendQuant(const DeviceTensor<int8_t>& dstTensor, const DeviceTensor<T>& srcTensor,
+                 const DeviceTensor<T>& scaleTensor, const DeviceTensor<T>& offsetTensor, uint32_t scaleCount,
+                 uint32_t offsetCount, uint32_t calCount, void* stream = nullptr)
+{
+    if (scaleCount != offsetCount) {
+        throw Error(ASCQ_EINVAL, "AscendQuant: scaleCount must equal offsetCount");
+    }
+    ascq_quant_desc d{};
+    d.policy = ASCQ_PER_CHANNEL;
+    d.src_dtype = d.scale_dtype = DTypeOf<T>::value;
+    d.compute = ASCQ_COMPUTE_F16;
+    d.round_mode = ASCQ_CAST_RINT;
+    d.offset_kind = ASCQ_OFFSET_TENSOR;
+    d.n = scaleCount;
+    d.m = scaleCount ? calCount / scaleCount : 0;
+    d.cal_count = calCount;
+    Check(ascq_quant(&d, dstTensor.GetPhyAddr(), srcTensor.GetPhyAddr(), scaleTensor.GetPhyAddr(),
+                     offsetTensor.GetPhyAddr(), stream));
+}
+
+// PER_TOKEN / PER_GROUP with the arithmetic in scaleT (ref: ascend_quant.h:667-762).  The reference passes config and
+// policy as template arguments; they are ordinary arguments here.
+template <typename srcT, typename scaleT>
+void AscendQuant(const DeviceTensor<int8_t>& dstTensor, const DeviceTensor<srcT>& srcTensor,
+                 const DeviceTensor<scaleT>& scaleTensor, const DeviceTensor<scaleT>& offsetTensor,
+                 const AscendQuantParam& para, const AscendQuantConfig& config, AscendQuantPolicy policy,
+                 void* stream = nullptr)
+{
+    ascq_quant_desc d{};
+    d.policy = static_cast<int32_t>(policy);
+    d.src_dtype = DTypeOf<srcT>::value;
+    d.scale_dtype = DTypeOf<scaleT>::value;
+    d.compute = ASCQ_COMPUTE_SCALE_T;
+    d.round_mode = static_cast<int32_t>(config.roundMode);
+    d.offset_kind = config.hasOffset ? ASCQ_OFFSET_TENSOR : ASCQ_OFFSET_NONE;
+    d.k_dim = config.kDim;
+    d.m = para.m;
+    d.n = para.n;
+    d.cal_count = para.calCount;
+    d.group_size = para.groupSize;
+    Check(ascq_quant(&d, dstTensor.GetPhyAddr(), srcTensor.GetPhyAddr(), scaleTensor.GetPhyAddr(),
+                     config.hasOffset ? offsetTensor.GetPhyAddr() : nullptr, stream));
+}
+
+// ref: include/adv_api/quantization/ascend_dequant_utils.h:26-30, impl/basic_api/utils/kernel_utils_mode.h:181-184
+struct DequantParams {
+    uint32_t m;
+    uint32_t n;
+    uint32_t calCount;
+};
+enum class DeQuantMode : int32_t { DEQUANT_WITH_SINGLE_ROW = 0, DEQUANT_WITH_MULTI_ROW = 1 };
+
+// Tensor scale (ref: ascend_dequant.h:58-175).  dst rows are ascq_dequant_dst_stride(dstT, n) elements apart.
+template <typename dstT, typename scaleT, DeQuantMode mode = DeQuantMode::DEQUANT_WITH_SINGLE_ROW>
+void AscendDequant(const DeviceTensor<dstT>& dstTensor, const DeviceTensor<int32_t>& srcTensor,
+                   const DeviceTensor<scaleT>& deqScale, DequantParams params, void* stream = nullptr)
+{
+    ascq_dequant_desc d{};
+    d.policy = ASCQ_PER_CHANNEL;
+    d.src_dtype = ASCQ_I32;
+    d.scale_dtype = DTypeOf<scaleT>::value;
+    d.dst_dtype = DTypeOf<dstT>::value;
+    d.mode = static_cast<int32_t>(mode);
+    d.m = params.m;
+    d.n = params.n;
+    d.cal_count = params.calCount;
+    Check(ascq_dequant(&d, dstTensor.GetPhyAddr(), srcTensor.GetPhyAddr(), deqScale.GetPhyAddr(), stream));
+}
+
+// Scalar scale (ref: ascend_dequant.h:205-281).
+template <typename dstT, DeQuantMode mode = DeQuantMode::DEQUANT_WITH_SINGLE_ROW>
+void AscendDequant(const DeviceTensor<dstT>& dstTensor, const DeviceTensor<int32_t>& srcTensor, float deqScale,
+                   DequantParams params, void* stream = nullptr)
+{
+    ascq_dequant_desc d{};
+    d.policy = ASCQ_PER_TENSOR;
+    d.src_dtype = ASCQ_I32;
+    d.scale_dtype = ASCQ_F32;
+    d.dst_dtype = DTypeOf<dstT>::value;
+    d.mode = static_cast<int32_t>(mode);
+    d.scale = deqScale;
+    d.m = params.m;
+    d.n = params.n;
+    d.cal_count = params.calCount;
+    Check(ascq_dequant(&d, dstTensor.GetPhyAddr(), srcTensor.GetPhyAddr(), nullptr, stream));
+}
+
+// ref: include/adv_api/quantization/ascend_antiquant_utils.h:27-32
+struct AntiQuantShapeInfo {
+    uint32_t offsetHeight{0};
+    uint32_t offsetWidth{0};
+    uint32_t scaleHeight{0};
+    uint32_t scaleWidth{0};
+};
+
+// Offset and scale tensors (ref: ascend_antiquant.h:46-134).  src is [k, n] (or [n, k] when isTranspose); n is derived
+// from the source size as the reference derives it from the tensor's shape.
+template <typename InputDataType, typename OutputDataType, bool isTranspose>
+void AscendAntiQuant(const DeviceTensor<OutputDataType>& dst, const DeviceTensor<InputDataType>& src,
+                     const DeviceTensor<OutputDataType>& offset, const DeviceTensor<OutputDataType>& scale, uint32_t k,
+                     const AntiQuantShapeInfo& shapeInfo = {}, void* stream = nullptr)
+{
+    ascq_antiquant_desc d{};
+    d.src_dtype = DTypeOf<InputDataType>::value;
+    d.dst_dtype = DTypeOf<OutputDataType>::value;
+    d.is_transpose = isTranspose ? 1 : 0;
+    d.has_offset = 1;
+    d.k = k;
+    d.n = k ? src.GetSize() / k : 0;
+    d.offset_height = shapeInfo.offsetHeight;
+    d.offset_width = shapeInfo.offsetWidth;
+    d.scale_height = shapeInfo.scaleHeight;
+    d.scale_width = shapeInfo.scaleWidth;
+    Check(ascq_antiquant(&d, dst.GetPhyAddr(), src.GetPhyAddr(), offset.GetPhyAddr(), scale.GetPhyAddr(), stream));
+}
+
+// Scale only (ref: ascend_antiquant.h:136-210).
+template <typename InputDataType, typename OutputDataType, bool isTranspose>
+void AscendAntiQuant(const DeviceTensor<OutputDataType>& dst, const DeviceTensor<InputDataType>& src,
+                     const DeviceTensor<OutputDataType>& scale, uint32_t k, const AntiQuantShapeInfo& shapeInfo = {},
+                     void* stream = nullptr)
+{
+    ascq_antiquant_desc d{};
+    d.src_dtype = DTypeOf<InputDataType>::value;
+    d.dst_dtype = DTypeOf<OutputDataType>::value;
+    d.is_transpose = isTranspose ? 1 : 0;
+    d.has_offset = 0;
+    d.k = k;
+    d.n = k ? src.GetSize() / k : 0;
+    d.scale_height = shapeInfo.scaleHeight;
+    d.scale_width = shapeInfo.scaleWidth;
+    Check(ascq_antiquant(&d, dst.GetPhyAddr(), src.GetPhyAddr(), nullptr, scale.GetPhyAddr(), stream));
+}
+
+// Scalar offset and scale (ref: ascend_antiquant.h:211-262); the scalars are given as float and rounded once to
+// OutputDataType.
+template <typename InputDataType, typename OutputDataType, bool isTranspose>
+void AscendAntiQuant(const DeviceTensor<OutputDataType>& dst, const DeviceTensor<InputDataType>& src, float offset,
+                     float scale, uint32_t k, void* stream = nullptr)
+{
+    ascq_antiquant_desc d{};
+    d.src_dtype = DTypeOf<InputDataType>::value;
+    d.dst_dtype = DTypeOf<OutputDataType>::value;
+    d.is_transpose = isTranspose ? 1 : 0;
+    d.has_offset = 1;
+    d.per_tensor = 1;
+    d.scale = scale;
+    d.offset = offset;
+    d.k = k;
+    d.n = k ? src.GetSize() / k : 0;
+    Check(ascq_antiquant(&d, dst.GetPhyAddr(), src.GetPhyAddr(), nullptr, nullptr, stream));
+}
+
+// The int8 Matmul object with the quant epilogue (ref: include/adv_api/matmul/matmul.h:138-185; the quant parameters
+// are consumed at copy-out, impl/adv_api/detail/matmul/stage/copy_cube_out/quant/quant_processor_fixpipe.h:74-222).
+// CType selects the output: int32_t (no quant), half / bfloat16_t / float / int8_t (quant epilogue).
+template <typename CType>
+class Matmul {
+public:
+    Matmul(uint32_t m, uint32_t n, uint32_t k)
+    {
+        desc_ = ascq_matmul_desc{};
+        desc_.m = m;
+        desc_.n = n;
+        desc_.k = k;
+        desc_.out_dtype = DTypeOf<CType>::value;
+        desc_.quant_mode = ASCQ_MM_QUANT_NONE;
+    }
+    void SetTensorA(const DeviceTensor<int8_t>& a, bool isTransposeA = false)
+    {
+        a_ = a.GetPhyAddr();
+        desc_.trans_a = isTransposeA ? 1 : 0;
+    }
+    void SetTensorB(const DeviceTensor<int8_t>& b, bool isTransposeB = false)
+    {
+        b_ = b.GetPhyAddr();
+        desc_.trans_b = isTransposeB ? 1 : 0;
+    }
+    // int32 bias: the accumulator's initial value, as in the reference.
+    void SetBias(const DeviceTensor<int32_t>& bias)
+    {
+        bias_ = bias.GetPhyAddr();
+        desc_.bias_kind = ASCQ_MM_BIAS_I32_PRE;
+    }
+    // fp32 / bf16 bias added after dequantisation (not a reference combination; used by LLM linears).
+    void SetBias(const DeviceTensor<float>& bias)
+    {
+        bias_ = bias.GetPhyAddr();
+        desc_.bias_kind = ASCQ_MM_BIAS_F32_POST;
+    }
+    void SetBias(const DeviceTensor<bfloat16_t>& bias)
+    {
+        bias_ = bias.GetPhyAddr();
+        desc_.bias_kind = ASCQ_MM_BIAS_BF16_POST;
+    }
+    void DisableBias()
+    {
+        bias_ = nullptr;
+        desc_.bias_kind = ASCQ_MM_BIAS_NONE;
+    }
+    void SetQuantScalar(uint64_t quantScalar)
+    {
+        desc_.quant_mode = ASCQ_MM_QUANT_SCALAR;
+        desc_.scale_format = ASCQ_MM_SCALE_U64;
+        desc_.quant_scalar = quantScalar;
+    }
+    void SetQuantVector(const DeviceTensor<uint64_t>& quantTensor)
+    {
+        desc_.quant_mode = ASCQ_MM_QUANT_VECTOR;
+        desc_.scale_format = ASCQ_MM_SCALE_U64;
+        quant_ = quantTensor.GetPhyAddr();
+    }
+    // Plain fp32 per-channel scales (all 23 mantissa bits), optionally with per-token scales.
+    void SetQuantVector(const DeviceTensor<float>& scaleTensor)
+    {
+        desc_.quant_mode = ASCQ_MM_QUANT_VECTOR;
+        desc_.scale_format = ASCQ_MM_SCALE_F32;
+        quant_ = scaleTensor.GetPhyAddr();
+    }
+    void SetTokenScale(const DeviceTensor<float>& tokScale)
+    {
+        tok_ = tokScale.GetPhyAddr();
+        desc_.has_tok_scale = 1;
+    }
+    void SetWorkspace(void* workspace, size_t bytes)
+    {
+        workspace_ = workspace;
+        workspace_bytes_ = bytes;
+    }
+    size_t GetWorkspaceSize() const
+    {
+        size_t bytes = 0;
+        Check(ascq_matmul_w8a8_workspace_size(&desc_, &bytes));
+        return bytes;
+    }
+    void IterateAll(const DeviceTensor<CType>& c, void* stream = nullptr)
+    {
+        Check(ascq_matmul_w8a8(&desc_, c.GetPhyAddr(), a_, b_, bias_, quant_, tok_, workspace_, workspace_bytes_,
+                               stream));
+    }
+    const ascq_matmul_desc& Desc() const { return desc_; }
+
+private:
+    ascq_matmul_desc desc_;
+    const void* a_ = nullptr;
+    const void* b_ = nullptr;
+    const void* bias_ = nullptr;
+    const void* quant_ = nullptr;
+    const void* tok_ = nullptr;
+    void* workspace_ = nullptr;
+    size_t workspace_bytes_ = 0;
+};
+
+}  // namespace ascq
+
+#endif  // ASCQ_ASCENDC_HPP

@@ -1,0 +1,284 @@
+// Drives the HIP library through the C++ host mirror (include/ascq_ascendc.hpp) the way a reference user drives
+// AscendC::AscendQuant / AscendDequant / AscendAntiQuant / Matmul, and compares every result bit-for-bit with the CPU
+// oracle.  Host code only: device memory comes from the HIP runtime, the kernels from libascq.so.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "../../include/ascq_ascendc.hpp"
+#include "../../oracle/ascq_oracle.h"
+
+namespace {
+
+int g_failed = 0;
+
+#define HIP_OK(expr)                                                                    \
+    do {                                                                                \
+        hipError_t e_ = (expr);                                                         \
+        if (e_ != hipSuccess) {                                                         \
+            std::fprintf(stderr, "%s failed: %s\n", #expr, hipGetErrorString(e_));      \
+            std::exit(2);                                                               \
+        }                                                                               \
+    } while (0)
+
+struct Rng {  // SplitMix64
+    uint64_t s;
+    uint64_t next()
+    {
+        uint64_t z = (s += 0x9E3779B97F4A7C15ull);
+        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+        z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+        return z ^ (z >> 31);
+    }
+    float uniform(float lo, float hi) { return lo + (hi - lo) * static_cast<float>(next() >> 40) / 16777216.0f; }
+    int integer(int lo, int hi) { return lo + static_cast<int>(next() % static_cast<uint64_t>(hi - lo + 1)); }
+};
+
+template <typename T>
+class DeviceBuffer {
+public:
+    explicit DeviceBuffer(size_t count) : count_(count) { HIP_OK(hipMalloc(&ptr_, count * sizeof(T) + 16)); }
+    DeviceBuffer(const std::vector<T>& host) : DeviceBuffer(host.size())
+    {
+        HIP_OK(hipMemcpy(ptr_, host.data(), host.size() * sizeof(T), hipMemcpyHostToDevice));
+    }
+    ~DeviceBuffer() { (void)hipFree(ptr_); }
+    template <typename U>
+    ascq::DeviceTensor<U> view(uint32_t size) const
+    {
+        return ascq::DeviceTensor<U>(static_cast<U*>(ptr_), size);
+    }
+    std::vector<T> download() const
+    {
+        std::vector<T> h(count_);
+        HIP_OK(hipDeviceSynchronize());
+        HIP_OK(hipMemcpy(h.data(), ptr_, count_ * sizeof(T), hipMemcpyDeviceToHost));
+        return h;
+    }
+
+private:
+    void* ptr_ = nullptr;
+    size_t count_;
+};
+
+template <typename T>
+void expect_equal(const char* what, const std::vector<T>& got, const std::vector<T>& want)
+{
+    size_t bad = 0;
+    for (size_t i = 0; i < want.size(); ++i) bad += got[i] != want[i];
+    std::printf("[%s] %s: %zu of %zu elements differ\n", bad ? "FAIL" : " ok ", what, bad, want.size());
+    std::fflush(stdout);
+    g_failed += bad != 0;
+}
+
+std::vector<uint16_t> random_halves(Rng& r, size_t n, float lo, float hi)
+{
+    std::vector<uint16_t> v(n);
+    for (auto& e : v) e = orc_f32_to_f16(r.uniform(lo, hi));
+    return v;
+}
+
+void test_quant_per_channel()
+{
+    std::printf("[case] AscendQuant<half> per channel 64x256\n");
+    Rng r{1};
+    const uint32_t m = 64, n = 256;
+    auto x = random_halves(r, m * n, -6.0f, 6.0f), s = random_halves(r, n, 5.0f, 40.0f), o = random_halves(r, n, -3.0f, 3.0f);
+    DeviceBuffer<uint16_t> dx(x), ds(s), dof(o);
+    DeviceBuffer<int8_t> dq(m * n);
+    ascq::AscendQuant<ascq::half>(dq.view<int8_t>(m * n), dx.view<ascq::half>(m * n), ds.view<ascq::half>(n),
+                                  dof.view<ascq::half>(n), n, n, m * n);
+    ascq_quant_desc d{};
+    d.policy = ASCQ_PER_CHANNEL;
+    d.src_dtype = d.scale_dtype = ASCQ_F16;
+    d.compute = ASCQ_COMPUTE_F16;
+    d.round_mode = ASCQ_CAST_RINT;
+    d.offset_kind = ASCQ_OFFSET_TENSOR;
+    d.m = m;
+    d.n = n;
+    d.cal_count = m * n;
+    std::vector<int8_t> want(m * n);
+    orc_quant(&d, want.data(), x.data(), s.data(), o.data());
+    expect_equal("AscendQuant per channel", dq.download(), want);
+
+    std::printf("[case] AscendQuant<half> per tensor 1024\n");
+    ascq::AscendQuant<ascq::half>(dq.view<int8_t>(1024), dx.view<ascq::half>(1024), 2.0f, 0.9f, 1024);
+    d = ascq_quant_desc{};
+    d.policy = ASCQ_PER_TENSOR;
+    d.src_dtype = d.scale_dtype = ASCQ_F16;
+    d.compute = ASCQ_COMPUTE_F16;
+    d.round_mode = ASCQ_CAST_RINT;
+    d.offset_kind = ASCQ_OFFSET_SCALAR;
+    d.scale = 2.0f;
+    d.offset = 0.9f;
+    d.m = 1;
+    d.n = d.cal_count = 1024;
+    want.assign(1024, 0);
+    orc_quant(&d, want.data(), x.data(), nullptr, nullptr);
+    auto got = dq.download();
+    got.resize(1024);
+    expect_equal("AscendQuant per tensor", got, want);
+}
+
+void test_dequant()
+{
+    std::printf("[case] AscendDequant<bfloat16_t, float, MULTI_ROW> 32x40, calCount 36\n");
+    Rng r{2};
+    const uint32_t m = 32, n = 40, cal = 36;
+    std::vector<int32_t> src(m * n);
+    for (auto& e : src) e = r.integer(-(1 << 20), 1 << 20);
+    std::vector<float> sc(n);
+    for (auto& e : sc) e = r.uniform(1e-5f, 1e-3f);
+    const uint32_t stride = ascq_dequant_dst_stride(ASCQ_BF16, n);
+    DeviceBuffer<int32_t> dsrc(src);
+    DeviceBuffer<float> dsc(sc);
+    std::vector<uint16_t> init(m * stride, 0x7FC0);
+    DeviceBuffer<uint16_t> ddst(init);
+    ascq::AscendDequant<ascq::bfloat16_t, float, ascq::DeQuantMode::DEQUANT_WITH_MULTI_ROW>(
+        ddst.view<ascq::bfloat16_t>(m * stride), dsrc.view<int32_t>(m * n), dsc.view<float>(n),
+        ascq::DequantParams{m, n, cal});
+    ascq_dequant_desc d{};
+    d.policy = ASCQ_PER_CHANNEL;
+    d.src_dtype = ASCQ_I32;
+    d.scale_dtype = ASCQ_F32;
+    d.dst_dtype = ASCQ_BF16;
+    d.mode = ASCQ_DEQUANT_WITH_MULTI_ROW;
+    d.m = m;
+    d.n = n;
+    d.cal_count = cal;
+    std::vector<uint16_t> want(init);
+    orc_dequant(&d, want.data(), src.data(), sc.data());
+    expect_equal("AscendDequant", ddst.download(), want);
+}
+
+void test_antiquant()
+{
+    std::printf("[case] AscendAntiQuant<int8_t, half, false> 64x128, 2 groups\n");
+    Rng r{3};
+    const uint32_t k = 64, n = 128, groups = 2;
+    std::vector<int8_t> w(k * n);
+    for (auto& e : w) e = static_cast<int8_t>(r.integer(-128, 127));
+    auto sc = random_halves(r, groups * n, 1e-3f, 1e-1f);
+    std::vector<uint16_t> of(groups * n);
+    for (auto& e : of) e = orc_f32_to_f16(static_cast<float>(r.integer(-8, 8)));
+    DeviceBuffer<int8_t> dw(w);
+    DeviceBuffer<uint16_t> dsc(sc), dof(of), ddst(k * n);
+    ascq::AntiQuantShapeInfo info{groups, n, groups, n};
+    ascq::AscendAntiQuant<int8_t, ascq::half, false>(ddst.view<ascq::half>(k * n), dw.view<int8_t>(k * n),
+                                                     dof.view<ascq::half>(groups * n), dsc.view<ascq::half>(groups * n),
+                                                     k, info);
+    ascq_antiquant_desc d{};
+    d.src_dtype = ASCQ_I8;
+    d.dst_dtype = ASCQ_F16;
+    d.has_offset = 1;
+    d.k = k;
+    d.n = n;
+    d.offset_height = d.scale_height = groups;
+    d.offset_width = d.scale_width = n;
+    std::vector<uint16_t> want(k * n);
+    orc_antiquant(&d, want.data(), w.data(), of.data(), sc.data());
+    expect_equal("AscendAntiQuant", ddst.download(), want);
+}
+
+void test_matmul()
+{
+    Rng r{4};
+    const uint32_t m = 96, n = 160, k = 256;
+    std::vector<int8_t> a(m * k), b(k * n);
+    for (auto& e : a) e = static_cast<int8_t>(r.integer(-127, 127));
+    for (auto& e : b) e = static_cast<int8_t>(r.integer(-127, 127));
+    std::vector<float> cs(n), ts(m);
+    for (auto& e : cs) e = r.uniform(1e-4f, 1e-2f);
+    for (auto& e : ts) e = r.uniform(1e-3f, 1e-1f);
+    std::vector<int32_t> bias(n);
+    for (auto& e : bias) e = r.integer(-1000, 1000);
+    DeviceBuffer<int8_t> da(a), db(b);
+    DeviceBuffer<float> dcs(cs), dts(ts);
+    DeviceBuffer<int32_t> dbias(bias);
+
+    std::printf("[case] Matmul<bfloat16_t> 96x160x256, SetQuantVector(float) + token scale\n");
+    {
+        DeviceBuffer<uint16_t> dc(m * n);
+        ascq::Matmul<ascq::bfloat16_t> mm(m, n, k);
+        mm.SetTensorA(da.view<int8_t>(m * k));
+        mm.SetTensorB(db.view<int8_t>(k * n));
+        mm.SetQuantVector(dcs.view<float>(n));
+        mm.SetTokenScale(dts.view<float>(m));
+        mm.IterateAll(dc.view<ascq::bfloat16_t>(m * n));
+        std::vector<uint16_t> want(m * n);
+        orc_matmul_w8a8(&mm.Desc(), want.data(), a.data(), b.data(), nullptr, cs.data(), ts.data());
+        expect_equal("Matmul bf16 epilogue", dc.download(), want);
+    }
+    std::printf("[case] Matmul<half> 96x160x256, int32 bias + SetQuantScalar(uint64)\n");
+    {
+        DeviceBuffer<uint16_t> dc(m * n);
+        ascq::Matmul<ascq::half> mm(m, n, k);
+        mm.SetTensorA(da.view<int8_t>(m * k));
+        mm.SetTensorB(db.view<int8_t>(k * n));
+        mm.SetBias(dbias.view<int32_t>(n));
+        mm.SetQuantScalar(ascq_pack_quant_param(0.00123f, 0, 0));
+        mm.IterateAll(dc.view<ascq::half>(m * n));
+        std::vector<uint16_t> want(m * n);
+        orc_matmul_w8a8(&mm.Desc(), want.data(), a.data(), b.data(), bias.data(), nullptr, nullptr);
+        expect_equal("Matmul DEQF16 epilogue", dc.download(), want);
+    }
+    std::printf("[case] Matmul<int32_t> 96x160x256, no quant\n");
+    {
+        DeviceBuffer<int32_t> dc(m * n);
+        ascq::Matmul<int32_t> mm(m, n, k);
+        mm.SetTensorA(da.view<int8_t>(m * k));
+        mm.SetTensorB(db.view<int8_t>(k * n));
+        mm.IterateAll(dc.view<int32_t>(m * n));
+        std::vector<int32_t> want(m * n);
+        orc_matmul_w8a8(&mm.Desc(), want.data(), a.data(), b.data(), nullptr, nullptr, nullptr);
+        expect_equal("Matmul int32", dc.download(), want);
+    }
+}
+
+void test_errors()
+{
+    std::printf("[case] argument errors surface as ascq::Error\n");
+    DeviceBuffer<uint16_t> x(64);
+    DeviceBuffer<int8_t> q(64);
+    bool threw = false;
+    try {
+        ascq::AscendQuant<ascq::half>(q.view<int8_t>(64), x.view<ascq::half>(64), x.view<ascq::half>(32),
+                                      x.view<ascq::half>(16), 32, 16, 64);
+    } catch (const ascq::Error& e) {
+        threw = e.status() == ASCQ_EINVAL;
+    }
+    int ok = threw;
+    threw = false;
+    try {
+        ascq::Matmul<ascq::half> mm(16, 16, 16);  // no tensors set
+        mm.SetQuantScalar(ascq_pack_quant_param(1.0f, 0, 0));
+        mm.IterateAll(x.view<ascq::half>(64));
+    } catch (const ascq::Error& e) {
+        threw = e.status() != ASCQ_OK && std::strlen(e.what()) > 0;
+    }
+    ok += threw;
+    std::printf("[%s] error paths: %d of 2 raised\n", ok == 2 ? " ok " : "FAIL", ok);
+    g_failed += ok != 2;
+}
+
+}  // namespace
+
+int main()
+{
+    int ndev = 0;
+    if (hipGetDeviceCount(&ndev) != hipSuccess || ndev == 0) {
+        std::fprintf(stderr, "no GPU\n");
+        return 2;
+    }
+    std::printf("library: %s\n", ascq_version());
+    test_quant_per_channel();
+    test_dequant();
+    test_antiquant();
+    test_matmul();
+    test_errors();
+    std::printf("%s\n", g_failed ? "FAILED" : "ALL PASSED");
+    return g_failed ? 1 : 0;
+}

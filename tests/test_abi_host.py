@@ -182,3 +182,13 @@ def test_pack_quant_param():
     import numpy as np
     w = L.ascq_pack_quant_param(0.1, 5, 1)
     assert (w & 0xFFFFFFFF) == int(np.float32(0.1).view(np.uint32)) and (w >> 37) & 0x1FF == 5 and (w >> 46) & 1 == 1
+
+
+def test_cpp_host_mirror_header_compiles_standalone(tmp_path):
+    """include/ascq_ascendc.hpp is plain C++17 on top of ascq.h: it must compile with the host compiler alone."""
+    import subprocess
+    src = tmp_path / "t.cpp"
+    src.write_text('#include "ascq_ascendc.hpp"\n'
+                   'int main() { ascq::Matmul<ascq::bfloat16_t> mm(1, 1, 1); return mm.Desc().m == 1 ? 0 : 1; }\n')
+    inc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
+    subprocess.check_call(["g++", "-std=c++17", "-Wall", "-Wextra", "-Werror", "-fsyntax-only", "-I", inc, str(src)])
