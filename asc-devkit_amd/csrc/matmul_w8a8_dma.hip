@@ -19,6 +19,8 @@
 // LDS layouts (all reads and writes conflict-free, measured at ~220-250 B/clk/CU):
 //   A stage: row r = 128 bytes = 8 pieces of 16; piece c is stored at position c ^ ((r >> 1) & 7).
 //   B stage: row k = 256 bytes = 16 pieces of 16; piece q is stored at position q ^ (2 * (k & 7)).
+#include <type_traits>
+
 #include "matmul_w8a8.h"
 
 namespace ascq {
@@ -42,15 +44,15 @@ __device__ __forceinline__ uint32_t to_bits16(float v)
     }
 }
 
-__device__ __forceinline__ float epi_value(const EpiParams& e, int32_t acc, const ChannelQ& q, float tok,
-                                           float bias_post)
+template <bool kBiasPost, bool kGelu>
+__device__ __forceinline__ float epi_value(int32_t acc, float chan, float tok, float bias_post)
 {
-    float v = static_cast<float>(acc) * q.s;
+    float v = static_cast<float>(acc) * chan;
     v = v * tok;  // tok is 1.0f without a token scale: an exact identity
-    if (e.bias_kind >= ASCQ_MM_BIAS_F32_POST) {
+    if constexpr (kBiasPost) {
         v = v + bias_post;
     }
-    if (e.activation == ASCQ_MM_ACT_FASTER_GELU) {
+    if constexpr (kGelu) {
         v = faster_gelu(v);
     }
     return v;
@@ -72,6 +74,7 @@ __global__ __launch_bounds__(kThreads) void gemm_dma_kernel(GemmParams p, int gr
     __shared__ __attribute__((aligned(1024))) char B0[BK * BN];
     __shared__ __attribute__((aligned(1024))) char A1[BM * BK];
     __shared__ __attribute__((aligned(1024))) char B1[BK * BN];
+    __shared__ __attribute__((aligned(16))) float TS[BM];  // token scales of the tile's rows (1.0f when there are none)
 
     const uint32_t total = p.tiles_m * p.tiles_n;
     const uint32_t t = xcd_remap(blockIdx.x, total);
@@ -119,6 +122,11 @@ __global__ __launch_bounds__(kThreads) void gemm_dma_kernel(GemmParams p, int gr
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t wm = wave / kWN, wn = wave % kWN;
+    if (tid < BM) {
+        // read by the epilogue only; the barriers of the main loop order this store before those reads
+        const uint32_t row = row0 + tid;
+        TS[tid] = (p.epi.has_tok && row < row_end) ? p.epi.tok_scale[row] : 1.0f;
+    }
 
     // ---- DMA sources: 4 A and 4 B instructions per wavefront and K step; lane owns LDS slot (instr * 64 + lane)
     uint32_t aoff[4], boff[kBInstr];
@@ -249,54 +257,92 @@ __global__ __launch_bounds__(kThreads) void gemm_dma_kernel(GemmParams p, int gr
     const EpiParams& e = p.epi;
     auto run = [&](auto tag) {
         constexpr int kOut = decltype(tag)::value;
+        const uint32_t colw = n0 + wn * (TJ * 32u);  // first column of this wavefront
+        ChannelQ q[TJ];
+        float bias_post[TJ];
+        int32_t bias_pre[TJ];
+        bool cvalid[TJ];
 #pragma unroll
         for (int j = 0; j < TJ; ++j) {
-            const uint32_t col = n0 + (wn * TJ + j) * 32u + lrow;
-            const bool cvalid = col < N;
-            ChannelQ q{1.0f, 0, 1};
-            float bias_post = 0.0f;
-            int32_t bias_pre = 0;
-            if (cvalid) {
-                q = load_channel_q(e, chan_off + col);
-                bias_post = load_bias_post(e, chan_off + col);
+            const uint32_t col = colw + j * 32u + lrow;
+            cvalid[j] = col < N;
+            q[j] = ChannelQ{1.0f, 0, 1};
+            bias_post[j] = 0.0f;
+            bias_pre[j] = 0;
+            if (cvalid[j]) {
+                q[j] = load_channel_q(e, chan_off + col);
+                bias_post[j] = load_bias_post(e, chan_off + col);
                 if (e.bias_kind == ASCQ_MM_BIAS_I32_PRE) {
-                    bias_pre = static_cast<const int32_t*>(e.bias)[chan_off + col];
+                    bias_pre[j] = static_cast<const int32_t*>(e.bias)[chan_off + col];
                 }
             }
-#pragma unroll
+        }
+        // The uniform choices (post-dequant bias, activation) are made once, outside the element loops, so that each
+        // wavefront runs one compact straight-line epilogue.
+        auto store_all = [&](auto bias_tag, auto gelu_tag) {
+            constexpr bool kBiasPost = decltype(bias_tag)::value;
+            constexpr bool kGelu = decltype(gelu_tag)::value;
+            (void)kBiasPost;
+            (void)kGelu;
+    #pragma unroll
             for (int i = 0; i < TI; ++i) {
-                const uint32_t rbase = row0 + (wm * TI + i) * 32u + 4u * g;
-                if constexpr (kOut == ASCQ_BF16 || kOut == ASCQ_F16) {
-                    // two adjacent columns per dword store: even lanes keep row r, odd lanes row r + 1
-                    const bool odd = (lane & 1u) != 0;
-#pragma unroll
-                    for (int r = 0; r < 16; r += 2) {
-                        const uint32_t ra = rbase + 8u * (r >> 2) + (r & 3);
-                        const float ta = (e.has_tok && ra < row_end) ? e.tok_scale[ra] : 1.0f;
-                        const float tb = (e.has_tok && ra + 1 < row_end) ? e.tok_scale[ra + 1] : 1.0f;
-                        const uint32_t ha = to_bits16<kOut>(epi_value(e, acc[i][j][r] + bias_pre, q, ta, bias_post));
-                        const uint32_t hb = to_bits16<kOut>(epi_value(e, acc[i][j][r + 1] + bias_pre, q, tb, bias_post));
-                        const uint32_t send = odd ? ha : hb;
-                        const uint32_t recv = static_cast<uint32_t>(
-                            __builtin_amdgcn_mov_dpp(static_cast<int>(send), 0xB1, 0xF, 0xF, true));  // lane ^ 1
-                        const uint32_t word = odd ? (recv | (hb << 16)) : (ha | (recv << 16));
-                        const uint32_t row = odd ? ra + 1 : ra;
-                        if (cvalid && row < row_end) {
-                            *reinterpret_cast<uint32_t*>(static_cast<uint16_t*>(e.c) +
-                                                         static_cast<size_t>(row) * e.ldc + (col & ~1u)) = word;
-                        }
-                    }
-                } else {
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const uint32_t row = rbase + 8u * (r >> 2) + (r & 3);
-                        if (cvalid && row < row_end) {
-                            const float tok = e.has_tok ? e.tok_scale[row] : 1.0f;
-                            epilogue_store<kOut>(e, row, col, acc[i][j][r] + bias_pre, q, tok, bias_post);
+                const uint32_t lbase = (wm * TI + i) * 32u + 4u * g;  // row inside the tile of register 0
+    #pragma unroll
+                for (int rq = 0; rq < 4; ++rq) {
+                    const f32x4 tok4 = *reinterpret_cast<const f32x4*>(&TS[lbase + 8u * rq]);
+    #pragma unroll
+                    for (int rr = 0; rr < 4; ++rr) {
+                        const int r = 4 * rq + rr;
+                        const uint32_t row = row0 + lbase + 8u * rq + rr;
+                        if constexpr (kOut == ASCQ_BF16 || kOut == ASCQ_F16) {
+                            // One dword store per lane covers a full 128-byte line per row: even lanes write columns
+                            // (l, l+1) of the first 32-column block, odd lanes columns (l-1, l) of the second one.
+                            static_assert(TJ == 2, "the paired store assumes two column blocks per wavefront");
+                            const bool odd = (lane & 1u) != 0;
+                            const uint32_t h0 =
+                                to_bits16<kOut>(
+                                    epi_value<kBiasPost, kGelu>(acc[i][0][r] + bias_pre[0], q[0].s, tok4[rr], bias_post[0]));
+                            const uint32_t h1 =
+                                to_bits16<kOut>(
+                                    epi_value<kBiasPost, kGelu>(acc[i][1][r] + bias_pre[1], q[1].s, tok4[rr], bias_post[1]));
+                            const uint32_t send = odd ? h0 : h1;
+                            const uint32_t recv = static_cast<uint32_t>(
+                                __builtin_amdgcn_mov_dpp(static_cast<int>(send), 0xB1, 0xF, 0xF, true));  // lane ^ 1
+                            const uint32_t word = odd ? (recv | (h1 << 16)) : (h0 | (recv << 16));
+                            const uint32_t col = odd ? colw + 32u + (lrow - 1u) : colw + lrow;
+                            if (row < row_end && col < N) {
+                                *reinterpret_cast<uint32_t*>(static_cast<uint16_t*>(e.c) +
+                                                             static_cast<size_t>(row) * e.ldc + col) = word;
+                            }
+                        } else {
+    #pragma unroll
+                            for (int j = 0; j < TJ; ++j) {
+                                if (cvalid[j] && row < row_end) {
+                                    epilogue_store<kOut>(e, row, colw + j * 32u + lrow, acc[i][j][r] + bias_pre[j], q[j],
+                                                         tok4[rr], bias_post[j]);
+                                }
+                            }
                         }
                     }
                 }
             }
+        };
+        if constexpr (kOut == ASCQ_BF16 || kOut == ASCQ_F16) {
+            const bool bias_post_on = e.bias_kind >= ASCQ_MM_BIAS_F32_POST;
+            const bool gelu_on = e.activation == ASCQ_MM_ACT_FASTER_GELU;
+            if (gelu_on) {
+                if (bias_post_on) {
+                    store_all(std::true_type{}, std::true_type{});
+                } else {
+                    store_all(std::false_type{}, std::true_type{});
+                }
+            } else if (bias_post_on) {
+                store_all(std::true_type{}, std::false_type{});
+            } else {
+                store_all(std::false_type{}, std::false_type{});
+            }
+        } else {
+            store_all(std::false_type{}, std::false_type{});  // the generic store reads both choices at run time
         }
     };
     dispatch_out(e, run);
