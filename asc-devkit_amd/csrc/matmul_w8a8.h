@@ -158,5 +158,7 @@ __device__ __forceinline__ uint32_t xcd_remap(uint32_t pid, uint32_t total)
 // Large-M kernel built on direct-to-LDS loads and transposing LDS reads (matmul_w8a8_dma.hip).
 bool gemm_dma_supported(const GemmParams& p);
 int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st);
+uint32_t gemm_dma_skinny_splits(uint32_t m, uint32_t n, uint32_t k);
+int launch_gemm_dma_skinny(GemmParams& p, void* workspace, size_t workspace_bytes, hipStream_t st);
 
 }  // namespace ascq

@@ -531,6 +531,9 @@ bool fast_path_ok(const ascq_matmul_desc* d, const void* a, const void* b)
     return d->n % 8 == 0 && d->n >= 8 && (reinterpret_cast<uintptr_t>(b) & 7u) == 0;
 }
 
+// Up to this many rows the 128 x 128 direct-to-LDS kernel (K split over workgroups) is used when the shape allows.
+constexpr uint32_t kSkinnyMaxM = 512;
+
 // split-K factor for the small-M kernel: enough workgroups to cover the chip ~3 times
 uint32_t pick_k_splits(uint32_t n, uint32_t k)
 {
@@ -553,6 +556,13 @@ extern "C" int ascq_matmul_w8a8_workspace_size(const ascq_matmul_desc* d, size_t
     *bytes = 0;
     if (d->m <= 32 && !d->trans_a && pick_k_splits(d->n, d->k) > 1) {
         *bytes = static_cast<size_t>(d->m) * d->n * sizeof(int32_t);
+    }
+    if (d->m <= kSkinnyMaxM && !d->trans_a && !d->trans_b && d->k % 128 == 0 && d->n % 16 == 0) {
+        const size_t need =
+            static_cast<size_t>(gemm_dma_skinny_splits(d->m, d->n, d->k)) * d->m * d->n * sizeof(int32_t);
+        if (need > *bytes && need > static_cast<size_t>(d->m) * d->n * sizeof(int32_t)) {
+            *bytes = need;
+        }
     }
     return ASCQ_OK;
 }
@@ -581,6 +591,9 @@ extern "C" int ascq_matmul_w8a8(const ascq_matmul_desc* d, void* c, const void* 
         if (blocks > 65536) blocks = 65536;
         gemm_generic_kernel<<<static_cast<uint32_t>(blocks), kThreads, 0, st>>>(p, d->trans_a, d->trans_b);
         return launch_status("ascq_matmul_w8a8 (generic)");
+    }
+    if (d->m <= kSkinnyMaxM && !d->trans_b && gemm_dma_supported(p)) {
+        return launch_gemm_dma_skinny(p, workspace, workspace_bytes, st);
     }
     if (d->m <= 32) {
         const uint32_t splits = pick_k_splits(d->n, d->k);

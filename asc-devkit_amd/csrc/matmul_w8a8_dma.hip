@@ -27,7 +27,7 @@ namespace ascq {
 namespace {
 
 constexpr int kThreads = 512;
-constexpr int BM = 256, BK = 128;
+constexpr int BK = 128;
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef __attribute__((address_space(1))) const void* gptr_t;
@@ -58,18 +58,24 @@ __device__ __forceinline__ float epi_value(int32_t acc, float chan, float tok, f
     return v;
 }
 
-// BN = 256: wavefronts 2 (M) x 4 (N), 128 x 64 each.  BN = 128: wavefronts 4 (M) x 2 (N), 64 x 64 each (used for the
-// last, partially filled round of tiles: half-width tiles finish it in half the time).
-template <int BN>
-__global__ __launch_bounds__(kThreads) void gemm_dma_kernel(GemmParams p, int grouped, uint32_t col_begin)
+// 256 x 256: wavefronts 2 (M) x 4 (N), 128 x 64 each.  256 x 128: wavefronts 4 (M) x 2 (N), 64 x 64 each (used for the
+// last, partially filled round of tiles: half-width tiles finish it in half the time).  128 x 128: 32 x 64 per
+// wavefront, 64 KiB of LDS so that two workgroups share a CU; with kSplitK the K range is divided over blockIdx.y and
+// the int32 partial tiles go to a workspace [split][m][n] that a second kernel sums (small M: the weights are read
+// once, by enough workgroups to fill the chip).
+template <int BM, int BN, bool kSplitK>
+__global__ __launch_bounds__(kThreads, (BM * BK + BK * BN) * 2 <= 65536 ? 2 : 1) void gemm_dma_kernel(
+    GemmParams p, int grouped, uint32_t col_begin)
 {
     constexpr int kWN = BN / 64;            // wavefronts along N
     constexpr int kWM = 8 / kWN;            // wavefronts along M
     constexpr int TI = BM / 32 / kWM;       // 32x32 blocks per wavefront along M
     constexpr int TJ = 2;                   // and along N
     constexpr int kPieces = BN / 16;        // 16-byte pieces per B row
+    constexpr int kAInstr = BM * BK / 1024 / 8;  // A DMA instructions per wavefront and K step
     constexpr int kBInstr = BK * BN / 1024 / 8;  // B DMA instructions per wavefront and K step
     constexpr int kKsB = 32 * BN;           // bytes of B per K sub-step of 32 rows
+    static_assert(TI >= 1 && TI * 32 * kWM == BM && kAInstr >= 1, "tile shape does not fit eight wavefronts");
     __shared__ __attribute__((aligned(1024))) char A0[BM * BK];
     __shared__ __attribute__((aligned(1024))) char B0[BK * BN];
     __shared__ __attribute__((aligned(1024))) char A1[BM * BK];
@@ -129,10 +135,10 @@ __global__ __launch_bounds__(kThreads) void gemm_dma_kernel(GemmParams p, int gr
     }
 
     // ---- DMA sources: 4 A and 4 B instructions per wavefront and K step; lane owns LDS slot (instr * 64 + lane)
-    uint32_t aoff[4], boff[kBInstr];
+    uint32_t aoff[kAInstr], boff[kBInstr];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-        const uint32_t s = (wave * 4 + u) * 64 + lane;
+    for (int u = 0; u < kAInstr; ++u) {
+        const uint32_t s = (wave * kAInstr + u) * 64 + lane;
         const uint32_t r = s >> 3, c = (s & 7u) ^ ((r >> 1) & 7u);
         uint32_t row = row0 + r;
         row = row < row_end ? row : row_end - 1;  // rows past the end are never stored: any valid row will do
@@ -148,14 +154,21 @@ __global__ __launch_bounds__(kThreads) void gemm_dma_kernel(GemmParams p, int gr
         col = col + 16u <= N ? col : N - 16u;      // columns past the end are never stored
         boff[u] = kb * N + (col - n0);
     }
-    const int8_t* Abase = p.a + static_cast<size_t>(row0) * K;
-    const int8_t* Bbase = Bmat + n0;
+    // K range of this workgroup, in steps of BK
+    uint32_t s_begin = 0, steps = K / BK;
+    if constexpr (kSplitK) {
+        s_begin = steps * blockIdx.y / p.k_splits;
+        steps = steps * (blockIdx.y + 1u) / p.k_splits - s_begin;
+    }
+    const int8_t* Abase = p.a + static_cast<size_t>(row0) * K + static_cast<size_t>(s_begin) * BK;
+    const int8_t* Bbase = Bmat + n0 + static_cast<size_t>(s_begin) * BK * N;
     auto issue = [&](uint32_t k0, char* As, char* Bs) {
         const int8_t* ab = Abase + k0;
         const int8_t* bb = Bbase + static_cast<size_t>(k0) * N;
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            __builtin_amdgcn_global_load_lds((gptr_t)(ab + aoff[u]), (lds_ptr_t)(As + (wave * 4 + u) * 1024), 16, 0, 0);
+        for (int u = 0; u < kAInstr; ++u) {
+            __builtin_amdgcn_global_load_lds((gptr_t)(ab + aoff[u]), (lds_ptr_t)(As + (wave * kAInstr + u) * 1024), 16,
+                                             0, 0);
         }
 #pragma unroll
         for (int u = 0; u < kBInstr; ++u) {
@@ -232,8 +245,9 @@ __global__ __launch_bounds__(kThreads) void gemm_dma_kernel(GemmParams p, int gr
         }
     };
 
-    const uint32_t steps = K / BK;
-    issue(0, A0, B0);
+    if (steps != 0) {
+        issue(0, A0, B0);
+    }
     asm volatile("s_waitcnt vmcnt(0)");
     __syncthreads();
     uint32_t s = 0;
@@ -254,6 +268,24 @@ __global__ __launch_bounds__(kThreads) void gemm_dma_kernel(GemmParams p, int gr
     }
 
     // ---- epilogue: register r of lane l in a 32x32 block is row 8*(r/4) + 4*(l/32) + r%4, column l%32
+    if constexpr (kSplitK) {
+        int32_t* part = p.partial + static_cast<size_t>(blockIdx.y) * p.m * N;
+#pragma unroll
+        for (int i = 0; i < TI; ++i) {
+#pragma unroll
+            for (int j = 0; j < TJ; ++j) {
+                const uint32_t col = n0 + (wn * TJ + j) * 32u + lrow;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const uint32_t row = row0 + (wm * TI + i) * 32u + 8u * (r >> 2) + 4u * g + (r & 3);
+                    if (row < row_end && col < N) {
+                        part[static_cast<size_t>(row) * N + col] = acc[i][j][r];
+                    }
+                }
+            }
+        }
+        return;
+    }
     const EpiParams& e = p.epi;
     auto run = [&](auto tag) {
         constexpr int kOut = decltype(tag)::value;
@@ -348,6 +380,36 @@ __global__ __launch_bounds__(kThreads) void gemm_dma_kernel(GemmParams p, int gr
     dispatch_out(e, run);
 }
 
+// Second pass of the split-K path: sums the int32 partial tiles [split][m][n] in split order (integer addition: exact in
+// any order) and applies the epilogue.  One lane = four consecutive columns.
+__global__ __launch_bounds__(256) void splitk_sum_epilogue_kernel(GemmParams p)
+{
+    const size_t quads = static_cast<size_t>(p.m) * p.n / 4u;
+    const size_t plane = static_cast<size_t>(p.m) * p.n;
+    for (size_t qd = static_cast<size_t>(blockIdx.x) * 256u + threadIdx.x; qd < quads;
+         qd += static_cast<size_t>(gridDim.x) * 256u) {
+        const size_t idx = qd * 4u;
+        i32x4 acc = *reinterpret_cast<const i32x4*>(p.partial + idx);
+        for (uint32_t sp = 1; sp < p.k_splits; ++sp) {
+            const i32x4 v = *reinterpret_cast<const i32x4*>(p.partial + sp * plane + idx);
+            acc += v;
+        }
+        const size_t row = idx / p.n, col = idx % p.n;
+        const float tok = p.epi.has_tok ? p.epi.tok_scale[row] : 1.0f;
+        dispatch_out(p.epi, [&](auto tag) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                int32_t a = acc[c];
+                if (p.epi.bias_kind == ASCQ_MM_BIAS_I32_PRE) {
+                    a += static_cast<const int32_t*>(p.epi.bias)[col + c];
+                }
+                epilogue_store<decltype(tag)::value>(p.epi, row, col + c, a, load_channel_q(p.epi, col + c), tok,
+                                                     load_bias_post(p.epi, col + c));
+            }
+        });
+    }
+}
+
 }  // namespace
 
 bool gemm_dma_supported(const GemmParams& p)
@@ -357,7 +419,7 @@ bool gemm_dma_supported(const GemmParams& p)
 
 int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st)
 {
-    p.tiles_m = (p.m + BM - 1) / BM + (grouped ? p.groups : 0u);  // every group adds at most one partial tile
+    p.tiles_m = (p.m + 255u) / 256u + (grouped ? p.groups : 0u);  // every group adds at most one partial tile
     uint32_t tiles_n = (p.n + 255u) / 256u;
     // Tile quantisation: when the last round of 256-wide tiles would fill less than half of the 256 CUs, its
     // columns are computed by a second launch with 128-wide tiles, which finishes that round in about half the time.
@@ -379,15 +441,57 @@ int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st)
         if (narrow_cols) {
             q.n = p.n;  // row pitch stays n; columns >= wide_cols * 256 are simply not assigned to any tile
         }
-        gemm_dma_kernel<256><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(q, grouped ? 1 : 0, 0u);
+        gemm_dma_kernel<256, 256, false><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(q, grouped ? 1 : 0, 0u);
     }
     if (narrow_cols) {
         const uint32_t col_begin = wide_cols * 256u;
         p.tiles_n = (p.n - col_begin + 127u) / 128u;
         const uint32_t t = p.tiles_m * p.tiles_n;
-        gemm_dma_kernel<128><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(p, 0, col_begin);
+        gemm_dma_kernel<256, 128, false><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(p, 0, col_begin);
     }
     return launch_status(grouped ? "ascq_group_matmul_w8a8" : "ascq_matmul_w8a8");
+}
+
+// Split factor of the 128 x 128 kernel: two workgroups per CU when the partial tiles are small next to the weights,
+// one per CU otherwise; never more splits than K steps.
+uint32_t gemm_dma_skinny_splits(uint32_t m, uint32_t n, uint32_t k)
+{
+    const uint32_t tiles = ((m + 127u) / 128u) * ((n + 127u) / 128u);
+    const uint32_t target = m <= 64u ? 512u : 300u;
+    uint32_t s = (target + tiles - 1u) / tiles;
+    const uint32_t steps = k / BK;
+    if (s > steps) s = steps;
+    if (s > 16u) s = 16u;
+    return s ? s : 1u;
+}
+
+// M up to a few hundred rows: 128 x 128 tiles, K split over blockIdx.y when a workspace of
+// splits * m * n * 4 bytes (16-byte aligned) is given.
+int launch_gemm_dma_skinny(GemmParams& p, void* workspace, size_t workspace_bytes, hipStream_t st)
+{
+    p.tiles_m = (p.m + 127u) / 128u;
+    p.tiles_n = (p.n + 127u) / 128u;
+    const uint32_t t = (p.tiles_m * p.tiles_n + 7u) / 8u * 8u;
+    uint32_t splits = gemm_dma_skinny_splits(p.m, p.n, p.k);
+    const size_t need = static_cast<size_t>(splits) * p.m * p.n * sizeof(int32_t);
+    if (splits > 1 && (workspace == nullptr || workspace_bytes < need || !aligned16(workspace))) {
+        splits = 1;
+    }
+    if (splits == 1) {
+        gemm_dma_kernel<128, 128, false><<<t, kThreads, 0, st>>>(p, 0, 0u);
+        return launch_status("ascq_matmul_w8a8");
+    }
+    p.k_splits = splits;
+    p.partial = static_cast<int32_t*>(workspace);
+    gemm_dma_kernel<128, 128, true><<<dim3(t, splits), kThreads, 0, st>>>(p, 0, 0u);
+    int rc = launch_status("ascq_matmul_w8a8 (split-K)");
+    if (rc != ASCQ_OK) {
+        return rc;
+    }
+    size_t blocks = (static_cast<size_t>(p.m) * p.n / 4u + 255u) / 256u;
+    if (blocks > 8192u) blocks = 8192u;
+    splitk_sum_epilogue_kernel<<<static_cast<uint32_t>(blocks), 256, 0, st>>>(p);
+    return launch_status("ascq_matmul_w8a8 (split-K epilogue)");
 }
 
 }  // namespace ascq
