@@ -1,42 +1,59 @@
 // W4A16 weight-only linear for decode: y[m, n] = sum_k x[m, k] * antiquant(w[k, n]) with int4 weights de-quantised in
 // registers (never materialised in memory).
 //
-// The kernel is bound by the HBM read of the packed weights (k * n / 2 bytes).  Layout of the work:
-//   * a lane owns 16 bytes = 32 adjacent columns of a weight row; the 16 lanes of a quarter-wavefront cover 512
-//     columns (256 contiguous bytes) and the four quarters take four different k rows, so one load instruction of a
-//     wavefront reads 4 rows x 256 bytes; 8 such loads are in flight per lane;
-//   * the four wavefronts of a workgroup take different k ranges of the same 512 columns, K is further split over
-//     gridDim.y, so that about 450 workgroups stream the weights;
+// The kernel is bound by the HBM read of the packed weights (k * n / 2 bytes), so it is built as a set of independent
+// streams, one per wavefront, each with its own deep queue of loads:
+//   * the weight matrix is cut into chunks of 32 rows x 512 columns (8 KiB); the chunks, in column-block-major order,
+//     are dealt out in equal contiguous runs to 1024 wavefronts (one per SIMD of the chip), so every SIMD streams the
+//     same number of bytes whatever the shape;
+//   * a wavefront moves a chunk HBM -> LDS with global_load_lds_dwordx4 (no registers, tracked by vmcnt) into a private
+//     ring of three stages: two chunks (plus the matching scale / offset rows and activations) are always in flight
+//     behind the one being computed, independent of register pressure and of where the compiler places its waits;
+//     a lane reads back from LDS exactly the bytes it fetched, so there are no bank conflicts and no barriers at all;
+//   * a lane owns 16 bytes = 32 adjacent columns of a weight row; the 16 lanes of a quarter-wavefront cover the 512
+//     columns and the four quarters take 4 x 8 rows;
 //   * de-quantisation follows AscendAntiQuant<int4b_t, half> exactly: the nibble becomes an exact half via the
-//     0x6400 exponent trick (1024 + u) - 1032, then one rounded half add of the offset and one rounded half
-//     multiply by the scale (packed v_pk_add_f16 / v_pk_mul_f16 on two columns at a time);
-//   * the multiply-accumulate runs on the matrix core instead of the VALU: the 8 de-quantised halves of one dword
-//     are the B operand of v_mfma_f32_16x16x32_f16 as they are (k slot (g, b) = row of quarter g, column b of the
-//     dword); the A operand of output row i carries x[k_g] in slot i and zeros elsewhere, so row i of the result is
-//     the running dot product of column i of the dword.  Rows 0-7 serve one activation row, rows 8-15 a second one;
-//     more activation rows take more MFMAs on the same de-quantised operand.  Accumulation is fp32;
-//   * partial sums are reduced across the wavefronts through LDS and written as fp32; a second small kernel adds
-//     the K-splits in a fixed order and rounds once to half, so results are deterministic.
+//     0x6400 exponent trick (1024 + u, or 1024 + 16 u for the nibbles read 4 bits up, which saves the shift), one
+//     exact packed add / fma turns it into w, then one rounded half add of the offset and one rounded half multiply by
+//     the scale;
+//   * the multiply-accumulate runs on the matrix core: the 8 de-quantised halves of one dword are the B operand of
+//     v_mfma_f32_16x16x32_f16 as they are; the A operand of output row i carries x[k_g] in slot i and zeros elsewhere,
+//     so row i of the result is the running dot product of column i of the dword.  Rows 0-7 serve one activation row,
+//     rows 8-15 a second one; more activation rows take more MFMAs on the same de-quantised operand (fp32 sums);
+//   * when a wavefront's run leaves a column block (and at its end) the accumulators go to a workspace as they lie in
+//     registers; a second kernel adds, for every output, the pieces of all wavefronts that worked on its column block
+//     in ascending k order and rounds once to half, so results are deterministic.
+#include <type_traits>
+
 #include "ascq_common.h"
 #include "ascq_device.h"
 
 namespace ascq {
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kColsPerBlock = 512;
-constexpr int kRowsPerPass = 128;
+constexpr int kThreads = 256;          // four independent wavefronts per workgroup
+constexpr uint32_t kColsPerBlock = 512;
+constexpr uint32_t kChunkRows = 32;
+constexpr uint32_t kMaxWaves = 1024;   // 256 compute units x 4 SIMDs
+constexpr int kMaxPairs = 4;           // activation-row pairs per pass over the weights
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef __attribute__((address_space(1))) const void* gptr_t;
 
 struct W4Params {
     const uint16_t* x;
     const uint8_t* w;
     const uint16_t* scale;
     const uint16_t* offset;
-    float* partial;  // [splits, m, n]
+    float* partial;  // [waves][max_seg][pairs][16 registers][64 lanes]
     uint16_t* y;
     uint32_t m, n, k, group_size, has_offset;
-    uint32_t splits, k_per_split;
-    uint32_t m0;  // first activation row handled by this launch
+    uint32_t m0;                // first activation row of this pass
+    uint32_t waves;             // streams
+    uint32_t chunks_per_block;  // k / 32
+    uint32_t total_chunks;      // column blocks * chunks_per_block
+    uint32_t max_seg;           // column blocks one stream can touch
+    uint32_t per, rem;          // total_chunks = waves * per + rem
 };
 
 __device__ __forceinline__ f16x2 bits_to_h2(uint32_t b)
@@ -55,25 +72,80 @@ __device__ __forceinline__ void pair_up(u32x4 v, f16x2 (&out)[4])
     out[3] = bits_to_h2(__builtin_amdgcn_perm(v[3], v[1], 0x07060302u));
 }
 
-// slot b of the de-quantised operand holds column (b >> 1) + 4 * (b & 1) of the dword
-__device__ __forceinline__ uint32_t slot_to_col(uint32_t b) { return (b >> 1) + 4u * (b & 1u); }
-
-// MP = number of activation-row pairs handled per pass over the weights (m <= 2 * MP).
-// Requires n % 32 == 0, group_size % 32 == 0, k_per_split % 128 == 0.
-template <int MP, bool kHasOffset>
-__global__ __launch_bounds__(kThreads) void w4a16_mfma_kernel(W4Params p)
+// Stream `wave` owns chunks [stream_begin(wave), stream_begin(wave + 1)): the first `rem` streams take per + 1 chunks.
+__device__ __forceinline__ uint32_t stream_begin(const W4Params& p, uint32_t wave)
 {
-    __shared__ float red[4][2][kColsPerBlock];
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    const uint32_t g = lane >> 4, jj = lane & 15u;
-    // Lanes past the last column work on a duplicate of the last 32 columns (their results are never stored): the
-    // MFMA ignores the execution mask, so every lane must hold a valid A operand.
-    uint32_t col0 = blockIdx.x * kColsPerBlock + jj * 32u;
-    col0 = col0 < p.n ? col0 : p.n - 32u;
-    const uint32_t rows_per_wave = p.k_per_split / 4u;
-    const uint32_t kw0 = blockIdx.y * p.k_per_split + wave * rows_per_wave;
-    const size_t row_bytes = p.n / 2;
+    return wave * p.per + (wave < p.rem ? wave : p.rem);
+}
 
+// s_waitcnt vmcnt(n) only (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8)
+#define ASCQ_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | (7 << 4) | (15 << 8))
+
+// MP = number of activation-row pairs handled per pass over the weights (rows m0 .. m0 + 2 MP - 1).
+// Requires n % 32 == 0, k % 32 == 0, group_size % 32 == 0.
+template <int MP, bool kHasOffset>
+__global__ __launch_bounds__(kThreads) void w4a16_stream_kernel(W4Params p)
+{
+    constexpr int kParamInstr = kHasOffset ? 2 : 1;
+    constexpr int kInstr = 8 + kParamInstr + 1;   // 1 KiB DMA instructions per chunk
+    constexpr int kStage = kInstr * 1024;         // bytes per wavefront and stage
+    __shared__ __attribute__((aligned(1024))) char S0[4 * kStage];
+    __shared__ __attribute__((aligned(1024))) char S1[4 * kStage];
+    __shared__ __attribute__((aligned(1024))) char S2[4 * kStage];
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t gw = blockIdx.x * 4u + wave;
+    if (gw >= p.waves) {
+        return;  // whole wavefront; the kernel has no barriers
+    }
+    const uint32_t g = lane >> 4, jj = lane & 15u;
+    const uint32_t c_begin = stream_begin(p, gw), c_end = stream_begin(p, gw + 1u);
+    if (c_begin == c_end) {
+        return;
+    }
+    const size_t row_bytes = p.n / 2;
+    const uint32_t cb_chunks = p.chunks_per_block;
+
+    // ---- producer side: chunk (block ib, k-chunk ik) -> stage
+    uint32_t ib = c_begin / cb_chunks, ik = c_begin % cb_chunks, issued = c_begin;
+    auto issue = [&](char* stage) {
+        // Lanes past the last column work on a duplicate of the last 32 columns (never stored): the MFMA ignores the
+        // execution mask, so every lane must hold valid operands.
+        uint32_t col0 = ib * kColsPerBlock + jj * 32u;
+        col0 = col0 < p.n ? col0 : p.n - 32u;
+        const uint32_t krow = ik * kChunkRows;
+        const uint8_t* wsrc = p.w + static_cast<size_t>(krow + 8u * g) * row_bytes + col0 / 2;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            __builtin_amdgcn_global_load_lds((gptr_t)(wsrc + static_cast<size_t>(u) * row_bytes),
+                                             (lds_ptr_t)(stage + u * 1024), 16, 0, 0);
+        }
+        // parameters of the chunk's group: lane (g, jj) fetches piece g (8 halves) of the 32 columns of jj
+        const size_t prow = static_cast<size_t>(krow / p.group_size) * p.n + col0 + 8u * g;
+        __builtin_amdgcn_global_load_lds((gptr_t)(p.scale + prow), (lds_ptr_t)(stage + 8 * 1024), 16, 0, 0);
+        if constexpr (kHasOffset) {
+            __builtin_amdgcn_global_load_lds((gptr_t)(p.offset + prow), (lds_ptr_t)(stage + 9 * 1024), 16, 0, 0);
+        }
+        // activations of the chunk's 32 k for up to 16 rows in one instruction: lane l fetches piece (l & 3) of row
+        // m0 + (l >> 2); rows past m fetch row m - 1 and are zeroed when used
+        {
+            const uint32_t m = p.m0 + (lane >> 2);
+            const uint32_t mc = m < p.m ? m : p.m - 1u;
+            __builtin_amdgcn_global_load_lds((gptr_t)(p.x + static_cast<size_t>(mc) * p.k + krow + 8u * (lane & 3u)),
+                                             (lds_ptr_t)(stage + (8 + kParamInstr) * 1024), 16, 0, 0);
+        }
+        // advance, staying on the last chunk once the run is exhausted (harmless repeated fetches at the tail)
+        if (issued + 1u < c_end) {
+            ++issued;
+            if (++ik == cb_chunks) {
+                ik = 0;
+                ++ib;
+            }
+        }
+    };
+
+    // ---- consumer side
     f32x4 acc[MP][4];
 #pragma unroll
     for (int q = 0; q < MP; ++q) {
@@ -88,142 +160,258 @@ __global__ __launch_bounds__(kThreads) void w4a16_mfma_kernel(W4Params p)
         amask[r] = (static_cast<uint32_t>(r) == (slot >> 1)) ? ((slot & 1u) ? 0xFFFF0000u : 0x0000FFFFu) : 0u;
     }
     const f16x2 k1032 = {static_cast<half_t>(1032.0f), static_cast<half_t>(1032.0f)};
+    const f16x2 k72 = {static_cast<half_t>(72.0f), static_cast<half_t>(72.0f)};
+    const f16x2 k16th = {static_cast<half_t>(0.0625f), static_cast<half_t>(0.0625f)};
 
-    // Software pipeline over chunks of 32 rows: the 8 weight loads (and the activations) of chunk c + 1 are issued
-    // before chunk c is de-quantised, so a lane always has 8-16 loads of 16 bytes in flight.
-    const uint8_t* wbase = p.w + static_cast<size_t>(kw0 + 8u * g) * row_bytes + col0 / 2;
-    const uint32_t chunks = rows_per_wave / 32u;
-    u32x4 wv[2][8];
-    u32x4 xv[2][MP];
-    f16x2 sc[4][4], of[4][4];
-    uint32_t cur_group = 0xFFFFFFFFu;
-    auto load_chunk = [&](uint32_t c, u32x4 (&wd)[8], u32x4 (&xd)[MP]) {
-        const uint8_t* src = wbase + static_cast<size_t>(c) * 32u * row_bytes;
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            wd[u] = *reinterpret_cast<const u32x4*>(src + static_cast<size_t>(u) * row_bytes);
-        }
+    uint32_t seg = 0, done_in_block = c_begin % cb_chunks;
+    uint32_t checked_group = 0xFFFFFFFFu;
+    bool int_offsets = false;  // every offset of the current group (all lanes) is an integer of magnitude <= 512
+    // the accumulators as they lie in registers: [16 registers][64 lanes] per pair
+    auto flush = [&]() {
 #pragma unroll
         for (int q = 0; q < MP; ++q) {
-            const uint32_t m = p.m0 + 2u * q + (jj >> 3);
-            xd[q] = u32x4{0u, 0u, 0u, 0u};
-            if (m < p.m) {
-                xd[q] = *reinterpret_cast<const u32x4*>(p.x + static_cast<size_t>(m) * p.k + kw0 + c * 32u + 8u * g);
-            }
-        }
-    };
-    auto compute_chunk = [&](uint32_t c, const u32x4 (&wd)[8], const u32x4 (&xd)[MP]) {
-        const uint32_t grp = (kw0 + c * 32u) / p.group_size;  // the 32 rows of a chunk share a group
-        if (grp != cur_group) {
-            cur_group = grp;
-            const size_t prow = static_cast<size_t>(grp) * p.n + col0;
+            float* dst = p.partial + ((static_cast<size_t>(gw) * p.max_seg + seg) * MP + q) * 1024u + lane;
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
-                pair_up(*reinterpret_cast<const u32x4*>(p.scale + prow + 8 * d), sc[d]);
-                if constexpr (kHasOffset) {
-                    pair_up(*reinterpret_cast<const u32x4*>(p.offset + prow + 8 * d), of[d]);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    dst[(d * 4 + r) * 64] = acc[q][d][r];
                 }
+                acc[q][d] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
             }
         }
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            f16x8 a[MP];
-#pragma unroll
-            for (int q = 0; q < MP; ++q) {
-                const uint32_t xw = xd[q][u >> 1];
-                const uint32_t xx = (u & 1) ? __builtin_amdgcn_perm(xw, xw, 0x03020302u)
-                                            : __builtin_amdgcn_perm(xw, xw, 0x01000100u);
-                u32x4 av = u32x4{xx & amask[0], xx & amask[1], xx & amask[2], xx & amask[3]};
-                __builtin_memcpy(&a[q], &av, 16);
-            }
-#pragma unroll
-            for (int d = 0; d < 4; ++d) {
-                const uint32_t qd = wd[u][d] ^ 0x88888888u;  // two's complement nibble -> offset binary u = w + 8
-                f16x2 h[4];
-#pragma unroll
-                for (int c2 = 0; c2 < 4; ++c2) {
-                    uint32_t bits;  // (nibble c2, nibble c2 + 4) -> two halves 1024 + u, exact
-                    asm("v_and_or_b32 %0, %1, %2, %3"
-                        : "=v"(bits)
-                        : "v"(qd >> (4 * c2)), "s"(0x000F000Fu), "v"(0x64006400u));
-                    h[c2] = bits_to_h2(bits) - k1032;  // w, exact
-                    if constexpr (kHasOffset) {
-                        h[c2] = h[c2] + of[d][c2];  // one rounding
-                    }
-                    h[c2] = sc[d][c2] * h[c2];      // one rounding
-                }
-                f16x8 b;
-                __builtin_memcpy(&b, h, 16);
-#pragma unroll
-                for (int q = 0; q < MP; ++q) {
-                    acc[q][d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[q], b, acc[q][d], 0, 0, 0);
-                }
-            }
-        }
+        ++seg;
+        checked_group = 0xFFFFFFFFu;  // the next column block has other offsets
+        // Stores and loads retire out of order with respect to each other, so the counted waits on the load queue
+        // are only meaningful while no store is pending: drain here (once per column block and stream).
+        ASCQ_WAIT_VMCNT(0);
     };
-    load_chunk(0, wv[0], xv[0]);
-    for (uint32_t c = 0; c < chunks; c += 2) {
-        if (c + 1 < chunks) {
-            load_chunk(c + 1, wv[1], xv[1]);
+    // The stages are read back with explicit ds_read instructions and one explicit wait: the reads only ever follow
+    // the counted wait on the stage's loads above them, and the compiler's own bookkeeping of LDS reads against
+    // direct-to-LDS loads in flight (which is conservative around the loop) stays out of the way.
+#define ASCQ_DS_READ128(dst, addr, off) \
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(off) : "memory")
+    auto compute = [&](const char* stage) {
+        const uint32_t sa = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)stage));
+        const uint32_t a_own = sa + lane * 16u;                      // what this lane fetched itself
+        const uint32_t a_par = sa + jj * 16u;                        // parameter pieces of the lane's 32 columns
+        const uint32_t a_x = sa + (((jj >> 3) * 4u + g) * 16u);      // activations: row (jj >> 3) of a pair, piece g
+        u32x4 wd[8], sraw[4], oraw[4], xraw[MP];
+        ASCQ_DS_READ128(wd[0], a_own, 0 * 1024);
+        ASCQ_DS_READ128(wd[1], a_own, 1 * 1024);
+        ASCQ_DS_READ128(wd[2], a_own, 2 * 1024);
+        ASCQ_DS_READ128(wd[3], a_own, 3 * 1024);
+        ASCQ_DS_READ128(wd[4], a_own, 4 * 1024);
+        ASCQ_DS_READ128(wd[5], a_own, 5 * 1024);
+        ASCQ_DS_READ128(wd[6], a_own, 6 * 1024);
+        ASCQ_DS_READ128(wd[7], a_own, 7 * 1024);
+        ASCQ_DS_READ128(sraw[0], a_par, 8 * 1024 + 0 * 256);
+        ASCQ_DS_READ128(sraw[1], a_par, 8 * 1024 + 1 * 256);
+        ASCQ_DS_READ128(sraw[2], a_par, 8 * 1024 + 2 * 256);
+        ASCQ_DS_READ128(sraw[3], a_par, 8 * 1024 + 3 * 256);
+        if constexpr (kHasOffset) {
+            ASCQ_DS_READ128(oraw[0], a_par, 9 * 1024 + 0 * 256);
+            ASCQ_DS_READ128(oraw[1], a_par, 9 * 1024 + 1 * 256);
+            ASCQ_DS_READ128(oraw[2], a_par, 9 * 1024 + 2 * 256);
+            ASCQ_DS_READ128(oraw[3], a_par, 9 * 1024 + 3 * 256);
         }
-        compute_chunk(c, wv[0], xv[0]);
-        if (c + 1 < chunks) {
-            if (c + 2 < chunks) {
-                load_chunk(c + 2, wv[0], xv[0]);
-            }
-            compute_chunk(c + 1, wv[1], xv[1]);
+        // pair q sits 128 bytes (two rows of four pieces) further on
+        ASCQ_DS_READ128(xraw[0], a_x, (8 + kParamInstr) * 1024);
+        if constexpr (MP > 1) ASCQ_DS_READ128(xraw[1], a_x, (8 + kParamInstr) * 1024 + 128);
+        if constexpr (MP > 2) ASCQ_DS_READ128(xraw[2], a_x, (8 + kParamInstr) * 1024 + 256);
+        if constexpr (MP > 3) ASCQ_DS_READ128(xraw[3], a_x, (8 + kParamInstr) * 1024 + 384);
+        // every value read above is an in/out operand of the wait, so nothing uses one before it has arrived
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(wd[0]), "+v"(wd[1]), "+v"(wd[2]), "+v"(wd[3]), "+v"(wd[4]), "+v"(wd[5]), "+v"(wd[6]),
+                       "+v"(wd[7]), "+v"(sraw[0]), "+v"(sraw[1]), "+v"(sraw[2]), "+v"(sraw[3])
+                     :
+                     : "memory");
+        if constexpr (kHasOffset) {
+            asm volatile("" : "+v"(oraw[0]), "+v"(oraw[1]), "+v"(oraw[2]), "+v"(oraw[3]));
         }
-    }
-
-    // result tile d of pair q: register r of lane (g, jj) is row 4 g + r -> activation row 2 q + (g >> 1),
-    // slot 4 (g & 1) + r -> column jj * 32 + d * 8 + slot_to_col(slot)
 #pragma unroll
-    for (int q = 0; q < MP; ++q) {
-        __syncthreads();
+        for (int q = 0; q < MP; ++q) asm volatile("" : "+v"(xraw[q]));
+        f16x2 sc[4][4], of[4][4];
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                red[wave][g >> 1][jj * 32 + d * 8 + slot_to_col(4u * (g & 1u) + r)] = acc[q][d][r];
+            pair_up(sraw[d], sc[d]);
+            if constexpr (kHasOffset) {
+                pair_up(oraw[d], of[d]);
             }
         }
-        __syncthreads();
+        if constexpr (kHasOffset) {
+            // With integer offsets w + offset is exact, and so is (1024 + u) + (offset - 1032): the constant can be
+            // folded and one packed operation per column pair saved without changing a bit of the result.  The test
+            // (o + 1536) - 1536 == o holds exactly for integers |o| <= 512; it runs once per quantisation group and
+            // its outcome is made uniform over the wavefront, because the matrix instruction ignores the execution
+            // mask and so both paths must never run in one wavefront.
+            const uint32_t grp = (done_in_block * kChunkRows) / p.group_size;
+            if (grp != checked_group) {
+                checked_group = grp;
+                const f16x2 k1536 = {static_cast<half_t>(1536.0f), static_cast<half_t>(1536.0f)};
+                uint32_t differ = 0;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const uint32_t idx = tid + e * kThreads;  // 0..1023: (row of the pair, column)
-            const uint32_t mr = idx >> 9, c = idx & 511u;
-            const uint32_t m = p.m0 + 2u * q + mr;
-            const uint32_t col = blockIdx.x * kColsPerBlock + c;
-            if (m < p.m && col < p.n) {
-                const float s = ((red[0][mr][c] + red[1][mr][c]) + red[2][mr][c]) + red[3][mr][c];
-                p.partial[(static_cast<size_t>(blockIdx.y) * p.m + m) * p.n + col] = s;
+                for (int d = 0; d < 4; ++d) {
+#pragma unroll
+                    for (int c2 = 0; c2 < 4; ++c2) {
+                        const f16x2 t = (of[d][c2] + k1536) - k1536;
+                        uint32_t tb, ob;
+                        __builtin_memcpy(&tb, &t, 4);
+                        __builtin_memcpy(&ob, &of[d][c2], 4);
+                        differ |= (tb ^ ob) & 0x7FFF7FFFu;  // -0 counts as the integer 0
+                    }
+                }
+                int_offsets = __builtin_amdgcn_ballot_w64(differ != 0) == 0;
             }
         }
+        u32x4 xc[MP];
+#pragma unroll
+        for (int q = 0; q < MP; ++q) {
+            // lane (g, jj) carries x[m][krow + 8 g .. + 8) for m = m0 + 2 q + (jj >> 3)
+            xc[q] = (p.m0 + 2u * q + (jj >> 3) < p.m) ? xraw[q] : u32x4{0u, 0u, 0u, 0u};
+        }
+        auto body = [&](auto fold_tag) {
+            constexpr bool kFold = decltype(fold_tag)::value;
+            if constexpr (kFold && kHasOffset) {
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+#pragma unroll
+                    for (int c2 = 0; c2 < 4; ++c2) {
+                        of[d][c2] = (c2 & 1) ? of[d][c2] - k72 : of[d][c2] - k1032;  // exact
+                    }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                f16x8 a[MP];
+#pragma unroll
+                for (int q = 0; q < MP; ++q) {
+                    const uint32_t xw = xc[q][u >> 1];
+                    const uint32_t xx = (u & 1) ? __builtin_amdgcn_perm(xw, xw, 0x03020302u)
+                                                : __builtin_amdgcn_perm(xw, xw, 0x01000100u);
+                    u32x4 av = u32x4{xx & amask[0], xx & amask[1], xx & amask[2], xx & amask[3]};
+                    __builtin_memcpy(&a[q], &av, 16);
+                }
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+                    const uint32_t qd = wd[u][d] ^ 0x88888888u;  // two's complement nibble -> offset binary u = w + 8
+                    const uint32_t qh = qd >> 8;
+                    f16x2 h[4];
+#pragma unroll
+                    for (int c2 = 0; c2 < 4; ++c2) {
+                        // (nibble c2, nibble c2 + 4) -> two exact halves: 1024 + u read in place (c2 even),
+                        // 1024 + 16 u read 4 bits up (c2 odd, saves the shift)
+                        uint32_t bits;
+                        if (c2 & 1) {
+                            asm("v_and_or_b32 %0, %1, %2, %3"
+                                : "=v"(bits)
+                                : "v"(c2 == 1 ? qd : qh), "s"(0x00F000F0u), "v"(0x64006400u));
+                        } else {
+                            asm("v_and_or_b32 %0, %1, %2, %3"
+                                : "=v"(bits)
+                                : "v"(c2 == 0 ? qd : qh), "s"(0x000F000Fu), "v"(0x64006400u));
+                        }
+                        if constexpr (kFold && kHasOffset) {
+                            // w + offset in one exact operation
+                            h[c2] = (c2 & 1) ? __builtin_elementwise_fma(bits_to_h2(bits), k16th, of[d][c2])
+                                             : bits_to_h2(bits) + of[d][c2];
+                        } else {
+                            h[c2] = (c2 & 1) ? __builtin_elementwise_fma(bits_to_h2(bits), k16th, -k72)
+                                             : bits_to_h2(bits) - k1032;  // w, exact
+                            if constexpr (kHasOffset) {
+                                h[c2] = h[c2] + of[d][c2];  // one rounding
+                            }
+                        }
+                        h[c2] = sc[d][c2] * h[c2];  // one rounding
+                    }
+                    f16x8 b;
+                    __builtin_memcpy(&b, h, 16);
+#pragma unroll
+                    for (int q = 0; q < MP; ++q) {
+                        acc[q][d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[q], b, acc[q][d], 0, 0, 0);
+                    }
+                }
+            }
+        };
+        if (kHasOffset && int_offsets) {
+            body(std::true_type{});
+        } else {
+            body(std::false_type{});
+        }
+        if (++done_in_block == cb_chunks) {  // the run leaves this column block
+            done_in_block = 0;
+            flush();
+        }
+    };
+
+    char* s0 = S0 + wave * kStage;
+    char* s1 = S1 + wave * kStage;
+    char* s2 = S2 + wave * kStage;
+    issue(s0);
+    issue(s1);
+    issue(s2);
+    uint32_t c = c_begin;
+    while (true) {
+        ASCQ_WAIT_VMCNT(2 * kInstr);  // everything but the two newest chunks has landed
+        compute(s0);
+        if (++c == c_end) break;
+        issue(s0);
+        ASCQ_WAIT_VMCNT(2 * kInstr);
+        compute(s1);
+        if (++c == c_end) break;
+        issue(s1);
+        ASCQ_WAIT_VMCNT(2 * kInstr);
+        compute(s2);
+        if (++c == c_end) break;
+        issue(s2);
+    }
+    ASCQ_WAIT_VMCNT(0);
+    if (done_in_block != 0) {
+        flush();
     }
 }
 
-// Adds the K-splits in a fixed order (deterministic) and rounds once to half.  Launched after the partial kernel: the
-// kernel boundary makes the partial sums visible, which is far cheaper here than device-scope fences in 900 workgroups.
-__global__ __launch_bounds__(kThreads) void w4a16_reduce_kernel(W4Params p)
+// For every output of the pass: adds the pieces of all streams that worked on its column block, in ascending k order
+// (deterministic), and rounds once to half.  One lane per (activation row of the pass, column).
+template <int MP>
+__global__ __launch_bounds__(kThreads) void w4a16_sum_kernel(W4Params p)
 {
-    const size_t total = static_cast<size_t>(p.m) * p.n;
-    const size_t idx = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x;
-    if (idx >= total) {
+    const uint32_t col = blockIdx.x * kThreads + threadIdx.x;
+    const uint32_t mrow = blockIdx.y;  // 0 .. 2 MP - 1
+    const uint32_t m = p.m0 + mrow;
+    if (col >= p.n || m >= p.m) {
         return;
     }
-    float s = 0.0f;
-    uint32_t sp = 0;
-    for (; sp + 8 <= p.splits; sp += 8) {
+    const uint32_t q = mrow >> 1, mr = mrow & 1u;
+    const uint32_t blk = col / kColsPerBlock, cl = col % kColsPerBlock;
+    const uint32_t jj = cl / 32u, d = (cl % 32u) / 8u, cc = cl % 8u;
+    // register r of lane (g, jj) in tile d holds column slot b8 of the dword, with column = (b8 >> 1) + 4 (b8 & 1)
+    const uint32_t b8 = cc < 4u ? 2u * cc : 2u * (cc - 4u) + 1u;
+    const uint32_t r = b8 & 3u, g = 2u * mr + (b8 >> 2);
+    const uint32_t e = (d * 4u + r) * 64u + g * 16u + jj;
+    const uint32_t first_chunk = blk * p.chunks_per_block, end_chunk = first_chunk + p.chunks_per_block;
+    // the stream that holds first_chunk, and the first one past the block
+    const uint32_t big = p.rem * (p.per + 1u);  // chunks owned by the longer streams
+    uint32_t w0 = first_chunk < big ? first_chunk / (p.per + 1u) : p.rem + (first_chunk - big) / p.per;
+    uint32_t w1 = end_chunk <= big ? (end_chunk + p.per) / (p.per + 1u) : p.rem + (end_chunk - big + p.per - 1u) / p.per;
+    w1 = w1 < p.waves ? w1 : p.waves;
+    const size_t stride = static_cast<size_t>(p.max_seg) * MP * 1024u;  // floats between streams
+    // the first stream may have begun in an earlier block; all later ones begin inside this block (piece 0)
+    const uint32_t seg0 = blk - stream_begin(p, w0) / p.chunks_per_block;
+    const float* src = p.partial + (static_cast<size_t>(w0) * p.max_seg * MP + q) * 1024u + e;
+    float s = src[static_cast<size_t>(seg0) * MP * 1024u];
+    src += stride;
+    for (uint32_t w = w0 + 1u; w < w1; w += 8u) {
         float v[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = p.partial[static_cast<size_t>(sp + u) * total + idx];  // 8 loads in flight
+        for (uint32_t u = 0; u < 8u; ++u) {  // 8 independent loads in flight, then an ordered sum
+            v[u] = (w + u < w1) ? src[static_cast<size_t>(u) * stride] : 0.0f;
+        }
 #pragma unroll
-        for (int u = 0; u < 8; ++u) s += v[u];
+        for (uint32_t u = 0; u < 8u; ++u) s += v[u];
+        src += 8u * stride;
     }
-    for (; sp < p.splits; ++sp) {
-        s += p.partial[static_cast<size_t>(sp) * total + idx];
-    }
-    p.y[idx] = static_cast<uint16_t>(f32_to_half_bits(s));
+    p.y[static_cast<size_t>(m) * p.n + col] = static_cast<uint16_t>(f32_to_half_bits(s));
 }
 
 // Any shape: one lane per output element.
@@ -250,24 +438,28 @@ __global__ __launch_bounds__(kThreads) void w4a16_generic_kernel(W4Params p)
     }
 }
 
-uint32_t pick_splits(uint32_t n, uint32_t k, uint32_t group_size)
+struct W4Plan {
+    uint32_t waves, chunks_per_block, total_chunks, max_seg;
+};
+
+W4Plan make_plan(uint32_t n, uint32_t k)
 {
-    // K range per workgroup: a multiple of 128 rows (32 per wavefront) and of the group size; aim at ~450 workgroups (measured best on 256 CUs)
-    (void)group_size;
-    const uint32_t blocks_n = (n + kColsPerBlock - 1) / kColsPerBlock;
-    const uint32_t units = k / kRowsPerPass;
-    const uint32_t target = 448u;  // workgroups per launch that measured fastest on 256 compute units
-    uint32_t want = (target + blocks_n - 1) / blocks_n;
-    uint32_t splits = units < want ? units : want;
-    if (splits == 0) splits = 1;
-    while (units % splits != 0) --splits;
-    return splits;
+    W4Plan pl;
+    const uint32_t blocks_n = (n + kColsPerBlock - 1u) / kColsPerBlock;
+    pl.chunks_per_block = k / kChunkRows;
+    pl.total_chunks = blocks_n * pl.chunks_per_block;
+    pl.waves = pl.total_chunks < kMaxWaves ? pl.total_chunks : kMaxWaves;
+    const uint32_t per = (pl.total_chunks + pl.waves - 1u) / pl.waves;  // longest run
+    pl.max_seg = (per + pl.chunks_per_block - 2u) / pl.chunks_per_block + 1u;
+    return pl;
 }
 
 bool fast_ok(const ascq_w4a16_desc* d, const void* x, const void* w, const void* scale, const void* offset)
 {
-    return d->n % 32 == 0 && d->k % kRowsPerPass == 0 && d->group_size % 32 == 0 && aligned16(x) && aligned16(w) &&
-           aligned16(scale) && (!d->has_offset || aligned16(offset));
+    // total_chunks must fit 32 bits with room for the 64-bit products; k % 8 == 0 keeps activation loads aligned
+    return d->n % 32 == 0 && d->k % kChunkRows == 0 && d->group_size % kChunkRows == 0 && aligned16(x) &&
+           aligned16(w) && aligned16(scale) && (!d->has_offset || aligned16(offset)) &&
+           static_cast<uint64_t>((d->n + kColsPerBlock - 1u) / kColsPerBlock) * (d->k / kChunkRows) < (1ull << 31);
 }
 
 }  // namespace
@@ -292,8 +484,11 @@ extern "C" int ascq_matmul_w4a16_workspace_size(const ascq_w4a16_desc* d, size_t
         return rc;
     }
     ASCQ_REQUIRE(bytes != nullptr, ASCQ_ENULL, "ascq_matmul_w4a16_workspace_size: bytes is NULL");
-    const uint32_t splits = pick_splits(d->n, d->k, d->group_size);
-    *bytes = static_cast<size_t>(splits) * d->m * d->n * sizeof(float);
+    *bytes = 0;
+    if (d->k % kChunkRows == 0) {
+        const W4Plan pl = make_plan(d->n, d->k);
+        *bytes = static_cast<size_t>(pl.waves) * pl.max_seg * kMaxPairs * 1024u * sizeof(float);
+    }
     return ASCQ_OK;
 }
 
@@ -308,50 +503,59 @@ extern "C" int ascq_matmul_w4a16(const ascq_w4a16_desc* d, void* y, const void* 
     ASCQ_REQUIRE(y && x && w && scale, ASCQ_ENULL, "ascq_matmul_w4a16: y / x / w / scale is NULL");
     ASCQ_REQUIRE(!d->has_offset || offset, ASCQ_ENULL, "ascq_matmul_w4a16: offset is NULL");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    W4Params p{static_cast<const uint16_t*>(x), static_cast<const uint8_t*>(w), static_cast<const uint16_t*>(scale),
-               static_cast<const uint16_t*>(offset), static_cast<float*>(workspace), static_cast<uint16_t*>(y),
-               d->m, d->n, d->k, d->group_size, static_cast<uint32_t>(d->has_offset ? 1 : 0), 1, d->k, 0};
-    const size_t total = static_cast<size_t>(d->m) * d->n;
+    W4Params p{};
+    p.x = static_cast<const uint16_t*>(x);
+    p.w = static_cast<const uint8_t*>(w);
+    p.scale = static_cast<const uint16_t*>(scale);
+    p.offset = static_cast<const uint16_t*>(offset);
+    p.partial = static_cast<float*>(workspace);
+    p.y = static_cast<uint16_t*>(y);
+    p.m = d->m;
+    p.n = d->n;
+    p.k = d->k;
+    p.group_size = d->group_size;
+    p.has_offset = d->has_offset ? 1u : 0u;
     if (!fast_ok(d, x, w, scale, offset)) {
+        const size_t total = static_cast<size_t>(d->m) * d->n;
         size_t blocks = (total + kThreads - 1) / kThreads;
         if (blocks > 65536) blocks = 65536;
         w4a16_generic_kernel<<<static_cast<uint32_t>(blocks), kThreads, 0, st>>>(p);
         return launch_status("ascq_matmul_w4a16 (generic)");
     }
-    p.splits = pick_splits(d->n, d->k, d->group_size);
-    p.k_per_split = d->k / p.splits;
-    const size_t need = static_cast<size_t>(p.splits) * total * sizeof(float);
+    const W4Plan pl = make_plan(d->n, d->k);
+    p.waves = pl.waves;
+    p.chunks_per_block = pl.chunks_per_block;
+    p.total_chunks = pl.total_chunks;
+    p.max_seg = pl.max_seg;
+    p.per = pl.total_chunks / pl.waves;
+    p.rem = pl.total_chunks % pl.waves;
+    const size_t need = static_cast<size_t>(pl.waves) * pl.max_seg * kMaxPairs * 1024u * sizeof(float);
     ASCQ_REQUIRE(workspace != nullptr && workspace_bytes >= need, ASCQ_EINVAL,
                  "ascq_matmul_w4a16: workspace of %zu bytes required (see ascq_matmul_w4a16_workspace_size)", need);
     ASCQ_REQUIRE(aligned16(workspace), ASCQ_EALIGN, "ascq_matmul_w4a16: workspace must be 16-byte aligned");
-    dim3 grid((d->n + kColsPerBlock - 1) / kColsPerBlock, p.splits);
-    for (uint32_t m0 = 0; m0 < d->m; m0 += 16) {
+    const uint32_t grid = (pl.waves + 3u) / 4u;
+    const uint32_t col_blocks = (d->n + kThreads - 1) / kThreads;
+    // at most 8 activation rows per pass over the weights
+    for (uint32_t m0 = 0; m0 < d->m; m0 += 2 * kMaxPairs) {
         const uint32_t left = d->m - m0;
         p.m0 = m0;
-#define ASCQ_W4_LAUNCH(MPV)                                                  \
-    do {                                                                     \
-        if (d->has_offset) {                                                 \
-            w4a16_mfma_kernel<MPV, true><<<grid, kThreads, 0, st>>>(p);      \
-        } else {                                                             \
-            w4a16_mfma_kernel<MPV, false><<<grid, kThreads, 0, st>>>(p);     \
-        }                                                                    \
+#define ASCQ_W4_LAUNCH(MPV)                                                              \
+    do {                                                                                 \
+        if (d->has_offset) {                                                             \
+            w4a16_stream_kernel<MPV, true><<<grid, kThreads, 0, st>>>(p);                \
+        } else {                                                                         \
+            w4a16_stream_kernel<MPV, false><<<grid, kThreads, 0, st>>>(p);               \
+        }                                                                                \
+        w4a16_sum_kernel<MPV><<<dim3(col_blocks, 2 * MPV), kThreads, 0, st>>>(p);        \
     } while (0)
         if (left <= 2) {
             ASCQ_W4_LAUNCH(1);
         } else if (left <= 4) {
             ASCQ_W4_LAUNCH(2);
-        } else if (left <= 8) {
-            ASCQ_W4_LAUNCH(4);
         } else {
-            ASCQ_W4_LAUNCH(8);
+            ASCQ_W4_LAUNCH(4);
         }
 #undef ASCQ_W4_LAUNCH
     }
-    rc = launch_status("ascq_matmul_w4a16");
-    if (rc != ASCQ_OK) {
-        return rc;
-    }
-    const size_t blocks = (total + kThreads - 1) / kThreads;
-    w4a16_reduce_kernel<<<static_cast<uint32_t>(blocks), kThreads, 0, st>>>(p);
-    return launch_status("ascq_matmul_w4a16 (reduce)");
+    return launch_status("ascq_matmul_w4a16");
 }

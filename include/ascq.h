@@ -263,8 +263,8 @@ int ascq_group_matmul_w8a8(const ascq_group_matmul_desc* desc, void* y, const vo
  * x f16 [m, k]; w int4 [k, n] packed along n (n even); scale, offset f16 [k/group_size, n].
  *   wdq[k,j] = f16( scale[k/g][j] * f16( f16(w[k,j]) + offset[k/g][j] ) )     (offset optional)
  *   y[i,j]   = f16( sum_k f32(x[i,k]) * f32(wdq[k,j]) )                       fp32 accumulation
- * workspace: ascq_matmul_w4a16_workspace_size bytes of scratch for the K-split partial sums (contents need not be
- * initialised); calls that share a workspace must not overlap.
+ * workspace: ascq_matmul_w4a16_workspace_size bytes of scratch for the partial sums of the weight streams (contents
+ * need not be initialised); calls that share a workspace must not overlap.
  */
 typedef struct ascq_w4a16_desc {
     uint32_t m, n, k;
