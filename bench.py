@@ -28,8 +28,8 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E peak, GB/s
 # `bench.py --quick --no-cpu --copy-probe`; each counter is scaled by its reading for the 1 GiB copy of the same run
 # (FETCH_SIZE reads 0.5 per KiB there, WRITE_SIZE 1.0 per KiB).  Measured offline and recorded here; a run of this
 # file does not re-measure them.
-GEMM_TRAFFIC_BYTES = 249316454   # M=2048 GEMM, both launches: 191.7 MB fetched + 57.6 MB written
-GEMV_TRAFFIC_BYTES = 127087616   # W4A16 M=1 GEMV, partial + reduce kernels: 126.1 MB fetched + 1.0 MB written
+GEMM_TRAFFIC_BYTES = 228336230   # M=2048 GEMM, both launches: 183.2 MB fetched + 45.1 MB written
+GEMV_TRAFFIC_BYTES = 135269990   # W4A16 M=1 GEMV, stream + sum kernels: 130.8 MB fetched + 4.4 MB written
 
 
 def main():
@@ -262,11 +262,11 @@ def main():
                                "dequant to bf16; one step = quant kernel + GEMM kernel",
                    "m": 2048, "k": 4096, "n": 11008, "ops_per_step": head["ops"]},
         # The GEMM is two launches of one kernel template back to back: 256x256 tiles for the full rounds of 256
-        # workgroups and 256x128 tiles for the last partial round; the events bracket both, so `achieved` is the
-        # 2*M*K*N operations over the sum of the two durations.  `traffic` is HBM bytes per GEMM (both launches) from
+        # workgroups and 256x128 tiles for the last partial round; `achieved` is the 2*M*K*N operations over the
+        # average duration of the pair, from one pair of events around `steps` back-to-back GEMMs.  `traffic` is HBM bytes per GEMM (both launches) from
         # rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of `bench.py --only w8a8 --copy-probe`, each counter scaled by
         # its reading for the 1 GiB copy; it is a constant measured offline, not re-measured by this run.
-        "roofline": {"bound": "mfma", "kernel": "gemm_dma_kernel<256> + gemm_dma_kernel<128> (last partial round)",
+        "roofline": {"bound": "mfma", "kernel": "gemm_dma_kernel<256,256> + gemm_dma_kernel<256,128> (last partial round)",
                      "achieved": head["gemm_tops"], "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                      "frac": head["gemm_tops"] / PEAK_INT8_TOPS, "traffic": GEMM_TRAFFIC_BYTES,
                      "avg_kernel_ms": head["gemm_kernel_ms"], "ops_per_launch": head["ops"],
@@ -280,7 +280,7 @@ def main():
     out["w4a16_gemv"] = {"metric": "w4a16_decode_gemv_hbm_gbs_m1_k8192_n28672", "value": gemv["gbs"], "unit": "GB/s",
                          "workload": "BASELINE configs[3] at M=1, 4 rotating weight sets (500 MB > Infinity Cache)",
                          "ms_per_step": gemv["ms_per_step"],
-                         "roofline": {"bound": "hbm", "kernel": "w4a16_mfma_kernel<1, offset> + w4a16_reduce_kernel",
+                         "roofline": {"bound": "hbm", "kernel": "w4a16_stream_kernel<1, offset> + w4a16_sum_kernel<1>",
                                       "achieved": gemv["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                       "frac": gemv["gbs"] / PEAK_HBM_GBS, "traffic": GEMV_TRAFFIC_BYTES,
                                       "avg_kernel_ms": gemv["kernel_ms"], "bytes_per_launch": gemv["bytes"]}}
