@@ -78,6 +78,91 @@ __device__ __forceinline__ uint32_t stream_begin(const W4Params& p, uint32_t wav
     return wave * p.per + (wave < p.rem ? wave : p.rem);
 }
 
+// De-quantises the 32 x 32 weights a lane holds of one chunk (8 rows x 4 dwords) and accumulates them against the
+// activations on the matrix core.  kFold: ofc holds offset - 1032 (even nibble pairs) / offset - 72 (odd pairs), which
+// is exact for integer offsets, so that w + offset is one exact operation; otherwise ofc is the offset itself.
+template <int MP, bool kHasOffset, bool kFold>
+__device__ __forceinline__ void w4_accumulate(const u32x4 (&wd)[8], const u32x4 (&xc)[MP], const f16x2 (&sc)[4][4],
+                                              const f16x2 (&ofc)[4][4], const uint32_t (&amask)[4],
+                                              f32x4 (&acc)[MP][4])
+{
+    const f16x2 k1032 = {static_cast<half_t>(1032.0f), static_cast<half_t>(1032.0f)};
+    const f16x2 k72 = {static_cast<half_t>(72.0f), static_cast<half_t>(72.0f)};
+    const f16x2 k16th = {static_cast<half_t>(0.0625f), static_cast<half_t>(0.0625f)};
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+        f16x8 a[MP];
+#pragma unroll
+        for (int q = 0; q < MP; ++q) {
+            const uint32_t xw = xc[q][u >> 1];
+            const uint32_t xx =
+                (u & 1) ? __builtin_amdgcn_perm(xw, xw, 0x03020302u) : __builtin_amdgcn_perm(xw, xw, 0x01000100u);
+            u32x4 av = u32x4{xx & amask[0], xx & amask[1], xx & amask[2], xx & amask[3]};
+            __builtin_memcpy(&a[q], &av, 16);
+        }
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            const uint32_t qd = wd[u][d] ^ 0x88888888u;  // two's complement nibble -> offset binary u = w + 8
+            const uint32_t qh = qd >> 8;
+            f16x2 h[4];
+#pragma unroll
+            for (int c2 = 0; c2 < 4; ++c2) {
+                // (nibble c2, nibble c2 + 4) -> two exact halves: 1024 + u read in place (c2 even), 1024 + 16 u read
+                // 4 bits up (c2 odd, saves the shift)
+                uint32_t bits;
+                if (c2 & 1) {
+                    asm("v_and_or_b32 %0, %1, %2, %3"
+                        : "=v"(bits)
+                        : "v"(c2 == 1 ? qd : qh), "s"(0x00F000F0u), "v"(0x64006400u));
+                } else {
+                    asm("v_and_or_b32 %0, %1, %2, %3"
+                        : "=v"(bits)
+                        : "v"(c2 == 0 ? qd : qh), "s"(0x000F000Fu), "v"(0x64006400u));
+                }
+                if constexpr (kFold && kHasOffset) {
+                    // w + offset in one exact operation
+                    h[c2] = (c2 & 1) ? __builtin_elementwise_fma(bits_to_h2(bits), k16th, ofc[d][c2])
+                                     : bits_to_h2(bits) + ofc[d][c2];
+                } else {
+                    h[c2] = (c2 & 1) ? __builtin_elementwise_fma(bits_to_h2(bits), k16th, -k72)
+                                     : bits_to_h2(bits) - k1032;  // w, exact
+                    if constexpr (kHasOffset) {
+                        h[c2] = h[c2] + ofc[d][c2];  // one rounding
+                    }
+                }
+                h[c2] = sc[d][c2] * h[c2];  // one rounding
+            }
+            f16x8 b;
+            __builtin_memcpy(&b, h, 16);
+#pragma unroll
+            for (int q = 0; q < MP; ++q) {
+                acc[q][d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[q], b, acc[q][d], 0, 0, 0);
+            }
+        }
+    }
+}
+
+// True on every lane iff every offset held by any lane of the wavefront is an integer of magnitude <= 512 (then
+// (o + 1536) - 1536 == o exactly).  Uniform over the wavefront on purpose: the matrix instruction ignores the execution
+// mask, so the two arithmetic paths must never run in one wavefront.
+__device__ __forceinline__ bool all_offsets_integral(const f16x2 (&of)[4][4])
+{
+    const f16x2 k1536 = {static_cast<half_t>(1536.0f), static_cast<half_t>(1536.0f)};
+    uint32_t differ = 0;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+#pragma unroll
+        for (int c2 = 0; c2 < 4; ++c2) {
+            const f16x2 t = (of[d][c2] + k1536) - k1536;
+            uint32_t tb, ob;
+            __builtin_memcpy(&tb, &t, 4);
+            __builtin_memcpy(&ob, &of[d][c2], 4);
+            differ |= (tb ^ ob) & 0x7FFF7FFFu;  // -0 counts as the integer 0
+        }
+    }
+    return __builtin_amdgcn_ballot_w64(differ != 0) == 0;
+}
+
 // s_waitcnt vmcnt(n) only (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8)
 #define ASCQ_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | (7 << 4) | (15 << 8))
 
@@ -161,7 +246,6 @@ __global__ __launch_bounds__(kThreads) void w4a16_stream_kernel(W4Params p)
     }
     const f16x2 k1032 = {static_cast<half_t>(1032.0f), static_cast<half_t>(1032.0f)};
     const f16x2 k72 = {static_cast<half_t>(72.0f), static_cast<half_t>(72.0f)};
-    const f16x2 k16th = {static_cast<half_t>(0.0625f), static_cast<half_t>(0.0625f)};
 
     uint32_t seg = 0, done_in_block = c_begin % cb_chunks;
     uint32_t checked_group = 0xFFFFFFFFu;
@@ -241,27 +325,12 @@ __global__ __launch_bounds__(kThreads) void w4a16_stream_kernel(W4Params p)
         }
         if constexpr (kHasOffset) {
             // With integer offsets w + offset is exact, and so is (1024 + u) + (offset - 1032): the constant can be
-            // folded and one packed operation per column pair saved without changing a bit of the result.  The test
-            // (o + 1536) - 1536 == o holds exactly for integers |o| <= 512; it runs once per quantisation group and
-            // its outcome is made uniform over the wavefront, because the matrix instruction ignores the execution
-            // mask and so both paths must never run in one wavefront.
+            // folded and one packed operation per column pair saved without changing a bit of the result.  Tested
+            // once per quantisation group.
             const uint32_t grp = (done_in_block * kChunkRows) / p.group_size;
             if (grp != checked_group) {
                 checked_group = grp;
-                const f16x2 k1536 = {static_cast<half_t>(1536.0f), static_cast<half_t>(1536.0f)};
-                uint32_t differ = 0;
-#pragma unroll
-                for (int d = 0; d < 4; ++d) {
-#pragma unroll
-                    for (int c2 = 0; c2 < 4; ++c2) {
-                        const f16x2 t = (of[d][c2] + k1536) - k1536;
-                        uint32_t tb, ob;
-                        __builtin_memcpy(&tb, &t, 4);
-                        __builtin_memcpy(&ob, &of[d][c2], 4);
-                        differ |= (tb ^ ob) & 0x7FFF7FFFu;  // -0 counts as the integer 0
-                    }
-                }
-                int_offsets = __builtin_amdgcn_ballot_w64(differ != 0) == 0;
+                int_offsets = all_offsets_integral(of);
             }
         }
         u32x4 xc[MP];
@@ -270,73 +339,17 @@ __global__ __launch_bounds__(kThreads) void w4a16_stream_kernel(W4Params p)
             // lane (g, jj) carries x[m][krow + 8 g .. + 8) for m = m0 + 2 q + (jj >> 3)
             xc[q] = (p.m0 + 2u * q + (jj >> 3) < p.m) ? xraw[q] : u32x4{0u, 0u, 0u, 0u};
         }
-        auto body = [&](auto fold_tag) {
-            constexpr bool kFold = decltype(fold_tag)::value;
-            if constexpr (kFold && kHasOffset) {
-#pragma unroll
-                for (int d = 0; d < 4; ++d) {
-#pragma unroll
-                    for (int c2 = 0; c2 < 4; ++c2) {
-                        of[d][c2] = (c2 & 1) ? of[d][c2] - k72 : of[d][c2] - k1032;  // exact
-                    }
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                f16x8 a[MP];
-#pragma unroll
-                for (int q = 0; q < MP; ++q) {
-                    const uint32_t xw = xc[q][u >> 1];
-                    const uint32_t xx = (u & 1) ? __builtin_amdgcn_perm(xw, xw, 0x03020302u)
-                                                : __builtin_amdgcn_perm(xw, xw, 0x01000100u);
-                    u32x4 av = u32x4{xx & amask[0], xx & amask[1], xx & amask[2], xx & amask[3]};
-                    __builtin_memcpy(&a[q], &av, 16);
-                }
-#pragma unroll
-                for (int d = 0; d < 4; ++d) {
-                    const uint32_t qd = wd[u][d] ^ 0x88888888u;  // two's complement nibble -> offset binary u = w + 8
-                    const uint32_t qh = qd >> 8;
-                    f16x2 h[4];
-#pragma unroll
-                    for (int c2 = 0; c2 < 4; ++c2) {
-                        // (nibble c2, nibble c2 + 4) -> two exact halves: 1024 + u read in place (c2 even),
-                        // 1024 + 16 u read 4 bits up (c2 odd, saves the shift)
-                        uint32_t bits;
-                        if (c2 & 1) {
-                            asm("v_and_or_b32 %0, %1, %2, %3"
-                                : "=v"(bits)
-                                : "v"(c2 == 1 ? qd : qh), "s"(0x00F000F0u), "v"(0x64006400u));
-                        } else {
-                            asm("v_and_or_b32 %0, %1, %2, %3"
-                                : "=v"(bits)
-                                : "v"(c2 == 0 ? qd : qh), "s"(0x000F000Fu), "v"(0x64006400u));
-                        }
-                        if constexpr (kFold && kHasOffset) {
-                            // w + offset in one exact operation
-                            h[c2] = (c2 & 1) ? __builtin_elementwise_fma(bits_to_h2(bits), k16th, of[d][c2])
-                                             : bits_to_h2(bits) + of[d][c2];
-                        } else {
-                            h[c2] = (c2 & 1) ? __builtin_elementwise_fma(bits_to_h2(bits), k16th, -k72)
-                                             : bits_to_h2(bits) - k1032;  // w, exact
-                            if constexpr (kHasOffset) {
-                                h[c2] = h[c2] + of[d][c2];  // one rounding
-                            }
-                        }
-                        h[c2] = sc[d][c2] * h[c2];  // one rounding
-                    }
-                    f16x8 b;
-                    __builtin_memcpy(&b, h, 16);
-#pragma unroll
-                    for (int q = 0; q < MP; ++q) {
-                        acc[q][d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[q], b, acc[q][d], 0, 0, 0);
-                    }
-                }
-            }
-        };
         if (kHasOffset && int_offsets) {
-            body(std::true_type{});
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+#pragma unroll
+                for (int c2 = 0; c2 < 4; ++c2) {
+                    of[d][c2] = (c2 & 1) ? of[d][c2] - k72 : of[d][c2] - k1032;  // exact
+                }
+            }
+            w4_accumulate<MP, kHasOffset, true>(wd, xc, sc, of, amask, acc);
         } else {
-            body(std::false_type{});
+            w4_accumulate<MP, kHasOffset, false>(wd, xc, sc, of, amask, acc);
         }
         if (++done_in_block == cb_chunks) {  // the run leaves this column block
             done_in_block = 0;
@@ -371,47 +384,231 @@ __global__ __launch_bounds__(kThreads) void w4a16_stream_kernel(W4Params p)
     }
 }
 
-// For every output of the pass: adds the pieces of all streams that worked on its column block, in ascending k order
-// (deterministic), and rounds once to half.  One lane per (activation row of the pass, column).
-template <int MP>
-__global__ __launch_bounds__(kThreads) void w4a16_sum_kernel(W4Params p)
+// One or two activation rows (the decode GEMV): the same streams, two per SIMD.  To fit 8 rings into the LDS the
+// ring has two stages and holds only the weights (8 KiB) and the activations (256 bytes); the scale / offset rows of
+// a quantisation group are fetched into registers when a chunk opens a new group, ahead of that chunk's weights, so
+// they have landed whenever the weights have.  With two stages one chunk is in flight behind the one being computed
+// and the wait before a chunk is simply for everything outstanding; the second wavefront of the SIMD fills the time
+// a wavefront spends waiting or stalled on its own dependent instructions.
+template <bool kHasOffset>
+__global__ __launch_bounds__(512) void w4a16_gemv_kernel(W4Params p)
 {
-    const uint32_t col = blockIdx.x * kThreads + threadIdx.x;
-    const uint32_t mrow = blockIdx.y;  // 0 .. 2 MP - 1
-    const uint32_t m = p.m0 + mrow;
-    if (col >= p.n || m >= p.m) {
+    constexpr int kStage = 8 * 1024 + 256;  // bytes per wavefront and stage
+    __shared__ __attribute__((aligned(1024))) char S0[8 * kStage];
+    __shared__ __attribute__((aligned(1024))) char S1[8 * kStage];
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t gw = blockIdx.x * 8u + wave;
+    if (gw >= p.waves) {
+        return;  // whole wavefront; the kernel has no barriers
+    }
+    const uint32_t g = lane >> 4, jj = lane & 15u;
+    const uint32_t c_begin = stream_begin(p, gw), c_end = stream_begin(p, gw + 1u);
+    if (c_begin == c_end) {
         return;
     }
-    const uint32_t q = mrow >> 1, mr = mrow & 1u;
-    const uint32_t blk = col / kColsPerBlock, cl = col % kColsPerBlock;
-    const uint32_t jj = cl / 32u, d = (cl % 32u) / 8u, cc = cl % 8u;
-    // register r of lane (g, jj) in tile d holds column slot b8 of the dword, with column = (b8 >> 1) + 4 (b8 & 1)
-    const uint32_t b8 = cc < 4u ? 2u * cc : 2u * (cc - 4u) + 1u;
-    const uint32_t r = b8 & 3u, g = 2u * mr + (b8 >> 2);
-    const uint32_t e = (d * 4u + r) * 64u + g * 16u + jj;
+    const size_t row_bytes = p.n / 2;
+    const uint32_t cb_chunks = p.chunks_per_block;
+    const uint32_t chunks_per_group = p.group_size / kChunkRows;
+
+    // ---- producer side: chunk (block ib, k-chunk ik) -> stage; parameters of a new group -> registers
+    uint32_t ib = c_begin / cb_chunks, ik = c_begin % cb_chunks;
+    u32x4 sraw[4], oraw[4];
+    bool params_pending = false;
+    auto issue = [&](char* stage, bool first) {
+        // Lanes past the last column work on a duplicate of the last 32 columns (never stored): the MFMA ignores the
+        // execution mask, so every lane must hold valid operands.
+        uint32_t col0 = ib * kColsPerBlock + jj * 32u;
+        col0 = col0 < p.n ? col0 : p.n - 32u;
+        const uint32_t krow = ik * kChunkRows;
+        if (first || ik % chunks_per_group == 0u) {  // the chunk opens the run, a group or a column block
+            const size_t prow = static_cast<size_t>(krow / p.group_size) * p.n + col0;
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                sraw[d] = *reinterpret_cast<const u32x4*>(p.scale + prow + 8 * d);
+                if constexpr (kHasOffset) {
+                    oraw[d] = *reinterpret_cast<const u32x4*>(p.offset + prow + 8 * d);
+                }
+            }
+            params_pending = true;
+        }
+        const uint8_t* wsrc = p.w + static_cast<size_t>(krow + 8u * g) * row_bytes + col0 / 2;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            __builtin_amdgcn_global_load_lds((gptr_t)(wsrc + static_cast<size_t>(u) * row_bytes),
+                                             (lds_ptr_t)(stage + u * 1024), 16, 0, 0);
+        }
+        // activations of the chunk's 32 k for two rows, one dword per lane: lane l fetches dword (l & 15) of row
+        // m0 + ((l >> 4) & 1); a missing second row fetches the first and is zeroed when used
+        {
+            const uint32_t m = p.m0 + ((lane >> 4) & 1u);
+            const uint32_t mc = m < p.m ? m : p.m - 1u;
+            __builtin_amdgcn_global_load_lds((gptr_t)(p.x + static_cast<size_t>(mc) * p.k + krow + 2u * (lane & 15u)),
+                                             (lds_ptr_t)(stage + 8 * 1024), 4, 0, 0);
+        }
+        if (++ik == cb_chunks) {
+            ik = 0;
+            ++ib;
+        }
+    };
+
+    // ---- consumer side
+    f32x4 acc[1][4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) acc[0][t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    const uint32_t slot = jj & 7u;
+    uint32_t amask[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        amask[r] = (static_cast<uint32_t>(r) == (slot >> 1)) ? ((slot & 1u) ? 0xFFFF0000u : 0x0000FFFFu) : 0u;
+    }
+    const f16x2 k1032 = {static_cast<half_t>(1032.0f), static_cast<half_t>(1032.0f)};
+    const f16x2 k72 = {static_cast<half_t>(72.0f), static_cast<half_t>(72.0f)};
+    f16x2 sc[4][4], ofc[4][4];
+    bool folded = false;
+    uint32_t seg = 0, done_in_block = c_begin % cb_chunks;
+    auto flush = [&]() {
+        float* dst = p.partial + (static_cast<size_t>(gw) * p.max_seg + seg) * 1024u + lane;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                dst[(d * 4 + r) * 64] = acc[0][d][r];
+            }
+            acc[0][d] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+        ++seg;
+    };
+    // called after the wait: turns freshly landed parameter rows into the packed constants of the group
+    auto adopt_params = [&]() {
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            pair_up(sraw[d], sc[d]);
+            if constexpr (kHasOffset) {
+                pair_up(oraw[d], ofc[d]);
+            }
+        }
+        folded = false;
+        if constexpr (kHasOffset) {
+            folded = all_offsets_integral(ofc);
+            if (folded) {
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+#pragma unroll
+                    for (int c2 = 0; c2 < 4; ++c2) {
+                        ofc[d][c2] = (c2 & 1) ? ofc[d][c2] - k72 : ofc[d][c2] - k1032;  // exact
+                    }
+                }
+            }
+        }
+        params_pending = false;
+    };
+    auto compute = [&](const char* stage) {
+        const uint32_t sa = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)stage));
+        const uint32_t a_own = sa + lane * 16u;                           // what this lane fetched itself
+        const uint32_t a_x = sa + 8u * 1024u + (jj >> 3) * 64u + g * 16u;  // row (jj >> 3), k 8 g .. 8 g + 7
+        u32x4 wd[8], xraw[1];
+        ASCQ_DS_READ128(wd[0], a_own, 0 * 1024);
+        ASCQ_DS_READ128(wd[1], a_own, 1 * 1024);
+        ASCQ_DS_READ128(wd[2], a_own, 2 * 1024);
+        ASCQ_DS_READ128(wd[3], a_own, 3 * 1024);
+        ASCQ_DS_READ128(wd[4], a_own, 4 * 1024);
+        ASCQ_DS_READ128(wd[5], a_own, 5 * 1024);
+        ASCQ_DS_READ128(wd[6], a_own, 6 * 1024);
+        ASCQ_DS_READ128(wd[7], a_own, 7 * 1024);
+        ASCQ_DS_READ128(xraw[0], a_x, 0);
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(wd[0]), "+v"(wd[1]), "+v"(wd[2]), "+v"(wd[3]), "+v"(wd[4]), "+v"(wd[5]), "+v"(wd[6]),
+                       "+v"(wd[7]), "+v"(xraw[0])
+                     :
+                     : "memory");
+        u32x4 xc[1];
+        xc[0] = (p.m0 + (jj >> 3) < p.m) ? xraw[0] : u32x4{0u, 0u, 0u, 0u};
+        if (kHasOffset && folded) {
+            w4_accumulate<1, kHasOffset, true>(wd, xc, sc, ofc, amask, acc);
+        } else {
+            w4_accumulate<1, kHasOffset, false>(wd, xc, sc, ofc, amask, acc);
+        }
+        if (++done_in_block == cb_chunks) {  // the run leaves this column block
+            done_in_block = 0;
+            flush();
+        }
+    };
+
+    char* s0 = S0 + wave * kStage;
+    char* s1 = S1 + wave * kStage;
+    issue(s0, true);
+    uint32_t c = c_begin;
+    while (true) {
+        ASCQ_WAIT_VMCNT(0);  // chunk c (and parameter rows fetched ahead of it) has landed
+        if (params_pending) adopt_params();
+        if (c + 1u < c_end) issue(s1, false);
+        compute(s0);
+        if (++c == c_end) break;
+        ASCQ_WAIT_VMCNT(0);
+        if (params_pending) adopt_params();
+        if (c + 1u < c_end) issue(s0, false);
+        compute(s1);
+        if (++c == c_end) break;
+    }
+    if (done_in_block != 0) {
+        flush();
+    }
+}
+
+// Adds the pieces of all streams that worked on a column block and rounds once to half.  A piece is the image of
+// the accumulators of a wavefront, [16 registers][64 lanes] = the 2 rows x 512 columns of the block, so the pieces are
+// added element by element in that layout with fully coalesced 16-byte loads, and only the final store is scattered.
+// One workgroup per (column block, row pair): 4 sub-groups of 256 lanes take the pieces i = sub, sub + 4, ... in
+// ascending k order, the four sums are combined as (s0 + s1) + (s2 + s3): deterministic.
+template <int MP>
+__global__ __launch_bounds__(1024) void w4a16_sum_kernel(W4Params p)
+{
+    __shared__ f32x4 part[4][256];
+    const uint32_t sub = threadIdx.x >> 8, t = threadIdx.x & 255u;
+    const uint32_t blk = blockIdx.x, q = blockIdx.y;
     const uint32_t first_chunk = blk * p.chunks_per_block, end_chunk = first_chunk + p.chunks_per_block;
     // the stream that holds first_chunk, and the first one past the block
     const uint32_t big = p.rem * (p.per + 1u);  // chunks owned by the longer streams
-    uint32_t w0 = first_chunk < big ? first_chunk / (p.per + 1u) : p.rem + (first_chunk - big) / p.per;
+    const uint32_t w0 = first_chunk < big ? first_chunk / (p.per + 1u) : p.rem + (first_chunk - big) / p.per;
     uint32_t w1 = end_chunk <= big ? (end_chunk + p.per) / (p.per + 1u) : p.rem + (end_chunk - big + p.per - 1u) / p.per;
     w1 = w1 < p.waves ? w1 : p.waves;
     const size_t stride = static_cast<size_t>(p.max_seg) * MP * 1024u;  // floats between streams
     // the first stream may have begun in an earlier block; all later ones begin inside this block (piece 0)
-    const uint32_t seg0 = blk - stream_begin(p, w0) / p.chunks_per_block;
-    const float* src = p.partial + (static_cast<size_t>(w0) * p.max_seg * MP + q) * 1024u + e;
-    float s = src[static_cast<size_t>(seg0) * MP * 1024u];
-    src += stride;
-    for (uint32_t w = w0 + 1u; w < w1; w += 8u) {
-        float v[8];
+    const size_t first_extra = static_cast<size_t>(blk - stream_begin(p, w0) / p.chunks_per_block) * MP * 1024u;
+    const float* base = p.partial + (static_cast<size_t>(w0) * p.max_seg * MP + q) * 1024u + 4u * t;
+    f32x4 s = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (uint32_t w = w0 + sub; w < w1; w += 32u) {
+        f32x4 v[8];
 #pragma unroll
         for (uint32_t u = 0; u < 8u; ++u) {  // 8 independent loads in flight, then an ordered sum
-            v[u] = (w + u < w1) ? src[static_cast<size_t>(u) * stride] : 0.0f;
+            const uint32_t wu = w + 4u * u;
+            const size_t off = static_cast<size_t>(wu - w0) * stride + (wu == w0 ? first_extra : 0u);
+            v[u] = wu < w1 ? *reinterpret_cast<const f32x4*>(base + off) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
         }
 #pragma unroll
         for (uint32_t u = 0; u < 8u; ++u) s += v[u];
-        src += 8u * stride;
     }
-    p.y[static_cast<size_t>(m) * p.n + col] = static_cast<uint16_t>(f32_to_half_bits(s));
+    part[sub][t] = s;
+    __syncthreads();
+    if (sub != 0u) {
+        return;
+    }
+    const f32x4 tot = (part[0][t] + part[1][t]) + (part[2][t] + part[3][t]);
+    // element e = (d * 4 + r) * 64 + g * 16 + jj: register r of lane (g, jj) in tile d holds row (g >> 1) of the pair
+    // and column slot b8 = 4 (g & 1) + r of the dword, with column = (b8 >> 1) + 4 (b8 & 1)
+#pragma unroll
+    for (uint32_t i = 0; i < 4u; ++i) {
+        const uint32_t e = 4u * t + i;
+        const uint32_t jj = e & 15u, g = (e >> 4) & 3u, r = (e >> 6) & 3u, d = e >> 8;
+        const uint32_t b8 = 4u * (g & 1u) + r;
+        const uint32_t col = blk * kColsPerBlock + jj * 32u + d * 8u + (b8 >> 1) + 4u * (b8 & 1u);
+        const uint32_t m = p.m0 + 2u * q + (g >> 1);
+        if (col < p.n && m < p.m) {
+            p.y[static_cast<size_t>(m) * p.n + col] = static_cast<uint16_t>(f32_to_half_bits(tot[i]));
+        }
+    }
 }
 
 // Any shape: one lane per output element.
@@ -442,16 +639,24 @@ struct W4Plan {
     uint32_t waves, chunks_per_block, total_chunks, max_seg;
 };
 
-W4Plan make_plan(uint32_t n, uint32_t k)
+W4Plan make_plan(uint32_t n, uint32_t k, uint32_t max_waves)
 {
     W4Plan pl;
     const uint32_t blocks_n = (n + kColsPerBlock - 1u) / kColsPerBlock;
     pl.chunks_per_block = k / kChunkRows;
     pl.total_chunks = blocks_n * pl.chunks_per_block;
-    pl.waves = pl.total_chunks < kMaxWaves ? pl.total_chunks : kMaxWaves;
+    pl.waves = pl.total_chunks < max_waves ? pl.total_chunks : max_waves;
     const uint32_t per = (pl.total_chunks + pl.waves - 1u) / pl.waves;  // longest run
     pl.max_seg = (per + pl.chunks_per_block - 2u) / pl.chunks_per_block + 1u;
     return pl;
+}
+
+// bytes of workspace: the larger of the two kernels' needs (two streams per SIMD with one row pair, one with four)
+size_t workspace_need(uint32_t n, uint32_t k)
+{
+    const W4Plan a = make_plan(n, k, kMaxWaves), b = make_plan(n, k, 2u * kMaxWaves);
+    const size_t na = static_cast<size_t>(a.waves) * a.max_seg * kMaxPairs, nb = static_cast<size_t>(b.waves) * b.max_seg;
+    return (na > nb ? na : nb) * 1024u * sizeof(float);
 }
 
 bool fast_ok(const ascq_w4a16_desc* d, const void* x, const void* w, const void* scale, const void* offset)
@@ -486,8 +691,7 @@ extern "C" int ascq_matmul_w4a16_workspace_size(const ascq_w4a16_desc* d, size_t
     ASCQ_REQUIRE(bytes != nullptr, ASCQ_ENULL, "ascq_matmul_w4a16_workspace_size: bytes is NULL");
     *bytes = 0;
     if (d->k % kChunkRows == 0) {
-        const W4Plan pl = make_plan(d->n, d->k);
-        *bytes = static_cast<size_t>(pl.waves) * pl.max_seg * kMaxPairs * 1024u * sizeof(float);
+        *bytes = workspace_need(d->n, d->k);
     }
     return ASCQ_OK;
 }
@@ -522,23 +726,37 @@ extern "C" int ascq_matmul_w4a16(const ascq_w4a16_desc* d, void* y, const void* 
         w4a16_generic_kernel<<<static_cast<uint32_t>(blocks), kThreads, 0, st>>>(p);
         return launch_status("ascq_matmul_w4a16 (generic)");
     }
-    const W4Plan pl = make_plan(d->n, d->k);
-    p.waves = pl.waves;
-    p.chunks_per_block = pl.chunks_per_block;
-    p.total_chunks = pl.total_chunks;
-    p.max_seg = pl.max_seg;
-    p.per = pl.total_chunks / pl.waves;
-    p.rem = pl.total_chunks % pl.waves;
-    const size_t need = static_cast<size_t>(pl.waves) * pl.max_seg * kMaxPairs * 1024u * sizeof(float);
+    const size_t need = workspace_need(d->n, d->k);
     ASCQ_REQUIRE(workspace != nullptr && workspace_bytes >= need, ASCQ_EINVAL,
                  "ascq_matmul_w4a16: workspace of %zu bytes required (see ascq_matmul_w4a16_workspace_size)", need);
     ASCQ_REQUIRE(aligned16(workspace), ASCQ_EALIGN, "ascq_matmul_w4a16: workspace must be 16-byte aligned");
-    const uint32_t grid = (pl.waves + 3u) / 4u;
-    const uint32_t col_blocks = (d->n + kThreads - 1) / kThreads;
+    const uint32_t col_blocks = (d->n + kColsPerBlock - 1u) / kColsPerBlock;
+    auto set_plan = [&](uint32_t max_waves) {
+        const W4Plan pl = make_plan(d->n, d->k, max_waves);
+        p.waves = pl.waves;
+        p.chunks_per_block = pl.chunks_per_block;
+        p.total_chunks = pl.total_chunks;
+        p.max_seg = pl.max_seg;
+        p.per = pl.total_chunks / pl.waves;
+        p.rem = pl.total_chunks % pl.waves;
+    };
     // at most 8 activation rows per pass over the weights
     for (uint32_t m0 = 0; m0 < d->m; m0 += 2 * kMaxPairs) {
         const uint32_t left = d->m - m0;
         p.m0 = m0;
+        if (left <= 2) {
+            set_plan(2u * kMaxWaves);  // two streams per SIMD
+            const uint32_t grid = (p.waves + 7u) / 8u;
+            if (d->has_offset) {
+                w4a16_gemv_kernel<true><<<grid, 512, 0, st>>>(p);
+            } else {
+                w4a16_gemv_kernel<false><<<grid, 512, 0, st>>>(p);
+            }
+            w4a16_sum_kernel<1><<<dim3(col_blocks, 1), 1024, 0, st>>>(p);
+            continue;
+        }
+        set_plan(kMaxWaves);
+        const uint32_t grid = (p.waves + 3u) / 4u;
 #define ASCQ_W4_LAUNCH(MPV)                                                              \
     do {                                                                                 \
         if (d->has_offset) {                                                             \
@@ -546,11 +764,9 @@ extern "C" int ascq_matmul_w4a16(const ascq_w4a16_desc* d, void* y, const void* 
         } else {                                                                         \
             w4a16_stream_kernel<MPV, false><<<grid, kThreads, 0, st>>>(p);               \
         }                                                                                \
-        w4a16_sum_kernel<MPV><<<dim3(col_blocks, 2 * MPV), kThreads, 0, st>>>(p);        \
+        w4a16_sum_kernel<MPV><<<dim3(col_blocks, MPV), 1024, 0, st>>>(p);           \
     } while (0)
-        if (left <= 2) {
-            ASCQ_W4_LAUNCH(1);
-        } else if (left <= 4) {
+        if (left <= 4) {
             ASCQ_W4_LAUNCH(2);
         } else {
             ASCQ_W4_LAUNCH(4);
