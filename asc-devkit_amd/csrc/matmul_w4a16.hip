@@ -35,7 +35,7 @@ constexpr int kThreads = 256;          // four independent wavefronts per workgr
 constexpr uint32_t kColsPerBlock = 512;
 constexpr uint32_t kChunkRows = 32;
 constexpr uint32_t kMaxWaves = 1024;   // 256 compute units x 4 SIMDs
-constexpr int kMaxPairs = 4;           // activation-row pairs per pass over the weights
+constexpr int kMaxPairs = 8;           // activation-row pairs per pass over the weights
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef __attribute__((address_space(1))) const void* gptr_t;
@@ -304,6 +304,12 @@ __global__ __launch_bounds__(kThreads) void w4a16_stream_kernel(W4Params p)
         if constexpr (MP > 1) ASCQ_DS_READ128(xraw[1], a_x, (8 + kParamInstr) * 1024 + 128);
         if constexpr (MP > 2) ASCQ_DS_READ128(xraw[2], a_x, (8 + kParamInstr) * 1024 + 256);
         if constexpr (MP > 3) ASCQ_DS_READ128(xraw[3], a_x, (8 + kParamInstr) * 1024 + 384);
+        if constexpr (MP > 4) {
+            ASCQ_DS_READ128(xraw[4], a_x, (8 + kParamInstr) * 1024 + 512);
+            ASCQ_DS_READ128(xraw[5], a_x, (8 + kParamInstr) * 1024 + 640);
+            ASCQ_DS_READ128(xraw[6], a_x, (8 + kParamInstr) * 1024 + 768);
+            ASCQ_DS_READ128(xraw[7], a_x, (8 + kParamInstr) * 1024 + 896);
+        }
         // every value read above is an in/out operand of the wait, so nothing uses one before it has arrived
         asm volatile("s_waitcnt lgkmcnt(0)"
                      : "+v"(wd[0]), "+v"(wd[1]), "+v"(wd[2]), "+v"(wd[3]), "+v"(wd[4]), "+v"(wd[5]), "+v"(wd[6]),
@@ -740,7 +746,7 @@ extern "C" int ascq_matmul_w4a16(const ascq_w4a16_desc* d, void* y, const void* 
         p.per = pl.total_chunks / pl.waves;
         p.rem = pl.total_chunks % pl.waves;
     };
-    // at most 8 activation rows per pass over the weights
+    // at most 16 activation rows per pass over the weights
     for (uint32_t m0 = 0; m0 < d->m; m0 += 2 * kMaxPairs) {
         const uint32_t left = d->m - m0;
         p.m0 = m0;
@@ -768,8 +774,10 @@ extern "C" int ascq_matmul_w4a16(const ascq_w4a16_desc* d, void* y, const void* 
     } while (0)
         if (left <= 4) {
             ASCQ_W4_LAUNCH(2);
-        } else {
+        } else if (left <= 8) {
             ASCQ_W4_LAUNCH(4);
+        } else {
+            ASCQ_W4_LAUNCH(8);
         }
 #undef ASCQ_W4_LAUNCH
     }
