@@ -159,6 +159,9 @@ __device__ __forceinline__ uint32_t xcd_remap(uint32_t pid, uint32_t total)
 bool gemm_dma_supported(const GemmParams& p);
 int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st);
 uint32_t gemm_dma_skinny_splits(uint32_t m, uint32_t n, uint32_t k);
+bool gemm_stream_supported(const GemmParams& p);
+size_t gemm_stream_workspace(uint32_t m, uint32_t n, uint32_t k);
+int launch_gemm_stream(const GemmParams& p, void* workspace, hipStream_t st);
 int launch_gemm_dma_skinny(GemmParams& p, void* workspace, size_t workspace_bytes, hipStream_t st);
 
 }  // namespace ascq

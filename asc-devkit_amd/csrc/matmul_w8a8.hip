@@ -564,6 +564,12 @@ extern "C" int ascq_matmul_w8a8_workspace_size(const ascq_matmul_desc* d, size_t
             *bytes = need;
         }
     }
+    if (!d->trans_a && !d->trans_b && d->n % 16 == 0) {
+        const size_t need = gemm_stream_workspace(d->m, d->n, d->k);
+        if (need > *bytes) {
+            *bytes = need;
+        }
+    }
     return ASCQ_OK;
 }
 
@@ -591,6 +597,10 @@ extern "C" int ascq_matmul_w8a8(const ascq_matmul_desc* d, void* c, const void* 
         if (blocks > 65536) blocks = 65536;
         gemm_generic_kernel<<<static_cast<uint32_t>(blocks), kThreads, 0, st>>>(p, d->trans_a, d->trans_b);
         return launch_status("ascq_matmul_w8a8 (generic)");
+    }
+    if (!d->trans_b && gemm_stream_supported(p) && workspace != nullptr && aligned16(workspace) &&
+        workspace_bytes >= gemm_stream_workspace(d->m, d->n, d->k)) {
+        return launch_gemm_stream(p, workspace, st);
     }
     if (d->m <= kSkinnyMaxM && !d->trans_b && gemm_dma_supported(p)) {
         return launch_gemm_dma_skinny(p, workspace, workspace_bytes, st);
