@@ -29,7 +29,7 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E peak, GB/s
 # (FETCH_SIZE reads 0.5 per KiB there, WRITE_SIZE 1.0 per KiB).  Measured offline and recorded here; a run of this
 # file does not re-measure them.
 GEMM_TRAFFIC_BYTES = 228336230   # M=2048 GEMM, both launches: 183.2 MB fetched + 45.1 MB written
-GEMV_TRAFFIC_BYTES = 135269990   # W4A16 M=1 GEMV, stream + sum kernels: 130.8 MB fetched + 4.4 MB written
+GEMV_TRAFFIC_BYTES = 145573273   # W4A16 M=1 GEMV, stream + sum kernels: 136.9 MB fetched + 8.6 MB written
 
 
 def main():
