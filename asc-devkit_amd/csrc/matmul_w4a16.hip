@@ -255,11 +255,14 @@ __global__ __launch_bounds__(kThreads) void w4a16_stream_kernel(W4Params p)
 #pragma unroll
         for (int q = 0; q < MP; ++q) {
             float* dst = p.partial + ((static_cast<size_t>(gw) * p.max_seg + seg) * MP + q) * 1024u + lane;
+            const bool row_valid = p.m0 + 2u * q + (g >> 1) < p.m;  // lanes of a missing second row hold zeros
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
+                if (row_valid) {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    dst[(d * 4 + r) * 64] = acc[q][d][r];
+                    for (int r = 0; r < 4; ++r) {
+                        dst[(d * 4 + r) * 64] = acc[q][d][r];
+                    }
                 }
                 acc[q][d] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
             }
@@ -476,11 +479,14 @@ __global__ __launch_bounds__(512) void w4a16_gemv_kernel(W4Params p)
     uint32_t seg = 0, done_in_block = c_begin % cb_chunks;
     auto flush = [&]() {
         float* dst = p.partial + (static_cast<size_t>(gw) * p.max_seg + seg) * 1024u + lane;
+        const bool row_valid = p.m0 + (g >> 1) < p.m;  // lanes of a missing second row hold zeros: not stored
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
+            if (row_valid) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                dst[(d * 4 + r) * 64] = acc[0][d][r];
+                for (int r = 0; r < 4; ++r) {
+                    dst[(d * 4 + r) * 64] = acc[0][d][r];
+                }
             }
             acc[0][d] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
         }
@@ -584,8 +590,10 @@ __global__ __launch_bounds__(1024) void w4a16_sum_kernel(W4Params p)
     // the first stream may have begun in an earlier block; all later ones begin inside this block (piece 0)
     const size_t first_extra = static_cast<size_t>(blk - stream_begin(p, w0) / p.chunks_per_block) * MP * 1024u;
     const float* base = p.partial + (static_cast<size_t>(w0) * p.max_seg * MP + q) * 1024u + 4u * t;
+    // the four elements of a lane share their row (g >> 1 of the pair); a row past m was never written
+    const bool row_valid = p.m0 + 2u * q + ((t >> 2) & 3u) / 2u < p.m;
     f32x4 s = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-    for (uint32_t w = w0 + sub; w < w1; w += 32u) {
+    for (uint32_t w = w0 + sub; row_valid && w < w1; w += 32u) {
         f32x4 v[8];
 #pragma unroll
         for (uint32_t u = 0; u < 8u; ++u) {  // 8 independent loads in flight, then an ordered sum
