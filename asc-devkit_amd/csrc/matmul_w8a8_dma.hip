@@ -63,9 +63,9 @@ __device__ __forceinline__ float epi_value(int32_t acc, float chan, float tok, f
 // wavefront, 64 KiB of LDS so that two workgroups share a CU; with kSplitK the K range is divided over blockIdx.y and
 // the int32 partial tiles go to a workspace [split][m][n] that a second kernel sums (small M: the weights are read
 // once, by enough workgroups to fill the chip).
-template <int BM, int BN, bool kSplitK>
+template <int BM, int BN, bool kSplitK, bool kGrouped = false>
 __global__ __launch_bounds__(kThreads, (BM * BK + BK * BN) * 2 <= 65536 ? 2 : 1) void gemm_dma_kernel(
-    GemmParams p, int grouped, uint32_t col_begin)
+    GemmParams p, uint32_t col_begin)
 {
     constexpr int kWN = BN / 64;            // wavefronts along N
     constexpr int kWM = 8 / kWN;            // wavefronts along M
@@ -92,7 +92,7 @@ __global__ __launch_bounds__(kThreads, (BM * BK + BK * BN) * 2 <= 65536 ? 2 : 1)
     uint32_t row0 = ms * BM, row_end = p.m;
     const int8_t* Bmat = p.b;
     size_t chan_off = 0;
-    if (grouped) {
+    if constexpr (kGrouped) {
         // walk the groups: group g owns tile slots [slot, slot + ceil(rows / BM))
         uint32_t slot = 0;
         int64_t off = 0;
@@ -250,21 +250,24 @@ __global__ __launch_bounds__(kThreads, (BM * BK + BK * BN) * 2 <= 65536 ? 2 : 1)
     }
     asm volatile("s_waitcnt vmcnt(0)");
     __syncthreads();
+    // A wavefront whose rows all lie past the end of the tile's group (ragged grouped tiles) skips the matrix work and
+    // only keeps the loads and barriers going: its SIMD then runs one wavefront's MFMAs per K step instead of two.
+    const bool wave_active = !kGrouped || row0 + wm * (TI * 32u) < row_end;
     uint32_t s = 0;
     for (; s + 1 < steps; s += 2) {
         issue((s + 1) * BK, A1, B1);
-        compute(A0, B0);
+        if (wave_active) compute(A0, B0);
         asm volatile("s_waitcnt vmcnt(0)");
         __syncthreads();
         if (s + 2 < steps) {
             issue((s + 2) * BK, A0, B0);
         }
-        compute(A1, B1);
+        if (wave_active) compute(A1, B1);
         asm volatile("s_waitcnt vmcnt(0)");
         __syncthreads();
     }
     if (s < steps) {  // odd number of K steps: the last one sits in stage 0
-        compute(A0, B0);
+        if (wave_active) compute(A0, B0);
     }
 
     // ---- epilogue: register r of lane l in a 32x32 block is row 8*(r/4) + 4*(l/32) + r%4, column l%32
@@ -441,13 +444,17 @@ int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st)
         if (narrow_cols) {
             q.n = p.n;  // row pitch stays n; columns >= wide_cols * 256 are simply not assigned to any tile
         }
-        gemm_dma_kernel<256, 256, false><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(q, grouped ? 1 : 0, 0u);
+        if (grouped) {
+            gemm_dma_kernel<256, 256, false, true><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(q, 0u);
+        } else {
+            gemm_dma_kernel<256, 256, false><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(q, 0u);
+        }
     }
     if (narrow_cols) {
         const uint32_t col_begin = wide_cols * 256u;
         p.tiles_n = (p.n - col_begin + 127u) / 128u;
         const uint32_t t = p.tiles_m * p.tiles_n;
-        gemm_dma_kernel<256, 128, false><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(p, 0, col_begin);
+        gemm_dma_kernel<256, 128, false><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(p, col_begin);
     }
     return launch_status(grouped ? "ascq_group_matmul_w8a8" : "ascq_matmul_w8a8");
 }
@@ -478,12 +485,12 @@ int launch_gemm_dma_skinny(GemmParams& p, void* workspace, size_t workspace_byte
         splits = 1;
     }
     if (splits == 1) {
-        gemm_dma_kernel<128, 128, false><<<t, kThreads, 0, st>>>(p, 0, 0u);
+        gemm_dma_kernel<128, 128, false><<<t, kThreads, 0, st>>>(p, 0u);
         return launch_status("ascq_matmul_w8a8");
     }
     p.k_splits = splits;
     p.partial = static_cast<int32_t*>(workspace);
-    gemm_dma_kernel<128, 128, true><<<dim3(t, splits), kThreads, 0, st>>>(p, 0, 0u);
+    gemm_dma_kernel<128, 128, true><<<dim3(t, splits), kThreads, 0, st>>>(p, 0u);
     int rc = launch_status("ascq_matmul_w8a8 (split-K)");
     if (rc != ASCQ_OK) {
         return rc;
