@@ -46,7 +46,13 @@ def oracle_mm(desc, a, b, bias=None, quant=None, tok=None):
 # shapes chosen to hit: the 32-row split-K tile, the 128-row tile with a row tail, the 256-row tile with row and
 # column tails, K tails (K not a multiple of 128), and the generic kernel (odd sizes)
 SHAPES = [(1, 256, 512), (16, 1024, 4096), (32, 264, 1040), (33, 256, 256), (128, 512, 384), (300, 520, 272),
-          (1100, 776, 400), (2048, 512, 128), (19, 23, 77), (40, 100, 48)]
+          (1100, 776, 400), (2048, 512, 128), (19, 23, 77), (40, 100, 48),
+          # the weight-stream kernel (m <= 32, k % 64 == 0): one chunk, column tails, runs that cross column blocks
+          (1, 16, 64), (7, 144, 192), (32, 400, 64), (32, 1040, 2048), (5, 2064, 8192),
+          # 128 x 128 tiles with and without a K split, row / column tails
+          (33, 144, 128), (200, 528, 384), (512, 272, 256), (130, 2064, 1024),
+          # 256-row tiles: a partial last round (narrow tiles), K steps odd and even
+          (513, 528, 256), (2048, 2832, 384)]
 
 
 @pytest.mark.parametrize("m,n,k", SHAPES)
