@@ -393,13 +393,13 @@ __global__ __launch_bounds__(kThreads) void w4a16_stream_kernel(W4Params p)
     }
 }
 
-// One or two activation rows (the decode GEMV): the same streams, two per SIMD.  To fit 8 rings into the LDS the
+// Up to four activation rows (MP = 1 or 2 row pairs; the decode GEMV): the same streams, two per SIMD.  To fit 8 rings into the LDS the
 // ring has two stages and holds only the weights (8 KiB) and the activations (256 bytes); the scale / offset rows of
 // a quantisation group are fetched into registers when a chunk opens a new group, ahead of that chunk's weights, so
 // they have landed whenever the weights have.  With two stages one chunk is in flight behind the one being computed
 // and the wait before a chunk is simply for everything outstanding; the second wavefront of the SIMD fills the time
 // a wavefront spends waiting or stalled on its own dependent instructions.
-template <bool kHasOffset>
+template <int MP, bool kHasOffset>
 __global__ __launch_bounds__(512) void w4a16_gemv_kernel(W4Params p)
 {
     constexpr int kStage = 8 * 1024 + 256;  // bytes per wavefront and stage
@@ -448,10 +448,10 @@ __global__ __launch_bounds__(512) void w4a16_gemv_kernel(W4Params p)
             __builtin_amdgcn_global_load_lds((gptr_t)(wsrc + static_cast<size_t>(u) * row_bytes),
                                              (lds_ptr_t)(stage + u * 1024), 16, 0, 0);
         }
-        // activations of the chunk's 32 k for two rows, one dword per lane: lane l fetches dword (l & 15) of row
-        // m0 + ((l >> 4) & 1); a missing second row fetches the first and is zeroed when used
+        // activations of the chunk's 32 k for 2 MP rows, one dword per lane: lane l fetches dword (l & 15) of row
+        // m0 + ((l >> 4) & (2 MP - 1)); a missing row fetches the last one and is zeroed when used
         {
-            const uint32_t m = p.m0 + ((lane >> 4) & 1u);
+            const uint32_t m = p.m0 + ((lane >> 4) & (2u * MP - 1u));
             const uint32_t mc = m < p.m ? m : p.m - 1u;
             __builtin_amdgcn_global_load_lds((gptr_t)(p.x + static_cast<size_t>(mc) * p.k + krow + 2u * (lane & 15u)),
                                              (lds_ptr_t)(stage + 8 * 1024), 4, 0, 0);
@@ -463,9 +463,12 @@ __global__ __launch_bounds__(512) void w4a16_gemv_kernel(W4Params p)
     };
 
     // ---- consumer side
-    f32x4 acc[1][4];
+    f32x4 acc[MP][4];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) acc[0][t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int q = 0; q < MP; ++q) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) acc[q][t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
     const uint32_t slot = jj & 7u;
     uint32_t amask[4];
 #pragma unroll
@@ -478,17 +481,20 @@ __global__ __launch_bounds__(512) void w4a16_gemv_kernel(W4Params p)
     bool folded = false;
     uint32_t seg = 0, done_in_block = c_begin % cb_chunks;
     auto flush = [&]() {
-        float* dst = p.partial + (static_cast<size_t>(gw) * p.max_seg + seg) * 1024u + lane;
-        const bool row_valid = p.m0 + (g >> 1) < p.m;  // lanes of a missing second row hold zeros: not stored
 #pragma unroll
-        for (int d = 0; d < 4; ++d) {
-            if (row_valid) {
+        for (int q = 0; q < MP; ++q) {
+            float* dst = p.partial + ((static_cast<size_t>(gw) * p.max_seg + seg) * MP + q) * 1024u + lane;
+            const bool row_valid = p.m0 + 2u * q + (g >> 1) < p.m;  // lanes of a missing row hold zeros: not stored
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    dst[(d * 4 + r) * 64] = acc[0][d][r];
+            for (int d = 0; d < 4; ++d) {
+                if (row_valid) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        dst[(d * 4 + r) * 64] = acc[q][d][r];
+                    }
                 }
+                acc[q][d] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
             }
-            acc[0][d] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
         }
         ++seg;
     };
@@ -519,8 +525,8 @@ __global__ __launch_bounds__(512) void w4a16_gemv_kernel(W4Params p)
     auto compute = [&](const char* stage) {
         const uint32_t sa = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)stage));
         const uint32_t a_own = sa + lane * 16u;                           // what this lane fetched itself
-        const uint32_t a_x = sa + 8u * 1024u + (jj >> 3) * 64u + g * 16u;  // row (jj >> 3), k 8 g .. 8 g + 7
-        u32x4 wd[8], xraw[1];
+        const uint32_t a_x = sa + 8u * 1024u + (jj >> 3) * 64u + g * 16u;  // row (jj >> 3) of a pair, k 8 g .. 8 g + 7
+        u32x4 wd[8], xraw[MP];
         ASCQ_DS_READ128(wd[0], a_own, 0 * 1024);
         ASCQ_DS_READ128(wd[1], a_own, 1 * 1024);
         ASCQ_DS_READ128(wd[2], a_own, 2 * 1024);
@@ -530,17 +536,22 @@ __global__ __launch_bounds__(512) void w4a16_gemv_kernel(W4Params p)
         ASCQ_DS_READ128(wd[6], a_own, 6 * 1024);
         ASCQ_DS_READ128(wd[7], a_own, 7 * 1024);
         ASCQ_DS_READ128(xraw[0], a_x, 0);
+        if constexpr (MP > 1) ASCQ_DS_READ128(xraw[1], a_x, 128);  // the next pair: two rows of 64 bytes further on
         asm volatile("s_waitcnt lgkmcnt(0)"
                      : "+v"(wd[0]), "+v"(wd[1]), "+v"(wd[2]), "+v"(wd[3]), "+v"(wd[4]), "+v"(wd[5]), "+v"(wd[6]),
                        "+v"(wd[7]), "+v"(xraw[0])
                      :
                      : "memory");
-        u32x4 xc[1];
-        xc[0] = (p.m0 + (jj >> 3) < p.m) ? xraw[0] : u32x4{0u, 0u, 0u, 0u};
+        if constexpr (MP > 1) asm volatile("" : "+v"(xraw[1]));
+        u32x4 xc[MP];
+#pragma unroll
+        for (int q = 0; q < MP; ++q) {
+            xc[q] = (p.m0 + 2u * q + (jj >> 3) < p.m) ? xraw[q] : u32x4{0u, 0u, 0u, 0u};
+        }
         if (kHasOffset && folded) {
-            w4_accumulate<1, kHasOffset, true>(wd, xc, sc, ofc, amask, acc);
+            w4_accumulate<MP, kHasOffset, true>(wd, xc, sc, ofc, amask, acc);
         } else {
-            w4_accumulate<1, kHasOffset, false>(wd, xc, sc, ofc, amask, acc);
+            w4_accumulate<MP, kHasOffset, false>(wd, xc, sc, ofc, amask, acc);
         }
         if (++done_in_block == cb_chunks) {  // the run leaves this column block
             done_in_block = 0;
@@ -665,11 +676,12 @@ W4Plan make_plan(uint32_t n, uint32_t k, uint32_t max_waves)
     return pl;
 }
 
-// bytes of workspace: the larger of the two kernels' needs (two streams per SIMD with one row pair, one with four)
+// bytes of workspace: the larger of the two kernels' needs (two streams per SIMD with up to two row pairs, one with
+// up to eight)
 size_t workspace_need(uint32_t n, uint32_t k)
 {
     const W4Plan a = make_plan(n, k, kMaxWaves), b = make_plan(n, k, 2u * kMaxWaves);
-    const size_t na = static_cast<size_t>(a.waves) * a.max_seg * kMaxPairs, nb = static_cast<size_t>(b.waves) * b.max_seg;
+    const size_t na = static_cast<size_t>(a.waves) * a.max_seg * kMaxPairs, nb = static_cast<size_t>(b.waves) * b.max_seg * 2u;
     return (na > nb ? na : nb) * 1024u * sizeof(float);
 }
 
@@ -758,15 +770,24 @@ extern "C" int ascq_matmul_w4a16(const ascq_w4a16_desc* d, void* y, const void* 
     for (uint32_t m0 = 0; m0 < d->m; m0 += 2 * kMaxPairs) {
         const uint32_t left = d->m - m0;
         p.m0 = m0;
-        if (left <= 2) {
+        if (left <= 4) {
             set_plan(2u * kMaxWaves);  // two streams per SIMD
             const uint32_t grid = (p.waves + 7u) / 8u;
-            if (d->has_offset) {
-                w4a16_gemv_kernel<true><<<grid, 512, 0, st>>>(p);
+#define ASCQ_W4_GEMV(MPV)                                                           \
+    do {                                                                            \
+        if (d->has_offset) {                                                        \
+            w4a16_gemv_kernel<MPV, true><<<grid, 512, 0, st>>>(p);                  \
+        } else {                                                                    \
+            w4a16_gemv_kernel<MPV, false><<<grid, 512, 0, st>>>(p);                 \
+        }                                                                           \
+        w4a16_sum_kernel<MPV><<<dim3(col_blocks, MPV), 1024, 0, st>>>(p);           \
+    } while (0)
+            if (left <= 2) {
+                ASCQ_W4_GEMV(1);
             } else {
-                w4a16_gemv_kernel<false><<<grid, 512, 0, st>>>(p);
+                ASCQ_W4_GEMV(2);
             }
-            w4a16_sum_kernel<1><<<dim3(col_blocks, 1), 1024, 0, st>>>(p);
+#undef ASCQ_W4_GEMV
             continue;
         }
         set_plan(kMaxWaves);
@@ -780,9 +801,7 @@ extern "C" int ascq_matmul_w4a16(const ascq_w4a16_desc* d, void* y, const void* 
         }                                                                                \
         w4a16_sum_kernel<MPV><<<dim3(col_blocks, MPV), 1024, 0, st>>>(p);           \
     } while (0)
-        if (left <= 4) {
-            ASCQ_W4_LAUNCH(2);
-        } else if (left <= 8) {
+        if (left <= 8) {
             ASCQ_W4_LAUNCH(4);
         } else {
             ASCQ_W4_LAUNCH(8);
