@@ -16,10 +16,11 @@
 //     0x6400 exponent trick (1024 + u, or 1024 + 16 u for the nibbles read 4 bits up, which saves the shift), one
 //     exact packed add / fma turns it into w, then one rounded half add of the offset and one rounded half multiply by
 //     the scale;
-//   * the multiply-accumulate runs on the matrix core: the 8 de-quantised halves of one dword are the B operand of
-//     v_mfma_f32_16x16x32_f16 as they are; the A operand of output row i carries x[k_g] in slot i and zeros elsewhere,
-//     so row i of the result is the running dot product of column i of the dword.  Rows 0-7 serve one activation row,
-//     rows 8-15 a second one; more activation rows take more MFMAs on the same de-quantised operand (fp32 sums);
+//   * the multiply-accumulate runs on the matrix core (v_mfma_f32_16x16x32_f16, fp32 sums).  For up to four
+//     activation rows the 8 de-quantised halves of one dword are the B operand as they are; the A operand of output
+//     row i carries x[k_g] in slot i and zeros elsewhere, so row i of the result is the running dot product of column
+//     i of the dword (rows 0-7 serve one activation row, rows 8-15 a second one).  From five rows on, the halves are
+//     regrouped so that a B operand is 8 consecutive k of one column and 16 activation rows fill the A operand;
 //   * when a wavefront's run leaves a column block (and at its end) the accumulators go to a workspace as they lie in
 //     registers; a second kernel adds, for every output, the pieces of all wavefronts that worked on its column block
 //     in ascending k order and rounds once to half, so results are deterministic.
@@ -35,7 +36,7 @@ constexpr int kThreads = 256;          // four independent wavefronts per workgr
 constexpr uint32_t kColsPerBlock = 512;
 constexpr uint32_t kChunkRows = 32;
 constexpr uint32_t kMaxWaves = 1024;   // 256 compute units x 4 SIMDs
-constexpr int kMaxPairs = 8;           // activation-row pairs per pass over the weights
+constexpr uint32_t kTileRows = 16;     // activation rows per pass over the weights
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef __attribute__((address_space(1))) const void* gptr_t;
@@ -45,7 +46,7 @@ struct W4Params {
     const uint8_t* w;
     const uint16_t* scale;
     const uint16_t* offset;
-    float* partial;  // [waves][max_seg][pairs][16 registers][64 lanes]
+    float* partial;  // [waves][max_seg][row pairs, or 8 slices of a 16-row tile][16 registers][64 lanes]
     uint16_t* y;
     uint32_t m, n, k, group_size, has_offset;
     uint32_t m0;                // first activation row of this pass
@@ -78,17 +79,55 @@ __device__ __forceinline__ uint32_t stream_begin(const W4Params& p, uint32_t wav
     return wave * p.per + (wave < p.rem ? wave : p.rem);
 }
 
-// De-quantises the 32 x 32 weights a lane holds of one chunk (8 rows x 4 dwords) and accumulates them against the
-// activations on the matrix core.  kFold: ofc holds offset - 1032 (even nibble pairs) / offset - 72 (odd pairs), which
-// is exact for integer offsets, so that w + offset is one exact operation; otherwise ofc is the offset itself.
+// De-quantises one dword (8 nibbles = 8 adjacent columns of one weight row) into 4 packed half pairs; pair c2 holds
+// columns (c2, c2 + 4).  kFold: ofc holds offset - 1032 (even pairs) / offset - 72 (odd pairs), which is exact for
+// integer offsets, so that w + offset is one exact operation; otherwise ofc is the offset itself.
+template <bool kHasOffset, bool kFold>
+__device__ __forceinline__ void w4_dequant_dword(uint32_t word, const f16x2 (&sc)[4], const f16x2 (&ofc)[4],
+                                                 f16x2 (&h)[4])
+{
+    const f16x2 k1032 = {static_cast<half_t>(1032.0f), static_cast<half_t>(1032.0f)};
+    const f16x2 k72 = {static_cast<half_t>(72.0f), static_cast<half_t>(72.0f)};
+    const f16x2 k16th = {static_cast<half_t>(0.0625f), static_cast<half_t>(0.0625f)};
+    const uint32_t qd = word ^ 0x88888888u;  // two's complement nibble -> offset binary u = w + 8
+    const uint32_t qh = qd >> 8;
+#pragma unroll
+    for (int c2 = 0; c2 < 4; ++c2) {
+        // (nibble c2, nibble c2 + 4) -> two exact halves: 1024 + u read in place (c2 even), 1024 + 16 u read
+        // 4 bits up (c2 odd, saves the shift)
+        uint32_t bits;
+        if (c2 & 1) {
+            asm("v_and_or_b32 %0, %1, %2, %3"
+                : "=v"(bits)
+                : "v"(c2 == 1 ? qd : qh), "s"(0x00F000F0u), "v"(0x64006400u));
+        } else {
+            asm("v_and_or_b32 %0, %1, %2, %3"
+                : "=v"(bits)
+                : "v"(c2 == 0 ? qd : qh), "s"(0x000F000Fu), "v"(0x64006400u));
+        }
+        if constexpr (kFold && kHasOffset) {
+            // w + offset in one exact operation
+            h[c2] = (c2 & 1) ? __builtin_elementwise_fma(bits_to_h2(bits), k16th, ofc[c2])
+                             : bits_to_h2(bits) + ofc[c2];
+        } else {
+            h[c2] = (c2 & 1) ? __builtin_elementwise_fma(bits_to_h2(bits), k16th, -k72)
+                             : bits_to_h2(bits) - k1032;  // w, exact
+            if constexpr (kHasOffset) {
+                h[c2] = h[c2] + ofc[c2];  // one rounding
+            }
+        }
+        h[c2] = sc[c2] * h[c2];  // one rounding
+    }
+}
+
+// De-quantises the 32 x 32 weights a lane holds of one chunk (8 rows x 4 dwords) and accumulates them against one or
+// two pairs of activation rows on the matrix core: the 8 halves of a dword are the B operand as they are, and the A
+// operand of output row i carries x[k_g] in slot i and zeros elsewhere.
 template <int MP, bool kHasOffset, bool kFold>
 __device__ __forceinline__ void w4_accumulate(const u32x4 (&wd)[8], const u32x4 (&xc)[MP], const f16x2 (&sc)[4][4],
                                               const f16x2 (&ofc)[4][4], const uint32_t (&amask)[4],
                                               f32x4 (&acc)[MP][4])
 {
-    const f16x2 k1032 = {static_cast<half_t>(1032.0f), static_cast<half_t>(1032.0f)};
-    const f16x2 k72 = {static_cast<half_t>(72.0f), static_cast<half_t>(72.0f)};
-    const f16x2 k16th = {static_cast<half_t>(0.0625f), static_cast<half_t>(0.0625f)};
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
         f16x8 a[MP];
@@ -102,41 +141,52 @@ __device__ __forceinline__ void w4_accumulate(const u32x4 (&wd)[8], const u32x4 
         }
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
-            const uint32_t qd = wd[u][d] ^ 0x88888888u;  // two's complement nibble -> offset binary u = w + 8
-            const uint32_t qh = qd >> 8;
             f16x2 h[4];
-#pragma unroll
-            for (int c2 = 0; c2 < 4; ++c2) {
-                // (nibble c2, nibble c2 + 4) -> two exact halves: 1024 + u read in place (c2 even), 1024 + 16 u read
-                // 4 bits up (c2 odd, saves the shift)
-                uint32_t bits;
-                if (c2 & 1) {
-                    asm("v_and_or_b32 %0, %1, %2, %3"
-                        : "=v"(bits)
-                        : "v"(c2 == 1 ? qd : qh), "s"(0x00F000F0u), "v"(0x64006400u));
-                } else {
-                    asm("v_and_or_b32 %0, %1, %2, %3"
-                        : "=v"(bits)
-                        : "v"(c2 == 0 ? qd : qh), "s"(0x000F000Fu), "v"(0x64006400u));
-                }
-                if constexpr (kFold && kHasOffset) {
-                    // w + offset in one exact operation
-                    h[c2] = (c2 & 1) ? __builtin_elementwise_fma(bits_to_h2(bits), k16th, ofc[d][c2])
-                                     : bits_to_h2(bits) + ofc[d][c2];
-                } else {
-                    h[c2] = (c2 & 1) ? __builtin_elementwise_fma(bits_to_h2(bits), k16th, -k72)
-                                     : bits_to_h2(bits) - k1032;  // w, exact
-                    if constexpr (kHasOffset) {
-                        h[c2] = h[c2] + ofc[d][c2];  // one rounding
-                    }
-                }
-                h[c2] = sc[d][c2] * h[c2];  // one rounding
-            }
+            w4_dequant_dword<kHasOffset, kFold>(wd[u][d], sc[d], ofc[d], h);
             f16x8 b;
             __builtin_memcpy(&b, h, 16);
 #pragma unroll
             for (int q = 0; q < MP; ++q) {
                 acc[q][d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[q], b, acc[q][d], 0, 0, 0);
+            }
+        }
+    }
+}
+
+// The same weights against a tile of 16 activation rows.  Over the 8 rows a lane holds, column c of dword d is the
+// 8 consecutive k the B operand of v_mfma_f32_16x16x32_f16 wants for one column, so the de-quantised halves only
+// have to be regrouped (one byte permute per operand dword) and x[16 rows][32 k] is the A operand as it lies in
+// memory.  Accumulator e = 8 d + 2 c2 + hi (kept as acc[e / 4][e % 4]) holds, for the lane's quarter g and column
+// group jj, rows 4 g .. 4 g + 3 of column 32 jj + 8 d + c2 + 4 hi.
+template <bool kHasOffset, bool kFold>
+__device__ __forceinline__ void w4_accumulate_tile(const u32x4 (&wd)[8], const u32x4& xa, const f16x2 (&sc)[4][4],
+                                                   const f16x2 (&ofc)[4][4], f32x4 (&acc)[8][4])
+{
+    f16x8 a;
+    __builtin_memcpy(&a, &xa, 16);
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+        f16x2 h[8][4];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            w4_dequant_dword<kHasOffset, kFold>(wd[u][d], sc[d], ofc[d], h[u]);
+        }
+#pragma unroll
+        for (int qh = 0; qh < 2; ++qh) {
+#pragma unroll
+            for (int dd = 0; dd < 4; ++dd) {
+                const int c2 = 2 * qh + (dd >> 1), hi = dd & 1;  // accumulator e = 8 d + 4 qh + dd
+                u32x4 bv;
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    uint32_t even, odd;
+                    __builtin_memcpy(&even, &h[2 * t][c2], 4);
+                    __builtin_memcpy(&odd, &h[2 * t + 1][c2], 4);
+                    bv[t] = __builtin_amdgcn_perm(odd, even, hi ? 0x07060302u : 0x05040100u);
+                }
+                f16x8 b;
+                __builtin_memcpy(&b, &bv, 16);
+                acc[2 * d + qh][dd] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[2 * d + qh][dd], 0, 0, 0);
             }
         }
     }
@@ -166,10 +216,11 @@ __device__ __forceinline__ bool all_offsets_integral(const f16x2 (&of)[4][4])
 // s_waitcnt vmcnt(n) only (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8)
 #define ASCQ_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | (7 << 4) | (15 << 8))
 
-// MP = number of activation-row pairs handled per pass over the weights (rows m0 .. m0 + 2 MP - 1).
+// Five to sixteen activation rows per pass over the weights (rows m0 .. m0 + 15): one stream per SIMD, the rows are
+// the rows of one MFMA tile (w4_accumulate_tile).  A piece of the workspace is [8 slices][16 registers][64 lanes].
 // Requires n % 32 == 0, k % 32 == 0, group_size % 32 == 0.
-template <int MP, bool kHasOffset>
-__global__ __launch_bounds__(kThreads) void w4a16_stream_kernel(W4Params p)
+template <bool kHasOffset>
+__global__ __launch_bounds__(kThreads) void w4a16_tile_kernel(W4Params p)
 {
     constexpr int kParamInstr = kHasOffset ? 2 : 1;
     constexpr int kInstr = 8 + kParamInstr + 1;   // 1 KiB DMA instructions per chunk
@@ -231,18 +282,11 @@ __global__ __launch_bounds__(kThreads) void w4a16_stream_kernel(W4Params p)
     };
 
     // ---- consumer side
-    f32x4 acc[MP][4];
+    f32x4 acc[8][4];  // accumulator e of w4_accumulate_tile is acc[e / 4][e % 4]
 #pragma unroll
-    for (int q = 0; q < MP; ++q) {
+    for (int q = 0; q < 8; ++q) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) acc[q][t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-    }
-    // A operand: lane (g, i) carries x[m][k_g] in half-slot (i & 7) for m = 2 * pair + (i >> 3)
-    const uint32_t slot = jj & 7u;
-    uint32_t amask[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        amask[r] = (static_cast<uint32_t>(r) == (slot >> 1)) ? ((slot & 1u) ? 0xFFFF0000u : 0x0000FFFFu) : 0u;
     }
     const f16x2 k1032 = {static_cast<half_t>(1032.0f), static_cast<half_t>(1032.0f)};
     const f16x2 k72 = {static_cast<half_t>(72.0f), static_cast<half_t>(72.0f)};
@@ -250,17 +294,18 @@ __global__ __launch_bounds__(kThreads) void w4a16_stream_kernel(W4Params p)
     uint32_t seg = 0, done_in_block = c_begin % cb_chunks;
     uint32_t checked_group = 0xFFFFFFFFu;
     bool int_offsets = false;  // every offset of the current group (all lanes) is an integer of magnitude <= 512
-    // the accumulators as they lie in registers: [16 registers][64 lanes] per pair
-    auto flush = [&]() {
+    // the accumulators as they lie in registers: [16 registers][64 lanes] per slice of four accumulators
+    auto flush = [&]() __attribute__((always_inline)) {
 #pragma unroll
-        for (int q = 0; q < MP; ++q) {
-            float* dst = p.partial + ((static_cast<size_t>(gw) * p.max_seg + seg) * MP + q) * 1024u + lane;
-            const bool row_valid = p.m0 + 2u * q + (g >> 1) < p.m;  // lanes of a missing second row hold zeros
+        for (int q = 0; q < 8; ++q) {
+            float* dst = p.partial + ((static_cast<size_t>(gw) * p.max_seg + seg) * 8u + q) * 1024u + lane;
+            // register r holds row 4 g + r; lanes of a missing row hold zeros: not stored
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
-                if (row_valid) {
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
+                for (int r = 0; r < 4; ++r) {
+                    const bool row_valid = p.m0 + 4u * g + r < p.m;
+                    if (row_valid) {
                         dst[(d * 4 + r) * 64] = acc[q][d][r];
                     }
                 }
@@ -278,12 +323,12 @@ __global__ __launch_bounds__(kThreads) void w4a16_stream_kernel(W4Params p)
     // direct-to-LDS loads in flight (which is conservative around the loop) stays out of the way.
 #define ASCQ_DS_READ128(dst, addr, off) \
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(off) : "memory")
-    auto compute = [&](const char* stage) {
+    auto compute = [&](const char* stage) __attribute__((always_inline)) {
         const uint32_t sa = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)stage));
         const uint32_t a_own = sa + lane * 16u;                      // what this lane fetched itself
         const uint32_t a_par = sa + jj * 16u;                        // parameter pieces of the lane's 32 columns
-        const uint32_t a_x = sa + (((jj >> 3) * 4u + g) * 16u);      // activations: row (jj >> 3) of a pair, piece g
-        u32x4 wd[8], sraw[4], oraw[4], xraw[MP];
+        const uint32_t a_x = sa + (jj * 4u + g) * 16u;               // activations: row jj of the tile, piece g
+        u32x4 wd[8], sraw[4], oraw[4], xraw;
         ASCQ_DS_READ128(wd[0], a_own, 0 * 1024);
         ASCQ_DS_READ128(wd[1], a_own, 1 * 1024);
         ASCQ_DS_READ128(wd[2], a_own, 2 * 1024);
@@ -302,17 +347,7 @@ __global__ __launch_bounds__(kThreads) void w4a16_stream_kernel(W4Params p)
             ASCQ_DS_READ128(oraw[2], a_par, 9 * 1024 + 2 * 256);
             ASCQ_DS_READ128(oraw[3], a_par, 9 * 1024 + 3 * 256);
         }
-        // pair q sits 128 bytes (two rows of four pieces) further on
-        ASCQ_DS_READ128(xraw[0], a_x, (8 + kParamInstr) * 1024);
-        if constexpr (MP > 1) ASCQ_DS_READ128(xraw[1], a_x, (8 + kParamInstr) * 1024 + 128);
-        if constexpr (MP > 2) ASCQ_DS_READ128(xraw[2], a_x, (8 + kParamInstr) * 1024 + 256);
-        if constexpr (MP > 3) ASCQ_DS_READ128(xraw[3], a_x, (8 + kParamInstr) * 1024 + 384);
-        if constexpr (MP > 4) {
-            ASCQ_DS_READ128(xraw[4], a_x, (8 + kParamInstr) * 1024 + 512);
-            ASCQ_DS_READ128(xraw[5], a_x, (8 + kParamInstr) * 1024 + 640);
-            ASCQ_DS_READ128(xraw[6], a_x, (8 + kParamInstr) * 1024 + 768);
-            ASCQ_DS_READ128(xraw[7], a_x, (8 + kParamInstr) * 1024 + 896);
-        }
+        ASCQ_DS_READ128(xraw, a_x, (8 + kParamInstr) * 1024);
         // every value read above is an in/out operand of the wait, so nothing uses one before it has arrived
         asm volatile("s_waitcnt lgkmcnt(0)"
                      : "+v"(wd[0]), "+v"(wd[1]), "+v"(wd[2]), "+v"(wd[3]), "+v"(wd[4]), "+v"(wd[5]), "+v"(wd[6]),
@@ -322,8 +357,7 @@ __global__ __launch_bounds__(kThreads) void w4a16_stream_kernel(W4Params p)
         if constexpr (kHasOffset) {
             asm volatile("" : "+v"(oraw[0]), "+v"(oraw[1]), "+v"(oraw[2]), "+v"(oraw[3]));
         }
-#pragma unroll
-        for (int q = 0; q < MP; ++q) asm volatile("" : "+v"(xraw[q]));
+        asm volatile("" : "+v"(xraw));
         f16x2 sc[4][4], of[4][4];
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
@@ -342,12 +376,8 @@ __global__ __launch_bounds__(kThreads) void w4a16_stream_kernel(W4Params p)
                 int_offsets = all_offsets_integral(of);
             }
         }
-        u32x4 xc[MP];
-#pragma unroll
-        for (int q = 0; q < MP; ++q) {
-            // lane (g, jj) carries x[m][krow + 8 g .. + 8) for m = m0 + 2 q + (jj >> 3)
-            xc[q] = (p.m0 + 2u * q + (jj >> 3) < p.m) ? xraw[q] : u32x4{0u, 0u, 0u, 0u};
-        }
+        // lane (g, jj) carries x[m0 + jj][krow + 8 g .. + 8): the A operand of the tile
+        const u32x4 xa = p.m0 + jj < p.m ? xraw : u32x4{0u, 0u, 0u, 0u};
         if (kHasOffset && int_offsets) {
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
@@ -356,9 +386,9 @@ __global__ __launch_bounds__(kThreads) void w4a16_stream_kernel(W4Params p)
                     of[d][c2] = (c2 & 1) ? of[d][c2] - k72 : of[d][c2] - k1032;  // exact
                 }
             }
-            w4_accumulate<MP, kHasOffset, true>(wd, xc, sc, of, amask, acc);
+            w4_accumulate_tile<kHasOffset, true>(wd, xa, sc, of, acc);
         } else {
-            w4_accumulate<MP, kHasOffset, false>(wd, xc, sc, of, amask, acc);
+            w4_accumulate_tile<kHasOffset, false>(wd, xa, sc, of, acc);
         }
         if (++done_in_block == cb_chunks) {  // the run leaves this column block
             done_in_block = 0;
@@ -480,7 +510,7 @@ __global__ __launch_bounds__(512) void w4a16_gemv_kernel(W4Params p)
     f16x2 sc[4][4], ofc[4][4];
     bool folded = false;
     uint32_t seg = 0, done_in_block = c_begin % cb_chunks;
-    auto flush = [&]() {
+    auto flush = [&]() __attribute__((always_inline)) {
 #pragma unroll
         for (int q = 0; q < MP; ++q) {
             float* dst = p.partial + ((static_cast<size_t>(gw) * p.max_seg + seg) * MP + q) * 1024u + lane;
@@ -522,7 +552,7 @@ __global__ __launch_bounds__(512) void w4a16_gemv_kernel(W4Params p)
         }
         params_pending = false;
     };
-    auto compute = [&](const char* stage) {
+    auto compute = [&](const char* stage) __attribute__((always_inline)) {
         const uint32_t sa = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)stage));
         const uint32_t a_own = sa + lane * 16u;                           // what this lane fetched itself
         const uint32_t a_x = sa + 8u * 1024u + (jj >> 3) * 64u + g * 16u;  // row (jj >> 3) of a pair, k 8 g .. 8 g + 7
@@ -585,7 +615,7 @@ __global__ __launch_bounds__(512) void w4a16_gemv_kernel(W4Params p)
 // added element by element in that layout with fully coalesced 16-byte loads, and only the final store is scattered.
 // One workgroup per (column block, row pair): 4 sub-groups of 256 lanes take the pieces i = sub, sub + 4, ... in
 // ascending k order, the four sums are combined as (s0 + s1) + (s2 + s3): deterministic.
-template <int MP>
+template <int MP, bool kTile = false>
 __global__ __launch_bounds__(1024) void w4a16_sum_kernel(W4Params p)
 {
     __shared__ f32x4 part[4][256];
@@ -601,8 +631,10 @@ __global__ __launch_bounds__(1024) void w4a16_sum_kernel(W4Params p)
     // the first stream may have begun in an earlier block; all later ones begin inside this block (piece 0)
     const size_t first_extra = static_cast<size_t>(blk - stream_begin(p, w0) / p.chunks_per_block) * MP * 1024u;
     const float* base = p.partial + (static_cast<size_t>(w0) * p.max_seg * MP + q) * 1024u + 4u * t;
-    // the four elements of a lane share their row (g >> 1 of the pair); a row past m was never written
-    const bool row_valid = p.m0 + 2u * q + ((t >> 2) & 3u) / 2u < p.m;
+    // the four elements of a lane share their register (t >> 4) and quarter g = (t >> 2) & 3, hence their row (g / 2 of
+    // the pair, or 4 g + r of a tile); a row past m was never written
+    const uint32_t my_row = kTile ? 4u * ((t >> 2) & 3u) + ((t >> 4) & 3u) : 2u * q + ((t >> 2) & 3u) / 2u;
+    const bool row_valid = p.m0 + my_row < p.m;
     f32x4 s = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     for (uint32_t w = w0 + sub; row_valid && w < w1; w += 32u) {
         f32x4 v[8];
@@ -627,9 +659,17 @@ __global__ __launch_bounds__(1024) void w4a16_sum_kernel(W4Params p)
     for (uint32_t i = 0; i < 4u; ++i) {
         const uint32_t e = 4u * t + i;
         const uint32_t jj = e & 15u, g = (e >> 4) & 3u, r = (e >> 6) & 3u, d = e >> 8;
-        const uint32_t b8 = 4u * (g & 1u) + r;
-        const uint32_t col = blk * kColsPerBlock + jj * 32u + d * 8u + (b8 >> 1) + 4u * (b8 & 1u);
-        const uint32_t m = p.m0 + 2u * q + (g >> 1);
+        uint32_t col, m;
+        if constexpr (kTile) {
+            // slice q holds accumulators 4 q + d of w4_accumulate_tile
+            const uint32_t acc_e = 4u * q + d;
+            col = blk * kColsPerBlock + jj * 32u + (acc_e >> 3) * 8u + ((acc_e >> 1) & 3u) + 4u * (acc_e & 1u);
+            m = p.m0 + 4u * g + r;
+        } else {
+            const uint32_t b8 = 4u * (g & 1u) + r;
+            col = blk * kColsPerBlock + jj * 32u + d * 8u + (b8 >> 1) + 4u * (b8 & 1u);
+            m = p.m0 + 2u * q + (g >> 1);
+        }
         if (col < p.n && m < p.m) {
             p.y[static_cast<size_t>(m) * p.n + col] = static_cast<uint16_t>(f32_to_half_bits(tot[i]));
         }
@@ -681,7 +721,7 @@ W4Plan make_plan(uint32_t n, uint32_t k, uint32_t max_waves)
 size_t workspace_need(uint32_t n, uint32_t k)
 {
     const W4Plan a = make_plan(n, k, kMaxWaves), b = make_plan(n, k, 2u * kMaxWaves);
-    const size_t na = static_cast<size_t>(a.waves) * a.max_seg * kMaxPairs, nb = static_cast<size_t>(b.waves) * b.max_seg * 2u;
+    const size_t na = static_cast<size_t>(a.waves) * a.max_seg * (kTileRows / 2u), nb = static_cast<size_t>(b.waves) * b.max_seg * 2u;
     return (na > nb ? na : nb) * 1024u * sizeof(float);
 }
 
@@ -767,7 +807,7 @@ extern "C" int ascq_matmul_w4a16(const ascq_w4a16_desc* d, void* y, const void* 
         p.rem = pl.total_chunks % pl.waves;
     };
     // at most 16 activation rows per pass over the weights
-    for (uint32_t m0 = 0; m0 < d->m; m0 += 2 * kMaxPairs) {
+    for (uint32_t m0 = 0; m0 < d->m; m0 += kTileRows) {
         const uint32_t left = d->m - m0;
         p.m0 = m0;
         if (left <= 4) {
@@ -790,23 +830,14 @@ extern "C" int ascq_matmul_w4a16(const ascq_w4a16_desc* d, void* y, const void* 
 #undef ASCQ_W4_GEMV
             continue;
         }
-        set_plan(kMaxWaves);
+        set_plan(kMaxWaves);  // one stream per SIMD, 16 rows
         const uint32_t grid = (p.waves + 3u) / 4u;
-#define ASCQ_W4_LAUNCH(MPV)                                                              \
-    do {                                                                                 \
-        if (d->has_offset) {                                                             \
-            w4a16_stream_kernel<MPV, true><<<grid, kThreads, 0, st>>>(p);                \
-        } else {                                                                         \
-            w4a16_stream_kernel<MPV, false><<<grid, kThreads, 0, st>>>(p);               \
-        }                                                                                \
-        w4a16_sum_kernel<MPV><<<dim3(col_blocks, MPV), 1024, 0, st>>>(p);           \
-    } while (0)
-        if (left <= 8) {
-            ASCQ_W4_LAUNCH(4);
+        if (d->has_offset) {
+            w4a16_tile_kernel<true><<<grid, kThreads, 0, st>>>(p);
         } else {
-            ASCQ_W4_LAUNCH(8);
+            w4a16_tile_kernel<false><<<grid, kThreads, 0, st>>>(p);
         }
-#undef ASCQ_W4_LAUNCH
+        w4a16_sum_kernel<8, true><<<dim3(col_blocks, 8), 1024, 0, st>>>(p);
     }
     return launch_status("ascq_matmul_w4a16");
 }
