@@ -67,6 +67,11 @@ class W4A16Desc(C.Structure):
                 ("has_offset", C.c_int32)]
 
 
+class W8A16Desc(C.Structure):
+    _fields_ = [("m", C.c_uint32), ("n", C.c_uint32), ("k", C.c_uint32), ("per_tensor", C.c_int32),
+                ("has_offset", C.c_int32), ("scale", C.c_float), ("offset", C.c_float), ("out_dtype", C.c_int32)]
+
+
 _P = C.c_void_p
 # name -> (restype, argtypes): every symbol include/ascq.h declares
 SIGNATURES = {
@@ -80,6 +85,8 @@ SIGNATURES = {
     "ascq_group_matmul_w8a8": (C.c_int, [C.POINTER(GroupMatmulDesc), _P, _P, _P, _P, _P, _P, _P, _P]),
     "ascq_matmul_w4a16": (C.c_int, [C.POINTER(W4A16Desc), _P, _P, _P, _P, _P, _P, C.c_size_t, _P]),
     "ascq_matmul_w4a16_workspace_size": (C.c_int, [C.POINTER(W4A16Desc), C.POINTER(C.c_size_t)]),
+    "ascq_matmul_w8a16": (C.c_int, [C.POINTER(W8A16Desc), _P, _P, _P, _P, _P, _P, C.c_size_t, _P]),
+    "ascq_matmul_w8a16_workspace_size": (C.c_int, [C.POINTER(W8A16Desc), C.POINTER(C.c_size_t)]),
     "ascq_get_ascend_quant_max_min_tmp_size": (C.c_int, [C.POINTER(C.c_uint32), C.c_uint32, C.c_uint32,
                                                          C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
     "ascq_get_ascend_dequant_max_min_tmp_size": (C.c_int, [C.POINTER(C.c_uint32), C.c_uint32, C.c_uint32,

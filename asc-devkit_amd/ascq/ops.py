@@ -285,6 +285,33 @@ def matmul_w4a16(y, x, w_packed, scale, offset=None, group_size=128, workspace=N
     return y
 
 
+# ------------------------------------------------------------------------------------------------------ W8A16
+def matmul_w8a16(y, x, w, offset=None, scale=None, workspace=None):
+    """y f16 / f32 [m, n] = x f16 [m, k] @ AscendAntiQuant<int8_t, half>(w int8 [k, n]).
+
+    scale / offset: f16 tensors of n elements (SetAntiQuantVector) or Python floats (SetAntiQuantScalar); offset None =
+    MatmulConfig::hasAntiQuantOffset false.
+    """
+    m, k = x.shape
+    n = y.shape[1]
+    per_tensor = not torch.is_tensor(scale)
+    d = abi.W8A16Desc(m=m, n=n, k=k, per_tensor=int(per_tensor), has_offset=int(offset is not None),
+                      scale=float(scale) if per_tensor else 0.0,
+                      offset=float(offset) if per_tensor and offset is not None else 0.0, out_dtype=_DT[y.dtype])
+    lib = load_library()
+    need = C.c_size_t(0)
+    check(lib.ascq_matmul_w8a16_workspace_size(C.byref(d), C.byref(need)))
+    if workspace is None:
+        key = (x.device, need.value)
+        if key not in _w4_ws:
+            _w4_ws[key] = torch.zeros(max(need.value // 4, 4), dtype=torch.float32, device=x.device)
+        workspace = _w4_ws[key]
+    check(lib.ascq_matmul_w8a16(C.byref(d), _ptr(y), _ptr(x), _ptr(w), None if per_tensor else _ptr(offset),
+                                None if per_tensor else _ptr(scale), _ptr(workspace),
+                                workspace.numel() * workspace.element_size(), _stream()))
+    return y
+
+
 # ------------------------------------------------------------------------------------------- host size queries
 def _shape(shape):
     return (C.c_uint32 * len(shape))(*shape), len(shape)

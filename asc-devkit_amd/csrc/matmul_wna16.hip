@@ -33,7 +33,8 @@ namespace ascq {
 namespace {
 
 constexpr int kThreads = 256;          // four independent wavefronts per workgroup
-constexpr uint32_t kColsPerBlock = 512;
+constexpr uint32_t kColsPerBlock = 512;    // int4: 16 lanes x 32 columns
+constexpr uint32_t kW8ColsPerBlock = 256;  // int8: 16 lanes x 16 columns
 constexpr uint32_t kChunkRows = 32;
 constexpr uint32_t kMaxWaves = 1024;   // 256 compute units x 4 SIMDs
 constexpr uint32_t kTileRows = 16;     // activation rows per pass over the weights
@@ -41,7 +42,7 @@ constexpr uint32_t kTileRows = 16;     // activation rows per pass over the weig
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef __attribute__((address_space(1))) const void* gptr_t;
 
-struct W4Params {
+struct WnParams {
     const uint16_t* x;
     const uint8_t* w;
     const uint16_t* scale;
@@ -55,6 +56,9 @@ struct W4Params {
     uint32_t total_chunks;      // column blocks * chunks_per_block
     uint32_t max_seg;           // column blocks one stream can touch
     uint32_t per, rem;          // total_chunks = waves * per + rem
+    // W8A16 only
+    uint32_t out_f32;                  // y is float instead of half
+    uint32_t scale_bits, offset_bits;  // per-tensor parameters as half bits, used when scale == nullptr
 };
 
 __device__ __forceinline__ f16x2 bits_to_h2(uint32_t b)
@@ -74,7 +78,7 @@ __device__ __forceinline__ void pair_up(u32x4 v, f16x2 (&out)[4])
 }
 
 // Stream `wave` owns chunks [stream_begin(wave), stream_begin(wave + 1)): the first `rem` streams take per + 1 chunks.
-__device__ __forceinline__ uint32_t stream_begin(const W4Params& p, uint32_t wave)
+__device__ __forceinline__ uint32_t stream_begin(const WnParams& p, uint32_t wave)
 {
     return wave * p.per + (wave < p.rem ? wave : p.rem);
 }
@@ -195,14 +199,15 @@ __device__ __forceinline__ void w4_accumulate_tile(const u32x4 (&wd)[8], const u
 // True on every lane iff every offset held by any lane of the wavefront is an integer of magnitude <= 512 (then
 // (o + 1536) - 1536 == o exactly).  Uniform over the wavefront on purpose: the matrix instruction ignores the execution
 // mask, so the two arithmetic paths must never run in one wavefront.
-__device__ __forceinline__ bool all_offsets_integral(const f16x2 (&of)[4][4])
+template <int A, int B>
+__device__ __forceinline__ bool all_offsets_integral(const f16x2 (&of)[A][B])
 {
     const f16x2 k1536 = {static_cast<half_t>(1536.0f), static_cast<half_t>(1536.0f)};
     uint32_t differ = 0;
 #pragma unroll
-    for (int d = 0; d < 4; ++d) {
+    for (int d = 0; d < A; ++d) {
 #pragma unroll
-        for (int c2 = 0; c2 < 4; ++c2) {
+        for (int c2 = 0; c2 < B; ++c2) {
             const f16x2 t = (of[d][c2] + k1536) - k1536;
             uint32_t tb, ob;
             __builtin_memcpy(&tb, &t, 4);
@@ -220,7 +225,7 @@ __device__ __forceinline__ bool all_offsets_integral(const f16x2 (&of)[4][4])
 // the rows of one MFMA tile (w4_accumulate_tile).  A piece of the workspace is [8 slices][16 registers][64 lanes].
 // Requires n % 32 == 0, k % 32 == 0, group_size % 32 == 0.
 template <bool kHasOffset>
-__global__ __launch_bounds__(kThreads) void w4a16_tile_kernel(W4Params p)
+__global__ __launch_bounds__(kThreads) void w4a16_tile_kernel(WnParams p)
 {
     constexpr int kParamInstr = kHasOffset ? 2 : 1;
     constexpr int kInstr = 8 + kParamInstr + 1;   // 1 KiB DMA instructions per chunk
@@ -430,7 +435,7 @@ __global__ __launch_bounds__(kThreads) void w4a16_tile_kernel(W4Params p)
 // and the wait before a chunk is simply for everything outstanding; the second wavefront of the SIMD fills the time
 // a wavefront spends waiting or stalled on its own dependent instructions.
 template <int MP, bool kHasOffset>
-__global__ __launch_bounds__(512) void w4a16_gemv_kernel(W4Params p)
+__global__ __launch_bounds__(512) void w4a16_gemv_kernel(WnParams p)
 {
     constexpr int kStage = 8 * 1024 + 256;  // bytes per wavefront and stage
     __shared__ __attribute__((aligned(1024))) char S0[8 * kStage];
@@ -610,14 +615,236 @@ __global__ __launch_bounds__(512) void w4a16_gemv_kernel(W4Params p)
     }
 }
 
+// W8A16 (A half, B int8 de-quantised per channel or per tensor while it is read): the same streams, two per SIMD, on
+// chunks of 32 rows x 256 columns of int8 (8 KiB).  A lane owns 16 adjacent columns of a weight row; over the 8 rows
+// it holds, one column is the 8 consecutive k of a B operand, so up to 16 activation rows fill one MFMA tile per
+// column.  A byte becomes an exact half by a byte permute into 0x6400 | (w + 128) = 1152 + w; one exact subtraction
+// gives w, then one rounded half add of the offset and one rounded half multiply by the scale, as
+// AscendAntiQuant<int8_t, half>.  The scale / offset of a column do not depend on k: they are fetched into registers
+// when the stream enters a column block.  Accumulator c (kept as acc[c / 4][c % 4]) holds rows 4 g .. 4 g + 3 of
+// column 16 jj + c; a piece of the workspace is [4 slices][16 registers][64 lanes].
+// Requires n % 16 == 0, k % 32 == 0.
+template <bool kHasOffset>
+__global__ __launch_bounds__(512) void w8a16_tile_kernel(WnParams p)
+{
+    constexpr int kStage = 8 * 1024 + 1024;  // bytes per wavefront and stage: weights, activations
+    __shared__ __attribute__((aligned(1024))) char S0[8 * kStage];
+    __shared__ __attribute__((aligned(1024))) char S1[8 * kStage];
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t gw = blockIdx.x * 8u + wave;
+    if (gw >= p.waves) {
+        return;  // whole wavefront; the kernel has no barriers
+    }
+    const uint32_t g = lane >> 4, jj = lane & 15u;
+    const uint32_t c_begin = stream_begin(p, gw), c_end = stream_begin(p, gw + 1u);
+    if (c_begin == c_end) {
+        return;
+    }
+    const size_t row_bytes = p.n;
+    const uint32_t cb_chunks = p.chunks_per_block;
+    const bool per_tensor = p.scale == nullptr;
+
+    // ---- producer side: chunk (block ib, k-chunk ik) -> stage; parameters of a new column block -> registers
+    uint32_t ib = c_begin / cb_chunks, ik = c_begin % cb_chunks;
+    u32x4 sraw[2], oraw[2];
+    bool params_pending = false;
+    auto issue = [&](char* stage, bool first) {
+        // Lanes past the last column work on a duplicate of the last 16 columns (never stored): the MFMA ignores the
+        // execution mask, so every lane must hold valid operands.
+        uint32_t col0 = ib * kW8ColsPerBlock + jj * 16u;
+        col0 = col0 < p.n ? col0 : p.n - 16u;
+        const uint32_t krow = ik * kChunkRows;
+        if (first || ik == 0u) {  // the chunk opens the run or a column block
+            if (!per_tensor) {
+#pragma unroll
+                for (int d = 0; d < 2; ++d) {
+                    sraw[d] = *reinterpret_cast<const u32x4*>(p.scale + col0 + 8 * d);
+                    if constexpr (kHasOffset) {
+                        oraw[d] = *reinterpret_cast<const u32x4*>(p.offset + col0 + 8 * d);
+                    }
+                }
+            }
+            params_pending = true;
+        }
+        const uint8_t* wsrc = p.w + static_cast<size_t>(krow + 8u * g) * row_bytes + col0;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            __builtin_amdgcn_global_load_lds((gptr_t)(wsrc + static_cast<size_t>(u) * row_bytes),
+                                             (lds_ptr_t)(stage + u * 1024), 16, 0, 0);
+        }
+        // activations of the chunk's 32 k for up to 16 rows in one instruction: lane l fetches piece (l & 3) of row
+        // m0 + (l >> 2); rows past m fetch row m - 1 and are zeroed when used
+        {
+            const uint32_t m = p.m0 + (lane >> 2);
+            const uint32_t mc = m < p.m ? m : p.m - 1u;
+            __builtin_amdgcn_global_load_lds((gptr_t)(p.x + static_cast<size_t>(mc) * p.k + krow + 8u * (lane & 3u)),
+                                             (lds_ptr_t)(stage + 8 * 1024), 16, 0, 0);
+        }
+        if (++ik == cb_chunks) {
+            ik = 0;
+            ++ib;
+        }
+    };
+
+    // ---- consumer side
+    f32x4 acc[4][4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) acc[q][t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    const f16x2 k1152 = {static_cast<half_t>(1152.0f), static_cast<half_t>(1152.0f)};
+    f16x2 sc[2][4], ofc[2][4];  // pair i of dword-half d: columns 8 d + 2 i, 8 d + 2 i + 1
+    bool folded = false;
+    uint32_t seg = 0, done_in_block = c_begin % cb_chunks;
+    auto flush = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            float* dst = p.partial + ((static_cast<size_t>(gw) * p.max_seg + seg) * 4u + q) * 1024u + lane;
+            // register r holds row 4 g + r; lanes of a missing row hold zeros: not stored
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if (p.m0 + 4u * g + r < p.m) {
+                        dst[(d * 4 + r) * 64] = acc[q][d][r];
+                    }
+                }
+                acc[q][d] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            }
+        }
+        ++seg;
+    };
+    // called after the wait: turns freshly landed parameters into the packed constants of the column block
+    auto adopt_params = [&]() {
+#pragma unroll
+        for (int d = 0; d < 2; ++d) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                sc[d][i] = bits_to_h2(per_tensor ? p.scale_bits * 0x00010001u : sraw[d][i]);
+                if constexpr (kHasOffset) {
+                    ofc[d][i] = bits_to_h2(per_tensor ? p.offset_bits * 0x00010001u : oraw[d][i]);
+                }
+            }
+        }
+        folded = false;
+        if constexpr (kHasOffset) {
+            // with integer offsets w + offset is exact, and so is (1152 + w) + (offset - 1152)
+            folded = all_offsets_integral(ofc);
+            if (folded) {
+#pragma unroll
+                for (int d = 0; d < 2; ++d) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) ofc[d][i] = ofc[d][i] - k1152;  // exact
+                }
+            }
+        }
+        params_pending = false;
+    };
+    auto compute = [&](const char* stage) __attribute__((always_inline)) {
+        const uint32_t sa = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)stage));
+        const uint32_t a_own = sa + lane * 16u;                       // what this lane fetched itself
+        const uint32_t a_x = sa + 8u * 1024u + (jj * 4u + g) * 16u;   // activations: row jj of the tile, piece g
+        u32x4 wd[8], xraw;
+        ASCQ_DS_READ128(wd[0], a_own, 0 * 1024);
+        ASCQ_DS_READ128(wd[1], a_own, 1 * 1024);
+        ASCQ_DS_READ128(wd[2], a_own, 2 * 1024);
+        ASCQ_DS_READ128(wd[3], a_own, 3 * 1024);
+        ASCQ_DS_READ128(wd[4], a_own, 4 * 1024);
+        ASCQ_DS_READ128(wd[5], a_own, 5 * 1024);
+        ASCQ_DS_READ128(wd[6], a_own, 6 * 1024);
+        ASCQ_DS_READ128(wd[7], a_own, 7 * 1024);
+        ASCQ_DS_READ128(xraw, a_x, 0);
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(wd[0]), "+v"(wd[1]), "+v"(wd[2]), "+v"(wd[3]), "+v"(wd[4]), "+v"(wd[5]), "+v"(wd[6]),
+                       "+v"(wd[7]), "+v"(xraw)
+                     :
+                     : "memory");
+        // lane (g, jj) carries x[m0 + jj][krow + 8 g .. + 8): the A operand of the tile
+        const u32x4 xa = p.m0 + jj < p.m ? xraw : u32x4{0u, 0u, 0u, 0u};
+        f16x8 a;
+        __builtin_memcpy(&a, &xa, 16);
+#pragma unroll
+        for (int d = 0; d < 2; ++d) {  // columns 8 d .. 8 d + 7 of the lane's 16
+            f16x2 h[8][4];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t word = wd[u][2 * d + (i >> 1)] ^ 0x80808080u;  // two's complement -> w + 128
+                    // bytes (2 (i & 1), 2 (i & 1) + 1) of the word -> two exact halves 1024 + (w + 128)
+                    const uint32_t bits = __builtin_amdgcn_perm(0x64646464u, word, (i & 1) ? 0x04030402u : 0x04010400u);
+                    f16x2 v;
+                    if (kHasOffset && folded) {
+                        v = bits_to_h2(bits) + ofc[d][i];  // w + offset, exact
+                    } else {
+                        v = bits_to_h2(bits) - k1152;  // w, exact
+                        if constexpr (kHasOffset) {
+                            v = v + ofc[d][i];  // one rounding
+                        }
+                    }
+                    h[u][i] = sc[d][i] * v;  // one rounding
+                }
+            }
+#pragma unroll
+            for (int qh = 0; qh < 2; ++qh) {
+#pragma unroll
+                for (int dd = 0; dd < 4; ++dd) {
+                    const int i = 2 * qh + (dd >> 1), hi = dd & 1;  // column 8 d + 4 qh + dd
+                    u32x4 bv;
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        uint32_t even, odd;
+                        __builtin_memcpy(&even, &h[2 * t][i], 4);
+                        __builtin_memcpy(&odd, &h[2 * t + 1][i], 4);
+                        bv[t] = __builtin_amdgcn_perm(odd, even, hi ? 0x07060302u : 0x05040100u);
+                    }
+                    f16x8 b;
+                    __builtin_memcpy(&b, &bv, 16);
+                    acc[2 * d + qh][dd] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[2 * d + qh][dd], 0, 0, 0);
+                }
+            }
+        }
+        if (++done_in_block == cb_chunks) {  // the run leaves this column block
+            done_in_block = 0;
+            flush();
+        }
+    };
+
+    char* s0 = S0 + wave * kStage;
+    char* s1 = S1 + wave * kStage;
+    issue(s0, true);
+    uint32_t c = c_begin;
+    while (true) {
+        ASCQ_WAIT_VMCNT(0);  // chunk c (and parameters fetched ahead of it) has landed
+        if (params_pending) adopt_params();
+        if (c + 1u < c_end) issue(s1, false);
+        compute(s0);
+        if (++c == c_end) break;
+        ASCQ_WAIT_VMCNT(0);
+        if (params_pending) adopt_params();
+        if (c + 1u < c_end) issue(s0, false);
+        compute(s1);
+        if (++c == c_end) break;
+    }
+    if (done_in_block != 0) {
+        flush();
+    }
+}
+
 // Adds the pieces of all streams that worked on a column block and rounds once to half.  A piece is the image of
 // the accumulators of a wavefront, [16 registers][64 lanes] = the 2 rows x 512 columns of the block, so the pieces are
 // added element by element in that layout with fully coalesced 16-byte loads, and only the final store is scattered.
 // One workgroup per (column block, row pair): 4 sub-groups of 256 lanes take the pieces i = sub, sub + 4, ... in
 // ascending k order, the four sums are combined as (s0 + s1) + (s2 + s3): deterministic.
-template <int MP, bool kTile = false>
-__global__ __launch_bounds__(1024) void w4a16_sum_kernel(W4Params p)
+enum PieceLayout { kPiecePairs = 0, kPieceTileW4 = 1, kPieceTileW8 = 2 };
+
+template <int MP, int kLayout = kPiecePairs>
+__global__ __launch_bounds__(1024) void stream_sum_kernel(WnParams p)
 {
+    constexpr bool kTile = kLayout != kPiecePairs;
     __shared__ f32x4 part[4][256];
     const uint32_t sub = threadIdx.x >> 8, t = threadIdx.x & 255u;
     const uint32_t blk = blockIdx.x, q = blockIdx.y;
@@ -660,10 +887,14 @@ __global__ __launch_bounds__(1024) void w4a16_sum_kernel(W4Params p)
         const uint32_t e = 4u * t + i;
         const uint32_t jj = e & 15u, g = (e >> 4) & 3u, r = (e >> 6) & 3u, d = e >> 8;
         uint32_t col, m;
-        if constexpr (kTile) {
+        if constexpr (kLayout == kPieceTileW4) {
             // slice q holds accumulators 4 q + d of w4_accumulate_tile
             const uint32_t acc_e = 4u * q + d;
             col = blk * kColsPerBlock + jj * 32u + (acc_e >> 3) * 8u + ((acc_e >> 1) & 3u) + 4u * (acc_e & 1u);
+            m = p.m0 + 4u * g + r;
+        } else if constexpr (kLayout == kPieceTileW8) {
+            // slice q holds accumulators 4 q + d of the int8 tile kernel = columns 4 q + d of the lane's 16
+            col = blk * kW8ColsPerBlock + jj * 16u + 4u * q + d;
             m = p.m0 + 4u * g + r;
         } else {
             const uint32_t b8 = 4u * (g & 1u) + r;
@@ -671,13 +902,17 @@ __global__ __launch_bounds__(1024) void w4a16_sum_kernel(W4Params p)
             m = p.m0 + 2u * q + (g >> 1);
         }
         if (col < p.n && m < p.m) {
-            p.y[static_cast<size_t>(m) * p.n + col] = static_cast<uint16_t>(f32_to_half_bits(tot[i]));
+            if (kLayout == kPieceTileW8 && p.out_f32) {
+                reinterpret_cast<float*>(p.y)[static_cast<size_t>(m) * p.n + col] = tot[i];
+            } else {
+                p.y[static_cast<size_t>(m) * p.n + col] = static_cast<uint16_t>(f32_to_half_bits(tot[i]));
+            }
         }
     }
 }
 
 // Any shape: one lane per output element.
-__global__ __launch_bounds__(kThreads) void w4a16_generic_kernel(W4Params p)
+__global__ __launch_bounds__(kThreads) void w4a16_generic_kernel(WnParams p)
 {
     const size_t total = static_cast<size_t>(p.m) * p.n;
     for (size_t idx = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x; idx < total;
@@ -700,14 +935,41 @@ __global__ __launch_bounds__(kThreads) void w4a16_generic_kernel(W4Params p)
     }
 }
 
+// W8A16, any shape: one lane per output element.
+__global__ __launch_bounds__(kThreads) void w8a16_generic_kernel(WnParams p)
+{
+    const size_t total = static_cast<size_t>(p.m) * p.n;
+    for (size_t idx = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x; idx < total;
+         idx += static_cast<size_t>(gridDim.x) * kThreads) {
+        const size_t row = idx / p.n, col = idx % p.n;
+        const half_t scale = static_cast<half_t>(half_bits_to_f32(p.scale ? p.scale[col] : p.scale_bits));
+        const half_t offset =
+            p.has_offset ? static_cast<half_t>(half_bits_to_f32(p.scale ? p.offset[col] : p.offset_bits)) : half_t(0);
+        float s = 0.0f;
+        for (uint32_t kk = 0; kk < p.k; ++kk) {
+            half_t h = static_cast<half_t>(static_cast<float>(static_cast<int8_t>(p.w[static_cast<size_t>(kk) * p.n + col])));
+            if (p.has_offset) {
+                h = h + offset;
+            }
+            h = scale * h;
+            s += half_bits_to_f32(p.x[row * p.k + kk]) * static_cast<float>(h);
+        }
+        if (p.out_f32) {
+            reinterpret_cast<float*>(p.y)[idx] = s;
+        } else {
+            p.y[idx] = static_cast<uint16_t>(f32_to_half_bits(s));
+        }
+    }
+}
+
 struct W4Plan {
     uint32_t waves, chunks_per_block, total_chunks, max_seg;
 };
 
-W4Plan make_plan(uint32_t n, uint32_t k, uint32_t max_waves)
+W4Plan make_plan(uint32_t n, uint32_t k, uint32_t max_waves, uint32_t cols_per_block = kColsPerBlock)
 {
     W4Plan pl;
-    const uint32_t blocks_n = (n + kColsPerBlock - 1u) / kColsPerBlock;
+    const uint32_t blocks_n = (n + cols_per_block - 1u) / cols_per_block;
     pl.chunks_per_block = k / kChunkRows;
     pl.total_chunks = blocks_n * pl.chunks_per_block;
     pl.waves = pl.total_chunks < max_waves ? pl.total_chunks : max_waves;
@@ -773,7 +1035,7 @@ extern "C" int ascq_matmul_w4a16(const ascq_w4a16_desc* d, void* y, const void* 
     ASCQ_REQUIRE(y && x && w && scale, ASCQ_ENULL, "ascq_matmul_w4a16: y / x / w / scale is NULL");
     ASCQ_REQUIRE(!d->has_offset || offset, ASCQ_ENULL, "ascq_matmul_w4a16: offset is NULL");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    W4Params p{};
+    WnParams p{};
     p.x = static_cast<const uint16_t*>(x);
     p.w = static_cast<const uint8_t*>(w);
     p.scale = static_cast<const uint16_t*>(scale);
@@ -820,7 +1082,7 @@ extern "C" int ascq_matmul_w4a16(const ascq_w4a16_desc* d, void* y, const void* 
         } else {                                                                    \
             w4a16_gemv_kernel<MPV, false><<<grid, 512, 0, st>>>(p);                 \
         }                                                                           \
-        w4a16_sum_kernel<MPV><<<dim3(col_blocks, MPV), 1024, 0, st>>>(p);           \
+        stream_sum_kernel<MPV><<<dim3(col_blocks, MPV), 1024, 0, st>>>(p);           \
     } while (0)
             if (left <= 2) {
                 ASCQ_W4_GEMV(1);
@@ -837,7 +1099,106 @@ extern "C" int ascq_matmul_w4a16(const ascq_w4a16_desc* d, void* y, const void* 
         } else {
             w4a16_tile_kernel<false><<<grid, kThreads, 0, st>>>(p);
         }
-        w4a16_sum_kernel<8, true><<<dim3(col_blocks, 8), 1024, 0, st>>>(p);
+        stream_sum_kernel<8, kPieceTileW4><<<dim3(col_blocks, 8), 1024, 0, st>>>(p);
     }
     return launch_status("ascq_matmul_w4a16");
+}
+
+// ------------------------------------------------------------------------------------------------------------ W8A16
+static int validate_w8a16(const ascq_w8a16_desc* d)
+{
+    ASCQ_REQUIRE(d != nullptr, ASCQ_ENULL, "ascq_matmul_w8a16: desc is NULL");
+    ASCQ_REQUIRE(d->m > 0 && d->n > 0 && d->k > 0, ASCQ_EINVAL, "ascq_matmul_w8a16: m, n, k must be greater than 0");
+    ASCQ_REQUIRE(d->out_dtype == ASCQ_F16 || d->out_dtype == ASCQ_F32, ASCQ_EUNSUPPORTED,
+                 "ascq_matmul_w8a16: out_dtype must be ASCQ_F16 or ASCQ_F32");
+    return ASCQ_OK;
+}
+
+static bool w8a16_fast_ok(const ascq_w8a16_desc* d, const void* x, const void* w, const void* scale, const void* offset)
+{
+    return d->n % 16 == 0 && d->k % kChunkRows == 0 && aligned16(x) && aligned16(w) &&
+           (d->per_tensor || (aligned16(scale) && (!d->has_offset || aligned16(offset)))) &&
+           static_cast<uint64_t>((d->n + kW8ColsPerBlock - 1u) / kW8ColsPerBlock) * (d->k / kChunkRows) < (1ull << 31);
+}
+
+static size_t w8a16_workspace_need(uint32_t n, uint32_t k)
+{
+    const W4Plan pl = make_plan(n, k, 2u * kMaxWaves, kW8ColsPerBlock);
+    return static_cast<size_t>(pl.waves) * pl.max_seg * 4u * 1024u * sizeof(float);
+}
+
+extern "C" int ascq_matmul_w8a16_workspace_size(const ascq_w8a16_desc* d, size_t* bytes)
+{
+    int rc = validate_w8a16(d);
+    if (rc != ASCQ_OK) {
+        return rc;
+    }
+    ASCQ_REQUIRE(bytes != nullptr, ASCQ_ENULL, "ascq_matmul_w8a16_workspace_size: bytes is NULL");
+    *bytes = (d->n % 16 == 0 && d->k % kChunkRows == 0) ? w8a16_workspace_need(d->n, d->k) : 0;
+    return ASCQ_OK;
+}
+
+// ref: include/adv_api/matmul/matmul.h:161-168 (SetAntiQuantScalar / SetAntiQuantVector);
+// impl/adv_api/detail/matmul/stage/copy_cube_in/antiquant/antiquant_processor_using_ub.h:53-130 (AscendAntiQuant of B)
+extern "C" int ascq_matmul_w8a16(const ascq_w8a16_desc* d, void* y, const void* x, const void* w, const void* offset,
+                                 const void* scale, void* workspace, size_t workspace_bytes, void* stream)
+{
+    int rc = validate_w8a16(d);
+    if (rc != ASCQ_OK) {
+        return rc;
+    }
+    ASCQ_REQUIRE(y && x && w, ASCQ_ENULL, "ascq_matmul_w8a16: y / x / w is NULL");
+    ASCQ_REQUIRE(d->per_tensor || scale, ASCQ_ENULL, "ascq_matmul_w8a16: scale vector is NULL");
+    ASCQ_REQUIRE(d->per_tensor || !d->has_offset || offset, ASCQ_ENULL, "ascq_matmul_w8a16: offset vector is NULL");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    WnParams p{};
+    p.x = static_cast<const uint16_t*>(x);
+    p.w = static_cast<const uint8_t*>(w);
+    p.scale = d->per_tensor ? nullptr : static_cast<const uint16_t*>(scale);
+    p.offset = d->per_tensor ? nullptr : static_cast<const uint16_t*>(offset);
+    // the per-tensor scalars are halves in the reference (SrcT of SetAntiQuantScalar): one rounding here
+    const _Float16 scale_h = static_cast<_Float16>(d->scale), offset_h = static_cast<_Float16>(d->offset);
+    uint16_t scale_b, offset_b;
+    __builtin_memcpy(&scale_b, &scale_h, 2);
+    __builtin_memcpy(&offset_b, &offset_h, 2);
+    p.scale_bits = scale_b;
+    p.offset_bits = offset_b;
+    p.partial = static_cast<float*>(workspace);
+    p.y = static_cast<uint16_t*>(y);
+    p.m = d->m;
+    p.n = d->n;
+    p.k = d->k;
+    p.has_offset = d->has_offset ? 1u : 0u;
+    p.out_f32 = d->out_dtype == ASCQ_F32 ? 1u : 0u;
+    if (!w8a16_fast_ok(d, x, w, scale, offset)) {
+        const size_t total = static_cast<size_t>(d->m) * d->n;
+        size_t blocks = (total + kThreads - 1) / kThreads;
+        if (blocks > 65536) blocks = 65536;
+        w8a16_generic_kernel<<<static_cast<uint32_t>(blocks), kThreads, 0, st>>>(p);
+        return launch_status("ascq_matmul_w8a16 (generic)");
+    }
+    const size_t need = w8a16_workspace_need(d->n, d->k);
+    ASCQ_REQUIRE(workspace != nullptr && workspace_bytes >= need, ASCQ_EINVAL,
+                 "ascq_matmul_w8a16: workspace of %zu bytes required (see ascq_matmul_w8a16_workspace_size)", need);
+    ASCQ_REQUIRE(aligned16(workspace), ASCQ_EALIGN, "ascq_matmul_w8a16: workspace must be 16-byte aligned");
+    const W4Plan pl = make_plan(d->n, d->k, 2u * kMaxWaves, kW8ColsPerBlock);
+    p.waves = pl.waves;
+    p.chunks_per_block = pl.chunks_per_block;
+    p.total_chunks = pl.total_chunks;
+    p.max_seg = pl.max_seg;
+    p.per = pl.total_chunks / pl.waves;
+    p.rem = pl.total_chunks % pl.waves;
+    const uint32_t col_blocks = (d->n + kW8ColsPerBlock - 1u) / kW8ColsPerBlock;
+    const uint32_t grid = (p.waves + 7u) / 8u;
+    // 16 activation rows per pass over the weights
+    for (uint32_t m0 = 0; m0 < d->m; m0 += kTileRows) {
+        p.m0 = m0;
+        if (d->has_offset) {
+            w8a16_tile_kernel<true><<<grid, 512, 0, st>>>(p);
+        } else {
+            w8a16_tile_kernel<false><<<grid, 512, 0, st>>>(p);
+        }
+        stream_sum_kernel<4, kPieceTileW8><<<dim3(col_blocks, 4), 1024, 0, st>>>(p);
+    }
+    return launch_status("ascq_matmul_w8a16");
 }

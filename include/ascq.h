@@ -276,6 +276,33 @@ int ascq_matmul_w4a16(const ascq_w4a16_desc* desc, void* y, const void* x, const
                       const void* offset, void* workspace, size_t workspace_bytes, void* stream);
 int ascq_matmul_w4a16_workspace_size(const ascq_w4a16_desc* desc, size_t* bytes);
 
+/* ------------------------------------------------------------------- W8A16 */
+/*
+ * Matmul with A half and B int8 de-quantised on the way in ("anti-quant" matmul): the B matrix is turned into half by
+ * AscendAntiQuant<int8_t, half> with one scalar pair (SetAntiQuantScalar, MatmulConfig::isPerTensor) or one pair per
+ * output channel (SetAntiQuantVector), then a half matmul with fp32 accumulation.
+ * ref: include/adv_api/matmul/matmul.h:161-168;
+ *      impl/adv_api/detail/matmul/stage/copy_cube_in/antiquant/antiquant_processor_using_ub.h:53-130.
+ * x f16 [m, k]; w int8 [k, n]; scale, offset f16 [n] (per channel) or the desc's scalars (per tensor).
+ *   wdq[k,j] = f16( scale[j] * f16( f16(w[k,j]) + offset[j] ) )               (offset iff has_offset)
+ *   y[i,j]   = out( sum_k f32(x[i,k]) * f32(wdq[k,j]) )                       fp32 accumulation
+ * The kernel is a weight-streaming one built for few activation rows (decode): the weights are read once per 16
+ * rows of x.  B as [n, k] (isTransposeB) is not supported.
+ * workspace: ascq_matmul_w8a16_workspace_size bytes (contents need not be initialised); calls that share a
+ * workspace must not overlap.
+ */
+typedef struct ascq_w8a16_desc {
+    uint32_t m, n, k;
+    int32_t per_tensor;  /* 1: scale / offset below (SetAntiQuantScalar); 0: vectors of n halves (SetAntiQuantVector) */
+    int32_t has_offset;  /* MatmulConfig::hasAntiQuantOffset */
+    float scale, offset; /* per-tensor parameters, rounded to half as the reference's half scalars */
+    int32_t out_dtype;   /* ASCQ_F16 | ASCQ_F32 */
+} ascq_w8a16_desc;
+
+int ascq_matmul_w8a16(const ascq_w8a16_desc* desc, void* y, const void* x, const void* w, const void* offset,
+                      const void* scale, void* workspace, size_t workspace_bytes, void* stream);
+int ascq_matmul_w8a16_workspace_size(const ascq_w8a16_desc* desc, size_t* bytes);
+
 /* --------------------------------------------- host "tiling" size queries */
 /*
  * Scratch-size queries with the reference's answers, for callers that size a

@@ -411,6 +411,63 @@ private:
     size_t workspace_bytes_ = 0;
 };
 
+// Matmul with A half and B int8 de-quantised on the way in (MatmulType<.., half> x MatmulType<.., int8_t>).
+// ref: include/adv_api/matmul/matmul.h:161-168 (SetAntiQuantScalar / SetAntiQuantVector); hasAntiQuantOffset is the
+// MatmulConfig field of that name.  CType: half or float.
+template <typename CType, bool hasAntiQuantOffset = true>
+class AntiQuantMatmul {
+public:
+    AntiQuantMatmul(uint32_t m, uint32_t n, uint32_t k)
+    {
+        desc_ = ascq_w8a16_desc{};
+        desc_.m = m;
+        desc_.n = n;
+        desc_.k = k;
+        desc_.has_offset = hasAntiQuantOffset ? 1 : 0;
+        desc_.out_dtype = DTypeOf<CType>::value;
+    }
+    void SetTensorA(const DeviceTensor<half>& a) { a_ = a.GetPhyAddr(); }
+    void SetTensorB(const DeviceTensor<int8_t>& b) { b_ = b.GetPhyAddr(); }
+    void SetAntiQuantScalar(float offsetScalar, float scaleScalar)
+    {
+        desc_.per_tensor = 1;
+        desc_.offset = offsetScalar;
+        desc_.scale = scaleScalar;
+    }
+    void SetAntiQuantVector(const DeviceTensor<half>& offsetTensor, const DeviceTensor<half>& scaleTensor)
+    {
+        desc_.per_tensor = 0;
+        offset_ = offsetTensor.GetPhyAddr();
+        scale_ = scaleTensor.GetPhyAddr();
+    }
+    void SetWorkspace(void* workspace, size_t bytes)
+    {
+        workspace_ = workspace;
+        workspace_bytes_ = bytes;
+    }
+    size_t GetWorkspaceSize() const
+    {
+        size_t bytes = 0;
+        Check(ascq_matmul_w8a16_workspace_size(&desc_, &bytes));
+        return bytes;
+    }
+    void IterateAll(const DeviceTensor<CType>& c, void* stream = nullptr)
+    {
+        Check(ascq_matmul_w8a16(&desc_, c.GetPhyAddr(), a_, b_, offset_, scale_, workspace_, workspace_bytes_,
+                                stream));
+    }
+    const ascq_w8a16_desc& Desc() const { return desc_; }
+
+private:
+    ascq_w8a16_desc desc_;
+    const void* a_ = nullptr;
+    const void* b_ = nullptr;
+    const void* offset_ = nullptr;
+    const void* scale_ = nullptr;
+    void* workspace_ = nullptr;
+    size_t workspace_bytes_ = 0;
+};
+
 }  // namespace ascq
 
 #endif  // ASCQ_ASCENDC_HPP

@@ -679,6 +679,62 @@ int orc_matmul_w4a16_cols(const ascq_w4a16_desc* d, uint16_t* y, const uint16_t*
     return 0;
 }
 
+/* ------------------------------------------------------------------- W8A16 */
+/* Matmul with A half and B int8 that is de-quantised on the way in: B goes through AscendAntiQuant<int8_t, half>
+ * (half math: f16(w) + offset, then * scale, one rounding each;
+ * ref: impl/adv_api/detail/matmul/stage/copy_cube_in/antiquant/antiquant_processor_using_ub.h:53-130 calling
+ * impl/adv_api/detail/quantization/antiquant/ascend_antiquant_impl.h) with one scalar pair
+ * (SetAntiQuantScalar) or one pair per output channel (SetAntiQuantVector, include/adv_api/matmul/matmul.h:161-168),
+ * followed by a dot product accumulated wider than the output and rounded once. */
+int orc_matmul_w8a16(const ascq_w8a16_desc* d, void* y, const uint16_t* x, const int8_t* w, const uint16_t* offset,
+                     const uint16_t* scale)
+{
+    size_t M = d->m, N = d->n, K = d->k;
+    const size_t blk = 64;
+    size_t nblk = (N + blk - 1) / blk;
+    uint16_t scale_s = orc_f32_to_f16(d->scale), offset_s = orc_f32_to_f16(d->offset);
+    float* xf = (float*)malloc(M * K * sizeof(float));
+    for (size_t i = 0; i < M * K; ++i) {
+        xf[i] = orc_f16_to_f32(x[i]);
+    }
+#pragma omp parallel
+    {
+        double* acc = (double*)malloc(M * blk * sizeof(double));
+#pragma omp for schedule(dynamic, 1)
+        for (size_t b = 0; b < nblk; ++b) {
+            size_t c0 = b * blk, c1 = c0 + blk < N ? c0 + blk : N;
+            for (size_t t = 0; t < M * blk; ++t) {
+                acc[t] = 0.0;
+            }
+            for (size_t kk = 0; kk < K; ++kk) {
+                for (size_t j = c0; j < c1; ++j) {
+                    uint16_t h = orc_f32_to_f16((float)w[kk * N + j]);
+                    if (d->has_offset) {
+                        h = orc_f16_add(h, d->per_tensor ? offset_s : offset[j]);
+                    }
+                    double wd = (double)orc_f16_to_f32(orc_f16_mul(d->per_tensor ? scale_s : scale[j], h));
+                    for (size_t i = 0; i < M; ++i) {
+                        acc[i * blk + (j - c0)] += (double)xf[i * K + kk] * wd;
+                    }
+                }
+            }
+            for (size_t i = 0; i < M; ++i) {
+                for (size_t j = c0; j < c1; ++j) {
+                    double v = acc[i * blk + (j - c0)];
+                    if (d->out_dtype == ASCQ_F32) {
+                        ((float*)y)[i * N + j] = (float)v;
+                    } else {
+                        ((uint16_t*)y)[i * N + j] = orc_f64_to_f16(v);
+                    }
+                }
+            }
+        }
+        free(acc);
+    }
+    free(xf);
+    return 0;
+}
+
 /* ------------------------------------------------ vectorised array helpers */
 void orc_f32_to_f16_array(uint16_t* dst, const float* src, size_t n)
 {

@@ -57,6 +57,7 @@ def lib():
         L.orc_group_matmul_w8a8.argtypes = [C.POINTER(abi.GroupMatmulDesc), _P, _P, _P, _P, _P, _P, _P]
         L.orc_matmul_w4a16.argtypes = [C.POINTER(abi.W4A16Desc), _P, _P, _P, _P, _P]
         L.orc_matmul_w4a16_cols.argtypes = [C.POINTER(abi.W4A16Desc), _P, _P, _P, _P, _P, C.c_uint32, C.c_uint32]
+        L.orc_matmul_w8a16.argtypes = [C.POINTER(abi.W8A16Desc), _P, _P, _P, _P, _P]
         for name in ("orc_f32_to_f16_array", "orc_f16_to_f32_array", "orc_f32_to_bf16_array"):
             getattr(L, name).argtypes = [_P, _P, C.c_size_t]
         for name in ("orc_f16_mul_array", "orc_f16_add_array"):
@@ -196,4 +197,10 @@ def matmul_w4a16(desc, x, w, scale, offset=None, cols=None):
     else:
         lib().orc_matmul_w4a16_cols(C.byref(desc), _ptr(y), _ptr(x), _ptr(w), _ptr(scale), _ptr(offset), cols[0],
                                     cols[1])
+    return y
+
+
+def matmul_w8a16(desc, x, w, offset=None, scale=None):
+    y = np.zeros((desc.m, desc.n), dtype=_NP[desc.out_dtype])
+    lib().orc_matmul_w8a16(C.byref(desc), _ptr(y), _ptr(x), _ptr(w), _ptr(offset), _ptr(scale))
     return y

@@ -1,6 +1,6 @@
 // Drives the HIP library through the C++ host mirror (include/ascq_ascendc.hpp) the way a reference user drives
-// AscendC::AscendQuant / AscendDequant / AscendAntiQuant / Matmul, and compares every result bit-for-bit with the CPU
-// oracle.  Host code only: device memory comes from the HIP runtime, the kernels from libascq.so.
+// AscendC::AscendQuant / AscendDequant / AscendAntiQuant / Matmul (int8 and anti-quant), and compares every result
+// bit-for-bit with the CPU oracle.  Host code only: device memory comes from the HIP runtime, the kernels from libascq.so.
 #include <hip/hip_runtime.h>
 
 #include <cstdio>
@@ -238,6 +238,34 @@ void test_matmul()
     }
 }
 
+void test_antiquant_matmul()
+{
+    // small integers, a power-of-two scale and an integer offset: every product and partial sum is exact in fp32, so
+    // the result does not depend on the order of accumulation and must equal the oracle's bit for bit
+    std::printf("[case] AntiQuantMatmul<float> 5x272x128, SetAntiQuantVector\n");
+    Rng r{6};
+    const uint32_t m = 5, n = 272, k = 128;
+    std::vector<uint16_t> x(m * k), sc(n), of(n);
+    std::vector<int8_t> w(k * n);
+    for (auto& e : x) e = orc_f32_to_f16(static_cast<float>(r.integer(-4, 4)));
+    for (auto& e : w) e = static_cast<int8_t>(r.integer(-128, 127));
+    for (auto& e : sc) e = orc_f32_to_f16(r.integer(0, 1) ? 0.5f : 0.25f);
+    for (auto& e : of) e = orc_f32_to_f16(static_cast<float>(r.integer(-8, 8)));
+    DeviceBuffer<uint16_t> dx(x), dsc(sc), dof(of);
+    DeviceBuffer<int8_t> dw(w);
+    DeviceBuffer<float> dc(m * n);
+    ascq::AntiQuantMatmul<float> mm(m, n, k);
+    DeviceBuffer<uint8_t> ws(mm.GetWorkspaceSize() + 16);
+    mm.SetTensorA(dx.view<ascq::half>(m * k));
+    mm.SetTensorB(dw.view<int8_t>(k * n));
+    mm.SetAntiQuantVector(dof.view<ascq::half>(n), dsc.view<ascq::half>(n));
+    mm.SetWorkspace(ws.view<uint8_t>(1).GetPhyAddr(), mm.GetWorkspaceSize());
+    mm.IterateAll(dc.view<float>(m * n));
+    std::vector<float> want(m * n);
+    orc_matmul_w8a16(&mm.Desc(), want.data(), x.data(), w.data(), of.data(), sc.data());
+    expect_equal("AntiQuantMatmul", dc.download(), want);
+}
+
 void test_errors()
 {
     std::printf("[case] argument errors surface as ascq::Error\n");
@@ -278,6 +306,7 @@ int main()
     test_dequant();
     test_antiquant();
     test_matmul();
+    test_antiquant_matmul();
     test_errors();
     std::printf("%s\n", g_failed ? "FAILED" : "ALL PASSED");
     return g_failed ? 1 : 0;

@@ -247,3 +247,78 @@ def test_config4_w4a16_decode(m):
     tol = 1e-3 * np.maximum(np.abs(want.astype(np.float64)), 1.0)
     assert np.all(err <= tol + 2e-3)
     assert max_ulp(got.view(np.uint16), want.view(np.uint16), "f16") <= 4 or np.mean(err <= tol) > 0.999
+
+
+# ------------------------------------------------------------------ W8A16 (Matmul anti-quant path)
+def w8a16_check(got, want, x, out_f32):
+    # fp32 accumulation in a different order than the oracle's wide one: error bounded relative to sum |x| |w| (w up
+    # to 137 * 1e-2 in these cases), and bit-identical halves nearly everywhere
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    ref = np.abs(x.astype(np.float64)).sum(axis=1, keepdims=True) * 1.4
+    assert np.all(err <= 1e-5 * ref + 1e-6) if out_f32 else np.all(err <= 1e-3 * ref + 1e-6)
+    if not out_f32:
+        assert np.mean(got.view(np.uint16) == want.view(np.uint16)) > 0.9
+
+
+@pytest.mark.parametrize("m", [1, 3, 16, 17, 40])
+@pytest.mark.parametrize("k,n", [(256, 256), (512, 1040), (96, 48), (100, 30), (2048, 512)])
+@pytest.mark.parametrize("mode", ["vector+offset", "vector", "scalar+offset", "scalar", "vector+intoffset"])
+def test_w8a16_small(m, k, n, mode):
+    announce("w8a16", m, k, n, mode)
+    rng = np.random.default_rng(m * 7 + k + n)
+    x = rng.standard_normal((m, k)).astype(np.float16)
+    w = rng.integers(-128, 128, (k, n)).astype(np.int8)
+    per_tensor = mode.startswith("scalar")
+    has_offset = "offset" in mode
+    out_f32 = (m + k) % 2 == 1
+    if per_tensor:
+        sc, of = 0.0077, (2.5 if has_offset else None)
+    else:
+        sc = rng.uniform(1e-3, 1e-2, n).astype(np.float16)
+        of = None
+        if has_offset:
+            of = (rng.integers(-9, 10, n) if "int" in mode else rng.uniform(-9, 9, n)).astype(np.float16)
+    y = torch.zeros((m, n), dtype=torch.float32 if out_f32 else torch.float16, device=DEV)
+    ops.matmul_w8a16(y, to_dev(x), to_dev(w), of if per_tensor else (None if of is None else to_dev(of)),
+                     sc if per_tensor else to_dev(sc))
+    d = abi.W8A16Desc(m=m, n=n, k=k, per_tensor=int(per_tensor), has_offset=int(has_offset),
+                      scale=sc if per_tensor else 0.0, offset=of if per_tensor and has_offset else 0.0,
+                      out_dtype=abi.F32 if out_f32 else abi.F16)
+    want = orc.matmul_w8a16(d, x, w, None if per_tensor else of, None if per_tensor else sc)
+    w8a16_check(y.cpu().numpy(), want, x, out_f32)
+
+
+@pytest.mark.parametrize("m", [1, 16])
+def test_w8a16_decode_shape(m):
+    """fp16 [M,4096] x int8 [4096,11008], per-channel scale and offset (the W8A8 headline weight shape)."""
+    announce("w8a16 decode", m)
+    rng = np.random.default_rng(0xA16 + m)
+    k, n = 4096, 11008
+    x = rng.standard_normal((m, k)).astype(np.float16)
+    w = rng.integers(-128, 128, (k, n)).astype(np.int8)
+    sc = rng.uniform(1e-3, 1e-2, n).astype(np.float16)
+    of = rng.uniform(-9, 9, n).astype(np.float16)
+    y = torch.zeros((m, n), dtype=torch.float16, device=DEV)
+    ops.matmul_w8a16(y, to_dev(x), to_dev(w), to_dev(of), to_dev(sc))
+    d = abi.W8A16Desc(m=m, n=n, k=k, per_tensor=0, has_offset=1, out_dtype=abi.F16)
+    orc.set_threads(16)
+    want = orc.matmul_w8a16(d, x, w, of, sc)
+    w8a16_check(y.cpu().numpy(), want, x, False)
+
+
+@pytest.mark.parametrize("m", [2, 16])
+def test_w8a16_exact_integers_full_size(m):
+    """Small integer activations, power-of-two scales and integer offsets make every product and partial sum exact in
+    fp32, so the result is independent of the accumulation order: bit-equal to plain integer arithmetic at full size."""
+    announce("w8a16 exact", m)
+    rng = np.random.default_rng(0xE8 + m)
+    k, n = 4096, 11008
+    xi = rng.integers(-2, 3, (m, k))
+    w = rng.integers(-128, 128, (k, n)).astype(np.int8)
+    sc = rng.choice([0.25, 0.5, 1.0], n)
+    of = rng.integers(-9, 10, n)
+    y = torch.zeros((m, n), dtype=torch.float32, device=DEV)
+    ops.matmul_w8a16(y, to_dev(xi.astype(np.float16)), to_dev(w), to_dev(of.astype(np.float16)),
+                     to_dev(sc.astype(np.float16)))
+    want = (xi.astype(np.float64) @ (w.astype(np.float64) + of[None, :])) * sc[None, :]
+    assert np.array_equal(y.cpu().numpy().astype(np.float64), want)

@@ -453,3 +453,31 @@ def test_w4a16_against_numpy_half_dequant():
     assert np.array_equal(got.view(U16), want.view(U16))
     sub = orc.matmul_w4a16(d, x, packed, sc, of, cols=(8, 24))
     assert np.array_equal(sub[:, 8:24].view(U16), want[:, 8:24].view(U16))
+
+
+@pytest.mark.parametrize("per_tensor", [False, True])
+@pytest.mark.parametrize("has_offset", [True, False])
+def test_w8a16_is_antiquant_then_half_matmul(per_tensor, has_offset):
+    """The W8A16 oracle = the AscendAntiQuant<int8_t, half> oracle (pinned by the documentation examples) applied to
+    B, followed by numpy's float64 matmul and one rounding; non-integer offsets make both half roundings matter."""
+    rng = np.random.default_rng(23 + per_tensor + 2 * has_offset)
+    M, K, N = 5, 192, 80
+    x = h(rng.standard_normal((M, K)))
+    w = rng.integers(-128, 128, (K, N)).astype(np.int8)
+    if per_tensor:
+        sc_s, of_s = 0.0123, 3.3
+        sc, of = h(np.full(N, sc_s)), h(np.full(N, of_s))
+    else:
+        sc, of = h(rng.uniform(1e-3, 1e-2, N)), h(rng.uniform(-9, 9, N))
+    wdq = (sc[None, :] * ((w.astype(np.float16) + of[None, :]).astype(np.float16) if has_offset
+                          else w.astype(np.float16))).astype(np.float16)
+    ad = aq_desc(has_offset=int(has_offset), k=K, n=N, scale_height=1, scale_width=N, offset_height=1, offset_width=N)
+    assert np.array_equal(orc.antiquant(ad, w, of[None, :] if has_offset else None, sc[None, :]).view(U16),
+                          wdq.view(U16))
+    for out_dtype, npdt in ((abi.F16, np.float16), (abi.F32, np.float32)):
+        d = abi.W8A16Desc(m=M, n=N, k=K, per_tensor=int(per_tensor), has_offset=int(has_offset),
+                          scale=sc_s if per_tensor else 0.0, offset=of_s if per_tensor else 0.0, out_dtype=out_dtype)
+        got = orc.matmul_w8a16(d, x, w, None if per_tensor else (of if has_offset else None),
+                               None if per_tensor else sc)
+        want = (x.astype(np.float64) @ wdq.astype(np.float64)).astype(npdt)
+        assert np.array_equal(got, want)
