@@ -280,7 +280,7 @@ def main():
     out["w4a16_gemv"] = {"metric": "w4a16_decode_gemv_hbm_gbs_m1_k8192_n28672", "value": gemv["gbs"], "unit": "GB/s",
                          "workload": "BASELINE configs[3] at M=1, 4 rotating weight sets (500 MB > Infinity Cache)",
                          "ms_per_step": gemv["ms_per_step"],
-                         "roofline": {"bound": "hbm", "kernel": "w4a16_gemv_kernel<offset> + w4a16_sum_kernel<1>",
+                         "roofline": {"bound": "hbm", "kernel": "w4a16_gemv_kernel<1, offset> + stream_sum_kernel<1>",
                                       "achieved": gemv["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                       "frac": gemv["gbs"] / PEAK_HBM_GBS, "traffic": GEMV_TRAFFIC_BYTES,
                                       "avg_kernel_ms": gemv["kernel_ms"], "bytes_per_launch": gemv["bytes"]}}
