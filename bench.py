@@ -28,8 +28,8 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E peak, GB/s
 # `bench.py --quick --no-cpu --copy-probe`; each counter is scaled by its reading for the 1 GiB copy of the same run
 # (FETCH_SIZE reads 0.5 per KiB there, WRITE_SIZE 1.0 per KiB).  Measured offline and recorded here; a run of this
 # file does not re-measure them.
-GEMM_TRAFFIC_BYTES = 228336230   # M=2048 GEMM, both launches: 183.2 MB fetched + 45.1 MB written
-GEMV_TRAFFIC_BYTES = 145573273   # W4A16 M=1 GEMV, stream + sum kernels: 136.9 MB fetched + 8.6 MB written
+GEMM_TRAFFIC_BYTES = 228345446   # M=2048 GEMM, both launches: 183.2 MB fetched + 45.1 MB written
+GEMV_TRAFFIC_BYTES = 137013862   # W4A16 M=1 GEMV, stream + sum kernels: 132.7 MB fetched + 4.3 MB written
 
 
 def main():
