@@ -18,6 +18,7 @@ CAST_NONE, CAST_RINT, CAST_FLOOR, CAST_CEIL, CAST_ROUND, CAST_TRUNC = range(6)
 COMPUTE_F16, COMPUTE_SCALE_T, COMPUTE_F32 = range(3)
 # ascq_offset_kind
 OFFSET_NONE, OFFSET_SCALAR, OFFSET_TENSOR = range(3)
+QDST_I8, QDST_FP8_E4M3FN, QDST_FP8_E5M2 = range(3)
 # ascq_dequant_mode
 DEQUANT_WITH_SINGLE_ROW, DEQUANT_WITH_MULTI_ROW = range(2)
 # ascq_mm_*
@@ -35,7 +36,7 @@ class QuantDesc(C.Structure):
     _fields_ = [("policy", C.c_int32), ("src_dtype", C.c_int32), ("scale_dtype", C.c_int32), ("compute", C.c_int32),
                 ("round_mode", C.c_int32), ("offset_kind", C.c_int32), ("k_dim", C.c_int32), ("scale", C.c_float),
                 ("offset", C.c_float), ("m", C.c_uint32), ("n", C.c_uint32), ("cal_count", C.c_uint32),
-                ("group_size", C.c_uint32)]
+                ("group_size", C.c_uint32), ("dst_format", C.c_int32)]
 
 
 class DequantDesc(C.Structure):

@@ -17,6 +17,7 @@ _DT = {torch.float16: abi.F16, torch.bfloat16: abi.BF16, torch.float32: abi.F32,
        torch.int32: abi.I32, torch.int64: abi.U64, torch.uint8: abi.I4}
 if hasattr(torch, "uint64"):
     _DT[torch.uint64] = abi.U64
+_QDST = {torch.int8: abi.QDST_I8, torch.float8_e4m3fn: abi.QDST_FP8_E4M3FN, torch.float8_e5m2: abi.QDST_FP8_E5M2}
 _TORCH = {abi.F16: torch.float16, abi.BF16: torch.bfloat16, abi.F32: torch.float32, abi.I8: torch.int8,
           abi.I32: torch.int32}
 
@@ -86,7 +87,8 @@ def ascend_quant(dst, src, scale, offset, cal_count=None, scale_count=None, offs
 
 def _policy_quant(compute, dst, src, scale, offset, para, policy, config):
     d = abi.QuantDesc(policy=policy, src_dtype=_dt(src), compute=compute, round_mode=config.round_mode,
-                      k_dim=config.k_dim, m=para.m, n=para.n, cal_count=para.cal_count, group_size=para.group_size)
+                      k_dim=config.k_dim, m=para.m, n=para.n, cal_count=para.cal_count, group_size=para.group_size,
+                      dst_format=_QDST[dst.dtype])
     if policy == abi.PER_TENSOR:
         d.scale, d.scale_dtype = float(scale), _dt(src)
         scale = None
@@ -103,7 +105,7 @@ def _policy_quant(compute, dst, src, scale, offset, para, policy, config):
 
 def ascend_quant_policy(dst, src, scale, offset, para, policy, config=AscendQuantConfig()):
     """AscendQuant<dstT, srcT, scaleT, config, policy>(dst, src, scale, offset, para) for PER_TOKEN / PER_GROUP:
-    arithmetic in the scale's dtype.  ref: include/adv_api/quantization/ascend_quant.h:667-762."""
+    arithmetic in the scale's dtype for an int8 dst, in fp32 for a torch.float8_e4m3fn / float8_e5m2 dst.  ref: include/adv_api/quantization/ascend_quant.h:667-762."""
     return _policy_quant(abi.COMPUTE_SCALE_T, dst, src, scale, offset, para, policy, config)
 
 

@@ -219,6 +219,37 @@ __device__ __forceinline__ void store1(void* base, size_t idx, float v)
     }
 }
 
+// fp32 -> OCP 8-bit floats, round-half-even, saturating to the largest finite value; NaN -> 0x7F with the sign.
+// kE5M2 false: e4m3fn (bias 7, max 448 = 0x7E); true: e5m2 (bias 15, max 57344 = 0x7B).
+template <bool kE5M2>
+__device__ __forceinline__ int f32_to_fp8_sat(float f)
+{
+    constexpr int kMant = kE5M2 ? 2 : 3;
+    constexpr int kBias = kE5M2 ? 15 : 7;
+    constexpr int kShift = 23 - kMant;
+    constexpr uint32_t kMaxBits = kE5M2 ? 0x47600000u : 0x43E00000u;      // 57344.0f / 448.0f
+    constexpr uint32_t kMinNormalBits = static_cast<uint32_t>(127 - kBias + 1) << 23;
+    uint32_t u;
+    __builtin_memcpy(&u, &f, 4);
+    const uint32_t sign = (u >> 24) & 0x80u;
+    const uint32_t a = u & 0x7FFFFFFFu;
+    uint32_t code;
+    if (a > 0x7F800000u) {
+        code = 0x7Fu;
+    } else if (a >= kMaxBits) {
+        code = kE5M2 ? 0x7Bu : 0x7Eu;  // everything from the largest finite value up, infinity included
+    } else if (a >= kMinNormalBits) {
+        const uint32_t r = a + ((1u << (kShift - 1)) - 1u) + ((a >> kShift) & 1u);  // ties to even
+        code = (r >> kShift) - (static_cast<uint32_t>(127 - kBias) << kMant);
+    } else {
+        // subnormal range: a multiple of the smallest subnormal, 2^(1 - bias - mant); 2^mant is the smallest normal
+        float mag;
+        __builtin_memcpy(&mag, &a, 4);
+        code = static_cast<uint32_t>(__builtin_rintf(mag * (kE5M2 ? 65536.0f : 512.0f)));
+    }
+    return static_cast<int>(sign | code);
+}
+
 __device__ __forceinline__ uint32_t pack4_i8(int a, int b, int c, int d)
 {
     return (static_cast<uint32_t>(a) & 0xFFu) | ((static_cast<uint32_t>(b) & 0xFFu) << 8) |

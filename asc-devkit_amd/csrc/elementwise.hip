@@ -24,7 +24,18 @@ struct QuantArgs {
     int policy, offset_kind, k_dim, round_mode;
     float sscale, soffset;
     uint32_t group_size, params_per_row;
+    int dst_format;  // ascq_quant_dst
 };
+
+// the last step: int8 with the requested rounding, or an 8-bit float (always half-even, saturating)
+template <bool kRint>
+__device__ __forceinline__ int quant_final(float t, const QuantArgs& a)
+{
+    if (a.dst_format == ASCQ_QDST_I8) {
+        return round_sat8<kRint>(t, a.round_mode);
+    }
+    return a.dst_format == ASCQ_QDST_FP8_E5M2 ? f32_to_fp8_sat<true>(t) : f32_to_fp8_sat<false>(t);
+}
 
 template <int kPar>
 __device__ __forceinline__ void quant_params8(const QuantArgs& a, const void* base, float scalar, uint32_t i,
@@ -127,7 +138,7 @@ __global__ __launch_bounds__(kThreads) void quant_vec_kernel(QuantArgs a)
                 if (has_off) {
                     t = Fmt<kCt>::add(t, o[e]);
                 }
-                q[e] = round_sat8<kRint>(t, a.round_mode);
+                q[e] = quant_final<kRint>(t, a);
             }
             u32x2 out;
             out[0] = pack4_i8(q[0], q[1], q[2], q[3]);
@@ -153,7 +164,7 @@ __global__ __launch_bounds__(kThreads) void quant_scalar_kernel(QuantArgs a)
                                                             : a.soffset;
             t = Fmt<kCt>::add(t, Fmt<kCt>::cvt(o));
         }
-        a.dst[e] = static_cast<int8_t>(round_sat8<false>(t, a.round_mode));
+        a.dst[e] = static_cast<int8_t>(quant_final<false>(t, a));
     }
 }
 
@@ -249,7 +260,8 @@ int launch_quant(const QuantArgs& a, bool vec, hipStream_t st)
         const bool rint = a.round_mode == ASCQ_CAST_RINT || a.round_mode == ASCQ_CAST_NONE;
         if constexpr (kSrc == ASCQ_F16 && kCt == ASCQ_F16) {
             // fp16 contract on a half source: scale / offset are half tensors or scalars
-            if (rint && (a.policy == ASCQ_PER_TENSOR || (a.policy == ASCQ_PER_CHANNEL && kPar == ASCQ_F16))) {
+            if (rint && a.dst_format == ASCQ_QDST_I8 &&
+                (a.policy == ASCQ_PER_TENSOR || (a.policy == ASCQ_PER_CHANNEL && kPar == ASCQ_F16))) {
                 quant_f16_fast_kernel<<<grid, kThreads, 0, st>>>(a);
                 return launch_status("ascq_quant");
             }
@@ -796,6 +808,10 @@ extern "C" int ascq_quant(const ascq_quant_desc* d, void* dst, const void* src, 
                  "ascq_quant: round mode %d is not supported for int8 output", d->round_mode);
     ASCQ_REQUIRE(d->offset_kind >= ASCQ_OFFSET_NONE && d->offset_kind <= ASCQ_OFFSET_TENSOR, ASCQ_EINVAL,
                  "ascq_quant: unknown offset kind %d", d->offset_kind);
+    ASCQ_REQUIRE(d->dst_format >= ASCQ_QDST_I8 && d->dst_format <= ASCQ_QDST_FP8_E5M2, ASCQ_EUNSUPPORTED,
+                 "ascq_quant: destination format %d is not int8 / fp8_e4m3fn / fp8_e5m2", d->dst_format);
+    ASCQ_REQUIRE(d->dst_format == ASCQ_QDST_I8 || d->compute != ASCQ_COMPUTE_F16, ASCQ_EUNSUPPORTED,
+                 "ascq_quant: the fp16 contract (AscendQuant per tensor / per channel) has int8 output only");
     const bool tensor_scale = d->policy != ASCQ_PER_TENSOR;
     int par = tensor_scale ? d->scale_dtype : ASCQ_F32;
     if (tensor_scale) {
@@ -850,7 +866,7 @@ extern "C" int ascq_quant(const ascq_quant_desc* d, void* dst, const void* src, 
                  ASCQ_EINVAL, "ascq_quant: dst overlaps src (in-place operation is not supported on the GPU)");
 
     QuantArgs a{static_cast<int8_t*>(dst), src, scale, offset, rows, n, d->policy, d->offset_kind, d->k_dim,
-                d->round_mode, d->scale, d->offset, d->group_size ? d->group_size : 1u, ppr};
+                d->round_mode, d->scale, d->offset, d->group_size ? d->group_size : 1u, ppr, d->dst_format};
     bool vec = (n % 8 == 0) && aligned16(src) && ((reinterpret_cast<uintptr_t>(dst) & 7u) == 0);
     if (tensor_scale) {
         vec = vec && aligned16(scale) && (d->offset_kind != ASCQ_OFFSET_TENSOR || aligned16(offset));
@@ -868,7 +884,10 @@ extern "C" int ascq_quant(const ascq_quant_desc* d, void* dst, const void* src, 
     if (src_dt == (S) && par == (P) && ct == (C)) {                \
         return launch_quant<S, P, C>(a, vec, st);                  \
     }
-    const int ct = d->compute == ASCQ_COMPUTE_F16 ? ASCQ_F16 : (d->compute == ASCQ_COMPUTE_F32 ? ASCQ_F32 : par);
+    // 8-bit float outputs are computed in fp32 whatever the parameter type
+    const int ct = d->compute == ASCQ_COMPUTE_F16
+                       ? ASCQ_F16
+                       : ((d->compute == ASCQ_COMPUTE_F32 || d->dst_format != ASCQ_QDST_I8) ? ASCQ_F32 : par);
     if (!tensor_scale) {
         ASCQ_Q(ASCQ_F16, ASCQ_F32, ASCQ_F16)
         ASCQ_Q(ASCQ_BF16, ASCQ_F32, ASCQ_F16)

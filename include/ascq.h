@@ -73,6 +73,11 @@ typedef enum ascq_quant_compute {
     ASCQ_COMPUTE_F32 = 2      /* Quantize: always fp32 (ref: impl/.../quantize/quantize_impl.h:641-968) */
 } ascq_quant_compute;
 
+/* Destination format of AscendQuant / Quantize.  The 8-bit floats are the OCP formats the reference names
+ * fp8_e4m3fn_t (bias 7, no infinity, NaN = S.1111.111, max 448) and fp8_e5m2_t (bias 15, max 57344)
+ * (ref: docs/zh/api/SIMD-API/基础API/数据结构/内置数据类型.md table 5). */
+typedef enum ascq_quant_dst { ASCQ_QDST_I8 = 0, ASCQ_QDST_FP8_E4M3FN = 1, ASCQ_QDST_FP8_E5M2 = 2 } ascq_quant_dst;
+
 typedef enum ascq_offset_kind { ASCQ_OFFSET_NONE = 0, ASCQ_OFFSET_SCALAR = 1, ASCQ_OFFSET_TENSOR = 2 } ascq_offset_kind;
 
 /* ref: impl/basic_api/utils/kernel_utils_mode.h:181-184 (DeQuantMode) */
@@ -93,6 +98,12 @@ typedef enum ascq_dequant_mode { ASCQ_DEQUANT_WITH_SINGLE_ROW = 0, ASCQ_DEQUANT_
  * COMPUTE_SCALE_T / F32: v = cvt(x) * s [+ o] with one rounding per operation in the compute
  *               type, y = sat8(round_mode(v)).
  * Tensor scale/offset dtype = scale_dtype (COMPUTE_F16: must equal src_dtype).
+ * dst_format FP8_E4M3FN / FP8_E5M2 (one byte per element): the arithmetic is fp32 whatever `compute` says
+ *               (source and parameters widened, one rounding per operation), then one conversion to the 8-bit
+ *               float, round-half-even, saturating to the largest finite value (448 / 57344); the reference falls
+ *               back to this rounding for every round_mode
+ *               (ref: impl/adv_api/detail/quantization/quant/ascend_quant_per_group_3510_impl.h:33-79,
+ *               impl/adv_api/detail/quantization/quantize/quantize_impl.h:64-73).
  */
 typedef struct ascq_quant_desc {
     int32_t policy;      /* ascq_policy */
@@ -107,6 +118,7 @@ typedef struct ascq_quant_desc {
     uint32_t m, n;       /* PER_TOKEN / PER_GROUP row count and row length; PER_CHANNEL: n = scale_count */
     uint32_t cal_count;  /* number of elements processed */
     uint32_t group_size; /* PER_GROUP */
+    int32_t dst_format;  /* ascq_quant_dst; 0 = int8 */
 } ascq_quant_desc;
 
 int ascq_quant(const ascq_quant_desc* desc, void* dst, const void* src, const void* scale, const void* offset,

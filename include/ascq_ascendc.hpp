@@ -50,6 +50,28 @@ struct bfloat16_t {
 struct int4b_t {  // two values per byte, even element in the low nibble
     uint8_t pair;
 };
+struct fp8_e4m3fn_t {
+    uint8_t bits;
+};
+struct fp8_e5m2_t {
+    uint8_t bits;
+};
+
+// destination types of AscendQuant
+template <typename T>
+struct QuantDstOf;
+template <>
+struct QuantDstOf<int8_t> {
+    static constexpr int32_t value = ASCQ_QDST_I8;
+};
+template <>
+struct QuantDstOf<fp8_e4m3fn_t> {
+    static constexpr int32_t value = ASCQ_QDST_FP8_E4M3FN;
+};
+template <>
+struct QuantDstOf<fp8_e5m2_t> {
+    static constexpr int32_t value = ASCQ_QDST_FP8_E5M2;
+};
 
 template <typename T>
 struct DTypeOf;
@@ -178,10 +200,11 @@ void AscendQuant(const DeviceTensor<int8_t>& dstTensor, const DeviceTensor<T>& s
                      offsetTensor.GetPhyAddr(), stream));
 }
 
-// PER_TOKEN / PER_GROUP with the arithmetic in scaleT (ref: ascend_quant.h:667-762).  The reference passes config and
-// policy as template arguments; they are ordinary arguments here.
-template <typename srcT, typename scaleT>
-void AscendQuant(const DeviceTensor<int8_t>& dstTensor, const DeviceTensor<srcT>& srcTensor,
+// PER_TOKEN / PER_GROUP (ref: ascend_quant.h:667-762): dstT int8_t with the arithmetic in scaleT, or fp8_e4m3fn_t /
+// fp8_e5m2_t with fp32 arithmetic.  The reference passes config and policy as template arguments; they are ordinary
+// arguments here.
+template <typename dstT, typename srcT, typename scaleT>
+void AscendQuant(const DeviceTensor<dstT>& dstTensor, const DeviceTensor<srcT>& srcTensor,
                  const DeviceTensor<scaleT>& scaleTensor, const DeviceTensor<scaleT>& offsetTensor,
                  const AscendQuantParam& para, const AscendQuantConfig& config, AscendQuantPolicy policy,
                  void* stream = nullptr)
@@ -198,6 +221,7 @@ void AscendQuant(const DeviceTensor<int8_t>& dstTensor, const DeviceTensor<srcT>
     d.n = para.n;
     d.cal_count = para.calCount;
     d.group_size = para.groupSize;
+    d.dst_format = QuantDstOf<dstT>::value;
     Check(ascq_quant(&d, dstTensor.GetPhyAddr(), srcTensor.GetPhyAddr(), scaleTensor.GetPhyAddr(),
                      config.hasOffset ? offsetTensor.GetPhyAddr() : nullptr, stream));
 }

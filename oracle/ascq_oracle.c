@@ -14,6 +14,13 @@
  * Each operator cites the reference file it restates (paths relative to the
  * asc-devkit tree).  Pinning status of every function is listed in
  * oracle/README.md.
+ *
+ * Parity unpinned (no reference vector, document table or independent
+ * implementation fixes these; the choice made is stated at the function):
+ *   - the fixpipe int32 -> bf16 modes (defined by analogy with DEQF16);
+ *   - NaN / Inf inputs, and fp16 overflow inside the half chains;
+ *   - fixpipe rounding for |acc| > 2^24, REQ8 offset signedness;
+ *   - 8-bit float outputs from the largest finite value up (saturation).
  */
 #include "ascq_oracle.h"
 
@@ -190,6 +197,64 @@ int8_t orc_round_sat8(double v, int round_mode)
     return (int8_t)r;
 }
 
+/* The value of an OCP 8-bit float code (sign handled by the caller): e4m3fn has bias 7, 3 mantissa bits and no
+ * infinity (0x7F is NaN, 0x7E = 448 the largest finite); e5m2 has bias 15, 2 mantissa bits, 0x7B = 57344 the largest
+ * finite.  ref: docs/zh/api/SIMD-API/基础API/数据结构/内置数据类型.md table 5. */
+static double fp8_code_value(int code, int e5m2)
+{
+    int mant_bits = e5m2 ? 2 : 3, bias = e5m2 ? 15 : 7;
+    int e = code >> mant_bits, m = code & ((1 << mant_bits) - 1);
+    if (e == 0) {
+        return ldexp((double)m, 1 - bias - mant_bits);
+    }
+    return ldexp((double)((1 << mant_bits) + m), e - bias - mant_bits);
+}
+
+/* fp32 -> 8-bit float by search: the nearest representable magnitude, ties to the even code, everything beyond the
+ * largest finite value (infinity included) saturates to it (SatMode::SAT of the reference's cast trait,
+ * ref: impl/adv_api/detail/quantization/quant/ascend_quant_per_group_3510_impl.h:41-42); NaN -> 0x7F with the sign. */
+uint8_t orc_f32_to_fp8(float f, int e5m2)
+{
+    int max_code = e5m2 ? 0x7B : 0x7E;
+    uint8_t sign = signbit(f) ? 0x80 : 0;
+    double a = fabs((double)f);
+    if (f != f) {
+        return (uint8_t)(sign | 0x7F);
+    }
+    if (a >= fp8_code_value(max_code, e5m2)) {
+        return (uint8_t)(sign | max_code);
+    }
+    int lo = 0; /* largest code whose value is <= a */
+    for (int c = 1; c <= max_code; ++c) {
+        if (fp8_code_value(c, e5m2) <= a) {
+            lo = c;
+        }
+    }
+    double below = fp8_code_value(lo, e5m2), above = fp8_code_value(lo + 1, e5m2);
+    int pick;
+    if (a - below < above - a) {
+        pick = lo;
+    } else if (a - below > above - a) {
+        pick = lo + 1;
+    } else {
+        pick = (lo & 1) ? lo + 1 : lo;
+    }
+    return (uint8_t)(sign | pick);
+}
+
+float orc_fp8_to_f32(uint8_t code, int e5m2)
+{
+    int mag = code & 0x7F;
+    if ((!e5m2 && mag == 0x7F) || (e5m2 && mag > 0x7C)) {
+        return NAN;
+    }
+    if (e5m2 && mag == 0x7C) {
+        return (code & 0x80) ? -INFINITY : INFINITY;
+    }
+    double v = fp8_code_value(mag, e5m2);
+    return (float)((code & 0x80) ? -v : v);
+}
+
 static inline float load_as_f32(const void* p, size_t i, int dtype)
 {
     switch (dtype) {
@@ -254,6 +319,10 @@ int orc_quant(const ascq_quant_desc* d, int8_t* dst, const void* src, const void
     size_t rows = total / n;
     int comp = d->compute;
     int ctype = (comp == ASCQ_COMPUTE_F16) ? ASCQ_F16 : (comp == ASCQ_COMPUTE_F32 ? ASCQ_F32 : d->scale_dtype);
+    if (d->dst_format != ASCQ_QDST_I8) {
+        ctype = ASCQ_F32; /* the 8-bit float paths widen everything to fp32:
+                             ascend_quant_per_group_3510_impl.h:54-74, quantize_impl.h:64-73 */
+    }
     int rmode = (comp == ASCQ_COMPUTE_F16) ? ASCQ_CAST_RINT : d->round_mode;
 
 #pragma omp parallel for schedule(static) if (rows * n > 65536)
@@ -294,7 +363,11 @@ int orc_quant(const ascq_quant_desc* d, int8_t* dst, const void* src, const void
                 }
                 v = (double)t;
             }
-            dst[e] = orc_round_sat8(v, rmode);
+            if (d->dst_format == ASCQ_QDST_I8) {
+                dst[e] = orc_round_sat8(v, rmode);
+            } else {
+                dst[e] = (int8_t)orc_f32_to_fp8((float)v, d->dst_format == ASCQ_QDST_FP8_E5M2);
+            }
         }
     }
     return 0;

@@ -123,6 +123,43 @@ void test_quant_per_channel()
     expect_equal("AscendQuant per tensor", got, want);
 }
 
+void test_quant_per_token_fp8()
+{
+    std::printf("[case] AscendQuant<fp8_e4m3fn_t, half, float> PER_TOKEN 12x256\n");
+    Rng r{7};
+    const uint32_t m = 12, n = 256;
+    auto x = random_halves(r, m * n, -3.0f, 3.0f);
+    std::vector<float> sc(m), of(m);
+    for (auto& e : sc) e = r.uniform(0.01f, 200.0f);  // the largest products pass 448 and saturate
+    for (auto& e : of) e = r.uniform(-1.0f, 1.0f);
+    DeviceBuffer<uint16_t> dx(x);
+    DeviceBuffer<float> dsc(sc), dof(of);
+    DeviceBuffer<uint8_t> dq(m * n);
+    ascq::AscendQuantConfig cfg{};
+    cfg.hasOffset = true;
+    ascq::AscendQuantParam para{};
+    para.m = m;
+    para.n = n;
+    para.calCount = m * n;
+    ascq::AscendQuant(dq.view<ascq::fp8_e4m3fn_t>(m * n), dx.view<ascq::half>(m * n), dsc.view<float>(m),
+                      dof.view<float>(m), para, cfg, ascq::AscendQuantPolicy::PER_TOKEN);
+    ascq_quant_desc d{};
+    d.policy = ASCQ_PER_TOKEN;
+    d.src_dtype = ASCQ_F16;
+    d.scale_dtype = ASCQ_F32;
+    d.compute = ASCQ_COMPUTE_SCALE_T;
+    d.round_mode = ASCQ_CAST_RINT;
+    d.offset_kind = ASCQ_OFFSET_TENSOR;
+    d.k_dim = 1;
+    d.m = m;
+    d.n = n;
+    d.cal_count = m * n;
+    d.dst_format = ASCQ_QDST_FP8_E4M3FN;
+    std::vector<uint8_t> want(m * n);
+    orc_quant(&d, reinterpret_cast<int8_t*>(want.data()), x.data(), sc.data(), of.data());
+    expect_equal("AscendQuant fp8 per token", dq.download(), want);
+}
+
 void test_dequant()
 {
     std::printf("[case] AscendDequant<bfloat16_t, float, MULTI_ROW> 32x40, calCount 36\n");
@@ -303,6 +340,7 @@ int main()
     }
     std::printf("library: %s\n", ascq_version());
     test_quant_per_channel();
+    test_quant_per_token_fp8();
     test_dequant();
     test_antiquant();
     test_matmul();

@@ -29,12 +29,13 @@ def test_every_declared_symbol_is_exported_and_bound():
 
 def test_struct_sizes_match_the_header():
     # field-by-field layout is 4-byte scalars; the matmul descriptor ends with an 8-byte word
-    assert C.sizeof(abi.QuantDesc) == 13 * 4
+    assert C.sizeof(abi.QuantDesc) == 14 * 4
     assert C.sizeof(abi.DequantDesc) == 11 * 4
     assert C.sizeof(abi.AntiQuantDesc) == 13 * 4
     assert C.sizeof(abi.MatmulDesc) == 11 * 4 + 4 + 8
     assert C.sizeof(abi.GroupMatmulDesc) == C.sizeof(abi.MatmulDesc) + 8
     assert C.sizeof(abi.W4A16Desc) == 5 * 4
+    assert C.sizeof(abi.W8A16Desc) == 8 * 4
 
 
 def q(**kw):
@@ -56,6 +57,8 @@ def test_quant_rejections():
     assert call(q(n=0)) == abi.EINVAL
     assert call(q(src_dtype=abi.I8)) == abi.EUNSUPPORTED
     assert call(q(round_mode=6)) == abi.EUNSUPPORTED                                   # CAST_ODD has no int8 form
+    assert call(q(dst_format=3)) == abi.EUNSUPPORTED                                   # int8 / fp8_e4m3fn / fp8_e5m2 only
+    assert call(q(dst_format=abi.QDST_FP8_E5M2)) == abi.EUNSUPPORTED                   # the fp16 contract is int8 only
     assert call(q(policy=abi.PER_TOKEN)) == abi.EUNSUPPORTED                           # fp16 compute is tensor/channel only
     assert call(q(scale_dtype=abi.F32)) == abi.EUNSUPPORTED                            # legacy: scale dtype == src dtype
     tok = dict(policy=abi.PER_TOKEN, compute=abi.COMPUTE_SCALE_T, m=10, n=288, cal_count=2880)

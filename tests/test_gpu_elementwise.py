@@ -131,6 +131,69 @@ def test_dynamic_quant_per_token(src_dt, m, n):
     assert np.array_equal(q.cpu().numpy(), wq)
 
 
+# ------------------------------------------------------------------ 8-bit float destinations
+FP8 = {abi.QDST_FP8_E4M3FN: torch.float8_e4m3fn, abi.QDST_FP8_E5M2: torch.float8_e5m2}
+
+
+def typed(x, dtype):
+    """fp32 values -> (host array in `dtype`'s representation, device tensor)."""
+    x = np.asarray(x, dtype=np.float32)
+    if dtype == abi.F32:
+        return x, to_dev(x)
+    if dtype == abi.F16:
+        return x.astype(np.float16), to_dev(x.astype(np.float16))
+    b = orc.f32_to_bf16_bits(x)
+    return b, to_dev(b, "bf16")
+
+
+@pytest.mark.parametrize("fmt", [abi.QDST_FP8_E4M3FN, abi.QDST_FP8_E5M2])
+@pytest.mark.parametrize("pair", PAIRS)
+@pytest.mark.parametrize("policy", ["token", "group0", "group1", "channel", "tensor"])
+def test_quant_fp8(fmt, pair, policy):
+    """fp8_e4m3fn / fp8_e5m2 outputs (fp32 arithmetic, half-even, saturating): bit-exact against the oracle.  The
+    scales push part of the data past the largest finite value and part of it into the subnormal range."""
+    src_dt, sc_dt = pair
+    for (m, n, cal) in [(10, 288, 1152), (8, 512, 3584), (6, 36 * 8, 6 * 36 * 8)]:
+        announce("quant fp8", fmt, pair, policy, m, n, cal)
+        rng = np.random.default_rng(m + n + fmt)
+        x, xd = src_array(rng, (m, n), src_dt, 1.0)
+        top = 300.0 if fmt == abi.QDST_FP8_E4M3FN else 40000.0
+        gs = 32
+        pol = {"token": abi.PER_TOKEN, "group0": abi.PER_GROUP, "group1": abi.PER_GROUP, "channel": abi.PER_CHANNEL,
+               "tensor": abi.PER_TENSOR}[policy]
+        k_dim = 0 if policy == "group0" else 1
+        sshape = {"token": (m,), "group0": (-(-m // gs), n), "group1": (m, -(-n // gs)), "channel": (n,),
+                  "tensor": (1,)}[policy]
+        # log-uniform scales: products from 1e-3 (subnormal for e4m3fn) to beyond the largest finite value
+        s = np.exp(rng.uniform(np.log(1e-3), np.log(top), sshape)).astype(np.float32)
+        s.flat[0], s.flat[-1] = min(top * 8, 6e4), 1e-3  # both ends are present whatever the draw (finite in half)
+        o = rng.uniform(-0.5, 0.5, sshape).astype(np.float32)
+        (s, sdev), (o, odev) = typed(s, sc_dt), typed(o, sc_dt)
+        dst = torch.zeros((m, n), dtype=FP8[fmt], device=DEV)
+        cfg = ops.AscendQuantConfig(has_offset=True, k_dim=k_dim, round_mode=abi.CAST_RINT)
+        para = ops.AscendQuantParam(m=m, n=n, cal_count=cal, group_size=gs if pol == abi.PER_GROUP else 0)
+        d = abi.QuantDesc(policy=pol, src_dtype=src_dt, scale_dtype=sc_dt, compute=abi.COMPUTE_F32,
+                          round_mode=abi.CAST_RINT, k_dim=k_dim, m=m, n=n, cal_count=cal,
+                          group_size=para.group_size, dst_format=fmt, offset_kind=abi.OFFSET_TENSOR)
+        if pol == abi.PER_TENSOR:
+            sv, ov = float(np.float32(3.7)), 0.25
+            ops.quantize(dst, xd, sv, ov, para, pol, cfg)
+            d.scale, d.offset, d.offset_kind, d.scale_dtype = sv, ov, abi.OFFSET_SCALAR, src_dt
+            want = orc.quant(d, x.reshape(-1)[:cal].copy())
+        else:
+            fn = ops.ascend_quant_policy if pol in (abi.PER_TOKEN, abi.PER_GROUP) else ops.quantize
+            if fn is ops.ascend_quant_policy:
+                d.compute = abi.COMPUTE_SCALE_T        # the library widens to fp32 by itself for these outputs
+            fn(dst, xd, sdev, odev, para, pol, cfg)
+            want = orc.quant(d, x.reshape(-1)[:cal].copy(), s, o)
+        got = dst.view(torch.uint8).cpu().numpy().reshape(-1)
+        assert np.array_equal(got[:cal], want.view(np.uint8))
+        assert np.all(got[cal:] == 0)
+        if pol != abi.PER_TENSOR and cal == m * n:
+            top_code = 0x7E if fmt == abi.QDST_FP8_E4M3FN else 0x7B
+            assert np.any((got[:cal] & 0x7F) == top_code)          # saturation was exercised
+
+
 # ------------------------------------------------------------------ AscendDequant
 @pytest.mark.parametrize("dst_dt,sc_dt", [(abi.F16, abi.U64), (abi.F32, abi.F32), (abi.F32, abi.BF16),
                                           (abi.BF16, abi.BF16), (abi.BF16, abi.F32)])

@@ -1,5 +1,7 @@
 """Pins of the oracle's scalar numerics against independent implementations (numpy's float16, torch's bfloat16),
 closed forms, and the worked examples of the reference's precision-conversion document."""
+import ctypes as C
+
 import numpy as np
 import pytest
 import torch
@@ -110,3 +112,57 @@ def test_round_sat8_doc_example():
         assert orc.round_sat8(np.array([127.5], np.float32), mode)[0] == 127
     # ties to even under RINT
     assert list(orc.round_sat8(np.array([0.5, 1.5, 2.5, -0.5, -1.5, -2.5], np.float32))) == [0, 2, 2, 0, -2, -2]
+
+
+# ------------------------------------------------------------------ 8-bit floats
+def _fp8_lib():
+    L = orc.lib()
+    L.orc_f32_to_fp8.restype = C.c_uint8
+    L.orc_f32_to_fp8.argtypes = [C.c_float, C.c_int]
+    L.orc_fp8_to_f32.restype = C.c_float
+    L.orc_fp8_to_f32.argtypes = [C.c_uint8, C.c_int]
+    return L
+
+
+@pytest.mark.parametrize("e5m2", [0, 1])
+def test_fp8_codes_decode_like_torch_and_round_trip(e5m2):
+    """All 256 codes: the value equals torch's float8 (the OCP formats the reference's own golden scripts take from
+    ml_dtypes, examples/.../matmul_fp8/scripts/gen_data.py:142-147), and encoding a representable value gives its
+    code back."""
+    L = _fp8_lib()
+    tdt = torch.float8_e5m2 if e5m2 else torch.float8_e4m3fn
+    vals = torch.arange(256, dtype=torch.int32).to(torch.uint8).view(tdt).float().numpy()
+    for code in range(256):
+        mine = L.orc_fp8_to_f32(code, e5m2)
+        if np.isnan(vals[code]):
+            assert np.isnan(mine)
+            continue
+        assert mine == vals[code]
+        if np.isfinite(mine):
+            back = L.orc_f32_to_fp8(mine, e5m2)
+            assert back == code or (mine == 0 and (back & 0x7F) == 0)
+
+
+@pytest.mark.parametrize("e5m2", [0, 1])
+def test_fp8_encode_matches_torch_in_range_and_saturates(e5m2):
+    """Round-half-even to the nearest representable value agrees with torch's conversion for every input below the
+    overflow threshold (random values, every midpoint between neighbours and its two fp32 neighbours); from the
+    largest finite value up the result saturates (the reference's SatMode::SAT) where torch gives NaN / infinity."""
+    L = _fp8_lib()
+    tdt = torch.float8_e5m2 if e5m2 else torch.float8_e4m3fn
+    top_code = 0x7B if e5m2 else 0x7E
+    top = L.orc_fp8_to_f32(top_code, e5m2)
+    grid = np.array([L.orc_fp8_to_f32(c, e5m2) for c in range(top_code + 1)], dtype=np.float64)
+    mids = ((grid[:-1] + grid[1:]) / 2).astype(np.float32)
+    rng = np.random.default_rng(8)
+    rand = (np.exp(rng.uniform(np.log(1e-8), np.log(top), 20000)) * rng.choice([-1, 1], 20000)).astype(np.float32)
+    xs = np.concatenate([mids, np.nextafter(mids, np.float32(0)), np.nextafter(mids, np.float32(np.inf)), -mids, rand,
+                         grid.astype(np.float32), np.float32([0.0, -0.0])])
+    want = torch.from_numpy(xs).to(tdt).view(torch.uint8).numpy()
+    got = np.array([L.orc_f32_to_fp8(float(v), e5m2) for v in xs], dtype=np.uint8)
+    assert np.array_equal(got, want)
+    for v in (top, np.nextafter(np.float32(top), np.float32(np.inf)), top * 1.04, top * 2, 1e30, np.inf):
+        assert L.orc_f32_to_fp8(float(v), e5m2) == top_code
+        assert L.orc_f32_to_fp8(-float(v), e5m2) == 0x80 | top_code
+    assert L.orc_f32_to_fp8(float("nan"), e5m2) & 0x7F == 0x7F
+

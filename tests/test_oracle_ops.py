@@ -5,6 +5,7 @@ import os
 
 import numpy as np
 import pytest
+import torch
 
 import orc
 from ascq import _abi as abi
@@ -481,3 +482,26 @@ def test_w8a16_is_antiquant_then_half_matmul(per_tensor, has_offset):
                                None if per_tensor else sc)
         want = (x.astype(np.float64) @ wdq.astype(np.float64)).astype(npdt)
         assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("fmt,tdt,top", [(abi.QDST_FP8_E4M3FN, torch.float8_e4m3fn, 448.0),
+                                         (abi.QDST_FP8_E5M2, torch.float8_e5m2, 57344.0)])
+@pytest.mark.parametrize("sc_dt", [abi.F16, abi.F32])
+def test_quant_fp8_is_fp32_arithmetic_then_one_conversion(fmt, tdt, top, sc_dt):
+    """8-bit float outputs: source and parameters widened to fp32, one fp32 multiply, one fp32 add, one conversion
+    (ascend_quant_per_group_3510_impl.h:54-74), checked against numpy fp32 arithmetic + torch's float8 conversion on
+    data kept below the overflow threshold; whatever the scale dtype or `compute` says."""
+    rng = np.random.default_rng(fmt * 10 + sc_dt)
+    m, n = 6, 64
+    x = h(rng.standard_normal((m, n)))
+    npdt = np.float16 if sc_dt == abi.F16 else np.float32
+    s = rng.uniform(1e-3, top / 8, m).astype(npdt)
+    o = rng.uniform(-1, 1, m).astype(npdt)
+    v = (x.astype(np.float32) * s.astype(np.float32)[:, None]) + o.astype(np.float32)[:, None]
+    assert np.abs(v).max() < top
+    want = torch.from_numpy(v).to(tdt).view(torch.uint8).numpy()
+    for compute in (abi.COMPUTE_SCALE_T, abi.COMPUTE_F32):
+        d = abi.QuantDesc(policy=abi.PER_TOKEN, src_dtype=abi.F16, scale_dtype=sc_dt, compute=compute,
+                          round_mode=abi.CAST_FLOOR, offset_kind=abi.OFFSET_TENSOR, k_dim=1, m=m, n=n, cal_count=m * n,
+                          dst_format=fmt)
+        assert np.array_equal(orc.quant(d, x, s, o).view(np.uint8), want)
