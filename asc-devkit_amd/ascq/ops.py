@@ -203,8 +203,10 @@ class Matmul:
     def set_tensor_a(self, a):
         self.a = a
 
-    def set_tensor_b(self, b):
+    def set_tensor_b(self, b, nz=False):
+        """b: int8 [k, n] row-major, or with nz=True the fractal layout [n/32, k/16, 16, 32] (CubeFormat::NZ)."""
         self.b = b
+        self.desc.b_format = abi.MM_B_NZ if nz else abi.MM_B_ND
 
     def set_bias(self, bias):
         """int32 bias: initial value of the accumulator; float32 / bfloat16 bias: added after dequantisation."""
@@ -248,15 +250,19 @@ class Matmul:
 
 
 def quant_group_matmul(y, x, weight, group_list, scale, per_token_scale=None, bias=None,
-                       group_list_kind=abi.GROUP_LIST_COUNTS, activation=abi.MM_ACT_NONE):
-    """The quantized grouped matmul of the reference's MoE example: x int8 [m, k], weight int8 [g, k, n], scale
-    float32 [g, n], per_token_scale float32 [m], group_list int64 [g] (counts or prefix sums).
+                       group_list_kind=abi.GROUP_LIST_COUNTS, activation=abi.MM_ACT_NONE, weight_nz=False):
+    """The quantized grouped matmul of the reference's MoE example: x int8 [m, k], weight int8 [g, k, n] (or, with
+    weight_nz, the example's fractal layout [g, n/32, k/16, 16, 32]), scale float32 [g, n], per_token_scale float32
+    [m], group_list int64 [g] (counts or prefix sums).
     ref: examples/01_simd_cpp_api/05_best_practices/03_fusion_compute/quant_group_matmul_high_performance/
     quant_group_matmul_custom.asc:255-454."""
-    g, k, n = weight.shape
+    if weight_nz:
+        g, k, n = weight.shape[0], weight.shape[2] * weight.shape[3], weight.shape[1] * weight.shape[4]
+    else:
+        g, k, n = weight.shape
     mm = abi.MatmulDesc(m=x.shape[0], n=n, k=k, out_dtype=_dt(y), quant_mode=abi.MM_QUANT_VECTOR,
                         scale_format=abi.MM_SCALE_F32, has_tok_scale=int(per_token_scale is not None),
-                        activation=activation)
+                        activation=activation, b_format=abi.MM_B_NZ if weight_nz else abi.MM_B_ND)
     if bias is not None:
         mm.bias_kind = abi.MM_BIAS_F32_POST if bias.dtype == torch.float32 else abi.MM_BIAS_BF16_POST
     d = abi.GroupMatmulDesc(mm=mm, groups=g, group_list_kind=group_list_kind)

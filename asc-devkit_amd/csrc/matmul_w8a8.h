@@ -19,6 +19,7 @@ struct GemmParams {
     const int8_t* a;
     const int8_t* b;
     uint32_t m, n, k;
+    uint32_t b_nz;  // B is in the fractal layout [n/32][k][32] (direct-to-LDS tile kernels only)
     uint32_t tiles_m, tiles_n;
     uint32_t k_splits, k_per_split;  // split-K: bytes of K per grid.z slice (multiple of kBK)
     int32_t* partial;                // split-K int32 accumulator [m, n]

@@ -495,6 +495,17 @@ int validate_mm(const ascq_matmul_desc* d, const char* who, const void* c, const
                  "%s: unknown bias kind %d", who, d->bias_kind);
     ASCQ_REQUIRE(d->activation == ASCQ_MM_ACT_NONE || d->activation == ASCQ_MM_ACT_FASTER_GELU, ASCQ_EINVAL,
                  "%s: unknown activation %d", who, d->activation);
+    ASCQ_REQUIRE(d->b_format == ASCQ_MM_B_ND || d->b_format == ASCQ_MM_B_NZ, ASCQ_EINVAL, "%s: unknown B format %d",
+                 who, d->b_format);
+    if (d->b_format == ASCQ_MM_B_NZ) {
+        ASCQ_REQUIRE(!d->trans_a && !d->trans_b, ASCQ_EUNSUPPORTED, "%s: fractal (NZ) B takes no transposition", who);
+        ASCQ_REQUIRE(d->n % 32 == 0 && d->k % 128 == 0, ASCQ_EALIGN,
+                     "%s: fractal (NZ) B needs n %% 32 == 0 and k %% 128 == 0 (n=%u, k=%u)", who, d->n, d->k);
+        ASCQ_REQUIRE(static_cast<uint64_t>(d->k) * d->n < (1ull << 32), ASCQ_EUNSUPPORTED,
+                     "%s: fractal (NZ) B is limited to k * n < 2^32", who);
+        ASCQ_REQUIRE(aligned16(a) && aligned16(b), ASCQ_EALIGN, "%s: fractal (NZ) B needs 16-byte aligned a and b",
+                     who);
+    }
     if (d->quant_mode == ASCQ_MM_QUANT_NONE) {
         ASCQ_REQUIRE(d->out_dtype == ASCQ_I32, ASCQ_EUNSUPPORTED, "%s: without a quant mode the output is int32", who);
         ASCQ_REQUIRE(d->bias_kind <= ASCQ_MM_BIAS_I32_PRE && !d->has_tok_scale && d->activation == ASCQ_MM_ACT_NONE,
@@ -591,6 +602,12 @@ extern "C" int ascq_matmul_w8a8(const ascq_matmul_desc* d, void* c, const void* 
     p.n = d->n;
     p.k = d->k;
     p.epi = make_epi(d, c, bias, quant_vector, tok_scale);
+    if (d->b_format == ASCQ_MM_B_NZ) {
+        // only the direct-to-LDS tile kernels address the fractal layout; validate_mm has checked what they need
+        p.b_nz = 1;
+        return d->m <= kSkinnyMaxM ? launch_gemm_dma_skinny(p, workspace, workspace_bytes, st)
+                                   : launch_gemm_dma(p, false, st);
+    }
     if (!fast_path_ok(d, a, b)) {
         size_t total = static_cast<size_t>(d->m) * d->n;
         size_t blocks = (total + kThreads - 1) / kThreads;
@@ -672,9 +689,11 @@ extern "C" int ascq_group_matmul_w8a8(const ascq_group_matmul_desc* g, void* y, 
     p.groups = g->groups;
     p.group_list_kind = g->group_list_kind;
     p.epi = make_epi(d, y, bias, scale, tok_scale);
+    p.b_nz = d->b_format == ASCQ_MM_B_NZ ? 1u : 0u;
     if (gemm_dma_supported(p)) {
         return launch_gemm_dma(p, true, st);
     }
+    ASCQ_REQUIRE(!p.b_nz, ASCQ_EUNSUPPORTED, "ascq_group_matmul_w8a8: fractal (NZ) weights need the tile kernel's shape");
     typedef TileL T;
     // every group adds at most one partial tile along M
     p.tiles_m = (d->m + T::BM - 1) / T::BM + g->groups;

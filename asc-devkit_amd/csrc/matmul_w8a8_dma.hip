@@ -152,8 +152,10 @@ __global__ __launch_bounds__(kThreads, (BM * BK + BK * BN) * 2 <= 65536 ? 2 : 1)
         const uint32_t q = (s % kPieces) ^ swz;
         uint32_t col = n0 + 16u * q;
         col = col + 16u <= N ? col : N - 16u;      // columns past the end are never stored
-        boff[u] = kb * N + (col - n0);
+        // fractal B: panels of 32 columns, each a contiguous row-major [K][32] block
+        boff[u] = p.b_nz ? ((col >> 5) * K + kb) * 32u + (col & 31u) : kb * N + (col - n0);
     }
+    const uint32_t ldb = p.b_nz ? 32u : N;  // bytes from one k to the next
     // K range of this workgroup, in steps of BK
     uint32_t s_begin = 0, steps = K / BK;
     if constexpr (kSplitK) {
@@ -161,10 +163,10 @@ __global__ __launch_bounds__(kThreads, (BM * BK + BK * BN) * 2 <= 65536 ? 2 : 1)
         steps = steps * (blockIdx.y + 1u) / p.k_splits - s_begin;
     }
     const int8_t* Abase = p.a + static_cast<size_t>(row0) * K + static_cast<size_t>(s_begin) * BK;
-    const int8_t* Bbase = Bmat + n0 + static_cast<size_t>(s_begin) * BK * N;
+    const int8_t* Bbase = Bmat + (p.b_nz ? 0u : n0) + static_cast<size_t>(s_begin) * BK * ldb;
     auto issue = [&](uint32_t k0, char* As, char* Bs) {
         const int8_t* ab = Abase + k0;
-        const int8_t* bb = Bbase + static_cast<size_t>(k0) * N;
+        const int8_t* bb = Bbase + static_cast<size_t>(k0) * ldb;
 #pragma unroll
         for (int u = 0; u < kAInstr; ++u) {
             __builtin_amdgcn_global_load_lds((gptr_t)(ab + aoff[u]), (lds_ptr_t)(As + (wave * kAInstr + u) * 1024), 16,

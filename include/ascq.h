@@ -202,6 +202,17 @@ typedef enum ascq_mm_scale_format {
     ASCQ_MM_SCALE_F32 = 1  /* plain fp32, all 23 mantissa bits used */
 } ascq_mm_scale_format;
 
+/* Layout of the B (weight) matrix in memory. */
+typedef enum ascq_mm_b_format {
+    ASCQ_MM_B_ND = 0, /* row-major [k, n] ([n, k] with trans_b) */
+    ASCQ_MM_B_NZ = 1  /* the reference's fractal weight format for int8: [n/32][k/16][16][32], i.e. panels of 32
+                         columns, each a row-major [k][32] block; element (k, j) lies at
+                         ((j/32) * K + k) * 32 + j % 32
+                         (ref: examples/.../quant_group_matmul_high_performance/scripts/gen_data.py:62-65;
+                         CubeFormat::NZ of MatmulType, include/adv_api/matmul/matmul.h).
+                         Needs n % 32 == 0, k % 128 == 0, k * n < 2^32, no transposition. */
+} ascq_mm_b_format;
+
 typedef enum ascq_mm_bias_kind {
     ASCQ_MM_BIAS_NONE = 0,
     ASCQ_MM_BIAS_I32_PRE = 1,   /* int32 [n], initial value of the accumulator
@@ -235,6 +246,7 @@ typedef struct ascq_matmul_desc {
     int32_t bias_kind;     /* ascq_mm_bias_kind */
     int32_t has_tok_scale; /* fp32 [m] multiplied after the channel scale */
     int32_t activation;    /* ascq_mm_activation */
+    int32_t b_format;      /* ascq_mm_b_format; for the grouped matmul every group's [k, n] block is in this format */
     uint64_t quant_scalar; /* QUANT_SCALAR: U64 word, or fp32 bits in the low half for F32 format */
 } ascq_matmul_desc;
 

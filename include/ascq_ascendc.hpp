@@ -335,9 +335,13 @@ void AscendAntiQuant(const DeviceTensor<OutputDataType>& dst, const DeviceTensor
     Check(ascq_antiquant(&d, dst.GetPhyAddr(), src.GetPhyAddr(), nullptr, nullptr, stream));
 }
 
+// Memory layout of a matrix operand, as the CubeFormat argument of the reference's MatmulType.
+enum class CubeFormat : int32_t { ND = 0, NZ = 1 };
+
 // The int8 Matmul object with the quant epilogue (ref: include/adv_api/matmul/matmul.h:138-185; the quant parameters
 // are consumed at copy-out, impl/adv_api/detail/matmul/stage/copy_cube_out/quant/quant_processor_fixpipe.h:74-222).
 // CType selects the output: int32_t (no quant), half / bfloat16_t / float / int8_t (quant epilogue).
+
 template <typename CType>
 class Matmul {
 public:
@@ -355,10 +359,12 @@ public:
         a_ = a.GetPhyAddr();
         desc_.trans_a = isTransposeA ? 1 : 0;
     }
-    void SetTensorB(const DeviceTensor<int8_t>& b, bool isTransposeB = false)
+    // format: the CubeFormat of the reference's MatmulType for B (ND, or the fractal NZ layout [n/32][k/16][16][32])
+    void SetTensorB(const DeviceTensor<int8_t>& b, bool isTransposeB = false, CubeFormat format = CubeFormat::ND)
     {
         b_ = b.GetPhyAddr();
         desc_.trans_b = isTransposeB ? 1 : 0;
+        desc_.b_format = format == CubeFormat::NZ ? ASCQ_MM_B_NZ : ASCQ_MM_B_ND;
     }
     // int32 bias: the accumulator's initial value, as in the reference.
     void SetBias(const DeviceTensor<int32_t>& bias)

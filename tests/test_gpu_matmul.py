@@ -322,3 +322,63 @@ def test_w8a16_exact_integers_full_size(m):
                      to_dev(sc.astype(np.float16)))
     want = (xi.astype(np.float64) @ (w.astype(np.float64) + of[None, :])) * sc[None, :]
     assert np.array_equal(y.cpu().numpy().astype(np.float64), want)
+
+# ------------------------------------------------------------------ fractal (NZ) weights
+def to_nz(w):
+    """[.., k, n] -> [.., n/32, k/16, 16, 32], as the reference example packs its weights
+    (quant_group_matmul_high_performance/scripts/gen_data.py:62-65)."""
+    *lead, k, n = w.shape
+    nd = len(lead)
+    perm = list(range(nd)) + [nd + 2, nd + 0, nd + 1, nd + 3]
+    return np.ascontiguousarray(w.reshape(*lead, k // 16, 16, n // 32, 32).transpose(perm))
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 64, 128), (48, 160, 256), (200, 544, 384), (513, 288, 128), (2048, 2848, 256)])
+@pytest.mark.parametrize("out", [torch.int32, torch.bfloat16])
+def test_matmul_nz_weights(m, n, k, out):
+    """The same product from fractal weights: bit-equal to the oracle on the row-major weights."""
+    announce("nz weights", m, n, k, out)
+    rng = np.random.default_rng(m + n + k)
+    a = rng.integers(-127, 128, (m, k)).astype(np.int8)
+    w = rng.integers(-127, 128, (k, n)).astype(np.int8)
+    c = torch.zeros((m, n), dtype=out, device=DEV)
+    mm = ops.Matmul(m, n, k)
+    mm.set_tensor_a(to_dev(a))
+    mm.set_tensor_b(to_dev(to_nz(w)), nz=True)
+    d = abi.MatmulDesc(m=m, n=n, k=k, out_dtype=abi.I32)
+    cs = ts = None
+    if out != torch.int32:
+        cs = rng.uniform(1e-4, 1e-2, n).astype(np.float32)
+        ts = rng.uniform(1e-3, 1e-1, m).astype(np.float32)
+        mm.set_quant_vector(to_dev(cs))
+        mm.set_token_scale(to_dev(ts))
+        d = abi.MatmulDesc(m=m, n=n, k=k, out_dtype=abi.BF16, quant_mode=abi.MM_QUANT_VECTOR,
+                           scale_format=abi.MM_SCALE_F32, has_tok_scale=1)
+    mm.iterate_all(c)
+    orc.set_threads(16)
+    want = orc.matmul_w8a8(d, a, w, None, cs, ts)
+    assert np.array_equal(bits(c), want)
+
+
+def test_group_matmul_nz_weights_as_the_reference_example_packs_them():
+    """The example's configuration in small: counts group list, fractal weights, FasterGelu, fp16 out."""
+    announce("group nz")
+    rng = np.random.default_rng(0x6E7A)
+    groups, k, n = 4, 256, 320
+    counts = [100, 0, 257, 31]
+    m = sum(counts)
+    x = rng.integers(-10, 10, (m, k)).astype(np.int8)
+    w = rng.integers(-10, 10, (groups, k, n)).astype(np.int8)
+    sc = rng.normal(0, 0.01, (groups, n)).astype(np.float32)
+    ts = rng.normal(0, 0.01, m).astype(np.float32)
+    y = torch.zeros((m, n), dtype=torch.float16, device=DEV)
+    gl = torch.tensor(counts, dtype=torch.int64, device=DEV)
+    ops.quant_group_matmul(y, to_dev(x), to_dev(to_nz(w)), gl, to_dev(sc), to_dev(ts),
+                           activation=abi.MM_ACT_FASTER_GELU, weight_nz=True)
+    mmd = abi.MatmulDesc(m=m, n=n, k=k, out_dtype=abi.F16, quant_mode=abi.MM_QUANT_VECTOR,
+                         scale_format=abi.MM_SCALE_F32, has_tok_scale=1, activation=abi.MM_ACT_FASTER_GELU)
+    gd = abi.GroupMatmulDesc(mm=mmd, groups=groups, group_list_kind=abi.GROUP_LIST_COUNTS)
+    want = orc.group_matmul_w8a8(gd, x, w, None, sc, ts, np.array(counts, dtype=np.int64))
+    got = bits(y)
+    assert max_ulp(got, want.view(np.uint16), "f16") <= 1
+
