@@ -382,3 +382,30 @@ def test_group_matmul_nz_weights_as_the_reference_example_packs_them():
     got = bits(y)
     assert max_ulp(got, want.view(np.uint16), "f16") <= 1
 
+
+def test_group_matmul_example_full_size_nz_equals_nd():
+    """The reference example's own size (8 groups x 1024 tokens, k=1024, n=8192, FasterGelu, fp16): the result from
+    the fractal weights is bit-equal to the one from row-major weights (which the other tests tie to the oracle), and
+    a sample of rows is checked against the example's golden formula in float64."""
+    announce("group example full size")
+    rng = np.random.default_rng(0xE8A)
+    groups, m, k, n = 8, 8192, 1024, 8192
+    counts = [1024] * groups
+    x = rng.integers(-10, 10, (m, k)).astype(np.int8)
+    w = rng.integers(-10, 10, (groups, k, n)).astype(np.int8)
+    sc = rng.normal(0, 0.01, (groups, n)).astype(np.float32)
+    ts = rng.normal(0, 0.01, m).astype(np.float32)
+    gl = torch.tensor(counts, dtype=torch.int64, device=DEV)
+    xd, scd, tsd = to_dev(x), to_dev(sc), to_dev(ts)
+    y_nd = torch.zeros((m, n), dtype=torch.float16, device=DEV)
+    y_nz = torch.zeros((m, n), dtype=torch.float16, device=DEV)
+    ops.quant_group_matmul(y_nd, xd, to_dev(w), gl, scd, tsd, activation=abi.MM_ACT_FASTER_GELU)
+    ops.quant_group_matmul(y_nz, xd, to_dev(to_nz(w)), gl, scd, tsd, activation=abi.MM_ACT_FASTER_GELU, weight_nz=True)
+    assert torch.equal(y_nd.view(torch.int16), y_nz.view(torch.int16))
+    rows = rng.choice(m, 64, replace=False)
+    got = y_nz[torch.from_numpy(rows).to(DEV)].float().cpu().numpy().astype(np.float64)
+    for i, r in enumerate(rows):
+        g = r // 1024
+        v = (x[r].astype(np.float64) @ w[g].astype(np.float64)) * sc[g].astype(np.float64) * float(ts[r])
+        gold = v / (1.0 + np.exp(-1.702 * v))                       # the example's FastGelu, in closed form
+        assert np.all(np.abs(got[i] - gold) <= 2e-3 * np.abs(gold) + 1e-6)
