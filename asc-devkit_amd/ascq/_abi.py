@@ -53,6 +53,12 @@ class AntiQuantDesc(C.Structure):
                 ("scale_height", C.c_uint32), ("scale_width", C.c_uint32)]
 
 
+class AntiQuantPolicyDesc(C.Structure):
+    _fields_ = [("policy", C.c_int32), ("src_format", C.c_int32), ("scale_dtype", C.c_int32), ("dst_dtype", C.c_int32),
+                ("compute", C.c_int32), ("has_offset", C.c_int32), ("is_transpose", C.c_int32), ("k_dim", C.c_int32),
+                ("m", C.c_uint32), ("n", C.c_uint32), ("cal_count", C.c_uint32), ("group_size", C.c_uint32)]
+
+
 class MatmulDesc(C.Structure):
     _fields_ = [("m", C.c_uint32), ("n", C.c_uint32), ("k", C.c_uint32), ("trans_a", C.c_int32),
                 ("trans_b", C.c_int32), ("out_dtype", C.c_int32), ("quant_mode", C.c_int32),
@@ -82,6 +88,7 @@ SIGNATURES = {
     "ascq_dequant": (C.c_int, [C.POINTER(DequantDesc), _P, _P, _P, _P]),
     "ascq_dequant_dst_stride": (C.c_uint32, [C.c_int32, C.c_uint32]),
     "ascq_antiquant": (C.c_int, [C.POINTER(AntiQuantDesc), _P, _P, _P, _P, _P]),
+    "ascq_antiquant_policy": (C.c_int, [C.POINTER(AntiQuantPolicyDesc), _P, _P, _P, _P, _P]),
     "ascq_matmul_w8a8": (C.c_int, [C.POINTER(MatmulDesc), _P, _P, _P, _P, _P, _P, _P, C.c_size_t, _P]),
     "ascq_matmul_w8a8_workspace_size": (C.c_int, [C.POINTER(MatmulDesc), C.POINTER(C.c_size_t)]),
     "ascq_group_matmul_w8a8": (C.c_int, [C.POINTER(GroupMatmulDesc), _P, _P, _P, _P, _P, _P, _P, _P]),

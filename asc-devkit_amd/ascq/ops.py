@@ -188,6 +188,44 @@ def ascend_antiquant(dst, src, offset, scale, k, shape_info=AntiQuantShapeInfo()
     return dst
 
 
+@dataclass
+class AscendAntiQuantConfig:
+    """ref: include/adv_api/quantization/ascend_antiquant_common.h:45-65"""
+    has_offset: bool = False
+    is_transpose: bool = False
+    k_dim: int = 1
+
+
+@dataclass
+class AscendAntiQuantParam:
+    m: int
+    n: int
+    cal_count: int
+    group_size: int = 0
+
+
+def _antiquant_policy(compute, dst, src, scale, offset, para, policy, config):
+    d = abi.AntiQuantPolicyDesc(policy=policy, src_format=_QDST[src.dtype], scale_dtype=_dt(scale), dst_dtype=_dt(dst),
+                                compute=compute, has_offset=int(config.has_offset),
+                                is_transpose=int(config.is_transpose), k_dim=config.k_dim, m=para.m, n=para.n,
+                                cal_count=para.cal_count, group_size=para.group_size)
+    check(load_library().ascq_antiquant_policy(C.byref(d), _ptr(dst), _ptr(src), _ptr(scale),
+                                               _ptr(offset) if config.has_offset else None, _stream()))
+    return dst
+
+
+def ascend_antiquant_policy(dst, src, scale, offset, para, policy, config=AscendAntiQuantConfig()):
+    """AscendAntiQuant<dstT, srcT, scaleT, config, policy>(dst, src, scale, offset, para) for PER_TOKEN / PER_GROUP:
+    src int8 / torch.float8_e4m3fn / torch.float8_e5m2 [m, n], arithmetic in the scale's dtype.
+    ref: impl/adv_api/detail/quantization/antiquant/ascend_antiquant_3510_impl.h:2166-2222."""
+    return _antiquant_policy(abi.COMPUTE_SCALE_T, dst, src, scale, offset, para, policy, config)
+
+
+def antiquantize(dst, src, scale, offset, para, policy, config=AscendAntiQuantConfig()):
+    """AntiQuantize: the same with fp32 arithmetic whatever the parameter type."""
+    return _antiquant_policy(abi.COMPUTE_F32, dst, src, scale, offset, para, policy, config)
+
+
 # ------------------------------------------------------------------------------------------ Matmul quant path
 class Matmul:
     """Host-side mirror of `Matmul<A int8, B int8, C, Bias>` on the quant path: SetTensorA/B, SetBias,

@@ -785,6 +785,141 @@ bool ranges_overlap(const void* a, size_t abytes, const void* b, size_t bbytes)
     return a0 < b0 + bbytes && b0 < a0 + abytes;
 }
 
+
+// ============================================== AscendAntiQuant PER_TOKEN / PER_GROUP (one-byte sources)
+struct AntiQuantPolicyArgs {
+    void* dst;
+    const uint8_t* src;
+    const void* scale;
+    const void* offset;
+    uint32_t rows, n;
+    int policy, along_n, has_offset, src_format;
+    uint32_t group_size, params_per_row;
+};
+
+// int8 / fp8_e4m3fn / fp8_e5m2 byte -> fp32 (exact); the 8-bit floats go through the hardware converters
+__device__ __forceinline__ float decode_b8(uint32_t word, int byte, int fmt)
+{
+    const uint32_t b = (word >> (8 * byte)) & 0xFFu;
+    if (fmt == ASCQ_QDST_I8) {
+        return static_cast<float>(static_cast<int8_t>(b));
+    }
+    return fmt == ASCQ_QDST_FP8_E5M2 ? __builtin_amdgcn_cvt_f32_bf8(static_cast<int>(b), 0)
+                                     : __builtin_amdgcn_cvt_f32_fp8(static_cast<int>(b), 0);
+}
+
+template <int kPar>
+__device__ __forceinline__ void aqp_params8(const AntiQuantPolicyArgs& a, const void* base, uint32_t i, uint32_t j,
+                                            float (&p)[8])
+{
+    if (a.policy == ASCQ_PER_GROUP && !a.along_n) {
+        load8<kPar>(base, static_cast<size_t>(i / a.group_size) * a.n + j, p);
+        return;
+    }
+    const float s = a.policy == ASCQ_PER_TOKEN
+                        ? load1<kPar>(base, i)
+                        : load1<kPar>(base, static_cast<size_t>(i) * a.params_per_row + j / a.group_size);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) p[e] = s;
+}
+
+// fp32 -> destination with the reference's saturating cast for 16-bit outputs
+template <int kDst>
+__device__ __forceinline__ float aqp_saturate(float v)
+{
+    if constexpr (kDst == ASCQ_F16) {
+        return (v != v) ? v : fminf(fmaxf(v, -65504.0f), 65504.0f);
+    } else if constexpr (kDst == ASCQ_BF16) {
+        return (v != v) ? v : fminf(fmaxf(v, -3.3895313892515355e38f), 3.3895313892515355e38f);
+    } else {
+        return v;
+    }
+}
+
+// One lane = 8 consecutive columns.  Requires n % 8 == 0, 8-byte aligned src, 16-byte aligned dst and parameters.
+template <int kPar, int kCt, int kDst>
+__global__ __launch_bounds__(kThreads) void antiquant_policy_vec_kernel(AntiQuantPolicyArgs a)
+{
+    const uint32_t j = (blockIdx.x * kThreads + threadIdx.x) * 8u;
+    if (j >= a.n) {
+        return;
+    }
+    for (uint32_t r0 = blockIdx.y * kRowsInFlight; r0 < a.rows; r0 += gridDim.y * kRowsInFlight) {
+        u32x2 raw[kRowsInFlight];
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; ++u) {
+            if (r0 + u < a.rows) {
+                raw[u] = *reinterpret_cast<const u32x2*>(a.src + static_cast<size_t>(r0 + u) * a.n + j);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; ++u) {
+            const uint32_t r = r0 + u;
+            if (r >= a.rows) {
+                break;
+            }
+            float s[8], o[8], v[8];
+            aqp_params8<kPar>(a, a.scale, r, j, s);
+            if (a.has_offset) {
+                aqp_params8<kPar>(a, a.offset, r, j, o);
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                float t = decode_b8(raw[u][e >> 2], e & 3, a.src_format);  // exact in every compute type
+                if (a.has_offset) {
+                    t = Fmt<kCt>::add(t, Fmt<kCt>::cvt(o[e]));
+                }
+                t = Fmt<kCt>::mul(t, Fmt<kCt>::cvt(s[e]));
+                v[e] = kCt == kDst ? t : aqp_saturate<kDst>(t);
+            }
+            store8<kDst>(a.dst, static_cast<size_t>(r) * a.n + j, v);
+        }
+    }
+}
+
+// Any shape / alignment: one element per lane.
+template <int kPar, int kCt, int kDst>
+__global__ __launch_bounds__(kThreads) void antiquant_policy_scalar_kernel(AntiQuantPolicyArgs a)
+{
+    const size_t total = static_cast<size_t>(a.rows) * a.n;
+    for (size_t e = static_cast<size_t>(blockIdx.x) * kThreads + threadIdx.x; e < total;
+         e += static_cast<size_t>(gridDim.x) * kThreads) {
+        const uint32_t i = static_cast<uint32_t>(e / a.n), j = static_cast<uint32_t>(e % a.n);
+        size_t pi;
+        if (a.policy == ASCQ_PER_TOKEN) {
+            pi = i;
+        } else if (a.along_n) {
+            pi = static_cast<size_t>(i) * a.params_per_row + j / a.group_size;
+        } else {
+            pi = static_cast<size_t>(i / a.group_size) * a.n + j;
+        }
+        float t = decode_b8(a.src[e], 0, a.src_format);
+        if (a.has_offset) {
+            t = Fmt<kCt>::add(t, Fmt<kCt>::cvt(load1<kPar>(a.offset, pi)));
+        }
+        t = Fmt<kCt>::mul(t, Fmt<kCt>::cvt(load1<kPar>(a.scale, pi)));
+        store1<kDst>(a.dst, e, kCt == kDst ? t : aqp_saturate<kDst>(t));
+    }
+}
+
+template <int kPar, int kCt, int kDst>
+int launch_antiquant_policy(const AntiQuantPolicyArgs& a, bool vec, hipStream_t st)
+{
+    if (vec) {
+        dim3 grid((a.n / 8 + kThreads - 1) / kThreads, 1);
+        const uint32_t row_groups = (a.rows + kRowsInFlight - 1) / kRowsInFlight;
+        const uint32_t want = (8192u + grid.x - 1) / grid.x;
+        grid.y = row_groups < want ? row_groups : want;
+        if (grid.y > 65535u) grid.y = 65535u;
+        antiquant_policy_vec_kernel<kPar, kCt, kDst><<<grid, kThreads, 0, st>>>(a);
+    } else {
+        size_t blocks = (static_cast<size_t>(a.rows) * a.n + kThreads - 1) / kThreads;
+        if (blocks > 65536) blocks = 65536;
+        antiquant_policy_scalar_kernel<kPar, kCt, kDst><<<static_cast<uint32_t>(blocks), kThreads, 0, st>>>(a);
+    }
+    return launch_status("ascq_antiquant_policy");
+}
+
 }  // namespace
 }  // namespace ascq
 
@@ -1082,4 +1217,73 @@ extern "C" int ascq_antiquant(const ascq_antiquant_desc* d, void* dst, const voi
     }
     return d->dst_dtype == ASCQ_F16 ? launch_antiquant<ASCQ_I4, ASCQ_F16>(a, vec, st)
                                     : launch_antiquant<ASCQ_I4, ASCQ_BF16>(a, vec, st);
+}
+
+// ------------------------------------------------------------------------------------- ascq_antiquant_policy
+// Checks mirror the reference's (impl/adv_api/detail/quantization/antiquant/ascend_antiquant_3510_impl.h:2176-2215).
+extern "C" int ascq_antiquant_policy(const ascq_antiquant_policy_desc* d, void* dst, const void* src,
+                                     const void* scale, const void* offset, void* stream)
+{
+    ASCQ_REQUIRE(d != nullptr, ASCQ_ENULL, "ascq_antiquant_policy: desc is NULL");
+    ASCQ_REQUIRE(dst != nullptr && src != nullptr && scale != nullptr, ASCQ_ENULL,
+                 "ascq_antiquant_policy: dst / src / scale is NULL");
+    ASCQ_REQUIRE(!d->has_offset || offset != nullptr, ASCQ_ENULL, "ascq_antiquant_policy: offset tensor is NULL");
+    ASCQ_REQUIRE(d->policy == ASCQ_PER_TOKEN || d->policy == ASCQ_PER_GROUP, ASCQ_EUNSUPPORTED,
+                 "ascq_antiquant_policy: policy %d is not PER_TOKEN / PER_GROUP", d->policy);
+    ASCQ_REQUIRE(d->src_format >= ASCQ_QDST_I8 && d->src_format <= ASCQ_QDST_FP8_E5M2, ASCQ_EUNSUPPORTED,
+                 "ascq_antiquant_policy: source format %d is not int8 / fp8_e4m3fn / fp8_e5m2", d->src_format);
+    const int par = d->scale_dtype, dt = d->dst_dtype;
+    ASCQ_REQUIRE(par == ASCQ_F16 || par == ASCQ_BF16 || par == ASCQ_F32, ASCQ_EUNSUPPORTED,
+                 "ascq_antiquant_policy: scale dtype %d is not half / bfloat16 / float", par);
+    ASCQ_REQUIRE(dt == ASCQ_F16 || dt == ASCQ_BF16 || dt == ASCQ_F32, ASCQ_EUNSUPPORTED,
+                 "ascq_antiquant_policy: dst dtype %d is not half / bfloat16 / float", dt);
+    ASCQ_REQUIRE(d->compute == ASCQ_COMPUTE_SCALE_T || d->compute == ASCQ_COMPUTE_F32, ASCQ_EINVAL,
+                 "ascq_antiquant_policy: compute must be SCALE_T or F32");
+    const int ct = d->compute == ASCQ_COMPUTE_F32 ? ASCQ_F32 : par;
+    ASCQ_REQUIRE(ct == ASCQ_F32 || dt == ct, ASCQ_EUNSUPPORTED,
+                 "ascq_antiquant_policy: with %s arithmetic the output has the same type (dst dtype %d)",
+                 ct == ASCQ_F16 ? "half" : "bfloat16", dt);
+    ASCQ_REQUIRE(d->n > 0, ASCQ_EINVAL, "ascq_antiquant_policy: n must be greater than 0");
+    ASCQ_REQUIRE(d->cal_count % d->n == 0, ASCQ_EINVAL,
+                 "ascq_antiquant_policy: calCount %u must be an integer multiple of n %u", d->cal_count, d->n);
+    ASCQ_REQUIRE(static_cast<uint64_t>(d->m) * d->n >= d->cal_count, ASCQ_EINVAL,
+                 "ascq_antiquant_policy: calCount %u exceeds m*n = %u*%u", d->cal_count, d->m, d->n);
+    ASCQ_REQUIRE(d->n % 32 == 0, ASCQ_EALIGN, "ascq_antiquant_policy: a row of n=%u bytes must be a multiple of 32 bytes",
+                 d->n);
+    int along_n = 1;
+    uint32_t ppr = 0;
+    if (d->policy == ASCQ_PER_GROUP) {
+        ASCQ_REQUIRE(d->k_dim == 0 || d->k_dim == 1, ASCQ_EINVAL, "ascq_antiquant_policy: kDim must be 0 or 1");
+        ASCQ_REQUIRE(d->group_size > 0 && d->group_size % 32 == 0, ASCQ_EINVAL,
+                     "ascq_antiquant_policy: groupSize %u must be a positive multiple of 32", d->group_size);
+        along_n = (d->k_dim == 1) != (d->is_transpose != 0) ? 1 : 0;
+        ppr = (d->n + d->group_size - 1) / d->group_size;
+    }
+    if (d->cal_count == 0) {
+        return ASCQ_OK;
+    }
+    ASCQ_REQUIRE(!ranges_overlap(dst, static_cast<size_t>(d->cal_count) * dtype_size(dt), src, d->cal_count),
+                 ASCQ_EINVAL, "ascq_antiquant_policy: dst overlaps src");
+    AntiQuantPolicyArgs a{dst, static_cast<const uint8_t*>(src), scale, offset, d->cal_count / d->n, d->n, d->policy,
+                          along_n, d->has_offset ? 1 : 0, d->src_format, d->group_size ? d->group_size : 1u, ppr};
+    const bool vec = (reinterpret_cast<uintptr_t>(src) & 7u) == 0 && aligned16(dst) && aligned16(scale) &&
+                     (!d->has_offset || aligned16(offset));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+#define ASCQ_AQP(P, C, D)                                         \
+    if (par == (P) && ct == (C) && dt == (D)) {                   \
+        return launch_antiquant_policy<P, C, D>(a, vec, st);      \
+    }
+    ASCQ_AQP(ASCQ_F16, ASCQ_F16, ASCQ_F16)
+    ASCQ_AQP(ASCQ_BF16, ASCQ_BF16, ASCQ_BF16)
+    ASCQ_AQP(ASCQ_F32, ASCQ_F32, ASCQ_F32)
+    ASCQ_AQP(ASCQ_F32, ASCQ_F32, ASCQ_F16)
+    ASCQ_AQP(ASCQ_F32, ASCQ_F32, ASCQ_BF16)
+    ASCQ_AQP(ASCQ_F16, ASCQ_F32, ASCQ_F32)
+    ASCQ_AQP(ASCQ_F16, ASCQ_F32, ASCQ_F16)
+    ASCQ_AQP(ASCQ_F16, ASCQ_F32, ASCQ_BF16)
+    ASCQ_AQP(ASCQ_BF16, ASCQ_F32, ASCQ_F32)
+    ASCQ_AQP(ASCQ_BF16, ASCQ_F32, ASCQ_F16)
+    ASCQ_AQP(ASCQ_BF16, ASCQ_F32, ASCQ_BF16)
+#undef ASCQ_AQP
+    return fail(ASCQ_EUNSUPPORTED, "ascq_antiquant_policy: no kernel for scale %d, compute %d, dst %d", par, ct, dt);
 }

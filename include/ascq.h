@@ -189,6 +189,38 @@ typedef struct ascq_antiquant_desc {
 int ascq_antiquant(const ascq_antiquant_desc* desc, void* dst, const void* src, const void* offset, const void* scale,
                    void* stream);
 
+/*
+ * AscendAntiQuant<dstT, srcT, scaleT, config, policy> for PER_TOKEN / PER_GROUP, and AntiQuantize
+ * (ref: include/adv_api/quantization/ascend_antiquant.h, the AscendAntiQuantParam overloads;
+ *  impl/adv_api/detail/quantization/antiquant/ascend_antiquant_3510_impl.h:1386-1403 (source conversion),
+ *  :1458-1495 (per token), :2170-2222 (dispatch); type table docs/zh/api/SIMD-API/高阶API/量化操作/AscendAntiQuant.md 表3).
+ * src [m, n] one byte per element: int8, fp8_e4m3fn or fp8_e5m2 (src_format, an ascq_quant_dst value);
+ * dst [m, n] of dst_dtype; only the first cal_count elements (a multiple of n) are processed.
+ *   PER_TOKEN: scale / offset [m].
+ *   PER_GROUP: the group axis is k_dim XOR is_transpose: 1 = along n, parameters [m, ceil(n / group_size)];
+ *              0 = along m, parameters [ceil(m / group_size), n].  The data stay [m, n] row-major either way.
+ *   v = ct(src) ; v = ct(v + offset) if has_offset ; v = ct(v * scale) ; dst = dstT(v)
+ * with ct = the scale dtype (ASCQ_COMPUTE_SCALE_T: AscendAntiQuant) or fp32 (ASCQ_COMPUTE_F32: AntiQuantize); every
+ * source value is exact in every ct.  A 16-bit ct requires dst_dtype == scale_dtype; an fp32 result is rounded
+ * half-even to a 16-bit dst, saturating at the largest finite value.
+ */
+typedef struct ascq_antiquant_policy_desc {
+    int32_t policy;      /* ASCQ_PER_TOKEN | ASCQ_PER_GROUP */
+    int32_t src_format;  /* ASCQ_QDST_I8 | ASCQ_QDST_FP8_E4M3FN | ASCQ_QDST_FP8_E5M2 */
+    int32_t scale_dtype; /* ASCQ_F16 | ASCQ_BF16 | ASCQ_F32: dtype of the scale / offset tensors */
+    int32_t dst_dtype;   /* ASCQ_F16 | ASCQ_BF16 | ASCQ_F32 */
+    int32_t compute;     /* ASCQ_COMPUTE_SCALE_T | ASCQ_COMPUTE_F32 */
+    int32_t has_offset;
+    int32_t is_transpose;
+    int32_t k_dim;       /* PER_GROUP: AscendAntiQuantConfig::kDim */
+    uint32_t m, n;
+    uint32_t cal_count;
+    uint32_t group_size; /* PER_GROUP: positive multiple of 32 */
+} ascq_antiquant_policy_desc;
+
+int ascq_antiquant_policy(const ascq_antiquant_policy_desc* desc, void* dst, const void* src, const void* scale,
+                          const void* offset, void* stream);
+
 /* ------------------------------------------------- Matmul int8 quant path */
 typedef enum ascq_mm_quant_mode {
     ASCQ_MM_QUANT_NONE = 0,   /* int32 out */

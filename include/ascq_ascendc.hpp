@@ -269,6 +269,45 @@ void AscendDequant(const DeviceTensor<dstT>& dstTensor, const DeviceTensor<int32
     Check(ascq_dequant(&d, dstTensor.GetPhyAddr(), srcTensor.GetPhyAddr(), nullptr, stream));
 }
 
+// AscendAntiQuant<dstT, srcT, scaleT, config, policy> for PER_TOKEN / PER_GROUP (ref: ascend_antiquant.h, the
+// AscendAntiQuantParam overloads; ascend_antiquant_common.h:45-65): srcT int8_t / fp8_e4m3fn_t / fp8_e5m2_t, the
+// arithmetic in scaleT.  config and policy are ordinary arguments here.
+struct AscendAntiQuantConfig {
+    bool hasOffset = false;
+    bool isTranspose = false;
+    int32_t kDim = 1;
+};
+struct AscendAntiQuantParam {
+    uint32_t m;
+    uint32_t n;
+    uint32_t calCount;
+    uint32_t groupSize = 0;
+};
+enum class AscendAntiQuantPolicy : int32_t { PER_TENSOR, PER_CHANNEL, PER_TOKEN, PER_GROUP };
+
+template <typename dstT, typename srcT, typename scaleT>
+void AscendAntiQuant(const DeviceTensor<dstT>& dstTensor, const DeviceTensor<srcT>& srcTensor,
+                     const DeviceTensor<scaleT>& scaleTensor, const DeviceTensor<scaleT>& offsetTensor,
+                     const AscendAntiQuantParam& para, const AscendAntiQuantConfig& config,
+                     AscendAntiQuantPolicy policy, void* stream = nullptr)
+{
+    ascq_antiquant_policy_desc d{};
+    d.policy = static_cast<int32_t>(policy);
+    d.src_format = QuantDstOf<srcT>::value;
+    d.scale_dtype = DTypeOf<scaleT>::value;
+    d.dst_dtype = DTypeOf<dstT>::value;
+    d.compute = ASCQ_COMPUTE_SCALE_T;
+    d.has_offset = config.hasOffset ? 1 : 0;
+    d.is_transpose = config.isTranspose ? 1 : 0;
+    d.k_dim = config.kDim;
+    d.m = para.m;
+    d.n = para.n;
+    d.cal_count = para.calCount;
+    d.group_size = para.groupSize;
+    Check(ascq_antiquant_policy(&d, dstTensor.GetPhyAddr(), srcTensor.GetPhyAddr(), scaleTensor.GetPhyAddr(),
+                                config.hasOffset ? offsetTensor.GetPhyAddr() : nullptr, stream));
+}
+
 // ref: include/adv_api/quantization/ascend_antiquant_utils.h:27-32
 struct AntiQuantShapeInfo {
     uint32_t offsetHeight{0};

@@ -752,6 +752,91 @@ int orc_matmul_w4a16_cols(const ascq_w4a16_desc* d, uint16_t* y, const uint16_t*
     return 0;
 }
 
+/* ------------------------------------- AscendAntiQuant PER_TOKEN / PER_GROUP */
+/* One-byte sources (int8, fp8_e4m3fn, fp8_e5m2): the source is converted to the compute type (exact for every source
+ * value), the offset is added and the scale multiplied in that type, one rounding each; an fp32 result going to a
+ * 16-bit destination is rounded half-even and saturates (LayoutZMrgZRndRSatS).
+ * ref: impl/adv_api/detail/quantization/antiquant/ascend_antiquant_3510_impl.h:1386-1403 (ConvertSrc),
+ *      :1458-1495 (per token), :2176-2222 (group axis = kDim XOR isTranspose); fp32 arithmetic for AntiQuantize. */
+static uint16_t f32_to_f16_sat(float v)
+{
+    if (v == v && v > 65504.0f) {
+        v = 65504.0f;
+    }
+    if (v == v && v < -65504.0f) {
+        v = -65504.0f;
+    }
+    return orc_f32_to_f16(v);
+}
+
+static uint16_t f32_to_bf16_sat(float v)
+{
+    const float top = 3.3895313892515355e38f; /* largest finite bfloat16 */
+    if (v == v && v > top) {
+        v = top;
+    }
+    if (v == v && v < -top) {
+        v = -top;
+    }
+    return orc_f32_to_bf16(v);
+}
+
+int orc_antiquant_policy(const ascq_antiquant_policy_desc* d, void* dst, const uint8_t* src, const void* scale,
+                         const void* offset)
+{
+    size_t n = d->n, rows = n ? d->cal_count / n : 0;
+    int along_n = (d->k_dim == 1) != (d->is_transpose != 0);
+    size_t ppr = d->group_size ? (n + d->group_size - 1) / d->group_size : 0;
+    int ct = d->compute == ASCQ_COMPUTE_F32 ? ASCQ_F32 : d->scale_dtype;
+#pragma omp parallel for schedule(static) if (rows * n > 65536)
+    for (size_t i = 0; i < rows; ++i) {
+        for (size_t j = 0; j < n; ++j) {
+            size_t e = i * n + j, pi;
+            if (d->policy == ASCQ_PER_TOKEN) {
+                pi = i;
+            } else if (along_n) {
+                pi = i * ppr + j / d->group_size;
+            } else {
+                pi = (i / d->group_size) * n + j;
+            }
+            float x = d->src_format == ASCQ_QDST_I8 ? (float)(int8_t)src[e]
+                                                    : orc_fp8_to_f32(src[e], d->src_format == ASCQ_QDST_FP8_E5M2);
+            float s = load_as_f32(scale, pi, d->scale_dtype);
+            float o = d->has_offset ? load_as_f32(offset, pi, d->scale_dtype) : 0.0f;
+            float v;
+            if (ct == ASCQ_F16) {
+                uint16_t t = orc_f32_to_f16(x);
+                if (d->has_offset) {
+                    t = orc_f16_add(t, orc_f32_to_f16(o));
+                }
+                v = orc_f16_to_f32(orc_f16_mul(t, orc_f32_to_f16(s)));
+            } else if (ct == ASCQ_BF16) {
+                uint16_t t = orc_f32_to_bf16(x);
+                if (d->has_offset) {
+                    t = orc_bf16_add(t, orc_f32_to_bf16(o));
+                }
+                v = orc_bf16_to_f32(orc_bf16_mul(t, orc_f32_to_bf16(s)));
+            } else {
+                volatile float t = x;
+                if (d->has_offset) {
+                    volatile float t2 = t + o;
+                    t = t2;
+                }
+                volatile float t3 = t * s;
+                v = t3;
+            }
+            if (d->dst_dtype == ASCQ_F32) {
+                ((float*)dst)[e] = v;
+            } else if (d->dst_dtype == ASCQ_F16) {
+                ((uint16_t*)dst)[e] = ct == ASCQ_F16 ? orc_f32_to_f16(v) : f32_to_f16_sat(v);
+            } else {
+                ((uint16_t*)dst)[e] = ct == ASCQ_BF16 ? orc_f32_to_bf16(v) : f32_to_bf16_sat(v);
+            }
+        }
+    }
+    return 0;
+}
+
 /* ------------------------------------------------------------------- W8A16 */
 /* Matmul with A half and B int8 that is de-quantised on the way in: B goes through AscendAntiQuant<int8_t, half>
  * (half math: f16(w) + offset, then * scale, one rounding each;

@@ -44,6 +44,8 @@ int orc_matmul_w4a16(const ascq_w4a16_desc* d, uint16_t* y, const uint16_t* x, c
                      const uint16_t* scale, const uint16_t* offset);
 int orc_matmul_w4a16_cols(const ascq_w4a16_desc* d, uint16_t* y, const uint16_t* x, const uint8_t* w,
                           const uint16_t* scale, const uint16_t* offset, uint32_t j0, uint32_t j1);
+int orc_antiquant_policy(const ascq_antiquant_policy_desc* d, void* dst, const uint8_t* src, const void* scale,
+                         const void* offset);
 int orc_matmul_w8a16(const ascq_w8a16_desc* d, void* y, const uint16_t* x, const int8_t* w, const uint16_t* offset,
                      const uint16_t* scale);
 

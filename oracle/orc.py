@@ -58,6 +58,7 @@ def lib():
         L.orc_matmul_w4a16.argtypes = [C.POINTER(abi.W4A16Desc), _P, _P, _P, _P, _P]
         L.orc_matmul_w4a16_cols.argtypes = [C.POINTER(abi.W4A16Desc), _P, _P, _P, _P, _P, C.c_uint32, C.c_uint32]
         L.orc_matmul_w8a16.argtypes = [C.POINTER(abi.W8A16Desc), _P, _P, _P, _P, _P]
+        L.orc_antiquant_policy.argtypes = [C.POINTER(abi.AntiQuantPolicyDesc), _P, _P, _P, _P]
         for name in ("orc_f32_to_f16_array", "orc_f16_to_f32_array", "orc_f32_to_bf16_array"):
             getattr(L, name).argtypes = [_P, _P, C.c_size_t]
         for name in ("orc_f16_mul_array", "orc_f16_add_array"):
@@ -204,3 +205,11 @@ def matmul_w8a16(desc, x, w, offset=None, scale=None):
     y = np.zeros((desc.m, desc.n), dtype=_NP[desc.out_dtype])
     lib().orc_matmul_w8a16(C.byref(desc), _ptr(y), _ptr(x), _ptr(w), _ptr(offset), _ptr(scale))
     return y
+
+
+def antiquant_policy(desc, src, scale, offset=None):
+    """src: uint8 / int8 array [m, n] (raw bytes of the one-byte source format)."""
+    dst = np.zeros((desc.m, desc.n), dtype=_NP[desc.dst_dtype])
+    lib().orc_antiquant_policy(C.byref(desc), _ptr(dst), _ptr(src), _ptr(scale), _ptr(offset))
+    return dst
+

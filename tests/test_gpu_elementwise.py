@@ -295,6 +295,54 @@ def test_antiquant(int4, dst_dt, transpose, K, N, G, has_offset):
     assert np.array_equal(bits(dst), want.view(np.uint16))
 
 
+# ------------------------------------------------------------------ AscendAntiQuant PER_TOKEN / PER_GROUP
+B8 = {abi.QDST_I8: torch.int8, abi.QDST_FP8_E4M3FN: torch.float8_e4m3fn, abi.QDST_FP8_E5M2: torch.float8_e5m2}
+AQP_TYPES = [(abi.F16, abi.F16, abi.COMPUTE_SCALE_T), (abi.BF16, abi.BF16, abi.COMPUTE_SCALE_T),
+             (abi.F32, abi.F32, abi.COMPUTE_SCALE_T), (abi.F32, abi.F16, abi.COMPUTE_SCALE_T),
+             (abi.F32, abi.BF16, abi.COMPUTE_SCALE_T), (abi.F16, abi.F16, abi.COMPUTE_F32),
+             (abi.BF16, abi.F32, abi.COMPUTE_F32)]                     # (scale, dst, arithmetic)
+
+
+@pytest.mark.parametrize("fmt", [abi.QDST_I8, abi.QDST_FP8_E4M3FN, abi.QDST_FP8_E5M2])
+@pytest.mark.parametrize("types", AQP_TYPES)
+@pytest.mark.parametrize("mode", ["token", "group_n", "group_m", "group_m_via_transpose"])
+def test_antiquant_policy(fmt, types, mode):
+    """Every source code of the one-byte formats (NaN / infinity codes aside), every legal type combination, both
+    group axes: bit-exact against the oracle."""
+    sc_dt, dst_dt, compute = types
+    for (m, n, cal, has_offset) in [(64, 256, 64 * 256, True), (40, 96, 32 * 96, False), (33, 2080, 33 * 2080, True)]:
+        announce("antiquant policy", fmt, types, mode, m, n, cal)
+        rng = np.random.default_rng(m + n + fmt)
+        codes = rng.integers(0, 256, (m, n)).astype(np.uint8)
+        codes.reshape(-1)[:256] = np.arange(256, dtype=np.uint8)          # every code at least once
+        if fmt == abi.QDST_FP8_E4M3FN:
+            codes[(codes & 0x7F) == 0x7F] = 0x3C
+        elif fmt == abi.QDST_FP8_E5M2:
+            codes[(codes & 0x7F) >= 0x7C] = 0x3C
+        gs = 32
+        policy = abi.PER_TOKEN if mode == "token" else abi.PER_GROUP
+        k_dim, tr = {"token": (1, 0), "group_n": (1, 0), "group_m": (0, 0), "group_m_via_transpose": (1, 1)}[mode]
+        pshape = {"token": (m,), "group_n": (m, -(-n // gs))}.get(mode, (-(-m // gs), n))
+        (s, sdev), (o, odev) = typed(rng.uniform(0.01, 2.0, pshape), sc_dt), typed(rng.uniform(-3, 3, pshape), sc_dt)
+        dst = torch.zeros((m, n), dtype=TDT[dst_dt], device=DEV)
+        cfg = ops.AscendAntiQuantConfig(has_offset=has_offset, is_transpose=bool(tr), k_dim=k_dim)
+        para = ops.AscendAntiQuantParam(m=m, n=n, cal_count=cal, group_size=gs if policy == abi.PER_GROUP else 0)
+        fn = ops.ascend_antiquant_policy if compute == abi.COMPUTE_SCALE_T else ops.antiquantize
+        fn(dst, to_dev(codes).view(B8[fmt]), sdev, odev, para, policy, cfg)
+        d = abi.AntiQuantPolicyDesc(policy=policy, src_format=fmt, scale_dtype=sc_dt, dst_dtype=dst_dt, compute=compute,
+                                    has_offset=int(has_offset), is_transpose=tr, k_dim=k_dim, m=m, n=n, cal_count=cal,
+                                    group_size=para.group_size)
+        want = orc.antiquant_policy(d, codes, s, o)
+        got = bits(dst)
+        want = want.view(np.uint16) if want.dtype == np.float16 else want
+        rows = cal // n
+        if dst_dt == abi.F32:
+            assert np.array_equal(got[:rows].view(np.uint32), want[:rows].view(np.uint32))
+        else:
+            assert np.array_equal(got[:rows], want[:rows])
+        assert not got[rows:].any()
+
+
 def test_antiquant_per_tensor():
     announce("antiquant per-tensor")
     w = np.arange(-128, 128, dtype=np.int8).reshape(8, 32)

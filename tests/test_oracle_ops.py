@@ -505,3 +505,65 @@ def test_quant_fp8_is_fp32_arithmetic_then_one_conversion(fmt, tdt, top, sc_dt):
                           round_mode=abi.CAST_FLOOR, offset_kind=abi.OFFSET_TENSOR, k_dim=1, m=m, n=n, cal_count=m * n,
                           dst_format=fmt)
         assert np.array_equal(orc.quant(d, x, s, o).view(np.uint8), want)
+
+
+# ------------------------------------------------------------------ AscendAntiQuant PER_TOKEN / PER_GROUP
+def _b8_source(rng, fmt, shape):
+    """Random one-byte sources (no NaN / infinity codes) and their exact fp32 values."""
+    codes = rng.integers(0, 256, shape).astype(np.uint8)
+    if fmt == abi.QDST_I8:
+        return codes, codes.view(np.int8).astype(np.float32)
+    if fmt == abi.QDST_FP8_E4M3FN:
+        codes[(codes & 0x7F) == 0x7F] = 0x3C
+        return codes, torch.from_numpy(codes).view(torch.float8_e4m3fn).float().numpy()
+    codes[(codes & 0x7F) >= 0x7C] = 0x3C
+    return codes, torch.from_numpy(codes).view(torch.float8_e5m2).float().numpy()
+
+
+@pytest.mark.filterwarnings("ignore:overflow encountered")      # half arithmetic on the largest e5m2 values overflows
+@pytest.mark.parametrize("fmt", [abi.QDST_I8, abi.QDST_FP8_E4M3FN, abi.QDST_FP8_E5M2])
+@pytest.mark.parametrize("mode", ["token", "group_n", "group_m", "group_n_via_transpose"])
+def test_antiquant_policy_against_numpy_and_torch_arithmetic(fmt, mode):
+    """(src + offset) * scale in the scale's type: numpy float16 arithmetic, torch bfloat16 arithmetic (both round
+    once per operation) and numpy float32 arithmetic are the independent implementations; the group axis is
+    kDim XOR isTranspose (ascend_antiquant_3510_impl.h:2204-2212)."""
+    rng = np.random.default_rng(31 + fmt)
+    m, n, gs = 64, 96, 32
+    codes, x = _b8_source(rng, fmt, (m, n))
+    policy = abi.PER_TOKEN if mode == "token" else abi.PER_GROUP
+    k_dim, tr = {"token": (1, 0), "group_n": (1, 0), "group_m": (0, 0), "group_n_via_transpose": (0, 1)}[mode]
+    if mode == "token":
+        pshape, expand = (m,), lambda p: p[:, None]
+    elif mode == "group_m":
+        pshape, expand = (m // gs, n), lambda p: np.repeat(p, gs, axis=0)
+    else:
+        pshape, expand = (m, n // gs), lambda p: np.repeat(p, gs, axis=1)
+    s32 = rng.uniform(0.01, 2.0, pshape).astype(np.float32)
+    o32 = rng.uniform(-3.0, 3.0, pshape).astype(np.float32)
+
+    def desc(sc_dt, dst_dt, compute):
+        return abi.AntiQuantPolicyDesc(policy=policy, src_format=fmt, scale_dtype=sc_dt, dst_dtype=dst_dt,
+                                       compute=compute, has_offset=1, is_transpose=tr, k_dim=k_dim, m=m, n=n,
+                                       cal_count=m * n, group_size=gs if policy == abi.PER_GROUP else 0)
+
+    # half arithmetic
+    s16, o16 = s32.astype(np.float16), o32.astype(np.float16)
+    want = ((x.astype(np.float16) + expand(o16)).astype(np.float16) * expand(s16)).astype(np.float16)
+    got = orc.antiquant_policy(desc(abi.F16, abi.F16, abi.COMPUTE_SCALE_T), codes, s16, o16)
+    assert np.array_equal(got.view(U16), want.view(U16))
+    # bfloat16 arithmetic
+    sb, ob = torch.from_numpy(s32).bfloat16(), torch.from_numpy(o32).bfloat16()
+    tb = (torch.from_numpy(x).bfloat16() + torch.from_numpy(expand(ob.float().numpy())).bfloat16())
+    wantb = (tb * torch.from_numpy(expand(sb.float().numpy())).bfloat16()).view(torch.int16).numpy().view(U16)
+    gotb = orc.antiquant_policy(desc(abi.BF16, abi.BF16, abi.COMPUTE_SCALE_T), codes,
+                                sb.view(torch.int16).numpy().view(U16), ob.view(torch.int16).numpy().view(U16))
+    assert np.array_equal(gotb.view(U16), wantb)
+    # fp32 arithmetic, fp32 and half outputs; and AntiQuantize (fp32 arithmetic on half parameters)
+    want32 = (x + expand(o32)) * expand(s32)
+    assert np.array_equal(orc.antiquant_policy(desc(abi.F32, abi.F32, abi.COMPUTE_SCALE_T), codes, s32, o32), want32)
+    got16 = orc.antiquant_policy(desc(abi.F32, abi.F16, abi.COMPUTE_SCALE_T), codes, s32, o32)
+    sat = lambda v: np.clip(v, -65504.0, 65504.0).astype(np.float16)   # the fp32 -> half cast saturates (RndR SatS)
+    assert np.array_equal(got16.view(U16), sat(want32).view(U16))
+    wantq = sat((x + expand(o16).astype(np.float32)) * expand(s16).astype(np.float32))
+    gotq = orc.antiquant_policy(desc(abi.F16, abi.F16, abi.COMPUTE_F32), codes, s16, o16)
+    assert np.array_equal(gotq.view(U16), wantq.view(U16))
