@@ -163,6 +163,23 @@ def main():
         return {"ms_per_step": ms, "kernel_ms": kern_ms, "gbs": bytes_ / (kern_ms * 1e-3) / 1e9, "bytes": bytes_,
                 "tops": 2.0 * M * K * N / (kern_ms * 1e-3) / 1e12, "tensors": (xs, ws[0], sc[0], of[0])}
 
+    # ------------------------------------------------------------------ W8A16 decode (Matmul anti-quant path)
+    def w8a16(M, steps, warmup, sets=3):
+        K, N = 8192, 28672
+        xs = torch.randn((M, K), device=dev, generator=gen).to(torch.float16)
+        ws = [rand_i8(K, N) for _ in range(sets)]
+        sc = [(torch.rand((N,), device=dev, generator=gen) * 9e-3 + 1e-3).to(torch.float16) for _ in range(sets)]
+        of = [(torch.rand((N,), device=dev, generator=gen) * 18 - 9).to(torch.float16) for _ in range(sets)]
+        y = torch.empty((M, N), dtype=torch.float16, device=dev)
+
+        def step(i, starts, stops):
+            j = i % sets
+            bracket(starts, stops, lambda: ops.matmul_w8a16(y, xs, ws[j], of[j], sc[j]))
+
+        ms, kern_ms = timed(step, steps, warmup)
+        bytes_ = K * N + 2 * N * 2 + M * K * 2 + M * N * 2
+        return {"ms_per_step": ms, "kernel_ms": kern_ms, "gbs": bytes_ / (kern_ms * 1e-3) / 1e9, "bytes": bytes_}
+
     # ------------------------------------------------------------------ elementwise (config 2)
     def quant2a(steps, warmup, sets=3):
         m, n = 8192, 4096
@@ -302,6 +319,11 @@ def main():
         for M in (4, 16):
             r = strip(w4a16(M, s2, w2))
             others[f"w4a16_m{M}"] = {"kernel_ms": r["kernel_ms"], "gbs": r["gbs"], "hbm_frac": r["gbs"] / PEAK_HBM_GBS}
+            torch.cuda.empty_cache()
+        for M in (1, 16):
+            r = w8a16(M, s2, w2)
+            others[f"w8a16_m{M}_k8192_n28672"] = {"kernel_ms": r["kernel_ms"], "gbs": r["gbs"], "bytes": r["bytes"],
+                                                  "hbm_frac": r["gbs"] / PEAK_HBM_GBS}
             torch.cuda.empty_cache()
         r = group5(max(5, args.steps // 5), 2)
         r["mfma_frac"] = r["tops"] / PEAK_INT8_TOPS
