@@ -1,5 +1,7 @@
-// W4A16 weight-only linear for decode: y[m, n] = sum_k x[m, k] * antiquant(w[k, n]) with int4 weights de-quantised in
-// registers (never materialised in memory).
+// Weight-only linears for decode: y[m, n] = sum_k x[m, k] * antiquant(w[k, n]) with int4 (W4A16, per-group
+// parameters) or int8 (W8A16, per-channel / per-tensor parameters: the Matmul anti-quant path) weights de-quantised in
+// registers, never materialised in memory.  The description below is the int4 kernels'; the int8 kernel at the end of
+// the file follows the same design.
 //
 // The kernel is bound by the HBM read of the packed weights (k * n / 2 bytes), so it is built as a set of independent
 // streams, one per wavefront, each with its own deep queue of loads:
@@ -428,8 +430,8 @@ __global__ __launch_bounds__(kThreads) void w4a16_tile_kernel(WnParams p)
     }
 }
 
-// Up to four activation rows (MP = 1 or 2 row pairs; the decode GEMV): the same streams, two per SIMD.  To fit 8 rings into the LDS the
-// ring has two stages and holds only the weights (8 KiB) and the activations (256 bytes); the scale / offset rows of
+// Up to four activation rows (MP = 1 or 2 row pairs; the decode GEMV): the same streams, two per SIMD.  To fit 8
+// rings into the LDS the ring has two stages and holds only the weights (8 KiB) and the activations (256 bytes); the scale / offset rows of
 // a quantisation group are fetched into registers when a chunk opens a new group, ahead of that chunk's weights, so
 // they have landed whenever the weights have.  With two stages one chunk is in flight behind the one being computed
 // and the wait before a chunk is simply for everything outstanding; the second wavefront of the SIMD fills the time
