@@ -5,7 +5,7 @@ Headline (the `value` of the JSON line): the W8A8 LLM linear at M=2048, K=4096, 
 per-token quantisation of the bf16 activations + the int8 MFMA GEMM with the fused dequant epilogue to bf16 - reported
 as int8 TOPS (2*M*K*N per step).  The same line carries the roofline of the dominant kernel (the GEMM, timed alone with
 events on the launch stream), the CPU baseline (the oracle, timed on the host cores), the W4A16 decode GEMV as HBM GB/s
-and, unless --quick, the other BASELINE workloads (elementwise ops, small-M linears, W4A16 M=4/16, the MoE grouped
+and, unless --quick, the other workloads of the path (elementwise ops, small-M linears, W4A16 M=4/16, the MoE grouped
 matmul) under "others".
 
 Inputs are synthetic, seeded and resident in HBM before the timed region.  Memory-bound workloads rotate among
@@ -45,8 +45,9 @@ def main():
                          "FETCH_SIZE / WRITE_SIZE counters when this command runs under rocprofv3 --pmc")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build measures one GPU; run it with --gpus 1 (the path shards without communication, "
-              "see DESIGN.md).", file=sys.stderr)
+        print("bench.py: this build measures one GPU; run it with --gpus 1 (the path shards over output columns, rows "
+              "or experts without any communication, so N GPUs are N independent copies of this run).",
+              file=sys.stderr)
         sys.exit(2)
 
     import numpy as np
