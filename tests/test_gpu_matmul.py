@@ -409,3 +409,44 @@ def test_group_matmul_example_full_size_nz_equals_nd():
         v = (x[r].astype(np.float64) @ w[g].astype(np.float64)) * sc[g].astype(np.float64) * float(ts[r])
         gold = v / (1.0 + np.exp(-1.702 * v))                       # the example's FastGelu, in closed form
         assert np.all(np.abs(got[i] - gold) <= 2e-3 * np.abs(gold) + 1e-6)
+
+# ------------------------------------------------------------------ workspace contract, determinism
+@pytest.mark.parametrize("m", [1, 5, 16, 19, 130])
+def test_workspaces_need_no_initialisation_and_results_repeat(m):
+    """The scratch of the weight-stream and split-K paths may hold anything (here: all-ones bytes = NaN / -1) and two
+    calls give the same bits."""
+    announce("workspace garbage", m)
+    rng = np.random.default_rng(0x5C + m)
+    k, n = 1024, 1056
+    # W8A8 (stream kernel for m <= 32, split-K tiles above)
+    a = rng.integers(-127, 128, (m, k)).astype(np.int8)
+    w = rng.integers(-127, 128, (k, n)).astype(np.int8)
+    cs = rng.uniform(1e-4, 1e-2, n).astype(np.float32)
+    mm = ops.Matmul(m, n, k)
+    mm.set_tensor_a(to_dev(a))
+    mm.set_tensor_b(to_dev(w))
+    mm.set_quant_vector(to_dev(cs))
+    c1 = torch.zeros((m, n), dtype=torch.bfloat16, device=DEV)
+    mm.iterate_all(c1)
+    if mm._ws is not None:
+        mm._ws.fill_(-1)
+    c2 = torch.zeros((m, n), dtype=torch.bfloat16, device=DEV)
+    mm.iterate_all(c2)
+    d = abi.MatmulDesc(m=m, n=n, k=k, out_dtype=abi.BF16, quant_mode=abi.MM_QUANT_VECTOR, scale_format=abi.MM_SCALE_F32)
+    want = orc.matmul_w8a8(d, a, w, None, cs, None)
+    assert np.array_equal(bits(c1), want) and np.array_equal(bits(c2), want)
+    # W4A16 and W8A16
+    x = rng.standard_normal((m, k)).astype(np.float16)
+    xw, wp, sc, of = w4_case(rng, m, k, n, 128, True)
+    garbage = torch.full((1 << 22,), float("nan"), dtype=torch.float32, device=DEV)
+    outs = []
+    for ws in (None, garbage, garbage):
+        y4 = torch.zeros((m, n), dtype=torch.float16, device=DEV)
+        ops.matmul_w4a16(y4, to_dev(xw), to_dev(wp), to_dev(sc), to_dev(of), 128, workspace=ws)
+        y8 = torch.zeros((m, n), dtype=torch.float16, device=DEV)
+        ops.matmul_w8a16(y8, to_dev(x), to_dev(w), to_dev(of[0]), to_dev(sc[0]), workspace=ws)
+        outs.append((bits(y4), bits(y8)))
+        garbage.fill_(float("nan"))
+    for y4, y8 in outs[1:]:
+        assert np.array_equal(y4, outs[0][0]) and np.array_equal(y8, outs[0][1])
+    assert not np.isnan(outs[0][0].view(np.float16)).any() and not np.isnan(outs[0][1].view(np.float16)).any()
