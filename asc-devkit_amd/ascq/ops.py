@@ -287,6 +287,31 @@ class Matmul:
         return c
 
 
+_lin_ws = {}
+
+
+def linear_w8a8_dynamic(c, x, weight, channel_scale, bias=None, activation=abi.MM_ACT_NONE, trans_b=False):
+    """c = dequant(dynamic_quant_per_token(x) @ weight): the activation quantiser and the int8 matmul in one call, with
+    the results of calling the two one after the other.  x half / bfloat16 / float32 [m, k]; weight int8 [k, n];
+    channel_scale float32 [n]; bias float32 / bfloat16 [n] (added after dequantisation)."""
+    m, k = x.shape
+    n = c.shape[1]
+    d = abi.MatmulDesc(m=m, n=n, k=k, trans_b=int(trans_b), out_dtype=_dt(c), quant_mode=abi.MM_QUANT_VECTOR,
+                       scale_format=abi.MM_SCALE_F32, activation=activation)
+    if bias is not None:
+        d.bias_kind = abi.MM_BIAS_F32_POST if bias.dtype == torch.float32 else abi.MM_BIAS_BF16_POST
+    lib = load_library()
+    need = C.c_size_t(0)
+    check(lib.ascq_linear_w8a8_dynamic_workspace_size(C.byref(d), C.byref(need)))
+    key = (x.device, need.value)
+    if key not in _lin_ws:
+        _lin_ws[key] = torch.empty(max(need.value, 16), dtype=torch.uint8, device=x.device)
+    ws = _lin_ws[key]
+    check(lib.ascq_linear_w8a8_dynamic(C.byref(d), _dt(x), _ptr(c), _ptr(x), _ptr(weight), _ptr(bias),
+                                       _ptr(channel_scale), _ptr(ws), ws.numel(), _stream()))
+    return c
+
+
 def quant_group_matmul(y, x, weight, group_list, scale, per_token_scale=None, bias=None,
                        group_list_kind=abi.GROUP_LIST_COUNTS, activation=abi.MM_ACT_NONE, weight_nz=False):
     """The quantized grouped matmul of the reference's MoE example: x int8 [m, k], weight int8 [g, k, n] (or, with

@@ -656,6 +656,72 @@ extern "C" int ascq_matmul_w8a8(const ascq_matmul_desc* d, void* c, const void* 
     return d->trans_b ? launch_gemm<TileLT, true, false>(p, st) : launch_gemm<TileL, false, false>(p, st);
 }
 
+// ---------------------------------------------------------------------------- fused dynamic quantisation + matmul
+namespace {
+inline size_t round256(size_t v) { return (v + 255u) & ~static_cast<size_t>(255u); }
+}  // namespace
+
+extern "C" int ascq_linear_w8a8_dynamic_workspace_size(const ascq_matmul_desc* d, size_t* bytes)
+{
+    ASCQ_REQUIRE(d != nullptr && bytes != nullptr, ASCQ_ENULL, "ascq_linear_w8a8_dynamic_workspace_size: NULL argument");
+    size_t mm = 0;
+    ascq_matmul_desc dd = *d;
+    dd.has_tok_scale = 1;
+    int rc = ascq_matmul_w8a8_workspace_size(&dd, &mm);
+    if (rc != ASCQ_OK) {
+        return rc;
+    }
+    // q [m, k] int8, token scales [m], then the matmul's own scratch
+    *bytes = round256(static_cast<size_t>(d->m) * d->k) + round256(static_cast<size_t>(d->m) * sizeof(float)) + mm;
+    return ASCQ_OK;
+}
+
+// The activation quantiser of a W8A8 linear and the matmul in one call: q, tok = dynamic per-token quantisation of x
+// (ascq_dynamic_quant_per_token), c = matmul(q, b) with the token scales in the epilogue; q and tok live in the
+// caller's workspace.  (A variant that quantised inside the weight-streaming matmul kernel for up to 8 rows - row
+// maxima per workgroup, quantisation in registers on the way into the MFMA operand - was bit-identical but not faster
+// than the two launches, 21 us against 20 us at m = 1, and is not kept.)  The reference composes this
+// from ReduceMax / AscendQuant PER_TOKEN and Matmul (impl/adv_api/detail/quantization/quant/
+// ascend_quant_per_group_3510_impl.h:142-178, include/adv_api/matmul/matmul.h:175-185).
+extern "C" int ascq_linear_w8a8_dynamic(const ascq_matmul_desc* d, int32_t x_dtype, void* c, const void* x,
+                                        const void* b, const void* bias, const void* quant_vector, void* workspace,
+                                        size_t workspace_bytes, void* stream)
+{
+    ASCQ_REQUIRE(d != nullptr, ASCQ_ENULL, "ascq_linear_w8a8_dynamic: desc is NULL");
+    ASCQ_REQUIRE(x_dtype == ASCQ_F16 || x_dtype == ASCQ_BF16 || x_dtype == ASCQ_F32, ASCQ_EUNSUPPORTED,
+                 "ascq_linear_w8a8_dynamic: x dtype %d is not half / bfloat16 / float", x_dtype);
+    ASCQ_REQUIRE(!d->trans_a, ASCQ_EUNSUPPORTED, "ascq_linear_w8a8_dynamic: x is [m, k] row-major");
+    ASCQ_REQUIRE(d->quant_mode != ASCQ_MM_QUANT_NONE && d->out_dtype != ASCQ_I8, ASCQ_EUNSUPPORTED,
+                 "ascq_linear_w8a8_dynamic: the token scales need a floating-point dequantising epilogue");
+    ascq_matmul_desc dd = *d;
+    dd.has_tok_scale = 1;
+    ASCQ_REQUIRE(workspace != nullptr, ASCQ_ENULL, "ascq_linear_w8a8_dynamic: workspace is NULL");
+    ASCQ_REQUIRE(aligned16(workspace), ASCQ_EALIGN, "ascq_linear_w8a8_dynamic: workspace must be 16-byte aligned");
+    size_t need = 0;
+    int rc = ascq_linear_w8a8_dynamic_workspace_size(d, &need);
+    if (rc != ASCQ_OK) {
+        return rc;
+    }
+    ASCQ_REQUIRE(workspace_bytes >= need, ASCQ_EINVAL,
+                 "ascq_linear_w8a8_dynamic: workspace of %zu bytes required (see ascq_linear_w8a8_dynamic_workspace_size)",
+                 need);
+    char* ws = static_cast<char*>(workspace);
+    // validate with a stand-in for the quantised activations (the checks only look at NULL-ness)
+    rc = validate_mm(&dd, "ascq_linear_w8a8_dynamic", c, x, b, bias, quant_vector, ws);
+    if (rc != ASCQ_OK) {
+        return rc;
+    }
+    int8_t* q = reinterpret_cast<int8_t*>(ws);
+    float* tok = reinterpret_cast<float*>(ws + round256(static_cast<size_t>(d->m) * d->k));
+    char* rest = reinterpret_cast<char*>(tok) + round256(static_cast<size_t>(d->m) * sizeof(float));
+    rc = ascq_dynamic_quant_per_token(x_dtype, d->m, d->k, q, tok, x, stream);
+    if (rc != ASCQ_OK) {
+        return rc;
+    }
+    return ascq_matmul_w8a8(&dd, c, q, b, bias, quant_vector, tok, rest,
+                            workspace_bytes - static_cast<size_t>(rest - ws), stream);
+}
+
 // ref: examples/.../quant_group_matmul_high_performance/quant_group_matmul_custom.asc:255-454
 extern "C" int ascq_group_matmul_w8a8(const ascq_group_matmul_desc* g, void* y, const void* x, const void* w,
                                       const void* bias, const void* scale, const void* tok_scale,

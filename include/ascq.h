@@ -287,6 +287,20 @@ int ascq_matmul_w8a8(const ascq_matmul_desc* desc, void* c, const void* a, const
                      void* stream);
 int ascq_matmul_w8a8_workspace_size(const ascq_matmul_desc* desc, size_t* bytes);
 
+/*
+ * The W8A8 linear with dynamic activation quantisation in one call:
+ *   q, tok = ascq_dynamic_quant_per_token(x) ;  c = ascq_matmul_w8a8(q, b, ..., tok_scale = tok)
+ * with exactly those results.  x [m, k] of x_dtype (ASCQ_F16 | ASCQ_BF16 | ASCQ_F32); desc as for ascq_matmul_w8a8 with
+ * a dequantising epilogue (quant_mode SCALAR or VECTOR, floating-point out_dtype); desc->has_tok_scale is ignored.
+ * The two kernels run one after the other on the stream, with q and tok in the workspace (sized by
+ * ascq_linear_w8a8_dynamic_workspace_size).  No single reference operator does this: the reference composes it from
+ * ReduceMax / AscendQuant PER_TOKEN (ascend_quant_per_group_3510_impl.h:142-178) and Matmul (matmul.h:175-185).
+ */
+int ascq_linear_w8a8_dynamic(const ascq_matmul_desc* desc, int32_t x_dtype, void* c, const void* x, const void* b,
+                             const void* bias, const void* quant_vector, void* workspace, size_t workspace_bytes,
+                             void* stream);
+int ascq_linear_w8a8_dynamic_workspace_size(const ascq_matmul_desc* desc, size_t* bytes);
+
 /* ------------------------------------------------ quantized grouped matmul */
 typedef enum ascq_group_list_kind {
     ASCQ_GROUP_LIST_COUNTS = 0,    /* rows per group (ref: examples/.../quant_group_matmul_custom.asc:264) */

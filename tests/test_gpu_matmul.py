@@ -450,3 +450,27 @@ def test_workspaces_need_no_initialisation_and_results_repeat(m):
     for y4, y8 in outs[1:]:
         assert np.array_equal(y4, outs[0][0]) and np.array_equal(y8, outs[0][1])
     assert not np.isnan(outs[0][0].view(np.float16)).any() and not np.isnan(outs[0][1].view(np.float16)).any()
+
+# ------------------------------------------------------------------ fused dynamic quantisation + matmul
+@pytest.mark.parametrize("m", [1, 2, 5, 8, 9, 40])
+@pytest.mark.parametrize("k,n", [(256, 128), (1024, 1056), (4096, 2064), (320, 48)])
+@pytest.mark.parametrize("xdt", [torch.bfloat16, torch.float16, torch.float32])
+def test_linear_w8a8_dynamic_equals_quantise_then_matmul(m, k, n, xdt):
+    """One call = per-token quantisation followed by the matmul, bit for bit (oracle of the two steps)."""
+    announce("linear dynamic", m, k, n, xdt)
+    rng = np.random.default_rng(m * 3 + k + n)
+    xf = rng.standard_normal((m, k)).astype(np.float32) * rng.uniform(0.1, 30.0, (m, 1)).astype(np.float32)
+    if m > 2:
+        xf[1] = 0.0                                       # an all-zero row: scale 1, zeros
+    x = torch.from_numpy(xf).to(DEV).to(xdt)
+    w = rng.integers(-127, 128, (k, n)).astype(np.int8)
+    cs = rng.uniform(1e-4, 1e-2, n).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    c = torch.zeros((m, n), dtype=torch.bfloat16, device=DEV)
+    ops.linear_w8a8_dynamic(c, x, to_dev(w), to_dev(cs), to_dev(bias))
+    xdt_abi = {torch.bfloat16: abi.BF16, torch.float16: abi.F16, torch.float32: abi.F32}[xdt]
+    q, ts = orc.dynamic_quant_per_token(xdt_abi, bits(x))
+    d = abi.MatmulDesc(m=m, n=n, k=k, out_dtype=abi.BF16, quant_mode=abi.MM_QUANT_VECTOR, scale_format=abi.MM_SCALE_F32,
+                       has_tok_scale=1, bias_kind=abi.MM_BIAS_F32_POST)
+    want = orc.matmul_w8a8(d, q, w, bias, cs, ts)
+    assert np.array_equal(bits(c), want)
