@@ -664,26 +664,29 @@ __global__ __launch_bounds__(kThreads) void antiquant_scalar_kernel(AntiQuantArg
 template <bool kHasOffset>
 __global__ __launch_bounds__(kThreads) void antiquant_i8_f16_fast_kernel(AntiQuantArgs a)
 {
-    const uint32_t j = (blockIdx.x * kThreads + threadIdx.x) * 16u;
+    // one lane = 8 columns: 8 bytes in, one 16-byte store out, so that every store instruction of a wavefront writes
+    // 1 KiB of consecutive bytes
+    const uint32_t j = (blockIdx.x * kThreads + threadIdx.x) * 8u;
     if (j >= a.cols) {
         return;
     }
+    constexpr int kRows = 2 * kRowsInFlight;
     const f16x2 k1152 = {static_cast<half_t>(1152.0f), static_cast<half_t>(1152.0f)};
-    f16x2 s[8], o[8];
+    f16x2 s[4], o[4];
     uint32_t cached_group = 0xFFFFFFFFu;
     const int8_t* src = static_cast<const int8_t*>(a.src);
     uint16_t* dst = static_cast<uint16_t*>(a.dst);
-    for (uint32_t r0 = blockIdx.y * kRowsInFlight; r0 < a.rows; r0 += gridDim.y * kRowsInFlight) {
-        u32x4 raw[kRowsInFlight];
+    for (uint32_t r0 = blockIdx.y * kRows; r0 < a.rows; r0 += gridDim.y * kRows) {
+        u32x2 raw[kRows];
 #pragma unroll
-        for (int u = 0; u < kRowsInFlight; ++u) {
+        for (int u = 0; u < kRows; ++u) {
             if (r0 + u < a.rows) {
                 raw[u] = __builtin_nontemporal_load(
-                    reinterpret_cast<const u32x4*>(src + static_cast<size_t>(r0 + u) * a.cols + j));
+                    reinterpret_cast<const u32x2*>(src + static_cast<size_t>(r0 + u) * a.cols + j));
             }
         }
 #pragma unroll
-        for (int u = 0; u < kRowsInFlight; ++u) {
+        for (int u = 0; u < kRows; ++u) {
             const uint32_t r = r0 + u;
             if (r >= a.rows) {
                 break;
@@ -694,34 +697,25 @@ __global__ __launch_bounds__(kThreads) void antiquant_i8_f16_fast_kernel(AntiQua
                 if (a.per_tensor) {
                     const half_t hs = static_cast<half_t>(a.sscale), ho = static_cast<half_t>(a.soffset);
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) {
+                    for (int e = 0; e < 4; ++e) {
                         s[e] = f16x2{hs, hs};
                         o[e] = f16x2{ho, ho};
                     }
                 } else {
                     const size_t pi = static_cast<size_t>(g) * a.cols + j;
                     const u32x4 s0 = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(a.scale) + pi);
-                    const u32x4 s1 = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(a.scale) + pi + 8);
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        s[e] = h2_from_bits(s0[e]);
-                        s[4 + e] = h2_from_bits(s1[e]);
-                    }
+                    for (int e = 0; e < 4; ++e) s[e] = h2_from_bits(s0[e]);
                     if constexpr (kHasOffset) {
                         const u32x4 o0 = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(a.offset) + pi);
-                        const u32x4 o1 =
-                            *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(a.offset) + pi + 8);
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            o[e] = h2_from_bits(o0[e]);
-                            o[4 + e] = h2_from_bits(o1[e]);
-                        }
+                        for (int e = 0; e < 4; ++e) o[e] = h2_from_bits(o0[e]);
                     }
                 }
             }
-            u32x4 y0, y1;
+            u32x4 y;
 #pragma unroll
-            for (int d = 0; d < 4; ++d) {
+            for (int d = 0; d < 2; ++d) {
                 const uint32_t x = raw[u][d] ^ 0x80808080u;
                 f16x2 lo = h2_from_bits(__builtin_amdgcn_perm(0x64646464u, x, 0x04010400u)) - k1152;  // bytes 0, 1
                 f16x2 hi = h2_from_bits(__builtin_amdgcn_perm(0x64646464u, x, 0x04030402u)) - k1152;  // bytes 2, 3
@@ -734,17 +728,10 @@ __global__ __launch_bounds__(kThreads) void antiquant_i8_f16_fast_kernel(AntiQua
                 uint32_t blo, bhi;
                 __builtin_memcpy(&blo, &lo, 4);
                 __builtin_memcpy(&bhi, &hi, 4);
-                if (d < 2) {
-                    y0[2 * d] = blo;
-                    y0[2 * d + 1] = bhi;
-                } else {
-                    y1[2 * (d - 2)] = blo;
-                    y1[2 * (d - 2) + 1] = bhi;
-                }
+                y[2 * d] = blo;
+                y[2 * d + 1] = bhi;
             }
-            const size_t oe = static_cast<size_t>(r) * a.cols + j;
-            __builtin_nontemporal_store(y0, reinterpret_cast<u32x4*>(dst + oe));
-            __builtin_nontemporal_store(y1, reinterpret_cast<u32x4*>(dst + oe + 8));
+            __builtin_nontemporal_store(y, reinterpret_cast<u32x4*>(dst + static_cast<size_t>(r) * a.cols + j));
         }
     }
 }
@@ -761,10 +748,15 @@ int launch_antiquant(const AntiQuantArgs& a, bool vec, hipStream_t st)
         if (grid.y > 65535u) grid.y = 65535u;
         if constexpr (kSrc == ASCQ_I8 && kDst == ASCQ_F16) {
             if (!a.transpose) {
+                dim3 fgrid((a.cols / 8 + kThreads - 1) / kThreads, 1);
+                const uint32_t frow_groups = (a.rows + 2 * kRowsInFlight - 1) / (2 * kRowsInFlight);
+                const uint32_t fwant = (8192u + fgrid.x - 1) / fgrid.x;
+                fgrid.y = frow_groups < fwant ? frow_groups : fwant;
+                if (fgrid.y > 65535u) fgrid.y = 65535u;
                 if (a.has_offset) {
-                    antiquant_i8_f16_fast_kernel<true><<<grid, kThreads, 0, st>>>(a);
+                    antiquant_i8_f16_fast_kernel<true><<<fgrid, kThreads, 0, st>>>(a);
                 } else {
-                    antiquant_i8_f16_fast_kernel<false><<<grid, kThreads, 0, st>>>(a);
+                    antiquant_i8_f16_fast_kernel<false><<<fgrid, kThreads, 0, st>>>(a);
                 }
                 return launch_status("ascq_antiquant");
             }
