@@ -626,10 +626,11 @@ __global__ __launch_bounds__(512) void w4a16_gemv_kernel(WnParams p)
 // when the stream enters a column block.  Accumulator c (kept as acc[c / 4][c % 4]) holds rows 4 g .. 4 g + 3 of
 // column 16 jj + c; a piece of the workspace is [4 slices][16 registers][64 lanes].
 // Requires n % 16 == 0, k % 32 == 0.
-template <bool kHasOffset>
+template <bool kHasOffset, int kRT>
 __global__ __launch_bounds__(512) void w8a16_tile_kernel(WnParams p)
 {
-    constexpr int kStage = 8 * 1024 + 1024;  // bytes per wavefront and stage: weights, activations
+    static_assert(kRT == 1 || kRT == 2, "one or two tiles of 16 activation rows per pass");
+    constexpr int kStage = 8 * 1024 + kRT * 1024;  // bytes per wavefront and stage: weights, activations
     __shared__ __attribute__((aligned(1024))) char S0[8 * kStage];
     __shared__ __attribute__((aligned(1024))) char S1[8 * kStage];
 
@@ -676,13 +677,14 @@ __global__ __launch_bounds__(512) void w8a16_tile_kernel(WnParams p)
             __builtin_amdgcn_global_load_lds((gptr_t)(wsrc + static_cast<size_t>(u) * row_bytes),
                                              (lds_ptr_t)(stage + u * 1024), 16, 0, 0);
         }
-        // activations of the chunk's 32 k for up to 16 rows in one instruction: lane l fetches piece (l & 3) of row
-        // m0 + (l >> 2); rows past m fetch row m - 1 and are zeroed when used
-        {
-            const uint32_t m = p.m0 + (lane >> 2);
+        // activations of the chunk's 32 k, 16 rows per instruction: lane l fetches piece (l & 3) of row
+        // m0 + 16 t + (l >> 2); rows past m fetch row m - 1 and are zeroed when used
+#pragma unroll
+        for (int t = 0; t < kRT; ++t) {
+            const uint32_t m = p.m0 + 16u * t + (lane >> 2);
             const uint32_t mc = m < p.m ? m : p.m - 1u;
             __builtin_amdgcn_global_load_lds((gptr_t)(p.x + static_cast<size_t>(mc) * p.k + krow + 8u * (lane & 3u)),
-                                             (lds_ptr_t)(stage + 8 * 1024), 16, 0, 0);
+                                             (lds_ptr_t)(stage + (8 + t) * 1024), 16, 0, 0);
         }
         if (++ik == cb_chunks) {
             ik = 0;
@@ -691,9 +693,9 @@ __global__ __launch_bounds__(512) void w8a16_tile_kernel(WnParams p)
     };
 
     // ---- consumer side
-    f32x4 acc[4][4];
+    f32x4 acc[kRT * 4][4];  // row tile t: acc[4 t + c / 4][c % 4]
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
+    for (int q = 0; q < kRT * 4; ++q) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) acc[q][t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     }
@@ -703,14 +705,14 @@ __global__ __launch_bounds__(512) void w8a16_tile_kernel(WnParams p)
     uint32_t seg = 0, done_in_block = c_begin % cb_chunks;
     auto flush = [&]() __attribute__((always_inline)) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            float* dst = p.partial + ((static_cast<size_t>(gw) * p.max_seg + seg) * 4u + q) * 1024u + lane;
-            // register r holds row 4 g + r; lanes of a missing row hold zeros: not stored
+        for (int q = 0; q < kRT * 4; ++q) {
+            float* dst = p.partial + ((static_cast<size_t>(gw) * p.max_seg + seg) * (kRT * 4u) + q) * 1024u + lane;
+            // register r holds row 16 (q / 4) + 4 g + r; lanes of a missing row hold zeros: not stored
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    if (p.m0 + 4u * g + r < p.m) {
+                    if (p.m0 + 16u * (q >> 2) + 4u * g + r < p.m) {
                         dst[(d * 4 + r) * 64] = acc[q][d][r];
                     }
                 }
@@ -749,7 +751,7 @@ __global__ __launch_bounds__(512) void w8a16_tile_kernel(WnParams p)
         const uint32_t sa = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)stage));
         const uint32_t a_own = sa + lane * 16u;                       // what this lane fetched itself
         const uint32_t a_x = sa + 8u * 1024u + (jj * 4u + g) * 16u;   // activations: row jj of the tile, piece g
-        u32x4 wd[8], xraw;
+        u32x4 wd[8], xraw[kRT];
         ASCQ_DS_READ128(wd[0], a_own, 0 * 1024);
         ASCQ_DS_READ128(wd[1], a_own, 1 * 1024);
         ASCQ_DS_READ128(wd[2], a_own, 2 * 1024);
@@ -758,16 +760,21 @@ __global__ __launch_bounds__(512) void w8a16_tile_kernel(WnParams p)
         ASCQ_DS_READ128(wd[5], a_own, 5 * 1024);
         ASCQ_DS_READ128(wd[6], a_own, 6 * 1024);
         ASCQ_DS_READ128(wd[7], a_own, 7 * 1024);
-        ASCQ_DS_READ128(xraw, a_x, 0);
+        ASCQ_DS_READ128(xraw[0], a_x, 0);
+        if constexpr (kRT > 1) ASCQ_DS_READ128(xraw[1], a_x, 1024);
         asm volatile("s_waitcnt lgkmcnt(0)"
                      : "+v"(wd[0]), "+v"(wd[1]), "+v"(wd[2]), "+v"(wd[3]), "+v"(wd[4]), "+v"(wd[5]), "+v"(wd[6]),
-                       "+v"(wd[7]), "+v"(xraw)
+                       "+v"(wd[7]), "+v"(xraw[0])
                      :
                      : "memory");
-        // lane (g, jj) carries x[m0 + jj][krow + 8 g .. + 8): the A operand of the tile
-        const u32x4 xa = p.m0 + jj < p.m ? xraw : u32x4{0u, 0u, 0u, 0u};
-        f16x8 a;
-        __builtin_memcpy(&a, &xa, 16);
+        if constexpr (kRT > 1) asm volatile("" : "+v"(xraw[1]));
+        // lane (g, jj) carries x[m0 + 16 t + jj][krow + 8 g .. + 8): the A operand of row tile t
+        f16x8 a[kRT];
+#pragma unroll
+        for (int t = 0; t < kRT; ++t) {
+            const u32x4 xa = p.m0 + 16u * t + jj < p.m ? xraw[t] : u32x4{0u, 0u, 0u, 0u};
+            __builtin_memcpy(&a[t], &xa, 16);
+        }
 #pragma unroll
         for (int d = 0; d < 2; ++d) {  // columns 8 d .. 8 d + 7 of the lane's 16
             f16x2 h[8][4];
@@ -805,7 +812,11 @@ __global__ __launch_bounds__(512) void w8a16_tile_kernel(WnParams p)
                     }
                     f16x8 b;
                     __builtin_memcpy(&b, &bv, 16);
-                    acc[2 * d + qh][dd] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[2 * d + qh][dd], 0, 0, 0);
+#pragma unroll
+                    for (int t = 0; t < kRT; ++t) {
+                        acc[4 * t + 2 * d + qh][dd] =
+                            __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t], b, acc[4 * t + 2 * d + qh][dd], 0, 0, 0);
+                    }
                 }
             }
         }
@@ -862,7 +873,8 @@ __global__ __launch_bounds__(1024) void stream_sum_kernel(WnParams p)
     const float* base = p.partial + (static_cast<size_t>(w0) * p.max_seg * MP + q) * 1024u + 4u * t;
     // the four elements of a lane share their register (t >> 4) and quarter g = (t >> 2) & 3, hence their row (g / 2 of
     // the pair, or 4 g + r of a tile); a row past m was never written
-    const uint32_t my_row = kTile ? 4u * ((t >> 2) & 3u) + ((t >> 4) & 3u) : 2u * q + ((t >> 2) & 3u) / 2u;
+    const uint32_t my_row = kLayout == kPieceTileW8 ? 16u * (q >> 2) + 4u * ((t >> 2) & 3u) + ((t >> 4) & 3u)
+                            : (kTile ? 4u * ((t >> 2) & 3u) + ((t >> 4) & 3u) : 2u * q + ((t >> 2) & 3u) / 2u);
     const bool row_valid = p.m0 + my_row < p.m;
     f32x4 s = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     for (uint32_t w = w0 + sub; row_valid && w < w1; w += 32u) {
@@ -895,9 +907,9 @@ __global__ __launch_bounds__(1024) void stream_sum_kernel(WnParams p)
             col = blk * kColsPerBlock + jj * 32u + (acc_e >> 3) * 8u + ((acc_e >> 1) & 3u) + 4u * (acc_e & 1u);
             m = p.m0 + 4u * g + r;
         } else if constexpr (kLayout == kPieceTileW8) {
-            // slice q holds accumulators 4 q + d of the int8 tile kernel = columns 4 q + d of the lane's 16
-            col = blk * kW8ColsPerBlock + jj * 16u + 4u * q + d;
-            m = p.m0 + 4u * g + r;
+            // slice q of row tile q / 4 holds columns 4 (q % 4) + d of the lane's 16
+            col = blk * kW8ColsPerBlock + jj * 16u + 4u * (q & 3u) + d;
+            m = p.m0 + 16u * (q >> 2) + 4u * g + r;
         } else {
             const uint32_t b8 = 4u * (g & 1u) + r;
             col = blk * kColsPerBlock + jj * 32u + d * 8u + (b8 >> 1) + 4u * (b8 & 1u);
@@ -1126,7 +1138,7 @@ static bool w8a16_fast_ok(const ascq_w8a16_desc* d, const void* x, const void* w
 static size_t w8a16_workspace_need(uint32_t n, uint32_t k)
 {
     const W4Plan pl = make_plan(n, k, 2u * kMaxWaves, kW8ColsPerBlock);
-    return static_cast<size_t>(pl.waves) * pl.max_seg * 4u * 1024u * sizeof(float);
+    return static_cast<size_t>(pl.waves) * pl.max_seg * 8u * 1024u * sizeof(float);  // two row tiles of 4 slices
 }
 
 extern "C" int ascq_matmul_w8a16_workspace_size(const ascq_w8a16_desc* d, size_t* bytes)
@@ -1192,15 +1204,26 @@ extern "C" int ascq_matmul_w8a16(const ascq_w8a16_desc* d, void* y, const void* 
     p.rem = pl.total_chunks % pl.waves;
     const uint32_t col_blocks = (d->n + kW8ColsPerBlock - 1u) / kW8ColsPerBlock;
     const uint32_t grid = (p.waves + 7u) / 8u;
-    // 16 activation rows per pass over the weights
-    for (uint32_t m0 = 0; m0 < d->m; m0 += kTileRows) {
+    // 32 activation rows per pass over the weights (16 when no more are left: fewer MFMAs and a smaller ring)
+    for (uint32_t m0 = 0; m0 < d->m;) {
         p.m0 = m0;
-        if (d->has_offset) {
-            w8a16_tile_kernel<true><<<grid, 512, 0, st>>>(p);
+        if (d->m - m0 > kTileRows) {
+            if (d->has_offset) {
+                w8a16_tile_kernel<true, 2><<<grid, 512, 0, st>>>(p);
+            } else {
+                w8a16_tile_kernel<false, 2><<<grid, 512, 0, st>>>(p);
+            }
+            stream_sum_kernel<8, kPieceTileW8><<<dim3(col_blocks, 8), 1024, 0, st>>>(p);
+            m0 += 2u * kTileRows;
         } else {
-            w8a16_tile_kernel<false><<<grid, 512, 0, st>>>(p);
+            if (d->has_offset) {
+                w8a16_tile_kernel<true, 1><<<grid, 512, 0, st>>>(p);
+            } else {
+                w8a16_tile_kernel<false, 1><<<grid, 512, 0, st>>>(p);
+            }
+            stream_sum_kernel<4, kPieceTileW8><<<dim3(col_blocks, 4), 1024, 0, st>>>(p);
+            m0 += kTileRows;
         }
-        stream_sum_kernel<4, kPieceTileW8><<<dim3(col_blocks, 4), 1024, 0, st>>>(p);
     }
     return launch_status("ascq_matmul_w8a16");
 }

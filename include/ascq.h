@@ -356,7 +356,7 @@ int ascq_matmul_w4a16_workspace_size(const ascq_w4a16_desc* desc, size_t* bytes)
  * x f16 [m, k]; w int8 [k, n]; scale, offset f16 [n] (per channel) or the desc's scalars (per tensor).
  *   wdq[k,j] = f16( scale[j] * f16( f16(w[k,j]) + offset[j] ) )               (offset iff has_offset)
  *   y[i,j]   = out( sum_k f32(x[i,k]) * f32(wdq[k,j]) )                       fp32 accumulation
- * The kernel is a weight-streaming one built for few activation rows (decode): the weights are read once per 16
+ * The kernel is a weight-streaming one built for few activation rows (decode): the weights are read once per 32
  * rows of x.  B as [n, k] (isTransposeB) is not supported.
  * workspace: ascq_matmul_w8a16_workspace_size bytes (contents need not be initialised); calls that share a
  * workspace must not overlap.

@@ -260,7 +260,7 @@ def w8a16_check(got, want, x, out_f32):
         assert np.mean(got.view(np.uint16) == want.view(np.uint16)) > 0.9
 
 
-@pytest.mark.parametrize("m", [1, 3, 16, 17, 40])
+@pytest.mark.parametrize("m", [1, 3, 16, 17, 32, 33, 40, 70])
 @pytest.mark.parametrize("k,n", [(256, 256), (512, 1040), (96, 48), (100, 30), (2048, 512)])
 @pytest.mark.parametrize("mode", ["vector+offset", "vector", "scalar+offset", "scalar", "vector+intoffset"])
 def test_w8a16_small(m, k, n, mode):
