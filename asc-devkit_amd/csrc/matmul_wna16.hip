@@ -22,7 +22,8 @@
 //     activation rows the 8 de-quantised halves of one dword are the B operand as they are; the A operand of output
 //     row i carries x[k_g] in slot i and zeros elsewhere, so row i of the result is the running dot product of column
 //     i of the dword (rows 0-7 serve one activation row, rows 8-15 a second one).  From five rows on, the halves are
-//     regrouped so that a B operand is 8 consecutive k of one column and 16 activation rows fill the A operand;
+//     regrouped so that a B operand is 8 consecutive k of one column and 16 activation rows fill the A operand (two
+//     such row tiles per pass when more than 16 rows remain);
 //   * when a wavefront's run leaves a column block (and at its end) the accumulators go to a workspace as they lie in
 //     registers; a second kernel adds, for every output, the pieces of all wavefronts that worked on its column block
 //     in ascending k order and rounds once to half, so results are deterministic.
@@ -164,12 +165,14 @@ __device__ __forceinline__ void w4_accumulate(const u32x4 (&wd)[8], const u32x4 
 // have to be regrouped (one byte permute per operand dword) and x[16 rows][32 k] is the A operand as it lies in
 // memory.  Accumulator e = 8 d + 2 c2 + hi (kept as acc[e / 4][e % 4]) holds, for the lane's quarter g and column
 // group jj, rows 4 g .. 4 g + 3 of column 32 jj + 8 d + c2 + 4 hi.
-template <bool kHasOffset, bool kFold>
-__device__ __forceinline__ void w4_accumulate_tile(const u32x4 (&wd)[8], const u32x4& xa, const f16x2 (&sc)[4][4],
-                                                   const f16x2 (&ofc)[4][4], f32x4 (&acc)[8][4])
+template <bool kHasOffset, bool kFold, int kRT>
+__device__ __forceinline__ void w4_accumulate_tile(const u32x4 (&wd)[8], const u32x4 (&xa)[kRT],
+                                                   const f16x2 (&sc)[4][4], const f16x2 (&ofc)[4][4],
+                                                   f32x4 (&acc)[kRT * 8][4])
 {
-    f16x8 a;
-    __builtin_memcpy(&a, &xa, 16);
+    f16x8 a[kRT];
+#pragma unroll
+    for (int t = 0; t < kRT; ++t) __builtin_memcpy(&a[t], &xa[t], 16);
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
         f16x2 h[8][4];
@@ -192,7 +195,11 @@ __device__ __forceinline__ void w4_accumulate_tile(const u32x4 (&wd)[8], const u
                 }
                 f16x8 b;
                 __builtin_memcpy(&b, &bv, 16);
-                acc[2 * d + qh][dd] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[2 * d + qh][dd], 0, 0, 0);
+#pragma unroll
+                for (int t = 0; t < kRT; ++t) {
+                    acc[8 * t + 2 * d + qh][dd] =
+                        __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t], b, acc[8 * t + 2 * d + qh][dd], 0, 0, 0);
+                }
             }
         }
     }
@@ -223,14 +230,15 @@ __device__ __forceinline__ bool all_offsets_integral(const f16x2 (&of)[A][B])
 // s_waitcnt vmcnt(n) only (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8)
 #define ASCQ_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | (7 << 4) | (15 << 8))
 
-// Five to sixteen activation rows per pass over the weights (rows m0 .. m0 + 15): one stream per SIMD, the rows are
-// the rows of one MFMA tile (w4_accumulate_tile).  A piece of the workspace is [8 slices][16 registers][64 lanes].
-// Requires n % 32 == 0, k % 32 == 0, group_size % 32 == 0.
-template <bool kHasOffset>
+// Five to 16 kRT activation rows per pass over the weights (rows m0 .. m0 + 16 kRT - 1): one stream per SIMD, the rows
+// are the rows of kRT MFMA tiles that share every de-quantised B operand (w4_accumulate_tile).  A piece of the
+// workspace is [8 kRT slices][16 registers][64 lanes].  Requires n % 32 == 0, k % 32 == 0, group_size % 32 == 0.
+template <bool kHasOffset, int kRT>
 __global__ __launch_bounds__(kThreads) void w4a16_tile_kernel(WnParams p)
 {
+    static_assert(kRT == 1 || kRT == 2, "one or two tiles of 16 activation rows per pass");
     constexpr int kParamInstr = kHasOffset ? 2 : 1;
-    constexpr int kInstr = 8 + kParamInstr + 1;   // 1 KiB DMA instructions per chunk
+    constexpr int kInstr = 8 + kParamInstr + kRT;  // 1 KiB DMA instructions per chunk
     constexpr int kStage = kInstr * 1024;         // bytes per wavefront and stage
     __shared__ __attribute__((aligned(1024))) char S0[4 * kStage];
     __shared__ __attribute__((aligned(1024))) char S1[4 * kStage];
@@ -270,13 +278,14 @@ __global__ __launch_bounds__(kThreads) void w4a16_tile_kernel(WnParams p)
         if constexpr (kHasOffset) {
             __builtin_amdgcn_global_load_lds((gptr_t)(p.offset + prow), (lds_ptr_t)(stage + 9 * 1024), 16, 0, 0);
         }
-        // activations of the chunk's 32 k for up to 16 rows in one instruction: lane l fetches piece (l & 3) of row
-        // m0 + (l >> 2); rows past m fetch row m - 1 and are zeroed when used
-        {
-            const uint32_t m = p.m0 + (lane >> 2);
+        // activations of the chunk's 32 k, 16 rows per instruction: lane l fetches piece (l & 3) of row
+        // m0 + 16 t + (l >> 2); rows past m fetch row m - 1 and are zeroed when used
+#pragma unroll
+        for (int t = 0; t < kRT; ++t) {
+            const uint32_t m = p.m0 + 16u * t + (lane >> 2);
             const uint32_t mc = m < p.m ? m : p.m - 1u;
             __builtin_amdgcn_global_load_lds((gptr_t)(p.x + static_cast<size_t>(mc) * p.k + krow + 8u * (lane & 3u)),
-                                             (lds_ptr_t)(stage + (8 + kParamInstr) * 1024), 16, 0, 0);
+                                             (lds_ptr_t)(stage + (8 + kParamInstr + t) * 1024), 16, 0, 0);
         }
         // advance, staying on the last chunk once the run is exhausted (harmless repeated fetches at the tail)
         if (issued + 1u < c_end) {
@@ -289,9 +298,9 @@ __global__ __launch_bounds__(kThreads) void w4a16_tile_kernel(WnParams p)
     };
 
     // ---- consumer side
-    f32x4 acc[8][4];  // accumulator e of w4_accumulate_tile is acc[e / 4][e % 4]
+    f32x4 acc[kRT * 8][4];  // accumulator e of row tile t is acc[8 t + e / 4][e % 4]
 #pragma unroll
-    for (int q = 0; q < 8; ++q) {
+    for (int q = 0; q < kRT * 8; ++q) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) acc[q][t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     }
@@ -304,14 +313,14 @@ __global__ __launch_bounds__(kThreads) void w4a16_tile_kernel(WnParams p)
     // the accumulators as they lie in registers: [16 registers][64 lanes] per slice of four accumulators
     auto flush = [&]() __attribute__((always_inline)) {
 #pragma unroll
-        for (int q = 0; q < 8; ++q) {
-            float* dst = p.partial + ((static_cast<size_t>(gw) * p.max_seg + seg) * 8u + q) * 1024u + lane;
-            // register r holds row 4 g + r; lanes of a missing row hold zeros: not stored
+        for (int q = 0; q < kRT * 8; ++q) {
+            float* dst = p.partial + ((static_cast<size_t>(gw) * p.max_seg + seg) * (kRT * 8u) + q) * 1024u + lane;
+            // register r holds row 16 (q / 8) + 4 g + r; lanes of a missing row hold zeros: not stored
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const bool row_valid = p.m0 + 4u * g + r < p.m;
+                    const bool row_valid = p.m0 + 16u * (q >> 3) + 4u * g + r < p.m;
                     if (row_valid) {
                         dst[(d * 4 + r) * 64] = acc[q][d][r];
                     }
@@ -335,7 +344,7 @@ __global__ __launch_bounds__(kThreads) void w4a16_tile_kernel(WnParams p)
         const uint32_t a_own = sa + lane * 16u;                      // what this lane fetched itself
         const uint32_t a_par = sa + jj * 16u;                        // parameter pieces of the lane's 32 columns
         const uint32_t a_x = sa + (jj * 4u + g) * 16u;               // activations: row jj of the tile, piece g
-        u32x4 wd[8], sraw[4], oraw[4], xraw;
+        u32x4 wd[8], sraw[4], oraw[4], xraw[kRT];
         ASCQ_DS_READ128(wd[0], a_own, 0 * 1024);
         ASCQ_DS_READ128(wd[1], a_own, 1 * 1024);
         ASCQ_DS_READ128(wd[2], a_own, 2 * 1024);
@@ -354,7 +363,8 @@ __global__ __launch_bounds__(kThreads) void w4a16_tile_kernel(WnParams p)
             ASCQ_DS_READ128(oraw[2], a_par, 9 * 1024 + 2 * 256);
             ASCQ_DS_READ128(oraw[3], a_par, 9 * 1024 + 3 * 256);
         }
-        ASCQ_DS_READ128(xraw, a_x, (8 + kParamInstr) * 1024);
+        ASCQ_DS_READ128(xraw[0], a_x, (8 + kParamInstr) * 1024);
+        if constexpr (kRT > 1) ASCQ_DS_READ128(xraw[1], a_x, (8 + kParamInstr + 1) * 1024);
         // every value read above is an in/out operand of the wait, so nothing uses one before it has arrived
         asm volatile("s_waitcnt lgkmcnt(0)"
                      : "+v"(wd[0]), "+v"(wd[1]), "+v"(wd[2]), "+v"(wd[3]), "+v"(wd[4]), "+v"(wd[5]), "+v"(wd[6]),
@@ -364,7 +374,8 @@ __global__ __launch_bounds__(kThreads) void w4a16_tile_kernel(WnParams p)
         if constexpr (kHasOffset) {
             asm volatile("" : "+v"(oraw[0]), "+v"(oraw[1]), "+v"(oraw[2]), "+v"(oraw[3]));
         }
-        asm volatile("" : "+v"(xraw));
+#pragma unroll
+        for (int t = 0; t < kRT; ++t) asm volatile("" : "+v"(xraw[t]));
         f16x2 sc[4][4], of[4][4];
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
@@ -373,29 +384,38 @@ __global__ __launch_bounds__(kThreads) void w4a16_tile_kernel(WnParams p)
                 pair_up(oraw[d], of[d]);
             }
         }
-        if constexpr (kHasOffset) {
+        if constexpr (kHasOffset && kRT == 1) {
             // With integer offsets w + offset is exact, and so is (1024 + u) + (offset - 1032): the constant can be
             // folded and one packed operation per column pair saved without changing a bit of the result.  Tested
-            // once per quantisation group.
+            // once per quantisation group.  (Not with two row tiles: two arithmetic paths that merge with 256 live
+            // accumulators make the register allocator spill.)
             const uint32_t grp = (done_in_block * kChunkRows) / p.group_size;
             if (grp != checked_group) {
                 checked_group = grp;
                 int_offsets = all_offsets_integral(of);
             }
         }
-        // lane (g, jj) carries x[m0 + jj][krow + 8 g .. + 8): the A operand of the tile
-        const u32x4 xa = p.m0 + jj < p.m ? xraw : u32x4{0u, 0u, 0u, 0u};
-        if (kHasOffset && int_offsets) {
+        // lane (g, jj) carries x[m0 + 16 t + jj][krow + 8 g .. + 8): the A operand of row tile t
+        u32x4 xa[kRT];
 #pragma unroll
-            for (int d = 0; d < 4; ++d) {
+        for (int t = 0; t < kRT; ++t) {
+            xa[t] = p.m0 + 16u * t + jj < p.m ? xraw[t] : u32x4{0u, 0u, 0u, 0u};
+        }
+        if constexpr (kHasOffset && kRT == 1) {
+            if (int_offsets) {
 #pragma unroll
-                for (int c2 = 0; c2 < 4; ++c2) {
-                    of[d][c2] = (c2 & 1) ? of[d][c2] - k72 : of[d][c2] - k1032;  // exact
+                for (int d = 0; d < 4; ++d) {
+#pragma unroll
+                    for (int c2 = 0; c2 < 4; ++c2) {
+                        of[d][c2] = (c2 & 1) ? of[d][c2] - k72 : of[d][c2] - k1032;  // exact
+                    }
                 }
+                w4_accumulate_tile<kHasOffset, true, kRT>(wd, xa, sc, of, acc);
+            } else {
+                w4_accumulate_tile<kHasOffset, false, kRT>(wd, xa, sc, of, acc);
             }
-            w4_accumulate_tile<kHasOffset, true>(wd, xa, sc, of, acc);
         } else {
-            w4_accumulate_tile<kHasOffset, false>(wd, xa, sc, of, acc);
+            w4_accumulate_tile<kHasOffset, false, kRT>(wd, xa, sc, of, acc);
         }
         if (++done_in_block == cb_chunks) {  // the run leaves this column block
             done_in_block = 0;
@@ -857,7 +877,6 @@ enum PieceLayout { kPiecePairs = 0, kPieceTileW4 = 1, kPieceTileW8 = 2 };
 template <int MP, int kLayout = kPiecePairs>
 __global__ __launch_bounds__(1024) void stream_sum_kernel(WnParams p)
 {
-    constexpr bool kTile = kLayout != kPiecePairs;
     __shared__ f32x4 part[4][256];
     const uint32_t sub = threadIdx.x >> 8, t = threadIdx.x & 255u;
     const uint32_t blk = blockIdx.x, q = blockIdx.y;
@@ -873,8 +892,9 @@ __global__ __launch_bounds__(1024) void stream_sum_kernel(WnParams p)
     const float* base = p.partial + (static_cast<size_t>(w0) * p.max_seg * MP + q) * 1024u + 4u * t;
     // the four elements of a lane share their register (t >> 4) and quarter g = (t >> 2) & 3, hence their row (g / 2 of
     // the pair, or 4 g + r of a tile); a row past m was never written
-    const uint32_t my_row = kLayout == kPieceTileW8 ? 16u * (q >> 2) + 4u * ((t >> 2) & 3u) + ((t >> 4) & 3u)
-                            : (kTile ? 4u * ((t >> 2) & 3u) + ((t >> 4) & 3u) : 2u * q + ((t >> 2) & 3u) / 2u);
+    const uint32_t my_row = kLayout == kPieceTileW8   ? 16u * (q >> 2) + 4u * ((t >> 2) & 3u) + ((t >> 4) & 3u)
+                            : kLayout == kPieceTileW4 ? 16u * (q >> 3) + 4u * ((t >> 2) & 3u) + ((t >> 4) & 3u)
+                                                      : 2u * q + ((t >> 2) & 3u) / 2u;
     const bool row_valid = p.m0 + my_row < p.m;
     f32x4 s = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     for (uint32_t w = w0 + sub; row_valid && w < w1; w += 32u) {
@@ -902,10 +922,10 @@ __global__ __launch_bounds__(1024) void stream_sum_kernel(WnParams p)
         const uint32_t jj = e & 15u, g = (e >> 4) & 3u, r = (e >> 6) & 3u, d = e >> 8;
         uint32_t col, m;
         if constexpr (kLayout == kPieceTileW4) {
-            // slice q holds accumulators 4 q + d of w4_accumulate_tile
-            const uint32_t acc_e = 4u * q + d;
+            // slice q of row tile q / 8 holds accumulators 4 (q % 8) + d of w4_accumulate_tile
+            const uint32_t acc_e = 4u * (q & 7u) + d;
             col = blk * kColsPerBlock + jj * 32u + (acc_e >> 3) * 8u + ((acc_e >> 1) & 3u) + 4u * (acc_e & 1u);
-            m = p.m0 + 4u * g + r;
+            m = p.m0 + 16u * (q >> 3) + 4u * g + r;
         } else if constexpr (kLayout == kPieceTileW8) {
             // slice q of row tile q / 4 holds columns 4 (q % 4) + d of the lane's 16
             col = blk * kW8ColsPerBlock + jj * 16u + 4u * (q & 3u) + d;
@@ -993,11 +1013,12 @@ W4Plan make_plan(uint32_t n, uint32_t k, uint32_t max_waves, uint32_t cols_per_b
 }
 
 // bytes of workspace: the larger of the two kernels' needs (two streams per SIMD with up to two row pairs, one with
-// up to eight)
+// up to sixteen)
 size_t workspace_need(uint32_t n, uint32_t k)
 {
     const W4Plan a = make_plan(n, k, kMaxWaves), b = make_plan(n, k, 2u * kMaxWaves);
-    const size_t na = static_cast<size_t>(a.waves) * a.max_seg * (kTileRows / 2u), nb = static_cast<size_t>(b.waves) * b.max_seg * 2u;
+    const size_t na = static_cast<size_t>(a.waves) * a.max_seg * kTileRows;
+    const size_t nb = static_cast<size_t>(b.waves) * b.max_seg * 2u;
     return (na > nb ? na : nb) * 1024u * sizeof(float);
 }
 
@@ -1082,11 +1103,12 @@ extern "C" int ascq_matmul_w4a16(const ascq_w4a16_desc* d, void* y, const void* 
         p.per = pl.total_chunks / pl.waves;
         p.rem = pl.total_chunks % pl.waves;
     };
-    // at most 16 activation rows per pass over the weights
-    for (uint32_t m0 = 0; m0 < d->m; m0 += kTileRows) {
+    // at most 32 activation rows per pass over the weights
+    for (uint32_t m0 = 0; m0 < d->m;) {
         const uint32_t left = d->m - m0;
         p.m0 = m0;
         if (left <= 4) {
+            m0 += 4u;
             set_plan(2u * kMaxWaves);  // two streams per SIMD
             const uint32_t grid = (p.waves + 7u) / 8u;
 #define ASCQ_W4_GEMV(MPV)                                                           \
@@ -1106,14 +1128,25 @@ extern "C" int ascq_matmul_w4a16(const ascq_w4a16_desc* d, void* y, const void* 
 #undef ASCQ_W4_GEMV
             continue;
         }
-        set_plan(kMaxWaves);  // one stream per SIMD, 16 rows
+        set_plan(kMaxWaves);  // one stream per SIMD, one or two tiles of 16 rows
         const uint32_t grid = (p.waves + 3u) / 4u;
-        if (d->has_offset) {
-            w4a16_tile_kernel<true><<<grid, kThreads, 0, st>>>(p);
+        if (left > kTileRows) {
+            if (d->has_offset) {
+                w4a16_tile_kernel<true, 2><<<grid, kThreads, 0, st>>>(p);
+            } else {
+                w4a16_tile_kernel<false, 2><<<grid, kThreads, 0, st>>>(p);
+            }
+            stream_sum_kernel<16, kPieceTileW4><<<dim3(col_blocks, 16), 1024, 0, st>>>(p);
+            m0 += 2u * kTileRows;
         } else {
-            w4a16_tile_kernel<false><<<grid, kThreads, 0, st>>>(p);
+            if (d->has_offset) {
+                w4a16_tile_kernel<true, 1><<<grid, kThreads, 0, st>>>(p);
+            } else {
+                w4a16_tile_kernel<false, 1><<<grid, kThreads, 0, st>>>(p);
+            }
+            stream_sum_kernel<8, kPieceTileW4><<<dim3(col_blocks, 8), 1024, 0, st>>>(p);
+            m0 += kTileRows;
         }
-        stream_sum_kernel<8, kPieceTileW4><<<dim3(col_blocks, 8), 1024, 0, st>>>(p);
     }
     return launch_status("ascq_matmul_w4a16");
 }

@@ -209,7 +209,7 @@ def w4_case(rng, m, k, n, gs, has_offset):
     return x, pack_int4(w), sc, of
 
 
-@pytest.mark.parametrize("m", [1, 2, 3, 4, 7, 9, 16, 19])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 7, 9, 16, 19, 32, 33, 37, 70])
 @pytest.mark.parametrize("k,n,gs", [(512, 1024, 128), (1024, 544, 64), (256, 66, 128), (384, 512, 384)])
 @pytest.mark.parametrize("has_offset", [True, False])
 def test_w4a16_small(m, k, n, gs, has_offset):
