@@ -165,7 +165,7 @@ __device__ __forceinline__ void w4_accumulate(const u32x4 (&wd)[8], const u32x4 
 // have to be regrouped (one byte permute per operand dword) and x[16 rows][32 k] is the A operand as it lies in
 // memory.  Accumulator e = 8 d + 2 c2 + hi (kept as acc[e / 4][e % 4]) holds, for the lane's quarter g and column
 // group jj, rows 4 g .. 4 g + 3 of column 32 jj + 8 d + c2 + 4 hi.
-template <bool kHasOffset, bool kFold, int kRT>
+template <bool kHasOffset, int kRT>
 __device__ __forceinline__ void w4_accumulate_tile(const u32x4 (&wd)[8], const u32x4 (&xa)[kRT],
                                                    const f16x2 (&sc)[4][4], const f16x2 (&ofc)[4][4],
                                                    f32x4 (&acc)[kRT * 8][4])
@@ -178,7 +178,7 @@ __device__ __forceinline__ void w4_accumulate_tile(const u32x4 (&wd)[8], const u
         f16x2 h[8][4];
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
-            w4_dequant_dword<kHasOffset, kFold>(wd[u][d], sc[d], ofc[d], h[u]);
+            w4_dequant_dword<kHasOffset, false>(wd[u][d], sc[d], ofc[d], h[u]);
         }
 #pragma unroll
         for (int qh = 0; qh < 2; ++qh) {
@@ -304,12 +304,8 @@ __global__ __launch_bounds__(kThreads) void w4a16_tile_kernel(WnParams p)
 #pragma unroll
         for (int t = 0; t < 4; ++t) acc[q][t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     }
-    const f16x2 k1032 = {static_cast<half_t>(1032.0f), static_cast<half_t>(1032.0f)};
-    const f16x2 k72 = {static_cast<half_t>(72.0f), static_cast<half_t>(72.0f)};
 
     uint32_t seg = 0, done_in_block = c_begin % cb_chunks;
-    uint32_t checked_group = 0xFFFFFFFFu;
-    bool int_offsets = false;  // every offset of the current group (all lanes) is an integer of magnitude <= 512
     // the accumulators as they lie in registers: [16 registers][64 lanes] per slice of four accumulators
     auto flush = [&]() __attribute__((always_inline)) {
 #pragma unroll
@@ -329,7 +325,6 @@ __global__ __launch_bounds__(kThreads) void w4a16_tile_kernel(WnParams p)
             }
         }
         ++seg;
-        checked_group = 0xFFFFFFFFu;  // the next column block has other offsets
         // Stores and loads retire out of order with respect to each other, so the counted waits on the load queue
         // are only meaningful while no store is pending: drain here (once per column block and stream).
         ASCQ_WAIT_VMCNT(0);
@@ -384,39 +379,15 @@ __global__ __launch_bounds__(kThreads) void w4a16_tile_kernel(WnParams p)
                 pair_up(oraw[d], of[d]);
             }
         }
-        if constexpr (kHasOffset && kRT == 1) {
-            // With integer offsets w + offset is exact, and so is (1024 + u) + (offset - 1032): the constant can be
-            // folded and one packed operation per column pair saved without changing a bit of the result.  Tested
-            // once per quantisation group.  (Not with two row tiles: two arithmetic paths that merge with 256 live
-            // accumulators make the register allocator spill.)
-            const uint32_t grp = (done_in_block * kChunkRows) / p.group_size;
-            if (grp != checked_group) {
-                checked_group = grp;
-                int_offsets = all_offsets_integral(of);
-            }
-        }
         // lane (g, jj) carries x[m0 + 16 t + jj][krow + 8 g .. + 8): the A operand of row tile t
         u32x4 xa[kRT];
 #pragma unroll
         for (int t = 0; t < kRT; ++t) {
             xa[t] = p.m0 + 16u * t + jj < p.m ? xraw[t] : u32x4{0u, 0u, 0u, 0u};
         }
-        if constexpr (kHasOffset && kRT == 1) {
-            if (int_offsets) {
-#pragma unroll
-                for (int d = 0; d < 4; ++d) {
-#pragma unroll
-                    for (int c2 = 0; c2 < 4; ++c2) {
-                        of[d][c2] = (c2 & 1) ? of[d][c2] - k72 : of[d][c2] - k1032;  // exact
-                    }
-                }
-                w4_accumulate_tile<kHasOffset, true, kRT>(wd, xa, sc, of, acc);
-            } else {
-                w4_accumulate_tile<kHasOffset, false, kRT>(wd, xa, sc, of, acc);
-            }
-        } else {
-            w4_accumulate_tile<kHasOffset, false, kRT>(wd, xa, sc, of, acc);
-        }
+        // (the integer-offset fold of the GEMV kernel is left out: two arithmetic paths that merge with 128 or 256 live
+        // accumulators cost more in register shuffling, or spills, than the packed operation they save)
+        w4_accumulate_tile<kHasOffset, kRT>(wd, xa, sc, of, acc);
         if (++done_in_block == cb_chunks) {  // the run leaves this column block
             done_in_block = 0;
             flush();
