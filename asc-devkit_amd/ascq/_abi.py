@@ -80,6 +80,15 @@ class W8A16Desc(C.Structure):
                 ("has_offset", C.c_int32), ("scale", C.c_float), ("offset", C.c_float), ("out_dtype", C.c_int32)]
 
 
+class MatmulPlan(C.Structure):
+    _fields_ = [("kernel", C.c_int32), ("tile_m", C.c_uint32), ("tile_n", C.c_uint32), ("tile_k", C.c_uint32),
+                ("workgroups", C.c_uint32), ("k_splits", C.c_uint32), ("launches", C.c_uint32),
+                ("lds_bytes", C.c_uint32), ("narrow_tile_n", C.c_uint32), ("narrow_workgroups", C.c_uint32),
+                ("workspace_bytes", C.c_size_t)]
+
+
+MM_KERNEL_GENERIC, MM_KERNEL_STREAM, MM_KERNEL_DMA_128, MM_KERNEL_DMA_256, MM_KERNEL_STAGED = 0, 1, 2, 3, 4
+
 _P = C.c_void_p
 # name -> (restype, argtypes): every symbol include/ascq.h declares
 SIGNATURES = {
@@ -92,6 +101,8 @@ SIGNATURES = {
     "ascq_matmul_w8a8": (C.c_int, [C.POINTER(MatmulDesc), _P, _P, _P, _P, _P, _P, _P, C.c_size_t, _P]),
     "ascq_matmul_w8a8_workspace_size": (C.c_int, [C.POINTER(MatmulDesc), C.POINTER(C.c_size_t)]),
     "ascq_linear_w8a8_dynamic": (C.c_int, [C.POINTER(MatmulDesc), C.c_int32, _P, _P, _P, _P, _P, _P, C.c_size_t, _P]),
+    "ascq_matmul_w8a8_plan": (C.c_int, [C.POINTER(MatmulDesc), _P, _P, _P, _P, _P, _P, _P, C.c_size_t,
+                                        C.POINTER(MatmulPlan)]),
     "ascq_linear_w8a8_dynamic_workspace_size": (C.c_int, [C.POINTER(MatmulDesc), C.POINTER(C.c_size_t)]),
     "ascq_group_matmul_w8a8": (C.c_int, [C.POINTER(GroupMatmulDesc), _P, _P, _P, _P, _P, _P, _P, _P]),
     "ascq_matmul_w4a16": (C.c_int, [C.POINTER(W4A16Desc), _P, _P, _P, _P, _P, _P, C.c_size_t, _P]),
@@ -107,6 +118,7 @@ SIGNATURES = {
                                                              C.c_int32, C.POINTER(C.c_uint32),
                                                              C.POINTER(C.c_uint32)]),
     "ascq_pack_quant_param": (C.c_uint64, [C.c_float, C.c_int32, C.c_int32]),
+    "ascq_pack_weight_nz": (C.c_int, [C.c_uint32, C.c_uint32, C.c_uint32, _P, _P, _P]),
     "ascq_zero_fill": (C.c_int, [_P, C.c_size_t, _P]),
     "ascq_last_error": (C.c_char_p, []),
     "ascq_version": (C.c_char_p, []),

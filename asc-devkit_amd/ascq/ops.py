@@ -286,6 +286,22 @@ class Matmul:
                                    need.value, _stream()))
         return c
 
+    def plan(self, c):
+        """The launch plan `iterate_all(c)` would follow (kernel family, tile shape, workgroups, K splits), as a
+        MatmulPlan; nothing is launched.  The counterpart of the reference's host-side TCubeTiling
+        (include/adv_api/matmul/matmul_tilingdata.h:21-72)."""
+        self.desc.out_dtype = _dt(c)
+        lib = load_library()
+        need = C.c_size_t(0)
+        check(lib.ascq_matmul_w8a8_workspace_size(C.byref(self.desc), C.byref(need)))
+        if need.value and (self._ws is None or self._ws.numel() * 4 < need.value):
+            self._ws = torch.empty((need.value + 3) // 4, dtype=torch.int32, device=c.device)
+        plan = abi.MatmulPlan()
+        check(lib.ascq_matmul_w8a8_plan(C.byref(self.desc), _ptr(c), _ptr(self.a), _ptr(self.b), _ptr(self.bias),
+                                        _ptr(self.quant), _ptr(self.tok), _ptr(self._ws) if need.value else None,
+                                        need.value, C.byref(plan)))
+        return plan
+
 
 _lin_ws = {}
 
@@ -416,3 +432,16 @@ def get_ascend_antiquant_max_min_tmp_size(src_shape, scale_shape, is_transpose, 
 
 def pack_quant_param(scale, offset9=0, is_signed=True):
     return int(load_library().ascq_pack_quant_param(float(scale), int(offset9), int(is_signed)))
+
+
+def pack_weight_nz(w, out=None):
+    """int8 [k, n] or [g, k, n] row-major -> the fractal layout [(g,) n/32, k/16, 16, 32] of CubeFormat::NZ, as the
+    reference example packs its weights offline (quant_group_matmul_high_performance/scripts/gen_data.py:62-64)."""
+    if w.dim() not in (2, 3) or w.dtype != torch.int8 or not w.is_contiguous():
+        raise ValueError("pack_weight_nz: a contiguous int8 tensor [k, n] or [g, k, n] is expected")
+    g = w.shape[0] if w.dim() == 3 else 1
+    k, n = w.shape[-2:]
+    if out is None:
+        out = torch.empty(tuple(w.shape[:-2]) + (n // 32, k // 16, 16, 32), dtype=torch.int8, device=w.device)
+    check(load_library().ascq_pack_weight_nz(g, k, n, _ptr(out), _ptr(w), _stream()))
+    return out

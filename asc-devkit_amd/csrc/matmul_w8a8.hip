@@ -472,12 +472,16 @@ int launch_gemm(GemmParams& p, hipStream_t st)
     p.tiles_m = (p.m + T::BM - 1) / T::BM;
     p.tiles_n = (p.n + T::BN - 1) / T::BN;
     auto kernel = gemm_kernel<T, kTransB, kSplitK>;
+    const uint32_t total = p.tiles_m * p.tiles_n;
+    dim3 grid((total + 7u) / 8u * 8u, kSplitK ? p.k_splits : 1u);
+    if (plan_note(ASCQ_MM_KERNEL_STAGED, T::BM, T::BN, kBK, grid.x * grid.y, grid.y, T::kLds,
+                  kSplitK ? static_cast<size_t>(p.m) * p.n * sizeof(int32_t) : 0)) {
+        return ASCQ_OK;
+    }
     int rc = set_lds(kernel, T::kLds);
     if (rc != ASCQ_OK) {
         return rc;
     }
-    const uint32_t total = p.tiles_m * p.tiles_n;
-    dim3 grid((total + 7u) / 8u * 8u, kSplitK ? p.k_splits : 1u);
     kernel<<<grid, kThreads, T::kLds, st>>>(p);
     return launch_status("ascq_matmul_w8a8");
 }
@@ -612,6 +616,9 @@ extern "C" int ascq_matmul_w8a8(const ascq_matmul_desc* d, void* c, const void* 
         size_t total = static_cast<size_t>(d->m) * d->n;
         size_t blocks = (total + kThreads - 1) / kThreads;
         if (blocks > 65536) blocks = 65536;
+        if (plan_note(ASCQ_MM_KERNEL_GENERIC, 1, 1, 1, static_cast<uint32_t>(blocks), 1, 0, 0)) {
+            return ASCQ_OK;
+        }
         gemm_generic_kernel<<<static_cast<uint32_t>(blocks), kThreads, 0, st>>>(p, d->trans_a, d->trans_b);
         return launch_status("ascq_matmul_w8a8 (generic)");
     }
@@ -631,13 +638,19 @@ extern "C" int ascq_matmul_w8a8(const ascq_matmul_desc* d, void* c, const void* 
             const uint32_t steps = (d->k + kBK - 1) / kBK;
             p.k_per_split = (steps + splits - 1) / splits * kBK;
             p.partial = static_cast<int32_t*>(workspace);
-            rc = ascq_zero_fill(workspace, need, stream);
-            if (rc != ASCQ_OK) {
-                return rc;
+            if (!plan_recording()) {
+                rc = ascq_zero_fill(workspace, need, stream);
+                if (rc != ASCQ_OK) {
+                    return rc;
+                }
             }
             rc = d->trans_b ? launch_gemm<TileST, true, true>(p, st) : launch_gemm<TileS, false, true>(p, st);
             if (rc != ASCQ_OK) {
                 return rc;
+            }
+            if (plan_note(0, 0, 0, 0, 0, 0, 0, 0)) {   // the zero fill ...
+                plan_note(0, 0, 0, 0, 0, 0, 0, 0);     // ... and the epilogue kernel
+                return ASCQ_OK;
             }
             size_t total = static_cast<size_t>(d->m) * d->n;
             size_t blocks = (total + kThreads - 1) / kThreads;
@@ -654,6 +667,20 @@ extern "C" int ascq_matmul_w8a8(const ascq_matmul_desc* d, void* c, const void* 
         return d->trans_b ? launch_gemm<TileMT, true, false>(p, st) : launch_gemm<TileM, false, false>(p, st);
     }
     return d->trans_b ? launch_gemm<TileLT, true, false>(p, st) : launch_gemm<TileL, false, false>(p, st);
+}
+
+// ref: include/adv_api/matmul/matmul_tilingdata.h:21-72 (TCubeTiling, the reference's host-side plan of a matmul)
+extern "C" int ascq_matmul_w8a8_plan(const ascq_matmul_desc* d, const void* c, const void* a, const void* b,
+                                     const void* bias, const void* quant_vector, const void* tok_scale,
+                                     const void* workspace, size_t workspace_bytes, ascq_matmul_plan* plan)
+{
+    ASCQ_REQUIRE(plan != nullptr, ASCQ_ENULL, "ascq_matmul_w8a8_plan: plan is NULL");
+    // the call itself, with every launch site describing its launch instead of making it
+    plan_begin(plan);
+    const int rc = ascq_matmul_w8a8(d, const_cast<void*>(c), a, b, bias, quant_vector, tok_scale,
+                                    const_cast<void*>(workspace), workspace_bytes, nullptr);
+    plan_end();
+    return rc;
 }
 
 // ---------------------------------------------------------------------------- fused dynamic quantisation + matmul

@@ -438,6 +438,22 @@ int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st)
         }
     }
     const uint32_t wide_cols = tiles_n - narrow_cols;
+    if (plan_recording()) {
+        constexpr uint32_t kLdsWide = 2u * (256u * BK + BK * 256u) + 256u * 4u;
+        constexpr uint32_t kLdsNarrow = 2u * (256u * BK + BK * 128u) + 256u * 4u;
+        const uint32_t wide_wg = (p.tiles_m * wide_cols + 7u) / 8u * 8u;
+        const uint32_t narrow_tiles = narrow_cols ? (p.n - wide_cols * 256u + 127u) / 128u : 0u;
+        const uint32_t narrow_wg = (p.tiles_m * narrow_tiles + 7u) / 8u * 8u;
+        if (wide_cols) {
+            plan_note(ASCQ_MM_KERNEL_DMA_256, 256, 256, BK, wide_wg, 1, kLdsWide, 0);
+            if (narrow_cols) {
+                plan_note_extra(128, narrow_wg);
+            }
+        } else {
+            plan_note(ASCQ_MM_KERNEL_DMA_256, 256, 128, BK, narrow_wg, 1, kLdsNarrow, 0);
+        }
+        return ASCQ_OK;
+    }
     if (wide_cols) {
         p.tiles_n = wide_cols;
         const uint32_t t = p.tiles_m * p.tiles_n;
@@ -485,6 +501,14 @@ int launch_gemm_dma_skinny(GemmParams& p, void* workspace, size_t workspace_byte
     const size_t need = static_cast<size_t>(splits) * p.m * p.n * sizeof(int32_t);
     if (splits > 1 && (workspace == nullptr || workspace_bytes < need || !aligned16(workspace))) {
         splits = 1;
+    }
+    if (plan_recording()) {
+        constexpr uint32_t kLds = 2u * (128u * BK + BK * 128u) + 128u * 4u;
+        plan_note(ASCQ_MM_KERNEL_DMA_128, 128, 128, BK, t * splits, splits, kLds, splits > 1 ? need : 0);
+        if (splits > 1) {
+            plan_note(0, 0, 0, 0, 0, 0, 0, 0);  // the kernel that adds the partial tiles and applies the epilogue
+        }
+        return ASCQ_OK;
     }
     if (splits == 1) {
         gemm_dma_kernel<128, 128, false><<<t, kThreads, 0, st>>>(p, 0u);

@@ -333,6 +333,14 @@ int launch_gemm_stream(const GemmParams& g, void* workspace, hipStream_t st)
     p.per = pl.total_chunks / pl.waves;
     p.rem = pl.total_chunks % pl.waves;
     p.epi = g.epi;
+    if (plan_recording()) {
+        // at most this many streams work on one column block: the partial results the second kernel adds
+        const uint32_t pieces = p.per ? (pl.chunks_per_block + p.per - 1u) / p.per + 1u : pl.chunks_per_block;
+        plan_note(ASCQ_MM_KERNEL_STREAM, kMaxRows, kChunkN, kChunkK, (pl.waves + 3u) / 4u, pieces, 3u * 4u * kStage,
+                  gemm_stream_workspace(g.m, g.n, g.k));
+        plan_note(0, 0, 0, 0, 0, 0, 0, 0);  // the kernel that adds the pieces and applies the epilogue
+        return ASCQ_OK;
+    }
     gemm_stream_kernel<<<(pl.waves + 3u) / 4u, kThreads, 0, st>>>(p);
     int rc = launch_status("ascq_matmul_w8a8 (stream)");
     if (rc != ASCQ_OK) {

@@ -8,6 +8,46 @@ namespace ascq {
 
 static thread_local char g_error[512] = "";
 
+static thread_local ascq_matmul_plan* g_plan = nullptr;
+
+void plan_begin(ascq_matmul_plan* plan)
+{
+    std::memset(plan, 0, sizeof(*plan));
+    plan->kernel = -1;
+    g_plan = plan;
+}
+void plan_end() { g_plan = nullptr; }
+bool plan_recording() { return g_plan != nullptr; }
+bool plan_note(int kernel, uint32_t tile_m, uint32_t tile_n, uint32_t tile_k, uint32_t workgroups, uint32_t k_splits,
+               uint32_t lds_bytes, size_t workspace_bytes)
+{
+    if (g_plan == nullptr) {
+        return false;
+    }
+    if (g_plan->kernel < 0) {
+        g_plan->kernel = kernel;
+        g_plan->tile_m = tile_m;
+        g_plan->tile_n = tile_n;
+        g_plan->tile_k = tile_k;
+        g_plan->workgroups = workgroups;
+        g_plan->k_splits = k_splits;
+        g_plan->lds_bytes = lds_bytes;
+        g_plan->workspace_bytes = workspace_bytes;
+    }
+    g_plan->launches += 1;
+    return true;
+}
+bool plan_note_extra(uint32_t narrow_tile_n, uint32_t narrow_workgroups)
+{
+    if (g_plan == nullptr) {
+        return false;
+    }
+    g_plan->launches += 1;
+    g_plan->narrow_tile_n = narrow_tile_n;
+    g_plan->narrow_workgroups = narrow_workgroups;
+    return true;
+}
+
 int fail(int code, const char* fmt, ...)
 {
     va_list ap;
@@ -23,6 +63,28 @@ __global__ __launch_bounds__(256) void zero_fill_kernel(uint32_t* p, size_t word
     for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < words;
          i += static_cast<size_t>(gridDim.x) * 256) {
         p[i] = 0u;
+    }
+}
+// int8 [g][k][n] -> fractal [g][n / 32][k][32]: a workgroup moves 64 rows x 128 columns.  A wavefront reads 8 rows x
+// 128 bytes (full lines) per instruction and writes, for each of the 4 column panels, the 8 rows x 32 bytes that are
+// consecutive in the destination.
+__global__ __launch_bounds__(256) void pack_nz_kernel(uint8_t* dst, const uint8_t* src, uint32_t k, uint32_t n)
+{
+    const uint32_t piece = threadIdx.x & 7u, r0 = threadIdx.x >> 3;
+    const uint32_t col = blockIdx.x * 128u + piece * 16u;
+    if (col >= n) {
+        return;
+    }
+    const size_t plane = static_cast<size_t>(blockIdx.z) * k * n;
+    const uint8_t* s = src + plane + col;
+    uint8_t* d = dst + plane + static_cast<size_t>(col >> 5) * k * 32u + (col & 16u);
+#pragma unroll
+    for (uint32_t i = 0; i < 2u; ++i) {
+        const uint32_t row = blockIdx.y * 64u + i * 32u + r0;
+        if (row < k) {
+            const uint4 v = *reinterpret_cast<const uint4*>(s + static_cast<size_t>(row) * n);
+            *reinterpret_cast<uint4*>(d + static_cast<size_t>(row) * 32u) = v;
+        }
     }
 }
 uint64_t shape_size(const uint32_t* shape, uint32_t ndim)
@@ -52,6 +114,25 @@ extern "C" int ascq_zero_fill(void* ptr, size_t bytes, void* stream)
     zero_fill_kernel<<<static_cast<uint32_t>(blocks), 256, 0, static_cast<hipStream_t>(stream)>>>(
         static_cast<uint32_t*>(ptr), words);
     return launch_status("ascq_zero_fill");
+}
+
+// ref: examples/01_simd_cpp_api/05_best_practices/03_fusion_compute/quant_group_matmul_high_performance/scripts/
+// gen_data.py:62-64 (weight.reshape([g, k/16, 16, n/32, 32]).transpose([0, 3, 1, 2, 4]))
+extern "C" int ascq_pack_weight_nz(uint32_t groups, uint32_t k, uint32_t n, void* dst, const void* src, void* stream)
+{
+    ASCQ_REQUIRE(dst && src, ASCQ_ENULL, "ascq_pack_weight_nz: dst / src is NULL");
+    ASCQ_REQUIRE(groups > 0 && k > 0 && n > 0, ASCQ_EINVAL, "ascq_pack_weight_nz: groups, k, n must be greater than 0");
+    ASCQ_REQUIRE(k % 16 == 0 && n % 32 == 0, ASCQ_EINVAL,
+                 "ascq_pack_weight_nz: the fractal layout needs k %% 16 == 0 and n %% 32 == 0 (k %u, n %u)", k, n);
+    ASCQ_REQUIRE(groups <= 65535u && (k + 63u) / 64u <= 65535u, ASCQ_EUNSUPPORTED,
+                 "ascq_pack_weight_nz: at most 65535 groups and k <= 4194240");
+    ASCQ_REQUIRE(((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & 15u) == 0, ASCQ_EALIGN,
+                 "ascq_pack_weight_nz: dst and src must be 16-byte aligned");
+    ASCQ_REQUIRE(dst != src, ASCQ_EINVAL, "ascq_pack_weight_nz: dst and src must not be the same buffer");
+    const dim3 grid((n + 127u) / 128u, (k + 63u) / 64u, groups);
+    pack_nz_kernel<<<grid, 256, 0, static_cast<hipStream_t>(stream)>>>(static_cast<uint8_t*>(dst),
+                                                                      static_cast<const uint8_t*>(src), k, n);
+    return launch_status("ascq_pack_weight_nz");
 }
 
 // Bit layout: docs/zh/api/SIMD-API/基础API/矩阵计算（ISASI）/矩阵计算的搬出/关键特性说明/随路量化.md (tables 1 and 2):

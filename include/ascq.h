@@ -288,6 +288,41 @@ int ascq_matmul_w8a8(const ascq_matmul_desc* desc, void* c, const void* a, const
 int ascq_matmul_w8a8_workspace_size(const ascq_matmul_desc* desc, size_t* bytes);
 
 /*
+ * The launch plan of a matmul call: which kernel family the library picks for these arguments and how it tiles the
+ * problem.  The counterpart of the host-side tiling result the reference computes before a launch
+ * (ref: include/adv_api/matmul/matmul_tilingdata.h:21-72, TCubeTiling: usedCoreNum ~ workgroups, baseM / baseN /
+ * baseK ~ tile_m / tile_n / tile_k, shareL1Size ~ lds_bytes); here it is informational, the call plans by itself.
+ */
+typedef enum ascq_mm_kernel {
+    ASCQ_MM_KERNEL_GENERIC = 0,      /* one lane per output element: unaligned or transposed-A inputs */
+    ASCQ_MM_KERNEL_STREAM = 1,       /* m <= 32: weight streams, one per SIMD, then a kernel that adds their pieces */
+    ASCQ_MM_KERNEL_DMA_128 = 2,      /* m <= 512: 128 x 128 direct-to-LDS tiles, K split over workgroups when a
+                                        workspace is given (k_splits > 1: a second kernel adds the partial tiles) */
+    ASCQ_MM_KERNEL_DMA_256 = 3,      /* 256 x 256 direct-to-LDS tiles; a last partial round of the chip may be run
+                                        by a second launch with 256 x narrow_tile_n tiles */
+    ASCQ_MM_KERNEL_STAGED = 4        /* register-staged tiles: transposed B, or K not a multiple of 128 */
+} ascq_mm_kernel;
+
+typedef struct ascq_matmul_plan {
+    int32_t kernel;             /* ascq_mm_kernel */
+    uint32_t tile_m, tile_n;    /* rows x columns of C per workgroup (per wavefront stream for KERNEL_STREAM: the
+                                   rows x columns a stream accumulates at a time); 1 x 1 for KERNEL_GENERIC */
+    uint32_t tile_k;            /* K per main-loop step */
+    uint32_t workgroups;        /* workgroups of the main launch */
+    uint32_t k_splits;          /* partial sums per output element (1: the main kernel writes C itself) */
+    uint32_t launches;          /* kernel launches per call */
+    uint32_t lds_bytes;         /* LDS per workgroup of the main launch */
+    uint32_t narrow_tile_n;     /* KERNEL_DMA_256: columns per tile of the second launch, 0 if there is none */
+    uint32_t narrow_workgroups; /* workgroups of that launch */
+    size_t workspace_bytes;     /* bytes of the workspace this plan uses (0: the call runs without) */
+} ascq_matmul_plan;
+
+/* Same arguments as ascq_matmul_w8a8 (pointers are only inspected: NULL checks and alignment), no launch. */
+int ascq_matmul_w8a8_plan(const ascq_matmul_desc* desc, const void* c, const void* a, const void* b, const void* bias,
+                          const void* quant_vector, const void* tok_scale, const void* workspace,
+                          size_t workspace_bytes, ascq_matmul_plan* plan);
+
+/*
  * The W8A8 linear with dynamic activation quantisation in one call:
  *   q, tok = ascq_dynamic_quant_per_token(x) ;  c = ascq_matmul_w8a8(q, b, ..., tok_scale = tok)
  * with exactly those results.  x [m, k] of x_dtype (ASCQ_F16 | ASCQ_BF16 | ASCQ_F32); desc as for ascq_matmul_w8a8 with
@@ -393,6 +428,16 @@ int ascq_get_ascend_antiquant_max_min_tmp_size(const uint32_t* src_shape, uint32
 /* -------------------------------------------------------------- utilities */
 /* Pack an fp32 scale (and optional REQ8 offset / sign) into the fixpipe uint64 word. Host-side, pure. */
 uint64_t ascq_pack_quant_param(float scale, int32_t offset9, int32_t is_signed);
+/*
+ * Weight pre-pack: int8 [groups][k][n] (row-major, "ND") -> the fractal "NZ" layout
+ * [groups][n/32][k/16][16][32] that ASCQ_MM_B_NZ consumes (element (g, kk, c) at
+ * ((g * n/32 + c/32) * k + kk) * 32 + c%32).  k % 16 == 0, n % 32 == 0, both
+ * pointers 16-byte aligned, dst != src.  The device-side form of the packing the
+ * reference does offline.
+ * ref: examples/01_simd_cpp_api/05_best_practices/03_fusion_compute/
+ *      quant_group_matmul_high_performance/scripts/gen_data.py:62-64
+ */
+int ascq_pack_weight_nz(uint32_t groups, uint32_t k, uint32_t n, void* dst, const void* src, void* stream);
 /* Fill `bytes` of device memory with zero using a kernel (safe inside stream capture). */
 int ascq_zero_fill(void* ptr, size_t bytes, void* stream);
 const char* ascq_last_error(void);

@@ -467,6 +467,15 @@ public:
         Check(ascq_matmul_w8a8(&desc_, c.GetPhyAddr(), a_, b_, bias_, quant_, tok_, workspace_, workspace_bytes_,
                                stream));
     }
+    // The plan IterateAll(c) would follow; nothing is launched.  The counterpart of the reference's host-side
+    // TCubeTiling (include/adv_api/matmul/matmul_tilingdata.h:21-72).
+    ascq_matmul_plan GetPlan(const DeviceTensor<CType>& c) const
+    {
+        ascq_matmul_plan plan;
+        Check(ascq_matmul_w8a8_plan(&desc_, c.GetPhyAddr(), a_, b_, bias_, quant_, tok_, workspace_, workspace_bytes_,
+                                    &plan));
+        return plan;
+    }
     const ascq_matmul_desc& Desc() const { return desc_; }
 
 private:

@@ -213,3 +213,16 @@ def antiquant_policy(desc, src, scale, offset=None):
     lib().orc_antiquant_policy(C.byref(desc), _ptr(dst), _ptr(src), _ptr(scale), _ptr(offset))
     return dst
 
+
+
+def pack_weight_nz(w):
+    """[.., k, n] -> [.., n/32, k/16, 16, 32]: the packing of the reference example's data script
+    (quant_group_matmul_high_performance/scripts/gen_data.py:62-64) restated with explicit indices, so that a test
+    can hold it against the script's reshape / transpose expression."""
+    *lead, k, n = w.shape
+    w3 = w.reshape(-1, k, n)
+    out = np.empty((w3.shape[0], n // 32, k // 16, 16, 32), dtype=w.dtype)
+    for c in range(n // 32):
+        for kb in range(k // 16):
+            out[:, c, kb] = w3[:, 16 * kb:16 * kb + 16, 32 * c:32 * c + 32]
+    return out.reshape(*lead, n // 32, k // 16, 16, 32)

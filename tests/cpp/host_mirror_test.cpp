@@ -244,6 +244,14 @@ void test_matmul()
         mm.SetTensorB(db.view<int8_t>(k * n));
         mm.SetQuantVector(dcs.view<float>(n));
         mm.SetTokenScale(dts.view<float>(m));
+        // the plan query launches nothing and leaves the object ready for the call: 96 rows without a workspace are
+        // one launch of 128 x 128 tiles
+        const ascq_matmul_plan plan = mm.GetPlan(dc.view<ascq::bfloat16_t>(m * n));
+        if (plan.kernel != ASCQ_MM_KERNEL_DMA_128 || plan.tile_m != 128 || plan.k_splits != 1 || plan.launches != 1) {
+            std::printf("FAIL Matmul plan: kernel %d tile_m %u k_splits %u launches %u\n", plan.kernel, plan.tile_m,
+                        plan.k_splits, plan.launches);
+            ++g_failed;
+        }
         mm.IterateAll(dc.view<ascq::bfloat16_t>(m * n));
         std::vector<uint16_t> want(m * n);
         orc_matmul_w8a8(&mm.Desc(), want.data(), a.data(), b.data(), nullptr, cs.data(), ts.data());

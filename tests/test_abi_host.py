@@ -196,3 +196,49 @@ def test_cpp_host_mirror_header_compiles_standalone(tmp_path):
                    'int main() { ascq::Matmul<ascq::bfloat16_t> mm(1, 1, 1); return mm.Desc().m == 1 ? 0 : 1; }\n')
     inc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
     subprocess.check_call(["g++", "-std=c++17", "-Wall", "-Wextra", "-Werror", "-fsyntax-only", "-I", inc, str(src)])
+
+
+def _plan(m, n, k, a=0x10000, b=0x20000, ws=True, **kw):
+    d = abi.MatmulDesc(m=m, n=n, k=k, out_dtype=abi.BF16, quant_mode=abi.MM_QUANT_VECTOR,
+                       scale_format=abi.MM_SCALE_F32, has_tok_scale=1, **kw)
+    need = C.c_size_t(0)
+    assert L.ascq_matmul_w8a8_workspace_size(C.byref(d), C.byref(need)) == abi.OK
+    p = abi.MatmulPlan()
+    have = need.value if ws else 0
+    rc = L.ascq_matmul_w8a8_plan(C.byref(d), C.c_void_p(0x30000), C.c_void_p(a), C.c_void_p(b), None,
+                                 C.c_void_p(0x40000), C.c_void_p(0x50000), C.c_void_p(0x60000) if have else None,
+                                 have, C.byref(p))
+    assert rc == abi.OK, err()
+    return p, need.value
+
+
+def test_matmul_plan_of_the_benchmark_shapes():
+    """The plan query answers without a GPU (pointers are only inspected) and names what the dispatcher does."""
+    assert C.sizeof(abi.MatmulPlan) == 10 * 4 + 8
+    # M=2048, K=4096, N=11008: 8 x 43 tiles of 256 x 256 = 344 = one full round of 256 + 88; the last 11 tile columns
+    # (2816 columns of C) go to a second launch with 256 x 128 tiles
+    p, _ = _plan(2048, 11008, 4096)
+    assert (p.kernel, p.tile_m, p.tile_n, p.tile_k) == (abi.MM_KERNEL_DMA_256, 256, 256, 128)
+    assert (p.workgroups, p.narrow_tile_n, p.narrow_workgroups, p.launches) == (256, 128, 176, 2)
+    assert p.k_splits == 1 and p.workspace_bytes == 0 and p.lds_bytes == 2 * (256 * 128 * 2) + 1024
+    # decode: weight streams, one per SIMD of 256 compute units, and a kernel that adds their pieces
+    p, need = _plan(1, 11008, 4096)
+    assert (p.kernel, p.tile_m, p.tile_n, p.tile_k) == (abi.MM_KERNEL_STREAM, 32, 128, 64)
+    assert p.workgroups == 256 and p.launches == 2 and p.k_splits > 1 and p.workspace_bytes == need > 0
+    # without the workspace the same call cannot run the streams: 128 x 128 tiles, no K split
+    p, _ = _plan(1, 11008, 4096, ws=False)
+    assert (p.kernel, p.k_splits, p.launches, p.workspace_bytes) == (abi.MM_KERNEL_DMA_128, 1, 1, 0)
+    # M=128: 86 tiles of 128 x 128, K split 4 ways to put some 300 workgroups on the chip
+    p, need = _plan(128, 11008, 4096)
+    assert (p.kernel, p.tile_m, p.tile_n) == (abi.MM_KERNEL_DMA_128, 128, 128)
+    assert (p.k_splits, p.workgroups, p.launches) == (4, 88 * 4, 2) and p.workspace_bytes == 4 * 128 * 11008 * 4
+    # transposed B and odd addresses fall to the register-staged and the generic kernels
+    p, _ = _plan(2048, 11008, 4096, trans_b=1)
+    assert (p.kernel, p.tile_m, p.tile_n, p.launches) == (abi.MM_KERNEL_STAGED, 256, 256, 1)
+    p, _ = _plan(2048, 11008, 4096, a=0x10001)
+    assert (p.kernel, p.launches) == (abi.MM_KERNEL_GENERIC, 1)
+    # a rejected descriptor is rejected by the plan query as by the call
+    d = abi.MatmulDesc(m=0, n=8, k=16, out_dtype=abi.I32)
+    assert L.ascq_matmul_w8a8_plan(C.byref(d), FAKE, FAKE, FAKE, None, None, None, None, 0,
+                                   C.byref(abi.MatmulPlan())) == abi.EINVAL
+    assert L.ascq_matmul_w8a8_plan(C.byref(d), FAKE, FAKE, FAKE, None, None, None, None, 0, None) == abi.ENULL

@@ -360,6 +360,68 @@ def test_matmul_nz_weights(m, n, k, out):
     assert np.array_equal(bits(c), want)
 
 
+@pytest.mark.parametrize("m,kernel", [(1, abi.MM_KERNEL_STREAM), (100, abi.MM_KERNEL_DMA_128),
+                                      (700, abi.MM_KERNEL_DMA_256)])
+def test_matmul_plan_then_call(m, kernel):
+    """The plan query names the kernel family and launches nothing; the call that follows is unaffected."""
+    announce("plan", m)
+    rng = np.random.default_rng(m)
+    n, k = 544, 384
+    a = rng.integers(-127, 128, (m, k)).astype(np.int8)
+    w = rng.integers(-127, 128, (k, n)).astype(np.int8)
+    c = torch.full((m, n), -7, dtype=torch.int32, device=DEV)
+    mm = ops.Matmul(m, n, k)
+    mm.set_tensor_a(to_dev(a))
+    mm.set_tensor_b(to_dev(w))
+    plan = mm.plan(c)
+    torch.cuda.synchronize()
+    assert plan.kernel == kernel and plan.launches >= 1 and plan.workgroups >= 1
+    assert bool((c == -7).all())                      # nothing ran
+    mm.iterate_all(c)
+    assert np.array_equal(c.cpu().numpy(), a.astype(np.int32) @ w.astype(np.int32))
+
+
+@pytest.mark.parametrize("g,k,n", [(1, 16, 32), (1, 128, 160), (3, 208, 544), (2, 4096, 1024), (1, 80, 11008)])
+def test_pack_weight_nz(g, k, n):
+    """The device-side packer against the reference script's reshape / transpose, and its error paths."""
+    announce("pack nz", g, k, n)
+    rng = np.random.default_rng(g + k + n)
+    w = rng.integers(-128, 128, (g, k, n)).astype(np.int8)
+    got = ops.pack_weight_nz(to_dev(w)).cpu().numpy()
+    assert np.array_equal(got, to_nz(w))
+    if g == 1:
+        got2 = ops.pack_weight_nz(to_dev(w[0])).cpu().numpy()
+        assert got2.shape == (n // 32, k // 16, 16, 32) and np.array_equal(got2, to_nz(w[0]))
+
+
+def test_pack_weight_nz_feeds_the_matmul():
+    """ND weights packed on the device give the product of the ND weights, bit for bit."""
+    announce("pack nz + matmul")
+    rng = np.random.default_rng(0x4E5A)
+    m, n, k = 300, 544, 384
+    a = rng.integers(-127, 128, (m, k)).astype(np.int8)
+    w = rng.integers(-127, 128, (k, n)).astype(np.int8)
+    c = torch.zeros((m, n), dtype=torch.int32, device=DEV)
+    mm = ops.Matmul(m, n, k)
+    mm.set_tensor_a(to_dev(a))
+    mm.set_tensor_b(ops.pack_weight_nz(to_dev(w)), nz=True)
+    mm.iterate_all(c)
+    assert np.array_equal(c.cpu().numpy(), a.astype(np.int32) @ w.astype(np.int32))
+
+
+def test_pack_weight_nz_rejects():
+    announce("pack nz rejects")
+    w = torch.zeros((24, 32), dtype=torch.int8, device=DEV)
+    with pytest.raises(ops.AscqError, match="k % 16"):
+        ops.pack_weight_nz(w)
+    w = torch.zeros((16, 48), dtype=torch.int8, device=DEV)
+    with pytest.raises(ops.AscqError, match="n % 32"):
+        ops.pack_weight_nz(w)
+    w = torch.zeros((16, 32), dtype=torch.int8, device=DEV)
+    with pytest.raises(ops.AscqError, match="same buffer"):
+        ops.pack_weight_nz(w, out=w)
+
+
 def test_group_matmul_nz_weights_as_the_reference_example_packs_them():
     """The example's configuration in small: counts group list, fractal weights, FasterGelu, fp16 out."""
     announce("group nz")

@@ -567,3 +567,17 @@ def test_antiquant_policy_against_numpy_and_torch_arithmetic(fmt, mode):
     wantq = sat((x + expand(o16).astype(np.float32)) * expand(s16).astype(np.float32))
     gotq = orc.antiquant_policy(desc(abi.F16, abi.F16, abi.COMPUTE_F32), codes, s16, o16)
     assert np.array_equal(gotq.view(U16), wantq.view(U16))
+
+
+def test_pack_weight_nz_is_the_data_scripts_reshape_transpose():
+    """The explicit-index packing against the expression of the reference example's script (gen_data.py:62-64), and
+    the element address the C header states."""
+    rng = np.random.default_rng(62)
+    g, k, n = 3, 48, 96
+    w = rng.integers(-128, 128, (g, k, n)).astype(np.int8)
+    want = w.reshape([g, k // 16, 16, n // 32, 32]).transpose([0, 3, 1, 2, 4])
+    got = orc.pack_weight_nz(w)
+    assert got.shape == (g, n // 32, k // 16, 16, 32) and np.array_equal(got, want)
+    flat = got.reshape(-1)
+    for gi, kk, c in [(0, 0, 0), (1, 17, 33), (2, 47, 95), (1, 16, 31), (0, 15, 32)]:
+        assert flat[((gi * (n // 32) + c // 32) * k + kk) * 32 + c % 32] == w[gi, kk, c]
