@@ -303,6 +303,36 @@ class Matmul:
         return plan
 
 
+class MatmulInt4(Matmul):
+    """`Matmul<int4b_t, int4b_t, C>`: a and b are uint8 / int8 tensors holding two int4 per byte (even element in the
+    low nibble): a [m, k/2], b [k, n/2] ([n, k/2] with trans_b).  Everything else as Matmul.
+    ref: examples/01_simd_cpp_api/04_advanced_api/00_matmul/matmul_int4/matmul_int4.asc:52-58."""
+
+    def iterate_all(self, c):
+        self.desc.out_dtype = _dt(c)
+        lib = load_library()
+        need = C.c_size_t(0)
+        check(lib.ascq_matmul_w4a4_workspace_size(C.byref(self.desc), C.byref(need)))
+        if self._ws is None or self._ws.numel() * 4 < need.value:
+            self._ws = torch.empty((need.value + 3) // 4, dtype=torch.int32, device=c.device)
+        check(lib.ascq_matmul_w4a4(C.byref(self.desc), _ptr(c), _ptr(self.a), _ptr(self.b), _ptr(self.bias),
+                                   _ptr(self.quant), _ptr(self.tok), _ptr(self._ws), need.value, _stream()))
+        return c
+
+    def plan(self, c):
+        raise NotImplementedError("the plan query describes the int8 matmul; widen the operands with unpack_int4")
+
+
+def unpack_int4(src, out=None):
+    """Packed int4 (two per byte, even element in the low nibble) -> int8, same leading shape, last dimension doubled."""
+    if not src.is_contiguous() or src.element_size() != 1:
+        raise ValueError("unpack_int4: a contiguous one-byte tensor is expected")
+    if out is None:
+        out = torch.empty(tuple(src.shape[:-1]) + (src.shape[-1] * 2,), dtype=torch.int8, device=src.device)
+    check(load_library().ascq_unpack_int4(_ptr(out), _ptr(src), src.numel() * 2, _stream()))
+    return out
+
+
 _lin_ws = {}
 
 

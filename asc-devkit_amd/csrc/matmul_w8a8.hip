@@ -749,6 +749,136 @@ extern "C" int ascq_linear_w8a8_dynamic(const ascq_matmul_desc* d, int32_t x_dty
                             workspace_bytes - static_cast<size_t>(rest - ws), stream);
 }
 
+// ------------------------------------------------------------------------------------------ int4 x int4 matmul
+namespace {
+// 16 source bytes (32 nibbles, even element in the low nibble) -> 32 sign-extended int8 per lane and step
+__global__ __launch_bounds__(256) void unpack_i4_kernel(uint8_t* dst, const uint8_t* src, size_t bytes)
+{
+    const size_t quads = bytes / 16u;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * 256u + threadIdx.x; i < quads;
+         i += static_cast<size_t>(gridDim.x) * 256u) {
+        const u32x4 w = *reinterpret_cast<const u32x4*>(src + i * 16u);
+        u32x4 lo8, hi8;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            // per byte: nibble u -> ((u ^ 8) | 0x80) - 8 has no borrow between bytes, and flipping bit 7 afterwards
+            // leaves the two's complement value of the nibble
+            const uint32_t lo = ((((w[j] & 0x0F0F0F0Fu) ^ 0x08080808u) | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
+            const uint32_t hi = (((((w[j] >> 4) & 0x0F0F0F0Fu) ^ 0x08080808u) | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
+            const uint32_t e0123 = __builtin_amdgcn_perm(hi, lo, 0x05010400u);
+            const uint32_t e4567 = __builtin_amdgcn_perm(hi, lo, 0x07030602u);
+            if (j < 2) {
+                lo8[2 * j] = e0123;
+                lo8[2 * j + 1] = e4567;
+            } else {
+                hi8[2 * (j - 2)] = e0123;
+                hi8[2 * (j - 2) + 1] = e4567;
+            }
+        }
+        *reinterpret_cast<u32x4*>(dst + i * 32u) = lo8;
+        *reinterpret_cast<u32x4*>(dst + i * 32u + 16u) = hi8;
+    }
+    // the last bytes of a buffer that is not a multiple of 16 bytes
+    const size_t tail = quads * 16u;
+    for (size_t i = tail + static_cast<size_t>(blockIdx.x) * 256u + threadIdx.x; i < bytes;
+         i += static_cast<size_t>(gridDim.x) * 256u) {
+        const uint32_t b = src[i];
+        dst[2u * i] = static_cast<uint8_t>(static_cast<int>((b & 15u) ^ 8u) - 8);
+        dst[2u * i + 1u] = static_cast<uint8_t>(static_cast<int>((b >> 4) ^ 8u) - 8);
+    }
+}
+}  // namespace
+
+// ref: AscendC::int4b_t tensors are two values per byte, even element in the low nibble
+// (examples/01_simd_cpp_api/04_advanced_api/00_matmul/matmul_int4/scripts/gen_data.py:32-42)
+extern "C" int ascq_unpack_int4(void* dst, const void* src, size_t elements, void* stream)
+{
+    ASCQ_REQUIRE(elements == 0 || (dst && src), ASCQ_ENULL, "ascq_unpack_int4: dst / src is NULL");
+    ASCQ_REQUIRE(elements % 2 == 0, ASCQ_EINVAL, "ascq_unpack_int4: an even number of int4 elements is required");
+    ASCQ_REQUIRE(aligned16(dst) && aligned16(src), ASCQ_EALIGN, "ascq_unpack_int4: dst and src must be 16-byte aligned");
+    if (elements == 0) {
+        return ASCQ_OK;
+    }
+    const size_t bytes = elements / 2u;
+    size_t blocks = (bytes / 16u + 255u) / 256u;
+    blocks = blocks < 1u ? 1u : (blocks > 8192u ? 8192u : blocks);
+    unpack_i4_kernel<<<static_cast<uint32_t>(blocks), 256, 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<uint8_t*>(dst), static_cast<const uint8_t*>(src), bytes);
+    return launch_status("ascq_unpack_int4");
+}
+
+static int validate_w4a4(const ascq_matmul_desc* d)
+{
+    ASCQ_REQUIRE(d != nullptr, ASCQ_ENULL, "ascq_matmul_w4a4: desc is NULL");
+    // README of the reference example: "When the left matrix A is of int4 data type, transpose is not supported."
+    ASCQ_REQUIRE(!d->trans_a, ASCQ_EUNSUPPORTED, "ascq_matmul_w4a4: an int4 A cannot be transposed");
+    ASCQ_REQUIRE(d->b_format == ASCQ_MM_B_ND, ASCQ_EUNSUPPORTED, "ascq_matmul_w4a4: int4 B is row-major (ND) only");
+    ASCQ_REQUIRE(d->k % 2 == 0, ASCQ_EINVAL, "ascq_matmul_w4a4: k %u must be even (two int4 per byte)", d->k);
+    ASCQ_REQUIRE(d->trans_b || d->n % 2 == 0, ASCQ_EINVAL, "ascq_matmul_w4a4: n %u must be even (two int4 per byte)",
+                 d->n);
+    return ASCQ_OK;
+}
+
+extern "C" int ascq_matmul_w4a4_workspace_size(const ascq_matmul_desc* d, size_t* bytes)
+{
+    int rc = validate_w4a4(d);
+    if (rc != ASCQ_OK) {
+        return rc;
+    }
+    ASCQ_REQUIRE(bytes != nullptr, ASCQ_ENULL, "ascq_matmul_w4a4_workspace_size: bytes is NULL");
+    size_t mm = 0;
+    rc = ascq_matmul_w8a8_workspace_size(d, &mm);
+    if (rc != ASCQ_OK) {
+        return rc;
+    }
+    // A and B as int8, then the int8 matmul's own scratch
+    *bytes = round256(static_cast<size_t>(d->m) * d->k) + round256(static_cast<size_t>(d->k) * d->n) + mm;
+    return ASCQ_OK;
+}
+
+// Matmul<int4b_t, int4b_t, C>: both operands are widened to int8 in the caller's workspace (exact) and the int8
+// matmul with its epilogues does the rest.  The matrix core of this GPU has no int4 operand format, so the widening is
+// what any kernel would do on the way into the MFMA; weights that are used more than once can be widened once with
+// ascq_unpack_int4 and given to ascq_matmul_w8a8.
+// ref: examples/01_simd_cpp_api/04_advanced_api/00_matmul/matmul_int4/matmul_int4.asc:52-58, 155
+extern "C" int ascq_matmul_w4a4(const ascq_matmul_desc* d, void* c, const void* a, const void* b, const void* bias,
+                                const void* quant_vector, const void* tok_scale, void* workspace,
+                                size_t workspace_bytes, void* stream)
+{
+    int rc = validate_w4a4(d);
+    if (rc != ASCQ_OK) {
+        return rc;
+    }
+    rc = validate_mm(d, "ascq_matmul_w4a4", c, a, b, bias, quant_vector, tok_scale);
+    if (rc != ASCQ_OK) {
+        return rc;
+    }
+    ASCQ_REQUIRE(workspace != nullptr, ASCQ_ENULL, "ascq_matmul_w4a4: workspace is NULL");
+    ASCQ_REQUIRE(aligned16(workspace) && aligned16(a) && aligned16(b), ASCQ_EALIGN,
+                 "ascq_matmul_w4a4: a, b and workspace must be 16-byte aligned");
+    size_t need = 0;
+    rc = ascq_matmul_w4a4_workspace_size(d, &need);
+    if (rc != ASCQ_OK) {
+        return rc;
+    }
+    ASCQ_REQUIRE(workspace_bytes >= need, ASCQ_EINVAL,
+                 "ascq_matmul_w4a4: workspace of %zu bytes required (see ascq_matmul_w4a4_workspace_size)", need);
+    char* ws = static_cast<char*>(workspace);
+    char* a8 = ws;
+    char* b8 = a8 + round256(static_cast<size_t>(d->m) * d->k);
+    char* rest = b8 + round256(static_cast<size_t>(d->k) * d->n);
+    rc = ascq_unpack_int4(a8, a, static_cast<size_t>(d->m) * d->k, stream);
+    if (rc != ASCQ_OK) {
+        return rc;
+    }
+    rc = ascq_unpack_int4(b8, b, static_cast<size_t>(d->k) * d->n, stream);
+    if (rc != ASCQ_OK) {
+        return rc;
+    }
+    return ascq_matmul_w8a8(d, c, a8, b8, bias, quant_vector, tok_scale, rest,
+                            workspace_bytes - static_cast<size_t>(rest - ws), stream);
+}
+
 // ref: examples/.../quant_group_matmul_high_performance/quant_group_matmul_custom.asc:255-454
 extern "C" int ascq_group_matmul_w8a8(const ascq_group_matmul_desc* g, void* y, const void* x, const void* w,
                                       const void* bias, const void* scale, const void* tok_scale,

@@ -288,6 +288,22 @@ int ascq_matmul_w8a8(const ascq_matmul_desc* desc, void* c, const void* a, const
 int ascq_matmul_w8a8_workspace_size(const ascq_matmul_desc* desc, size_t* bytes);
 
 /*
+ * Matmul<int4b_t A, int4b_t B, C>: the same descriptor, epilogues and outputs as ascq_matmul_w8a8 with both operands
+ * packed two int4 per byte, even element in the low nibble: A [m, k/2] bytes, B [k, n/2] bytes ([n, k/2] with
+ * trans_b).  trans_a is not supported (the reference's rule for an int4 A), b_format is ND, k is even, n is even
+ * unless trans_b.  Both operands are widened to int8 in the workspace (mandatory; size from the query below), then the
+ * int8 matmul runs.  a, b and the workspace are 16-byte aligned.
+ * ref: examples/01_simd_cpp_api/04_advanced_api/00_matmul/matmul_int4/matmul_int4.asc:52-58, 155; README.md
+ *      ("Constraints"); packing: scripts/gen_data.py:32-42.
+ */
+int ascq_matmul_w4a4(const ascq_matmul_desc* desc, void* c, const void* a, const void* b, const void* bias,
+                     const void* quant_vector, const void* tok_scale, void* workspace, size_t workspace_bytes,
+                     void* stream);
+int ascq_matmul_w4a4_workspace_size(const ascq_matmul_desc* desc, size_t* bytes);
+/* int4 (two per byte, even element in the low nibble) -> int8, `elements` values (even); 16-byte aligned pointers. */
+int ascq_unpack_int4(void* dst, const void* src, size_t elements, void* stream);
+
+/*
  * The launch plan of a matmul call: which kernel family the library picks for these arguments and how it tiles the
  * problem.  The counterpart of the host-side tiling result the reference computes before a launch
  * (ref: include/adv_api/matmul/matmul_tilingdata.h:21-72, TCubeTiling: usedCoreNum ~ workgroups, baseM / baseN /

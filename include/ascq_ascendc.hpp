@@ -19,6 +19,7 @@
 #include <cstdint>
 #include <stdexcept>
 #include <string>
+#include <type_traits>
 
 #include "ascq.h"
 
@@ -381,8 +382,15 @@ enum class CubeFormat : int32_t { ND = 0, NZ = 1 };
 // are consumed at copy-out, impl/adv_api/detail/matmul/stage/copy_cube_out/quant/quant_processor_fixpipe.h:74-222).
 // CType selects the output: int32_t (no quant), half / bfloat16_t / float / int8_t (quant epilogue).
 
-template <typename CType>
+// ABType: int8_t, or int4b_t for Matmul<int4b_t, int4b_t, C> (both operands two values per byte; the workspace is
+// then mandatory, no transposed A, ND only;
+// ref: examples/01_simd_cpp_api/04_advanced_api/00_matmul/matmul_int4/matmul_int4.asc:52-58).
+template <typename CType, typename ABType = int8_t>
 class Matmul {
+    static_assert(std::is_same<ABType, int8_t>::value || std::is_same<ABType, int4b_t>::value,
+                  "Matmul: A and B are int8_t or int4b_t");
+    static constexpr bool kInt4 = std::is_same<ABType, int4b_t>::value;
+
 public:
     Matmul(uint32_t m, uint32_t n, uint32_t k)
     {
@@ -393,13 +401,13 @@ public:
         desc_.out_dtype = DTypeOf<CType>::value;
         desc_.quant_mode = ASCQ_MM_QUANT_NONE;
     }
-    void SetTensorA(const DeviceTensor<int8_t>& a, bool isTransposeA = false)
+    void SetTensorA(const DeviceTensor<ABType>& a, bool isTransposeA = false)
     {
         a_ = a.GetPhyAddr();
         desc_.trans_a = isTransposeA ? 1 : 0;
     }
     // format: the CubeFormat of the reference's MatmulType for B (ND, or the fractal NZ layout [n/32][k/16][16][32])
-    void SetTensorB(const DeviceTensor<int8_t>& b, bool isTransposeB = false, CubeFormat format = CubeFormat::ND)
+    void SetTensorB(const DeviceTensor<ABType>& b, bool isTransposeB = false, CubeFormat format = CubeFormat::ND)
     {
         b_ = b.GetPhyAddr();
         desc_.trans_b = isTransposeB ? 1 : 0;
@@ -459,18 +467,20 @@ public:
     size_t GetWorkspaceSize() const
     {
         size_t bytes = 0;
-        Check(ascq_matmul_w8a8_workspace_size(&desc_, &bytes));
+        Check(kInt4 ? ascq_matmul_w4a4_workspace_size(&desc_, &bytes)
+                    : ascq_matmul_w8a8_workspace_size(&desc_, &bytes));
         return bytes;
     }
     void IterateAll(const DeviceTensor<CType>& c, void* stream = nullptr)
     {
-        Check(ascq_matmul_w8a8(&desc_, c.GetPhyAddr(), a_, b_, bias_, quant_, tok_, workspace_, workspace_bytes_,
-                               stream));
+        Check((kInt4 ? ascq_matmul_w4a4 : ascq_matmul_w8a8)(&desc_, c.GetPhyAddr(), a_, b_, bias_, quant_, tok_,
+                                                            workspace_, workspace_bytes_, stream));
     }
     // The plan IterateAll(c) would follow; nothing is launched.  The counterpart of the reference's host-side
     // TCubeTiling (include/adv_api/matmul/matmul_tilingdata.h:21-72).
     ascq_matmul_plan GetPlan(const DeviceTensor<CType>& c) const
     {
+        static_assert(!kInt4, "the plan query describes the int8 matmul");
         ascq_matmul_plan plan;
         Check(ascq_matmul_w8a8_plan(&desc_, c.GetPhyAddr(), a_, b_, bias_, quant_, tok_, workspace_, workspace_bytes_,
                                     &plan));

@@ -281,6 +281,32 @@ void test_matmul()
         orc_matmul_w8a8(&mm.Desc(), want.data(), a.data(), b.data(), nullptr, nullptr, nullptr);
         expect_equal("Matmul int32", dc.download(), want);
     }
+    std::printf("[case] Matmul<int32_t, int4b_t> 96x160x256, int32 bias\n");
+    {
+        // int4 operands, two per byte with the even element in the low nibble; the oracle sees the same values as int8
+        std::vector<int8_t> a4v(m * k), b4v(k * n);
+        for (auto& e : a4v) e = static_cast<int8_t>(r.integer(-8, 7));
+        for (auto& e : b4v) e = static_cast<int8_t>(r.integer(-8, 7));
+        auto pack = [](const std::vector<int8_t>& v) {
+            std::vector<uint8_t> p(v.size() / 2);
+            for (size_t i = 0; i < p.size(); ++i) {
+                p[i] = static_cast<uint8_t>((v[2 * i] & 0x0F) | ((v[2 * i + 1] & 0x0F) << 4));
+            }
+            return p;
+        };
+        DeviceBuffer<uint8_t> da4(pack(a4v)), db4(pack(b4v));
+        DeviceBuffer<int32_t> dc(m * n);
+        ascq::Matmul<int32_t, ascq::int4b_t> mm(m, n, k);
+        mm.SetTensorA(da4.view<ascq::int4b_t>(m * k));
+        mm.SetTensorB(db4.view<ascq::int4b_t>(k * n));
+        mm.SetBias(dbias.view<int32_t>(n));
+        DeviceBuffer<uint8_t> ws(mm.GetWorkspaceSize());
+        mm.SetWorkspace(ws.view<uint8_t>(0).GetPhyAddr(), mm.GetWorkspaceSize());
+        mm.IterateAll(dc.view<int32_t>(m * n));
+        std::vector<int32_t> want(m * n);
+        orc_matmul_w8a8(&mm.Desc(), want.data(), a4v.data(), b4v.data(), bias.data(), nullptr, nullptr);
+        expect_equal("Matmul int4 x int4", dc.download(), want);
+    }
 }
 
 void test_antiquant_matmul()

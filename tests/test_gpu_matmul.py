@@ -536,3 +536,78 @@ def test_linear_w8a8_dynamic_equals_quantise_then_matmul(m, k, n, xdt):
                        has_tok_scale=1, bias_kind=abi.MM_BIAS_F32_POST)
     want = orc.matmul_w8a8(d, q, w, bias, cs, ts)
     assert np.array_equal(bits(c), want)
+
+
+# ------------------------------------------------------------------ Matmul<int4b_t, int4b_t, C>
+def ref_pack_int4(x):
+    """The packing of the reference example's script (matmul_int4/scripts/gen_data.py:32-42): byte j of a row is
+    (x[2j+1] << 4) + (x[2j] & 0x0F), kept in int8."""
+    return ((x[..., 1::2].astype(np.int32) << 4) + (x[..., 0::2].astype(np.int32) & 0x0F)).astype(np.int8)
+
+
+def test_matmul_int4_reference_example():
+    """The example at its own size and with its own data recipe: M=256, N=7680, K=128, values from
+    uniform(-5, 5) cast to int8, int32 bias, int32 out (matmul_int4/scripts/gen_data.py:20-31)."""
+    announce("int4 example")
+    rng = np.random.default_rng(0x14)
+    m, n, k = 256, 7680, 128
+    x1 = rng.uniform(-5, 5, (m, k)).astype(np.int8)
+    x2 = rng.uniform(-5, 5, (k, n)).astype(np.int8)
+    bias = rng.uniform(-5, 5, n).astype(np.int32)
+    golden = x1.astype(np.int32) @ x2.astype(np.int32) + bias
+    c = torch.zeros((m, n), dtype=torch.int32, device=DEV)
+    mm = ops.MatmulInt4(m, n, k)
+    mm.set_tensor_a(to_dev(ref_pack_int4(x1)))
+    mm.set_tensor_b(to_dev(ref_pack_int4(x2)))
+    mm.set_bias(to_dev(bias))
+    mm.iterate_all(c)
+    assert np.array_equal(c.cpu().numpy(), golden)
+
+
+@pytest.mark.parametrize("m,n,k,trans_b", [(1, 64, 128, False), (33, 160, 96, False), (200, 544, 384, True),
+                                           (513, 34, 130, False), (70, 33, 64, True)])
+@pytest.mark.parametrize("out", [torch.int32, torch.float16])
+def test_matmul_int4_full_range(m, n, k, trans_b, out):
+    """Every nibble value, both B orientations, int32 and the half output the reference allows (through the
+    fixpipe scale words), bit-equal to the int8 oracle on the widened operands."""
+    announce("int4", m, n, k, trans_b, out)
+    rng = np.random.default_rng(m + n + k)
+    a = rng.integers(-8, 8, (m, k)).astype(np.int8)
+    b = rng.integers(-8, 8, (n, k) if trans_b else (k, n)).astype(np.int8)
+    c = torch.zeros((m, n), dtype=out, device=DEV)
+    mm = ops.MatmulInt4(m, n, k, trans_b=trans_b)
+    mm.set_tensor_a(to_dev(pack_int4(a)))
+    mm.set_tensor_b(to_dev(pack_int4(b)))
+    d = abi.MatmulDesc(m=m, n=n, k=k, trans_b=int(trans_b), out_dtype=abi.I32)
+    qv = None
+    if out != torch.int32:
+        qv = np.array([ops.pack_quant_param(s) for s in rng.uniform(1e-3, 1e-1, n)], dtype=np.uint64)
+        mm.set_quant_vector(to_dev(qv.view(np.int64)))
+        d = abi.MatmulDesc(m=m, n=n, k=k, trans_b=int(trans_b), out_dtype=abi.F16, quant_mode=abi.MM_QUANT_VECTOR,
+                           scale_format=abi.MM_SCALE_U64)
+    mm.iterate_all(c)
+    want = orc.matmul_w8a8(d, a, b, None, qv, None)
+    assert np.array_equal(bits(c), want if out == torch.int32 else want.view(np.uint16))
+
+
+@pytest.mark.parametrize("count", [2, 30, 32, 4096 + 34, 1 << 20])
+def test_unpack_int4(count):
+    announce("unpack int4", count)
+    rng = np.random.default_rng(count)
+    v = rng.integers(-8, 8, count).astype(np.int8)
+    got = ops.unpack_int4(to_dev(pack_int4(v))).cpu().numpy()
+    assert got.dtype == np.int8 and np.array_equal(got, v)
+    assert np.array_equal(ops.unpack_int4(to_dev(ref_pack_int4(v))).cpu().numpy(), v)
+
+
+def test_matmul_int4_rejects():
+    announce("int4 rejects")
+    z = torch.zeros(64, dtype=torch.int8, device=DEV)
+    c = torch.zeros((4, 4), dtype=torch.int32, device=DEV)
+    for kw, msg in [(dict(m=4, n=4, k=3), "k 3 must be even"), (dict(m=4, n=3, k=4), "n 3 must be even"),
+                    (dict(m=4, n=4, k=4, trans_a=True), "cannot be transposed")]:
+        mm = ops.MatmulInt4(**kw)
+        mm.set_tensor_a(z)
+        mm.set_tensor_b(z)
+        with pytest.raises(ops.AscqError, match=msg):
+            mm.iterate_all(c)
