@@ -18,7 +18,7 @@ CAST_NONE, CAST_RINT, CAST_FLOOR, CAST_CEIL, CAST_ROUND, CAST_TRUNC = range(6)
 COMPUTE_F16, COMPUTE_SCALE_T, COMPUTE_F32 = range(3)
 # ascq_offset_kind
 OFFSET_NONE, OFFSET_SCALAR, OFFSET_TENSOR = range(3)
-QDST_I8, QDST_FP8_E4M3FN, QDST_FP8_E5M2 = range(3)
+QDST_I8, QDST_FP8_E4M3FN, QDST_FP8_E5M2, QDST_FP4_E2M1, QDST_FP4_E1M2 = range(5)
 # ascq_dequant_mode
 DEQUANT_WITH_SINGLE_ROW, DEQUANT_WITH_MULTI_ROW = range(2)
 # ascq_mm_*

@@ -85,10 +85,10 @@ def ascend_quant(dst, src, scale, offset, cal_count=None, scale_count=None, offs
     return _quant(d, dst, src, None, None)
 
 
-def _policy_quant(compute, dst, src, scale, offset, para, policy, config):
+def _policy_quant(compute, dst, src, scale, offset, para, policy, config, dst_format=None):
     d = abi.QuantDesc(policy=policy, src_dtype=_dt(src), compute=compute, round_mode=config.round_mode,
                       k_dim=config.k_dim, m=para.m, n=para.n, cal_count=para.cal_count, group_size=para.group_size,
-                      dst_format=_QDST[dst.dtype])
+                      dst_format=_QDST[dst.dtype] if dst_format is None else dst_format)
     if policy == abi.PER_TENSOR:
         d.scale, d.scale_dtype = float(scale), _dt(src)
         scale = None
@@ -103,10 +103,13 @@ def _policy_quant(compute, dst, src, scale, offset, para, policy, config):
     return _quant(d, dst, src, scale, offset)
 
 
-def ascend_quant_policy(dst, src, scale, offset, para, policy, config=AscendQuantConfig()):
+def ascend_quant_policy(dst, src, scale, offset, para, policy, config=AscendQuantConfig(), dst_format=None):
     """AscendQuant<dstT, srcT, scaleT, config, policy>(dst, src, scale, offset, para) for PER_TOKEN / PER_GROUP:
-    arithmetic in the scale's dtype for an int8 dst, in fp32 for a torch.float8_e4m3fn / float8_e5m2 dst.  ref: include/adv_api/quantization/ascend_quant.h:667-762."""
-    return _policy_quant(abi.COMPUTE_SCALE_T, dst, src, scale, offset, para, policy, config)
+    arithmetic in the scale's dtype for an int8 dst, in fp32 for a torch.float8_e4m3fn / float8_e5m2 dst.
+    dst_format=abi.QDST_FP4_E2M1 / QDST_FP4_E1M2 (PER_GROUP only): dst is a uint8 tensor of cal_count / 2 bytes, two
+    4-bit floats per byte with the even element in the low nibble (fp4x2_e2m1_t / fp4x2_e1m2_t).
+    ref: include/adv_api/quantization/ascend_quant.h:667-762."""
+    return _policy_quant(abi.COMPUTE_SCALE_T, dst, src, scale, offset, para, policy, config, dst_format)
 
 
 def quantize(dst, src, scale, offset, para, policy, config=AscendQuantConfig()):

@@ -219,7 +219,7 @@ __device__ __forceinline__ void store1(void* base, size_t idx, float v)
     }
 }
 
-// fp32 -> OCP 8-bit floats, round-half-even, saturating to the largest finite value; NaN -> 0x7F with the sign.
+// fp32 -> OCP 8-bit floats, round-half-even, saturating to the largest finite value; NaN -> +0.
 // kE5M2 false: e4m3fn (bias 7, max 448 = 0x7E); true: e5m2 (bias 15, max 57344 = 0x7B).
 template <bool kE5M2>
 __device__ __forceinline__ int f32_to_fp8_sat(float f)
@@ -235,7 +235,7 @@ __device__ __forceinline__ int f32_to_fp8_sat(float f)
     const uint32_t a = u & 0x7FFFFFFFu;
     uint32_t code;
     if (a > 0x7F800000u) {
-        code = 0x7Fu;
+        return 0;  // NaN -> +0: what the reference's saturating casts give
     } else if (a >= kMaxBits) {
         code = kE5M2 ? 0x7Bu : 0x7Eu;  // everything from the largest finite value up, infinity included
     } else if (a >= kMinNormalBits) {
@@ -248,6 +248,44 @@ __device__ __forceinline__ int f32_to_fp8_sat(float f)
         code = static_cast<uint32_t>(__builtin_rintf(mag * (kE5M2 ? 65536.0f : 512.0f)));
     }
     return static_cast<int>(sign | code);
+}
+
+// A value already rounded to bfloat16 -> 4-bit float code (sign, then e2m1 or e1m2, both bias 1), rounded with the
+// given mode, saturating to the largest magnitude (6 / 1.75); NaN -> +0.  The grid is uniform inside each of the
+// ranges used below, so the value is scaled to integers, rounded as a signed number (which makes FLOOR and CEIL right
+// for negative inputs, and half-even on the scaled integer is half-even on the code), and scaled back.
+template <bool kE1M2>
+__device__ __forceinline__ uint32_t f32_to_fp4_sat(float v, int round_mode)
+{
+    if (v != v) {
+        return 0u;
+    }
+    const uint32_t sign = (__float_as_uint(v) >> 28) & 8u;
+    const float a = fminf(fabsf(v), 8.0f);  // everything from 8 up saturates like 8 (and infinity becomes finite)
+    float unit;                             // spacing of the grid around |v|
+    if (kE1M2) {
+        unit = 0.25f;
+    } else {
+        unit = a < 2.0f ? 0.5f : (a < 4.0f ? 1.0f : 2.0f);
+    }
+    const float t = (sign ? -a : a) / unit;  // exact: a power-of-two divisor
+    float r;
+    switch (round_mode) {
+        case ASCQ_CAST_FLOOR: r = __builtin_floorf(t); break;
+        case ASCQ_CAST_CEIL: r = __builtin_ceilf(t); break;
+        case ASCQ_CAST_ROUND: r = __builtin_roundf(t); break;
+        case ASCQ_CAST_TRUNC: r = __builtin_truncf(t); break;
+        default: r = __builtin_rintf(t); break;
+    }
+    const float q = fminf(fabsf(r) * unit, kE1M2 ? 1.75f : 6.0f);
+    uint32_t code;
+    if (kE1M2) {
+        code = static_cast<uint32_t>(q * 4.0f);
+    } else {
+        code = q < 2.0f ? static_cast<uint32_t>(q * 2.0f)
+                        : (q < 4.0f ? static_cast<uint32_t>(q) + 2u : static_cast<uint32_t>(q * 0.5f) + 4u);
+    }
+    return sign | code;
 }
 
 __device__ __forceinline__ uint32_t pack4_i8(int a, int b, int c, int d)

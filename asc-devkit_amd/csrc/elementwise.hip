@@ -34,6 +34,12 @@ __device__ __forceinline__ int quant_final(float t, const QuantArgs& a)
     if (a.dst_format == ASCQ_QDST_I8) {
         return round_sat8<kRint>(t, a.round_mode);
     }
+    if (a.dst_format >= ASCQ_QDST_FP4_E2M1) {
+        // through bfloat16 (half-even), then the 4-bit float with the requested rounding
+        const float b = bf16_bits_to_f32(f32_to_bf16_bits(t));
+        return static_cast<int>(a.dst_format == ASCQ_QDST_FP4_E1M2 ? f32_to_fp4_sat<true>(b, a.round_mode)
+                                                                   : f32_to_fp4_sat<false>(b, a.round_mode));
+    }
     return a.dst_format == ASCQ_QDST_FP8_E5M2 ? f32_to_fp8_sat<true>(t) : f32_to_fp8_sat<false>(t);
 }
 
@@ -139,6 +145,14 @@ __global__ __launch_bounds__(kThreads) void quant_vec_kernel(QuantArgs a)
                     t = Fmt<kCt>::add(t, o[e]);
                 }
                 q[e] = quant_final<kRint>(t, a);
+            }
+            if (a.dst_format >= ASCQ_QDST_FP4_E2M1) {
+                // two codes per byte, the even element in the low nibble: 8 columns are one dword
+                uint32_t out = 0;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) out |= static_cast<uint32_t>(q[e]) << (4 * e);
+                *reinterpret_cast<uint32_t*>(a.dst + (static_cast<size_t>(r) * a.n + j) / 2u) = out;
+                continue;
             }
             u32x2 out;
             out[0] = pack4_i8(q[0], q[1], q[2], q[3]);
@@ -935,8 +949,17 @@ extern "C" int ascq_quant(const ascq_quant_desc* d, void* dst, const void* src, 
                  "ascq_quant: round mode %d is not supported for int8 output", d->round_mode);
     ASCQ_REQUIRE(d->offset_kind >= ASCQ_OFFSET_NONE && d->offset_kind <= ASCQ_OFFSET_TENSOR, ASCQ_EINVAL,
                  "ascq_quant: unknown offset kind %d", d->offset_kind);
-    ASCQ_REQUIRE(d->dst_format >= ASCQ_QDST_I8 && d->dst_format <= ASCQ_QDST_FP8_E5M2, ASCQ_EUNSUPPORTED,
-                 "ascq_quant: destination format %d is not int8 / fp8_e4m3fn / fp8_e5m2", d->dst_format);
+    ASCQ_REQUIRE(d->dst_format >= ASCQ_QDST_I8 && d->dst_format <= ASCQ_QDST_FP4_E1M2, ASCQ_EUNSUPPORTED,
+                 "ascq_quant: destination format %d is not int8 / fp8_e4m3fn / fp8_e5m2 / fp4_e2m1 / fp4_e1m2",
+                 d->dst_format);
+    const bool fp4 = d->dst_format >= ASCQ_QDST_FP4_E2M1;
+    if (fp4) {
+        // ref: AscendQuant.md table 4 (the fp4x2 rows), ascend_quant_per_group_3510_impl.h:1383-1385
+        ASCQ_REQUIRE(d->policy == ASCQ_PER_GROUP && d->compute == ASCQ_COMPUTE_SCALE_T, ASCQ_EUNSUPPORTED,
+                     "ascq_quant: fp4 destinations exist for AscendQuant PER_GROUP only");
+        ASCQ_REQUIRE(d->src_dtype != ASCQ_F32, ASCQ_EUNSUPPORTED,
+                     "ascq_quant: fp4 destinations take half / bfloat16 sources");
+    }
     ASCQ_REQUIRE(d->dst_format == ASCQ_QDST_I8 || d->compute != ASCQ_COMPUTE_F16, ASCQ_EUNSUPPORTED,
                  "ascq_quant: the fp16 contract (AscendQuant per tensor / per channel) has int8 output only");
     const bool tensor_scale = d->policy != ASCQ_PER_TENSOR;
@@ -989,14 +1012,22 @@ extern "C" int ascq_quant(const ascq_quant_desc* d, void* dst, const void* src, 
     if (d->cal_count == 0) {
         return ASCQ_OK;
     }
-    ASCQ_REQUIRE(!ranges_overlap(dst, d->cal_count, src, static_cast<size_t>(d->cal_count) * dtype_size(d->src_dtype)),
+    if (fp4) {
+        ASCQ_REQUIRE(n % 8 == 0 && aligned16(src) && aligned16(scale) && (reinterpret_cast<uintptr_t>(dst) & 3u) == 0,
+                     ASCQ_EALIGN, "ascq_quant: fp4 destinations need n %% 8 == 0, 16-byte aligned src / scale and a "
+                                  "4-byte aligned dst");
+    }
+    ASCQ_REQUIRE(!ranges_overlap(dst, fp4 ? d->cal_count / 2u : d->cal_count, src,
+                                 static_cast<size_t>(d->cal_count) * dtype_size(d->src_dtype)),
                  ASCQ_EINVAL, "ascq_quant: dst overlaps src (in-place operation is not supported on the GPU)");
 
-    QuantArgs a{static_cast<int8_t*>(dst), src, scale, offset, rows, n, d->policy, d->offset_kind, d->k_dim,
+    // the fp4 path of the reference is not given the offset at all
+    const int offset_kind = fp4 ? static_cast<int>(ASCQ_OFFSET_NONE) : d->offset_kind;
+    QuantArgs a{static_cast<int8_t*>(dst), src, scale, offset, rows, n, d->policy, offset_kind, d->k_dim,
                 d->round_mode, d->scale, d->offset, d->group_size ? d->group_size : 1u, ppr, d->dst_format};
-    bool vec = (n % 8 == 0) && aligned16(src) && ((reinterpret_cast<uintptr_t>(dst) & 7u) == 0);
+    bool vec = (n % 8 == 0) && aligned16(src) && ((reinterpret_cast<uintptr_t>(dst) & 7u) == 0 || fp4);
     if (tensor_scale) {
-        vec = vec && aligned16(scale) && (d->offset_kind != ASCQ_OFFSET_TENSOR || aligned16(offset));
+        vec = vec && aligned16(scale) && (offset_kind != ASCQ_OFFSET_TENSOR || aligned16(offset));
     }
     if (!tensor_scale && n > 8 * kThreads) {
         // a per-tensor call is a flat array: view it as rows of 2048 when that divides, so the launch is 2-D
@@ -1014,7 +1045,7 @@ extern "C" int ascq_quant(const ascq_quant_desc* d, void* dst, const void* src, 
     // 8-bit float outputs are computed in fp32 whatever the parameter type
     const int ct = d->compute == ASCQ_COMPUTE_F16
                        ? ASCQ_F16
-                       : ((d->compute == ASCQ_COMPUTE_F32 || d->dst_format != ASCQ_QDST_I8) ? ASCQ_F32 : par);
+                       : ((d->compute == ASCQ_COMPUTE_F32 || (d->dst_format != ASCQ_QDST_I8 && !fp4)) ? ASCQ_F32 : par);
     if (!tensor_scale) {
         ASCQ_Q(ASCQ_F16, ASCQ_F32, ASCQ_F16)
         ASCQ_Q(ASCQ_BF16, ASCQ_F32, ASCQ_F16)

@@ -76,7 +76,16 @@ typedef enum ascq_quant_compute {
 /* Destination format of AscendQuant / Quantize.  The 8-bit floats are the OCP formats the reference names
  * fp8_e4m3fn_t (bias 7, no infinity, NaN = S.1111.111, max 448) and fp8_e5m2_t (bias 15, max 57344)
  * (ref: docs/zh/api/SIMD-API/基础API/数据结构/内置数据类型.md table 5). */
-typedef enum ascq_quant_dst { ASCQ_QDST_I8 = 0, ASCQ_QDST_FP8_E4M3FN = 1, ASCQ_QDST_FP8_E5M2 = 2 } ascq_quant_dst;
+typedef enum ascq_quant_dst {
+    ASCQ_QDST_I8 = 0,
+    ASCQ_QDST_FP8_E4M3FN = 1,
+    ASCQ_QDST_FP8_E5M2 = 2,
+    /* 4-bit floats, two per byte with the even element in the low nibble (the packing rule the reference states for
+     * int4x2 and both fp4x2 types together: docs/zh/api/SIMD-API/C-API/reg/reg_data_types/data_type_definition.md:17):
+     * sign, then e2m1 (bias 1; 0, 0.5, 1, 1.5, 2, 3, 4, 6) or e1m2 (bias 1; 0, 0.25 .. 1.75 in steps of 0.25). */
+    ASCQ_QDST_FP4_E2M1 = 3,
+    ASCQ_QDST_FP4_E1M2 = 4
+} ascq_quant_dst;
 
 typedef enum ascq_offset_kind { ASCQ_OFFSET_NONE = 0, ASCQ_OFFSET_SCALAR = 1, ASCQ_OFFSET_TENSOR = 2 } ascq_offset_kind;
 
@@ -103,7 +112,16 @@ typedef enum ascq_dequant_mode { ASCQ_DEQUANT_WITH_SINGLE_ROW = 0, ASCQ_DEQUANT_
  *               float, round-half-even, saturating to the largest finite value (448 / 57344); the reference falls
  *               back to this rounding for every round_mode
  *               (ref: impl/adv_api/detail/quantization/quant/ascend_quant_per_group_3510_impl.h:33-79,
- *               impl/adv_api/detail/quantization/quantize/quantize_impl.h:64-73).
+ *               impl/adv_api/detail/quantization/quantize/quantize_impl.h:64-73).  NaN gives +0, as the reference's
+ *               saturating casts do (docs/zh/api/附录/Reg矢量计算接口边界值汇总.md, rows float/fp8_e5m2_t; the table
+ *               leaves the e4m3 NaN cell empty, the same is done there).
+ * dst_format FP4_E2M1 / FP4_E1M2 (dst holds cal_count / 2 bytes): PER_GROUP with COMPUTE_SCALE_T only, (src, scale)
+ *               = (half, half), (half, float), (bfloat16, bfloat16), (bfloat16, float); v = cvt(x) * s in the scale
+ *               type, one rounding; the offset is not applied ("fp4 doesn't count offset"); then bf16(v) (half-even)
+ *               and bf16 -> fp4 with round_mode, saturating to +-6 / +-1.75, NaN -> +0.  n is a multiple of 8.
+ *               (ref: impl/adv_api/detail/quantization/quant/ascend_quant_per_group_3510_impl.h:346-379, 1383-1385;
+ *               ascend_quant_3510_impl.h:994-1032; boundary values: the table named above, rows
+ *               bfloat16_t/fp4x2_e2m1_t and bfloat16_t/fp4x2_e1m2_t.)
  */
 typedef struct ascq_quant_desc {
     int32_t policy;      /* ascq_policy */

@@ -57,6 +57,12 @@ struct fp8_e4m3fn_t {
 struct fp8_e5m2_t {
     uint8_t bits;
 };
+struct fp4x2_e2m1_t {  // two 4-bit floats per byte, even element in the low nibble
+    uint8_t pair;
+};
+struct fp4x2_e1m2_t {
+    uint8_t pair;
+};
 
 // destination types of AscendQuant
 template <typename T>
@@ -72,6 +78,14 @@ struct QuantDstOf<fp8_e4m3fn_t> {
 template <>
 struct QuantDstOf<fp8_e5m2_t> {
     static constexpr int32_t value = ASCQ_QDST_FP8_E5M2;
+};
+template <>
+struct QuantDstOf<fp4x2_e2m1_t> {  // AscendQuant PER_GROUP only
+    static constexpr int32_t value = ASCQ_QDST_FP4_E2M1;
+};
+template <>
+struct QuantDstOf<fp4x2_e1m2_t> {
+    static constexpr int32_t value = ASCQ_QDST_FP4_E1M2;
 };
 
 template <typename T>

@@ -18,9 +18,12 @@
  * Parity unpinned (no reference vector, document table or independent
  * implementation fixes these; the choice made is stated at the function):
  *   - the fixpipe int32 -> bf16 modes (defined by analogy with DEQF16);
- *   - NaN / Inf inputs, and fp16 overflow inside the half chains;
+ *   - NaN / Inf inputs of the int8 and half paths, and fp16 overflow inside the half chains;
  *   - fixpipe rounding for |acc| > 2^24, REQ8 offset signedness;
- *   - 8-bit float outputs from the largest finite value up (saturation).
+ *   - NaN -> fp8_e4m3fn (the reference's boundary table leaves that cell empty; +0 here, as for every other
+ *     saturating cast in that table);
+ *   - the nibble order of the fp4x2 types (the reference states one packing rule for int4x2 and both fp4x2 types;
+ *     its int4 data scripts fix "even element in the low nibble", no fp4 vector exists).
  */
 #include "ascq_oracle.h"
 
@@ -212,14 +215,16 @@ static double fp8_code_value(int code, int e5m2)
 
 /* fp32 -> 8-bit float by search: the nearest representable magnitude, ties to the even code, everything beyond the
  * largest finite value (infinity included) saturates to it (SatMode::SAT of the reference's cast trait,
- * ref: impl/adv_api/detail/quantization/quant/ascend_quant_per_group_3510_impl.h:41-42); NaN -> 0x7F with the sign. */
+ * ref: impl/adv_api/detail/quantization/quant/ascend_quant_per_group_3510_impl.h:41-42); NaN -> +0, the saturating
+ * cast's answer (ref: docs/zh/api/附录/Reg矢量计算接口边界值汇总.md, rows float/fp8_e5m2_t; the e4m3 NaN cell of that
+ * table is empty and is given the same answer here). */
 uint8_t orc_f32_to_fp8(float f, int e5m2)
 {
     int max_code = e5m2 ? 0x7B : 0x7E;
     uint8_t sign = signbit(f) ? 0x80 : 0;
     double a = fabs((double)f);
     if (f != f) {
-        return (uint8_t)(sign | 0x7F);
+        return 0;
     }
     if (a >= fp8_code_value(max_code, e5m2)) {
         return (uint8_t)(sign | max_code);
@@ -238,6 +243,55 @@ uint8_t orc_f32_to_fp8(float f, int e5m2)
         pick = lo + 1;
     } else {
         pick = (lo & 1) ? lo + 1 : lo;
+    }
+    return (uint8_t)(sign | pick);
+}
+
+/* The 8 magnitudes of the 4-bit floats, code 0..7 (sign in bit 3).  e2m1: exponent bias 1, one mantissa bit, code 0/1
+ * subnormal; e1m2: bias 1, two mantissa bits, codes 0..3 subnormal.  Largest values 6 and 1.75 as the reference's
+ * boundary table has them (docs/zh/api/附录/Reg矢量计算接口边界值汇总.md, rows bfloat16_t/fp4x2_e2m1_t, .../e1m2_t). */
+static const double kFp4E2M1[8] = {0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0};
+static const double kFp4E1M2[8] = {0.0, 0.25, 0.5, 0.75, 1.0, 1.25, 1.5, 1.75};
+
+float orc_fp4_to_f32(uint8_t code, int e1m2)
+{
+    double v = (e1m2 ? kFp4E1M2 : kFp4E2M1)[code & 7];
+    return (float)((code & 8) ? -v : v);
+}
+
+/* A (bfloat16) value -> 4-bit float by search over the 15 signed grid points: the two neighbours of the value, then
+ * the rounding mode picks one; beyond the largest magnitude (infinity included) the result saturates; NaN -> +0; a
+ * zero result keeps the sign of the input.  RINT ties go to the even code, ROUND ties away from zero.
+ * ref: impl/adv_api/detail/quantization/quant/ascend_quant_3510_impl.h:994-1032 (Cast<fp4, bfloat16_t, castTrait>,
+ * SatMode::SAT), boundary table named above. */
+uint8_t orc_f32_to_fp4(float f, int e1m2, int round_mode)
+{
+    const double* grid = e1m2 ? kFp4E1M2 : kFp4E2M1;
+    if (f != f) {
+        return 0;
+    }
+    uint8_t sign = signbit(f) ? 8 : 0;
+    double a = fabs((double)f);
+    if (a >= grid[7]) {
+        return (uint8_t)(sign | 7);
+    }
+    int lo = 0; /* largest code whose magnitude is <= a; lo + 1 exists because a < grid[7] */
+    for (int c = 1; c < 8; ++c) {
+        if (grid[c] <= a) {
+            lo = c;
+        }
+    }
+    if (grid[lo] == a) {
+        return (uint8_t)(sign | lo);
+    }
+    int pick;
+    double below = a - grid[lo], above = grid[lo + 1] - a;
+    switch (round_mode) {
+        case ASCQ_CAST_TRUNC: pick = lo; break;
+        case ASCQ_CAST_FLOOR: pick = sign ? lo + 1 : lo; break; /* towards minus infinity */
+        case ASCQ_CAST_CEIL: pick = sign ? lo : lo + 1; break;
+        case ASCQ_CAST_ROUND: pick = below < above ? lo : lo + 1; break;
+        default: pick = below < above ? lo : (below > above ? lo + 1 : ((lo & 1) ? lo + 1 : lo)); break;
     }
     return (uint8_t)(sign | pick);
 }
@@ -324,6 +378,13 @@ int orc_quant(const ascq_quant_desc* d, int8_t* dst, const void* src, const void
                              ascend_quant_per_group_3510_impl.h:54-74, quantize_impl.h:64-73 */
     }
     int rmode = (comp == ASCQ_COMPUTE_F16) ? ASCQ_CAST_RINT : d->round_mode;
+    const int fp4 = d->dst_format == ASCQ_QDST_FP4_E2M1 || d->dst_format == ASCQ_QDST_FP4_E1M2;
+    if (fp4) {
+        ctype = d->scale_dtype; /* the fp4 path multiplies in the scale type ...
+                                   ascend_quant_per_group_3510_impl.h:346-379 */
+    }
+    /* ... and is not given the offset ("fp4 doesn't count offset", :1384) */
+    const int offset_kind = fp4 ? (int)ASCQ_OFFSET_NONE : d->offset_kind;
 
 #pragma omp parallel for schedule(static) if (rows * n > 65536)
     for (size_t i = 0; i < rows; ++i) {
@@ -335,9 +396,9 @@ int orc_quant(const ascq_quant_desc* d, int8_t* dst, const void* src, const void
             } else {
                 s = load_as_f32(scale, quant_param_index(d, i, j), d->scale_dtype);
             }
-            if (d->offset_kind == ASCQ_OFFSET_SCALAR) {
+            if (offset_kind == ASCQ_OFFSET_SCALAR) {
                 o = d->offset;
-            } else if (d->offset_kind == ASCQ_OFFSET_TENSOR) {
+            } else if (offset_kind == ASCQ_OFFSET_TENSOR) {
                 o = load_as_f32(offset, quant_param_index(d, i, j), d->scale_dtype);
             }
             float x = load_as_f32(src, e, d->src_dtype);
@@ -345,19 +406,19 @@ int orc_quant(const ascq_quant_desc* d, int8_t* dst, const void* src, const void
             if (ctype == ASCQ_F16) {
                 uint16_t xh = orc_f32_to_f16(x); /* exact for a half source */
                 uint16_t t = orc_f16_mul(xh, orc_f32_to_f16(s));
-                if (comp == ASCQ_COMPUTE_F16 || d->offset_kind != ASCQ_OFFSET_NONE) {
+                if (comp == ASCQ_COMPUTE_F16 || offset_kind != ASCQ_OFFSET_NONE) {
                     t = orc_f16_add(t, orc_f32_to_f16(o)); /* the legacy op always executes Adds/Add */
                 }
                 v = (double)orc_f16_to_f32(t);
             } else if (ctype == ASCQ_BF16) {
                 uint16_t t = orc_bf16_mul(orc_f32_to_bf16(x), orc_f32_to_bf16(s));
-                if (d->offset_kind != ASCQ_OFFSET_NONE) {
+                if (offset_kind != ASCQ_OFFSET_NONE) {
                     t = orc_bf16_add(t, orc_f32_to_bf16(o));
                 }
                 v = (double)orc_bf16_to_f32(t);
             } else {
                 volatile float t = x * s; /* one fp32 rounding, never fused with the add */
-                if (d->offset_kind != ASCQ_OFFSET_NONE) {
+                if (offset_kind != ASCQ_OFFSET_NONE) {
                     volatile float t2 = t + o;
                     t = t2;
                 }
@@ -365,6 +426,13 @@ int orc_quant(const ascq_quant_desc* d, int8_t* dst, const void* src, const void
             }
             if (d->dst_format == ASCQ_QDST_I8) {
                 dst[e] = orc_round_sat8(v, rmode);
+            } else if (fp4) {
+                /* to bfloat16 first (half-even), then to the 4-bit float with the requested rounding; two codes per
+                 * byte, the even element in the low nibble.  Rows are whole bytes (n is even). */
+                float b = orc_bf16_to_f32(orc_f32_to_bf16((float)v));
+                uint8_t code = orc_f32_to_fp4(b, d->dst_format == ASCQ_QDST_FP4_E1M2, rmode);
+                uint8_t* byte = (uint8_t*)dst + e / 2;
+                *byte = (e & 1) ? (uint8_t)((*byte & 0x0F) | (code << 4)) : code;
             } else {
                 dst[e] = (int8_t)orc_f32_to_fp8((float)v, d->dst_format == ASCQ_QDST_FP8_E5M2);
             }

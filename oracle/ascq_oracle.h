@@ -29,6 +29,8 @@ float orc_quant_word_scale(uint64_t w, int scale_format);
 
 uint8_t orc_f32_to_fp8(float f, int e5m2);
 float orc_fp8_to_f32(uint8_t code, int e5m2);
+uint8_t orc_f32_to_fp4(float f, int e1m2, int round_mode);
+float orc_fp4_to_f32(uint8_t code, int e1m2);
 int orc_quant(const ascq_quant_desc* d, int8_t* dst, const void* src, const void* scale, const void* offset);
 int orc_dynamic_quant_per_token(int src_dtype, uint32_t m, uint32_t n, int8_t* q, float* tok_scale, const void* x);
 uint32_t orc_dequant_dst_stride(int dst_dtype, uint32_t n);

@@ -47,6 +47,10 @@ def lib():
         L.orc_quant_word_scale.argtypes = [C.c_uint64, C.c_int]
         L.orc_dequant_dst_stride.restype = C.c_uint32
         L.orc_dequant_dst_stride.argtypes = [C.c_int, C.c_uint32]
+        L.orc_f32_to_fp4.restype = C.c_uint8
+        L.orc_f32_to_fp4.argtypes = [C.c_float, C.c_int, C.c_int]
+        L.orc_fp4_to_f32.restype = C.c_float
+        L.orc_fp4_to_f32.argtypes = [C.c_uint8, C.c_int]
         L.orc_set_threads.argtypes = [C.c_int]
         L.orc_quant.argtypes = [C.POINTER(abi.QuantDesc), _P, _P, _P, _P]
         L.orc_dynamic_quant_per_token.argtypes = [C.c_int, C.c_uint32, C.c_uint32, _P, _P, _P]
@@ -134,6 +138,10 @@ def round_sat8(x, round_mode=abi.CAST_RINT):
 
 # ------------------------------------------------------------------ operators (host numpy arrays)
 def quant(desc, src, scale=None, offset=None):
+    if desc.dst_format in (abi.QDST_FP4_E2M1, abi.QDST_FP4_E1M2):
+        dst = np.zeros(src.size // 2, dtype=np.uint8)      # two codes per byte, even element in the low nibble
+        lib().orc_quant(C.byref(desc), _ptr(dst), _ptr(src), _ptr(scale), _ptr(offset))
+        return dst.reshape(*src.shape[:-1], src.shape[-1] // 2)
     dst = np.zeros(src.size, dtype=np.int8)
     lib().orc_quant(C.byref(desc), _ptr(dst), _ptr(src), _ptr(scale), _ptr(offset))
     return dst.reshape(src.shape)

@@ -160,6 +160,45 @@ void test_quant_per_token_fp8()
     expect_equal("AscendQuant fp8 per token", dq.download(), want);
 }
 
+void test_quant_per_group_fp4()
+{
+    std::printf("[case] AscendQuant<fp4x2_e2m1_t, half, float> PER_GROUP 12x256, groupSize 64, CAST_FLOOR\n");
+    Rng r{9};
+    const uint32_t m = 12, n = 256, gs = 64;
+    auto x = random_halves(r, m * n, -3.0f, 3.0f);
+    std::vector<float> sc(m * n / gs);
+    for (auto& e : sc) e = r.uniform(0.05f, 4.0f);  // the largest products pass 6 and saturate
+    DeviceBuffer<uint16_t> dx(x);
+    DeviceBuffer<float> dsc(sc);
+    DeviceBuffer<uint8_t> dq(m * n / 2);
+    ascq::AscendQuantConfig cfg{};
+    cfg.hasOffset = false;
+    cfg.roundMode = ascq::RoundMode::CAST_FLOOR;
+    ascq::AscendQuantParam para{};
+    para.m = m;
+    para.n = n;
+    para.calCount = m * n;
+    para.groupSize = gs;
+    ascq::AscendQuant(dq.view<ascq::fp4x2_e2m1_t>(m * n), dx.view<ascq::half>(m * n), dsc.view<float>(m * n / gs),
+                      dsc.view<float>(m * n / gs), para, cfg, ascq::AscendQuantPolicy::PER_GROUP);
+    ascq_quant_desc d{};
+    d.policy = ASCQ_PER_GROUP;
+    d.src_dtype = ASCQ_F16;
+    d.scale_dtype = ASCQ_F32;
+    d.compute = ASCQ_COMPUTE_SCALE_T;
+    d.round_mode = ASCQ_CAST_FLOOR;
+    d.offset_kind = ASCQ_OFFSET_NONE;
+    d.k_dim = 1;
+    d.m = m;
+    d.n = n;
+    d.cal_count = m * n;
+    d.group_size = gs;
+    d.dst_format = ASCQ_QDST_FP4_E2M1;
+    std::vector<uint8_t> want(m * n / 2);
+    orc_quant(&d, reinterpret_cast<int8_t*>(want.data()), x.data(), sc.data(), nullptr);
+    expect_equal("AscendQuant fp4 per group", dq.download(), want);
+}
+
 void test_dequant()
 {
     std::printf("[case] AscendDequant<bfloat16_t, float, MULTI_ROW> 32x40, calCount 36\n");
@@ -375,6 +414,7 @@ int main()
     std::printf("library: %s\n", ascq_version());
     test_quant_per_channel();
     test_quant_per_token_fp8();
+    test_quant_per_group_fp4();
     test_dequant();
     test_antiquant();
     test_matmul();

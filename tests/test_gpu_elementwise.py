@@ -194,6 +194,69 @@ def test_quant_fp8(fmt, pair, policy):
             assert np.any((got[:cal] & 0x7F) == top_code)          # saturation was exercised
 
 
+@pytest.mark.parametrize("fmt", [abi.QDST_FP4_E2M1, abi.QDST_FP4_E1M2])
+@pytest.mark.parametrize("pair", [(abi.F16, abi.F16), (abi.F16, abi.F32), (abi.BF16, abi.BF16), (abi.BF16, abi.F32)])
+@pytest.mark.parametrize("mode", [abi.CAST_RINT, abi.CAST_ROUND, abi.CAST_FLOOR, abi.CAST_CEIL, abi.CAST_TRUNC])
+@pytest.mark.parametrize("k_dim", [0, 1])
+def test_quant_fp4(fmt, pair, mode, k_dim):
+    """fp4x2_e2m1_t / fp4x2_e1m2_t outputs of AscendQuant PER_GROUP, every type pair of the reference's table and
+    every rounding mode: the packed bytes are bit-equal to the oracle's.  The scales put part of the data past the
+    largest magnitude and the data holds exact midpoints of the grid; the offset tensor is passed and must be ignored,
+    as in the reference."""
+    src_dt, sc_dt = pair
+    top = 6.0 if fmt == abi.QDST_FP4_E2M1 else 1.75
+    for (m, n, cal) in [(10, 288, 1152), (64, 512, 64 * 512), (6, 64, 6 * 64)]:
+        announce("quant fp4", fmt, pair, mode, k_dim, m, n, cal)
+        rng = np.random.default_rng(m + n + fmt + mode)
+        x, xd = src_array(rng, (m, n), src_dt, 1.0)
+        gs = 32
+        sshape = (m, -(-n // gs)) if k_dim == 1 else (-(-m // gs), n)
+        s = np.exp(rng.uniform(np.log(0.05), np.log(4 * top), sshape)).astype(np.float32)
+        if k_dim == 1:
+            s[0, 0] = 1.0                                        # this group keeps the midpoints planted below
+        else:
+            s[0, :10] = 1.0
+        (s, sdev) = typed(s, sc_dt)
+        mids = np.float32([0.25, 0.75, 1.25, 2.5, 5.0, -0.125, -0.375, -3.5, 7.0, -9.0])
+        if src_dt == abi.F16:
+            x[0, :10] = mids.astype(np.float16)
+            xd = to_dev(x)
+        else:
+            x[0, :10] = orc.f32_to_bf16_bits(mids)
+            xd = to_dev(x, "bf16")
+        o = rng.uniform(-3, 3, sshape).astype(np.float32)
+        (o, odev) = typed(o, sc_dt)
+        dst = torch.zeros(m * n // 2, dtype=torch.uint8, device=DEV)
+        cfg = ops.AscendQuantConfig(has_offset=True, k_dim=k_dim, round_mode=mode)
+        para = ops.AscendQuantParam(m=m, n=n, cal_count=cal, group_size=gs)
+        ops.ascend_quant_policy(dst, xd, sdev, odev, para, abi.PER_GROUP, cfg, dst_format=fmt)
+        d = abi.QuantDesc(policy=abi.PER_GROUP, src_dtype=src_dt, scale_dtype=sc_dt, compute=abi.COMPUTE_SCALE_T,
+                          round_mode=mode, k_dim=k_dim, m=m, n=n, cal_count=cal, group_size=gs, dst_format=fmt,
+                          offset_kind=abi.OFFSET_TENSOR)
+        want = orc.quant(d, x.reshape(-1)[:cal].copy(), s, o).reshape(-1)
+        got = dst.cpu().numpy()
+        assert np.array_equal(got[:cal // 2], want)
+        assert np.all(got[cal // 2:] == 0)
+        codes = np.concatenate([got[:cal // 2] & 15, got[:cal // 2] >> 4])
+        assert set(np.unique(codes & 7)) == set(range(8)) and np.any(codes & 8)    # every magnitude, both signs
+
+
+def test_quant_fp4_rejects():
+    announce("quant fp4 rejects")
+    x = torch.zeros((4, 64), dtype=torch.float16, device=DEV)
+    s = torch.ones((4, 2), dtype=torch.float16, device=DEV)
+    dst = torch.zeros(128, dtype=torch.uint8, device=DEV)
+    para = ops.AscendQuantParam(m=4, n=64, cal_count=256, group_size=32)
+    cfg = ops.AscendQuantConfig(has_offset=False, k_dim=1)
+    with pytest.raises(ops.AscqError, match="PER_GROUP only"):
+        ops.ascend_quant_policy(dst, x, s[:, 0].contiguous(), None, para, abi.PER_TOKEN, cfg,
+                                dst_format=abi.QDST_FP4_E2M1)
+    xf = torch.zeros((4, 64), dtype=torch.float32, device=DEV)
+    sf = torch.ones((4, 2), dtype=torch.float32, device=DEV)
+    with pytest.raises(ops.AscqError, match="half / bfloat16 sources"):
+        ops.ascend_quant_policy(dst, xf, sf, None, para, abi.PER_GROUP, cfg, dst_format=abi.QDST_FP4_E1M2)
+
+
 # ------------------------------------------------------------------ AscendDequant
 @pytest.mark.parametrize("dst_dt,sc_dt", [(abi.F16, abi.U64), (abi.F32, abi.F32), (abi.F32, abi.BF16),
                                           (abi.BF16, abi.BF16), (abi.BF16, abi.F32)])

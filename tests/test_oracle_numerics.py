@@ -164,5 +164,81 @@ def test_fp8_encode_matches_torch_in_range_and_saturates(e5m2):
     for v in (top, np.nextafter(np.float32(top), np.float32(np.inf)), top * 1.04, top * 2, 1e30, np.inf):
         assert L.orc_f32_to_fp8(float(v), e5m2) == top_code
         assert L.orc_f32_to_fp8(-float(v), e5m2) == 0x80 | top_code
-    assert L.orc_f32_to_fp8(float("nan"), e5m2) & 0x7F == 0x7F
+    # NaN -> +0: the saturation-mode column of the reference's boundary table for float -> fp8_e5m2_t
+    # (docs/zh/api/附录/Reg矢量计算接口边界值汇总.md); its e4m3 cell is empty and follows the same rule here
+    assert L.orc_f32_to_fp8(float("nan"), e5m2) == 0
 
+
+
+# ---------------------------------------------------------------- 4-bit floats (fp4x2_e2m1_t / fp4x2_e1m2_t)
+def _fp4_lib():
+    return orc.lib()
+
+
+@pytest.mark.parametrize("e1m2", [0, 1])
+def test_fp4_value_grid_and_the_reference_boundary_table(e1m2):
+    """The value sets of the two formats (e2m1 is the OCP microscaling FP4: 0, 0.5, 1, 1.5, 2, 3, 4, 6; e1m2 with the
+    same bias has 0 .. 1.75 in steps of 0.25), built here from sign / exponent / mantissa fields, and the rows
+    bfloat16_t/fp4x2_* of the reference's boundary table in saturation mode: MIN / -inf -> -max, MAX / inf -> +max,
+    nan -> 0.0 (docs/zh/api/附录/Reg矢量计算接口边界值汇总.md)."""
+    L = _fp4_lib()
+    ebits, mbits = (1, 2) if e1m2 else (2, 1)
+    for code in range(16):
+        e, m = (code >> mbits) & ((1 << ebits) - 1), code & ((1 << mbits) - 1)
+        mag = (m / (1 << mbits)) if e == 0 else (1 + m / (1 << mbits)) * 2.0 ** (e - 1)   # bias 1, e == 0 subnormal
+        want = -mag if code & 8 else mag
+        got = L.orc_fp4_to_f32(code, e1m2)
+        assert got == want and np.signbit(got) == bool(code & 8)
+        for mode in (abi.CAST_RINT, abi.CAST_FLOOR, abi.CAST_CEIL, abi.CAST_ROUND, abi.CAST_TRUNC):
+            assert L.orc_f32_to_fp4(want, e1m2, mode) == code          # representable values are fixed points
+    top = 1.75 if e1m2 else 6.0
+    bf16_max = float(np.float32(3.3895313892515355e38))
+    for mode in (abi.CAST_RINT, abi.CAST_FLOOR, abi.CAST_CEIL, abi.CAST_ROUND, abi.CAST_TRUNC):
+        for v in (bf16_max, float("inf"), top * 1.01, 8.0):
+            assert L.orc_fp4_to_f32(L.orc_f32_to_fp4(v, e1m2, mode), e1m2) == top
+            assert L.orc_fp4_to_f32(L.orc_f32_to_fp4(-v, e1m2, mode), e1m2) == -top
+        assert L.orc_f32_to_fp4(float("nan"), e1m2, mode) == 0
+        assert L.orc_f32_to_fp4(0.0, e1m2, mode) == 0
+
+
+def test_fp4_rounding_modes_known_answers():
+    """Midpoints and off-grid values worked by hand for each rounding mode: half-even goes to the even code (the one
+    whose mantissa bit is 0), ROUND away from zero, FLOOR / CEIL are directed on the signed value, TRUNC towards 0."""
+    L = _fp4_lib()
+    R, F, Cc, A, T = abi.CAST_RINT, abi.CAST_FLOOR, abi.CAST_CEIL, abi.CAST_ROUND, abi.CAST_TRUNC
+
+    def q(v, e1m2, mode):
+        return L.orc_fp4_to_f32(L.orc_f32_to_fp4(v, e1m2, mode), e1m2)
+
+    # e2m1: neighbours (0, .5) (.5, 1) (1, 1.5) (1.5, 2) (2, 3) (3, 4) (4, 6); even codes are 0, 1, 2, 4
+    for v, want in [(0.25, 0.0), (0.75, 1.0), (1.25, 1.0), (1.75, 2.0), (2.5, 2.0), (3.5, 4.0), (5.0, 4.0),
+                    (-0.25, -0.0), (-2.5, -2.0), (-5.0, -4.0), (0.26, 0.5), (2.49, 2.0), (2.51, 3.0), (5.01, 6.0)]:
+        assert q(v, 0, R) == want, (v, want)
+    for v, want in [(0.25, 0.5), (1.25, 1.5), (2.5, 3.0), (5.0, 6.0), (-0.25, -0.5), (-2.5, -3.0), (4.9, 4.0)]:
+        assert q(v, 0, A) == want, (v, want)
+    for v, f, c, t in [(0.3, 0.0, 0.5, 0.0), (2.2, 2.0, 3.0, 2.0), (5.9, 4.0, 6.0, 4.0), (-0.3, -0.5, -0.0, -0.0),
+                       (-2.2, -3.0, -2.0, -2.0), (-5.9, -6.0, -4.0, -4.0)]:
+        assert (q(v, 0, F), q(v, 0, Cc), q(v, 0, T)) == (f, c, t), v
+    # e1m2: a uniform grid of 0.25; even codes are the even multiples
+    for v, want in [(0.125, 0.0), (0.375, 0.5), (0.625, 0.5), (1.625, 1.5), (1.7, 1.75), (-0.875, -1.0)]:
+        assert q(v, 1, R) == want, (v, want)
+    for v, want in [(0.125, 0.25), (0.625, 0.75), (-0.875, -1.0), (-0.125, -0.25)]:
+        assert q(v, 1, A) == want, (v, want)
+    for v, f, c, t in [(0.3, 0.25, 0.5, 0.25), (-0.3, -0.5, -0.25, -0.25), (1.74, 1.5, 1.75, 1.5)]:
+        assert (q(v, 1, F), q(v, 1, Cc), q(v, 1, T)) == (f, c, t), v
+    # a zero result keeps the sign of the input
+    assert L.orc_f32_to_fp4(-0.1, 0, R) == 8 and L.orc_f32_to_fp4(-0.0, 1, R) == 8
+
+
+@pytest.mark.parametrize("e1m2", [0, 1])
+def test_fp4_rint_is_monotone_and_nearest(e1m2):
+    """Over a dense sweep: the result is one of the two neighbours, never farther than the other neighbour, and the
+    map is monotone."""
+    L = _fp4_lib()
+    xs = np.linspace(-7, 7, 5601).astype(np.float32)
+    out = np.array([L.orc_fp4_to_f32(L.orc_f32_to_fp4(float(v), e1m2, abi.CAST_RINT), e1m2) for v in xs])
+    assert np.all(np.diff(out) >= 0)
+    grid = np.array(sorted({L.orc_fp4_to_f32(c, e1m2) for c in range(16)}))
+    clipped = np.clip(xs, grid[0], grid[-1])
+    best = np.min(np.abs(clipped[:, None] - grid[None, :]), axis=1)
+    assert np.allclose(np.abs(out - clipped), best, atol=0)

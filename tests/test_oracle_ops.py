@@ -507,6 +507,42 @@ def test_quant_fp8_is_fp32_arithmetic_then_one_conversion(fmt, tdt, top, sc_dt):
         assert np.array_equal(orc.quant(d, x, s, o).view(np.uint8), want)
 
 
+@pytest.mark.parametrize("fmt", [abi.QDST_FP4_E2M1, abi.QDST_FP4_E1M2])
+@pytest.mark.parametrize("src_t,sc_t", [(torch.float16, torch.float16), (torch.float16, torch.float32),
+                                        (torch.bfloat16, torch.bfloat16), (torch.bfloat16, torch.float32)])
+@pytest.mark.parametrize("k_dim", [0, 1])
+def test_quant_fp4_is_a_product_in_the_scale_type_then_bf16_then_fp4(fmt, src_t, sc_t, k_dim):
+    """fp4 outputs (ascend_quant_per_group_3510_impl.h:346-379, ascend_quant_3510_impl.h:994-1032): the product is
+    formed in the scale's type by torch (an independent implementation of half / bfloat16 / float multiplication),
+    rounded to bfloat16 by torch, converted element by element with the scalar conversion pinned in
+    test_oracle_numerics.py, and packed with the even element in the low nibble; the offset must have no effect."""
+    rng = np.random.default_rng(fmt + k_dim)
+    m, n, gs = 64, 96, 32
+    xt = torch.from_numpy(rng.standard_normal((m, n)).astype(np.float32)).to(src_t)
+    sshape = (m, n // gs) if k_dim == 1 else (m // gs, n)
+    st = torch.from_numpy(rng.uniform(0.1, 8.0, sshape).astype(np.float32)).to(sc_t)
+    full = st.repeat_interleave(gs, dim=1) if k_dim == 1 else st.repeat_interleave(gs, dim=0)
+    prod = (xt.to(sc_t) * full).to(torch.bfloat16).to(torch.float32).numpy()
+    e1m2 = int(fmt == abi.QDST_FP4_E1M2)
+    L = orc.lib()
+    codes = np.array([L.orc_f32_to_fp4(float(v), e1m2, abi.CAST_ROUND) for v in prod.reshape(-1)], dtype=np.uint8)
+    want = (codes[0::2] | (codes[1::2] << 4)).astype(np.uint8)
+
+    def raw(t):
+        return t.view(torch.int16).numpy().view(np.uint16) if t.dtype != torch.float32 else t.numpy()
+
+    x_np = raw(xt) if src_t == torch.bfloat16 else xt.numpy()
+    s_np = raw(st) if sc_t == torch.bfloat16 else st.numpy()
+    o_np = (np.full(sshape, 5.0, dtype=np.float32) if sc_t == torch.float32
+            else raw(torch.full(sshape, 5.0).to(sc_t)) if sc_t == torch.bfloat16 else np.full(sshape, 5.0, np.float16))
+    d = abi.QuantDesc(policy=abi.PER_GROUP, src_dtype=abi.F16 if src_t == torch.float16 else abi.BF16,
+                      scale_dtype={torch.float16: abi.F16, torch.bfloat16: abi.BF16, torch.float32: abi.F32}[sc_t],
+                      compute=abi.COMPUTE_SCALE_T, round_mode=abi.CAST_ROUND, offset_kind=abi.OFFSET_TENSOR,
+                      k_dim=k_dim, m=m, n=n, cal_count=m * n, group_size=gs, dst_format=fmt)
+    got = orc.quant(d, x_np, s_np, o_np)
+    assert got.shape == (m, n // 2) and np.array_equal(got.reshape(-1), want)
+
+
 # ------------------------------------------------------------------ AscendAntiQuant PER_TOKEN / PER_GROUP
 def _b8_source(rng, fmt, shape):
     """Random one-byte sources (no NaN / infinity codes) and their exact fp32 values."""
