@@ -829,14 +829,15 @@ __device__ __forceinline__ void aqp_params8(const AntiQuantPolicyArgs& a, const 
     for (int e = 0; e < 8; ++e) p[e] = s;
 }
 
-// fp32 -> destination with the reference's saturating cast for 16-bit outputs
+// fp32 -> destination with the reference's saturating cast for 16-bit outputs: infinity and everything beyond the
+// largest finite value give that value, NaN gives +0
 template <int kDst>
 __device__ __forceinline__ float aqp_saturate(float v)
 {
     if constexpr (kDst == ASCQ_F16) {
-        return (v != v) ? v : fminf(fmaxf(v, -65504.0f), 65504.0f);
+        return (v != v) ? 0.0f : fminf(fmaxf(v, -65504.0f), 65504.0f);
     } else if constexpr (kDst == ASCQ_BF16) {
-        return (v != v) ? v : fminf(fmaxf(v, -3.3895313892515355e38f), 3.3895313892515355e38f);
+        return (v != v) ? 0.0f : fminf(fmaxf(v, -3.3895313892515355e38f), 3.3895313892515355e38f);
     } else {
         return v;
     }

@@ -823,11 +823,16 @@ int orc_matmul_w4a16_cols(const ascq_w4a16_desc* d, uint16_t* y, const uint16_t*
 /* ------------------------------------- AscendAntiQuant PER_TOKEN / PER_GROUP */
 /* One-byte sources (int8, fp8_e4m3fn, fp8_e5m2): the source is converted to the compute type (exact for every source
  * value), the offset is added and the scale multiplied in that type, one rounding each; an fp32 result going to a
- * 16-bit destination is rounded half-even and saturates (LayoutZMrgZRndRSatS).
+ * 16-bit destination is rounded half-even and saturates (LayoutZMrgZRndRSatS): beyond the largest finite value, and
+ * infinity, give that value, NaN gives +0 (ref: docs/zh/api/附录/Reg矢量计算接口边界值汇总.md, saturation-mode column
+ * of the rows float/half and float/bfloat16_t).
  * ref: impl/adv_api/detail/quantization/antiquant/ascend_antiquant_3510_impl.h:1386-1403 (ConvertSrc),
  *      :1458-1495 (per token), :2176-2222 (group axis = kDim XOR isTranspose); fp32 arithmetic for AntiQuantize. */
 static uint16_t f32_to_f16_sat(float v)
 {
+    if (v != v) {
+        return 0;
+    }
     if (v == v && v > 65504.0f) {
         v = 65504.0f;
     }
@@ -840,6 +845,9 @@ static uint16_t f32_to_f16_sat(float v)
 static uint16_t f32_to_bf16_sat(float v)
 {
     const float top = 3.3895313892515355e38f; /* largest finite bfloat16 */
+    if (v != v) {
+        return 0;
+    }
     if (v == v && v > top) {
         v = top;
     }

@@ -406,6 +406,36 @@ def test_antiquant_policy(fmt, types, mode):
         assert not got[rows:].any()
 
 
+@pytest.mark.parametrize("fmt", [abi.QDST_FP8_E4M3FN, abi.QDST_FP8_E5M2])
+@pytest.mark.parametrize("dst_dt", [abi.F16, abi.BF16])
+def test_antiquant_policy_nan_and_infinity_codes_through_the_saturating_cast(fmt, dst_dt):
+    """fp8 sources that are NaN or infinity, fp32 arithmetic, 16-bit destination: the saturating cast gives the
+    largest finite value for infinities and +0 for NaN (the saturation-mode column of the reference's boundary table,
+    rows float/half and float/bfloat16_t); bit-equal to the oracle, and the expected patterns spelt out."""
+    announce("antiquant policy nan/inf", fmt, dst_dt)
+    m, n = 8, 64
+    codes = np.full((m, n), 0x3C, dtype=np.uint8)
+    nan_codes = [0x7F, 0xFF] if fmt == abi.QDST_FP8_E4M3FN else [0x7D, 0x7E, 0x7F, 0xFD]
+    inf_codes = [] if fmt == abi.QDST_FP8_E4M3FN else [0x7C, 0xFC]
+    special = nan_codes + inf_codes
+    codes[0, :len(special)] = special
+    s = np.full(m, 2.0, dtype=np.float32)
+    dst = torch.zeros((m, n), dtype=TDT[dst_dt], device=DEV)
+    cfg = ops.AscendAntiQuantConfig(has_offset=False, is_transpose=False, k_dim=1)
+    para = ops.AscendAntiQuantParam(m=m, n=n, cal_count=m * n, group_size=0)
+    ops.ascend_antiquant_policy(dst, to_dev(codes).view(B8[fmt]), to_dev(s), None, para, abi.PER_TOKEN, cfg)
+    d = abi.AntiQuantPolicyDesc(policy=abi.PER_TOKEN, src_format=fmt, scale_dtype=abi.F32, dst_dtype=dst_dt,
+                                compute=abi.COMPUTE_SCALE_T, has_offset=0, is_transpose=0, k_dim=1, m=m, n=n,
+                                cal_count=m * n, group_size=0)
+    want = orc.antiquant_policy(d, codes, s, None)
+    want = want.view(np.uint16) if want.dtype == np.float16 else want
+    got = bits(dst)
+    assert np.array_equal(got, want)
+    top = 0x7BFF if dst_dt == abi.F16 else 0x7F7F
+    assert list(got[0, :len(nan_codes)]) == [0] * len(nan_codes)
+    assert list(got[0, len(nan_codes):len(special)]) == [top, 0x8000 | top][:len(inf_codes)]
+
+
 def test_antiquant_per_tensor():
     announce("antiquant per-tensor")
     w = np.arange(-128, 128, dtype=np.int8).reshape(8, 32)
