@@ -56,7 +56,8 @@ class AntiQuantDesc(C.Structure):
 class AntiQuantPolicyDesc(C.Structure):
     _fields_ = [("policy", C.c_int32), ("src_format", C.c_int32), ("scale_dtype", C.c_int32), ("dst_dtype", C.c_int32),
                 ("compute", C.c_int32), ("has_offset", C.c_int32), ("is_transpose", C.c_int32), ("k_dim", C.c_int32),
-                ("m", C.c_uint32), ("n", C.c_uint32), ("cal_count", C.c_uint32), ("group_size", C.c_uint32)]
+                ("m", C.c_uint32), ("n", C.c_uint32), ("cal_count", C.c_uint32), ("group_size", C.c_uint32),
+                ("scale", C.c_float), ("offset", C.c_float)]
 
 
 class MatmulDesc(C.Structure):

@@ -208,10 +208,15 @@ class AscendAntiQuantParam:
 
 
 def _antiquant_policy(compute, dst, src, scale, offset, para, policy, config):
-    d = abi.AntiQuantPolicyDesc(policy=policy, src_format=_QDST[src.dtype], scale_dtype=_dt(scale), dst_dtype=_dt(dst),
+    d = abi.AntiQuantPolicyDesc(policy=policy, src_format=_QDST[src.dtype], dst_dtype=_dt(dst),
                                 compute=compute, has_offset=int(config.has_offset),
                                 is_transpose=int(config.is_transpose), k_dim=config.k_dim, m=para.m, n=para.n,
                                 cal_count=para.cal_count, group_size=para.group_size)
+    if policy == abi.PER_TENSOR:
+        d.scale_dtype, d.scale, d.offset = _dt(dst), float(scale), float(offset) if config.has_offset else 0.0
+        scale = offset = None
+    else:
+        d.scale_dtype = _dt(scale)
     check(load_library().ascq_antiquant_policy(C.byref(d), _ptr(dst), _ptr(src), _ptr(scale),
                                                _ptr(offset) if config.has_offset else None, _stream()))
     return dst
@@ -225,8 +230,23 @@ def ascend_antiquant_policy(dst, src, scale, offset, para, policy, config=Ascend
 
 
 def antiquantize(dst, src, scale, offset, para, policy, config=AscendAntiQuantConfig()):
-    """AntiQuantize: the same with fp32 arithmetic whatever the parameter type."""
+    """AntiQuantize<config>(dst, src, scale, offset, params): fp32 arithmetic whatever the parameter type, any policy.
+    PER_TENSOR takes Python floats (values of the output's type), PER_CHANNEL tensors [n] of the output's type.
+    ref: include/adv_api/quantization/antiquantize.h:59-95, impl/adv_api/detail/quantization/antiquantize/
+    antiquantize_impl.h:36-135."""
     return _antiquant_policy(abi.COMPUTE_F32, dst, src, scale, offset, para, policy, config)
+
+
+def dequantize(dst, src, scale, para, policy, k_dim=1):
+    """Dequantize<config>(dst, src, scale, offset, params) (the offset is not supported by the reference either):
+    PER_TENSOR (scale a Python float) and PER_CHANNEL are AscendDequant in DEQUANT_WITH_MULTI_ROW mode on {m, n, n},
+    PER_TOKEN / PER_GROUP the policy form.  `para` has m, n (and group_size for PER_GROUP).
+    ref: impl/adv_api/detail/quantization/dequantize/dequantize_impl.h:94-196."""
+    if policy in (abi.PER_TENSOR, abi.PER_CHANNEL):
+        return ascend_dequant(dst, src, scale, DequantParams(m=para.m, n=para.n, cal_count=para.n),
+                              mode=abi.DEQUANT_WITH_MULTI_ROW)
+    p = AscendQuantParam(m=para.m, n=para.n, cal_count=para.m * para.n, group_size=getattr(para, "group_size", 0))
+    return ascend_dequant_policy(dst, src, scale, p, policy, k_dim=k_dim)
 
 
 # ------------------------------------------------------------------------------------------ Matmul quant path

@@ -801,6 +801,7 @@ struct AntiQuantPolicyArgs {
     uint32_t rows, n;
     int policy, along_n, has_offset, src_format;
     uint32_t group_size, params_per_row;
+    float sscale, soffset;  // PER_TENSOR
 };
 
 // int8 / fp8_e4m3fn / fp8_e5m2 byte -> fp32 (exact); the 8-bit floats go through the hardware converters
@@ -815,11 +816,17 @@ __device__ __forceinline__ float decode_b8(uint32_t word, int byte, int fmt)
 }
 
 template <int kPar>
-__device__ __forceinline__ void aqp_params8(const AntiQuantPolicyArgs& a, const void* base, uint32_t i, uint32_t j,
-                                            float (&p)[8])
+__device__ __forceinline__ void aqp_params8(const AntiQuantPolicyArgs& a, const void* base, bool is_offset, uint32_t i,
+                                            uint32_t j, float (&p)[8])
 {
     if (a.policy == ASCQ_PER_GROUP && !a.along_n) {
         load8<kPar>(base, static_cast<size_t>(i / a.group_size) * a.n + j, p);
+        return;
+    }
+    if (a.policy == ASCQ_PER_TENSOR) {
+        const float s = is_offset ? a.soffset : a.sscale;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) p[e] = s;
         return;
     }
     const float s = a.policy == ASCQ_PER_TOKEN
@@ -866,9 +873,9 @@ __global__ __launch_bounds__(kThreads) void antiquant_policy_vec_kernel(AntiQuan
                 break;
             }
             float s[8], o[8], v[8];
-            aqp_params8<kPar>(a, a.scale, r, j, s);
+            aqp_params8<kPar>(a, a.scale, false, r, j, s);
             if (a.has_offset) {
-                aqp_params8<kPar>(a, a.offset, r, j, o);
+                aqp_params8<kPar>(a, a.offset, true, r, j, o);
             }
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
@@ -900,11 +907,12 @@ __global__ __launch_bounds__(kThreads) void antiquant_policy_scalar_kernel(AntiQ
         } else {
             pi = static_cast<size_t>(i / a.group_size) * a.n + j;
         }
+        const bool scalar = a.policy == ASCQ_PER_TENSOR;
         float t = decode_b8(a.src[e], 0, a.src_format);
         if (a.has_offset) {
-            t = Fmt<kCt>::add(t, Fmt<kCt>::cvt(load1<kPar>(a.offset, pi)));
+            t = Fmt<kCt>::add(t, Fmt<kCt>::cvt(scalar ? a.soffset : load1<kPar>(a.offset, pi)));
         }
-        t = Fmt<kCt>::mul(t, Fmt<kCt>::cvt(load1<kPar>(a.scale, pi)));
+        t = Fmt<kCt>::mul(t, Fmt<kCt>::cvt(scalar ? a.sscale : load1<kPar>(a.scale, pi)));
         store1<kDst>(a.dst, e, kCt == kDst ? t : aqp_saturate<kDst>(t));
     }
 }
@@ -1131,9 +1139,23 @@ extern "C" int ascq_dequant(const ascq_dequant_desc* d, void* dst, const void* s
     ASCQ_REQUIRE(d->n > 0 && d->m > 0, ASCQ_EINVAL, "ascq_dequant: m and n must be greater than 0");
     ASCQ_REQUIRE((d->n * 4u) % 32 == 0, ASCQ_EALIGN, "ascq_dequant: a source row (n=%u int32) must be 32-byte aligned",
                  d->n);
-    ASCQ_REQUIRE(d->cal_count <= d->n, ASCQ_EINVAL, "ascq_dequant: calCount %u must not exceed n %u", d->cal_count,
-                 d->n);
     uint32_t m = d->m, n = d->n, cal = d->cal_count, ppr = 0;
+    if (legacy) {
+        ASCQ_REQUIRE(d->cal_count <= d->n, ASCQ_EINVAL, "ascq_dequant: calCount %u must not exceed n %u", d->cal_count,
+                     d->n);
+    } else {
+        // the policy form counts elements: the first calCount / n rows are processed, every column of them scaled
+        // (ref: impl/adv_api/detail/quantization/dequant/ascend_dequant_3510_impl.h:230, 272, 341, 397, 533, 601)
+        ASCQ_REQUIRE(d->cal_count % d->n == 0, ASCQ_EINVAL,
+                     "ascq_dequant: calCount %u must be an integer multiple of n %u", d->cal_count, d->n);
+        ASCQ_REQUIRE(static_cast<uint64_t>(d->m) * d->n >= d->cal_count, ASCQ_EINVAL,
+                     "ascq_dequant: calCount %u exceeds m*n = %u*%u", d->cal_count, d->m, d->n);
+        m = d->cal_count / d->n;
+        cal = n;
+        if (m == 0) {
+            return ASCQ_OK;
+        }
+    }
     if (legacy && d->mode == ASCQ_DEQUANT_WITH_SINGLE_ROW) {
         const uint32_t per_blk = (d->dst_dtype == ASCQ_F32) ? 8u : 16u;
         if (m == 1 && cal != 0 && cal % per_blk == 0 && n % cal == 0) {
@@ -1249,11 +1271,22 @@ extern "C" int ascq_antiquant_policy(const ascq_antiquant_policy_desc* d, void* 
                                      const void* scale, const void* offset, void* stream)
 {
     ASCQ_REQUIRE(d != nullptr, ASCQ_ENULL, "ascq_antiquant_policy: desc is NULL");
-    ASCQ_REQUIRE(dst != nullptr && src != nullptr && scale != nullptr, ASCQ_ENULL,
+    const bool per_tensor = d->policy == ASCQ_PER_TENSOR, per_channel = d->policy == ASCQ_PER_CHANNEL;
+    ASCQ_REQUIRE(dst != nullptr && src != nullptr && (per_tensor || scale != nullptr), ASCQ_ENULL,
                  "ascq_antiquant_policy: dst / src / scale is NULL");
-    ASCQ_REQUIRE(!d->has_offset || offset != nullptr, ASCQ_ENULL, "ascq_antiquant_policy: offset tensor is NULL");
-    ASCQ_REQUIRE(d->policy == ASCQ_PER_TOKEN || d->policy == ASCQ_PER_GROUP, ASCQ_EUNSUPPORTED,
-                 "ascq_antiquant_policy: policy %d is not PER_TOKEN / PER_GROUP", d->policy);
+    ASCQ_REQUIRE(!d->has_offset || per_tensor || offset != nullptr, ASCQ_ENULL,
+                 "ascq_antiquant_policy: offset tensor is NULL");
+    ASCQ_REQUIRE(d->policy >= ASCQ_PER_TENSOR && d->policy <= ASCQ_PER_GROUP, ASCQ_EINVAL,
+                 "ascq_antiquant_policy: unknown policy %d", d->policy);
+    if (per_tensor || per_channel) {
+        // ref: antiquantize_impl.h:42-45 (scale type == dst type, half or bfloat16), 70-110
+        ASCQ_REQUIRE(d->compute == ASCQ_COMPUTE_F32, ASCQ_EUNSUPPORTED,
+                     "ascq_antiquant_policy: PER_TENSOR / PER_CHANNEL exist for AntiQuantize (fp32 arithmetic) only");
+        ASCQ_REQUIRE((d->dst_dtype == ASCQ_F16 || d->dst_dtype == ASCQ_BF16) && d->scale_dtype == d->dst_dtype,
+                     ASCQ_EUNSUPPORTED,
+                     "ascq_antiquant_policy: PER_TENSOR / PER_CHANNEL take half or bfloat16 parameters of the output's "
+                     "type (scale dtype %d, dst dtype %d)", d->scale_dtype, d->dst_dtype);
+    }
     ASCQ_REQUIRE(d->src_format >= ASCQ_QDST_I8 && d->src_format <= ASCQ_QDST_FP8_E5M2, ASCQ_EUNSUPPORTED,
                  "ascq_antiquant_policy: source format %d is not int8 / fp8_e4m3fn / fp8_e5m2", d->src_format);
     const int par = d->scale_dtype, dt = d->dst_dtype;
@@ -1289,9 +1322,31 @@ extern "C" int ascq_antiquant_policy(const ascq_antiquant_policy_desc* d, void* 
     ASCQ_REQUIRE(!ranges_overlap(dst, static_cast<size_t>(d->cal_count) * dtype_size(dt), src, d->cal_count),
                  ASCQ_EINVAL, "ascq_antiquant_policy: dst overlaps src");
     AntiQuantPolicyArgs a{dst, static_cast<const uint8_t*>(src), scale, offset, d->cal_count / d->n, d->n, d->policy,
-                          along_n, d->has_offset ? 1 : 0, d->src_format, d->group_size ? d->group_size : 1u, ppr};
-    const bool vec = (reinterpret_cast<uintptr_t>(src) & 7u) == 0 && aligned16(dst) && aligned16(scale) &&
-                     (!d->has_offset || aligned16(offset));
+                          along_n, d->has_offset ? 1 : 0, d->src_format, d->group_size ? d->group_size : 1u, ppr,
+                          0.0f, 0.0f};
+    if (per_channel) {
+        // one parameter row for every data row: a group along m that is never left
+        a.policy = ASCQ_PER_GROUP;
+        a.along_n = 0;
+        a.group_size = 0xFFFFFFFFu;
+    }
+    if (per_tensor) {
+        // the scalars arrive as values of the output type
+        auto round_to = [&](float f) {
+            if (dt == ASCQ_F16) {
+                return static_cast<float>(static_cast<_Float16>(f));
+            }
+            uint32_t u;
+            __builtin_memcpy(&u, &f, 4);
+            u = (u + 0x7FFFu + ((u >> 16) & 1u)) & 0xFFFF0000u;
+            __builtin_memcpy(&f, &u, 4);
+            return f;
+        };
+        a.sscale = round_to(d->scale);
+        a.soffset = round_to(d->offset);
+    }
+    const bool vec = (reinterpret_cast<uintptr_t>(src) & 7u) == 0 && aligned16(dst) &&
+                     (per_tensor || (aligned16(scale) && (!d->has_offset || aligned16(offset))));
     hipStream_t st = static_cast<hipStream_t>(stream);
 #define ASCQ_AQP(P, C, D)                                         \
     if (par == (P) && ct == (C) && dt == (D)) {                   \

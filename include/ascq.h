@@ -163,6 +163,9 @@ int ascq_dynamic_quant_per_token(int32_t src_dtype, uint32_t m, uint32_t n, void
  *   n <= j < n_dst: not written.
  * scale: PER_TENSOR scalar `scale`; PER_CHANNEL tensor [>=cal_count] of F32 | BF16 | U64
  * (U64: the low 32 bits are the fp32 scale); PER_TOKEN [m]; PER_GROUP as for quant.
+ * PER_TOKEN / PER_GROUP (AscendDeQuantParam): cal_count counts elements, a multiple of n and at most m * n; the
+ * first cal_count / n rows are processed and every column of them is scaled (ref: impl/adv_api/detail/quantization/
+ * dequant/ascend_dequant_3510_impl.h:230, 341, 533).
  * SINGLE_ROW mode applies the reference's {1, m*n, n} -> {m, n, n} reshape rule.
  */
 typedef struct ascq_dequant_desc {
@@ -220,10 +223,15 @@ int ascq_antiquant(const ascq_antiquant_desc* desc, void* dst, const void* src, 
  *   v = ct(src) ; v = ct(v + offset) if has_offset ; v = ct(v * scale) ; dst = dstT(v)
  * with ct = the scale dtype (ASCQ_COMPUTE_SCALE_T: AscendAntiQuant) or fp32 (ASCQ_COMPUTE_F32: AntiQuantize); every
  * source value is exact in every ct.  A 16-bit ct requires dst_dtype == scale_dtype; an fp32 result is rounded
- * half-even to a 16-bit dst, saturating at the largest finite value.
+ * half-even to a 16-bit dst, saturating at the largest finite value (NaN -> +0).
+ *   PER_CHANNEL (AntiQuantize only, ASCQ_COMPUTE_F32): scale / offset [n] of dst_dtype (half | bfloat16).
+ *   PER_TENSOR  (AntiQuantize only, ASCQ_COMPUTE_F32): the scalars `scale` / `offset` of the descriptor, taken as
+ *              dst_dtype values (rounded once to it); the scale / offset pointers are ignored.
+ *              (ref: impl/adv_api/detail/quantization/antiquantize/antiquantize_impl.h:42-45, 70-110;
+ *               antiquantize_3510_impl.h:253-362: fp32 arithmetic, saturating cast to half / bfloat16.)
  */
 typedef struct ascq_antiquant_policy_desc {
-    int32_t policy;      /* ASCQ_PER_TOKEN | ASCQ_PER_GROUP */
+    int32_t policy;      /* ASCQ_PER_TOKEN | ASCQ_PER_GROUP; with ASCQ_COMPUTE_F32 also PER_TENSOR | PER_CHANNEL */
     int32_t src_format;  /* ASCQ_QDST_I8 | ASCQ_QDST_FP8_E4M3FN | ASCQ_QDST_FP8_E5M2 */
     int32_t scale_dtype; /* ASCQ_F16 | ASCQ_BF16 | ASCQ_F32: dtype of the scale / offset tensors */
     int32_t dst_dtype;   /* ASCQ_F16 | ASCQ_BF16 | ASCQ_F32 */
@@ -234,6 +242,7 @@ typedef struct ascq_antiquant_policy_desc {
     uint32_t m, n;
     uint32_t cal_count;
     uint32_t group_size; /* PER_GROUP: positive multiple of 32 */
+    float scale, offset; /* PER_TENSOR scalars */
 } ascq_antiquant_policy_desc;
 
 int ascq_antiquant_policy(const ascq_antiquant_policy_desc* desc, void* dst, const void* src, const void* scale,

@@ -323,6 +323,195 @@ void AscendAntiQuant(const DeviceTensor<dstT>& dstTensor, const DeviceTensor<src
                                 config.hasOffset ? offsetTensor.GetPhyAddr() : nullptr, stream));
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// AscendDequant<dstT, srcT, scaleT, config, policy> for PER_TOKEN / PER_GROUP (ref: ascend_dequant.h:284-305,
+// ascend_dequant_utils.h:32-44); srcT int32_t or float; the offset tensor is accepted and unused, as in the reference.
+struct AscendDeQuantConfig {
+    bool hasOffset = false;
+    int32_t kDim = 1;
+};
+enum class AscendDeQuantPolicy : int32_t { PER_TENSOR, PER_CHANNEL, PER_TOKEN, PER_GROUP };
+struct AscendDeQuantParam {
+    uint32_t m;
+    uint32_t n;
+    uint32_t calCount;
+    uint32_t groupSize = 0;
+};
+template <typename dstT, typename srcT, typename scaleT>
+void AscendDequant(const DeviceTensor<dstT>& dstTensor, const DeviceTensor<srcT>& srcTensor,
+                   const DeviceTensor<scaleT>& scaleTensor, const DeviceTensor<scaleT>& /*offsetTensor*/,
+                   const AscendDeQuantParam& para, const AscendDeQuantConfig& config, AscendDeQuantPolicy policy,
+                   void* stream = nullptr)
+{
+    ascq_dequant_desc d{};
+    d.policy = static_cast<int32_t>(policy);
+    d.src_dtype = DTypeOf<srcT>::value;
+    d.scale_dtype = DTypeOf<scaleT>::value;
+    d.dst_dtype = DTypeOf<dstT>::value;
+    d.mode = ASCQ_DEQUANT_WITH_MULTI_ROW;
+    d.k_dim = config.kDim;
+    d.m = para.m;
+    d.n = para.n;
+    d.cal_count = para.calCount;
+    d.group_size = para.groupSize;
+    Check(ascq_dequant(&d, dstTensor.GetPhyAddr(), srcTensor.GetPhyAddr(), scaleTensor.GetPhyAddr(), stream));
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// The unified surface: Quantize / Dequantize / AntiQuantize, one config type each with the policy inside
+// (ref: include/adv_api/quantization/quantize.h:53-90, quantize_utils.h:32-45; dequantize.h:57-91,
+// impl/adv_api/detail/quantization/dequantize/dequantize_common.h:26-45; antiquantize.h:59-95,
+// .../antiquantize/antiquantize_common.h:26-45).  The reference passes the config as a template argument; it is an
+// ordinary argument here.  Tensor parameters for every policy but PER_TENSOR, which takes scalars.
+enum class QuantizePolicy : int32_t { PER_TENSOR, PER_CHANNEL, PER_TOKEN, PER_GROUP };
+struct QuantizeConfig {
+    QuantizePolicy policy;
+    bool hasOffset;
+    RoundMode roundMode = RoundMode::CAST_RINT;
+    int32_t kDim = 1;
+};
+struct QuantizeParams {
+    uint32_t m;
+    uint32_t n;
+    uint32_t groupSize = 0;
+};
+// Always fp32 arithmetic (ref: impl/adv_api/detail/quantization/quantize/quantize_impl.h:641-968).
+template <typename DstT, typename SrcT, typename ScaleT>
+void Quantize(const DeviceTensor<DstT>& dstTensor, const DeviceTensor<SrcT>& srcTensor,
+              const DeviceTensor<ScaleT>& scale, const DeviceTensor<ScaleT>& offset, const QuantizeParams& params,
+              const QuantizeConfig& config, void* stream = nullptr)
+{
+    ascq_quant_desc d{};
+    d.policy = static_cast<int32_t>(config.policy);
+    d.src_dtype = DTypeOf<SrcT>::value;
+    d.scale_dtype = DTypeOf<ScaleT>::value;
+    d.compute = ASCQ_COMPUTE_F32;
+    d.round_mode = static_cast<int32_t>(config.roundMode);
+    d.offset_kind = config.hasOffset ? ASCQ_OFFSET_TENSOR : ASCQ_OFFSET_NONE;
+    d.k_dim = config.kDim;
+    d.m = params.m;
+    d.n = params.n;
+    d.cal_count = params.m * params.n;
+    d.group_size = params.groupSize;
+    d.dst_format = QuantDstOf<DstT>::value;
+    Check(ascq_quant(&d, dstTensor.GetPhyAddr(), srcTensor.GetPhyAddr(), scale.GetPhyAddr(),
+                     config.hasOffset ? offset.GetPhyAddr() : nullptr, stream));
+}
+template <typename DstT, typename SrcT>
+void Quantize(const DeviceTensor<DstT>& dstTensor, const DeviceTensor<SrcT>& srcTensor, float scale, float offset,
+              const QuantizeParams& params, const QuantizeConfig& config, void* stream = nullptr)
+{
+    ascq_quant_desc d{};
+    d.policy = ASCQ_PER_TENSOR;
+    d.src_dtype = DTypeOf<SrcT>::value;
+    d.scale_dtype = DTypeOf<SrcT>::value;
+    d.compute = ASCQ_COMPUTE_F32;
+    d.round_mode = static_cast<int32_t>(config.roundMode);
+    d.offset_kind = config.hasOffset ? ASCQ_OFFSET_SCALAR : ASCQ_OFFSET_NONE;
+    d.scale = scale;
+    d.offset = offset;
+    d.m = params.m;
+    d.n = params.n;
+    d.cal_count = params.m * params.n;
+    d.dst_format = QuantDstOf<DstT>::value;
+    Check(ascq_quant(&d, dstTensor.GetPhyAddr(), srcTensor.GetPhyAddr(), nullptr, nullptr, stream));
+}
+
+enum class DequantizePolicy : int32_t { PER_TENSOR, PER_CHANNEL, PER_TOKEN, PER_GROUP };
+struct DequantizeConfig {
+    DequantizePolicy policy;
+    bool hasOffset = false;  // not supported by the reference either
+    int32_t kDim = 1;
+};
+struct DequantizeParams {
+    uint32_t m;
+    uint32_t n;
+    uint32_t groupSize = 0;
+};
+// PER_CHANNEL is AscendDequant in DEQUANT_WITH_MULTI_ROW mode on {m, n, n}; PER_TOKEN / PER_GROUP the policy form
+// (ref: impl/adv_api/detail/quantization/dequantize/dequantize_impl.h:117-196).
+template <typename DstT, typename SrcT, typename ScaleT>
+void Dequantize(const DeviceTensor<DstT>& dstTensor, const DeviceTensor<SrcT>& srcTensor,
+                const DeviceTensor<ScaleT>& scale, const DeviceTensor<ScaleT>& /*offset*/,
+                const DequantizeParams& params, const DequantizeConfig& config, void* stream = nullptr)
+{
+    ascq_dequant_desc d{};
+    d.policy = static_cast<int32_t>(config.policy);
+    d.src_dtype = DTypeOf<SrcT>::value;
+    d.scale_dtype = DTypeOf<ScaleT>::value;
+    d.dst_dtype = DTypeOf<DstT>::value;
+    d.mode = ASCQ_DEQUANT_WITH_MULTI_ROW;
+    d.k_dim = config.kDim;
+    d.m = params.m;
+    d.n = params.n;
+    d.cal_count = config.policy == DequantizePolicy::PER_CHANNEL ? params.n : params.m * params.n;
+    d.group_size = params.groupSize;
+    Check(ascq_dequant(&d, dstTensor.GetPhyAddr(), srcTensor.GetPhyAddr(), scale.GetPhyAddr(), stream));
+}
+// PER_TENSOR (ref: dequantize_impl.h:94-115)
+template <typename DstT>
+void Dequantize(const DeviceTensor<DstT>& dstTensor, const DeviceTensor<int32_t>& srcTensor, float scale,
+                float /*offset*/, const DequantizeParams& params, const DequantizeConfig& /*config*/,
+                void* stream = nullptr)
+{
+    AscendDequant<DstT, DeQuantMode::DEQUANT_WITH_MULTI_ROW>(dstTensor, srcTensor, scale,
+                                                            DequantParams{params.m, params.n, params.n}, stream);
+}
+
+enum class AntiQuantizePolicy : int32_t { PER_TENSOR, PER_CHANNEL, PER_TOKEN, PER_GROUP };
+struct AntiQuantizeConfig {
+    AntiQuantizePolicy policy;
+    bool hasOffset;
+    int32_t kDim = 1;
+};
+struct AntiQuantizeParams {
+    uint32_t m;
+    uint32_t n;
+    uint32_t groupSize = 0;
+};
+// fp32 arithmetic whatever the parameter type; SrcT int8_t / fp8_e4m3fn_t / fp8_e5m2_t; PER_CHANNEL takes parameters
+// [n] of the output's type (ref: impl/adv_api/detail/quantization/antiquantize/antiquantize_impl.h:36-135,
+// antiquantize_3510_impl.h:200-362).
+template <typename DstT, typename SrcT, typename ScaleT>
+void AntiQuantize(const DeviceTensor<DstT>& dstTensor, const DeviceTensor<SrcT>& srcTensor,
+                  const DeviceTensor<ScaleT>& scale, const DeviceTensor<ScaleT>& offset,
+                  const AntiQuantizeParams& params, const AntiQuantizeConfig& config, void* stream = nullptr)
+{
+    ascq_antiquant_policy_desc d{};
+    d.policy = static_cast<int32_t>(config.policy);
+    d.src_format = QuantDstOf<SrcT>::value;
+    d.scale_dtype = DTypeOf<ScaleT>::value;
+    d.dst_dtype = DTypeOf<DstT>::value;
+    d.compute = ASCQ_COMPUTE_F32;
+    d.has_offset = config.hasOffset ? 1 : 0;
+    d.k_dim = config.kDim;
+    d.m = params.m;
+    d.n = params.n;
+    d.cal_count = params.m * params.n;
+    d.group_size = params.groupSize;
+    Check(ascq_antiquant_policy(&d, dstTensor.GetPhyAddr(), srcTensor.GetPhyAddr(), scale.GetPhyAddr(),
+                                config.hasOffset ? offset.GetPhyAddr() : nullptr, stream));
+}
+// PER_TENSOR: the scalars are values of the output's type (ref: antiquantize_3510_impl.h:253-302).
+template <typename DstT, typename SrcT>
+void AntiQuantize(const DeviceTensor<DstT>& dstTensor, const DeviceTensor<SrcT>& srcTensor, float scale, float offset,
+                  const AntiQuantizeParams& params, const AntiQuantizeConfig& config, void* stream = nullptr)
+{
+    ascq_antiquant_policy_desc d{};
+    d.policy = ASCQ_PER_TENSOR;
+    d.src_format = QuantDstOf<SrcT>::value;
+    d.scale_dtype = DTypeOf<DstT>::value;
+    d.dst_dtype = DTypeOf<DstT>::value;
+    d.compute = ASCQ_COMPUTE_F32;
+    d.has_offset = config.hasOffset ? 1 : 0;
+    d.m = params.m;
+    d.n = params.n;
+    d.cal_count = params.m * params.n;
+    d.scale = scale;
+    d.offset = offset;
+    Check(ascq_antiquant_policy(&d, dstTensor.GetPhyAddr(), srcTensor.GetPhyAddr(), nullptr, nullptr, stream));
+}
+
 // ref: include/adv_api/quantization/ascend_antiquant_utils.h:27-32
 struct AntiQuantShapeInfo {
     uint32_t offsetHeight{0};

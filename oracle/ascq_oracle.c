@@ -486,6 +486,12 @@ uint32_t orc_dequant_dst_stride(int dst_dtype, uint32_t n)
 int orc_dequant(const ascq_dequant_desc* d, void* dst, const void* src, const void* scale)
 {
     uint32_t m = d->m, n = d->n, cal = d->cal_count;
+    if (d->policy >= ASCQ_PER_TOKEN) {
+        /* the policy form counts elements: the first calCount / n rows are processed, every column of them scaled
+         * (ref: impl/adv_api/detail/quantization/dequant/ascend_dequant_3510_impl.h:230, 272, 341, 397, 533) */
+        m = n ? cal / n : 0;
+        cal = n;
+    }
     if (d->mode == ASCQ_DEQUANT_WITH_SINGLE_ROW && d->policy <= ASCQ_PER_CHANNEL) {
         uint32_t per_blk = (d->dst_dtype == ASCQ_F32) ? 8u : 16u;
         if (m == 1 && cal != 0 && cal % per_blk == 0 && n % cal == 0) {
@@ -870,6 +876,10 @@ int orc_antiquant_policy(const ascq_antiquant_policy_desc* d, void* dst, const u
             size_t e = i * n + j, pi;
             if (d->policy == ASCQ_PER_TOKEN) {
                 pi = i;
+            } else if (d->policy == ASCQ_PER_CHANNEL) {
+                pi = j; /* AntiQuantize PER_CHANNEL: antiquantize_3510_impl.h:319-350 */
+            } else if (d->policy == ASCQ_PER_TENSOR) {
+                pi = 0;
             } else if (along_n) {
                 pi = i * ppr + j / d->group_size;
             } else {
@@ -877,8 +887,19 @@ int orc_antiquant_policy(const ascq_antiquant_policy_desc* d, void* dst, const u
             }
             float x = d->src_format == ASCQ_QDST_I8 ? (float)(int8_t)src[e]
                                                     : orc_fp8_to_f32(src[e], d->src_format == ASCQ_QDST_FP8_E5M2);
-            float s = load_as_f32(scale, pi, d->scale_dtype);
-            float o = d->has_offset ? load_as_f32(offset, pi, d->scale_dtype) : 0.0f;
+            float s, o = 0.0f;
+            if (d->policy == ASCQ_PER_TENSOR) {
+                /* scalars of the output's type (antiquantize_3510_impl.h:253-283) */
+                s = d->dst_dtype == ASCQ_F16 ? orc_f16_to_f32(orc_f32_to_f16(d->scale))
+                                             : orc_bf16_to_f32(orc_f32_to_bf16(d->scale));
+                if (d->has_offset) {
+                    o = d->dst_dtype == ASCQ_F16 ? orc_f16_to_f32(orc_f32_to_f16(d->offset))
+                                                 : orc_bf16_to_f32(orc_f32_to_bf16(d->offset));
+                }
+            } else {
+                s = load_as_f32(scale, pi, d->scale_dtype);
+                o = d->has_offset ? load_as_f32(offset, pi, d->scale_dtype) : 0.0f;
+            }
             float v;
             if (ct == ASCQ_F16) {
                 uint16_t t = orc_f32_to_f16(x);

@@ -156,8 +156,11 @@ def dynamic_quant_per_token(src_dtype, x):
 
 
 def dequant(desc, src, scale=None, fill=0):
-    """Returns dst [m', stride] (padded columns keep `fill`) after the single-row reshape rule."""
+    """Returns dst [m', stride] (padded columns keep `fill`) after the single-row reshape rule; for PER_TOKEN /
+    PER_GROUP m' = cal_count / n, the rows the operator processes."""
     m, n, cal = desc.m, desc.n, desc.cal_count
+    if desc.policy >= abi.PER_TOKEN:
+        m = cal // n
     per_blk = 8 if desc.dst_dtype == abi.F32 else 16
     if (desc.mode == abi.DEQUANT_WITH_SINGLE_ROW and desc.policy <= abi.PER_CHANNEL and m == 1 and cal
             and cal % per_blk == 0 and n % cal == 0):

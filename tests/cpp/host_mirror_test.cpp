@@ -376,6 +376,97 @@ void test_antiquant_matmul()
     expect_equal("AntiQuantMatmul", dc.download(), want);
 }
 
+void test_unified_surface()
+{
+    // Quantize / Dequantize / AntiQuantize with the policy inside the config, each against the oracle entry point of
+    // the operator it forwards to
+    Rng r{13};
+    const uint32_t m = 24, n = 128, gs = 32;
+    std::printf("[case] Quantize<PER_GROUP kDim=1, CAST_ROUND, offset> half -> int8 24x128\n");
+    {
+        auto x = random_halves(r, m * n, -4.0f, 4.0f);
+        std::vector<float> sc(m * n / gs), of(m * n / gs);
+        for (auto& e : sc) e = r.uniform(5.0f, 40.0f);
+        for (auto& e : of) e = r.uniform(-3.0f, 3.0f);
+        DeviceBuffer<uint16_t> dx(x);
+        DeviceBuffer<float> dsc(sc), dof(of);
+        DeviceBuffer<int8_t> dq(m * n);
+        ascq::QuantizeConfig cfg{ascq::QuantizePolicy::PER_GROUP, true, ascq::RoundMode::CAST_ROUND, 1};
+        ascq::Quantize(dq.view<int8_t>(m * n), dx.view<ascq::half>(m * n), dsc.view<float>(m * n / gs),
+                       dof.view<float>(m * n / gs), ascq::QuantizeParams{m, n, gs}, cfg);
+        ascq_quant_desc d{};
+        d.policy = ASCQ_PER_GROUP;
+        d.src_dtype = ASCQ_F16;
+        d.scale_dtype = ASCQ_F32;
+        d.compute = ASCQ_COMPUTE_F32;
+        d.round_mode = ASCQ_CAST_ROUND;
+        d.offset_kind = ASCQ_OFFSET_TENSOR;
+        d.k_dim = 1;
+        d.m = m;
+        d.n = n;
+        d.cal_count = m * n;
+        d.group_size = gs;
+        std::vector<int8_t> want(m * n);
+        orc_quant(&d, want.data(), x.data(), sc.data(), of.data());
+        expect_equal("Quantize per group", dq.download(), want);
+    }
+    std::printf("[case] Dequantize<PER_TOKEN> int32 -> bfloat16 24x128\n");
+    {
+        std::vector<int32_t> src(m * n);
+        for (auto& e : src) e = r.integer(-(1 << 20), 1 << 20);
+        std::vector<float> sc(m);
+        for (auto& e : sc) e = r.uniform(1e-5f, 1e-3f);
+        DeviceBuffer<int32_t> ds(src);
+        DeviceBuffer<float> dsc(sc);
+        DeviceBuffer<uint16_t> dd(m * n);
+        ascq::DequantizeConfig cfg{ascq::DequantizePolicy::PER_TOKEN, false, 1};
+        ascq::Dequantize(dd.view<ascq::bfloat16_t>(m * n), ds.view<int32_t>(m * n), dsc.view<float>(m),
+                         dsc.view<float>(m), ascq::DequantizeParams{m, n, 0}, cfg);
+        ascq_dequant_desc d{};
+        d.policy = ASCQ_PER_TOKEN;
+        d.src_dtype = ASCQ_I32;
+        d.scale_dtype = ASCQ_F32;
+        d.dst_dtype = ASCQ_BF16;
+        d.mode = ASCQ_DEQUANT_WITH_MULTI_ROW;
+        d.k_dim = 1;
+        d.m = m;
+        d.n = n;
+        d.cal_count = m * n;
+        std::vector<uint16_t> want(m * n);
+        orc_dequant(&d, want.data(), src.data(), sc.data());
+        expect_equal("Dequantize per token", dd.download(), want);
+    }
+    std::printf("[case] AntiQuantize<PER_TENSOR, offset> fp8_e4m3fn -> half 24x128\n");
+    {
+        std::vector<uint8_t> codes(m * n);
+        for (auto& e : codes) {
+            e = static_cast<uint8_t>(r.integer(0, 255));
+            if ((e & 0x7F) == 0x7F) e = 0x3C;  // no NaN codes
+        }
+        DeviceBuffer<uint8_t> dc(codes);
+        DeviceBuffer<uint16_t> dd(m * n);
+        ascq::AntiQuantizeConfig cfg{ascq::AntiQuantizePolicy::PER_TENSOR, true, 1};
+        ascq::AntiQuantize(dd.view<ascq::half>(m * n), dc.view<ascq::fp8_e4m3fn_t>(m * n), 0.37123f, -3.2517f,
+                           ascq::AntiQuantizeParams{m, n, 0}, cfg);
+        ascq_antiquant_policy_desc d{};
+        d.policy = ASCQ_PER_TENSOR;
+        d.src_format = ASCQ_QDST_FP8_E4M3FN;
+        d.scale_dtype = ASCQ_F16;
+        d.dst_dtype = ASCQ_F16;
+        d.compute = ASCQ_COMPUTE_F32;
+        d.has_offset = 1;
+        d.k_dim = 1;
+        d.m = m;
+        d.n = n;
+        d.cal_count = m * n;
+        d.scale = 0.37123f;
+        d.offset = -3.2517f;
+        std::vector<uint16_t> want(m * n);
+        orc_antiquant_policy(&d, want.data(), codes.data(), nullptr, nullptr);
+        expect_equal("AntiQuantize per tensor", dd.download(), want);
+    }
+}
+
 void test_errors()
 {
     std::printf("[case] argument errors surface as ascq::Error\n");
@@ -419,6 +510,7 @@ int main()
     test_antiquant();
     test_matmul();
     test_antiquant_matmul();
+    test_unified_surface();
     test_errors();
     std::printf("%s\n", g_failed ? "FAILED" : "ALL PASSED");
     return g_failed ? 1 : 0;

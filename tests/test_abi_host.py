@@ -36,7 +36,7 @@ def test_struct_sizes_match_the_header():
     assert C.sizeof(abi.GroupMatmulDesc) == C.sizeof(abi.MatmulDesc) + 8
     assert C.sizeof(abi.W4A16Desc) == 5 * 4
     assert C.sizeof(abi.W8A16Desc) == 8 * 4
-    assert C.sizeof(abi.AntiQuantPolicyDesc) == 12 * 4
+    assert C.sizeof(abi.AntiQuantPolicyDesc) == 14 * 4
 
 
 def q(**kw):

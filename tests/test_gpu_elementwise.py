@@ -316,12 +316,16 @@ def test_dequant_scalar_single_row_and_policies():
                 s, sd = src_array_uniform(rng, sshape, sc_dt, 0.01, 1.0)
                 sin = src.astype(np.float32) * np.float32(0.37) if src_f32 else src
                 dstb = torch.zeros((12, 256), dtype=torch.bfloat16, device=DEV)
-                para = ops.AscendQuantParam(12, 256, 256, gs)
-                ops.ascend_dequant_policy(dstb, to_dev(sin), sd, para, policy, k_dim)
-                d = abi.DequantDesc(policy=policy, src_dtype=abi.F32 if src_f32 else abi.I32, scale_dtype=sc_dt,
-                                    dst_dtype=abi.BF16, mode=abi.DEQUANT_WITH_MULTI_ROW, k_dim=k_dim, m=12, n=256,
-                                    cal_count=256, group_size=gs)
-                assert np.array_equal(bits(dstb), orc.dequant(d, sin, s))
+                for cal in (12 * 256, 5 * 256):       # every row, and the first five only (the rest stays untouched)
+                    dstb.zero_()
+                    para = ops.AscendQuantParam(12, 256, cal, gs)
+                    ops.ascend_dequant_policy(dstb, to_dev(sin), sd, para, policy, k_dim)
+                    d = abi.DequantDesc(policy=policy, src_dtype=abi.F32 if src_f32 else abi.I32, scale_dtype=sc_dt,
+                                        dst_dtype=abi.BF16, mode=abi.DEQUANT_WITH_MULTI_ROW, k_dim=k_dim, m=12, n=256,
+                                        cal_count=cal, group_size=gs)
+                    got = bits(dstb)
+                    assert np.array_equal(got[:cal // 256], orc.dequant(d, sin, s))
+                    assert not got[cal // 256:].any()
 
 
 # ------------------------------------------------------------------ AscendAntiQuant
@@ -434,6 +438,68 @@ def test_antiquant_policy_nan_and_infinity_codes_through_the_saturating_cast(fmt
     top = 0x7BFF if dst_dt == abi.F16 else 0x7F7F
     assert list(got[0, :len(nan_codes)]) == [0] * len(nan_codes)
     assert list(got[0, len(nan_codes):len(special)]) == [top, 0x8000 | top][:len(inf_codes)]
+
+
+@pytest.mark.parametrize("fmt", [abi.QDST_I8, abi.QDST_FP8_E4M3FN, abi.QDST_FP8_E5M2])
+@pytest.mark.parametrize("dst_dt", [abi.F16, abi.BF16])
+@pytest.mark.parametrize("policy", [abi.PER_CHANNEL, abi.PER_TENSOR])
+@pytest.mark.parametrize("has_offset", [True, False])
+def test_antiquantize_per_channel_and_per_tensor(fmt, dst_dt, policy, has_offset):
+    """AntiQuantize PER_CHANNEL / PER_TENSOR: fp32 arithmetic on parameters of the output's type, saturating cast;
+    every source code, bit-exact against the oracle."""
+    for (m, n) in [(64, 256), (33, 2080), (5, 32)]:
+        announce("antiquantize", fmt, dst_dt, policy, has_offset, m, n)
+        rng = np.random.default_rng(m + n + fmt)
+        codes = rng.integers(0, 256, (m, n)).astype(np.uint8)
+        codes.reshape(-1)[:min(256, m * n)] = np.arange(min(256, m * n), dtype=np.uint8)
+        if fmt == abi.QDST_FP8_E4M3FN:
+            codes[(codes & 0x7F) == 0x7F] = 0x3C
+        elif fmt == abi.QDST_FP8_E5M2:
+            codes[(codes & 0x7F) >= 0x7C] = 0x3C
+        dst = torch.zeros((m, n), dtype=TDT[dst_dt], device=DEV)
+        cfg = ops.AscendAntiQuantConfig(has_offset=has_offset, is_transpose=False, k_dim=1)
+        para = ops.AscendAntiQuantParam(m=m, n=n, cal_count=m * n, group_size=0)
+        d = abi.AntiQuantPolicyDesc(policy=policy, src_format=fmt, scale_dtype=dst_dt, dst_dtype=dst_dt,
+                                    compute=abi.COMPUTE_F32, has_offset=int(has_offset), is_transpose=0, k_dim=1,
+                                    m=m, n=n, cal_count=m * n, group_size=0)
+        if policy == abi.PER_CHANNEL:
+            (s, sdev), (o, odev) = typed(rng.uniform(0.01, 2.0, n), dst_dt), typed(rng.uniform(-3, 3, n), dst_dt)
+            ops.antiquantize(dst, to_dev(codes).view(B8[fmt]), sdev, odev, para, policy, cfg)
+            want = orc.antiquant_policy(d, codes, s, o)
+        else:
+            sv, ov = 0.37123, -3.2517                      # not representable in half / bfloat16: rounded once
+            ops.antiquantize(dst, to_dev(codes).view(B8[fmt]), sv, ov, para, policy, cfg)
+            d.scale, d.offset = sv, ov
+            want = orc.antiquant_policy(d, codes, None, None)
+        want = want.view(np.uint16) if want.dtype == np.float16 else want
+        assert np.array_equal(bits(dst), want)
+
+
+@pytest.mark.parametrize("policy", ["tensor", "channel", "token", "group0", "group1"])
+def test_dequantize_is_the_matching_ascend_dequant(policy):
+    """The unified Dequantize: each policy gives what the operator it forwards to gives (and the oracle)."""
+    announce("dequantize", policy)
+    rng = np.random.default_rng(17)
+    m, n, gs = 40, 96, 32
+    src = rng.integers(-2 ** 20, 2 ** 20, (m, n)).astype(np.int32)
+    pol = {"tensor": abi.PER_TENSOR, "channel": abi.PER_CHANNEL, "token": abi.PER_TOKEN, "group0": abi.PER_GROUP,
+           "group1": abi.PER_GROUP}[policy]
+    k_dim = 0 if policy == "group0" else 1
+    sshape = {"channel": (n,), "token": (m,), "group0": (-(-m // gs), n), "group1": (m, -(-n // gs))}.get(policy)
+    para = ops.AscendQuantParam(m=m, n=n, cal_count=m * n, group_size=gs if pol == abi.PER_GROUP else 0)
+    dst = torch.zeros((m, n), dtype=torch.bfloat16, device=DEV)
+    d = abi.DequantDesc(policy=pol, src_dtype=abi.I32, scale_dtype=abi.F32, dst_dtype=abi.BF16,
+                        mode=abi.DEQUANT_WITH_MULTI_ROW, k_dim=k_dim, m=m, n=n,
+                        cal_count=n if pol in (abi.PER_TENSOR, abi.PER_CHANNEL) else m * n, group_size=para.group_size)
+    if pol == abi.PER_TENSOR:
+        ops.dequantize(dst, to_dev(src), 3.1e-4, para, pol)
+        d.scale = 3.1e-4
+        want = orc.dequant(d, src)
+    else:
+        s = rng.uniform(1e-5, 1e-3, sshape).astype(np.float32)
+        ops.dequantize(dst, to_dev(src), to_dev(s), para, pol, k_dim=k_dim)
+        want = orc.dequant(d, src, s)
+    assert np.array_equal(bits(dst), np.asarray(want).reshape(m, -1)[:, :n])
 
 
 def test_antiquant_per_tensor():

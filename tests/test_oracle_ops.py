@@ -212,8 +212,12 @@ def test_dequant_per_token_and_group():
     src = rng.integers(-1000, 1000, (m, n), dtype=np.int32)
     st = rng.uniform(0.01, 1, m).astype(np.float32)
     d = abi.DequantDesc(policy=abi.PER_TOKEN, src_dtype=abi.I32, scale_dtype=abi.F32, dst_dtype=abi.F32,
-                        mode=abi.DEQUANT_WITH_MULTI_ROW, m=m, n=n, cal_count=n)
+                        mode=abi.DEQUANT_WITH_MULTI_ROW, m=m, n=n, cal_count=m * n)
     assert np.array_equal(orc.dequant(d, src, st), src.astype(np.float32) * st[:, None])
+    # calCount counts elements: calCount / n rows are processed (ascend_dequant_3510_impl.h:230)
+    d.cal_count = 3 * n
+    assert np.array_equal(orc.dequant(d, src, st), (src.astype(np.float32) * st[:, None])[:3])
+    d.cal_count = m * n
     sg = rng.uniform(0.01, 1, (m, n // gs)).astype(np.float32)
     d.policy, d.group_size, d.k_dim = abi.PER_GROUP, gs, 1
     assert np.array_equal(orc.dequant(d, src, sg), src.astype(np.float32) * np.repeat(sg, gs, axis=1))
@@ -221,7 +225,7 @@ def test_dequant_per_token_and_group():
     src2 = rng.integers(-1000, 1000, (m2, 32), dtype=np.int32)
     sg0 = rng.uniform(0.01, 1, (m2 // gs, 32)).astype(np.float32)
     d2 = abi.DequantDesc(policy=abi.PER_GROUP, src_dtype=abi.I32, scale_dtype=abi.F32, dst_dtype=abi.F32,
-                         mode=abi.DEQUANT_WITH_MULTI_ROW, k_dim=0, m=m2, n=32, cal_count=32, group_size=gs)
+                         mode=abi.DEQUANT_WITH_MULTI_ROW, k_dim=0, m=m2, n=32, cal_count=m2 * 32, group_size=gs)
     assert np.array_equal(orc.dequant(d2, src2, sg0), src2.astype(np.float32) * np.repeat(sg0, gs, axis=0))
 
 
@@ -617,3 +621,44 @@ def test_pack_weight_nz_is_the_data_scripts_reshape_transpose():
     flat = got.reshape(-1)
     for gi, kk, c in [(0, 0, 0), (1, 17, 33), (2, 47, 95), (1, 16, 31), (0, 15, 32)]:
         assert flat[((gi * (n // 32) + c // 32) * k + kk) * 32 + c % 32] == w[gi, kk, c]
+
+
+@pytest.mark.filterwarnings("ignore:overflow encountered")
+@pytest.mark.parametrize("fmt", [abi.QDST_I8, abi.QDST_FP8_E4M3FN, abi.QDST_FP8_E5M2])
+def test_antiquantize_per_channel_and_per_tensor_against_numpy_fp32(fmt):
+    """AntiQuantize PER_CHANNEL / PER_TENSOR (antiquantize_3510_impl.h:253-362): parameters of the output's type are
+    widened to fp32, (src + offset) * scale in fp32 (numpy), one saturating half-even cast (numpy / torch)."""
+    rng = np.random.default_rng(53 + fmt)
+    m, n = 48, 64
+    codes, x = _b8_source(rng, fmt, (m, n))
+    s16 = rng.uniform(0.01, 2.0, n).astype(np.float16)
+    o16 = rng.uniform(-3.0, 3.0, n).astype(np.float16)
+    sat = lambda v: np.clip(v, -65504.0, 65504.0).astype(np.float16)
+
+    def desc(policy, dst_dt, has_offset=1, **kw):
+        return abi.AntiQuantPolicyDesc(policy=policy, src_format=fmt, scale_dtype=dst_dt, dst_dtype=dst_dt,
+                                       compute=abi.COMPUTE_F32, has_offset=has_offset, is_transpose=0, k_dim=1, m=m,
+                                       n=n, cal_count=m * n, group_size=0, **kw)
+
+    want = sat((x + o16.astype(np.float32)[None, :]) * s16.astype(np.float32)[None, :])
+    got = orc.antiquant_policy(desc(abi.PER_CHANNEL, abi.F16), codes, s16, o16)
+    assert np.array_equal(got.view(U16), want.view(U16))
+    want = sat(x * s16.astype(np.float32)[None, :])
+    got = orc.antiquant_policy(desc(abi.PER_CHANNEL, abi.F16, has_offset=0), codes, s16, None)
+    assert np.array_equal(got.view(U16), want.view(U16))
+    # bfloat16 parameters and output
+    sb, ob = torch.from_numpy(s16.astype(np.float32)).bfloat16(), torch.from_numpy(o16.astype(np.float32)).bfloat16()
+    wantb = ((torch.from_numpy(x) + ob.float()[None, :]) * sb.float()[None, :]).bfloat16()
+    gotb = orc.antiquant_policy(desc(abi.PER_CHANNEL, abi.BF16), codes, sb.view(torch.int16).numpy().view(U16),
+                                ob.view(torch.int16).numpy().view(U16))
+    assert np.array_equal(gotb.view(U16), wantb.view(torch.int16).numpy().view(U16))
+    # per tensor: the scalars are rounded once to the output's type
+    sv, ov = 0.37123, -3.2517
+    want = sat((x + np.float32(np.float16(ov))) * np.float32(np.float16(sv)))
+    got = orc.antiquant_policy(desc(abi.PER_TENSOR, abi.F16, scale=sv, offset=ov), codes, None, None)
+    assert np.array_equal(got.view(U16), want.view(U16))
+    svb = torch.tensor(sv).bfloat16().float().item()
+    ovb = torch.tensor(ov).bfloat16().float().item()
+    wantb = ((torch.from_numpy(x) + np.float32(ovb)) * np.float32(svb)).bfloat16()
+    gotb = orc.antiquant_policy(desc(abi.PER_TENSOR, abi.BF16, scale=sv, offset=ov), codes, None, None)
+    assert np.array_equal(gotb.view(U16), wantb.view(torch.int16).numpy().view(U16))
