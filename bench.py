@@ -29,7 +29,7 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E peak, GB/s
 # (FETCH_SIZE reads 0.5 per KiB there, WRITE_SIZE 1.0 per KiB).  Measured offline and recorded here; a run of this
 # file does not re-measure them.
 GEMM_TRAFFIC_BYTES = 228345446   # M=2048 GEMM, both launches: 183.2 MB fetched + 45.1 MB written
-GEMV_TRAFFIC_BYTES = 137013862   # W4A16 M=1 GEMV, stream + sum kernels: 132.7 MB fetched + 4.3 MB written
+GEMV_TRAFFIC_BYTES = 133853594   # W4A16 M=1 GEMV, stream + sum kernels: 129.5 MB fetched + 4.3 MB written
 
 
 def main():
