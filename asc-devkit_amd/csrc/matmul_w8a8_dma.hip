@@ -348,8 +348,9 @@ __global__ __launch_bounds__(kThreads, (BM * BK + BK * BN) * 2 <= 65536 ? 2 : 1)
                             const uint32_t word = odd ? (recv | (h1 << 16)) : (h0 | (recv << 16));
                             const uint32_t col = odd ? colw + 32u + (lrow - 1u) : colw + lrow;
                             if (row < row_end && col < N) {
-                                *reinterpret_cast<uint32_t*>(static_cast<uint16_t*>(e.c) +
-                                                             static_cast<size_t>(row) * e.ldc + col) = word;
+                                __builtin_nontemporal_store(
+                                    word, reinterpret_cast<uint32_t*>(static_cast<uint16_t*>(e.c) +
+                                                                      static_cast<size_t>(row) * e.ldc + col));
                             }
                         } else {
     #pragma unroll
