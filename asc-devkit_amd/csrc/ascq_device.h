@@ -139,22 +139,42 @@ struct Elem<ASCQ_I32> {
     static __device__ __forceinline__ float to_f32(int32_t v) { return static_cast<float>(v); }  // RNE
 };
 
+// 16-byte load / store with or without the non-temporal cache policy (data that is touched once per call).
+template <bool kNT>
+__device__ __forceinline__ u32x4 ld16(const void* p)
+{
+    if constexpr (kNT) {
+        return __builtin_nontemporal_load(static_cast<const u32x4*>(p));
+    } else {
+        return *static_cast<const u32x4*>(p);
+    }
+}
+template <bool kNT, class V>
+__device__ __forceinline__ void st16(void* p, V v)
+{
+    if constexpr (kNT) {
+        __builtin_nontemporal_store(v, static_cast<V*>(p));
+    } else {
+        *static_cast<V*>(p) = v;
+    }
+}
+
 // Load 8 consecutive elements (16-byte aligned group for 2-byte types) widened to fp32.
-template <int kDt>
+template <int kDt, bool kNT = false>
 __device__ __forceinline__ void load8(const void* base, size_t idx, float (&out)[8])
 {
     typedef typename Elem<kDt>::type T;
     const T* p = static_cast<const T*>(base) + idx;
     if constexpr (sizeof(T) == 2) {
-        u32x4 v = *reinterpret_cast<const u32x4*>(p);
+        u32x4 v = ld16<kNT>(p);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             out[2 * i] = Elem<kDt>::to_f32(static_cast<uint16_t>(v[i] & 0xFFFFu));
             out[2 * i + 1] = Elem<kDt>::to_f32(static_cast<uint16_t>(v[i] >> 16));
         }
     } else if constexpr (sizeof(T) == 4) {
-        u32x4 a = reinterpret_cast<const u32x4*>(p)[0];
-        u32x4 b = reinterpret_cast<const u32x4*>(p)[1];
+        u32x4 a = ld16<kNT>(reinterpret_cast<const u32x4*>(p));
+        u32x4 b = ld16<kNT>(reinterpret_cast<const u32x4*>(p) + 1);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const uint32_t ua = a[i], ub = b[i];
@@ -182,13 +202,13 @@ __device__ __forceinline__ float load1(const void* base, size_t idx)
 }
 
 // Store 8 fp32 values as the destination type (rounded once).
-template <int kDt>
+template <int kDt, bool kNT = false>
 __device__ __forceinline__ void store8(void* base, size_t idx, const float (&v)[8])
 {
     if constexpr (kDt == ASCQ_F32) {
         f32x4* p = reinterpret_cast<f32x4*>(static_cast<float*>(base) + idx);
-        p[0] = f32x4{v[0], v[1], v[2], v[3]};
-        p[1] = f32x4{v[4], v[5], v[6], v[7]};
+        st16<kNT>(p, f32x4{v[0], v[1], v[2], v[3]});
+        st16<kNT>(p + 1, f32x4{v[4], v[5], v[6], v[7]});
     } else {
         u32x4 o;
 #pragma unroll
@@ -203,7 +223,7 @@ __device__ __forceinline__ void store8(void* base, size_t idx, const float (&v)[
             }
             o[i] = lo | (hi << 16);
         }
-        *reinterpret_cast<u32x4*>(static_cast<uint16_t*>(base) + idx) = o;
+        st16<kNT>(static_cast<uint16_t*>(base) + idx, o);
     }
 }
 

@@ -138,7 +138,7 @@ __global__ __launch_bounds__(kThreads) void quant_vec_kernel(QuantArgs a)
 #pragma unroll
         for (int u = 0; u < kRowsInFlight; ++u) {
             if (r0 + u < a.rows) {
-                load8<kSrc>(a.src, static_cast<size_t>(r0 + u) * a.n + j, x[u]);
+                load8<kSrc, true>(a.src, static_cast<size_t>(r0 + u) * a.n + j, x[u]);  // read once: non-temporal
             }
         }
 #pragma unroll
@@ -175,13 +175,14 @@ __global__ __launch_bounds__(kThreads) void quant_vec_kernel(QuantArgs a)
                 uint32_t out = 0;
 #pragma unroll
                 for (int e = 0; e < 8; ++e) out |= static_cast<uint32_t>(q[e]) << (4 * e);
-                *reinterpret_cast<uint32_t*>(a.dst + (static_cast<size_t>(r) * a.n + j) / 2u) = out;
+                __builtin_nontemporal_store(
+                    out, reinterpret_cast<uint32_t*>(a.dst + (static_cast<size_t>(r) * a.n + j) / 2u));
                 continue;
             }
             u32x2 out;
             out[0] = pack4_i8(q[0], q[1], q[2], q[3]);
             out[1] = pack4_i8(q[4], q[5], q[6], q[7]);
-            *reinterpret_cast<u32x2*>(a.dst + static_cast<size_t>(r) * a.n + j) = out;
+            __builtin_nontemporal_store(out, reinterpret_cast<u32x2*>(a.dst + static_cast<size_t>(r) * a.n + j));
         }
     }
 }
@@ -469,7 +470,7 @@ __global__ __launch_bounds__(kThreads) void dequant_vec_kernel(DequantArgs a)
 #pragma unroll
         for (int u = 0; u < kRowsInFlight; ++u) {
             if (r0 + u < a.rows) {
-                load8<kSrc>(a.src, static_cast<size_t>(r0 + u) * a.n + j, x[u]);
+                load8<kSrc, true>(a.src, static_cast<size_t>(r0 + u) * a.n + j, x[u]);  // read once: non-temporal
             }
         }
 #pragma unroll
@@ -487,7 +488,7 @@ __global__ __launch_bounds__(kThreads) void dequant_vec_kernel(DequantArgs a)
             float y[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) y[e] = x[u][e] * s[e];
-            store8<kDst>(a.dst, static_cast<size_t>(r) * a.dst_stride + j, y);
+            store8<kDst, true>(a.dst, static_cast<size_t>(r) * a.dst_stride + j, y);
         }
     }
 }
@@ -656,8 +657,8 @@ __global__ __launch_bounds__(kThreads) void antiquant_vec_kernel(AntiQuantArgs a
                 }
             }
             const size_t oe = static_cast<size_t>(r) * a.cols + j;
-            store8<kDst>(a.dst, oe, y0);
-            store8<kDst>(a.dst, oe + 8, y1);
+            store8<kDst, true>(a.dst, oe, y0);
+            store8<kDst, true>(a.dst, oe + 8, y1);
         }
     }
 }
@@ -873,7 +874,8 @@ __global__ __launch_bounds__(kThreads) void antiquant_policy_vec_kernel(AntiQuan
 #pragma unroll
         for (int u = 0; u < kRowsInFlight; ++u) {
             if (r0 + u < a.rows) {
-                raw[u] = *reinterpret_cast<const u32x2*>(a.src + static_cast<size_t>(r0 + u) * a.n + j);
+                raw[u] = __builtin_nontemporal_load(
+                    reinterpret_cast<const u32x2*>(a.src + static_cast<size_t>(r0 + u) * a.n + j));
             }
         }
 #pragma unroll
@@ -896,7 +898,7 @@ __global__ __launch_bounds__(kThreads) void antiquant_policy_vec_kernel(AntiQuan
                 t = Fmt<kCt>::mul(t, Fmt<kCt>::cvt(s[e]));
                 v[e] = kCt == kDst ? t : aqp_saturate<kDst>(t);
             }
-            store8<kDst>(a.dst, static_cast<size_t>(r) * a.n + j, v);
+            store8<kDst, true>(a.dst, static_cast<size_t>(r) * a.n + j, v);
         }
     }
 }
