@@ -174,8 +174,9 @@ __global__ __launch_bounds__(kThreads, (BM * BK + BK * BN) * 2 <= 65536 ? 2 : 1)
         }
 #pragma unroll
         for (int u = 0; u < kBInstr; ++u) {
+            // split-K (few rows): the weights are read once, or by a handful of row tiles at the same time
             __builtin_amdgcn_global_load_lds((gptr_t)(bb + boff[u]), (lds_ptr_t)(Bs + (wave * kBInstr + u) * 1024), 16, 0,
-                                             0);
+                                             kSplitK ? 2 : 0);
         }
     };
 
