@@ -39,8 +39,8 @@ inline int launch_status(const char* what)
 
 // Plan recording (ascq_matmul_w8a8_plan): while a plan is being recorded on this thread, every launch site of the int8
 // matmul describes the launch it would make and returns true, and the caller then skips the launch.  The first note of
-// a call fills the main fields; later ones (a second tile shape for the last partial round, the kernel that sums
-// partial results) only add to `launches` and the narrow-tile fields.
+// a call fills the main fields; later ones (the kernel that sums partial results) only add to `launches`;
+// plan_note_extra records the second tile shape that the same launch runs for the last partial round.
 bool plan_recording();
 bool plan_note(int kernel, uint32_t tile_m, uint32_t tile_n, uint32_t tile_k, uint32_t workgroups, uint32_t k_splits,
                uint32_t lds_bytes, size_t workspace_bytes);

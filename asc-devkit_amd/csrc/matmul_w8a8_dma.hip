@@ -63,9 +63,11 @@ __device__ __forceinline__ float epi_value(int32_t acc, float chan, float tok, f
 // wavefront, 64 KiB of LDS so that two workgroups share a CU; with kSplitK the K range is divided over blockIdx.y and
 // the int32 partial tiles go to a workspace [split][m][n] that a second kernel sums (small M: the weights are read
 // once, by enough workgroups to fill the chip).
-template <int BM, int BN, bool kSplitK, bool kGrouped = false>
-__global__ __launch_bounds__(kThreads, (BM * BK + BK * BN) * 2 <= 65536 ? 2 : 1) void gemm_dma_kernel(
-    GemmParams p, uint32_t col_begin)
+// The body of a workgroup: tile number `bid` (before the XCD remapping) of the launch, K split `bidy`.  The LDS arrays
+// are declared by the kernels and handed in, so that one kernel can run tiles of two shapes.
+template <int BM, int BN, bool kSplitK, bool kGrouped>
+__device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_begin, uint32_t bid, uint32_t bidy,
+                                              char* A0, char* B0, char* A1, char* B1, float* TS)
 {
     constexpr int kWN = BN / 64;            // wavefronts along N
     constexpr int kWM = 8 / kWN;            // wavefronts along M
@@ -76,14 +78,9 @@ __global__ __launch_bounds__(kThreads, (BM * BK + BK * BN) * 2 <= 65536 ? 2 : 1)
     constexpr int kBInstr = BK * BN / 1024 / 8;  // B DMA instructions per wavefront and K step
     constexpr int kKsB = 32 * BN;           // bytes of B per K sub-step of 32 rows
     static_assert(TI >= 1 && TI * 32 * kWM == BM && kAInstr >= 1, "tile shape does not fit eight wavefronts");
-    __shared__ __attribute__((aligned(1024))) char A0[BM * BK];
-    __shared__ __attribute__((aligned(1024))) char B0[BK * BN];
-    __shared__ __attribute__((aligned(1024))) char A1[BM * BK];
-    __shared__ __attribute__((aligned(1024))) char B1[BK * BN];
-    __shared__ __attribute__((aligned(16))) float TS[BM];  // token scales of the tile's rows (1.0f when there are none)
 
     const uint32_t total = p.tiles_m * p.tiles_n;
-    const uint32_t t = xcd_remap(blockIdx.x, total);
+    const uint32_t t = xcd_remap(bid, total);
     if (t >= total) {
         return;
     }
@@ -159,8 +156,8 @@ __global__ __launch_bounds__(kThreads, (BM * BK + BK * BN) * 2 <= 65536 ? 2 : 1)
     // K range of this workgroup, in steps of BK
     uint32_t s_begin = 0, steps = K / BK;
     if constexpr (kSplitK) {
-        s_begin = steps * blockIdx.y / p.k_splits;
-        steps = steps * (blockIdx.y + 1u) / p.k_splits - s_begin;
+        s_begin = steps * bidy / p.k_splits;
+        steps = steps * (bidy + 1u) / p.k_splits - s_begin;
     }
     const int8_t* Abase = p.a + static_cast<size_t>(row0) * K + static_cast<size_t>(s_begin) * BK;
     const int8_t* Bbase = Bmat + (p.b_nz ? 0u : n0) + static_cast<size_t>(s_begin) * BK * ldb;
@@ -275,7 +272,7 @@ __global__ __launch_bounds__(kThreads, (BM * BK + BK * BN) * 2 <= 65536 ? 2 : 1)
 
     // ---- epilogue: register r of lane l in a 32x32 block is row 8*(r/4) + 4*(l/32) + r%4, column l%32
     if constexpr (kSplitK) {
-        int32_t* part = p.partial + static_cast<size_t>(blockIdx.y) * p.m * N;
+        int32_t* part = p.partial + static_cast<size_t>(bidy) * p.m * N;
 #pragma unroll
         for (int i = 0; i < TI; ++i) {
 #pragma unroll
@@ -387,6 +384,38 @@ __global__ __launch_bounds__(kThreads, (BM * BK + BK * BN) * 2 <= 65536 ? 2 : 1)
     dispatch_out(e, run);
 }
 
+template <int BM, int BN, bool kSplitK, bool kGrouped = false>
+__global__ __launch_bounds__(kThreads, (BM * BK + BK * BN) * 2 <= 65536 ? 2 : 1) void gemm_dma_kernel(
+    GemmParams p, uint32_t col_begin)
+{
+    __shared__ __attribute__((aligned(1024))) char A0[BM * BK];
+    __shared__ __attribute__((aligned(1024))) char B0[BK * BN];
+    __shared__ __attribute__((aligned(1024))) char A1[BM * BK];
+    __shared__ __attribute__((aligned(1024))) char B1[BK * BN];
+    __shared__ __attribute__((aligned(16))) float TS[BM];  // token scales of the tile's rows (1.0f when there are none)
+    gemm_dma_tile<BM, BN, kSplitK, kGrouped>(p, col_begin, blockIdx.x, blockIdx.y, A0, B0, A1, B1, TS);
+}
+
+// One launch for a matrix whose last round of 256 x 256 tiles would be mostly empty: workgroups [0, wide_wgs) run the
+// 256 x 256 tiles of the first `p.tiles_n` tile columns, the rest 256 x 128 tiles of the remaining columns.  A compute
+// unit that has finished its wide tile takes a narrow one at once, without the drain between two launches.
+__global__ __launch_bounds__(kThreads, 1) void gemm_dma_dual_kernel(GemmParams p, uint32_t wide_wgs,
+                                                                    uint32_t narrow_tiles_n, uint32_t col_begin)
+{
+    __shared__ __attribute__((aligned(1024))) char A0[256 * BK];
+    __shared__ __attribute__((aligned(1024))) char B0[BK * 256];
+    __shared__ __attribute__((aligned(1024))) char A1[256 * BK];
+    __shared__ __attribute__((aligned(1024))) char B1[BK * 256];
+    __shared__ __attribute__((aligned(16))) float TS[256];
+    if (blockIdx.x < wide_wgs) {
+        gemm_dma_tile<256, 256, false, false>(p, 0u, blockIdx.x, 0u, A0, B0, A1, B1, TS);
+    } else {
+        GemmParams q = p;
+        q.tiles_n = narrow_tiles_n;
+        gemm_dma_tile<256, 128, false, false>(q, col_begin, blockIdx.x - wide_wgs, 0u, A0, B0, A1, B1, TS);
+    }
+}
+
 // Second pass of the split-K path: sums the int32 partial tiles [split][m][n] in split order (integer addition: exact in
 // any order) and applies the epilogue.  One lane = four consecutive columns.
 __global__ __launch_bounds__(256) void splitk_sum_epilogue_kernel(GemmParams p)
@@ -429,7 +458,7 @@ int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st)
     p.tiles_m = (p.m + 255u) / 256u + (grouped ? p.groups : 0u);  // every group adds at most one partial tile
     uint32_t tiles_n = (p.n + 255u) / 256u;
     // Tile quantisation: when the last round of 256-wide tiles would fill less than half of the 256 CUs, its
-    // columns are computed by a second launch with 128-wide tiles, which finishes that round in about half the time.
+    // columns are computed with 128-wide tiles, which finish that round in about half the time.
     uint32_t narrow_cols = 0;  // number of 256-wide column tiles handed to the 128-wide kernel
     const uint32_t total = p.tiles_m * tiles_n;
     const uint32_t rem = total % 256u;
@@ -449,12 +478,22 @@ int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st)
         if (wide_cols) {
             plan_note(ASCQ_MM_KERNEL_DMA_256, 256, 256, BK, wide_wg, 1, kLdsWide, 0);
             if (narrow_cols) {
-                plan_note_extra(128, narrow_wg);
+                plan_note_extra(128, narrow_wg);  // workgroups of the same launch
             }
         } else {
             plan_note(ASCQ_MM_KERNEL_DMA_256, 256, 128, BK, narrow_wg, 1, kLdsNarrow, 0);
         }
         return ASCQ_OK;
+    }
+    if (wide_cols && narrow_cols) {
+        // both tile shapes in one launch (narrow_cols is only ever non-zero for the plain matmul)
+        const uint32_t col_begin = wide_cols * 256u;
+        const uint32_t narrow_tiles_n = (p.n - col_begin + 127u) / 128u;
+        const uint32_t wide_wgs = (p.tiles_m * wide_cols + 7u) / 8u * 8u;
+        const uint32_t narrow_wgs = (p.tiles_m * narrow_tiles_n + 7u) / 8u * 8u;
+        p.tiles_n = wide_cols;
+        gemm_dma_dual_kernel<<<wide_wgs + narrow_wgs, kThreads, 0, st>>>(p, wide_wgs, narrow_tiles_n, col_begin);
+        return launch_status("ascq_matmul_w8a8");
     }
     if (wide_cols) {
         p.tiles_n = wide_cols;

@@ -42,7 +42,6 @@ bool plan_note_extra(uint32_t narrow_tile_n, uint32_t narrow_workgroups)
     if (g_plan == nullptr) {
         return false;
     }
-    g_plan->launches += 1;
     g_plan->narrow_tile_n = narrow_tile_n;
     g_plan->narrow_workgroups = narrow_workgroups;
     return true;

@@ -28,7 +28,7 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E peak, GB/s
 # `bench.py --quick --no-cpu --copy-probe`; each counter is scaled by its reading for the 1 GiB copy of the same run
 # (FETCH_SIZE reads 0.5 per KiB there, WRITE_SIZE 1.0 per KiB).  Measured offline and recorded here; a run of this
 # file does not re-measure them.
-GEMM_TRAFFIC_BYTES = 228345446   # M=2048 GEMM, both launches: 183.2 MB fetched + 45.1 MB written
+GEMM_TRAFFIC_BYTES = 228293837   # M=2048 GEMM, both tile shapes: 183.2 MB fetched + 45.1 MB written
 GEMV_TRAFFIC_BYTES = 133853594   # W4A16 M=1 GEMV, stream + sum kernels: 129.5 MB fetched + 4.3 MB written
 
 
@@ -279,12 +279,12 @@ def main():
                                "per-token int8 quant -> int8 GEMM with W [4096,11008] -> fused (channel x token) "
                                "dequant to bf16; one step = quant kernel + GEMM kernel",
                    "m": 2048, "k": 4096, "n": 11008, "ops_per_step": head["ops"]},
-        # The GEMM is two launches of one kernel template back to back: 256x256 tiles for the full rounds of 256
-        # workgroups and 256x128 tiles for the last partial round; `achieved` is the 2*M*K*N operations over the
-        # average duration of the pair, from one pair of events around `steps` back-to-back GEMMs.  `traffic` is HBM bytes per GEMM (both launches) from
+        # The GEMM is one launch that runs two tile shapes: 256x256 tiles for the full round of 256 workgroups and
+        # 256x128 tiles for the last partial round; `achieved` is the 2*M*K*N operations over the average duration of
+        # the launch, from one pair of events around `steps` back-to-back GEMMs.  `traffic` is HBM bytes per GEMM from
         # rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of `bench.py --only w8a8 --copy-probe`, each counter scaled by
         # its reading for the 1 GiB copy; it is a constant measured offline, not re-measured by this run.
-        "roofline": {"bound": "mfma", "kernel": "gemm_dma_kernel<256,256> + gemm_dma_kernel<256,128> (last partial round)",
+        "roofline": {"bound": "mfma", "kernel": "gemm_dma_dual_kernel (256x256 tiles, then 256x128 tiles for the last partial round)",
                      "achieved": head["gemm_tops"], "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                      "frac": head["gemm_tops"] / PEAK_INT8_TOPS, "traffic": GEMM_TRAFFIC_BYTES,
                      "avg_kernel_ms": head["gemm_kernel_ms"], "ops_per_launch": head["ops"],

@@ -342,7 +342,7 @@ typedef enum ascq_mm_kernel {
     ASCQ_MM_KERNEL_DMA_128 = 2,      /* m <= 512: 128 x 128 direct-to-LDS tiles, K split over workgroups when a
                                         workspace is given (k_splits > 1: a second kernel adds the partial tiles) */
     ASCQ_MM_KERNEL_DMA_256 = 3,      /* 256 x 256 direct-to-LDS tiles; a last partial round of the chip may be run
-                                        by a second launch with 256 x narrow_tile_n tiles */
+                                        by further workgroups of the same launch with 256 x narrow_tile_n tiles */
     ASCQ_MM_KERNEL_STAGED = 4        /* register-staged tiles: transposed B, or K not a multiple of 128 */
 } ascq_mm_kernel;
 
@@ -355,8 +355,8 @@ typedef struct ascq_matmul_plan {
     uint32_t k_splits;          /* partial sums per output element (1: the main kernel writes C itself) */
     uint32_t launches;          /* kernel launches per call */
     uint32_t lds_bytes;         /* LDS per workgroup of the main launch */
-    uint32_t narrow_tile_n;     /* KERNEL_DMA_256: columns per tile of the second launch, 0 if there is none */
-    uint32_t narrow_workgroups; /* workgroups of that launch */
+    uint32_t narrow_tile_n;     /* KERNEL_DMA_256: columns per tile of the narrow tiles, 0 if there are none */
+    uint32_t narrow_workgroups; /* workgroups that run them, beyond `workgroups` */
     size_t workspace_bytes;     /* bytes of the workspace this plan uses (0: the call runs without) */
 } ascq_matmul_plan;
 

@@ -216,10 +216,10 @@ def test_matmul_plan_of_the_benchmark_shapes():
     """The plan query answers without a GPU (pointers are only inspected) and names what the dispatcher does."""
     assert C.sizeof(abi.MatmulPlan) == 10 * 4 + 8
     # M=2048, K=4096, N=11008: 8 x 43 tiles of 256 x 256 = 344 = one full round of 256 + 88; the last 11 tile columns
-    # (2816 columns of C) go to a second launch with 256 x 128 tiles
+    # (2816 columns of C) go to further workgroups of the same launch with 256 x 128 tiles
     p, _ = _plan(2048, 11008, 4096)
     assert (p.kernel, p.tile_m, p.tile_n, p.tile_k) == (abi.MM_KERNEL_DMA_256, 256, 256, 128)
-    assert (p.workgroups, p.narrow_tile_n, p.narrow_workgroups, p.launches) == (256, 128, 176, 2)
+    assert (p.workgroups, p.narrow_tile_n, p.narrow_workgroups, p.launches) == (256, 128, 176, 1)
     assert p.k_splits == 1 and p.workspace_bytes == 0 and p.lds_bytes == 2 * (256 * 128 * 2) + 1024
     # decode: weight streams, one per SIMD of 256 compute units, and a kernel that adds their pieces
     p, need = _plan(1, 11008, 4096)
