@@ -9,7 +9,7 @@ import os
 # ascq_status
 OK, EINVAL, EUNSUPPORTED, EALIGN, EHIP, ENULL = range(6)
 # ascq_dtype
-F16, BF16, F32, I8, I4, I32, U64 = range(7)
+F16, BF16, F32, I8, I4, I32, U64, E8M0 = range(8)
 # ascq_policy
 PER_TENSOR, PER_CHANNEL, PER_TOKEN, PER_GROUP = range(4)
 # ascq_round_mode (values of the reference's RoundMode enum)

@@ -207,14 +207,17 @@ class AscendAntiQuantParam:
     group_size: int = 0
 
 
-def _antiquant_policy(compute, dst, src, scale, offset, para, policy, config):
-    d = abi.AntiQuantPolicyDesc(policy=policy, src_format=_QDST[src.dtype], dst_dtype=_dt(dst),
+def _antiquant_policy(compute, dst, src, scale, offset, para, policy, config, src_format=None):
+    d = abi.AntiQuantPolicyDesc(policy=policy, src_format=_QDST[src.dtype] if src_format is None else src_format,
+                                dst_dtype=_dt(dst),
                                 compute=compute, has_offset=int(config.has_offset),
                                 is_transpose=int(config.is_transpose), k_dim=config.k_dim, m=para.m, n=para.n,
                                 cal_count=para.cal_count, group_size=para.group_size)
     if policy == abi.PER_TENSOR:
         d.scale_dtype, d.scale, d.offset = _dt(dst), float(scale), float(offset) if config.has_offset else 0.0
         scale = offset = None
+    elif d.src_format in (abi.QDST_FP4_E2M1, abi.QDST_FP4_E1M2):
+        d.scale_dtype = abi.E8M0        # one byte per group: 2^(code - 127)
     else:
         d.scale_dtype = _dt(scale)
     check(load_library().ascq_antiquant_policy(C.byref(d), _ptr(dst), _ptr(src), _ptr(scale),
@@ -222,11 +225,13 @@ def _antiquant_policy(compute, dst, src, scale, offset, para, policy, config):
     return dst
 
 
-def ascend_antiquant_policy(dst, src, scale, offset, para, policy, config=AscendAntiQuantConfig()):
+def ascend_antiquant_policy(dst, src, scale, offset, para, policy, config=AscendAntiQuantConfig(), src_format=None):
     """AscendAntiQuant<dstT, srcT, scaleT, config, policy>(dst, src, scale, offset, para) for PER_TOKEN / PER_GROUP:
     src int8 / torch.float8_e4m3fn / torch.float8_e5m2 [m, n], arithmetic in the scale's dtype.
-    ref: impl/adv_api/detail/quantization/antiquant/ascend_antiquant_3510_impl.h:2166-2222."""
-    return _antiquant_policy(abi.COMPUTE_SCALE_T, dst, src, scale, offset, para, policy, config)
+    src_format=abi.QDST_FP4_E2M1 / QDST_FP4_E1M2 (PER_GROUP, no offset): src is a uint8 tensor [m, n / 2] holding two
+    4-bit floats per byte (fp4x2_e2m1_t / fp4x2_e1m2_t), scale a uint8 tensor of fp8_e8m0 codes, dst half / bfloat16.
+    ref: impl/adv_api/detail/quantization/antiquant/ascend_antiquant_3510_impl.h:1727-1779, 2166-2222."""
+    return _antiquant_policy(abi.COMPUTE_SCALE_T, dst, src, scale, offset, para, policy, config, src_format)
 
 
 def antiquantize(dst, src, scale, offset, para, policy, config=AscendAntiQuantConfig()):

@@ -929,6 +929,53 @@ __global__ __launch_bounds__(kThreads) void antiquant_policy_scalar_kernel(AntiQ
     }
 }
 
+// fp4 sources with fp8_e8m0 scales (PER_GROUP): one lane = 8 columns (4 source bytes, 16 bytes out).  The product of
+// a 4-bit float and a power of two is exact in fp32 and in bfloat16 (infinity on overflow), so dst(bf16) is that
+// product and dst(half) its saturating half-even cast.
+__device__ __forceinline__ float fp4_code_to_f32(uint32_t code, bool e1m2)
+{
+    const uint32_t mag = code & 7u;
+    float v;
+    if (e1m2) {
+        v = static_cast<float>(mag) * 0.25f;  // 0, 0.25 .. 1.75
+    } else {
+        // e2m1: 0, 0.5, then (1 + m / 2) * 2^(e - 1)
+        const uint32_t e = mag >> 1, m = mag & 1u;
+        v = e == 0u ? 0.5f * static_cast<float>(m)
+                    : (1.0f + 0.5f * static_cast<float>(m)) * static_cast<float>(1u << (e - 1u));
+    }
+    return (code & 8u) ? -v : v;
+}
+__device__ __forceinline__ float e8m0_to_f32(uint32_t code)
+{
+    // 2^(code - 127): the code is the fp32 exponent field; 0 is 2^-127 (a subnormal), 255 is NaN
+    const uint32_t bits = code == 0u ? 0x00400000u : (code == 255u ? 0x7FC00000u : code << 23);
+    return __uint_as_float(bits);
+}
+template <int kDst>
+__global__ __launch_bounds__(kThreads) void antiquant_fp4_kernel(AntiQuantPolicyArgs a)
+{
+    const uint32_t j = (blockIdx.x * blockDim.x + threadIdx.x) * 8u;
+    if (j >= a.n) {
+        return;
+    }
+    const bool e1m2 = a.src_format == ASCQ_QDST_FP4_E1M2;
+    const uint8_t* sc = static_cast<const uint8_t*>(a.scale);
+    for (uint32_t r = blockIdx.y; r < a.rows; r += gridDim.y) {
+        const uint32_t raw = __builtin_nontemporal_load(
+            reinterpret_cast<const uint32_t*>(a.src + (static_cast<size_t>(r) * a.n + j) / 2u));
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const size_t pi = a.along_n ? static_cast<size_t>(r) * a.params_per_row + (j + e) / a.group_size
+                                        : static_cast<size_t>(r / a.group_size) * a.n + j + e;
+            const float p = fp4_code_to_f32((raw >> (4 * e)) & 15u, e1m2) * e8m0_to_f32(sc[pi]);
+            v[e] = kDst == ASCQ_F16 ? aqp_saturate<ASCQ_F16>(p) : p;
+        }
+        store8<kDst, true>(a.dst, static_cast<size_t>(r) * a.n + j, v);
+    }
+}
+
 template <int kPar, int kCt, int kDst>
 int launch_antiquant_policy(const AntiQuantPolicyArgs& a, bool vec, hipStream_t st)
 {
@@ -1295,8 +1342,46 @@ extern "C" int ascq_antiquant_policy(const ascq_antiquant_policy_desc* d, void* 
                      "ascq_antiquant_policy: PER_TENSOR / PER_CHANNEL take half or bfloat16 parameters of the output's "
                      "type (scale dtype %d, dst dtype %d)", d->scale_dtype, d->dst_dtype);
     }
-    ASCQ_REQUIRE(d->src_format >= ASCQ_QDST_I8 && d->src_format <= ASCQ_QDST_FP8_E5M2, ASCQ_EUNSUPPORTED,
-                 "ascq_antiquant_policy: source format %d is not int8 / fp8_e4m3fn / fp8_e5m2", d->src_format);
+    ASCQ_REQUIRE(d->src_format >= ASCQ_QDST_I8 && d->src_format <= ASCQ_QDST_FP4_E1M2, ASCQ_EUNSUPPORTED,
+                 "ascq_antiquant_policy: source format %d is not int8 / fp8_e4m3fn / fp8_e5m2 / fp4_e2m1 / fp4_e1m2",
+                 d->src_format);
+    if (d->src_format >= ASCQ_QDST_FP4_E2M1) {
+        // ref: AscendAntiQuant.md table 3 (the fp4x2 rows), antiquantize_impl.h:53-58
+        ASCQ_REQUIRE(d->policy == ASCQ_PER_GROUP, ASCQ_EUNSUPPORTED,
+                     "ascq_antiquant_policy: fp4 sources exist for PER_GROUP only");
+        ASCQ_REQUIRE(d->scale_dtype == ASCQ_E8M0 && (d->dst_dtype == ASCQ_F16 || d->dst_dtype == ASCQ_BF16),
+                     ASCQ_EUNSUPPORTED,
+                     "ascq_antiquant_policy: fp4 sources take fp8_e8m0 scales and give half or bfloat16 (scale dtype "
+                     "%d, dst dtype %d)", d->scale_dtype, d->dst_dtype);
+        ASCQ_REQUIRE(!d->has_offset, ASCQ_EUNSUPPORTED, "ascq_antiquant_policy: fp4 sources have no offset");
+        ASCQ_REQUIRE(d->k_dim == 0 || d->k_dim == 1, ASCQ_EINVAL, "ascq_antiquant_policy: kDim must be 0 or 1");
+        ASCQ_REQUIRE(d->group_size > 0 && d->group_size % 32 == 0, ASCQ_EINVAL,
+                     "ascq_antiquant_policy: groupSize %u must be a positive multiple of 32", d->group_size);
+        ASCQ_REQUIRE(d->n > 0 && d->n % 8 == 0, ASCQ_EALIGN, "ascq_antiquant_policy: fp4 rows need n %% 8 == 0 (n %u)",
+                     d->n);
+        ASCQ_REQUIRE(d->cal_count % d->n == 0 && static_cast<uint64_t>(d->m) * d->n >= d->cal_count, ASCQ_EINVAL,
+                     "ascq_antiquant_policy: calCount %u must be a multiple of n %u and at most m*n", d->cal_count,
+                     d->n);
+        ASCQ_REQUIRE((reinterpret_cast<uintptr_t>(src) & 3u) == 0 && aligned16(dst), ASCQ_EALIGN,
+                     "ascq_antiquant_policy: fp4 sources need a 4-byte aligned src and a 16-byte aligned dst");
+        if (d->cal_count == 0) {
+            return ASCQ_OK;
+        }
+        ASCQ_REQUIRE(!ranges_overlap(dst, static_cast<size_t>(d->cal_count) * 2u, src, d->cal_count / 2u), ASCQ_EINVAL,
+                     "ascq_antiquant_policy: dst overlaps src");
+        const int along = (d->k_dim == 1) != (d->is_transpose != 0) ? 1 : 0;
+        AntiQuantPolicyArgs fa{dst, static_cast<const uint8_t*>(src), scale, nullptr, d->cal_count / d->n, d->n,
+                               d->policy, along, 0, d->src_format, d->group_size,
+                               (d->n + d->group_size - 1) / d->group_size, 0.0f, 0.0f};
+        RowLaunch rl = row_launch(d->n / 8, fa.rows, 1);
+        hipStream_t fst = static_cast<hipStream_t>(stream);
+        if (d->dst_dtype == ASCQ_F16) {
+            antiquant_fp4_kernel<ASCQ_F16><<<rl.grid, rl.block, 0, fst>>>(fa);
+        } else {
+            antiquant_fp4_kernel<ASCQ_BF16><<<rl.grid, rl.block, 0, fst>>>(fa);
+        }
+        return launch_status("ascq_antiquant_policy");
+    }
     const int par = d->scale_dtype, dt = d->dst_dtype;
     ASCQ_REQUIRE(par == ASCQ_F16 || par == ASCQ_BF16 || par == ASCQ_F32, ASCQ_EUNSUPPORTED,
                  "ascq_antiquant_policy: scale dtype %d is not half / bfloat16 / float", par);

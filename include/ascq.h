@@ -43,7 +43,8 @@ typedef enum ascq_dtype {
     ASCQ_I8 = 3,
     ASCQ_I4 = 4, /* two per byte, element 2j in the low nibble (ref: impl/utils/common_types.h:57-111) */
     ASCQ_I32 = 5,
-    ASCQ_U64 = 6 /* fixpipe quant parameter word, fp32 scale in the low 32 bits */
+    ASCQ_U64 = 6, /* fixpipe quant parameter word, fp32 scale in the low 32 bits */
+    ASCQ_E8M0 = 7 /* fp8_e8m0_t: one byte, the value 2^(code - 127); code 255 is NaN (scales of the fp4 sources) */
 } ascq_dtype;
 
 /* ref: include/adv_api/quantization/ascend_quant_utils.h:73-80 (AscendQuantPolicy) */
@@ -224,6 +225,13 @@ int ascq_antiquant(const ascq_antiquant_desc* desc, void* dst, const void* src, 
  * with ct = the scale dtype (ASCQ_COMPUTE_SCALE_T: AscendAntiQuant) or fp32 (ASCQ_COMPUTE_F32: AntiQuantize); every
  * source value is exact in every ct.  A 16-bit ct requires dst_dtype == scale_dtype; an fp32 result is rounded
  * half-even to a 16-bit dst, saturating at the largest finite value (NaN -> +0).
+ *   fp4 sources (src_format ASCQ_QDST_FP4_E2M1 / FP4_E1M2: two values per byte, even element in the low nibble, src
+ *              holds cal_count / 2 bytes): PER_GROUP only, scale_dtype ASCQ_E8M0 (one byte per group, same indexing
+ *              as above), no offset, dst half | bfloat16: dst = bf16(src) * bf16(2^(code - 127)) as a bfloat16
+ *              product (exact: at most 3 significant bits times a power of two; overflow gives infinity), a scale
+ *              code of 255 is NaN; a half dst is the saturating half-even cast of that product (NaN -> +0).
+ *              n % 8 == 0.  (ref: impl/adv_api/detail/quantization/antiquant/ascend_antiquant_3510_impl.h:49-57
+ *              (codes 0 and 255), :1727-1779 (groups along n), :1793-1850 (along m); AscendAntiQuant.md 表3.)
  *   PER_CHANNEL (AntiQuantize only, ASCQ_COMPUTE_F32): scale / offset [n] of dst_dtype (half | bfloat16).
  *   PER_TENSOR  (AntiQuantize only, ASCQ_COMPUTE_F32): the scalars `scale` / `offset` of the descriptor, taken as
  *              dst_dtype values (rounded once to it); the scale / offset pointers are ignored.
@@ -232,8 +240,8 @@ int ascq_antiquant(const ascq_antiquant_desc* desc, void* dst, const void* src, 
  */
 typedef struct ascq_antiquant_policy_desc {
     int32_t policy;      /* ASCQ_PER_TOKEN | ASCQ_PER_GROUP; with ASCQ_COMPUTE_F32 also PER_TENSOR | PER_CHANNEL */
-    int32_t src_format;  /* ASCQ_QDST_I8 | ASCQ_QDST_FP8_E4M3FN | ASCQ_QDST_FP8_E5M2 */
-    int32_t scale_dtype; /* ASCQ_F16 | ASCQ_BF16 | ASCQ_F32: dtype of the scale / offset tensors */
+    int32_t src_format;  /* ASCQ_QDST_I8 | ASCQ_QDST_FP8_E4M3FN | ASCQ_QDST_FP8_E5M2 | ASCQ_QDST_FP4_E2M1 | _E1M2 */
+    int32_t scale_dtype; /* ASCQ_F16 | ASCQ_BF16 | ASCQ_F32: dtype of the scale / offset tensors; ASCQ_E8M0 for fp4 */
     int32_t dst_dtype;   /* ASCQ_F16 | ASCQ_BF16 | ASCQ_F32 */
     int32_t compute;     /* ASCQ_COMPUTE_SCALE_T | ASCQ_COMPUTE_F32 */
     int32_t has_offset;

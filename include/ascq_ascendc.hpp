@@ -57,6 +57,9 @@ struct fp8_e4m3fn_t {
 struct fp8_e5m2_t {
     uint8_t bits;
 };
+struct fp8_e8m0_t {  // a power of two: 2^(bits - 127); the scales of the fp4 sources of AscendAntiQuant
+    uint8_t bits;
+};
 struct fp4x2_e2m1_t {  // two 4-bit floats per byte, even element in the low nibble
     uint8_t pair;
 };
@@ -117,6 +120,10 @@ struct DTypeOf<int32_t> {
 template <>
 struct DTypeOf<uint64_t> {
     static constexpr int32_t value = ASCQ_U64;
+};
+template <>
+struct DTypeOf<fp8_e8m0_t> {
+    static constexpr int32_t value = ASCQ_E8M0;
 };
 
 // View of a caller-owned device buffer: the counterpart of LocalTensor / GlobalTensor.  `size` counts elements

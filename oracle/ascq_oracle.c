@@ -863,9 +863,35 @@ static uint16_t f32_to_bf16_sat(float v)
     return orc_f32_to_bf16(v);
 }
 
+/* fp4 sources, fp8_e8m0 scales (PER_GROUP): scale = 2^(code - 127) held as a bfloat16 (code 0: bits 0x0040 = 2^-127,
+ * code 255: NaN), dst = bf16(src) * scale as a bfloat16 product, then the saturating cast when dst is half.
+ * ref: impl/adv_api/detail/quantization/antiquant/ascend_antiquant_3510_impl.h:49-57, 69-74, 1727-1779. */
+static void antiquant_fp4(const ascq_antiquant_policy_desc* d, uint16_t* dst, const uint8_t* src, const uint8_t* scale)
+{
+    size_t n = d->n, rows = n ? d->cal_count / n : 0;
+    int along_n = (d->k_dim == 1) != (d->is_transpose != 0);
+    size_t ppr = (n + d->group_size - 1) / d->group_size;
+    for (size_t i = 0; i < rows; ++i) {
+        for (size_t j = 0; j < n; ++j) {
+            size_t e = i * n + j;
+            size_t pi = along_n ? i * ppr + j / d->group_size : (i / d->group_size) * n + j;
+            uint8_t code = (e & 1) ? (uint8_t)(src[e / 2] >> 4) : (uint8_t)(src[e / 2] & 15);
+            uint16_t xb = orc_f32_to_bf16(orc_fp4_to_f32(code, d->src_format == ASCQ_QDST_FP4_E1M2)); /* exact */
+            uint8_t c = scale[pi];
+            uint16_t sb = c == 0 ? 0x0040 : (c == 255 ? 0x7FFF : (uint16_t)(c << 7));
+            uint16_t prod = orc_bf16_mul(xb, sb);
+            dst[e] = d->dst_dtype == ASCQ_BF16 ? prod : f32_to_f16_sat(orc_bf16_to_f32(prod));
+        }
+    }
+}
+
 int orc_antiquant_policy(const ascq_antiquant_policy_desc* d, void* dst, const uint8_t* src, const void* scale,
                          const void* offset)
 {
+    if (d->src_format == ASCQ_QDST_FP4_E2M1 || d->src_format == ASCQ_QDST_FP4_E1M2) {
+        antiquant_fp4(d, (uint16_t*)dst, src, (const uint8_t*)scale);
+        return 0;
+    }
     size_t n = d->n, rows = n ? d->cal_count / n : 0;
     int along_n = (d->k_dim == 1) != (d->is_transpose != 0);
     size_t ppr = d->group_size ? (n + d->group_size - 1) / d->group_size : 0;

@@ -467,6 +467,42 @@ void test_unified_surface()
     }
 }
 
+void test_antiquant_fp4()
+{
+    std::printf("[case] AscendAntiQuant<half, fp4x2_e2m1_t, fp8_e8m0_t> PER_GROUP 12x256, groupSize 64\n");
+    Rng r{21};
+    const uint32_t m = 12, n = 256, gs = 64;
+    std::vector<uint8_t> packed(m * n / 2), sc(m * n / gs);
+    for (auto& e : packed) e = static_cast<uint8_t>(r.integer(0, 255));
+    for (auto& e : sc) e = static_cast<uint8_t>(r.integer(100, 150));  // 2^-27 .. 2^23: part of it past half's range
+    DeviceBuffer<uint8_t> dp(packed), dsc(sc);
+    DeviceBuffer<uint16_t> dd(m * n);
+    ascq::AscendAntiQuantConfig cfg{};
+    cfg.hasOffset = false;
+    ascq::AscendAntiQuantParam para{};
+    para.m = m;
+    para.n = n;
+    para.calCount = m * n;
+    para.groupSize = gs;
+    ascq::AscendAntiQuant(dd.view<ascq::half>(m * n), dp.view<ascq::fp4x2_e2m1_t>(m * n),
+                          dsc.view<ascq::fp8_e8m0_t>(m * n / gs), dsc.view<ascq::fp8_e8m0_t>(m * n / gs), para, cfg,
+                          ascq::AscendAntiQuantPolicy::PER_GROUP);
+    ascq_antiquant_policy_desc d{};
+    d.policy = ASCQ_PER_GROUP;
+    d.src_format = ASCQ_QDST_FP4_E2M1;
+    d.scale_dtype = ASCQ_E8M0;
+    d.dst_dtype = ASCQ_F16;
+    d.compute = ASCQ_COMPUTE_SCALE_T;
+    d.k_dim = 1;
+    d.m = m;
+    d.n = n;
+    d.cal_count = m * n;
+    d.group_size = gs;
+    std::vector<uint16_t> want(m * n);
+    orc_antiquant_policy(&d, want.data(), packed.data(), sc.data(), nullptr);
+    expect_equal("AscendAntiQuant fp4 per group", dd.download(), want);
+}
+
 void test_errors()
 {
     std::printf("[case] argument errors surface as ascq::Error\n");
@@ -511,6 +547,7 @@ int main()
     test_matmul();
     test_antiquant_matmul();
     test_unified_surface();
+    test_antiquant_fp4();
     test_errors();
     std::printf("%s\n", g_failed ? "FAILED" : "ALL PASSED");
     return g_failed ? 1 : 0;

@@ -475,6 +475,65 @@ def test_antiquantize_per_channel_and_per_tensor(fmt, dst_dt, policy, has_offset
         assert np.array_equal(bits(dst), want)
 
 
+@pytest.mark.parametrize("fmt", [abi.QDST_FP4_E2M1, abi.QDST_FP4_E1M2])
+@pytest.mark.parametrize("dst_dt", [abi.F16, abi.BF16])
+@pytest.mark.parametrize("mode", ["group_n", "group_m", "group_m_via_transpose"])
+def test_antiquant_fp4_sources(fmt, dst_dt, mode):
+    """fp4x2 sources with fp8_e8m0 scales, PER_GROUP along either axis, half and bfloat16 outputs: bit-equal to the
+    oracle (NaN outputs compared as NaN).  The scales cover both ends of the exponent range, NaN, and products beyond
+    half's range."""
+    k_dim, tr = {"group_n": (1, 0), "group_m": (0, 0), "group_m_via_transpose": (1, 1)}[mode]
+    along_n = (k_dim == 1) != bool(tr)
+    for (m, n, cal) in [(64, 256, 64 * 256), (40, 96, 32 * 96), (33, 2080, 33 * 2080)]:
+        announce("antiquant fp4", fmt, dst_dt, mode, m, n, cal)
+        rng = np.random.default_rng(m + n + fmt)
+        gs = 32
+        packed = rng.integers(0, 256, (m, n // 2)).astype(np.uint8)
+        packed.reshape(-1)[:256] = np.arange(256, dtype=np.uint8)                 # every code in both nibbles
+        sshape = (m, -(-n // gs)) if along_n else (-(-m // gs), n)
+        sc = rng.integers(96, 160, sshape).astype(np.uint8)
+        sc.reshape(-1)[:6] = [0, 1, 254, 255, 127, 143]
+        dst = torch.zeros((m, n), dtype=TDT[dst_dt], device=DEV)
+        cfg = ops.AscendAntiQuantConfig(has_offset=False, is_transpose=bool(tr), k_dim=k_dim)
+        para = ops.AscendAntiQuantParam(m=m, n=n, cal_count=cal, group_size=gs)
+        ops.ascend_antiquant_policy(dst, to_dev(packed), to_dev(sc), None, para, abi.PER_GROUP, cfg, src_format=fmt)
+        d = abi.AntiQuantPolicyDesc(policy=abi.PER_GROUP, src_format=fmt, scale_dtype=abi.E8M0, dst_dtype=dst_dt,
+                                    compute=abi.COMPUTE_SCALE_T, has_offset=0, is_transpose=tr, k_dim=k_dim, m=m, n=n,
+                                    cal_count=cal, group_size=gs)
+        want = orc.antiquant_policy(d, packed, sc, None).view(np.uint16)
+        got = bits(dst)
+        rows = cal // n
+        if dst_dt == abi.BF16:
+            nan_w = (want & 0x7FFF) > 0x7F80
+            nan_g = (got & 0x7FFF) > 0x7F80
+            assert np.array_equal(nan_w[:rows], nan_g[:rows]) and nan_w.any()
+            assert np.array_equal(got[:rows][~nan_w[:rows]], want[:rows][~nan_w[:rows]])
+            if fmt == abi.QDST_FP4_E2M1:          # 6 * 2^127 overflows bfloat16; 1.75 * 2^127 (e1m2) does not
+                assert np.any((want[:rows] & 0x7FFF) == 0x7F80)
+        else:
+            assert np.array_equal(got[:rows], want[:rows])
+            assert np.any((want[:rows] & 0x7FFF) == 0x7BFF)                      # saturation was exercised
+        assert not got[rows:].any()
+
+
+def test_antiquant_fp4_rejects():
+    announce("antiquant fp4 rejects")
+    src = torch.zeros((4, 32), dtype=torch.uint8, device=DEV)
+    sc = torch.full((4, 2), 127, dtype=torch.uint8, device=DEV)
+    dst = torch.zeros((4, 64), dtype=torch.float16, device=DEV)
+    para = ops.AscendAntiQuantParam(m=4, n=64, cal_count=256, group_size=32)
+    with pytest.raises(ops.AscqError, match="PER_GROUP only"):
+        ops.ascend_antiquant_policy(dst, src, sc[:, 0].contiguous(), None, para, abi.PER_TOKEN,
+                                    ops.AscendAntiQuantConfig(has_offset=False), src_format=abi.QDST_FP4_E2M1)
+    with pytest.raises(ops.AscqError, match="no offset"):
+        ops.ascend_antiquant_policy(dst, src, sc, sc, para, abi.PER_GROUP,
+                                    ops.AscendAntiQuantConfig(has_offset=True), src_format=abi.QDST_FP4_E1M2)
+    dst32 = torch.zeros((4, 64), dtype=torch.float32, device=DEV)
+    with pytest.raises(ops.AscqError, match="half or bfloat16"):
+        ops.ascend_antiquant_policy(dst32, src, sc, None, para, abi.PER_GROUP,
+                                    ops.AscendAntiQuantConfig(has_offset=False), src_format=abi.QDST_FP4_E2M1)
+
+
 @pytest.mark.parametrize("policy", ["tensor", "channel", "token", "group0", "group1"])
 def test_dequantize_is_the_matching_ascend_dequant(policy):
     """The unified Dequantize: each policy gives what the operator it forwards to gives (and the oracle)."""

@@ -662,3 +662,43 @@ def test_antiquantize_per_channel_and_per_tensor_against_numpy_fp32(fmt):
     wantb = ((torch.from_numpy(x) + np.float32(ovb)) * np.float32(svb)).bfloat16()
     gotb = orc.antiquant_policy(desc(abi.PER_TENSOR, abi.BF16, scale=sv, offset=ov), codes, None, None)
     assert np.array_equal(gotb.view(U16), wantb.view(torch.int16).numpy().view(U16))
+
+
+@pytest.mark.parametrize("fmt", [abi.QDST_FP4_E2M1, abi.QDST_FP4_E1M2])
+@pytest.mark.parametrize("k_dim", [0, 1])
+def test_antiquant_fp4_sources_are_value_times_power_of_two(fmt, k_dim):
+    """fp4 sources with fp8_e8m0 scales (ascend_antiquant_3510_impl.h:1727-1779): every product of a 4-bit float and
+    2^(code - 127) is exact, so the expected bfloat16 output is the closed form ldexp(value, code - 127) (numpy float64,
+    then torch's bfloat16 conversion, which has nothing to round), and the half output its clipped half-even cast.
+    The special scale codes follow the reference's constants (:69-74): 0 is 2^-127, 255 is NaN."""
+    rng = np.random.default_rng(fmt * 2 + k_dim)
+    m, n, gs = 64, 96, 32
+    codes = rng.integers(0, 16, (m, n)).astype(np.uint8)
+    codes.reshape(-1)[:16] = np.arange(16)
+    packed = (codes[:, 0::2] | (codes[:, 1::2] << 4)).astype(np.uint8)
+    grid = np.array([0, .5, 1, 1.5, 2, 3, 4, 6] if fmt == abi.QDST_FP4_E2M1 else [0, .25, .5, .75, 1, 1.25, 1.5, 1.75])
+    vals = np.where(codes & 8, -1.0, 1.0) * grid[codes & 7]
+    sshape = (m, n // gs) if k_dim == 1 else (m // gs, n)
+    sc = rng.integers(100, 150, sshape).astype(np.uint8)             # 2^-27 .. 2^22: inside half's range and beyond it
+    sc.reshape(-1)[:4] = [0, 1, 254, 127]                            # the ends of the exponent range, and 1.0
+    full = np.repeat(sc, gs, axis=1) if k_dim == 1 else np.repeat(sc, gs, axis=0)
+    exact = np.ldexp(vals, full.astype(np.int64) - 127)              # float64: exact, 6 * 2^127 overflows bfloat16 only
+    with np.errstate(over="ignore"):
+        want_bf16 = torch.from_numpy(exact.astype(np.float32)).bfloat16().view(torch.int16).numpy().view(U16)
+    d = abi.AntiQuantPolicyDesc(policy=abi.PER_GROUP, src_format=fmt, scale_dtype=abi.E8M0, dst_dtype=abi.BF16,
+                                compute=abi.COMPUTE_SCALE_T, has_offset=0, is_transpose=0, k_dim=k_dim, m=m, n=n,
+                                cal_count=m * n, group_size=gs)
+    got = orc.antiquant_policy(d, packed, sc, None)
+    assert np.array_equal(got.view(U16), want_bf16)
+    d.dst_dtype = abi.F16
+    got16 = orc.antiquant_policy(d, packed, sc, None)
+    with np.errstate(over="ignore"):
+        want16 = np.clip(exact, -65504.0, 65504.0).astype(np.float16)
+    assert np.array_equal(got16.view(U16), want16.view(U16))
+    # a NaN scale: NaN in bfloat16, +0 through the saturating cast to half
+    sc2 = np.full(sshape, 255, dtype=np.uint8)
+    d.dst_dtype = abi.BF16
+    nb = orc.antiquant_policy(d, packed, sc2, None).view(U16)
+    assert np.all((nb & 0x7F80) == 0x7F80) and np.all(nb & 0x7F)
+    d.dst_dtype = abi.F16
+    assert not orc.antiquant_policy(d, packed, sc2, None).view(U16).any()
