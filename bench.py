@@ -14,6 +14,8 @@ several buffer sets larger than the 256 MB Infinity Cache so that their input is
 The default of 1000 timed steps after 100 warm-up steps keeps the GPU busy for about 0.1 s.  After an idle period the
 clocks take a few milliseconds of load to reach their sustained state: a 50-step region (6 ms) measured 124 us per
 step and 108 us per GEMM, a 1000-step region 102-106 us per step and 95 us per GEMM, on the same box minutes apart.
+For the same reason `--settle` untimed steps (300, about 30 ms; reported as config.settle_steps) run before the W
+warm-up steps of the headline, so that a caller's short --steps/--warmup is measured at the sustained clock as well.
 """
 import argparse
 import json
@@ -41,6 +43,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=100)
+    ap.add_argument("--settle", type=int, default=300,
+                    help="untimed steps of the headline workload before its warm-up, so that short --steps/--warmup "
+                         "runs are also measured at the sustained clock (0 disables)")
     ap.add_argument("--quick", action="store_true", help="headline + W4A16 GEMV only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="run a single workload: w8a8 | w4a16 | quant | dequant | antiquant | group")
@@ -108,7 +113,7 @@ def main():
         torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------ W8A8 linear (config 3)
-    def w8a8(M, steps, warmup, sets=1):
+    def w8a8(M, steps, warmup, sets=1, settle=0):
         """`sets` > 1 rotates the weights over several copies (together larger than the Infinity Cache) so that the
         weight-bound small-M cases read them from HBM."""
         K, N = 4096, 11008
@@ -135,6 +140,8 @@ def main():
         # Pass 1: the timed region proper (quant + GEMM per step), no events inside it: an event record idles the
         # queue for ~6 us.  Pass 2: the GEMM launches of the same steps back to back between one pair of events on
         # the launch stream, which gives the average duration of the GEMM launch itself.
+        for i in range(settle):
+            step(i, None, None)
         ms, _ = timed(lambda i, a, b: step(i, None, None), steps, warmup)
         ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
@@ -265,7 +272,7 @@ def main():
         print(json.dumps({only: strip(fn())}))
         return
 
-    head = w8a8(2048, args.steps, args.warmup)
+    head = w8a8(2048, args.steps, args.warmup, settle=args.settle)
     out = {
         "metric": "w8a8_linear_int8_tops_m2048_k4096_n11008",
         "value": head["tops"],
@@ -282,7 +289,8 @@ def main():
         "config": {"workload": "BASELINE configs[2] (W8A8 LLM linear) at M=2048: bf16 x [2048,4096] -> dynamic "
                                "per-token int8 quant -> int8 GEMM with W [4096,11008] -> fused (channel x token) "
                                "dequant to bf16; one step = quant kernel + GEMM kernel",
-                   "m": 2048, "k": 4096, "n": 11008, "ops_per_step": head["ops"]},
+                   "m": 2048, "k": 4096, "n": 11008, "ops_per_step": head["ops"],
+                   "settle_steps": args.settle},
         # The GEMM is one launch that runs two tile shapes: 256x256 tiles for the full round of 256 workgroups and
         # 256x128 tiles for the last partial round; `achieved` is the 2*M*K*N operations over the average duration of
         # the launch, from one pair of events around `steps` back-to-back GEMMs.  `traffic` is HBM bytes per GEMM from
