@@ -77,21 +77,25 @@ def main():
         return torch.randint(-127, 128, shape, dtype=torch.int8, device=dev, generator=gen)
 
     def timed(fn, steps, warmup, inner=None):
-        """Times `steps` calls of fn(i) after `warmup`; returns (ms per step, ms per step of the `inner` section).
-        `inner` events are recorded by fn itself through the two lists it receives."""
-        starts, stops = [], []
+        """Times `steps` calls of fn(i, None, None) after `warmup` by the host clock between two synchronizes, then
+        the same `steps` calls again between one pair of events on the launch stream.  Returns (ms per step by the
+        host clock, ms per step by the events).  No event is recorded inside either region: a record between two
+        launches idles the queue for 3-6 us, which is a tenth of a 35 us decode step."""
         for i in range(warmup):
             fn(i, None, None)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for i in range(steps):
-            fn(warmup + i, starts, stops)
+            fn(warmup + i, None, None)
         torch.cuda.synchronize()
         wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-        kern_ms = None
-        if starts:
-            kern_ms = sum(a.elapsed_time(b) for a, b in zip(starts, stops)) / len(starts)
-        return wall_ms, kern_ms
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+        for i in range(steps):
+            fn(warmup + i, None, None)
+        ev1.record()
+        torch.cuda.synchronize()
+        return wall_ms, ev0.elapsed_time(ev1) / steps
 
     def bracket(starts, stops, call):
         if starts is None:
@@ -137,9 +141,8 @@ def main():
             ops.dynamic_quant_per_token(x, q, ts)
             bracket(starts, stops, lambda: mms[i % sets].iterate_all(c))
 
-        # Pass 1: the timed region proper (quant + GEMM per step), no events inside it: an event record idles the
-        # queue for ~6 us.  Pass 2: the GEMM launches of the same steps back to back between one pair of events on
-        # the launch stream, which gives the average duration of the GEMM launch itself.
+        # The timed region proper is quant + GEMM per step.  Then the GEMM launches of the same steps run back to
+        # back between one pair of events on the launch stream, which gives the average duration of the GEMM launch.
         for i in range(settle):
             step(i, None, None)
         ms, _ = timed(lambda i, a, b: step(i, None, None), steps, warmup)
@@ -306,9 +309,8 @@ def main():
         print(json.dumps(out))
         return
 
-    # The other workloads record a pair of events per step, which costs host time per step: past a few hundred steps
-    # the host falls behind the GPU and the kernels start from an idle queue.  They run a bounded number of steps.
-    side_steps, side_warmup = min(args.steps, 200), min(args.warmup, 20)
+    # The other workloads run a bounded number of steps so that the whole file finishes in about a minute.
+    side_steps, side_warmup = min(args.steps, 500), min(args.warmup, 50)
     gemv = w4a16(1, side_steps, side_warmup)
     out["w4a16_gemv"] = {"metric": "w4a16_decode_gemv_hbm_gbs_m1_k8192_n28672", "value": gemv["gbs"], "unit": "GB/s",
                          "workload": "BASELINE configs[3] at M=1, 4 rotating weight sets (500 MB > Infinity Cache)",
