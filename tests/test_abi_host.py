@@ -242,3 +242,14 @@ def test_matmul_plan_of_the_benchmark_shapes():
     assert L.ascq_matmul_w8a8_plan(C.byref(d), FAKE, FAKE, FAKE, None, None, None, None, 0,
                                    C.byref(abi.MatmulPlan())) == abi.EINVAL
     assert L.ascq_matmul_w8a8_plan(C.byref(d), FAKE, FAKE, FAKE, None, None, None, None, 0, None) == abi.ENULL
+
+
+def test_missing_library_is_a_loud_error_with_no_fallback(monkeypatch, tmp_path):
+    """The package has no CPU path: without libascq.so the first call raises instead of computing something else."""
+    monkeypatch.setattr(abi, "_lib", None)
+    monkeypatch.setattr(abi, "LIB_PATH", str(tmp_path / "libascq.so"))
+    with pytest.raises(RuntimeError, match="is missing"):
+        abi.load_library()
+    from ascq import ops
+    with pytest.raises(RuntimeError, match="is missing"):
+        ops.dequant_dst_stride("float16", 40)
