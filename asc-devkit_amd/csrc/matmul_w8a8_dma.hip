@@ -212,37 +212,48 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_
             bf[j] = i32x4{lo[0], lo[1], hi[0], hi[1]};
         }
     };
-    auto compute = [&](const char* As, const char* Bs) {
-        i32x4 af[2][TI], bf[2][TJ];
+    // Fragment registers live across K steps: buffer 0 holds sub-steps 0 and 2, buffer 1 sub-steps 1 and 3.
+    i32x4 af[2][TI], bf[2][TJ];
+    auto mfma_block = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < TI; ++i) {
+#pragma unroll
+            for (int j = 0; j < TJ; ++j) {
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[buf][i], bf[buf][j], acc[i][j], 0, 0, 0);
+            }
+        }
+    };
+    // one LDS read behind each MFMA
+    auto interleave = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int n = 0; n < TI * TJ; ++n) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, (TI + 2 * TJ + TI * TJ - 1) / (TI * TJ), 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // Sub-steps 0-2 of a K step whose sub-step-0 fragments are already in buffer 0; on return the fragments of
+    // sub-step 3 are on their way into buffer 1 and nothing else of the stage will be read.
+    auto head = [&](const char* As, const char* Bs) __attribute__((always_inline)) {
         // Re-materialise the bases inside the loop body: the constant parts of every address then fold into the
         // 16-bit offset field of the DS instructions instead of being hoisted into dozens of registers.
 #pragma unroll
         for (int q = 0; q < 4; ++q) asm volatile("" : "+v"(a_base[q]));
 #pragma unroll
         for (int q = 0; q < 2; ++q) asm volatile("" : "+v"(b_base[q]));
-        load_frags(As, Bs, 0, af[0], bf[0]);
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            if (ks < 3) {
-                load_frags(As, Bs, ks + 1, af[(ks + 1) & 1], bf[(ks + 1) & 1]);
-            }
-#pragma unroll
-            for (int i = 0; i < TI; ++i) {
-#pragma unroll
-                for (int j = 0; j < TJ; ++j) {
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks & 1][i], bf[ks & 1][j], acc[i][j], 0, 0, 0);
-                }
-            }
-            if (ks < 3) {
-                // one LDS read of the next sub-step behind each MFMA of this one
-#pragma unroll
-                for (int n = 0; n < TI * TJ; ++n) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x100, (TI + 2 * TJ + TI * TJ - 1) / (TI * TJ), 0);
-                }
-            }
-            __builtin_amdgcn_sched_barrier(0);
+        for (int ks = 0; ks < 3; ++ks) {
+            load_frags(As, Bs, ks + 1, af[(ks + 1) & 1], bf[(ks + 1) & 1]);
+            mfma_block(ks & 1);
+            interleave();
         }
+    };
+    // Behind the barrier: the MFMAs of sub-step 3 run while the first fragments of the next K step (stage An, Bn)
+    // arrive, so the matrix pipe has work during the burst of LDS reads that follows every barrier.
+    auto tail = [&](const char* An, const char* Bn) __attribute__((always_inline)) {
+        load_frags(An, Bn, 0, af[0], bf[0]);
+        mfma_block(1);
+        interleave();
     };
 
     if (steps != 0) {
@@ -253,21 +264,45 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_
     // A wavefront whose rows all lie past the end of the tile's group (ragged grouped tiles) skips the matrix work and
     // only keeps the loads and barriers going: its SIMD then runs one wavefront's MFMAs per K step instead of two.
     const bool wave_active = !kGrouped || row0 + wm * (TI * 32u) < row_end;
-    uint32_t s = 0;
-    for (; s + 1 < steps; s += 2) {
-        issue((s + 1) * BK, A1, B1);
-        if (wave_active) compute(A0, B0);
-        asm volatile("s_waitcnt vmcnt(0)");
-        __syncthreads();
-        if (s + 2 < steps) {
-            issue((s + 2) * BK, A0, B0);
-        }
-        if (wave_active) compute(A1, B1);
-        asm volatile("s_waitcnt vmcnt(0)");
-        __syncthreads();
+    if (steps > 1) {
+        issue(BK, A1, B1);
     }
-    if (s < steps) {  // odd number of K steps: the last one sits in stage 0
-        if (wave_active) compute(A0, B0);
+    if (wave_active && steps != 0) {
+        load_frags(A0, B0, 0, af[0], bf[0]);
+    }
+    // Per K step: sub-steps 0-2, wait for the next stage's DMA, barrier (every wavefront has the last fragments of
+    // this stage in registers, so the stage is free), DMA of the step after next into this stage, sub-step 3.
+    // The loop body never branches between two ways of updating the accumulators (that would make the compiler
+    // shuffle all 256 of them): the steady state always has a next step, the last one or two steps are peeled.
+    uint32_t s = 0;
+    for (; s + 2 < steps; s += 2) {
+        if (wave_active) head(A0, B0);
+        asm volatile("s_waitcnt vmcnt(0)");
+        __syncthreads();
+        issue((s + 2) * BK, A0, B0);
+        if (wave_active) tail(A1, B1);
+        if (wave_active) head(A1, B1);
+        asm volatile("s_waitcnt vmcnt(0)");
+        __syncthreads();
+        if (s + 3 < steps) {
+            issue((s + 3) * BK, A1, B1);
+        }
+        if (wave_active) tail(A0, B0);
+    }
+    if (s + 1 < steps) {  // two steps left: this one in stage 0, the last one on its way into stage 1
+        if (wave_active) head(A0, B0);
+        asm volatile("s_waitcnt vmcnt(0)");
+        __syncthreads();
+        if (wave_active) tail(A1, B1);
+        ++s;
+    }
+    if (s < steps) {  // the last step: stage 0 for an odd number of steps, stage 1 for an even one
+        const char* Al = (steps & 1u) ? A0 : A1;
+        const char* Bl = (steps & 1u) ? B0 : B1;
+        if (wave_active) {
+            head(Al, Bl);
+            mfma_block(1);
+        }
     }
 
     // ---- epilogue: register r of lane l in a 32x32 block is row 8*(r/4) + 4*(l/32) + r%4, column l%32
