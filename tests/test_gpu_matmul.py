@@ -52,7 +52,9 @@ SHAPES = [(1, 256, 512), (16, 1024, 4096), (32, 264, 1040), (33, 256, 256), (128
           # 128 x 128 tiles with and without a K split, row / column tails
           (33, 144, 128), (200, 528, 384), (512, 272, 256), (130, 2064, 1024),
           # 256-row tiles: a partial last round (narrow tiles), K steps odd and even
-          (513, 528, 256), (2048, 2832, 384)]
+          (513, 528, 256), (2048, 2832, 384),
+          # four and five K steps: the steady-state loop runs once, then two steps / one step are peeled
+          (600, 528, 512), (600, 528, 640), (300, 272, 512), (300, 272, 640)]
 
 
 @pytest.mark.parametrize("m,n,k", SHAPES)
