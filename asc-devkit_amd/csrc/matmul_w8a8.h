@@ -158,7 +158,8 @@ __device__ __forceinline__ uint32_t xcd_remap(uint32_t pid, uint32_t total)
 
 // Large-M kernel built on direct-to-LDS loads and transposing LDS reads (matmul_w8a8_dma.hip).
 bool gemm_dma_supported(const GemmParams& p);
-int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st);
+// b_nk: B is [n][k] (the transposed operand of the plain matmul); not with grouped or fractal B
+int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st, bool b_nk = false);
 uint32_t gemm_dma_skinny_splits(uint32_t m, uint32_t n, uint32_t k);
 bool gemm_stream_supported(const GemmParams& p);
 size_t gemm_stream_workspace(uint32_t m, uint32_t n, uint32_t k);

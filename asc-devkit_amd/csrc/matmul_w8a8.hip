@@ -663,6 +663,9 @@ extern "C" int ascq_matmul_w8a8(const ascq_matmul_desc* d, void* c, const void* 
     if (d->m > 128 && !d->trans_b && gemm_dma_supported(p)) {
         return launch_gemm_dma(p, false, st);
     }
+    if (d->m > 512 && d->trans_b && !d->trans_a && gemm_dma_supported(p)) {
+        return launch_gemm_dma(p, false, st, true);  // B as [n][k]: its tiles are staged and read like A's
+    }
     if (d->m <= 1024) {
         return d->trans_b ? launch_gemm<TileMT, true, false>(p, st) : launch_gemm<TileM, false, false>(p, st);
     }

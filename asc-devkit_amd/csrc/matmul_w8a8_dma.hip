@@ -65,7 +65,9 @@ __device__ __forceinline__ float epi_value(int32_t acc, float chan, float tok, f
 // once, by enough workgroups to fill the chip).
 // The body of a workgroup: tile number `bid` (before the XCD remapping) of the launch, K split `bidy`.  The LDS arrays
 // are declared by the kernels and handed in, so that one kernel can run tiles of two shapes.
-template <int BM, int BN, bool kSplitK, bool kGrouped>
+// kBT: B is given as [n][k] (transposed operand): its tile is staged and read exactly like A's, with plain 16-byte
+// LDS reads instead of the transposing ones.
+template <int BM, int BN, bool kSplitK, bool kGrouped, bool kBT = false>
 __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_begin, uint32_t bid, uint32_t bidy,
                                               char* A0, char* B0, char* A1, char* B1, float* TS)
 {
@@ -144,6 +146,13 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_
 #pragma unroll
     for (int u = 0; u < kBInstr; ++u) {
         const uint32_t s = (wave * kBInstr + u) * 64 + lane;
+        if constexpr (kBT) {
+            const uint32_t r = s >> 3, c = (s & 7u) ^ ((r >> 1) & 7u);
+            uint32_t col = n0 + r;
+            col = col < N ? col : N - 1u;  // columns past the end are never stored
+            boff[u] = (col - n0) * K + 16u * c;
+            continue;
+        }
         const uint32_t kb = s / kPieces;
         const uint32_t swz = BN == 256 ? 2u * (kb & 7u) : 2u * ((kb >> 1) & 3u);
         const uint32_t q = (s % kPieces) ^ swz;
@@ -152,7 +161,7 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_
         // fractal B: panels of 32 columns, each a contiguous row-major [K][32] block
         boff[u] = p.b_nz ? ((col >> 5) * K + kb) * 32u + (col & 31u) : kb * N + (col - n0);
     }
-    const uint32_t ldb = p.b_nz ? 32u : N;  // bytes from one k to the next
+    const uint32_t ldb = kBT ? 1u : p.b_nz ? 32u : N;  // bytes from one k to the next
     // K range of this workgroup, in steps of BK
     uint32_t s_begin = 0, steps = K / BK;
     if constexpr (kSplitK) {
@@ -160,7 +169,7 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_
         steps = steps * (bidy + 1u) / p.k_splits - s_begin;
     }
     const int8_t* Abase = p.a + static_cast<size_t>(row0) * K + static_cast<size_t>(s_begin) * BK;
-    const int8_t* Bbase = Bmat + (p.b_nz ? 0u : n0) + static_cast<size_t>(s_begin) * BK * ldb;
+    const int8_t* Bbase = Bmat + (kBT ? static_cast<size_t>(n0) * K : p.b_nz ? 0u : n0) + static_cast<size_t>(s_begin) * BK * ldb;
     auto issue = [&](uint32_t k0, char* As, char* Bs) {
         const int8_t* ab = Abase + k0;
         const int8_t* bb = Bbase + static_cast<size_t>(k0) * ldb;
@@ -190,10 +199,11 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_
     // ---- fragment addresses: one base per K sub-step (A) / per column block (B), everything else is an immediate
     const uint32_t lrow = lane & 31u, g = lane >> 5;
     const uint32_t grp16 = (lane >> 4) & 1u, bsub = (lane & 15u) >> 1, psub = lane & 1u;
-    uint32_t a_base[4], b_base[2];
+    uint32_t a_base[4], b_base[2], bt_base[4];
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
         a_base[ks] = (wm * (TI * 32) + lrow) * 128 + (((2 * ks + g) ^ ((lrow >> 1) & 7u)) << 4);
+        bt_base[ks] = (wn * (TJ * 32) + lrow) * 128 + (((2 * ks + g) ^ ((lrow >> 1) & 7u)) << 4);
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
@@ -204,6 +214,13 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_
 #pragma unroll
         for (int i = 0; i < TI; ++i) {
             af[i] = *reinterpret_cast<const i32x4*>(As + a_base[ks] + i * 4096);
+        }
+        if constexpr (kBT) {
+#pragma unroll
+            for (int j = 0; j < TJ; ++j) {
+                bf[j] = *reinterpret_cast<const i32x4*>(Bs + bt_base[ks] + j * 4096);
+            }
+            return;
         }
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
@@ -228,7 +245,7 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_
 #pragma unroll
         for (int n = 0; n < TI * TJ; ++n) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, (TI + 2 * TJ + TI * TJ - 1) / (TI * TJ), 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, (TI + (kBT ? TJ : 2 * TJ) + TI * TJ - 1) / (TI * TJ), 0);
         }
         __builtin_amdgcn_sched_barrier(0);
     };
@@ -241,6 +258,10 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_
         for (int q = 0; q < 4; ++q) asm volatile("" : "+v"(a_base[q]));
 #pragma unroll
         for (int q = 0; q < 2; ++q) asm volatile("" : "+v"(b_base[q]));
+        if constexpr (kBT) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) asm volatile("" : "+v"(bt_base[q]));
+        }
 #pragma unroll
         for (int ks = 0; ks < 3; ++ks) {
             load_frags(As, Bs, ks + 1, af[(ks + 1) & 1], bf[(ks + 1) & 1]);
@@ -419,7 +440,7 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_
     dispatch_out(e, run);
 }
 
-template <int BM, int BN, bool kSplitK, bool kGrouped = false>
+template <int BM, int BN, bool kSplitK, bool kGrouped = false, bool kBT = false>
 __global__ __launch_bounds__(kThreads, (BM * BK + BK * BN) * 2 <= 65536 ? 2 : 1) void gemm_dma_kernel(
     GemmParams p, uint32_t col_begin)
 {
@@ -428,12 +449,13 @@ __global__ __launch_bounds__(kThreads, (BM * BK + BK * BN) * 2 <= 65536 ? 2 : 1)
     __shared__ __attribute__((aligned(1024))) char A1[BM * BK];
     __shared__ __attribute__((aligned(1024))) char B1[BK * BN];
     __shared__ __attribute__((aligned(16))) float TS[BM];  // token scales of the tile's rows (1.0f when there are none)
-    gemm_dma_tile<BM, BN, kSplitK, kGrouped>(p, col_begin, blockIdx.x, blockIdx.y, A0, B0, A1, B1, TS);
+    gemm_dma_tile<BM, BN, kSplitK, kGrouped, kBT>(p, col_begin, blockIdx.x, blockIdx.y, A0, B0, A1, B1, TS);
 }
 
 // One launch for a matrix whose last round of 256 x 256 tiles would be mostly empty: workgroups [0, wide_wgs) run the
 // 256 x 256 tiles of the first `p.tiles_n` tile columns, the rest 256 x 128 tiles of the remaining columns.  A compute
 // unit that has finished its wide tile takes a narrow one at once, without the drain between two launches.
+template <bool kBT>
 __global__ __launch_bounds__(kThreads, 1) void gemm_dma_dual_kernel(GemmParams p, uint32_t wide_wgs,
                                                                     uint32_t narrow_tiles_n, uint32_t col_begin)
 {
@@ -443,11 +465,11 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_dma_dual_kernel(GemmParams p
     __shared__ __attribute__((aligned(1024))) char B1[BK * 256];
     __shared__ __attribute__((aligned(16))) float TS[256];
     if (blockIdx.x < wide_wgs) {
-        gemm_dma_tile<256, 256, false, false>(p, 0u, blockIdx.x, 0u, A0, B0, A1, B1, TS);
+        gemm_dma_tile<256, 256, false, false, kBT>(p, 0u, blockIdx.x, 0u, A0, B0, A1, B1, TS);
     } else {
         GemmParams q = p;
         q.tiles_n = narrow_tiles_n;
-        gemm_dma_tile<256, 128, false, false>(q, col_begin, blockIdx.x - wide_wgs, 0u, A0, B0, A1, B1, TS);
+        gemm_dma_tile<256, 128, false, false, kBT>(q, col_begin, blockIdx.x - wide_wgs, 0u, A0, B0, A1, B1, TS);
     }
 }
 
@@ -488,7 +510,7 @@ bool gemm_dma_supported(const GemmParams& p)
     return p.k % BK == 0 && p.n % 16 == 0 && p.n >= 16 && aligned16(p.a) && aligned16(p.b);
 }
 
-int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st)
+int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st, bool b_nk)
 {
     p.tiles_m = (p.m + 255u) / 256u + (grouped ? p.groups : 0u);  // every group adds at most one partial tile
     uint32_t tiles_n = (p.n + 255u) / 256u;
@@ -527,7 +549,11 @@ int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st)
         const uint32_t wide_wgs = (p.tiles_m * wide_cols + 7u) / 8u * 8u;
         const uint32_t narrow_wgs = (p.tiles_m * narrow_tiles_n + 7u) / 8u * 8u;
         p.tiles_n = wide_cols;
-        gemm_dma_dual_kernel<<<wide_wgs + narrow_wgs, kThreads, 0, st>>>(p, wide_wgs, narrow_tiles_n, col_begin);
+        if (b_nk) {
+            gemm_dma_dual_kernel<true><<<wide_wgs + narrow_wgs, kThreads, 0, st>>>(p, wide_wgs, narrow_tiles_n, col_begin);
+        } else {
+            gemm_dma_dual_kernel<false><<<wide_wgs + narrow_wgs, kThreads, 0, st>>>(p, wide_wgs, narrow_tiles_n, col_begin);
+        }
         return launch_status("ascq_matmul_w8a8");
     }
     if (wide_cols) {
@@ -540,6 +566,8 @@ int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st)
         }
         if (grouped) {
             gemm_dma_kernel<256, 256, false, true><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(q, 0u);
+        } else if (b_nk) {
+            gemm_dma_kernel<256, 256, false, false, true><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(q, 0u);
         } else {
             gemm_dma_kernel<256, 256, false><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(q, 0u);
         }
@@ -548,7 +576,11 @@ int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st)
         const uint32_t col_begin = wide_cols * 256u;
         p.tiles_n = (p.n - col_begin + 127u) / 128u;
         const uint32_t t = p.tiles_m * p.tiles_n;
-        gemm_dma_kernel<256, 128, false><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(p, col_begin);
+        if (b_nk) {
+            gemm_dma_kernel<256, 128, false, false, true><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(p, col_begin);
+        } else {
+            gemm_dma_kernel<256, 128, false><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(p, col_begin);
+        }
     }
     return launch_status(grouped ? "ascq_group_matmul_w8a8" : "ascq_matmul_w8a8");
 }
