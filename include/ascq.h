@@ -351,7 +351,8 @@ typedef enum ascq_mm_kernel {
                                         workspace is given (k_splits > 1: a second kernel adds the partial tiles) */
     ASCQ_MM_KERNEL_DMA_256 = 3,      /* 256 x 256 direct-to-LDS tiles; a last partial round of the chip may be run
                                         by further workgroups of the same launch with 256 x narrow_tile_n tiles */
-    ASCQ_MM_KERNEL_STAGED = 4        /* register-staged tiles: transposed B, or K not a multiple of 128 */
+    ASCQ_MM_KERNEL_STAGED = 4        /* register-staged tiles: transposed B with at most 512 rows of A, or K not a
+                                        multiple of 128 (a transposed B with more rows runs on KERNEL_DMA_256) */
 } ascq_mm_kernel;
 
 typedef struct ascq_matmul_plan {

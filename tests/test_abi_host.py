@@ -232,9 +232,12 @@ def test_matmul_plan_of_the_benchmark_shapes():
     p, need = _plan(128, 11008, 4096)
     assert (p.kernel, p.tile_m, p.tile_n) == (abi.MM_KERNEL_DMA_128, 128, 128)
     assert (p.k_splits, p.workgroups, p.launches) == (4, 88 * 4, 2) and p.workspace_bytes == 4 * 128 * 11008 * 4
-    # transposed B and odd addresses fall to the register-staged and the generic kernels
+    # B as [n, k]: the same direct-to-LDS tiles when A has more than 512 rows, the register-staged kernel below that
     p, _ = _plan(2048, 11008, 4096, trans_b=1)
-    assert (p.kernel, p.tile_m, p.tile_n, p.launches) == (abi.MM_KERNEL_STAGED, 256, 256, 1)
+    assert (p.kernel, p.tile_m, p.tile_n, p.narrow_tile_n, p.launches) == (abi.MM_KERNEL_DMA_256, 256, 256, 128, 1)
+    p, _ = _plan(300, 11008, 4096, trans_b=1)
+    assert (p.kernel, p.launches) == (abi.MM_KERNEL_STAGED, 1)
+    # odd addresses fall to the generic kernel
     p, _ = _plan(2048, 11008, 4096, a=0x10001)
     assert (p.kernel, p.launches) == (abi.MM_KERNEL_GENERIC, 1)
     # a rejected descriptor is rejected by the plan query as by the call
