@@ -20,8 +20,17 @@
 //   A stage: row r = 128 bytes = 8 pieces of 16; piece c is stored at position c ^ ((r >> 1) & 7).
 //   B stage: row k = 256 bytes = 16 pieces of 16; piece q is stored at position q ^ (2 * (k & 7)).
 #include <type_traits>
+#include <utility>
 
 #include "matmul_w8a8.h"
+
+#ifdef ASCQ_EXP_CLOCK
+__device__ unsigned long long ascq_dbg_clk[4];
+extern "C" int ascq_debug_clock(unsigned long long* out)
+{
+    return hipMemcpyFromSymbol(out, HIP_SYMBOL(ascq_dbg_clk), sizeof(ascq_dbg_clk)) == hipSuccess ? 0 : 1;
+}
+#endif
 
 namespace ascq {
 namespace {
@@ -32,6 +41,18 @@ constexpr int BK = 128;
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef __attribute__((address_space(1))) const void* gptr_t;
 typedef i32x2_t __attribute__((address_space(3)))* lds_v2_t;
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant expression.
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>)
+{
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f)
+{
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
 
 // 16-bit output of two adjacent columns packed into one dword store.
 template <int kOut>
@@ -86,6 +107,9 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_
     if (t >= total) {
         return;
     }
+#ifdef ASCQ_EXP_CLOCK
+    const unsigned long long dbg_c0 = __builtin_readcyclecounter(), dbg_r0 = wall_clock64();
+#endif
     const uint32_t ms = t % p.tiles_m, tn = t / p.tiles_m;
     const uint32_t K = p.k, N = p.n;
     uint32_t row0 = ms * BM, row_end = p.m;
@@ -210,23 +234,24 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_
         const uint32_t swz = BN == 256 ? 2u * bsub : 2u * ((bsub >> 1) & 3u);
         b_base[j] = (16 * g + bsub) * BN + (((4 * wn + 2 * j + grp16) ^ swz) << 4) + 8 * psub;
     }
+    // In the order the MFMAs of a sub-step want them (they run row block by row block): B0, A0, B1, A1, A2, ...
     auto load_frags = [&](const char* As, const char* Bs, int ks, i32x4 (&af)[TI], i32x4 (&bf)[TJ]) {
-#pragma unroll
-        for (int i = 0; i < TI; ++i) {
-            af[i] = *reinterpret_cast<const i32x4*>(As + a_base[ks] + i * 4096);
-        }
-        if constexpr (kBT) {
-#pragma unroll
-            for (int j = 0; j < TJ; ++j) {
+        auto load_b = [&](int j) {
+            if constexpr (kBT) {
                 bf[j] = *reinterpret_cast<const i32x4*>(Bs + bt_base[ks] + j * 4096);
+            } else {
+                const i32x2_t lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2_t)(Bs + b_base[j] + ks * kKsB));
+                const i32x2_t hi =
+                    __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2_t)(Bs + b_base[j] + ks * kKsB + 8 * BN));
+                bf[j] = i32x4{lo[0], lo[1], hi[0], hi[1]};
             }
-            return;
-        }
+        };
+        load_b(0);
+        af[0] = *reinterpret_cast<const i32x4*>(As + a_base[ks]);
+        load_b(1);
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const i32x2_t lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2_t)(Bs + b_base[j] + ks * kKsB));
-            const i32x2_t hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2_t)(Bs + b_base[j] + ks * kKsB + 8 * BN));
-            bf[j] = i32x4{lo[0], lo[1], hi[0], hi[1]};
+        for (int i = 1; i < TI; ++i) {
+            af[i] = *reinterpret_cast<const i32x4*>(As + a_base[ks] + i * 4096);
         }
     };
     // Fragment registers live across K steps: buffer 0 holds sub-steps 0 and 2, buffer 1 sub-steps 1 and 3.
@@ -240,13 +265,25 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_
             }
         }
     };
-    // one LDS read behind each MFMA
+    // The LDS reads of a sub-step go out behind its first MFMAs (kReadsPerMfma behind each), so that the matrix
+    // instructions of its second half run while the last reads are still on their way: the next sub-step starts by
+    // waiting for all of them.
     auto interleave = [&]() __attribute__((always_inline)) {
-#pragma unroll
-        for (int n = 0; n < TI * TJ; ++n) {
+        constexpr int kReads = TI + (kBT ? TJ : 2 * TJ);
+        constexpr int kMfmas = TI * TJ;
+#ifdef ASCQ_EXP_FRONT_DIV
+        constexpr int kFront = (kMfmas + ASCQ_EXP_FRONT_DIV - 1) / ASCQ_EXP_FRONT_DIV;
+#else
+        constexpr int kFront = (kMfmas + 1) / 2;
+#endif
+        constexpr int kPer = (kReads + kFront - 1) / kFront;
+        static_for<kMfmas>([&](auto n) {
+            constexpr int kLeft = kReads - decltype(n)::value * kPer;
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, (TI + (kBT ? TJ : 2 * TJ) + TI * TJ - 1) / (TI * TJ), 0);
-        }
+            if constexpr (kLeft > 0) {
+                __builtin_amdgcn_sched_group_barrier(0x100, kLeft < kPer ? kLeft : kPer, 0);
+            }
+        });
         __builtin_amdgcn_sched_barrier(0);
     };
     // Sub-steps 0-2 of a K step whose sub-step-0 fragments are already in buffer 0; on return the fragments of
@@ -296,15 +333,32 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_
     // The loop body never branches between two ways of updating the accumulators (that would make the compiler
     // shuffle all 256 of them): the steady state always has a next step, the last one or two steps are peeled.
     uint32_t s = 0;
+#ifdef ASCQ_EXP_CLOCK
+    unsigned long long dbg_vm = 0, dbg_bar = 0;
+#define ASCQ_WAIT_AND_BARRIER()                                          \
+    do {                                                                 \
+        const unsigned long long t0_ = __builtin_readcyclecounter();     \
+        asm volatile("s_waitcnt vmcnt(0)");                              \
+        const unsigned long long t1_ = __builtin_readcyclecounter();     \
+        __syncthreads();                                                 \
+        const unsigned long long t2_ = __builtin_readcyclecounter();     \
+        dbg_vm += t1_ - t0_;                                             \
+        dbg_bar += t2_ - t1_;                                            \
+    } while (0)
+#else
+#define ASCQ_WAIT_AND_BARRIER()             \
+    do {                                    \
+        asm volatile("s_waitcnt vmcnt(0)"); \
+        __syncthreads();                    \
+    } while (0)
+#endif
     for (; s + 2 < steps; s += 2) {
         if (wave_active) head(A0, B0);
-        asm volatile("s_waitcnt vmcnt(0)");
-        __syncthreads();
+        ASCQ_WAIT_AND_BARRIER();
         issue((s + 2) * BK, A0, B0);
         if (wave_active) tail(A1, B1);
         if (wave_active) head(A1, B1);
-        asm volatile("s_waitcnt vmcnt(0)");
-        __syncthreads();
+        ASCQ_WAIT_AND_BARRIER();
         if (s + 3 < steps) {
             issue((s + 3) * BK, A1, B1);
         }
@@ -326,6 +380,14 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_
         }
     }
 
+#ifdef ASCQ_EXP_CLOCK
+    if (bid == 8 && threadIdx.x == 0 && BN == 256) {
+        ascq_dbg_clk[0] = __builtin_readcyclecounter() - dbg_c0;
+        ascq_dbg_clk[1] = wall_clock64() - dbg_r0;
+        ascq_dbg_clk[2] = dbg_vm;
+        ascq_dbg_clk[3] = dbg_bar;
+    }
+#endif
     // ---- epilogue: register r of lane l in a 32x32 block is row 8*(r/4) + 4*(l/32) + r%4, column l%32
     if constexpr (kSplitK) {
         int32_t* part = p.partial + static_cast<size_t>(bidy) * p.m * N;
