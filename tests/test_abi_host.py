@@ -256,3 +256,34 @@ def test_missing_library_is_a_loud_error_with_no_fallback(monkeypatch, tmp_path)
     from ascq import ops
     with pytest.raises(RuntimeError, match="is missing"):
         ops.dequant_dst_stride("float16", 40)
+
+
+def test_inline_assembly_kernels_have_no_scratch_frame():
+    """The build records every kernel's register / scratch figures (asc-devkit_amd/csrc/check_resources.py).  Kernels
+    that load through inline assembly and wait by hand must have no scratch frame and no spills: the compiler does not
+    know that their destination registers are still being written."""
+    import json
+    path = os.path.join(ROOT, "asc-devkit_amd", "lib", "kernel_resources.json")
+    assert os.path.exists(path), "build the library first (make -C asc-devkit_amd/csrc writes this file)"
+    rec = json.load(open(path))
+    guarded = [k for k in rec["kernels"] if k["guarded"]]
+    seen = {k["name"].replace("void ", "").split("<")[0].split("(")[0] for k in guarded}
+    for name in ("w4a16_gemv_kernel", "w4a16_tile_kernel", "w8a16_tile_kernel", "gemm_stream_kernel", "gemm_dma_kernel",
+                 "gemm_dma_dual_kernel"):
+        assert name in seen, f"{name} is missing from the build record"
+    for k in guarded:
+        assert k["scratch_bytes_per_lane"] == 0 and k["vgpr_spills"] == 0 and k["sgpr_spills"] == 0, k
+        assert k["vgprs"] + k["agprs"] <= 512 and k["lds_bytes"] <= 160 * 1024, k
+
+
+def test_resource_checker_rejects_a_guarded_kernel_with_scratch(tmp_path):
+    import subprocess
+    import sys
+    remarks = tmp_path / "fake.remarks"
+    lines = ["Function Name: _ZN4ascq12_GLOBAL__N_118gemm_stream_kernelENS0_12StreamParamsE", "    TotalSGPRs: 10",
+             "    VGPRs: 256", "    AGPRs: 0", "    ScratchSize [bytes/lane]: 100", "    Occupancy [waves/SIMD]: 1",
+             "    SGPRs Spill: 0", "    VGPRs Spill: 25", "    LDS Size [bytes/block]: 0"]
+    remarks.write_text("".join(f"x.hip:1:1: remark: {l} [-Rpass-analysis=kernel-resource-usage]\n" for l in lines))
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "asc-devkit_amd", "csrc", "check_resources.py"), str(remarks)],
+                       capture_output=True, text=True)
+    assert r.returncode == 1 and "100 bytes of scratch" in r.stderr
