@@ -111,6 +111,9 @@ SIGNATURES = {
     "ascq_group_matmul_w8a8": (C.c_int, [C.POINTER(GroupMatmulDesc), _P, _P, _P, _P, _P, _P, _P, _P]),
     "ascq_matmul_w4a16": (C.c_int, [C.POINTER(W4A16Desc), _P, _P, _P, _P, _P, _P, C.c_size_t, _P]),
     "ascq_matmul_w4a16_workspace_size": (C.c_int, [C.POINTER(W4A16Desc), C.POINTER(C.c_size_t)]),
+    "ascq_pack_weight_w4_size": (C.c_int, [C.c_uint32, C.c_uint32, C.POINTER(C.c_size_t)]),
+    "ascq_pack_weight_w4": (C.c_int, [_P, _P, C.c_uint32, C.c_uint32, _P]),
+    "ascq_matmul_w4a16_packed": (C.c_int, [C.POINTER(W4A16Desc), _P, _P, _P, _P, _P, _P]),
     "ascq_matmul_w8a16": (C.c_int, [C.POINTER(W8A16Desc), _P, _P, _P, _P, _P, _P, C.c_size_t, _P]),
     "ascq_matmul_w8a16_workspace_size": (C.c_int, [C.POINTER(W8A16Desc), C.POINTER(C.c_size_t)]),
     "ascq_get_ascend_quant_max_min_tmp_size": (C.c_int, [C.POINTER(C.c_uint32), C.c_uint32, C.c_uint32,

@@ -430,6 +430,26 @@ def matmul_w4a16(y, x, w_packed, scale, offset=None, group_size=128, workspace=N
     return y
 
 
+def pack_weight_w4(w_nd, k, n):
+    """int4 weights [k, n / 2] bytes (two per byte along n) -> the GPU-native packed layout of matmul_w4a16_packed."""
+    lib = load_library()
+    need = C.c_size_t(0)
+    check(lib.ascq_pack_weight_w4_size(k, n, C.byref(need)))
+    out = torch.empty(need.value, dtype=torch.uint8, device=w_nd.device)
+    check(lib.ascq_pack_weight_w4(_ptr(w_nd), _ptr(out), k, n, _stream()))
+    return out
+
+
+def matmul_w4a16_packed(y, x, w_gpu, scale, offset=None, group_size=128):
+    """matmul_w4a16 on weights packed by pack_weight_w4: one launch, no workspace, same arithmetic."""
+    m, k = x.shape
+    n = y.shape[1]
+    d = abi.W4A16Desc(m=m, n=n, k=k, group_size=group_size, has_offset=int(offset is not None))
+    check(load_library().ascq_matmul_w4a16_packed(C.byref(d), _ptr(y), _ptr(x), _ptr(w_gpu), _ptr(scale),
+                                                  _ptr(offset), _stream()))
+    return y
+
+
 # ------------------------------------------------------------------------------------------------------ W8A16
 def matmul_w8a16(y, x, w, offset=None, scale=None, workspace=None):
     """y f16 / f32 [m, n] = x f16 [m, k] @ AscendAntiQuant<int8_t, half>(w int8 [k, n]).

@@ -1,0 +1,517 @@
+// W4A16 decode GEMV / skinny GEMM on pre-packed int4 weights: one launch, one flat sweep over the weights.
+//
+// Packed layout (ascq_pack_weight_w4): the [k, n] matrix is cut into slabs of 16 columns and tiles of 128 k; a tile of
+// a slab is 1 KiB and the tiles of a slab, then the slabs, follow each other in memory, so the 16 columns of a slab
+// are one contiguous run of k / 128 KiB.  Inside a tile, lane l of a wavefront owns 16 bytes: column l % 16 of the
+// slab, k = 32 (l / 16) .. + 31; dword d of the 16 bytes holds k = 32 (l / 16) + 8 d .. + 7.  A nibble is stored
+// as u = w + 8 (offset binary), and the 8 nibbles of a dword sit in the order in which the 0x6400 exponent trick
+// yields pairs: k offsets 0 1 2 3 4 5 6 7 live in nibbles 0 4 1 5 2 6 3 7.  Columns past n and k past the end hold
+// w = 0.
+//
+// With that layout one 16-byte load per lane is a fully coalesced 1 KiB read and the only memory instruction a tile
+// costs; a lane needs one scale and one offset per tile (a quantisation group is a multiple of 32 k), and the 8
+// de-quantised halves of a dword are, as they lie in the registers, the B operand of v_mfma_f32_16x16x32_f16 for
+// column l % 16 and k group l / 16: the matrix core does the multiply-accumulate and the reduction over the four k
+// groups, for up to 16 activation rows at the cost of one.  Activations and the workgroup's scale / offset columns are
+// staged in LDS once per pass over k (coalesced 16-byte loads); operand row i of a lane reads activation row i % m, so
+// there are no zero rows to materialise (result rows >= m repeat earlier ones and are not stored).
+//
+// A workgroup owns whole slabs: its wavefronts split k, every wavefront streams a contiguous piece of each slab with
+// two batches of tiles in flight behind the one being computed, and the per-wavefront sums meet in LDS, where they
+// are added in wavefront order and rounded once to half: no second kernel, no workspace, deterministic.
+// De-quantisation follows AscendAntiQuant<int4b_t, half> exactly (one rounded half add of the offset, one rounded half
+// multiply by the scale per weight); the products and sums are fp32.
+#include <type_traits>
+
+#include "ascq_common.h"
+#include "ascq_device.h"
+
+namespace ascq {
+namespace {
+
+constexpr uint32_t kSlabCols = 16, kTileK = 128, kTileBytes = 1024;
+constexpr int kBuf = 3;                  // register buffers: two batches in flight behind the one being computed
+constexpr uint32_t kPadTiles = 16;       // tiles of padding behind the last slab of a packed matrix (a batch may read on)
+constexpr uint32_t kMaxSlabs = 8;        // slabs per workgroup
+constexpr uint32_t kMaxRows = 16;        // activation rows per launch
+constexpr uint32_t kPool = 152 * 1024;   // LDS of a workgroup: staged activations, parameters, per-wavefront sums
+constexpr uint32_t kXBytes = 72 * 1024;  // at most this much of it for the activations of one pass over k
+constexpr uint32_t kParBytes = 32 * 1024;// and this much for the (scale, offset) pairs of one pass
+constexpr uint32_t kPastEnd = 0x7FFFFFF0u;  // a per-lane buffer offset beyond any buffer this kernel accepts (< 2 GiB)
+constexpr int kNt = 2;                   // cache policy of the weight loads: non-temporal (read once per call)
+constexpr uint32_t kRowPad = 16;         // bytes added to a staged activation row: rows start 4 banks apart
+
+struct NibbleMasks {
+    uint32_t even, odd, exp;  // 0x000F000F, 0x00F000F0, 0x64006400
+};
+
+struct W4pParams {
+    const uint16_t* x;       // [m, k] halves, first row of this launch
+    const u32x4* wp;         // packed weights
+    const uint16_t* scale;   // [k / group_size, n]
+    const uint16_t* offset;  // same, or nullptr
+    uint16_t* y;             // [m, n] halves, first row of this launch
+    uint32_t m;              // rows of this launch, 1 .. 16
+    uint32_t n, k;
+    uint32_t gs_shift;       // log2(group_size / 32)
+    uint32_t slabs, ktiles;  // ceil(n / 16), k / 128
+    uint32_t slabs_per_wg;   // 1 .. kMaxSlabs
+    uint32_t pass_tiles;     // tiles of k staged per pass (multiple of the wavefront count)
+    uint32_t ppr_magic;      // ceil(2^32 / (tiles per wavefront * 16)): i / that = mulhi(i, ppr_magic) for i < 65536
+    uint32_t par_magic;      // ceil(2^32 / (slabs_per_wg * 2)), likewise
+    uint32_t xs_wave, par_wave;  // bytes of staged activations / parameters per wavefront
+    uint32_t par_pitch;          // entries per column of a wavefront's parameter table (odd)
+    uint32_t par_off, red_off;   // byte offsets of the parameter tables and of the sums inside the LDS pool
+    NibbleMasks mk;
+    uint32_t red_lanes;      // lanes of a result register that hold rows < m: 16 for m <= 4, else 64
+};
+
+__device__ __forceinline__ f16x2 bits_h2(uint32_t b)
+{
+    f16x2 r;
+    __builtin_memcpy(&r, &b, 4);
+    return r;
+}
+__device__ __forceinline__ uint32_t h2_bits(f16x2 h)
+{
+    uint32_t r;
+    __builtin_memcpy(&r, &h, 4);
+    return r;
+}
+
+// One dword of packed weights (8 consecutive k of one column, offset binary) -> the 8 de-quantised halves in k order.
+// kFold: ofe holds offset - 1032 and ofo offset - 72 (both halves), exact for integer offsets of magnitude <= 512, so
+// that conversion and offset are one exact operation; otherwise ofe is the offset itself.
+template <bool kHasOffset, bool kFold>
+__device__ __forceinline__ f16x8 dequant8(uint32_t qd, f16x2 sc, f16x2 ofe, f16x2 ofo, const NibbleMasks& mk)
+{
+    const f16x2 k1032 = {static_cast<half_t>(1032.0f), static_cast<half_t>(1032.0f)};
+    const f16x2 k72 = {static_cast<half_t>(72.0f), static_cast<half_t>(72.0f)};
+    const f16x2 k16th = {static_cast<half_t>(0.0625f), static_cast<half_t>(0.0625f)};
+    const uint32_t qh = qd >> 8;
+    f16x2 h[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const uint32_t src = c < 2 ? qd : qh;
+        // 1024 + u read in place (even c), 1024 + 16 u read four bits up (odd c).  The masks arrive as kernel arguments:
+        // with values it cannot fold the compiler emits one v_and_or_b32 (VOP3 takes no literals) instead of two
+        // instructions with literal operands.
+        const uint32_t bits = (src & ((c & 1) ? mk.odd : mk.even)) | mk.exp;
+        if constexpr (kHasOffset && kFold) {
+            h[c] = (c & 1) ? __builtin_elementwise_fma(bits_h2(bits), k16th, ofo) : bits_h2(bits) + ofe;
+        } else {
+            h[c] = (c & 1) ? __builtin_elementwise_fma(bits_h2(bits), k16th, -k72) : bits_h2(bits) - k1032;  // w, exact
+            if constexpr (kHasOffset) {
+                h[c] = h[c] + ofe;  // one rounding
+            }
+        }
+        h[c] = sc * h[c];  // one rounding
+    }
+    f16x8 b;
+    __builtin_memcpy(&b, h, 16);
+    return b;
+}
+
+template <bool kHasOffset, uint32_t kWaves, uint32_t kBatch>
+__global__ __launch_bounds__(kWaves * 64) void w4a16_packed_kernel(W4pParams p)
+{
+    constexpr uint32_t kThreadsWg = kWaves * 64u;
+    constexpr uint32_t kXPieces = (kXBytes / 16u + kThreadsWg - 1u) / kThreadsWg;    // 16-byte pieces per lane
+    constexpr uint32_t kParPieces = 2;  // 8-column parameter pieces per lane (the host keeps a wavefront's table within 128)
+    __shared__ __attribute__((aligned(16))) char POOL[kPool];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t j = lane & 15u, g = lane >> 4;
+    // every wavefront stages what its own share of k needs and reads nothing another wavefront wrote: no barriers
+    // until the final sum
+    char* const XS = POOL + wave * p.xs_wave;               // [m][tiles per wavefront * 128 halves + pad]
+    char* const PAR = POOL + p.par_off + wave * p.par_wave;  // [column of the workgroup][group of the wavefront's k] (scale | offset << 16)
+    float* const RED = reinterpret_cast<float*>(POOL + p.red_off);    // [wave][slab][register][lane < red_lanes]
+
+    const uint32_t spw = p.slabs_per_wg;
+    const uint32_t slab0 = blockIdx.x * spw;
+    const uint32_t nslabs = min(spw, p.slabs - slab0);
+    const uint32_t tpw = p.pass_tiles / kWaves;             // tiles of a pass per wavefront
+    const uint32_t pitch = tpw * kTileK * 2u + kRowPad;     // bytes of a staged activation row
+    const uint32_t ppr = tpw * (kTileK / 8u);               // 16-byte pieces of a staged row
+    const uint32_t x_lane = ((lane & 15u) % p.m) * pitch + g * 64u;  // operand row i reads row i % m; + tile * 256 + d * 16
+    const uint32_t row_bytes = p.n * 2u;                          // one row of scale / offset in memory
+    const uint32_t par_col = p.par_pitch * 4u;                    // bytes of one column of the table in LDS (odd number of entries)
+    // The quantisation group of a lane's 32 k, (4 tile + g) / (group_size / 32) with group_size / 32 = 2^s, splits into
+    // a part that is the same for every lane, (4 tile) >> s, and a per-lane constant, g >> s (s <= 2); for s > 2 the
+    // lanes of a tile share one group, tile >> (s - 2).
+    const uint32_t gsh = p.gs_shift;
+    const uint32_t par_lane0 = (gsh <= 2u ? (g >> gsh) * 4u : 0u) + j * par_col;  // + slab * 16 columns
+
+    // Buffer descriptors: a load takes a per-lane 32-bit offset (range-checked: an offset past the end makes the load
+    // return zero without moving data) and a scalar offset that moves with the tile (not range-checked), so no vector
+    // instruction is spent on weight addresses inside the loop.
+    // the exponent constant lives in a vector register so that mask (scalar) and constant fit one v_and_or_b32
+    NibbleMasks mk = p.mk;
+    asm volatile("" : "+v"(mk.exp));
+    const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<u32x4*>(p.wp), 0, static_cast<int>((p.slabs * p.ktiles + kPadTiles) * kTileBytes), 0x00020000);
+    const int par_bytes = static_cast<int>(((p.k / 32u) >> gsh) * row_bytes);
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.scale), 0, par_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t*>(kHasOffset ? p.offset : p.scale), 0, par_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t*>(p.x), 0, static_cast<int>(p.m * p.k * 2u), 0x00020000);
+
+    // sums of this wavefront per slab, kept in LDS between passes
+    const uint32_t rl = p.red_lanes, red_wave = spw * 4u * rl;  // floats per wavefront
+    float* red = RED + wave * red_wave;
+    if (lane < rl) {
+        for (uint32_t s = 0; s < nslabs * 4u; ++s) red[s * rl + lane] = 0.0f;
+    }
+
+    for (uint32_t pt0 = 0; pt0 < p.ktiles; pt0 += p.pass_tiles) {
+        const uint32_t ptiles = min(p.pass_tiles, p.ktiles - pt0);
+        // ---- this wavefront's work of the pass: tiles [ta, tb) (relative to pt0) of each of its slabs, in batches of
+        // kBatch tiles that never straddle a slab: batch q = (slab q / nb, tiles ta + (q % nb) kBatch ...)
+        const uint32_t ta = min(wave * tpw, ptiles), tb = min(ta + tpw, ptiles);
+        const uint32_t cnt = tb - ta;
+        const uint32_t nb = (cnt + kBatch - 1u) / kBatch;
+        const uint32_t batches = nb * nslabs;
+        const uint32_t g_base = ((pt0 + ta) * 4u) >> gsh;                                          // first group of its k
+        const uint32_t g_rows = cnt != 0u ? ((((pt0 + tb) * 4u - 1u) >> gsh) - g_base + 1u) : 0u;  // groups it touches
+
+        // Every weight load is unconditional, so the loop body is straight-line as far as memory loads go and the waits
+        // the compiler inserts count exactly: two batches stay in flight while one is computed.  A tile past the end of
+        // its slab's range re-reads the last one (and is not computed); once every batch has been requested the
+        // per-lane offset points past the end of the buffer and the loads of the loop's last rounds are dropped.
+        u32x4 wq[kBuf][kBatch];
+        uint32_t l_slab = slab0, l_b = 0, l_q = 0;  // load cursor: slab, batch within the slab, batch number
+        bool l_done = batches == 0u;               // every batch has been requested
+        auto load = [&](int buf) __attribute__((always_inline)) {
+            const uint32_t l_w = l_done ? kPastEnd : lane * 16u;
+            // tiles past the wavefront's range (a short last batch) read on into the next tiles or the padding behind the
+            // last slab: valid memory, not computed
+            const uint32_t base = (l_slab * p.ktiles + pt0 + ta + l_b * kBatch) * kTileBytes;  // scalar
+#pragma unroll
+            for (uint32_t t = 0; t < kBatch; ++t) {
+                wq[buf][t] = __builtin_amdgcn_raw_buffer_load_b128(rw, l_w, base + t * kTileBytes, kNt);
+            }
+            if (l_q + 1u < batches) {  // uniform
+                ++l_q;
+                if (++l_b == nb) {
+                    l_b = 0;
+                    ++l_slab;
+                }
+            } else {
+                l_done = true;
+            }
+        };
+
+        // ---- The wavefront's activations (m rows x its tiles' k) and parameters (its groups x the workgroup's columns)
+        // travel through registers into its part of the LDS.  Their loads are issued first and the first weight batch
+        // behind them: loads return in order, so the wait for the staged data leaves the weights in flight.
+        // Activation piece i (16 bytes) is piece i % ppr of row i / ppr; pieces past the last row lie past the end of
+        // the buffer (dropped loads), pieces past the wavefront's tiles are never read back.  Parameter piece i is 8
+        // columns: piece i % (2 spw) of group row i / (2 spw).
+        u32x4 xr[kXPieces], sr[kParPieces], orr[kParPieces];
+#pragma unroll
+        for (uint32_t u = 0; u < kXPieces; ++u) {
+            const uint32_t i = lane + u * 64u;
+            const uint32_t r = __umulhi(i, p.ppr_magic), c = i - r * ppr;
+            xr[u] = __builtin_amdgcn_raw_buffer_load_b128(
+                rx, (r < p.m && cnt != 0u) ? (r * p.k + (pt0 + ta) * kTileK + c * 8u) * 2u : kPastEnd, 0, 0);
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < kParPieces; ++u) {
+            const uint32_t i = lane + u * 64u;
+            const uint32_t r = __umulhi(i, p.par_magic), c = i - r * (2u * spw);
+            const uint32_t col = slab0 * kSlabCols + c * 8u;
+            const uint32_t off = (r < g_rows && col < p.n) ? ((g_base + r) * p.n + col) * 2u : kPastEnd;
+            sr[u] = __builtin_amdgcn_raw_buffer_load_b128(rs, off, 0, 0);
+            if constexpr (kHasOffset) {
+                orr[u] = __builtin_amdgcn_raw_buffer_load_b128(ro, off, 0, 0);
+            }
+        }
+        load(0);
+#pragma unroll
+        for (uint32_t u = 0; u < kXPieces; ++u) {
+            const uint32_t i = lane + u * 64u;
+            const uint32_t r = __umulhi(i, p.ppr_magic), c = i - r * ppr;
+            if (r < p.m) {
+                *reinterpret_cast<u32x4*>(XS + r * pitch + c * 16u) = xr[u];
+            }
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < kParPieces; ++u) {
+            const uint32_t i = lane + u * 64u;
+            const uint32_t r = __umulhi(i, p.par_magic), c = i - r * (2u * spw);
+            if (r < g_rows) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const uint32_t o2 = kHasOffset ? orr[u][e] : 0u;
+                    char* dst = PAR + (c * 8u + 2u * e) * par_col + r * 4u;
+                    *reinterpret_cast<uint32_t*>(dst) = __builtin_amdgcn_perm(o2, sr[u][e], 0x05040100u);            // (s, o) of column 2e
+                    *reinterpret_cast<uint32_t*>(dst + par_col) = __builtin_amdgcn_perm(o2, sr[u][e], 0x07060302u);  // column 2e + 1
+                }
+            }
+        }
+        load(1);
+        if (batches == 0u) {
+            continue;  // uniform over the wavefront
+        }
+
+        f32x4 acc[2] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
+        uint32_t c_slab = 0, c_b = 0, c_q = 0;  // compute cursor (slab relative to slab0)
+        auto compute = [&](int buf) __attribute__((always_inline)) {
+            if (c_q >= batches) {
+                return;  // uniform; nothing but arithmetic is skipped
+            }
+            const uint32_t t0 = ta + c_b * kBatch;       // first tile of the batch, relative to pt0
+            const uint32_t live = min(kBatch, tb - t0);  // tiles of the batch inside the range
+            const char* xa0 = XS + x_lane + (t0 - ta) * 256u;
+            // (scale, offset) of every tile of the batch; whether every offset is an integer of magnitude <= 512 (it
+            // survives (o + 1536) - 1536): then conversion and offset are one exact operation.  With group_size 128 the
+            // tiles' entries are consecutive, one address serves the batch; a tile past the range reads on into the next
+            // column's entries (or, behind the last table, into the sums: still inside the pool) and is not computed.
+            const uint32_t tt0 = pt0 + t0;
+            const char* pa0 = PAR + par_lane0 + c_slab * (kSlabCols * par_col) +
+                              ((gsh <= 2u ? (tt0 * 4u) >> gsh : tt0 >> (gsh - 2u)) - g_base) * 4u;
+            uint32_t pp[kBatch];
+            uint32_t frac = 0;
+            if (gsh == 2u) {
+#pragma unroll
+                for (uint32_t t = 0; t < kBatch; ++t) pp[t] = *reinterpret_cast<const uint32_t*>(pa0 + t * 4u);
+            } else {
+#pragma unroll
+                for (uint32_t t = 0; t < kBatch; ++t) {
+                    const uint32_t tt = tt0 + t;
+                    const uint32_t grow = (gsh <= 2u ? (tt * 4u) >> gsh : tt >> (gsh - 2u)) - (gsh <= 2u ? (tt0 * 4u) >> gsh : tt0 >> (gsh - 2u));
+                    pp[t] = *reinterpret_cast<const uint32_t*>(pa0 + grow * 4u);
+                }
+            }
+            if constexpr (kHasOffset) {
+#pragma unroll
+                for (uint32_t t = 0; t < kBatch; ++t) {
+                    const f16x2 k1536 = {static_cast<half_t>(1536.0f), static_cast<half_t>(1536.0f)};
+                    const f16x2 rt = (bits_h2(pp[t]) + k1536) - k1536;
+                    frac |= (h2_bits(rt) ^ pp[t]) & 0x7FFF0000u;  // the offset is the high half
+                }
+            }
+            const bool fold = kHasOffset && __builtin_amdgcn_ballot_w64(frac != 0u) == 0;  // uniform
+            auto tiles = [&](auto folded) __attribute__((always_inline)) {
+                constexpr bool kFold = decltype(folded)::value;
+#pragma unroll
+                for (uint32_t t = 0; t < kBatch; ++t) {
+                    if (t < live) {  // uniform; no memory loads inside, so the wait counts stay exact
+                        const f16x2 sp = bits_h2(pp[t]);
+                        const f16x2 sc = {sp[0], sp[0]};
+                        f16x2 ofe = {sp[1], sp[1]}, ofo = ofe;
+                        if constexpr (kFold) {
+                            ofo = ofe - f16x2{static_cast<half_t>(72.0f), static_cast<half_t>(72.0f)};    // exact
+                            ofe = ofe - f16x2{static_cast<half_t>(1032.0f), static_cast<half_t>(1032.0f)};  // exact
+                        }
+#pragma unroll
+                        for (int d = 0; d < 4; ++d) {
+                            const f16x8 a = *reinterpret_cast<const f16x8*>(xa0 + t * 256u + d * 16);
+                            const f16x8 b = dequant8<kHasOffset, kFold>(wq[buf][t][d], sc, ofe, ofo, mk);
+                            acc[d & 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[d & 1], 0, 0, 0);
+                        }
+                    }
+                }
+            };
+            if (fold) {
+                tiles(std::true_type{});
+            } else {
+                tiles(std::false_type{});
+            }
+            ++c_q;
+            if (++c_b == nb) {  // the slab is done for this pass: add to the wavefront's sums in LDS
+                if (lane < rl) {
+                    float* dst = red + c_slab * 4u * rl + lane;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) dst[r * rl] += acc[0][r] + acc[1][r];
+                }
+                acc[0] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                acc[1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                c_b = 0;
+                ++c_slab;
+            }
+        };
+
+        for (uint32_t q = 0; q < batches; q += 3u) {
+            load(2);
+            compute(0);
+            load(0);
+            compute(1);
+            load(1);
+            compute(2);
+        }
+    }
+
+    // ---- add the wavefronts' sums in wavefront order, round once, store
+    __syncthreads();
+    const uint32_t outs = nslabs * p.m * kSlabCols;
+    for (uint32_t i = tid; i < outs; i += kThreadsWg) {
+        const uint32_t s = i / (p.m * kSlabCols), rc = i % (p.m * kSlabCols);
+        const uint32_t r = rc / kSlabCols, c = rc % kSlabCols;
+        const uint32_t col = (slab0 + s) * kSlabCols + c;
+        // result row r of column c: lane 16 (r / 4) + c, register r % 4
+        const uint32_t at = (s * 4u + (r & 3u)) * rl + (r >> 2) * 16u + c;
+        float sum = 0.0f;
+#pragma unroll
+        for (uint32_t w = 0; w < kWaves; ++w) sum += RED[w * red_wave + at];
+        if (col < p.n) {
+            p.y[static_cast<size_t>(r) * p.n + col] = static_cast<uint16_t>(f32_to_half_bits(sum));
+        }
+    }
+}
+
+// ND [k, n / 2] (even column in the low nibble, two's complement) -> packed; one thread per lane of a tile.
+__global__ __launch_bounds__(256) void pack_w4_kernel(const uint8_t* __restrict__ w, u32x4* __restrict__ out, uint32_t k,
+                                                      uint32_t n, uint32_t slabs, uint32_t ktiles)
+{
+    const size_t total = static_cast<size_t>(slabs) * ktiles * 64u;
+    const size_t i = static_cast<size_t>(blockIdx.x) * 256u + threadIdx.x;
+    if (i >= total + kPadTiles * 64u) {
+        return;
+    }
+    if (i >= total) {  // padding behind the last slab: w = 0
+        out[i] = u32x4{0x88888888u, 0x88888888u, 0x88888888u, 0x88888888u};
+        return;
+    }
+    const uint32_t lane = static_cast<uint32_t>(i & 63u);
+    const size_t tile_id = i >> 6;
+    const uint32_t slab = static_cast<uint32_t>(tile_id / ktiles), tile = static_cast<uint32_t>(tile_id % ktiles);
+    const uint32_t col = slab * kSlabCols + (lane & 15u), g = lane >> 4;
+    const size_t row_bytes = n / 2u;
+    u32x4 v;
+#pragma unroll
+    for (uint32_t d = 0; d < 4; ++d) {
+        uint32_t word = 0;
+#pragma unroll
+        for (uint32_t e = 0; e < 8; ++e) {
+            const uint32_t kk = tile * kTileK + g * 32u + d * 8u + e;
+            uint32_t u = 8u;  // w = 0
+            if (kk < k && col < n) {
+                const uint8_t byte = w[static_cast<size_t>(kk) * row_bytes + col / 2u];
+                u = ((col & 1u) ? (byte >> 4) : (byte & 15u)) ^ 8u;
+            }
+            const uint32_t nib = (e >> 1) + 4u * (e & 1u);  // k offsets 0..7 -> nibbles 0 4 1 5 2 6 3 7
+            word |= u << (4u * nib);
+        }
+        v[d] = word;
+    }
+    out[i] = v;
+}
+
+}  // namespace
+}  // namespace ascq
+
+using namespace ascq;
+
+extern "C" int ascq_pack_weight_w4_size(uint32_t k, uint32_t n, size_t* bytes)
+{
+    ASCQ_REQUIRE(bytes != nullptr, ASCQ_ENULL, "ascq_pack_weight_w4_size: bytes is NULL");
+    ASCQ_REQUIRE(k > 0 && n > 0 && n % 2 == 0, ASCQ_EINVAL, "ascq_pack_weight_w4_size: k, n must be positive and n even");
+    *bytes = (static_cast<size_t>((n + kSlabCols - 1u) / kSlabCols) * ((k + kTileK - 1u) / kTileK) + kPadTiles) * kTileBytes;
+    return ASCQ_OK;
+}
+
+extern "C" int ascq_pack_weight_w4(const void* w, void* packed, uint32_t k, uint32_t n, void* stream)
+{
+    ASCQ_REQUIRE(w && packed, ASCQ_ENULL, "ascq_pack_weight_w4: w / packed is NULL");
+    ASCQ_REQUIRE(k > 0 && n > 0 && n % 2 == 0, ASCQ_EINVAL, "ascq_pack_weight_w4: k, n must be positive and n even");
+    ASCQ_REQUIRE(aligned16(packed), ASCQ_EALIGN, "ascq_pack_weight_w4: packed must be 16-byte aligned");
+    const uint32_t slabs = (n + kSlabCols - 1u) / kSlabCols, ktiles = (k + kTileK - 1u) / kTileK;
+    const size_t lanes = (static_cast<size_t>(slabs) * ktiles + kPadTiles) * 64u;
+    ASCQ_REQUIRE((lanes + 255u) / 256u < (1ull << 31), ASCQ_EINVAL, "ascq_pack_weight_w4: matrix too large");
+    pack_w4_kernel<<<static_cast<uint32_t>((lanes + 255u) / 256u), 256, 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<const uint8_t*>(w), static_cast<u32x4*>(packed), k, n, slabs, ktiles);
+    return launch_status("ascq_pack_weight_w4");
+}
+
+// ref: include/adv_api/quantization/ascend_antiquant.h:50-54 (AscendAntiQuant<int4b_t, half>, per group along k)
+extern "C" int ascq_matmul_w4a16_packed(const ascq_w4a16_desc* d, void* y, const void* x, const void* w_packed,
+                                        const void* scale, const void* offset, void* stream)
+{
+    ASCQ_REQUIRE(d != nullptr, ASCQ_ENULL, "ascq_matmul_w4a16_packed: desc is NULL");
+    ASCQ_REQUIRE(d->m > 0 && d->n > 0 && d->k > 0, ASCQ_EINVAL, "ascq_matmul_w4a16_packed: m, n, k must be greater than 0");
+    ASCQ_REQUIRE(d->n % 2 == 0, ASCQ_EINVAL, "ascq_matmul_w4a16_packed: n must be even (two int4 per byte)");
+    ASCQ_REQUIRE(d->group_size > 0 && d->k % d->group_size == 0, ASCQ_EINVAL,
+                 "ascq_matmul_w4a16_packed: k %u must be a multiple of group_size %u", d->k, d->group_size);
+    ASCQ_REQUIRE(y && x && w_packed && scale, ASCQ_ENULL, "ascq_matmul_w4a16_packed: y / x / w_packed / scale is NULL");
+    ASCQ_REQUIRE(!d->has_offset || offset, ASCQ_ENULL, "ascq_matmul_w4a16_packed: offset is NULL");
+    const uint32_t g32 = d->group_size / 32u;
+    ASCQ_REQUIRE(d->k % kTileK == 0 && d->n % 8u == 0 && d->group_size % 32u == 0 && (g32 & (g32 - 1u)) == 0, ASCQ_EUNSUPPORTED,
+                 "ascq_matmul_w4a16_packed: k must be a multiple of 128, n of 8 and group_size 32 times a power of two "
+                 "(use ascq_matmul_w4a16 otherwise)");
+    ASCQ_REQUIRE((static_cast<uint64_t>((d->n + kSlabCols - 1u) / kSlabCols) * (d->k / kTileK) + kPadTiles) * kTileBytes < (1ull << 31) &&
+                     static_cast<uint64_t>(d->k / d->group_size) * d->n * 2u < (1ull << 31) &&
+                     static_cast<uint64_t>(kMaxRows) * d->k * 2u < (1ull << 31),
+                 ASCQ_EUNSUPPORTED, "ascq_matmul_w4a16_packed: packed weights, parameter tables and 16 activation rows must "
+                                    "each stay below 2 GiB");
+    ASCQ_REQUIRE(aligned16(x) && aligned16(w_packed) && aligned16(scale) && (!d->has_offset || aligned16(offset)), ASCQ_EALIGN,
+                 "ascq_matmul_w4a16_packed: x, w_packed, scale and offset must be 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    W4pParams p{};
+    p.wp = static_cast<const u32x4*>(w_packed);
+    p.scale = static_cast<const uint16_t*>(scale);
+    p.offset = d->has_offset ? static_cast<const uint16_t*>(offset) : nullptr;
+    p.n = d->n;
+    p.k = d->k;
+    p.mk = NibbleMasks{0x000F000Fu, 0x00F000F0u, 0x64006400u};
+    p.gs_shift = 0;
+    while ((1u << p.gs_shift) < g32) ++p.gs_shift;
+    p.slabs = (d->n + kSlabCols - 1u) / kSlabCols;
+    p.ktiles = d->k / kTileK;
+    static int cached_cus = 0;  // compute units of the device first used (one GPU per process in this library's use)
+    if (cached_cus == 0) {
+        int dev = 0, n_cu = 0;
+        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess &&
+            n_cu > 0) {
+            cached_cus = n_cu;
+        } else {
+            cached_cus = 256;
+        }
+    }
+    const uint32_t cus = static_cast<uint32_t>(cached_cus);
+    constexpr uint32_t waves = 8u, batch = 8u;  // 16 wavefronts with batches of 4 tiles measured slower (37 against 30 us)
+    for (uint32_t m0 = 0; m0 < d->m; m0 += kMaxRows) {
+        p.m = d->m - m0 < kMaxRows ? d->m - m0 : kMaxRows;
+        p.x = static_cast<const uint16_t*>(x) + static_cast<size_t>(m0) * d->k;
+        p.y = static_cast<uint16_t*>(y) + static_cast<size_t>(m0) * d->n;
+        p.red_lanes = p.m <= 4u ? 16u : 64u;
+        // Whole slabs per workgroup, one workgroup per compute unit when the slabs allow it; then the longest pass over
+        // k whose activations and parameters fit their shares of the LDS (a multiple of the wavefront count), and fewer
+        // slabs if the per-wavefront sums would not fit beside them.
+        uint32_t spw = (p.slabs + cus - 1u) / cus;
+        spw = spw < 1u ? 1u : (spw > kMaxSlabs ? kMaxSlabs : spw);
+        uint32_t pt = 0, xs_wave = 0, par_wave = 0, red_bytes = 0;
+        // entries per column of a wavefront's table: the groups its tiles can touch, rounded up to an odd number
+        auto par_rows = [&](uint32_t tiles) { return ((((tiles * 4u - 1u) >> p.gs_shift) + 2u) | 1u); };
+        for (;; --spw) {
+            const uint32_t all = (p.ktiles + waves - 1u) / waves * waves;
+            pt = ((kXBytes / p.m - waves * kRowPad) / (kTileK * 2u)) / waves * waves;
+            pt = pt < all ? pt : all;
+            while (pt > waves && (waves * par_rows(pt / waves) * spw * kSlabCols * 4u > kParBytes || par_rows(pt / waves) * 2u * spw > 128u)) pt -= waves;
+            xs_wave = p.m * (pt / waves * kTileK * 2u + kRowPad);
+            par_wave = par_rows(pt / waves) * spw * kSlabCols * 4u;
+            red_bytes = waves * spw * 4u * p.red_lanes * 4u;
+            if ((waves * par_wave <= kParBytes && par_rows(pt / waves) * 2u * spw <= 128u && waves * (xs_wave + par_wave) + red_bytes <= kPool) || spw == 1u) break;
+        }
+        ASCQ_REQUIRE(waves * par_wave <= kParBytes && par_rows(pt / waves) * 2u * spw <= 128u && waves * (xs_wave + par_wave) + red_bytes <= kPool, ASCQ_EUNSUPPORTED,
+                     "ascq_matmul_w4a16_packed: group_size %u too small for this shape", d->group_size);
+        p.slabs_per_wg = spw;
+        p.pass_tiles = pt;
+        p.ppr_magic = static_cast<uint32_t>(((1ull << 32) + pt / waves * 16u - 1u) / (pt / waves * 16u));
+        p.par_magic = static_cast<uint32_t>(((1ull << 32) + spw * 2u - 1u) / (spw * 2u));
+        p.xs_wave = xs_wave;
+        p.par_wave = par_wave;
+        p.par_pitch = par_rows(pt / waves);
+        p.par_off = waves * xs_wave;
+        p.red_off = p.par_off + waves * par_wave;
+        const uint32_t grid = (p.slabs + spw - 1u) / spw;
+        if (d->has_offset) {
+            w4a16_packed_kernel<true, waves, batch><<<grid, waves * 64u, 0, st>>>(p);
+        } else {
+            w4a16_packed_kernel<false, waves, batch><<<grid, waves * 64u, 0, st>>>(p);
+        }
+    }
+    return launch_status("ascq_matmul_w4a16_packed");
+}

@@ -433,6 +433,25 @@ int ascq_matmul_w4a16(const ascq_w4a16_desc* desc, void* y, const void* x, const
                       const void* offset, void* workspace, size_t workspace_bytes, void* stream);
 int ascq_matmul_w4a16_workspace_size(const ascq_w4a16_desc* desc, size_t* bytes);
 
+/*
+ * The same operator on weights pre-packed for this GPU (the step the reference does offline for its own L1 / L0
+ * layout: examples/.../quant_group_matmul_high_performance/scripts/gen_data.py:62-64 packs ND -> NZ before the kernel
+ * runs).  ascq_pack_weight_w4 turns w int4 [k, n] (two per byte along n, even column in the low nibble) into
+ * ascq_pack_weight_w4_size(k, n) bytes: slabs of 16 columns, each one contiguous run of tiles of 128 k (1 KiB: lane l
+ * of a wavefront owns column l % 16 and k 32 (l / 16) .. + 31; dword d of its 16 bytes holds k + 8 d .. + 7 with k
+ * offsets 0..7 in nibbles 0 4 1 5 2 6 3 7, nibbles stored as w + 8); columns past n and k past the end hold w = 0, and
+ * 16 tiles of w = 0 follow the last slab.  scale / offset stay [k / group_size, n].
+ * ascq_matmul_w4a16_packed computes exactly what ascq_matmul_w4a16 computes (same roundings per weight, fp32 sums, one
+ * rounding to half) in one launch with no workspace: a workgroup owns whole columns and adds its wavefronts' partial
+ * sums in a fixed order, so repeated calls give identical bits.  It is built for 1-4 activation rows (decode) and takes
+ * up to 16 per pass over the weights.  Requires k % 128 == 0, n % 8 == 0, group_size = 32 * 2^i (ASCQ_EUNSUPPORTED
+ * otherwise: use ascq_matmul_w4a16), and x, w_packed, scale, offset 16-byte aligned.
+ */
+int ascq_pack_weight_w4_size(uint32_t k, uint32_t n, size_t* bytes);
+int ascq_pack_weight_w4(const void* w, void* w_packed, uint32_t k, uint32_t n, void* stream);
+int ascq_matmul_w4a16_packed(const ascq_w4a16_desc* desc, void* y, const void* x, const void* w_packed,
+                             const void* scale, const void* offset, void* stream);
+
 /* ------------------------------------------------------------------- W8A16 */
 /*
  * Matmul with A half and B int8 de-quantised on the way in ("anti-quant" matmul): the B matrix is turned into half by

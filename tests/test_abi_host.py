@@ -287,3 +287,23 @@ def test_resource_checker_rejects_a_guarded_kernel_with_scratch(tmp_path):
     r = subprocess.run([sys.executable, os.path.join(ROOT, "asc-devkit_amd", "csrc", "check_resources.py"), str(remarks)],
                        capture_output=True, text=True)
     assert r.returncode == 1 and "100 bytes of scratch" in r.stderr
+
+
+def test_w4a16_packed_rejections_and_size():
+    d = abi.W4A16Desc(m=1, n=64, k=256, group_size=128, has_offset=0)
+    call = lambda d, y=FAKE, x=FAKE, w=FAKE, sc=FAKE, of=None: L.ascq_matmul_w4a16_packed(C.byref(d), y, x, w, sc, of, None)
+    assert L.ascq_matmul_w4a16_packed(None, FAKE, FAKE, FAKE, FAKE, None, None) == abi.ENULL
+    assert call(d, w=None) == abi.ENULL
+    assert call(abi.W4A16Desc(m=1, n=64, k=256, group_size=128, has_offset=1)) == abi.ENULL       # offset missing
+    assert call(abi.W4A16Desc(m=1, n=63, k=256, group_size=128, has_offset=0)) == abi.EINVAL
+    assert call(abi.W4A16Desc(m=1, n=64, k=256, group_size=100, has_offset=0)) == abi.EINVAL      # k % group_size
+    assert call(abi.W4A16Desc(m=1, n=64, k=160, group_size=32, has_offset=0)) == abi.EUNSUPPORTED  # k % 128
+    assert call(abi.W4A16Desc(m=1, n=66, k=256, group_size=128, has_offset=0)) == abi.EUNSUPPORTED  # n % 8
+    assert call(abi.W4A16Desc(m=1, n=64, k=384, group_size=96, has_offset=0)) == abi.EUNSUPPORTED  # 96 = 32 * 3
+    assert call(d, x=C.c_void_p(0x1008)) == abi.EALIGN
+    size = C.c_size_t(0)
+    assert L.ascq_pack_weight_w4_size(8192, 28672, C.byref(size)) == abi.OK
+    assert size.value == (28672 // 16 * (8192 // 128) + 16) * 1024               # slabs * tiles + 16 tiles of padding
+    assert L.ascq_pack_weight_w4_size(100, 30, C.byref(size)) == abi.OK and size.value == (2 * 1 + 16) * 1024
+    assert L.ascq_pack_weight_w4_size(128, 15, C.byref(size)) == abi.EINVAL
+    assert L.ascq_pack_weight_w4(None, FAKE, 128, 16, None) == abi.ENULL

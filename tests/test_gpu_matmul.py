@@ -233,24 +233,110 @@ def test_w4a16_small(m, k, n, gs, has_offset):
     assert np.mean(got.view(np.uint16) == want.view(np.uint16)) > 0.9
 
 
+def w4_packed_reference(w_bytes, k, n):
+    """The packed int4 layout restated in numpy: slabs of 16 columns, tiles of 128 k, lane l of a tile owns column l % 16
+    and k 32 (l / 16) .. + 31, dword d holds k + 8 d .. + 7 with k offsets 0..7 in nibbles 0 4 1 5 2 6 3 7, nibbles stored as
+    w + 8; 16 tiles of w = 0 behind the last slab."""
+    slabs, ktiles = (n + 15) // 16, (k + 127) // 128
+    u = np.full((ktiles * 128, slabs * 16), 8, dtype=np.uint32)                    # w = 0 where there is no weight
+    lo, hi = w_bytes & 15, w_bytes >> 4
+    nib = np.empty((k, n), dtype=np.uint32)
+    nib[:, 0::2], nib[:, 1::2] = lo, hi
+    u[:k, :n] = nib ^ 8
+    u = u.reshape(ktiles, 4, 4, 8, slabs, 16)                                      # tile, g, d, e, slab, j
+    pos = np.array([0, 4, 1, 5, 2, 6, 3, 7], dtype=np.uint32)                      # nibble of k offset e
+    words = (u << (4 * pos)[None, None, None, :, None, None]).sum(axis=3, dtype=np.uint64).astype(np.uint32)
+    words = words.transpose(3, 0, 1, 4, 2)                                         # slab, tile, g, j, d
+    body = np.ascontiguousarray(words).reshape(-1)
+    pad = np.full(16 * 256, 0x88888888, dtype=np.uint32)
+    return np.concatenate([body, pad]).view(np.uint8)
+
+
+@pytest.mark.parametrize("k,n", [(128, 16), (256, 40), (384, 1040), (1024, 272)])
+def test_pack_weight_w4_layout(k, n):
+    announce("pack w4", k, n)
+    rng = np.random.default_rng(k + n)
+    wp = pack_int4(rng.integers(-8, 8, (k, n)).astype(np.int8))
+    got = ops.pack_weight_w4(to_dev(wp), k, n).cpu().numpy()
+    assert np.array_equal(got, w4_packed_reference(wp, k, n))
+
+
+def w4_check(got, want, x):
+    # fp32 accumulation in a different order than the oracle's: rel-err <= 1e-3 of the row scale, and bit-identical
+    # halves nearly everywhere (<= 1 fp16 ulp wherever the result is not close to a cancellation)
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    ref = np.abs(x.astype(np.float64)).sum(axis=1, keepdims=True) * 8 * 1e-2      # bound on sum |x||w|
+    assert np.all(err <= 1e-3 * ref + 1e-6)
+    assert np.mean(got.view(np.uint16) == want.view(np.uint16)) > 0.9
+
+
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 9, 16, 17, 33])
+@pytest.mark.parametrize("k,n,gs", [(512, 1024, 128), (1024, 544, 64), (256, 40, 32), (384, 512, 128), (2048, 272, 256),
+                                     (2048, 64, 512), (128, 4112, 128)])
+@pytest.mark.parametrize("offset", ["int", "frac", None])
+def test_w4a16_packed_small(m, k, n, gs, offset):
+    """The pre-packed weight path computes what the [k, n / 2] path computes (same oracle)."""
+    announce("w4a16 packed", m, k, n, gs, offset)
+    rng = np.random.default_rng(m + k + n)
+    x, wp, sc, of = w4_case(rng, m, k, n, gs, offset is not None)
+    if offset == "frac":
+        of = (rng.standard_normal((k // gs, n)) * 3).astype(np.float16)
+    w_gpu = ops.pack_weight_w4(to_dev(wp), k, n)
+    y = torch.zeros((m, n), dtype=torch.float16, device=DEV)
+    ops.matmul_w4a16_packed(y, to_dev(x), w_gpu, to_dev(sc), None if of is None else to_dev(of), gs)
+    d = abi.W4A16Desc(m=m, n=n, k=k, group_size=gs, has_offset=int(of is not None))
+    w4_check(y.cpu().numpy(), orc.matmul_w4a16(d, x, wp, sc, of), x)
+
+
+def test_w4a16_packed_multi_pass_and_repeatable():
+    """k too long for one pass of staged activations (several passes per wavefront), and two calls give identical bits."""
+    m, k, n, gs = 4, 24576, 256, 128
+    announce("w4a16 packed long k", m, k, n)
+    rng = np.random.default_rng(5)
+    x, wp, sc, of = w4_case(rng, m, k, n, gs, True)
+    w_gpu = ops.pack_weight_w4(to_dev(wp), k, n)
+    xs, scs, ofs = to_dev(x), to_dev(sc), to_dev(of)
+    y1 = torch.zeros((m, n), dtype=torch.float16, device=DEV)
+    y2 = torch.zeros((m, n), dtype=torch.float16, device=DEV)
+    ops.matmul_w4a16_packed(y1, xs, w_gpu, scs, ofs, gs)
+    ops.matmul_w4a16_packed(y2, xs, w_gpu, scs, ofs, gs)
+    d = abi.W4A16Desc(m=m, n=n, k=k, group_size=gs, has_offset=1)
+    w4_check(y1.cpu().numpy(), orc.matmul_w4a16(d, x, wp, sc, of), x)
+    assert torch.equal(y1, y2)
+
+
+def config4_columns(m, n):
+    """The oracle covers every column at M=1 (about 6 s on 16 threads); for more rows three slabs: the first and the last
+    512 columns (the kernels' first and last column blocks) and one from the middle."""
+    return [(0, n)] if m == 1 else [(0, 512), (n // 2 - 256, n // 2 + 256), (n - 512, n)]
+
+
+def config4_check(got, x, wp, sc, of, d, cols):
+    orc.set_threads(16)
+    for c0, c1 in cols:
+        want = orc.matmul_w4a16(d, x, wp, sc, of, cols=(c0, c1))[:, c0:c1]
+        g = got[:, c0:c1]
+        err = np.abs(g.astype(np.float64) - want.astype(np.float64))
+        tol = 1e-3 * np.maximum(np.abs(want.astype(np.float64)), 1.0)          # fp32 epilogue rel-err <= 1e-3
+        assert np.all(err <= tol + 2e-3)
+        assert np.mean(g.view(np.uint16) == want.view(np.uint16)) > 0.99
+
+
+@pytest.mark.parametrize("packed", [False, True])
 @pytest.mark.parametrize("m", [1, 4, 16])
-def test_config4_w4a16_decode(m):
-    """fp16 [M,8192] x int4 [8192,28672], group 128, fp16 scale and offset."""
-    announce("config 4", m)
+def test_config4_w4a16_decode(m, packed):
+    """fp16 [M,8192] x int4 [8192,28672], group 128, fp16 scale and offset; both weight layouts."""
+    announce("config 4", m, "packed" if packed else "nd")
     rng = np.random.default_rng(0xC4 + m)
     k, n, gs = 8192, 28672, 128
     x, wp, sc, of = w4_case(rng, m, k, n, gs, True)
     y = torch.zeros((m, n), dtype=torch.float16, device=DEV)
-    ops.matmul_w4a16(y, to_dev(x), to_dev(wp), to_dev(sc), to_dev(of), gs)
+    if packed:
+        ops.matmul_w4a16_packed(y, to_dev(x), ops.pack_weight_w4(to_dev(wp), k, n), to_dev(sc), to_dev(of), gs)
+    else:
+        ops.matmul_w4a16(y, to_dev(x), to_dev(wp), to_dev(sc), to_dev(of), gs)
     d = abi.W4A16Desc(m=m, n=n, k=k, group_size=gs, has_offset=1)
-    orc.set_threads(16)
-    cols = (0, n) if m == 1 else (4096, 4096 + 2048)             # the oracle covers every column at M=1, a slab otherwise
-    want = orc.matmul_w4a16(d, x, wp, sc, of, cols=cols)[:, cols[0]:cols[1]]
-    got = y.cpu().numpy()[:, cols[0]:cols[1]]
-    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
-    tol = 1e-3 * np.maximum(np.abs(want.astype(np.float64)), 1.0)
-    assert np.all(err <= tol + 2e-3)
-    assert max_ulp(got.view(np.uint16), want.view(np.uint16), "f16") <= 4 or np.mean(err <= tol) > 0.999
+    config4_check(y.cpu().numpy(), x, wp, sc, of, d, config4_columns(m, n))
 
 
 # ------------------------------------------------------------------ W8A16 (Matmul anti-quant path)
