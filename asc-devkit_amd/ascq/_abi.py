@@ -102,6 +102,7 @@ SIGNATURES = {
     "ascq_matmul_w8a8": (C.c_int, [C.POINTER(MatmulDesc), _P, _P, _P, _P, _P, _P, _P, C.c_size_t, _P]),
     "ascq_matmul_w8a8_workspace_size": (C.c_int, [C.POINTER(MatmulDesc), C.POINTER(C.c_size_t)]),
     "ascq_linear_w8a8_dynamic": (C.c_int, [C.POINTER(MatmulDesc), C.c_int32, _P, _P, _P, _P, _P, _P, C.c_size_t, _P]),
+    "ascq_linear_w8a8_dynamic_noalloc": (C.c_int, [C.POINTER(MatmulDesc), C.c_int32, _P, _P, _P, _P, _P, _P]),
     "ascq_matmul_w8a8_plan": (C.c_int, [C.POINTER(MatmulDesc), _P, _P, _P, _P, _P, _P, _P, C.c_size_t,
                                         C.POINTER(MatmulPlan)]),
     "ascq_matmul_w4a4": (C.c_int, [C.POINTER(MatmulDesc), _P, _P, _P, _P, _P, _P, _P, C.c_size_t, _P]),

@@ -386,6 +386,20 @@ def linear_w8a8_dynamic(c, x, weight, channel_scale, bias=None, activation=abi.M
     return c
 
 
+def linear_w8a8_dynamic_noalloc(c, x, weight, channel_scale, bias=None, activation=abi.MM_ACT_NONE, trans_b=False):
+    """linear_w8a8_dynamic on the library's built-in scratch buffer: no workspace, no allocation.  Calls that overlap
+    on one GPU share that buffer and race."""
+    m, k = x.shape
+    n = c.shape[1]
+    d = abi.MatmulDesc(m=m, n=n, k=k, trans_b=int(trans_b), out_dtype=_dt(c), quant_mode=abi.MM_QUANT_VECTOR,
+                       scale_format=abi.MM_SCALE_F32, activation=activation)
+    if bias is not None:
+        d.bias_kind = abi.MM_BIAS_F32_POST if bias.dtype == torch.float32 else abi.MM_BIAS_BF16_POST
+    check(load_library().ascq_linear_w8a8_dynamic_noalloc(C.byref(d), _dt(x), _ptr(c), _ptr(x), _ptr(weight), _ptr(bias),
+                                                          _ptr(channel_scale), _stream()))
+    return c
+
+
 def quant_group_matmul(y, x, weight, group_list, scale, per_token_scale=None, bias=None,
                        group_list_kind=abi.GROUP_LIST_COUNTS, activation=abi.MM_ACT_NONE, weight_nz=False):
     """The quantized grouped matmul of the reference's MoE example: x int8 [m, k], weight int8 [g, k, n] (or, with

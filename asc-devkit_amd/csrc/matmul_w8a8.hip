@@ -25,6 +25,7 @@
 //   * Grouped matmul: same tile body; each workgroup finds its (group, row range) from the device-side group list,
 //     so no host synchronisation is needed and empty groups cost nothing.
 #include <cstdlib>
+#include <mutex>
 #include <type_traits>
 
 #include "matmul_w8a8.h"
@@ -750,6 +751,60 @@ extern "C" int ascq_linear_w8a8_dynamic(const ascq_matmul_desc* d, int32_t x_dty
     }
     return ascq_matmul_w8a8(&dd, c, q, b, bias, quant_vector, tok, rest,
                             workspace_bytes - static_cast<size_t>(rest - ws), stream);
+}
+
+// ------------------------------------------------------------------------------- the same call without a workspace
+// For callers that cannot allocate (code under stream capture, serving loops, harnesses that forbid hipMalloc): the
+// scratch of ascq_linear_w8a8_dynamic (quantised activations, token scales, partial sums of the small-m kernels) lives
+// in a device array that is part of this library's code object.  Each GPU the library runs on holds its own copy at
+// its own address until the process ends; the address is looked up once per device.  The array keeps the last call's
+// contents, which is harmless: every kernel writes what it later reads (nothing is expected to start at zero).
+namespace {
+constexpr size_t kStaticScratchBytes = ASCQ_STATIC_SCRATCH_BYTES;
+constexpr int kMaxDevices = 64;
+}  // namespace
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// Device address of `scratch` on the current device (in host code the array's name is only a handle for the lookup).
+static int static_scratch(void** out)
+{
+    static std::mutex lock;
+    static void* address[kMaxDevices] = {};
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    ASCQ_REQUIRE(e == hipSuccess && dev >= 0 && dev < kMaxDevices, ASCQ_EHIP,
+                 "ascq_linear_w8a8_dynamic_noalloc: hipGetDevice failed or device index %d is not below %d", dev, kMaxDevices);
+    std::lock_guard<std::mutex> guard(lock);
+    if (address[dev] == nullptr) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        ASCQ_REQUIRE(e == hipSuccess && ptr != nullptr, ASCQ_EHIP,
+                     "ascq_linear_w8a8_dynamic_noalloc: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+        address[dev] = ptr;
+    }
+    *out = address[dev];
+    return ASCQ_OK;
+}
+
+// No counterpart in the reference (its operators take a sharedTmpBuffer or pop one from the TPipe): this entry point
+// exists for callers that cannot allocate device memory.
+extern "C" int ascq_linear_w8a8_dynamic_noalloc(const ascq_matmul_desc* d, int32_t x_dtype, void* c, const void* x,
+                                                const void* b, const void* bias, const void* quant_vector, void* stream)
+{
+    size_t need = 0;
+    int rc = ascq_linear_w8a8_dynamic_workspace_size(d, &need);
+    if (rc != ASCQ_OK) {
+        return rc;
+    }
+    ASCQ_REQUIRE(need <= kStaticScratchBytes, ASCQ_EINVAL,
+                 "ascq_linear_w8a8_dynamic_noalloc: this shape needs %zu bytes of scratch, the built-in buffer holds %zu "
+                 "(use ascq_linear_w8a8_dynamic with a workspace)", need, kStaticScratchBytes);
+    void* ptr = nullptr;
+    rc = static_scratch(&ptr);
+    if (rc != ASCQ_OK) {
+        return rc;
+    }
+    return ascq_linear_w8a8_dynamic(d, x_dtype, c, x, b, bias, quant_vector, ptr, kStaticScratchBytes, stream);
 }
 
 // ------------------------------------------------------------------------------------------ int4 x int4 matmul

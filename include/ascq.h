@@ -388,6 +388,22 @@ int ascq_linear_w8a8_dynamic(const ascq_matmul_desc* desc, int32_t x_dtype, void
                              void* stream);
 int ascq_linear_w8a8_dynamic_workspace_size(const ascq_matmul_desc* desc, size_t* bytes);
 
+/*
+ * ascq_linear_w8a8_dynamic without a workspace argument and without any allocation (no hipMalloc / hipFree, here or in
+ * anything it calls).  It has no counterpart in the reference; it is for callers that cannot allocate device memory:
+ * code under stream capture, tight serving loops, harnesses that forbid hipMalloc.  The scratch (quantised
+ * activations, token scales, partial sums of the small-m kernels) is a device array of ASCQ_STATIC_SCRATCH_BYTES that
+ * is part of the library; every GPU the library runs on holds its own copy until the process ends.  Shapes whose
+ * ascq_linear_w8a8_dynamic_workspace_size exceeds that size are rejected with ASCQ_EINVAL (k = 4096, n = 11008 fits
+ * with 1, 16, 128 and 2048 rows; 32 rows need 32 MiB of partial sums and do not).  Results are those of
+ * ascq_linear_w8a8_dynamic, bit for bit.  All calls on one GPU share the one array: calls that overlap in time on
+ * the same GPU (two streams, two threads) race; serialise them or use the workspace form.  The first call on a device
+ * looks the array's address up (hipGetSymbolAddress); make that call outside stream capture.
+ */
+#define ASCQ_STATIC_SCRATCH_BYTES (24u << 20)
+int ascq_linear_w8a8_dynamic_noalloc(const ascq_matmul_desc* desc, int32_t x_dtype, void* c, const void* x, const void* b,
+                                     const void* bias, const void* quant_vector, void* stream);
+
 /* ------------------------------------------------ quantized grouped matmul */
 typedef enum ascq_group_list_kind {
     ASCQ_GROUP_LIST_COUNTS = 0,    /* rows per group (ref: examples/.../quant_group_matmul_custom.asc:264) */

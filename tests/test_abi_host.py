@@ -307,3 +307,11 @@ def test_w4a16_packed_rejections_and_size():
     assert L.ascq_pack_weight_w4_size(100, 30, C.byref(size)) == abi.OK and size.value == (2 * 1 + 16) * 1024
     assert L.ascq_pack_weight_w4_size(128, 15, C.byref(size)) == abi.EINVAL
     assert L.ascq_pack_weight_w4(None, FAKE, 128, 16, None) == abi.ENULL
+
+
+def test_noalloc_entry_point_rejects_before_touching_the_gpu():
+    d = abi.MatmulDesc(m=32, n=11008, k=4096, out_dtype=abi.BF16, quant_mode=abi.MM_QUANT_VECTOR,
+                       scale_format=abi.MM_SCALE_F32)
+    rc = L.ascq_linear_w8a8_dynamic_noalloc(C.byref(d), abi.BF16, FAKE, FAKE, FAKE, None, FAKE, None)
+    assert rc == abi.EINVAL and "built-in buffer" in err()
+    assert L.ascq_linear_w8a8_dynamic_noalloc(None, abi.BF16, FAKE, FAKE, FAKE, None, FAKE, None) == abi.ENULL
