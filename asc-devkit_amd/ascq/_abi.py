@@ -11,7 +11,7 @@ OK, EINVAL, EUNSUPPORTED, EALIGN, EHIP, ENULL = range(6)
 # ascq_dtype
 F16, BF16, F32, I8, I4, I32, U64, E8M0 = range(8)
 # ascq_policy
-PER_TENSOR, PER_CHANNEL, PER_TOKEN, PER_GROUP = range(4)
+PER_TENSOR, PER_CHANNEL, PER_TOKEN, PER_GROUP, PER_CHANNEL_PER_GROUP, PER_TOKEN_PER_GROUP = range(6)
 # ascq_round_mode (values of the reference's RoundMode enum)
 CAST_NONE, CAST_RINT, CAST_FLOOR, CAST_CEIL, CAST_ROUND, CAST_TRUNC = range(6)
 # ascq_quant_compute
@@ -125,6 +125,13 @@ SIGNATURES = {
                                                              C.POINTER(C.c_uint32), C.c_uint32, C.c_int32, C.c_int32,
                                                              C.c_int32, C.POINTER(C.c_uint32),
                                                              C.POINTER(C.c_uint32)]),
+    "ascq_get_ascend_quant_tmp_buffer_factor_size": (C.c_int, [C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
+    "ascq_get_ascend_dequant_tmp_buffer_factor_size": (C.c_int, [C.POINTER(C.c_uint32), C.c_uint32, C.POINTER(C.c_uint32),
+                                                                 C.POINTER(C.c_uint32)]),
+    "ascq_get_ascend_antiquant_tmp_buffer_factor_size": (C.c_int, [C.POINTER(C.c_uint32), C.c_uint32,
+                                                                   C.POINTER(C.c_uint32), C.c_uint32, C.c_int32, C.c_int32,
+                                                                   C.c_int32, C.POINTER(C.c_uint32),
+                                                                   C.POINTER(C.c_uint32)]),
     "ascq_pack_quant_param": (C.c_uint64, [C.c_float, C.c_int32, C.c_int32]),
     "ascq_pack_weight_nz": (C.c_int, [C.c_uint32, C.c_uint32, C.c_uint32, _P, _P, _P]),
     "ascq_zero_fill": (C.c_int, [_P, C.c_size_t, _P]),

@@ -155,8 +155,16 @@ def ascend_dequant(dst, src, deq_scale, params, mode=abi.DEQUANT_WITH_SINGLE_ROW
     return dst
 
 
+class AscendDeQuantPolicy:
+    """ref: include/adv_api/quantization/ascend_dequant_utils.h:37 (same members, same values)"""
+    PER_TOKEN, PER_GROUP, PER_CHANNEL_PER_GROUP, PER_TOKEN_PER_GROUP = range(4)
+    TO_ABI = {0: abi.PER_TOKEN, 1: abi.PER_GROUP, 2: abi.PER_CHANNEL_PER_GROUP, 3: abi.PER_TOKEN_PER_GROUP}
+
+
 def ascend_dequant_policy(dst, src, scale, para, policy, k_dim=1):
-    """AscendDequant<dstT, srcT, scaleT, config, policy> for PER_TOKEN / PER_GROUP.
+    """AscendDequant<dstT, srcT, scaleT, config, policy> for PER_TOKEN / PER_GROUP; `policy` is an ascq policy value
+    (abi.PER_TOKEN ...); AscendDeQuantPolicy.TO_ABI maps the reference's own enumerators.  The two combined policies the
+    reference declares are answered with ASCQ_EUNSUPPORTED.
     ref: include/adv_api/quantization/ascend_dequant.h:284-305."""
     d = abi.DequantDesc(policy=policy, src_dtype=_dt(src), scale_dtype=_dt(scale), dst_dtype=_dt(dst),
                         mode=abi.DEQUANT_WITH_MULTI_ROW, k_dim=k_dim, m=para.m, n=para.n, cal_count=para.cal_count,

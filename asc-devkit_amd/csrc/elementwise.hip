@@ -1003,6 +1003,9 @@ extern "C" int ascq_quant(const ascq_quant_desc* d, void* dst, const void* src, 
 {
     ASCQ_REQUIRE(d != nullptr, ASCQ_ENULL, "ascq_quant: desc is NULL");
     ASCQ_REQUIRE(dst != nullptr && src != nullptr, ASCQ_ENULL, "ascq_quant: dst/src is NULL");
+    ASCQ_REQUIRE(d->policy != ASCQ_PER_CHANNEL_PER_GROUP && d->policy != ASCQ_PER_TOKEN_PER_GROUP, ASCQ_EUNSUPPORTED,
+                 "ascq_quant: the combined policies PER_CHANNEL_PER_GROUP / PER_TOKEN_PER_GROUP are declared by the reference "
+                 "but implemented by none of its operators");
     ASCQ_REQUIRE(d->policy >= ASCQ_PER_TENSOR && d->policy <= ASCQ_PER_GROUP, ASCQ_EINVAL,
                  "ascq_quant: unknown policy %d", d->policy);
     ASCQ_REQUIRE(d->src_dtype == ASCQ_F16 || d->src_dtype == ASCQ_BF16 || d->src_dtype == ASCQ_F32, ASCQ_EUNSUPPORTED,
@@ -1162,6 +1165,9 @@ extern "C" int ascq_dequant(const ascq_dequant_desc* d, void* dst, const void* s
 {
     ASCQ_REQUIRE(d != nullptr, ASCQ_ENULL, "ascq_dequant: desc is NULL");
     ASCQ_REQUIRE(dst != nullptr && src != nullptr, ASCQ_ENULL, "ascq_dequant: dst/src is NULL");
+    ASCQ_REQUIRE(d->policy != ASCQ_PER_CHANNEL_PER_GROUP && d->policy != ASCQ_PER_TOKEN_PER_GROUP, ASCQ_EUNSUPPORTED,
+                 "ascq_dequant: the combined policies PER_CHANNEL_PER_GROUP / PER_TOKEN_PER_GROUP are declared by the reference "
+                 "but implemented by none of its operators");
     ASCQ_REQUIRE(d->policy >= ASCQ_PER_TENSOR && d->policy <= ASCQ_PER_GROUP, ASCQ_EINVAL,
                  "ascq_dequant: unknown policy %d", d->policy);
     ASCQ_REQUIRE(d->dst_dtype == ASCQ_F16 || d->dst_dtype == ASCQ_BF16 || d->dst_dtype == ASCQ_F32,
@@ -1331,6 +1337,9 @@ extern "C" int ascq_antiquant_policy(const ascq_antiquant_policy_desc* d, void* 
                  "ascq_antiquant_policy: dst / src / scale is NULL");
     ASCQ_REQUIRE(!d->has_offset || per_tensor || offset != nullptr, ASCQ_ENULL,
                  "ascq_antiquant_policy: offset tensor is NULL");
+    ASCQ_REQUIRE(d->policy != ASCQ_PER_CHANNEL_PER_GROUP && d->policy != ASCQ_PER_TOKEN_PER_GROUP, ASCQ_EUNSUPPORTED,
+                 "ascq_antiquant_policy: the combined policies PER_CHANNEL_PER_GROUP / PER_TOKEN_PER_GROUP are declared by the reference "
+                 "but implemented by none of its operators");
     ASCQ_REQUIRE(d->policy >= ASCQ_PER_TENSOR && d->policy <= ASCQ_PER_GROUP, ASCQ_EINVAL,
                  "ascq_antiquant_policy: unknown policy %d", d->policy);
     if (per_tensor || per_channel) {

@@ -222,3 +222,64 @@ extern "C" int ascq_get_ascend_antiquant_max_min_tmp_size(const uint32_t* src_sh
     }
     return ASCQ_OK;
 }
+
+// The "factor" queries: a temporary buffer of maxLiveNodeCount * (bytes of the data processed at once) + extraBuf bytes
+// serves the operator; host code that carves one shared buffer for several operators sizes it from them.
+// ref: impl/adv_api/tiling/quantization/ascend_quant_tiling_impl.cpp:57-61 (GetAscendQuantTmpBufferFactorSize; the
+// Quantize form, quantize_tiling_impl.cpp, answers the same)
+extern "C" int ascq_get_ascend_quant_tmp_buffer_factor_size(uint32_t* max_live_node_count, uint32_t* extra_buf)
+{
+    ASCQ_REQUIRE(max_live_node_count && extra_buf, ASCQ_ENULL, "GetAscendQuantTmpBufferFactorSize: NULL argument");
+    *max_live_node_count = 2u;
+    *extra_buf = 0u;
+    return ASCQ_OK;
+}
+
+// ref: impl/adv_api/tiling/quantization/ascend_dequant_tiling_impl.cpp:67-81
+extern "C" int ascq_get_ascend_dequant_tmp_buffer_factor_size(const uint32_t* shape, uint32_t ndim,
+                                                              uint32_t* max_live_node_count, uint32_t* extra_buf)
+{
+    ASCQ_REQUIRE(max_live_node_count && extra_buf && (shape || ndim == 0), ASCQ_ENULL,
+                 "GetAscendDequantTmpBufferFactorSize: NULL argument");
+    *extra_buf = 8u + 64u;  // floats per 32-byte block + floats per 256-byte repeat
+    if (ndim == 2) {
+        *extra_buf += shape[1];
+        *max_live_node_count = 1u;
+    } else if (ndim == 1) {
+        *max_live_node_count = 2u;
+    } else {  // the reference answers any other rank with zeros
+        *extra_buf = 0u;
+        *max_live_node_count = 0u;
+    }
+    return ASCQ_OK;
+}
+
+// ref: impl/adv_api/tiling/quantization/ascend_antiquant_tiling_impl.cpp:145-169 (int8 / int4 and the 4-bit float sources)
+extern "C" int ascq_get_ascend_antiquant_tmp_buffer_factor_size(const uint32_t* src_shape, uint32_t src_ndim,
+                                                                const uint32_t* scale_shape, uint32_t scale_ndim,
+                                                                int32_t is_transpose, int32_t input_format,
+                                                                int32_t output_dtype, uint32_t* max_live_node_count,
+                                                                uint32_t* extra_buf)
+{
+    ASCQ_REQUIRE(src_shape && scale_shape && max_live_node_count && extra_buf, ASCQ_ENULL,
+                 "GetAscendAntiQuantTmpBufferFactorSize: NULL argument");
+    ASCQ_REQUIRE(src_ndim >= 1, ASCQ_EINVAL, "[AscendAntiQuant] srcShape has no dimension");
+    *extra_buf = 0u;
+    *max_live_node_count = 0u;
+    const uint32_t scale_size = static_cast<uint32_t>(std::max<uint64_t>(shape_size(scale_shape, scale_ndim), 1));
+    const bool per_channel = scale_size != 1;
+    if (input_format == ASCQ_QDST_FP4_E2M1 || input_format == ASCQ_QDST_FP4_E1M2) {
+        if (is_transpose) {
+            *extra_buf = (scale_size + 31u) / 32u * 32u * 2u;
+        }
+    } else if (output_dtype == ASCQ_F16) {
+        // nothing
+    } else if (is_transpose && per_channel) {
+        *extra_buf = 80u * scale_size * 4u;
+    } else if (!per_channel) {
+        *max_live_node_count = 1u;
+    } else {
+        *extra_buf = scale_size * 2u * 4u + 64u * src_shape[0] * 4u;
+    }
+    return ASCQ_OK;
+}

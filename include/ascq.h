@@ -52,7 +52,11 @@ typedef enum ascq_policy {
     ASCQ_PER_TENSOR = 0,
     ASCQ_PER_CHANNEL = 1,
     ASCQ_PER_TOKEN = 2,
-    ASCQ_PER_GROUP = 3
+    ASCQ_PER_GROUP = 3,
+    /* declared by the reference (same header, and ascend_dequant_utils.h:37), implemented by none of its operators:
+       every entry point answers them with ASCQ_EUNSUPPORTED */
+    ASCQ_PER_CHANNEL_PER_GROUP = 4,
+    ASCQ_PER_TOKEN_PER_GROUP = 5
 } ascq_policy;
 
 /* ref: impl/basic_api/utils/kernel_utils_mode.h:94-109 (RoundMode), same values */
@@ -314,7 +318,11 @@ typedef struct ascq_matmul_desc {
     int32_t has_tok_scale; /* fp32 [m] multiplied after the channel scale */
     int32_t activation;    /* ascq_mm_activation */
     int32_t b_format;      /* ascq_mm_b_format; for the grouped matmul every group's [k, n] block is in this format */
-    uint64_t quant_scalar; /* QUANT_SCALAR: U64 word, or fp32 bits in the low half for F32 format */
+    uint64_t quant_scalar; /* QUANT_SCALAR: U64 word, or fp32 bits in the low half for F32 format.  A U64 word with
+                              the mode-control bit 36 set (pre-shift by bits [35:32], fixpipe_l0c2gm/scripts/
+                              gen_data_s322f16.py:48-58,84-90) is rejected with ASCQ_EUNSUPPORTED; words of a quant
+                              vector live on the device and are not inspected: bit 36 and the shift are outside the
+                              supported domain there */
 } ascq_matmul_desc;
 
 int ascq_matmul_w8a8(const ascq_matmul_desc* desc, void* c, const void* a, const void* b, const void* bias,
@@ -511,6 +519,20 @@ int ascq_get_ascend_antiquant_max_min_tmp_size(const uint32_t* src_shape, uint32
                                                const uint32_t* scale_shape, uint32_t scale_ndim, int32_t is_transpose,
                                                int32_t input_dtype, int32_t output_dtype, uint32_t* max_value,
                                                uint32_t* min_value);
+/*
+ * The reference's Get*TmpBufferFactorSize: a temporary buffer of maxLiveNodeCount * (bytes processed at once) + extraBuf
+ * bytes serves the operator (ascend_quant_tiling_impl.cpp:57-61, ascend_dequant_tiling_impl.cpp:67-81,
+ * ascend_antiquant_tiling_impl.cpp:145-169; GetQuantizeTmpBufferFactorSize answers as the AscendQuant form).  Same
+ * values, for host code that sizes a shared buffer from them; input_format of the AntiQuant form is an ascq_quant_dst
+ * value (the source formats of ascq_antiquant_policy; int4 sources answer as ASCQ_QDST_I8).
+ */
+int ascq_get_ascend_quant_tmp_buffer_factor_size(uint32_t* max_live_node_count, uint32_t* extra_buf);
+int ascq_get_ascend_dequant_tmp_buffer_factor_size(const uint32_t* shape, uint32_t ndim, uint32_t* max_live_node_count,
+                                                   uint32_t* extra_buf);
+int ascq_get_ascend_antiquant_tmp_buffer_factor_size(const uint32_t* src_shape, uint32_t src_ndim,
+                                                     const uint32_t* scale_shape, uint32_t scale_ndim,
+                                                     int32_t is_transpose, int32_t input_format, int32_t output_dtype,
+                                                     uint32_t* max_live_node_count, uint32_t* extra_buf);
 
 /* -------------------------------------------------------------- utilities */
 /* Pack an fp32 scale (and optional REQ8 offset / sign) into the fixpipe uint64 word. Host-side, pure. */

@@ -143,7 +143,9 @@ private:
 
 // ref: include/adv_api/quantization/ascend_quant_utils.h:31-87
 enum class RoundMode : int32_t { CAST_NONE = 0, CAST_RINT, CAST_FLOOR, CAST_CEIL, CAST_ROUND, CAST_TRUNC };
-enum class AscendQuantPolicy : int32_t { PER_TENSOR, PER_CHANNEL, PER_TOKEN, PER_GROUP };
+// ref: include/adv_api/quantization/ascend_quant_utils.h:73-80 (same members, same values; the two combined policies are
+// declared there and implemented by none of the reference's operators: ascq_quant answers ASCQ_EUNSUPPORTED)
+enum class AscendQuantPolicy : int32_t { PER_TENSOR, PER_CHANNEL, PER_TOKEN, PER_GROUP, PER_CHANNEL_PER_GROUP, PER_TOKEN_PER_GROUP };
 struct AscendQuantConfig {
     bool hasOffset = false;
     int32_t kDim = 1;
@@ -337,7 +339,17 @@ struct AscendDeQuantConfig {
     bool hasOffset = false;
     int32_t kDim = 1;
 };
-enum class AscendDeQuantPolicy : int32_t { PER_TENSOR, PER_CHANNEL, PER_TOKEN, PER_GROUP };
+// ref: include/adv_api/quantization/ascend_dequant_utils.h:37 (same members, same values: PER_TOKEN is 0 here)
+enum class AscendDeQuantPolicy : int32_t { PER_TOKEN, PER_GROUP, PER_CHANNEL_PER_GROUP, PER_TOKEN_PER_GROUP };
+inline int32_t ToAscqPolicy(AscendDeQuantPolicy p)
+{
+    switch (p) {
+        case AscendDeQuantPolicy::PER_TOKEN: return ASCQ_PER_TOKEN;
+        case AscendDeQuantPolicy::PER_GROUP: return ASCQ_PER_GROUP;
+        case AscendDeQuantPolicy::PER_CHANNEL_PER_GROUP: return ASCQ_PER_CHANNEL_PER_GROUP;  // rejected by ascq_dequant
+        default: return ASCQ_PER_TOKEN_PER_GROUP;                                            // likewise
+    }
+}
 struct AscendDeQuantParam {
     uint32_t m;
     uint32_t n;
@@ -351,7 +363,7 @@ void AscendDequant(const DeviceTensor<dstT>& dstTensor, const DeviceTensor<srcT>
                    void* stream = nullptr)
 {
     ascq_dequant_desc d{};
-    d.policy = static_cast<int32_t>(policy);
+    d.policy = ToAscqPolicy(policy);
     d.src_dtype = DTypeOf<srcT>::value;
     d.scale_dtype = DTypeOf<scaleT>::value;
     d.dst_dtype = DTypeOf<dstT>::value;

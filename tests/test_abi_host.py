@@ -315,3 +315,67 @@ def test_noalloc_entry_point_rejects_before_touching_the_gpu():
     rc = L.ascq_linear_w8a8_dynamic_noalloc(C.byref(d), abi.BF16, FAKE, FAKE, FAKE, None, FAKE, None)
     assert rc == abi.EINVAL and "built-in buffer" in err()
     assert L.ascq_linear_w8a8_dynamic_noalloc(None, abi.BF16, FAKE, FAKE, FAKE, None, FAKE, None) == abi.ENULL
+
+
+def test_integration_snippet_matches_the_abi():
+    """The ctypes struct printed in INTEGRATION.md has the fields of the struct the library reads."""
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    block = text[text.index("class QuantDesc(C.Structure)"):]
+    block = block[:block.index("lib.ascq_quant.restype")]
+    fields = re.findall(r'\("([a-z_]+)", C\.(c_[a-z0-9]+)\)', block)
+    # compare names and the ctypes types themselves (c_int32 is an alias of c_int on this platform)
+    got = [(n, getattr(C, t)) for n, t in fields]
+    assert got == list(abi.QuantDesc._fields_), (got, abi.QuantDesc._fields_)
+
+
+def test_combined_policies_are_rejected_by_name():
+    FAKE2 = C.c_void_p(0x100000)
+    for pol in (abi.PER_CHANNEL_PER_GROUP, abi.PER_TOKEN_PER_GROUP):
+        assert L.ascq_quant(C.byref(q(policy=pol)), FAKE, FAKE2, FAKE, FAKE, None) == abi.EUNSUPPORTED
+        assert "PER_CHANNEL_PER_GROUP" in err()
+        dq = abi.DequantDesc(policy=pol, src_dtype=abi.I32, scale_dtype=abi.F32, dst_dtype=abi.F32, m=4, n=8, cal_count=32,
+                             group_size=8)
+        assert L.ascq_dequant(C.byref(dq), FAKE, FAKE2, FAKE, None) == abi.EUNSUPPORTED
+        aq = abi.AntiQuantPolicyDesc(policy=pol, dst_dtype=abi.F16, scale_dtype=abi.F16, m=4, n=32, cal_count=128,
+                                     group_size=8)
+        assert L.ascq_antiquant_policy(C.byref(aq), FAKE, FAKE2, FAKE, None, None) == abi.EUNSUPPORTED
+    assert L.ascq_quant(C.byref(q(policy=6)), FAKE, FAKE2, FAKE, FAKE, None) == abi.EINVAL
+    from ascq import ops
+    assert ops.AscendDeQuantPolicy.TO_ABI[ops.AscendDeQuantPolicy.PER_TOKEN] == abi.PER_TOKEN
+    assert ops.AscendDeQuantPolicy.PER_TOKEN == 0 and ops.AscendDeQuantPolicy.PER_TOKEN_PER_GROUP == 3
+
+
+def test_quant_word_with_pre_shift_bit_is_rejected():
+    d = abi.MatmulDesc(m=16, n=32, k=64, out_dtype=abi.F16, quant_mode=abi.MM_QUANT_SCALAR, scale_format=abi.MM_SCALE_U64,
+                       quant_scalar=(1 << 36) | (3 << 32) | (0x3F800000 & 0xFFFFE000))
+    rc = L.ascq_matmul_w8a8(C.byref(d), FAKE, FAKE, FAKE, None, None, None, None, 0, None)
+    assert rc == abi.EUNSUPPORTED and "bit 36" in err()
+
+
+def test_tmp_buffer_factor_sizes_known_answers():
+    """tests/api/adv_api/tiling/test_tiling.cpp:6549-6553, 6565-6569, 6583-6608, 6621-6625, 6643-6647, 6662-6666,
+    6684-6688 of the reference."""
+    U = C.c_uint32
+    live, extra = U(9), U(9)
+    assert L.ascq_get_ascend_quant_tmp_buffer_factor_size(C.byref(live), C.byref(extra)) == abi.OK
+    assert (live.value, extra.value) == (2, 0)
+    shape = (U * 2)(10, 32)
+    assert L.ascq_get_ascend_dequant_tmp_buffer_factor_size(shape, 2, C.byref(live), C.byref(extra)) == abi.OK
+    assert (live.value, extra.value) == (1, 104)
+    shape1 = (U * 1)(320)
+    assert L.ascq_get_ascend_dequant_tmp_buffer_factor_size(shape1, 1, C.byref(live), C.byref(extra)) == abi.OK
+    assert (live.value, extra.value) == (2, 72)
+    shape3 = (U * 3)(2, 3, 4)
+    assert L.ascq_get_ascend_dequant_tmp_buffer_factor_size(shape3, 3, C.byref(live), C.byref(extra)) == abi.OK
+    assert (live.value, extra.value) == (0, 0)
+
+    def aq(src, scale, transpose, out):
+        s, c = (U * len(src))(*src), (U * len(scale))(*scale)
+        assert L.ascq_get_ascend_antiquant_tmp_buffer_factor_size(s, len(src), c, len(scale), int(transpose), 0, out,
+                                                                  C.byref(live), C.byref(extra)) == abi.OK
+        return live.value, extra.value
+    assert aq((640, 5120), (1, 5120), False, abi.F16) == (0, 0)
+    assert aq((640, 5120), (1, 5120), False, abi.BF16) == (0, 5120 * 2 * 4 + 64 * 640 * 4)
+    assert aq((640, 5120), (1,), False, abi.BF16) == (1, 0)
+    assert aq((64, 512), (64, 1), True, abi.BF16) == (0, 80 * 64 * 4)
+    assert aq((640, 5120), (1,), True, abi.BF16) == (1, 0)
