@@ -272,7 +272,7 @@ class Matmul:
         self.desc = abi.MatmulDesc(m=m, n=n, k=k, trans_a=int(trans_a), trans_b=int(trans_b), out_dtype=abi.I32,
                                    quant_mode=abi.MM_QUANT_NONE, scale_format=abi.MM_SCALE_U64)
         self.a = self.b = self.bias = self.quant = self.tok = None
-        self._ws = None
+        self._ws_by_stream = {}   # scratch per stream handle: calls of one object on two streams may overlap
 
     def set_tensor_a(self, a):
         self.a = a
@@ -310,13 +310,26 @@ class Matmul:
     def set_activation(self, activation):
         self.desc.activation = activation
 
+    def _scratch(self, need_bytes, device):
+        """The object's scratch buffer for the current stream (grown when a larger one is needed)."""
+        key = _stream().value
+        ws = self._ws_by_stream.get(key)
+        if ws is None or ws.numel() * 4 < need_bytes:
+            ws = torch.empty((need_bytes + 3) // 4, dtype=torch.int32, device=device)
+            self._ws_by_stream[key] = ws
+        return ws
+
+    @property
+    def _ws(self):
+        return self._ws_by_stream.get(_stream().value)
+
     def iterate_all(self, c):
         self.desc.out_dtype = _dt(c)
         lib = load_library()
         need = C.c_size_t(0)
         check(lib.ascq_matmul_w8a8_workspace_size(C.byref(self.desc), C.byref(need)))
-        if need.value and (self._ws is None or self._ws.numel() * 4 < need.value):
-            self._ws = torch.empty((need.value + 3) // 4, dtype=torch.int32, device=c.device)
+        if need.value:
+            self._scratch(need.value, c.device)
         check(lib.ascq_matmul_w8a8(C.byref(self.desc), _ptr(c), _ptr(self.a), _ptr(self.b), _ptr(self.bias),
                                    _ptr(self.quant), _ptr(self.tok), _ptr(self._ws) if need.value else None,
                                    need.value, _stream()))
@@ -330,8 +343,8 @@ class Matmul:
         lib = load_library()
         need = C.c_size_t(0)
         check(lib.ascq_matmul_w8a8_workspace_size(C.byref(self.desc), C.byref(need)))
-        if need.value and (self._ws is None or self._ws.numel() * 4 < need.value):
-            self._ws = torch.empty((need.value + 3) // 4, dtype=torch.int32, device=c.device)
+        if need.value:
+            self._scratch(need.value, c.device)
         plan = abi.MatmulPlan()
         check(lib.ascq_matmul_w8a8_plan(C.byref(self.desc), _ptr(c), _ptr(self.a), _ptr(self.b), _ptr(self.bias),
                                         _ptr(self.quant), _ptr(self.tok), _ptr(self._ws) if need.value else None,
@@ -349,8 +362,7 @@ class MatmulInt4(Matmul):
         lib = load_library()
         need = C.c_size_t(0)
         check(lib.ascq_matmul_w4a4_workspace_size(C.byref(self.desc), C.byref(need)))
-        if self._ws is None or self._ws.numel() * 4 < need.value:
-            self._ws = torch.empty((need.value + 3) // 4, dtype=torch.int32, device=c.device)
+        self._scratch(max(need.value, 4), c.device)
         check(lib.ascq_matmul_w4a4(C.byref(self.desc), _ptr(c), _ptr(self.a), _ptr(self.b), _ptr(self.bias),
                                    _ptr(self.quant), _ptr(self.tok), _ptr(self._ws), need.value, _stream()))
         return c
@@ -385,7 +397,7 @@ def linear_w8a8_dynamic(c, x, weight, channel_scale, bias=None, activation=abi.M
     lib = load_library()
     need = C.c_size_t(0)
     check(lib.ascq_linear_w8a8_dynamic_workspace_size(C.byref(d), C.byref(need)))
-    key = (x.device, need.value)
+    key = (x.device, need.value, _stream().value)    # one scratch buffer per stream: calls on two streams may overlap
     if key not in _lin_ws:
         _lin_ws[key] = torch.empty(max(need.value, 16), dtype=torch.uint8, device=x.device)
     ws = _lin_ws[key]
@@ -443,7 +455,7 @@ def matmul_w4a16(y, x, w_packed, scale, offset=None, group_size=128, workspace=N
     need = C.c_size_t(0)
     check(lib.ascq_matmul_w4a16_workspace_size(C.byref(d), C.byref(need)))
     if workspace is None:
-        key = (x.device, need.value)
+        key = (x.device, need.value, _stream().value)   # one scratch buffer per stream: calls on two streams may overlap
         if key not in _w4_ws:
             _w4_ws[key] = torch.zeros(max(need.value // 4, 4), dtype=torch.float32, device=x.device)
         workspace = _w4_ws[key]
@@ -489,7 +501,7 @@ def matmul_w8a16(y, x, w, offset=None, scale=None, workspace=None):
     need = C.c_size_t(0)
     check(lib.ascq_matmul_w8a16_workspace_size(C.byref(d), C.byref(need)))
     if workspace is None:
-        key = (x.device, need.value)
+        key = (x.device, need.value, _stream().value)   # one scratch buffer per stream: calls on two streams may overlap
         if key not in _w4_ws:
             _w4_ws[key] = torch.zeros(max(need.value // 4, 4), dtype=torch.float32, device=x.device)
         workspace = _w4_ws[key]
