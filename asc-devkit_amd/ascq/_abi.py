@@ -25,7 +25,7 @@ DEQUANT_WITH_SINGLE_ROW, DEQUANT_WITH_MULTI_ROW = range(2)
 MM_QUANT_NONE, MM_QUANT_SCALAR, MM_QUANT_VECTOR = range(3)
 MM_SCALE_U64, MM_SCALE_F32 = range(2)
 MM_BIAS_NONE, MM_BIAS_I32_PRE, MM_BIAS_F32_POST, MM_BIAS_BF16_POST = range(4)
-MM_ACT_NONE, MM_ACT_FASTER_GELU = range(2)
+MM_ACT_NONE, MM_ACT_FASTER_GELU, MM_ACT_SWIGLU = range(3)
 MM_B_ND, MM_B_NZ = range(2)
 GROUP_LIST_COUNTS, GROUP_LIST_PREFIX_SUM = range(2)
 
@@ -64,7 +64,8 @@ class MatmulDesc(C.Structure):
     _fields_ = [("m", C.c_uint32), ("n", C.c_uint32), ("k", C.c_uint32), ("trans_a", C.c_int32),
                 ("trans_b", C.c_int32), ("out_dtype", C.c_int32), ("quant_mode", C.c_int32),
                 ("scale_format", C.c_int32), ("bias_kind", C.c_int32), ("has_tok_scale", C.c_int32),
-                ("activation", C.c_int32), ("b_format", C.c_int32), ("quant_scalar", C.c_uint64)]
+                ("activation", C.c_int32), ("b_format", C.c_int32), ("quant_scalar", C.c_uint64),
+                ("act_beta", C.c_float), ("reserved", C.c_int32)]
 
 
 class GroupMatmulDesc(C.Structure):

@@ -307,8 +307,11 @@ class Matmul:
     def set_token_scale(self, tok_scale):
         self.tok, self.desc.has_tok_scale = tok_scale, 1
 
-    def set_activation(self, activation):
+    def set_activation(self, activation, beta=1.0):
+        """MM_ACT_FASTER_GELU, or MM_ACT_SWIGLU: columns 2j / 2j + 1 of the product are src0 / src1 of
+        SwiGLU(src0, src1, beta) and c is [m, n / 2] (ref: include/adv_api/activation/swiglu.h)."""
         self.desc.activation = activation
+        self.desc.act_beta = beta
 
     def _scratch(self, need_bytes, device):
         """The object's scratch buffer for the current stream (grown when a larger one is needed)."""
@@ -384,14 +387,14 @@ def unpack_int4(src, out=None):
 _lin_ws = {}
 
 
-def linear_w8a8_dynamic(c, x, weight, channel_scale, bias=None, activation=abi.MM_ACT_NONE, trans_b=False):
+def linear_w8a8_dynamic(c, x, weight, channel_scale, bias=None, activation=abi.MM_ACT_NONE, trans_b=False, act_beta=1.0):
     """c = dequant(dynamic_quant_per_token(x) @ weight): the activation quantiser and the int8 matmul in one call, with
     the results of calling the two one after the other.  x half / bfloat16 / float32 [m, k]; weight int8 [k, n];
     channel_scale float32 [n]; bias float32 / bfloat16 [n] (added after dequantisation)."""
     m, k = x.shape
-    n = c.shape[1]
+    n = weight.shape[0] if trans_b else weight.shape[1]    # with SwiGLU c has n / 2 columns
     d = abi.MatmulDesc(m=m, n=n, k=k, trans_b=int(trans_b), out_dtype=_dt(c), quant_mode=abi.MM_QUANT_VECTOR,
-                       scale_format=abi.MM_SCALE_F32, activation=activation)
+                       scale_format=abi.MM_SCALE_F32, activation=activation, act_beta=act_beta)
     if bias is not None:
         d.bias_kind = abi.MM_BIAS_F32_POST if bias.dtype == torch.float32 else abi.MM_BIAS_BF16_POST
     lib = load_library()
@@ -421,7 +424,7 @@ def linear_w8a8_dynamic_noalloc(c, x, weight, channel_scale, bias=None, activati
 
 
 def quant_group_matmul(y, x, weight, group_list, scale, per_token_scale=None, bias=None,
-                       group_list_kind=abi.GROUP_LIST_COUNTS, activation=abi.MM_ACT_NONE, weight_nz=False):
+                       group_list_kind=abi.GROUP_LIST_COUNTS, activation=abi.MM_ACT_NONE, weight_nz=False, act_beta=1.0):
     """The quantized grouped matmul of the reference's MoE example: x int8 [m, k], weight int8 [g, k, n] (or, with
     weight_nz, the example's fractal layout [g, n/32, k/16, 16, 32]), scale float32 [g, n], per_token_scale float32
     [m], group_list int64 [g] (counts or prefix sums).
@@ -433,7 +436,7 @@ def quant_group_matmul(y, x, weight, group_list, scale, per_token_scale=None, bi
         g, k, n = weight.shape
     mm = abi.MatmulDesc(m=x.shape[0], n=n, k=k, out_dtype=_dt(y), quant_mode=abi.MM_QUANT_VECTOR,
                         scale_format=abi.MM_SCALE_F32, has_tok_scale=int(per_token_scale is not None),
-                        activation=activation, b_format=abi.MM_B_NZ if weight_nz else abi.MM_B_ND)
+                        activation=activation, act_beta=act_beta, b_format=abi.MM_B_NZ if weight_nz else abi.MM_B_ND)
     if bias is not None:
         mm.bias_kind = abi.MM_BIAS_F32_POST if bias.dtype == torch.float32 else abi.MM_BIAS_BF16_POST
     d = abi.GroupMatmulDesc(mm=mm, groups=g, group_list_kind=group_list_kind)

@@ -13,6 +13,7 @@ struct EpiParams {
     uint32_t ldc;
     int out_dtype, quant_mode, scale_format, bias_kind, has_tok, activation;
     uint64_t quant_scalar;
+    float act_beta;  // SwiGLU
 };
 
 struct GemmParams {
@@ -68,6 +69,40 @@ __device__ __forceinline__ float faster_gelu(float x)
     const float x2 = expf(0.851f * (x - ax));
     const float x3 = 1.0f + expf(-1.702f * ax);
     return x * x2 / x3;
+}
+
+// SwiGLU of one column pair in fp32, one rounding per step, in the order of the reference's vector instructions
+// (Muls by -beta, Exp, Adds 1, Div, Mul: impl/adv_api/detail/activation/swiglu/swiglu_common_impl.h:154-190).
+__device__ __forceinline__ float swiglu(float src0, float src1, float beta)
+{
+    const float t = src1 * (-1.0f * beta);
+    const float d = expf(t) + 1.0f;
+    return src0 * (src1 / d);
+}
+
+// v of one accumulator before any activation: channel scale, token scale, post-dequant bias.
+__device__ __forceinline__ float epilogue_value(const EpiParams& e, int32_t acc, const ChannelQ& q, float tok, float bias_post)
+{
+    float v = static_cast<float>(acc) * q.s;
+    if (e.has_tok) {
+        v = v * tok;
+    }
+    if (e.bias_kind >= ASCQ_MM_BIAS_F32_POST) {
+        v = v + bias_post;
+    }
+    return v;
+}
+
+// Stores one floating-point value of the SwiGLU epilogue (C is [m, n / 2], e.ldc = n / 2).
+__device__ __forceinline__ void store_float_out(const EpiParams& e, size_t idx, float v)
+{
+    if (e.out_dtype == ASCQ_BF16) {
+        static_cast<uint16_t*>(e.c)[idx] = static_cast<uint16_t>(f32_to_bf16_bits(v));
+    } else if (e.out_dtype == ASCQ_F16) {
+        static_cast<uint16_t*>(e.c)[idx] = static_cast<uint16_t>(f32_to_half_bits_sat(v));
+    } else {
+        static_cast<float*>(e.c)[idx] = v;
+    }
 }
 
 // Everything after the int32 accumulator, for one output element.  `bias_post` is already widened to fp32.

@@ -498,8 +498,16 @@ int validate_mm(const ascq_matmul_desc* d, const char* who, const void* c, const
                  "%s: unknown scale format %d", who, d->scale_format);
     ASCQ_REQUIRE(d->bias_kind >= ASCQ_MM_BIAS_NONE && d->bias_kind <= ASCQ_MM_BIAS_BF16_POST, ASCQ_EINVAL,
                  "%s: unknown bias kind %d", who, d->bias_kind);
-    ASCQ_REQUIRE(d->activation == ASCQ_MM_ACT_NONE || d->activation == ASCQ_MM_ACT_FASTER_GELU, ASCQ_EINVAL,
+    ASCQ_REQUIRE(d->activation >= ASCQ_MM_ACT_NONE && d->activation <= ASCQ_MM_ACT_SWIGLU, ASCQ_EINVAL,
                  "%s: unknown activation %d", who, d->activation);
+    if (d->activation == ASCQ_MM_ACT_SWIGLU) {
+        ASCQ_REQUIRE(d->n % 2 == 0, ASCQ_EINVAL, "%s: SwiGLU combines column pairs: n = %u must be even", who, d->n);
+        ASCQ_REQUIRE(d->quant_mode != ASCQ_MM_QUANT_NONE &&
+                         (d->out_dtype == ASCQ_F16 || d->out_dtype == ASCQ_BF16 || d->out_dtype == ASCQ_F32),
+                     ASCQ_EUNSUPPORTED, "%s: SwiGLU needs a dequantising epilogue and a half / bfloat16 / float output", who);
+        ASCQ_REQUIRE(d->act_beta == d->act_beta && d->act_beta - d->act_beta == 0.0f, ASCQ_EINVAL,
+                     "%s: act_beta must be finite", who);
+    }
     ASCQ_REQUIRE(d->b_format == ASCQ_MM_B_ND || d->b_format == ASCQ_MM_B_NZ, ASCQ_EINVAL, "%s: unknown B format %d",
                  who, d->b_format);
     if (d->b_format == ASCQ_MM_B_NZ) {
@@ -537,8 +545,10 @@ int validate_mm(const ascq_matmul_desc* d, const char* who, const void* c, const
 
 EpiParams make_epi(const ascq_matmul_desc* d, void* c, const void* bias, const void* qv, const void* tok)
 {
-    return EpiParams{c, bias, qv, static_cast<const float*>(tok), d->n, d->out_dtype, d->quant_mode, d->scale_format,
-                     d->bias_kind, d->has_tok_scale, d->activation, d->quant_scalar};
+    // the SwiGLU epilogue writes one column per column pair
+    const uint32_t ldc = d->activation == ASCQ_MM_ACT_SWIGLU && d->quant_mode != ASCQ_MM_QUANT_NONE ? d->n / 2u : d->n;
+    return EpiParams{c, bias, qv, static_cast<const float*>(tok), ldc, d->out_dtype, d->quant_mode, d->scale_format,
+                     d->bias_kind, d->has_tok_scale, d->activation, d->quant_scalar, d->act_beta};
 }
 
 bool fast_path_ok(const ascq_matmul_desc* d, const void* a, const void* b)
@@ -566,6 +576,51 @@ uint32_t pick_k_splits(uint32_t n, uint32_t k)
     return s ? s : 1u;
 }
 
+// SwiGLU for the shapes the large tile kernel does not take: the matmul leaves its int32 accumulators in the workspace
+// ([m][n], pre-dequant bias included) and this kernel applies scale, token scale, bias and the activation to each
+// column pair.  One lane = one pair.
+__global__ __launch_bounds__(256) void swiglu_epilogue_kernel(GemmParams p)
+{
+    const EpiParams& e = p.epi;
+    const size_t half_n = p.n / 2u, total = static_cast<size_t>(p.m) * half_n;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * 256u + threadIdx.x; i < total;
+         i += static_cast<size_t>(gridDim.x) * 256u) {
+        const size_t row = i / half_n, jp = i % half_n, col = 2u * jp;
+        const int32_t a0 = p.partial[row * p.n + col], a1 = p.partial[row * p.n + col + 1u];
+        const float tok = e.has_tok ? e.tok_scale[row] : 1.0f;
+        const float v0 = epilogue_value(e, a0, load_channel_q(e, col), tok, load_bias_post(e, col));
+        const float v1 = epilogue_value(e, a1, load_channel_q(e, col + 1u), tok, load_bias_post(e, col + 1u));
+        store_float_out(e, row * e.ldc + jp, swiglu(v0, v1, e.act_beta));
+    }
+}
+
+// True when the plain matmul of this descriptor runs on the large direct-to-LDS tile kernel, whose epilogue applies
+// SwiGLU in registers (16-bit outputs).
+bool swiglu_in_tile_kernel(const ascq_matmul_desc* d, const GemmParams& p, const void* a, const void* b)
+{
+    if (d->out_dtype != ASCQ_F16 && d->out_dtype != ASCQ_BF16) {
+        return false;
+    }
+    if (d->m <= kSkinnyMaxM || !gemm_dma_supported(p)) {
+        return false;
+    }
+    return d->b_format == ASCQ_MM_B_NZ || fast_path_ok(d, a, b);
+}
+
+inline size_t round256(size_t v) { return (v + 255u) & ~static_cast<size_t>(255u); }
+
+// the matmul that leaves raw accumulators: same operands, no quantisation, at most the pre-dequant bias
+ascq_matmul_desc raw_accumulator_desc(const ascq_matmul_desc* d)
+{
+    ascq_matmul_desc r = *d;
+    r.quant_mode = ASCQ_MM_QUANT_NONE;
+    r.out_dtype = ASCQ_I32;
+    r.activation = ASCQ_MM_ACT_NONE;
+    r.has_tok_scale = 0;
+    r.bias_kind = d->bias_kind == ASCQ_MM_BIAS_I32_PRE ? ASCQ_MM_BIAS_I32_PRE : ASCQ_MM_BIAS_NONE;
+    return r;
+}
+
 }  // namespace
 }  // namespace ascq
 
@@ -575,6 +630,18 @@ extern "C" int ascq_matmul_w8a8_workspace_size(const ascq_matmul_desc* d, size_t
 {
     ASCQ_REQUIRE(d != nullptr && bytes != nullptr, ASCQ_ENULL, "ascq_matmul_w8a8_workspace_size: NULL argument");
     *bytes = 0;
+    if (d->activation == ASCQ_MM_ACT_SWIGLU && d->quant_mode != ASCQ_MM_QUANT_NONE) {
+        // Shapes outside the large tile kernel keep their int32 accumulators [m][n] in the workspace, behind the
+        // scratch of the matmul that produces them.  (The size does not depend on the pointers: it is the bound.)
+        const ascq_matmul_desc r = raw_accumulator_desc(d);
+        size_t inner = 0;
+        const int rc = ascq_matmul_w8a8_workspace_size(&r, &inner);
+        if (rc != ASCQ_OK) {
+            return rc;
+        }
+        *bytes = round256(inner) + static_cast<size_t>(d->m) * d->n * sizeof(int32_t);
+        return ASCQ_OK;
+    }
     if (d->m <= 32 && !d->trans_a && pick_k_splits(d->n, d->k) > 1) {
         *bytes = static_cast<size_t>(d->m) * d->n * sizeof(int32_t);
     }
@@ -612,6 +679,35 @@ extern "C" int ascq_matmul_w8a8(const ascq_matmul_desc* d, void* c, const void* 
     p.n = d->n;
     p.k = d->k;
     p.epi = make_epi(d, c, bias, quant_vector, tok_scale);
+    if (d->activation == ASCQ_MM_ACT_SWIGLU && !swiglu_in_tile_kernel(d, p, a, b)) {
+        // raw accumulators into the workspace, then the pairwise epilogue
+        const ascq_matmul_desc r = raw_accumulator_desc(d);
+        size_t inner = 0;
+        rc = ascq_matmul_w8a8_workspace_size(&r, &inner);
+        if (rc != ASCQ_OK) {
+            return rc;
+        }
+        inner = round256(inner);
+        const size_t need = inner + static_cast<size_t>(d->m) * d->n * sizeof(int32_t);
+        ASCQ_REQUIRE(workspace != nullptr && workspace_bytes >= need, ASCQ_EINVAL,
+                     "ascq_matmul_w8a8: SwiGLU at this shape needs a workspace of %zu bytes (see "
+                     "ascq_matmul_w8a8_workspace_size)", need);
+        ASCQ_REQUIRE(aligned16(workspace), ASCQ_EALIGN, "ascq_matmul_w8a8: workspace must be 16-byte aligned");
+        p.partial = reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + inner);
+        rc = ascq_matmul_w8a8(&r, p.partial, a, b, r.bias_kind == ASCQ_MM_BIAS_I32_PRE ? bias : nullptr, nullptr, nullptr,
+                              inner ? workspace : nullptr, inner, stream);
+        if (rc != ASCQ_OK) {
+            return rc;
+        }
+        const size_t pairs = static_cast<size_t>(d->m) * (d->n / 2u);
+        size_t blocks = (pairs + 255u) / 256u;
+        if (blocks > 8192) blocks = 8192;
+        if (plan_note(0, 0, 0, 0, 0, 0, 0, 0)) {  // the pairwise epilogue kernel
+            return ASCQ_OK;
+        }
+        swiglu_epilogue_kernel<<<static_cast<uint32_t>(blocks), 256, 0, st>>>(p);
+        return launch_status("ascq_matmul_w8a8 (SwiGLU epilogue)");
+    }
     if (d->b_format == ASCQ_MM_B_NZ) {
         // only the direct-to-LDS tile kernels address the fractal layout; validate_mm has checked what they need
         p.b_nz = 1;
@@ -693,10 +789,6 @@ extern "C" int ascq_matmul_w8a8_plan(const ascq_matmul_desc* d, const void* c, c
 }
 
 // ---------------------------------------------------------------------------- fused dynamic quantisation + matmul
-namespace {
-inline size_t round256(size_t v) { return (v + 255u) & ~static_cast<size_t>(255u); }
-}  // namespace
-
 extern "C" int ascq_linear_w8a8_dynamic_workspace_size(const ascq_matmul_desc* d, size_t* bytes)
 {
     ASCQ_REQUIRE(d != nullptr && bytes != nullptr, ASCQ_ENULL, "ascq_linear_w8a8_dynamic_workspace_size: NULL argument");
@@ -976,10 +1068,14 @@ extern "C" int ascq_group_matmul_w8a8(const ascq_group_matmul_desc* g, void* y, 
     p.group_list_kind = g->group_list_kind;
     p.epi = make_epi(d, y, bias, scale, tok_scale);
     p.b_nz = d->b_format == ASCQ_MM_B_NZ ? 1u : 0u;
+    ASCQ_REQUIRE(d->activation != ASCQ_MM_ACT_SWIGLU || d->out_dtype == ASCQ_F16 || d->out_dtype == ASCQ_BF16,
+                 ASCQ_EUNSUPPORTED, "ascq_group_matmul_w8a8: SwiGLU writes half or bfloat16 here");
     if (gemm_dma_supported(p)) {
         return launch_gemm_dma(p, true, st);
     }
     ASCQ_REQUIRE(!p.b_nz, ASCQ_EUNSUPPORTED, "ascq_group_matmul_w8a8: fractal (NZ) weights need the tile kernel's shape");
+    ASCQ_REQUIRE(d->activation != ASCQ_MM_ACT_SWIGLU, ASCQ_EUNSUPPORTED,
+                 "ascq_group_matmul_w8a8: SwiGLU needs the tile kernel's shape (k %% 128 == 0, n %% 16 == 0)");
     typedef TileL T;
     // every group adds at most one partial tile along M
     p.tiles_m = (d->m + T::BM - 1) / T::BM + g->groups;

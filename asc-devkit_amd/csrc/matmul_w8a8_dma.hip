@@ -432,11 +432,13 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_
         }
         // The uniform choices (post-dequant bias, activation) are made once, outside the element loops, so that each
         // wavefront runs one compact straight-line epilogue.
-        auto store_all = [&](auto bias_tag, auto gelu_tag) {
+        auto store_all = [&](auto bias_tag, auto gelu_tag, auto swiglu_tag) {
             constexpr bool kBiasPost = decltype(bias_tag)::value;
             constexpr bool kGelu = decltype(gelu_tag)::value;
+            constexpr bool kSwiGlu = decltype(swiglu_tag)::value;
             (void)kBiasPost;
             (void)kGelu;
+            (void)kSwiGlu;
     #pragma unroll
             for (int i = 0; i < TI; ++i) {
                 const uint32_t lbase = (wm * TI + i) * 32u + 4u * g;  // row inside the tile of register 0
@@ -452,6 +454,25 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_
                             // (l, l+1) of the first 32-column block, odd lanes columns (l-1, l) of the second one.
                             static_assert(TJ == 2, "the paired store assumes two column blocks per wavefront");
                             const bool odd = (lane & 1u) != 0;
+                            if constexpr (kSwiGlu) {
+                                // Adjacent lanes hold the two columns of a pair.  After one lane swap the even lane
+                                // owns the pair of the first 32-column block (src0 its own value, src1 its
+                                // neighbour's), the odd lane the pair of the second block (src0 its neighbour's).
+                                const float v0 = epi_value<kBiasPost, false>(acc[i][0][r] + bias_pre[0], q[0].s, tok4[rr],
+                                                                             bias_post[0]);
+                                const float v1 = epi_value<kBiasPost, false>(acc[i][1][r] + bias_pre[1], q[1].s, tok4[rr],
+                                                                             bias_post[1]);
+                                const float recv = __int_as_float(__builtin_amdgcn_mov_dpp(
+                                    __float_as_int(odd ? v0 : v1), 0xB1, 0xF, 0xF, true));  // lane ^ 1
+                                const float o = swiglu(odd ? recv : v0, odd ? v1 : recv, e.act_beta);
+                                const uint32_t col = odd ? colw + 32u + (lrow - 1u) : colw + lrow;  // first column of the pair
+                                if (row < row_end && col < N) {
+                                    __builtin_nontemporal_store(
+                                        static_cast<uint16_t>(to_bits16<kOut>(o)),
+                                        static_cast<uint16_t*>(e.c) + static_cast<size_t>(row) * e.ldc + (col >> 1));
+                                }
+                                continue;
+                            }
                             const uint32_t h0 =
                                 to_bits16<kOut>(
                                     epi_value<kBiasPost, kGelu>(acc[i][0][r] + bias_pre[0], q[0].s, tok4[rr], bias_post[0]));
@@ -484,19 +505,26 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_
         if constexpr (kOut == ASCQ_BF16 || kOut == ASCQ_F16) {
             const bool bias_post_on = e.bias_kind >= ASCQ_MM_BIAS_F32_POST;
             const bool gelu_on = e.activation == ASCQ_MM_ACT_FASTER_GELU;
-            if (gelu_on) {
+            if (e.activation == ASCQ_MM_ACT_SWIGLU) {
                 if (bias_post_on) {
-                    store_all(std::true_type{}, std::true_type{});
+                    store_all(std::true_type{}, std::false_type{}, std::true_type{});
                 } else {
-                    store_all(std::false_type{}, std::true_type{});
+                    store_all(std::false_type{}, std::false_type{}, std::true_type{});
+                }
+            } else if (gelu_on) {
+                if (bias_post_on) {
+                    store_all(std::true_type{}, std::true_type{}, std::false_type{});
+                } else {
+                    store_all(std::false_type{}, std::true_type{}, std::false_type{});
                 }
             } else if (bias_post_on) {
-                store_all(std::true_type{}, std::false_type{});
+                store_all(std::true_type{}, std::false_type{}, std::false_type{});
             } else {
-                store_all(std::false_type{}, std::false_type{});
+                store_all(std::false_type{}, std::false_type{}, std::false_type{});
             }
         } else {
-            store_all(std::false_type{}, std::false_type{});  // the generic store reads both choices at run time
+            // the generic store reads both choices at run time (the host sends SwiGLU with these outputs elsewhere)
+            store_all(std::false_type{}, std::false_type{}, std::false_type{});
         }
     };
     dispatch_out(e, run);

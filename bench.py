@@ -15,7 +15,14 @@ The default of 1000 timed steps after 100 warm-up steps keeps the GPU busy for a
 clocks take a few milliseconds of load to reach their sustained state: a 50-step region (6 ms) measured 124 us per
 step and 108 us per GEMM, a 1000-step region 102-106 us per step and 95 us per GEMM, on the same box minutes apart.
 For the same reason `--settle` untimed steps (300, about 30 ms; reported as config.settle_steps) run before the W
-warm-up steps of the headline, so that a caller's short --steps/--warmup is measured at the sustained clock as well.
+warm-up steps of every workload, the headline and the others alike, so that a caller's short --steps/--warmup is
+measured at the sustained clock as well; the workloads under "others" time at least 100 steps.
+
+Besides the workloads the line carries "ceilings": the figures the stand-alone program asc-devkit_amd/lib/machine_probe
+measures on this GPU in the same run (matrix-pipe rate with constant and with random int8 operands and the shader clock
+during each, HBM copy / read / fill, LDS read rate), and "roofline.same_kernel_zero_operands": the headline GEMM
+launched on all-zero operands, which shows what the same instruction stream reaches when the operands do not toggle
+the multipliers (the power management then leaves the clock at its maximum).
 """
 import argparse
 import json
@@ -35,7 +42,8 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E peak, GB/s
 # (FETCH_SIZE reads 0.5 per KiB there, WRITE_SIZE 1.0 per KiB).  Measured offline and recorded here; a run of this
 # file does not re-measure them.
 GEMM_TRAFFIC_BYTES = 228293837   # M=2048 GEMM, both tile shapes: 183.2 MB fetched + 45.1 MB written
-GEMV_TRAFFIC_BYTES = 133853594   # W4A16 M=1 GEMV, stream + sum kernels: 129.5 MB fetched + 4.3 MB written
+GEMV_TRAFFIC_BYTES = 133853594   # W4A16 M=1 GEMV, [k, n / 2] layout, stream + sum kernels: 129.5 MB fetched + 4.3 MB written
+GEMV_PACKED_TRAFFIC_BYTES = None  # W4A16 M=1 GEMV on packed weights: not measured yet
 
 
 def main():
@@ -48,7 +56,9 @@ def main():
                          "runs are also measured at the sustained clock (0 disables)")
     ap.add_argument("--quick", action="store_true", help="headline + W4A16 GEMV only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="run a single workload: w8a8 | w4a16 | quant | dequant | antiquant | group")
+    ap.add_argument("--only", default="", help="run a single workload: w8a8 | w4a16 | w4a16_nd | w4a16_m4 | w4a16_m16 | w4a16_nd_m4 | w4a16_nd_m16 | "
+                         "w8a8_m1 | w8a8_m16 | w8a8_m128 | w8a16_m1 | w8a16_m16 | quant | dequant | antiquant | group | "
+                         "group_example (a W4A16 name without _nd is the packed-weight path)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch one device-to-device copy of 1 GiB: the known-size kernel that calibrates the "
                          "FETCH_SIZE / WRITE_SIZE counters when this command runs under rocprofv3 --pmc")
@@ -76,11 +86,13 @@ def main():
     def rand_i8(*shape):
         return torch.randint(-127, 128, shape, dtype=torch.int8, device=dev, generator=gen)
 
-    def timed(fn, steps, warmup, inner=None):
-        """Times `steps` calls of fn(i, None, None) after `warmup` by the host clock between two synchronizes, then
-        the same `steps` calls again between one pair of events on the launch stream.  Returns (ms per step by the
-        host clock, ms per step by the events).  No event is recorded inside either region: a record between two
-        launches idles the queue for 3-6 us, which is a tenth of a 35 us decode step."""
+    def timed(fn, steps, warmup, settle=None):
+        """Times `steps` calls of fn(i, None, None) after `settle` + `warmup` untimed ones by the host clock between two
+        synchronizes, then the same `steps` calls again between one pair of events on the launch stream.  Returns (ms
+        per step by the host clock, ms per step by the events).  No event is recorded inside either region: a record
+        between two launches idles the queue for 3-6 us, which is a tenth of a 35 us decode step."""
+        for i in range(args.settle if settle is None else settle):
+            fn(i, None, None)
         for i in range(warmup):
             fn(i, None, None)
         torch.cuda.synchronize()
@@ -117,12 +129,16 @@ def main():
         torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------ W8A8 linear (config 3)
-    def w8a8(M, steps, warmup, sets=1, settle=0):
+    def w8a8(M, steps, warmup, sets=1, settle=None, zero=False):
         """`sets` > 1 rotates the weights over several copies (together larger than the Infinity Cache) so that the
         weight-bound small-M cases read them from HBM."""
         K, N = 4096, 11008
         x = torch.randn((M, K), device=dev, generator=gen).to(torch.bfloat16)
         ws = [rand_i8(K, N) for _ in range(sets)]
+        if zero:          # all-zero activations and weights: the same launches, nothing toggles in the multipliers
+            x.zero_()
+            for wj in ws:
+                wj.zero_()
         w = ws[0]
         cs = torch.rand(N, device=dev, generator=gen) * (1e-2 - 1e-4) + 1e-4
         q = torch.empty((M, K), dtype=torch.int8, device=dev)
@@ -143,9 +159,7 @@ def main():
 
         # The timed region proper is quant + GEMM per step.  Then the GEMM launches of the same steps run back to
         # back between one pair of events on the launch stream, which gives the average duration of the GEMM launch.
-        for i in range(settle):
-            step(i, None, None)
-        ms, _ = timed(lambda i, a, b: step(i, None, None), steps, warmup)
+        ms, _ = timed(lambda i, a, b: step(i, None, None), steps, warmup, settle)
         ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         ev0.record()
@@ -174,17 +188,23 @@ def main():
                 "ops": flops, "bytes": bytes_, "tensors": (x, w, cs)}
 
     # ------------------------------------------------------------------ W4A16 decode (config 4)
-    def w4a16(M, steps, warmup, sets=4):
+    def w4a16(M, steps, warmup, sets=4, packed=False):
+        """packed: the weights in the layout of ascq_pack_weight_w4 (packed once, outside the timed region) and the
+        one-launch kernel; otherwise the [k, n / 2] layout and the stream + sum kernels."""
         K, N, gs = 8192, 28672, 128
         xs = torch.randn((M, K), device=dev, generator=gen).to(torch.float16)
         ws = [torch.randint(0, 256, (K, N // 2), dtype=torch.uint8, device=dev, generator=gen) for _ in range(sets)]
         sc = [(torch.rand((K // gs, N), device=dev, generator=gen) * 9e-3 + 1e-3).to(torch.float16) for _ in range(sets)]
         of = [torch.randint(-8, 8, (K // gs, N), device=dev, generator=gen).to(torch.float16) for _ in range(sets)]
         y = torch.empty((M, N), dtype=torch.float16, device=dev)
+        wps = [ops.pack_weight_w4(w, K, N) for w in ws] if packed else None
 
         def step(i, starts, stops):
             j = i % sets
-            bracket(starts, stops, lambda: ops.matmul_w4a16(y, xs, ws[j], sc[j], of[j], gs))
+            if packed:
+                bracket(starts, stops, lambda: ops.matmul_w4a16_packed(y, xs, wps[j], sc[j], of[j], gs))
+            else:
+                bracket(starts, stops, lambda: ops.matmul_w4a16(y, xs, ws[j], sc[j], of[j], gs))
 
         ms, kern_ms = timed(step, steps, warmup)
         bytes_ = K * N // 2 + 2 * (K // gs) * N * 2 + M * K * 2 + M * N * 2
@@ -276,12 +296,59 @@ def main():
         return {"kernel_ms": kern_ms, "tops": flops / (kern_ms * 1e-3) / 1e12, "gbs": bytes_ / (kern_ms * 1e-3) / 1e9,
                 "ops": flops, "bytes": bytes_}
 
+    def group_example(steps, warmup):
+        """The reference example's own shape and options (quant_group_matmul_high_performance: 8 groups x 1024 tokens,
+        k = 1024, n = 8192, weights in the fractal NZ layout, FasterGelu, fp16 output; data as its gen_data.py draws
+        them).  Its README reports 204.129 us and mac_ratio 0.887 on an Ascend 950PR (context only)."""
+        G, T, K, N = 8, 8192, 1024, 8192
+        gl = torch.full((G,), T // G, dtype=torch.int64, device=dev)
+        x = torch.randint(-10, 10, (T, K), dtype=torch.int8, device=dev, generator=gen)
+        w = ops.pack_weight_nz(torch.randint(-10, 10, (G, K, N), dtype=torch.int8, device=dev, generator=gen))
+        cs = torch.randn((G, N), device=dev, generator=gen) * 0.01
+        ts = torch.randn(T, device=dev, generator=gen) * 0.01
+        y = torch.empty((T, N), dtype=torch.float16, device=dev)
+
+        def step(i, starts, stops):
+            bracket(starts, stops, lambda: ops.quant_group_matmul(y, x, w, gl, cs, ts, None, abi.GROUP_LIST_COUNTS,
+                                                                  abi.MM_ACT_FASTER_GELU, True))
+
+        ms, kern_ms = timed(step, steps, warmup)
+        flops = 2.0 * T * K * N
+        bytes_ = T * K + G * K * N + G * N * 4 + T * 4 + T * N * 2 + G * 8
+        return {"kernel_ms": kern_ms, "tops": flops / (kern_ms * 1e-3) / 1e12, "gbs": bytes_ / (kern_ms * 1e-3) / 1e9,
+                "ops": flops, "bytes": bytes_, "reference_published_us_ascend_950pr": 204.129,
+                "reference_published_mac_ratio": 0.887}
+
     def strip(d):
         return {k: v for k, v in d.items() if k != "tensors"}
 
+    def machine_ceilings():
+        """Runs the stand-alone probe (its own process, before this one launches anything large) and returns its JSON."""
+        import subprocess
+        exe = os.path.join(ROOT, "asc-devkit_amd", "lib", "machine_probe")
+        if not os.path.exists(exe):
+            return {"error": "asc-devkit_amd/lib/machine_probe is not built"}
+        try:
+            r = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+            return json.loads(r.stdout) if r.returncode == 0 else {"error": r.stderr.strip()[-200:]}
+        except Exception as e:     # the probe is evidence, not part of the measurement: report and go on
+            return {"error": str(e)}
+
+    ceilings = None if args.quick or args.only else machine_ceilings()
     only = args.only
     if only and only != "w8a8":
-        fn = {"w4a16": lambda: w4a16(1, args.steps, args.warmup), "quant": lambda: quant2a(args.steps, args.warmup),
+        fn = {"w4a16": lambda: w4a16(1, args.steps, args.warmup, packed=True),
+              "w4a16_nd": lambda: w4a16(1, args.steps, args.warmup),
+              "group_example": lambda: group_example(args.steps, args.warmup),
+              "w4a16_m4": lambda: w4a16(4, args.steps, args.warmup, packed=True),
+              "w4a16_m16": lambda: w4a16(16, args.steps, args.warmup, packed=True),
+              "w4a16_nd_m4": lambda: w4a16(4, args.steps, args.warmup),
+              "w4a16_nd_m16": lambda: w4a16(16, args.steps, args.warmup),
+              "w8a8_m1": lambda: w8a8(1, args.steps, args.warmup, sets=7),
+              "w8a8_m16": lambda: w8a8(16, args.steps, args.warmup, sets=7),
+              "w8a8_m128": lambda: w8a8(128, args.steps, args.warmup, sets=7),
+              "w8a16_m1": lambda: w8a16(1, args.steps, args.warmup),
+              "w8a16_m16": lambda: w8a16(16, args.steps, args.warmup), "quant": lambda: quant2a(args.steps, args.warmup),
               "dequant": lambda: dequant2b(args.steps, args.warmup),
               "antiquant": lambda: antiquant2c(args.steps, args.warmup),
               "group": lambda: group5(args.steps, args.warmup)}[only]
@@ -322,21 +389,39 @@ def main():
     if only == "w8a8":
         print(json.dumps(out))
         return
+    if not args.quick:
+        z = w8a8(2048, min(args.steps, 300), min(args.warmup, 50), zero=True)
+        out["roofline"]["same_kernel_zero_operands"] = {
+            "avg_kernel_ms": z["gemm_kernel_ms"], "achieved": z["gemm_tops"], "frac": z["gemm_tops"] / PEAK_INT8_TOPS,
+            "note": "the same GEMM launches on all-zero activations and weights: the instruction stream, tiling and "
+                    "memory traffic are those of the headline, only the operand values differ"}
+        del z
+        torch.cuda.empty_cache()
+    if ceilings is not None:
+        out["ceilings"] = ceilings
 
     # The other workloads run a bounded number of steps so that the whole file finishes in about a minute.
-    side_steps, side_warmup = min(args.steps, 500), min(args.warmup, 50)
-    gemv = w4a16(1, side_steps, side_warmup)
+    side_steps, side_warmup = max(100, min(args.steps, 500)), min(args.warmup, 50)
+    gemv = w4a16(1, side_steps, side_warmup, packed=True)
+    gemv_nd = w4a16(1, side_steps, side_warmup)
     out["w4a16_gemv"] = {"metric": "w4a16_decode_gemv_hbm_gbs_m1_k8192_n28672", "value": gemv["gbs"], "unit": "GB/s",
-                         "workload": "BASELINE configs[3] at M=1, 4 rotating weight sets (500 MB > Infinity Cache)",
+                         "workload": "BASELINE configs[3] at M=1, weights pre-packed by ascq_pack_weight_w4 (outside "
+                                     "the timed region), 4 rotating weight sets (500 MB > Infinity Cache)",
                          "ms_per_step": gemv["ms_per_step"],
-                         "roofline": {"bound": "hbm", "kernel": "w4a16_gemv_kernel<1, offset> + stream_sum_kernel<1>",
+                         "roofline": {"bound": "hbm", "kernel": "w4a16_packed_kernel<offset, 8, 8> (one launch)",
                                       "achieved": gemv["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                      "frac": gemv["gbs"] / PEAK_HBM_GBS, "traffic": GEMV_TRAFFIC_BYTES,
-                                      "avg_kernel_ms": gemv["kernel_ms"], "bytes_per_launch": gemv["bytes"]}}
+                                      "frac": gemv["gbs"] / PEAK_HBM_GBS, "traffic": GEMV_PACKED_TRAFFIC_BYTES,
+                                      "avg_kernel_ms": gemv["kernel_ms"], "bytes_per_launch": gemv["bytes"]},
+                         "nd_layout": {"kernel": "w4a16_gemv_kernel<1, offset> + stream_sum_kernel<1>",
+                                       "workload": "the same GEMV on the reference's [k, n / 2] weight layout",
+                                       "avg_kernel_ms": gemv_nd["kernel_ms"], "gbs": gemv_nd["gbs"],
+                                       "hbm_frac": gemv_nd["gbs"] / PEAK_HBM_GBS, "traffic": GEMV_TRAFFIC_BYTES}}
+    del gemv_nd
+    torch.cuda.empty_cache()
 
     if not args.quick:
         others = {}
-        s2, w2 = max(10, side_steps // 2), max(3, side_warmup // 2)
+        s2, w2 = max(100, side_steps // 2), max(3, side_warmup // 2)
         for name, fn in (("quant_2a", lambda: quant2a(s2, w2)), ("dequant_2b", lambda: dequant2b(s2, w2)),
                          ("antiquant_2c", lambda: antiquant2c(s2, w2))):
             r = strip(fn())
@@ -352,15 +437,24 @@ def main():
             r = strip(w4a16(M, s2, w2))
             others[f"w4a16_m{M}"] = {"kernel_ms": r["kernel_ms"], "gbs": r["gbs"], "hbm_frac": r["gbs"] / PEAK_HBM_GBS}
             torch.cuda.empty_cache()
+            r = strip(w4a16(M, s2, w2, packed=True))
+            others[f"w4a16_packed_m{M}"] = {"kernel_ms": r["kernel_ms"], "gbs": r["gbs"],
+                                            "hbm_frac": r["gbs"] / PEAK_HBM_GBS}
+            torch.cuda.empty_cache()
         for M in (1, 16):
             r = w8a16(M, s2, w2)
             others[f"w8a16_m{M}_k8192_n28672"] = {"kernel_ms": r["kernel_ms"], "gbs": r["gbs"], "bytes": r["bytes"],
                                                   "hbm_frac": r["gbs"] / PEAK_HBM_GBS}
             torch.cuda.empty_cache()
-        r = group5(max(5, side_steps // 5), 2)
+        r = group5(max(20, side_steps // 5), 5)
         r["mfma_frac"] = r["tops"] / PEAK_INT8_TOPS
         r["hbm_frac"] = r["gbs"] / PEAK_HBM_GBS
         others["group_matmul_config5"] = r
+        torch.cuda.empty_cache()
+        r = group_example(max(20, side_steps // 5), 5)
+        r["mfma_frac"] = r["tops"] / PEAK_INT8_TOPS
+        others["group_matmul_reference_example"] = r
+        torch.cuda.empty_cache()
         out["others"] = others
 
     # ------------------------------------------------------------------ CPU baseline (the oracle; a checker being timed)
@@ -381,10 +475,28 @@ def main():
             dt = time.perf_counter() - t0
             if dt >= 12.0 or reps >= 64:
                 break
+        cpu_model = "unknown"
+        try:
+            with open("/proc/cpuinfo") as f:
+                cpu_model = next((ln.split(":", 1)[1].strip() for ln in f if ln.startswith("model name")), "unknown")
+        except OSError:
+            pass
         out["cpu_baseline"] = {"value": reps * 2.0 * 2048 * 4096 * 11008 / dt / 1e12, "unit": "TOPS", "cores": cores,
-                               "kind": "port",
+                               "kind": "port", "cpu_model": cpu_model,
+                               "label": "CPU restatement of asc-devkit semantics (oracle/), not the reference's CPU-debug build",
                                "sample": f"{reps} whole steps of the same workload (per-token quant + int8 GEMM + "
                                          f"epilogue, all 2048 rows) in {dt:.2f} s, OpenMP over rows"}
+        # the same on one thread, on a row sample: 256 of the 2048 rows (the work is independent per row)
+        orc.set_threads(1)
+        d1 = abi.MatmulDesc(m=256, n=11008, k=4096, out_dtype=abi.BF16, quant_mode=abi.MM_QUANT_VECTOR,
+                            scale_format=abi.MM_SCALE_F32, has_tok_scale=1)
+        t0 = time.perf_counter()
+        q1, ts1 = orc.dynamic_quant_per_token(abi.BF16, xb[:256])
+        orc.matmul_w8a8(d1, q1, wn, None, csn, ts1)
+        dt1 = time.perf_counter() - t0
+        out["cpu_baseline"]["single_thread"] = {"value": 2.0 * 256 * 4096 * 11008 / dt1 / 1e12, "unit": "TOPS", "cores": 1,
+                                                "sample": f"rows 0..255 of the same step (an eighth of it) in {dt1:.2f} s"}
+        orc.set_threads(cores)
         xs, w4, sc4, of4 = gemv["tensors"]
         d4 = abi.W4A16Desc(m=1, n=28672, k=8192, group_size=128, has_offset=1)
         a4 = (xs.cpu().numpy(), w4.cpu().numpy(), sc4.cpu().numpy(), of4.cpu().numpy())
@@ -396,7 +508,7 @@ def main():
             if dt >= 6.0 or reps >= 64:
                 break
         out["w4a16_gemv"]["cpu_baseline"] = {"value": reps * gemv["bytes"] / dt / 1e9, "unit": "GB/s",
-                                             "cores": cores, "kind": "port",
+                                             "cores": cores, "kind": "port", "cpu_model": cpu_model,
                                              "sample": f"{reps} whole GEMVs (all 28672 columns) in {dt:.2f} s"}
     print(json.dumps(out))
 

@@ -294,7 +294,15 @@ typedef enum ascq_mm_bias_kind {
 
 typedef enum ascq_mm_activation {
     ASCQ_MM_ACT_NONE = 0,
-    ASCQ_MM_ACT_FASTER_GELU = 1 /* x*exp(0.851(x-|x|))/(1+exp(-1.702|x|)) (ref: examples/.../quant_group_matmul_high_performance/scripts/gen_data.py:19-23) */
+    ASCQ_MM_ACT_FASTER_GELU = 1, /* x*exp(0.851(x-|x|))/(1+exp(-1.702|x|)) (ref: examples/.../quant_group_matmul_high_performance/scripts/gen_data.py:19-23) */
+    /* SwiGLU over interleaved column pairs: column 2j of the matmul is src0, column 2j + 1 is src1, and output
+       column j (C is [m, n / 2]) is src0 * swish(src1) with swish(x) = x / (1 + exp(-beta x)), computed in fp32 in
+       the reference's order: t = x * (-beta); e = exp(t); d = e + 1; s = x / d; out = src0 * s, one rounding each
+       (ref: impl/adv_api/detail/activation/swiglu/swiglu_common_impl.h:154-190; golden
+       examples/.../01_activation/swiglu/scripts/gen_data.py:32).  n must be even, the output floating point
+       (F16 / BF16 / F32); beta is ascq_matmul_desc.act_beta.  A gate / up projection whose weight columns are
+       stored interleaved (up_0, gate_0, up_1, gate_1, ...) produces silu(gate) * up directly with beta = 1. */
+    ASCQ_MM_ACT_SWIGLU = 2
 } ascq_mm_activation;
 
 /*
@@ -304,6 +312,7 @@ typedef enum ascq_mm_activation {
  *   acc[i,j] = sum_k A[i,k]*B[k,j] (+ bias_i32[j])                          exact int32
  *   QUANT_NONE: C int32 = acc.
  *   else v = f32(acc) * s_j  [* tok_scale[i]]  [+ bias_post[j]]  [act]      one fp32 rounding per op
+ *        (ASCQ_MM_ACT_SWIGLU combines the v of columns 2j and 2j + 1 into output column j: C is [m, n / 2])
  *        C = F16: f16(v) saturated to +-65504;  BF16: bf16 rne;  F32: v;
  *            I8 (U64 format only): sat( sat9(rint(v)) + offset9 ), offset9 = bits[45:37] taken as unsigned,
  *            saturating to int8 when bit 46 is set and to uint8 otherwise.
@@ -323,6 +332,8 @@ typedef struct ascq_matmul_desc {
                               gen_data_s322f16.py:48-58,84-90) is rejected with ASCQ_EUNSUPPORTED; words of a quant
                               vector live on the device and are not inspected: bit 36 and the shift are outside the
                               supported domain there */
+    float act_beta;        /* ASCQ_MM_ACT_SWIGLU: the constant of the swish function (1 = SiLU); ignored otherwise */
+    int32_t reserved;      /* set to 0 */
 } ascq_matmul_desc;
 
 int ascq_matmul_w8a8(const ascq_matmul_desc* desc, void* c, const void* a, const void* b, const void* bias,

@@ -681,6 +681,14 @@ public:
         tok_ = tokScale.GetPhyAddr();
         desc_.has_tok_scale = 1;
     }
+    // Fused activation of the dequantised result (no reference counterpart on the Matmul object: the reference applies
+    // FasterGelu / SwiGLU as separate vector operators, gelu_impl.h:140-143, swiglu_common_impl.h:154-190).
+    // ASCQ_MM_ACT_SWIGLU: columns 2j / 2j + 1 of the product are src0 / src1 and C is [m, n / 2].
+    void SetActivation(ascq_mm_activation activation, float beta = 1.0f)
+    {
+        desc_.activation = activation;
+        desc_.act_beta = beta;
+    }
     void SetWorkspace(void* workspace, size_t bytes)
     {
         workspace_ = workspace;

@@ -617,13 +617,10 @@ float orc_quant_word_scale(uint64_t w, int scale_format)
  *      fixpipe_l0c2gm/scripts/gen_data_s322f16.py:76-102 (deqf16: fp32 multiply, saturate to the fp16 range),
  *      gen_data_s322s8.py:76-97 (req8: round, saturate to 9 bits, add offset, saturate to 8 bits),
  *      quant_group_matmul_custom.asc:433-452 (channel scale, then token scale, then activation). */
-static inline void mm_epilogue(const ascq_matmul_desc* d, void* c, size_t idx, int32_t acc, uint64_t qword,
-                               const float* tok_scale, size_t row, const void* bias, size_t bias_idx)
+/* v of one accumulator: channel scale, token scale, post-dequant bias, each one fp32 rounding (no activation yet). */
+static inline float mm_value(const ascq_matmul_desc* d, int32_t acc, uint64_t qword, const float* tok_scale, size_t row,
+                             const void* bias, size_t bias_idx)
 {
-    if (d->quant_mode == ASCQ_MM_QUANT_NONE) {
-        ((int32_t*)c)[idx] = acc;
-        return;
-    }
     float s = orc_quant_word_scale(qword, d->scale_format);
     volatile float v = (float)acc * s;
     if (d->has_tok_scale) {
@@ -637,10 +634,25 @@ static inline void mm_epilogue(const ascq_matmul_desc* d, void* c, size_t idx, i
         volatile float t = v + orc_bf16_to_f32(((const uint16_t*)bias)[bias_idx]);
         v = t;
     }
-    if (d->activation == ASCQ_MM_ACT_FASTER_GELU) {
-        v = orc_faster_gelu(v);
-    }
-    float r = v;
+    return v;
+}
+
+/* SwiGLU in fp32, step by step as the reference's vector instructions round:
+ * ref: impl/adv_api/detail/activation/swiglu/swiglu_common_impl.h:154-190 (Muls by -beta, Exp, Adds 1, Div, Mul). */
+float orc_swiglu(float src0, float src1, float beta)
+{
+    volatile float nb = -1.0f * beta;
+    volatile float t = src1 * nb;
+    volatile float e = expf(t);
+    volatile float dd = e + 1.0f;
+    volatile float sw = src1 / dd;
+    volatile float r = src0 * sw;
+    return r;
+}
+
+/* Output conversion of one value (everything after the activation). */
+static inline void mm_store(const ascq_matmul_desc* d, void* c, size_t idx, float r, uint64_t qword)
+{
     switch (d->out_dtype) {
         case ASCQ_F16: {
             if (r > 65504.0f) r = 65504.0f;
@@ -672,6 +684,20 @@ static inline void mm_epilogue(const ascq_matmul_desc* d, void* c, size_t idx, i
         }
         default: break;
     }
+}
+
+static inline void mm_epilogue(const ascq_matmul_desc* d, void* c, size_t idx, int32_t acc, uint64_t qword,
+                               const float* tok_scale, size_t row, const void* bias, size_t bias_idx)
+{
+    if (d->quant_mode == ASCQ_MM_QUANT_NONE) {
+        ((int32_t*)c)[idx] = acc;
+        return;
+    }
+    float v = mm_value(d, acc, qword, tok_scale, row, bias, bias_idx);
+    if (d->activation == ASCQ_MM_ACT_FASTER_GELU) {
+        v = orc_faster_gelu(v);
+    }
+    mm_store(d, c, idx, v, qword);
 }
 
 /* Exact int32 accumulation of rows [r0, r1) of A [.., k] with B [k, n] (or [n, k] when trans_b). */
@@ -707,16 +733,23 @@ static void mm_rows(const ascq_matmul_desc* d, void* c, const int8_t* a, const i
                     acc[j] += s;
                 }
             }
-            for (size_t j = 0; j < n; ++j) {
-                uint64_t w;
-                if (d->quant_mode == ASCQ_MM_QUANT_VECTOR) {
-                    w = (d->scale_format == ASCQ_MM_SCALE_U64) ? qv[bias_row_off + j]
-                                                                : (uint64_t)f32_bits(qvf[bias_row_off + j]);
-                } else {
-                    w = d->quant_scalar;
+#define ORC_QWORD(j)                                                                                              \
+    ((d->quant_mode == ASCQ_MM_QUANT_VECTOR)                                                                      \
+         ? ((d->scale_format == ASCQ_MM_SCALE_U64) ? qv[bias_row_off + (j)] : (uint64_t)f32_bits(qvf[bias_row_off + (j)])) \
+         : d->quant_scalar)
+            if (d->quant_mode != ASCQ_MM_QUANT_NONE && d->activation == ASCQ_MM_ACT_SWIGLU) {
+                /* columns 2j (src0) and 2j + 1 (src1) -> output column j of a row of n / 2 */
+                for (size_t j = 0; j + 1 < n; j += 2) {
+                    float v0 = mm_value(d, acc[j], ORC_QWORD(j), tok_scale, i, bias, bias_row_off + j);
+                    float v1 = mm_value(d, acc[j + 1], ORC_QWORD(j + 1), tok_scale, i, bias, bias_row_off + j + 1);
+                    mm_store(d, c, i * (n / 2) + j / 2, orc_swiglu(v0, v1, d->act_beta), 0);
                 }
-                mm_epilogue(d, c, i * n + j, acc[j], w, tok_scale, i, bias, bias_row_off + j);
+            } else {
+                for (size_t j = 0; j < n; ++j) {
+                    mm_epilogue(d, c, i * n + j, acc[j], ORC_QWORD(j), tok_scale, i, bias, bias_row_off + j);
+                }
             }
+#undef ORC_QWORD
         }
         free(acc);
     }

@@ -25,6 +25,7 @@ uint16_t orc_bf16_mul(uint16_t a, uint16_t b);
 uint16_t orc_bf16_add(uint16_t a, uint16_t b);
 int8_t orc_round_sat8(double v, int round_mode);
 float orc_faster_gelu(float x);
+float orc_swiglu(float src0, float src1, float beta);
 float orc_quant_word_scale(uint64_t w, int scale_format);
 
 uint8_t orc_f32_to_fp8(float f, int e5m2);

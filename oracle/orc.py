@@ -43,6 +43,8 @@ def lib():
         L.orc_round_sat8.argtypes = [C.c_double, C.c_int]
         L.orc_faster_gelu.restype = C.c_float
         L.orc_faster_gelu.argtypes = [C.c_float]
+        L.orc_swiglu.restype = C.c_float
+        L.orc_swiglu.argtypes = [C.c_float, C.c_float, C.c_float]
         L.orc_quant_word_scale.restype = C.c_float
         L.orc_quant_word_scale.argtypes = [C.c_uint64, C.c_int]
         L.orc_dequant_dst_stride.restype = C.c_uint32
@@ -183,8 +185,13 @@ def antiquant(desc, src, offset=None, scale=None):
     return dst
 
 
+def _out_cols(mm):
+    """Columns of the output: n, or n / 2 when the SwiGLU epilogue combines column pairs (activation value 2)."""
+    return mm.n // 2 if mm.activation == 2 and mm.quant_mode != 0 else mm.n
+
+
 def matmul_w8a8(desc, a, b, bias=None, quant_vector=None, tok_scale=None, rows=None):
-    c = np.zeros((desc.m, desc.n), dtype=_NP[desc.out_dtype])
+    c = np.zeros((desc.m, _out_cols(desc)), dtype=_NP[desc.out_dtype])
     if rows is None:
         lib().orc_matmul_w8a8(C.byref(desc), _ptr(c), _ptr(a), _ptr(b), _ptr(bias), _ptr(quant_vector),
                               _ptr(tok_scale))
@@ -195,7 +202,7 @@ def matmul_w8a8(desc, a, b, bias=None, quant_vector=None, tok_scale=None, rows=N
 
 
 def group_matmul_w8a8(desc, x, w, bias, scale, tok_scale, group_list, fill=0):
-    y = np.full((desc.mm.m, desc.mm.n), fill, dtype=_NP[desc.mm.out_dtype])
+    y = np.full((desc.mm.m, _out_cols(desc.mm)), fill, dtype=_NP[desc.mm.out_dtype])
     gl = np.ascontiguousarray(group_list, dtype=np.int64)
     lib().orc_group_matmul_w8a8(C.byref(desc), _ptr(y), _ptr(x), _ptr(w), _ptr(bias), _ptr(scale), _ptr(tok_scale),
                                 _ptr(gl))

@@ -32,7 +32,7 @@ def test_struct_sizes_match_the_header():
     assert C.sizeof(abi.QuantDesc) == 14 * 4
     assert C.sizeof(abi.DequantDesc) == 11 * 4
     assert C.sizeof(abi.AntiQuantDesc) == 13 * 4
-    assert C.sizeof(abi.MatmulDesc) == 11 * 4 + 4 + 8
+    assert C.sizeof(abi.MatmulDesc) == 11 * 4 + 4 + 8 + 8
     assert C.sizeof(abi.GroupMatmulDesc) == C.sizeof(abi.MatmulDesc) + 8
     assert C.sizeof(abi.W4A16Desc) == 5 * 4
     assert C.sizeof(abi.W8A16Desc) == 8 * 4
@@ -379,3 +379,18 @@ def test_tmp_buffer_factor_sizes_known_answers():
     assert aq((640, 5120), (1,), False, abi.BF16) == (1, 0)
     assert aq((64, 512), (64, 1), True, abi.BF16) == (0, 80 * 64 * 4)
     assert aq((640, 5120), (1,), True, abi.BF16) == (1, 0)
+
+
+def test_swiglu_rejections_and_workspace():
+    mk = lambda **kw: abi.MatmulDesc(**{**dict(m=16, n=64, k=128, out_dtype=abi.BF16, quant_mode=abi.MM_QUANT_VECTOR,
+                                               scale_format=abi.MM_SCALE_F32, activation=abi.MM_ACT_SWIGLU, act_beta=1.0), **kw})
+    call = lambda d, ws=None, nb=0: L.ascq_matmul_w8a8(C.byref(d), FAKE, FAKE, FAKE, None, FAKE, None, ws, nb, None)
+    assert call(mk(n=63)) == abi.EINVAL and "even" in err()
+    assert call(mk(out_dtype=abi.I8, scale_format=abi.MM_SCALE_U64)) == abi.EUNSUPPORTED
+    assert call(mk(quant_mode=abi.MM_QUANT_NONE, out_dtype=abi.I32)) == abi.EUNSUPPORTED
+    assert call(mk(act_beta=float("inf"))) == abi.EINVAL
+    assert call(mk(activation=3)) == abi.EINVAL
+    need = C.c_size_t(0)
+    assert L.ascq_matmul_w8a8_workspace_size(C.byref(mk()), C.byref(need)) == abi.OK
+    assert need.value >= 16 * 64 * 4                                  # the int32 accumulators of the pairwise epilogue
+    assert call(mk()) == abi.EINVAL and "workspace" in err()          # small m: not the large tile kernel

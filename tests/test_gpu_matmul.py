@@ -562,6 +562,78 @@ def test_group_matmul_example_full_size_nz_equals_nd():
         gold = v / (1.0 + np.exp(-1.702 * v))                       # the example's FastGelu, in closed form
         assert np.all(np.abs(got[i] - gold) <= 2e-3 * np.abs(gold) + 1e-6)
 
+# ------------------------------------------------------------------ SwiGLU epilogue
+def swiglu_close(got_bits, want_bits, fmt):
+    # expf of the device library against libm: the activation may differ by an ulp of the output type
+    assert max_ulp(got_bits, want_bits, fmt) <= 1
+    assert np.mean(got_bits == want_bits) > 0.98
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 64, 128), (16, 1040, 2048), (33, 144, 128), (200, 528, 384), (600, 528, 640),
+                                   (1100, 784, 384), (19, 22, 77), (2048, 2832, 384)])
+@pytest.mark.parametrize("out,bias", [(torch.bfloat16, None), (torch.float16, "f32"), (torch.float32, "bf16")])
+def test_matmul_swiglu_epilogue(m, n, k, out, bias):
+    """Columns 2j / 2j + 1 -> output column j; every kernel family (weight streams, K-split tiles, large tiles with the
+    in-register form, generic) against the oracle."""
+    announce("swiglu", m, n, k, out, bias)
+    rng = np.random.default_rng(m * 3 + n + k)
+    a, b = rand_i8(rng, (m, k)), rand_i8(rng, (k, n))
+    cs = rng.uniform(1e-4, 4e-4, n).astype(np.float32)
+    ts = rng.uniform(0.5, 2.0, m).astype(np.float32)
+    bv = None
+    if bias == "f32":
+        bv = (rng.standard_normal(n).astype(np.float32), None)
+    elif bias == "bf16":
+        bv = (orc.f32_to_bf16_bits(rng.standard_normal(n).astype(np.float32)), "bf16")
+    mm = ops.Matmul(m, n, k)
+    mm.set_tensor_a(to_dev(a))
+    mm.set_tensor_b(to_dev(b))
+    mm.set_quant_vector(to_dev(cs))
+    mm.set_token_scale(to_dev(ts))
+    if bv is not None:
+        mm.set_bias(to_dev(bv[0], bv[1]))
+    mm.set_activation(abi.MM_ACT_SWIGLU, 1.0 if m % 2 else 1.702)
+    c = torch.zeros((m, n // 2), dtype=out, device=DEV)
+    mm.iterate_all(c)
+    want = oracle_mm(mm.desc, a, b, bv, cs, ts)
+    if out == torch.float32:
+        got = c.cpu().numpy()
+        assert np.all(np.abs(got - want) <= 4 * np.spacing(np.abs(want)) + 1e-30)
+    else:
+        fmt = "bf16" if out == torch.bfloat16 else "f16"
+        swiglu_close(bits(c), want.view(np.uint16), fmt)
+
+
+def test_group_matmul_swiglu_and_dynamic_linear():
+    """The grouped matmul (MoE gate / up projection with interleaved columns) and the fused quantise + linear call."""
+    announce("group swiglu")
+    rng = np.random.default_rng(0x51)
+    groups, m, k, n = 4, 700, 256, 544
+    counts = np.array([300, 0, 1, 399], dtype=np.int64)
+    x, w = rand_i8(rng, (m, k)), rand_i8(rng, (groups, k, n))
+    sc = rng.uniform(1e-4, 4e-4, (groups, n)).astype(np.float32)
+    ts = rng.uniform(0.5, 2.0, m).astype(np.float32)
+    y = torch.zeros((m, n // 2), dtype=torch.bfloat16, device=DEV)
+    ops.quant_group_matmul(y, to_dev(x), to_dev(w), to_dev(counts), to_dev(sc), to_dev(ts),
+                           activation=abi.MM_ACT_SWIGLU, act_beta=1.0)
+    mmd = abi.MatmulDesc(m=m, n=n, k=k, out_dtype=abi.BF16, quant_mode=abi.MM_QUANT_VECTOR, scale_format=abi.MM_SCALE_F32,
+                         has_tok_scale=1, activation=abi.MM_ACT_SWIGLU, act_beta=1.0)
+    gd = abi.GroupMatmulDesc(mm=mmd, groups=groups, group_list_kind=abi.GROUP_LIST_COUNTS)
+    want = orc.group_matmul_w8a8(gd, x, w, None, sc, ts, counts)
+    swiglu_close(bits(y), want.view(np.uint16), "bf16")
+    # dynamic quantisation + linear + SwiGLU in one call, decode and prefill sizes
+    for mm_rows in (3, 640):
+        xa = orc.f32_to_bf16_bits(rng.standard_normal((mm_rows, k)).astype(np.float32))
+        wl = rand_i8(rng, (k, n))
+        cs = rng.uniform(1e-4, 4e-4, n).astype(np.float32)
+        c = torch.zeros((mm_rows, n // 2), dtype=torch.bfloat16, device=DEV)
+        ops.linear_w8a8_dynamic(c, to_dev(xa, "bf16"), to_dev(wl), to_dev(cs), activation=abi.MM_ACT_SWIGLU)
+        q, tsn = orc.dynamic_quant_per_token(abi.BF16, xa)
+        d = abi.MatmulDesc(m=mm_rows, n=n, k=k, out_dtype=abi.BF16, quant_mode=abi.MM_QUANT_VECTOR,
+                           scale_format=abi.MM_SCALE_F32, has_tok_scale=1, activation=abi.MM_ACT_SWIGLU, act_beta=1.0)
+        swiglu_close(bits(c), orc.matmul_w8a8(d, q, wl, None, cs, tsn).view(np.uint16), "bf16")
+
+
 # ------------------------------------------------------------------ workspace contract, determinism
 @pytest.mark.parametrize("m", [1, 5, 16, 19, 130])
 def test_workspaces_need_no_initialisation_and_results_repeat(m):

@@ -702,3 +702,47 @@ def test_antiquant_fp4_sources_are_value_times_power_of_two(fmt, k_dim):
     assert np.all((nb & 0x7F80) == 0x7F80) and np.all(nb & 0x7F)
     d.dst_dtype = abi.F16
     assert not orc.antiquant_policy(d, packed, sc2, None).view(U16).any()
+
+
+def test_swiglu_epilogue_is_the_reference_vector_chain():
+    """SwiGLU in the matmul epilogue: columns 2j / 2j + 1 are src0 / src1 and out[j] = src0 * (src1 / (1 + exp(-beta src1)))
+    in fp32, one rounding per step (swiglu_common_impl.h:154-190), pinned by numpy float32 arithmetic written as the
+    reference's five vector instructions, by the example's golden formula (swiglu/scripts/gen_data.py:32: src0 * src1 /
+    (1 + exp(-src1)) in float32) and by torch's bfloat16 rounding of the result."""
+    import torch
+    rng = np.random.default_rng(11)
+    m, k, n = 9, 64, 48
+    a = rng.integers(-127, 128, (m, k)).astype(np.int8)
+    b = rng.integers(-127, 128, (k, n)).astype(np.int8)
+    cs = rng.uniform(1e-4, 4e-4, n).astype(np.float32)
+    ts = rng.uniform(0.5, 2.0, m).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    acc = a.astype(np.int64) @ b.astype(np.int64)
+    v = ((acc.astype(np.float32) * cs[None, :]) * ts[:, None] + bias[None, :]).astype(np.float32)
+    for beta in (1.0, 1.702):
+        d = abi.MatmulDesc(m=m, n=n, k=k, out_dtype=abi.F32, quant_mode=abi.MM_QUANT_VECTOR, scale_format=abi.MM_SCALE_F32,
+                           has_tok_scale=1, bias_kind=abi.MM_BIAS_F32_POST, activation=abi.MM_ACT_SWIGLU, act_beta=beta)
+        got = orc.matmul_w8a8(d, a, b, bias, cs, ts)
+        assert got.shape == (m, n // 2)
+        s0, s1 = v[:, 0::2], v[:, 1::2]
+        t = (s1 * np.float32(-beta)).astype(np.float32)                       # Muls
+        with np.errstate(over="ignore"):                                    # exp of a large argument is inf: swish -> 0
+            e = np.exp(t.astype(np.float32)).astype(np.float32)              # Exp
+        dd = (e + np.float32(1.0)).astype(np.float32)                        # Adds
+        sw = (s1 / dd).astype(np.float32)                                    # Div
+        want = (s0 * sw).astype(np.float32)                                  # Mul
+        # expf of libm against numpy's float32 exp: at most 1 ulp apart, which the later steps carry through
+        assert np.all(np.abs(got - want) <= 4 * np.spacing(np.abs(want)) + 1e-30)
+        if beta == 1.0:
+            with np.errstate(over="ignore"):
+                gold = (s0 * s1 / (1 + np.exp(-1 * s1))).astype(np.float32)  # the example's golden
+            assert np.allclose(got, gold, rtol=1e-5, atol=1e-7)
+        # bf16 output = torch's rounding of the fp32 result
+        d.out_dtype = abi.BF16
+        got16 = orc.matmul_w8a8(d, a, b, bias, cs, ts)
+        ref16 = torch.from_numpy(got).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+        assert np.array_equal(got16, ref16)
+    # the scalar function itself on special arguments: swish(0) = 0, large |x| saturates to x or to -0
+    assert orc.lib().orc_swiglu(3.0, 0.0, 1.0) == 0.0
+    assert orc.lib().orc_swiglu(2.0, 100.0, 1.0) == 200.0
+    assert abs(orc.lib().orc_swiglu(2.0, -100.0, 1.0)) < 1e-40
