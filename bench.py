@@ -43,7 +43,7 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E peak, GB/s
 # file does not re-measure them.
 GEMM_TRAFFIC_BYTES = 228293837   # M=2048 GEMM, both tile shapes: 183.2 MB fetched + 45.1 MB written
 GEMV_TRAFFIC_BYTES = 133853594   # W4A16 M=1 GEMV, [k, n / 2] layout, stream + sum kernels: 129.5 MB fetched + 4.3 MB written
-GEMV_PACKED_TRAFFIC_BYTES = None  # W4A16 M=1 GEMV on packed weights: not measured yet
+GEMV_PACKED_TRAFFIC_BYTES = 128_487_629   # the same on packed weights, one launch: 128.4 MB fetched + 0.06 MB written (profiles/w4a16_packed_gemv_m1_trace_and_counters.md)
 
 
 def main():
@@ -129,12 +129,20 @@ def main():
         torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------ W8A8 linear (config 3)
-    def w8a8(M, steps, warmup, sets=1, settle=None, zero=False):
+    def w8a8(M, steps, warmup, sets=1, settle=None, zero=False, gauss=False):
         """`sets` > 1 rotates the weights over several copies (together larger than the Infinity Cache) so that the
-        weight-bound small-M cases read them from HBM."""
+        weight-bound small-M cases read them from HBM.  The weights are uniform over [-127, 127] unless `gauss`: then
+        they are normal weights quantised per output channel by their absolute maximum, as a checkpoint's would be."""
         K, N = 4096, 11008
         x = torch.randn((M, K), device=dev, generator=gen).to(torch.bfloat16)
-        ws = [rand_i8(K, N) for _ in range(sets)]
+        if gauss:
+            ws = []
+            for _ in range(sets):
+                wf = torch.randn((K, N), device=dev, generator=gen)
+                ws.append(torch.round(wf / wf.abs().amax(dim=0, keepdim=True) * 127).clamp(-127, 127).to(torch.int8))
+                del wf
+        else:
+            ws = [rand_i8(K, N) for _ in range(sets)]
         if zero:          # all-zero activations and weights: the same launches, nothing toggles in the multipliers
             x.zero_()
             for wj in ws:
@@ -396,6 +404,14 @@ def main():
             "note": "the same GEMM launches on all-zero activations and weights: the instruction stream, tiling and "
                     "memory traffic are those of the headline, only the operand values differ"}
         del z
+        torch.cuda.empty_cache()
+        g = w8a8(2048, min(args.steps, 300), min(args.warmup, 50), gauss=True)
+        out["roofline"]["same_kernel_normal_weights"] = {
+            "avg_kernel_ms": g["gemm_kernel_ms"], "achieved": g["gemm_tops"], "frac": g["gemm_tops"] / PEAK_INT8_TOPS,
+            "note": "the same GEMM launches on normally distributed weights quantised per output channel by their "
+                    "absolute maximum (the headline's weights are uniform over [-127, 127], the most switching "
+                    "activity a weight matrix can cause)"}
+        del g
         torch.cuda.empty_cache()
     if ceilings is not None:
         out["ceilings"] = ceilings
