@@ -6,7 +6,9 @@ A guarded kernel reads LDS or global memory through inline assembly (`ds_read_b1
 result visible to the compiler only at a later counted wait.  Until then the compiler takes the destination registers
 for valid.  If register pressure makes it spill or copy one of them in between, stale data is stored, or the load that
 is still in flight writes into a register that now belongs to something else (a memory fault was seen from exactly
-this).  A scratch frame of zero bytes and zero spilled registers is the build-time proof that no such move exists.
+this).  A scratch frame of zero bytes and zero spilled vector registers is the build-time proof that no such move
+exists.  Spilled scalar registers are recorded but allowed: the compiler parks them in lanes of a vector register it
+reserves for that purpose, which is never the destination of a load.
 """
 import json
 import re
@@ -15,7 +17,7 @@ import sys
 
 # kernels built on the inline-assembly read pattern, by the name they have in the sources
 GUARDED = ("w4a16_gemv_kernel", "w4a16_tile_kernel", "w8a16_tile_kernel", "gemm_stream_kernel", "gemm_dma_kernel",
-           "gemm_dma_dual_kernel", "w4a16_packed_kernel")
+           "gemm_dma_dual_kernel", "gemm_dma_group_kernel", "w4a16_packed_kernel")
 
 FIELDS = {
     "TotalSGPRs": "sgprs", "VGPRs": "vgprs", "AGPRs": "agprs", "ScratchSize [bytes/lane]": "scratch_bytes_per_lane",
@@ -52,8 +54,7 @@ def main(paths):
         k["name"] = name.replace("ascq::(anonymous namespace)::", "")
         base = re.sub(r"^void ", "", k["name"]).split("<")[0].split("(")[0]
         k["guarded"] = base in GUARDED
-    bad = [k for k in kernels if k["guarded"] and (k.get("scratch_bytes_per_lane", 1) or k.get("vgpr_spills", 1)
-                                                   or k.get("sgpr_spills", 1))]
+    bad = [k for k in kernels if k["guarded"] and (k.get("scratch_bytes_per_lane", 1) or k.get("vgpr_spills", 1))]
     json.dump({"guarded_names": GUARDED, "kernels": kernels}, sys.stdout, indent=1)
     for k in bad:
         sys.stderr.write("check_resources: %s (%s) has %d bytes of scratch per lane, %d VGPR and %d SGPR spills; a kernel "

@@ -361,16 +361,24 @@ __global__ __launch_bounds__(kThreads) void dynq_row_kernel(int8_t* __restrict__
     if (threadIdx.x == 0) {
         ts[row] = zero ? 1.0f : amax / 127.0f;
     }
+    // |v * inv| <= 127 (1 + 2^-23) by construction, so the product needs no clamp for finite inputs (the median keeps
+    // infinities inside int8; NaN becomes -128).  Adding 1.5 * 2^23 rounds the fp32 product to the nearest integer, ties
+    // to even, exactly as rint does (the sum's spacing is 1 and the constant is even), and leaves that integer in two's
+    // complement in the low mantissa bits: one add replaces rint, the conversion and the sign handling, and one byte
+    // permute per pair gathers the low bytes.
 #pragma unroll
     for (int k = 0; k < kVecs; ++k) {
         const uint32_t j = (k * kThreads + threadIdx.x) * 8u;
         if (j < n) {
-            int r[8];
+            uint32_t u[8];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) r[e] = round_sat8<true>(v[k][e] * inv, 0);
+            for (int e = 0; e < 8; ++e) {
+                const float t = __builtin_amdgcn_fmed3f(v[k][e] * inv, -128.0f, 127.0f);
+                u[e] = __float_as_uint(t + 12582912.0f);
+            }
             u32x2 out;
-            out[0] = pack4_i8(r[0], r[1], r[2], r[3]);
-            out[1] = pack4_i8(r[4], r[5], r[6], r[7]);
+            out[0] = __builtin_amdgcn_perm(u[1], u[0], 0x0c0c0400u) | __builtin_amdgcn_perm(u[3], u[2], 0x04000c0cu);
+            out[1] = __builtin_amdgcn_perm(u[5], u[4], 0x0c0c0400u) | __builtin_amdgcn_perm(u[7], u[6], 0x04000c0cu);
             *reinterpret_cast<u32x2*>(q + static_cast<size_t>(row) * n + j) = out;
         }
     }

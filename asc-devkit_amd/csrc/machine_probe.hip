@@ -5,7 +5,9 @@
 //   * the shader clock during each of those loops, from the ratio of the shader-clock counter to the constant
 //     100 MHz real-time counter read inside the kernel;
 //   * device-to-device copy, read-only sweep and write-only fill of 1 GiB (HBM bandwidth actually reachable);
-//   * LDS read bandwidth per compute unit with 16-byte reads.
+//   * LDS read bandwidth per compute unit with 16-byte reads;
+//   * a small streaming job, 2048 workgroups that each read one 8 KiB row and write 4 KiB (16 MiB in, 8 MiB out, the
+//     same buffers every launch): what launch, ramp-up and drain cost a kernel of that size whatever it computes.
 // Every figure is the mean of the second half of `reps` back-to-back launches (the first half brings the clocks to
 // their sustained state).  No input, no dependence on libascq.
 #include <hip/hip_runtime.h>
@@ -88,6 +90,19 @@ __global__ __launch_bounds__(256) void fill_kernel(u32x4* __restrict__ b, size_t
 
 // 8 x 16-byte LDS reads per lane and iteration, rows of 128 bytes with the XOR swizzle of the GEMM's A tile.  The reads
 // and the wait for them are one asm statement, so the compiler never sees a register whose load is still in flight.
+// One workgroup per row of 8 KiB: two 16-byte loads per lane, the even bytes of each stored as 8 bytes.
+__global__ __launch_bounds__(256) void row_2to1_kernel(const u32x4* __restrict__ a, unsigned long long* __restrict__ b)
+{
+    const size_t base = static_cast<size_t>(blockIdx.x) * 512;
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        const u32x4 v = a[base + k * 256 + threadIdx.x];
+        const unsigned lo = __builtin_amdgcn_perm(v[1], v[0], 0x06040200u);
+        const unsigned hi = __builtin_amdgcn_perm(v[3], v[2], 0x06040200u);
+        b[base + k * 256 + threadIdx.x] = (static_cast<unsigned long long>(hi) << 32) | lo;
+    }
+}
+
 __global__ __launch_bounds__(256) void lds_read_loop(int* out, int iters)
 {
     __shared__ __attribute__((aligned(16))) char smem[65536];
@@ -198,7 +213,16 @@ int main()
     CK(hipEventSynchronize(e1));
     CK(hipEventElapsedTime(&ms, e0, e1));
     const double lds_bytes = 16.0 * 256 * 8 * lds_iters * cus * 4 * 8;
-    printf(", \"lds_read_bytes_per_clock_per_cu_at_max_clock\": %.0f}\n",
+    printf(", \"lds_read_bytes_per_clock_per_cu_at_max_clock\": %.0f",
            lds_bytes / (ms * 1e-3) / (clock_khz * 1e3) / cus);
+
+    // ---- a 24 MiB streaming job
+    for (int r = 0; r < 100; ++r) row_2to1_kernel<<<2048, 256>>>(a, reinterpret_cast<unsigned long long*>(b));
+    CK(hipEventRecord(e0));
+    for (int r = 0; r < 400; ++r) row_2to1_kernel<<<2048, 256>>>(a, reinterpret_cast<unsigned long long*>(b));
+    CK(hipEventRecord(e1));
+    CK(hipEventSynchronize(e1));
+    CK(hipEventElapsedTime(&ms, e0, e1));
+    printf(", \"rows_2048x8kib_read_4kib_written_us\": %.2f}\n", ms * 1e3 / 400);
     return 0;
 }

@@ -63,12 +63,15 @@ __device__ __forceinline__ ChannelQ load_channel_q(const EpiParams& e, size_t co
     return q;
 }
 
+// FasterGelu, x * exp(0.851 (x - |x|)) / (1 + exp(-1.702 |x|)).  For x < 0 the two exponentials are the same number
+// (0.851 * 2x and 1.702 * x round alike in fp32) and for x >= 0 the first is exactly 1, so one exponential serves
+// both; it and the reciprocal are the hardware's approximations (about one fp32 ulp each), far inside one ulp of
+// the 16-bit outputs this activation is used with.
 __device__ __forceinline__ float faster_gelu(float x)
 {
-    const float ax = fabsf(x);
-    const float x2 = expf(0.851f * (x - ax));
-    const float x3 = 1.0f + expf(-1.702f * ax);
-    return x * x2 / x3;
+    const float e = __builtin_amdgcn_exp2f((-1.702f * 1.44269504088896341f) * fabsf(x));
+    const float num = x < 0.0f ? x * e : x;
+    return num * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
 // SwiGLU of one column pair in fp32, one rounding per step, in the order of the reference's vector instructions
@@ -183,7 +186,7 @@ __device__ __forceinline__ uint32_t xcd_remap(uint32_t pid, uint32_t total)
     }
     const uint32_t xcd = pid & 7u, local = pid >> 3;
     if (xcd < tall) {
-        return xcd * per + local;
+        return local < per ? xcd * per + local : 0xFFFFFFFFu;  // a launch may be larger than `total`
     }
     if (local + 1u >= per) {
         return 0xFFFFFFFFu;  // the short XCDs own one tile less: this workgroup has nothing to do

@@ -24,14 +24,6 @@
 
 #include "matmul_w8a8.h"
 
-#ifdef ASCQ_EXP_CLOCK
-__device__ unsigned long long ascq_dbg_clk[4];
-extern "C" int ascq_debug_clock(unsigned long long* out)
-{
-    return hipMemcpyFromSymbol(out, HIP_SYMBOL(ascq_dbg_clk), sizeof(ascq_dbg_clk)) == hipSuccess ? 0 : 1;
-}
-#endif
-
 namespace ascq {
 namespace {
 
@@ -88,9 +80,17 @@ __device__ __forceinline__ float epi_value(int32_t acc, float chan, float tok, f
 // are declared by the kernels and handed in, so that one kernel can run tiles of two shapes.
 // kBT: B is given as [n][k] (transposed operand): its tile is staged and read exactly like A's, with plain 16-byte
 // LDS reads instead of the transposing ones.
+// Where a tile lies: rows [row0, row_end) of A and C (row_end clips the tile), columns from n0, the weight matrix it
+// multiplies with and the offset of that matrix's per-channel parameters (grouped: those of the tile's group).
+struct TilePlace {
+    uint32_t row0, row_end, n0;
+    const int8_t* b;
+    size_t chan_off;
+};
+
 template <int BM, int BN, bool kSplitK, bool kGrouped, bool kBT = false>
-__device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_begin, uint32_t bid, uint32_t bidy,
-                                              char* A0, char* B0, char* A1, char* B1, float* TS)
+__device__ __forceinline__ void gemm_dma_tile_at(const GemmParams& p, const TilePlace& at, uint32_t bidy, char* A0,
+                                                 char* B0, char* A1, char* B1, float* TS)
 {
     constexpr int kWN = BN / 64;            // wavefronts along N
     constexpr int kWM = 8 / kWN;            // wavefronts along M
@@ -102,53 +102,17 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_
     constexpr int kKsB = 32 * BN;           // bytes of B per K sub-step of 32 rows
     static_assert(TI >= 1 && TI * 32 * kWM == BM && kAInstr >= 1, "tile shape does not fit eight wavefronts");
 
-    const uint32_t total = p.tiles_m * p.tiles_n;
-    const uint32_t t = xcd_remap(bid, total);
-    if (t >= total) {
-        return;
-    }
-#ifdef ASCQ_EXP_CLOCK
-    const unsigned long long dbg_c0 = __builtin_readcyclecounter(), dbg_r0 = wall_clock64();
-#endif
-    const uint32_t ms = t % p.tiles_m, tn = t / p.tiles_m;
     const uint32_t K = p.k, N = p.n;
-    uint32_t row0 = ms * BM, row_end = p.m;
-    const int8_t* Bmat = p.b;
-    size_t chan_off = 0;
+    const uint32_t row0 = at.row0, row_end = at.row_end, n0 = at.n0;
+    const int8_t* Bmat = at.b;
+    const size_t chan_off = at.chan_off;
+    uint32_t tid = threadIdx.x;
     if constexpr (kGrouped) {
-        // walk the groups: group g owns tile slots [slot, slot + ceil(rows / BM))
-        uint32_t slot = 0;
-        int64_t off = 0;
-        bool found = false;
-        for (uint32_t g = 0; g < p.groups; ++g) {
-            const int64_t v = p.group_list[g];
-            const int64_t cnt = p.group_list_kind == ASCQ_GROUP_LIST_PREFIX_SUM ? v - off : v;
-            if (cnt <= 0) {
-                continue;
-            }
-            int64_t end = off + cnt;
-            if (end > static_cast<int64_t>(p.m)) {
-                end = p.m;
-            }
-            const uint32_t rows = end > off ? static_cast<uint32_t>(end - off) : 0u;
-            const uint32_t tiles = (rows + BM - 1) / BM;
-            if (ms < slot + tiles) {
-                row0 = static_cast<uint32_t>(off) + (ms - slot) * BM;
-                row_end = static_cast<uint32_t>(end);
-                Bmat = p.b + static_cast<size_t>(g) * K * N;
-                chan_off = static_cast<size_t>(g) * N;
-                found = true;
-                break;
-            }
-            slot += tiles;
-            off += cnt;
-        }
-        if (!found) {
-            return;
-        }
+        // The grouped kernel runs tiles in a loop: without this the compiler computes everything that depends only on
+        // the lane once, ahead of the loop, and those registers are missing in the tile's main loop.
+        asm volatile("" : "+v"(tid));
     }
-    const uint32_t n0 = col_begin + tn * BN;
-    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t wm = wave / kWN, wn = wave % kWN;
     if (tid < BM) {
@@ -271,11 +235,7 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_
     auto interleave = [&]() __attribute__((always_inline)) {
         constexpr int kReads = TI + (kBT ? TJ : 2 * TJ);
         constexpr int kMfmas = TI * TJ;
-#ifdef ASCQ_EXP_FRONT_DIV
-        constexpr int kFront = (kMfmas + ASCQ_EXP_FRONT_DIV - 1) / ASCQ_EXP_FRONT_DIV;
-#else
         constexpr int kFront = (kMfmas + 1) / 2;
-#endif
         constexpr int kPer = (kReads + kFront - 1) / kFront;
         static_for<kMfmas>([&](auto n) {
             constexpr int kLeft = kReads - decltype(n)::value * kPer;
@@ -333,25 +293,11 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_
     // The loop body never branches between two ways of updating the accumulators (that would make the compiler
     // shuffle all 256 of them): the steady state always has a next step, the last one or two steps are peeled.
     uint32_t s = 0;
-#ifdef ASCQ_EXP_CLOCK
-    unsigned long long dbg_vm = 0, dbg_bar = 0;
-#define ASCQ_WAIT_AND_BARRIER()                                          \
-    do {                                                                 \
-        const unsigned long long t0_ = __builtin_readcyclecounter();     \
-        asm volatile("s_waitcnt vmcnt(0)");                              \
-        const unsigned long long t1_ = __builtin_readcyclecounter();     \
-        __syncthreads();                                                 \
-        const unsigned long long t2_ = __builtin_readcyclecounter();     \
-        dbg_vm += t1_ - t0_;                                             \
-        dbg_bar += t2_ - t1_;                                            \
-    } while (0)
-#else
 #define ASCQ_WAIT_AND_BARRIER()             \
     do {                                    \
         asm volatile("s_waitcnt vmcnt(0)"); \
         __syncthreads();                    \
     } while (0)
-#endif
     for (; s + 2 < steps; s += 2) {
         if (wave_active) head(A0, B0);
         ASCQ_WAIT_AND_BARRIER();
@@ -380,14 +326,6 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_
         }
     }
 
-#ifdef ASCQ_EXP_CLOCK
-    if (bid == 8 && threadIdx.x == 0 && BN == 256) {
-        ascq_dbg_clk[0] = __builtin_readcyclecounter() - dbg_c0;
-        ascq_dbg_clk[1] = wall_clock64() - dbg_r0;
-        ascq_dbg_clk[2] = dbg_vm;
-        ascq_dbg_clk[3] = dbg_bar;
-    }
-#endif
     // ---- epilogue: register r of lane l in a 32x32 block is row 8*(r/4) + 4*(l/32) + r%4, column l%32
     if constexpr (kSplitK) {
         int32_t* part = p.partial + static_cast<size_t>(bidy) * p.m * N;
@@ -530,7 +468,168 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_
     dispatch_out(e, run);
 }
 
-template <int BM, int BN, bool kSplitK, bool kGrouped = false, bool kBT = false>
+// The plain matmul: tile number `bid` of the launch (before the XCD remapping), column tiles counted from col_begin,
+// row tiles innermost so that the tiles an XCD runs side by side share their B columns.
+template <int BM, int BN, bool kSplitK, bool kBT>
+__device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_begin, uint32_t bid, uint32_t bidy,
+                                              char* A0, char* B0, char* A1, char* B1, float* TS)
+{
+    const uint32_t total = p.tiles_m * p.tiles_n;
+    const uint32_t t = xcd_remap(bid, total);
+    if (t >= total) {
+        return;
+    }
+    const uint32_t ms = t % p.tiles_m, tn = t / p.tiles_m;
+    const TilePlace at{ms * BM, p.m, col_begin + tn * BN, p.b, 0};
+    gemm_dma_tile_at<BM, BN, kSplitK, false, kBT>(p, at, bidy, A0, B0, A1, B1, TS);
+}
+
+// Rows [off, end) of group g (clipped to m); false when the group owns none.  `off` is carried from group to group.
+__device__ __forceinline__ bool group_rows(const GemmParams& p, uint32_t g, int64_t& off, uint32_t& first, uint32_t& end)
+{
+    const int64_t v = p.group_list[g];
+    const int64_t cnt = p.group_list_kind == ASCQ_GROUP_LIST_PREFIX_SUM ? v - off : v;
+    if (cnt <= 0) {
+        return false;
+    }
+    const int64_t begin = off;
+    off += cnt;
+    const int64_t stop = off > static_cast<int64_t>(p.m) ? static_cast<int64_t>(p.m) : off;
+    first = static_cast<uint32_t>(begin);
+    end = static_cast<uint32_t>(stop);
+    return stop > begin;
+}
+
+// Row tiles of a group: `big` tiles of 256 rows (a remainder of more than 128 rows is one of them) and at most one
+// small tile of 128 rows for a shorter remainder.
+__device__ __forceinline__ void group_row_tiles(uint32_t rows, uint32_t& big, uint32_t& small)
+{
+    const uint32_t rem = rows & 255u;
+    big = (rows >> 8) + (rem > 128u ? 1u : 0u);
+    small = (rem != 0u && rem <= 128u) ? 1u : 0u;
+}
+
+// One phase of the grouped kernel's plan (see gemm_dma_group_kernel): the workgroup's ids that fall into it.
+template <uint32_t phase>
+__device__ __forceinline__ void gemm_dma_group_phase(const GemmParams& p, const uint32_t* PLAN, char* A0, char* B0,
+                                                     char* A1, char* B1, float* TS)
+{
+    for (uint32_t id = blockIdx.x;; id += gridDim.x) {
+        const uint32_t tiles_n = p.tiles_n;
+        const uint32_t big_tiles = __builtin_amdgcn_readfirstlane(PLAN[0]);
+        const uint32_t small_tiles = __builtin_amdgcn_readfirstlane(PLAN[1]);
+        const uint32_t wide = __builtin_amdgcn_readfirstlane(PLAN[2]);
+        const uint32_t col_narrow = wide * 256u;
+        const uint32_t narrow = col_narrow < p.n ? (p.n - col_narrow + 127u) / 128u : 0u;
+        const uint32_t count0 = big_tiles * wide, count1 = big_tiles * narrow, count2 = small_tiles * tiles_n;
+        const uint32_t first1 = (count0 + 7u) & ~7u, first2 = first1 + ((count1 + 7u) & ~7u);
+        const uint32_t first = phase == 0 ? 0u : phase == 1 ? first1 : first2;
+        const uint32_t count = phase == 0 ? count0 : phase == 1 ? count1 : count2;
+        const uint32_t cols = phase == 0 ? wide : phase == 1 ? narrow : tiles_n;
+        if (id < first) {
+            continue;  // an id of an earlier phase
+        }
+        if (id >= first + ((count + 7u) & ~7u)) {
+            break;
+        }
+        const uint32_t t = xcd_remap(id - first, count);
+        if (t >= count) {
+            continue;  // padding of the phase
+        }
+        TilePlace at{0, 0, 0, nullptr, 0};
+        {
+            uint32_t base = 0;
+            int64_t off = 0;
+            for (uint32_t g = 0; g < p.groups; ++g) {
+                uint32_t first, end, big, small;
+                if (!group_rows(p, g, off, first, end)) {
+                    continue;
+                }
+                group_row_tiles(end - first, big, small);
+                const uint32_t mine = phase == 2 ? small : big;
+                if (t >= base + mine * cols) {
+                    base += mine * cols;
+                    continue;
+                }
+                const uint32_t local = t - base;
+                const uint32_t tn = local / mine, tr = local - tn * mine;
+                at.row0 = first + (phase == 2 ? ((end - first) >> 8) * 256u : tr * 256u);
+                at.row_end = end;
+                at.n0 = phase == 1 ? col_narrow + tn * 128u : tn * 256u;
+                at.b = p.b + static_cast<size_t>(g) * p.k * p.n;
+                at.chan_off = static_cast<size_t>(g) * p.n;
+                break;
+            }
+        }
+        if (at.b == nullptr) {
+            continue;
+        }
+        if constexpr (phase == 0) {
+            gemm_dma_tile_at<256, 256, false, true>(p, at, 0u, A0, B0, A1, B1, TS);
+        } else if constexpr (phase == 1) {
+            gemm_dma_tile_at<256, 128, false, true>(p, at, 0u, A0, B0, A1, B1, TS);
+        } else {
+            gemm_dma_tile_at<128, 256, false, true>(p, at, 0u, A0, B0, A1, B1, TS);
+        }
+        __syncthreads();  // the next tile's loads and token scales overwrite what slower wavefronts may still read
+    }
+}
+
+// The grouped matmul in one launch of persistent workgroups, one per compute unit.  Every workgroup reads the group
+// list and derives the same plan from it:
+//   phase 0: the big row tiles x the first `wide` 256-wide tile columns, as many as fill whole rounds of the chip;
+//   phase 1: the big row tiles x the remaining columns as 256 x 128 tiles (the last, partial round in half-size pieces);
+//   phase 2: the groups' short remainders (at most 128 rows) as 128 x 256 tiles, cheapest last.
+// Tile ids run through the phases in this order (each phase padded to a multiple of 8 ids, so that id mod 8 stays the
+// XCD of the workgroup that takes it); workgroup w takes ids w, w + gridDim.x, ...  Inside a phase the tiles are
+// ordered group by group, column by column, the row tiles of a column adjacent, and an XCD takes a contiguous share:
+// about one group per XCD, whose rows of A stay in that L2 while each B tile is fetched once for the row tiles that
+// run side by side.  The group sizes are known only on the device, so a launch sized by the host for the worst case
+// would consist mostly of workgroups with nothing to do; the loop has none.  gridDim.x must be a multiple of 8;
+// p.tiles_n = 256-wide tile columns of the whole matrix.
+__global__ __launch_bounds__(kThreads, 1) void gemm_dma_group_kernel(GemmParams p)
+{
+    __shared__ __attribute__((aligned(1024))) char A0[256 * BK];
+    __shared__ __attribute__((aligned(1024))) char B0[BK * 256];
+    __shared__ __attribute__((aligned(1024))) char A1[256 * BK];
+    __shared__ __attribute__((aligned(1024))) char B1[BK * 256];
+    __shared__ __attribute__((aligned(16))) float TS[256];
+    uint32_t n_big = 0, n_small = 0;
+    {
+        int64_t off = 0;
+        for (uint32_t g = 0; g < p.groups; ++g) {
+            uint32_t first, end, big, small;
+            if (group_rows(p, g, off, first, end)) {
+                group_row_tiles(end - first, big, small);
+                n_big += big;
+                n_small += small;
+            }
+        }
+    }
+    // The plan is parked in LDS and re-read per tile: held in scalar registers across the tile bodies it would push
+    // the compiler into spilling them.
+    __shared__ uint32_t PLAN[4];
+    {
+        const uint32_t units = n_big * p.tiles_n + (n_small * p.tiles_n + 1u) / 2u;  // work in 256 x 256 tiles
+        uint32_t wide = n_big ? units / gridDim.x * gridDim.x / n_big : 0u;
+        if (wide > p.tiles_n) {
+            wide = p.tiles_n;
+        }
+        if (threadIdx.x == 0) {
+            PLAN[0] = n_big;
+            PLAN[1] = n_small;
+            PLAN[2] = wide;
+        }
+        __syncthreads();
+    }
+    // One loop per phase (a workgroup's ids ascend, so it passes through the phases in order anyway): each loop holds
+    // one tile shape's code and registers.
+    gemm_dma_group_phase<0>(p, PLAN, A0, B0, A1, B1, TS);
+    gemm_dma_group_phase<1>(p, PLAN, A0, B0, A1, B1, TS);
+    gemm_dma_group_phase<2>(p, PLAN, A0, B0, A1, B1, TS);
+}
+
+template <int BM, int BN, bool kSplitK, bool kBT = false>
 __global__ __launch_bounds__(kThreads, (BM * BK + BK * BN) * 2 <= 65536 ? 2 : 1) void gemm_dma_kernel(
     GemmParams p, uint32_t col_begin)
 {
@@ -539,7 +638,7 @@ __global__ __launch_bounds__(kThreads, (BM * BK + BK * BN) * 2 <= 65536 ? 2 : 1)
     __shared__ __attribute__((aligned(1024))) char A1[BM * BK];
     __shared__ __attribute__((aligned(1024))) char B1[BK * BN];
     __shared__ __attribute__((aligned(16))) float TS[BM];  // token scales of the tile's rows (1.0f when there are none)
-    gemm_dma_tile<BM, BN, kSplitK, kGrouped, kBT>(p, col_begin, blockIdx.x, blockIdx.y, A0, B0, A1, B1, TS);
+    gemm_dma_tile<BM, BN, kSplitK, kBT>(p, col_begin, blockIdx.x, blockIdx.y, A0, B0, A1, B1, TS);
 }
 
 // One launch for a matrix whose last round of 256 x 256 tiles would be mostly empty: workgroups [0, wide_wgs) run the
@@ -555,11 +654,11 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_dma_dual_kernel(GemmParams p
     __shared__ __attribute__((aligned(1024))) char B1[BK * 256];
     __shared__ __attribute__((aligned(16))) float TS[256];
     if (blockIdx.x < wide_wgs) {
-        gemm_dma_tile<256, 256, false, false, kBT>(p, 0u, blockIdx.x, 0u, A0, B0, A1, B1, TS);
+        gemm_dma_tile<256, 256, false, kBT>(p, 0u, blockIdx.x, 0u, A0, B0, A1, B1, TS);
     } else {
         GemmParams q = p;
         q.tiles_n = narrow_tiles_n;
-        gemm_dma_tile<256, 128, false, false, kBT>(q, col_begin, blockIdx.x - wide_wgs, 0u, A0, B0, A1, B1, TS);
+        gemm_dma_tile<256, 128, false, kBT>(q, col_begin, blockIdx.x - wide_wgs, 0u, A0, B0, A1, B1, TS);
     }
 }
 
@@ -595,6 +694,24 @@ __global__ __launch_bounds__(256) void splitk_sum_epilogue_kernel(GemmParams p)
 
 }  // namespace
 
+// Compute units of the current device (cached for the first 64 devices).
+static uint32_t device_compute_units()
+{
+    static int cached[64];
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+        return 256u;
+    }
+    n = __atomic_load_n(&cached[dev], __ATOMIC_RELAXED);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+            n = 256;
+        }
+        __atomic_store_n(&cached[dev], n, __ATOMIC_RELAXED);
+    }
+    return static_cast<uint32_t>(n);
+}
+
 bool gemm_dma_supported(const GemmParams& p)
 {
     return p.k % BK == 0 && p.n % 16 == 0 && p.n >= 16 && aligned16(p.a) && aligned16(p.b);
@@ -602,14 +719,38 @@ bool gemm_dma_supported(const GemmParams& p)
 
 int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st, bool b_nk)
 {
-    p.tiles_m = (p.m + 255u) / 256u + (grouped ? p.groups : 0u);  // every group adds at most one partial tile
     uint32_t tiles_n = (p.n + 255u) / 256u;
+    if (grouped) {
+        // The group sizes are on the device; the kernel plans its tiles there.  One persistent workgroup per compute
+        // unit (a multiple of 8, so that a workgroup's id mod 8 is its XCD), fewer when no group list over m rows
+        // can need that many tiles: big row tiles hold more than 128 rows each, at most m / 256 + groups of them, and
+        // every group adds at most one short remainder.
+        const uint32_t big = p.m / 129u < p.m / 256u + p.groups ? p.m / 129u : p.m / 256u + p.groups;
+        const uint32_t small = p.groups < p.m ? p.groups : p.m;
+        const uint64_t most = static_cast<uint64_t>(big) * 2u * tiles_n + static_cast<uint64_t>(small) * tiles_n + 24u;
+        uint32_t wgs = device_compute_units() / 8u * 8u;
+        if (wgs == 0u) {
+            wgs = 8u;
+        }
+        if (most < wgs) {
+            wgs = static_cast<uint32_t>((most + 7u) / 8u * 8u);
+        }
+        p.tiles_m = big + small;
+        p.tiles_n = tiles_n;
+        if (plan_recording()) {
+            plan_note(ASCQ_MM_KERNEL_DMA_256, 256, 256, BK, wgs, 1, 2u * (256u * BK + BK * 256u) + 256u * 4u, 0);
+            return ASCQ_OK;
+        }
+        gemm_dma_group_kernel<<<wgs, kThreads, 0, st>>>(p);
+        return launch_status("ascq_group_matmul_w8a8");
+    }
+    p.tiles_m = (p.m + 255u) / 256u;
     // Tile quantisation: when the last round of 256-wide tiles would fill less than half of the 256 CUs, its
     // columns are computed with 128-wide tiles, which finish that round in about half the time.
     uint32_t narrow_cols = 0;  // number of 256-wide column tiles handed to the 128-wide kernel
     const uint32_t total = p.tiles_m * tiles_n;
     const uint32_t rem = total % 256u;
-    if (!grouped && total > 256u && rem != 0 && rem <= 128u) {
+    if (total > 256u && rem != 0 && rem <= 128u) {
         narrow_cols = (rem + p.tiles_m - 1) / p.tiles_m;
         if (narrow_cols > tiles_n) {
             narrow_cols = tiles_n;
@@ -654,10 +795,8 @@ int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st, bool b_nk)
         if (narrow_cols) {
             q.n = p.n;  // row pitch stays n; columns >= wide_cols * 256 are simply not assigned to any tile
         }
-        if (grouped) {
+        if (b_nk) {
             gemm_dma_kernel<256, 256, false, true><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(q, 0u);
-        } else if (b_nk) {
-            gemm_dma_kernel<256, 256, false, false, true><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(q, 0u);
         } else {
             gemm_dma_kernel<256, 256, false><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(q, 0u);
         }
@@ -667,12 +806,12 @@ int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st, bool b_nk)
         p.tiles_n = (p.n - col_begin + 127u) / 128u;
         const uint32_t t = p.tiles_m * p.tiles_n;
         if (b_nk) {
-            gemm_dma_kernel<256, 128, false, false, true><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(p, col_begin);
+            gemm_dma_kernel<256, 128, false, true><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(p, col_begin);
         } else {
             gemm_dma_kernel<256, 128, false><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(p, col_begin);
         }
     }
-    return launch_status(grouped ? "ascq_group_matmul_w8a8" : "ascq_matmul_w8a8");
+    return launch_status("ascq_matmul_w8a8");
 }
 
 // Split factor of the 128 x 128 kernel: two workgroups per CU when the partial tiles are small next to the weights,

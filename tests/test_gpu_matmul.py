@@ -204,6 +204,45 @@ def test_config5_moe_up_projection():
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("counts,act", [([600, 40, 560], abi.MM_ACT_NONE), ([200, 0, 513, 129, 128, 1], abi.MM_ACT_FASTER_GELU),
+                                        ([300, 300, 300, 300], abi.MM_ACT_SWIGLU)])
+def test_group_matmul_all_tile_shapes(counts, act):
+    """Enough 256-row tiles and tile columns that the launch holds a whole round of 256 x 256 tiles, a partial round
+    of 256 x 128 tiles (the last of them 80 columns wide) and 128-row tiles for the groups' short remainders; groups
+    with 128, 129 and 200 remainder rows sit on either side of the rule that picks the row-tile height."""
+    announce("grouped matmul, every tile shape", counts, act)
+    rng = np.random.default_rng(len(counts))
+    m, k, n = sum(counts) + 3, 128, 16976
+    out = torch.float16 if act == abi.MM_ACT_FASTER_GELU else torch.bfloat16
+    if act == abi.MM_ACT_SWIGLU:
+        x, w = rand_i8(rng, (m, k)), rand_i8(rng, (len(counts), k, n))
+        cs = rng.uniform(1e-4, 1e-3, (len(counts), n)).astype(np.float32)
+        ts = rng.uniform(1e-2, 1e-1, m).astype(np.float32)
+        gl = np.asarray(counts, dtype=np.int64)
+        y = torch.zeros((m, n // 2), dtype=out, device=DEV)
+        y.view(torch.int16).fill_(0x7E7E)
+        ops.quant_group_matmul(y, to_dev(x), to_dev(w), to_dev(gl), to_dev(cs), to_dev(ts), None, abi.GROUP_LIST_COUNTS,
+                               act, act_beta=1.0)
+        torch.cuda.synchronize()
+        mm = abi.MatmulDesc(m=m, n=n, k=k, out_dtype=abi.BF16, quant_mode=abi.MM_QUANT_VECTOR,
+                            scale_format=abi.MM_SCALE_F32, has_tok_scale=1, activation=act, act_beta=1.0)
+        orc.set_threads(16)
+        want = orc.group_matmul_w8a8(abi.GroupMatmulDesc(mm=mm, groups=len(counts), group_list_kind=abi.GROUP_LIST_COUNTS),
+                                     x, w, None, cs, ts, gl, fill=0x7E7E)
+        got = bits(y)
+        assert np.all(got[sum(counts):] == 0x7E7E)
+        rows = sum(counts)
+        assert max_ulp(got[:rows], want.view(np.uint16)[:rows], "bf16") <= 1  # expf differs by at most an ulp of fp32
+        assert np.mean(got[:rows] == want.view(np.uint16)[:rows]) > 0.98
+        return
+    got, want = run_group(m, k, n, counts, abi.GROUP_LIST_COUNTS, out, rng, act == abi.MM_ACT_NONE, act)
+    if act == abi.MM_ACT_NONE:
+        assert np.array_equal(got, want)
+    else:
+        assert np.all(got[sum(counts):] == 0x7E7E)
+        assert max_ulp(got[:sum(counts)], want[:sum(counts)]) <= 1
+
+
 # ------------------------------------------------------------------ W4A16
 def w4_case(rng, m, k, n, gs, has_offset):
     x = rng.standard_normal((m, k)).astype(np.float16)
