@@ -13,12 +13,12 @@ F16, BF16, F32, I8, I4, I32, U64, E8M0 = range(8)
 # ascq_policy
 PER_TENSOR, PER_CHANNEL, PER_TOKEN, PER_GROUP, PER_CHANNEL_PER_GROUP, PER_TOKEN_PER_GROUP = range(6)
 # ascq_round_mode (values of the reference's RoundMode enum)
-CAST_NONE, CAST_RINT, CAST_FLOOR, CAST_CEIL, CAST_ROUND, CAST_TRUNC = range(6)
+CAST_NONE, CAST_RINT, CAST_FLOOR, CAST_CEIL, CAST_ROUND, CAST_TRUNC, CAST_ODD, CAST_HYBRID = range(8)
 # ascq_quant_compute
 COMPUTE_F16, COMPUTE_SCALE_T, COMPUTE_F32 = range(3)
 # ascq_offset_kind
 OFFSET_NONE, OFFSET_SCALAR, OFFSET_TENSOR = range(3)
-QDST_I8, QDST_FP8_E4M3FN, QDST_FP8_E5M2, QDST_FP4_E2M1, QDST_FP4_E1M2 = range(5)
+QDST_I8, QDST_FP8_E4M3FN, QDST_FP8_E5M2, QDST_FP4_E2M1, QDST_FP4_E1M2, QDST_HIF8 = range(6)
 # ascq_dequant_mode
 DEQUANT_WITH_SINGLE_ROW, DEQUANT_WITH_MULTI_ROW = range(2)
 # ascq_mm_*

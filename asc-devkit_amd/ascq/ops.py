@@ -63,12 +63,15 @@ def _quant(desc, dst, src, scale, offset):
     return dst
 
 
-def ascend_quant(dst, src, scale, offset, cal_count=None, scale_count=None, offset_count=None):
+def ascend_quant(dst, src, scale, offset, cal_count=None, scale_count=None, offset_count=None, dst_format=None):
     """AscendQuant<T>(dst, src, scale, offset, [scaleCount, offsetCount,] calCount): per-tensor when `scale` is a
     float, per-channel when it is a tensor (offset: float or tensor).  Every intermediate is fp16.
+    dst_format=abi.QDST_HIF8: dst is a uint8 tensor of hifloat8 codes (the half chain, then the cast that rounds ties
+    away from zero: ascend_quant_3510_impl.h:82-111).
     ref: include/adv_api/quantization/ascend_quant.h:63-347."""
     cal = src.numel() if cal_count is None else cal_count
-    d = abi.QuantDesc(src_dtype=_dt(src), compute=abi.COMPUTE_F16, round_mode=abi.CAST_RINT, k_dim=1, cal_count=cal)
+    d = abi.QuantDesc(src_dtype=_dt(src), compute=abi.COMPUTE_F16, round_mode=abi.CAST_RINT, k_dim=1, cal_count=cal,
+                      dst_format=abi.QDST_I8 if dst_format is None else dst_format)
     if torch.is_tensor(scale):
         n = scale.numel() if scale_count is None else scale_count
         d.policy, d.scale_dtype, d.n = abi.PER_CHANNEL, _dt(scale), n
@@ -108,14 +111,17 @@ def ascend_quant_policy(dst, src, scale, offset, para, policy, config=AscendQuan
     arithmetic in the scale's dtype for an int8 dst, in fp32 for a torch.float8_e4m3fn / float8_e5m2 dst.
     dst_format=abi.QDST_FP4_E2M1 / QDST_FP4_E1M2 (PER_GROUP only): dst is a uint8 tensor of cal_count / 2 bytes, two
     4-bit floats per byte with the even element in the low nibble (fp4x2_e2m1_t / fp4x2_e1m2_t).
+    dst_format=abi.QDST_HIF8: dst is a uint8 tensor of hifloat8 codes; arithmetic in the scale's dtype as for int8,
+    config.round_mode CAST_ROUND (CAST_HYBRID is refused).
     ref: include/adv_api/quantization/ascend_quant.h:667-762."""
     return _policy_quant(abi.COMPUTE_SCALE_T, dst, src, scale, offset, para, policy, config, dst_format)
 
 
-def quantize(dst, src, scale, offset, para, policy, config=AscendQuantConfig()):
-    """Quantize<config>(dst, src, scale, offset, params): always fp32 arithmetic, any policy.
+def quantize(dst, src, scale, offset, para, policy, config=AscendQuantConfig(), dst_format=None):
+    """Quantize<config>(dst, src, scale, offset, params): always fp32 arithmetic, any policy; dst_format=abi.QDST_HIF8
+    for hifloat8 codes in a uint8 dst.
     ref: include/adv_api/quantization/quantize.h, impl/adv_api/detail/quantization/quantize/quantize_impl.h:923-968."""
-    return _policy_quant(abi.COMPUTE_F32, dst, src, scale, offset, para, policy, config)
+    return _policy_quant(abi.COMPUTE_F32, dst, src, scale, offset, para, policy, config, dst_format)
 
 
 def dynamic_quant_per_token(x, q=None, tok_scale=None):
@@ -242,12 +248,13 @@ def ascend_antiquant_policy(dst, src, scale, offset, para, policy, config=Ascend
     return _antiquant_policy(abi.COMPUTE_SCALE_T, dst, src, scale, offset, para, policy, config, src_format)
 
 
-def antiquantize(dst, src, scale, offset, para, policy, config=AscendAntiQuantConfig()):
+def antiquantize(dst, src, scale, offset, para, policy, config=AscendAntiQuantConfig(), src_format=None):
     """AntiQuantize<config>(dst, src, scale, offset, params): fp32 arithmetic whatever the parameter type, any policy.
     PER_TENSOR takes Python floats (values of the output's type), PER_CHANNEL tensors [n] of the output's type.
+    src_format=abi.QDST_HIF8: src is a uint8 tensor of hifloat8 codes.
     ref: include/adv_api/quantization/antiquantize.h:59-95, impl/adv_api/detail/quantization/antiquantize/
     antiquantize_impl.h:36-135."""
-    return _antiquant_policy(abi.COMPUTE_F32, dst, src, scale, offset, para, policy, config)
+    return _antiquant_policy(abi.COMPUTE_F32, dst, src, scale, offset, para, policy, config, src_format)
 
 
 def dequantize(dst, src, scale, para, policy, k_dim=1):

@@ -59,6 +59,85 @@ __device__ __forceinline__ uint32_t f32_to_half_bits_sat(float f)
     return f32_to_half_bits((f != f) ? f : c);
 }
 
+// fp32 -> hifloat8, RoundMode::CAST_ROUND (nearest on the grid of the value's own exponent, ties away from zero; a
+// mantissa that rounds up past all-ones carries into the exponent), saturating: NaN -> 0, magnitudes from 1.25 * 2^15
+// on (infinity included) -> the largest finite code 0x6E, below 1.5 * 2^-23 -> 0 without sign.  Mantissa bits: 3 for
+// |e| <= 3, 2 for |e| <= 7, 1 up to 15, none for the powers of two 2^-22 .. 2^-16 (codes 1..7).
+__device__ __forceinline__ uint32_t f32_to_hif8_sat(float f)
+{
+    const uint32_t u = __float_as_uint(f), au = u & 0x7FFFFFFFu, sign = (u >> 24) & 0x80u;
+    if (au > 0x7F800000u) {
+        return 0u;
+    }
+    if (au >= 0x47200000u) {  // 1.25 * 2^15
+        return sign | 0x6Eu;
+    }
+    int e = static_cast<int>(au >> 23) - 127;
+    if (e < -23) {
+        return 0u;
+    }
+    const int ae0 = e < 0 ? -e : e;
+    const int mbits = e < -15 ? 0 : ae0 <= 3 ? 3 : ae0 <= 7 ? 2 : 1;
+    const uint32_t tmp = (au & 0x7FFFFFu) >> (22 - mbits);  // the mantissa and one more bit
+    uint32_t mant = (tmp + 1u) >> 1;
+    if (tmp == (2u << mbits) - 1u) {
+        mant = 0u;
+        e += 1;
+    }
+    if (e < -22) {
+        return 0u;
+    }
+    const uint32_t ae = static_cast<uint32_t>(e < 0 ? -e : e), neg = e < 0 ? 1u : 0u;
+    uint32_t code;
+    if (e < -15) {
+        code = static_cast<uint32_t>(e + 23);
+    } else if (ae == 0u) {
+        code = 0x08u | mant;
+    } else if (ae == 1u) {
+        code = 0x10u | (neg << 3) | mant;
+    } else if (ae <= 3u) {
+        code = 0x20u | (neg << 4) | ((ae - 2u) << 3) | mant;
+    } else if (ae <= 7u) {
+        // a carry from exponent 3 (three mantissa bits) arrives with mant = 0, as does one from -8
+        code = 0x40u | (neg << 4) | ((ae - 4u) << 2) | mant;
+    } else {
+        code = 0x60u | (neg << 4) | ((ae - 8u) << 1) | mant;
+    }
+    return sign | code;
+}
+
+// hifloat8 -> fp32 (exact): 0x80 is NaN, 0x6F / 0xEF the infinities.
+__device__ __forceinline__ float hif8_to_f32(uint32_t code)
+{
+    const uint32_t c = code & 0x7Fu;
+    if (c == 0u) {
+        return (code & 0x80u) ? __uint_as_float(0x7FC00000u) : 0.0f;
+    }
+    int e;
+    uint32_t mant23;  // the mantissa, left-aligned in the 23 fraction bits of a float
+    if (c < 8u) {
+        e = static_cast<int>(c) - 23, mant23 = 0u;
+    } else if (c < 16u) {
+        e = 0, mant23 = (c & 7u) << 20;
+    } else if (c < 32u) {
+        e = (c & 8u) ? -1 : 1, mant23 = (c & 7u) << 20;
+    } else if (c < 64u) {
+        const int f = static_cast<int>((c >> 3) & 3u);
+        e = f >= 2 ? -f : f + 2, mant23 = (c & 7u) << 20;
+    } else if (c < 96u) {
+        const int f = static_cast<int>((c >> 2) & 7u);
+        e = f >= 4 ? -f : f + 4, mant23 = (c & 3u) << 21;
+    } else {
+        const int f = static_cast<int>((c >> 1) & 15u);
+        e = f >= 8 ? -f : f + 8, mant23 = (c & 1u) << 22;
+    }
+    uint32_t bits = (static_cast<uint32_t>(e + 127) << 23) | mant23;
+    if (c == 0x6Fu) {
+        bits = 0x7F800000u;
+    }
+    return __uint_as_float(bits | ((code & 0x80u) << 24));
+}
+
 // Round a value (already exact in fp32) to an integer with the given mode and saturate to int8.
 template <bool kRint>
 __device__ __forceinline__ int round_sat8(float v, int round_mode)

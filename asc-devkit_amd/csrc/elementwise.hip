@@ -51,14 +51,18 @@ struct QuantArgs {
     int dst_format;  // ascq_quant_dst
 };
 
-// the last step: int8 with the requested rounding, or an 8-bit float (always half-even, saturating)
+// the last step: int8 with the requested rounding, hifloat8 (ties away from zero, saturating), or an 8-bit float
+// (always half-even, saturating)
 template <bool kRint>
 __device__ __forceinline__ int quant_final(float t, const QuantArgs& a)
 {
     if (a.dst_format == ASCQ_QDST_I8) {
         return round_sat8<kRint>(t, a.round_mode);
     }
-    if (a.dst_format >= ASCQ_QDST_FP4_E2M1) {
+    if (a.dst_format == ASCQ_QDST_HIF8) {
+        return static_cast<int>(f32_to_hif8_sat(t));
+    }
+    if (a.dst_format == ASCQ_QDST_FP4_E2M1 || a.dst_format == ASCQ_QDST_FP4_E1M2) {
         // through bfloat16 (half-even), then the 4-bit float with the requested rounding
         const float b = bf16_bits_to_f32(f32_to_bf16_bits(t));
         return static_cast<int>(a.dst_format == ASCQ_QDST_FP4_E1M2 ? f32_to_fp4_sat<true>(b, a.round_mode)
@@ -170,7 +174,7 @@ __global__ __launch_bounds__(kThreads) void quant_vec_kernel(QuantArgs a)
                 }
                 q[e] = quant_final<kRint>(t, a);
             }
-            if (a.dst_format >= ASCQ_QDST_FP4_E2M1) {
+            if (a.dst_format == ASCQ_QDST_FP4_E2M1 || a.dst_format == ASCQ_QDST_FP4_E1M2) {
                 // two codes per byte, the even element in the low nibble: 8 columns are one dword
                 uint32_t out = 0;
 #pragma unroll
@@ -823,12 +827,15 @@ struct AntiQuantPolicyArgs {
     float sscale, soffset;  // PER_TENSOR
 };
 
-// int8 / fp8_e4m3fn / fp8_e5m2 byte -> fp32 (exact); the 8-bit floats go through the hardware converters
+// int8 / fp8_e4m3fn / fp8_e5m2 / hifloat8 byte -> fp32 (exact); the OCP 8-bit floats go through the hardware converters
 __device__ __forceinline__ float decode_b8(uint32_t word, int byte, int fmt)
 {
     const uint32_t b = (word >> (8 * byte)) & 0xFFu;
     if (fmt == ASCQ_QDST_I8) {
         return static_cast<float>(static_cast<int8_t>(b));
+    }
+    if (fmt == ASCQ_QDST_HIF8) {
+        return hif8_to_f32(b);
     }
     return fmt == ASCQ_QDST_FP8_E5M2 ? __builtin_amdgcn_cvt_f32_bf8(static_cast<int>(b), 0)
                                      : __builtin_amdgcn_cvt_f32_fp8(static_cast<int>(b), 0);
@@ -1021,13 +1028,15 @@ extern "C" int ascq_quant(const ascq_quant_desc* d, void* dst, const void* src, 
     ASCQ_REQUIRE(d->compute >= ASCQ_COMPUTE_F16 && d->compute <= ASCQ_COMPUTE_F32, ASCQ_EINVAL,
                  "ascq_quant: unknown compute mode %d", d->compute);
     ASCQ_REQUIRE(d->round_mode >= ASCQ_CAST_NONE && d->round_mode <= ASCQ_CAST_TRUNC, ASCQ_EUNSUPPORTED,
-                 "ascq_quant: round mode %d is not supported for int8 output", d->round_mode);
+                 "ascq_quant: round mode %d is not supported (CAST_ODD belongs to no quantisation operator; CAST_HYBRID, "
+                 "for hifloat8 outputs, has no usable specification in the reference)", d->round_mode);
     ASCQ_REQUIRE(d->offset_kind >= ASCQ_OFFSET_NONE && d->offset_kind <= ASCQ_OFFSET_TENSOR, ASCQ_EINVAL,
                  "ascq_quant: unknown offset kind %d", d->offset_kind);
-    ASCQ_REQUIRE(d->dst_format >= ASCQ_QDST_I8 && d->dst_format <= ASCQ_QDST_FP4_E1M2, ASCQ_EUNSUPPORTED,
-                 "ascq_quant: destination format %d is not int8 / fp8_e4m3fn / fp8_e5m2 / fp4_e2m1 / fp4_e1m2",
+    ASCQ_REQUIRE(d->dst_format >= ASCQ_QDST_I8 && d->dst_format <= ASCQ_QDST_HIF8, ASCQ_EUNSUPPORTED,
+                 "ascq_quant: destination format %d is not int8 / fp8_e4m3fn / fp8_e5m2 / fp4_e2m1 / fp4_e1m2 / hifloat8",
                  d->dst_format);
-    const bool fp4 = d->dst_format >= ASCQ_QDST_FP4_E2M1;
+    const bool fp4 = d->dst_format == ASCQ_QDST_FP4_E2M1 || d->dst_format == ASCQ_QDST_FP4_E1M2;
+    const bool hif8 = d->dst_format == ASCQ_QDST_HIF8;
     if (fp4) {
         // ref: AscendQuant.md table 4 (the fp4x2 rows), ascend_quant_per_group_3510_impl.h:1383-1385
         ASCQ_REQUIRE(d->policy == ASCQ_PER_GROUP && d->compute == ASCQ_COMPUTE_SCALE_T, ASCQ_EUNSUPPORTED,
@@ -1035,8 +1044,9 @@ extern "C" int ascq_quant(const ascq_quant_desc* d, void* dst, const void* src, 
         ASCQ_REQUIRE(d->src_dtype != ASCQ_F32, ASCQ_EUNSUPPORTED,
                      "ascq_quant: fp4 destinations take half / bfloat16 sources");
     }
-    ASCQ_REQUIRE(d->dst_format == ASCQ_QDST_I8 || d->compute != ASCQ_COMPUTE_F16, ASCQ_EUNSUPPORTED,
-                 "ascq_quant: the fp16 contract (AscendQuant per tensor / per channel) has int8 output only");
+    // ref: ascend_quant_3510_impl.h:69-111 ("pertensor process for int8/hif8 output": the half chain, then the cast)
+    ASCQ_REQUIRE(d->dst_format == ASCQ_QDST_I8 || hif8 || d->compute != ASCQ_COMPUTE_F16, ASCQ_EUNSUPPORTED,
+                 "ascq_quant: the fp16 contract (AscendQuant per tensor / per channel) has int8 and hifloat8 outputs only");
     const bool tensor_scale = d->policy != ASCQ_PER_TENSOR;
     int par = tensor_scale ? d->scale_dtype : ASCQ_F32;
     if (tensor_scale) {
@@ -1120,7 +1130,7 @@ extern "C" int ascq_quant(const ascq_quant_desc* d, void* dst, const void* src, 
     // 8-bit float outputs are computed in fp32 whatever the parameter type
     const int ct = d->compute == ASCQ_COMPUTE_F16
                        ? ASCQ_F16
-                       : ((d->compute == ASCQ_COMPUTE_F32 || (d->dst_format != ASCQ_QDST_I8 && !fp4)) ? ASCQ_F32 : par);
+                       : ((d->compute == ASCQ_COMPUTE_F32 || (d->dst_format != ASCQ_QDST_I8 && !fp4 && !hif8)) ? ASCQ_F32 : par);
     if (!tensor_scale) {
         ASCQ_Q(ASCQ_F16, ASCQ_F32, ASCQ_F16)
         ASCQ_Q(ASCQ_BF16, ASCQ_F32, ASCQ_F16)
@@ -1359,10 +1369,10 @@ extern "C" int ascq_antiquant_policy(const ascq_antiquant_policy_desc* d, void* 
                      "ascq_antiquant_policy: PER_TENSOR / PER_CHANNEL take half or bfloat16 parameters of the output's "
                      "type (scale dtype %d, dst dtype %d)", d->scale_dtype, d->dst_dtype);
     }
-    ASCQ_REQUIRE(d->src_format >= ASCQ_QDST_I8 && d->src_format <= ASCQ_QDST_FP4_E1M2, ASCQ_EUNSUPPORTED,
-                 "ascq_antiquant_policy: source format %d is not int8 / fp8_e4m3fn / fp8_e5m2 / fp4_e2m1 / fp4_e1m2",
-                 d->src_format);
-    if (d->src_format >= ASCQ_QDST_FP4_E2M1) {
+    ASCQ_REQUIRE(d->src_format >= ASCQ_QDST_I8 && d->src_format <= ASCQ_QDST_HIF8, ASCQ_EUNSUPPORTED,
+                 "ascq_antiquant_policy: source format %d is not int8 / fp8_e4m3fn / fp8_e5m2 / fp4_e2m1 / fp4_e1m2 / "
+                 "hifloat8", d->src_format);
+    if (d->src_format == ASCQ_QDST_FP4_E2M1 || d->src_format == ASCQ_QDST_FP4_E1M2) {
         // ref: AscendAntiQuant.md table 3 (the fp4x2 rows), antiquantize_impl.h:53-58
         ASCQ_REQUIRE(d->policy == ASCQ_PER_GROUP, ASCQ_EUNSUPPORTED,
                      "ascq_antiquant_policy: fp4 sources exist for PER_GROUP only");

@@ -66,7 +66,14 @@ typedef enum ascq_round_mode {
     ASCQ_CAST_FLOOR = 2,
     ASCQ_CAST_CEIL = 3,
     ASCQ_CAST_ROUND = 4, /* half away from zero */
-    ASCQ_CAST_TRUNC = 5
+    ASCQ_CAST_TRUNC = 5,
+    /* Declared so that they can be named and refused (ASCQ_EUNSUPPORTED): no operator of this library documents ODD,
+     * and HYBRID (hifloat8 destinations only) has no usable specification in the reference: its one executable
+     * statement, examples/.../matmul_fp8/scripts/hif8.py, rounds exactly representable values upward in its float32
+     * path (:121-140: the comparison of the discarded bits with their own low half holds for 0 >= 0) and drops the
+     * carry into the exponent in its float16 path (:160-178). */
+    ASCQ_CAST_ODD = 6,
+    ASCQ_CAST_HYBRID = 7
 } ascq_round_mode;
 
 /* Which arithmetic contract AscendQuant follows (the reference has three). */
@@ -89,7 +96,16 @@ typedef enum ascq_quant_dst {
      * int4x2 and both fp4x2 types together: docs/zh/api/SIMD-API/C-API/reg/reg_data_types/data_type_definition.md:17):
      * sign, then e2m1 (bias 1; 0, 0.5, 1, 1.5, 2, 3, 4, 6) or e1m2 (bias 1; 0, 0.25 .. 1.75 in steps of 0.25). */
     ASCQ_QDST_FP4_E2M1 = 3,
-    ASCQ_QDST_FP4_E1M2 = 4
+    ASCQ_QDST_FP4_E1M2 = 4,
+    /* hifloat8_t: sign, a prefix-coded field that says how many exponent bits follow, a sign-magnitude exponent and
+     * 3 / 3 / 3 / 2 / 1 mantissa bits for |exponent| 0 / 1 / 2-3 / 4-7 / 8-15; codes 1..7 are 2^-22 .. 2^-16; 0x80 is
+     * NaN, 0x6F / 0xEF the infinities, 0x6E = 2^15 the largest finite value (the codec the reference ships as
+     * examples/01_simd_cpp_api/04_advanced_api/00_matmul/matmul_fp8/scripts/hif8.py).  As a destination (AscendQuant
+     * per tensor / per channel / PER_TOKEN / PER_GROUP, Quantize: AscendQuant.md table 4) the value is computed like
+     * the int8 result, in the same arithmetic type, then cast with RoundMode::CAST_ROUND (nearest, ties away from
+     * zero), saturating: every round mode except HYBRID means that cast, as in the reference
+     * (ascend_quant_3510_impl.h:900-933). */
+    ASCQ_QDST_HIF8 = 5
 } ascq_quant_dst;
 
 typedef enum ascq_offset_kind { ASCQ_OFFSET_NONE = 0, ASCQ_OFFSET_SCALAR = 1, ASCQ_OFFSET_TENSOR = 2 } ascq_offset_kind;

@@ -57,6 +57,9 @@ struct fp8_e4m3fn_t {
 struct fp8_e5m2_t {
     uint8_t bits;
 };
+struct hifloat8_t {  // see ASCQ_QDST_HIF8 for the encoding
+    uint8_t bits;
+};
 struct fp8_e8m0_t {  // a power of two: 2^(bits - 127); the scales of the fp4 sources of AscendAntiQuant
     uint8_t bits;
 };
@@ -81,6 +84,10 @@ struct QuantDstOf<fp8_e4m3fn_t> {
 template <>
 struct QuantDstOf<fp8_e5m2_t> {
     static constexpr int32_t value = ASCQ_QDST_FP8_E5M2;
+};
+template <>
+struct QuantDstOf<hifloat8_t> {
+    static constexpr int32_t value = ASCQ_QDST_HIF8;
 };
 template <>
 struct QuantDstOf<fp4x2_e2m1_t> {  // AscendQuant PER_GROUP only
@@ -142,7 +149,7 @@ private:
 };
 
 // ref: include/adv_api/quantization/ascend_quant_utils.h:31-87
-enum class RoundMode : int32_t { CAST_NONE = 0, CAST_RINT, CAST_FLOOR, CAST_CEIL, CAST_ROUND, CAST_TRUNC };
+enum class RoundMode : int32_t { CAST_NONE = 0, CAST_RINT, CAST_FLOOR, CAST_CEIL, CAST_ROUND, CAST_TRUNC, CAST_ODD, CAST_HYBRID };
 // ref: include/adv_api/quantization/ascend_quant_utils.h:73-80 (same members, same values; the two combined policies are
 // declared there and implemented by none of the reference's operators: ascq_quant answers ASCQ_EUNSUPPORTED)
 enum class AscendQuantPolicy : int32_t { PER_TENSOR, PER_CHANNEL, PER_TOKEN, PER_GROUP, PER_CHANNEL_PER_GROUP, PER_TOKEN_PER_GROUP };

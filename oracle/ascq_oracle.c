@@ -309,6 +309,77 @@ float orc_fp8_to_f32(uint8_t code, int e5m2)
     return (float)((code & 0x80) ? -v : v);
 }
 
+/* ---- hifloat8: sign, a prefix-coded "dot" field that says how many exponent bits follow (0-4), a sign-magnitude
+ * exponent and 3 / 3 / 3 / 2 / 1 mantissa bits for |exponent| 0 / 1 / 2-3 / 4-7 / 8-15; codes 1..7 are the powers of two
+ * 2^-22 .. 2^-16 without mantissa; 0 is zero, 0x80 NaN, 0x6F / 0xEF the infinities; the largest finite value is
+ * 2^15 (0x6E).  ref: examples/01_simd_cpp_api/04_advanced_api/00_matmul/matmul_fp8/scripts/hif8.py:387-468
+ * (cvt_hifuint8_to_float, over_mode True). */
+float orc_hif8_to_f32(uint8_t code)
+{
+    int c = code & 0x7F, e;
+    double m;
+    if (c == 0) {
+        return code == 0x80 ? NAN : 0.0f;
+    }
+    if (c == 0x6F) {
+        return (code & 0x80) ? -INFINITY : INFINITY;
+    }
+    if (c < 8) {
+        e = c - 23, m = 1.0;
+    } else if (c < 16) {
+        e = 0, m = 1.0 + (c & 7) / 8.0;
+    } else if (c < 32) {
+        e = (c & 8) ? -1 : 1, m = 1.0 + (c & 7) / 8.0;
+    } else if (c < 64) {
+        int f = (c >> 3) & 3;
+        e = f >= 2 ? -f : f + 2, m = 1.0 + (c & 7) / 8.0;
+    } else if (c < 96) {
+        int f = (c >> 2) & 7;
+        e = f >= 4 ? -f : f + 4, m = 1.0 + (c & 3) / 4.0;
+    } else {
+        int f = (c >> 1) & 15;
+        e = f >= 8 ? -f : f + 8, m = 1.0 + (c & 1) / 2.0;
+    }
+    double v = ldexp(m, e);
+    return (float)((code & 0x80) ? -v : v);
+}
+
+/* fp32 (or any narrower float, widened exactly) -> hifloat8 with RoundMode::CAST_ROUND, the cast's "round to nearest,
+ * ties away from zero" (hif8.py:104-118 keeps one bit more than the mantissa and rounds an odd value up), written
+ * here as a search over the code values rather than on the bits.  Between 2^-23 and 2^-22 the script rounds on the
+ * grid of powers of two and then flushes 2^-23 to zero (:353-361), so the tie point of the smallest code is
+ * 1.5 * 2^-23.  Saturating (SatMode::SAT, the trait every quantisation operator passes,
+ * ascend_quant_per_group_3510_impl.h:100-101): magnitudes from 1.25 * 2^15 on, infinities included, give the largest
+ * finite code, NaN gives 0 (hif8.py:198-214,318-331 with over_mode False); zero and everything that rounds to it
+ * lose their sign. */
+uint8_t orc_f32_to_hif8(float f)
+{
+    if (f != f) {
+        return 0;
+    }
+    uint8_t sign = signbit(f) ? 0x80 : 0;
+    double a = fabs((double)f);
+    if (a >= 1.25 * 32768.0) {
+        return (uint8_t)(sign | 0x6E);
+    }
+    if (a < ldexp(1.5, -23)) {
+        return 0;
+    }
+    int best = 1;
+    double best_d = fabs(a - (double)orc_hif8_to_f32(1));
+    for (int c = 2; c <= 0x7F; ++c) {
+        if (c == 0x6F) {
+            continue; /* infinity */
+        }
+        double v = (double)orc_hif8_to_f32((uint8_t)c), dd = fabs(a - v);
+        double bv = (double)orc_hif8_to_f32((uint8_t)best);
+        if (dd < best_d || (dd == best_d && v > bv)) {
+            best = c, best_d = dd;
+        }
+    }
+    return (uint8_t)(sign | best);
+}
+
 static inline float load_as_f32(const void* p, size_t i, int dtype)
 {
     switch (dtype) {
@@ -373,8 +444,9 @@ int orc_quant(const ascq_quant_desc* d, int8_t* dst, const void* src, const void
     size_t rows = total / n;
     int comp = d->compute;
     int ctype = (comp == ASCQ_COMPUTE_F16) ? ASCQ_F16 : (comp == ASCQ_COMPUTE_F32 ? ASCQ_F32 : d->scale_dtype);
-    if (d->dst_format != ASCQ_QDST_I8) {
-        ctype = ASCQ_F32; /* the 8-bit float paths widen everything to fp32:
+    if (d->dst_format != ASCQ_QDST_I8 && d->dst_format != ASCQ_QDST_HIF8) {
+        ctype = ASCQ_F32; /* the fp8 paths widen everything to fp32 (hifloat8 is computed like int8, in the scale type:
+                             ascend_quant_per_group_3510_impl.h:93-127, ascend_quant_3510_impl.h:82-111):
                              ascend_quant_per_group_3510_impl.h:54-74, quantize_impl.h:64-73 */
     }
     int rmode = (comp == ASCQ_COMPUTE_F16) ? ASCQ_CAST_RINT : d->round_mode;
@@ -426,6 +498,9 @@ int orc_quant(const ascq_quant_desc* d, int8_t* dst, const void* src, const void
             }
             if (d->dst_format == ASCQ_QDST_I8) {
                 dst[e] = orc_round_sat8(v, rmode);
+            } else if (d->dst_format == ASCQ_QDST_HIF8) {
+                dst[e] = (int8_t)orc_f32_to_hif8((float)v); /* every round mode but HYBRID means CAST_ROUND here:
+                                                               ascend_quant_3510_impl.h:900-933 */
             } else if (fp4) {
                 /* to bfloat16 first (half-even), then to the 4-bit float with the requested rounding; two codes per
                  * byte, the even element in the low nibble.  Rows are whole bytes (n is even). */
@@ -944,8 +1019,9 @@ int orc_antiquant_policy(const ascq_antiquant_policy_desc* d, void* dst, const u
             } else {
                 pi = (i / d->group_size) * n + j;
             }
-            float x = d->src_format == ASCQ_QDST_I8 ? (float)(int8_t)src[e]
-                                                    : orc_fp8_to_f32(src[e], d->src_format == ASCQ_QDST_FP8_E5M2);
+            float x = d->src_format == ASCQ_QDST_I8     ? (float)(int8_t)src[e]
+                      : d->src_format == ASCQ_QDST_HIF8 ? orc_hif8_to_f32(src[e])
+                                                        : orc_fp8_to_f32(src[e], d->src_format == ASCQ_QDST_FP8_E5M2);
             float s, o = 0.0f;
             if (d->policy == ASCQ_PER_TENSOR) {
                 /* scalars of the output's type (antiquantize_3510_impl.h:253-283) */

@@ -30,6 +30,8 @@ float orc_quant_word_scale(uint64_t w, int scale_format);
 
 uint8_t orc_f32_to_fp8(float f, int e5m2);
 float orc_fp8_to_f32(uint8_t code, int e5m2);
+uint8_t orc_f32_to_hif8(float f);
+float orc_hif8_to_f32(uint8_t code);
 uint8_t orc_f32_to_fp4(float f, int e1m2, int round_mode);
 float orc_fp4_to_f32(uint8_t code, int e1m2);
 int orc_quant(const ascq_quant_desc* d, int8_t* dst, const void* src, const void* scale, const void* offset);

@@ -53,6 +53,10 @@ def lib():
         L.orc_f32_to_fp4.argtypes = [C.c_float, C.c_int, C.c_int]
         L.orc_fp4_to_f32.restype = C.c_float
         L.orc_fp4_to_f32.argtypes = [C.c_uint8, C.c_int]
+        L.orc_f32_to_hif8.restype = C.c_uint8
+        L.orc_f32_to_hif8.argtypes = [C.c_float]
+        L.orc_hif8_to_f32.restype = C.c_float
+        L.orc_hif8_to_f32.argtypes = [C.c_uint8]
         L.orc_set_threads.argtypes = [C.c_int]
         L.orc_quant.argtypes = [C.POINTER(abi.QuantDesc), _P, _P, _P, _P]
         L.orc_dynamic_quant_per_token.argtypes = [C.c_int, C.c_uint32, C.c_uint32, _P, _P, _P]

@@ -346,6 +346,22 @@ def test_combined_policies_are_rejected_by_name():
     assert ops.AscendDeQuantPolicy.PER_TOKEN == 0 and ops.AscendDeQuantPolicy.PER_TOKEN_PER_GROUP == 3
 
 
+def test_hifloat8_surface_and_refused_round_modes():
+    """hifloat8 is a destination of ascq_quant and a source of ascq_antiquant_policy; CAST_HYBRID and CAST_ODD have
+    the reference's values (kernel_utils_mode.h:94-109) and are refused by name; format 6 does not exist."""
+    FAKE2 = C.c_void_p(0x100000)
+    assert (abi.CAST_ODD, abi.CAST_HYBRID, abi.QDST_HIF8) == (6, 7, 5)
+    for mode in (abi.CAST_ODD, abi.CAST_HYBRID):
+        assert L.ascq_quant(C.byref(q(round_mode=mode, dst_format=abi.QDST_HIF8)), FAKE, FAKE2, FAKE, FAKE, None) == abi.EUNSUPPORTED
+        assert "CAST_HYBRID" in err()
+    assert L.ascq_quant(C.byref(q(dst_format=6)), FAKE, FAKE2, FAKE, FAKE, None) == abi.EUNSUPPORTED and "hifloat8" in err()
+    aq = abi.AntiQuantPolicyDesc(policy=abi.PER_TOKEN, src_format=6, dst_dtype=abi.F16, scale_dtype=abi.F16, m=4, n=32,
+                                 cal_count=128)
+    assert L.ascq_antiquant_policy(C.byref(aq), FAKE, FAKE2, FAKE, None, None) == abi.EUNSUPPORTED and "hifloat8" in err()
+    hdr = open(os.path.join(ROOT, "include", "ascq.h")).read()
+    assert "ASCQ_QDST_HIF8 = 5" in hdr and "ASCQ_CAST_HYBRID = 7" in hdr
+
+
 def test_quant_word_with_pre_shift_bit_is_rejected():
     d = abi.MatmulDesc(m=16, n=32, k=64, out_dtype=abi.F16, quant_mode=abi.MM_QUANT_SCALAR, scale_format=abi.MM_SCALE_U64,
                        quant_scalar=(1 << 36) | (3 << 32) | (0x3F800000 & 0xFFFFE000))

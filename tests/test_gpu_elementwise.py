@@ -194,6 +194,85 @@ def test_quant_fp8(fmt, pair, policy):
             assert np.any((got[:cal] & 0x7F) == top_code)          # saturation was exercised
 
 
+@pytest.mark.parametrize("pair", PAIRS)
+@pytest.mark.parametrize("policy", ["token", "group0", "group1", "channel", "tensor"])
+def test_quant_hifloat8(pair, policy):
+    """hifloat8 outputs: arithmetic in the scale's type (PER_TOKEN / PER_GROUP) or in fp32 (Quantize), then the cast
+    that rounds ties away from zero and saturates: bit-exact against the oracle.  The scales spread the products from
+    below the smallest code (2^-22) to beyond the largest (2^15)."""
+    src_dt, sc_dt = pair
+    for (m, n, cal) in [(10, 288, 1152), (8, 512, 3584), (6, 36 * 8, 6 * 36 * 8)]:
+        announce("quant hifloat8", pair, policy, m, n, cal)
+        rng = np.random.default_rng(m + n + 5)
+        x, xd = src_array(rng, (m, n), src_dt, 1.0)
+        gs = 32
+        pol = {"token": abi.PER_TOKEN, "group0": abi.PER_GROUP, "group1": abi.PER_GROUP, "channel": abi.PER_CHANNEL,
+               "tensor": abi.PER_TENSOR}[policy]
+        k_dim = 0 if policy == "group0" else 1
+        sshape = {"token": (m,), "group0": (-(-m // gs), n), "group1": (m, -(-n // gs)), "channel": (n,),
+                  "tensor": (1,)}[policy]
+        s = np.exp(rng.uniform(np.log(1e-7), np.log(3e4), sshape)).astype(np.float32)
+        s.flat[0], s.flat[-1] = 6e4, 1e-7
+        o = rng.uniform(-1e-6, 1e-6, sshape).astype(np.float32)
+        (s, sdev), (o, odev) = typed(s, sc_dt), typed(o, sc_dt)
+        dst = torch.zeros((m, n), dtype=torch.uint8, device=DEV)
+        cfg = ops.AscendQuantConfig(has_offset=True, k_dim=k_dim, round_mode=abi.CAST_ROUND)
+        para = ops.AscendQuantParam(m=m, n=n, cal_count=cal, group_size=gs if pol == abi.PER_GROUP else 0)
+        d = abi.QuantDesc(policy=pol, src_dtype=src_dt, scale_dtype=sc_dt, compute=abi.COMPUTE_F32,
+                          round_mode=abi.CAST_ROUND, k_dim=k_dim, m=m, n=n, cal_count=cal,
+                          group_size=para.group_size, dst_format=abi.QDST_HIF8, offset_kind=abi.OFFSET_TENSOR)
+        if pol == abi.PER_TENSOR:
+            sv, ov = float(np.float32(3.7)), 0.25
+            ops.quantize(dst, xd, sv, ov, para, pol, cfg, dst_format=abi.QDST_HIF8)
+            d.scale, d.offset, d.offset_kind, d.scale_dtype = sv, ov, abi.OFFSET_SCALAR, src_dt
+            want = orc.quant(d, x.reshape(-1)[:cal].copy())
+        elif pol in (abi.PER_TOKEN, abi.PER_GROUP):
+            d.compute = abi.COMPUTE_SCALE_T
+            ops.ascend_quant_policy(dst, xd, sdev, odev, para, pol, cfg, dst_format=abi.QDST_HIF8)
+            want = orc.quant(d, x.reshape(-1)[:cal].copy(), s, o)
+        else:
+            ops.quantize(dst, xd, sdev, odev, para, pol, cfg, dst_format=abi.QDST_HIF8)
+            want = orc.quant(d, x.reshape(-1)[:cal].copy(), s, o)
+        got = dst.cpu().numpy().reshape(-1)
+        assert np.array_equal(got[:cal], want.view(np.uint8))
+        assert np.all(got[cal:] == 0)
+        if pol != abi.PER_TENSOR and cal == m * n:
+            # both ends were exercised: the largest code, and zero or the mantissa-less powers of two 2^-22 .. 2^-16
+            assert np.any((got[:cal] & 0x7F) == 0x6E) and np.any((got[:cal] & 0x7F) < 8)
+
+
+def test_hifloat8_cast_against_the_reference_script_vectors():
+    """The device's cast itself, not through the oracle: Quantize per tensor with scale 1 on the float32 inputs of the
+    committed vectors (the reference script's answers), and AscendQuant's half chain (scale 1, offset 0) on every
+    float16 value the script answers correctly; then AntiQuantize of all codes against the script's decoding."""
+    import os
+    announce("hifloat8 vectors")
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "hif8_vectors.npz"))
+    x = g["f32_in"][:-(g["f32_in"].size % 32) or None].copy()
+    n = 32
+    m = x.size // n
+    dst = torch.zeros((m, n), dtype=torch.uint8, device=DEV)
+    cfg = ops.AscendQuantConfig(has_offset=False, k_dim=1, round_mode=abi.CAST_ROUND)
+    ops.quantize(dst, to_dev(x.reshape(m, n)), 1.0, 0.0, ops.AscendQuantParam(m=m, n=n, cal_count=m * n, group_size=0),
+                 abi.PER_TENSOR, cfg, dst_format=abi.QDST_HIF8)
+    assert np.array_equal(dst.cpu().numpy().reshape(-1), g["f32_round"][:x.size])
+    halves = np.arange(65536, dtype=np.uint16).view(np.float16)
+    h32 = halves.astype(np.float32)
+    pinned = ~g["f16_round_raised"] & ~(h32 <= -40960.0) & ~np.isnan(h32)
+    dsth = torch.zeros(65536, dtype=torch.uint8, device=DEV)
+    ops.ascend_quant(dsth, to_dev(halves), 1.0, 0.0, dst_format=abi.QDST_HIF8)
+    assert np.array_equal(dsth.cpu().numpy()[pinned], g["f16_round"][pinned])
+    codes = np.arange(256, dtype=np.uint8).repeat(32).reshape(256, 32)
+    out = torch.zeros((256, 32), dtype=torch.float32, device=DEV)
+    ones = torch.ones(256, dtype=torch.float32, device=DEV)
+    ops.ascend_antiquant_policy(out, to_dev(codes), ones, None, ops.AscendAntiQuantParam(m=256, n=32, cal_count=256 * 32),
+                                abi.PER_TOKEN, ops.AscendAntiQuantConfig(has_offset=False), src_format=abi.QDST_HIF8)
+    got = out.cpu().numpy()[:, 0]
+    want = g["decode"]
+    fin = ~np.isnan(want)
+    assert np.array_equal(got[fin].view(np.uint32), want[fin].view(np.uint32)) and np.isnan(got[0x80])
+
+
 @pytest.mark.parametrize("fmt", [abi.QDST_FP4_E2M1, abi.QDST_FP4_E1M2])
 @pytest.mark.parametrize("pair", [(abi.F16, abi.F16), (abi.F16, abi.F32), (abi.BF16, abi.BF16), (abi.BF16, abi.F32)])
 @pytest.mark.parametrize("mode", [abi.CAST_RINT, abi.CAST_ROUND, abi.CAST_FLOOR, abi.CAST_CEIL, abi.CAST_TRUNC])
@@ -363,14 +442,15 @@ def test_antiquant(int4, dst_dt, transpose, K, N, G, has_offset):
 
 
 # ------------------------------------------------------------------ AscendAntiQuant PER_TOKEN / PER_GROUP
-B8 = {abi.QDST_I8: torch.int8, abi.QDST_FP8_E4M3FN: torch.float8_e4m3fn, abi.QDST_FP8_E5M2: torch.float8_e5m2}
+B8 = {abi.QDST_I8: torch.int8, abi.QDST_FP8_E4M3FN: torch.float8_e4m3fn, abi.QDST_FP8_E5M2: torch.float8_e5m2,
+      abi.QDST_HIF8: torch.uint8}
 AQP_TYPES = [(abi.F16, abi.F16, abi.COMPUTE_SCALE_T), (abi.BF16, abi.BF16, abi.COMPUTE_SCALE_T),
              (abi.F32, abi.F32, abi.COMPUTE_SCALE_T), (abi.F32, abi.F16, abi.COMPUTE_SCALE_T),
              (abi.F32, abi.BF16, abi.COMPUTE_SCALE_T), (abi.F16, abi.F16, abi.COMPUTE_F32),
              (abi.BF16, abi.F32, abi.COMPUTE_F32)]                     # (scale, dst, arithmetic)
 
 
-@pytest.mark.parametrize("fmt", [abi.QDST_I8, abi.QDST_FP8_E4M3FN, abi.QDST_FP8_E5M2])
+@pytest.mark.parametrize("fmt", [abi.QDST_I8, abi.QDST_FP8_E4M3FN, abi.QDST_FP8_E5M2, abi.QDST_HIF8])
 @pytest.mark.parametrize("types", AQP_TYPES)
 @pytest.mark.parametrize("mode", ["token", "group_n", "group_m", "group_m_via_transpose"])
 def test_antiquant_policy(fmt, types, mode):
@@ -386,6 +466,8 @@ def test_antiquant_policy(fmt, types, mode):
             codes[(codes & 0x7F) == 0x7F] = 0x3C
         elif fmt == abi.QDST_FP8_E5M2:
             codes[(codes & 0x7F) >= 0x7C] = 0x3C
+        elif fmt == abi.QDST_HIF8:
+            codes[(codes == 0x80) | ((codes & 0x7F) == 0x6F)] = 0x3C
         gs = 32
         policy = abi.PER_TOKEN if mode == "token" else abi.PER_GROUP
         k_dim, tr = {"token": (1, 0), "group_n": (1, 0), "group_m": (0, 0), "group_m_via_transpose": (1, 1)}[mode]
@@ -395,7 +477,7 @@ def test_antiquant_policy(fmt, types, mode):
         cfg = ops.AscendAntiQuantConfig(has_offset=has_offset, is_transpose=bool(tr), k_dim=k_dim)
         para = ops.AscendAntiQuantParam(m=m, n=n, cal_count=cal, group_size=gs if policy == abi.PER_GROUP else 0)
         fn = ops.ascend_antiquant_policy if compute == abi.COMPUTE_SCALE_T else ops.antiquantize
-        fn(dst, to_dev(codes).view(B8[fmt]), sdev, odev, para, policy, cfg)
+        fn(dst, to_dev(codes).view(B8[fmt]), sdev, odev, para, policy, cfg, src_format=fmt)
         d = abi.AntiQuantPolicyDesc(policy=policy, src_format=fmt, scale_dtype=sc_dt, dst_dtype=dst_dt, compute=compute,
                                     has_offset=int(has_offset), is_transpose=tr, k_dim=k_dim, m=m, n=n, cal_count=cal,
                                     group_size=para.group_size)

@@ -746,3 +746,39 @@ def test_swiglu_epilogue_is_the_reference_vector_chain():
     assert orc.lib().orc_swiglu(3.0, 0.0, 1.0) == 0.0
     assert orc.lib().orc_swiglu(2.0, 100.0, 1.0) == 200.0
     assert abs(orc.lib().orc_swiglu(2.0, -100.0, 1.0)) < 1e-40
+
+
+def test_hifloat8_codec_is_the_reference_script():
+    """hifloat8 has no document table in the reference; its codec ships as a Python script beside the fp8 matmul example
+    (matmul_fp8/scripts/hif8.py).  tests/golden/hif8_vectors.npz holds that script's answers (made by
+    tests/golden/make_hif8_vectors.py): the decoding of all 256 codes, the float32 encoder with "round" on 13,625 inputs
+    (every code value, every midpoint between neighbours and the float32 values beside them, the range ends, random
+    values) and the float16 encoder on all 65,536 halves.  The oracle's encoder is a nearest-value search, not the
+    script's bit arithmetic.  Outside the pin, because the script is wrong there: the 1,024 halves on which it raises
+    (a mantissa that rounds up into a smaller negative exponent: hif8.py:262-265 shifts by a negative count; the float32
+    path, which has no such shift, gives what the oracle gives), and negative float16 overflow (hif8.py:228-233 tests for
+    overflow before it has looked at the sign and answers with the positive code)."""
+    import os
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "hif8_vectors.npz"))
+    L = orc.lib()
+    dec = np.array([L.orc_hif8_to_f32(c) for c in range(256)], dtype=np.float32)
+    assert np.array_equal(np.isnan(dec), np.isnan(g["decode"])) and np.isnan(dec).sum() == 1 and np.isnan(dec[0x80])
+    ok = ~np.isnan(dec)
+    assert np.array_equal(dec[ok].view(np.uint32), g["decode"][ok].view(np.uint32))
+    enc = np.array([L.orc_f32_to_hif8(float(x)) for x in g["f32_in"]], dtype=np.uint8)
+    assert np.array_equal(enc, g["f32_round"])
+    # the non-saturating form of the script differs only where this one saturates: infinities and NaN
+    differs = enc != g["f32_round_inf"]
+    assert set(g["f32_round_inf"][differs].tolist()) <= {0x6F, 0xEF, 0x80}
+    halves = np.arange(65536, dtype=np.uint16).view(np.float16).astype(np.float32)
+    ench = np.array([L.orc_f32_to_hif8(float(x)) for x in halves], dtype=np.uint8)
+    pinned = ~g["f16_round_raised"] & ~(halves <= -40960.0)
+    assert pinned.sum() == 65536 - 1024 - int((halves <= -40960.0).sum())
+    assert np.array_equal(ench[pinned], g["f16_round"][pinned])
+    assert set(ench[halves <= -40960.0].tolist()) == {0xEE}             # the float32 path's answer for the same values
+    # what the mathematics fixes: encode(decode(c)) == c for every finite code; monotone in the value
+    finite = [c for c in range(256) if c not in (0x80, 0x6F, 0xEF)]
+    assert all(L.orc_f32_to_hif8(float(dec[c])) == c for c in finite)
+    xs = np.sort(np.abs(g["f32_in"][np.isfinite(g["f32_in"])]))
+    vals = np.array([L.orc_hif8_to_f32(L.orc_f32_to_hif8(float(x))) for x in xs])
+    assert np.all(np.diff(vals) >= 0)
