@@ -10,6 +10,7 @@
 
 #include "../../include/ascq_ascendc.hpp"
 #include "../../oracle/ascq_oracle.h"
+#include "../splitmix64.h"
 
 namespace {
 
@@ -24,17 +25,12 @@ int g_failed = 0;
         }                                                                               \
     } while (0)
 
-struct Rng {  // SplitMix64
-    uint64_t s;
-    uint64_t next()
-    {
-        uint64_t z = (s += 0x9E3779B97F4A7C15ull);
-        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
-        z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
-        return z ^ (z >> 31);
-    }
-    float uniform(float lo, float hi) { return lo + (hi - lo) * static_cast<float>(next() >> 40) / 16777216.0f; }
-    int integer(int lo, int hi) { return lo + static_cast<int>(next() % static_cast<uint64_t>(hi - lo + 1)); }
+struct Rng {  // the generator shared with the Python tests (tests/splitmix64.h)
+    splitmix64 g;
+    explicit Rng(uint64_t seed) : g{seed} {}
+    uint64_t next() { return splitmix64_next(&g); }
+    float uniform(float lo, float hi) { return splitmix64_uniform(&g, lo, hi); }
+    int integer(int lo, int hi) { return splitmix64_integer(&g, lo, hi); }
 };
 
 template <typename T>
@@ -81,12 +77,20 @@ std::vector<uint16_t> random_halves(Rng& r, size_t n, float lo, float hi)
     return v;
 }
 
-void test_quant_per_channel()
+// The first case's inputs and, with a GPU, its output as checksums: tests/test_gpu_cpp_host.py draws the same inputs
+// with the Python generator, runs the same operator through the Python mirror and must arrive at the same numbers.
+void test_quant_per_channel(bool inputs_only)
 {
     std::printf("[case] AscendQuant<half> per channel 64x256\n");
     Rng r{1};
     const uint32_t m = 64, n = 256;
     auto x = random_halves(r, m * n, -6.0f, 6.0f), s = random_halves(r, n, 5.0f, 40.0f), o = random_halves(r, n, -3.0f, 3.0f);
+    std::printf("[inputs] quant_per_channel x=%016llx s=%016llx o=%016llx\n",
+                (unsigned long long)fnv1a64(x.data(), x.size() * 2), (unsigned long long)fnv1a64(s.data(), s.size() * 2),
+                (unsigned long long)fnv1a64(o.data(), o.size() * 2));
+    if (inputs_only) {
+        return;
+    }
     DeviceBuffer<uint16_t> dx(x), ds(s), dof(o);
     DeviceBuffer<int8_t> dq(m * n);
     ascq::AscendQuant<ascq::half>(dq.view<int8_t>(m * n), dx.view<ascq::half>(m * n), ds.view<ascq::half>(n),
@@ -103,6 +107,10 @@ void test_quant_per_channel()
     std::vector<int8_t> want(m * n);
     orc_quant(&d, want.data(), x.data(), s.data(), o.data());
     expect_equal("AscendQuant per channel", dq.download(), want);
+    {
+        auto q = dq.download();
+        std::printf("[output] quant_per_channel q=%016llx\n", (unsigned long long)fnv1a64(q.data(), q.size()));
+    }
 
     std::printf("[case] AscendQuant<half> per tensor 1024\n");
     ascq::AscendQuant<ascq::half>(dq.view<int8_t>(1024), dx.view<ascq::half>(1024), 2.0f, 0.9f, 1024);
@@ -531,15 +539,19 @@ void test_errors()
 
 }  // namespace
 
-int main()
+int main(int argc, char** argv)
 {
+    if (argc > 1 && std::strcmp(argv[1], "--inputs") == 0) {  // no GPU needed: the generated inputs only
+        test_quant_per_channel(true);
+        return 0;
+    }
     int ndev = 0;
     if (hipGetDeviceCount(&ndev) != hipSuccess || ndev == 0) {
         std::fprintf(stderr, "no GPU\n");
         return 2;
     }
     std::printf("library: %s\n", ascq_version());
-    test_quant_per_channel();
+    test_quant_per_channel(false);
     test_quant_per_token_fp8();
     test_quant_per_group_fp4();
     test_dequant();
