@@ -79,7 +79,8 @@ class W4A16Desc(C.Structure):
 
 class W8A16Desc(C.Structure):
     _fields_ = [("m", C.c_uint32), ("n", C.c_uint32), ("k", C.c_uint32), ("per_tensor", C.c_int32),
-                ("has_offset", C.c_int32), ("scale", C.c_float), ("offset", C.c_float), ("out_dtype", C.c_int32)]
+                ("has_offset", C.c_int32), ("scale", C.c_float), ("offset", C.c_float), ("out_dtype", C.c_int32),
+                ("trans_b", C.c_int32)]
 
 
 class MatmulPlan(C.Structure):

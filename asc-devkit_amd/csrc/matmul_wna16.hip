@@ -1128,6 +1128,13 @@ extern "C" int ascq_matmul_w4a16(const ascq_w4a16_desc* d, void* y, const void* 
 }
 
 // ------------------------------------------------------------------------------------------------------------ W8A16
+// matmul_w8a16_nk.hip
+namespace ascq {
+bool w8a16_nk_supported(uint32_t k, const void* x, const void* w);
+int launch_w8a16_nk(const void* x, const void* w, const void* scale, const void* offset, void* y, uint32_t m, uint32_t n,
+                    uint32_t k, bool has_offset, bool out_f32, uint32_t scale_bits, uint32_t offset_bits, hipStream_t st);
+}  // namespace ascq
+
 static int validate_w8a16(const ascq_w8a16_desc* d)
 {
     ASCQ_REQUIRE(d != nullptr, ASCQ_ENULL, "ascq_matmul_w8a16: desc is NULL");
@@ -1157,6 +1164,10 @@ extern "C" int ascq_matmul_w8a16_workspace_size(const ascq_w8a16_desc* d, size_t
         return rc;
     }
     ASCQ_REQUIRE(bytes != nullptr, ASCQ_ENULL, "ascq_matmul_w8a16_workspace_size: bytes is NULL");
+    if (d->trans_b) {
+        *bytes = 0;  // whole columns per workgroup: nothing to add across workgroups
+        return ASCQ_OK;
+    }
     *bytes = (d->n % 16 == 0 && d->k % kChunkRows == 0) ? w8a16_workspace_need(d->n, d->k) : 0;
     return ASCQ_OK;
 }
@@ -1193,6 +1204,14 @@ extern "C" int ascq_matmul_w8a16(const ascq_w8a16_desc* d, void* y, const void* 
     p.k = d->k;
     p.has_offset = d->has_offset ? 1u : 0u;
     p.out_f32 = d->out_dtype == ASCQ_F32 ? 1u : 0u;
+    if (d->trans_b) {
+        ASCQ_REQUIRE(d->k % 128u == 0, ASCQ_EUNSUPPORTED,
+                     "ascq_matmul_w8a16: with trans_b k must be a multiple of 128 (k %u)", d->k);
+        ASCQ_REQUIRE(w8a16_nk_supported(d->k, x, w), ASCQ_EALIGN,
+                     "ascq_matmul_w8a16: with trans_b x and w must be 16-byte aligned");
+        return launch_w8a16_nk(x, w, p.scale, p.offset, y, d->m, d->n, d->k, d->has_offset != 0, d->out_dtype == ASCQ_F32,
+                               p.scale_bits, p.offset_bits, st);
+    }
     if (!w8a16_fast_ok(d, x, w, scale, offset)) {
         const size_t total = static_cast<size_t>(d->m) * d->n;
         size_t blocks = (total + kThreads - 1) / kThreads;

@@ -510,11 +510,14 @@ int ascq_matmul_w4a16_packed(const ascq_w4a16_desc* desc, void* y, const void* x
  * output channel (SetAntiQuantVector), then a half matmul with fp32 accumulation.
  * ref: include/adv_api/matmul/matmul.h:161-168;
  *      impl/adv_api/detail/matmul/stage/copy_cube_in/antiquant/antiquant_processor_using_ub.h:53-130.
- * x f16 [m, k]; w int8 [k, n]; scale, offset f16 [n] (per channel) or the desc's scalars (per tensor).
+ * x f16 [m, k]; w int8 [k, n], or [n, k] with trans_b (the reference's isTransposeB: SetTensorB(b, true));
+ * scale, offset f16 [n] (per channel) or the desc's scalars (per tensor).
  *   wdq[k,j] = f16( scale[j] * f16( f16(w[k,j]) + offset[j] ) )               (offset iff has_offset)
  *   y[i,j]   = out( sum_k f32(x[i,k]) * f32(wdq[k,j]) )                       fp32 accumulation
- * The kernel is a weight-streaming one built for few activation rows (decode): the weights are read once per 32
- * rows of x.  B as [n, k] (isTransposeB) is not supported.
+ * The kernels are weight-streaming ones built for few activation rows (decode): the weights are read once per 32
+ * rows of x ([k, n]) or per 16 rows ([n, k]).  With trans_b a column's weights are one contiguous run, so whole
+ * columns belong to one workgroup: one launch, no workspace (the size query answers 0), identical bits from call to
+ * call; that form needs k % 128 == 0 and 16-byte aligned x and w (ASCQ_EUNSUPPORTED / ASCQ_EALIGN otherwise).
  * workspace: ascq_matmul_w8a16_workspace_size bytes (contents need not be initialised); calls that share a
  * workspace must not overlap.
  */
@@ -524,6 +527,7 @@ typedef struct ascq_w8a16_desc {
     int32_t has_offset;  /* MatmulConfig::hasAntiQuantOffset */
     float scale, offset; /* per-tensor parameters, rounded to half as the reference's half scalars */
     int32_t out_dtype;   /* ASCQ_F16 | ASCQ_F32 */
+    int32_t trans_b;     /* 0: w is [k, n]; 1: w is [n, k] */
 } ascq_w8a16_desc;
 
 int ascq_matmul_w8a16(const ascq_w8a16_desc* desc, void* y, const void* x, const void* w, const void* offset,

@@ -752,7 +752,12 @@ public:
         desc_.out_dtype = DTypeOf<CType>::value;
     }
     void SetTensorA(const DeviceTensor<half>& a) { a_ = a.GetPhyAddr(); }
-    void SetTensorB(const DeviceTensor<int8_t>& b) { b_ = b.GetPhyAddr(); }
+    // isTransposeB: b is [n, k] (ref: include/adv_api/matmul/matmul.h:129)
+    void SetTensorB(const DeviceTensor<int8_t>& b, bool isTransposeB = false)
+    {
+        b_ = b.GetPhyAddr();
+        desc_.trans_b = isTransposeB ? 1 : 0;
+    }
     void SetAntiQuantScalar(float offsetScalar, float scaleScalar)
     {
         desc_.per_tensor = 1;

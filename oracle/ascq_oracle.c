@@ -1098,7 +1098,7 @@ int orc_matmul_w8a16(const ascq_w8a16_desc* d, void* y, const uint16_t* x, const
             }
             for (size_t kk = 0; kk < K; ++kk) {
                 for (size_t j = c0; j < c1; ++j) {
-                    uint16_t h = orc_f32_to_f16((float)w[kk * N + j]);
+                    uint16_t h = orc_f32_to_f16((float)(d->trans_b ? w[j * K + kk] : w[kk * N + j]));
                     if (d->has_offset) {
                         h = orc_f16_add(h, d->per_tensor ? offset_s : offset[j]);
                     }

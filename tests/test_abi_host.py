@@ -35,7 +35,7 @@ def test_struct_sizes_match_the_header():
     assert C.sizeof(abi.MatmulDesc) == 11 * 4 + 4 + 8 + 8
     assert C.sizeof(abi.GroupMatmulDesc) == C.sizeof(abi.MatmulDesc) + 8
     assert C.sizeof(abi.W4A16Desc) == 5 * 4
-    assert C.sizeof(abi.W8A16Desc) == 8 * 4
+    assert C.sizeof(abi.W8A16Desc) == 9 * 4
     assert C.sizeof(abi.AntiQuantPolicyDesc) == 14 * 4
 
 
@@ -360,6 +360,19 @@ def test_hifloat8_surface_and_refused_round_modes():
     assert L.ascq_antiquant_policy(C.byref(aq), FAKE, FAKE2, FAKE, None, None) == abi.EUNSUPPORTED and "hifloat8" in err()
     hdr = open(os.path.join(ROOT, "include", "ascq.h")).read()
     assert "ASCQ_QDST_HIF8 = 5" in hdr and "ASCQ_CAST_HYBRID = 7" in hdr
+
+
+def test_w8a16_transposed_weights_surface():
+    """[n, k] weights: no workspace; k must be a multiple of 128; the descriptor carries trans_b as its last field."""
+    assert C.sizeof(abi.W8A16Desc) == 9 * 4 and abi.W8A16Desc._fields_[-1][0] == "trans_b"
+    need = C.c_size_t(77)
+    d = abi.W8A16Desc(m=4, n=64, k=256, per_tensor=1, scale=0.5, out_dtype=abi.F16, trans_b=1)
+    assert L.ascq_matmul_w8a16_workspace_size(C.byref(d), C.byref(need)) == abi.OK and need.value == 0
+    d.k = 192
+    assert L.ascq_matmul_w8a16(C.byref(d), FAKE, FAKE, FAKE, None, None, None, 0, None) == abi.EUNSUPPORTED
+    assert "multiple of 128" in err()
+    d.k = 256
+    assert L.ascq_matmul_w8a16(C.byref(d), FAKE, C.c_void_p(0x100008), FAKE, None, None, None, 0, None) == abi.EALIGN
 
 
 def test_quant_word_with_pre_shift_bit_is_rejected():

@@ -452,6 +452,62 @@ def test_w8a16_exact_integers_full_size(m):
     want = (xi.astype(np.float64) @ (w.astype(np.float64) + of[None, :])) * sc[None, :]
     assert np.array_equal(y.cpu().numpy().astype(np.float64), want)
 
+@pytest.mark.parametrize("m", [1, 3, 16, 17, 40])
+@pytest.mark.parametrize("k,n", [(128, 16), (256, 256), (512, 1040), (384, 30), (2048, 520), (8192, 144)])
+@pytest.mark.parametrize("mode", ["vector+offset", "vector", "scalar+offset", "scalar"])
+def test_w8a16_trans_b(m, k, n, mode):
+    """B given as [n, k] (isTransposeB): one launch, no workspace.  Against the oracle on the same transposed weights,
+    and bit-equal between two calls (the summation order is fixed)."""
+    announce("w8a16 [n, k]", m, k, n, mode)
+    rng = np.random.default_rng(m * 5 + k + n)
+    x = rng.standard_normal((m, k)).astype(np.float16)
+    wt = rng.integers(-128, 128, (n, k)).astype(np.int8)
+    per_tensor = mode.startswith("scalar")
+    has_offset = "offset" in mode
+    out_f32 = (m + k // 128) % 2 == 1
+    if per_tensor:
+        sc, of = 0.0077, (2.5 if has_offset else None)
+    else:
+        sc = rng.uniform(1e-3, 1e-2, n).astype(np.float16)
+        of = rng.uniform(-9, 9, n).astype(np.float16) if has_offset else None
+    ys = []
+    for _ in range(2):
+        y = torch.zeros((m, n), dtype=torch.float32 if out_f32 else torch.float16, device=DEV)
+        y.view(torch.int16).fill_(0x7E7E)
+        ops.matmul_w8a16(y, to_dev(x), to_dev(wt), of if per_tensor else (None if of is None else to_dev(of)),
+                         sc if per_tensor else to_dev(sc), workspace=torch.empty(4, device=DEV), trans_b=True)
+        ys.append(y.cpu().numpy())
+    assert np.array_equal(ys[0].view(np.uint16), ys[1].view(np.uint16))
+    d = abi.W8A16Desc(m=m, n=n, k=k, per_tensor=int(per_tensor), has_offset=int(has_offset),
+                      scale=sc if per_tensor else 0.0, offset=of if per_tensor and has_offset else 0.0,
+                      out_dtype=abi.F32 if out_f32 else abi.F16, trans_b=1)
+    want = orc.matmul_w8a16(d, x, wt, None if per_tensor else of, None if per_tensor else sc)
+    w8a16_check(ys[0], want, x, out_f32)
+    # the oracle's own transposed indexing: the same answer from the [k, n] form
+    d.trans_b = 0
+    assert np.array_equal(np.asarray(want).view(np.uint8),
+                          np.asarray(orc.matmul_w8a16(d, x, np.ascontiguousarray(wt.T), None if per_tensor else of,
+                                                      None if per_tensor else sc)).view(np.uint8))
+
+
+@pytest.mark.parametrize("m", [1, 16])
+def test_w8a16_trans_b_exact_integers_full_size(m):
+    """K=8192, N=28672 as [n, k]: small integer activations, power-of-two scales and integer offsets make every partial
+    sum exact in fp32, so the result must equal plain integer arithmetic bit for bit on every column."""
+    announce("w8a16 [n, k] exact", m)
+    rng = np.random.default_rng(0xE9 + m)
+    k, n = 8192, 28672
+    xi = rng.integers(-2, 3, (m, k))
+    wt = rng.integers(-128, 128, (n, k)).astype(np.int8)
+    sc = rng.choice([0.25, 0.5, 1.0], n)
+    of = rng.integers(-9, 10, n)
+    y = torch.zeros((m, n), dtype=torch.float32, device=DEV)
+    ops.matmul_w8a16(y, to_dev(xi.astype(np.float16)), to_dev(wt), to_dev(of.astype(np.float16)),
+                     to_dev(sc.astype(np.float16)), trans_b=True)
+    want = ((wt.astype(np.float32) + of[:, None].astype(np.float32)) @ xi.T.astype(np.float32)).T * sc[None, :]
+    assert np.array_equal(y.cpu().numpy().astype(np.float64), want.astype(np.float64))
+
+
 # ------------------------------------------------------------------ fractal (NZ) weights
 def to_nz(w):
     """[.., k, n] -> [.., n/32, k/16, 16, 32], as the reference example packs its weights
