@@ -231,6 +231,8 @@ int launch_w8a16_nk(const void* x, const void* w, const void* scale, const void*
         cus = 256;
     }
     const uint32_t n_groups = (n + 15u) / 16u;
+    // one workgroup per compute unit: two, three or seven times as many smaller ones measured slower at every m
+    // (49.7 against 52.7-57.8 us at m = 1, k = 8192, n = 28672)
     uint32_t per = (n_groups + static_cast<uint32_t>(cus) - 1u) / static_cast<uint32_t>(cus);
     per = per > kMaxGroups ? kMaxGroups : per;
     p.groups = per;

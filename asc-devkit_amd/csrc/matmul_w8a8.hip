@@ -642,7 +642,8 @@ extern "C" int ascq_matmul_w8a8_workspace_size(const ascq_matmul_desc* d, size_t
         *bytes = round256(inner) + static_cast<size_t>(d->m) * d->n * sizeof(int32_t);
         return ASCQ_OK;
     }
-    if (d->m <= 32 && !d->trans_a && pick_k_splits(d->n, d->k) > 1) {
+    if (d->m <= 32 && !d->trans_a && pick_k_splits(d->n, d->k) > 1 && !(d->trans_b && d->k % 128 == 0)) {
+        // (few rows on [n, k] weights with k % 128 == 0 run the whole-column kernel, which needs none)
         *bytes = static_cast<size_t>(d->m) * d->n * sizeof(int32_t);
     }
     if (d->m <= kSkinnyMaxM && !d->trans_a && !d->trans_b && d->k % 128 == 0 && d->n % 16 == 0) {
@@ -730,6 +731,9 @@ extern "C" int ascq_matmul_w8a8(const ascq_matmul_desc* d, void* c, const void* 
     }
     if (d->m <= kSkinnyMaxM && !d->trans_b && gemm_dma_supported(p)) {
         return launch_gemm_dma_skinny(p, workspace, workspace_bytes, st);
+    }
+    if (d->m <= 32 && d->trans_b && !d->trans_a && gemm_nk_supported(p)) {
+        return launch_gemm_nk(p, st);
     }
     if (d->m <= 32) {
         const uint32_t splits = pick_k_splits(d->n, d->k);

@@ -57,8 +57,9 @@ def main():
     ap.add_argument("--quick", action="store_true", help="headline + W4A16 GEMV only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="run a single workload: w8a8 | w4a16 | w4a16_nd | w4a16_m4 | w4a16_m16 | w4a16_nd_m4 | w4a16_nd_m16 | "
-                         "w8a8_m1 | w8a8_m16 | w8a8_m128 | w8a16_m1 | w8a16_m16 | quant | dequant | antiquant | group | "
-                         "group_example (a W4A16 name without _nd is the packed-weight path)")
+                         "w8a8_m1 | w8a8_m16 | w8a8_m128 | w8a8_nk_m1 | w8a8_nk_m16 | w8a16_m1 | w8a16_m16 | w8a16_nk_m1 | "
+                         "w8a16_nk_m16 | quant | dequant | antiquant | group | group_example (a W4A16 name without _nd "
+                         "is the packed-weight path; _nk: weights kept as [n, k])")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch one device-to-device copy of 1 GiB: the known-size kernel that calibrates the "
                          "FETCH_SIZE / WRITE_SIZE counters when this command runs under rocprofv3 --pmc")
@@ -129,10 +130,11 @@ def main():
         torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------ W8A8 linear (config 3)
-    def w8a8(M, steps, warmup, sets=1, settle=None, zero=False, gauss=False):
+    def w8a8(M, steps, warmup, sets=1, settle=None, zero=False, gauss=False, b_nk=False):
         """`sets` > 1 rotates the weights over several copies (together larger than the Infinity Cache) so that the
         weight-bound small-M cases read them from HBM.  The weights are uniform over [-127, 127] unless `gauss`: then
-        they are normal weights quantised per output channel by their absolute maximum, as a checkpoint's would be."""
+        they are normal weights quantised per output channel by their absolute maximum, as a checkpoint's would be.
+        b_nk: the weights are kept as [n, k] (isTransposeB)."""
         K, N = 4096, 11008
         x = torch.randn((M, K), device=dev, generator=gen).to(torch.bfloat16)
         if gauss:
@@ -142,7 +144,7 @@ def main():
                 ws.append(torch.round(wf / wf.abs().amax(dim=0, keepdim=True) * 127).clamp(-127, 127).to(torch.int8))
                 del wf
         else:
-            ws = [rand_i8(K, N) for _ in range(sets)]
+            ws = [rand_i8(N, K) if b_nk else rand_i8(K, N) for _ in range(sets)]
         if zero:          # all-zero activations and weights: the same launches, nothing toggles in the multipliers
             x.zero_()
             for wj in ws:
@@ -154,7 +156,7 @@ def main():
         c = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
         mms = []
         for wj in ws:
-            mm = ops.Matmul(M, N, K)
+            mm = ops.Matmul(M, N, K, False, b_nk)
             mm.set_tensor_a(q)
             mm.set_tensor_b(wj)
             mm.set_quant_vector(cs)
@@ -220,17 +222,17 @@ def main():
                 "tops": 2.0 * M * K * N / (kern_ms * 1e-3) / 1e12, "tensors": (xs, ws[0], sc[0], of[0])}
 
     # ------------------------------------------------------------------ W8A16 decode (Matmul anti-quant path)
-    def w8a16(M, steps, warmup, sets=3):
+    def w8a16(M, steps, warmup, sets=3, b_nk=False):
         K, N = 8192, 28672
         xs = torch.randn((M, K), device=dev, generator=gen).to(torch.float16)
-        ws = [rand_i8(K, N) for _ in range(sets)]
+        ws = [rand_i8(N, K) if b_nk else rand_i8(K, N) for _ in range(sets)]
         sc = [(torch.rand((N,), device=dev, generator=gen) * 9e-3 + 1e-3).to(torch.float16) for _ in range(sets)]
         of = [(torch.rand((N,), device=dev, generator=gen) * 18 - 9).to(torch.float16) for _ in range(sets)]
         y = torch.empty((M, N), dtype=torch.float16, device=dev)
 
         def step(i, starts, stops):
             j = i % sets
-            bracket(starts, stops, lambda: ops.matmul_w8a16(y, xs, ws[j], of[j], sc[j]))
+            bracket(starts, stops, lambda: ops.matmul_w8a16(y, xs, ws[j], of[j], sc[j], trans_b=b_nk))
 
         ms, kern_ms = timed(step, steps, warmup)
         bytes_ = K * N + 2 * N * 2 + M * K * 2 + M * N * 2
@@ -355,6 +357,10 @@ def main():
               "w8a8_m1": lambda: w8a8(1, args.steps, args.warmup, sets=7),
               "w8a8_m16": lambda: w8a8(16, args.steps, args.warmup, sets=7),
               "w8a8_m128": lambda: w8a8(128, args.steps, args.warmup, sets=7),
+              "w8a8_nk_m1": lambda: w8a8(1, args.steps, args.warmup, sets=7, b_nk=True),
+              "w8a8_nk_m16": lambda: w8a8(16, args.steps, args.warmup, sets=7, b_nk=True),
+              "w8a16_nk_m1": lambda: w8a16(1, args.steps, args.warmup, b_nk=True),
+              "w8a16_nk_m16": lambda: w8a16(16, args.steps, args.warmup, b_nk=True),
               "w8a16_m1": lambda: w8a16(1, args.steps, args.warmup),
               "w8a16_m16": lambda: w8a16(16, args.steps, args.warmup), "quant": lambda: quant2a(args.steps, args.warmup),
               "dequant": lambda: dequant2b(args.steps, args.warmup),
@@ -449,6 +455,12 @@ def main():
             others[f"w8a8_m{M}"] = {"gemm_kernel_ms": r["gemm_kernel_ms"], "gemm_tops": r["gemm_tops"],
                                     "gemm_gbs": r["gemm_gbs"], "hbm_frac": r["gemm_gbs"] / PEAK_HBM_GBS,
                                     "mfma_frac": r["gemm_tops"] / PEAK_INT8_TOPS}
+        for M in (1, 16):
+            r = strip(w8a8(M, s2, w2, sets=7, b_nk=True))
+            others[f"w8a8_nk_m{M}"] = {"gemm_kernel_ms": r["gemm_kernel_ms"], "gemm_gbs": r["gemm_gbs"],
+                                       "hbm_frac": r["gemm_gbs"] / PEAK_HBM_GBS,
+                                       "note": "weights kept as [n, k] (isTransposeB): one launch, no workspace"}
+            torch.cuda.empty_cache()
         for M in (4, 16):
             r = strip(w4a16(M, s2, w2))
             others[f"w4a16_m{M}"] = {"kernel_ms": r["kernel_ms"], "gbs": r["gbs"], "hbm_frac": r["gbs"] / PEAK_HBM_GBS}
@@ -461,6 +473,11 @@ def main():
             r = w8a16(M, s2, w2)
             others[f"w8a16_m{M}_k8192_n28672"] = {"kernel_ms": r["kernel_ms"], "gbs": r["gbs"], "bytes": r["bytes"],
                                                   "hbm_frac": r["gbs"] / PEAK_HBM_GBS}
+            torch.cuda.empty_cache()
+            r = w8a16(M, s2, w2, b_nk=True)
+            others[f"w8a16_nk_m{M}_k8192_n28672"] = {"kernel_ms": r["kernel_ms"], "gbs": r["gbs"], "bytes": r["bytes"],
+                                                     "hbm_frac": r["gbs"] / PEAK_HBM_GBS,
+                                                     "note": "weights kept as [n, k]: one launch, no workspace"}
             torch.cuda.empty_cache()
         r = group5(max(20, side_steps // 5), 5)
         r["mfma_frac"] = r["tops"] / PEAK_INT8_TOPS

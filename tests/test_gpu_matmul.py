@@ -2,6 +2,8 @@
 the C ABI.  int32 accumulators and every epilogue without a transcendental are compared bit for bit (each epilogue
 step rounds once in fp32, in the reference's order); FasterGelu outputs within 1 ulp of the output type; W4A16
 (free summation order) within the stated tolerance."""
+import ctypes as C
+
 import numpy as np
 import pytest
 import torch
@@ -112,6 +114,29 @@ def test_config3_w8a8_linear(m):
     got = bits(c)
     assert max_ulp(got, want) <= 1
     assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("m", [1, 16, 17, 32])
+def test_config3_w8a8_linear_weights_as_n_k(m):
+    """Config 3's decode sizes on weights kept as [n, k] (isTransposeB): the whole-column kernel, one launch, no
+    workspace; bf16 output with channel and token scales, bit-exact against the oracle on the same weights."""
+    announce("config 3 [n, k]", m)
+    rng = np.random.default_rng(0xC3 + 100 + m)
+    k, n = 4096, 11008
+    a = rand_i8(rng, (m, k))
+    wt = rand_i8(rng, (n, k))
+    cs = rng.uniform(1e-4, 1e-2, n).astype(np.float32)
+    ts = rng.uniform(1e-2, 1e-1, m).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    c, desc = run_mm(m, n, k, a, wt, out=torch.bfloat16, bias=(bias, None), quant=cs, tok=ts, trans_b=True)
+    orc.set_threads(16)
+    assert np.array_equal(bits(c), oracle_mm(desc, a, wt, (bias, None), cs, ts))
+    wsz = C.c_size_t(1)
+    assert abi.load_library().ascq_matmul_w8a8_workspace_size(C.byref(desc), C.byref(wsz)) == abi.OK and wsz.value == 0
+    # int8 requantised output and SwiGLU through the same kernel
+    words = (cs * 50).astype(np.float32).view(np.uint32).astype(np.uint64) | (np.uint64(1) << np.uint64(46))
+    c8, d8 = run_mm(m, n, k, a, wt, out=torch.int8, quant=words, trans_b=True)
+    assert np.array_equal(bits(c8), oracle_mm(d8, a, wt, None, words))
 
 
 def test_fixpipe_modes_uint64_words():
