@@ -24,6 +24,9 @@ typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 
 constexpr uint32_t kWaves = 8, kMaxGroups = 8, kRows = 16, kRun = 128;
+// up to this many rows the whole-column kernel runs, 16 rows per pass (two passes cost what one pass of the tile GEMM
+// over up to 128 rows costs: 120 us at k = 8192, n = 28672)
+constexpr uint32_t kDecodeRows = 32;
 
 struct NkParams {
     const uint16_t* x;       // [m, k] halves (this pass's first row)
@@ -205,11 +208,204 @@ void launch_nk(const NkParams& p, uint32_t grid, hipStream_t st)
     }
 }
 
+// ---- many activation rows: a half GEMM whose B-tile loader de-quantises.
+// Workgroup = 4 wavefronts (2 x 2) on a 128 x 128 tile, K step 64, two LDS stages of 32 KiB (two workgroups per compute
+// unit).  Both tiles sit in LDS as [row or column][64 k] halves, 128 bytes per line in 8 pieces of 16 bytes, piece c of
+// line r stored at position c ^ (r & 7), so that the 16-byte operand reads of eight neighbouring lines fall into
+// different banks.  A thread stages 32 bytes of one column of B per K step (registers: load, de-quantise exactly as
+// the decode kernel does, four 16-byte LDS writes) and two 16-byte pieces of A; the global loads of the next K step are
+// issued before the MFMAs of the current one.  v_mfma_f32_32x32x16_f16: lane l holds row (column) l % 32 and the 8
+// consecutive k 8 (l / 32) .. + 7 of a K sub-step, i.e. one 16-byte piece of a line.
+constexpr uint32_t kGM = 128, kGN = 128, kGK = 64;
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+template <bool kHasOffset>
+__global__ __launch_bounds__(256, 2) void w8a16_nk_gemm_kernel(NkParams p, uint32_t tiles_m)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t AS[2][kGM * kGK * 2];
+    __shared__ __attribute__((aligned(16))) uint8_t BS[2][kGN * kGK * 2];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t wm = wave >> 1, wn = wave & 1u;
+    // row tiles innermost: the workgroups that run side by side share their columns of B
+    const uint32_t tm = blockIdx.x % tiles_m, tn = blockIdx.x / tiles_m;
+    const uint32_t row0 = tm * kGM, col0 = tn * kGN;
+
+    // ---- staging roles
+    // B: thread t stages bytes 32 (t & 1) .. + 31 of column col0 + t / 2 (pieces 4 (t & 1) .. + 3 of its LDS line)
+    const uint32_t bcol_l = tid >> 1, bhalf = tid & 1u;
+    uint32_t bcol = col0 + bcol_l;
+    bcol = bcol < p.n ? bcol : p.n - 1u;
+    const uint8_t* bsrc = p.w + static_cast<size_t>(bcol) * p.k + 32u * bhalf;
+    const uint32_t sb = p.scale ? p.scale[bcol] : p.scale_bits;
+    const uint32_t ob = kHasOffset ? (p.scale ? p.offset[bcol] : p.offset_bits) : 0u;
+    const f16x2_t sc2 = h2_from_bits(sb | (sb << 16)), of2 = h2_from_bits(ob | (ob << 16));
+    // A: thread t stages pieces (t & 7) of rows t / 8 and t / 8 + 32 .. (four rows, 16 bytes each)
+    const uint32_t apiece = tid & 7u, arow_l = tid >> 3;
+    const uint16_t* asrc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        uint32_t r = row0 + arow_l + 32u * j;
+        r = r < p.m ? r : p.m - 1u;
+        asrc[j] = p.x + static_cast<size_t>(r) * p.k + 8u * apiece;
+    }
+
+    u32x4 braw[2], araw[4];
+    auto fetch = [&](uint32_t k0) __attribute__((always_inline)) {
+        braw[0] = *reinterpret_cast<const u32x4*>(bsrc + k0);
+        braw[1] = *reinterpret_cast<const u32x4*>(bsrc + k0 + 16u);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) araw[j] = *reinterpret_cast<const u32x4*>(asrc[j] + k0);
+    };
+    auto stage = [&](uint32_t st) __attribute__((always_inline)) {
+        // B: 32 bytes -> 32 halves = four pieces
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            uint32_t h0, h1, h2, h3;
+            dequant4<kHasOffset>(braw[q >> 1][2 * (q & 1)], sc2, of2, h0, h1);
+            dequant4<kHasOffset>(braw[q >> 1][2 * (q & 1) + 1], sc2, of2, h2, h3);
+            const uint32_t piece = 4u * bhalf + static_cast<uint32_t>(q);
+            *reinterpret_cast<u32x4*>(&BS[st][bcol_l * 128u + ((piece ^ (bcol_l & 7u)) << 4)]) = u32x4{h0, h1, h2, h3};
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t r = arow_l + 32u * j;
+            *reinterpret_cast<u32x4*>(&AS[st][r * 128u + ((apiece ^ (r & 7u)) << 4)]) = araw[j];
+        }
+    };
+
+    f32x16_t acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    const uint32_t lrow = lane & 31u, lk = lane >> 5;  // operand line and which 8 k of a sub-step
+    auto compute = [&](uint32_t st) __attribute__((always_inline)) {
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const uint32_t piece = 2u * ks + lk;
+            f16x8_t af[2], bf[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const uint32_t r = wm * 64u + i * 32u + lrow;
+                af[i] = *reinterpret_cast<const f16x8_t*>(&AS[st][r * 128u + ((piece ^ (r & 7u)) << 4)]);
+                const uint32_t c = wn * 64u + i * 32u + lrow;
+                bf[i] = *reinterpret_cast<const f16x8_t*>(&BS[st][c * 128u + ((piece ^ (c & 7u)) << 4)]);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+        }
+    };
+
+    const uint32_t steps = p.k / kGK;
+    fetch(0);
+    stage(0);
+    __syncthreads();
+    for (uint32_t s = 0; s < steps; ++s) {
+        const uint32_t cur = s & 1u;
+        if (s + 1u < steps) {
+            fetch((s + 1u) * kGK);
+        }
+        compute(cur);
+        if (s + 1u < steps) {
+            stage(cur ^ 1u);  // the other stage was last read before the barrier that ended the previous step
+        }
+        __syncthreads();
+    }
+
+    // ---- register r of lane l in a 32 x 32 block: row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const uint32_t col = col0 + wn * 64u + j * 32u + lrow;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint32_t row = row0 + wm * 64u + i * 32u + 8u * (r >> 2) + 4u * lk + (r & 3);
+                if (row < p.m && col < p.n) {
+                    const size_t idx = static_cast<size_t>(row) * p.n + col;
+                    if (p.out_f32) {
+                        static_cast<float*>(p.y)[idx] = acc[i][j][r];
+                    } else {
+                        static_cast<uint16_t*>(p.y)[idx] = static_cast<uint16_t>(f32_to_half_bits(acc[i][j][r]));
+                    }
+                }
+            }
+        }
+    }
+}
+
+// int8 [k, n] -> [n, k] through 64 x 64 tiles in LDS (the tile GEMM wants k-contiguous weights).  k % 64 == 0.
+// kVec: n % 16 == 0 and src 16-byte aligned, so a thread's 16 columns of a row are one load.
+template <bool kVec>
+__global__ __launch_bounds__(256) void transpose_i8_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
+                                                           uint32_t k, uint32_t n)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t T[64][68];
+    const uint32_t tiles_n = (n + 63u) / 64u;
+    const uint32_t k0 = (blockIdx.x / tiles_n) * 64u, n0 = (blockIdx.x % tiles_n) * 64u;
+    const uint32_t t = threadIdx.x, r = t >> 2, c = (t & 3u) * 16u;
+    const uint8_t* row = src + static_cast<size_t>(k0 + r) * n;
+    if constexpr (kVec) {
+        u32x4 v = u32x4{0u, 0u, 0u, 0u};
+        if (n0 + c < n) {
+            v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(row + n0 + c));
+        }
+#pragma unroll
+        for (uint32_t w = 0; w < 4; ++w) *reinterpret_cast<uint32_t*>(&T[r][c + 4u * w]) = v[w];
+    } else {
+#pragma unroll
+        for (uint32_t i = 0; i < 16; ++i) {
+            const uint32_t col = n0 + c + i;
+            T[r][c + i] = row[col < n ? col : n - 1u];
+        }
+    }
+    __syncthreads();
+    if (n0 + r < n) {
+        uint32_t out[4];
+#pragma unroll
+        for (uint32_t w = 0; w < 4; ++w) {
+            out[w] = 0;
+#pragma unroll
+            for (uint32_t b = 0; b < 4; ++b) out[w] |= static_cast<uint32_t>(T[c + 4u * w + b][r]) << (8u * b);
+        }
+        *reinterpret_cast<u32x4*>(dst + static_cast<size_t>(n0 + r) * k + k0 + c) = u32x4{out[0], out[1], out[2], out[3]};
+    }
+}
+
 }  // namespace
 
 bool w8a16_nk_supported(uint32_t k, const void* x, const void* w)
 {
     return k % kRun == 0 && aligned16(x) && aligned16(w);
+}
+
+int launch_w8a16_nk(const void* x, const void* w, const void* scale, const void* offset, void* y, uint32_t m, uint32_t n,
+                    uint32_t k, bool has_offset, bool out_f32, uint32_t scale_bits, uint32_t offset_bits, hipStream_t st);
+
+// Weights given as [k, n] and many rows: transposed once into the caller's workspace (k * n bytes), then the tile GEMM.
+bool w8a16_kn_gemm_supported(uint32_t m, uint32_t k, const void* x, const void* w)
+{
+    return m > 96u && k % kGK == 0 && aligned16(x) && (reinterpret_cast<uintptr_t>(w) & 3u) == 0;
+}
+
+int launch_w8a16_kn_via_transpose(const void* x, const void* w, const void* scale, const void* offset, void* y,
+                                  uint32_t m, uint32_t n, uint32_t k, bool has_offset, bool out_f32, uint32_t scale_bits,
+                                  uint32_t offset_bits, void* workspace, hipStream_t st)
+{
+    const uint32_t tiles = (k / 64u) * ((n + 63u) / 64u);
+    if (n % 16u == 0 && aligned16(w)) {
+        transpose_i8_kernel<true><<<tiles, 256, 0, st>>>(static_cast<const uint8_t*>(w), static_cast<uint8_t*>(workspace), k, n);
+    } else {
+        transpose_i8_kernel<false><<<tiles, 256, 0, st>>>(static_cast<const uint8_t*>(w), static_cast<uint8_t*>(workspace), k, n);
+    }
+    return launch_w8a16_nk(x, workspace, scale, offset, y, m, n, k, has_offset, out_f32, scale_bits, offset_bits, st);
 }
 
 // x, y: first row of the whole problem; m rows in passes of 16.
@@ -237,6 +433,19 @@ int launch_w8a16_nk(const void* x, const void* w, const void* scale, const void*
     per = per > kMaxGroups ? kMaxGroups : per;
     p.groups = per;
     const uint32_t grid = (n_groups + per - 1u) / per;
+    if (m > kDecodeRows && k % kGK == 0) {
+        // more rows than a few passes of the decode kernel: the tile GEMM reads the weights once per 128 rows
+        p.m = m;
+        p.x = static_cast<const uint16_t*>(x);
+        p.y = y;
+        const uint32_t tiles_m = (m + kGM - 1u) / kGM, tiles_n = (n + kGN - 1u) / kGN;
+        if (has_offset) {
+            w8a16_nk_gemm_kernel<true><<<tiles_m * tiles_n, 256, 0, st>>>(p, tiles_m);
+        } else {
+            w8a16_nk_gemm_kernel<false><<<tiles_m * tiles_n, 256, 0, st>>>(p, tiles_m);
+        }
+        return launch_status("ascq_matmul_w8a16");
+    }
     for (uint32_t m0 = 0; m0 < m; m0 += kRows) {
         p.m = m - m0 < kRows ? m - m0 : kRows;
         p.x = static_cast<const uint16_t*>(x) + static_cast<size_t>(m0) * k;

@@ -1133,6 +1133,10 @@ namespace ascq {
 bool w8a16_nk_supported(uint32_t k, const void* x, const void* w);
 int launch_w8a16_nk(const void* x, const void* w, const void* scale, const void* offset, void* y, uint32_t m, uint32_t n,
                     uint32_t k, bool has_offset, bool out_f32, uint32_t scale_bits, uint32_t offset_bits, hipStream_t st);
+bool w8a16_kn_gemm_supported(uint32_t m, uint32_t k, const void* x, const void* w);
+int launch_w8a16_kn_via_transpose(const void* x, const void* w, const void* scale, const void* offset, void* y,
+                                  uint32_t m, uint32_t n, uint32_t k, bool has_offset, bool out_f32, uint32_t scale_bits,
+                                  uint32_t offset_bits, void* workspace, hipStream_t st);
 }  // namespace ascq
 
 static int validate_w8a16(const ascq_w8a16_desc* d)
@@ -1169,6 +1173,14 @@ extern "C" int ascq_matmul_w8a16_workspace_size(const ascq_w8a16_desc* d, size_t
         return ASCQ_OK;
     }
     *bytes = (d->n % 16 == 0 && d->k % kChunkRows == 0) ? w8a16_workspace_need(d->n, d->k) : 0;
+    if (d->m > 96u && d->k % 64u == 0) {
+        // many rows: the weights are transposed into the workspace once and a tile GEMM runs on them (a smaller
+        // workspace is accepted and the weight-stream kernel then passes over the weights once per 32 rows)
+        const size_t need = static_cast<size_t>(d->k) * d->n;
+        if (need > *bytes) {
+            *bytes = need;
+        }
+    }
     return ASCQ_OK;
 }
 
@@ -1211,6 +1223,11 @@ extern "C" int ascq_matmul_w8a16(const ascq_w8a16_desc* d, void* y, const void* 
                      "ascq_matmul_w8a16: with trans_b x and w must be 16-byte aligned");
         return launch_w8a16_nk(x, w, p.scale, p.offset, y, d->m, d->n, d->k, d->has_offset != 0, d->out_dtype == ASCQ_F32,
                                p.scale_bits, p.offset_bits, st);
+    }
+    if (w8a16_kn_gemm_supported(d->m, d->k, x, w) && workspace != nullptr && aligned16(workspace) &&
+        workspace_bytes >= static_cast<size_t>(d->k) * d->n) {
+        return launch_w8a16_kn_via_transpose(x, w, p.scale, p.offset, y, d->m, d->n, d->k, d->has_offset != 0,
+                                             d->out_dtype == ASCQ_F32, p.scale_bits, p.offset_bits, workspace, st);
     }
     if (!w8a16_fast_ok(d, x, w, scale, offset)) {
         const size_t total = static_cast<size_t>(d->m) * d->n;

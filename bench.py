@@ -58,7 +58,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="run a single workload: w8a8 | w4a16 | w4a16_nd | w4a16_m4 | w4a16_m16 | w4a16_nd_m4 | w4a16_nd_m16 | "
                          "w8a8_m1 | w8a8_m16 | w8a8_m128 | w8a8_nk_m1 | w8a8_nk_m16 | w8a16_m1 | w8a16_m16 | w8a16_nk_m1 | "
-                         "w8a16_nk_m16 | quant | dequant | antiquant | group | group_example (a W4A16 name without _nd "
+                         "w8a16_nk_m16 | w8a16_m2048 | w8a16_nk_m2048 | quant | dequant | antiquant | group | group_example (a W4A16 name without _nd "
                          "is the packed-weight path; _nk: weights kept as [n, k])")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch one device-to-device copy of 1 GiB: the known-size kernel that calibrates the "
@@ -234,9 +234,10 @@ def main():
             j = i % sets
             bracket(starts, stops, lambda: ops.matmul_w8a16(y, xs, ws[j], of[j], sc[j], trans_b=b_nk))
 
-        ms, kern_ms = timed(step, steps, warmup)
+        ms, kern_ms = timed(step, steps, warmup, settle=min(args.settle, 300 if M <= 64 else 20))
         bytes_ = K * N + 2 * N * 2 + M * K * 2 + M * N * 2
-        return {"ms_per_step": ms, "kernel_ms": kern_ms, "gbs": bytes_ / (kern_ms * 1e-3) / 1e9, "bytes": bytes_}
+        return {"ms_per_step": ms, "kernel_ms": kern_ms, "gbs": bytes_ / (kern_ms * 1e-3) / 1e9, "bytes": bytes_,
+                "tflops": 2.0 * M * K * N / (kern_ms * 1e-3) / 1e12}
 
     # ------------------------------------------------------------------ elementwise (config 2)
     def quant2a(steps, warmup, sets=3):
@@ -361,6 +362,8 @@ def main():
               "w8a8_nk_m16": lambda: w8a8(16, args.steps, args.warmup, sets=7, b_nk=True),
               "w8a16_nk_m1": lambda: w8a16(1, args.steps, args.warmup, b_nk=True),
               "w8a16_nk_m16": lambda: w8a16(16, args.steps, args.warmup, b_nk=True),
+              "w8a16_nk_m2048": lambda: w8a16(2048, min(args.steps, 30), min(args.warmup, 5), sets=1, b_nk=True),
+              "w8a16_m2048": lambda: w8a16(2048, min(args.steps, 30), min(args.warmup, 5), sets=1),
               "w8a16_m1": lambda: w8a16(1, args.steps, args.warmup),
               "w8a16_m16": lambda: w8a16(16, args.steps, args.warmup), "quant": lambda: quant2a(args.steps, args.warmup),
               "dequant": lambda: dequant2b(args.steps, args.warmup),
@@ -478,6 +481,13 @@ def main():
             others[f"w8a16_nk_m{M}_k8192_n28672"] = {"kernel_ms": r["kernel_ms"], "gbs": r["gbs"], "bytes": r["bytes"],
                                                      "hbm_frac": r["gbs"] / PEAK_HBM_GBS,
                                                      "note": "weights kept as [n, k]: one launch, no workspace"}
+            torch.cuda.empty_cache()
+        for nk in (True, False):
+            r = w8a16(2048, 30, 5, sets=1, b_nk=nk)
+            others["w8a16_nk_m2048_k8192_n28672" if nk else "w8a16_m2048_k8192_n28672"] = {
+                "kernel_ms": r["kernel_ms"], "tflops": r["tflops"], "f16_mfma_frac": r["tflops"] / 2500.0,
+                "note": "half GEMM whose B-tile loader de-quantises (w8a16_nk_gemm_kernel)" +
+                        ("" if nk else ", after one transposed copy of the [k, n] weights into the workspace")}
             torch.cuda.empty_cache()
         r = group5(max(20, side_steps // 5), 5)
         r["mfma_frac"] = r["tops"] / PEAK_INT8_TOPS

@@ -514,10 +514,13 @@ int ascq_matmul_w4a16_packed(const ascq_w4a16_desc* desc, void* y, const void* x
  * scale, offset f16 [n] (per channel) or the desc's scalars (per tensor).
  *   wdq[k,j] = f16( scale[j] * f16( f16(w[k,j]) + offset[j] ) )               (offset iff has_offset)
  *   y[i,j]   = out( sum_k f32(x[i,k]) * f32(wdq[k,j]) )                       fp32 accumulation
- * The kernels are weight-streaming ones built for few activation rows (decode): the weights are read once per 32
- * rows of x ([k, n]) or per 16 rows ([n, k]).  With trans_b a column's weights are one contiguous run, so whole
- * columns belong to one workgroup: one launch, no workspace (the size query answers 0), identical bits from call to
- * call; that form needs k % 128 == 0 and 16-byte aligned x and w (ASCQ_EUNSUPPORTED / ASCQ_EALIGN otherwise).
+ * Few activation rows (decode) run weight-streaming kernels: the weights are read once per 32 rows of x ([k, n]) or
+ * per 16 rows ([n, k]).  With trans_b a column's weights are one contiguous run, so whole columns belong to one
+ * workgroup: one launch, no workspace (the size query answers 0), identical bits from call to call; that form needs
+ * k % 128 == 0 and 16-byte aligned x and w (ASCQ_EUNSUPPORTED / ASCQ_EALIGN otherwise).
+ * Many rows (more than 32 on [n, k] weights, more than 96 on [k, n]) run a half GEMM on 128 x 128 tiles whose B-tile
+ * loader de-quantises; [k, n] weights are first copied transposed into the workspace (k * n bytes, which the size query
+ * then asks for; given less, the call falls back to one pass over the weights per 32 rows).
  * workspace: ascq_matmul_w8a16_workspace_size bytes (contents need not be initialised); calls that share a
  * workspace must not overlap.
  */

@@ -414,8 +414,8 @@ def w8a16_check(got, want, x, out_f32):
         assert np.mean(got.view(np.uint16) == want.view(np.uint16)) > 0.9
 
 
-@pytest.mark.parametrize("m", [1, 3, 16, 17, 32, 33, 40, 70])
-@pytest.mark.parametrize("k,n", [(256, 256), (512, 1040), (96, 48), (100, 30), (2048, 512)])
+@pytest.mark.parametrize("m", [1, 3, 16, 17, 32, 33, 40, 70, 97, 300])   # above 96 rows: transposed copy + tile GEMM
+@pytest.mark.parametrize("k,n", [(256, 256), (512, 1040), (96, 48), (100, 30), (2048, 512), (192, 30)])
 @pytest.mark.parametrize("mode", ["vector+offset", "vector", "scalar+offset", "scalar", "vector+intoffset"])
 def test_w8a16_small(m, k, n, mode):
     announce("w8a16", m, k, n, mode)
@@ -477,12 +477,13 @@ def test_w8a16_exact_integers_full_size(m):
     want = (xi.astype(np.float64) @ (w.astype(np.float64) + of[None, :])) * sc[None, :]
     assert np.array_equal(y.cpu().numpy().astype(np.float64), want)
 
-@pytest.mark.parametrize("m", [1, 3, 16, 17, 40])
+@pytest.mark.parametrize("m", [1, 3, 16, 17, 40, 49, 130, 300])
 @pytest.mark.parametrize("k,n", [(128, 16), (256, 256), (512, 1040), (384, 30), (2048, 520), (8192, 144)])
 @pytest.mark.parametrize("mode", ["vector+offset", "vector", "scalar+offset", "scalar"])
 def test_w8a16_trans_b(m, k, n, mode):
-    """B given as [n, k] (isTransposeB): one launch, no workspace.  Against the oracle on the same transposed weights,
-    and bit-equal between two calls (the summation order is fixed)."""
+    """B given as [n, k] (isTransposeB): one launch, no workspace; the whole-column kernel up to 48 rows, the
+    de-quantising tile GEMM above.  Against the oracle on the same transposed weights, and bit-equal between two calls
+    (the summation order is fixed)."""
     announce("w8a16 [n, k]", m, k, n, mode)
     rng = np.random.default_rng(m * 5 + k + n)
     x = rng.standard_normal((m, k)).astype(np.float16)
