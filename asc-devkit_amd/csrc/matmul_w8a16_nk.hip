@@ -211,8 +211,9 @@ void launch_nk(const NkParams& p, uint32_t grid, hipStream_t st)
 // ---- many activation rows: a half GEMM whose B-tile loader de-quantises.
 // Workgroup = 4 wavefronts (2 x 2) on a 128 x 128 tile, K step 64, two LDS stages of 32 KiB (two workgroups per compute
 // unit).  Both tiles sit in LDS as [row or column][64 k] halves, 128 bytes per line in 8 pieces of 16 bytes, piece c of
-// line r stored at position c ^ (r & 7), so that the 16-byte operand reads of eight neighbouring lines fall into
-// different banks.  A thread stages 32 bytes of one column of B per K step (registers: load, de-quantise exactly as
+// line r stored at position c ^ ((r >> 1) & 7): a 16-byte access is served 16 lanes (256 bytes, all 64 banks) at a
+// time, two lines fill one 256-byte bank row, so the sixteen neighbouring lines of such a group must put their piece
+// into eight different positions per line parity.  A thread stages 32 bytes of one column of B per K step (registers: load, de-quantise exactly as
 // the decode kernel does, four 16-byte LDS writes) and two 16-byte pieces of A; the global loads of the next K step are
 // issued before the MFMAs of the current one.  v_mfma_f32_32x32x16_f16: lane l holds row (column) l % 32 and the 8
 // consecutive k 8 (l / 32) .. + 7 of a K sub-step, i.e. one 16-byte piece of a line.
@@ -250,28 +251,28 @@ __global__ __launch_bounds__(256, 2) void w8a16_nk_gemm_kernel(NkParams p, uint3
         asrc[j] = p.x + static_cast<size_t>(r) * p.k + 8u * apiece;
     }
 
-    u32x4 braw[2], araw[4];
-    auto fetch = [&](uint32_t k0) __attribute__((always_inline)) {
-        braw[0] = *reinterpret_cast<const u32x4*>(bsrc + k0);
-        braw[1] = *reinterpret_cast<const u32x4*>(bsrc + k0 + 16u);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) araw[j] = *reinterpret_cast<const u32x4*>(asrc[j] + k0);
+    // Two register sets for the raw data of the next two K steps: the loads of step s + 2 are issued while step s
+    // computes, and the data of step s + 1 is de-quantised and written to the other LDS stage in four parts, one behind
+    // the MFMAs of each K sub-step, so that the vector ALU works while the matrix pipe is busy.
+    struct Raw {
+        u32x4 b[2], a[4];
     };
-    auto stage = [&](uint32_t st) __attribute__((always_inline)) {
-        // B: 32 bytes -> 32 halves = four pieces
+    auto fetch = [&](Raw& raw, uint32_t step) __attribute__((always_inline)) {
+        const uint32_t k0 = step * kGK;
+        raw.b[0] = *reinterpret_cast<const u32x4*>(bsrc + k0);
+        raw.b[1] = *reinterpret_cast<const u32x4*>(bsrc + k0 + 16u);
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            uint32_t h0, h1, h2, h3;
-            dequant4<kHasOffset>(braw[q >> 1][2 * (q & 1)], sc2, of2, h0, h1);
-            dequant4<kHasOffset>(braw[q >> 1][2 * (q & 1) + 1], sc2, of2, h2, h3);
-            const uint32_t piece = 4u * bhalf + static_cast<uint32_t>(q);
-            *reinterpret_cast<u32x4*>(&BS[st][bcol_l * 128u + ((piece ^ (bcol_l & 7u)) << 4)]) = u32x4{h0, h1, h2, h3};
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const uint32_t r = arow_l + 32u * j;
-            *reinterpret_cast<u32x4*>(&AS[st][r * 128u + ((apiece ^ (r & 7u)) << 4)]) = araw[j];
-        }
+        for (int j = 0; j < 4; ++j) raw.a[j] = *reinterpret_cast<const u32x4*>(asrc[j] + k0);
+    };
+    // part q of a step's staging: piece q of the thread's half line of B, piece q of its A pieces
+    auto stage_part = [&](const Raw& raw, uint32_t st, int q) __attribute__((always_inline)) {
+        uint32_t h0, h1, h2, h3;
+        dequant4<kHasOffset>(raw.b[q >> 1][2 * (q & 1)], sc2, of2, h0, h1);
+        dequant4<kHasOffset>(raw.b[q >> 1][2 * (q & 1) + 1], sc2, of2, h2, h3);
+        const uint32_t piece = 4u * bhalf + static_cast<uint32_t>(q);
+        *reinterpret_cast<u32x4*>(&BS[st][bcol_l * 128u + ((piece ^ ((bcol_l >> 1) & 7u)) << 4)]) = u32x4{h0, h1, h2, h3};
+        const uint32_t r = arow_l + 32u * static_cast<uint32_t>(q);
+        *reinterpret_cast<u32x4*>(&AS[st][r * 128u + ((apiece ^ ((r >> 1) & 7u)) << 4)]) = raw.a[q];
     };
 
     f32x16_t acc[2][2];
@@ -283,7 +284,8 @@ __global__ __launch_bounds__(256, 2) void w8a16_nk_gemm_kernel(NkParams p, uint3
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
     const uint32_t lrow = lane & 31u, lk = lane >> 5;  // operand line and which 8 k of a sub-step
-    auto compute = [&](uint32_t st) __attribute__((always_inline)) {
+    // one K step on LDS stage st; `next` (data of the following step) is staged into the other LDS stage when do_stage
+    auto step_body = [&](uint32_t st, const Raw& next, bool do_stage) __attribute__((always_inline)) {
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
             const uint32_t piece = 2u * ks + lk;
@@ -291,32 +293,39 @@ __global__ __launch_bounds__(256, 2) void w8a16_nk_gemm_kernel(NkParams p, uint3
 #pragma unroll
             for (int i = 0; i < 2; ++i) {
                 const uint32_t r = wm * 64u + i * 32u + lrow;
-                af[i] = *reinterpret_cast<const f16x8_t*>(&AS[st][r * 128u + ((piece ^ (r & 7u)) << 4)]);
+                af[i] = *reinterpret_cast<const f16x8_t*>(&AS[st][r * 128u + ((piece ^ ((r >> 1) & 7u)) << 4)]);
                 const uint32_t c = wn * 64u + i * 32u + lrow;
-                bf[i] = *reinterpret_cast<const f16x8_t*>(&BS[st][c * 128u + ((piece ^ (c & 7u)) << 4)]);
+                bf[i] = *reinterpret_cast<const f16x8_t*>(&BS[st][c * 128u + ((piece ^ ((c >> 1) & 7u)) << 4)]);
             }
 #pragma unroll
             for (int i = 0; i < 2; ++i)
 #pragma unroll
                 for (int j = 0; j < 2; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+            if (do_stage) {  // uniform; the other stage was last read before the barrier that ended the previous step
+                stage_part(next, st ^ 1u, ks);
+            }
         }
     };
 
     const uint32_t steps = p.k / kGK;
-    fetch(0);
-    stage(0);
+    const uint32_t last = steps - 1u;
+    Raw r0, r1;
+    fetch(r0, 0);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) stage_part(r0, 0, q);
+    fetch(r1, 1u < last ? 1u : last);  // data of step 1 (clamped: a single-step problem re-reads step 0 and drops it)
     __syncthreads();
-    for (uint32_t s = 0; s < steps; ++s) {
-        const uint32_t cur = s & 1u;
-        if (s + 1u < steps) {
-            fetch((s + 1u) * kGK);
-        }
-        compute(cur);
-        if (s + 1u < steps) {
-            stage(cur ^ 1u);  // the other stage was last read before the barrier that ended the previous step
-        }
+    for (uint32_t s = 0; s < steps; s += 2) {
+        // step s on stage 0: r1 holds step s + 1; fetch step s + 2 into r0 (clamped at the end: harmless re-reads)
+        fetch(r0, s + 2u < last ? s + 2u : last);
+        step_body(0u, r1, s + 1u < steps);
         __syncthreads();
+        if (s + 1u < steps) {
+            fetch(r1, s + 3u < last ? s + 3u : last);
+            step_body(1u, r0, s + 2u < steps);
+            __syncthreads();
+        }
     }
 
     // ---- register r of lane l in a 32 x 32 block: row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32
