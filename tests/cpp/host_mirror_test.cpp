@@ -166,6 +166,16 @@ void test_quant_per_token_fp8()
     std::vector<uint8_t> want(m * n);
     orc_quant(&d, reinterpret_cast<int8_t*>(want.data()), x.data(), sc.data(), of.data());
     expect_equal("AscendQuant fp8 per token", dq.download(), want);
+
+    // the same call with a hifloat8_t destination (RoundMode::CAST_ROUND, the type's default)
+    std::printf("[case] AscendQuant<hifloat8_t, half, float> PER_TOKEN 12x256\n");
+    cfg.roundMode = ascq::RoundMode::CAST_ROUND;
+    ascq::AscendQuant(dq.view<ascq::hifloat8_t>(m * n), dx.view<ascq::half>(m * n), dsc.view<float>(m),
+                      dof.view<float>(m), para, cfg, ascq::AscendQuantPolicy::PER_TOKEN);
+    d.round_mode = ASCQ_CAST_ROUND;
+    d.dst_format = ASCQ_QDST_HIF8;
+    orc_quant(&d, reinterpret_cast<int8_t*>(want.data()), x.data(), sc.data(), of.data());
+    expect_equal("AscendQuant hifloat8 per token", dq.download(), want);
 }
 
 void test_quant_per_group_fp4()
@@ -382,6 +392,24 @@ void test_antiquant_matmul()
     std::vector<float> want(m * n);
     orc_matmul_w8a16(&mm.Desc(), want.data(), x.data(), w.data(), of.data(), sc.data());
     expect_equal("AntiQuantMatmul", dc.download(), want);
+
+    // the same product from weights kept as [n, k] (SetTensorB(b, isTransposeB = true)): no workspace
+    std::printf("[case] AntiQuantMatmul<float> 5x272x128, B as [n, k]\n");
+    std::vector<int8_t> wt(n * k);
+    for (uint32_t j = 0; j < n; ++j)
+        for (uint32_t kk = 0; kk < k; ++kk) wt[j * k + kk] = w[kk * n + j];
+    DeviceBuffer<int8_t> dwt(wt);
+    DeviceBuffer<float> dc2(m * n);
+    ascq::AntiQuantMatmul<float> mt(m, n, k);
+    mt.SetTensorA(dx.view<ascq::half>(m * k));
+    mt.SetTensorB(dwt.view<int8_t>(k * n), true);
+    mt.SetAntiQuantVector(dof.view<ascq::half>(n), dsc.view<ascq::half>(n));
+    if (mt.GetWorkspaceSize() != 0) {
+        std::printf("[FAIL] [n, k] weights asked for a workspace\n");
+        ++g_failed;
+    }
+    mt.IterateAll(dc2.view<float>(m * n));
+    expect_equal("AntiQuantMatmul [n, k]", dc2.download(), want);
 }
 
 void test_unified_surface()
