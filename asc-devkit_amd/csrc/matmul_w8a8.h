@@ -63,15 +63,15 @@ __device__ __forceinline__ ChannelQ load_channel_q(const EpiParams& e, size_t co
     return q;
 }
 
-// FasterGelu, x * exp(0.851 (x - |x|)) / (1 + exp(-1.702 |x|)).  For x < 0 the two exponentials are the same number
-// (0.851 * 2x and 1.702 * x round alike in fp32) and for x >= 0 the first is exactly 1, so one exponential serves
-// both; it and the reciprocal are the hardware's approximations (about one fp32 ulp each), far inside one ulp of
-// the 16-bit outputs this activation is used with.
+// FasterGelu, x * exp(0.851 (x - |x|)) / (1 + exp(-1.702 |x|)) = x / (1 + exp(-1.702 x)): the reference's form keeps
+// both exponentials at or below 1 for its vector unit; the quotient form needs one exponential, and its overflow is
+// harmless in fp32 (exp -> inf gives 1 / inf = 0, the right limit; exp -> 0 gives x).  The exponential and the
+// reciprocal are the hardware's approximations (about one fp32 ulp each), far inside one ulp of the 16-bit outputs
+// this activation is used with.
 __device__ __forceinline__ float faster_gelu(float x)
 {
-    const float e = __builtin_amdgcn_exp2f((-1.702f * 1.44269504088896341f) * fabsf(x));
-    const float num = x < 0.0f ? x * e : x;
-    return num * __builtin_amdgcn_rcpf(1.0f + e);
+    const float e = __builtin_amdgcn_exp2f((-1.702f * 1.44269504088896341f) * x);
+    return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
 // SwiGLU of one column pair in fp32, one rounding per step, in the order of the reference's vector instructions
