@@ -202,7 +202,7 @@ uint32_t gemm_dma_skinny_splits(uint32_t m, uint32_t n, uint32_t k);
 bool gemm_stream_supported(const GemmParams& p);
 size_t gemm_stream_workspace(uint32_t m, uint32_t n, uint32_t k);
 int launch_gemm_stream(const GemmParams& p, void* workspace, hipStream_t st);
-int launch_gemm_dma_skinny(GemmParams& p, void* workspace, size_t workspace_bytes, hipStream_t st);
+int launch_gemm_dma_skinny(GemmParams& p, void* workspace, size_t workspace_bytes, hipStream_t st, bool b_nk = false);
 // Few rows, B as [n][k]: whole columns per workgroup, one launch, no workspace (matmul_w8a8_nk.hip).
 bool gemm_nk_supported(const GemmParams& p);
 int launch_gemm_nk(const GemmParams& p, hipStream_t st);

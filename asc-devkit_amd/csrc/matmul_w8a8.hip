@@ -646,7 +646,7 @@ extern "C" int ascq_matmul_w8a8_workspace_size(const ascq_matmul_desc* d, size_t
         // (few rows on [n, k] weights with k % 128 == 0 run the whole-column kernel, which needs none)
         *bytes = static_cast<size_t>(d->m) * d->n * sizeof(int32_t);
     }
-    if (d->m <= kSkinnyMaxM && !d->trans_a && !d->trans_b && d->k % 128 == 0 && d->n % 16 == 0) {
+    if (d->m <= kSkinnyMaxM && !d->trans_a && d->k % 128 == 0 && d->n % 16 == 0 && !(d->m <= 32 && d->trans_b)) {
         const size_t need =
             static_cast<size_t>(gemm_dma_skinny_splits(d->m, d->n, d->k)) * d->m * d->n * sizeof(int32_t);
         if (need > *bytes && need > static_cast<size_t>(d->m) * d->n * sizeof(int32_t)) {
@@ -729,11 +729,11 @@ extern "C" int ascq_matmul_w8a8(const ascq_matmul_desc* d, void* c, const void* 
         workspace_bytes >= gemm_stream_workspace(d->m, d->n, d->k)) {
         return launch_gemm_stream(p, workspace, st);
     }
-    if (d->m <= kSkinnyMaxM && !d->trans_b && gemm_dma_supported(p)) {
-        return launch_gemm_dma_skinny(p, workspace, workspace_bytes, st);
-    }
     if (d->m <= 32 && d->trans_b && !d->trans_a && gemm_nk_supported(p)) {
         return launch_gemm_nk(p, st);
+    }
+    if (d->m <= kSkinnyMaxM && !d->trans_a && gemm_dma_supported(p)) {
+        return launch_gemm_dma_skinny(p, workspace, workspace_bytes, st, d->trans_b != 0);
     }
     if (d->m <= 32) {
         const uint32_t splits = pick_k_splits(d->n, d->k);

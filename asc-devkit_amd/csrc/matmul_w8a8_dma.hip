@@ -818,9 +818,16 @@ int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st, bool b_nk)
 // one per CU otherwise; never more splits than K steps.
 uint32_t gemm_dma_skinny_splits(uint32_t m, uint32_t n, uint32_t k)
 {
+    // Measured at k = 4096, n = 11008 (86 column tiles) with the weights coming from HBM: one row tile (m <= 128) is
+    // fastest with 4 splits (17-25 us; 2 splits 21-25, 6 splits 25-32, none 30), two or more row tiles are fastest
+    // with none (30-32 us for m = 160 .. 384 against 32-55 with 2): once the tiles alone cover most of the compute
+    // units the int32 partial tiles, written and read back, cost more than the idle units.  Hence: no split from 160
+    // tiles on, otherwise about 1.35 workgroups per compute unit, all resident at once (two fit a unit).
     const uint32_t tiles = ((m + 127u) / 128u) * ((n + 127u) / 128u);
-    const uint32_t target = m <= 64u ? 512u : 300u;
-    uint32_t s = (target + tiles - 1u) / tiles;
+    if (tiles >= 160u) {
+        return 1u;
+    }
+    uint32_t s = 344u / tiles;
     const uint32_t steps = k / BK;
     if (s > steps) s = steps;
     if (s > 16u) s = 16u;
@@ -828,8 +835,8 @@ uint32_t gemm_dma_skinny_splits(uint32_t m, uint32_t n, uint32_t k)
 }
 
 // M up to a few hundred rows: 128 x 128 tiles, K split over blockIdx.y when a workspace of
-// splits * m * n * 4 bytes (16-byte aligned) is given.
-int launch_gemm_dma_skinny(GemmParams& p, void* workspace, size_t workspace_bytes, hipStream_t st)
+// splits * m * n * 4 bytes (16-byte aligned) is given.  b_nk: B is [n][k].
+int launch_gemm_dma_skinny(GemmParams& p, void* workspace, size_t workspace_bytes, hipStream_t st, bool b_nk)
 {
     p.tiles_m = (p.m + 127u) / 128u;
     p.tiles_n = (p.n + 127u) / 128u;
@@ -848,12 +855,20 @@ int launch_gemm_dma_skinny(GemmParams& p, void* workspace, size_t workspace_byte
         return ASCQ_OK;
     }
     if (splits == 1) {
-        gemm_dma_kernel<128, 128, false><<<t, kThreads, 0, st>>>(p, 0u);
+        if (b_nk) {
+            gemm_dma_kernel<128, 128, false, true><<<t, kThreads, 0, st>>>(p, 0u);
+        } else {
+            gemm_dma_kernel<128, 128, false><<<t, kThreads, 0, st>>>(p, 0u);
+        }
         return launch_status("ascq_matmul_w8a8");
     }
     p.k_splits = splits;
     p.partial = static_cast<int32_t*>(workspace);
-    gemm_dma_kernel<128, 128, true><<<dim3(t, splits), kThreads, 0, st>>>(p, 0u);
+    if (b_nk) {
+        gemm_dma_kernel<128, 128, true, true><<<dim3(t, splits), kThreads, 0, st>>>(p, 0u);
+    } else {
+        gemm_dma_kernel<128, 128, true><<<dim3(t, splits), kThreads, 0, st>>>(p, 0u);
+    }
     int rc = launch_status("ascq_matmul_w8a8 (split-K)");
     if (rc != ASCQ_OK) {
         return rc;

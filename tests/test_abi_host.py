@@ -232,10 +232,17 @@ def test_matmul_plan_of_the_benchmark_shapes():
     p, need = _plan(128, 11008, 4096)
     assert (p.kernel, p.tile_m, p.tile_n) == (abi.MM_KERNEL_DMA_128, 128, 128)
     assert (p.k_splits, p.workgroups, p.launches) == (4, 88 * 4, 2) and p.workspace_bytes == 4 * 128 * 11008 * 4
-    # B as [n, k]: the same direct-to-LDS tiles when A has more than 512 rows, the register-staged kernel below that
+    # two or more row tiles cover most of the compute units by themselves: no split
+    p, need = _plan(300, 11008, 4096)
+    assert (p.kernel, p.k_splits, p.workgroups, p.launches, p.workspace_bytes) == (abi.MM_KERNEL_DMA_128, 1, 264, 1, 0)
+    # B as [n, k] runs the same direct-to-LDS tiles at every m; a K that is no multiple of 128 the register-staged kernel
     p, _ = _plan(2048, 11008, 4096, trans_b=1)
     assert (p.kernel, p.tile_m, p.tile_n, p.narrow_tile_n, p.launches) == (abi.MM_KERNEL_DMA_256, 256, 256, 128, 1)
     p, _ = _plan(300, 11008, 4096, trans_b=1)
+    assert (p.kernel, p.tile_m, p.tile_n, p.k_splits, p.launches) == (abi.MM_KERNEL_DMA_128, 128, 128, 1, 1)
+    p, need = _plan(100, 11008, 4096, trans_b=1)
+    assert (p.kernel, p.k_splits, p.launches) == (abi.MM_KERNEL_DMA_128, 4, 2) and p.workspace_bytes == need
+    p, _ = _plan(300, 11008, 4096 + 64, trans_b=1)
     assert (p.kernel, p.launches) == (abi.MM_KERNEL_STAGED, 1)
     # odd addresses fall to the generic kernel
     p, _ = _plan(2048, 11008, 4096, a=0x10001)

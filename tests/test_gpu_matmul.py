@@ -139,6 +139,28 @@ def test_config3_w8a8_linear_weights_as_n_k(m):
     assert np.array_equal(bits(c8), oracle_mm(d8, a, wt, None, words))
 
 
+@pytest.mark.parametrize("m", [48, 128, 300, 512])
+def test_config3_w8a8_mid_m_both_weight_layouts(m):
+    """Config 3 between the decode sizes and the large tiles: 128 x 128 direct-to-LDS tiles, K split four ways for one
+    row tile and not at all for more, on weights as [k, n] and as [n, k]; bit-exact against the oracle."""
+    announce("config 3 mid m", m)
+    rng = np.random.default_rng(0xC3 + 200 + m)
+    k, n = 4096, 11008
+    a = rand_i8(rng, (m, k))
+    w = rand_i8(rng, (k, n))
+    cs = rng.uniform(1e-4, 1e-2, n).astype(np.float32)
+    ts = rng.uniform(1e-2, 1e-1, m).astype(np.float32)
+    c, desc = run_mm(m, n, k, a, w, out=torch.bfloat16, quant=cs, tok=ts)
+    want = oracle_mm(desc, a, w, None, cs, ts)
+    assert np.array_equal(bits(c), want)
+    ct, _ = run_mm(m, n, k, a, np.ascontiguousarray(w.T), out=torch.bfloat16, quant=cs, tok=ts, trans_b=True)
+    assert np.array_equal(bits(ct), want)
+    desc.trans_b = 1
+    wsz = C.c_size_t(0)
+    assert abi.load_library().ascq_matmul_w8a8_workspace_size(C.byref(desc), C.byref(wsz)) == abi.OK
+    assert wsz.value == (4 * m * n * 4 if m <= 128 else 0)
+
+
 def test_fixpipe_modes_uint64_words():
     announce("matmul fixpipe words: VDEQF16, DEQF16 scalar, VREQ8, bf16")
     rng = np.random.default_rng(21)
