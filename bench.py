@@ -57,7 +57,7 @@ def main():
     ap.add_argument("--quick", action="store_true", help="headline + W4A16 GEMV only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="run a single workload: w8a8 | w4a16 | w4a16_nd | w4a16_m4 | w4a16_m16 | w4a16_nd_m4 | w4a16_nd_m16 | "
-                         "w8a8_m1 | w8a8_m16 | w8a8_m128 | w8a8_nk_m1 | w8a8_nk_m16 | w8a16_m1 | w8a16_m16 | w8a16_nk_m1 | "
+                         "w8a8_m1 | w8a8_m8 | w8a8_m16 | w8a8_m128 | w8a8_m512 | w8a8_nk_m1 | w8a8_nk_m16 | w8a8_nk_m128 | w8a16_m1 | w8a16_m16 | w8a16_nk_m1 | "
                          "w8a16_nk_m16 | w8a16_m2048 | w8a16_nk_m2048 | quant | dequant | antiquant | group | group_example (a W4A16 name without _nd "
                          "is the packed-weight path; _nk: weights kept as [n, k])")
     ap.add_argument("--copy-probe", action="store_true",
@@ -356,7 +356,10 @@ def main():
               "w4a16_nd_m4": lambda: w4a16(4, args.steps, args.warmup),
               "w4a16_nd_m16": lambda: w4a16(16, args.steps, args.warmup),
               "w8a8_m1": lambda: w8a8(1, args.steps, args.warmup, sets=7),
+              "w8a8_m8": lambda: w8a8(8, args.steps, args.warmup, sets=7),
               "w8a8_m16": lambda: w8a8(16, args.steps, args.warmup, sets=7),
+              "w8a8_m512": lambda: w8a8(512, args.steps, args.warmup, sets=7),
+              "w8a8_nk_m128": lambda: w8a8(128, args.steps, args.warmup, sets=7, b_nk=True),
               "w8a8_m128": lambda: w8a8(128, args.steps, args.warmup, sets=7),
               "w8a8_nk_m1": lambda: w8a8(1, args.steps, args.warmup, sets=7, b_nk=True),
               "w8a8_nk_m16": lambda: w8a8(16, args.steps, args.warmup, sets=7, b_nk=True),
@@ -453,16 +456,17 @@ def main():
             r["hbm_frac"] = r["gbs"] / PEAK_HBM_GBS
             others[name] = r
             torch.cuda.empty_cache()
-        for M in (1, 16, 128):
+        for M in (1, 8, 16, 128, 512):
             r = strip(w8a8(M, s2, w2, sets=7))
             others[f"w8a8_m{M}"] = {"gemm_kernel_ms": r["gemm_kernel_ms"], "gemm_tops": r["gemm_tops"],
                                     "gemm_gbs": r["gemm_gbs"], "hbm_frac": r["gemm_gbs"] / PEAK_HBM_GBS,
                                     "mfma_frac": r["gemm_tops"] / PEAK_INT8_TOPS}
-        for M in (1, 16):
+        for M in (1, 16, 128):
             r = strip(w8a8(M, s2, w2, sets=7, b_nk=True))
             others[f"w8a8_nk_m{M}"] = {"gemm_kernel_ms": r["gemm_kernel_ms"], "gemm_gbs": r["gemm_gbs"],
                                        "hbm_frac": r["gemm_gbs"] / PEAK_HBM_GBS,
-                                       "note": "weights kept as [n, k] (isTransposeB): one launch, no workspace"}
+                                       "note": "weights kept as [n, k] (isTransposeB)" +
+                                               (": one launch, no workspace" if M <= 32 else "")}
             torch.cuda.empty_cache()
         for M in (4, 16):
             r = strip(w4a16(M, s2, w2))

@@ -381,13 +381,13 @@ int ascq_unpack_int4(void* dst, const void* src, size_t elements, void* stream);
  */
 typedef enum ascq_mm_kernel {
     ASCQ_MM_KERNEL_GENERIC = 0,      /* one lane per output element: unaligned or transposed-A inputs */
-    ASCQ_MM_KERNEL_STREAM = 1,       /* m <= 32: weight streams, one per SIMD, then a kernel that adds their pieces */
+    ASCQ_MM_KERNEL_STREAM = 1,       /* few rows: weight streams, one per SIMD, then a kernel that adds their pieces */
     ASCQ_MM_KERNEL_DMA_128 = 2,      /* m <= 512: 128 x 128 direct-to-LDS tiles, K split over workgroups when a
                                         workspace is given (k_splits > 1: a second kernel adds the partial tiles) */
     ASCQ_MM_KERNEL_DMA_256 = 3,      /* 256 x 256 direct-to-LDS tiles; a last partial round of the chip may be run
                                         by further workgroups of the same launch with 256 x narrow_tile_n tiles */
-    ASCQ_MM_KERNEL_STAGED = 4        /* register-staged tiles: transposed B with at most 512 rows of A, or K not a
-                                        multiple of 128 (a transposed B with more rows runs on KERNEL_DMA_256) */
+    ASCQ_MM_KERNEL_STAGED = 4        /* register-staged tiles: K not a multiple of 128, or n not a multiple of 16
+                                        (a transposed B otherwise runs on the direct-to-LDS kernels like a plain one) */
 } ascq_mm_kernel;
 
 typedef struct ascq_matmul_plan {
