@@ -362,6 +362,194 @@ __global__ __launch_bounds__(kWaves * 64) void w4a16_packed_kernel(W4pParams p)
     }
 }
 
+// 5 to 16 activation rows: the activations of a whole pass over k no longer fit the LDS wavefront by wavefront (the
+// kernel above would need several passes, each refetching parameters and restarting its stream), so the roles turn
+// round.  A wavefront owns one slab over all of k: its weights are one contiguous run and the sums of its 16 columns
+// never leave its registers - no reduction in LDS, no second pass.  The wavefronts of a workgroup walk k together and
+// share the activations: chunk c (8 tiles = 1024 k of all m rows) lies in one of two LDS buffers while the next is
+// fetched, one barrier per chunk.  The (scale, offset) pairs of a slab for all of k are staged once per wavefront.
+constexpr uint32_t kRowsBatch = 8;          // tiles per batch of weight loads = tiles per activation chunk
+constexpr uint32_t kRowsMaxGroups = 128;    // quantisation groups along k this kernel has LDS for
+constexpr uint32_t kRowsChunkBytes = kRowsBatch * kTileK * 2u;  // bytes of one activation row per chunk
+constexpr uint32_t kRowsPitch = kRowsChunkBytes + kRowPad;
+
+template <bool kHasOffset, uint32_t kW>
+__global__ __launch_bounds__(kW * 64) void w4a16_packed_rows_kernel(W4pParams p)
+{
+    constexpr uint32_t kT = kW * 64u;
+    constexpr uint32_t kXP = (kMaxRows * kRowsChunkBytes / 16u + kT - 1u) / kT;  // 16-byte pieces per thread and chunk
+    constexpr uint32_t kParWave = kSlabCols * (kRowsMaxGroups + 1u) * 4u;
+    __shared__ __attribute__((aligned(16))) char XS[2][kMaxRows * kRowsPitch];
+    __shared__ __attribute__((aligned(16))) char PARS[kW * kParWave];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t j = lane & 15u, g = lane >> 4;
+    const uint32_t slab = blockIdx.x * kW + wave;
+    const bool live = slab < p.slabs;  // a wavefront without a slab still stages activations and meets the barriers
+    char* const PAR = PARS + wave * kParWave;  // [column of the slab][group] (scale | offset << 16)
+    const uint32_t gsh = p.gs_shift;
+    const uint32_t groups = (p.k / 32u) >> gsh;
+    const uint32_t par_col = p.par_pitch * 4u;  // bytes of one column of the table (odd number of entries)
+    const uint32_t par_lane0 = (gsh <= 2u ? (g >> gsh) * 4u : 0u) + j * par_col;
+    const uint32_t x_lane = (j % p.m) * kRowsPitch + g * 64u;  // operand row i reads row i % m; + tile * 256 + d * 16
+    const uint32_t nb = (p.ktiles + kRowsBatch - 1u) / kRowsBatch;
+
+    NibbleMasks mk = p.mk;
+    asm volatile("" : "+v"(mk.exp));
+    const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<u32x4*>(p.wp), 0, static_cast<int>((p.slabs * p.ktiles + kPadTiles) * kTileBytes), 0x00020000);
+    const int par_bytes = static_cast<int>(groups * p.n * 2u);
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.scale), 0, par_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t*>(kHasOffset ? p.offset : p.scale), 0, par_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t*>(p.x), 0, static_cast<int>(p.m * p.k * 2u), 0x00020000);
+
+    // ---- the slab's parameters: lane i fetches 8 columns of group row r0 + i / 2
+    for (uint32_t r0 = 0; r0 < groups; r0 += 32u) {
+        const uint32_t r = r0 + (lane >> 1), c8 = (lane & 1u) * 8u;
+        const uint32_t col = slab * kSlabCols + c8;
+        const uint32_t off = (live && r < groups && col < p.n) ? (r * p.n + col) * 2u : kPastEnd;
+        const u32x4 sr = __builtin_amdgcn_raw_buffer_load_b128(rs, off, 0, 0);
+        u32x4 orr = u32x4{0, 0, 0, 0};
+        if constexpr (kHasOffset) {
+            orr = __builtin_amdgcn_raw_buffer_load_b128(ro, off, 0, 0);
+        }
+        if (r < groups) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                char* dst = PAR + (c8 + 2u * e) * par_col + r * 4u;
+                *reinterpret_cast<uint32_t*>(dst) = __builtin_amdgcn_perm(orr[e], sr[e], 0x05040100u);            // column 2e
+                *reinterpret_cast<uint32_t*>(dst + par_col) = __builtin_amdgcn_perm(orr[e], sr[e], 0x07060302u);  // column 2e + 1
+            }
+        }
+    }
+
+    // ---- activations of chunk c: piece i (16 bytes) is piece i % 128 of row i / 128
+    u32x4 xr[kXP];
+    auto xload = [&](uint32_t c) __attribute__((always_inline)) {
+#pragma unroll
+        for (uint32_t u = 0; u < kXP; ++u) {
+            const uint32_t i = tid + u * kT;
+            const uint32_t r = i >> 7, kk = c * (kRowsBatch * kTileK) + (i & 127u) * 8u;
+            xr[u] = __builtin_amdgcn_raw_buffer_load_b128(rx, (c < nb && r < p.m && kk < p.k) ? (r * p.k + kk) * 2u : kPastEnd, 0, 0);
+        }
+    };
+    auto xstore = [&](uint32_t c) __attribute__((always_inline)) {
+        char* dst = XS[c & 1u];
+#pragma unroll
+        for (uint32_t u = 0; u < kXP; ++u) {
+            const uint32_t i = tid + u * kT;
+            const uint32_t r = i >> 7;
+            if (c < nb && r < p.m) {
+                *reinterpret_cast<u32x4*>(dst + r * kRowsPitch + (i & 127u) * 16u) = xr[u];
+            }
+        }
+    };
+    // ---- weights of batch q: unconditional loads (a batch past the end, or of a wavefront without a slab, is given an
+    // offset beyond the buffer and moves no data; the last batch may read on into the next slab or the padding)
+    u32x4 wq[kBuf][kRowsBatch];
+    auto wload = [&](int buf, uint32_t q) __attribute__((always_inline)) {
+        const uint32_t l_w = (live && q < nb) ? lane * 16u : kPastEnd;
+        const uint32_t base = (slab * p.ktiles + q * kRowsBatch) * kTileBytes;  // scalar
+#pragma unroll
+        for (uint32_t t = 0; t < kRowsBatch; ++t) {
+            wq[buf][t] = __builtin_amdgcn_raw_buffer_load_b128(rw, l_w, base + t * kTileBytes, kNt);
+        }
+    };
+
+    f32x4 acc[2] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
+    auto compute = [&](int buf, uint32_t q) __attribute__((always_inline)) {
+        const uint32_t tt0 = q * kRowsBatch;
+        const uint32_t live_t = min(kRowsBatch, p.ktiles - tt0);
+        const char* xa0 = XS[q & 1u] + x_lane;
+        const char* pa0 = PAR + par_lane0 + (gsh <= 2u ? (tt0 * 4u) >> gsh : tt0 >> (gsh - 2u)) * 4u;
+        uint32_t pp[kRowsBatch];
+        uint32_t frac = 0;
+        if (gsh == 2u) {
+#pragma unroll
+            for (uint32_t t = 0; t < kRowsBatch; ++t) pp[t] = *reinterpret_cast<const uint32_t*>(pa0 + t * 4u);
+        } else {
+#pragma unroll
+            for (uint32_t t = 0; t < kRowsBatch; ++t) {
+                const uint32_t tt = tt0 + t;
+                const uint32_t grow = (gsh <= 2u ? (tt * 4u) >> gsh : tt >> (gsh - 2u)) - (gsh <= 2u ? (tt0 * 4u) >> gsh : tt0 >> (gsh - 2u));
+                pp[t] = *reinterpret_cast<const uint32_t*>(pa0 + grow * 4u);
+            }
+        }
+        if constexpr (kHasOffset) {
+#pragma unroll
+            for (uint32_t t = 0; t < kRowsBatch; ++t) {
+                const f16x2 k1536 = {static_cast<half_t>(1536.0f), static_cast<half_t>(1536.0f)};
+                const f16x2 rt = (bits_h2(pp[t]) + k1536) - k1536;
+                frac |= (h2_bits(rt) ^ pp[t]) & 0x7FFF0000u;  // the offset is the high half
+            }
+        }
+        const bool fold = kHasOffset && __builtin_amdgcn_ballot_w64(frac != 0u) == 0;  // uniform
+        auto tiles = [&](auto folded) __attribute__((always_inline)) {
+            constexpr bool kFold = decltype(folded)::value;
+#pragma unroll
+            for (uint32_t t = 0; t < kRowsBatch; ++t) {
+                if (t < live_t) {  // uniform
+                    const f16x2 sp = bits_h2(pp[t]);
+                    const f16x2 sc = {sp[0], sp[0]};
+                    f16x2 ofe = {sp[1], sp[1]}, ofo = ofe;
+                    if constexpr (kFold) {
+                        ofo = ofe - f16x2{static_cast<half_t>(72.0f), static_cast<half_t>(72.0f)};      // exact
+                        ofe = ofe - f16x2{static_cast<half_t>(1032.0f), static_cast<half_t>(1032.0f)};  // exact
+                    }
+#pragma unroll
+                    for (int d = 0; d < 4; ++d) {
+                        const f16x8 a = *reinterpret_cast<const f16x8*>(xa0 + t * 256u + d * 16);
+                        const f16x8 b = dequant8<kHasOffset, kFold>(wq[buf][t][d], sc, ofe, ofo, mk);
+                        acc[d & 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[d & 1], 0, 0, 0);
+                    }
+                }
+            }
+        };
+        if (fold) {
+            tiles(std::true_type{});
+        } else {
+            tiles(std::false_type{});
+        }
+    };
+
+    // One step: request the activations of the next chunk, then the weights of the batch after next (in that order:
+    // loads return in order, so the wait for the activations at the end of the step leaves that batch in flight),
+    // compute, hand the activations over, meet the other wavefronts.
+    auto step = [&](int buf, uint32_t q) __attribute__((always_inline)) {
+        xload(q + 1u);
+        wload((buf + 2) % kBuf, q + 2u);
+        if (live && q < nb) {  // uniform over the wavefront
+            compute(buf, q);
+        }
+        xstore(q + 1u);
+        __syncthreads();
+    };
+    xload(0);
+    wload(0, 0);
+    wload(1, 1);
+    xstore(0);
+    __syncthreads();
+    for (uint32_t q = 0; q < nb; q += 3u) {
+        step(0, q);
+        step(1, q + 1u);
+        step(2, q + 2u);
+    }
+
+    // ---- result row 4 (lane / 16) + r of column lane % 16: one rounding to half
+    const uint32_t col = slab * kSlabCols + j;
+    if (live && col < p.n) {
+#pragma unroll
+        for (uint32_t r = 0; r < 4; ++r) {
+            const uint32_t row = 4u * g + r;
+            if (row < p.m) {
+                p.y[static_cast<size_t>(row) * p.n + col] = static_cast<uint16_t>(f32_to_half_bits(acc[0][r] + acc[1][r]));
+            }
+        }
+    }
+}
+
 // ND [k, n / 2] (even column in the low nibble, two's complement) -> packed; one thread per lane of a tile.
 __global__ __launch_bounds__(256) void pack_w4_kernel(const uint8_t* __restrict__ w, u32x4* __restrict__ out, uint32_t k,
                                                       uint32_t n, uint32_t slabs, uint32_t ktiles)
@@ -476,6 +664,31 @@ extern "C" int ascq_matmul_w4a16_packed(const ascq_w4a16_desc* d, void* y, const
         p.m = d->m - m0 < kMaxRows ? d->m - m0 : kMaxRows;
         p.x = static_cast<const uint16_t*>(x) + static_cast<size_t>(m0) * d->k;
         p.y = static_cast<uint16_t*>(y) + static_cast<size_t>(m0) * d->n;
+        const uint32_t groups = d->k / d->group_size;
+        if (p.m > 4u && groups <= kRowsMaxGroups) {
+            // one wavefront per slab, the activations shared chunk by chunk: as many wavefronts per workgroup as give
+            // every compute unit a workgroup (7 at n = 28672 on 256 units), between 4 and 8
+            uint32_t kw = (p.slabs + cus - 1u) / cus;
+            kw = kw < 4u ? 4u : (kw > 8u ? 8u : kw);
+            p.par_pitch = groups | 1u;
+            const uint32_t grid = (p.slabs + kw - 1u) / kw;
+            auto go = [&](auto has_offset) {
+                constexpr bool kOff = decltype(has_offset)::value;
+                switch (kw) {
+                    case 4: w4a16_packed_rows_kernel<kOff, 4><<<grid, 4 * 64, 0, st>>>(p); break;
+                    case 5: w4a16_packed_rows_kernel<kOff, 5><<<grid, 5 * 64, 0, st>>>(p); break;
+                    case 6: w4a16_packed_rows_kernel<kOff, 6><<<grid, 6 * 64, 0, st>>>(p); break;
+                    case 7: w4a16_packed_rows_kernel<kOff, 7><<<grid, 7 * 64, 0, st>>>(p); break;
+                    default: w4a16_packed_rows_kernel<kOff, 8><<<grid, 8 * 64, 0, st>>>(p); break;
+                }
+            };
+            if (d->has_offset) {
+                go(std::true_type{});
+            } else {
+                go(std::false_type{});
+            }
+            continue;
+        }
         p.red_lanes = p.m <= 4u ? 16u : 64u;
         // Whole slabs per workgroup, one workgroup per compute unit when the slabs allow it; then the longest pass over
         // k whose activations and parameters fit their shares of the LDS (a multiple of the wavefront count), and fewer

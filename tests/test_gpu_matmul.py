@@ -391,6 +391,27 @@ def test_w4a16_packed_multi_pass_and_repeatable():
     assert torch.equal(y1, y2)
 
 
+@pytest.mark.parametrize("m,k,n,gs", [(7, 3200, 144, 64), (16, 5248, 48, 128), (12, 1024, 2320, 1024),
+                                      (8, 8192, 64, 32)])
+def test_w4a16_packed_more_than_four_rows(m, k, n, gs):
+    """5 to 16 rows on packed weights: one wavefront per slab over all of k, activations shared chunk by chunk.  k of
+    several chunks with a short last one, a last workgroup with idle wavefronts, one group per chunk; the last case has
+    more quantisation groups than that kernel stages and runs the kernel of the few-row case in several passes.  Two
+    calls give identical bits."""
+    announce("w4a16 packed rows", m, k, n, gs)
+    rng = np.random.default_rng(m * 131 + k + n)
+    x, wp, sc, of = w4_case(rng, m, k, n, gs, True)
+    w_gpu = ops.pack_weight_w4(to_dev(wp), k, n)
+    xs, scs, ofs = to_dev(x), to_dev(sc), to_dev(of)
+    y1 = torch.zeros((m, n), dtype=torch.float16, device=DEV)
+    y2 = torch.full((m, n), 7.0, dtype=torch.float16, device=DEV)
+    ops.matmul_w4a16_packed(y1, xs, w_gpu, scs, ofs, gs)
+    ops.matmul_w4a16_packed(y2, xs, w_gpu, scs, ofs, gs)
+    d = abi.W4A16Desc(m=m, n=n, k=k, group_size=gs, has_offset=1)
+    w4_check(y1.cpu().numpy(), orc.matmul_w4a16(d, x, wp, sc, of), x)
+    assert torch.equal(y1, y2)
+
+
 def config4_columns(m, n):
     """The oracle covers every column at M=1 (about 6 s on 16 threads); for more rows three slabs: the first and the last
     512 columns (the kernels' first and last column blocks) and one from the middle."""
