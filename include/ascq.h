@@ -494,9 +494,10 @@ int ascq_matmul_w4a16_workspace_size(const ascq_w4a16_desc* desc, size_t* bytes)
  * 16 tiles of w = 0 follow the last slab.  scale / offset stay [k / group_size, n].
  * ascq_matmul_w4a16_packed computes exactly what ascq_matmul_w4a16 computes (same roundings per weight, fp32 sums, one
  * rounding to half) in one launch with no workspace: a workgroup owns whole columns and adds its wavefronts' partial
- * sums in a fixed order, so repeated calls give identical bits.  It is built for 1-4 activation rows (decode) and takes
- * up to 16 per pass over the weights.  Requires k % 128 == 0, n % 8 == 0, group_size = 32 * 2^i (ASCQ_EUNSUPPORTED
- * otherwise: use ascq_matmul_w4a16), and x, w_packed, scale, offset 16-byte aligned.
+ * sums in a fixed order, so repeated calls give identical bits.  Up to 4 activation rows (decode) its wavefronts
+ * split k and add their sums in LDS; 5 to 16 rows run one wavefront per slab with the activations shared chunk by
+ * chunk; more rows take further passes of 16 over the weights.  Requires k % 128 == 0, n % 8 == 0, group_size =
+ * 32 * 2^i (ASCQ_EUNSUPPORTED otherwise: use ascq_matmul_w4a16), and x, w_packed, scale, offset 16-byte aligned.
  */
 int ascq_pack_weight_w4_size(uint32_t k, uint32_t n, size_t* bytes);
 int ascq_pack_weight_w4(const void* w, void* w_packed, uint32_t k, uint32_t n, void* stream);
