@@ -35,8 +35,13 @@ for _p in (os.path.join(ROOT, "asc-devkit_amd"), os.path.join(ROOT, "oracle")):
     if _p not in sys.path:
         sys.path.insert(0, _p)
 
-PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 matrix peak, TOP/s
-PEAK_HBM_GBS = 8000.0     # MI355X HBM3E peak, GB/s
+# MI355X published peaks (dense int8 matrix TOP/s, HBM3E GB/s, dense f16 matrix TFLOP/s): peaks.json beside this file
+# holds them together with the ceilings measured on the machine
+with open(os.path.join(ROOT, "peaks.json")) as _f:
+    _PEAKS = json.load(_f)["published"]
+PEAK_INT8_TOPS = float(_PEAKS["int8_dense_tops"])
+PEAK_HBM_GBS = float(_PEAKS["hbm_gbs"])
+PEAK_F16_TFLOPS = float(_PEAKS["f16_dense_tflops"])
 # Bytes that left / entered the L2 caches per launch, from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs of
 # `bench.py --quick --no-cpu --copy-probe`; each counter is scaled by its reading for the 1 GiB copy of the same run
 # (FETCH_SIZE reads 0.5 per KiB there, WRITE_SIZE 1.0 per KiB).  Measured offline and recorded here; a run of this
@@ -489,7 +494,7 @@ def main():
         for nk in (True, False):
             r = w8a16(2048, 30, 5, sets=1, b_nk=nk)
             others["w8a16_nk_m2048_k8192_n28672" if nk else "w8a16_m2048_k8192_n28672"] = {
-                "kernel_ms": r["kernel_ms"], "tflops": r["tflops"], "f16_mfma_frac": r["tflops"] / 2500.0,
+                "kernel_ms": r["kernel_ms"], "tflops": r["tflops"], "f16_mfma_frac": r["tflops"] / PEAK_F16_TFLOPS,
                 "note": "half GEMM whose B-tile loader de-quantises (w8a16_nk_gemm_kernel)" +
                         ("" if nk else ", after one transposed copy of the [k, n] weights into the workspace")}
             torch.cuda.empty_cache()
