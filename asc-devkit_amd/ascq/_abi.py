@@ -83,6 +83,11 @@ class W8A16Desc(C.Structure):
                 ("trans_b", C.c_int32)]
 
 
+class MxDesc(C.Structure):
+    _fields_ = [("m", C.c_uint32), ("n", C.c_uint32), ("k", C.c_uint32), ("scale_k", C.c_uint32),
+                ("a_format", C.c_int32), ("b_format", C.c_int32), ("out_dtype", C.c_int32), ("has_bias", C.c_int32)]
+
+
 class MatmulPlan(C.Structure):
     _fields_ = [("kernel", C.c_int32), ("tile_m", C.c_uint32), ("tile_n", C.c_uint32), ("tile_k", C.c_uint32),
                 ("workgroups", C.c_uint32), ("k_splits", C.c_uint32), ("launches", C.c_uint32),
@@ -119,6 +124,8 @@ SIGNATURES = {
     "ascq_matmul_w4a16_packed": (C.c_int, [C.POINTER(W4A16Desc), _P, _P, _P, _P, _P, _P]),
     "ascq_matmul_w8a16": (C.c_int, [C.POINTER(W8A16Desc), _P, _P, _P, _P, _P, _P, C.c_size_t, _P]),
     "ascq_matmul_w8a16_workspace_size": (C.c_int, [C.POINTER(W8A16Desc), C.POINTER(C.c_size_t)]),
+    "ascq_matmul_mx": (C.c_int, [C.POINTER(MxDesc), _P, _P, _P, _P, _P, _P, _P, C.c_size_t, _P]),
+    "ascq_matmul_mx_workspace_size": (C.c_int, [C.POINTER(MxDesc), C.POINTER(C.c_size_t)]),
     "ascq_get_ascend_quant_max_min_tmp_size": (C.c_int, [C.POINTER(C.c_uint32), C.c_uint32, C.c_uint32,
                                                          C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
     "ascq_get_ascend_dequant_max_min_tmp_size": (C.c_int, [C.POINTER(C.c_uint32), C.c_uint32, C.c_uint32,

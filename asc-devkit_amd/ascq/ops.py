@@ -523,6 +523,30 @@ def matmul_w8a16(y, x, w, offset=None, scale=None, workspace=None, trans_b=False
     return y
 
 
+# ------------------------------------------------------------------------------------------------- MX matmul
+_mx_ws = {}
+
+
+def matmul_mx(c, a, b, a_scale, b_scale, a_format, b_format, k, bias=None, workspace=None):
+    """MmadMx on whole matrices: c f32 / bf16 / f16 [m, n] = A @ B^T with a uint8 [m, k or k / 2] and b uint8
+    [n, k or k / 2] holding fp8 (abi.QDST_FP8_E4M3FN / _E5M2) or fp4 (abi.QDST_FP4_E2M1 / _E1M2, two per byte along k)
+    values and a_scale / b_scale uint8 [rows, scale_k] the fp8_e8m0 scale of every 32 k; bias f32 [n] or None."""
+    m, n = c.shape
+    d = abi.MxDesc(m=m, n=n, k=k, scale_k=a_scale.shape[1], a_format=a_format, b_format=b_format, out_dtype=_DT[c.dtype],
+                   has_bias=int(bias is not None))
+    lib = load_library()
+    need = C.c_size_t(0)
+    check(lib.ascq_matmul_mx_workspace_size(C.byref(d), C.byref(need)))
+    if workspace is None and need.value:
+        key = (c.device, need.value, _stream().value)   # one scratch buffer per stream: calls on two streams may overlap
+        if key not in _mx_ws:
+            _mx_ws[key] = torch.empty(need.value, dtype=torch.uint8, device=c.device)
+        workspace = _mx_ws[key]
+    check(lib.ascq_matmul_mx(C.byref(d), _ptr(c), _ptr(a), _ptr(b), _ptr(a_scale), _ptr(b_scale), _ptr(bias),
+                             _ptr(workspace), workspace.numel() if workspace is not None else 0, _stream()))
+    return c
+
+
 # ------------------------------------------------------------------------------------------- host size queries
 def _shape(shape):
     return (C.c_uint32 * len(shape))(*shape), len(shape)

@@ -1,0 +1,441 @@
+// Block-scaled (MX) matmul: c[m, n] = sum_k a[m, k] 2^(sa[m, k / 32] - 127) * b[n, k] 2^(sb[n, k / 32] - 127) (+ bias).
+// a and b are fp8 (e4m3fn, e5m2) or fp4 (e2m1, e1m2; two per byte along k), both k-contiguous; the scales are one
+// fp8_e8m0 byte per row and 32 k.
+//
+// The tile kernel feeds v_mfma_scale_f32_32x32x64_f8f6f4 straight from the given buffers: 256 x 256 tiles, K step of
+// 128 bytes of a row (128 fp8 or 256 fp4 values), two LDS stages filled by global_load_lds_dwordx4, 8 wavefronts as
+// 2 x 4, each on 128 x 64 of the tile (4 x 2 blocks of 32 x 32, 128 fp32 accumulators).  A tile row is a 128-byte line
+// in LDS whose 16-byte pieces are XOR-swizzled by half the row number, applied on the source side of the load.
+//   * 8-bit operands: one instruction takes 64 k; registers 0-3 of lane l hold k = 16 (l / 32) .. + 15 and registers
+//     4-7 k = 32 + 16 (l / 32) .. + 15 of row l % 32, and the scale of k < 32 comes from lanes 0-31, that of k >= 32
+//     from lanes 32-63: two 16-byte LDS reads per operand and instruction.
+//   * 4-bit operands: registers 0-3 of lane l hold its row's k = 32 (l / 32) .. + 31 (16 bytes), scaled by the lane's
+//     own scale byte: one read per operand and instruction.
+// In both cases lane l needs scale byte 2 j + l / 32 of its row's bytes for this K step in sub-step j; the bytes of a
+// K step are fetched as one dword (8-bit) or two (4-bit) per row and shifted right by 8 (l / 32) once, so that the
+// byte selector of the instruction is the constant 0 or 2.
+// The element-wise kernel (one lane per output) takes every other shape; 4-bit operands that have no tile path of
+// their own (e1m2, or a 4-bit operand beside an 8-bit one) are first widened to e4m3, which holds every fp4 value.
+#include "matmul_w8a8.h"
+
+namespace ascq {
+namespace {
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef __attribute__((address_space(1))) const void* gptr_t;
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr uint32_t kMxBM = 256, kMxBN = 256, kMxBK = 128;  // BK in bytes of an operand row
+constexpr int kMxThreads = 512;
+
+struct MxParams {
+    const uint8_t* a;
+    const uint8_t* b;
+    const uint8_t* sa;
+    const uint8_t* sb;
+    const float* bias;
+    void* c;
+    uint32_t m, n, k;       // k in elements
+    uint32_t row_bytes;     // bytes of a row of a / b in the tile kernel (both operands have the same width there)
+    uint32_t sk;            // bytes of a scale row
+    uint32_t tiles_m, tiles_n;
+    int32_t a_format, b_format, out_dtype;
+};
+
+__device__ __forceinline__ void mx_store(const MxParams& p, size_t idx, float v)
+{
+    if (p.out_dtype == ASCQ_F32) {
+        static_cast<float*>(p.c)[idx] = v;
+    } else if (p.out_dtype == ASCQ_BF16) {
+        static_cast<uint16_t*>(p.c)[idx] = static_cast<uint16_t>(f32_to_bf16_bits(v));
+    } else {
+        static_cast<uint16_t*>(p.c)[idx] = static_cast<uint16_t>(f32_to_half_bits_sat(v));
+    }
+}
+
+// kFour: both operands 4-bit (e2m1); otherwise both 8-bit with the instruction's format codes kCa / kCb
+// (0 = e4m3, 1 = e5m2; 4 = e2m1).
+template <bool kFour, int kCa, int kCb>
+__global__ __launch_bounds__(kMxThreads, 1) void mx_tile_kernel(MxParams p)
+{
+    __shared__ __attribute__((aligned(1024))) char A0[kMxBM * kMxBK];
+    __shared__ __attribute__((aligned(1024))) char B0[kMxBN * kMxBK];
+    __shared__ __attribute__((aligned(1024))) char A1[kMxBM * kMxBK];
+    __shared__ __attribute__((aligned(1024))) char B1[kMxBN * kMxBK];
+    constexpr int TI = 4, TJ = 2;
+    constexpr int kSub = kFour ? 4 : 2;       // instructions (64 k each) per K step and block pair
+    constexpr int kScaleDw = kFour ? 2 : 1;   // dwords of scale bytes per row and K step
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t wm = wave >> 2, wn = wave & 3u;
+    const uint32_t total = p.tiles_m * p.tiles_n;
+    const uint32_t t = xcd_remap(blockIdx.x, total);  // every XCD takes a contiguous share, row tiles innermost
+    if (t >= total) {
+        return;
+    }
+    const uint32_t row0 = (t % p.tiles_m) * kMxBM, n0 = (t / p.tiles_m) * kMxBN;
+    const uint32_t RB = p.row_bytes;
+
+    // ---- DMA sources: 4 A and 4 B instructions per wavefront and K step; lane owns LDS slot (instr * 64 + lane) of
+    // 16 bytes: row slot / 8, position slot % 8, which holds piece position ^ ((row / 2) % 8) of the row's 128 bytes
+    uint32_t aoff[4], boff[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const uint32_t s = (wave * 4u + u) * 64u + lane;
+        const uint32_t r = s >> 3, c = (s & 7u) ^ ((r >> 1) & 7u);
+        uint32_t row = row0 + r, col = n0 + r;
+        row = row < p.m ? row : p.m - 1u;  // rows and columns past the end are never stored: any valid one will do
+        col = col < p.n ? col : p.n - 1u;
+        aoff[u] = (row - row0) * RB + 16u * c;
+        boff[u] = (col - n0) * RB + 16u * c;
+    }
+    const uint8_t* Abase = p.a + static_cast<size_t>(row0) * RB;
+    const uint8_t* Bbase = p.b + static_cast<size_t>(n0) * RB;
+    auto issue = [&](uint32_t k0, char* As, char* Bs) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            __builtin_amdgcn_global_load_lds((gptr_t)(Abase + k0 + aoff[u]), (lds_ptr_t)(As + (wave * 4u + u) * 1024u), 16, 0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            __builtin_amdgcn_global_load_lds((gptr_t)(Bbase + k0 + boff[u]), (lds_ptr_t)(Bs + (wave * 4u + u) * 1024u), 16, 0, 0);
+        }
+    };
+
+    // ---- scale bytes of a K step: one or two dwords per operand row, already shifted for this lane's half
+    const uint32_t lrow = lane & 31u, h = lane >> 5;
+    const uint8_t* sa_row[TI];
+    const uint8_t* sb_row[TJ];
+#pragma unroll
+    for (int i = 0; i < TI; ++i) {
+        uint32_t row = row0 + (wm * TI + i) * 32u + lrow;
+        row = row < p.m ? row : p.m - 1u;
+        sa_row[i] = p.sa + static_cast<size_t>(row) * p.sk;
+    }
+#pragma unroll
+    for (int j = 0; j < TJ; ++j) {
+        uint32_t col = n0 + (wn * TJ + j) * 32u + lrow;
+        col = col < p.n ? col : p.n - 1u;
+        sb_row[j] = p.sb + static_cast<size_t>(col) * p.sk;
+    }
+    struct Scales {
+        uint32_t a[TI][kScaleDw], b[TJ][kScaleDw];
+    };
+    auto load_scales = [&](Scales& sc, uint32_t step) __attribute__((always_inline)) {
+        const uint32_t o = step * (4u * kScaleDw);
+#pragma unroll
+        for (int i = 0; i < TI; ++i) {
+#pragma unroll
+            for (int d = 0; d < kScaleDw; ++d) sc.a[i][d] = *reinterpret_cast<const uint32_t*>(sa_row[i] + o + 4u * d) >> (8u * h);
+        }
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) {
+#pragma unroll
+            for (int d = 0; d < kScaleDw; ++d) sc.b[j][d] = *reinterpret_cast<const uint32_t*>(sb_row[j] + o + 4u * d) >> (8u * h);
+        }
+    };
+
+    f32x16 acc[TI][TJ];
+#pragma unroll
+    for (int i = 0; i < TI; ++i) {
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+        }
+    }
+
+    // ---- fragments: piece q of tile line r sits at r * 128 + ((q ^ ((r / 2) % 8)) * 16)
+    const uint32_t swz = (lrow >> 1) & 7u;
+    auto frag = [&](const char* S, uint32_t line0, uint32_t piece) __attribute__((always_inline)) {
+        return *reinterpret_cast<const i32x4*>(S + (line0 + lrow) * 128u + ((piece ^ swz) << 4));
+    };
+    auto compute = [&](const char* As, const char* Bs, const Scales& sc) __attribute__((always_inline)) {
+#pragma unroll
+        for (int s = 0; s < kSub; ++s) {
+            v8i av[TI], bv[TJ];
+#pragma unroll
+            for (int i = 0; i < TI; ++i) {
+                const uint32_t line0 = (wm * TI + i) * 32u;  // (lines 32 apart share the swizzle of lrow)
+                if constexpr (kFour) {
+                    const i32x4 lo = frag(As, line0, 2u * s + h);
+                    av[i] = v8i{lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
+                } else {
+                    const i32x4 lo = frag(As, line0, 4u * s + h), hi = frag(As, line0, 4u * s + 2u + h);
+                    av[i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < TJ; ++j) {
+                const uint32_t line0 = (wn * TJ + j) * 32u;
+                if constexpr (kFour) {
+                    const i32x4 lo = frag(Bs, line0, 2u * s + h);
+                    bv[j] = v8i{lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
+                } else {
+                    const i32x4 lo = frag(Bs, line0, 4u * s + h), hi = frag(Bs, line0, 4u * s + 2u + h);
+                    bv[j] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < TI; ++i) {
+#pragma unroll
+                for (int j = 0; j < TJ; ++j) {
+                    // sub-step s uses scale byte 2 s (+ the lane's half, shifted in) of the step's bytes
+                    if (s & 1) {
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                            av[i], bv[j], acc[i][j], kCa, kCb, 2, static_cast<int>(sc.a[i][s >> 1]), 2,
+                            static_cast<int>(sc.b[j][s >> 1]));
+                    } else {
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                            av[i], bv[j], acc[i][j], kCa, kCb, 0, static_cast<int>(sc.a[i][s >> 1]), 0,
+                            static_cast<int>(sc.b[j][s >> 1]));
+                    }
+                }
+            }
+        }
+    };
+
+    // ---- main loop: the loads of step s + 1 (tiles by DMA, scales into registers) run under the arithmetic of step
+    // s; one wait and one barrier per step (the next stage has landed, and everyone has left the stage that the step
+    // after next will overwrite)
+    const uint32_t steps = RB / kMxBK;
+    Scales s0, s1;
+    issue(0, A0, B0);
+    load_scales(s0, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    for (uint32_t s = 0; s < steps; s += 2) {
+        if (s + 1u < steps) {
+            issue((s + 1u) * kMxBK, A1, B1);
+            load_scales(s1, s + 1u);
+        }
+        compute(A0, B0, s0);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (s + 1u < steps) {
+            if (s + 2u < steps) {
+                issue((s + 2u) * kMxBK, A0, B0);
+                load_scales(s0, s + 2u);
+            }
+            compute(A1, B1, s1);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+        }
+    }
+
+    // ---- register r of lane l in a 32 x 32 block: row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32
+#pragma unroll
+    for (int j = 0; j < TJ; ++j) {
+        const uint32_t col = n0 + (wn * TJ + j) * 32u + lrow;
+        const float bias = (p.bias != nullptr && col < p.n) ? p.bias[col] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < TI; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint32_t row = row0 + (wm * TI + i) * 32u + 8u * (r >> 2) + 4u * h + (r & 3);
+                if (row < p.m && col < p.n) {
+                    mx_store(p, static_cast<size_t>(row) * p.n + col, acc[i][j][r] + bias);
+                }
+            }
+        }
+    }
+}
+
+// value of an operand element: 8-bit formats by the hardware conversions (exact), 4-bit ones by their tables
+__device__ __forceinline__ float mx_value(const uint8_t* row, uint32_t k, int fmt)
+{
+    if (fmt == ASCQ_QDST_FP8_E4M3FN) {
+        return __builtin_amdgcn_cvt_f32_fp8(static_cast<int>(row[k]), 0);
+    }
+    if (fmt == ASCQ_QDST_FP8_E5M2) {
+        return __builtin_amdgcn_cvt_f32_bf8(static_cast<int>(row[k]), 0);
+    }
+    const uint32_t code = (row[k >> 1] >> (4u * (k & 1u))) & 15u;
+    const uint32_t mag = code & 7u;
+    float v;
+    if (fmt == ASCQ_QDST_FP4_E2M1) {
+        v = mag < 2u ? 0.5f * static_cast<float>(mag) : static_cast<float>(2u + (mag & 1u)) * static_cast<float>(1u << ((mag >> 1) - 1u)) * 0.5f;
+    } else {
+        v = 0.25f * static_cast<float>(mag);
+    }
+    return (code & 8u) ? -v : v;
+}
+
+__device__ __forceinline__ float e8m0_value(uint8_t e)
+{
+    // 2^(e - 127); e = 0 is 2^-127 (a subnormal float), e = 255 (NaN in the format) is passed on as NaN
+    return e == 255u ? __uint_as_float(0x7FC00000u) : (e == 0u ? __uint_as_float(0x00400000u) : __uint_as_float(static_cast<uint32_t>(e) << 23));
+}
+
+// One lane per output element; the sum of a block of 32 k is formed in fp32, scaled, and added to the total.
+__global__ __launch_bounds__(256) void mx_elementwise_kernel(MxParams p, uint32_t a_row_bytes, uint32_t b_row_bytes)
+{
+    const size_t total = static_cast<size_t>(p.m) * p.n;
+    for (size_t idx = static_cast<size_t>(blockIdx.x) * 256u + threadIdx.x; idx < total;
+         idx += static_cast<size_t>(gridDim.x) * 256u) {
+        const uint32_t i = static_cast<uint32_t>(idx / p.n), j = static_cast<uint32_t>(idx % p.n);
+        const uint8_t* ar = p.a + static_cast<size_t>(i) * a_row_bytes;
+        const uint8_t* br = p.b + static_cast<size_t>(j) * b_row_bytes;
+        float sum = 0.0f;
+        for (uint32_t k0 = 0; k0 < p.k; k0 += 32u) {
+            const uint32_t k1 = k0 + 32u < p.k ? k0 + 32u : p.k;
+            float part = 0.0f;
+            for (uint32_t k = k0; k < k1; ++k) {
+                part = __builtin_fmaf(mx_value(ar, k, p.a_format), mx_value(br, k, p.b_format), part);
+            }
+            const float sc = e8m0_value(p.sa[static_cast<size_t>(i) * p.sk + (k0 >> 5)]) * e8m0_value(p.sb[static_cast<size_t>(j) * p.sk + (k0 >> 5)]);
+            sum = __builtin_fmaf(part, sc, sum);
+        }
+        if (p.bias != nullptr) {
+            sum += p.bias[j];
+        }
+        mx_store(p, idx, sum);
+    }
+}
+
+// fp4 [rows, k / 2 bytes] -> e4m3 [rows, k bytes]; every fp4 value of either format is an e4m3 value.
+// e2m1 magnitudes 0 .5 1 1.5 2 3 4 6 and e1m2 magnitudes 0 .25 .. 1.75 as e4m3 codes (bias 7, 3 mantissa bits)
+__global__ __launch_bounds__(256) void mx_widen_fp4_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
+                                                           size_t bytes, int fmt)
+{
+    const uint64_t lut = fmt == ASCQ_QDST_FP4_E2M1 ? 0x4C4844403C383000ull : 0x3E3C3A3834302800ull;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * 256u + threadIdx.x; i < bytes; i += static_cast<size_t>(gridDim.x) * 256u) {
+        const uint32_t v = src[i];
+        const uint32_t lo = v & 15u, hi = v >> 4;
+        const uint32_t c0 = static_cast<uint32_t>(lut >> (8u * (lo & 7u))) & 0xFFu, c1 = static_cast<uint32_t>(lut >> (8u * (hi & 7u))) & 0xFFu;
+        reinterpret_cast<uint16_t*>(dst)[i] = static_cast<uint16_t>((c0 | ((lo & 8u) << 4)) | ((c1 | ((hi & 8u) << 4)) << 8));
+    }
+}
+
+inline bool is_fp8(int f) { return f == ASCQ_QDST_FP8_E4M3FN || f == ASCQ_QDST_FP8_E5M2; }
+inline bool is_fp4(int f) { return f == ASCQ_QDST_FP4_E2M1 || f == ASCQ_QDST_FP4_E1M2; }
+
+// which operands the tile path widens to e4m3 first: a 4-bit operand unless both are e2m1
+inline void mx_widen_plan(const ascq_mx_desc* d, bool& widen_a, bool& widen_b)
+{
+    const bool both_e2m1 = d->a_format == ASCQ_QDST_FP4_E2M1 && d->b_format == ASCQ_QDST_FP4_E2M1;
+    widen_a = is_fp4(d->a_format) && !both_e2m1;
+    widen_b = is_fp4(d->b_format) && !both_e2m1;
+}
+
+inline bool mx_tile_shape_ok(const ascq_mx_desc* d)
+{
+    bool wa, wb;
+    mx_widen_plan(d, wa, wb);
+    const bool four = is_fp4(d->a_format) && !wa;  // both e2m1
+    return d->k % (four ? 256u : 128u) == 0 && d->scale_k % 8u == 0 && d->m >= 64u && d->n >= 64u;
+}
+
+int mx_validate(const ascq_mx_desc* d, const char* who)
+{
+    ASCQ_REQUIRE(d != nullptr, ASCQ_ENULL, "%s: desc is NULL", who);
+    ASCQ_REQUIRE(d->m > 0 && d->n > 0 && d->k > 0, ASCQ_EINVAL, "%s: m, n, k must be greater than 0", who);
+    ASCQ_REQUIRE((is_fp8(d->a_format) || is_fp4(d->a_format)) && (is_fp8(d->b_format) || is_fp4(d->b_format)), ASCQ_EINVAL,
+                 "%s: a_format / b_format must be one of FP8_E4M3FN, FP8_E5M2, FP4_E2M1, FP4_E1M2", who);
+    ASCQ_REQUIRE(!(is_fp4(d->a_format) || is_fp4(d->b_format)) || d->k % 2u == 0, ASCQ_EINVAL,
+                 "%s: k %u must be even for a 4-bit operand (two values per byte)", who, d->k);
+    ASCQ_REQUIRE(d->scale_k >= (d->k + 31u) / 32u, ASCQ_EINVAL, "%s: scale_k %u is less than ceil(k / 32) = %u", who,
+                 d->scale_k, (d->k + 31u) / 32u);
+    ASCQ_REQUIRE(d->out_dtype == ASCQ_F32 || d->out_dtype == ASCQ_BF16 || d->out_dtype == ASCQ_F16, ASCQ_EINVAL,
+                 "%s: out_dtype must be F32, BF16 or F16", who);
+    return ASCQ_OK;
+}
+
+}  // namespace
+}  // namespace ascq
+
+using namespace ascq;
+
+extern "C" int ascq_matmul_mx_workspace_size(const ascq_mx_desc* d, size_t* bytes)
+{
+    ASCQ_REQUIRE(bytes != nullptr, ASCQ_ENULL, "ascq_matmul_mx_workspace_size: bytes is NULL");
+    const int rc = mx_validate(d, "ascq_matmul_mx_workspace_size");
+    if (rc != ASCQ_OK) {
+        return rc;
+    }
+    *bytes = 0;
+    bool wa, wb;
+    mx_widen_plan(d, wa, wb);
+    if ((wa || wb) && mx_tile_shape_ok(d)) {
+        *bytes = (wa ? static_cast<size_t>(d->m) * d->k : 0u) + (wb ? static_cast<size_t>(d->n) * d->k : 0u);
+    }
+    return ASCQ_OK;
+}
+
+// ref: include/basic_api/kernel_operator_mm_intf.h:321-340 (MmadMx); golden: examples/01_simd_cpp_api/03_basic_api/
+// 03_matrix_compute/mmad_mx/scripts/gen_data.py:52-140
+extern "C" int ascq_matmul_mx(const ascq_mx_desc* d, void* c, const void* a, const void* b, const void* a_scale,
+                              const void* b_scale, const void* bias, void* workspace, size_t workspace_bytes, void* stream)
+{
+    const int rc = mx_validate(d, "ascq_matmul_mx");
+    if (rc != ASCQ_OK) {
+        return rc;
+    }
+    ASCQ_REQUIRE(c && a && b && a_scale && b_scale, ASCQ_ENULL, "ascq_matmul_mx: c / a / b / a_scale / b_scale is NULL");
+    ASCQ_REQUIRE(!d->has_bias || bias, ASCQ_ENULL, "ascq_matmul_mx: bias is NULL");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    MxParams p{};
+    p.a = static_cast<const uint8_t*>(a);
+    p.b = static_cast<const uint8_t*>(b);
+    p.sa = static_cast<const uint8_t*>(a_scale);
+    p.sb = static_cast<const uint8_t*>(b_scale);
+    p.bias = d->has_bias ? static_cast<const float*>(bias) : nullptr;
+    p.c = c;
+    p.m = d->m;
+    p.n = d->n;
+    p.k = d->k;
+    p.sk = d->scale_k;
+    p.a_format = d->a_format;
+    p.b_format = d->b_format;
+    p.out_dtype = d->out_dtype;
+
+    bool wa, wb;
+    mx_widen_plan(d, wa, wb);
+    const size_t need = (wa ? static_cast<size_t>(d->m) * d->k : 0u) + (wb ? static_cast<size_t>(d->n) * d->k : 0u);
+    const bool tile = mx_tile_shape_ok(d) && aligned16(a) && aligned16(b) && (reinterpret_cast<uintptr_t>(a_scale) & 7u) == 0 &&
+                      (reinterpret_cast<uintptr_t>(b_scale) & 7u) == 0 &&
+                      (need == 0 || (workspace != nullptr && workspace_bytes >= need && aligned16(workspace)));
+    if (!tile) {
+        const uint32_t arb = is_fp4(d->a_format) ? d->k / 2u : d->k, brb = is_fp4(d->b_format) ? d->k / 2u : d->k;
+        size_t blocks = (static_cast<size_t>(d->m) * d->n + 255u) / 256u;
+        if (blocks > 65536u) blocks = 65536u;
+        mx_elementwise_kernel<<<static_cast<uint32_t>(blocks), 256, 0, st>>>(p, arb, brb);
+        return launch_status("ascq_matmul_mx (element-wise)");
+    }
+    int fa = d->a_format, fb = d->b_format;
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
+    auto widen = [&](const uint8_t*& src, int& fmt, size_t rows) {
+        const size_t bytes = rows * (d->k / 2u);
+        size_t blocks = (bytes + 255u) / 256u;
+        if (blocks > 65536u) blocks = 65536u;
+        mx_widen_fp4_kernel<<<static_cast<uint32_t>(blocks), 256, 0, st>>>(src, ws, bytes, fmt);
+        src = ws;
+        ws += rows * d->k;
+        fmt = ASCQ_QDST_FP8_E4M3FN;
+    };
+    if (wa) {
+        widen(p.a, fa, d->m);
+    }
+    if (wb) {
+        widen(p.b, fb, d->n);
+    }
+    const bool four = is_fp4(fa);
+    p.row_bytes = four ? d->k / 2u : d->k;
+    p.tiles_m = (d->m + kMxBM - 1u) / kMxBM;
+    p.tiles_n = (d->n + kMxBN - 1u) / kMxBN;
+    const uint32_t grid = (p.tiles_m * p.tiles_n + 7u) / 8u * 8u;
+    if (four) {
+        mx_tile_kernel<true, 4, 4><<<grid, kMxThreads, 0, st>>>(p);
+    } else if (fa == ASCQ_QDST_FP8_E4M3FN && fb == ASCQ_QDST_FP8_E4M3FN) {
+        mx_tile_kernel<false, 0, 0><<<grid, kMxThreads, 0, st>>>(p);
+    } else if (fa == ASCQ_QDST_FP8_E4M3FN) {
+        mx_tile_kernel<false, 0, 1><<<grid, kMxThreads, 0, st>>>(p);
+    } else if (fb == ASCQ_QDST_FP8_E4M3FN) {
+        mx_tile_kernel<false, 1, 0><<<grid, kMxThreads, 0, st>>>(p);
+    } else {
+        mx_tile_kernel<false, 1, 1><<<grid, kMxThreads, 0, st>>>(p);
+    }
+    return launch_status("ascq_matmul_mx");
+}

@@ -538,6 +538,39 @@ int ascq_matmul_w8a16(const ascq_w8a16_desc* desc, void* y, const void* x, const
                       const void* scale, void* workspace, size_t workspace_bytes, void* stream);
 int ascq_matmul_w8a16_workspace_size(const ascq_w8a16_desc* desc, size_t* bytes);
 
+/* --------------------------------------------- block-scaled (MX) matmul */
+/*
+ * MmadMx as a whole-matrix operator: c[m, n] = sum_k A[i, k] * B[j, k] (+ bias[j]) with
+ *   A[i, k] = value(a[i, k]) * 2^(a_scale[i, k / 32] - 127),  B[j, k] = value(b[j, k]) * 2^(b_scale[j, k / 32] - 127):
+ * every 32 consecutive k of a row share one fp8_e8m0 scale.  a is [m, k] and b is [n, k] (the right matrix and its
+ * scales transposed, the form the reference's examples feed), row-major; 4-bit formats are packed two per byte along k,
+ * even k in the low nibble, rows of k / 2 bytes (k even).  a_scale is [m, scale_k] and b_scale [n, scale_k] bytes with
+ * scale_k >= ceil(k / 32) (the reference rounds it up to an even number).  Products and sums are fp32 in the matrix
+ * core (exact products; the sum's order is the hardware's), c is rounded once: the reference's golden is the float64
+ * product rounded to the output type, compared at rtol = atol = 1e-3.
+ * a_format / b_format: ASCQ_QDST_FP8_E4M3FN | ASCQ_QDST_FP8_E5M2 | ASCQ_QDST_FP4_E2M1 | ASCQ_QDST_FP4_E1M2.
+ * Two 8-bit operands, or two e2m1 operands, with k % 128 == 0 (8-bit) / k % 256 == 0 (4-bit), 16-byte aligned a, b and
+ * scale_k % 8 == 0 run v_mfma_scale_f32_32x32x64_f8f6f4 on 256 x 256 tiles straight from the given buffers.  Other
+ * format pairs first widen their 4-bit operands to e4m3 (exact) in the workspace; other shapes take a kernel with one
+ * lane per output element.
+ * ref: include/basic_api/kernel_operator_mm_intf.h:321-340 (MmadMx), examples/01_simd_cpp_api/03_basic_api/
+ *      03_matrix_compute/mmad_mx/README.md:5,131-152 and scripts/gen_data.py:52-140 (layouts, golden),
+ *      examples/01_simd_cpp_api/05_best_practices/01_matrix_compute/matmul_mxfp4_basic_api_high_performance/
+ *      scripts/gen_data.py:36-72 (m = n = k = 8192, bfloat16 output).
+ */
+typedef struct ascq_mx_desc {
+    uint32_t m, n, k;
+    uint32_t scale_k;    /* bytes per row of a_scale / b_scale */
+    int32_t a_format;    /* ascq_quant_dst: FP8_E4M3FN, FP8_E5M2, FP4_E2M1, FP4_E1M2 */
+    int32_t b_format;
+    int32_t out_dtype;   /* ASCQ_F32 | ASCQ_BF16 | ASCQ_F16 */
+    int32_t has_bias;    /* bias is fp32 [n], added to the fp32 sum before the rounding */
+} ascq_mx_desc;
+
+int ascq_matmul_mx(const ascq_mx_desc* desc, void* c, const void* a, const void* b, const void* a_scale,
+                   const void* b_scale, const void* bias, void* workspace, size_t workspace_bytes, void* stream);
+int ascq_matmul_mx_workspace_size(const ascq_mx_desc* desc, size_t* bytes);
+
 /* --------------------------------------------- host "tiling" size queries */
 /*
  * Scratch-size queries with the reference's answers, for callers that size a

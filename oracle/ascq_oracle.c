@@ -1125,6 +1125,71 @@ int orc_matmul_w8a16(const ascq_w8a16_desc* d, void* y, const uint16_t* x, const
     return 0;
 }
 
+/* ------------------------------------------------ block-scaled (MX) matmul */
+/* Restates the golden of the reference's MmadMx examples: every operand element is its format's value times
+ * 2^(scale - 127) of its row and block of 32 k, the product of the two decompressed matrices is formed in float64 and
+ * rounded to the output type (examples/01_simd_cpp_api/03_basic_api/03_matrix_compute/mmad_mx/scripts/
+ * gen_data.py:52-83,117-126; .../matmul_mxfp4_basic_api_high_performance/scripts/gen_data.py:50-63); a float32 bias
+ * is added to the float32 result (gen_data.py:123-126).  b is [n, k] (the transposed right matrix the examples
+ * write), 4-bit operands two per byte with the even k in the low nibble (pack_fp4_to_fp4x2, gen_data.py:38-49).
+ * rows [r0, r1) and columns [c0, c1) are computed (the others of c are left alone).  Test infrastructure only. */
+static double mx_elem(const uint8_t* row, size_t k, int fmt)
+{
+    if (fmt == ASCQ_QDST_FP8_E4M3FN || fmt == ASCQ_QDST_FP8_E5M2) {
+        return (double)orc_fp8_to_f32(row[k], fmt == ASCQ_QDST_FP8_E5M2);
+    }
+    return (double)orc_fp4_to_f32((uint8_t)((row[k >> 1] >> (4 * (k & 1))) & 15), fmt == ASCQ_QDST_FP4_E1M2);
+}
+
+int orc_matmul_mx(const ascq_mx_desc* d, void* c, const uint8_t* a, const uint8_t* b, const uint8_t* sa,
+                  const uint8_t* sb, const float* bias, uint32_t r0, uint32_t r1, uint32_t c0, uint32_t c1)
+{
+    const size_t K = d->k, N = d->n, SK = d->scale_k;
+    const size_t arb = (d->a_format == ASCQ_QDST_FP4_E2M1 || d->a_format == ASCQ_QDST_FP4_E1M2) ? K / 2 : K;
+    const size_t brb = (d->b_format == ASCQ_QDST_FP4_E2M1 || d->b_format == ASCQ_QDST_FP4_E1M2) ? K / 2 : K;
+    /* decompress the columns once */
+    double* bd = (double*)malloc((size_t)(c1 - c0) * K * sizeof(double));
+    if (!bd) {
+        return -1;
+    }
+#pragma omp parallel for schedule(static)
+    for (long j = c0; j < (long)c1; ++j) {
+        for (size_t k = 0; k < K; ++k) {
+            bd[(size_t)(j - c0) * K + k] = mx_elem(b + (size_t)j * brb, k, d->b_format) * ldexp(1.0, (int)sb[(size_t)j * SK + k / 32] - 127);
+        }
+    }
+#pragma omp parallel
+    {
+        double* ad = (double*)malloc(K * sizeof(double));
+#pragma omp for schedule(dynamic, 1)
+        for (long i = r0; i < (long)r1; ++i) {
+            for (size_t k = 0; k < K; ++k) {
+                ad[k] = mx_elem(a + (size_t)i * arb, k, d->a_format) * ldexp(1.0, (int)sa[(size_t)i * SK + k / 32] - 127);
+            }
+            for (size_t j = c0; j < c1; ++j) {
+                const double* bj = bd + (j - c0) * K;
+                double acc = 0.0;
+                for (size_t k = 0; k < K; ++k) acc += ad[k] * bj[k];
+                float v = (float)acc;
+                if (d->has_bias) {
+                    v = v + bias[j];
+                }
+                const size_t idx = (size_t)i * N + j;
+                if (d->out_dtype == ASCQ_F32) {
+                    ((float*)c)[idx] = v;
+                } else if (d->out_dtype == ASCQ_BF16) {
+                    ((uint16_t*)c)[idx] = orc_f32_to_bf16(v);
+                } else {
+                    ((uint16_t*)c)[idx] = orc_f32_to_f16(v);
+                }
+            }
+        }
+        free(ad);
+    }
+    free(bd);
+    return 0;
+}
+
 /* ------------------------------------------------ vectorised array helpers */
 void orc_f32_to_f16_array(uint16_t* dst, const float* src, size_t n)
 {

@@ -54,6 +54,8 @@ int orc_antiquant_policy(const ascq_antiquant_policy_desc* d, void* dst, const u
 int orc_matmul_w8a16(const ascq_w8a16_desc* d, void* y, const uint16_t* x, const int8_t* w, const uint16_t* offset,
                      const uint16_t* scale);
 
+int orc_matmul_mx(const ascq_mx_desc* d, void* c, const uint8_t* a, const uint8_t* b, const uint8_t* sa,
+                  const uint8_t* sb, const float* bias, uint32_t r0, uint32_t r1, uint32_t c0, uint32_t c1);
 void orc_f32_to_f16_array(uint16_t* dst, const float* src, size_t n);
 void orc_f16_to_f32_array(float* dst, const uint16_t* src, size_t n);
 void orc_f32_to_bf16_array(uint16_t* dst, const float* src, size_t n);

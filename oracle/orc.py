@@ -68,6 +68,8 @@ def lib():
         L.orc_matmul_w4a16.argtypes = [C.POINTER(abi.W4A16Desc), _P, _P, _P, _P, _P]
         L.orc_matmul_w4a16_cols.argtypes = [C.POINTER(abi.W4A16Desc), _P, _P, _P, _P, _P, C.c_uint32, C.c_uint32]
         L.orc_matmul_w8a16.argtypes = [C.POINTER(abi.W8A16Desc), _P, _P, _P, _P, _P]
+        L.orc_matmul_mx.argtypes = [C.POINTER(abi.MxDesc), _P, _P, _P, _P, _P, _P, C.c_uint32, C.c_uint32, C.c_uint32,
+                                    C.c_uint32]
         L.orc_antiquant_policy.argtypes = [C.POINTER(abi.AntiQuantPolicyDesc), _P, _P, _P, _P]
         for name in ("orc_f32_to_f16_array", "orc_f16_to_f32_array", "orc_f32_to_bf16_array"):
             getattr(L, name).argtypes = [_P, _P, C.c_size_t]
@@ -227,6 +229,18 @@ def matmul_w8a16(desc, x, w, offset=None, scale=None):
     y = np.zeros((desc.m, desc.n), dtype=_NP[desc.out_dtype])
     lib().orc_matmul_w8a16(C.byref(desc), _ptr(y), _ptr(x), _ptr(w), _ptr(offset), _ptr(scale))
     return y
+
+
+def matmul_mx(desc, a, b, a_scale, b_scale, bias=None, rows=None, cols=None):
+    """a [m, k] / b [n, k] raw bytes (4-bit formats packed two per byte along k), scales uint8 [rows, scale_k].  Only
+    the rows / columns of the given ranges are computed; the rest of the result is zero."""
+    c = np.zeros((desc.m, desc.n), dtype=_NP[desc.out_dtype])
+    r0, r1 = rows if rows is not None else (0, desc.m)
+    c0, c1 = cols if cols is not None else (0, desc.n)
+    rc = lib().orc_matmul_mx(C.byref(desc), _ptr(c), _ptr(a), _ptr(b), _ptr(a_scale), _ptr(b_scale), _ptr(bias), r0, r1,
+                             c0, c1)
+    assert rc == 0
+    return c
 
 
 def antiquant_policy(desc, src, scale, offset=None):

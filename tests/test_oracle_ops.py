@@ -782,3 +782,81 @@ def test_hifloat8_codec_is_the_reference_script():
     xs = np.sort(np.abs(g["f32_in"][np.isfinite(g["f32_in"])]))
     vals = np.array([L.orc_hif8_to_f32(L.orc_f32_to_hif8(float(x))) for x in xs])
     assert np.all(np.diff(vals) >= 0)
+
+
+# ------------------------------------------------------------------------------------------------- MX matmul
+MX_FP4 = {abi.QDST_FP4_E2M1: [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0],
+          abi.QDST_FP4_E1M2: [0.0, 0.25, 0.5, 0.75, 1.0, 1.25, 1.5, 1.75]}
+MX_FP8 = {abi.QDST_FP8_E4M3FN: torch.float8_e4m3fn, abi.QDST_FP8_E5M2: torch.float8_e5m2}
+
+
+def mx_random_operand(rng, rows, k, fmt):
+    """Raw bytes of a [rows, k] operand with finite values: fp8 one per byte, fp4 two per byte (even k low)."""
+    if fmt in MX_FP8:
+        code = rng.integers(0, 256, (rows, k)).astype(np.uint8)
+        bad = (code & 0x7F) == 0x7F if fmt == abi.QDST_FP8_E4M3FN else (code & 0x7C) == 0x7C
+        code[bad] &= 0x80    # NaN / infinity codes become +-0
+        return code
+    return rng.integers(0, 256, (rows, k // 2)).astype(np.uint8)
+
+
+def mx_values(raw, k, fmt):
+    """The operand's values as float64 [rows, k], decoded by torch's 8-bit float types or the 4-bit formats' value
+    tables (an implementation that shares nothing with the oracle's)."""
+    if fmt in MX_FP8:
+        return torch.from_numpy(raw.copy()).view(MX_FP8[fmt]).to(torch.float64).numpy()
+    nib = np.stack([raw & 15, raw >> 4], axis=-1).reshape(raw.shape[0], k)
+    mag = np.array(MX_FP4[fmt])[nib & 7]
+    return np.where(nib & 8, -mag, mag)
+
+
+def mx_golden(a, b, sa, sb, k, fa, fb, bias=None):
+    """The data scripts' computation: decompress (value * 2^(scale - 127), block of 32 along k), float64 matmul, float32
+    (mmad_mx/scripts/gen_data.py:52-83, 117-126)."""
+    blk = np.arange(k) // 32
+    af = mx_values(a, k, fa) * np.power(2.0, sa.astype(np.float64) - 127.0)[:, blk]
+    bf = mx_values(b, k, fb) * np.power(2.0, sb.astype(np.float64) - 127.0)[:, blk]
+    out = np.matmul(af, bf.T).astype(np.float32)
+    return out if bias is None else out + bias
+
+
+@pytest.mark.parametrize("fa,fb", [(abi.QDST_FP4_E1M2, abi.QDST_FP4_E2M1), (abi.QDST_FP4_E2M1, abi.QDST_FP4_E1M2),
+                                   (abi.QDST_FP8_E4M3FN, abi.QDST_FP8_E5M2), (abi.QDST_FP8_E5M2, abi.QDST_FP8_E4M3FN),
+                                   (abi.QDST_FP8_E4M3FN, abi.QDST_FP4_E2M1)])
+@pytest.mark.parametrize("bias", [False, True])
+def test_matmul_mx_is_the_data_scripts_decompress_then_float64_matmul(fa, fb, bias):
+    """The reference example's own shape ([40, 70] x [50, 70], scale_k = ceil(70 / 32) rounded up to even = 4) and its
+    four format pairs plus a mixed one, against numpy float64 on operands decoded by torch / value tables."""
+    rng = np.random.default_rng(70 + fa * 8 + fb)
+    m, n, k, sk = 40, 50, 70, 4
+    a, b = mx_random_operand(rng, m, k, fa), mx_random_operand(rng, n, k, fb)
+    sa, sb = rng.integers(120, 135, (m, sk)).astype(np.uint8), rng.integers(120, 135, (n, sk)).astype(np.uint8)
+    bv = rng.integers(-10, 10, n).astype(np.float32) if bias else None
+    d = abi.MxDesc(m=m, n=n, k=k, scale_k=sk, a_format=fa, b_format=fb, out_dtype=abi.F32, has_bias=int(bias))
+    got = orc.matmul_mx(d, a, b, sa, sb, bv)
+    assert np.array_equal(got, mx_golden(a, b, sa, sb, k, fa, fb, bv))
+    d.out_dtype = abi.BF16
+    want16 = torch.from_numpy(mx_golden(a, b, sa, sb, k, fa, fb, bv)).to(torch.bfloat16).view(torch.int16).numpy()
+    assert np.array_equal(orc.matmul_mx(d, a, b, sa, sb, bv).view(np.int16), want16)
+
+
+def test_matmul_mx_closed_forms():
+    """All-ones operands count k; one more in a scale byte doubles exactly that row's block; the sub-range arguments
+    leave the rest of the result alone."""
+    m, n, k, sk = 3, 5, 96, 4
+    one8, one4 = 0x38, 0x22   # 1.0 in e4m3fn, (1.0, 1.0) in e2m1
+    a = np.full((m, k), one8, np.uint8)
+    b = np.full((n, k // 2), one4, np.uint8)
+    sa, sb = np.full((m, sk), 127, np.uint8), np.full((n, sk), 127, np.uint8)
+    d = abi.MxDesc(m=m, n=n, k=k, scale_k=sk, a_format=abi.QDST_FP8_E4M3FN, b_format=abi.QDST_FP4_E2M1,
+                   out_dtype=abi.F32, has_bias=0)
+    assert np.all(orc.matmul_mx(d, a, b, sa, sb) == k)
+    sa[1, 2] = 128
+    want = np.full((m, n), float(k), np.float32)
+    want[1, :] += 32
+    assert np.array_equal(orc.matmul_mx(d, a, b, sa, sb), want)
+    sb[4, 0] = 125
+    want[:, 4] -= 32 * 0.75
+    assert np.array_equal(orc.matmul_mx(d, a, b, sa, sb), want)
+    part = orc.matmul_mx(d, a, b, sa, sb, rows=(1, 2), cols=(3, 5))
+    assert np.array_equal(part[1, 3:5], want[1, 3:5]) and np.count_nonzero(part) == 2
