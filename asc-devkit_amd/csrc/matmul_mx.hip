@@ -16,6 +16,9 @@
 // byte selector of the instruction is the constant 0 or 2.
 // The element-wise kernel (one lane per output) takes every other shape; 4-bit operands that have no tile path of
 // their own (e1m2, or a 4-bit operand beside an 8-bit one) are first widened to e4m3, which holds every fp4 value.
+#include <type_traits>
+#include <utility>
+
 #include "matmul_w8a8.h"
 
 namespace ascq {
@@ -25,6 +28,18 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef __attribute__((address_space(1))) const void* gptr_t;
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant expression.
+template <class F, int... I>
+__device__ __forceinline__ void mx_static_for_impl(F&& f, std::integer_sequence<int, I...>)
+{
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void mx_static_for(F&& f)
+{
+    mx_static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
 
 constexpr uint32_t kMxBM = 256, kMxBN = 256, kMxBK = 128;  // BK in bytes of an operand row
 constexpr int kMxThreads = 512;
@@ -106,35 +121,33 @@ __global__ __launch_bounds__(kMxThreads, 1) void mx_tile_kernel(MxParams p)
 
     // ---- scale bytes of a K step: one or two dwords per operand row, already shifted for this lane's half
     const uint32_t lrow = lane & 31u, h = lane >> 5;
-    const uint8_t* sa_row[TI];
-    const uint8_t* sb_row[TJ];
+    uint32_t sa_row[TI], sb_row[TJ];  // byte offsets of the lane's scale rows (m * sk and n * sk stay below 2^32)
 #pragma unroll
     for (int i = 0; i < TI; ++i) {
         uint32_t row = row0 + (wm * TI + i) * 32u + lrow;
         row = row < p.m ? row : p.m - 1u;
-        sa_row[i] = p.sa + static_cast<size_t>(row) * p.sk;
+        sa_row[i] = row * p.sk;
     }
 #pragma unroll
     for (int j = 0; j < TJ; ++j) {
         uint32_t col = n0 + (wn * TJ + j) * 32u + lrow;
         col = col < p.n ? col : p.n - 1u;
-        sb_row[j] = p.sb + static_cast<size_t>(col) * p.sk;
+        sb_row[j] = col * p.sk;
     }
     struct Scales {
         uint32_t a[TI][kScaleDw], b[TJ][kScaleDw];
     };
+    // dword d of the scale bytes of a K step
+    auto load_scales_dw = [&](Scales& sc, uint32_t step, int d) __attribute__((always_inline)) {
+        const uint32_t o = step * (4u * kScaleDw) + 4u * d;
+#pragma unroll
+        for (int i = 0; i < TI; ++i) sc.a[i][d] = *reinterpret_cast<const uint32_t*>(p.sa + sa_row[i] + o) >> (8u * h);
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) sc.b[j][d] = *reinterpret_cast<const uint32_t*>(p.sb + sb_row[j] + o) >> (8u * h);
+    };
     auto load_scales = [&](Scales& sc, uint32_t step) __attribute__((always_inline)) {
-        const uint32_t o = step * (4u * kScaleDw);
 #pragma unroll
-        for (int i = 0; i < TI; ++i) {
-#pragma unroll
-            for (int d = 0; d < kScaleDw; ++d) sc.a[i][d] = *reinterpret_cast<const uint32_t*>(sa_row[i] + o + 4u * d) >> (8u * h);
-        }
-#pragma unroll
-        for (int j = 0; j < TJ; ++j) {
-#pragma unroll
-            for (int d = 0; d < kScaleDw; ++d) sc.b[j][d] = *reinterpret_cast<const uint32_t*>(sb_row[j] + o + 4u * d) >> (8u * h);
-        }
+        for (int d = 0; d < kScaleDw; ++d) load_scales_dw(sc, step, d);
     };
 
     f32x16 acc[TI][TJ];
@@ -147,61 +160,77 @@ __global__ __launch_bounds__(kMxThreads, 1) void mx_tile_kernel(MxParams p)
         }
     }
 
-    // ---- fragments: piece q of tile line r sits at r * 128 + ((q ^ ((r / 2) % 8)) * 16)
-    const uint32_t swz = (lrow >> 1) & 7u;
-    auto frag = [&](const char* S, uint32_t line0, uint32_t piece) __attribute__((always_inline)) {
-        return *reinterpret_cast<const i32x4*>(S + (line0 + lrow) * 128u + ((piece ^ swz) << 4));
+    // ---- fragments: piece q of tile line r sits at r * 128 + ((q ^ ((r / 2) % 8)) * 16).  A lane reads piece
+    // kPieceStep u + h (+ 2 for the upper registers of an 8-bit operand) of a line whose number is lrow + a multiple
+    // of 32, i.e. at lrow * 128 + (((kPieceStep u) ^ (h ^ swizzle)) * 16) + constants: one register per u.
+    constexpr int kPieceStep = 2;
+    constexpr int kPieces = 4;   // u = 0 .. 3: pieces 0 2 4 6 (+ h)
+    uint32_t foff[kPieces];
+#pragma unroll
+    for (int u = 0; u < kPieces; ++u) {
+        foff[u] = lrow * 128u + (((static_cast<uint32_t>(kPieceStep * u)) ^ (h ^ ((lrow >> 1) & 7u))) << 4);
+    }
+    auto frag = [&](const char* S, uint32_t line0, int u) __attribute__((always_inline)) {
+        return *reinterpret_cast<const i32x4*>(S + line0 * 128u + foff[u]);
     };
-    auto compute = [&](const char* As, const char* Bs, const Scales& sc) __attribute__((always_inline)) {
+    struct Frags {
+        v8i a[TI], b[TJ];
+    };
+    // the operands of sub-step s (64 k) of a stage
+    auto load_frags = [&](Frags& f, const char* As, const char* Bs, int s) __attribute__((always_inline)) {
 #pragma unroll
-        for (int s = 0; s < kSub; ++s) {
-            v8i av[TI], bv[TJ];
-#pragma unroll
-            for (int i = 0; i < TI; ++i) {
-                const uint32_t line0 = (wm * TI + i) * 32u;  // (lines 32 apart share the swizzle of lrow)
-                if constexpr (kFour) {
-                    const i32x4 lo = frag(As, line0, 2u * s + h);
-                    av[i] = v8i{lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
-                } else {
-                    const i32x4 lo = frag(As, line0, 4u * s + h), hi = frag(As, line0, 4u * s + 2u + h);
-                    av[i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                }
+        for (int i = 0; i < TI; ++i) {
+            const uint32_t line0 = (wm * TI + i) * 32u;  // (lines 32 apart share the swizzle of lrow)
+            if constexpr (kFour) {
+                const i32x4 lo = frag(As, line0, s);
+                f.a[i] = __builtin_shufflevector(lo, lo, 0, 1, 2, 3, -1, -1, -1, -1);  // the instruction reads 4 registers of a 4-bit operand
+            } else {
+                const i32x4 lo = frag(As, line0, 2 * s), hi = frag(As, line0, 2 * s + 1);
+                f.a[i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             }
+        }
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) {
+            const uint32_t line0 = (wn * TJ + j) * 32u;
+            if constexpr (kFour) {
+                const i32x4 lo = frag(Bs, line0, s);
+                f.b[j] = __builtin_shufflevector(lo, lo, 0, 1, 2, 3, -1, -1, -1, -1);
+            } else {
+                const i32x4 lo = frag(Bs, line0, 2 * s), hi = frag(Bs, line0, 2 * s + 1);
+                f.b[j] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            }
+        }
+    };
+    // the 8 matrix instructions of sub-step s: scale byte 2 s (+ the lane's half, shifted in) of the step's bytes
+    auto mfmas = [&](const Frags& f, const Scales& sc, auto sub) __attribute__((always_inline)) {
+        constexpr int s = decltype(sub)::value;
+#pragma unroll
+        for (int i = 0; i < TI; ++i) {
 #pragma unroll
             for (int j = 0; j < TJ; ++j) {
-                const uint32_t line0 = (wn * TJ + j) * 32u;
-                if constexpr (kFour) {
-                    const i32x4 lo = frag(Bs, line0, 2u * s + h);
-                    bv[j] = v8i{lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
-                } else {
-                    const i32x4 lo = frag(Bs, line0, 4u * s + h), hi = frag(Bs, line0, 4u * s + 2u + h);
-                    bv[j] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                }
-            }
-#pragma unroll
-            for (int i = 0; i < TI; ++i) {
-#pragma unroll
-                for (int j = 0; j < TJ; ++j) {
-                    // sub-step s uses scale byte 2 s (+ the lane's half, shifted in) of the step's bytes
-                    if (s & 1) {
-                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                            av[i], bv[j], acc[i][j], kCa, kCb, 2, static_cast<int>(sc.a[i][s >> 1]), 2,
-                            static_cast<int>(sc.b[j][s >> 1]));
-                    } else {
-                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                            av[i], bv[j], acc[i][j], kCa, kCb, 0, static_cast<int>(sc.a[i][s >> 1]), 0,
-                            static_cast<int>(sc.b[j][s >> 1]));
-                    }
-                }
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                    f.a[i], f.b[j], acc[i][j], kCa, kCb, (s & 1) ? 2 : 0, static_cast<int>(sc.a[i][s >> 1]),
+                    (s & 1) ? 2 : 0, static_cast<int>(sc.b[j][s >> 1]));
             }
         }
     };
 
     // ---- main loop: the loads of step s + 1 (tiles by DMA, scales into registers) run under the arithmetic of step
     // s; one wait and one barrier per step (the next stage has landed, and everyone has left the stage that the step
-    // after next will overwrite)
+    // after next will overwrite).  (A variant of the 4-bit loop with two operand sets, the reads of a sub-step under
+    // the instructions of the one before and the barrier moved in front of the last sub-step, measured slower: 579
+    // against 477 us at m = n = k = 8192.)
     const uint32_t steps = RB / kMxBK;
     Scales s0, s1;
+    Frags f;
+    auto compute = [&](const char* As, const char* Bs, const Scales& sc) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < kPieces; ++u) asm volatile("" : "+v"(foff[u]));
+        mx_static_for<kSub>([&](auto sub) {
+            load_frags(f, As, Bs, decltype(sub)::value);
+            mfmas(f, sc, sub);
+        });
+    };
     issue(0, A0, B0);
     load_scales(s0, 0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");

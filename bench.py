@@ -42,6 +42,8 @@ with open(os.path.join(ROOT, "peaks.json")) as _f:
 PEAK_INT8_TOPS = float(_PEAKS["int8_dense_tops"])
 PEAK_HBM_GBS = float(_PEAKS["hbm_gbs"])
 PEAK_F16_TFLOPS = float(_PEAKS["f16_dense_tflops"])
+PEAK_FP8_TFLOPS = float(_PEAKS["fp8_dense_tflops"])
+PEAK_FP4_TFLOPS = float(_PEAKS["fp4_dense_tflops"])
 # Bytes that left / entered the L2 caches per launch, from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs of
 # `bench.py --quick --no-cpu --copy-probe`; each counter is scaled by its reading for the 1 GiB copy of the same run
 # (FETCH_SIZE reads 0.5 per KiB there, WRITE_SIZE 1.0 per KiB).  Measured offline and recorded here; a run of this
@@ -63,7 +65,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="run a single workload: w8a8 | w4a16 | w4a16_nd | w4a16_m4 | w4a16_m16 | w4a16_nd_m4 | w4a16_nd_m16 | "
                          "w8a8_m1 | w8a8_m8 | w8a8_m16 | w8a8_m128 | w8a8_m512 | w8a8_nk_m1 | w8a8_nk_m16 | w8a8_nk_m128 | w8a16_m1 | w8a16_m16 | w8a16_nk_m1 | "
-                         "w8a16_nk_m16 | w8a16_m2048 | w8a16_nk_m2048 | quant | dequant | antiquant | group | group_example (a W4A16 name without _nd "
+                         "w8a16_nk_m16 | w8a16_m2048 | w8a16_nk_m2048 | quant | dequant | antiquant | group | group_example | mx_fp4 | mx_fp4_e1m2 | mx_fp8 (a W4A16 name without _nd "
                          "is the packed-weight path; _nk: weights kept as [n, k])")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch one device-to-device copy of 1 GiB: the known-size kernel that calibrates the "
@@ -335,6 +337,33 @@ def main():
                 "ops": flops, "bytes": bytes_, "reference_published_us_ascend_950pr": 204.129,
                 "reference_published_mac_ratio": 0.887}
 
+    def mx(fmt, steps, warmup):
+        """The shape of the reference's high-performance MxFP4 example (m = n = k = 8192, bfloat16 output, scale bytes
+        127..129 as its gen_data.py draws them; its README reports 681.056 us on an Ascend 950PR for fp4 e1m2 operands,
+        context only).  fmt: "fp4" = e2m1 x e2m1 straight on the scaled matrix instruction, "fp4_e1m2" = the example's
+        own format (widened to e4m3 first, inside the timed call), "fp8" = e4m3 x e4m3."""
+        M = N = K = 8192
+        f = {"fp4": abi.QDST_FP4_E2M1, "fp4_e1m2": abi.QDST_FP4_E1M2, "fp8": abi.QDST_FP8_E4M3FN}[fmt]
+        rb = K if fmt == "fp8" else K // 2
+        a = torch.randint(0, 256, (M, rb), dtype=torch.uint8, device=dev, generator=gen)
+        b = torch.randint(0, 256, (N, rb), dtype=torch.uint8, device=dev, generator=gen)
+        if fmt == "fp8":    # no NaN codes
+            a[(a & 0x7F) == 0x7F] = 0
+            b[(b & 0x7F) == 0x7F] = 0
+        sa = torch.randint(127, 130, (M, K // 32), dtype=torch.uint8, device=dev, generator=gen)
+        sb = torch.randint(127, 130, (N, K // 32), dtype=torch.uint8, device=dev, generator=gen)
+        c = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+
+        def step(i, starts, stops):
+            bracket(starts, stops, lambda: ops.matmul_mx(c, a, b, sa, sb, f, f, K))
+
+        ms, kern_ms = timed(step, steps, warmup)
+        flops = 2.0 * M * N * K
+        peak = PEAK_FP8_TFLOPS if fmt != "fp4" else PEAK_FP4_TFLOPS
+        return {"kernel_ms": kern_ms, "tflops": flops / (kern_ms * 1e-3) / 1e12,
+                "mfma_frac": flops / (kern_ms * 1e-3) / 1e12 / peak, "peak_tflops": peak,
+                "reference_published_us_ascend_950pr_fp4_e1m2": 681.056}
+
     def strip(d):
         return {k: v for k, v in d.items() if k != "tensors"}
 
@@ -356,6 +385,9 @@ def main():
         fn = {"w4a16": lambda: w4a16(1, args.steps, args.warmup, packed=True),
               "w4a16_nd": lambda: w4a16(1, args.steps, args.warmup),
               "group_example": lambda: group_example(args.steps, args.warmup),
+              "mx_fp4": lambda: mx("fp4", max(10, args.steps // 10), 3),
+              "mx_fp4_e1m2": lambda: mx("fp4_e1m2", max(10, args.steps // 10), 3),
+              "mx_fp8": lambda: mx("fp8", max(10, args.steps // 10), 3),
               "w4a16_m4": lambda: w4a16(4, args.steps, args.warmup, packed=True),
               "w4a16_m16": lambda: w4a16(16, args.steps, args.warmup, packed=True),
               "w4a16_nd_m4": lambda: w4a16(4, args.steps, args.warmup),
