@@ -539,6 +539,9 @@ def main():
         r["mfma_frac"] = r["tops"] / PEAK_INT8_TOPS
         others["group_matmul_reference_example"] = r
         torch.cuda.empty_cache()
+        for fmt in ("fp4", "fp8", "fp4_e1m2"):
+            others[f"mx_{fmt}_8192"] = mx(fmt, 10, 3)
+            torch.cuda.empty_cache()
         out["others"] = others
 
     # ------------------------------------------------------------------ CPU baseline (the oracle; a checker being timed)

@@ -37,6 +37,7 @@ def test_struct_sizes_match_the_header():
     assert C.sizeof(abi.W4A16Desc) == 5 * 4
     assert C.sizeof(abi.W8A16Desc) == 9 * 4
     assert C.sizeof(abi.AntiQuantPolicyDesc) == 14 * 4
+    assert C.sizeof(abi.MxDesc) == 8 * 4
 
 
 def q(**kw):
@@ -431,3 +432,22 @@ def test_swiglu_rejections_and_workspace():
     assert L.ascq_matmul_w8a8_workspace_size(C.byref(mk()), C.byref(need)) == abi.OK
     assert need.value >= 16 * 64 * 4                                  # the int32 accumulators of the pairwise epilogue
     assert call(mk()) == abi.EINVAL and "workspace" in err()          # small m: not the large tile kernel
+
+
+def test_mx_matmul_surface_without_a_gpu():
+    """Descriptor checks and the workspace rule of the block-scaled matmul answer on the host."""
+    lib = abi.load_library()
+    need = C.c_size_t(7)
+    e4, e5, f2, f1 = abi.QDST_FP8_E4M3FN, abi.QDST_FP8_E5M2, abi.QDST_FP4_E2M1, abi.QDST_FP4_E1M2
+    mk = lambda **kw: abi.MxDesc(**{**dict(m=512, n=512, k=1024, scale_k=32, a_format=e4, b_format=e5,
+                                           out_dtype=abi.BF16, has_bias=0), **kw})
+    for d, want in [(mk(), 0), (mk(a_format=f2, b_format=f2), 0),                      # straight from the given buffers
+                    (mk(a_format=f1, b_format=f1), 2 * 512 * 1024),                    # e1m2: both widened to e4m3
+                    (mk(a_format=f2), 512 * 1024),                                     # 4-bit beside 8-bit: a widened
+                    (mk(a_format=f1, k=70, scale_k=4), 0)]:                            # one lane per output: no scratch
+        assert lib.ascq_matmul_mx_workspace_size(C.byref(d), C.byref(need)) == abi.OK and need.value == want
+    for d, msg in [(mk(k=63, a_format=f2), "even"), (mk(scale_k=31), "scale_k"), (mk(a_format=abi.QDST_I8), "a_format"),
+                   (mk(out_dtype=abi.I8), "out_dtype"), (mk(m=0), "greater than 0")]:
+        assert lib.ascq_matmul_mx_workspace_size(C.byref(d), C.byref(need)) == abi.EINVAL
+        assert msg in lib.ascq_last_error().decode()
+    assert lib.ascq_matmul_mx(C.byref(mk()), None, None, None, None, None, None, None, 0, None) == abi.ENULL
