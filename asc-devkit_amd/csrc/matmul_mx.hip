@@ -239,36 +239,48 @@ __global__ __launch_bounds__(kMxThreads, 1) void mx_tile_kernel(MxParams p)
     const uint32_t steps = RB / kMxBK;
     Scales s0, s1;
     Frags f;
+    // A K step: all sub-steps but the last, then the last one's operands into registers, then the wait and the barrier
+    // (the next stage has landed; everyone has left this stage, which the step after next overwrites), and only then
+    // the last sub-step's instructions: behind the barrier the matrix pipe has work at once.
     auto compute = [&](const char* As, const char* Bs, const Scales& sc) __attribute__((always_inline)) {
 #pragma unroll
         for (int u = 0; u < kPieces; ++u) asm volatile("" : "+v"(foff[u]));
-        mx_static_for<kSub>([&](auto sub) {
+        mx_static_for<kSub - 1>([&](auto sub) {
             load_frags(f, As, Bs, decltype(sub)::value);
             mfmas(f, sc, sub);
         });
+        load_frags(f, As, Bs, kSub - 1);
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __syncthreads();
+    };
+    auto finish = [&](const Scales& sc) __attribute__((always_inline)) {
+        mfmas(f, sc, std::integral_constant<int, kSub - 1>{});
     };
     issue(0, A0, B0);
     load_scales(s0, 0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+    if (steps > 1u) {
+        issue(kMxBK, A1, B1);
+        load_scales(s1, 1u);
+    }
+    // Nothing between the instructions of a step is conditional (a branch there makes the compiler shuffle the
+    // accumulators): past the end the loads repeat the last step's, into a stage and registers nobody reads again.
+    const uint32_t last = steps - 1u;
     for (uint32_t s = 0; s < steps; s += 2) {
+        const uint32_t s2 = s + 2u < last ? s + 2u : last, s3 = s + 3u < last ? s + 3u : last;
+        compute(A0, B0, s0);                 // ends behind the barrier: stage 0 is free, stage 1 has landed
+        issue(s2 * kMxBK, A0, B0);
+        finish(s0);
+        load_scales(s0, s2);
         if (s + 1u < steps) {
-            issue((s + 1u) * kMxBK, A1, B1);
-            load_scales(s1, s + 1u);
-        }
-        compute(A0, B0, s0);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        if (s + 1u < steps) {
-            if (s + 2u < steps) {
-                issue((s + 2u) * kMxBK, A0, B0);
-                load_scales(s0, s + 2u);
-            }
             compute(A1, B1, s1);
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            __syncthreads();
+            issue(s3 * kMxBK, A1, B1);
+            finish(s1);
+            load_scales(s1, s3);
         }
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the repeated loads of the last steps
 
     // ---- register r of lane l in a 32 x 32 block: row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32
 #pragma unroll
