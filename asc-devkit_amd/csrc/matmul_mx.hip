@@ -283,17 +283,49 @@ __global__ __launch_bounds__(kMxThreads, 1) void mx_tile_kernel(MxParams p)
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the repeated loads of the last steps
 
     // ---- register r of lane l in a 32 x 32 block: row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32
+    float bias[TJ];
 #pragma unroll
     for (int j = 0; j < TJ; ++j) {
         const uint32_t col = n0 + (wn * TJ + j) * 32u + lrow;
-        const float bias = (p.bias != nullptr && col < p.n) ? p.bias[col] : 0.0f;
+        bias[j] = (p.bias != nullptr && col < p.n) ? p.bias[col] : 0.0f;
+    }
+    if (p.out_dtype != ASCQ_F32 && p.n % 2u == 0) {
+        // 16-bit outputs: after one swap between neighbouring lanes the even lane holds columns (l, l + 1) of the
+        // wavefront's first block of 32 and the odd lane columns (l - 1, l) of the second: one dword store per lane,
+        // and the 32 lanes of a row write one full 128-byte line
+        const bool odd = (lane & 1u) != 0;
+        const bool bf = p.out_dtype == ASCQ_BF16;
+        const uint32_t colw = n0 + wn * (TJ * 32u);
+        const uint32_t col = odd ? colw + 32u + (lrow - 1u) : colw + lrow;  // first column of the lane's pair
+#pragma unroll
+        for (int i = 0; i < TI; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint32_t row = row0 + (wm * TI + i) * 32u + 8u * (r >> 2) + 4u * h + (r & 3);
+                const float v0 = acc[i][0][r] + bias[0], v1 = acc[i][1][r] + bias[1];
+                const uint32_t h0 = bf ? f32_to_bf16_bits(v0) : f32_to_half_bits_sat(v0);
+                const uint32_t h1 = bf ? f32_to_bf16_bits(v1) : f32_to_half_bits_sat(v1);
+                const uint32_t recv = static_cast<uint32_t>(
+                    __builtin_amdgcn_mov_dpp(static_cast<int>(odd ? h0 : h1), 0xB1, 0xF, 0xF, true));  // lane ^ 1
+                const uint32_t word = odd ? (recv | (h1 << 16)) : (h0 | (recv << 16));
+                if (row < p.m && col < p.n) {
+                    __builtin_nontemporal_store(word, reinterpret_cast<uint32_t*>(static_cast<uint16_t*>(p.c) +
+                                                                                  static_cast<size_t>(row) * p.n + col));
+                }
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int j = 0; j < TJ; ++j) {
+        const uint32_t col = n0 + (wn * TJ + j) * 32u + lrow;
 #pragma unroll
         for (int i = 0; i < TI; ++i) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const uint32_t row = row0 + (wm * TI + i) * 32u + 8u * (r >> 2) + 4u * h + (r & 3);
                 if (row < p.m && col < p.n) {
-                    mx_store(p, static_cast<size_t>(row) * p.n + col, acc[i][j][r] + bias);
+                    mx_store(p, static_cast<size_t>(row) * p.n + col, acc[i][j][r] + bias[j]);
                 }
             }
         }
