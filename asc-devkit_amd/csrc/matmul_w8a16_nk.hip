@@ -329,6 +329,30 @@ __global__ __launch_bounds__(256, 2) void w8a16_nk_gemm_kernel(NkParams p, uint3
     }
 
     // ---- register r of lane l in a 32 x 32 block: row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32
+    if (!p.out_f32 && p.n % 2u == 0) {
+        // half output: after one swap between neighbouring lanes the even lane holds columns (l, l + 1) of the
+        // wavefront's first block of 32 and the odd lane columns (l - 1, l) of the second: one dword store per lane,
+        // and the 32 lanes of a row write one full 128-byte line
+        const bool odd = (lane & 1u) != 0;
+        const uint32_t colw = col0 + wn * 64u;
+        const uint32_t col = odd ? colw + 32u + (lrow - 1u) : colw + lrow;  // first column of the lane's pair
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint32_t row = row0 + wm * 64u + i * 32u + 8u * (r >> 2) + 4u * lk + (r & 3);
+                const uint32_t h0 = f32_to_half_bits(acc[i][0][r]), h1 = f32_to_half_bits(acc[i][1][r]);
+                const uint32_t recv = static_cast<uint32_t>(
+                    __builtin_amdgcn_mov_dpp(static_cast<int>(odd ? h0 : h1), 0xB1, 0xF, 0xF, true));  // lane ^ 1
+                const uint32_t word = odd ? (recv | (h1 << 16)) : (h0 | (recv << 16));
+                if (row < p.m && col < p.n) {
+                    __builtin_nontemporal_store(word, reinterpret_cast<uint32_t*>(static_cast<uint16_t*>(p.y) +
+                                                                                  static_cast<size_t>(row) * p.n + col));
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
 #pragma unroll
