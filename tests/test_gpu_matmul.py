@@ -58,7 +58,9 @@ SHAPES = [(1, 256, 512), (16, 1024, 4096), (32, 264, 1040), (33, 256, 256), (128
           # four and five K steps: the steady-state loop runs once, then two steps / one step are peeled
           (600, 528, 512), (600, 528, 640), (300, 272, 512), (300, 272, 640),
           # 344 tiles of 256 x 256: wide and narrow tiles in one launch, for B as [k, n] and as [n, k]
-          (2048, 11008, 128)]
+          (2048, 11008, 128),
+          # more than 8 row tiles: bands of 8 row tiles and a last band of 2 (with a partial last row tile)
+          (2500, 784, 128)]
 
 
 @pytest.mark.parametrize("m,n,k", SHAPES)
