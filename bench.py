@@ -64,7 +64,7 @@ def main():
     ap.add_argument("--quick", action="store_true", help="headline + W4A16 GEMV only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="run a single workload: w8a8 | w4a16 | w4a16_nd | w4a16_m4 | w4a16_m16 | w4a16_nd_m4 | w4a16_nd_m16 | "
-                         "w8a8_m1 | w8a8_m8 | w8a8_m16 | w8a8_m128 | w8a8_m512 | w8a8_nk_m1 | w8a8_nk_m16 | w8a8_nk_m128 | w8a16_m1 | w8a16_m16 | w8a16_nk_m1 | "
+                         "w8a8_m1 | w8a8_m8 | w8a8_m16 | w8a8_m128 | w8a8_m512 | w8a8_m8192 | w8a8_nk_m1 | w8a8_nk_m16 | w8a8_nk_m128 | w8a16_m1 | w8a16_m16 | w8a16_nk_m1 | "
                          "w8a16_nk_m16 | w8a16_m2048 | w8a16_nk_m2048 | quant | dequant | antiquant | group | group_example | mx_fp4 | mx_fp4_e1m2 | mx_fp8 (a W4A16 name without _nd "
                          "is the packed-weight path; _nk: weights kept as [n, k])")
     ap.add_argument("--copy-probe", action="store_true",
@@ -396,6 +396,7 @@ def main():
               "w8a8_m8": lambda: w8a8(8, args.steps, args.warmup, sets=7),
               "w8a8_m16": lambda: w8a8(16, args.steps, args.warmup, sets=7),
               "w8a8_m512": lambda: w8a8(512, args.steps, args.warmup, sets=7),
+              "w8a8_m8192": lambda: w8a8(8192, max(20, args.steps // 10), 5, settle=40),
               "w8a8_nk_m128": lambda: w8a8(128, args.steps, args.warmup, sets=7, b_nk=True),
               "w8a8_m128": lambda: w8a8(128, args.steps, args.warmup, sets=7),
               "w8a8_nk_m1": lambda: w8a8(1, args.steps, args.warmup, sets=7, b_nk=True),
@@ -498,6 +499,11 @@ def main():
             others[f"w8a8_m{M}"] = {"gemm_kernel_ms": r["gemm_kernel_ms"], "gemm_tops": r["gemm_tops"],
                                     "gemm_gbs": r["gemm_gbs"], "hbm_frac": r["gemm_gbs"] / PEAK_HBM_GBS,
                                     "mfma_frac": r["gemm_tops"] / PEAK_INT8_TOPS}
+        r = strip(w8a8(8192, 40, 5, settle=40))
+        others["w8a8_m8192"] = {"gemm_kernel_ms": r["gemm_kernel_ms"], "gemm_tops": r["gemm_tops"],
+                                "mfma_frac": r["gemm_tops"] / PEAK_INT8_TOPS,
+                                "note": "the same linear with 8192 rows: 1376 tiles, 5.4 rounds of the chip"}
+        torch.cuda.empty_cache()
         for M in (1, 16, 128):
             r = strip(w8a8(M, s2, w2, sets=7, b_nk=True))
             others[f"w8a8_nk_m{M}"] = {"gemm_kernel_ms": r["gemm_kernel_ms"], "gemm_gbs": r["gemm_gbs"],
