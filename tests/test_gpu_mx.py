@@ -86,12 +86,14 @@ def test_mx_tile_kernel(m, n, k, fa, fb):
     mx_check(run_mx(m, n, k, a, b, sa, sb, fa, fb).cpu().numpy(), want, mx_abs_dot(a, b, sa, sb, k, fa, fb), is8(fa, fb))
 
 
+@pytest.mark.parametrize("n", [320, 257])
 @pytest.mark.parametrize("out", [torch.bfloat16, torch.float16])
-def test_mx_sixteen_bit_outputs_and_bias(out):
-    """e2m1 operands (exact products, fp32 sums): a 16-bit result is the golden's or its neighbour."""
-    announce("mx 16-bit out", out)
+def test_mx_sixteen_bit_outputs_and_bias(out, n):
+    """e2m1 operands (exact products, fp32 sums): a 16-bit result is the golden's or its neighbour.  An even n leaves
+    the tile kernel as one dword per lane, an odd n element by element."""
+    announce("mx 16-bit out", out, n)
     rng = np.random.default_rng(5)
-    m, n, k = 256, 320, 512
+    m, k = 256, 512
     a, b, sa, sb, bv = mx_case(rng, m, n, k, F2, F2, bias=True, lo=124, hi=130)
     dt = abi.BF16 if out == torch.bfloat16 else abi.F16
     d = abi.MxDesc(m=m, n=n, k=k, scale_k=sa.shape[1], a_format=F2, b_format=F2, out_dtype=dt, has_bias=1)
