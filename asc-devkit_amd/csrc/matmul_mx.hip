@@ -267,17 +267,64 @@ __global__ __launch_bounds__(kMxThreads, 1) void mx_tile_kernel(MxParams p)
     // Nothing between the instructions of a step is conditional (a branch there makes the compiler shuffle the
     // accumulators): past the end the loads repeat the last step's, into a stage and registers nobody reads again.
     const uint32_t last = steps - 1u;
-    for (uint32_t s = 0; s < steps; s += 2) {
-        const uint32_t s2 = s + 2u < last ? s + 2u : last, s3 = s + 3u < last ? s + 3u : last;
-        compute(A0, B0, s0);                 // ends behind the barrier: stage 0 is free, stage 1 has landed
-        issue(s2 * kMxBK, A0, B0);
-        finish(s0);
-        load_scales(s0, s2);
-        if (s + 1u < steps) {
-            compute(A1, B1, s1);
-            issue(s3 * kMxBK, A1, B1);
-            finish(s1);
-            load_scales(s1, s3);
+    if constexpr (kFour) {
+        // 4-bit operands are 24 registers a set: two sets.  The LDS reads of a sub-step are spread behind the first
+        // matrix instructions of the sub-step before (scheduling groups: one instruction, two reads, ...), so that the
+        // LDS works while the matrix pipe does; the first operands of the next step, whose stage has landed, are read
+        // behind the barrier under this step's last instructions.
+        Frags g;
+        auto interleave = [&]() __attribute__((always_inline)) {
+            constexpr int kReads = TI + TJ, kMfmas = TI * TJ, kPer = 2;
+            mx_static_for<kMfmas>([&](auto n) {
+                constexpr int kLeft = kReads - decltype(n)::value * kPer;
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                if constexpr (kLeft > 0) {
+                    __builtin_amdgcn_sched_group_barrier(0x100, kLeft < kPer ? kLeft : kPer, 0);
+                }
+            });
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        load_frags(f, A0, B0, 0);
+        auto step2 = [&](char* Ax, char* Bx, const char* Ay, const char* By, Scales& sc, uint32_t next) __attribute__((always_inline)) {
+#pragma unroll
+            for (int u = 0; u < kPieces; ++u) asm volatile("" : "+v"(foff[u]));
+            load_frags(g, Ax, Bx, 1);
+            mfmas(f, sc, std::integral_constant<int, 0>{});
+            interleave();
+            load_frags(f, Ax, Bx, 2);
+            mfmas(g, sc, std::integral_constant<int, 1>{});
+            interleave();
+            load_frags(g, Ax, Bx, 3);
+            mfmas(f, sc, std::integral_constant<int, 2>{});
+            interleave();
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+            __syncthreads();
+            issue(next * kMxBK, Ax, Bx);
+            load_frags(f, Ay, By, 0);
+            mfmas(g, sc, std::integral_constant<int, 3>{});
+            interleave();
+            load_scales(sc, next);
+        };
+        for (uint32_t s = 0; s < steps; s += 2) {
+            const uint32_t s2 = s + 2u < last ? s + 2u : last, s3 = s + 3u < last ? s + 3u : last;
+            step2(A0, B0, A1, B1, s0, s2);
+            if (s + 1u < steps) {
+                step2(A1, B1, A0, B0, s1, s3);
+            }
+        }
+    } else {
+        for (uint32_t s = 0; s < steps; s += 2) {
+            const uint32_t s2 = s + 2u < last ? s + 2u : last, s3 = s + 3u < last ? s + 3u : last;
+            compute(A0, B0, s0);                 // ends behind the barrier: stage 0 is free, stage 1 has landed
+            issue(s2 * kMxBK, A0, B0);
+            finish(s0);
+            load_scales(s0, s2);
+            if (s + 1u < steps) {
+                compute(A1, B1, s1);
+                issue(s3 * kMxBK, A1, B1);
+                finish(s1);
+                load_scales(s1, s3);
+            }
         }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the repeated loads of the last steps
