@@ -385,9 +385,9 @@ def main():
         fn = {"w4a16": lambda: w4a16(1, args.steps, args.warmup, packed=True),
               "w4a16_nd": lambda: w4a16(1, args.steps, args.warmup),
               "group_example": lambda: group_example(args.steps, args.warmup),
-              "mx_fp4": lambda: mx("fp4", max(10, args.steps // 10), 3),
-              "mx_fp4_e1m2": lambda: mx("fp4_e1m2", max(10, args.steps // 10), 3),
-              "mx_fp8": lambda: mx("fp8", max(10, args.steps // 10), 3),
+              "mx_fp4": lambda: mx("fp4", args.steps, args.warmup),
+              "mx_fp4_e1m2": lambda: mx("fp4_e1m2", args.steps, args.warmup),
+              "mx_fp8": lambda: mx("fp8", args.steps, args.warmup),
               "w4a16_m4": lambda: w4a16(4, args.steps, args.warmup, packed=True),
               "w4a16_m16": lambda: w4a16(16, args.steps, args.warmup, packed=True),
               "w4a16_nd_m4": lambda: w4a16(4, args.steps, args.warmup),
