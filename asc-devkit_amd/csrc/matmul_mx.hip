@@ -43,6 +43,7 @@ __device__ __forceinline__ void mx_static_for(F&& f)
 
 constexpr uint32_t kMxBM = 256, kMxBN = 256, kMxBK = 128;  // BK in bytes of an operand row
 constexpr int kMxThreads = 512;
+constexpr uint32_t kMxScaleBuf = (kMxBM + kMxBN) * 16u;  // 16 scale bytes of every row of a tile's a and b
 
 struct MxParams {
     const uint8_t* a;
@@ -78,6 +79,7 @@ __global__ __launch_bounds__(kMxThreads, 1) void mx_tile_kernel(MxParams p)
     __shared__ __attribute__((aligned(1024))) char B0[kMxBN * kMxBK];
     __shared__ __attribute__((aligned(1024))) char A1[kMxBM * kMxBK];
     __shared__ __attribute__((aligned(1024))) char B1[kMxBN * kMxBK];
+    __shared__ __attribute__((aligned(1024))) char SC[2 * kMxScaleBuf];  // two buffers of scale bytes, see below
     constexpr int TI = 4, TJ = 2;
     constexpr int kSub = kFour ? 4 : 2;       // instructions (64 k each) per K step and block pair
     constexpr int kScaleDw = kFour ? 2 : 1;   // dwords of scale bytes per row and K step
@@ -124,46 +126,94 @@ __global__ __launch_bounds__(kMxThreads, 1) void mx_tile_kernel(MxParams p)
     }
     const uint8_t* Abase = p.a + static_cast<size_t>(row0) * RB;
     const uint8_t* Bbase = p.b + static_cast<size_t>(n0) * RB;
+    // A wavefront-uniform address, pinned to scalar registers: a load's address is then this base plus the lane's
+    // 32-bit offset, which the load instruction adds itself (otherwise the compiler folds the lane's offset into
+    // 64-bit per-lane addresses, twice the registers and an addition per load, in temporaries whose reuse by the
+    // next LDS reads makes it wait for the loads).
+    auto uniform = [](const uint8_t* q) __attribute__((always_inline)) {
+        const uint64_t v = reinterpret_cast<uint64_t>(q);
+        uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+        uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
+        asm volatile("" : "+s"(lo), "+s"(hi));  // opaque: keeps the compiler from re-associating base and lane offset
+        return reinterpret_cast<const uint8_t*>((static_cast<uint64_t>(hi) << 32) | lo);
+    };
     auto issue = [&](uint32_t k0, char* As, char* Bs) __attribute__((always_inline)) {
+        const uint8_t* ab = uniform(Abase + k0);
+        const uint8_t* bb = uniform(Bbase + k0);
+        // (re-materialised here: widened to 64 bits once, ahead of the loop, the offsets would no longer be seen as
+        // 32-bit offsets where the loads are selected)
+#pragma unroll
+        for (int u = 0; u < 4; ++u) asm volatile("" : "+v"(aoff[u]), "+v"(boff[u]));
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            __builtin_amdgcn_global_load_lds((gptr_t)(Abase + k0 + aoff[u]), (lds_ptr_t)(As + (wave * 4u + u) * 1024u), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(ab + aoff[u]), (lds_ptr_t)(As + (wave * 4u + u) * 1024u), 16, 0, 0);
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            __builtin_amdgcn_global_load_lds((gptr_t)(Bbase + k0 + boff[u]), (lds_ptr_t)(Bs + (wave * 4u + u) * 1024u), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(bb + boff[u]), (lds_ptr_t)(Bs + (wave * 4u + u) * 1024u), 16, 0, 0);
         }
     };
 
-    // ---- scale bytes of a K step: one or two dwords per operand row, already shifted for this lane's half
-    const uint32_t lrow = lane & 31u, h = lane >> 5;
-    uint32_t sa_row[TI], sb_row[TJ];  // byte offsets of the lane's scale rows (m * sk and n * sk stay below 2^32)
-#pragma unroll
-    for (int i = 0; i < TI; ++i) {
-        uint32_t row = row0 + (wm * TI + i) * 32u + lrow;
-        row = row < p.m ? row : p.m - 1u;
-        sa_row[i] = row * p.sk;
+    // ---- scale bytes.  They come through LDS: a wavefront reading its rows' bytes from memory fetched 32 lines per
+    // load for 8 bytes of each, three times the lines of the tile loads themselves, and the kernel took half as
+    // long again for it.  Here every second K step one 16-byte load per row (wavefronts 0-3: the 256 rows of a,
+    // 4-7: those of b) brings the bytes of the two steps of a "slot" (4-bit form: exactly those 16 bytes; 8-bit form:
+    // 8 of them) into buffer slot % 2, as a direct-to-LDS load beside the tile loads; at the row's end the 16 bytes
+    // are moved back to stay inside the row.  A lane then reads its rows' bytes of a step with one LDS read per row.
+    // The registers hold the bytes as loaded; the shift for the lane's half is applied where they are used.
+    const uint32_t lrow = lane & 31u, h = lane >> 5, hshift = 8u * h;
+    constexpr uint32_t kBs = 4u * kScaleDw;  // scale bytes per row and K step
+    const uint32_t steps = RB / kMxBK, last = steps - 1u, last_slot = last >> 1;
+    const bool sc_is_a = wave < 4u;
+    const uint8_t* sc_base = sc_is_a ? p.sa : p.sb;
+    uint32_t sc_lane;  // the lane's row of scale bytes (m * sk and n * sk stay below 2^32)
+    {
+        uint32_t r = (sc_is_a ? row0 : n0) + (wave & 3u) * 64u + lane;
+        const uint32_t lim = sc_is_a ? p.m : p.n;
+        r = r < lim ? r : lim - 1u;
+        sc_lane = r * p.sk;
     }
-#pragma unroll
-    for (int j = 0; j < TJ; ++j) {
-        uint32_t col = n0 + (wn * TJ + j) * 32u + lrow;
-        col = col < p.n ? col : p.n - 1u;
-        sb_row[j] = col * p.sk;
-    }
+    auto slot_off = [&](uint32_t slot) {  // first of the 16 bytes loaded for a slot
+        const uint32_t o = 2u * kBs * slot, cap = p.sk - 16u;
+        return o < cap ? o : cap;
+    };
+    // slot: counted on past the end (it picks the buffer); the bytes are those of the last slot then
+    auto issue_scales = [&](uint32_t slot) __attribute__((always_inline)) {
+        const uint32_t data = slot < last_slot ? slot : last_slot;
+        asm volatile("" : "+v"(sc_lane));
+        __builtin_amdgcn_global_load_lds((gptr_t)(uniform(sc_base + slot_off(data)) + sc_lane),
+                                         (lds_ptr_t)(SC + (slot & 1u) * kMxScaleBuf + wave * 1024u), 16, 0, 0);
+    };
     struct Scales {
         uint32_t a[TI][kScaleDw], b[TJ][kScaleDw];
     };
-    // dword d of the scale bytes of a K step
-    auto load_scales_dw = [&](Scales& sc, uint32_t step, int d) __attribute__((always_inline)) {
-        const uint32_t o = step * (4u * kScaleDw) + 4u * d;
+    const uint32_t sc_va = (wm * (TI * 32u) + lrow) * 16u, sc_vb = kMxBM * 16u + (wn * (TJ * 32u) + lrow) * 16u;
+    // the bytes of K step `step` (counted on past the end like the slot) from LDS into registers
+    auto read_scales = [&](Scales& sc, uint32_t step) __attribute__((always_inline)) {
+        const uint32_t slot = step >> 1, data = slot < last_slot ? slot : last_slot, st = step < last ? step : last;
+        const uint32_t off = (slot & 1u) * kMxScaleBuf + kBs * st - slot_off(data);
+        const char* pa = SC + sc_va + off;
+        const char* pb = SC + sc_vb + off;
 #pragma unroll
-        for (int i = 0; i < TI; ++i) sc.a[i][d] = *reinterpret_cast<const uint32_t*>(p.sa + sa_row[i] + o) >> (8u * h);
+        for (int i = 0; i < TI; ++i) {
+            if constexpr (kScaleDw == 2) {
+                const u32x2 v = *reinterpret_cast<const u32x2*>(pa + i * 512);
+                sc.a[i][0] = v[0];
+                sc.a[i][1] = v[1];
+            } else {
+                sc.a[i][0] = *reinterpret_cast<const uint32_t*>(pa + i * 512);
+            }
+        }
 #pragma unroll
-        for (int j = 0; j < TJ; ++j) sc.b[j][d] = *reinterpret_cast<const uint32_t*>(p.sb + sb_row[j] + o) >> (8u * h);
-    };
-    auto load_scales = [&](Scales& sc, uint32_t step) __attribute__((always_inline)) {
-#pragma unroll
-        for (int d = 0; d < kScaleDw; ++d) load_scales_dw(sc, step, d);
+        for (int j = 0; j < TJ; ++j) {
+            if constexpr (kScaleDw == 2) {
+                const u32x2 v = *reinterpret_cast<const u32x2*>(pb + j * 512);
+                sc.b[j][0] = v[0];
+                sc.b[j][1] = v[1];
+            } else {
+                sc.b[j][0] = *reinterpret_cast<const uint32_t*>(pb + j * 512);
+            }
+        }
     };
 
     f32x16 acc[TI][TJ];
@@ -225,48 +275,28 @@ __global__ __launch_bounds__(kMxThreads, 1) void mx_tile_kernel(MxParams p)
 #pragma unroll
             for (int j = 0; j < TJ; ++j) {
                 acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                    f.a[i], f.b[j], acc[i][j], kCa, kCb, (s & 1) ? 2 : 0, static_cast<int>(sc.a[i][s >> 1]),
-                    (s & 1) ? 2 : 0, static_cast<int>(sc.b[j][s >> 1]));
+                    f.a[i], f.b[j], acc[i][j], kCa, kCb, (s & 1) ? 2 : 0, static_cast<int>(sc.a[i][s >> 1] >> hshift),
+                    (s & 1) ? 2 : 0, static_cast<int>(sc.b[j][s >> 1] >> hshift));
             }
         }
     };
 
-    // ---- main loop: the loads of step s + 1 (tiles by DMA, scales into registers) run under the arithmetic of step
-    // s; one wait and one barrier per step (the next stage has landed, and everyone has left the stage that the step
-    // after next will overwrite).  (A variant of the 4-bit loop with two operand sets, the reads of a sub-step under
-    // the instructions of the one before and the barrier moved in front of the last sub-step, measured slower: 579
-    // against 477 us at m = n = k = 8192.)
-    const uint32_t steps = RB / kMxBK;
+    // ---- main loop: the loads of step s + 1 (tiles and, every second step, scale bytes, all direct to LDS) run under
+    // the arithmetic of step s; one wait and one barrier per step (the next stage has landed, and everyone has left
+    // the stage that the step after next will overwrite).  Behind the barrier a wavefront first reads the next
+    // step's scale bytes from LDS, then issues the loads: a load into the scale buffers ahead of those reads would
+    // make the compiler wait for it, and with it for the tile loads, before the reads.
     Scales s0, s1;
     Frags f;
-    // A K step: all sub-steps but the last, then the last one's operands into registers, then the wait and the barrier
-    // (the next stage has landed; everyone has left this stage, which the step after next overwrites), and only then
-    // the last sub-step's instructions: behind the barrier the matrix pipe has work at once.
-    auto compute = [&](const char* As, const char* Bs, const Scales& sc) __attribute__((always_inline)) {
-#pragma unroll
-        for (int u = 0; u < kPieces; ++u) asm volatile("" : "+v"(foff[u]));
-        mx_static_for<kSub - 1>([&](auto sub) {
-            load_frags(f, As, Bs, decltype(sub)::value);
-            mfmas(f, sc, sub);
-        });
-        load_frags(f, As, Bs, kSub - 1);
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-        __syncthreads();
-    };
-    auto finish = [&](const Scales& sc) __attribute__((always_inline)) {
-        mfmas(f, sc, std::integral_constant<int, kSub - 1>{});
-    };
+    // Nothing between the instructions of a step is conditional (a branch there makes the compiler shuffle the
+    // accumulators): past the end the loads repeat the last step's, into a stage and buffers nobody reads again.
+    auto next_step = [&](uint32_t s) { return s + 2u < last ? s + 2u : last; };
     issue(0, A0, B0);
-    load_scales(s0, 0);
+    issue_scales(0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (steps > 1u) {
-        issue(kMxBK, A1, B1);
-        load_scales(s1, 1u);
-    }
-    // Nothing between the instructions of a step is conditional (a branch there makes the compiler shuffle the
-    // accumulators): past the end the loads repeat the last step's, into a stage and registers nobody reads again.
-    const uint32_t last = steps - 1u;
+    read_scales(s0, 0);
+    issue((steps > 1u ? 1u : 0u) * kMxBK, A1, B1);  // a single step is loaded twice: stage 1 is then never read
     if constexpr (kFour) {
         // 4-bit operands are 24 registers a set: two sets.  The LDS reads of a sub-step are spread behind the first
         // matrix instructions of the sub-step before (scheduling groups: one instruction, two reads, ...), so that the
@@ -285,7 +315,9 @@ __global__ __launch_bounds__(kMxThreads, 1) void mx_tile_kernel(MxParams p)
             __builtin_amdgcn_sched_barrier(0);
         };
         load_frags(f, A0, B0, 0);
-        auto step2 = [&](char* Ax, char* Bx, const char* Ay, const char* By, Scales& sc, uint32_t next) __attribute__((always_inline)) {
+        // step s in stage x; `even` steps also load the scale bytes of the slot after the next
+        auto step2 = [&](char* Ax, char* Bx, const char* Ay, const char* By, const Scales& sc, Scales& sc_next, uint32_t s,
+                         auto even) __attribute__((always_inline)) {
 #pragma unroll
             for (int u = 0; u < kPieces; ++u) asm volatile("" : "+v"(foff[u]));
             load_frags(g, Ax, Bx, 1);
@@ -299,32 +331,55 @@ __global__ __launch_bounds__(kMxThreads, 1) void mx_tile_kernel(MxParams p)
             interleave();
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
             __syncthreads();
-            issue(next * kMxBK, Ax, Bx);
+            read_scales(sc_next, s + 1u);
+            __builtin_amdgcn_sched_barrier(0);
+            issue(next_step(s) * kMxBK, Ax, Bx);
+            if constexpr (decltype(even)::value) {
+                issue_scales((s >> 1) + 1u);
+            }
             load_frags(f, Ay, By, 0);
             mfmas(g, sc, std::integral_constant<int, 3>{});
             interleave();
-            load_scales(sc, next);
         };
-        for (uint32_t s = 0; s < steps; s += 2) {
-            const uint32_t s2 = s + 2u < last ? s + 2u : last, s3 = s + 3u < last ? s + 3u : last;
-            step2(A0, B0, A1, B1, s0, s2);
-            if (s + 1u < steps) {
-                step2(A1, B1, A0, B0, s1, s3);
-            }
+        // Steps in pairs, an odd last one behind the loop: with a second half that can be skipped inside the loop the
+        // compiler sees a path on which the tile loads of the first half are the newest at the loop's top, and
+        // waits there for all loads before the first LDS reads of every pass.
+        uint32_t s = 0;
+        for (; s + 1u < steps; s += 2) {
+            step2(A0, B0, A1, B1, s0, s1, s, std::true_type{});
+            step2(A1, B1, A0, B0, s1, s0, s + 1u, std::false_type{});
+        }
+        if (s < steps) {
+            step2(A0, B0, A1, B1, s0, s1, s, std::true_type{});
         }
     } else {
-        for (uint32_t s = 0; s < steps; s += 2) {
-            const uint32_t s2 = s + 2u < last ? s + 2u : last, s3 = s + 3u < last ? s + 3u : last;
-            compute(A0, B0, s0);                 // ends behind the barrier: stage 0 is free, stage 1 has landed
-            issue(s2 * kMxBK, A0, B0);
-            finish(s0);
-            load_scales(s0, s2);
-            if (s + 1u < steps) {
-                compute(A1, B1, s1);
-                issue(s3 * kMxBK, A1, B1);
-                finish(s1);
-                load_scales(s1, s3);
+        // A K step: all sub-steps but the last, then the last one's operands into registers, then the wait and the
+        // barrier, and only then the last sub-step's instructions: behind the barrier the matrix pipe has work at once.
+        auto step = [&](char* Ax, char* Bx, const Scales& sc, Scales& sc_next, uint32_t s, auto even) __attribute__((always_inline)) {
+#pragma unroll
+            for (int u = 0; u < kPieces; ++u) asm volatile("" : "+v"(foff[u]));
+            mx_static_for<kSub - 1>([&](auto sub) {
+                load_frags(f, Ax, Bx, decltype(sub)::value);
+                mfmas(f, sc, sub);
+            });
+            load_frags(f, Ax, Bx, kSub - 1);
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+            __syncthreads();
+            read_scales(sc_next, s + 1u);
+            __builtin_amdgcn_sched_barrier(0);
+            issue(next_step(s) * kMxBK, Ax, Bx);
+            if constexpr (decltype(even)::value) {
+                issue_scales((s >> 1) + 1u);
             }
+            mfmas(f, sc, std::integral_constant<int, kSub - 1>{});
+        };
+        uint32_t s = 0;
+        for (; s + 1u < steps; s += 2) {
+            step(A0, B0, s0, s1, s, std::true_type{});
+            step(A1, B1, s1, s0, s + 1u, std::false_type{});
+        }
+        if (s < steps) {
+            step(A0, B0, s0, s1, s, std::true_type{});
         }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the repeated loads of the last steps
@@ -471,7 +526,7 @@ inline bool mx_tile_shape_ok(const ascq_mx_desc* d)
     bool wa, wb;
     mx_widen_plan(d, wa, wb);
     const bool four = is_fp4(d->a_format) && !wa;  // both e2m1
-    return d->k % (four ? 256u : 128u) == 0 && d->scale_k % 8u == 0 && d->m >= 64u && d->n >= 64u;
+    return d->k % (four ? 256u : 128u) == 0 && d->scale_k % 8u == 0 && d->scale_k >= 16u && d->m >= 64u && d->n >= 64u;
 }
 
 int mx_validate(const ascq_mx_desc* d, const char* who)
