@@ -86,6 +86,22 @@ def test_mx_tile_kernel(m, n, k, fa, fb):
     mx_check(run_mx(m, n, k, a, b, sa, sb, fa, fb).cpu().numpy(), want, mx_abs_dot(a, b, sa, sb, k, fa, fb), is8(fa, fb))
 
 
+@pytest.mark.parametrize("m,n,k,sk", [(128, 128, 256, 16), (128, 192, 128, 16), (256, 256, 1280, 40), (200, 136, 640, 24),
+                                      (256, 256, 1024, 40), (320, 256, 2304, 72), (256, 256, 256, 8)])
+@pytest.mark.parametrize("fa,fb", [(E4, E5), (F2, F2), (F1, E4)])
+def test_mx_tile_kernel_scale_rows(m, n, k, sk, fa, fb):
+    """The tile kernel fetches 16 scale bytes per row for every two K steps and moves the last fetch back to stay inside
+    the row: rows of scale bytes that end in half a fetch, rows longer than k / 32, a single K step, odd numbers of
+    steps; rows shorter than one fetch (the last case) go through the element-wise kernel."""
+    announce("mx scale rows", m, n, k, sk, fa, fb)
+    rng = np.random.default_rng(m + 3 * n + 5 * k + 7 * sk + fa * 16 + fb)
+    a, b, sa, sb, _ = mx_case(rng, m, n, k, fa, fb, sk=sk)
+    d = abi.MxDesc(m=m, n=n, k=k, scale_k=sk, a_format=fa, b_format=fb, out_dtype=abi.F32, has_bias=0)
+    orc.set_threads(16)
+    want = orc.matmul_mx(d, a, b, sa, sb)
+    mx_check(run_mx(m, n, k, a, b, sa, sb, fa, fb).cpu().numpy(), want, mx_abs_dot(a, b, sa, sb, k, fa, fb), is8(fa, fb))
+
+
 @pytest.mark.parametrize("n", [320, 257])
 @pytest.mark.parametrize("out", [torch.bfloat16, torch.float16])
 def test_mx_sixteen_bit_outputs_and_bias(out, n):
