@@ -13,6 +13,7 @@
 //     antiquant_processor_using_ub.h:53-130); scale and offset belong to the lane's column, so they are lane constants;
 //   * the 8 partial sums of a column group are added in wavefront order in LDS and rounded once to the output type.
 // Up to 16 activation rows per pass; the host loops over more.  Requires k % 128 == 0, x / w 16-byte aligned.
+#include <type_traits>
 #include "ascq_common.h"
 #include "ascq_device.h"
 
@@ -285,7 +286,7 @@ __global__ __launch_bounds__(256, 2) void w8a16_nk_gemm_kernel(NkParams p, uint3
 
     const uint32_t lrow = lane & 31u, lk = lane >> 5;  // operand line and which 8 k of a sub-step
     // one K step on LDS stage st; `next` (data of the following step) is staged into the other LDS stage when do_stage
-    auto step_body = [&](uint32_t st, const Raw& next, bool do_stage) __attribute__((always_inline)) {
+    auto step_body = [&](uint32_t st, const Raw& next, auto do_stage) __attribute__((always_inline)) {
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
             const uint32_t piece = 2u * ks + lk;
@@ -302,7 +303,7 @@ __global__ __launch_bounds__(256, 2) void w8a16_nk_gemm_kernel(NkParams p, uint3
 #pragma unroll
                 for (int j = 0; j < 2; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
-            if (do_stage) {  // uniform; the other stage was last read before the barrier that ended the previous step
+            if constexpr (decltype(do_stage)::value) {  // the other stage was last read before the barrier that ended the previous step
                 stage_part(next, st ^ 1u, ks);
             }
         }
@@ -316,16 +317,23 @@ __global__ __launch_bounds__(256, 2) void w8a16_nk_gemm_kernel(NkParams p, uint3
     for (int q = 0; q < 4; ++q) stage_part(r0, 0, q);
     fetch(r1, 1u < last ? 1u : last);  // data of step 1 (clamped: a single-step problem re-reads step 0 and drops it)
     __syncthreads();
-    for (uint32_t s = 0; s < steps; s += 2) {
-        // step s on stage 0: r1 holds step s + 1; fetch step s + 2 into r0 (clamped at the end: harmless re-reads)
+    // Steps in pairs, an odd last one behind the loop, and nothing in a pair conditional (past the end the fetches
+    // repeat the last step's and the staging fills an LDS stage nobody reads): with a second half that can be skipped
+    // the compiler sees a path on which the first half's fetch is the newest load at the loop's top and waits there
+    // for every load in every pass, which takes the fetches' two-step lead away.
+    uint32_t s = 0;
+    for (; s + 1u < steps; s += 2) {
+        // step s on stage 0: r1 holds step s + 1; fetch step s + 2 into r0
         fetch(r0, s + 2u < last ? s + 2u : last);
-        step_body(0u, r1, s + 1u < steps);
+        step_body(0u, r1, std::true_type{});
         __syncthreads();
-        if (s + 1u < steps) {
-            fetch(r1, s + 3u < last ? s + 3u : last);
-            step_body(1u, r0, s + 2u < steps);
-            __syncthreads();
-        }
+        fetch(r1, s + 3u < last ? s + 3u : last);
+        step_body(1u, r0, std::true_type{});
+        __syncthreads();
+    }
+    if (s < steps) {
+        step_body(0u, r1, std::false_type{});
+        __syncthreads();
     }
 
     // ---- register r of lane l in a 32 x 32 block: row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32
