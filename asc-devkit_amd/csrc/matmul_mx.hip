@@ -70,8 +70,8 @@ __device__ __forceinline__ void mx_store(const MxParams& p, size_t idx, float v)
     }
 }
 
-// kFour: both operands 4-bit (e2m1); otherwise both 8-bit with the instruction's format codes kCa / kCb
-// (0 = e4m3, 1 = e5m2; 4 = e2m1).
+// kFour: both operands 4-bit (e2m1); otherwise both a byte per value in memory, with the instruction's format codes
+// kCa / kCb (0 = e4m3, 1 = e5m2, 2 = e2m3 as written by mx_widen_e1m2_kernel; 4 = e2m1).
 template <bool kFour, int kCa, int kCb>
 __global__ __launch_bounds__(kMxThreads, 1) void mx_tile_kernel(MxParams p)
 {
@@ -81,6 +81,8 @@ __global__ __launch_bounds__(kMxThreads, 1) void mx_tile_kernel(MxParams p)
     __shared__ __attribute__((aligned(1024))) char B1[kMxBN * kMxBK];
     __shared__ __attribute__((aligned(1024))) char SC[2 * kMxScaleBuf];  // two buffers of scale bytes, see below
     constexpr int TI = 4, TJ = 2;
+    constexpr bool kSix = !kFour && kCa == 2;  // e2m3 codes, the 24 bytes of every 32 values padded to 32
+    static_assert(!kSix || kCb == 2, "6-bit operands come in pairs");
     constexpr int kSub = kFour ? 4 : 2;       // instructions (64 k each) per K step and block pair
     constexpr int kScaleDw = kFour ? 2 : 1;   // dwords of scale bytes per row and K step
 
@@ -229,12 +231,14 @@ __global__ __launch_bounds__(kMxThreads, 1) void mx_tile_kernel(MxParams p)
     // ---- fragments: piece q of tile line r sits at r * 128 + ((q ^ ((r / 2) % 8)) * 16).  A lane reads piece
     // kPieceStep u + h (+ 2 for the upper registers of an 8-bit operand) of a line whose number is lrow + a multiple
     // of 32, i.e. at lrow * 128 + (((kPieceStep u) ^ (h ^ swizzle)) * 16) + constants: one register per u.
+    // (6-bit operands, 24 bytes per lane: pieces 4 s + 2 h and the first half of 4 s + 2 h + 1, u = 2 s and 2 s + 1)
     constexpr int kPieceStep = 2;
     constexpr int kPieces = 4;   // u = 0 .. 3: pieces 0 2 4 6 (+ h)
     uint32_t foff[kPieces];
 #pragma unroll
     for (int u = 0; u < kPieces; ++u) {
-        foff[u] = lrow * 128u + (((static_cast<uint32_t>(kPieceStep * u)) ^ (h ^ ((lrow >> 1) & 7u))) << 4);
+        const uint32_t piece = kSix ? 4u * (u >> 1) + 2u * h + (u & 1) : static_cast<uint32_t>(kPieceStep * u) ^ h;
+        foff[u] = lrow * 128u + ((piece ^ ((lrow >> 1) & 7u)) << 4);
     }
     auto frag = [&](const char* S, uint32_t line0, int u) __attribute__((always_inline)) {
         return *reinterpret_cast<const i32x4*>(S + line0 * 128u + foff[u]);
@@ -250,6 +254,13 @@ __global__ __launch_bounds__(kMxThreads, 1) void mx_tile_kernel(MxParams p)
             if constexpr (kFour) {
                 const i32x4 lo = frag(As, line0, s);
                 f.a[i] = __builtin_shufflevector(lo, lo, 0, 1, 2, 3, -1, -1, -1, -1);  // the instruction reads 4 registers of a 4-bit operand
+            } else if constexpr (kSix) {
+                const i32x4 lo = frag(As, line0, 2 * s);
+                const i32x2_t hi = *reinterpret_cast<const i32x2_t*>(As + line0 * 128u + foff[2 * s + 1]);
+                v8i t = __builtin_shufflevector(lo, lo, 0, 1, 2, 3, -1, -1, -1, -1);  // the instruction reads 6 registers
+                t[4] = hi[0];
+                t[5] = hi[1];
+                f.a[i] = t;
             } else {
                 const i32x4 lo = frag(As, line0, 2 * s), hi = frag(As, line0, 2 * s + 1);
                 f.a[i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
@@ -261,6 +272,13 @@ __global__ __launch_bounds__(kMxThreads, 1) void mx_tile_kernel(MxParams p)
             if constexpr (kFour) {
                 const i32x4 lo = frag(Bs, line0, s);
                 f.b[j] = __builtin_shufflevector(lo, lo, 0, 1, 2, 3, -1, -1, -1, -1);
+            } else if constexpr (kSix) {
+                const i32x4 lo = frag(Bs, line0, 2 * s);
+                const i32x2_t hi = *reinterpret_cast<const i32x2_t*>(Bs + line0 * 128u + foff[2 * s + 1]);
+                v8i t = __builtin_shufflevector(lo, lo, 0, 1, 2, 3, -1, -1, -1, -1);  // the instruction reads 6 registers
+                t[4] = hi[0];
+                t[5] = hi[1];
+                f.b[j] = t;
             } else {
                 const i32x4 lo = frag(Bs, line0, 2 * s), hi = frag(Bs, line0, 2 * s + 1);
                 f.b[j] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
@@ -510,6 +528,33 @@ __global__ __launch_bounds__(256) void mx_widen_fp4_kernel(const u32x4* __restri
     }
 }
 
+// e1m2 [rows, k / 2 bytes] -> e2m3 codes, 32 values as 24 bytes (little-endian 6-bit fields, the layout the matrix
+// instruction reads from a lane's six registers) followed by 8 unused bytes, so that a row is k bytes like an 8-bit
+// operand's.  An e1m2 value is +-(code / 4), code 0 .. 7, which is the e2m3 value with magnitude bits 2 * code (its
+// subnormals run 0, 1/8 .. 7/8 and its first binade 1, 9/8 .. 15/8).
+__global__ __launch_bounds__(256) void mx_widen_e1m2_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst,
+                                                            size_t pieces)
+{
+    for (size_t i = static_cast<size_t>(blockIdx.x) * 256u + threadIdx.x; i < pieces; i += static_cast<size_t>(gridDim.x) * 256u) {
+        const u32x4 q = __builtin_nontemporal_load(src + i);  // 32 values, value v of a dword in bits 4 v .. 4 v + 3
+        uint64_t c[4];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            uint64_t t = q[d];
+            t = (t & 0xFFFFull) | ((t & 0xFFFF0000ull) << 8);                              // values 0-3 | 4-7, 24 bits each
+            t = (t & 0x00000000FF0000FFull) | ((t & 0x000000FF0000FF00ull) << 4);          // pairs, 12 bits each
+            t = (t & 0x00000F00F00F00Full) | ((t & 0x0000F00F00F00F0ull) << 2);            // value v in bits 6 v .. 6 v + 3
+            c[d] = ((t & 0x0000208208208208ull) << 2) | ((t & 0x00001C71C71C71C7ull) << 1);  // sign to bit 5, magnitude doubled
+        }
+        const u32x4 lo = {static_cast<uint32_t>(c[0]), static_cast<uint32_t>(c[0] >> 32) | (static_cast<uint32_t>(c[1]) << 16),
+                          static_cast<uint32_t>(c[1] >> 16), static_cast<uint32_t>(c[2])};
+        const u32x4 hi = {static_cast<uint32_t>(c[2] >> 32) | (static_cast<uint32_t>(c[3]) << 16),
+                          static_cast<uint32_t>(c[3] >> 16), 0u, 0u};
+        dst[2 * i] = lo;
+        dst[2 * i + 1] = hi;
+    }
+}
+
 inline bool is_fp8(int f) { return f == ASCQ_QDST_FP8_E4M3FN || f == ASCQ_QDST_FP8_E5M2; }
 inline bool is_fp4(int f) { return f == ASCQ_QDST_FP4_E2M1 || f == ASCQ_QDST_FP4_E1M2; }
 
@@ -606,13 +651,20 @@ extern "C" int ascq_matmul_mx(const ascq_mx_desc* d, void* c, const void* a, con
         return launch_status("ascq_matmul_mx (element-wise)");
     }
     int fa = d->a_format, fb = d->b_format;
+    // two e1m2 operands become e2m3 codes, which the matrix core runs at the 4-bit rate; any other 4-bit operand e4m3
+    const bool six = fa == ASCQ_QDST_FP4_E1M2 && fb == ASCQ_QDST_FP4_E1M2;
     uint8_t* ws = static_cast<uint8_t*>(workspace);
     auto widen = [&](const uint8_t*& src, int& fmt, size_t rows) {
         const size_t pieces = rows * (d->k / 2u) / 16u;  // k is a multiple of 128 here
         size_t blocks = (pieces + 255u) / 256u;
         if (blocks > 65536u) blocks = 65536u;
-        mx_widen_fp4_kernel<<<static_cast<uint32_t>(blocks), 256, 0, st>>>(reinterpret_cast<const u32x4*>(src),
-                                                                          reinterpret_cast<u32x4*>(ws), pieces, fmt);
+        if (six) {
+            mx_widen_e1m2_kernel<<<static_cast<uint32_t>(blocks), 256, 0, st>>>(reinterpret_cast<const u32x4*>(src),
+                                                                               reinterpret_cast<u32x4*>(ws), pieces);
+        } else {
+            mx_widen_fp4_kernel<<<static_cast<uint32_t>(blocks), 256, 0, st>>>(reinterpret_cast<const u32x4*>(src),
+                                                                              reinterpret_cast<u32x4*>(ws), pieces, fmt);
+        }
         src = ws;
         ws += rows * d->k;
         fmt = ASCQ_QDST_FP8_E4M3FN;
@@ -623,13 +675,15 @@ extern "C" int ascq_matmul_mx(const ascq_mx_desc* d, void* c, const void* a, con
     if (wb) {
         widen(p.b, fb, d->n);
     }
-    const bool four = is_fp4(fa);
+    const bool four = is_fp4(fa);  // (after the widening: both e2m1)
     p.row_bytes = four ? d->k / 2u : d->k;
     p.tiles_m = (d->m + kMxBM - 1u) / kMxBM;
     p.tiles_n = (d->n + kMxBN - 1u) / kMxBN;
     const uint32_t grid = (p.tiles_m * p.tiles_n + 7u) / 8u * 8u;
     if (four) {
         mx_tile_kernel<true, 4, 4><<<grid, kMxThreads, 0, st>>>(p);
+    } else if (six) {
+        mx_tile_kernel<false, 2, 2><<<grid, kMxThreads, 0, st>>>(p);
     } else if (fa == ASCQ_QDST_FP8_E4M3FN && fb == ASCQ_QDST_FP8_E4M3FN) {
         mx_tile_kernel<false, 0, 0><<<grid, kMxThreads, 0, st>>>(p);
     } else if (fa == ASCQ_QDST_FP8_E4M3FN) {
