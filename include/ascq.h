@@ -551,7 +551,8 @@ int ascq_matmul_w8a16_workspace_size(const ascq_w8a16_desc* desc, size_t* bytes)
  * a_format / b_format: ASCQ_QDST_FP8_E4M3FN | ASCQ_QDST_FP8_E5M2 | ASCQ_QDST_FP4_E2M1 | ASCQ_QDST_FP4_E1M2.
  * Two 8-bit operands, or two e2m1 operands, with k % 128 == 0 (8-bit) / k % 256 == 0 (4-bit), 16-byte aligned a, b and
  * scale_k % 8 == 0, scale_k >= 16 run v_mfma_scale_f32_32x32x64_f8f6f4 on 256 x 256 tiles straight from the given buffers.  Other
- * format pairs first widen their 4-bit operands to e4m3 (exact) in the workspace; other shapes take a kernel with one
+ * format pairs first widen their 4-bit operands in the workspace (two e1m2 operands to 6-bit e2m3 codes, anything else
+ * to e4m3; both exact); other shapes take a kernel with one
  * lane per output element.
  * ref: include/basic_api/kernel_operator_mm_intf.h:321-340 (MmadMx), examples/01_simd_cpp_api/03_basic_api/
  *      03_matrix_compute/mmad_mx/README.md:5,131-152 and scripts/gen_data.py:52-140 (layouts, golden),
