@@ -547,7 +547,7 @@ def main():
         others["group_matmul_reference_example"] = r
         torch.cuda.empty_cache()
         for fmt in ("fp4", "fp8", "fp4_e1m2"):
-            others[f"mx_{fmt}_8192"] = mx(fmt, 10, 3)
+            others[f"mx_{fmt}_8192"] = mx(fmt, 100, 20)
             torch.cuda.empty_cache()
         out["others"] = others
 
