@@ -239,6 +239,9 @@ __global__ __launch_bounds__(kMxThreads, 1) void mx_tile_kernel(MxParams p)
     for (int u = 0; u < kPieces; ++u) {
         const uint32_t piece = kSix ? 4u * (u >> 1) + 2u * h + (u & 1) : static_cast<uint32_t>(kPieceStep * u) ^ h;
         foff[u] = lrow * 128u + ((piece ^ ((lrow >> 1) & 7u)) << 4);
+        if (kSix && (u & 1)) {
+            foff[u] += 8u * (lrow & 1u);  // odd rows keep these 8 bytes in the piece's second half
+        }
     }
     auto frag = [&](const char* S, uint32_t line0, int u) __attribute__((always_inline)) {
         return *reinterpret_cast<const i32x4*>(S + line0 * 128u + foff[u]);
@@ -532,8 +535,11 @@ __global__ __launch_bounds__(256) void mx_widen_fp4_kernel(const u32x4* __restri
 // instruction reads from a lane's six registers) followed by 8 unused bytes, so that a row is k bytes like an 8-bit
 // operand's.  An e1m2 value is +-(code / 4), code 0 .. 7, which is the e2m3 value with magnitude bits 2 * code (its
 // subnormals run 0, 1/8 .. 7/8 and its first binade 1, 9/8 .. 15/8).
+// The last 8 of the 24 bytes sit in the first half of the second 16-byte piece in even rows and in its second half in
+// odd rows: an 8-byte LDS read is served 16 lanes at a time, a row and its neighbour keep their pieces at the same
+// position of their 128-byte lines, and the two would meet in the same banks.
 __global__ __launch_bounds__(256) void mx_widen_e1m2_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst,
-                                                            size_t pieces)
+                                                            size_t pieces, uint32_t pieces_per_row)
 {
     for (size_t i = static_cast<size_t>(blockIdx.x) * 256u + threadIdx.x; i < pieces; i += static_cast<size_t>(gridDim.x) * 256u) {
         const u32x4 q = __builtin_nontemporal_load(src + i);  // 32 values, value v of a dword in bits 4 v .. 4 v + 3
@@ -548,10 +554,11 @@ __global__ __launch_bounds__(256) void mx_widen_e1m2_kernel(const u32x4* __restr
         }
         const u32x4 lo = {static_cast<uint32_t>(c[0]), static_cast<uint32_t>(c[0] >> 32) | (static_cast<uint32_t>(c[1]) << 16),
                           static_cast<uint32_t>(c[1] >> 16), static_cast<uint32_t>(c[2])};
-        const u32x4 hi = {static_cast<uint32_t>(c[2] >> 32) | (static_cast<uint32_t>(c[3]) << 16),
-                          static_cast<uint32_t>(c[3] >> 16), 0u, 0u};
+        const uint32_t w4 = static_cast<uint32_t>(c[2] >> 32) | (static_cast<uint32_t>(c[3]) << 16);
+        const uint32_t w5 = static_cast<uint32_t>(c[3] >> 16);
+        const bool upper = ((i / pieces_per_row) & 1u) != 0;
         dst[2 * i] = lo;
-        dst[2 * i + 1] = hi;
+        dst[2 * i + 1] = upper ? u32x4{0u, 0u, w4, w5} : u32x4{w4, w5, 0u, 0u};
     }
 }
 
@@ -660,7 +667,7 @@ extern "C" int ascq_matmul_mx(const ascq_mx_desc* d, void* c, const void* a, con
         if (blocks > 65536u) blocks = 65536u;
         if (six) {
             mx_widen_e1m2_kernel<<<static_cast<uint32_t>(blocks), 256, 0, st>>>(reinterpret_cast<const u32x4*>(src),
-                                                                               reinterpret_cast<u32x4*>(ws), pieces);
+                                                                               reinterpret_cast<u32x4*>(ws), pieces, d->k / 32u);
         } else {
             mx_widen_fp4_kernel<<<static_cast<uint32_t>(blocks), 256, 0, st>>>(reinterpret_cast<const u32x4*>(src),
                                                                               reinterpret_cast<u32x4*>(ws), pieces, fmt);
