@@ -158,9 +158,23 @@ __device__ __forceinline__ void gemm_dma_tile_at(const GemmParams& p, const Tile
     }
     const int8_t* Abase = p.a + static_cast<size_t>(row0) * K + static_cast<size_t>(s_begin) * BK;
     const int8_t* Bbase = Bmat + (kBT ? static_cast<size_t>(n0) * K : p.b_nz ? 0u : n0) + static_cast<size_t>(s_begin) * BK * ldb;
+    // A wavefront-uniform address, pinned to scalar registers: a load's address is then this base plus the lane's
+    // 32-bit offset, which the load instruction adds itself (otherwise the compiler widens the offsets to 64 bits
+    // ahead of the loop and adds the base per load: twice the registers and an addition per load).
+    auto uniform = [](const int8_t* q) __attribute__((always_inline)) {
+        const uint64_t v = reinterpret_cast<uint64_t>(q);
+        uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+        uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
+        asm volatile("" : "+s"(lo), "+s"(hi));
+        return reinterpret_cast<const int8_t*>((static_cast<uint64_t>(hi) << 32) | lo);
+    };
     auto issue = [&](uint32_t k0, char* As, char* Bs) {
-        const int8_t* ab = Abase + k0;
-        const int8_t* bb = Bbase + static_cast<size_t>(k0) * ldb;
+        const int8_t* ab = uniform(Abase + k0);
+        const int8_t* bb = uniform(Bbase + static_cast<size_t>(k0) * ldb);
+#pragma unroll
+        for (int u = 0; u < kAInstr; ++u) asm volatile("" : "+v"(aoff[u]));
+#pragma unroll
+        for (int u = 0; u < kBInstr; ++u) asm volatile("" : "+v"(boff[u]));
 #pragma unroll
         for (int u = 0; u < kAInstr; ++u) {
             __builtin_amdgcn_global_load_lds((gptr_t)(ab + aoff[u]), (lds_ptr_t)(As + (wave * kAInstr + u) * 1024), 16,
