@@ -11,11 +11,14 @@
 //     from lanes 32-63: two 16-byte LDS reads per operand and instruction.
 //   * 4-bit operands: registers 0-3 of lane l hold its row's k = 32 (l / 32) .. + 31 (16 bytes), scaled by the lane's
 //     own scale byte: one read per operand and instruction.
-// In both cases lane l needs scale byte 2 j + l / 32 of its row's bytes for this K step in sub-step j; the bytes of a
-// K step are fetched as one dword (8-bit) or two (4-bit) per row and shifted right by 8 (l / 32) once, so that the
-// byte selector of the instruction is the constant 0 or 2.
-// The element-wise kernel (one lane per output) takes every other shape; 4-bit operands that have no tile path of
-// their own (e1m2, or a 4-bit operand beside an 8-bit one) are first widened to e4m3, which holds every fp4 value.
+//   * 6-bit operands (e2m3 codes, what two e1m2 operands are rewritten as): registers 0-5 of lane l hold its row's
+//     k = 32 (l / 32) .. + 31 as little-endian 6-bit fields (24 bytes, padded to 32 in memory), scaled by the lane's
+//     own scale byte: a 16-byte and an 8-byte read per operand and instruction.
+// In every case lane l needs scale byte 2 j + l / 32 of its row's bytes for this K step in sub-step j; a lane holds
+// the bytes of a K step as one dword (8- and 6-bit) or two (4-bit) per row, staged through LDS, and shifts them right
+// by 8 (l / 32) where they are used, so that the byte selector of the instruction is the constant 0 or 2.
+// The element-wise kernel (one lane per output) takes every other shape; a 4-bit operand beside an 8-bit one, or e1m2
+// beside e2m1, is first widened to e4m3, which holds every fp4 value.
 #include <type_traits>
 #include <utility>
 
@@ -130,8 +133,7 @@ __global__ __launch_bounds__(kMxThreads, 1) void mx_tile_kernel(MxParams p)
     const uint8_t* Bbase = p.b + static_cast<size_t>(n0) * RB;
     // A wavefront-uniform address, pinned to scalar registers: a load's address is then this base plus the lane's
     // 32-bit offset, which the load instruction adds itself (otherwise the compiler folds the lane's offset into
-    // 64-bit per-lane addresses, twice the registers and an addition per load, in temporaries whose reuse by the
-    // next LDS reads makes it wait for the loads).
+    // 64-bit per-lane addresses: twice the registers and an addition per load).
     auto uniform = [](const uint8_t* q) __attribute__((always_inline)) {
         const uint64_t v = reinterpret_cast<uint64_t>(q);
         uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
