@@ -327,7 +327,7 @@ def test_noalloc_entry_point_rejects_before_touching_the_gpu():
 
 
 def test_integration_snippet_matches_the_abi():
-    """The ctypes struct printed in INTEGRATION.md has the fields of the struct the library reads."""
+    """The ctypes struct printed in the integration notes has the fields of the struct the library reads."""
     text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
     block = text[text.index("class QuantDesc(C.Structure)"):]
     block = block[:block.index("lib.ascq_quant.restype")]
