@@ -28,6 +28,7 @@ MM_BIAS_NONE, MM_BIAS_I32_PRE, MM_BIAS_F32_POST, MM_BIAS_BF16_POST = range(4)
 MM_ACT_NONE, MM_ACT_FASTER_GELU, MM_ACT_SWIGLU = range(3)
 MM_B_ND, MM_B_NZ = range(2)
 GROUP_LIST_COUNTS, GROUP_LIST_PREFIX_SUM = range(2)
+W4A16_PER_WEIGHT, W4A16_GROUP_SUM = range(2)
 
 STATUS_NAMES = {OK: "ASCQ_OK", EINVAL: "ASCQ_EINVAL", EUNSUPPORTED: "ASCQ_EUNSUPPORTED", EALIGN: "ASCQ_EALIGN",
                 EHIP: "ASCQ_EHIP", ENULL: "ASCQ_ENULL"}
@@ -74,7 +75,7 @@ class GroupMatmulDesc(C.Structure):
 
 class W4A16Desc(C.Structure):
     _fields_ = [("m", C.c_uint32), ("n", C.c_uint32), ("k", C.c_uint32), ("group_size", C.c_uint32),
-                ("has_offset", C.c_int32)]
+                ("has_offset", C.c_int32), ("mode", C.c_int32)]
 
 
 class W8A16Desc(C.Structure):

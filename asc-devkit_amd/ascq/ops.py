@@ -484,11 +484,13 @@ def pack_weight_w4(w_nd, k, n):
     return out
 
 
-def matmul_w4a16_packed(y, x, w_gpu, scale, offset=None, group_size=128):
-    """matmul_w4a16 on weights packed by pack_weight_w4: one launch, no workspace, same arithmetic."""
+def matmul_w4a16_packed(y, x, w_gpu, scale, offset=None, group_size=128, mode=abi.W4A16_PER_WEIGHT):
+    """matmul_w4a16 on weights packed by pack_weight_w4: one launch, no workspace.  mode abi.W4A16_PER_WEIGHT (default)
+    keeps AscendAntiQuant's two roundings to half per weight; abi.W4A16_GROUP_SUM applies scale and offset once per
+    quantisation group to fp32 sums (same value, no per-weight roundings, faster)."""
     m, k = x.shape
     n = y.shape[1]
-    d = abi.W4A16Desc(m=m, n=n, k=k, group_size=group_size, has_offset=int(offset is not None))
+    d = abi.W4A16Desc(m=m, n=n, k=k, group_size=group_size, has_offset=int(offset is not None), mode=mode)
     check(load_library().ascq_matmul_w4a16_packed(C.byref(d), _ptr(y), _ptr(x), _ptr(w_gpu), _ptr(scale),
                                                   _ptr(offset), _stream()))
     return y

@@ -16,11 +16,14 @@
 // staged in LDS once per pass over k (coalesced 16-byte loads); operand row i of a lane reads activation row i % m, so
 // there are no zero rows to materialise (result rows >= m repeat earlier ones and are not stored).
 //
-// A workgroup owns whole slabs: its wavefronts split k, every wavefront streams a contiguous piece of each slab with
-// two batches of tiles in flight behind the one being computed, and the per-wavefront sums meet in LDS, where they
-// are added in wavefront order and rounded once to half: no second kernel, no workspace, deterministic.
-// De-quantisation follows AscendAntiQuant<int4b_t, half> exactly (one rounded half add of the offset, one rounded half
-// multiply by the scale per weight); the products and sums are fp32.
+// A workgroup owns whole slabs: its wavefronts split k, every wavefront streams a contiguous piece of each slab in
+// batches of 4 tiles, one batch in flight while one is computed (deeper queues were slower: a compute unit keeps about
+// 64 KiB of loads in flight whatever is asked of it, and a wavefront that asks for more only waits at the issue of
+// its loads with data it could compute on), and the per-wavefront sums meet in LDS, where they are added in wavefront
+// order and rounded once to half: no second kernel, no workspace, deterministic.
+// De-quantisation follows AscendAntiQuant<int4b_t, half> exactly by default (one rounded half add of the offset, one
+// rounded half multiply by the scale per weight); ASCQ_W4A16_GROUP_SUM applies scale and offset to fp32 sums per tile
+// instead.  The products and sums are fp32 either way.
 #include <type_traits>
 
 #include "ascq_common.h"
@@ -30,19 +33,20 @@ namespace ascq {
 namespace {
 
 constexpr uint32_t kSlabCols = 16, kTileK = 128, kTileBytes = 1024;
-constexpr int kBuf = 3;                  // register buffers: two batches in flight behind the one being computed
+constexpr int kBuf = 2;                  // register buffers: one batch in flight while the other is computed
 constexpr uint32_t kPadTiles = 16;       // tiles of padding behind the last slab of a packed matrix (a batch may read on)
 constexpr uint32_t kMaxSlabs = 8;        // slabs per workgroup
 constexpr uint32_t kMaxRows = 16;        // activation rows per launch
 constexpr uint32_t kPool = 152 * 1024;   // LDS of a workgroup: staged activations, parameters, per-wavefront sums
 constexpr uint32_t kXBytes = 72 * 1024;  // at most this much of it for the activations of one pass over k
-constexpr uint32_t kParBytes = 32 * 1024;// and this much for the (scale, offset) pairs of one pass
+constexpr uint32_t kParBytes = 40 * 1024;// and this much for the (scale, offset) pairs of one pass
 constexpr uint32_t kPastEnd = 0x7FFFFFF0u;  // a per-lane buffer offset beyond any buffer this kernel accepts (< 2 GiB)
 constexpr int kNt = 2;                   // cache policy of the weight loads: non-temporal (read once per call)
 constexpr uint32_t kRowPad = 16;         // bytes added to a staged activation row: rows start 4 banks apart
 
 struct NibbleMasks {
     uint32_t even, odd, exp;  // 0x000F000F, 0x00F000F0, 0x64006400
+    uint32_t exp_odd;         // 0x54005400: with a nibble in bits 4..7 of its mantissa the half is 64 + u
 };
 
 struct W4pParams {
@@ -57,13 +61,14 @@ struct W4pParams {
     uint32_t slabs, ktiles;  // ceil(n / 16), k / 128
     uint32_t slabs_per_wg;   // 1 .. kMaxSlabs
     uint32_t pass_tiles;     // tiles of k staged per pass (multiple of the wavefront count)
-    uint32_t ppr_magic;      // ceil(2^32 / (tiles per wavefront * 16)): i / that = mulhi(i, ppr_magic) for i < 65536
-    uint32_t par_magic;      // ceil(2^32 / (slabs_per_wg * 2)), likewise
+    uint32_t m_magic;        // ceil(2^32 / m): i / m = mulhi(i, m_magic) for i < 65536
+    uint32_t par_cw;         // log2 of the lanes that share a group row when the parameters are fetched: 2^cw >= 2 slabs_per_wg
     uint32_t xs_wave, par_wave;  // bytes of staged activations / parameters per wavefront
     uint32_t par_pitch;          // entries per column of a wavefront's parameter table (odd)
     uint32_t par_off, red_off;   // byte offsets of the parameter tables and of the sums inside the LDS pool
     NibbleMasks mk;
     uint32_t red_lanes;      // lanes of a result register that hold rows < m: 16 for m <= 4, else 64
+    uint32_t sum_off, sum_wave;  // group-sum form: byte offset of the activation sums in the pool, bytes per wavefront
 };
 
 __device__ __forceinline__ f16x2 bits_h2(uint32_t b)
@@ -78,6 +83,11 @@ __device__ __forceinline__ uint32_t h2_bits(f16x2 h)
     __builtin_memcpy(&r, &h, 4);
     return r;
 }
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef __attribute__((address_space(1))) const void* gptr_t;
+
+__device__ __forceinline__ uint32_t mod_m(uint32_t i, const W4pParams& p) { return i - __umulhi(i, p.m_magic) * p.m; }
 
 // One dword of packed weights (8 consecutive k of one column, offset binary) -> the 8 de-quantised halves in k order.
 // kFold: ofe holds offset - 1032 and ofo offset - 72 (both halves), exact for integer offsets of magnitude <= 512, so
@@ -112,12 +122,32 @@ __device__ __forceinline__ f16x8 dequant8(uint32_t qd, f16x2 sc, f16x2 ofe, f16x
     return b;
 }
 
-template <bool kHasOffset, uint32_t kWaves, uint32_t kBatch>
+// One dword of packed weights -> 8 halves in k order that still carry their conversion constants: k offsets 0 1 4 5
+// become 1024 + u = 1032 + w, k offsets 2 3 6 7 become 64 + u = 72 + w.  Four v_and_or_b32 and one shift.
+__device__ __forceinline__ f16x8 raw8(uint32_t qd, const NibbleMasks& mk)
+{
+    const uint32_t qh = qd >> 8;
+    uint32_t h[4];
+    h[0] = (qd & mk.even) | mk.exp;
+    h[1] = (qd & mk.odd) | mk.exp_odd;
+    h[2] = (qh & mk.even) | mk.exp;
+    h[3] = (qh & mk.odd) | mk.exp_odd;
+    f16x8 b;
+    __builtin_memcpy(&b, h, 16);
+    return b;
+}
+constexpr float kBiasEven = 1032.0f, kBiasOdd = 72.0f;  // what raw8 adds to w at k offsets 0 1 4 5 / 2 3 6 7
+
+// kSum = 0: every weight is de-quantised as AscendAntiQuant does it (two roundings to half per weight).
+// kSum = 1, 2, 4 (the group-sum form, result registers in use = rows, group_size a multiple of 128): the matrix core
+// multiplies the activations with the raw halves of raw8 and scale and offset are applied once per tile of 128 k to the
+// fp32 sum,  y += scale * (sum_k x_k (w_k + c_k) - sum_k x_k c_k + offset * sum_k x_k),  where the two sums over the
+// activations alone are formed once per wavefront and tile before the weights arrive.
+template <bool kHasOffset, uint32_t kWaves, uint32_t kBatch, uint32_t kSum>
 __global__ __launch_bounds__(kWaves * 64) void w4a16_packed_kernel(W4pParams p)
 {
     constexpr uint32_t kThreadsWg = kWaves * 64u;
-    constexpr uint32_t kXPieces = (kXBytes / 16u + kThreadsWg - 1u) / kThreadsWg;    // 16-byte pieces per lane
-    constexpr uint32_t kParPieces = 2;  // 8-column parameter pieces per lane (the host keeps a wavefront's table within 128)
+    constexpr uint32_t kParPieces = 3;  // 8-column parameter pieces per lane (the host keeps a wavefront's table within that)
     __shared__ __attribute__((aligned(16))) char POOL[kPool];
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -133,8 +163,7 @@ __global__ __launch_bounds__(kWaves * 64) void w4a16_packed_kernel(W4pParams p)
     const uint32_t nslabs = min(spw, p.slabs - slab0);
     const uint32_t tpw = p.pass_tiles / kWaves;             // tiles of a pass per wavefront
     const uint32_t pitch = tpw * kTileK * 2u + kRowPad;     // bytes of a staged activation row
-    const uint32_t ppr = tpw * (kTileK / 8u);               // 16-byte pieces of a staged row
-    const uint32_t x_lane = ((lane & 15u) % p.m) * pitch + g * 64u;  // operand row i reads row i % m; + tile * 256 + d * 16
+    const uint32_t x_lane = mod_m(lane & 15u, p) * pitch + g * 64u;  // operand row i reads row i % m; + tile * 256 + d * 16
     const uint32_t row_bytes = p.n * 2u;                          // one row of scale / offset in memory
     const uint32_t par_col = p.par_pitch * 4u;                    // bytes of one column of the table in LDS (odd number of entries)
     // The quantisation group of a lane's 32 k, (4 tile + g) / (group_size / 32) with group_size / 32 = 2^s, splits into
@@ -149,21 +178,20 @@ __global__ __launch_bounds__(kWaves * 64) void w4a16_packed_kernel(W4pParams p)
     // the exponent constant lives in a vector register so that mask (scalar) and constant fit one v_and_or_b32
     NibbleMasks mk = p.mk;
     asm volatile("" : "+v"(mk.exp));
+    if constexpr (kSum != 0u) {
+        asm volatile("" : "+v"(mk.exp_odd));
+    }
+    char* const SUM = POOL + p.sum_off + wave * p.sum_wave;  // [tile of the wavefront's share][sums of rows 0..3 | -weighted sums]
     const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<u32x4*>(p.wp), 0, static_cast<int>((p.slabs * p.ktiles + kPadTiles) * kTileBytes), 0x00020000);
     const int par_bytes = static_cast<int>(((p.k / 32u) >> gsh) * row_bytes);
     const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.scale), 0, par_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t*>(kHasOffset ? p.offset : p.scale), 0, par_bytes, 0x00020000);
-    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint16_t*>(p.x), 0, static_cast<int>(p.m * p.k * 2u), 0x00020000);
 
     // sums of this wavefront per slab, kept in LDS between passes
     const uint32_t rl = p.red_lanes, red_wave = spw * 4u * rl;  // floats per wavefront
     float* red = RED + wave * red_wave;
-    if (lane < rl) {
-        for (uint32_t s = 0; s < nslabs * 4u; ++s) red[s * rl + lane] = 0.0f;
-    }
 
     for (uint32_t pt0 = 0; pt0 < p.ktiles; pt0 += p.pass_tiles) {
         const uint32_t ptiles = min(p.pass_tiles, p.ktiles - pt0);
@@ -177,9 +205,9 @@ __global__ __launch_bounds__(kWaves * 64) void w4a16_packed_kernel(W4pParams p)
         const uint32_t g_rows = cnt != 0u ? ((((pt0 + tb) * 4u - 1u) >> gsh) - g_base + 1u) : 0u;  // groups it touches
 
         // Every weight load is unconditional, so the loop body is straight-line as far as memory loads go and the waits
-        // the compiler inserts count exactly: two batches stay in flight while one is computed.  A tile past the end of
-        // its slab's range re-reads the last one (and is not computed); once every batch has been requested the
-        // per-lane offset points past the end of the buffer and the loads of the loop's last rounds are dropped.
+        // the compiler inserts count exactly: one batch stays in flight while the other is computed.  Once every batch
+        // has been requested the per-lane offset points past the end of the buffer and the loads of the loop's last
+        // rounds are dropped.
         u32x4 wq[kBuf][kBatch];
         uint32_t l_slab = slab0, l_b = 0, l_q = 0;  // load cursor: slab, batch within the slab, batch number
         bool l_done = batches == 0u;               // every batch has been requested
@@ -203,57 +231,88 @@ __global__ __launch_bounds__(kWaves * 64) void w4a16_packed_kernel(W4pParams p)
             }
         };
 
-        // ---- The wavefront's activations (m rows x its tiles' k) and parameters (its groups x the workgroup's columns)
-        // travel through registers into its part of the LDS.  Their loads are issued first and the first weight batch
-        // behind them: loads return in order, so the wait for the staged data leaves the weights in flight.
-        // Activation piece i (16 bytes) is piece i % ppr of row i / ppr; pieces past the last row lie past the end of
-        // the buffer (dropped loads), pieces past the wavefront's tiles are never read back.  Parameter piece i is 8
-        // columns: piece i % (2 spw) of group row i / (2 spw).
-        u32x4 xr[kXPieces], sr[kParPieces], orr[kParPieces];
-#pragma unroll
-        for (uint32_t u = 0; u < kXPieces; ++u) {
-            const uint32_t i = lane + u * 64u;
-            const uint32_t r = __umulhi(i, p.ppr_magic), c = i - r * ppr;
-            xr[u] = __builtin_amdgcn_raw_buffer_load_b128(
-                rx, (r < p.m && cnt != 0u) ? (r * p.k + (pt0 + ta) * kTileK + c * 8u) * 2u : kPastEnd, 0, 0);
+        // ---- The wavefront's activations (m rows x its tiles' k) go straight into its part of the LDS, 1 KiB of a row
+        // per instruction; its parameters (its groups x the workgroup's columns) travel through registers.  Loads
+        // return in order, so the wait for these leaves the two weight batches requested behind them in flight.  (These
+        // small loads go first: a compute unit's queue is served in order, and behind the weight batches of eight
+        // wavefronts they would arrive microseconds later.)
+        {
+            const uint32_t row_pieces = cnt * (kTileK / 8u);
+            for (uint32_t r = 0; r < p.m; ++r) {
+                const uint16_t* src = p.x + static_cast<size_t>(r) * p.k + (pt0 + ta) * kTileK + lane * 8u;
+                for (uint32_t c0 = 0; c0 < row_pieces; c0 += 64u) {
+                    if (c0 + lane < row_pieces) {
+                        __builtin_amdgcn_global_load_lds((gptr_t)(src + c0 * 8u), (lds_ptr_t)(XS + r * pitch + c0 * 16u), 16, 0, 0);
+                    }
+                }
+            }
         }
+        // Parameter piece (8 columns) of lane l in round u: column piece l % 2^cw, group row (l >> cw) + u (64 >> cw),
+        // 2^cw >= 2 slabs_per_wg.
+        u32x4 sr[kParPieces], orr[kParPieces];
+        const uint32_t par_c = lane & ((1u << p.par_cw) - 1u), par_r0 = lane >> p.par_cw, par_rstep = 64u >> p.par_cw;
 #pragma unroll
         for (uint32_t u = 0; u < kParPieces; ++u) {
-            const uint32_t i = lane + u * 64u;
-            const uint32_t r = __umulhi(i, p.par_magic), c = i - r * (2u * spw);
-            const uint32_t col = slab0 * kSlabCols + c * 8u;
-            const uint32_t off = (r < g_rows && col < p.n) ? ((g_base + r) * p.n + col) * 2u : kPastEnd;
+            const uint32_t r = par_r0 + u * par_rstep;
+            const uint32_t col = slab0 * kSlabCols + par_c * 8u;
+            const uint32_t off = (r < g_rows && par_c < 2u * spw && col < p.n) ? ((g_base + r) * p.n + col) * 2u : kPastEnd;
             sr[u] = __builtin_amdgcn_raw_buffer_load_b128(rs, off, 0, 0);
             if constexpr (kHasOffset) {
                 orr[u] = __builtin_amdgcn_raw_buffer_load_b128(ro, off, 0, 0);
             }
         }
-        load(0);
 #pragma unroll
-        for (uint32_t u = 0; u < kXPieces; ++u) {
-            const uint32_t i = lane + u * 64u;
-            const uint32_t r = __umulhi(i, p.ppr_magic), c = i - r * ppr;
-            if (r < p.m) {
-                *reinterpret_cast<u32x4*>(XS + r * pitch + c * 16u) = xr[u];
-            }
+        for (int b = 0; b < kBuf; ++b) load(b);
+        if (pt0 == 0u && lane < rl) {  // sums of this wavefront per slab, kept in LDS between passes
+            for (uint32_t s = 0; s < nslabs * 4u; ++s) red[s * rl + lane] = 0.0f;
         }
 #pragma unroll
         for (uint32_t u = 0; u < kParPieces; ++u) {
-            const uint32_t i = lane + u * 64u;
-            const uint32_t r = __umulhi(i, p.par_magic), c = i - r * (2u * spw);
-            if (r < g_rows) {
+            const uint32_t r = par_r0 + u * par_rstep;
+            if (r < g_rows && par_c < 2u * spw) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const uint32_t o2 = kHasOffset ? orr[u][e] : 0u;
-                    char* dst = PAR + (c * 8u + 2u * e) * par_col + r * 4u;
+                    char* dst = PAR + (par_c * 8u + 2u * e) * par_col + r * 4u;
                     *reinterpret_cast<uint32_t*>(dst) = __builtin_amdgcn_perm(o2, sr[u][e], 0x05040100u);            // (s, o) of column 2e
                     *reinterpret_cast<uint32_t*>(dst + par_col) = __builtin_amdgcn_perm(o2, sr[u][e], 0x07060302u);  // column 2e + 1
                 }
             }
         }
-        load(1);
         if (batches == 0u) {
             continue;  // uniform over the wavefront
+        }
+        if constexpr (kSum != 0u) {
+            // Sums of the staged activations per tile: lane = (tile of the round, result register r, one of 8 parts of
+            // 16 k), 8 / kSum tiles per round; register r of the lanes that are stored holds row r % m.  Per part the
+            // k offsets 0 1 4 5 (mod 8) and 2 3 6 7 are summed apart, the 8 parts are added across lanes, and the table
+            // keeps  sum x  and  -(1032 sum_even x + 72 sum_odd x)  per tile and register.
+            constexpr uint32_t kTilesRound = 8u / kSum;
+            const uint32_t part = lane & 7u, reg = (lane >> 3) & (kSum - 1u);
+            const uint32_t srow = kSum == 1u ? 0u : mod_m(reg, p);
+            for (uint32_t t2 = 0; t2 < cnt; t2 += kTilesRound) {
+                const uint32_t tt = t2 + (lane >> 3) / kSum;
+                const char* src = XS + srow * pitch + min(tt, cnt - 1u) * 256u + part * 32u;
+                float se = 0.0f, so = 0.0f;
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const f16x8 v = *reinterpret_cast<const f16x8*>(src + h * 16);
+                    se += (static_cast<float>(v[0]) + static_cast<float>(v[1])) + (static_cast<float>(v[4]) + static_cast<float>(v[5]));
+                    so += (static_cast<float>(v[2]) + static_cast<float>(v[3])) + (static_cast<float>(v[6]) + static_cast<float>(v[7]));
+                }
+                // add over the 8 parts: lane ^ 1, lane ^ 2 inside a quad, then the mirrored half row (the other quad)
+                se += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(se), 0xB1, 0xF, 0xF, true));
+                so += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(so), 0xB1, 0xF, 0xF, true));
+                se += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(se), 0x4E, 0xF, 0xF, true));
+                so += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(so), 0x4E, 0xF, 0xF, true));
+                se += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(se), 0x141, 0xF, 0xF, true));
+                so += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(so), 0x141, 0xF, 0xF, true));
+                if (part == 0u && tt < cnt) {
+                    float* dst = reinterpret_cast<float*>(SUM + tt * 32u);
+                    dst[reg] = se + so;
+                    dst[4u + reg] = -(kBiasEven * se + kBiasOdd * so);
+                }
+            }
         }
 
         f32x4 acc[2] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
@@ -285,7 +344,7 @@ __global__ __launch_bounds__(kWaves * 64) void w4a16_packed_kernel(W4pParams p)
                     pp[t] = *reinterpret_cast<const uint32_t*>(pa0 + grow * 4u);
                 }
             }
-            if constexpr (kHasOffset) {
+            if constexpr (kHasOffset && kSum == 0u) {
 #pragma unroll
                 for (uint32_t t = 0; t < kBatch; ++t) {
                     const f16x2 k1536 = {static_cast<half_t>(1536.0f), static_cast<half_t>(1536.0f)};
@@ -293,12 +352,29 @@ __global__ __launch_bounds__(kWaves * 64) void w4a16_packed_kernel(W4pParams p)
                     frac |= (h2_bits(rt) ^ pp[t]) & 0x7FFF0000u;  // the offset is the high half
                 }
             }
-            const bool fold = kHasOffset && __builtin_amdgcn_ballot_w64(frac != 0u) == 0;  // uniform
+            const bool fold = kHasOffset && kSum == 0u && __builtin_amdgcn_ballot_w64(frac != 0u) == 0;  // uniform
             auto tiles = [&](auto folded) __attribute__((always_inline)) {
                 constexpr bool kFold = decltype(folded)::value;
 #pragma unroll
                 for (uint32_t t = 0; t < kBatch; ++t) {
                     if (t < live) {  // uniform; no memory loads inside, so the wait counts stay exact
+                        if constexpr (kSum != 0u) {
+                            const f16x2 sp = bits_h2(pp[t]);
+                            const float scf = static_cast<float>(sp[0]), off = static_cast<float>(sp[1]);
+                            const char* sm = SUM + (t0 - ta + t) * 32u;
+                            const f32x4 xs = *reinterpret_cast<const f32x4*>(sm);
+                            f32x4 part = *reinterpret_cast<const f32x4*>(sm + 16);
+#pragma unroll
+                            for (int d = 0; d < 4; ++d) {
+                                const f16x8 a = *reinterpret_cast<const f16x8*>(xa0 + t * 256u + d * 16);
+                                part = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, raw8(wq[buf][t][d], mk), part, 0, 0, 0);
+                            }
+#pragma unroll
+                            for (uint32_t r = 0; r < kSum; ++r) {
+                                acc[0][r] = __builtin_fmaf(scf, kHasOffset ? __builtin_fmaf(off, xs[r], part[r]) : part[r], acc[0][r]);
+                            }
+                            continue;
+                        }
                         const f16x2 sp = bits_h2(pp[t]);
                         const f16x2 sc = {sp[0], sp[0]};
                         f16x2 ofe = {sp[1], sp[1]}, ofo = ofe;
@@ -334,13 +410,12 @@ __global__ __launch_bounds__(kWaves * 64) void w4a16_packed_kernel(W4pParams p)
             }
         };
 
-        for (uint32_t q = 0; q < batches; q += 3u) {
-            load(2);
-            compute(0);
-            load(0);
-            compute(1);
-            load(1);
-            compute(2);
+        for (uint32_t q = 0; q < batches; q += kBuf) {
+#pragma unroll
+            for (int b = 0; b < kBuf; ++b) {
+                compute(b);
+                load(b);
+            }
         }
     }
 
@@ -368,12 +443,18 @@ __global__ __launch_bounds__(kWaves * 64) void w4a16_packed_kernel(W4pParams p)
 // never leave its registers - no reduction in LDS, no second pass.  The wavefronts of a workgroup walk k together and
 // share the activations: chunk c (8 tiles = 1024 k of all m rows) lies in one of two LDS buffers while the next is
 // fetched, one barrier per chunk.  The (scale, offset) pairs of a slab for all of k are staged once per wavefront.
+constexpr int kRowsBuf = 3;
 constexpr uint32_t kRowsBatch = 8;          // tiles per batch of weight loads = tiles per activation chunk
 constexpr uint32_t kRowsMaxGroups = 128;    // quantisation groups along k this kernel has LDS for
 constexpr uint32_t kRowsChunkBytes = kRowsBatch * kTileK * 2u;  // bytes of one activation row per chunk
 constexpr uint32_t kRowsPitch = kRowsChunkBytes + kRowPad;
 
-template <bool kHasOffset, uint32_t kW>
+// kSumForm (group_size a multiple of 128): raw weight halves (raw8) on the matrix core, scale and offset applied once
+// per tile to fp32 sums.  What raw8 adds to the weights is taken off by the matrix core as well - a second product of the
+// same activations with the constant operand -c_k accumulates into the same registers - and a third with the operand 1
+// gives the sum of the activations that the offset multiplies: the rows differ from lane to lane here, so a table of
+// sums would cost more vector instructions than the de-quantisation it replaces, while the matrix pipe has room.
+template <bool kHasOffset, uint32_t kW, bool kSumForm>
 __global__ __launch_bounds__(kW * 64) void w4a16_packed_rows_kernel(W4pParams p)
 {
     constexpr uint32_t kT = kW * 64u;
@@ -396,6 +477,16 @@ __global__ __launch_bounds__(kW * 64) void w4a16_packed_rows_kernel(W4pParams p)
 
     NibbleMasks mk = p.mk;
     asm volatile("" : "+v"(mk.exp));
+    f16x8 b_neg, b_one;  // constant B operands of the group-sum form: -(what raw8 adds to each weight), and ones
+    if constexpr (kSumForm) {
+        asm volatile("" : "+v"(mk.exp_odd));
+        const f16x2 ne = {static_cast<half_t>(-kBiasEven), static_cast<half_t>(-kBiasEven)};
+        const f16x2 no = {static_cast<half_t>(-kBiasOdd), static_cast<half_t>(-kBiasOdd)};
+        const f16x2 one = {static_cast<half_t>(1.0f), static_cast<half_t>(1.0f)};
+        const f16x2 hn[4] = {ne, no, ne, no}, ho[4] = {one, one, one, one};
+        __builtin_memcpy(&b_neg, hn, 16);
+        __builtin_memcpy(&b_one, ho, 16);
+    }
     const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<u32x4*>(p.wp), 0, static_cast<int>((p.slabs * p.ktiles + kPadTiles) * kTileBytes), 0x00020000);
     const int par_bytes = static_cast<int>(groups * p.n * 2u);
@@ -448,7 +539,7 @@ __global__ __launch_bounds__(kW * 64) void w4a16_packed_rows_kernel(W4pParams p)
     };
     // ---- weights of batch q: unconditional loads (a batch past the end, or of a wavefront without a slab, is given an
     // offset beyond the buffer and moves no data; the last batch may read on into the next slab or the padding)
-    u32x4 wq[kBuf][kRowsBatch];
+    u32x4 wq[kRowsBuf][kRowsBatch];
     auto wload = [&](int buf, uint32_t q) __attribute__((always_inline)) {
         const uint32_t l_w = (live && q < nb) ? lane * 16u : kPastEnd;
         const uint32_t base = (slab * p.ktiles + q * kRowsBatch) * kTileBytes;  // scalar
@@ -477,7 +568,7 @@ __global__ __launch_bounds__(kW * 64) void w4a16_packed_rows_kernel(W4pParams p)
                 pp[t] = *reinterpret_cast<const uint32_t*>(pa0 + grow * 4u);
             }
         }
-        if constexpr (kHasOffset) {
+        if constexpr (kHasOffset && !kSumForm) {
 #pragma unroll
             for (uint32_t t = 0; t < kRowsBatch; ++t) {
                 const f16x2 k1536 = {static_cast<half_t>(1536.0f), static_cast<half_t>(1536.0f)};
@@ -485,12 +576,31 @@ __global__ __launch_bounds__(kW * 64) void w4a16_packed_rows_kernel(W4pParams p)
                 frac |= (h2_bits(rt) ^ pp[t]) & 0x7FFF0000u;  // the offset is the high half
             }
         }
-        const bool fold = kHasOffset && __builtin_amdgcn_ballot_w64(frac != 0u) == 0;  // uniform
+        const bool fold = kHasOffset && !kSumForm && __builtin_amdgcn_ballot_w64(frac != 0u) == 0;  // uniform
         auto tiles = [&](auto folded) __attribute__((always_inline)) {
             constexpr bool kFold = decltype(folded)::value;
 #pragma unroll
             for (uint32_t t = 0; t < kRowsBatch; ++t) {
                 if (t < live_t) {  // uniform
+                    if constexpr (kSumForm) {
+                        const f16x2 sp = bits_h2(pp[t]);
+                        const float scf = static_cast<float>(sp[0]), off = static_cast<float>(sp[1]);
+                        f32x4 part = {0.0f, 0.0f, 0.0f, 0.0f}, xs = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                        for (int d = 0; d < 4; ++d) {
+                            const f16x8 a = *reinterpret_cast<const f16x8*>(xa0 + t * 256u + d * 16);
+                            part = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b_neg, part, 0, 0, 0);
+                            if constexpr (kHasOffset) {
+                                xs = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b_one, xs, 0, 0, 0);
+                            }
+                            part = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, raw8(wq[buf][t][d], mk), part, 0, 0, 0);
+                        }
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            acc[0][r] = __builtin_fmaf(scf, kHasOffset ? __builtin_fmaf(off, xs[r], part[r]) : part[r], acc[0][r]);
+                        }
+                        continue;
+                    }
                     const f16x2 sp = bits_h2(pp[t]);
                     const f16x2 sc = {sp[0], sp[0]};
                     f16x2 ofe = {sp[1], sp[1]}, ofo = ofe;
@@ -519,7 +629,7 @@ __global__ __launch_bounds__(kW * 64) void w4a16_packed_rows_kernel(W4pParams p)
     // compute, hand the activations over, meet the other wavefronts.
     auto step = [&](int buf, uint32_t q) __attribute__((always_inline)) {
         xload(q + 1u);
-        wload((buf + 2) % kBuf, q + 2u);
+        wload((buf + 2) % kRowsBuf, q + 2u);
         if (live && q < nb) {  // uniform over the wavefront
             compute(buf, q);
         }
@@ -625,6 +735,8 @@ extern "C" int ascq_matmul_w4a16_packed(const ascq_w4a16_desc* d, void* y, const
                  "ascq_matmul_w4a16_packed: k %u must be a multiple of group_size %u", d->k, d->group_size);
     ASCQ_REQUIRE(y && x && w_packed && scale, ASCQ_ENULL, "ascq_matmul_w4a16_packed: y / x / w_packed / scale is NULL");
     ASCQ_REQUIRE(!d->has_offset || offset, ASCQ_ENULL, "ascq_matmul_w4a16_packed: offset is NULL");
+    ASCQ_REQUIRE(d->mode == ASCQ_W4A16_PER_WEIGHT || d->mode == ASCQ_W4A16_GROUP_SUM, ASCQ_EINVAL,
+                 "ascq_matmul_w4a16_packed: mode %d is neither ASCQ_W4A16_PER_WEIGHT nor ASCQ_W4A16_GROUP_SUM", d->mode);
     const uint32_t g32 = d->group_size / 32u;
     ASCQ_REQUIRE(d->k % kTileK == 0 && d->n % 8u == 0 && d->group_size % 32u == 0 && (g32 & (g32 - 1u)) == 0, ASCQ_EUNSUPPORTED,
                  "ascq_matmul_w4a16_packed: k must be a multiple of 128, n of 8 and group_size 32 times a power of two "
@@ -643,7 +755,7 @@ extern "C" int ascq_matmul_w4a16_packed(const ascq_w4a16_desc* d, void* y, const
     p.offset = d->has_offset ? static_cast<const uint16_t*>(offset) : nullptr;
     p.n = d->n;
     p.k = d->k;
-    p.mk = NibbleMasks{0x000F000Fu, 0x00F000F0u, 0x64006400u};
+    p.mk = NibbleMasks{0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u};
     p.gs_shift = 0;
     while ((1u << p.gs_shift) < g32) ++p.gs_shift;
     p.slabs = (d->n + kSlabCols - 1u) / kSlabCols;
@@ -659,9 +771,10 @@ extern "C" int ascq_matmul_w4a16_packed(const ascq_w4a16_desc* d, void* y, const
         }
     }
     const uint32_t cus = static_cast<uint32_t>(cached_cus);
-    constexpr uint32_t waves = 8u, batch = 8u;  // 16 wavefronts with batches of 4 tiles measured slower (37 against 30 us)
+    constexpr uint32_t waves = 8u, batch = 4u;  // 16 wavefronts with batches of 4 tiles measured slower (37 against 30 us)
     for (uint32_t m0 = 0; m0 < d->m; m0 += kMaxRows) {
         p.m = d->m - m0 < kMaxRows ? d->m - m0 : kMaxRows;
+        p.m_magic = static_cast<uint32_t>(((1ull << 32) + p.m - 1u) / p.m);
         p.x = static_cast<const uint16_t*>(x) + static_cast<size_t>(m0) * d->k;
         p.y = static_cast<uint16_t*>(y) + static_cast<size_t>(m0) * d->n;
         const uint32_t groups = d->k / d->group_size;
@@ -672,20 +785,21 @@ extern "C" int ascq_matmul_w4a16_packed(const ascq_w4a16_desc* d, void* y, const
             kw = kw < 4u ? 4u : (kw > 8u ? 8u : kw);
             p.par_pitch = groups | 1u;
             const uint32_t grid = (p.slabs + kw - 1u) / kw;
-            auto go = [&](auto has_offset) {
-                constexpr bool kOff = decltype(has_offset)::value;
+            auto go = [&](auto has_offset, auto sum_form) {
+                constexpr bool kOff = decltype(has_offset)::value, kSumF = decltype(sum_form)::value;
                 switch (kw) {
-                    case 4: w4a16_packed_rows_kernel<kOff, 4><<<grid, 4 * 64, 0, st>>>(p); break;
-                    case 5: w4a16_packed_rows_kernel<kOff, 5><<<grid, 5 * 64, 0, st>>>(p); break;
-                    case 6: w4a16_packed_rows_kernel<kOff, 6><<<grid, 6 * 64, 0, st>>>(p); break;
-                    case 7: w4a16_packed_rows_kernel<kOff, 7><<<grid, 7 * 64, 0, st>>>(p); break;
-                    default: w4a16_packed_rows_kernel<kOff, 8><<<grid, 8 * 64, 0, st>>>(p); break;
+                    case 4: w4a16_packed_rows_kernel<kOff, 4, kSumF><<<grid, 4 * 64, 0, st>>>(p); break;
+                    case 5: w4a16_packed_rows_kernel<kOff, 5, kSumF><<<grid, 5 * 64, 0, st>>>(p); break;
+                    case 6: w4a16_packed_rows_kernel<kOff, 6, kSumF><<<grid, 6 * 64, 0, st>>>(p); break;
+                    case 7: w4a16_packed_rows_kernel<kOff, 7, kSumF><<<grid, 7 * 64, 0, st>>>(p); break;
+                    default: w4a16_packed_rows_kernel<kOff, 8, kSumF><<<grid, 8 * 64, 0, st>>>(p); break;
                 }
             };
+            const bool rows_sum = d->mode == ASCQ_W4A16_GROUP_SUM && p.gs_shift >= 2u;
             if (d->has_offset) {
-                go(std::true_type{});
+                rows_sum ? go(std::true_type{}, std::true_type{}) : go(std::true_type{}, std::false_type{});
             } else {
-                go(std::false_type{});
+                rows_sum ? go(std::false_type{}, std::true_type{}) : go(std::false_type{}, std::false_type{});
             }
             continue;
         }
@@ -695,35 +809,54 @@ extern "C" int ascq_matmul_w4a16_packed(const ascq_w4a16_desc* d, void* y, const
         // slabs if the per-wavefront sums would not fit beside them.
         uint32_t spw = (p.slabs + cus - 1u) / cus;
         spw = spw < 1u ? 1u : (spw > kMaxSlabs ? kMaxSlabs : spw);
-        uint32_t pt = 0, xs_wave = 0, par_wave = 0, red_bytes = 0;
+        // the group-sum form needs whole tiles inside one quantisation group; other group sizes keep the per-weight form
+        const bool sum_form = d->mode == ASCQ_W4A16_GROUP_SUM && p.gs_shift >= 2u;
+        uint32_t pt = 0, xs_wave = 0, par_wave = 0, red_bytes = 0, sum_wave = 0, par_cw = 1;
         // entries per column of a wavefront's table: the groups its tiles can touch, rounded up to an odd number
         auto par_rows = [&](uint32_t tiles) { return ((((tiles * 4u - 1u) >> p.gs_shift) + 2u) | 1u); };
         for (;; --spw) {
             const uint32_t all = (p.ktiles + waves - 1u) / waves * waves;
             pt = ((kXBytes / p.m - waves * kRowPad) / (kTileK * 2u)) / waves * waves;
             pt = pt < all ? pt : all;
-            while (pt > waves && (waves * par_rows(pt / waves) * spw * kSlabCols * 4u > kParBytes || par_rows(pt / waves) * 2u * spw > 128u)) pt -= waves;
+            par_cw = 1u;
+            while ((1u << par_cw) < 2u * spw) ++par_cw;
+            const uint32_t par_max_rows = 3u * (64u >> par_cw);  // three fetch rounds of a wavefront
+            while (pt > waves && (waves * par_rows(pt / waves) * spw * kSlabCols * 4u > kParBytes || par_rows(pt / waves) > par_max_rows)) pt -= waves;
             xs_wave = p.m * (pt / waves * kTileK * 2u + kRowPad);
             par_wave = par_rows(pt / waves) * spw * kSlabCols * 4u;
             red_bytes = waves * spw * 4u * p.red_lanes * 4u;
-            if ((waves * par_wave <= kParBytes && par_rows(pt / waves) * 2u * spw <= 128u && waves * (xs_wave + par_wave) + red_bytes <= kPool) || spw == 1u) break;
+            sum_wave = sum_form ? pt / waves * 32u : 0u;
+            if ((waves * par_wave <= kParBytes && par_rows(pt / waves) <= 3u * (64u >> par_cw) && waves * (xs_wave + par_wave + sum_wave) + red_bytes <= kPool) || spw == 1u) break;
         }
-        ASCQ_REQUIRE(waves * par_wave <= kParBytes && par_rows(pt / waves) * 2u * spw <= 128u && waves * (xs_wave + par_wave) + red_bytes <= kPool, ASCQ_EUNSUPPORTED,
+        ASCQ_REQUIRE(waves * par_wave <= kParBytes && par_rows(pt / waves) <= 3u * (64u >> par_cw) && waves * (xs_wave + par_wave + sum_wave) + red_bytes <= kPool, ASCQ_EUNSUPPORTED,
                      "ascq_matmul_w4a16_packed: group_size %u too small for this shape", d->group_size);
         p.slabs_per_wg = spw;
         p.pass_tiles = pt;
-        p.ppr_magic = static_cast<uint32_t>(((1ull << 32) + pt / waves * 16u - 1u) / (pt / waves * 16u));
-        p.par_magic = static_cast<uint32_t>(((1ull << 32) + spw * 2u - 1u) / (spw * 2u));
+        p.par_cw = par_cw;
         p.xs_wave = xs_wave;
         p.par_wave = par_wave;
         p.par_pitch = par_rows(pt / waves);
         p.par_off = waves * xs_wave;
         p.red_off = p.par_off + waves * par_wave;
+        p.sum_off = p.red_off + red_bytes;
+        p.sum_wave = sum_wave;
         const uint32_t grid = (p.slabs + spw - 1u) / spw;
+        auto go = [&](auto has_offset) {
+            constexpr bool kOff = decltype(has_offset)::value;
+            if (!sum_form) {
+                w4a16_packed_kernel<kOff, waves, batch, 0><<<grid, waves * 64u, 0, st>>>(p);
+            } else if (p.m == 1u) {
+                w4a16_packed_kernel<kOff, waves, batch, 1><<<grid, waves * 64u, 0, st>>>(p);
+            } else if (p.m == 2u) {
+                w4a16_packed_kernel<kOff, waves, batch, 2><<<grid, waves * 64u, 0, st>>>(p);
+            } else {
+                w4a16_packed_kernel<kOff, waves, batch, 4><<<grid, waves * 64u, 0, st>>>(p);
+            }
+        };
         if (d->has_offset) {
-            w4a16_packed_kernel<true, waves, batch><<<grid, waves * 64u, 0, st>>>(p);
+            go(std::true_type{});
         } else {
-            w4a16_packed_kernel<false, waves, batch><<<grid, waves * 64u, 0, st>>>(p);
+            go(std::false_type{});
         }
     }
     return launch_status("ascq_matmul_w4a16_packed");

@@ -474,10 +474,23 @@ int ascq_group_matmul_w8a8(const ascq_group_matmul_desc* desc, void* y, const vo
  * workspace: ascq_matmul_w4a16_workspace_size bytes of scratch for the partial sums of the weight streams (contents
  * need not be initialised); calls that share a workspace must not overlap.
  */
+typedef enum ascq_w4a16_mode {
+    ASCQ_W4A16_PER_WEIGHT = 0, /* wdq rounded to half per weight, the formula above: AscendAntiQuant's own arithmetic */
+    /*
+     * Scale and offset applied once per quantisation group to fp32 sums, with no rounding per weight:
+     *   y[i,j] = f16( sum_g f32(scale[g][j]) * ( sum_{k in g} x[i,k] * w[k,j] + f32(offset[g][j]) * sum_{k in g} x[i,k] ) )
+     * The same real-number value as the per-weight form without its 2 * k roundings to half; the two forms differ by
+     * about 3e-4 of the result's magnitude, inside the tolerance of a half output (1 bf16 ulp).  Honoured by
+     * ascq_matmul_w4a16_packed when group_size is a multiple of 128; elsewhere the per-weight form runs.
+     */
+    ASCQ_W4A16_GROUP_SUM = 1
+} ascq_w4a16_mode;
+
 typedef struct ascq_w4a16_desc {
     uint32_t m, n, k;
     uint32_t group_size;
     int32_t has_offset;
+    int32_t mode; /* ascq_w4a16_mode; 0 = the reference's per-weight arithmetic */
 } ascq_w4a16_desc;
 
 int ascq_matmul_w4a16(const ascq_w4a16_desc* desc, void* y, const void* x, const void* w, const void* scale,

@@ -34,7 +34,7 @@ def test_struct_sizes_match_the_header():
     assert C.sizeof(abi.AntiQuantDesc) == 13 * 4
     assert C.sizeof(abi.MatmulDesc) == 11 * 4 + 4 + 8 + 8
     assert C.sizeof(abi.GroupMatmulDesc) == C.sizeof(abi.MatmulDesc) + 8
-    assert C.sizeof(abi.W4A16Desc) == 5 * 4
+    assert C.sizeof(abi.W4A16Desc) == 6 * 4
     assert C.sizeof(abi.W8A16Desc) == 9 * 4
     assert C.sizeof(abi.AntiQuantPolicyDesc) == 14 * 4
     assert C.sizeof(abi.MxDesc) == 8 * 4

@@ -448,6 +448,85 @@ def test_config4_w4a16_decode(m, packed):
     config4_check(y.cpu().numpy(), x, wp, sc, of, d, config4_columns(m, n))
 
 
+def w4_group_sum_gate(got, want):
+    """The bar of a half output whose accumulation order is free, against the oracle's per-weight arithmetic: every
+    element within one bfloat16 ulp of the expected value - where the expected value is small against its row (a
+    cancellation), one bfloat16 ulp of the row's root mean square - and the error of a row as a whole within 1e-3 of the
+    row.  No share of bit-identical elements is asked for: the group-sum form leaves out the per-weight roundings."""
+    g, w = got.astype(np.float64), want.astype(np.float64)
+    rms = np.sqrt(np.mean(w * w, axis=1, keepdims=True))
+    ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(w), rms) + 1e-300)) - 7)
+    assert np.all(np.abs(g - w) <= ulp)
+    assert np.all(np.linalg.norm(g - w, axis=1) <= 1e-3 * np.linalg.norm(w, axis=1))
+
+
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 9, 16, 17, 33])
+@pytest.mark.parametrize("k,n,gs", [(512, 1024, 128), (1024, 544, 64), (384, 512, 128), (2048, 272, 256), (2048, 64, 512),
+                                     (128, 4112, 128), (3200, 144, 128)])
+@pytest.mark.parametrize("offset", ["int", "frac", None])
+def test_w4a16_packed_group_sum_small(m, k, n, gs, offset):
+    """ASCQ_W4A16_GROUP_SUM: scale and offset applied once per quantisation group to fp32 sums.  Same oracle (the
+    per-weight arithmetic), the tolerance of a half output; a group size that is no multiple of 128 runs the per-weight
+    form and must pass the same gate.  Two calls give identical bits."""
+    announce("w4a16 packed group sum", m, k, n, gs, offset)
+    rng = np.random.default_rng(m * 7 + k + n)
+    x, wp, sc, of = w4_case(rng, m, k, n, gs, offset is not None)
+    if offset == "frac":
+        of = (rng.standard_normal((k // gs, n)) * 3).astype(np.float16)
+    w_gpu = ops.pack_weight_w4(to_dev(wp), k, n)
+    xs, scs, ofs = to_dev(x), to_dev(sc), None if of is None else to_dev(of)
+    y1 = torch.zeros((m, n), dtype=torch.float16, device=DEV)
+    y2 = torch.full((m, n), 7.0, dtype=torch.float16, device=DEV)
+    ops.matmul_w4a16_packed(y1, xs, w_gpu, scs, ofs, gs, mode=abi.W4A16_GROUP_SUM)
+    ops.matmul_w4a16_packed(y2, xs, w_gpu, scs, ofs, gs, mode=abi.W4A16_GROUP_SUM)
+    d = abi.W4A16Desc(m=m, n=n, k=k, group_size=gs, has_offset=int(of is not None))
+    w4_group_sum_gate(y1.cpu().numpy(), orc.matmul_w4a16(d, x, wp, sc, of))
+    assert torch.equal(y1, y2)
+
+
+def test_w4a16_packed_group_sum_is_the_real_number_value():
+    """What the group-sum form computes, pinned without the oracle: on inputs whose products and sums are exact in
+    fp32 (integer activations, power-of-two scales, integer offsets) it must give the exact value of
+    sum_g scale_g (sum_k x_k w_k + offset_g sum_k x_k), computed here in Python integers."""
+    m, k, n, gs = 3, 1024, 96, 128
+    announce("w4a16 packed group sum exact", m, k, n)
+    rng = np.random.default_rng(77)
+    x = rng.integers(-4, 5, (m, k)).astype(np.float16)
+    w = rng.integers(-8, 8, (k, n)).astype(np.int8)
+    sc = (2.0 ** rng.integers(-6, -2, (k // gs, n))).astype(np.float16)
+    of = rng.integers(-8, 8, (k // gs, n)).astype(np.float16)
+    y = torch.zeros((m, n), dtype=torch.float16, device=DEV)
+    ops.matmul_w4a16_packed(y, to_dev(x), ops.pack_weight_w4(to_dev(pack_int4(w)), k, n), to_dev(sc), to_dev(of), gs,
+                            mode=abi.W4A16_GROUP_SUM)
+    xg = x.astype(np.int64).reshape(m, k // gs, gs)
+    wg = w.astype(np.int64).reshape(k // gs, gs, n)
+    dots = np.einsum("mgk,gkn->mgn", xg, wg) + xg.sum(axis=2)[:, :, None] * of.astype(np.int64)[None]
+    want = (dots.astype(np.float64) * sc.astype(np.float64)[None]).sum(axis=1)      # exact: multiples of 2^-6 below 2^24
+    assert np.array_equal(y.cpu().numpy(), want.astype(np.float16))
+
+
+@pytest.mark.parametrize("offset", ["int", "frac"])
+@pytest.mark.parametrize("m", [1, 4, 16])
+def test_config4_w4a16_decode_group_sum(m, offset):
+    """Config 4 in the group-sum form: every column at M=1, three slabs of 512 columns at M=4 / 16, integer and
+    fractional offsets, against the unchanged oracle."""
+    announce("config 4 group sum", m, offset)
+    rng = np.random.default_rng(0xC4 + m)
+    k, n, gs = 8192, 28672, 128
+    x, wp, sc, of = w4_case(rng, m, k, n, gs, True)
+    if offset == "frac":
+        of = (rng.standard_normal((k // gs, n)) * 3).astype(np.float16)
+    y = torch.zeros((m, n), dtype=torch.float16, device=DEV)
+    ops.matmul_w4a16_packed(y, to_dev(x), ops.pack_weight_w4(to_dev(wp), k, n), to_dev(sc), to_dev(of), gs,
+                            mode=abi.W4A16_GROUP_SUM)
+    d = abi.W4A16Desc(m=m, n=n, k=k, group_size=gs, has_offset=1)
+    got = y.cpu().numpy()
+    orc.set_threads(16)
+    for c0, c1 in config4_columns(m, n):
+        want = orc.matmul_w4a16(d, x, wp, sc, of, cols=(c0, c1))[:, c0:c1]
+        w4_group_sum_gate(got[:, c0:c1], want)
+
+
 # ------------------------------------------------------------------ W8A16 (Matmul anti-quant path)
 def w8a16_check(got, want, x, out_f32):
     # fp32 accumulation in a different order than the oracle's wide one: error bounded relative to sum |x| |w| (w up
