@@ -136,6 +136,19 @@ __device__ __forceinline__ f16x8 raw8(uint32_t qd, const NibbleMasks& mk)
     __builtin_memcpy(&b, h, 16);
     return b;
 }
+// The same with every nibble moved into bits 4..7 of its half first (three shifts instead of one): all 8 halves are
+// 64 + u = 72 + w.
+__device__ __forceinline__ f16x8 raw8_72(uint32_t qd, const NibbleMasks& mk)
+{
+    uint32_t h[4];
+    h[0] = ((qd << 4) & mk.odd) | mk.exp_odd;
+    h[1] = (qd & mk.odd) | mk.exp_odd;
+    h[2] = ((qd >> 4) & mk.odd) | mk.exp_odd;
+    h[3] = ((qd >> 8) & mk.odd) | mk.exp_odd;
+    f16x8 b;
+    __builtin_memcpy(&b, h, 16);
+    return b;
+}
 constexpr float kBiasEven = 1032.0f, kBiasOdd = 72.0f;  // what raw8 adds to w at k offsets 0 1 4 5 / 2 3 6 7
 
 // kSum = 0: every weight is de-quantised as AscendAntiQuant does it (two roundings to half per weight).
@@ -443,17 +456,18 @@ __global__ __launch_bounds__(kWaves * 64) void w4a16_packed_kernel(W4pParams p)
 // never leave its registers - no reduction in LDS, no second pass.  The wavefronts of a workgroup walk k together and
 // share the activations: chunk c (8 tiles = 1024 k of all m rows) lies in one of two LDS buffers while the next is
 // fetched, one barrier per chunk.  The (scale, offset) pairs of a slab for all of k are staged once per wavefront.
-constexpr int kRowsBuf = 3;
+constexpr int kRowsBuf = 2;              // weight buffers: one batch in flight while the other is computed
 constexpr uint32_t kRowsBatch = 8;          // tiles per batch of weight loads = tiles per activation chunk
 constexpr uint32_t kRowsMaxGroups = 128;    // quantisation groups along k this kernel has LDS for
 constexpr uint32_t kRowsChunkBytes = kRowsBatch * kTileK * 2u;  // bytes of one activation row per chunk
 constexpr uint32_t kRowsPitch = kRowsChunkBytes + kRowPad;
 
-// kSumForm (group_size a multiple of 128): raw weight halves (raw8) on the matrix core, scale and offset applied once
-// per tile to fp32 sums.  What raw8 adds to the weights is taken off by the matrix core as well - a second product of the
-// same activations with the constant operand -c_k accumulates into the same registers - and a third with the operand 1
-// gives the sum of the activations that the offset multiplies: the rows differ from lane to lane here, so a table of
-// sums would cost more vector instructions than the de-quantisation it replaces, while the matrix pipe has room.
+// kSumForm (group_size a multiple of 128): raw weight halves on the matrix core, all of them 72 + w (raw8_72), scale and
+// offset applied once per tile to fp32 sums.  The sum of the activations that both the offset and the 72 multiply comes
+// from the matrix core as well - a second product of the same activations with an operand of ones:
+//   y += scale * (sum_k x_k (w_k + 72) + (offset - 72) * sum_k x_k).
+// The rows differ from lane to lane here, so a table of such sums would cost more vector instructions than the
+// de-quantisation it replaces, while the matrix pipe has room.
 template <bool kHasOffset, uint32_t kW, bool kSumForm>
 __global__ __launch_bounds__(kW * 64) void w4a16_packed_rows_kernel(W4pParams p)
 {
@@ -477,15 +491,13 @@ __global__ __launch_bounds__(kW * 64) void w4a16_packed_rows_kernel(W4pParams p)
 
     NibbleMasks mk = p.mk;
     asm volatile("" : "+v"(mk.exp));
-    f16x8 b_neg, b_one;  // constant B operands of the group-sum form: -(what raw8 adds to each weight), and ones
+    f16x8 b_one;  // the constant B operand of the group-sum form, kept in vector registers
     if constexpr (kSumForm) {
         asm volatile("" : "+v"(mk.exp_odd));
-        const f16x2 ne = {static_cast<half_t>(-kBiasEven), static_cast<half_t>(-kBiasEven)};
-        const f16x2 no = {static_cast<half_t>(-kBiasOdd), static_cast<half_t>(-kBiasOdd)};
         const f16x2 one = {static_cast<half_t>(1.0f), static_cast<half_t>(1.0f)};
-        const f16x2 hn[4] = {ne, no, ne, no}, ho[4] = {one, one, one, one};
-        __builtin_memcpy(&b_neg, hn, 16);
+        const f16x2 ho[4] = {one, one, one, one};
         __builtin_memcpy(&b_one, ho, 16);
+        asm volatile("" : "+v"(b_one));
     }
     const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<u32x4*>(p.wp), 0, static_cast<int>((p.slabs * p.ktiles + kPadTiles) * kTileBytes), 0x00020000);
@@ -585,19 +597,17 @@ __global__ __launch_bounds__(kW * 64) void w4a16_packed_rows_kernel(W4pParams p)
                     if constexpr (kSumForm) {
                         const f16x2 sp = bits_h2(pp[t]);
                         const float scf = static_cast<float>(sp[0]), off = static_cast<float>(sp[1]);
+                        const float off72 = (kHasOffset ? off : 0.0f) - kBiasOdd;
                         f32x4 part = {0.0f, 0.0f, 0.0f, 0.0f}, xs = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                         for (int d = 0; d < 4; ++d) {
                             const f16x8 a = *reinterpret_cast<const f16x8*>(xa0 + t * 256u + d * 16);
-                            part = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b_neg, part, 0, 0, 0);
-                            if constexpr (kHasOffset) {
-                                xs = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b_one, xs, 0, 0, 0);
-                            }
-                            part = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, raw8(wq[buf][t][d], mk), part, 0, 0, 0);
+                            xs = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b_one, xs, 0, 0, 0);
+                            part = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, raw8_72(wq[buf][t][d], mk), part, 0, 0, 0);
                         }
 #pragma unroll
                         for (int r = 0; r < 4; ++r) {
-                            acc[0][r] = __builtin_fmaf(scf, kHasOffset ? __builtin_fmaf(off, xs[r], part[r]) : part[r], acc[0][r]);
+                            acc[0][r] = __builtin_fmaf(scf, __builtin_fmaf(off72, xs[r], part[r]), acc[0][r]);
                         }
                         continue;
                     }
@@ -624,27 +634,27 @@ __global__ __launch_bounds__(kW * 64) void w4a16_packed_rows_kernel(W4pParams p)
         }
     };
 
-    // One step: request the activations of the next chunk, then the weights of the batch after next (in that order:
-    // loads return in order, so the wait for the activations at the end of the step leaves that batch in flight),
-    // compute, hand the activations over, meet the other wavefronts.
+    // One step: request the activations of the next chunk, compute, then request the weights of the batch after next
+    // into the buffer just computed (one batch in flight while one is computed: deeper queues were slower), hand the
+    // activations over - loads return in order, so that wait leaves the batch just requested in flight - and meet the
+    // other wavefronts.
     auto step = [&](int buf, uint32_t q) __attribute__((always_inline)) {
         xload(q + 1u);
-        wload((buf + 2) % kRowsBuf, q + 2u);
         if (live && q < nb) {  // uniform over the wavefront
             compute(buf, q);
         }
+        wload(buf, q + kRowsBuf);
         xstore(q + 1u);
         __syncthreads();
     };
     xload(0);
-    wload(0, 0);
-    wload(1, 1);
+#pragma unroll
+    for (int b = 0; b < kRowsBuf; ++b) wload(b, b);
     xstore(0);
     __syncthreads();
-    for (uint32_t q = 0; q < nb; q += 3u) {
-        step(0, q);
-        step(1, q + 1u);
-        step(2, q + 2u);
+    for (uint32_t q = 0; q < nb; q += kRowsBuf) {
+#pragma unroll
+        for (int b = 0; b < kRowsBuf; ++b) step(b, q + b);
     }
 
     // ---- result row 4 (lane / 16) + r of column lane % 16: one rounding to half
