@@ -279,6 +279,7 @@ class Matmul:
         self.desc = abi.MatmulDesc(m=m, n=n, k=k, trans_a=int(trans_a), trans_b=int(trans_b), out_dtype=abi.I32,
                                    quant_mode=abi.MM_QUANT_NONE, scale_format=abi.MM_SCALE_U64)
         self.a = self.b = self.bias = self.quant = self.tok = None
+        self.packed = False
         self._ws_by_stream = {}   # scratch per stream handle: calls of one object on two streams may overlap
 
     def set_tensor_a(self, a):
@@ -287,7 +288,15 @@ class Matmul:
     def set_tensor_b(self, b, nz=False):
         """b: int8 [k, n] row-major, or with nz=True the fractal layout [n/32, k/16, 16, 32] (CubeFormat::NZ)."""
         self.b = b
+        self.packed = False
         self.desc.b_format = abi.MM_B_NZ if nz else abi.MM_B_ND
+
+    def set_tensor_b_packed(self, w_packed):
+        """b in the layout of pack_weight_w8 (packed once, when the weights are loaded): iterate_all then runs the
+        one-launch kernel for few activation rows, which needs no scratch."""
+        self.b = w_packed
+        self.packed = True
+        self.desc.b_format = abi.MM_B_ND
 
     def set_bias(self, bias):
         """int32 bias: initial value of the accumulator; float32 / bfloat16 bias: added after dequantisation."""
@@ -336,6 +345,10 @@ class Matmul:
     def iterate_all(self, c):
         self.desc.out_dtype = _dt(c)
         lib = load_library()
+        if self.packed:
+            check(lib.ascq_matmul_w8a8_packed(C.byref(self.desc), _ptr(c), _ptr(self.a), _ptr(self.b), _ptr(self.bias),
+                                              _ptr(self.quant), _ptr(self.tok), _stream()))
+            return c
         need = C.c_size_t(0)
         check(lib.ascq_matmul_w8a8_workspace_size(C.byref(self.desc), C.byref(need)))
         if need.value:
@@ -472,6 +485,16 @@ def matmul_w4a16(y, x, w_packed, scale, offset=None, group_size=128, workspace=N
     check(lib.ascq_matmul_w4a16(C.byref(d), _ptr(y), _ptr(x), _ptr(w_packed), _ptr(scale), _ptr(offset),
                                 _ptr(workspace), workspace.numel() * workspace.element_size(), _stream()))
     return y
+
+
+def pack_weight_w8(b, k, n, trans_b=False):
+    """int8 weights [k, n] ([n, k] with trans_b) -> the GPU-native packed layout of Matmul.set_tensor_b_packed."""
+    lib = load_library()
+    need = C.c_size_t(0)
+    check(lib.ascq_pack_weight_w8_size(k, n, C.byref(need)))
+    out = torch.empty(need.value, dtype=torch.uint8, device=b.device)
+    check(lib.ascq_pack_weight_w8(_ptr(b), _ptr(out), k, n, int(trans_b), _stream()))
+    return out
 
 
 def pack_weight_w4(w_nd, k, n):

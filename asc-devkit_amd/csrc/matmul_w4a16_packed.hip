@@ -285,6 +285,11 @@ __global__ __launch_bounds__(kWaves * 64) void w4a16_packed_kernel(W4pParams p)
         }
 #pragma unroll
         for (int b = 0; b < kBuf; ++b) load(b);
+        // Loads return in order: once at most the weight loads just issued are outstanding, the activations have landed
+        // in LDS.  The compiler does not count direct-to-LDS loads issued in a loop; told here, with a wait it
+        // understands, it neither reads the LDS early nor waits for the weights in front of every LDS read.
+        __builtin_amdgcn_s_waitcnt(((kBuf * kBatch) & 15u) | (((kBuf * kBatch) >> 4) << 14) | (7u << 4) | (15u << 8));
+        asm volatile("" ::: "memory");
         if (pt0 == 0u && lane < rl) {  // sums of this wavefront per slab, kept in LDS between passes
             for (uint32_t s = 0; s < nslabs * 4u; ++s) red[s * rl + lane] = 0.0f;
         }

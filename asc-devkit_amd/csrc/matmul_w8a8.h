@@ -206,5 +206,9 @@ int launch_gemm_dma_skinny(GemmParams& p, void* workspace, size_t workspace_byte
 // Few rows, B as [n][k]: whole columns per workgroup, one launch, no workspace (matmul_w8a8_nk.hip).
 bool gemm_nk_supported(const GemmParams& p);
 int launch_gemm_nk(const GemmParams& p, hipStream_t st);
+// Few rows on weights packed by ascq_pack_weight_w8 (p.b): whole columns per workgroup, one launch, no workspace
+// (matmul_w8a8_packed.hip).
+bool gemm_packed_supported(const GemmParams& p);
+int launch_gemm_packed(const GemmParams& p, hipStream_t st);
 
 }  // namespace ascq

@@ -785,6 +785,34 @@ extern "C" int ascq_matmul_w8a8(const ascq_matmul_desc* d, void* c, const void* 
     return d->trans_b ? launch_gemm<TileLT, true, false>(p, st) : launch_gemm<TileL, false, false>(p, st);
 }
 
+// ref: include/adv_api/matmul/matmul.h:175-185 (the same Matmul with SetQuantScalar / SetQuantVector); the weights in the
+// layout of ascq_pack_weight_w8, the counterpart of the packing the reference does offline for its own L1 / L0 layout
+// (examples/.../quant_group_matmul_high_performance/scripts/gen_data.py:62-64)
+extern "C" int ascq_matmul_w8a8_packed(const ascq_matmul_desc* d, void* c, const void* a, const void* w_packed,
+                                       const void* bias, const void* quant_vector, const void* tok_scale, void* stream)
+{
+    ASCQ_REQUIRE(d != nullptr, ASCQ_ENULL, "ascq_matmul_w8a8_packed: desc is NULL");
+    int rc = validate_mm(d, "ascq_matmul_w8a8_packed", c, a, w_packed, bias, quant_vector, tok_scale);
+    if (rc != ASCQ_OK) {
+        return rc;
+    }
+    ASCQ_REQUIRE(!d->trans_a && d->b_format == ASCQ_MM_B_ND, ASCQ_EUNSUPPORTED,
+                 "ascq_matmul_w8a8_packed: a is [m, k] and the weights are in the packed layout (no trans_a, no NZ)");
+    ASCQ_REQUIRE(d->activation != ASCQ_MM_ACT_SWIGLU, ASCQ_EUNSUPPORTED,
+                 "ascq_matmul_w8a8_packed: SwiGLU is not available on packed weights (use ascq_matmul_w8a8)");
+    GemmParams p{};
+    p.a = static_cast<const int8_t*>(a);
+    p.b = static_cast<const int8_t*>(w_packed);
+    p.m = d->m;
+    p.n = d->n;
+    p.k = d->k;
+    p.epi = make_epi(d, c, bias, quant_vector, tok_scale);
+    ASCQ_REQUIRE(d->k % 64u == 0, ASCQ_EUNSUPPORTED, "ascq_matmul_w8a8_packed: k = %u must be a multiple of 64", d->k);
+    ASCQ_REQUIRE(aligned16(a) && aligned16(w_packed), ASCQ_EALIGN, "ascq_matmul_w8a8_packed: a and w_packed must be 16-byte aligned");
+    ASCQ_REQUIRE(gemm_packed_supported(p), ASCQ_EUNSUPPORTED, "ascq_matmul_w8a8_packed: the packed weights must stay below 2 GiB");
+    return launch_gemm_packed(p, static_cast<hipStream_t>(stream));
+}
+
 // ref: include/adv_api/matmul/matmul_tilingdata.h:21-72 (TCubeTiling, the reference's host-side plan of a matmul)
 extern "C" int ascq_matmul_w8a8_plan(const ascq_matmul_desc* d, const void* c, const void* a, const void* b,
                                      const void* bias, const void* quant_vector, const void* tok_scale,

@@ -1,0 +1,292 @@
+// int8 matmul for few activation rows (decode, small batches) on weights pre-packed for this GPU: one launch, no
+// workspace, one flat sweep over the weights.
+//
+// Packed layout (ascq_pack_weight_w8): the [k, n] matrix is cut into slabs of 16 columns and tiles of 64 k; a tile of a
+// slab is 1 KiB and the tiles of a slab, then the slabs, follow each other in memory.  Inside a tile lane l of a
+// wavefront owns 16 bytes: column l % 16 of the slab, k = 16 (l / 16) .. + 15 - the B operand of
+// v_mfma_i32_16x16x64_i8 as it lies.  Columns past n and k past the end hold 0; 16 tiles of zeros follow the last
+// slab.  So a tile costs one fully coalesced 16-byte load per lane and one matrix instruction, for up to 16 activation
+// rows at the cost of one, and nothing else: no vector ALU work in the loop.
+//
+// A workgroup owns whole slabs (whole columns: nothing is added across workgroups), its eight wavefronts split k.
+// A wavefront moves its share of the activations (its k range of every row) into its part of the LDS once, by
+// direct-to-LDS loads, and streams its tiles in batches of 4 with one batch in flight while one is computed (a compute
+// unit keeps about 64 KiB of loads in flight whatever is asked of it; deeper queues only make wavefronts wait at the
+// issue of their loads).  Operand row i of a lane reads activation row i % rows, so there are no zero rows to
+// materialise.  The eight partial sums of a column meet in LDS (integers: exact in any order) and go through the
+// element-wise epilogue of the int8 matmul.
+#include "matmul_w8a8.h"
+
+namespace ascq {
+namespace {
+
+constexpr uint32_t kPkCols = 16, kPkTileK = 64, kPkTileBytes = 1024;
+constexpr uint32_t kPkPadTiles = 16;   // tiles of zeros behind the last slab (a batch may read on)
+constexpr uint32_t kPkWaves = 8, kPkBatch = 4, kPkMaxSlabs = 8, kPkMaxRows = 16;
+constexpr int kPkBuf = 2;              // register buffers: one batch in flight while the other is computed
+constexpr uint32_t kPkRowPad = 16;     // bytes added to a staged activation row: rows start 4 banks apart
+constexpr uint32_t kPkXBytes = 88 * 1024;  // LDS for the staged activations of a workgroup (the partial sums take 64 KiB)
+constexpr uint32_t kPkPastEnd = 0x7FFFFFF0u;
+constexpr int kPkNt = 2;               // cache policy of the weight loads: non-temporal (read once per call)
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef __attribute__((address_space(1))) const void* gptr_t;
+
+struct PackedParams {
+    const int8_t* a;       // [m, k], first row of this pass
+    const i32x4* wp;       // packed weights
+    uint32_t m0, rows;     // first row and rows of this pass (1 .. 16)
+    uint32_t n, k;
+    uint32_t slabs, ktiles;
+    uint32_t tpw;          // tiles of k per wavefront
+    uint32_t rows_magic;   // ceil(2^32 / rows)
+    EpiParams epi;
+};
+
+// Workgroups are dealt to the 8 XCDs round-robin; in this order the workgroups of an XCD own neighbouring slabs.
+__device__ __forceinline__ uint32_t pk_xcd_order(uint32_t wg, uint32_t wgs)
+{
+    return (wgs & 7u) == 0u ? (wg & 7u) * (wgs >> 3) + (wg >> 3) : wg;
+}
+
+__global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_kernel(PackedParams p)
+{
+    __shared__ __attribute__((aligned(16))) char XS[kPkXBytes];
+    __shared__ int32_t RED[kPkWaves][kPkMaxSlabs][4][64];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t lc = lane & 15u, lq = lane >> 4;
+    // slabs [s0, s1) of this workgroup: the slabs are dealt out as evenly as they divide
+    const uint32_t wg = pk_xcd_order(blockIdx.x, gridDim.x);
+    const uint32_t s0 = static_cast<uint32_t>(static_cast<uint64_t>(wg) * p.slabs / gridDim.x);
+    const uint32_t s1 = static_cast<uint32_t>(static_cast<uint64_t>(wg + 1u) * p.slabs / gridDim.x);
+    const uint32_t nslabs = s1 - s0;
+    const uint32_t ta = min(wave * p.tpw, p.ktiles), tb = min(ta + p.tpw, p.ktiles), cnt = tb - ta;
+    const uint32_t pitch = p.tpw * kPkTileK + kPkRowPad;
+    char* const xs = XS + wave * (p.rows * pitch);
+
+    // ---- this wavefront's share of the activations: up to 1 KiB of a row per instruction, straight into LDS
+    {
+        const uint32_t row_pieces = cnt * (kPkTileK / 16u);
+        for (uint32_t r = 0; r < p.rows; ++r) {
+            const int8_t* src = p.a + static_cast<size_t>(p.m0 + r) * p.k + ta * kPkTileK + lane * 16u;
+            for (uint32_t c0 = 0; c0 < row_pieces; c0 += 64u) {
+                if (c0 + lane < row_pieces) {
+                    __builtin_amdgcn_global_load_lds((gptr_t)(src + c0 * 16u), (lds_ptr_t)(xs + r * pitch + c0 * 16u), 16, 0, 0);
+                }
+            }
+        }
+    }
+    const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<i32x4*>(p.wp), 0, static_cast<int>((p.slabs * p.ktiles + kPkPadTiles) * kPkTileBytes), 0x00020000);
+    // operand row i reads row i % rows; + tile * 64
+    const uint32_t x_lane = (lc - __umulhi(lc, p.rows_magic) * p.rows) * pitch + lq * 16u;
+
+    // ---- batches of kPkBatch tiles that never straddle a slab: batch q = (slab q / nb, tiles ta + (q % nb) kPkBatch ...)
+    const uint32_t nb = (cnt + kPkBatch - 1u) / kPkBatch;
+    const uint32_t batches = nb * nslabs;
+    i32x4 wq[kPkBuf][kPkBatch];
+    uint32_t l_slab = s0, l_b = 0, l_q = 0;
+    bool l_done = batches == 0u;
+    auto load = [&](int buf) __attribute__((always_inline)) {
+        // every load is issued, so the waits the compiler inserts count exactly; once every batch has been requested the
+        // per-lane offset lies past the end of the buffer and the loads move no data.  A short last batch reads on into
+        // the next tiles or the padding: valid memory, not computed.
+        const uint32_t l_w = l_done ? kPkPastEnd : lane * 16u;
+        const uint32_t base = (l_slab * p.ktiles + ta + l_b * kPkBatch) * kPkTileBytes;  // scalar
+#pragma unroll
+        for (uint32_t t = 0; t < kPkBatch; ++t) {
+            wq[buf][t] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, l_w, base + t * kPkTileBytes, kPkNt));
+        }
+        if (l_q + 1u < batches) {  // uniform
+            ++l_q;
+            if (++l_b == nb) {
+                l_b = 0;
+                ++l_slab;
+            }
+        } else {
+            l_done = true;
+        }
+    };
+#pragma unroll
+    for (int b = 0; b < kPkBuf; ++b) load(b);
+    // Loads return in order: once at most the weight loads just issued are outstanding, the activations have landed in
+    // LDS.  (The compiler does not count direct-to-LDS loads issued in a loop; it is told here, with a wait it
+    // understands, so that it neither reads the LDS early nor waits for the weights in front of every LDS read.)
+    __builtin_amdgcn_s_waitcnt(((kPkBuf * kPkBatch) & 15) | (((kPkBuf * kPkBatch) >> 4) << 14) | (7 << 4) | (15 << 8));
+    asm volatile("" ::: "memory");
+
+    i32x4 acc = {0, 0, 0, 0};
+    uint32_t c_slab = 0, c_b = 0, c_q = 0;
+    auto compute = [&](int buf) __attribute__((always_inline)) {
+        if (c_q >= batches) {
+            return;  // uniform
+        }
+        const uint32_t t0 = c_b * kPkBatch;             // first tile of the batch, relative to ta
+        const uint32_t live = min(kPkBatch, cnt - t0);
+        const char* xa0 = xs + x_lane + t0 * kPkTileK;
+#pragma unroll
+        for (uint32_t t = 0; t < kPkBatch; ++t) {
+            if (t < live) {  // uniform
+                const i32x4 a = *reinterpret_cast<const i32x4*>(xa0 + t * kPkTileK);
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, wq[buf][t], acc, 0, 0, 0);
+            }
+        }
+        ++c_q;
+        if (++c_b == nb) {  // the slab is done: register i of lane l is row 4 (l / 16) + i, column l % 16
+#pragma unroll
+            for (int i = 0; i < 4; ++i) RED[wave][c_slab][i][lane] = acc[i];
+            acc = i32x4{0, 0, 0, 0};
+            c_b = 0;
+            ++c_slab;
+        }
+    };
+    for (uint32_t q = 0; q < batches; q += kPkBuf) {
+#pragma unroll
+        for (int b = 0; b < kPkBuf; ++b) {
+            compute(b);
+            load(b);
+        }
+    }
+    if (batches == 0u) {  // a wavefront without tiles (k shorter than 8 tiles) contributes zeros
+        for (uint32_t s = 0; s < nslabs; ++s) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) RED[wave][s][i][lane] = 0;
+        }
+    }
+    __syncthreads();
+
+    // ---- the eight partial sums of every element, then the element-wise epilogue
+    const EpiParams& e = p.epi;
+    for (uint32_t s = wave; s < nslabs; s += kPkWaves) {
+        const uint32_t col = (s0 + s) * kPkCols + lc;
+        if (col >= p.n) {
+            continue;
+        }
+        const ChannelQ q = load_channel_q(e, col);
+        const float bp = load_bias_post(e, col);
+        const int32_t bias_pre = e.bias_kind == ASCQ_MM_BIAS_I32_PRE ? static_cast<const int32_t*>(e.bias)[col] : 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t row_in_pass = 4u * lq + static_cast<uint32_t>(i);
+            if (row_in_pass >= p.rows) {
+                continue;
+            }
+            int32_t sum = RED[0][s][i][lane];
+#pragma unroll
+            for (uint32_t wv = 1; wv < kPkWaves; ++wv) sum += RED[wv][s][i][lane];
+            sum += bias_pre;
+            const uint32_t row = p.m0 + row_in_pass;
+            const float tok = e.has_tok ? e.tok_scale[row] : 1.0f;
+            dispatch_out(e, [&](auto tag) { epilogue_store<decltype(tag)::value>(e, row, col, sum, q, tok, bp); });
+        }
+    }
+}
+
+// [k, n] (or [n, k] with trans) -> packed; one thread per lane of a tile.
+__global__ __launch_bounds__(256) void pack_w8_kernel(const int8_t* __restrict__ w, i32x4* __restrict__ out, uint32_t k,
+                                                      uint32_t n, uint32_t slabs, uint32_t ktiles, int trans)
+{
+    const size_t total = static_cast<size_t>(slabs) * ktiles * 64u;
+    const size_t i = static_cast<size_t>(blockIdx.x) * 256u + threadIdx.x;
+    if (i >= total + kPkPadTiles * 64u) {
+        return;
+    }
+    i32x4 v = {0, 0, 0, 0};
+    if (i < total) {
+        const uint32_t lane = static_cast<uint32_t>(i & 63u);
+        const size_t tile_id = i >> 6;
+        const uint32_t slab = static_cast<uint32_t>(tile_id / ktiles), tile = static_cast<uint32_t>(tile_id % ktiles);
+        const uint32_t col = slab * kPkCols + (lane & 15u), kq = lane >> 4;
+#pragma unroll
+        for (uint32_t d = 0; d < 4; ++d) {
+            uint32_t word = 0;
+#pragma unroll
+            for (uint32_t b = 0; b < 4; ++b) {
+                const uint32_t kk = tile * kPkTileK + kq * 16u + d * 4u + b;
+                uint32_t byte = 0;
+                if (kk < k && col < n) {
+                    byte = static_cast<uint8_t>(trans ? w[static_cast<size_t>(col) * k + kk] : w[static_cast<size_t>(kk) * n + col]);
+                }
+                word |= byte << (8u * b);
+            }
+            v[d] = static_cast<int32_t>(word);
+        }
+    }
+    out[i] = v;
+}
+
+}  // namespace
+
+bool gemm_packed_supported(const GemmParams& p)
+{
+    return p.k % kPkTileK == 0 && aligned16(p.a) && aligned16(p.b) &&
+           (static_cast<uint64_t>((p.n + kPkCols - 1u) / kPkCols) * (p.k / kPkTileK) + kPkPadTiles) * kPkTileBytes < (1ull << 31);
+}
+
+// p.b: the packed weights.  Any m: up to 16 rows per pass over the weights.
+int launch_gemm_packed(const GemmParams& p, hipStream_t st)
+{
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
+        cus = 256;
+    }
+    PackedParams q{};
+    q.wp = reinterpret_cast<const i32x4*>(p.b);
+    q.a = p.a;
+    q.n = p.n;
+    q.k = p.k;
+    q.slabs = (p.n + kPkCols - 1u) / kPkCols;
+    q.ktiles = p.k / kPkTileK;
+    q.tpw = (q.ktiles + kPkWaves - 1u) / kPkWaves;
+    q.epi = p.epi;
+    // one workgroup per compute unit when the slabs allow it, at most kPkMaxSlabs slabs per workgroup
+    uint32_t grid = q.slabs < static_cast<uint32_t>(cus) ? q.slabs : static_cast<uint32_t>(cus);
+    if ((q.slabs + grid - 1u) / grid > kPkMaxSlabs) {
+        grid = (q.slabs + kPkMaxSlabs - 1u) / kPkMaxSlabs;
+    }
+    // rows per pass: 16, fewer when k is so long that the staged activations of 16 rows would not fit the LDS
+    uint32_t pass_rows = kPkXBytes / (kPkWaves * (q.tpw * kPkTileK + kPkRowPad));
+    pass_rows = pass_rows > kPkMaxRows ? kPkMaxRows : pass_rows;
+    if (pass_rows == 0u) {
+        return fail(ASCQ_EUNSUPPORTED, "ascq_matmul_w8a8_packed: k = %u is too long for the staged activations", p.k);
+    }
+    for (uint32_t m0 = 0; m0 < p.m; m0 += pass_rows) {
+        q.m0 = m0;
+        q.rows = p.m - m0 < pass_rows ? p.m - m0 : pass_rows;
+        q.rows_magic = static_cast<uint32_t>(((1ull << 32) + q.rows - 1u) / q.rows);
+        if (plan_note(ASCQ_MM_KERNEL_STREAM, 16, 16 * ((q.slabs + grid - 1u) / grid), kPkTileK, grid, 1,
+                      kPkXBytes + kPkWaves * kPkMaxSlabs * 1024u, 0)) {
+            return ASCQ_OK;
+        }
+        gemm_packed_kernel<<<grid, kPkWaves * 64u, 0, st>>>(q);
+    }
+    return launch_status("ascq_matmul_w8a8_packed");
+}
+
+}  // namespace ascq
+
+using namespace ascq;
+
+extern "C" int ascq_pack_weight_w8_size(uint32_t k, uint32_t n, size_t* bytes)
+{
+    ASCQ_REQUIRE(bytes != nullptr, ASCQ_ENULL, "ascq_pack_weight_w8_size: bytes is NULL");
+    ASCQ_REQUIRE(k > 0 && n > 0, ASCQ_EINVAL, "ascq_pack_weight_w8_size: k, n must be positive");
+    *bytes = (static_cast<size_t>((n + kPkCols - 1u) / kPkCols) * ((k + kPkTileK - 1u) / kPkTileK) + kPkPadTiles) * kPkTileBytes;
+    return ASCQ_OK;
+}
+
+extern "C" int ascq_pack_weight_w8(const void* w, void* packed, uint32_t k, uint32_t n, int32_t trans_b, void* stream)
+{
+    ASCQ_REQUIRE(w && packed, ASCQ_ENULL, "ascq_pack_weight_w8: w / packed is NULL");
+    ASCQ_REQUIRE(k > 0 && n > 0, ASCQ_EINVAL, "ascq_pack_weight_w8: k, n must be positive");
+    ASCQ_REQUIRE(aligned16(packed), ASCQ_EALIGN, "ascq_pack_weight_w8: packed must be 16-byte aligned");
+    ASCQ_REQUIRE(w != packed, ASCQ_EINVAL, "ascq_pack_weight_w8: packed must not be w");
+    const uint32_t slabs = (n + kPkCols - 1u) / kPkCols, ktiles = (k + kPkTileK - 1u) / kPkTileK;
+    const size_t lanes = (static_cast<size_t>(slabs) * ktiles + kPkPadTiles) * 64u;
+    ASCQ_REQUIRE((lanes + 255u) / 256u < (1ull << 31), ASCQ_EINVAL, "ascq_pack_weight_w8: matrix too large");
+    pack_w8_kernel<<<static_cast<uint32_t>((lanes + 255u) / 256u), 256, 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<const int8_t*>(w), static_cast<i32x4*>(packed), k, n, slabs, ktiles, trans_b != 0);
+    return launch_status("ascq_pack_weight_w8");
+}

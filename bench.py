@@ -63,10 +63,10 @@ def main():
                          "runs are also measured at the sustained clock (0 disables)")
     ap.add_argument("--quick", action="store_true", help="headline + W4A16 GEMV only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="run a single workload: w8a8 | w4a16 | w4a16_nd | w4a16_m4 | w4a16_m16 | w4a16_nd_m4 | w4a16_nd_m16 | "
+    ap.add_argument("--only", default="", help="run a single workload: w8a8 | w4a16 | w4a16_per_weight | w4a16_per_weight_m4 | w4a16_per_weight_m16 | w4a16_nd | w4a16_m4 | w4a16_m16 | w4a16_nd_m4 | w4a16_nd_m16 | "
                          "w8a8_m1 | w8a8_m8 | w8a8_m16 | w8a8_m128 | w8a8_m512 | w8a8_m8192 | w8a8_nk_m1 | w8a8_nk_m16 | w8a8_nk_m128 | w8a16_m1 | w8a16_m16 | w8a16_nk_m1 | "
                          "w8a16_nk_m16 | w8a16_m2048 | w8a16_nk_m2048 | quant | dequant | antiquant | group | group_example | mx_fp4 | mx_fp4_e1m2 | mx_fp8 (a W4A16 name without _nd "
-                         "is the packed-weight path; _nk: weights kept as [n, k])")
+                         "is the packed-weight path, in the group-sum form unless it says per_weight; _nk: weights kept as [n, k])")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch one device-to-device copy of 1 GiB: the known-size kernel that calibrates the "
                          "FETCH_SIZE / WRITE_SIZE counters when this command runs under rocprofv3 --pmc")
@@ -76,6 +76,21 @@ def main():
               "or experts without any communication, so N GPUs are N independent copies of this run).",
               file=sys.stderr)
         sys.exit(2)
+
+    # The stand-alone probe of the machine's ceilings runs first, in a process of its own, before this process has
+    # touched the GPU.
+    ceilings = None
+    if not (args.quick or args.only):
+        import subprocess
+        exe = os.path.join(ROOT, "asc-devkit_amd", "lib", "machine_probe")
+        if not os.path.exists(exe):
+            ceilings = {"error": "asc-devkit_amd/lib/machine_probe is not built"}
+        else:
+            try:
+                r = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+                ceilings = json.loads(r.stdout) if r.returncode == 0 else {"error": r.stderr.strip()[-200:]}
+            except Exception as e:     # the probe is evidence, not part of the measurement: report and go on
+                ceilings = {"error": str(e)}
 
     import numpy as np
     import torch
@@ -205,9 +220,11 @@ def main():
                 "ops": flops, "bytes": bytes_, "tensors": (x, w, cs)}
 
     # ------------------------------------------------------------------ W4A16 decode (config 4)
-    def w4a16(M, steps, warmup, sets=4, packed=False):
+    def w4a16(M, steps, warmup, sets=4, packed=False, mode=abi.W4A16_PER_WEIGHT):
         """packed: the weights in the layout of ascq_pack_weight_w4 (packed once, outside the timed region) and the
-        one-launch kernel; otherwise the [k, n / 2] layout and the stream + sum kernels."""
+        one-launch kernel; otherwise the [k, n / 2] layout and the stream + sum kernels.  mode (packed only):
+        abi.W4A16_PER_WEIGHT = AscendAntiQuant's two roundings to half per weight, abi.W4A16_GROUP_SUM = scale and offset
+        applied once per quantisation group to fp32 sums."""
         K, N, gs = 8192, 28672, 128
         xs = torch.randn((M, K), device=dev, generator=gen).to(torch.float16)
         ws = [torch.randint(0, 256, (K, N // 2), dtype=torch.uint8, device=dev, generator=gen) for _ in range(sets)]
@@ -219,7 +236,7 @@ def main():
         def step(i, starts, stops):
             j = i % sets
             if packed:
-                bracket(starts, stops, lambda: ops.matmul_w4a16_packed(y, xs, wps[j], sc[j], of[j], gs))
+                bracket(starts, stops, lambda: ops.matmul_w4a16_packed(y, xs, wps[j], sc[j], of[j], gs, mode=mode))
             else:
                 bracket(starts, stops, lambda: ops.matmul_w4a16(y, xs, ws[j], sc[j], of[j], gs))
 
@@ -368,29 +385,20 @@ def main():
     def strip(d):
         return {k: v for k, v in d.items() if k != "tensors"}
 
-    def machine_ceilings():
-        """Runs the stand-alone probe (its own process, before this one launches anything large) and returns its JSON."""
-        import subprocess
-        exe = os.path.join(ROOT, "asc-devkit_amd", "lib", "machine_probe")
-        if not os.path.exists(exe):
-            return {"error": "asc-devkit_amd/lib/machine_probe is not built"}
-        try:
-            r = subprocess.run([exe], capture_output=True, text=True, timeout=120)
-            return json.loads(r.stdout) if r.returncode == 0 else {"error": r.stderr.strip()[-200:]}
-        except Exception as e:     # the probe is evidence, not part of the measurement: report and go on
-            return {"error": str(e)}
-
-    ceilings = None if args.quick or args.only else machine_ceilings()
     only = args.only
     if only and only != "w8a8":
-        fn = {"w4a16": lambda: w4a16(1, args.steps, args.warmup, packed=True),
+        gsum = abi.W4A16_GROUP_SUM
+        fn = {"w4a16": lambda: w4a16(1, args.steps, args.warmup, packed=True, mode=gsum),
+              "w4a16_per_weight": lambda: w4a16(1, args.steps, args.warmup, packed=True),
+              "w4a16_per_weight_m4": lambda: w4a16(4, args.steps, args.warmup, packed=True),
+              "w4a16_per_weight_m16": lambda: w4a16(16, args.steps, args.warmup, packed=True),
               "w4a16_nd": lambda: w4a16(1, args.steps, args.warmup),
               "group_example": lambda: group_example(args.steps, args.warmup),
               "mx_fp4": lambda: mx("fp4", args.steps, args.warmup),
               "mx_fp4_e1m2": lambda: mx("fp4_e1m2", args.steps, args.warmup),
               "mx_fp8": lambda: mx("fp8", args.steps, args.warmup),
-              "w4a16_m4": lambda: w4a16(4, args.steps, args.warmup, packed=True),
-              "w4a16_m16": lambda: w4a16(16, args.steps, args.warmup, packed=True),
+              "w4a16_m4": lambda: w4a16(4, args.steps, args.warmup, packed=True, mode=gsum),
+              "w4a16_m16": lambda: w4a16(16, args.steps, args.warmup, packed=True, mode=gsum),
               "w4a16_nd_m4": lambda: w4a16(4, args.steps, args.warmup),
               "w4a16_nd_m16": lambda: w4a16(16, args.steps, args.warmup),
               "w8a8_m1": lambda: w8a8(1, args.steps, args.warmup, sets=7),
@@ -469,21 +477,29 @@ def main():
 
     # The other workloads run a bounded number of steps so that the whole file finishes in about a minute.
     side_steps, side_warmup = max(100, min(args.steps, 500)), min(args.warmup, 50)
-    gemv = w4a16(1, side_steps, side_warmup, packed=True)
+    gemv = w4a16(1, side_steps, side_warmup, packed=True, mode=abi.W4A16_GROUP_SUM)
+    gemv_pw = w4a16(1, side_steps, side_warmup, packed=True)
     gemv_nd = w4a16(1, side_steps, side_warmup)
     out["w4a16_gemv"] = {"metric": "w4a16_decode_gemv_hbm_gbs_m1_k8192_n28672", "value": gemv["gbs"], "unit": "GB/s",
-                         "workload": "BASELINE configs[3] at M=1, weights pre-packed by ascq_pack_weight_w4 (outside "
+                         "workload": "BASELINE configs[3] at M=1 in the mode ASCQ_W4A16_GROUP_SUM (scale and offset "
+                                     "applied once per quantisation group to fp32 sums; fp16 output within one bf16 ulp "
+                                     "of the per-weight arithmetic), weights pre-packed by ascq_pack_weight_w4 (outside "
                                      "the timed region), 4 rotating weight sets (500 MB > Infinity Cache)",
                          "ms_per_step": gemv["ms_per_step"],
-                         "roofline": {"bound": "hbm", "kernel": "w4a16_packed_kernel<offset, 8, 8> (one launch)",
+                         "roofline": {"bound": "hbm", "kernel": "w4a16_packed_kernel<offset, 8, 4, group sum> (one launch)",
                                       "achieved": gemv["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                       "frac": gemv["gbs"] / PEAK_HBM_GBS, "traffic": GEMV_PACKED_TRAFFIC_BYTES,
                                       "avg_kernel_ms": gemv["kernel_ms"], "bytes_per_launch": gemv["bytes"]},
+                         "per_weight_mode": {"kernel": "w4a16_packed_kernel<offset, 8, 4, per weight> (one launch)",
+                                             "workload": "the same GEMV in the default mode ASCQ_W4A16_PER_WEIGHT: "
+                                                         "AscendAntiQuant's two roundings to half per weight",
+                                             "avg_kernel_ms": gemv_pw["kernel_ms"], "gbs": gemv_pw["gbs"],
+                                             "hbm_frac": gemv_pw["gbs"] / PEAK_HBM_GBS},
                          "nd_layout": {"kernel": "w4a16_gemv_kernel<1, offset> + stream_sum_kernel<1>",
                                        "workload": "the same GEMV on the reference's [k, n / 2] weight layout",
                                        "avg_kernel_ms": gemv_nd["kernel_ms"], "gbs": gemv_nd["gbs"],
                                        "hbm_frac": gemv_nd["gbs"] / PEAK_HBM_GBS, "traffic": GEMV_TRAFFIC_BYTES}}
-    del gemv_nd
+    del gemv_nd, gemv_pw
     torch.cuda.empty_cache()
 
     if not args.quick:
@@ -516,9 +532,14 @@ def main():
             r = strip(w4a16(M, s2, w2))
             others[f"w4a16_m{M}"] = {"kernel_ms": r["kernel_ms"], "gbs": r["gbs"], "hbm_frac": r["gbs"] / PEAK_HBM_GBS}
             torch.cuda.empty_cache()
-            r = strip(w4a16(M, s2, w2, packed=True))
+            r = strip(w4a16(M, s2, w2, packed=True, mode=abi.W4A16_GROUP_SUM))
             others[f"w4a16_packed_m{M}"] = {"kernel_ms": r["kernel_ms"], "gbs": r["gbs"],
-                                            "hbm_frac": r["gbs"] / PEAK_HBM_GBS}
+                                            "hbm_frac": r["gbs"] / PEAK_HBM_GBS, "mode": "ASCQ_W4A16_GROUP_SUM"}
+            torch.cuda.empty_cache()
+            r = strip(w4a16(M, s2, w2, packed=True))
+            others[f"w4a16_packed_per_weight_m{M}"] = {"kernel_ms": r["kernel_ms"], "gbs": r["gbs"],
+                                                       "hbm_frac": r["gbs"] / PEAK_HBM_GBS,
+                                                       "mode": "ASCQ_W4A16_PER_WEIGHT"}
             torch.cuda.empty_cache()
         for M in (1, 16):
             r = w8a16(M, s2, w2)

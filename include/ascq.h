@@ -358,6 +358,25 @@ int ascq_matmul_w8a8(const ascq_matmul_desc* desc, void* c, const void* a, const
 int ascq_matmul_w8a8_workspace_size(const ascq_matmul_desc* desc, size_t* bytes);
 
 /*
+ * The same matmul for few activation rows (decode, small batches) on weights pre-packed for this GPU, the step the
+ * reference does offline for its own L1 / L0 layout (examples/.../quant_group_matmul_high_performance/scripts/
+ * gen_data.py:62-64 packs ND -> NZ before the kernel runs).  ascq_pack_weight_w8 turns B int8 [k, n] (trans_b: [n, k])
+ * into ascq_pack_weight_w8_size(k, n) bytes: slabs of 16 columns, each one contiguous run of tiles of 64 k (1 KiB: lane l
+ * of a wavefront owns column l % 16 and the 16 consecutive bytes k 16 (l / 16) .. + 15); columns past n and k past the
+ * end hold 0, and 16 tiles of zeros follow the last slab.
+ * ascq_matmul_w8a8_packed computes exactly what ascq_matmul_w8a8 computes (same descriptor, epilogues and outputs;
+ * desc.trans_b is ignored, desc.trans_a and ASCQ_MM_ACT_SWIGLU are not supported) in one launch with no workspace: a
+ * workgroup owns whole columns, its wavefronts split k, and integer partial sums are exact in any order.  The weights
+ * are read once per 16 activation rows, so the call suits m up to a few dozen; requires k % 64 == 0 and a, w_packed
+ * 16-byte aligned.
+ * ref: include/adv_api/matmul/matmul.h:175-185 (the Matmul object and its quant epilogue)
+ */
+int ascq_pack_weight_w8_size(uint32_t k, uint32_t n, size_t* bytes);
+int ascq_pack_weight_w8(const void* b, void* w_packed, uint32_t k, uint32_t n, int32_t trans_b, void* stream);
+int ascq_matmul_w8a8_packed(const ascq_matmul_desc* desc, void* c, const void* a, const void* w_packed, const void* bias,
+                            const void* quant_vector, const void* tok_scale, void* stream);
+
+/*
  * Matmul<int4b_t A, int4b_t B, C>: the same descriptor, epilogues and outputs as ascq_matmul_w8a8 with both operands
  * packed two int4 per byte, even element in the low nibble: A [m, k/2] bytes, B [k, n/2] bytes ([n, k/2] with
  * trans_b).  trans_a is not supported (the reference's rule for an int4 A), b_format is ND, k is even, n is even

@@ -141,6 +141,111 @@ def test_config3_w8a8_linear_weights_as_n_k(m):
     assert np.array_equal(bits(c8), oracle_mm(d8, a, wt, None, words))
 
 
+def run_mm_packed(m, n, k, a, b, *, out, bias=None, quant=None, tok=None, trans_b=False, act=abi.MM_ACT_NONE,
+                  scalar=None):
+    """run_mm on weights packed by ops.pack_weight_w8 (from [k, n], or from [n, k] with trans_b); the descriptor it
+    returns describes the same matmul on the unpacked [k, n] weights, for the oracle."""
+    mm = ops.Matmul(m, n, k)
+    mm.set_tensor_a(to_dev(a))
+    mm.set_tensor_b_packed(ops.pack_weight_w8(to_dev(b), k, n, trans_b))
+    if bias is not None:
+        mm.set_bias(to_dev(bias[0], bias[1]))
+    if quant is not None:
+        mm.set_quant_vector(to_dev(quant))
+    if scalar is not None:
+        mm.set_quant_scalar(scalar)
+    if tok is not None:
+        mm.set_token_scale(to_dev(tok))
+    mm.set_activation(act)
+    c = torch.zeros((m, n), dtype=out, device=DEV)
+    mm.iterate_all(c)
+    torch.cuda.synchronize()
+    return c, mm.desc
+
+
+def w8_packed_reference(w, k, n):
+    """The packed int8 layout restated in numpy: slabs of 16 columns, tiles of 64 k, lane l of a tile owns column
+    l % 16 and the 16 bytes k 16 (l / 16) .. + 15; zeros past n and k, 16 tiles of zeros behind the last slab."""
+    slabs, ktiles = (n + 15) // 16, (k + 63) // 64
+    full = np.zeros((ktiles * 64, slabs * 16), dtype=np.int8)
+    full[:k, :n] = w
+    t = full.reshape(ktiles, 4, 16, slabs, 16)            # tile, k quarter, byte, slab, column
+    body = np.ascontiguousarray(t.transpose(3, 0, 1, 4, 2)).reshape(-1)   # slab, tile, k quarter, column, byte
+    return np.concatenate([body, np.zeros(16 * 1024, dtype=np.int8)]).view(np.uint8)
+
+
+@pytest.mark.parametrize("k,n", [(64, 16), (128, 40), (200, 1040), (1024, 272)])
+def test_pack_weight_w8_layout(k, n):
+    announce("pack w8", k, n)
+    rng = np.random.default_rng(k + n)
+    w = rand_i8(rng, (k, n))
+    want = w8_packed_reference(w, k, n)
+    assert np.array_equal(ops.pack_weight_w8(to_dev(w), k, n).cpu().numpy(), want)
+    assert np.array_equal(ops.pack_weight_w8(to_dev(np.ascontiguousarray(w.T)), k, n, trans_b=True).cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("m", [1, 2, 3, 5, 8, 16, 17, 33])
+@pytest.mark.parametrize("n,k", [(16, 64), (48, 128), (1040, 512), (272, 4096), (96, 8192), (32, 16384), (2064, 192)])
+def test_w8a8_packed_small(m, n, k):
+    """The one-launch kernel on packed weights computes what ascq_matmul_w8a8 computes: int32 accumulators and the
+    dequantising epilogues bit for bit against the oracle on the unpacked weights.  k of one tile (seven wavefronts
+    without work), column tails, more rows than a pass, k long enough for several batches per slab."""
+    announce("w8a8 packed", m, n, k)
+    rng = np.random.default_rng(m * 31 + n + k)
+    a, b = rand_i8(rng, (m, k)), rand_i8(rng, (k, n))
+    c, desc = run_mm_packed(m, n, k, a, b, out=torch.int32)
+    assert np.array_equal(c.cpu().numpy(), a.astype(np.int64) @ b.astype(np.int64))
+    cs = rng.uniform(1e-4, 1e-2, n).astype(np.float32)
+    ts = rng.uniform(1e-2, 1e-1, m).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    c, desc = run_mm_packed(m, n, k, a, np.ascontiguousarray(b.T), out=torch.bfloat16, bias=(bias, None), quant=cs, tok=ts,
+                            trans_b=True)
+    assert np.array_equal(bits(c), oracle_mm(desc, a, b, (bias, None), cs, ts))
+    # requantised int8 output from uint64 words, int32 bias ahead of the dequantisation, FasterGelu to half
+    words = (cs * 50).astype(np.float32).view(np.uint32).astype(np.uint64) | (np.uint64(1) << np.uint64(46))
+    bias_i = rng.integers(-1000, 1000, n).astype(np.int32)
+    c8, d8 = run_mm_packed(m, n, k, a, b, out=torch.int8, bias=(bias_i, None), quant=words)
+    assert np.array_equal(bits(c8), oracle_mm(d8, a, b, (bias_i, None), words))
+    cg, dg = run_mm_packed(m, n, k, a, b, out=torch.float16, scalar=1e-3, act=abi.MM_ACT_FASTER_GELU)
+    assert max_ulp(bits(cg), oracle_mm(dg, a, b).view(np.uint16), "f16") <= 1
+
+
+@pytest.mark.parametrize("m", [1, 16])
+def test_config3_w8a8_linear_packed(m):
+    """Config 3's decode sizes on packed weights: per-token quantisation on the GPU, one launch for the matmul, bf16
+    output bit-exact against the oracle."""
+    announce("config 3 packed", m)
+    rng = np.random.default_rng(0xC3 + m)
+    k, n = 4096, 11008
+    x = orc.f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32))
+    w = rand_i8(rng, (k, n))
+    cs = rng.uniform(1e-4, 1e-2, n).astype(np.float32)
+    q, ts = ops.dynamic_quant_per_token(to_dev(x, "bf16"))
+    wq, wts = orc.dynamic_quant_per_token(abi.BF16, x)
+    assert np.array_equal(q.cpu().numpy(), wq) and np.array_equal(ts.cpu().numpy(), wts)
+    c, desc = run_mm_packed(m, n, k, wq, w, out=torch.bfloat16, quant=cs, tok=wts)
+    assert np.array_equal(bits(c), oracle_mm(desc, wq, w, None, cs, wts))
+
+
+def test_w8a8_packed_rejects():
+    lib = abi.load_library()
+    t = torch.zeros(1 << 16, dtype=torch.int8, device=DEV)
+    c = torch.zeros(1 << 12, dtype=torch.int32, device=DEV)
+
+    def call(**kw):
+        d = abi.MatmulDesc(m=1, n=64, k=128, out_dtype=abi.I32, quant_mode=abi.MM_QUANT_NONE, scale_format=abi.MM_SCALE_U64)
+        for key, v in kw.items():
+            setattr(d, key, v)
+        return lib.ascq_matmul_w8a8_packed(C.byref(d), C.c_void_p(c.data_ptr()), C.c_void_p(t.data_ptr()),
+                                           C.c_void_p(t.data_ptr()), None, None, None, None)
+
+    assert call() == abi.OK
+    assert call(k=100) == abi.EUNSUPPORTED          # k % 64
+    assert call(trans_a=1) == abi.EUNSUPPORTED
+    assert call(b_format=abi.MM_B_NZ) != abi.OK
+    torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize("m", [48, 128, 300, 512])
 def test_config3_w8a8_mid_m_both_weight_layouts(m):
     """Config 3 between the decode sizes and the large tiles: 128 x 128 direct-to-LDS tiles, K split four ways for one
