@@ -64,7 +64,7 @@ def main():
     ap.add_argument("--quick", action="store_true", help="headline + W4A16 GEMV only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="run a single workload: w8a8 | w4a16 | w4a16_per_weight | w4a16_per_weight_m4 | w4a16_per_weight_m16 | w4a16_nd | w4a16_m4 | w4a16_m16 | w4a16_nd_m4 | w4a16_nd_m16 | "
-                         "w8a8_m1 | w8a8_m8 | w8a8_m16 | w8a8_m128 | w8a8_m512 | w8a8_m8192 | w8a8_nk_m1 | w8a8_nk_m16 | w8a8_nk_m128 | w8a16_m1 | w8a16_m16 | w8a16_nk_m1 | "
+                         "w8a8_m1 | w8a8_m8 | w8a8_m16 | w8a8_m128 | w8a8_m512 | w8a8_m8192 | w8a8_packed_m1 | w8a8_packed_m8 | w8a8_packed_m16 | w8a8_nk_m1 | w8a8_nk_m16 | w8a8_nk_m128 | w8a16_m1 | w8a16_m16 | w8a16_nk_m1 | "
                          "w8a16_nk_m16 | w8a16_m2048 | w8a16_nk_m2048 | quant | dequant | antiquant | group | group_example | mx_fp4 | mx_fp4_e1m2 | mx_fp8 (a W4A16 name without _nd "
                          "is the packed-weight path, in the group-sum form unless it says per_weight; _nk: weights kept as [n, k])")
     ap.add_argument("--copy-probe", action="store_true",
@@ -152,11 +152,12 @@ def main():
         torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------ W8A8 linear (config 3)
-    def w8a8(M, steps, warmup, sets=1, settle=None, zero=False, gauss=False, b_nk=False):
+    def w8a8(M, steps, warmup, sets=1, settle=None, zero=False, gauss=False, b_nk=False, packed=False):
         """`sets` > 1 rotates the weights over several copies (together larger than the Infinity Cache) so that the
         weight-bound small-M cases read them from HBM.  The weights are uniform over [-127, 127] unless `gauss`: then
         they are normal weights quantised per output channel by their absolute maximum, as a checkpoint's would be.
-        b_nk: the weights are kept as [n, k] (isTransposeB)."""
+        b_nk: the weights are kept as [n, k] (isTransposeB).  packed: the weights in the layout of ascq_pack_weight_w8
+        (packed once, outside the timed region) and the one-launch kernel for few rows."""
         K, N = 4096, 11008
         x = torch.randn((M, K), device=dev, generator=gen).to(torch.bfloat16)
         if gauss:
@@ -178,9 +179,12 @@ def main():
         c = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
         mms = []
         for wj in ws:
-            mm = ops.Matmul(M, N, K, False, b_nk)
+            mm = ops.Matmul(M, N, K, False, b_nk and not packed)
             mm.set_tensor_a(q)
-            mm.set_tensor_b(wj)
+            if packed:
+                mm.set_tensor_b_packed(ops.pack_weight_w8(wj, K, N, b_nk))
+            else:
+                mm.set_tensor_b(wj)
             mm.set_quant_vector(cs)
             mm.set_token_scale(ts)
             mms.append(mm)
@@ -408,6 +412,9 @@ def main():
               "w8a8_m8192": lambda: w8a8(8192, max(20, args.steps // 10), 5, settle=40),
               "w8a8_nk_m128": lambda: w8a8(128, args.steps, args.warmup, sets=7, b_nk=True),
               "w8a8_m128": lambda: w8a8(128, args.steps, args.warmup, sets=7),
+              "w8a8_packed_m1": lambda: w8a8(1, args.steps, args.warmup, sets=7, packed=True),
+              "w8a8_packed_m8": lambda: w8a8(8, args.steps, args.warmup, sets=7, packed=True),
+              "w8a8_packed_m16": lambda: w8a8(16, args.steps, args.warmup, sets=7, packed=True),
               "w8a8_nk_m1": lambda: w8a8(1, args.steps, args.warmup, sets=7, b_nk=True),
               "w8a8_nk_m16": lambda: w8a8(16, args.steps, args.warmup, sets=7, b_nk=True),
               "w8a16_nk_m1": lambda: w8a16(1, args.steps, args.warmup, b_nk=True),
@@ -516,6 +523,13 @@ def main():
             others[f"w8a8_m{M}"] = {"gemm_kernel_ms": r["gemm_kernel_ms"], "gemm_tops": r["gemm_tops"],
                                     "gemm_gbs": r["gemm_gbs"], "hbm_frac": r["gemm_gbs"] / PEAK_HBM_GBS,
                                     "mfma_frac": r["gemm_tops"] / PEAK_INT8_TOPS}
+        for M in (1, 8, 16):
+            r = strip(w8a8(M, s2, w2, sets=7, packed=True))
+            others[f"w8a8_packed_m{M}"] = {"gemm_kernel_ms": r["gemm_kernel_ms"], "gemm_gbs": r["gemm_gbs"],
+                                           "hbm_frac": r["gemm_gbs"] / PEAK_HBM_GBS,
+                                           "note": "weights pre-packed by ascq_pack_weight_w8 (outside the timed "
+                                                   "region): one launch, no workspace"}
+            torch.cuda.empty_cache()
         r = strip(w8a8(8192, 40, 5, settle=40))
         others["w8a8_m8192"] = {"gemm_kernel_ms": r["gemm_kernel_ms"], "gemm_tops": r["gemm_tops"],
                                 "mfma_frac": r["gemm_tops"] / PEAK_INT8_TOPS,
