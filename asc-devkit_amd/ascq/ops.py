@@ -429,13 +429,14 @@ def linear_w8a8_dynamic(c, x, weight, channel_scale, bias=None, activation=abi.M
     return c
 
 
-def linear_w8a8_dynamic_noalloc(c, x, weight, channel_scale, bias=None, activation=abi.MM_ACT_NONE, trans_b=False):
+def linear_w8a8_dynamic_noalloc(c, x, weight, channel_scale, bias=None, activation=abi.MM_ACT_NONE, trans_b=False,
+                                act_beta=1.0):
     """linear_w8a8_dynamic on the library's built-in scratch buffer: no workspace, no allocation.  Calls that overlap
     on one GPU share that buffer and race."""
     m, k = x.shape
-    n = c.shape[1]
+    n = weight.shape[0] if trans_b else weight.shape[1]    # with SwiGLU c has n / 2 columns
     d = abi.MatmulDesc(m=m, n=n, k=k, trans_b=int(trans_b), out_dtype=_dt(c), quant_mode=abi.MM_QUANT_VECTOR,
-                       scale_format=abi.MM_SCALE_F32, activation=activation)
+                       scale_format=abi.MM_SCALE_F32, activation=activation, act_beta=act_beta)
     if bias is not None:
         d.bias_kind = abi.MM_BIAS_F32_POST if bias.dtype == torch.float32 else abi.MM_BIAS_BF16_POST
     check(load_library().ascq_linear_w8a8_dynamic_noalloc(C.byref(d), _dt(x), _ptr(c), _ptr(x), _ptr(weight), _ptr(bias),

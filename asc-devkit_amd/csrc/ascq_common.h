@@ -37,6 +37,25 @@ inline int launch_status(const char* what)
     return ASCQ_OK;
 }
 
+// Compute units of the current device, looked up once per device (the first 64 devices are cached; any thread may
+// call this).  256 when the query fails.
+inline uint32_t device_compute_units()
+{
+    static int cached[64];
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+        return 256u;
+    }
+    n = __atomic_load_n(&cached[dev], __ATOMIC_RELAXED);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+            n = 256;
+        }
+        __atomic_store_n(&cached[dev], n, __ATOMIC_RELAXED);
+    }
+    return static_cast<uint32_t>(n);
+}
+
 // Plan recording (ascq_matmul_w8a8_plan): while a plan is being recorded on this thread, every launch site of the int8
 // matmul describes the launch it would make and returns true, and the caller then skips the launch.  The first note of
 // a call fills the main fields; later ones (the kernel that sums partial results) only add to `launches`;

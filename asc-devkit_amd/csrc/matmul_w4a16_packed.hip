@@ -788,17 +788,7 @@ extern "C" int ascq_matmul_w4a16_packed(const ascq_w4a16_desc* d, void* y, const
     while ((1u << p.gs_shift) < g32) ++p.gs_shift;
     p.slabs = (d->n + kSlabCols - 1u) / kSlabCols;
     p.ktiles = d->k / kTileK;
-    static int cached_cus = 0;  // compute units of the device first used (one GPU per process in this library's use)
-    if (cached_cus == 0) {
-        int dev = 0, n_cu = 0;
-        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess &&
-            n_cu > 0) {
-            cached_cus = n_cu;
-        } else {
-            cached_cus = 256;
-        }
-    }
-    const uint32_t cus = static_cast<uint32_t>(cached_cus);
+    const uint32_t cus = device_compute_units();
     constexpr uint32_t waves = 8u, batch = 4u;  // 16 wavefronts with batches of 4 tiles measured slower (37 against 30 us)
     for (uint32_t m0 = 0; m0 < d->m; m0 += kMaxRows) {
         p.m = d->m - m0 < kMaxRows ? d->m - m0 : kMaxRows;

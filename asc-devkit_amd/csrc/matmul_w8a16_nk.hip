@@ -462,11 +462,7 @@ int launch_w8a16_nk(const void* x, const void* w, const void* scale, const void*
     p.out_f32 = out_f32 ? 1u : 0u;
     p.scale_bits = scale_bits;
     p.offset_bits = offset_bits;
-    int dev = 0, cus = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
-        cus = 256;
-    }
+    const int cus = static_cast<int>(device_compute_units());
     const uint32_t n_groups = (n + 15u) / 16u;
     // one workgroup per compute unit: two, three or seven times as many smaller ones measured slower at every m
     // (49.7 against 52.7-57.8 us at m = 1, k = 8192, n = 28672)

@@ -34,7 +34,7 @@ struct GemmParams {
 struct ChannelQ {
     float s;
     int off9;
-    int sgn;
+    int ctl;  // bit 0: saturate the 8-bit result as signed; bit 1: pre-shift on; bits [5:2]: the pre-shift
 };
 
 __device__ __forceinline__ ChannelQ load_channel_q(const EpiParams& e, size_t col)
@@ -57,7 +57,8 @@ __device__ __forceinline__ ChannelQ load_channel_q(const EpiParams& e, size_t co
     if (e.scale_format == ASCQ_MM_SCALE_U64) {
         lo &= 0xFFFFE000u;  // the fixpipe reads sign, 8 exponent and 10 mantissa bits
         q.off9 = static_cast<int>((w >> 37) & 0x1FF);
-        q.sgn = static_cast<int>((w >> 46) & 1);
+        // sign bit 46 -> bit 0; mode-control bit 36 -> bit 1; shift bits [35:32] -> bits [5:2]
+        q.ctl = static_cast<int>((w >> 46) & 1) | static_cast<int>((w >> 35) & 2) | static_cast<int>((w >> 30) & 0x3C);
     }
     q.s = __uint_as_float(lo);
     return q;
@@ -83,10 +84,30 @@ __device__ __forceinline__ float swiglu(float src0, float src1, float beta)
     return src0 * (src1 / d);
 }
 
+// The accumulator as the float the scale multiplies.  A quant word with the mode-control bit set shifts the accumulator
+// right (arithmetically) first and saturates the result: to the half range with one rounding to half for half outputs
+// (ref: fixpipe_l0c2gm/scripts/gen_data_s322f16.py:84-90), to the int16 range for 8-bit outputs
+// (gen_data_s322s8.py:84-86); other outputs take the shifted value as it is.
+__device__ __forceinline__ float accumulator_value(int32_t acc, int ctl, int out_dtype)
+{
+    if (ctl & 2) {
+        const int32_t sh = acc >> ((ctl >> 2) & 15);
+        if (out_dtype == ASCQ_F16) {
+            const float f = fminf(fmaxf(static_cast<float>(sh), -65504.0f), 65504.0f);  // exact below 2^24, monotonic above
+            return static_cast<float>(static_cast<_Float16>(f));
+        }
+        if (out_dtype == ASCQ_I8) {
+            return static_cast<float>(min(max(sh, -32768), 32767));
+        }
+        return static_cast<float>(sh);
+    }
+    return static_cast<float>(acc);
+}
+
 // v of one accumulator before any activation: channel scale, token scale, post-dequant bias.
 __device__ __forceinline__ float epilogue_value(const EpiParams& e, int32_t acc, const ChannelQ& q, float tok, float bias_post)
 {
-    float v = static_cast<float>(acc) * q.s;
+    float v = accumulator_value(acc, q.ctl, e.out_dtype) * q.s;
     if (e.has_tok) {
         v = v * tok;
     }
@@ -118,7 +139,7 @@ __device__ __forceinline__ void epilogue_store(const EpiParams& e, size_t row, s
     if constexpr (kOut < 0) {
         static_cast<int32_t*>(e.c)[idx] = acc;
     } else {
-        float v = static_cast<float>(acc) * q.s;
+        float v = accumulator_value(acc, q.ctl, kOut) * q.s;
         if (e.has_tok) {
             v = v * tok;
         }
@@ -137,7 +158,7 @@ __device__ __forceinline__ void epilogue_store(const EpiParams& e, size_t row, s
         } else {  // int8 / uint8 requantisation
             float r = fminf(fmaxf(__builtin_rintf(v), -256.0f), 255.0f);
             int t = ((v != v) ? 0 : static_cast<int>(r)) + q.off9;
-            t = q.sgn ? min(max(t, -128), 127) : min(max(t, 0), 255);
+            t = (q.ctl & 1) ? min(max(t, -128), 127) : min(max(t, 0), 255);
             static_cast<uint8_t*>(e.c)[idx] = static_cast<uint8_t>(t);
         }
     }

@@ -531,11 +531,6 @@ int validate_mm(const ascq_matmul_desc* d, const char* who, const void* c, const
                      "%s: int8 output (requantisation) needs the uint64 quant parameter format", who);
         if (d->quant_mode == ASCQ_MM_QUANT_VECTOR) {
             ASCQ_REQUIRE(qv != nullptr, ASCQ_ENULL, "%s: quant vector is NULL", who);
-        } else if (d->scale_format == ASCQ_MM_SCALE_U64) {
-            // the fixpipe's pre-shift form (mode-control bit 36, shift in bits [35:32]) is not implemented: computing
-            // without the shift would be silently wrong
-            ASCQ_REQUIRE(((d->quant_scalar >> 36) & 1u) == 0, ASCQ_EUNSUPPORTED,
-                         "%s: quant word with mode-control bit 36 set (pre-shift by bits [35:32]) is not supported", who);
         }
     }
     ASCQ_REQUIRE(d->bias_kind == ASCQ_MM_BIAS_NONE || bias != nullptr, ASCQ_ENULL, "%s: bias is NULL", who);
@@ -632,9 +627,17 @@ extern "C" int ascq_matmul_w8a8_workspace_size(const ascq_matmul_desc* d, size_t
 {
     ASCQ_REQUIRE(d != nullptr && bytes != nullptr, ASCQ_ENULL, "ascq_matmul_w8a8_workspace_size: NULL argument");
     *bytes = 0;
-    if (d->activation == ASCQ_MM_ACT_SWIGLU && d->quant_mode != ASCQ_MM_QUANT_NONE) {
+    // The size is that for operands aligned to 16 bytes; it cannot see the pointers.  (A SwiGLU call whose misaligned
+    // operands keep it off the tile kernel names the size it needs in its error.)
+    GemmParams shape{};
+    shape.a = shape.b = reinterpret_cast<const int8_t*>(uintptr_t{16});
+    shape.m = d->m;
+    shape.n = d->n;
+    shape.k = d->k;
+    if (d->activation == ASCQ_MM_ACT_SWIGLU && d->quant_mode != ASCQ_MM_QUANT_NONE &&
+        !swiglu_in_tile_kernel(d, shape, shape.a, shape.b)) {
         // Shapes outside the large tile kernel keep their int32 accumulators [m][n] in the workspace, behind the
-        // scratch of the matmul that produces them.  (The size does not depend on the pointers: it is the bound.)
+        // scratch of the matmul that produces them.
         const ascq_matmul_desc r = raw_accumulator_desc(d);
         size_t inner = 0;
         const int rc = ascq_matmul_w8a8_workspace_size(&r, &inner);
@@ -1115,7 +1118,7 @@ extern "C" int ascq_group_matmul_w8a8(const ascq_group_matmul_desc* g, void* y, 
     ASCQ_REQUIRE(!p.b_nz, ASCQ_EUNSUPPORTED, "ascq_group_matmul_w8a8: fractal (NZ) weights need the tile kernel's shape");
     ASCQ_REQUIRE(d->activation != ASCQ_MM_ACT_SWIGLU, ASCQ_EUNSUPPORTED,
                  "ascq_group_matmul_w8a8: SwiGLU needs the tile kernel's shape (k %% 128 == 0, n %% 16 == 0)");
-    typedef TileL T;
+    typedef TileM T;  // 128 x 256: the 256-row tile spills here (the group bookkeeping on top of 256 accumulator registers)
     // every group adds at most one partial tile along M
     p.tiles_m = (d->m + T::BM - 1) / T::BM + g->groups;
     p.tiles_n = (d->n + T::BN - 1) / T::BN;

@@ -455,6 +455,48 @@ __device__ __forceinline__ void gemm_dma_tile_at(const GemmParams& p, const Tile
             }
         };
         if constexpr (kOut == ASCQ_BF16 || kOut == ASCQ_F16) {
+            // Quant words that shift the accumulator first (mode-control bit) are rare: when any column of the
+            // wavefront carries one, a compact epilogue that reads every choice at run time serves the whole
+            // wavefront, element by element, and the specialised ones below stay as they are.
+            if (e.scale_format == ASCQ_MM_SCALE_U64 && e.quant_mode != ASCQ_MM_QUANT_NONE &&
+                __builtin_amdgcn_ballot_w64(((q[0].ctl | q[TJ - 1].ctl) & 2) != 0) != 0) {
+                const bool odd = (lane & 1u) != 0;
+#pragma unroll 1
+                for (int i = 0; i < TI; ++i) {
+                    const uint32_t lbase = (wm * TI + i) * 32u + 4u * g;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const uint32_t lrow_t = lbase + 8u * (r >> 2) + (r & 3);
+                        const uint32_t row = row0 + lrow_t;
+                        const float tok = TS[lrow_t];
+                        float v[TJ];
+#pragma unroll
+                        for (int j = 0; j < TJ; ++j) {
+                            v[j] = epilogue_value(e, acc[i][j][r] + bias_pre[j], q[j], tok, bias_post[j]);
+                        }
+                        if (e.activation == ASCQ_MM_ACT_SWIGLU) {
+                            const float recv = __int_as_float(__builtin_amdgcn_mov_dpp(
+                                __float_as_int(odd ? v[0] : v[TJ - 1]), 0xB1, 0xF, 0xF, true));  // lane ^ 1
+                            const float o = swiglu(odd ? recv : v[0], odd ? v[TJ - 1] : recv, e.act_beta);
+                            const uint32_t col = odd ? colw + 32u + (lrow - 1u) : colw + lrow;
+                            if (row < row_end && col < N) {
+                                static_cast<uint16_t*>(e.c)[static_cast<size_t>(row) * e.ldc + (col >> 1)] =
+                                    static_cast<uint16_t>(to_bits16<kOut>(o));
+                            }
+                            continue;
+                        }
+#pragma unroll
+                        for (int j = 0; j < TJ; ++j) {
+                            if (cvalid[j] && row < row_end) {
+                                const float o = e.activation == ASCQ_MM_ACT_FASTER_GELU ? faster_gelu(v[j]) : v[j];
+                                static_cast<uint16_t*>(e.c)[static_cast<size_t>(row) * e.ldc + colw + j * 32u + lrow] =
+                                    static_cast<uint16_t>(to_bits16<kOut>(o));
+                            }
+                        }
+                    }
+                }
+                return;
+            }
             const bool bias_post_on = e.bias_kind >= ASCQ_MM_BIAS_F32_POST;
             const bool gelu_on = e.activation == ASCQ_MM_ACT_FASTER_GELU;
             if (e.activation == ASCQ_MM_ACT_SWIGLU) {
@@ -724,24 +766,6 @@ __global__ __launch_bounds__(256) void splitk_sum_epilogue_kernel(GemmParams p)
 }
 
 }  // namespace
-
-// Compute units of the current device (cached for the first 64 devices).
-static uint32_t device_compute_units()
-{
-    static int cached[64];
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
-        return 256u;
-    }
-    n = __atomic_load_n(&cached[dev], __ATOMIC_RELAXED);
-    if (n == 0) {
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
-            n = 256;
-        }
-        __atomic_store_n(&cached[dev], n, __ATOMIC_RELAXED);
-    }
-    return static_cast<uint32_t>(n);
-}
 
 bool gemm_dma_supported(const GemmParams& p)
 {

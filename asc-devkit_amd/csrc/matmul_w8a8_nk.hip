@@ -170,11 +170,7 @@ bool gemm_nk_supported(const GemmParams& p)
 // Any m; 32 rows per pass over the weights (16 in a last pass of at most 16 rows).
 int launch_gemm_nk(const GemmParams& p, hipStream_t st)
 {
-    int dev = 0, cus = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
-        cus = 256;
-    }
+    const int cus = static_cast<int>(device_compute_units());
     const uint32_t n_groups = (p.n + 15u) / 16u;
     // Column groups per workgroup: one workgroup per compute unit when several rows share the weights (every
     // workgroup reads all of a once); with at most 4 rows a is negligible and three times as many, smaller workgroups

@@ -227,11 +227,7 @@ bool gemm_packed_supported(const GemmParams& p)
 // p.b: the packed weights.  Any m: up to 16 rows per pass over the weights.
 int launch_gemm_packed(const GemmParams& p, hipStream_t st)
 {
-    int dev = 0, cus = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
-        cus = 256;
-    }
+    const int cus = static_cast<int>(device_compute_units());
     PackedParams q{};
     q.wp = reinterpret_cast<const i32x4*>(p.b);
     q.a = p.a;

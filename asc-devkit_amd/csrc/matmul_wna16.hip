@@ -67,6 +67,7 @@ struct WnParams {
     // W8A16 only
     uint32_t out_f32;                  // y is float instead of half
     uint32_t scale_bits, offset_bits;  // per-tensor parameters as half bits, used when scale == nullptr
+    uint32_t w_nk;                     // the weights are [n, k] (generic kernel only)
 };
 
 __device__ __forceinline__ f16x2 bits_to_h2(uint32_t b)
@@ -957,7 +958,8 @@ __global__ __launch_bounds__(kThreads) void w8a16_generic_kernel(WnParams p)
             p.has_offset ? static_cast<half_t>(half_bits_to_f32(p.scale ? p.offset[col] : p.offset_bits)) : half_t(0);
         float s = 0.0f;
         for (uint32_t kk = 0; kk < p.k; ++kk) {
-            half_t h = static_cast<half_t>(static_cast<float>(static_cast<int8_t>(p.w[static_cast<size_t>(kk) * p.n + col])));
+            const size_t at = p.w_nk ? col * p.k + kk : static_cast<size_t>(kk) * p.n + col;
+            half_t h = static_cast<half_t>(static_cast<float>(static_cast<int8_t>(p.w[at])));
             if (p.has_offset) {
                 h = h + offset;
             }
@@ -1216,11 +1218,16 @@ extern "C" int ascq_matmul_w8a16(const ascq_w8a16_desc* d, void* y, const void* 
     p.k = d->k;
     p.has_offset = d->has_offset ? 1u : 0u;
     p.out_f32 = d->out_dtype == ASCQ_F32 ? 1u : 0u;
+    p.w_nk = d->trans_b ? 1u : 0u;
+    if (d->trans_b && (d->k % 128u != 0 || !w8a16_nk_supported(d->k, x, w))) {
+        // k off the kernels' 128-element steps, or operands off 16-byte alignment: one lane per output element
+        const size_t total = static_cast<size_t>(d->m) * d->n;
+        size_t blocks = (total + kThreads - 1) / kThreads;
+        if (blocks > 65536) blocks = 65536;
+        w8a16_generic_kernel<<<static_cast<uint32_t>(blocks), kThreads, 0, st>>>(p);
+        return launch_status("ascq_matmul_w8a16 (generic, [n, k] weights)");
+    }
     if (d->trans_b) {
-        ASCQ_REQUIRE(d->k % 128u == 0, ASCQ_EUNSUPPORTED,
-                     "ascq_matmul_w8a16: with trans_b k must be a multiple of 128 (k %u)", d->k);
-        ASCQ_REQUIRE(w8a16_nk_supported(d->k, x, w), ASCQ_EALIGN,
-                     "ascq_matmul_w8a16: with trans_b x and w must be 16-byte aligned");
         return launch_w8a16_nk(x, w, p.scale, p.offset, y, d->m, d->n, d->k, d->has_offset != 0, d->out_dtype == ASCQ_F32,
                                p.scale_bits, p.offset_bits, st);
     }

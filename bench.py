@@ -362,7 +362,7 @@ def main():
         """The shape of the reference's high-performance MxFP4 example (m = n = k = 8192, bfloat16 output, scale bytes
         127..129 as its gen_data.py draws them; its README reports 681.056 us on an Ascend 950PR for fp4 e1m2 operands,
         context only).  fmt: "fp4" = e2m1 x e2m1 straight on the scaled matrix instruction, "fp4_e1m2" = the example's
-        own format (widened to e4m3 first, inside the timed call), "fp8" = e4m3 x e4m3."""
+        own format (repacked as 6-bit e2m3 codes first, inside the timed call), "fp8" = e4m3 x e4m3."""
         M = N = K = 8192
         f = {"fp4": abi.QDST_FP4_E2M1, "fp4_e1m2": abi.QDST_FP4_E1M2, "fp8": abi.QDST_FP8_E4M3FN}[fmt]
         rb = K if fmt == "fp8" else K // 2

@@ -122,8 +122,11 @@ typedef enum ascq_dequant_mode { ASCQ_DEQUANT_WITH_SINGLE_ROW = 0, ASCQ_DEQUANT_
  *   PER_TOKEN  : scale [m]; rows = cal_count / n.
  *   PER_GROUP  : k_dim=1: scale [m, ceil(n/group_size)]; k_dim=0: scale [ceil(m/group_size), n].
  * Offset follows the scale's indexing when offset_kind == TENSOR, is the scalar
- * `offset` when SCALAR.  dst may alias src only for identical element offsets
- * (the reference allows reuse for AscendQuant).
+ * `offset` when SCALAR.  dst must not overlap src: a call whose byte ranges intersect returns ASCQ_EINVAL.  (The
+ * reference lets the destination reuse the source's memory, docs/zh/api/SIMD-API/高阶API/量化操作/AscendQuant.md:435:
+ * one core walks its tile in order.  Here thousands of wavefronts read and write at once, and an output byte lies
+ * on top of an input element that another wavefront has yet to read.)  The same holds for ascq_dequant,
+ * ascq_antiquant and ascq_antiquant_policy.
  * COMPUTE_F16:  y = sat8(rint( f16( f16( f16(x) * f16(s) ) + f16(o) ) ))   (policy TENSOR | CHANNEL)
  * COMPUTE_SCALE_T / F32: v = cvt(x) * s [+ o] with one rounding per operation in the compute
  *               type, y = sat8(round_mode(v)).
@@ -285,7 +288,14 @@ typedef enum ascq_mm_quant_mode {
 
 typedef enum ascq_mm_scale_format {
     ASCQ_MM_SCALE_U64 = 0, /* fixpipe word: scale = f32(bits[31:0] & 0xFFFFE000)  (1-8-10 float), REQ8: bits[45:37]
-                              offset, bit 46 sign (ref: examples/.../fixpipe_l0c2gm/scripts/gen_data_s322f16.py:37-66) */
+                              offset, bit 46 sign (ref: examples/.../fixpipe_l0c2gm/scripts/gen_data_s322f16.py:37-66).
+                              Mode-control bit 36 (scalar word or any word of a vector): the accumulator is first
+                              shifted right arithmetically by bits [35:32] and saturated, to the half range with one
+                              rounding to half for F16 outputs (gen_data_s322f16.py:84-90), to the int16 range for I8
+                              outputs (gen_data_s322s8.py:84-86); BF16 / F32 outputs, which no reference script
+                              covers, take the shifted value unsaturated.  The fixpipe's separate relu_pre word
+                              (another scale for negative accumulators, gen_data_s322f16.py:20-34,92-97) is not part
+                              of SetQuantScalar / SetQuantVector and has no field here */
     ASCQ_MM_SCALE_F32 = 1  /* plain fp32, all 23 mantissa bits used */
 } ascq_mm_scale_format;
 
@@ -343,11 +353,7 @@ typedef struct ascq_matmul_desc {
     int32_t has_tok_scale; /* fp32 [m] multiplied after the channel scale */
     int32_t activation;    /* ascq_mm_activation */
     int32_t b_format;      /* ascq_mm_b_format; for the grouped matmul every group's [k, n] block is in this format */
-    uint64_t quant_scalar; /* QUANT_SCALAR: U64 word, or fp32 bits in the low half for F32 format.  A U64 word with
-                              the mode-control bit 36 set (pre-shift by bits [35:32], fixpipe_l0c2gm/scripts/
-                              gen_data_s322f16.py:48-58,84-90) is rejected with ASCQ_EUNSUPPORTED; words of a quant
-                              vector live on the device and are not inspected: bit 36 and the shift are outside the
-                              supported domain there */
+    uint64_t quant_scalar; /* QUANT_SCALAR: U64 word, or fp32 bits in the low half for F32 format */
     float act_beta;        /* ASCQ_MM_ACT_SWIGLU: the constant of the swish function (1 = SiLU); ignored otherwise */
     int32_t reserved;      /* set to 0 */
 } ascq_matmul_desc;
@@ -355,6 +361,9 @@ typedef struct ascq_matmul_desc {
 int ascq_matmul_w8a8(const ascq_matmul_desc* desc, void* c, const void* a, const void* b, const void* bias,
                      const void* quant_vector, const void* tok_scale, void* workspace, size_t workspace_bytes,
                      void* stream);
+/* The workspace ascq_matmul_w8a8 needs for this descriptor with operands aligned to 16 bytes (0 for most shapes; the
+ * partial sums of the few-row kernels; with ASCQ_MM_ACT_SWIGLU outside the large tile kernel the raw accumulators
+ * [m][n]).  A call that needs more than it was given (SwiGLU on misaligned operands) names the size in its error. */
 int ascq_matmul_w8a8_workspace_size(const ascq_matmul_desc* desc, size_t* bytes);
 
 /*
@@ -550,7 +559,8 @@ int ascq_matmul_w4a16_packed(const ascq_w4a16_desc* desc, void* y, const void* x
  * Few activation rows (decode) run weight-streaming kernels: the weights are read once per 32 rows of x ([k, n]) or
  * per 16 rows ([n, k]).  With trans_b a column's weights are one contiguous run, so whole columns belong to one
  * workgroup: one launch, no workspace (the size query answers 0), identical bits from call to call; that form needs
- * k % 128 == 0 and 16-byte aligned x and w (ASCQ_EUNSUPPORTED / ASCQ_EALIGN otherwise).
+ * k % 128 == 0 and 16-byte aligned x and w (other shapes and alignments run a slow kernel with one lane per output
+ * element, as they do for [k, n] weights).
  * Many rows (more than 32 on [n, k] weights, more than 96 on [k, n]) run a half GEMM on 128 x 128 tiles whose B-tile
  * loader de-quantises; [k, n] weights are first copied transposed into the workspace (k * n bytes, which the size query
  * then asks for; given less, the call falls back to one pass over the weights per 32 rows).

@@ -687,6 +687,33 @@ float orc_quant_word_scale(uint64_t w, int scale_format)
     return bits_f32(lo);
 }
 
+/* The accumulator as the fixpipe hands it to the multiplier.  With the mode-control bit 36 of the word set it is first
+ * shifted right arithmetically by bits [35:32] and saturated: for half outputs to the half range, rounded to half
+ * (ref: fixpipe_l0c2gm/scripts/gen_data_s322f16.py:48-58 the fields, :84-90 the shift and `saturation(..., float16)`);
+ * for 8-bit outputs to the int16 range (gen_data_s322s8.py:84-86).  No reference script covers the other output
+ * types: there the shifted value is used as it is (parity unpinned for bfloat16 / float outputs with bit 36 set). */
+float orc_prescaled_accumulator(int32_t acc, uint64_t qword, int scale_format, int out_dtype)
+{
+    if (scale_format != ASCQ_MM_SCALE_U64 || ((qword >> 36) & 1u) == 0) {
+        return (float)acc;
+    }
+    int n = (int)((qword >> 32) & 0xF);
+    /* arithmetic shift written out: floor division by 2^n */
+    int64_t q = (int64_t)acc;
+    int64_t sh = q >= 0 ? q / ((int64_t)1 << n) : -((-q + ((int64_t)1 << n) - 1) / ((int64_t)1 << n));
+    if (out_dtype == ASCQ_F16) {
+        double c = (double)sh;
+        if (c > 65504.0) c = 65504.0;
+        if (c < -65504.0) c = -65504.0;
+        return orc_f16_to_f32(orc_f64_to_f16(c));
+    }
+    if (out_dtype == ASCQ_I8) {
+        if (sh > 32767) sh = 32767;
+        if (sh < -32768) sh = -32768;
+    }
+    return (float)sh;
+}
+
 /* Epilogue applied to one int32 accumulator.
  * ref: impl/adv_api/detail/matmul/stage/copy_cube_out/quant/quant_processor_fixpipe.h:89-117,197-222 (mode selection),
  *      fixpipe_l0c2gm/scripts/gen_data_s322f16.py:76-102 (deqf16: fp32 multiply, saturate to the fp16 range),
@@ -697,7 +724,7 @@ static inline float mm_value(const ascq_matmul_desc* d, int32_t acc, uint64_t qw
                              const void* bias, size_t bias_idx)
 {
     float s = orc_quant_word_scale(qword, d->scale_format);
-    volatile float v = (float)acc * s;
+    volatile float v = orc_prescaled_accumulator(acc, qword, d->scale_format, d->out_dtype) * s;
     if (d->has_tok_scale) {
         volatile float t = v * tok_scale[row];
         v = t;

@@ -27,6 +27,7 @@ int8_t orc_round_sat8(double v, int round_mode);
 float orc_faster_gelu(float x);
 float orc_swiglu(float src0, float src1, float beta);
 float orc_quant_word_scale(uint64_t w, int scale_format);
+float orc_prescaled_accumulator(int32_t acc, uint64_t qword, int scale_format, int out_dtype);
 
 uint8_t orc_f32_to_fp8(float f, int e5m2);
 float orc_fp8_to_f32(uint8_t code, int e5m2);

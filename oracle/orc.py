@@ -47,6 +47,8 @@ def lib():
         L.orc_swiglu.argtypes = [C.c_float, C.c_float, C.c_float]
         L.orc_quant_word_scale.restype = C.c_float
         L.orc_quant_word_scale.argtypes = [C.c_uint64, C.c_int]
+        L.orc_prescaled_accumulator.restype = C.c_float
+        L.orc_prescaled_accumulator.argtypes = [C.c_int32, C.c_uint64, C.c_int, C.c_int]
         L.orc_dequant_dst_stride.restype = C.c_uint32
         L.orc_dequant_dst_stride.argtypes = [C.c_int, C.c_uint32]
         L.orc_f32_to_fp4.restype = C.c_uint8

@@ -76,6 +76,21 @@ def test_quant_rejections():
     assert call(q(cal_count=0)) == abi.OK                                              # nothing to do, nothing launched
 
 
+def test_in_place_calls_are_rejected():
+    """The reference lets AscendQuant's destination reuse the source's memory; the GPU kernels cannot (other wavefronts
+    still have to read what an output byte would cover), so dst == src, or any intersection of the byte ranges, is
+    ASCQ_EINVAL before anything is launched."""
+    src = C.c_void_p(0x100000)
+    for dst in (src, C.c_void_p(0x100000 + 2 * 640 - 1), C.c_void_p(0x100000 - 639)):
+        assert L.ascq_quant(C.byref(q()), dst, src, FAKE, FAKE, None) == abi.EINVAL and "overlaps" in err()
+    dq = abi.DequantDesc(policy=abi.PER_CHANNEL, src_dtype=abi.I32, scale_dtype=abi.F32, dst_dtype=abi.BF16,
+                         mode=abi.DEQUANT_WITH_MULTI_ROW, m=4, n=64, cal_count=64)
+    assert L.ascq_dequant(C.byref(dq), src, src, FAKE, None) == abi.EINVAL and "overlaps" in err()
+    aq = abi.AntiQuantDesc(src_dtype=abi.I8, dst_dtype=abi.F16, has_offset=1, k=64, n=128, scale_height=1,
+                           scale_width=128, offset_height=1, offset_width=128)
+    assert L.ascq_antiquant(C.byref(aq), src, src, FAKE, FAKE, None) == abi.EINVAL and "overlaps" in err()
+
+
 def test_dequant_rejections():
     def d(**kw):
         x = abi.DequantDesc(policy=abi.PER_CHANNEL, src_dtype=abi.I32, scale_dtype=abi.F32, dst_dtype=abi.BF16,
@@ -371,23 +386,24 @@ def test_hifloat8_surface_and_refused_round_modes():
 
 
 def test_w8a16_transposed_weights_surface():
-    """[n, k] weights: no workspace; k must be a multiple of 128; the descriptor carries trans_b as its last field."""
+    """[n, k] weights: no workspace at any k (a k off the kernels' 128-element steps runs the one-lane-per-output
+    kernel, which needs none either); the descriptor carries trans_b as its last field."""
     assert C.sizeof(abi.W8A16Desc) == 9 * 4 and abi.W8A16Desc._fields_[-1][0] == "trans_b"
     need = C.c_size_t(77)
     d = abi.W8A16Desc(m=4, n=64, k=256, per_tensor=1, scale=0.5, out_dtype=abi.F16, trans_b=1)
     assert L.ascq_matmul_w8a16_workspace_size(C.byref(d), C.byref(need)) == abi.OK and need.value == 0
     d.k = 192
-    assert L.ascq_matmul_w8a16(C.byref(d), FAKE, FAKE, FAKE, None, None, None, 0, None) == abi.EUNSUPPORTED
-    assert "multiple of 128" in err()
-    d.k = 256
-    assert L.ascq_matmul_w8a16(C.byref(d), FAKE, C.c_void_p(0x100008), FAKE, None, None, None, 0, None) == abi.EALIGN
+    need.value = 77
+    assert L.ascq_matmul_w8a16_workspace_size(C.byref(d), C.byref(need)) == abi.OK and need.value == 0
 
 
-def test_quant_word_with_pre_shift_bit_is_rejected():
+def test_quant_word_with_pre_shift_bit_passes_validation():
+    """The mode-control bit 36 of a quant word (pre-shift by bits [35:32]) is part of the supported domain: the
+    descriptor is accepted (the call then fails on the NULL output, which is checked after the descriptor)."""
     d = abi.MatmulDesc(m=16, n=32, k=64, out_dtype=abi.F16, quant_mode=abi.MM_QUANT_SCALAR, scale_format=abi.MM_SCALE_U64,
                        quant_scalar=(1 << 36) | (3 << 32) | (0x3F800000 & 0xFFFFE000))
-    rc = L.ascq_matmul_w8a8(C.byref(d), FAKE, FAKE, FAKE, None, None, None, None, 0, None)
-    assert rc == abi.EUNSUPPORTED and "bit 36" in err()
+    rc = L.ascq_matmul_w8a8(C.byref(d), None, FAKE, FAKE, None, None, None, None, 0, None)
+    assert rc == abi.ENULL and "bit 36" not in err()
 
 
 def test_tmp_buffer_factor_sizes_known_answers():

@@ -14,10 +14,10 @@ def _capture(fn):
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
-        fn()                                   # warm-up on a side stream: lazily created workspaces exist afterwards
-    torch.cuda.current_stream().wait_stream(side)
+        fn()                                   # warm-up on the stream that will capture: the wrappers key their scratch
+    torch.cuda.current_stream().wait_stream(side)  # buffers by stream, so those the capture uses exist afterwards
     graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
+    with torch.cuda.graph(graph, stream=side):
         fn()
     torch.cuda.synchronize()
     return graph

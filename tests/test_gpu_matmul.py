@@ -290,6 +290,49 @@ def test_fixpipe_modes_uint64_words():
     assert np.array_equal(bits(c), oracle_mm(desc, a, b))
 
 
+@pytest.mark.parametrize("m,n,k,trans_b", [(7, 144, 192, False), (64, 256, 256, False), (12, 272, 256, True),
+                                           (200, 528, 384, False), (600, 528, 640, False), (19, 23, 77, False)])
+def test_fixpipe_pre_shift_words(m, n, k, trans_b):
+    """Quant words with the mode-control bit 36: the accumulator is shifted right by bits [35:32] and saturated before
+    the multiply.  Every column draws its own bit and shift; all four output types, and a scalar word."""
+    announce(f"matmul fixpipe pre-shift words m={m} n={n} k={k} trans_b={trans_b}")
+    rng = np.random.default_rng(1000 + m)
+    a = rand_i8(rng, (m, k), -127, 128)
+    b = rand_i8(rng, (n, k) if trans_b else (k, n), -127, 128)
+    bias = rng.integers(-3000000, 3000000, n).astype(np.int32)
+    qf = rng.uniform(0.01, 1.5, n).astype(np.float32)
+    sh = rng.integers(0, 16, n).astype(np.uint64)
+    on = rng.integers(0, 2, n).astype(np.uint64)
+    on[:4], sh[:4] = 1, (0, 1, 4, 15)
+    words = (qf.view(np.uint32).astype(np.uint64) | (sh << np.uint64(32)) | (on << np.uint64(36)) |
+             (rng.integers(0, 512, n).astype(np.uint64) << np.uint64(37)) |
+             (rng.integers(0, 2, n).astype(np.uint64) << np.uint64(46)))
+    for out in (torch.float16, torch.int8, torch.bfloat16, torch.float32):
+        c, desc = run_mm(m, n, k, a, b, out=out, bias=(bias, None), quant=words, trans_b=trans_b)
+        want = oracle_mm(desc, a, b, (bias, None), words)
+        assert np.array_equal(bits(c), want.view(np.uint16) if out == torch.float16 else want), out
+    plain = words & ~(np.uint64(1) << np.uint64(36))
+    c0, _ = run_mm(m, n, k, a, b, out=torch.float16, bias=(bias, None), quant=plain, trans_b=trans_b)
+    c1, _ = run_mm(m, n, k, a, b, out=torch.float16, bias=(bias, None), quant=words, trans_b=trans_b)
+    assert not np.array_equal(bits(c0), bits(c1)), "bit 36 had no effect"
+    if n % 2 == 0 and not trans_b:      # SwiGLU over column pairs that shift differently (small scales keep exp in range)
+        sw = words & ~np.uint64(0xFFFFFFFF) | (qf * np.float32(1e-4)).view(np.uint32).astype(np.uint64)
+        mm = ops.Matmul(m, n, k)
+        mm.set_tensor_a(to_dev(a))
+        mm.set_tensor_b(to_dev(b))
+        mm.set_quant_vector(to_dev(sw))
+        mm.set_bias(to_dev(bias))
+        mm.set_activation(abi.MM_ACT_SWIGLU, 1.0)
+        c = torch.zeros((m, n // 2), dtype=torch.float16, device=DEV)
+        mm.iterate_all(c)
+        swiglu_close(bits(c), oracle_mm(mm.desc, a, b, (bias, None), sw).view(np.uint16), "f16")
+    scalar = int(np.float32(0.37).view(np.uint32)) | (3 << 32) | (1 << 36) | (9 << 37) | (1 << 46)
+    for out in (torch.float16, torch.int8):
+        c, desc = run_mm(m, n, k, a, b, out=out, bias=(bias, None), scalar=scalar, trans_b=trans_b)
+        want = oracle_mm(desc, a, b, (bias, None))
+        assert np.array_equal(bits(c), want.view(np.uint16) if out == torch.float16 else want), out
+
+
 def test_post_bias_bf16_and_gelu():
     announce("matmul bf16 bias + token scale + FasterGelu")
     rng = np.random.default_rng(22)
@@ -707,12 +750,13 @@ def test_w8a16_exact_integers_full_size(m):
     assert np.array_equal(y.cpu().numpy().astype(np.float64), want)
 
 @pytest.mark.parametrize("m", [1, 3, 16, 17, 40, 49, 130, 300])
-@pytest.mark.parametrize("k,n", [(128, 16), (256, 256), (512, 1040), (384, 30), (2048, 520), (8192, 144)])
+@pytest.mark.parametrize("k,n", [(128, 16), (256, 256), (512, 1040), (384, 30), (2048, 520), (8192, 144), (192, 40),
+                                 (77, 23)])
 @pytest.mark.parametrize("mode", ["vector+offset", "vector", "scalar+offset", "scalar"])
 def test_w8a16_trans_b(m, k, n, mode):
     """B given as [n, k] (isTransposeB): one launch, no workspace; the whole-column kernel up to 48 rows, the
-    de-quantising tile GEMM above.  Against the oracle on the same transposed weights, and bit-equal between two calls
-    (the summation order is fixed)."""
+    de-quantising tile GEMM above, one lane per output element when k is no multiple of 128.  Against the oracle on
+    the same transposed weights, and bit-equal between two calls (the summation order is fixed)."""
     announce("w8a16 [n, k]", m, k, n, mode)
     rng = np.random.default_rng(m * 5 + k + n)
     x = rng.standard_normal((m, k)).astype(np.float16)

@@ -377,6 +377,71 @@ def test_matmul_deqf16_vector_follows_fixpipe_spec():
     assert np.array_equal(got.view(U16), (acc2.astype(np.float32) * s01).astype(np.float16).view(U16))
 
 
+def _fixpipe_fields(word):
+    """extract_quant_params of the reference's golden scripts (gen_data_s322f16.py:37-66), field by field."""
+    bits = (word >> 13) & 0xFFFFF
+    sign_bit, exponent, mantissa = (bits >> 18) & 1, (bits >> 10) & 0xFF, bits & 0x3FF
+    alpha = (-1) ** sign_bit * (1 + mantissa / 1024) * (2.0 ** (exponent - 127))
+    return np.float32(alpha), (word >> 37) & 0x1FF, (word >> 46) & 1, (word >> 32) & 0xF, (word >> 36) & 1
+
+
+def test_matmul_pre_shift_follows_fixpipe_scripts():
+    """Mode-control bit 36: the scripts shift the accumulator right by bits [35:32] and saturate it (to the half range,
+    cast to half, in gen_data_s322f16.py:84-90; to int16 in gen_data_s322s8.py:84-86) before the multiply.  The
+    expected values below follow those lines with numpy's own >>, clip and casts."""
+    rng = np.random.default_rng(77)
+    m, n, k = 12, 40, 256
+    a = rng.integers(-127, 128, (m, k)).astype(np.int8)
+    b = rng.integers(-127, 128, (k, n)).astype(np.int8)
+    bias = rng.integers(-2000000, 2000000, n).astype(np.int32)       # accumulators beyond the half range and int16
+    acc = (a.astype(np.int64) @ b.astype(np.int64) + bias).astype(np.int32)
+    assert (np.abs(acc) > 70000).any() and (acc < 0).any()
+    scales = rng.uniform(0.01, 1.5, n).astype(np.float32)
+    shifts = rng.integers(0, 16, n)
+    on = rng.integers(0, 2, n)
+    on[:4], shifts[:4] = 1, (0, 1, 4, 15)
+    words = np.array([int(np.float32(s).view(np.uint32)) | (int(sh) << 32) | (int(o) << 36)
+                      for s, sh, o in zip(scales, shifts, on)], dtype=np.uint64)
+    # ---- half output (DEQF16)
+    d = mm_desc(m, n, k, out_dtype=abi.F16, quant_mode=abi.MM_QUANT_VECTOR, scale_format=abi.MM_SCALE_U64,
+                bias_kind=abi.MM_BIAS_I32_PRE)
+    got = orc.matmul_w8a8(d, a, b, bias, words)
+    want = np.empty((m, n), np.float16)
+    for j in range(n):
+        alpha, _, _, n_shift, mode = _fixpipe_fields(int(words[j]))
+        data = acc[:, j]
+        if mode == 1:
+            data = np.clip(data >> n_shift, np.finfo(np.float16).min, np.finfo(np.float16).max).astype(np.float16)
+        want[:, j] = np.clip(data.astype(np.float32) * alpha, -65504, 65504).astype(np.float16)
+    assert np.array_equal(got.view(U16), want.view(U16))
+    L = orc.lib()
+    # what the arithmetic fixes: a shift of 0 on accumulators a half holds exactly changes nothing; negative
+    # accumulators round towards minus infinity (-1 >> 4 == -1)
+    assert L.orc_prescaled_accumulator(1234, (1 << 36), abi.MM_SCALE_U64, abi.F16) == 1234.0
+    assert L.orc_prescaled_accumulator(-1, (1 << 36) | (4 << 32), abi.MM_SCALE_U64, abi.F16) == -1.0
+    assert L.orc_prescaled_accumulator(-4096, (1 << 36) | (4 << 32), abi.MM_SCALE_U64, abi.F16) == -256.0
+    assert L.orc_prescaled_accumulator(2 ** 31 - 1, (1 << 36), abi.MM_SCALE_U64, abi.F16) == 65504.0
+    assert L.orc_prescaled_accumulator(-2 ** 31, (1 << 36), abi.MM_SCALE_U64, abi.I8) == -32768.0
+    assert L.orc_prescaled_accumulator(4097, (1 << 36), abi.MM_SCALE_U64, abi.F16) == 4096.0      # rounded to half
+    assert L.orc_prescaled_accumulator(4097, (4 << 32), abi.MM_SCALE_U64, abi.F16) == 4097.0      # bit 36 clear
+    assert L.orc_prescaled_accumulator(4097, (1 << 36), abi.MM_SCALE_F32, abi.F16) == 4097.0      # plain float scales
+    # ---- 8-bit output (REQ8): shift, saturate to int16, multiply, round, 9 bits, + offset, 8 bits
+    offs = rng.integers(0, 512, n)
+    sgn = rng.integers(0, 2, n)
+    words8 = np.array([int(w) | (int(o) << 37) | (int(sg) << 46) for w, o, sg in zip(words, offs, sgn)], dtype=np.uint64)
+    d8 = mm_desc(m, n, k, out_dtype=abi.I8, quant_mode=abi.MM_QUANT_VECTOR, scale_format=abi.MM_SCALE_U64,
+                 bias_kind=abi.MM_BIAS_I32_PRE)
+    got8 = orc.matmul_w8a8(d8, a, b, bias, words8)
+    for j in range(n):
+        alpha, offset, sign, n_shift, mode = _fixpipe_fields(int(words8[j]))
+        data = acc[:, j]
+        if mode == 1:
+            data = np.clip(data >> n_shift, -32768, 32767).astype(np.int16)
+        q = np.clip(np.rint(data.astype(np.float32) * alpha), -256, 255).astype(np.int16) + offset
+        w8 = np.clip(q, -128, 127) if sign else np.clip(q, 0, 255)
+        assert np.array_equal(got8[:, j].view(np.uint8), w8.astype(np.int64).astype(np.uint8)), j
+
+
 def test_matmul_req8_follows_spec():
     # gen_data_s322s8.py:76-97: round, clip to [-256, 255], add the 9-bit offset, clip to int8 (sign = 1)
     rng = np.random.default_rng(16)

@@ -77,3 +77,25 @@ def test_noalloc_rejects_shapes_beyond_its_buffer():
     rc = L.ascq_linear_w8a8_dynamic_noalloc(C.byref(d), abi.BF16, C.c_void_p(0x1000), C.c_void_p(0x1000),
                                             C.c_void_p(0x1000), None, C.c_void_p(0x1000), None)
     assert rc == abi.EINVAL and "built-in buffer" in L.ascq_last_error().decode()
+
+
+@pytest.mark.parametrize("m,n,k", [(7, 544, 512), (300, 544, 512)])
+def test_noalloc_wrapper_with_swiglu(m, n, k):
+    """The Python wrapper takes n from the weight (with SwiGLU the output has n / 2 columns) and passes act_beta on: its
+    result is that of the workspace form's wrapper, bit for bit."""
+    from ascq import ops
+    announce("noalloc swiglu wrapper", m, n, k)
+    g = torch.Generator(device=DEV)
+    g.manual_seed(31)
+    x = torch.randn((m, k), device=DEV, generator=g).to(torch.bfloat16)
+    w = torch.randint(-127, 128, (k, n), dtype=torch.int8, device=DEV, generator=g)
+    cs = torch.rand(n, device=DEV, generator=g) * 1e-2 + 1e-4
+    want = torch.full((m, n // 2), -1.0, dtype=torch.bfloat16, device=DEV)
+    got = torch.full((m, n // 2), -2.0, dtype=torch.bfloat16, device=DEV)
+    ops.linear_w8a8_dynamic(want, x, w, cs, activation=abi.MM_ACT_SWIGLU, act_beta=1.702)
+    ops.linear_w8a8_dynamic_noalloc(got, x, w, cs, activation=abi.MM_ACT_SWIGLU, act_beta=1.702)
+    plain = torch.empty_like(want)
+    ops.linear_w8a8_dynamic(plain, x, w, cs, activation=abi.MM_ACT_SWIGLU, act_beta=1.0)
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    assert not torch.equal(plain.view(torch.int16), want.view(torch.int16)), "act_beta had no effect"
