@@ -7,7 +7,8 @@
 //   * device-to-device copy, read-only sweep and write-only fill of 1 GiB (HBM bandwidth actually reachable);
 //   * LDS read bandwidth per compute unit with 16-byte reads;
 //   * a small streaming job, 2048 workgroups that each read one 8 KiB row and write 4 KiB (16 MiB in, 8 MiB out, the
-//     same buffers every launch): what launch, ramp-up and drain cost a kernel of that size whatever it computes.
+//     same buffers every launch): what launch, ramp-up and drain cost a kernel of that size whatever it computes;
+//     and the same job on rows that no cache holds.
 // Every figure is the mean of the second half of `reps` back-to-back launches (the first half brings the clocks to
 // their sustained state).  No input, no dependence on libascq.
 #include <hip/hip_runtime.h>
@@ -223,6 +224,20 @@ int main()
     CK(hipEventRecord(e1));
     CK(hipEventSynchronize(e1));
     CK(hipEventElapsedTime(&ms, e0, e1));
-    printf(", \"rows_2048x8kib_read_4kib_written_us\": %.2f}\n", ms * 1e3 / 400);
+    printf(", \"rows_2048x8kib_read_4kib_written_us\": %.2f", ms * 1e3 / 400);
+    // the same job on fresh rows every launch (32 positions of the 1 GiB buffers in turn: 512 MiB in, 256 MiB out,
+    // more than the caches hold), as a kernel meets them whose input another kernel produced some launches earlier
+    const size_t step_a = static_cast<size_t>(2048) * 512, step_b = step_a / 2;  // in u32x4
+    for (int r = 0; r < 100; ++r) {
+        row_2to1_kernel<<<2048, 256>>>(a + (r % 32) * step_a, reinterpret_cast<unsigned long long*>(b + (r % 32) * step_b));
+    }
+    CK(hipEventRecord(e0));
+    for (int r = 0; r < 400; ++r) {
+        row_2to1_kernel<<<2048, 256>>>(a + (r % 32) * step_a, reinterpret_cast<unsigned long long*>(b + (r % 32) * step_b));
+    }
+    CK(hipEventRecord(e1));
+    CK(hipEventSynchronize(e1));
+    CK(hipEventElapsedTime(&ms, e0, e1));
+    printf(", \"rows_2048x8kib_fresh_rows_us\": %.2f}\n", ms * 1e3 / 400);
     return 0;
 }

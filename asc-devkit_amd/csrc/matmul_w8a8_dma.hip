@@ -461,7 +461,7 @@ __device__ __forceinline__ void gemm_dma_tile_at(const GemmParams& p, const Tile
             if (e.scale_format == ASCQ_MM_SCALE_U64 && e.quant_mode != ASCQ_MM_QUANT_NONE &&
                 __builtin_amdgcn_ballot_w64(((q[0].ctl | q[TJ - 1].ctl) & 2) != 0) != 0) {
                 const bool odd = (lane & 1u) != 0;
-#pragma unroll 1
+#pragma unroll  // (a run-time index into the accumulators would move them to scratch memory)
                 for (int i = 0; i < TI; ++i) {
                     const uint32_t lbase = (wm * TI + i) * 32u + 4u * g;
 #pragma unroll
