@@ -50,7 +50,7 @@ PEAK_FP4_TFLOPS = float(_PEAKS["fp4_dense_tflops"])
 # file does not re-measure them.
 GEMM_TRAFFIC_BYTES = 228293837   # M=2048 GEMM, both tile shapes: 183.2 MB fetched + 45.1 MB written
 GEMV_TRAFFIC_BYTES = 133853594   # W4A16 M=1 GEMV, [k, n / 2] layout, stream + sum kernels: 129.5 MB fetched + 4.3 MB written
-GEMV_PACKED_TRAFFIC_BYTES = 128_487_629   # the same on packed weights, one launch: 128.4 MB fetched + 0.06 MB written (profiles/w4a16_packed_gemv_m1_trace_and_counters.md)
+GEMV_PACKED_TRAFFIC_BYTES = 125_108_224   # the same on packed weights in the group-sum mode, one launch: 125.05 MB fetched + 0.06 MB written (profiles/w4a16_packed_group_sum_gemv_m1_trace_and_counters.md)
 
 
 def main():
