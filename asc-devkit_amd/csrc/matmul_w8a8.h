@@ -230,6 +230,7 @@ int launch_gemm_nk(const GemmParams& p, hipStream_t st);
 // Few rows on weights packed by ascq_pack_weight_w8 (p.b): whole columns per workgroup, one launch, no workspace
 // (matmul_w8a8_packed.hip).
 bool gemm_packed_supported(const GemmParams& p);
-int launch_gemm_packed(const GemmParams& p, hipStream_t st);
+bool gemm_packed_nk_supported(const GemmParams& p);
+int launch_gemm_packed(const GemmParams& p, hipStream_t st, bool b_nk = false);
 
 }  // namespace ascq

@@ -15,6 +15,12 @@
 // issue of their loads).  Operand row i of a lane reads activation row i % rows, so there are no zero rows to
 // materialise.  The eight partial sums of a column meet in LDS (integers: exact in any order) and go through the
 // element-wise epilogue of the int8 matmul.
+//
+// The same kernel reads weights kept as [n, k] (the reference's isTransposeB) without any packing: there a "tile" of a
+// slab is the 64 bytes k = 64 t .. + 63 of each of its 16 columns, lane l fetching bytes 16 (l / 16) .. + 15 of column
+// l % 16 - the same operand, gathered from 16 runs of 64 bytes instead of one run of 1 KiB.  Only the addresses differ:
+// the lane's offset is column * k + 16 (l / 16), the scalar offset slab * 16 k + 64 t, and columns past n fall outside
+// the buffer, whose range check returns zeros for them.
 #include "matmul_w8a8.h"
 
 namespace ascq {
@@ -49,6 +55,7 @@ __device__ __forceinline__ uint32_t pk_xcd_order(uint32_t wg, uint32_t wgs)
     return (wgs & 7u) == 0u ? (wg & 7u) * (wgs >> 3) + (wg >> 3) : wg;
 }
 
+template <bool kNK>
 __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_kernel(PackedParams p)
 {
     __shared__ __attribute__((aligned(16))) char XS[kPkXBytes];
@@ -78,7 +85,9 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_kernel(PackedParams
         }
     }
     const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<i32x4*>(p.wp), 0, static_cast<int>((p.slabs * p.ktiles + kPkPadTiles) * kPkTileBytes), 0x00020000);
+        const_cast<i32x4*>(p.wp), 0,
+        static_cast<int>(kNK ? p.n * p.k : (p.slabs * p.ktiles + kPkPadTiles) * kPkTileBytes), 0x00020000);
+    const uint32_t w_lane = kNK ? lc * p.k + lq * 16u : lane * 16u;  // the lane's 16 bytes inside a tile
     // operand row i reads row i % rows; + tile * 64
     const uint32_t x_lane = (lc - __umulhi(lc, p.rows_magic) * p.rows) * pitch + lq * 16u;
 
@@ -92,11 +101,13 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_kernel(PackedParams
         // every load is issued, so the waits the compiler inserts count exactly; once every batch has been requested the
         // per-lane offset lies past the end of the buffer and the loads move no data.  A short last batch reads on into
         // the next tiles or the padding: valid memory, not computed.
-        const uint32_t l_w = l_done ? kPkPastEnd : lane * 16u;
-        const uint32_t base = (l_slab * p.ktiles + ta + l_b * kPkBatch) * kPkTileBytes;  // scalar
+        const uint32_t l_w = l_done ? kPkPastEnd : w_lane;
+        constexpr uint32_t kStep = kNK ? kPkTileK : kPkTileBytes;  // bytes from a tile to the next of its slab
+        const uint32_t base = kNK ? l_slab * kPkCols * p.k + (ta + l_b * kPkBatch) * kPkTileK
+                                  : (l_slab * p.ktiles + ta + l_b * kPkBatch) * kPkTileBytes;  // scalar
 #pragma unroll
         for (uint32_t t = 0; t < kPkBatch; ++t) {
-            wq[buf][t] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, l_w, base + t * kPkTileBytes, kPkNt));
+            wq[buf][t] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, l_w, base + t * kStep, kPkNt));
         }
         if (l_q + 1u < batches) {  // uniform
             ++l_q;
@@ -218,14 +229,21 @@ __global__ __launch_bounds__(256) void pack_w8_kernel(const int8_t* __restrict__
 
 }  // namespace
 
+// B as [n, k], read in place by the same kernel (offsets are 32-bit and the range check marks the end at 2 GiB)
+bool gemm_packed_nk_supported(const GemmParams& p)
+{
+    return p.k % kPkTileK == 0 && aligned16(p.a) && aligned16(p.b) &&
+           static_cast<uint64_t>(p.n + kPkCols) * p.k < (1ull << 31) - 64u * kPkTileK;
+}
+
 bool gemm_packed_supported(const GemmParams& p)
 {
     return p.k % kPkTileK == 0 && aligned16(p.a) && aligned16(p.b) &&
            (static_cast<uint64_t>((p.n + kPkCols - 1u) / kPkCols) * (p.k / kPkTileK) + kPkPadTiles) * kPkTileBytes < (1ull << 31);
 }
 
-// p.b: the packed weights.  Any m: up to 16 rows per pass over the weights.
-int launch_gemm_packed(const GemmParams& p, hipStream_t st)
+// p.b: the packed weights, or with b_nk the plain [n, k] matrix.  Any m: up to 16 rows per pass over the weights.
+int launch_gemm_packed(const GemmParams& p, hipStream_t st, bool b_nk)
 {
     const int cus = static_cast<int>(device_compute_units());
     PackedParams q{};
@@ -256,9 +274,13 @@ int launch_gemm_packed(const GemmParams& p, hipStream_t st)
                       kPkXBytes + kPkWaves * kPkMaxSlabs * 1024u, 0)) {
             return ASCQ_OK;
         }
-        gemm_packed_kernel<<<grid, kPkWaves * 64u, 0, st>>>(q);
+        if (b_nk) {
+            gemm_packed_kernel<true><<<grid, kPkWaves * 64u, 0, st>>>(q);
+        } else {
+            gemm_packed_kernel<false><<<grid, kPkWaves * 64u, 0, st>>>(q);
+        }
     }
-    return launch_status("ascq_matmul_w8a8_packed");
+    return launch_status(b_nk ? "ascq_matmul_w8a8 ([n, k] weight stream)" : "ascq_matmul_w8a8_packed");
 }
 
 }  // namespace ascq
