@@ -642,6 +642,17 @@ public:
         desc_.trans_b = isTransposeB ? 1 : 0;
         desc_.b_format = format == CubeFormat::NZ ? ASCQ_MM_B_NZ : ASCQ_MM_B_ND;
     }
+    // B in the layout of ascq_pack_weight_w8 (PackWeightInt8 below), packed once per weight matrix: IterateAll then
+    // runs the one-launch decode kernel (up to 16 rows per pass over the weights), with the results of SetTensorB's
+    // matmul bit for bit.  No counterpart in the reference (the analogue of its offline ND -> NZ packing).
+    void SetTensorBPacked(const void* packed)
+    {
+        static_assert(!kInt4, "packed weights are int8");
+        b_ = packed;
+        packed_ = true;
+        desc_.trans_b = 0;
+        desc_.b_format = ASCQ_MM_B_ND;
+    }
     // int32 bias: the accumulator's initial value, as in the reference.
     void SetBias(const DeviceTensor<int32_t>& bias)
     {
@@ -710,6 +721,10 @@ public:
     }
     void IterateAll(const DeviceTensor<CType>& c, void* stream = nullptr)
     {
+        if (packed_) {
+            Check(ascq_matmul_w8a8_packed(&desc_, c.GetPhyAddr(), a_, b_, bias_, quant_, tok_, stream));
+            return;
+        }
         Check((kInt4 ? ascq_matmul_w4a4 : ascq_matmul_w8a8)(&desc_, c.GetPhyAddr(), a_, b_, bias_, quant_, tok_,
                                                             workspace_, workspace_bytes_, stream));
     }
@@ -734,7 +749,21 @@ private:
     const void* tok_ = nullptr;
     void* workspace_ = nullptr;
     size_t workspace_bytes_ = 0;
+    bool packed_ = false;
 };
+
+// Bytes of, and the packing into, the decode layout of int8 weights (b: [k, n], or [n, k] with isTransposeB).
+inline size_t PackWeightInt8Size(uint32_t k, uint32_t n)
+{
+    size_t bytes = 0;
+    Check(ascq_pack_weight_w8_size(k, n, &bytes));
+    return bytes;
+}
+inline void PackWeightInt8(const DeviceTensor<int8_t>& b, void* packed, uint32_t k, uint32_t n, bool isTransposeB = false,
+                           void* stream = nullptr)
+{
+    Check(ascq_pack_weight_w8(b.GetPhyAddr(), packed, k, n, isTransposeB ? 1 : 0, stream));
+}
 
 // Matmul with A half and B int8 de-quantised on the way in (MatmulType<.., half> x MatmulType<.., int8_t>).
 // ref: include/adv_api/matmul/matmul.h:161-168 (SetAntiQuantScalar / SetAntiQuantVector); hasAntiQuantOffset is the

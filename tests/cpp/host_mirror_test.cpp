@@ -47,6 +47,7 @@ public:
     {
         return ascq::DeviceTensor<U>(static_cast<U*>(ptr_), size);
     }
+    void* ptr() const { return ptr_; }
     std::vector<T> download() const
     {
         std::vector<T> h(count_);
@@ -337,6 +338,22 @@ void test_matmul()
         std::vector<int32_t> want(m * n);
         orc_matmul_w8a8(&mm.Desc(), want.data(), a.data(), b.data(), nullptr, nullptr, nullptr);
         expect_equal("Matmul int32", dc.download(), want);
+    }
+    std::printf("[case] Matmul<bfloat16_t> 7x160x256 on weights packed by PackWeightInt8 (decode kernel)\n");
+    {
+        const uint32_t rows = 7;
+        DeviceBuffer<uint8_t> dpacked(ascq::PackWeightInt8Size(k, n));
+        ascq::PackWeightInt8(db.view<int8_t>(k * n), dpacked.ptr(), k, n);
+        DeviceBuffer<uint16_t> dc(rows * n);
+        ascq::Matmul<ascq::bfloat16_t> mm(rows, n, k);
+        mm.SetTensorA(da.view<int8_t>(rows * k));
+        mm.SetTensorBPacked(dpacked.ptr());
+        mm.SetQuantVector(dcs.view<float>(n));
+        mm.SetTokenScale(dts.view<float>(rows));
+        mm.IterateAll(dc.view<ascq::bfloat16_t>(rows * n));
+        std::vector<uint16_t> want(rows * n);
+        orc_matmul_w8a8(&mm.Desc(), want.data(), a.data(), b.data(), nullptr, cs.data(), ts.data());
+        expect_equal("Matmul on packed int8 weights", dc.download(), want);
     }
     std::printf("[case] Matmul<int32_t, int4b_t> 96x160x256, int32 bias\n");
     {
