@@ -81,7 +81,10 @@ class W4A16Desc(C.Structure):
 class W8A16Desc(C.Structure):
     _fields_ = [("m", C.c_uint32), ("n", C.c_uint32), ("k", C.c_uint32), ("per_tensor", C.c_int32),
                 ("has_offset", C.c_int32), ("scale", C.c_float), ("offset", C.c_float), ("out_dtype", C.c_int32),
-                ("trans_b", C.c_int32)]
+                ("trans_b", C.c_int32), ("mode", C.c_int32)]
+
+
+W8A16_PER_WEIGHT, W8A16_CHANNEL_SUM = range(2)
 
 
 class MxDesc(C.Structure):

@@ -521,12 +521,13 @@ def matmul_w4a16_packed(y, x, w_gpu, scale, offset=None, group_size=128, mode=ab
 
 
 # ------------------------------------------------------------------------------------------------------ W8A16
-def matmul_w8a16(y, x, w, offset=None, scale=None, workspace=None, trans_b=False):
+def matmul_w8a16(y, x, w, offset=None, scale=None, workspace=None, trans_b=False, mode=abi.W8A16_PER_WEIGHT):
     """y f16 / f32 [m, n] = x f16 [m, k] @ AscendAntiQuant<int8_t, half>(w int8 [k, n]); trans_b: w is [n, k]
     (SetTensorB(b, isTransposeB=true)) and the call is one launch without a workspace.
 
     scale / offset: f16 tensors of n elements (SetAntiQuantVector) or Python floats (SetAntiQuantScalar); offset None =
-    MatmulConfig::hasAntiQuantOffset false.
+    MatmulConfig::hasAntiQuantOffset false.  mode: abi.W8A16_CHANNEL_SUM applies scale and offset once per output to
+    fp32 sums (up to 4 rows on [n, k] weights; elsewhere the per-weight form runs).
     """
     m, k = x.shape
     n = y.shape[1]
@@ -534,7 +535,7 @@ def matmul_w8a16(y, x, w, offset=None, scale=None, workspace=None, trans_b=False
     d = abi.W8A16Desc(m=m, n=n, k=k, per_tensor=int(per_tensor), has_offset=int(offset is not None),
                       scale=float(scale) if per_tensor else 0.0,
                       offset=float(offset) if per_tensor and offset is not None else 0.0, out_dtype=_DT[y.dtype],
-                      trans_b=int(trans_b))
+                      trans_b=int(trans_b), mode=mode)
     lib = load_library()
     need = C.c_size_t(0)
     check(lib.ascq_matmul_w8a16_workspace_size(C.byref(d), C.byref(need)))

@@ -209,6 +209,225 @@ void launch_nk(const NkParams& p, uint32_t grid, hipStream_t st)
     }
 }
 
+// ---- up to 4 activation rows: one flat sweep over the weights with the activations resident in LDS.
+// The kernel above fetches its rows of x from memory run by run, in the same in-order queue of the compute unit as
+// the weights; here a wavefront stages its k range of every row once (direct-to-LDS loads) and then has nothing but
+// weights in flight: batches of 4 tiles (64 k x 16 columns: the lane's 16 bytes are 16 consecutive k of its column),
+// two register buffers, buffer loads whose lane offset is column * k + 16 (l / 16) and whose scalar offset walks the
+// tiles, so that columns past n fall outside the buffer and read as zeros.  The workgroups of an XCD own neighbouring
+// column groups.
+//   kSum = false: the reference's arithmetic per weight (dequant4 above), two MFMAs per tile.
+//   kSum = true (ASCQ_W8A16_CHANNEL_SUM): y = scale * (sum_k x w + offset * sum_k x) with the sums in fp32.  The bytes
+//   go into the matrix core as the exact halves 1152 + w (one xor and two byte permutes per dword); the bias and the
+//   offset are one fma per column group and row, on sum_k x, which the matrix core adds up as well (the same A
+//   operands against a B operand of ones, during the wavefront's first column group only).
+constexpr uint32_t kSkTileK = 64, kSkBatch = 4, kSkMaxSlabs = 8, kSkMaxRows = 4;
+constexpr int kSkBuf = 2;
+constexpr uint32_t kSkRowPad = 32;             // bytes added to a staged row of x
+constexpr uint32_t kSkXBytes = 96 * 1024;      // LDS for the staged activations of a workgroup
+constexpr uint32_t kSkPastEnd = 0x7FFFFFF0u;
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef __attribute__((address_space(1))) const void* gptr_t;
+
+struct SkParams {
+    const uint16_t* x;       // [rows, k] halves (this pass's first row)
+    const uint8_t* w;        // [n, k] int8
+    const uint16_t* scale;   // [n] halves, or nullptr: scale_bits / offset_bits for every column
+    const uint16_t* offset;
+    void* y;                 // [rows, n] halves or floats (this pass's first row)
+    uint32_t rows, n, k;     // rows of this pass, 1 .. 4
+    uint32_t slabs, ktiles, tpw;
+    uint32_t out_f32;
+    uint32_t scale_bits, offset_bits;
+};
+
+__device__ __forceinline__ uint32_t sk_xcd_order(uint32_t wg, uint32_t wgs)
+{
+    return (wgs & 7u) == 0u ? (wg & 7u) * (wgs >> 3) + (wg >> 3) : wg;
+}
+
+template <bool kHasOffset, bool kSum>
+__global__ __launch_bounds__(kWaves * 64) void w8a16_nk_stream_kernel(SkParams p)
+{
+    __shared__ __attribute__((aligned(16))) char XS[kSkXBytes];
+    __shared__ float RED[kWaves][kSkMaxSlabs][4][16];
+    __shared__ uint32_t PAR[kSkMaxSlabs][16];  // (scale | offset << 16) of the workgroup's columns
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t lc = lane & 15u, lq = lane >> 4;
+    const uint32_t wg = sk_xcd_order(blockIdx.x, gridDim.x);
+    const uint32_t s0 = static_cast<uint32_t>(static_cast<uint64_t>(wg) * p.slabs / gridDim.x);
+    const uint32_t s1 = static_cast<uint32_t>(static_cast<uint64_t>(wg + 1u) * p.slabs / gridDim.x);
+    const uint32_t nslabs = s1 - s0;
+    const uint32_t ta = min(wave * p.tpw, p.ktiles), tb = min(ta + p.tpw, p.ktiles), cnt = tb - ta;
+    const uint32_t pitch = p.tpw * (kSkTileK * 2u) + kSkRowPad;
+    char* const xs = XS + wave * (p.rows * pitch);
+
+    // ---- this wavefront's k range of every row, straight into LDS (1 KiB of a row per instruction)
+    {
+        const uint32_t row_pieces = cnt * (kSkTileK * 2u / 16u);
+        for (uint32_t r = 0; r < p.rows; ++r) {
+            const uint16_t* src = p.x + static_cast<size_t>(r) * p.k + ta * kSkTileK + lane * 8u;
+            for (uint32_t c0 = 0; c0 < row_pieces; c0 += 64u) {
+                if (c0 + lane < row_pieces) {
+                    __builtin_amdgcn_global_load_lds((gptr_t)(src + c0 * 8u), (lds_ptr_t)(xs + r * pitch + c0 * 16u), 16, 0, 0);
+                }
+            }
+        }
+    }
+    // ---- the columns' parameters: thread t < 16 nslabs fetches those of column group t / 16, column t % 16
+    uint32_t my_par = 0;
+    if (tid < nslabs * 16u) {
+        uint32_t col = (s0 + (tid >> 4)) * 16u + (tid & 15u);
+        col = col < p.n ? col : p.n - 1u;
+        const uint32_t sb = p.scale ? p.scale[col] : p.scale_bits;
+        const uint32_t ob = kHasOffset ? (p.scale ? p.offset[col] : p.offset_bits) : 0u;
+        my_par = sb | (ob << 16);
+    }
+    const __amdgpu_buffer_rsrc_t rw =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.w), 0, static_cast<int>(p.n * p.k), 0x00020000);
+    const uint32_t w_lane = lc * p.k + lq * 16u;
+    // operand row i reads row i % rows (rows <= 4: a mask or a compare); + tile * 128
+    const uint32_t xrow = p.rows == 3u ? (lc % 3u) : (lc & (p.rows - 1u));
+    const uint32_t x_lane = xrow * pitch + lq * 32u;
+
+    const uint32_t nb = (cnt + kSkBatch - 1u) / kSkBatch;
+    const uint32_t batches = nb * nslabs;
+    u32x4 wq[kSkBuf][kSkBatch];
+    uint32_t l_slab = s0, l_b = 0, l_q = 0;
+    bool l_done = batches == 0u;
+    auto load = [&](int buf) __attribute__((always_inline)) {
+        // every load is issued, so the waits count exactly; once every batch has been requested the lane offset lies
+        // past the end of the buffer and the loads move no data.  A short last batch reads on along its columns (or
+        // past the buffer's end, as zeros): not computed.
+        const uint32_t l_w = l_done ? kSkPastEnd : w_lane;
+        const uint32_t base = l_slab * 16u * p.k + (ta + l_b * kSkBatch) * kSkTileK;  // scalar
+#pragma unroll
+        for (uint32_t t = 0; t < kSkBatch; ++t) {
+            wq[buf][t] = __builtin_amdgcn_raw_buffer_load_b128(rw, l_w, base + t * kSkTileK, 2);
+        }
+        if (l_q + 1u < batches) {  // uniform
+            ++l_q;
+            if (++l_b == nb) {
+                l_b = 0;
+                ++l_slab;
+            }
+        } else {
+            l_done = true;
+        }
+    };
+#pragma unroll
+    for (int b = 0; b < kSkBuf; ++b) load(b);
+    // Loads return in order: with at most the weight loads just issued outstanding, the activations have landed in LDS
+    // and the parameters in their register.  (The compiler does not count direct-to-LDS loads issued in a loop.)
+    __builtin_amdgcn_s_waitcnt(((kSkBuf * kSkBatch) & 15) | (((kSkBuf * kSkBatch) >> 4) << 14) | (7 << 4) | (15 << 8));
+    asm volatile("" ::: "memory");
+    if (tid < nslabs * 16u) {
+        PAR[tid >> 4][tid & 15u] = my_par;
+    }
+    __syncthreads();
+
+    f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f}, xsum = {0.0f, 0.0f, 0.0f, 0.0f};
+    f16x2_t sc2 = {}, of2 = {};
+    float corr = 0.0f;  // kSum: offset - 1152 of the lane's column
+    uint32_t c_slab = 0, c_b = 0, c_q = 0;
+    const f16x8_t ones = {1, 1, 1, 1, 1, 1, 1, 1};
+    auto compute = [&](int buf) __attribute__((always_inline)) {
+        constexpr uint32_t kBehind = (kSkBuf - 1) * kSkBatch;
+        __builtin_amdgcn_s_waitcnt((kBehind & 15u) | ((kBehind >> 4) << 14) | (7u << 4) | (15u << 8));
+        if (c_q >= batches) {
+            return;  // uniform
+        }
+        if (c_b == 0u) {  // a new column group: the lane's column parameters
+            const uint32_t pr = PAR[c_slab][lc];
+            sc2 = h2_from_bits((pr & 0xFFFFu) | (pr << 16));
+            of2 = h2_from_bits((pr >> 16) | (pr & 0xFFFF0000u));
+            corr = (kHasOffset ? static_cast<float>(of2[0]) : 0.0f) - 1152.0f;
+        }
+        const uint32_t t0 = c_b * kSkBatch;
+        const uint32_t live = min(kSkBatch, cnt - t0);
+        const char* xa0 = xs + x_lane + t0 * (kSkTileK * 2u);
+#pragma unroll
+        for (uint32_t t = 0; t < kSkBatch; ++t) {
+            if (t < live) {  // uniform
+                const f16x8_t a0 = *reinterpret_cast<const f16x8_t*>(xa0 + t * (kSkTileK * 2u));
+                const f16x8_t a1 = *reinterpret_cast<const f16x8_t*>(xa0 + t * (kSkTileK * 2u) + 16u);
+                uint32_t h[8];
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+                    if constexpr (kSum) {
+                        const uint32_t flipped = wq[buf][t][d] ^ 0x80808080u;  // w + 128 as an unsigned byte
+                        h[2 * d] = __builtin_amdgcn_perm(0x64646464u, flipped, 0x04010400u);      // (1152 + w0, 1152 + w1)
+                        h[2 * d + 1] = __builtin_amdgcn_perm(0x64646464u, flipped, 0x04030402u);  // (1152 + w2, 1152 + w3)
+                    } else {
+                        dequant4<kHasOffset>(wq[buf][t][d], sc2, of2, h[2 * d], h[2 * d + 1]);
+                    }
+                }
+                const u32x4 q0 = {h[0], h[1], h[2], h[3]}, q1 = {h[4], h[5], h[6], h[7]};
+                f16x8_t b0, b1;
+                __builtin_memcpy(&b0, &q0, 16);
+                __builtin_memcpy(&b1, &q1, 16);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, b0, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, b1, acc, 0, 0, 0);
+                if (kSum && c_slab == 0u) {  // uniform: sum_k x of this wavefront's k range, once
+                    xsum = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, ones, xsum, 0, 0, 0);
+                    xsum = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, ones, xsum, 0, 0, 0);
+                }
+            }
+        }
+        ++c_q;
+        if (++c_b == nb) {  // the column group is done: register i of lane l is row 4 (l / 16) + i, column l % 16
+            if (lq == 0u) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    RED[wave][c_slab][i][lc] = kSum ? __builtin_fmaf(corr, xsum[i], acc[i]) : acc[i];
+                }
+            }
+            acc = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+            c_b = 0;
+            ++c_slab;
+        }
+    };
+    for (uint32_t q = 0; q < batches; q += kSkBuf) {
+#pragma unroll
+        for (int b = 0; b < kSkBuf; ++b) {
+            compute(b);
+            load(b);
+        }
+    }
+    if (batches == 0u && lq == 0u) {  // a wavefront without tiles (k shorter than 8 tiles) contributes zeros
+        for (uint32_t s = 0; s < nslabs; ++s) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) RED[wave][s][i][lc] = 0.0f;
+        }
+    }
+    __syncthreads();
+
+    // ---- the eight partial sums of every element in wavefront order, one rounding, store
+    const uint32_t outs = nslabs * p.rows * 16u;
+    for (uint32_t i = tid; i < outs; i += kWaves * 64u) {
+        const uint32_t s = i / (p.rows * 16u), rc = i % (p.rows * 16u);
+        const uint32_t r = rc >> 4, c = rc & 15u;
+        const uint32_t col = (s0 + s) * 16u + c;
+        float sum = RED[0][s][r][c];
+#pragma unroll
+        for (uint32_t wv = 1; wv < kWaves; ++wv) sum += RED[wv][s][r][c];
+        if constexpr (kSum) {
+            const uint32_t pr = PAR[s][c];
+            sum = sum * half_bits_to_f32(pr & 0xFFFFu);
+        }
+        if (col < p.n) {
+            const size_t idx = static_cast<size_t>(r) * p.n + col;
+            if (p.out_f32) {
+                static_cast<float*>(p.y)[idx] = sum;
+            } else {
+                static_cast<uint16_t*>(p.y)[idx] = static_cast<uint16_t>(f32_to_half_bits(sum));
+            }
+        }
+    }
+}
+
 // ---- many activation rows: a half GEMM whose B-tile loader de-quantises.
 // Workgroup = 4 wavefronts (2 x 2) on a 128 x 128 tile, K step 64, two LDS stages of 32 KiB (two workgroups per compute
 // unit).  Both tiles sit in LDS as [row or column][64 k] halves, 128 bytes per line in 8 pieces of 16 bytes, piece c of
@@ -428,7 +647,8 @@ bool w8a16_nk_supported(uint32_t k, const void* x, const void* w)
 }
 
 int launch_w8a16_nk(const void* x, const void* w, const void* scale, const void* offset, void* y, uint32_t m, uint32_t n,
-                    uint32_t k, bool has_offset, bool out_f32, uint32_t scale_bits, uint32_t offset_bits, hipStream_t st);
+                    uint32_t k, bool has_offset, bool out_f32, uint32_t scale_bits, uint32_t offset_bits, hipStream_t st,
+                    bool channel_sum);
 
 // Weights given as [k, n] and many rows: transposed once into the caller's workspace (k * n bytes), then the tile GEMM.
 bool w8a16_kn_gemm_supported(uint32_t m, uint32_t k, const void* x, const void* w)
@@ -446,13 +666,53 @@ int launch_w8a16_kn_via_transpose(const void* x, const void* w, const void* scal
     } else {
         transpose_i8_kernel<false><<<tiles, 256, 0, st>>>(static_cast<const uint8_t*>(w), static_cast<uint8_t*>(workspace), k, n);
     }
-    return launch_w8a16_nk(x, workspace, scale, offset, y, m, n, k, has_offset, out_f32, scale_bits, offset_bits, st);
+    return launch_w8a16_nk(x, workspace, scale, offset, y, m, n, k, has_offset, out_f32, scale_bits, offset_bits, st,
+                           false);
 }
 
 // x, y: first row of the whole problem; m rows in passes of 16.
 int launch_w8a16_nk(const void* x, const void* w, const void* scale, const void* offset, void* y, uint32_t m, uint32_t n,
-                    uint32_t k, bool has_offset, bool out_f32, uint32_t scale_bits, uint32_t offset_bits, hipStream_t st)
+                    uint32_t k, bool has_offset, bool out_f32, uint32_t scale_bits, uint32_t offset_bits, hipStream_t st,
+                    bool channel_sum)
 {
+    // up to 4 rows (k % 64 == 0, offsets that fit the buffer loads' 31 bits, activations that fit the LDS): the stream
+    // kernel with the activations resident
+    if (m <= kSkMaxRows && k % kSkTileK == 0 && static_cast<uint64_t>(n + 16u) * k < (1ull << 31) - 64u * kSkTileK) {
+        SkParams q{};
+        q.x = static_cast<const uint16_t*>(x);
+        q.w = static_cast<const uint8_t*>(w);
+        q.scale = static_cast<const uint16_t*>(scale);
+        q.offset = static_cast<const uint16_t*>(offset);
+        q.y = y;
+        q.rows = m;
+        q.n = n;
+        q.k = k;
+        q.slabs = (n + 15u) / 16u;
+        q.ktiles = k / kSkTileK;
+        q.tpw = (q.ktiles + kWaves - 1u) / kWaves;
+        q.out_f32 = out_f32 ? 1u : 0u;
+        q.scale_bits = scale_bits;
+        q.offset_bits = offset_bits;
+        if (kWaves * m * (q.tpw * kSkTileK * 2u + kSkRowPad) <= kSkXBytes) {
+            const uint32_t cus = device_compute_units();
+            uint32_t grid = q.slabs < cus ? q.slabs : cus;
+            if ((q.slabs + grid - 1u) / grid > kSkMaxSlabs) {
+                grid = (q.slabs + kSkMaxSlabs - 1u) / kSkMaxSlabs;
+            }
+            if (channel_sum) {
+                if (has_offset) {
+                    w8a16_nk_stream_kernel<true, true><<<grid, kWaves * 64u, 0, st>>>(q);
+                } else {
+                    w8a16_nk_stream_kernel<false, true><<<grid, kWaves * 64u, 0, st>>>(q);
+                }
+            } else if (has_offset) {
+                w8a16_nk_stream_kernel<true, false><<<grid, kWaves * 64u, 0, st>>>(q);
+            } else {
+                w8a16_nk_stream_kernel<false, false><<<grid, kWaves * 64u, 0, st>>>(q);
+            }
+            return launch_status("ascq_matmul_w8a16");
+        }
+    }
     NkParams p{};
     p.w = static_cast<const uint8_t*>(w);
     p.scale = static_cast<const uint16_t*>(scale);

@@ -1134,7 +1134,8 @@ extern "C" int ascq_matmul_w4a16(const ascq_w4a16_desc* d, void* y, const void* 
 namespace ascq {
 bool w8a16_nk_supported(uint32_t k, const void* x, const void* w);
 int launch_w8a16_nk(const void* x, const void* w, const void* scale, const void* offset, void* y, uint32_t m, uint32_t n,
-                    uint32_t k, bool has_offset, bool out_f32, uint32_t scale_bits, uint32_t offset_bits, hipStream_t st);
+                    uint32_t k, bool has_offset, bool out_f32, uint32_t scale_bits, uint32_t offset_bits, hipStream_t st,
+                    bool channel_sum);
 bool w8a16_kn_gemm_supported(uint32_t m, uint32_t k, const void* x, const void* w);
 int launch_w8a16_kn_via_transpose(const void* x, const void* w, const void* scale, const void* offset, void* y,
                                   uint32_t m, uint32_t n, uint32_t k, bool has_offset, bool out_f32, uint32_t scale_bits,
@@ -1147,6 +1148,8 @@ static int validate_w8a16(const ascq_w8a16_desc* d)
     ASCQ_REQUIRE(d->m > 0 && d->n > 0 && d->k > 0, ASCQ_EINVAL, "ascq_matmul_w8a16: m, n, k must be greater than 0");
     ASCQ_REQUIRE(d->out_dtype == ASCQ_F16 || d->out_dtype == ASCQ_F32, ASCQ_EUNSUPPORTED,
                  "ascq_matmul_w8a16: out_dtype must be ASCQ_F16 or ASCQ_F32");
+    ASCQ_REQUIRE(d->mode == ASCQ_W8A16_PER_WEIGHT || d->mode == ASCQ_W8A16_CHANNEL_SUM, ASCQ_EINVAL,
+                 "ascq_matmul_w8a16: unknown mode %d", d->mode);
     return ASCQ_OK;
 }
 
@@ -1229,7 +1232,7 @@ extern "C" int ascq_matmul_w8a16(const ascq_w8a16_desc* d, void* y, const void* 
     }
     if (d->trans_b) {
         return launch_w8a16_nk(x, w, p.scale, p.offset, y, d->m, d->n, d->k, d->has_offset != 0, d->out_dtype == ASCQ_F32,
-                               p.scale_bits, p.offset_bits, st);
+                               p.scale_bits, p.offset_bits, st, d->mode == ASCQ_W8A16_CHANNEL_SUM);
     }
     if (w8a16_kn_gemm_supported(d->m, d->k, x, w) && workspace != nullptr && aligned16(workspace) &&
         workspace_bytes >= static_cast<size_t>(d->k) * d->n) {

@@ -64,7 +64,7 @@ def main():
     ap.add_argument("--quick", action="store_true", help="headline + W4A16 GEMV only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="run a single workload: w8a8 | w4a16 | w4a16_per_weight | w4a16_per_weight_m4 | w4a16_per_weight_m16 | w4a16_nd | w4a16_m4 | w4a16_m16 | w4a16_nd_m4 | w4a16_nd_m16 | "
-                         "w8a8_zeros | w8a8_m1 | w8a8_m8 | w8a8_m16 | w8a8_m128 | w8a8_m512 | w8a8_m8192 | w8a8_packed_m1 | w8a8_packed_m8 | w8a8_packed_m16 | w8a8_nk_m1 | w8a8_nk_m16 | w8a8_nk_m128 | w8a16_m1 | w8a16_m16 | w8a16_nk_m1 | "
+                         "w8a8_zeros | w8a8_m1 | w8a8_m8 | w8a8_m16 | w8a8_m128 | w8a8_m512 | w8a8_m8192 | w8a8_packed_m1 | w8a8_packed_m8 | w8a8_packed_m16 | w8a8_nk_m1 | w8a8_nk_m16 | w8a8_nk_m128 | w8a16_m1 | w8a16_m16 | w8a16_nk_m1 | w8a16_nk_m4 | w8a16_nk_sum_m1 | w8a16_nk_sum_m4 | "
                          "w8a16_nk_m16 | w8a16_m2048 | w8a16_nk_m2048 | quant | dequant | antiquant | group | group_example | mx_fp4 | mx_fp4_e1m2 | mx_fp8 (a W4A16 name without _nd "
                          "is the packed-weight path, in the group-sum form unless it says per_weight; _nk: weights kept as [n, k])")
     ap.add_argument("--copy-probe", action="store_true",
@@ -250,7 +250,7 @@ def main():
                 "tops": 2.0 * M * K * N / (kern_ms * 1e-3) / 1e12, "tensors": (xs, ws[0], sc[0], of[0])}
 
     # ------------------------------------------------------------------ W8A16 decode (Matmul anti-quant path)
-    def w8a16(M, steps, warmup, sets=3, b_nk=False):
+    def w8a16(M, steps, warmup, sets=3, b_nk=False, mode=abi.W8A16_PER_WEIGHT):
         K, N = 8192, 28672
         xs = torch.randn((M, K), device=dev, generator=gen).to(torch.float16)
         ws = [rand_i8(N, K) if b_nk else rand_i8(K, N) for _ in range(sets)]
@@ -260,7 +260,7 @@ def main():
 
         def step(i, starts, stops):
             j = i % sets
-            bracket(starts, stops, lambda: ops.matmul_w8a16(y, xs, ws[j], of[j], sc[j], trans_b=b_nk))
+            bracket(starts, stops, lambda: ops.matmul_w8a16(y, xs, ws[j], of[j], sc[j], trans_b=b_nk, mode=mode))
 
         ms, kern_ms = timed(step, steps, warmup, settle=min(args.settle, 300 if M <= 64 else 20))
         bytes_ = K * N + 2 * N * 2 + M * K * 2 + M * N * 2
@@ -418,6 +418,9 @@ def main():
               "w8a8_nk_m1": lambda: w8a8(1, args.steps, args.warmup, sets=7, b_nk=True),
               "w8a8_nk_m16": lambda: w8a8(16, args.steps, args.warmup, sets=7, b_nk=True),
               "w8a16_nk_m1": lambda: w8a16(1, args.steps, args.warmup, b_nk=True),
+              "w8a16_nk_sum_m1": lambda: w8a16(1, args.steps, args.warmup, b_nk=True, mode=abi.W8A16_CHANNEL_SUM),
+              "w8a16_nk_sum_m4": lambda: w8a16(4, args.steps, args.warmup, b_nk=True, mode=abi.W8A16_CHANNEL_SUM),
+              "w8a16_nk_m4": lambda: w8a16(4, args.steps, args.warmup, b_nk=True),
               "w8a16_nk_m16": lambda: w8a16(16, args.steps, args.warmup, b_nk=True),
               "w8a16_nk_m2048": lambda: w8a16(2048, min(args.steps, 30), min(args.warmup, 5), sets=1, b_nk=True),
               "w8a16_m2048": lambda: w8a16(2048, min(args.steps, 30), min(args.warmup, 5), sets=1),
@@ -566,6 +569,12 @@ def main():
                                                      "hbm_frac": r["gbs"] / PEAK_HBM_GBS,
                                                      "note": "weights kept as [n, k]: one launch, no workspace"}
             torch.cuda.empty_cache()
+            if M == 1:
+                r = w8a16(M, s2, w2, b_nk=True, mode=abi.W8A16_CHANNEL_SUM)
+                others["w8a16_nk_channel_sum_m1_k8192_n28672"] = {
+                    "kernel_ms": r["kernel_ms"], "gbs": r["gbs"], "bytes": r["bytes"], "hbm_frac": r["gbs"] / PEAK_HBM_GBS,
+                    "mode": "ASCQ_W8A16_CHANNEL_SUM", "note": "weights kept as [n, k]: one launch, no workspace"}
+                torch.cuda.empty_cache()
         for nk in (True, False):
             r = w8a16(2048, 30, 5, sets=1, b_nk=nk)
             others["w8a16_nk_m2048_k8192_n28672" if nk else "w8a16_m2048_k8192_n28672"] = {

@@ -567,6 +567,16 @@ int ascq_matmul_w4a16_packed(const ascq_w4a16_desc* desc, void* y, const void* x
  * workspace: ascq_matmul_w8a16_workspace_size bytes (contents need not be initialised); calls that share a
  * workspace must not overlap.
  */
+/* How the de-quantisation is carried out (ascq_w8a16_desc.mode).
+ * PER_WEIGHT (0, the default): the reference's arithmetic, f16(scale * f16(f16(w) + offset)) for every weight, then the
+ *   half matmul with fp32 sums.
+ * CHANNEL_SUM: y[i,j] = out( scale[j] * ( sum_k x[i,k] w[k,j] + offset[j] * sum_k x[i,k] ) ) with both sums in fp32 and
+ *   the int8 weights as exact halves: scale and offset applied once per output instead of twice rounded per weight.
+ *   Not the reference's bits; within one bf16 ulp and 1e-3 relative of them (and closer to the exact value of the
+ *   quantised product).  Honoured for up to 4 rows on [n, k] weights (trans_b) with k % 128 == 0; elsewhere the
+ *   per-weight form runs. */
+typedef enum ascq_w8a16_mode { ASCQ_W8A16_PER_WEIGHT = 0, ASCQ_W8A16_CHANNEL_SUM = 1 } ascq_w8a16_mode;
+
 typedef struct ascq_w8a16_desc {
     uint32_t m, n, k;
     int32_t per_tensor;  /* 1: scale / offset below (SetAntiQuantScalar); 0: vectors of n halves (SetAntiQuantVector) */
@@ -574,6 +584,7 @@ typedef struct ascq_w8a16_desc {
     float scale, offset; /* per-tensor parameters, rounded to half as the reference's half scalars */
     int32_t out_dtype;   /* ASCQ_F16 | ASCQ_F32 */
     int32_t trans_b;     /* 0: w is [k, n]; 1: w is [n, k] */
+    int32_t mode;        /* ascq_w8a16_mode */
 } ascq_w8a16_desc;
 
 int ascq_matmul_w8a16(const ascq_w8a16_desc* desc, void* y, const void* x, const void* w, const void* offset,

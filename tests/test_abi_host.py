@@ -35,7 +35,7 @@ def test_struct_sizes_match_the_header():
     assert C.sizeof(abi.MatmulDesc) == 11 * 4 + 4 + 8 + 8
     assert C.sizeof(abi.GroupMatmulDesc) == C.sizeof(abi.MatmulDesc) + 8
     assert C.sizeof(abi.W4A16Desc) == 6 * 4
-    assert C.sizeof(abi.W8A16Desc) == 9 * 4
+    assert C.sizeof(abi.W8A16Desc) == 10 * 4
     assert C.sizeof(abi.AntiQuantPolicyDesc) == 14 * 4
     assert C.sizeof(abi.MxDesc) == 8 * 4
 
@@ -388,7 +388,8 @@ def test_hifloat8_surface_and_refused_round_modes():
 def test_w8a16_transposed_weights_surface():
     """[n, k] weights: no workspace at any k (a k off the kernels' 128-element steps runs the one-lane-per-output
     kernel, which needs none either); the descriptor carries trans_b as its last field."""
-    assert C.sizeof(abi.W8A16Desc) == 9 * 4 and abi.W8A16Desc._fields_[-1][0] == "trans_b"
+    assert C.sizeof(abi.W8A16Desc) == 10 * 4 and abi.W8A16Desc._fields_[-2][0] == "trans_b"
+    assert abi.W8A16Desc._fields_[-1][0] == "mode" and (abi.W8A16_PER_WEIGHT, abi.W8A16_CHANNEL_SUM) == (0, 1)
     need = C.c_size_t(77)
     d = abi.W8A16Desc(m=4, n=64, k=256, per_tensor=1, scale=0.5, out_dtype=abi.F16, trans_b=1)
     assert L.ascq_matmul_w8a16_workspace_size(C.byref(d), C.byref(need)) == abi.OK and need.value == 0

@@ -789,6 +789,62 @@ def test_w8a16_trans_b(m, k, n, mode):
                                                       None if per_tensor else sc)).view(np.uint8))
 
 
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5])
+@pytest.mark.parametrize("k,n", [(128, 16), (256, 256), (512, 1040), (384, 30), (2048, 520), (8192, 144)])
+@pytest.mark.parametrize("mode", ["vector+offset", "vector", "scalar+offset", "scalar"])
+def test_w8a16_trans_b_channel_sum(m, k, n, mode):
+    """ASCQ_W8A16_CHANNEL_SUM on [n, k] weights: scale and offset applied once per output to fp32 sums.  Same oracle
+    (the per-weight arithmetic), the tolerance of a half output: every element within one bfloat16 ulp, the row error
+    within 1e-3; 5 rows run the per-weight kernel and pass the same gate.  Two calls give identical bits."""
+    announce("w8a16 [n, k] channel sum", m, k, n, mode)
+    rng = np.random.default_rng(m * 11 + k + n)
+    x = rng.standard_normal((m, k)).astype(np.float16)
+    wt = rng.integers(-128, 128, (n, k)).astype(np.int8)
+    per_tensor = mode.startswith("scalar")
+    has_offset = "offset" in mode
+    if per_tensor:
+        sc, of = 0.0077, (2.5 if has_offset else None)
+    else:
+        sc = rng.uniform(1e-3, 1e-2, n).astype(np.float16)
+        of = rng.uniform(-9, 9, n).astype(np.float16) if has_offset else None
+    ys = []
+    for _ in range(2):
+        y = torch.zeros((m, n), dtype=torch.float16, device=DEV)
+        y.view(torch.int16).fill_(0x7E7E)
+        ops.matmul_w8a16(y, to_dev(x), to_dev(wt), of if per_tensor else (None if of is None else to_dev(of)),
+                         sc if per_tensor else to_dev(sc), workspace=torch.empty(4, device=DEV), trans_b=True,
+                         mode=abi.W8A16_CHANNEL_SUM)
+        ys.append(y.cpu().numpy())
+    assert np.array_equal(ys[0].view(np.uint16), ys[1].view(np.uint16))
+    d = abi.W8A16Desc(m=m, n=n, k=k, per_tensor=int(per_tensor), has_offset=int(has_offset),
+                      scale=sc if per_tensor else 0.0, offset=of if per_tensor and has_offset else 0.0,
+                      out_dtype=abi.F16, trans_b=1)
+    want = orc.matmul_w8a16(d, x, wt, None if per_tensor else of, None if per_tensor else sc)
+    w4_group_sum_gate(ys[0], np.asarray(want))
+
+
+def test_w8a16_channel_sum_is_the_real_number_value():
+    """The channel-sum form rounds the exact value of the quantised product once; the per-weight form carries two
+    roundings per weight.  Against float64 arithmetic on the same quantised inputs the channel-sum result is at least
+    as close, on average, as the per-weight one."""
+    announce("w8a16 channel sum against float64")
+    rng = np.random.default_rng(91)
+    m, k, n = 4, 4096, 1024
+    x = rng.standard_normal((m, k)).astype(np.float16)
+    wt = rng.integers(-128, 128, (n, k)).astype(np.int8)
+    sc = rng.uniform(1e-3, 1e-2, n).astype(np.float16)
+    of = rng.uniform(-9, 9, n).astype(np.float16)
+    exact = (x.astype(np.float64) @ (wt.astype(np.float64).T + of.astype(np.float64)[None, :])) * sc.astype(np.float64)[None, :]
+    errs = []
+    for mode in (abi.W8A16_PER_WEIGHT, abi.W8A16_CHANNEL_SUM):
+        y = torch.zeros((m, n), dtype=torch.float32, device=DEV)
+        ops.matmul_w8a16(y, to_dev(x), to_dev(wt), to_dev(of), to_dev(sc), workspace=torch.empty(4, device=DEV), trans_b=True,
+                         mode=mode)
+        errs.append(np.abs(y.cpu().numpy().astype(np.float64) - exact).mean())
+    assert errs[1] <= errs[0]
+    assert errs[1] <= 1e-5 * np.abs(exact).mean()
+
+
 @pytest.mark.parametrize("m", [1, 16])
 def test_w8a16_trans_b_exact_integers_full_size(m):
     """K=8192, N=28672 as [n, k]: small integer activations, power-of-two scales and integer offsets make every partial
