@@ -231,6 +231,7 @@ int launch_gemm_nk(const GemmParams& p, hipStream_t st);
 // (matmul_w8a8_packed.hip).
 bool gemm_packed_supported(const GemmParams& p);
 bool gemm_packed_nk_supported(const GemmParams& p);
+bool gemm_packed_two_tiles_fit(uint32_t k);  // 17 to 32 rows in one pass over the weights
 int launch_gemm_packed(const GemmParams& p, hipStream_t st, bool b_nk = false);
 
 }  // namespace ascq

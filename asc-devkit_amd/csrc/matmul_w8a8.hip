@@ -739,7 +739,8 @@ extern "C" int ascq_matmul_w8a8(const ascq_matmul_desc* d, void* c, const void* 
         workspace_bytes >= gemm_stream_workspace(d->m, d->n, d->k)) {
         return launch_gemm_stream(p, workspace, st);
     }
-    if (d->m <= 16 && d->trans_b && !d->trans_a && gemm_packed_nk_supported(p)) {
+    if (d->m <= 32 && d->trans_b && !d->trans_a && gemm_packed_nk_supported(p) &&
+        (d->m <= 16 || gemm_packed_two_tiles_fit(d->k))) {
         return launch_gemm_packed(p, st, true);  // activations resident in LDS, nothing but weights in the load queue
     }
     if (d->m <= 32 && d->trans_b && !d->trans_a && gemm_nk_supported(p)) {

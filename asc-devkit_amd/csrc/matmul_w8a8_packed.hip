@@ -32,6 +32,9 @@ constexpr uint32_t kPkWaves = 8, kPkBatch = 4, kPkMaxSlabs = 8, kPkMaxRows = 16;
 constexpr int kPkBuf = 2;              // register buffers: one batch in flight while the other is computed
 constexpr uint32_t kPkRowPad = 16;     // bytes added to a staged activation row: rows start 4 banks apart
 constexpr uint32_t kPkXBytes = 88 * 1024;  // LDS for the staged activations of a workgroup (the partial sums take 64 KiB)
+// With two row tiles (17 to 32 rows per pass) the activations take up to 136 KiB and the wavefronts add their tiles
+// into one [slab][row][column] array with LDS atomics (integers: exact in any order) instead of keeping eight copies.
+constexpr uint32_t kPkXBytes2 = 136 * 1024;
 constexpr uint32_t kPkPastEnd = 0x7FFFFFF0u;
 constexpr int kPkNt = 2;               // cache policy of the weight loads: non-temporal (read once per call)
 
@@ -55,11 +58,11 @@ __device__ __forceinline__ uint32_t pk_xcd_order(uint32_t wg, uint32_t wgs)
     return (wgs & 7u) == 0u ? (wg & 7u) * (wgs >> 3) + (wg >> 3) : wg;
 }
 
-template <bool kNK>
+template <bool kNK, int RT>
 __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_kernel(PackedParams p)
 {
-    __shared__ __attribute__((aligned(16))) char XS[kPkXBytes];
-    __shared__ int32_t RED[kPkWaves][kPkMaxSlabs][4][64];
+    __shared__ __attribute__((aligned(16))) char XS[RT == 2 ? kPkXBytes2 : kPkXBytes];
+    __shared__ int32_t RED[RT == 2 ? 1 : kPkWaves][kPkMaxSlabs][RT == 2 ? 8 : 4][64];  // RT == 2: [slab][row / 4][..]
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t lc = lane & 15u, lq = lane >> 4;
@@ -88,8 +91,15 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_kernel(PackedParams
         const_cast<i32x4*>(p.wp), 0,
         static_cast<int>(kNK ? p.n * p.k : (p.slabs * p.ktiles + kPkPadTiles) * kPkTileBytes), 0x00020000);
     const uint32_t w_lane = kNK ? lc * p.k + lq * 16u : lane * 16u;  // the lane's 16 bytes inside a tile
-    // operand row i reads row i % rows; + tile * 64
+    // operand row i reads row i % rows; + tile * 64.  Second row tile (RT == 2, more than 16 rows): rows 16 + i, past
+    // the end the last row again (never stored).
     const uint32_t x_lane = (lc - __umulhi(lc, p.rows_magic) * p.rows) * pitch + lq * 16u;
+    const uint32_t x_lane2 = min(16u + lc, p.rows - 1u) * pitch + lq * 16u;
+    if constexpr (RT == 2) {
+        // the shared sums start at zero; the barrier also orders this against the first atomic
+        for (uint32_t i = tid; i < kPkMaxSlabs * 8u * 64u; i += kPkWaves * 64u) (&RED[0][0][0][0])[i] = 0;
+        __syncthreads();
+    }
 
     // ---- batches of kPkBatch tiles that never straddle a slab: batch q = (slab q / nb, tiles ta + (q % nb) kPkBatch ...)
     const uint32_t nb = (cnt + kPkBatch - 1u) / kPkBatch;
@@ -127,7 +137,7 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_kernel(PackedParams
     __builtin_amdgcn_s_waitcnt(((kPkBuf * kPkBatch) & 15) | (((kPkBuf * kPkBatch) >> 4) << 14) | (7 << 4) | (15 << 8));
     asm volatile("" ::: "memory");
 
-    i32x4 acc = {0, 0, 0, 0};
+    i32x4 acc = {0, 0, 0, 0}, acc2 = {0, 0, 0, 0};
     uint32_t c_slab = 0, c_b = 0, c_q = 0;
     auto compute = [&](int buf) __attribute__((always_inline)) {
         if (c_q >= batches) {
@@ -141,12 +151,26 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_kernel(PackedParams
             if (t < live) {  // uniform
                 const i32x4 a = *reinterpret_cast<const i32x4*>(xa0 + t * kPkTileK);
                 acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, wq[buf][t], acc, 0, 0, 0);
+                if constexpr (RT == 2) {
+                    const i32x4 a2 = *reinterpret_cast<const i32x4*>(xs + x_lane2 + (t0 + t) * kPkTileK);
+                    acc2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a2, wq[buf][t], acc2, 0, 0, 0);
+                }
             }
         }
         ++c_q;
         if (++c_b == nb) {  // the slab is done: register i of lane l is row 4 (l / 16) + i, column l % 16
+            if constexpr (RT == 2) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) RED[wave][c_slab][i][lane] = acc[i];
+                for (int i = 0; i < 4; ++i) {
+                    __hip_atomic_fetch_add(&RED[0][c_slab][i][lane], acc[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    __hip_atomic_fetch_add(&RED[0][c_slab][4 + i][lane], acc2[i], __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_WORKGROUP);
+                }
+                acc2 = i32x4{0, 0, 0, 0};
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) RED[wave][c_slab][i][lane] = acc[i];
+            }
             acc = i32x4{0, 0, 0, 0};
             c_b = 0;
             ++c_slab;
@@ -159,7 +183,7 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_kernel(PackedParams
             load(b);
         }
     }
-    if (batches == 0u) {  // a wavefront without tiles (k shorter than 8 tiles) contributes zeros
+    if (RT == 1 && batches == 0u) {  // a wavefront without tiles (k shorter than 8 tiles) contributes zeros
         for (uint32_t s = 0; s < nslabs; ++s) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) RED[wave][s][i][lane] = 0;
@@ -178,14 +202,16 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_kernel(PackedParams
         const float bp = load_bias_post(e, col);
         const int32_t bias_pre = e.bias_kind == ASCQ_MM_BIAS_I32_PRE ? static_cast<const int32_t*>(e.bias)[col] : 0;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const uint32_t row_in_pass = 4u * lq + static_cast<uint32_t>(i);
+        for (int i = 0; i < 4 * RT; ++i) {
+            const uint32_t row_in_pass = 16u * (i >> 2) + 4u * lq + static_cast<uint32_t>(i & 3);
             if (row_in_pass >= p.rows) {
                 continue;
             }
             int32_t sum = RED[0][s][i][lane];
+            if constexpr (RT == 1) {
 #pragma unroll
-            for (uint32_t wv = 1; wv < kPkWaves; ++wv) sum += RED[wv][s][i][lane];
+                for (uint32_t wv = 1; wv < kPkWaves; ++wv) sum += RED[wv][s][i][lane];
+            }
             sum += bias_pre;
             const uint32_t row = p.m0 + row_in_pass;
             const float tok = e.has_tok ? e.tok_scale[row] : 1.0f;
@@ -236,6 +262,12 @@ bool gemm_packed_nk_supported(const GemmParams& p)
            static_cast<uint64_t>(p.n + kPkCols) * p.k < (1ull << 31) - 64u * kPkTileK;
 }
 
+bool gemm_packed_two_tiles_fit(uint32_t k)
+{
+    const uint32_t tpw = (k / kPkTileK + kPkWaves - 1u) / kPkWaves;
+    return 2u * kPkMaxRows * kPkWaves * (tpw * kPkTileK + kPkRowPad) <= kPkXBytes2;
+}
+
 bool gemm_packed_supported(const GemmParams& p)
 {
     return p.k % kPkTileK == 0 && aligned16(p.a) && aligned16(p.b) &&
@@ -260,24 +292,35 @@ int launch_gemm_packed(const GemmParams& p, hipStream_t st, bool b_nk)
     if ((q.slabs + grid - 1u) / grid > kPkMaxSlabs) {
         grid = (q.slabs + kPkMaxSlabs - 1u) / kPkMaxSlabs;
     }
-    // rows per pass: 16, fewer when k is so long that the staged activations of 16 rows would not fit the LDS
-    uint32_t pass_rows = kPkXBytes / (kPkWaves * (q.tpw * kPkTileK + kPkRowPad));
+    // rows per pass: 16, fewer when k is so long that the staged activations of 16 rows would not fit the LDS; 32 (two
+    // row tiles sharing every weight fetch) while more than 16 rows are left and 32 rows fit the larger staging area
+    const uint32_t row_bytes = kPkWaves * (q.tpw * kPkTileK + kPkRowPad);
+    uint32_t pass_rows = kPkXBytes / row_bytes;
     pass_rows = pass_rows > kPkMaxRows ? kPkMaxRows : pass_rows;
     if (pass_rows == 0u) {
         return fail(ASCQ_EUNSUPPORTED, "ascq_matmul_w8a8_packed: k = %u is too long for the staged activations", p.k);
     }
-    for (uint32_t m0 = 0; m0 < p.m; m0 += pass_rows) {
+    const bool two_tiles_fit = 2u * kPkMaxRows * row_bytes <= kPkXBytes2;
+    for (uint32_t m0 = 0; m0 < p.m; m0 += q.rows) {
+        const uint32_t left = p.m - m0;
+        const bool two = two_tiles_fit && left > kPkMaxRows;
         q.m0 = m0;
-        q.rows = p.m - m0 < pass_rows ? p.m - m0 : pass_rows;
+        q.rows = two ? (left < 2u * kPkMaxRows ? left : 2u * kPkMaxRows) : (left < pass_rows ? left : pass_rows);
         q.rows_magic = static_cast<uint32_t>(((1ull << 32) + q.rows - 1u) / q.rows);
-        if (plan_note(ASCQ_MM_KERNEL_STREAM, 16, 16 * ((q.slabs + grid - 1u) / grid), kPkTileK, grid, 1,
-                      kPkXBytes + kPkWaves * kPkMaxSlabs * 1024u, 0)) {
+        if (plan_note(ASCQ_MM_KERNEL_STREAM, two ? 32 : 16, 16 * ((q.slabs + grid - 1u) / grid), kPkTileK, grid, 1,
+                      two ? kPkXBytes2 + kPkMaxSlabs * 8u * 256u : kPkXBytes + kPkWaves * kPkMaxSlabs * 1024u, 0)) {
             return ASCQ_OK;
         }
-        if (b_nk) {
-            gemm_packed_kernel<true><<<grid, kPkWaves * 64u, 0, st>>>(q);
+        if (two) {
+            if (b_nk) {
+                gemm_packed_kernel<true, 2><<<grid, kPkWaves * 64u, 0, st>>>(q);
+            } else {
+                gemm_packed_kernel<false, 2><<<grid, kPkWaves * 64u, 0, st>>>(q);
+            }
+        } else if (b_nk) {
+            gemm_packed_kernel<true, 1><<<grid, kPkWaves * 64u, 0, st>>>(q);
         } else {
-            gemm_packed_kernel<false><<<grid, kPkWaves * 64u, 0, st>>>(q);
+            gemm_packed_kernel<false, 1><<<grid, kPkWaves * 64u, 0, st>>>(q);
         }
     }
     return launch_status(b_nk ? "ascq_matmul_w8a8 ([n, k] weight stream)" : "ascq_matmul_w8a8_packed");

@@ -184,12 +184,13 @@ def test_pack_weight_w8_layout(k, n):
     assert np.array_equal(ops.pack_weight_w8(to_dev(np.ascontiguousarray(w.T)), k, n, trans_b=True).cpu().numpy(), want)
 
 
-@pytest.mark.parametrize("m", [1, 2, 3, 5, 8, 16, 17, 33])
+@pytest.mark.parametrize("m", [1, 2, 3, 5, 8, 16, 17, 20, 31, 32, 33, 50])
 @pytest.mark.parametrize("n,k", [(16, 64), (48, 128), (1040, 512), (272, 4096), (96, 8192), (32, 16384), (2064, 192)])
 def test_w8a8_packed_small(m, n, k):
     """The one-launch kernel on packed weights computes what ascq_matmul_w8a8 computes: int32 accumulators and the
     dequantising epilogues bit for bit against the oracle on the unpacked weights.  k of one tile (seven wavefronts
-    without work), column tails, more rows than a pass, k long enough for several batches per slab."""
+    without work), column tails, more rows than a pass, k long enough for several batches per slab; 17 to 32 rows in
+    one pass with two row tiles where the activations fit (k up to 4096), in passes of 16 or fewer where they do not."""
     announce("w8a8 packed", m, n, k)
     rng = np.random.default_rng(m * 31 + n + k)
     a, b = rand_i8(rng, (m, k)), rand_i8(rng, (k, n))
@@ -210,7 +211,7 @@ def test_w8a8_packed_small(m, n, k):
     assert max_ulp(bits(cg), oracle_mm(dg, a, b).view(np.uint16), "f16") <= 1
 
 
-@pytest.mark.parametrize("m", [1, 16])
+@pytest.mark.parametrize("m", [1, 16, 32])
 def test_config3_w8a8_linear_packed(m):
     """Config 3's decode sizes on packed weights: per-token quantisation on the GPU, one launch for the matmul, bf16
     output bit-exact against the oracle."""
