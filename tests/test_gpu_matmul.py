@@ -733,6 +733,31 @@ def test_w8a16_decode_shape(m):
     w8a16_check(y.cpu().numpy(), want, x, False)
 
 
+@pytest.mark.parametrize("m", [1, 4])
+@pytest.mark.parametrize("mode", [abi.W8A16_PER_WEIGHT, abi.W8A16_CHANNEL_SUM])
+def test_w8a16_decode_shape_weights_as_n_k(m, mode):
+    """fp16 [M, 8192] x int8 [28672, 8192] kept as [n, k] (the benchmark's decode shape), per-channel scale and offset,
+    on the stream kernel with the activations resident in LDS: the per-weight mode within the usual tolerance of a free
+    accumulation order, the channel-sum mode within one bfloat16 ulp per element and 1e-3 per row."""
+    announce("w8a16 decode [n, k]", m, mode)
+    rng = np.random.default_rng(0xB16 + m)
+    k, n = 8192, 28672
+    x = rng.standard_normal((m, k)).astype(np.float16)
+    wt = rng.integers(-128, 128, (n, k)).astype(np.int8)
+    sc = rng.uniform(1e-3, 1e-2, n).astype(np.float16)
+    of = rng.uniform(-9, 9, n).astype(np.float16)
+    y = torch.zeros((m, n), dtype=torch.float16, device=DEV)
+    ops.matmul_w8a16(y, to_dev(x), to_dev(wt), to_dev(of), to_dev(sc), workspace=torch.empty(4, device=DEV), trans_b=True,
+                     mode=mode)
+    d = abi.W8A16Desc(m=m, n=n, k=k, per_tensor=0, has_offset=1, out_dtype=abi.F16, trans_b=1)
+    orc.set_threads(16)
+    want = orc.matmul_w8a16(d, x, wt, of, sc)
+    if mode == abi.W8A16_PER_WEIGHT:
+        w8a16_check(y.cpu().numpy(), want, x, False)
+    else:
+        w4_group_sum_gate(y.cpu().numpy(), np.asarray(want))
+
+
 @pytest.mark.parametrize("m", [2, 16])
 def test_w8a16_exact_integers_full_size(m):
     """Small integer activations, power-of-two scales and integer offsets make every product and partial sum exact in
