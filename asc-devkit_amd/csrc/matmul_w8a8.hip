@@ -852,9 +852,10 @@ extern "C" int ascq_linear_w8a8_dynamic_workspace_size(const ascq_matmul_desc* d
 
 // The activation quantiser of a W8A8 linear and the matmul in one call: q, tok = dynamic per-token quantisation of x
 // (ascq_dynamic_quant_per_token), c = matmul(q, b) with the token scales in the epilogue; q and tok live in the
-// caller's workspace.  (A variant that quantised inside the weight-streaming matmul kernel for up to 8 rows - row
-// maxima per workgroup, quantisation in registers on the way into the MFMA operand - was bit-identical but not faster
-// than the two launches, 21 us against 20 us at m = 1, and is not kept.)  The reference composes this
+// caller's workspace.  Up to 4 rows of half / bfloat16 x on weights kept as [n, k] run as one launch instead: the
+// decode kernel quantises x inside every workgroup on its way into LDS (gemm_packed_dyn_kernel; the same bits, about
+// 12.5 us against 15.5 us at k = 4096, n = 11008; from 6 rows on the 256 redundant quantisations cost more than the
+// separate kernel's launch).  The reference composes this
 // from ReduceMax / AscendQuant PER_TOKEN and Matmul (impl/adv_api/detail/quantization/quant/
 // ascend_quant_per_group_3510_impl.h:142-178, include/adv_api/matmul/matmul.h:175-185).
 extern "C" int ascq_linear_w8a8_dynamic(const ascq_matmul_desc* d, int32_t x_dtype, void* c, const void* x,
@@ -884,6 +885,20 @@ extern "C" int ascq_linear_w8a8_dynamic(const ascq_matmul_desc* d, int32_t x_dty
     rc = validate_mm(&dd, "ascq_linear_w8a8_dynamic", c, x, b, bias, quant_vector, ws);
     if (rc != ASCQ_OK) {
         return rc;
+    }
+    if ((x_dtype == ASCQ_F16 || x_dtype == ASCQ_BF16) && d->trans_b && d->b_format == ASCQ_MM_B_ND &&
+        d->activation != ASCQ_MM_ACT_SWIGLU && aligned16(x) && gemm_packed_dyn_fits(d->m, d->k)) {
+        // decode on [n, k] weights: the quantisation happens inside the weight-streaming kernel (same bits, one launch)
+        GemmParams p{};
+        p.a = static_cast<const int8_t*>(x);  // only its alignment is looked at
+        p.b = static_cast<const int8_t*>(b);
+        p.m = d->m;
+        p.n = d->n;
+        p.k = d->k;
+        p.epi = make_epi(&dd, c, bias, quant_vector, reinterpret_cast<const float*>(ws));
+        if (gemm_packed_nk_supported(p)) {
+            return launch_gemm_packed_dyn(p, x, x_dtype == ASCQ_BF16, static_cast<hipStream_t>(stream), true);
+        }
     }
     int8_t* q = reinterpret_cast<int8_t*>(ws);
     float* tok = reinterpret_cast<float*>(ws + round256(static_cast<size_t>(d->m) * d->k));

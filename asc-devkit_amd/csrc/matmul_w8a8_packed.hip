@@ -220,6 +220,222 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_kernel(PackedParams
     }
 }
 
+// The decode kernel with the per-token quantisation of the activations inside (up to 4 rows of half or bfloat16 x):
+// q = ascq_dynamic_quant_per_token(x); c = matmul(q, w, tok_scale) in one launch, with those two calls' results bit for
+// bit.  Every workgroup needs all of x anyway, so every workgroup quantises it: a wavefront stages its k range of
+// every row as it is (2 bytes per element), the wavefronts exchange their rows' absolute maxima through LDS, and each
+// turns its own range into the int8 image the matrix instructions read, with the arithmetic of dynq_row_kernel:
+// inv = 127 / amax, the product rounded to the nearest integer, ties to even, by adding 1.5 * 2^23.  The weight
+// batches requested ahead of all this arrive meanwhile.  The quantisation costs every compute unit about 0.3 us per
+// row, which is why this form stops at 4 rows: from about 6 on the separate quantiser kernel (one pass over x by the
+// whole chip) is cheaper than 256 redundant ones.  The wavefronts' tiles are added into one LDS array with atomics.
+constexpr uint32_t kPkDynRows = 4;
+constexpr uint32_t kPkDynHBytes = 96 * 1024;   // the staged activations as they come (2 bytes per element)
+constexpr uint32_t kPkDynQBytes = 48 * 1024;   // their int8 image
+
+// The largest of the 64 lanes' values, none of which is negative or a NaN (so their bit patterns order like integers),
+// in every lane's copy of the result: four shifts inside the rows of 16 lanes and two row broadcasts, all in the
+// vector ALU, then lane 63 read back.
+__device__ __forceinline__ float pk_wave_max_nonneg(float v)
+{
+    int x = __float_as_int(v);
+    x = max(x, __builtin_amdgcn_update_dpp(0, x, 0x111, 0xF, 0xF, false));  // row_shr:1
+    x = max(x, __builtin_amdgcn_update_dpp(0, x, 0x112, 0xF, 0xF, false));  // row_shr:2
+    x = max(x, __builtin_amdgcn_update_dpp(0, x, 0x114, 0xF, 0xF, false));  // row_shr:4
+    x = max(x, __builtin_amdgcn_update_dpp(0, x, 0x118, 0xF, 0xF, false));  // row_shr:8
+    x = max(x, __builtin_amdgcn_update_dpp(0, x, 0x142, 0xA, 0xF, false));  // row_bcast:15 into rows 1 and 3
+    x = max(x, __builtin_amdgcn_update_dpp(0, x, 0x143, 0xC, 0xF, false));  // row_bcast:31 into rows 2 and 3
+    return __int_as_float(__builtin_amdgcn_readlane(x, 63));
+}
+
+template <bool kNK, bool kBf16>
+__global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_dyn_kernel(PackedParams p, const uint16_t* __restrict__ x)
+{
+    __shared__ __attribute__((aligned(16))) char XH[kPkDynHBytes];
+    __shared__ __attribute__((aligned(16))) char XS[kPkDynQBytes];
+    __shared__ int32_t OUT[kPkMaxSlabs][4][16];  // [slab][row][column]
+    __shared__ float ROWMAX[kPkWaves][kPkDynRows];
+    __shared__ float TOK[kPkDynRows];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t lc = lane & 15u, lq = lane >> 4;
+    const uint32_t wg = pk_xcd_order(blockIdx.x, gridDim.x);
+    const uint32_t s0 = static_cast<uint32_t>(static_cast<uint64_t>(wg) * p.slabs / gridDim.x);
+    const uint32_t s1 = static_cast<uint32_t>(static_cast<uint64_t>(wg + 1u) * p.slabs / gridDim.x);
+    const uint32_t nslabs = s1 - s0;
+    const uint32_t ta = min(wave * p.tpw, p.ktiles), tb = min(ta + p.tpw, p.ktiles), cnt = tb - ta;
+    const uint32_t pitch = p.tpw * kPkTileK + kPkRowPad;  // of an int8 row; a staged row is twice as long
+    char* const xh = XH + wave * (p.rows * 2u * pitch);
+    char* const xs = XS + wave * (p.rows * pitch);
+    const uint32_t row_pieces = cnt * (kPkTileK * 2u / 16u);  // 16-byte pieces (8 elements) of a staged row
+
+    // ---- this wavefront's k range of every row, as it is, straight into LDS
+    for (uint32_t r = 0; r < p.rows; ++r) {
+        const uint16_t* src = x + static_cast<size_t>(p.m0 + r) * p.k + ta * kPkTileK + lane * 8u;
+        for (uint32_t c0 = 0; c0 < row_pieces; c0 += 64u) {
+            if (c0 + lane < row_pieces) {
+                __builtin_amdgcn_global_load_lds((gptr_t)(src + c0 * 8u), (lds_ptr_t)(xh + r * 2u * pitch + c0 * 16u), 16, 0, 0);
+            }
+        }
+    }
+    const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<i32x4*>(p.wp), 0,
+        static_cast<int>(kNK ? p.n * p.k : (p.slabs * p.ktiles + kPkPadTiles) * kPkTileBytes), 0x00020000);
+    const uint32_t w_lane = kNK ? lc * p.k + lq * 16u : lane * 16u;
+    const uint32_t x_lane = (p.rows == 1u ? 0u : lc - __umulhi(lc, p.rows_magic) * p.rows) * pitch + lq * 16u;
+
+    const uint32_t nb = (cnt + kPkBatch - 1u) / kPkBatch;
+    const uint32_t batches = nb * nslabs;
+    i32x4 wq[kPkBuf][kPkBatch];
+    uint32_t l_slab = s0, l_b = 0, l_q = 0;
+    bool l_done = batches == 0u;
+    auto load = [&](int buf) __attribute__((always_inline)) {
+        const uint32_t l_w = l_done ? kPkPastEnd : w_lane;
+        constexpr uint32_t kStep = kNK ? kPkTileK : kPkTileBytes;
+        const uint32_t base = kNK ? l_slab * kPkCols * p.k + (ta + l_b * kPkBatch) * kPkTileK
+                                  : (l_slab * p.ktiles + ta + l_b * kPkBatch) * kPkTileBytes;  // scalar
+#pragma unroll
+        for (uint32_t t = 0; t < kPkBatch; ++t) {
+            wq[buf][t] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, l_w, base + t * kStep, kPkNt));
+        }
+        if (l_q + 1u < batches) {  // uniform
+            ++l_q;
+            if (++l_b == nb) {
+                l_b = 0;
+                ++l_slab;
+            }
+        } else {
+            l_done = true;
+        }
+    };
+#pragma unroll
+    for (int b = 0; b < kPkBuf; ++b) load(b);
+    // the staged activations have landed once at most the weight loads just issued are outstanding
+    __builtin_amdgcn_s_waitcnt(((kPkBuf * kPkBatch) & 15) | (((kPkBuf * kPkBatch) >> 4) << 14) | (7 << 4) | (15 << 8));
+    asm volatile("" ::: "memory");
+
+    // ---- absolute maximum of every row over this wavefront's range; the shared sums start at zero
+    auto widen = [](uint32_t half_bits) __attribute__((always_inline)) {
+        return kBf16 ? bf16_bits_to_f32(half_bits) : half_bits_to_f32(half_bits);
+    };
+    for (uint32_t i = tid; i < kPkMaxSlabs * 4u * 16u; i += kPkWaves * 64u) (&OUT[0][0][0])[i] = 0;
+#pragma unroll
+    for (uint32_t r = 0; r < kPkDynRows; ++r) {
+        if (r < p.rows) {  // uniform
+            float amax = 0.0f;
+            for (uint32_t c0 = 0; c0 < row_pieces; c0 += 64u) {
+                if (c0 + lane < row_pieces) {
+                    const u32x4 v = *reinterpret_cast<const u32x4*>(xh + r * 2u * pitch + (c0 + lane) * 16u);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        amax = fmaxf(amax, fabsf(widen(v[i] & 0xFFFFu)));
+                        amax = fmaxf(amax, fabsf(widen(v[i] >> 16)));
+                    }
+                }
+            }
+            const float wave_amax = pk_wave_max_nonneg(amax);
+            if (lane == 0u) {
+                ROWMAX[wave][r] = wave_amax;
+            }
+        }
+    }
+    // a plain barrier: the fence of __syncthreads() would also wait for the weight loads in flight
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    // ---- lane r works out row r's factor once; every lane then quantises its pieces of this wavefront's range
+    float lane_inv;
+    {
+        float amax = 0.0f;
+        if (lane < p.rows) {
+#pragma unroll
+            for (uint32_t wv = 0; wv < kPkWaves; ++wv) amax = fmaxf(amax, ROWMAX[wv][lane]);
+        }
+        const bool zero = !(amax > 0.0f);
+        lane_inv = zero ? 0.0f : 127.0f / amax;
+        if (tid < p.rows) {
+            TOK[tid] = zero ? 1.0f : amax / 127.0f;
+        }
+    }
+#pragma unroll
+    for (uint32_t r = 0; r < kPkDynRows; ++r) {
+        if (r < p.rows) {  // uniform
+            const float inv = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(lane_inv), static_cast<int>(r)));
+            for (uint32_t c0 = 0; c0 < row_pieces; c0 += 64u) {
+                if (c0 + lane < row_pieces) {
+                    const u32x4 v = *reinterpret_cast<const u32x4*>(xh + r * 2u * pitch + (c0 + lane) * 16u);
+                    uint32_t u[8];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float t0 = __builtin_amdgcn_fmed3f(widen(v[i] & 0xFFFFu) * inv, -128.0f, 127.0f);
+                        const float t1 = __builtin_amdgcn_fmed3f(widen(v[i] >> 16) * inv, -128.0f, 127.0f);
+                        u[2 * i] = __float_as_uint(t0 + 12582912.0f);
+                        u[2 * i + 1] = __float_as_uint(t1 + 12582912.0f);
+                    }
+                    u32x2 out;
+                    out[0] = __builtin_amdgcn_perm(u[1], u[0], 0x0c0c0400u) | __builtin_amdgcn_perm(u[3], u[2], 0x04000c0cu);
+                    out[1] = __builtin_amdgcn_perm(u[5], u[4], 0x0c0c0400u) | __builtin_amdgcn_perm(u[7], u[6], 0x04000c0cu);
+                    *reinterpret_cast<u32x2*>(xs + r * pitch + (c0 + lane) * 8u) = out;
+                }
+            }
+        }
+    }
+    // (the matrix operands below are read by the wavefront that wrote them: LDS operations of a wavefront stay in order)
+
+    i32x4 acc = {0, 0, 0, 0};
+    uint32_t c_slab = 0, c_b = 0, c_q = 0;
+    auto compute = [&](int buf) __attribute__((always_inline)) {
+        if (c_q >= batches) {
+            return;  // uniform
+        }
+        const uint32_t t0 = c_b * kPkBatch;
+        const uint32_t live = min(kPkBatch, cnt - t0);
+        const char* xa0 = xs + x_lane + t0 * kPkTileK;
+#pragma unroll
+        for (uint32_t t = 0; t < kPkBatch; ++t) {
+            if (t < live) {  // uniform
+                const i32x4 a = *reinterpret_cast<const i32x4*>(xa0 + t * kPkTileK);
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, wq[buf][t], acc, 0, 0, 0);
+            }
+        }
+        ++c_q;
+        if (++c_b == nb) {  // the slab is done: register i of lanes 0 .. 15 is row i, column = lane
+            if (lane < 16u) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    __hip_atomic_fetch_add(&OUT[c_slab][i][lane], acc[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                }
+            }
+            acc = i32x4{0, 0, 0, 0};
+            c_b = 0;
+            ++c_slab;
+        }
+    };
+    for (uint32_t q = 0; q < batches; q += kPkBuf) {
+#pragma unroll
+        for (int b = 0; b < kPkBuf; ++b) {
+            compute(b);
+            load(b);
+        }
+    }
+    __syncthreads();
+
+    // ---- element (row, column) of slab s is handled by thread s * 64 + row * 16 + column
+    const EpiParams& e = p.epi;
+    const uint32_t s = tid >> 6, row_in_pass = lq;
+    const uint32_t col = (s0 + s) * kPkCols + lc;
+    if (s < nslabs && col < p.n && row_in_pass < p.rows) {
+        const ChannelQ q = load_channel_q(e, col);
+        const float bp = load_bias_post(e, col);
+        const int32_t bias_pre = e.bias_kind == ASCQ_MM_BIAS_I32_PRE ? static_cast<const int32_t*>(e.bias)[col] : 0;
+        const int32_t sum = OUT[s][row_in_pass][lc] + bias_pre;
+        const float tok = TOK[row_in_pass];
+        dispatch_out(e, [&](auto tag) {
+            epilogue_store<decltype(tag)::value>(e, p.m0 + row_in_pass, col, sum, q, tok, bp);
+        });
+    }
+}
+
 // [k, n] (or [n, k] with trans) -> packed; one thread per lane of a tile.
 __global__ __launch_bounds__(256) void pack_w8_kernel(const int8_t* __restrict__ w, i32x4* __restrict__ out, uint32_t k,
                                                       uint32_t n, uint32_t slabs, uint32_t ktiles, int trans)
@@ -324,6 +540,51 @@ int launch_gemm_packed(const GemmParams& p, hipStream_t st, bool b_nk)
         }
     }
     return launch_status(b_nk ? "ascq_matmul_w8a8 ([n, k] weight stream)" : "ascq_matmul_w8a8_packed");
+}
+
+// The fused form: x [m, k] of halves or bfloat16s is quantised per token inside the kernel (p.epi.has_tok must be set;
+// p.a and p.epi.tok_scale are not read).  False when the shape does not fit (the caller then runs the two kernels).
+bool gemm_packed_dyn_fits(uint32_t m, uint32_t k)
+{
+    if (m == 0u || m > kPkDynRows || k % kPkTileK != 0) {
+        return false;
+    }
+    const uint32_t tpw = (k / kPkTileK + kPkWaves - 1u) / kPkWaves;
+    return m * kPkWaves * (tpw * kPkTileK + kPkRowPad) <= kPkDynQBytes;  // the staged rows take twice that, of twice the space
+}
+
+int launch_gemm_packed_dyn(const GemmParams& p, const void* x, bool x_bf16, hipStream_t st, bool b_nk)
+{
+    const uint32_t cus = device_compute_units();
+    PackedParams q{};
+    q.wp = reinterpret_cast<const i32x4*>(p.b);
+    q.a = nullptr;
+    q.n = p.n;
+    q.k = p.k;
+    q.slabs = (p.n + kPkCols - 1u) / kPkCols;
+    q.ktiles = p.k / kPkTileK;
+    q.tpw = (q.ktiles + kPkWaves - 1u) / kPkWaves;
+    q.epi = p.epi;
+    q.m0 = 0;
+    q.rows = p.m;
+    q.rows_magic = static_cast<uint32_t>(((1ull << 32) + q.rows - 1u) / q.rows);
+    uint32_t grid = q.slabs < cus ? q.slabs : cus;
+    if ((q.slabs + grid - 1u) / grid > kPkMaxSlabs) {
+        grid = (q.slabs + kPkMaxSlabs - 1u) / kPkMaxSlabs;
+    }
+    const uint16_t* xp = static_cast<const uint16_t*>(x);
+    if (b_nk) {
+        if (x_bf16) {
+            gemm_packed_dyn_kernel<true, true><<<grid, kPkWaves * 64u, 0, st>>>(q, xp);
+        } else {
+            gemm_packed_dyn_kernel<true, false><<<grid, kPkWaves * 64u, 0, st>>>(q, xp);
+        }
+    } else if (x_bf16) {
+        gemm_packed_dyn_kernel<false, true><<<grid, kPkWaves * 64u, 0, st>>>(q, xp);
+    } else {
+        gemm_packed_dyn_kernel<false, false><<<grid, kPkWaves * 64u, 0, st>>>(q, xp);
+    }
+    return launch_status("ascq_linear_w8a8_dynamic (fused decode kernel)");
 }
 
 }  // namespace ascq

@@ -11,6 +11,7 @@ import torch
 import orc
 from ascq import _abi as abi
 from ascq import ops
+import gpu_util
 from gpu_util import DEV, announce, bits, max_ulp, pack_int4, to_dev
 
 pytestmark = pytest.mark.gpu
@@ -1174,6 +1175,35 @@ def test_linear_w8a8_dynamic_equals_quantise_then_matmul(m, k, n, xdt):
                        has_tok_scale=1, bias_kind=abi.MM_BIAS_F32_POST)
     want = orc.matmul_w8a8(d, q, w, bias, cs, ts)
     assert np.array_equal(bits(c), want)
+
+
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 17])
+@pytest.mark.parametrize("k,n", [(64, 16), (192, 40), (256, 128), (1024, 1056), (4096, 2064), (320, 48), (8192, 100),
+                                 (11008, 272), (12288, 16)])
+@pytest.mark.parametrize("xdt,odt", [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16),
+                                     (torch.bfloat16, torch.float32)])
+def test_linear_w8a8_dynamic_on_n_k_weights(m, k, n, xdt, odt):
+    """Weights kept as [n, k] (isTransposeB): up to 4 rows are quantised inside the weight-streaming kernel, more rows
+    by the two kernels; either way the bits of quantise-then-matmul (oracle of the two steps)."""
+    announce("linear dynamic [n, k]", m, k, n, xdt, odt)
+    rng = np.random.default_rng(m * 7 + k + n)
+    xf = rng.standard_normal((m, k)).astype(np.float32) * rng.uniform(0.1, 30.0, (m, 1)).astype(np.float32)
+    if m > 2:
+        xf[1] = 0.0
+        xf[2, : k // 2] = 0.0                              # the row's maximum lies in the upper half of k only
+    x = torch.from_numpy(xf).to(DEV).to(xdt)
+    w = rng.integers(-127, 128, (n, k)).astype(np.int8)
+    cs = rng.uniform(1e-4, 1e-2, n).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    c = torch.zeros((m, n), dtype=odt, device=DEV)
+    ops.linear_w8a8_dynamic(c, x, to_dev(w), to_dev(cs), to_dev(bias), trans_b=True)
+    xdt_abi = {torch.bfloat16: abi.BF16, torch.float16: abi.F16}[xdt]
+    odt_abi = {torch.bfloat16: abi.BF16, torch.float16: abi.F16, torch.float32: abi.F32}[odt]
+    q, ts = orc.dynamic_quant_per_token(xdt_abi, bits(x))
+    d = abi.MatmulDesc(m=m, n=n, k=k, trans_b=1, out_dtype=odt_abi, quant_mode=abi.MM_QUANT_VECTOR,
+                       scale_format=abi.MM_SCALE_F32, has_tok_scale=1, bias_kind=abi.MM_BIAS_F32_POST)
+    want = orc.matmul_w8a8(d, q, w, bias, cs, ts)
+    assert np.array_equal(bits(c), gpu_util.as_bits(want))
 
 
 # ------------------------------------------------------------------ Matmul<int4b_t, int4b_t, C>
