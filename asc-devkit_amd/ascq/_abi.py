@@ -124,6 +124,8 @@ SIGNATURES = {
     "ascq_pack_weight_w8_size": (C.c_int, [C.c_uint32, C.c_uint32, C.POINTER(C.c_size_t)]),
     "ascq_pack_weight_w8": (C.c_int, [_P, _P, C.c_uint32, C.c_uint32, C.c_int32, _P]),
     "ascq_matmul_w8a8_packed": (C.c_int, [C.POINTER(MatmulDesc), _P, _P, _P, _P, _P, _P, _P]),
+    "ascq_linear_w8a8_dynamic_packed": (C.c_int, [C.POINTER(MatmulDesc), C.c_int32, _P, _P, _P, _P, _P, _P, C.c_size_t,
+                                                  _P]),
     "ascq_matmul_w4a16": (C.c_int, [C.POINTER(W4A16Desc), _P, _P, _P, _P, _P, _P, C.c_size_t, _P]),
     "ascq_matmul_w4a16_workspace_size": (C.c_int, [C.POINTER(W4A16Desc), C.POINTER(C.c_size_t)]),
     "ascq_pack_weight_w4_size": (C.c_int, [C.c_uint32, C.c_uint32, C.POINTER(C.c_size_t)]),

@@ -405,6 +405,23 @@ def unpack_int4(src, out=None):
 
 
 _lin_ws = {}
+_lin_need = {}
+
+
+def _linear_workspace(lib, d, device):
+    """The scratch buffer of the one-call linear: sized once per shape (the size query is a host call of its own, which
+    a decode step of a dozen microseconds notices), one buffer per stream (calls on two streams may overlap)."""
+    shape = (d.m, d.n, d.k, d.trans_b, d.out_dtype, d.activation, d.bias_kind)
+    need = _lin_need.get(shape)
+    if need is None:
+        size = C.c_size_t(0)
+        check(lib.ascq_linear_w8a8_dynamic_workspace_size(C.byref(d), C.byref(size)))
+        need = _lin_need[shape] = size.value
+    key = (device, need, _stream().value)
+    ws = _lin_ws.get(key)
+    if ws is None:
+        ws = _lin_ws[key] = torch.empty(max(need, 16), dtype=torch.uint8, device=device)
+    return ws
 
 
 def linear_w8a8_dynamic(c, x, weight, channel_scale, bias=None, activation=abi.MM_ACT_NONE, trans_b=False, act_beta=1.0):
@@ -418,15 +435,40 @@ def linear_w8a8_dynamic(c, x, weight, channel_scale, bias=None, activation=abi.M
     if bias is not None:
         d.bias_kind = abi.MM_BIAS_F32_POST if bias.dtype == torch.float32 else abi.MM_BIAS_BF16_POST
     lib = load_library()
-    need = C.c_size_t(0)
-    check(lib.ascq_linear_w8a8_dynamic_workspace_size(C.byref(d), C.byref(need)))
-    key = (x.device, need.value, _stream().value)    # one scratch buffer per stream: calls on two streams may overlap
-    if key not in _lin_ws:
-        _lin_ws[key] = torch.empty(max(need.value, 16), dtype=torch.uint8, device=x.device)
-    ws = _lin_ws[key]
+    ws = _linear_workspace(lib, d, x.device)
     check(lib.ascq_linear_w8a8_dynamic(C.byref(d), _dt(x), _ptr(c), _ptr(x), _ptr(weight), _ptr(bias),
                                        _ptr(channel_scale), _ptr(ws), ws.numel(), _stream()))
     return c
+
+
+class DynamicLinear:
+    """The one-call W8A8 linear with everything that does not change between calls prepared once (descriptor, scratch,
+    argument pointers): a decode step of ten microseconds notices a descriptor built per call.  weight: int8 [k, n],
+    [n, k] with trans_b, or, with packed_n, the buffer of pack_weight_w8 for n columns."""
+
+    def __init__(self, m, k, weight, channel_scale, bias=None, trans_b=False, packed_n=None, out_dtype=torch.bfloat16,
+                 x_dtype=torch.bfloat16, activation=abi.MM_ACT_NONE, act_beta=1.0):
+        n = packed_n if packed_n is not None else (weight.shape[0] if trans_b else weight.shape[1])
+        self.desc = abi.MatmulDesc(m=m, n=n, k=k, trans_b=int(trans_b and packed_n is None), out_dtype=_DT[out_dtype],
+                                   quant_mode=abi.MM_QUANT_VECTOR, scale_format=abi.MM_SCALE_F32, activation=activation,
+                                   act_beta=act_beta)
+        if bias is not None:
+            self.desc.bias_kind = abi.MM_BIAS_F32_POST if bias.dtype == torch.float32 else abi.MM_BIAS_BF16_POST
+        self.lib = load_library()
+        self.fn = self.lib.ascq_linear_w8a8_dynamic_packed if packed_n is not None else self.lib.ascq_linear_w8a8_dynamic
+        self.keep = (weight, channel_scale, bias)
+        self.ws = _linear_workspace(self.lib, self.desc, weight.device)
+        self.x_dt, self.out_dtype = _DT[x_dtype], out_dtype
+        self.args = (_ptr(weight), _ptr(bias), _ptr(channel_scale), _ptr(self.ws), self.ws.numel())
+        self.ref = C.byref(self.desc)
+
+    def __call__(self, c, x):
+        """c [m, n] of out_dtype (n / 2 columns with SwiGLU), x [m, k] of x_dtype, on the current stream (the scratch
+        belongs to the stream the object was made on: calls on other streams at the same time would share it)."""
+        if not (c.is_contiguous() and x.is_contiguous() and c.is_cuda and x.is_cuda):
+            raise ValueError("ascq operators take contiguous device tensors")
+        check(self.fn(self.ref, self.x_dt, c.data_ptr(), x.data_ptr(), *self.args, _stream()))
+        return c
 
 
 def linear_w8a8_dynamic_noalloc(c, x, weight, channel_scale, bias=None, activation=abi.MM_ACT_NONE, trans_b=False,
@@ -441,6 +483,21 @@ def linear_w8a8_dynamic_noalloc(c, x, weight, channel_scale, bias=None, activati
         d.bias_kind = abi.MM_BIAS_F32_POST if bias.dtype == torch.float32 else abi.MM_BIAS_BF16_POST
     check(load_library().ascq_linear_w8a8_dynamic_noalloc(C.byref(d), _dt(x), _ptr(c), _ptr(x), _ptr(weight), _ptr(bias),
                                                           _ptr(channel_scale), _stream()))
+    return c
+
+
+def linear_w8a8_dynamic_packed(c, x, w_packed, n, channel_scale, bias=None, activation=abi.MM_ACT_NONE):
+    """linear_w8a8_dynamic on weights packed by pack_weight_w8 (n = their column count): up to 8 rows of half /
+    bfloat16 x are one launch; the results are those of linear_w8a8_dynamic on the unpacked weights."""
+    m, k = x.shape
+    d = abi.MatmulDesc(m=m, n=n, k=k, out_dtype=_dt(c), quant_mode=abi.MM_QUANT_VECTOR, scale_format=abi.MM_SCALE_F32,
+                       activation=activation, act_beta=1.0)
+    if bias is not None:
+        d.bias_kind = abi.MM_BIAS_F32_POST if bias.dtype == torch.float32 else abi.MM_BIAS_BF16_POST
+    lib = load_library()
+    ws = _linear_workspace(lib, d, x.device)
+    check(lib.ascq_linear_w8a8_dynamic_packed(C.byref(d), _dt(x), _ptr(c), _ptr(x), _ptr(w_packed), _ptr(bias),
+                                              _ptr(channel_scale), _ptr(ws), ws.numel(), _stream()))
     return c
 
 

@@ -233,7 +233,7 @@ bool gemm_packed_supported(const GemmParams& p);
 bool gemm_packed_nk_supported(const GemmParams& p);
 bool gemm_packed_two_tiles_fit(uint32_t k);  // 17 to 32 rows in one pass over the weights
 int launch_gemm_packed(const GemmParams& p, hipStream_t st, bool b_nk = false);
-// The same kernel with the per-token quantisation of x (half or bfloat16, [m, k]) inside: m <= 4 rows that fit the LDS.
+// The same kernel with the per-token quantisation of x (half or bfloat16, [m, k]) inside: m <= 8 rows that fit the LDS.
 bool gemm_packed_dyn_fits(uint32_t m, uint32_t k);
 int launch_gemm_packed_dyn(const GemmParams& p, const void* x, bool x_bf16, hipStream_t st, bool b_nk);
 

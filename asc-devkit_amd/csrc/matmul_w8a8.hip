@@ -852,10 +852,10 @@ extern "C" int ascq_linear_w8a8_dynamic_workspace_size(const ascq_matmul_desc* d
 
 // The activation quantiser of a W8A8 linear and the matmul in one call: q, tok = dynamic per-token quantisation of x
 // (ascq_dynamic_quant_per_token), c = matmul(q, b) with the token scales in the epilogue; q and tok live in the
-// caller's workspace.  Up to 4 rows of half / bfloat16 x on weights kept as [n, k] run as one launch instead: the
+// caller's workspace.  Up to 8 rows of half / bfloat16 x on weights kept as [n, k] run as one launch instead: the
 // decode kernel quantises x inside every workgroup on its way into LDS (gemm_packed_dyn_kernel; the same bits, about
-// 12.5 us against 15.5 us at k = 4096, n = 11008; from 6 rows on the 256 redundant quantisations cost more than the
-// separate kernel's launch).  The reference composes this
+// 12 us against 15.5 us per step at k = 4096, n = 11008 and one row, 15.4 against 15.8 us at 8; from 9 rows on the 256
+// redundant quantisations cost more than the separate kernel's launch).  The reference composes this
 // from ReduceMax / AscendQuant PER_TOKEN and Matmul (impl/adv_api/detail/quantization/quant/
 // ascend_quant_per_group_3510_impl.h:142-178, include/adv_api/matmul/matmul.h:175-185).
 extern "C" int ascq_linear_w8a8_dynamic(const ascq_matmul_desc* d, int32_t x_dtype, void* c, const void* x,
@@ -909,6 +909,60 @@ extern "C" int ascq_linear_w8a8_dynamic(const ascq_matmul_desc* d, int32_t x_dty
     }
     return ascq_matmul_w8a8(&dd, c, q, b, bias, quant_vector, tok, rest,
                             workspace_bytes - static_cast<size_t>(rest - ws), stream);
+}
+
+// The same linear on weights packed by ascq_pack_weight_w8: up to 8 rows of half / bfloat16 x are one launch of the
+// packed decode kernel with the quantiser inside; anything else is the quantiser kernel followed by
+// ascq_matmul_w8a8_packed, with q and the token scales in the workspace.  The results are those of
+// ascq_linear_w8a8_dynamic on the unpacked weights, bit for bit.
+extern "C" int ascq_linear_w8a8_dynamic_packed(const ascq_matmul_desc* d, int32_t x_dtype, void* c, const void* x,
+                                               const void* w_packed, const void* bias, const void* quant_vector,
+                                               void* workspace, size_t workspace_bytes, void* stream)
+{
+    ASCQ_REQUIRE(d != nullptr, ASCQ_ENULL, "ascq_linear_w8a8_dynamic_packed: desc is NULL");
+    ASCQ_REQUIRE(x_dtype == ASCQ_F16 || x_dtype == ASCQ_BF16 || x_dtype == ASCQ_F32, ASCQ_EUNSUPPORTED,
+                 "ascq_linear_w8a8_dynamic_packed: x dtype %d is not half / bfloat16 / float", x_dtype);
+    ASCQ_REQUIRE(d->quant_mode != ASCQ_MM_QUANT_NONE && d->out_dtype != ASCQ_I8, ASCQ_EUNSUPPORTED,
+                 "ascq_linear_w8a8_dynamic_packed: the token scales need a floating-point dequantising epilogue");
+    ASCQ_REQUIRE(!d->trans_a && d->b_format == ASCQ_MM_B_ND && d->activation != ASCQ_MM_ACT_SWIGLU, ASCQ_EUNSUPPORTED,
+                 "ascq_linear_w8a8_dynamic_packed: x is [m, k], the weights are in the packed layout, SwiGLU is not "
+                 "available on packed weights");
+    ASCQ_REQUIRE(d->k % 64u == 0, ASCQ_EUNSUPPORTED, "ascq_linear_w8a8_dynamic_packed: k = %u must be a multiple of 64", d->k);
+    ascq_matmul_desc dd = *d;
+    dd.has_tok_scale = 1;
+    dd.trans_b = 0;
+    ASCQ_REQUIRE(workspace != nullptr, ASCQ_ENULL, "ascq_linear_w8a8_dynamic_packed: workspace is NULL");
+    ASCQ_REQUIRE(aligned16(workspace), ASCQ_EALIGN, "ascq_linear_w8a8_dynamic_packed: workspace must be 16-byte aligned");
+    const size_t q_bytes = round256(static_cast<size_t>(d->m) * d->k);
+    const size_t need = q_bytes + round256(static_cast<size_t>(d->m) * sizeof(float));
+    ASCQ_REQUIRE(workspace_bytes >= need, ASCQ_EINVAL,
+                 "ascq_linear_w8a8_dynamic_packed: workspace of %zu bytes required (ascq_linear_w8a8_dynamic_workspace_size "
+                 "covers it)", need);
+    char* ws = static_cast<char*>(workspace);
+    int rc = validate_mm(&dd, "ascq_linear_w8a8_dynamic_packed", c, x, w_packed, bias, quant_vector, ws);
+    if (rc != ASCQ_OK) {
+        return rc;
+    }
+    ASCQ_REQUIRE(aligned16(w_packed), ASCQ_EALIGN, "ascq_linear_w8a8_dynamic_packed: w_packed must be 16-byte aligned");
+    if ((x_dtype == ASCQ_F16 || x_dtype == ASCQ_BF16) && aligned16(x) && gemm_packed_dyn_fits(d->m, d->k)) {
+        GemmParams p{};
+        p.a = static_cast<const int8_t*>(x);  // only its alignment is looked at
+        p.b = static_cast<const int8_t*>(w_packed);
+        p.m = d->m;
+        p.n = d->n;
+        p.k = d->k;
+        p.epi = make_epi(&dd, c, bias, quant_vector, reinterpret_cast<const float*>(ws));
+        ASCQ_REQUIRE(gemm_packed_supported(p), ASCQ_EUNSUPPORTED,
+                     "ascq_linear_w8a8_dynamic_packed: the packed weights must stay below 2 GiB");
+        return launch_gemm_packed_dyn(p, x, x_dtype == ASCQ_BF16, static_cast<hipStream_t>(stream), false);
+    }
+    int8_t* q = reinterpret_cast<int8_t*>(ws);
+    float* tok = reinterpret_cast<float*>(ws + q_bytes);
+    rc = ascq_dynamic_quant_per_token(x_dtype, d->m, d->k, q, tok, x, stream);
+    if (rc != ASCQ_OK) {
+        return rc;
+    }
+    return ascq_matmul_w8a8_packed(&dd, c, q, w_packed, bias, quant_vector, tok, stream);
 }
 
 // ------------------------------------------------------------------------------- the same call without a workspace

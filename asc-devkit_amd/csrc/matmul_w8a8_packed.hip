@@ -220,16 +220,16 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_kernel(PackedParams
     }
 }
 
-// The decode kernel with the per-token quantisation of the activations inside (up to 4 rows of half or bfloat16 x):
+// The decode kernel with the per-token quantisation of the activations inside (up to 8 rows of half or bfloat16 x):
 // q = ascq_dynamic_quant_per_token(x); c = matmul(q, w, tok_scale) in one launch, with those two calls' results bit for
 // bit.  Every workgroup needs all of x anyway, so every workgroup quantises it: a wavefront stages its k range of
 // every row as it is (2 bytes per element), the wavefronts exchange their rows' absolute maxima through LDS, and each
 // turns its own range into the int8 image the matrix instructions read, with the arithmetic of dynq_row_kernel:
 // inv = 127 / amax, the product rounded to the nearest integer, ties to even, by adding 1.5 * 2^23.  The weight
-// batches requested ahead of all this arrive meanwhile.  The quantisation costs every compute unit about 0.3 us per
-// row, which is why this form stops at 4 rows: from about 6 on the separate quantiser kernel (one pass over x by the
-// whole chip) is cheaper than 256 redundant ones.  The wavefronts' tiles are added into one LDS array with atomics.
-constexpr uint32_t kPkDynRows = 4;
+// batches requested ahead of all this arrive meanwhile.  The quantisation costs every compute unit about 0.4 us per
+// row beyond the first, which is why this form stops at 8 rows: from there on the separate quantiser kernel (one pass
+// over x by the whole chip) is cheaper than 256 redundant ones.  The wavefronts' tiles are added into one LDS array with atomics.
+constexpr uint32_t kPkDynRows = 8;
 constexpr uint32_t kPkDynHBytes = 96 * 1024;   // the staged activations as they come (2 bytes per element)
 constexpr uint32_t kPkDynQBytes = 48 * 1024;   // their int8 image
 
@@ -253,7 +253,7 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_dyn_kernel(PackedPa
 {
     __shared__ __attribute__((aligned(16))) char XH[kPkDynHBytes];
     __shared__ __attribute__((aligned(16))) char XS[kPkDynQBytes];
-    __shared__ int32_t OUT[kPkMaxSlabs][4][16];  // [slab][row][column]
+    __shared__ int32_t OUT[kPkMaxSlabs][kPkDynRows][16];  // [slab][row][column]
     __shared__ float ROWMAX[kPkWaves][kPkDynRows];
     __shared__ float TOK[kPkDynRows];
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
@@ -318,7 +318,7 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_dyn_kernel(PackedPa
     auto widen = [](uint32_t half_bits) __attribute__((always_inline)) {
         return kBf16 ? bf16_bits_to_f32(half_bits) : half_bits_to_f32(half_bits);
     };
-    for (uint32_t i = tid; i < kPkMaxSlabs * 4u * 16u; i += kPkWaves * 64u) (&OUT[0][0][0])[i] = 0;
+    for (uint32_t i = tid; i < kPkMaxSlabs * kPkDynRows * 16u; i += kPkWaves * 64u) (&OUT[0][0][0])[i] = 0;
 #pragma unroll
     for (uint32_t r = 0; r < kPkDynRows; ++r) {
         if (r < p.rows) {  // uniform
@@ -399,11 +399,12 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_dyn_kernel(PackedPa
             }
         }
         ++c_q;
-        if (++c_b == nb) {  // the slab is done: register i of lanes 0 .. 15 is row i, column = lane
-            if (lane < 16u) {
+        if (++c_b == nb) {  // the slab is done: register i of lane l is row 4 (l / 16) + i, column l % 16
+            if (4u * lq < p.rows) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    __hip_atomic_fetch_add(&OUT[c_slab][i][lane], acc[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    __hip_atomic_fetch_add(&OUT[c_slab][4u * lq + i][lc], acc[i], __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_WORKGROUP);
                 }
             }
             acc = i32x4{0, 0, 0, 0};
@@ -420,19 +421,25 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_dyn_kernel(PackedPa
     }
     __syncthreads();
 
-    // ---- element (row, column) of slab s is handled by thread s * 64 + row * 16 + column
+    // ---- elements (row, column) and (row + 4, column) of slab s are handled by thread s * 64 + row * 16 + column
     const EpiParams& e = p.epi;
-    const uint32_t s = tid >> 6, row_in_pass = lq;
+    const uint32_t s = tid >> 6;
     const uint32_t col = (s0 + s) * kPkCols + lc;
-    if (s < nslabs && col < p.n && row_in_pass < p.rows) {
+    if (s < nslabs && col < p.n) {
         const ChannelQ q = load_channel_q(e, col);
         const float bp = load_bias_post(e, col);
         const int32_t bias_pre = e.bias_kind == ASCQ_MM_BIAS_I32_PRE ? static_cast<const int32_t*>(e.bias)[col] : 0;
-        const int32_t sum = OUT[s][row_in_pass][lc] + bias_pre;
-        const float tok = TOK[row_in_pass];
-        dispatch_out(e, [&](auto tag) {
-            epilogue_store<decltype(tag)::value>(e, p.m0 + row_in_pass, col, sum, q, tok, bp);
-        });
+#pragma unroll
+        for (uint32_t half = 0; half < kPkDynRows / 4u; ++half) {
+            const uint32_t row_in_pass = 4u * half + lq;
+            if (row_in_pass < p.rows) {
+                const int32_t sum = OUT[s][row_in_pass][lc] + bias_pre;
+                const float tok = TOK[row_in_pass];
+                dispatch_out(e, [&](auto tag) {
+                    epilogue_store<decltype(tag)::value>(e, p.m0 + row_in_pass, col, sum, q, tok, bp);
+                });
+            }
+        }
     }
 }
 

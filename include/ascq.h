@@ -444,8 +444,8 @@ int ascq_matmul_w8a8_plan(const ascq_matmul_desc* desc, const void* c, const voi
  * with exactly those results.  x [m, k] of x_dtype (ASCQ_F16 | ASCQ_BF16 | ASCQ_F32); desc as for ascq_matmul_w8a8 with
  * a dequantising epilogue (quant_mode SCALAR or VECTOR, floating-point out_dtype); desc->has_tok_scale is ignored.
  * The two kernels run one after the other on the stream, with q and tok in the workspace (sized by
- * ascq_linear_w8a8_dynamic_workspace_size; always required, whatever kernel runs).  Decode calls - up to 4 rows of half
- * or bfloat16 x on weights kept as [n, k] (desc->trans_b), k a multiple of 64 up to about 11700 at 4 rows - are one
+ * ascq_linear_w8a8_dynamic_workspace_size; always required, whatever kernel runs).  Decode calls - up to 8 rows of half
+ * or bfloat16 x on weights kept as [n, k] (desc->trans_b), k a multiple of 64 up to 5632 at 8 rows, 11776 at 4 - are one
  * launch: the weight-streaming kernel quantises x itself on its way into LDS (the same bits; the workspace is not
  * touched).  No single reference operator does this: the reference composes it from
  * ReduceMax / AscendQuant PER_TOKEN (ascend_quant_per_group_3510_impl.h:142-178) and Matmul (matmul.h:175-185).
@@ -454,6 +454,20 @@ int ascq_linear_w8a8_dynamic(const ascq_matmul_desc* desc, int32_t x_dtype, void
                              const void* bias, const void* quant_vector, void* workspace, size_t workspace_bytes,
                              void* stream);
 int ascq_linear_w8a8_dynamic_workspace_size(const ascq_matmul_desc* desc, size_t* bytes);
+
+/*
+ * The same linear on weights packed once by ascq_pack_weight_w8 (see ascq_matmul_w8a8_packed for the layout and what
+ * the descriptor may ask for: no trans_a, no NZ, no SwiGLU, k % 64 == 0; desc->trans_b is ignored).  Results are those
+ * of ascq_linear_w8a8_dynamic on the unpacked weights, bit for bit.  Up to 8 rows of half or bfloat16 x are one launch
+ * (the packed decode kernel quantises x itself); otherwise the quantiser kernel runs first and
+ * ascq_matmul_w8a8_packed after it, with q and the token scales in the workspace.  The workspace holds
+ * round256(m * k) + round256(4 * m) bytes; ascq_linear_w8a8_dynamic_workspace_size covers that.
+ * It has no counterpart in the reference (which composes the linear from ReduceMax / AscendQuant PER_TOKEN and Matmul,
+ * ascend_quant_per_group_3510_impl.h:142-178, matmul.h:175-185, on weights it packs offline, gen_data.py:62-64).
+ */
+int ascq_linear_w8a8_dynamic_packed(const ascq_matmul_desc* desc, int32_t x_dtype, void* c, const void* x,
+                                    const void* w_packed, const void* bias, const void* quant_vector, void* workspace,
+                                    size_t workspace_bytes, void* stream);
 
 /*
  * ascq_linear_w8a8_dynamic without a workspace argument and without any allocation (no hipMalloc / hipFree, here or in

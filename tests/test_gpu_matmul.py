@@ -1177,13 +1177,13 @@ def test_linear_w8a8_dynamic_equals_quantise_then_matmul(m, k, n, xdt):
     assert np.array_equal(bits(c), want)
 
 
-@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 17])
-@pytest.mark.parametrize("k,n", [(64, 16), (192, 40), (256, 128), (1024, 1056), (4096, 2064), (320, 48), (8192, 100),
-                                 (11008, 272), (12288, 16)])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 7, 8, 9, 17])
+@pytest.mark.parametrize("k,n", [(64, 16), (192, 40), (256, 128), (1024, 1056), (4096, 2064), (320, 48), (5632, 100),
+                                 (8192, 100), (11008, 272), (12288, 16)])
 @pytest.mark.parametrize("xdt,odt", [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16),
                                      (torch.bfloat16, torch.float32)])
 def test_linear_w8a8_dynamic_on_n_k_weights(m, k, n, xdt, odt):
-    """Weights kept as [n, k] (isTransposeB): up to 4 rows are quantised inside the weight-streaming kernel, more rows
+    """Weights kept as [n, k] (isTransposeB): up to 8 rows are quantised inside the weight-streaming kernel, more rows
     by the two kernels; either way the bits of quantise-then-matmul (oracle of the two steps)."""
     announce("linear dynamic [n, k]", m, k, n, xdt, odt)
     rng = np.random.default_rng(m * 7 + k + n)
@@ -1204,6 +1204,50 @@ def test_linear_w8a8_dynamic_on_n_k_weights(m, k, n, xdt, odt):
                        scale_format=abi.MM_SCALE_F32, has_tok_scale=1, bias_kind=abi.MM_BIAS_F32_POST)
     want = orc.matmul_w8a8(d, q, w, bias, cs, ts)
     assert np.array_equal(bits(c), gpu_util.as_bits(want))
+
+
+@pytest.mark.parametrize("m", [1, 3, 4, 5, 8, 9, 33])
+@pytest.mark.parametrize("k,n", [(64, 16), (192, 40), (1024, 1056), (4096, 2064), (11008, 272)])
+@pytest.mark.parametrize("xdt,src_nk", [(torch.bfloat16, False), (torch.float16, True), (torch.float32, False)])
+def test_linear_w8a8_dynamic_on_packed_weights(m, k, n, xdt, src_nk):
+    """ascq_linear_w8a8_dynamic_packed: up to 8 rows of half / bfloat16 x in one launch, anything else quantiser +
+    packed matmul; either way the bits of quantise-then-matmul (oracle of the two steps)."""
+    announce("linear dynamic packed", m, k, n, xdt, src_nk)
+    rng = np.random.default_rng(m * 11 + k + n)
+    xf = rng.standard_normal((m, k)).astype(np.float32) * rng.uniform(0.1, 30.0, (m, 1)).astype(np.float32)
+    if m > 2:
+        xf[1] = 0.0
+    x = torch.from_numpy(xf).to(DEV).to(xdt)
+    w = rng.integers(-127, 128, (k, n)).astype(np.int8)
+    wp = ops.pack_weight_w8(to_dev(np.ascontiguousarray(w.T)) if src_nk else to_dev(w), k, n, src_nk)
+    cs = rng.uniform(1e-4, 1e-2, n).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    c = torch.zeros((m, n), dtype=torch.bfloat16, device=DEV)
+    ops.linear_w8a8_dynamic_packed(c, x, wp, n, to_dev(cs), to_dev(bias))
+    xdt_abi = {torch.bfloat16: abi.BF16, torch.float16: abi.F16, torch.float32: abi.F32}[xdt]
+    q, ts = orc.dynamic_quant_per_token(xdt_abi, bits(x))
+    d = abi.MatmulDesc(m=m, n=n, k=k, out_dtype=abi.BF16, quant_mode=abi.MM_QUANT_VECTOR, scale_format=abi.MM_SCALE_F32,
+                       has_tok_scale=1, bias_kind=abi.MM_BIAS_F32_POST)
+    want = orc.matmul_w8a8(d, q, w, bias, cs, ts)
+    assert np.array_equal(bits(c), want)
+
+
+@pytest.mark.parametrize("m", [2, 9])
+def test_prepared_linear_object_equals_the_function(m):
+    """ops.DynamicLinear (descriptor and scratch prepared once) gives what ops.linear_w8a8_dynamic gives, on [k, n],
+    [n, k] and packed weights."""
+    k, n = 512, 208
+    rng = np.random.default_rng(m)
+    x = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).to(DEV).to(torch.bfloat16)
+    w = to_dev(rng.integers(-127, 128, (k, n)).astype(np.int8))
+    wt = w.t().contiguous()
+    cs, bias = to_dev(rng.uniform(1e-4, 1e-2, n).astype(np.float32)), to_dev(rng.standard_normal(n).astype(np.float32))
+    want = ops.linear_w8a8_dynamic(torch.zeros((m, n), dtype=torch.bfloat16, device=DEV), x, w, cs, bias)
+    for lin in (ops.DynamicLinear(m, k, w, cs, bias), ops.DynamicLinear(m, k, wt, cs, bias, trans_b=True),
+                ops.DynamicLinear(m, k, ops.pack_weight_w8(w, k, n), cs, bias, packed_n=n)):
+        for _ in range(2):
+            got = lin(torch.zeros((m, n), dtype=torch.bfloat16, device=DEV), x)
+            assert torch.equal(got, want)
 
 
 # ------------------------------------------------------------------ Matmul<int4b_t, int4b_t, C>
