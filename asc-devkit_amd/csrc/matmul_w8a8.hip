@@ -743,6 +743,9 @@ extern "C" int ascq_matmul_w8a8(const ascq_matmul_desc* d, void* c, const void* 
         (d->m <= 16 || gemm_packed_two_tiles_fit(d->k))) {
         return launch_gemm_packed(p, st, true);  // activations resident in LDS, nothing but weights in the load queue
     }
+    if (d->trans_b && !d->trans_a && gemm_ws_supported(p, true)) {
+        return launch_gemm_ws(p, st, true);  // 33 to 48 rows: the weights held in registers, the activations streamed
+    }
     if (d->m <= 32 && d->trans_b && !d->trans_a && gemm_nk_supported(p)) {
         return launch_gemm_nk(p, st);
     }
@@ -817,6 +820,9 @@ extern "C" int ascq_matmul_w8a8_packed(const ascq_matmul_desc* d, void* c, const
     ASCQ_REQUIRE(d->k % 64u == 0, ASCQ_EUNSUPPORTED, "ascq_matmul_w8a8_packed: k = %u must be a multiple of 64", d->k);
     ASCQ_REQUIRE(aligned16(a) && aligned16(w_packed), ASCQ_EALIGN, "ascq_matmul_w8a8_packed: a and w_packed must be 16-byte aligned");
     ASCQ_REQUIRE(gemm_packed_supported(p), ASCQ_EUNSUPPORTED, "ascq_matmul_w8a8_packed: the packed weights must stay below 2 GiB");
+    if (gemm_ws_supported(p, false)) {
+        return launch_gemm_ws(p, static_cast<hipStream_t>(stream), false);
+    }
     return launch_gemm_packed(p, static_cast<hipStream_t>(stream));
 }
 

@@ -443,6 +443,178 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_dyn_kernel(PackedPa
     }
 }
 
+// The weight-stationary form, for more than 32 activation rows (up to 128 per launch).  That many rows do not fit the LDS, and activations that
+// are streamed beside the weights share the compute unit's in-order load queue with them (every L2 hit of an
+// activation load then waits behind the weights' trips to memory).  So the two are separated in time: a workgroup
+// first requests all the weights of its columns (up to 3 slabs x 64 tiles = 192 KiB, a wavefront holding its k range
+// of them in 96 registers as ready matrix operands) in one burst with nothing else in the queue, and then streams the
+// activations, 16 rows at a time, from the L2 through a two-slot LDS ring per wavefront: one matrix instruction per
+// slab and tile on operands that are already in registers.  A row tile's sums over the wavefronts' k ranges meet in
+// one LDS array (atomic adds of integers: exact in any order); the epilogue runs once at the end.
+constexpr uint32_t kWsSlabs = 3, kWsTpw = 8, kWsRows = 128;
+constexpr uint32_t kWsRowBytes = kWsTpw * kPkTileK;   // 512: a staged row (the wavefront's k range, padded)
+constexpr uint32_t kWsSlot = 16u * kWsRowBytes;       // 8 KiB: 16 rows
+constexpr int kWsDma = 8;                             // direct-to-LDS instructions per slot (two rows each)
+
+template <bool kNK>
+__global__ __launch_bounds__(kPkWaves * 64) void gemm_ws_kernel(PackedParams p)
+{
+    __shared__ __attribute__((aligned(1024))) char R0[kPkWaves * kWsSlot];
+    __shared__ __attribute__((aligned(1024))) char R1[kPkWaves * kWsSlot];
+    __shared__ int32_t OUT[kWsRows][kWsSlabs * kPkCols];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t lc = lane & 15u, lq = lane >> 4;
+    const uint32_t wg = pk_xcd_order(blockIdx.x, gridDim.x);
+    const uint32_t s0 = static_cast<uint32_t>(static_cast<uint64_t>(wg) * p.slabs / gridDim.x);
+    const uint32_t s1 = static_cast<uint32_t>(static_cast<uint64_t>(wg + 1u) * p.slabs / gridDim.x);
+    const uint32_t nslabs = s1 - s0;  // at most kWsSlabs: the host has chosen the grid
+    const uint32_t ta = min(wave * p.tpw, p.ktiles), tb = min(ta + p.tpw, p.ktiles), cnt = tb - ta;  // at most kWsTpw
+    for (uint32_t i = tid; i < kWsRows * kWsSlabs * kPkCols; i += kPkWaves * 64u) (&OUT[0][0])[i] = 0;
+    __syncthreads();  // before any direct-to-LDS load is in flight
+
+    // ---- the weights of this wavefront's k range, all slabs: one burst, nothing else in the queue yet
+    const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<i32x4*>(p.wp), 0,
+        static_cast<int>(kNK ? p.n * p.k : (p.slabs * p.ktiles + kPkPadTiles) * kPkTileBytes), 0x00020000);
+    const uint32_t w_lane = kNK ? lc * p.k + lq * 16u : lane * 16u;
+    i32x4 wreg[kWsSlabs][kWsTpw];
+#pragma unroll
+    for (uint32_t s = 0; s < kWsSlabs; ++s) {
+#pragma unroll
+        for (uint32_t t = 0; t < kWsTpw; ++t) {
+            // a tile this wavefront does not have is requested past the end of the buffer: no data moves, the
+            // instruction count stays what the waits below assume
+            const uint32_t off = (s < nslabs && t < cnt) ? w_lane : kPkPastEnd;
+            const uint32_t base = kNK ? (s0 + s) * kPkCols * p.k + (ta + t) * kPkTileK
+                                      : ((s0 + s) * p.ktiles + ta + t) * kPkTileBytes;  // scalar
+            wreg[s][t] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, off, base, kPkNt));
+        }
+    }
+
+    // ---- activations: slot position (row r, piece q) holds the row's piece q ^ r of this wavefront's k range (the
+    // reader's 16 rows then fall on 16 different bank groups); pieces past the range fetch piece 0 and are not read
+    char* const r0w = R0 + wave * kWsSlot;
+    char* const r1w = R1 + wave * kWsSlot;
+    // A load's address is a wavefront-uniform base (the row tile) plus the lane's 32-bit offset, which the instruction
+    // adds itself; the last row tile, where rows past the end repeat the last row, has offsets of its own.
+    const uint32_t ntiles = (p.rows + 15u) / 16u;
+    const uint32_t rows_last = p.rows - (ntiles - 1u) * 16u;  // rows of the last row tile, 1 .. 16
+    uint32_t a_off[kWsDma], a_off_last[kWsDma];
+#pragma unroll
+    for (int u = 0; u < kWsDma; ++u) {
+        const uint32_t sidx = static_cast<uint32_t>(u) * 64u + lane;
+        const uint32_t r = sidx >> 5, q = (sidx & 31u) ^ r;
+        const uint32_t col = (q < cnt * 4u ? q : 0u) * 16u + ta * kPkTileK;
+        a_off[u] = r * p.k + col;
+        a_off_last[u] = min(r, rows_last - 1u) * p.k + col;
+    }
+    const int8_t* const a_base = p.a + static_cast<size_t>(p.m0) * p.k;
+    auto issue = [&](uint32_t rt, char* slot) __attribute__((always_inline)) {
+        // past the last row tile: the last one again (never read; keeps the count of loads in flight what the waits assume)
+        const uint32_t tile = rt < ntiles ? rt : ntiles - 1u;
+        const uint64_t bv = reinterpret_cast<uint64_t>(a_base + static_cast<size_t>(tile) * 16u * p.k);
+        uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bv));
+        uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bv >> 32));
+        asm volatile("" : "+s"(lo), "+s"(hi));
+        const int8_t* base = reinterpret_cast<const int8_t*>((static_cast<uint64_t>(hi) << 32) | lo);
+        if (tile + 1u == ntiles) {  // uniform
+#pragma unroll
+            for (int u = 0; u < kWsDma; ++u) {
+                __builtin_amdgcn_global_load_lds((gptr_t)(base + a_off_last[u]), (lds_ptr_t)(slot + u * 1024), 16, 0, 0);
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < kWsDma; ++u) {
+                __builtin_amdgcn_global_load_lds((gptr_t)(base + a_off[u]), (lds_ptr_t)(slot + u * 1024), 16, 0, 0);
+            }
+        }
+    };
+    // the lane's fragment of tile t: row lc, pieces 4 t + lq; its four sums of a row tile and slab: rows 4 lq + i
+    const uint32_t frag = lc * kWsRowBytes;
+    const uint32_t out_lane = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)&OUT[0][0])) +
+                              (4u * lq * kWsSlabs * kPkCols + lc) * 4u;
+    i32x4 acc[kWsSlabs];
+#pragma unroll
+    for (uint32_t s = 0; s < kWsSlabs; ++s) acc[s] = i32x4{0, 0, 0, 0};
+    auto compute = [&](uint32_t rt, char* slot) __attribute__((always_inline)) {
+        const uint32_t sa = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)slot)) + frag;
+        i32x4 a[kWsTpw];
+#pragma unroll
+        for (uint32_t t = 0; t < kWsTpw; ++t) {
+            const uint32_t addr = sa + (((4u * t + lq) ^ lc) << 4);
+            asm volatile("ds_read_b128 %0, %1" : "=v"(a[t]) : "v"(addr) : "memory");
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7]));
+#pragma unroll
+        for (uint32_t t = 0; t < kWsTpw; ++t) {
+            if (t < cnt) {  // uniform
+#pragma unroll
+                for (uint32_t s = 0; s < kWsSlabs; ++s) {
+                    if (s < nslabs) {  // uniform
+                        acc[s] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[t], wreg[s][t], acc[s], 0, 0, 0);
+                    }
+                }
+            }
+        }
+        // Register i of lane l is row 4 (l / 16) + i of the row tile, column l % 16 of the slab.  Rows past the last
+        // one (copies of it) are added to rows of OUT that nobody reads.  The additions are written as instructions:
+        // an LDS atomic the compiler knows of makes it wait for every direct-to-LDS load in flight first.
+        const uint32_t oa = out_lane + rt * (16u * kWsSlabs * kPkCols * 4u);
+#pragma unroll
+        for (uint32_t s = 0; s < kWsSlabs; ++s) {
+            if (s < nslabs) {  // uniform
+                asm volatile("ds_add_u32 %0, %1 offset:%5\n\tds_add_u32 %0, %2 offset:%6\n\t"
+                             "ds_add_u32 %0, %3 offset:%7\n\tds_add_u32 %0, %4 offset:%8"
+                             :
+                             : "v"(oa), "v"(acc[s][0]), "v"(acc[s][1]), "v"(acc[s][2]), "v"(acc[s][3]),
+                               "i"(s * kPkCols * 4u), "i"(s * kPkCols * 4u + kWsSlabs * kPkCols * 4u),
+                               "i"(s * kPkCols * 4u + 2u * kWsSlabs * kPkCols * 4u),
+                               "i"(s * kPkCols * 4u + 3u * kWsSlabs * kPkCols * 4u)
+                             : "memory");
+            }
+            acc[s] = i32x4{0, 0, 0, 0};
+        }
+    };
+    issue(0u, r0w);
+    issue(1u, r1w);
+    // Loads return in order: with at most the newest slot's kWsDma loads outstanding, everything older (the weights,
+    // the slot about to be read) has arrived.  A slot is refilled as soon as its fragments are in registers; past the
+    // last row tile the refills fetch the last row again, so that the count never changes.
+    for (uint32_t rt = 0; rt < ntiles; rt += 2u) {
+        __builtin_amdgcn_s_waitcnt((kWsDma & 15) | ((kWsDma >> 4) << 14) | (7 << 4) | (15 << 8));
+        compute(rt, r0w);
+        issue(rt + 2u, r0w);
+        if (rt + 1u < ntiles) {
+            __builtin_amdgcn_s_waitcnt((kWsDma & 15) | ((kWsDma >> 4) << 14) | (7 << 4) | (15 << 8));
+            compute(rt + 1u, r1w);
+            issue(rt + 3u, r1w);
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // nothing lands in LDS after the barrier
+    __syncthreads();
+
+    const EpiParams& e = p.epi;
+    const uint32_t width = nslabs * kPkCols;
+    for (uint32_t idx = tid; idx < p.rows * width; idx += kPkWaves * 64u) {
+        const uint32_t row = idx / width, c = idx - row * width;
+        const uint32_t col = s0 * kPkCols + c;
+        if (col >= p.n) {
+            continue;
+        }
+        int32_t sum = OUT[row][c];
+        if (e.bias_kind == ASCQ_MM_BIAS_I32_PRE) {
+            sum += static_cast<const int32_t*>(e.bias)[col];
+        }
+        const float tok = e.has_tok ? e.tok_scale[p.m0 + row] : 1.0f;
+        dispatch_out(e, [&](auto tag) {
+            epilogue_store<decltype(tag)::value>(e, p.m0 + row, col, sum, load_channel_q(e, col), tok,
+                                                 load_bias_post(e, col));
+        });
+    }
+}
+
 // [k, n] (or [n, k] with trans) -> packed; one thread per lane of a tile.
 __global__ __launch_bounds__(256) void pack_w8_kernel(const int8_t* __restrict__ w, i32x4* __restrict__ out, uint32_t k,
                                                       uint32_t n, uint32_t slabs, uint32_t ktiles, int trans)
@@ -547,6 +719,57 @@ int launch_gemm_packed(const GemmParams& p, hipStream_t st, bool b_nk)
         }
     }
     return launch_status(b_nk ? "ascq_matmul_w8a8 ([n, k] weight stream)" : "ascq_matmul_w8a8_packed");
+}
+
+// The weight-stationary form: more than 32 rows, k up to 4096 (a wavefront's k range of a slab fits 8 tile registers),
+// in passes of up to 128 rows.  On packed weights it is the path for every such call (one pass: 14.2 us at 33 rows,
+// 23.0 us at 128, k = 4096, n = 11008; the 32-row passes took 23 and 54 us).  On [n, k] weights, whose tiles arrive
+// as 16 runs of 64 bytes, it only leads the K-split tiles up to 48 rows (17.3 against 17.5-17.9 us; 26.5 against
+// 24.4 us at 128 rows): every workgroup streams all of the activations, which at 128 rows is 128 MB through the L2s.
+bool gemm_ws_supported(const GemmParams& p, bool b_nk)
+{
+    if (p.m <= 2u * kPkMaxRows || p.k % kPkTileK != 0 || p.k / kPkTileK > kPkWaves * kWsTpw) {
+        return false;
+    }
+    if (b_nk) {
+        return p.m <= 48u && gemm_packed_nk_supported(p);
+    }
+    return gemm_packed_supported(p);
+}
+
+int launch_gemm_ws(const GemmParams& p, hipStream_t st, bool b_nk)
+{
+    const uint32_t cus = device_compute_units();
+    PackedParams q{};
+    q.wp = reinterpret_cast<const i32x4*>(p.b);
+    q.a = p.a;
+    q.n = p.n;
+    q.k = p.k;
+    q.slabs = (p.n + kPkCols - 1u) / kPkCols;
+    q.ktiles = p.k / kPkTileK;
+    q.tpw = (q.ktiles + kPkWaves - 1u) / kPkWaves;
+    q.epi = p.epi;
+    q.rows_magic = 0;
+    // one workgroup per compute unit when that leaves it at most kWsSlabs slabs, otherwise more workgroups
+    uint32_t grid = q.slabs < cus ? q.slabs : cus;
+    if ((q.slabs + grid - 1u) / grid > kWsSlabs) {
+        grid = (q.slabs + kWsSlabs - 1u) / kWsSlabs;
+    }
+    for (uint32_t m0 = 0; m0 < p.m; m0 += kWsRows) {
+        q.m0 = m0;
+        q.rows = p.m - m0 < kWsRows ? p.m - m0 : kWsRows;
+        if (plan_note(ASCQ_MM_KERNEL_STREAM, kWsRows, kPkCols * ((q.slabs + grid - 1u) / grid), kPkTileK, grid, 1,
+                      2u * kPkWaves * kWsSlot + kWsRows * kWsSlabs * kPkCols * 4u, 0)) {
+            return ASCQ_OK;
+        }
+        if (b_nk) {
+            gemm_ws_kernel<true><<<grid, kPkWaves * 64u, 0, st>>>(q);
+        } else {
+            gemm_ws_kernel<false><<<grid, kPkWaves * 64u, 0, st>>>(q);
+        }
+    }
+    return launch_status(b_nk ? "ascq_matmul_w8a8 ([n, k] weights held in registers)"
+                              : "ascq_matmul_w8a8_packed (weights held in registers)");
 }
 
 // The fused form: x [m, k] of halves or bfloat16s is quantised per token inside the kernel (p.epi.has_tok must be set;

@@ -64,7 +64,7 @@ def main():
     ap.add_argument("--quick", action="store_true", help="headline + W4A16 GEMV only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="run a single workload: w8a8 | w4a16 | w4a16_per_weight | w4a16_per_weight_m4 | w4a16_per_weight_m16 | w4a16_nd | w4a16_m4 | w4a16_m16 | w4a16_nd_m4 | w4a16_nd_m16 | "
-                         "w8a8_zeros | w8a8_m1 | w8a8_m8 | w8a8_m16 | w8a8_m128 | w8a8_m512 | w8a8_m8192 | w8a8_packed_m1 | w8a8_packed_m8 | w8a8_packed_m16 | w8a8_packed_m32 | w8a8_nk_m32 | w8a8_m32 | w8a8_nk_m1 | w8a8_nk_m16 | w8a8_nk_m128 | w8a8_linear_nk_m1 | w8a8_linear_nk_m4 | w8a8_linear_nk_m16 | w8a8_linear_packed_m1 | w8a8_linear_packed_m4 | w8a16_m1 | w8a16_m16 | w8a16_nk_m1 | w8a16_nk_m4 | w8a16_nk_sum_m1 | w8a16_nk_sum_m4 | "
+                         "w8a8_zeros | w8a8_m1 | w8a8_m8 | w8a8_m16 | w8a8_m128 | w8a8_m512 | w8a8_m8192 | w8a8_packed_m1 | w8a8_packed_m8 | w8a8_packed_m16 | w8a8_packed_m32 | w8a8_packed_m64 | w8a8_packed_m128 | w8a8_nk_m32 | w8a8_nk_m64 | w8a8_m32 | w8a8_nk_m1 | w8a8_nk_m16 | w8a8_nk_m128 | w8a8_linear_nk_m1 | w8a8_linear_nk_m4 | w8a8_linear_nk_m16 | w8a8_linear_packed_m1 | w8a8_linear_packed_m4 | w8a16_m1 | w8a16_m16 | w8a16_nk_m1 | w8a16_nk_m4 | w8a16_nk_sum_m1 | w8a16_nk_sum_m4 | "
                          "w8a16_nk_m16 | w8a16_m2048 | w8a16_nk_m2048 | quant | dequant | antiquant | group | group_example | mx_fp4 | mx_fp4_e1m2 | mx_fp8 (a W4A16 name without _nd "
                          "is the packed-weight path, in the group-sum form unless it says per_weight; _nk: weights kept as [n, k])")
     ap.add_argument("--copy-probe", action="store_true",
@@ -434,6 +434,9 @@ def main():
               "w8a8_packed_m8": lambda: w8a8(8, args.steps, args.warmup, sets=7, packed=True),
               "w8a8_packed_m16": lambda: w8a8(16, args.steps, args.warmup, sets=7, packed=True),
               "w8a8_packed_m32": lambda: w8a8(32, args.steps, args.warmup, sets=7, packed=True),
+              "w8a8_packed_m64": lambda: w8a8(64, args.steps, args.warmup, sets=7, packed=True),
+              "w8a8_packed_m128": lambda: w8a8(128, args.steps, args.warmup, sets=7, packed=True),
+              "w8a8_nk_m64": lambda: w8a8(64, args.steps, args.warmup, sets=7, b_nk=True),
               "w8a8_nk_m32": lambda: w8a8(32, args.steps, args.warmup, sets=7, b_nk=True),
               "w8a8_m32": lambda: w8a8(32, args.steps, args.warmup, sets=7),
               "w8a8_linear_nk_m1": lambda: w8a8_linear(1, args.steps, args.warmup),
@@ -553,7 +556,7 @@ def main():
             others[f"w8a8_m{M}"] = {"gemm_kernel_ms": r["gemm_kernel_ms"], "gemm_tops": r["gemm_tops"],
                                     "gemm_gbs": r["gemm_gbs"], "hbm_frac": r["gemm_gbs"] / PEAK_HBM_GBS,
                                     "mfma_frac": r["gemm_tops"] / PEAK_INT8_TOPS}
-        for M in (1, 8, 16, 32):
+        for M in (1, 8, 16, 32, 64, 128):
             r = strip(w8a8(M, s2, w2, sets=7, packed=True))
             others[f"w8a8_packed_m{M}"] = {"gemm_kernel_ms": r["gemm_kernel_ms"], "gemm_gbs": r["gemm_gbs"],
                                            "hbm_frac": r["gemm_gbs"] / PEAK_HBM_GBS,

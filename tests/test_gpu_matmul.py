@@ -212,6 +212,32 @@ def test_w8a8_packed_small(m, n, k):
     assert max_ulp(bits(cg), oracle_mm(dg, a, b).view(np.uint16), "f16") <= 1
 
 
+@pytest.mark.parametrize("m", [33, 47, 48, 64, 100, 128, 129, 300])
+@pytest.mark.parametrize("n,k", [(16, 64), (48, 128), (1040, 512), (272, 4096), (2064, 192), (13000, 256), (96, 4160)])
+def test_w8a8_weights_held_in_registers(m, n, k):
+    """More than 32 rows on packed weights (33 to 48 on [n, k] weights): the weights of a workgroup's columns stay in
+    registers and the activations stream past them in passes of up to 128 rows (k up to 4096; longer k and, on [n, k]
+    weights, more rows take the other kernels).  int32 accumulators against int64 arithmetic, the dequantising
+    epilogue bit for bit against the oracle, both forms."""
+    announce("w8a8 weights in registers", m, n, k)
+    rng = np.random.default_rng(m * 37 + n + k)
+    a, b = rand_i8(rng, (m, k)), rand_i8(rng, (k, n))
+    bt = np.ascontiguousarray(b.T)
+    want = a.astype(np.int64) @ b.astype(np.int64)
+    c, _ = run_mm_packed(m, n, k, a, b, out=torch.int32)
+    assert np.array_equal(c.cpu().numpy(), want)
+    c, _ = run_mm(m, n, k, a, bt, out=torch.int32, trans_b=True)
+    assert np.array_equal(c.cpu().numpy(), want)
+    cs = rng.uniform(1e-4, 1e-2, n).astype(np.float32)
+    ts = rng.uniform(1e-2, 1e-1, m).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    c, desc = run_mm_packed(m, n, k, a, b, out=torch.bfloat16, bias=(bias, None), quant=cs, tok=ts)
+    gold = oracle_mm(desc, a, b, (bias, None), cs, ts)
+    assert np.array_equal(bits(c), gold)
+    c, desc = run_mm(m, n, k, a, bt, out=torch.bfloat16, bias=(bias, None), quant=cs, tok=ts, trans_b=True)
+    assert np.array_equal(bits(c), gold)
+
+
 @pytest.mark.parametrize("m", [1, 16, 32])
 def test_config3_w8a8_linear_packed(m):
     """Config 3's decode sizes on packed weights: per-token quantisation on the GPU, one launch for the matmul, bf16
