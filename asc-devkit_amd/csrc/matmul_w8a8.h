@@ -231,10 +231,9 @@ int launch_gemm_nk(const GemmParams& p, hipStream_t st);
 // (matmul_w8a8_packed.hip).
 bool gemm_packed_supported(const GemmParams& p);
 bool gemm_packed_nk_supported(const GemmParams& p);
-bool gemm_packed_two_tiles_fit(uint32_t k);  // 17 to 32 rows in one pass over the weights
 int launch_gemm_packed(const GemmParams& p, hipStream_t st, bool b_nk = false);
-// More than 32 rows on packed weights (33 to 48 on [n, k] weights): the weights of a workgroup's columns held in
-// registers, the activations streamed past them in passes of up to 128 rows (k up to 4096).
+// More than 16 rows on packed weights (17 to 224 on [n, k] weights): the weights of a workgroup's columns held in
+// registers, the activations streamed past them, one launch (k up to 4096).
 bool gemm_ws_supported(const GemmParams& p, bool b_nk);
 int launch_gemm_ws(const GemmParams& p, hipStream_t st, bool b_nk);
 // The same kernel with the per-token quantisation of x (half or bfloat16, [m, k]) inside: m <= 8 rows that fit the LDS.

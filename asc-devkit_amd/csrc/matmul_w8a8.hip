@@ -647,6 +647,11 @@ extern "C" int ascq_matmul_w8a8_workspace_size(const ascq_matmul_desc* d, size_t
         *bytes = round256(inner) + static_cast<size_t>(d->m) * d->n * sizeof(int32_t);
         return ASCQ_OK;
     }
+    // 17 to 224 rows on [n, k] weights with k up to 4096 run with the weights held in registers: no scratch
+    const bool ws_nk = d->trans_b && !d->trans_a && d->b_format == ASCQ_MM_B_ND && gemm_ws_supported(shape, true);
+    if (ws_nk) {
+        return ASCQ_OK;
+    }
     if (d->m <= 32 && !d->trans_a && pick_k_splits(d->n, d->k) > 1 && !(d->trans_b && d->k % 128 == 0)) {
         // (few rows on [n, k] weights with k % 128 == 0 run the whole-column kernel, which needs none)
         *bytes = static_cast<size_t>(d->m) * d->n * sizeof(int32_t);
@@ -739,12 +744,11 @@ extern "C" int ascq_matmul_w8a8(const ascq_matmul_desc* d, void* c, const void* 
         workspace_bytes >= gemm_stream_workspace(d->m, d->n, d->k)) {
         return launch_gemm_stream(p, workspace, st);
     }
-    if (d->m <= 32 && d->trans_b && !d->trans_a && gemm_packed_nk_supported(p) &&
-        (d->m <= 16 || gemm_packed_two_tiles_fit(d->k))) {
-        return launch_gemm_packed(p, st, true);  // activations resident in LDS, nothing but weights in the load queue
-    }
     if (d->trans_b && !d->trans_a && gemm_ws_supported(p, true)) {
-        return launch_gemm_ws(p, st, true);  // 33 to 48 rows: the weights held in registers, the activations streamed
+        return launch_gemm_ws(p, st, true);  // 17 to 224 rows: the weights held in registers, the activations streamed
+    }
+    if (d->m <= 16 && d->trans_b && !d->trans_a && gemm_packed_nk_supported(p)) {
+        return launch_gemm_packed(p, st, true);  // activations resident in LDS, nothing but weights in the load queue
     }
     if (d->m <= 32 && d->trans_b && !d->trans_a && gemm_nk_supported(p)) {
         return launch_gemm_nk(p, st);

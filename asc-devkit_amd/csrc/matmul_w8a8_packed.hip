@@ -1,5 +1,7 @@
 // int8 matmul for few activation rows (decode, small batches) on weights pre-packed for this GPU: one launch, no
-// workspace, one flat sweep over the weights.
+// workspace, one flat sweep over the weights.  Up to 16 rows the activations stay in LDS and the weights stream past
+// them (gemm_packed_kernel, and gemm_packed_dyn_kernel with the per-token quantiser inside); more rows turn the roles
+// round (gemm_ws_kernel: the weights stay in registers and the activations stream).
 //
 // Packed layout (ascq_pack_weight_w8): the [k, n] matrix is cut into slabs of 16 columns and tiles of 64 k; a tile of a
 // slab is 1 KiB and the tiles of a slab, then the slabs, follow each other in memory.  Inside a tile lane l of a
@@ -32,9 +34,6 @@ constexpr uint32_t kPkWaves = 8, kPkBatch = 4, kPkMaxSlabs = 8, kPkMaxRows = 16;
 constexpr int kPkBuf = 2;              // register buffers: one batch in flight while the other is computed
 constexpr uint32_t kPkRowPad = 16;     // bytes added to a staged activation row: rows start 4 banks apart
 constexpr uint32_t kPkXBytes = 88 * 1024;  // LDS for the staged activations of a workgroup (the partial sums take 64 KiB)
-// With two row tiles (17 to 32 rows per pass) the activations take up to 136 KiB and the wavefronts add their tiles
-// into one [slab][row][column] array with LDS atomics (integers: exact in any order) instead of keeping eight copies.
-constexpr uint32_t kPkXBytes2 = 136 * 1024;
 constexpr uint32_t kPkPastEnd = 0x7FFFFFF0u;
 constexpr int kPkNt = 2;               // cache policy of the weight loads: non-temporal (read once per call)
 
@@ -58,11 +57,11 @@ __device__ __forceinline__ uint32_t pk_xcd_order(uint32_t wg, uint32_t wgs)
     return (wgs & 7u) == 0u ? (wg & 7u) * (wgs >> 3) + (wg >> 3) : wg;
 }
 
-template <bool kNK, int RT>
+template <bool kNK>
 __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_kernel(PackedParams p)
 {
-    __shared__ __attribute__((aligned(16))) char XS[RT == 2 ? kPkXBytes2 : kPkXBytes];
-    __shared__ int32_t RED[RT == 2 ? 1 : kPkWaves][kPkMaxSlabs][RT == 2 ? 8 : 4][64];  // RT == 2: [slab][row / 4][..]
+    __shared__ __attribute__((aligned(16))) char XS[kPkXBytes];
+    __shared__ int32_t RED[kPkWaves][kPkMaxSlabs][4][64];
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t lc = lane & 15u, lq = lane >> 4;
@@ -91,15 +90,8 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_kernel(PackedParams
         const_cast<i32x4*>(p.wp), 0,
         static_cast<int>(kNK ? p.n * p.k : (p.slabs * p.ktiles + kPkPadTiles) * kPkTileBytes), 0x00020000);
     const uint32_t w_lane = kNK ? lc * p.k + lq * 16u : lane * 16u;  // the lane's 16 bytes inside a tile
-    // operand row i reads row i % rows; + tile * 64.  Second row tile (RT == 2, more than 16 rows): rows 16 + i, past
-    // the end the last row again (never stored).
+    // operand row i reads row i % rows; + tile * 64
     const uint32_t x_lane = (lc - __umulhi(lc, p.rows_magic) * p.rows) * pitch + lq * 16u;
-    const uint32_t x_lane2 = min(16u + lc, p.rows - 1u) * pitch + lq * 16u;
-    if constexpr (RT == 2) {
-        // the shared sums start at zero; the barrier also orders this against the first atomic
-        for (uint32_t i = tid; i < kPkMaxSlabs * 8u * 64u; i += kPkWaves * 64u) (&RED[0][0][0][0])[i] = 0;
-        __syncthreads();
-    }
 
     // ---- batches of kPkBatch tiles that never straddle a slab: batch q = (slab q / nb, tiles ta + (q % nb) kPkBatch ...)
     const uint32_t nb = (cnt + kPkBatch - 1u) / kPkBatch;
@@ -137,7 +129,7 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_kernel(PackedParams
     __builtin_amdgcn_s_waitcnt(((kPkBuf * kPkBatch) & 15) | (((kPkBuf * kPkBatch) >> 4) << 14) | (7 << 4) | (15 << 8));
     asm volatile("" ::: "memory");
 
-    i32x4 acc = {0, 0, 0, 0}, acc2 = {0, 0, 0, 0};
+    i32x4 acc = {0, 0, 0, 0};
     uint32_t c_slab = 0, c_b = 0, c_q = 0;
     auto compute = [&](int buf) __attribute__((always_inline)) {
         if (c_q >= batches) {
@@ -151,26 +143,12 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_kernel(PackedParams
             if (t < live) {  // uniform
                 const i32x4 a = *reinterpret_cast<const i32x4*>(xa0 + t * kPkTileK);
                 acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, wq[buf][t], acc, 0, 0, 0);
-                if constexpr (RT == 2) {
-                    const i32x4 a2 = *reinterpret_cast<const i32x4*>(xs + x_lane2 + (t0 + t) * kPkTileK);
-                    acc2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a2, wq[buf][t], acc2, 0, 0, 0);
-                }
             }
         }
         ++c_q;
         if (++c_b == nb) {  // the slab is done: register i of lane l is row 4 (l / 16) + i, column l % 16
-            if constexpr (RT == 2) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    __hip_atomic_fetch_add(&RED[0][c_slab][i][lane], acc[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                    __hip_atomic_fetch_add(&RED[0][c_slab][4 + i][lane], acc2[i], __ATOMIC_RELAXED,
-                                           __HIP_MEMORY_SCOPE_WORKGROUP);
-                }
-                acc2 = i32x4{0, 0, 0, 0};
-            } else {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) RED[wave][c_slab][i][lane] = acc[i];
-            }
+            for (int i = 0; i < 4; ++i) RED[wave][c_slab][i][lane] = acc[i];
             acc = i32x4{0, 0, 0, 0};
             c_b = 0;
             ++c_slab;
@@ -183,7 +161,7 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_kernel(PackedParams
             load(b);
         }
     }
-    if (RT == 1 && batches == 0u) {  // a wavefront without tiles (k shorter than 8 tiles) contributes zeros
+    if (batches == 0u) {  // a wavefront without tiles (k shorter than 8 tiles) contributes zeros
         for (uint32_t s = 0; s < nslabs; ++s) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) RED[wave][s][i][lane] = 0;
@@ -202,16 +180,14 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_kernel(PackedParams
         const float bp = load_bias_post(e, col);
         const int32_t bias_pre = e.bias_kind == ASCQ_MM_BIAS_I32_PRE ? static_cast<const int32_t*>(e.bias)[col] : 0;
 #pragma unroll
-        for (int i = 0; i < 4 * RT; ++i) {
-            const uint32_t row_in_pass = 16u * (i >> 2) + 4u * lq + static_cast<uint32_t>(i & 3);
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t row_in_pass = 4u * lq + static_cast<uint32_t>(i);
             if (row_in_pass >= p.rows) {
                 continue;
             }
             int32_t sum = RED[0][s][i][lane];
-            if constexpr (RT == 1) {
 #pragma unroll
-                for (uint32_t wv = 1; wv < kPkWaves; ++wv) sum += RED[wv][s][i][lane];
-            }
+            for (uint32_t wv = 1; wv < kPkWaves; ++wv) sum += RED[wv][s][i][lane];
             sum += bias_pre;
             const uint32_t row = p.m0 + row_in_pass;
             const float tok = e.has_tok ? e.tok_scale[row] : 1.0f;
@@ -443,7 +419,7 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_dyn_kernel(PackedPa
     }
 }
 
-// The weight-stationary form, for more than 32 activation rows (up to 128 per launch).  That many rows do not fit the LDS, and activations that
+// The weight-stationary form, for more than 16 activation rows.  Many rows do not fit the LDS, and activations that
 // are streamed beside the weights share the compute unit's in-order load queue with them (every L2 hit of an
 // activation load then waits behind the weights' trips to memory).  So the two are separated in time: a workgroup
 // first requests all the weights of its columns (up to 3 slabs x 64 tiles = 192 KiB, a wavefront holding its k range
@@ -452,6 +428,7 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_dyn_kernel(PackedPa
 // slab and tile on operands that are already in registers.  A row tile's sums over the wavefronts' k ranges meet in
 // one LDS array (atomic adds of integers: exact in any order); the epilogue runs once at the end.
 constexpr uint32_t kWsSlabs = 3, kWsTpw = 8, kWsRows = 128;
+constexpr uint32_t kWsNkMaxRows = 224;  // [n, k] weights: beyond this the tile kernels are level or ahead
 constexpr uint32_t kWsRowBytes = kWsTpw * kPkTileK;   // 512: a staged row (the wavefront's k range, padded)
 constexpr uint32_t kWsSlot = 16u * kWsRowBytes;       // 8 KiB: 16 rows
 constexpr int kWsDma = 8;                             // direct-to-LDS instructions per slot (two rows each)
@@ -462,6 +439,7 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_ws_kernel(PackedParams p)
     __shared__ __attribute__((aligned(1024))) char R0[kPkWaves * kWsSlot];
     __shared__ __attribute__((aligned(1024))) char R1[kPkWaves * kWsSlot];
     __shared__ int32_t OUT[kWsRows][kWsSlabs * kPkCols];
+    __shared__ float TS[kWsRows];
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t lc = lane & 15u, lq = lane >> 4;
@@ -470,8 +448,15 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_ws_kernel(PackedParams p)
     const uint32_t s1 = static_cast<uint32_t>(static_cast<uint64_t>(wg + 1u) * p.slabs / gridDim.x);
     const uint32_t nslabs = s1 - s0;  // at most kWsSlabs: the host has chosen the grid
     const uint32_t ta = min(wave * p.tpw, p.ktiles), tb = min(ta + p.tpw, p.ktiles), cnt = tb - ta;  // at most kWsTpw
-    for (uint32_t i = tid; i < kWsRows * kWsSlabs * kPkCols; i += kPkWaves * 64u) (&OUT[0][0])[i] = 0;
-    __syncthreads();  // before any direct-to-LDS load is in flight
+    // the sums of a block of kWsRows rows start at zero; the rows' token scales are kept for the epilogue
+    auto begin_block = [&](uint32_t b0) __attribute__((always_inline)) {
+        for (uint32_t i = tid; i < kWsRows * kWsSlabs * kPkCols; i += kPkWaves * 64u) (&OUT[0][0])[i] = 0;
+        if (tid < kWsRows) {
+            TS[tid] = (p.epi.has_tok && b0 + tid < p.rows) ? p.epi.tok_scale[p.m0 + b0 + tid] : 1.0f;
+        }
+        __syncthreads();  // no direct-to-LDS load is in flight here
+    };
+    begin_block(0u);
 
     // ---- the weights of this wavefront's k range, all slabs: one burst, nothing else in the queue yet
     const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(
@@ -498,18 +483,18 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_ws_kernel(PackedParams p)
     char* const r1w = R1 + wave * kWsSlot;
     // A load's address is a wavefront-uniform base (the row tile) plus the lane's 32-bit offset, which the instruction
     // adds itself; the last row tile, where rows past the end repeat the last row, has offsets of its own.
-    const uint32_t ntiles = (p.rows + 15u) / 16u;
-    const uint32_t rows_last = p.rows - (ntiles - 1u) * 16u;  // rows of the last row tile, 1 .. 16
-    uint32_t a_off[kWsDma], a_off_last[kWsDma];
+    // (ntiles, the offsets of the last tile and the base belong to the block of rows being worked on)
+    uint32_t ntiles = 0;
+    uint32_t a_off[kWsDma], a_off_last[kWsDma], a_col[kWsDma];
 #pragma unroll
     for (int u = 0; u < kWsDma; ++u) {
         const uint32_t sidx = static_cast<uint32_t>(u) * 64u + lane;
         const uint32_t r = sidx >> 5, q = (sidx & 31u) ^ r;
-        const uint32_t col = (q < cnt * 4u ? q : 0u) * 16u + ta * kPkTileK;
-        a_off[u] = r * p.k + col;
-        a_off_last[u] = min(r, rows_last - 1u) * p.k + col;
+        a_col[u] = (q < cnt * 4u ? q : 0u) * 16u + ta * kPkTileK;
+        a_off[u] = r * p.k + a_col[u];
+        a_off_last[u] = a_off[u];
     }
-    const int8_t* const a_base = p.a + static_cast<size_t>(p.m0) * p.k;
+    const int8_t* a_base = p.a;
     auto issue = [&](uint32_t rt, char* slot) __attribute__((always_inline)) {
         // past the last row tile: the last one again (never read; keeps the count of loads in flight what the waits assume)
         const uint32_t tile = rt < ntiles ? rt : ntiles - 1u;
@@ -577,41 +562,59 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_ws_kernel(PackedParams p)
             acc[s] = i32x4{0, 0, 0, 0};
         }
     };
+    const EpiParams& e = p.epi;
+    uint32_t brows = 0;
+    auto set_block = [&](uint32_t b0) __attribute__((always_inline)) {
+        brows = min(kWsRows, p.rows - b0);
+        ntiles = (brows + 15u) / 16u;
+        const uint32_t rows_last = brows - (ntiles - 1u) * 16u;  // rows of the block's last row tile, 1 .. 16
+#pragma unroll
+        for (int u = 0; u < kWsDma; ++u) {
+            const uint32_t r = (static_cast<uint32_t>(u) * 64u + lane) >> 5;
+            a_off_last[u] = min(r, rows_last - 1u) * p.k + a_col[u];
+        }
+        a_base = p.a + static_cast<size_t>(p.m0 + b0) * p.k;
+    };
+    // the first block's first two row tiles are requested right behind the weights
+    set_block(0u);
     issue(0u, r0w);
     issue(1u, r1w);
-    // Loads return in order: with at most the newest slot's kWsDma loads outstanding, everything older (the weights,
-    // the slot about to be read) has arrived.  A slot is refilled as soon as its fragments are in registers; past the
-    // last row tile the refills fetch the last row again, so that the count never changes.
-    for (uint32_t rt = 0; rt < ntiles; rt += 2u) {
-        __builtin_amdgcn_s_waitcnt((kWsDma & 15) | ((kWsDma >> 4) << 14) | (7 << 4) | (15 << 8));
-        compute(rt, r0w);
-        issue(rt + 2u, r0w);
-        if (rt + 1u < ntiles) {
+    for (uint32_t b0 = 0; b0 < p.rows; b0 += kWsRows) {  // blocks of kWsRows rows: the weights stay where they are
+        // Loads return in order: with at most the newest slot's kWsDma loads outstanding, everything older (the
+        // weights, the slot about to be read) has arrived.  A slot is refilled as soon as its fragments are in
+        // registers; past the last row tile the refills fetch the last tile again, so that the count never changes.
+        for (uint32_t rt = 0; rt < ntiles; rt += 2u) {
             __builtin_amdgcn_s_waitcnt((kWsDma & 15) | ((kWsDma >> 4) << 14) | (7 << 4) | (15 << 8));
-            compute(rt + 1u, r1w);
-            issue(rt + 3u, r1w);
+            compute(rt, r0w);
+            issue(rt + 2u, r0w);
+            if (rt + 1u < ntiles) {
+                __builtin_amdgcn_s_waitcnt((kWsDma & 15) | ((kWsDma >> 4) << 14) | (7 << 4) | (15 << 8));
+                compute(rt + 1u, r1w);
+                issue(rt + 3u, r1w);
+            }
         }
-    }
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // nothing lands in LDS after the barrier
-    __syncthreads();
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // nothing lands in LDS after the barrier
+        __syncthreads();
 
-    const EpiParams& e = p.epi;
-    const uint32_t width = nslabs * kPkCols;
-    for (uint32_t idx = tid; idx < p.rows * width; idx += kPkWaves * 64u) {
-        const uint32_t row = idx / width, c = idx - row * width;
-        const uint32_t col = s0 * kPkCols + c;
-        if (col >= p.n) {
-            continue;
+        // ---- a thread keeps one column (its parameters are fetched once) and walks down the rows, eight apart
+        const uint32_t c = lane, col = s0 * kPkCols + c;
+        if (c < nslabs * kPkCols && col < p.n) {
+            const ChannelQ q = load_channel_q(e, col);
+            const float bp = load_bias_post(e, col);
+            const int32_t bias_pre = e.bias_kind == ASCQ_MM_BIAS_I32_PRE ? static_cast<const int32_t*>(e.bias)[col] : 0;
+            dispatch_out(e, [&](auto tag) {
+                for (uint32_t row = wave; row < brows; row += kPkWaves) {
+                    epilogue_store<decltype(tag)::value>(e, p.m0 + b0 + row, col, OUT[row][c] + bias_pre, q, TS[row], bp);
+                }
+            });
         }
-        int32_t sum = OUT[row][c];
-        if (e.bias_kind == ASCQ_MM_BIAS_I32_PRE) {
-            sum += static_cast<const int32_t*>(e.bias)[col];
+        if (b0 + kWsRows < p.rows) {
+            __syncthreads();  // the next block clears what this epilogue read
+            begin_block(b0 + kWsRows);
+            set_block(b0 + kWsRows);
+            issue(0u, r0w);
+            issue(1u, r1w);
         }
-        const float tok = e.has_tok ? e.tok_scale[p.m0 + row] : 1.0f;
-        dispatch_out(e, [&](auto tag) {
-            epilogue_store<decltype(tag)::value>(e, p.m0 + row, col, sum, load_channel_q(e, col), tok,
-                                                 load_bias_post(e, col));
-        });
     }
 }
 
@@ -657,19 +660,14 @@ bool gemm_packed_nk_supported(const GemmParams& p)
            static_cast<uint64_t>(p.n + kPkCols) * p.k < (1ull << 31) - 64u * kPkTileK;
 }
 
-bool gemm_packed_two_tiles_fit(uint32_t k)
-{
-    const uint32_t tpw = (k / kPkTileK + kPkWaves - 1u) / kPkWaves;
-    return 2u * kPkMaxRows * kPkWaves * (tpw * kPkTileK + kPkRowPad) <= kPkXBytes2;
-}
-
 bool gemm_packed_supported(const GemmParams& p)
 {
     return p.k % kPkTileK == 0 && aligned16(p.a) && aligned16(p.b) &&
            (static_cast<uint64_t>((p.n + kPkCols - 1u) / kPkCols) * (p.k / kPkTileK) + kPkPadTiles) * kPkTileBytes < (1ull << 31);
 }
 
-// p.b: the packed weights, or with b_nk the plain [n, k] matrix.  Any m: up to 16 rows per pass over the weights.
+// p.b: the packed weights, or with b_nk the plain [n, k] matrix.  Any m: up to 16 rows per pass over the weights
+// (the callers send more than 16 rows here only when k is too long for the weight-stationary form).
 int launch_gemm_packed(const GemmParams& p, hipStream_t st, bool b_nk)
 {
     const int cus = static_cast<int>(device_compute_units());
@@ -687,52 +685,44 @@ int launch_gemm_packed(const GemmParams& p, hipStream_t st, bool b_nk)
     if ((q.slabs + grid - 1u) / grid > kPkMaxSlabs) {
         grid = (q.slabs + kPkMaxSlabs - 1u) / kPkMaxSlabs;
     }
-    // rows per pass: 16, fewer when k is so long that the staged activations of 16 rows would not fit the LDS; 32 (two
-    // row tiles sharing every weight fetch) while more than 16 rows are left and 32 rows fit the larger staging area
+    // rows per pass: 16, fewer when k is so long that the staged activations of 16 rows would not fit the LDS
     const uint32_t row_bytes = kPkWaves * (q.tpw * kPkTileK + kPkRowPad);
     uint32_t pass_rows = kPkXBytes / row_bytes;
     pass_rows = pass_rows > kPkMaxRows ? kPkMaxRows : pass_rows;
     if (pass_rows == 0u) {
         return fail(ASCQ_EUNSUPPORTED, "ascq_matmul_w8a8_packed: k = %u is too long for the staged activations", p.k);
     }
-    const bool two_tiles_fit = 2u * kPkMaxRows * row_bytes <= kPkXBytes2;
     for (uint32_t m0 = 0; m0 < p.m; m0 += q.rows) {
         const uint32_t left = p.m - m0;
-        const bool two = two_tiles_fit && left > kPkMaxRows;
         q.m0 = m0;
-        q.rows = two ? (left < 2u * kPkMaxRows ? left : 2u * kPkMaxRows) : (left < pass_rows ? left : pass_rows);
+        q.rows = left < pass_rows ? left : pass_rows;
         q.rows_magic = static_cast<uint32_t>(((1ull << 32) + q.rows - 1u) / q.rows);
-        if (plan_note(ASCQ_MM_KERNEL_STREAM, two ? 32 : 16, 16 * ((q.slabs + grid - 1u) / grid), kPkTileK, grid, 1,
-                      two ? kPkXBytes2 + kPkMaxSlabs * 8u * 256u : kPkXBytes + kPkWaves * kPkMaxSlabs * 1024u, 0)) {
+        if (plan_note(ASCQ_MM_KERNEL_STREAM, 16, 16 * ((q.slabs + grid - 1u) / grid), kPkTileK, grid, 1,
+                      kPkXBytes + kPkWaves * kPkMaxSlabs * 1024u, 0)) {
             return ASCQ_OK;
         }
-        if (two) {
-            if (b_nk) {
-                gemm_packed_kernel<true, 2><<<grid, kPkWaves * 64u, 0, st>>>(q);
-            } else {
-                gemm_packed_kernel<false, 2><<<grid, kPkWaves * 64u, 0, st>>>(q);
-            }
-        } else if (b_nk) {
-            gemm_packed_kernel<true, 1><<<grid, kPkWaves * 64u, 0, st>>>(q);
+        if (b_nk) {
+            gemm_packed_kernel<true><<<grid, kPkWaves * 64u, 0, st>>>(q);
         } else {
-            gemm_packed_kernel<false, 1><<<grid, kPkWaves * 64u, 0, st>>>(q);
+            gemm_packed_kernel<false><<<grid, kPkWaves * 64u, 0, st>>>(q);
         }
     }
     return launch_status(b_nk ? "ascq_matmul_w8a8 ([n, k] weight stream)" : "ascq_matmul_w8a8_packed");
 }
 
-// The weight-stationary form: more than 32 rows, k up to 4096 (a wavefront's k range of a slab fits 8 tile registers),
-// in passes of up to 128 rows.  On packed weights it is the path for every such call (one pass: 14.2 us at 33 rows,
-// 23.0 us at 128, k = 4096, n = 11008; the 32-row passes took 23 and 54 us).  On [n, k] weights, whose tiles arrive
-// as 16 runs of 64 bytes, it only leads the K-split tiles up to 48 rows (17.3 against 17.5-17.9 us; 26.5 against
-// 24.4 us at 128 rows): every workgroup streams all of the activations, which at 128 rows is 128 MB through the L2s.
+// The weight-stationary form: more than 16 rows, k up to 4096 (a wavefront's k range of a slab fits 8 tile registers),
+// any number of rows in one launch (the sums and the epilogue go in blocks of 128 rows).  At k = 4096, n = 11008 it
+// costs 9.5 us (packed weights; 11.5 us for [n, k] weights, whose tiles arrive as 16 runs of 64 bytes) plus about 1 us
+// per 16 rows: every workgroup streams all of the activations, 128 MB through the L2s at 128 rows.  On packed weights it
+// is the path for every call of more than 16 rows; on [n, k] weights up to 128 rows, where it leads the K-split tiles
+// (22.3 against 24.4 us at 128 rows).
 bool gemm_ws_supported(const GemmParams& p, bool b_nk)
 {
-    if (p.m <= 2u * kPkMaxRows || p.k % kPkTileK != 0 || p.k / kPkTileK > kPkWaves * kWsTpw) {
+    if (p.m <= kPkMaxRows || p.k % kPkTileK != 0 || p.k / kPkTileK > kPkWaves * kWsTpw) {
         return false;
     }
     if (b_nk) {
-        return p.m <= 48u && gemm_packed_nk_supported(p);
+        return p.m <= kWsNkMaxRows && gemm_packed_nk_supported(p);  // more rows: the tile kernels
     }
     return gemm_packed_supported(p);
 }
@@ -755,18 +745,16 @@ int launch_gemm_ws(const GemmParams& p, hipStream_t st, bool b_nk)
     if ((q.slabs + grid - 1u) / grid > kWsSlabs) {
         grid = (q.slabs + kWsSlabs - 1u) / kWsSlabs;
     }
-    for (uint32_t m0 = 0; m0 < p.m; m0 += kWsRows) {
-        q.m0 = m0;
-        q.rows = p.m - m0 < kWsRows ? p.m - m0 : kWsRows;
-        if (plan_note(ASCQ_MM_KERNEL_STREAM, kWsRows, kPkCols * ((q.slabs + grid - 1u) / grid), kPkTileK, grid, 1,
-                      2u * kPkWaves * kWsSlot + kWsRows * kWsSlabs * kPkCols * 4u, 0)) {
-            return ASCQ_OK;
-        }
-        if (b_nk) {
-            gemm_ws_kernel<true><<<grid, kPkWaves * 64u, 0, st>>>(q);
-        } else {
-            gemm_ws_kernel<false><<<grid, kPkWaves * 64u, 0, st>>>(q);
-        }
+    q.m0 = 0;
+    q.rows = p.m;
+    if (plan_note(ASCQ_MM_KERNEL_STREAM, kWsRows, kPkCols * ((q.slabs + grid - 1u) / grid), kPkTileK, grid, 1,
+                  2u * kPkWaves * kWsSlot + kWsRows * kWsSlabs * kPkCols * 4u, 0)) {
+        return ASCQ_OK;
+    }
+    if (b_nk) {
+        gemm_ws_kernel<true><<<grid, kPkWaves * 64u, 0, st>>>(q);
+    } else {
+        gemm_ws_kernel<false><<<grid, kPkWaves * 64u, 0, st>>>(q);
     }
     return launch_status(b_nk ? "ascq_matmul_w8a8 ([n, k] weights held in registers)"
                               : "ascq_matmul_w8a8_packed (weights held in registers)");

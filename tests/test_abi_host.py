@@ -256,7 +256,11 @@ def test_matmul_plan_of_the_benchmark_shapes():
     assert (p.kernel, p.tile_m, p.tile_n, p.narrow_tile_n, p.launches) == (abi.MM_KERNEL_DMA_256, 256, 256, 128, 1)
     p, _ = _plan(300, 11008, 4096, trans_b=1)
     assert (p.kernel, p.tile_m, p.tile_n, p.k_splits, p.launches) == (abi.MM_KERNEL_DMA_128, 128, 128, 1, 1)
+    # 17 to 224 rows on [n, k] weights (k up to 4096): weights held in registers, activations streamed, no scratch
     p, need = _plan(100, 11008, 4096, trans_b=1)
+    assert (p.kernel, p.k_splits, p.launches, p.workgroups) == (abi.MM_KERNEL_STREAM, 1, 1, 256)
+    assert p.workspace_bytes == need == 0
+    p, need = _plan(100, 11008, 8192, trans_b=1)
     assert (p.kernel, p.k_splits, p.launches) == (abi.MM_KERNEL_DMA_128, 4, 2) and p.workspace_bytes == need
     p, _ = _plan(300, 11008, 4096 + 64, trans_b=1)
     assert (p.kernel, p.launches) == (abi.MM_KERNEL_STAGED, 1)

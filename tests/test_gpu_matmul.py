@@ -190,8 +190,9 @@ def test_pack_weight_w8_layout(k, n):
 def test_w8a8_packed_small(m, n, k):
     """The one-launch kernel on packed weights computes what ascq_matmul_w8a8 computes: int32 accumulators and the
     dequantising epilogues bit for bit against the oracle on the unpacked weights.  k of one tile (seven wavefronts
-    without work), column tails, more rows than a pass, k long enough for several batches per slab; 17 to 32 rows in
-    one pass with two row tiles where the activations fit (k up to 4096), in passes of 16 or fewer where they do not."""
+    without work), column tails, more rows than a pass, k long enough for several batches per slab; more than 16 rows
+    with the weights held in registers where a wavefront's k range fits them (k up to 4096), in passes of 16 rows or
+    fewer where it does not."""
     announce("w8a8 packed", m, n, k)
     rng = np.random.default_rng(m * 31 + n + k)
     a, b = rand_i8(rng, (m, k)), rand_i8(rng, (k, n))
@@ -212,13 +213,13 @@ def test_w8a8_packed_small(m, n, k):
     assert max_ulp(bits(cg), oracle_mm(dg, a, b).view(np.uint16), "f16") <= 1
 
 
-@pytest.mark.parametrize("m", [33, 47, 48, 64, 100, 128, 129, 300])
+@pytest.mark.parametrize("m", [17, 33, 47, 64, 100, 128, 129, 224, 225, 300])
 @pytest.mark.parametrize("n,k", [(16, 64), (48, 128), (1040, 512), (272, 4096), (2064, 192), (13000, 256), (96, 4160)])
 def test_w8a8_weights_held_in_registers(m, n, k):
-    """More than 32 rows on packed weights (33 to 48 on [n, k] weights): the weights of a workgroup's columns stay in
-    registers and the activations stream past them in passes of up to 128 rows (k up to 4096; longer k and, on [n, k]
-    weights, more rows take the other kernels).  int32 accumulators against int64 arithmetic, the dequantising
-    epilogue bit for bit against the oracle, both forms."""
+    """More than 16 rows on packed weights (17 to 224 on [n, k] weights): the weights of a workgroup's columns stay in
+    registers and the activations stream past them, the sums and the epilogue in blocks of 128 rows (k up to 4096;
+    longer k and, on [n, k] weights, more rows take the other kernels).  int32 accumulators against int64
+    arithmetic, the dequantising epilogue bit for bit against the oracle, both forms."""
     announce("w8a8 weights in registers", m, n, k)
     rng = np.random.default_rng(m * 37 + n + k)
     a, b = rand_i8(rng, (m, k)), rand_i8(rng, (k, n))
@@ -277,7 +278,8 @@ def test_w8a8_packed_rejects():
 @pytest.mark.parametrize("m", [48, 128, 300, 512])
 def test_config3_w8a8_mid_m_both_weight_layouts(m):
     """Config 3 between the decode sizes and the large tiles: 128 x 128 direct-to-LDS tiles, K split four ways for one
-    row tile and not at all for more, on weights as [k, n] and as [n, k]; bit-exact against the oracle."""
+    row tile and not at all for more, on weights as [k, n]; on [n, k] weights the same tiles from 225 rows on and the
+    weights-in-registers kernel below; bit-exact against the oracle."""
     announce("config 3 mid m", m)
     rng = np.random.default_rng(0xC3 + 200 + m)
     k, n = 4096, 11008
@@ -290,10 +292,13 @@ def test_config3_w8a8_mid_m_both_weight_layouts(m):
     assert np.array_equal(bits(c), want)
     ct, _ = run_mm(m, n, k, a, np.ascontiguousarray(w.T), out=torch.bfloat16, quant=cs, tok=ts, trans_b=True)
     assert np.array_equal(bits(ct), want)
-    desc.trans_b = 1
+    # [k, n]: one row tile splits K four ways through the workspace; [n, k]: up to 224 rows need none
     wsz = C.c_size_t(0)
     assert abi.load_library().ascq_matmul_w8a8_workspace_size(C.byref(desc), C.byref(wsz)) == abi.OK
     assert wsz.value == (4 * m * n * 4 if m <= 128 else 0)
+    desc.trans_b = 1
+    assert abi.load_library().ascq_matmul_w8a8_workspace_size(C.byref(desc), C.byref(wsz)) == abi.OK
+    assert wsz.value == 0
 
 
 def test_fixpipe_modes_uint64_words():
