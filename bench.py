@@ -573,7 +573,7 @@ def main():
             others[f"w8a8_nk_m{M}"] = {"gemm_kernel_ms": r["gemm_kernel_ms"], "gemm_gbs": r["gemm_gbs"],
                                        "hbm_frac": r["gemm_gbs"] / PEAK_HBM_GBS,
                                        "note": "weights kept as [n, k] (isTransposeB)" +
-                                               (": one launch, no workspace" if M <= 32 else "")}
+                                               (": one launch, no workspace" if M <= 224 else "")}
             torch.cuda.empty_cache()
         for M in (1, 4):
             r = strip(w8a8_linear(M, s2, w2))
