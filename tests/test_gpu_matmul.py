@@ -237,6 +237,20 @@ def test_w8a8_weights_held_in_registers(m, n, k):
     assert np.array_equal(bits(c), gold)
     c, desc = run_mm(m, n, k, a, bt, out=torch.bfloat16, bias=(bias, None), quant=cs, tok=ts, trans_b=True)
     assert np.array_equal(bits(c), gold)
+    if n > 2064 or k > 4096:
+        return
+    # requantised int8 output from uint64 words (one of them with the pre-shift), int32 bias ahead of the
+    # dequantisation; FasterGelu to half from a scalar scale
+    words = (cs * 50).astype(np.float32).view(np.uint32).astype(np.uint64) | (np.uint64(1) << np.uint64(46))
+    words[n // 2] |= (np.uint64(1) << np.uint64(36)) | (np.uint64(3) << np.uint64(32))
+    bias_i = rng.integers(-1000, 1000, n).astype(np.int32)
+    c8, d8 = run_mm_packed(m, n, k, a, b, out=torch.int8, bias=(bias_i, None), quant=words)
+    gold8 = oracle_mm(d8, a, b, (bias_i, None), words)
+    assert np.array_equal(bits(c8), gold8)
+    c8, _ = run_mm(m, n, k, a, bt, out=torch.int8, bias=(bias_i, None), quant=words, trans_b=True)
+    assert np.array_equal(bits(c8), gold8)
+    cg, dg = run_mm_packed(m, n, k, a, b, out=torch.float16, scalar=1e-3, act=abi.MM_ACT_FASTER_GELU)
+    assert max_ulp(bits(cg), oracle_mm(dg, a, b).view(np.uint16), "f16") <= 1
 
 
 @pytest.mark.parametrize("m", [1, 16, 32])
