@@ -641,6 +641,8 @@ __device__ __forceinline__ void gemm_dma_group_phase(const GemmParams& p, const 
             gemm_dma_tile_at<256, 256, false, true>(p, at, 0u, A0, B0, A1, B1, TS);
         } else if constexpr (phase == 1) {
             gemm_dma_tile_at<256, 128, false, true>(p, at, 0u, A0, B0, A1, B1, TS);
+        } else if (at.row_end - at.row0 <= 64u) {  // uniform: a remainder of at most 64 rows
+            gemm_dma_tile_at<64, 256, false, true>(p, at, 0u, A0, B0, A1, B1, TS);
         } else {
             gemm_dma_tile_at<128, 256, false, true>(p, at, 0u, A0, B0, A1, B1, TS);
         }
@@ -652,7 +654,7 @@ __device__ __forceinline__ void gemm_dma_group_phase(const GemmParams& p, const 
 // list and derives the same plan from it:
 //   phase 0: the big row tiles x the first `wide` 256-wide tile columns, as many as fill whole rounds of the chip;
 //   phase 1: the big row tiles x the remaining columns as 256 x 128 tiles (the last, partial round in half-size pieces);
-//   phase 2: the groups' short remainders (at most 128 rows) as 128 x 256 tiles, cheapest last.
+//   phase 2: the groups' short remainders (at most 128 rows) as 128 x 256 tiles (64 x 256 up to 64 rows), cheapest last.
 // Tile ids run through the phases in this order (each phase padded to a multiple of 8 ids, so that id mod 8 stays the
 // XCD of the workgroup that takes it); workgroup w takes ids w, w + gridDim.x, ...  Inside a phase the tiles are
 // ordered group by group, column by column, the row tiles of a column adjacent, and an XCD takes a contiguous share:
