@@ -281,6 +281,7 @@ class Matmul:
         self.a = self.b = self.bias = self.quant = self.tok = None
         self.packed = False
         self._ws_by_stream = {}   # scratch per stream handle: calls of one object on two streams may overlap
+        self._need = {}           # scratch size per (shape, options)
 
     def set_tensor_a(self, a):
         self.a = a
@@ -349,13 +350,20 @@ class Matmul:
             check(lib.ascq_matmul_w8a8_packed(C.byref(self.desc), _ptr(c), _ptr(self.a), _ptr(self.b), _ptr(self.bias),
                                               _ptr(self.quant), _ptr(self.tok), _stream()))
             return c
-        need = C.c_size_t(0)
-        check(lib.ascq_matmul_w8a8_workspace_size(C.byref(self.desc), C.byref(need)))
-        if need.value:
-            self._scratch(need.value, c.device)
-        check(lib.ascq_matmul_w8a8(C.byref(self.desc), _ptr(c), _ptr(self.a), _ptr(self.b), _ptr(self.bias),
-                                   _ptr(self.quant), _ptr(self.tok), _ptr(self._ws) if need.value else None,
-                                   need.value, _stream()))
+        # the size query is a host call of its own, which a decode step of a dozen microseconds notices: asked once per
+        # shape and option set
+        d = self.desc
+        key = (d.m, d.n, d.k, d.trans_a, d.trans_b, d.out_dtype, d.quant_mode, d.scale_format, d.bias_kind,
+               d.has_tok_scale, d.activation, d.b_format)
+        need = self._need.get(key)
+        if need is None:
+            size = C.c_size_t(0)
+            check(lib.ascq_matmul_w8a8_workspace_size(C.byref(d), C.byref(size)))
+            need = self._need[key] = size.value
+        if need:
+            self._scratch(need, c.device)
+        check(lib.ascq_matmul_w8a8(C.byref(d), _ptr(c), _ptr(self.a), _ptr(self.b), _ptr(self.bias),
+                                   _ptr(self.quant), _ptr(self.tok), _ptr(self._ws) if need else None, need, _stream()))
         return c
 
     def plan(self, c):
