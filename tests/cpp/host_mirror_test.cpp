@@ -355,6 +355,49 @@ void test_matmul()
         orc_matmul_w8a8(&mm.Desc(), want.data(), a.data(), b.data(), nullptr, cs.data(), ts.data());
         expect_equal("Matmul on packed int8 weights", dc.download(), want);
     }
+    std::printf("[case] Matmul<bfloat16_t> 96x160x256 on packed weights (weights held in registers, activations streamed)\n");
+    {
+        DeviceBuffer<uint8_t> dpacked(ascq::PackWeightInt8Size(k, n));
+        ascq::PackWeightInt8(db.view<int8_t>(k * n), dpacked.ptr(), k, n);
+        DeviceBuffer<uint16_t> dc(m * n);
+        ascq::Matmul<ascq::bfloat16_t> mm(m, n, k);
+        mm.SetTensorA(da.view<int8_t>(m * k));
+        mm.SetTensorBPacked(dpacked.ptr());
+        mm.SetQuantVector(dcs.view<float>(n));
+        mm.SetTokenScale(dts.view<float>(m));
+        mm.IterateAll(dc.view<ascq::bfloat16_t>(m * n));
+        std::vector<uint16_t> want(m * n);
+        orc_matmul_w8a8(&mm.Desc(), want.data(), a.data(), b.data(), nullptr, cs.data(), ts.data());
+        expect_equal("Matmul on packed int8 weights, 96 rows", dc.download(), want);
+    }
+    std::printf("[case] ascq_linear_w8a8_dynamic_packed 3x160x256: bfloat16 x quantised per token inside the decode kernel\n");
+    {
+        const uint32_t rows = 3;
+        std::vector<uint16_t> x(rows * k);
+        for (auto& e : x) e = orc_f32_to_bf16(r.uniform(-4.0f, 4.0f));
+        DeviceBuffer<uint16_t> dx(x), dc(rows * n);
+        DeviceBuffer<uint8_t> dpacked(ascq::PackWeightInt8Size(k, n));
+        ascq::PackWeightInt8(db.view<int8_t>(k * n), dpacked.ptr(), k, n);
+        ascq_matmul_desc d{};
+        d.m = rows;
+        d.n = n;
+        d.k = k;
+        d.out_dtype = ASCQ_BF16;
+        d.quant_mode = ASCQ_MM_QUANT_VECTOR;
+        d.scale_format = ASCQ_MM_SCALE_F32;
+        size_t need = 0;
+        ascq::Check(ascq_linear_w8a8_dynamic_workspace_size(&d, &need));
+        DeviceBuffer<uint8_t> dws(need ? need : 16);
+        ascq::Check(ascq_linear_w8a8_dynamic_packed(&d, ASCQ_BF16, dc.ptr(), dx.ptr(), dpacked.ptr(), nullptr, dcs.ptr(),
+                                                    dws.ptr(), need ? need : 16, nullptr));
+        std::vector<int8_t> q(rows * k);
+        std::vector<float> tok(rows);
+        orc_dynamic_quant_per_token(ASCQ_BF16, rows, k, q.data(), tok.data(), x.data());
+        d.has_tok_scale = 1;
+        std::vector<uint16_t> want(rows * n);
+        orc_matmul_w8a8(&d, want.data(), q.data(), b.data(), nullptr, cs.data(), tok.data());
+        expect_equal("one-launch linear on packed weights", dc.download(), want);
+    }
     std::printf("[case] Matmul<int32_t, int4b_t> 96x160x256, int32 bias\n");
     {
         // int4 operands, two per byte with the even element in the low nibble; the oracle sees the same values as int8
