@@ -393,4 +393,44 @@ __device__ __forceinline__ uint32_t pack4_i8(int a, int b, int c, int d)
            ((static_cast<uint32_t>(c) & 0xFFu) << 16) | ((static_cast<uint32_t>(d) & 0xFFu) << 24);
 }
 
+// Maps a linear workgroup id to a tile id such that each XCD (id mod 8) gets a contiguous range of tiles.
+__device__ __forceinline__ uint32_t xcd_remap(uint32_t pid, uint32_t total)
+{
+    const uint32_t per = (total + 7u) / 8u;
+    uint32_t tall = total % 8u;
+    if (tall == 0) {
+        tall = 8;
+    }
+    const uint32_t xcd = pid & 7u, local = pid >> 3;
+    if (xcd < tall) {
+        return local < per ? xcd * per + local : 0xFFFFFFFFu;  // a launch may be larger than `total`
+    }
+    if (local + 1u >= per) {
+        return 0xFFFFFFFFu;  // the short XCDs own one tile less: this workgroup has nothing to do
+    }
+    return tall * per + (xcd - tall) * (per - 1u) + local;
+}
+
+// Tile t of a tiles_m x tiles_n grid in the order the tile kernels run them: bands of 8 row tiles, inside a band column
+// by column with the row tiles of a column adjacent (up to 8 row tiles that is the plain column-by-column order).
+// With xcd_remap an XCD's share is then a block of a few columns by 8 rows, whose rows of A and columns of B the
+// workgroups that run side by side share in that XCD's L2, however many rows the matrix has.
+__device__ __forceinline__ void band_order(uint32_t t, uint32_t tiles_m, uint32_t tiles_n, uint32_t& tm, uint32_t& tn)
+{
+    constexpr uint32_t kBand = 8;
+    const uint32_t per_band = kBand * tiles_n, full = tiles_m / kBand;
+    if (tiles_m <= kBand) {
+        tm = t % tiles_m;
+        tn = t / tiles_m;
+    } else if (t < full * per_band) {
+        const uint32_t r = t % per_band;
+        tm = (t / per_band) * kBand + r % kBand;
+        tn = r / kBand;
+    } else {
+        const uint32_t r = t - full * per_band, rows_last = tiles_m - full * kBand;
+        tm = full * kBand + r % rows_last;
+        tn = r / rows_last;
+    }
+}
+
 }  // namespace ascq

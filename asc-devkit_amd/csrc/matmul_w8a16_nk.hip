@@ -448,8 +448,15 @@ __global__ __launch_bounds__(256, 2) void w8a16_nk_gemm_kernel(NkParams p, uint3
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t wm = wave >> 1, wn = wave & 1u;
-    // row tiles innermost: the workgroups that run side by side share their columns of B
-    const uint32_t tm = blockIdx.x % tiles_m, tn = blockIdx.x / tiles_m;
+    // an XCD (workgroup id mod 8) takes a contiguous share of the tiles, ordered in bands of 8 row tiles: the
+    // workgroups that run side by side in it share their rows of x and their columns of B in its L2
+    const uint32_t tiles_n = (p.n + kGN - 1u) / kGN;
+    const uint32_t t = xcd_remap(blockIdx.x, tiles_m * tiles_n);
+    if (t == 0xFFFFFFFFu) {
+        return;  // whole workgroup (the launch is rounded up to a multiple of 8)
+    }
+    uint32_t tm, tn;
+    band_order(t, tiles_m, tiles_n, tm, tn);
     const uint32_t row0 = tm * kGM, col0 = tn * kGN;
 
     // ---- staging roles
@@ -737,9 +744,9 @@ int launch_w8a16_nk(const void* x, const void* w, const void* scale, const void*
         p.y = y;
         const uint32_t tiles_m = (m + kGM - 1u) / kGM, tiles_n = (n + kGN - 1u) / kGN;
         if (has_offset) {
-            w8a16_nk_gemm_kernel<true><<<tiles_m * tiles_n, 256, 0, st>>>(p, tiles_m);
+            w8a16_nk_gemm_kernel<true><<<(tiles_m * tiles_n + 7u) / 8u * 8u, 256, 0, st>>>(p, tiles_m);
         } else {
-            w8a16_nk_gemm_kernel<false><<<tiles_m * tiles_n, 256, 0, st>>>(p, tiles_m);
+            w8a16_nk_gemm_kernel<false><<<(tiles_m * tiles_n + 7u) / 8u * 8u, 256, 0, st>>>(p, tiles_m);
         }
         return launch_status("ascq_matmul_w8a16");
     }

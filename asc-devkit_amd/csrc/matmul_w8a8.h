@@ -197,23 +197,6 @@ __device__ __forceinline__ float load_bias_post(const EpiParams& e, size_t col)
 }
 
 
-// Maps a linear workgroup id to a tile id such that each XCD (id mod 8) gets a contiguous range of tiles.
-__device__ __forceinline__ uint32_t xcd_remap(uint32_t pid, uint32_t total)
-{
-    const uint32_t per = (total + 7u) / 8u;
-    uint32_t tall = total % 8u;
-    if (tall == 0) {
-        tall = 8;
-    }
-    const uint32_t xcd = pid & 7u, local = pid >> 3;
-    if (xcd < tall) {
-        return local < per ? xcd * per + local : 0xFFFFFFFFu;  // a launch may be larger than `total`
-    }
-    if (local + 1u >= per) {
-        return 0xFFFFFFFFu;  // the short XCDs own one tile less: this workgroup has nothing to do
-    }
-    return tall * per + (xcd - tall) * (per - 1u) + local;
-}
 
 // Large-M kernel built on direct-to-LDS loads and transposing LDS reads (matmul_w8a8_dma.hip).
 bool gemm_dma_supported(const GemmParams& p);

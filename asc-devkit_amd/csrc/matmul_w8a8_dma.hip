@@ -535,24 +535,10 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_
     if (t >= total) {
         return;
     }
-    // Tiles run in bands of 8 row tiles, inside a band column by column with the row tiles of a column adjacent (up to
-    // 8 row tiles that is the plain column-by-column order): an XCD's share stays a block of a few columns by 8 rows
-    // whose rows of A and columns of B it reuses from its L2, however many rows the matrix has.
-    constexpr uint32_t kBand = 8;
-    const uint32_t per_band = kBand * p.tiles_n, full = p.tiles_m / kBand;
+    // bands of 8 row tiles, inside a band column by column (band_order): an XCD's share stays a block of a few columns
+    // by 8 rows whose rows of A and columns of B it reuses from its L2, however many rows the matrix has
     uint32_t ms, tn;
-    if (p.tiles_m <= kBand) {
-        ms = t % p.tiles_m;
-        tn = t / p.tiles_m;
-    } else if (t < full * per_band) {
-        const uint32_t r = t % per_band;
-        ms = (t / per_band) * kBand + r % kBand;
-        tn = r / kBand;
-    } else {
-        const uint32_t r = t - full * per_band, rows_last = p.tiles_m - full * kBand;
-        ms = full * kBand + r % rows_last;
-        tn = r / rows_last;
-    }
+    band_order(t, p.tiles_m, p.tiles_n, ms, tn);
     const TilePlace at{ms * BM, p.m, col_begin + tn * BN, p.b, 0};
     gemm_dma_tile_at<BM, BN, kSplitK, false, kBT>(p, at, bidy, A0, B0, A1, B1, TS);
 }
