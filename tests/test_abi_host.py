@@ -411,6 +411,32 @@ def test_quant_word_with_pre_shift_bit_passes_validation():
     assert rc == abi.ENULL and "bit 36" not in err()
 
 
+def test_linear_dynamic_packed_argument_checks():
+    """ascq_linear_w8a8_dynamic_packed refuses what the packed layout cannot serve before anything is launched, and its
+    scratch need is covered by ascq_linear_w8a8_dynamic_workspace_size."""
+    def d(**kw):
+        x = abi.MatmulDesc(m=4, n=64, k=128, out_dtype=abi.BF16, quant_mode=abi.MM_QUANT_VECTOR, scale_format=abi.MM_SCALE_F32)
+        for key, v in kw.items():
+            setattr(x, key, v)
+        return x
+    big = C.c_void_p(0x200000)
+    call = lambda x, dt=abi.BF16, ws=big, nbytes=1 << 20: L.ascq_linear_w8a8_dynamic_packed(
+        C.byref(x), dt, FAKE, FAKE, FAKE, None, FAKE, ws, nbytes, None)
+    assert L.ascq_linear_w8a8_dynamic_packed(None, abi.BF16, FAKE, FAKE, FAKE, None, FAKE, big, 1 << 20, None) == abi.ENULL
+    assert call(d(), dt=abi.I8) == abi.EUNSUPPORTED and "x dtype" in err()
+    assert call(d(k=100)) == abi.EUNSUPPORTED and "multiple of 64" in err()
+    assert call(d(trans_a=1)) == abi.EUNSUPPORTED
+    assert call(d(activation=abi.MM_ACT_SWIGLU)) == abi.EUNSUPPORTED and "SwiGLU" in err()
+    assert call(d(quant_mode=abi.MM_QUANT_NONE)) == abi.EUNSUPPORTED
+    assert call(d(out_dtype=abi.I8)) == abi.EUNSUPPORTED
+    assert call(d(), ws=None) == abi.ENULL
+    assert call(d(), ws=C.c_void_p(0x200004)) == abi.EALIGN
+    assert call(d(), nbytes=256) == abi.EINVAL and "workspace" in err()
+    need = C.c_size_t(0)
+    assert L.ascq_linear_w8a8_dynamic_workspace_size(C.byref(d()), C.byref(need)) == abi.OK
+    assert need.value >= 4 * 128 + 4 * 4
+
+
 def test_tmp_buffer_factor_sizes_known_answers():
     """tests/api/adv_api/tiling/test_tiling.cpp:6549-6553, 6565-6569, 6583-6608, 6621-6625, 6643-6647, 6662-6666,
     6684-6688 of the reference."""
