@@ -490,7 +490,7 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_ws_kernel(PackedParams p)
     for (int u = 0; u < kWsDma; ++u) {
         const uint32_t sidx = static_cast<uint32_t>(u) * 64u + lane;
         const uint32_t r = sidx >> 5, q = (sidx & 31u) ^ r;
-        a_col[u] = (q < cnt * 4u ? q : 0u) * 16u + ta * kPkTileK;
+        a_col[u] = (q < cnt * 4u ? q : 0u) * 16u + (cnt != 0u ? ta : 0u) * kPkTileK;  // (no tiles: any valid piece)
         a_off[u] = r * p.k + a_col[u];
         a_off_last[u] = a_off[u];
     }
