@@ -185,6 +185,23 @@ __device__ __forceinline__ void dispatch_out(const EpiParams& e, F&& f)
     }
 }
 
+// The whole epilogue of one output element for kernels that hold one element per lane with the columns of a row in
+// neighbouring lanes (columns col and col ^ 1 in lanes l and l ^ 1, both active or both not): with SwiGLU the pair
+// exchanges its de-quantised values through the neighbouring lane and the even column stores output column col / 2.
+__device__ __forceinline__ void epilogue_store_lanes(const EpiParams& e, size_t row, uint32_t col, int32_t acc,
+                                                     const ChannelQ& q, float tok, float bias_post)
+{
+    if (e.activation == ASCQ_MM_ACT_SWIGLU) {  // uniform
+        const float v = epilogue_value(e, acc, q, tok, bias_post);
+        const float w = __shfl_xor(v, 1, 64);
+        if ((col & 1u) == 0u) {
+            store_float_out(e, row * e.ldc + (col >> 1), swiglu(v, w, e.act_beta));
+        }
+        return;
+    }
+    dispatch_out(e, [&](auto tag) { epilogue_store<decltype(tag)::value>(e, row, col, acc, q, tok, bias_post); });
+}
+
 __device__ __forceinline__ float load_bias_post(const EpiParams& e, size_t col)
 {
     if (e.bias_kind == ASCQ_MM_BIAS_F32_POST) {

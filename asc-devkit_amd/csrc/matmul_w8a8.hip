@@ -604,6 +604,16 @@ bool swiglu_in_tile_kernel(const ascq_matmul_desc* d, const GemmParams& p, const
     return d->b_format == ASCQ_MM_B_NZ || fast_path_ok(d, a, b);
 }
 
+// True when the plain matmul of this descriptor runs on the decode kernels for [n, k] weights (activations resident
+// in LDS, or weights held in registers), whose epilogue pairs the columns of a row through neighbouring lanes.
+bool swiglu_in_decode_kernel(const ascq_matmul_desc* d, const GemmParams& p, const void* a, const void* b)
+{
+    if (!d->trans_b || d->trans_a || d->b_format != ASCQ_MM_B_ND || !fast_path_ok(d, a, b)) {
+        return false;
+    }
+    return (d->m <= 16 && gemm_packed_nk_supported(p)) || gemm_ws_supported(p, true);
+}
+
 inline size_t round256(size_t v) { return (v + 255u) & ~static_cast<size_t>(255u); }
 
 // the matmul that leaves raw accumulators: same operands, no quantisation, at most the pre-dequant bias
@@ -635,7 +645,7 @@ extern "C" int ascq_matmul_w8a8_workspace_size(const ascq_matmul_desc* d, size_t
     shape.n = d->n;
     shape.k = d->k;
     if (d->activation == ASCQ_MM_ACT_SWIGLU && d->quant_mode != ASCQ_MM_QUANT_NONE &&
-        !swiglu_in_tile_kernel(d, shape, shape.a, shape.b)) {
+        !swiglu_in_tile_kernel(d, shape, shape.a, shape.b) && !swiglu_in_decode_kernel(d, shape, shape.a, shape.b)) {
         // Shapes outside the large tile kernel keep their int32 accumulators [m][n] in the workspace, behind the
         // scratch of the matmul that produces them.
         const ascq_matmul_desc r = raw_accumulator_desc(d);
@@ -690,7 +700,7 @@ extern "C" int ascq_matmul_w8a8(const ascq_matmul_desc* d, void* c, const void* 
     p.n = d->n;
     p.k = d->k;
     p.epi = make_epi(d, c, bias, quant_vector, tok_scale);
-    if (d->activation == ASCQ_MM_ACT_SWIGLU && !swiglu_in_tile_kernel(d, p, a, b)) {
+    if (d->activation == ASCQ_MM_ACT_SWIGLU && !swiglu_in_tile_kernel(d, p, a, b) && !swiglu_in_decode_kernel(d, p, a, b)) {
         // raw accumulators into the workspace, then the pairwise epilogue
         const ascq_matmul_desc r = raw_accumulator_desc(d);
         size_t inner = 0;
@@ -812,8 +822,6 @@ extern "C" int ascq_matmul_w8a8_packed(const ascq_matmul_desc* d, void* c, const
     }
     ASCQ_REQUIRE(!d->trans_a && d->b_format == ASCQ_MM_B_ND, ASCQ_EUNSUPPORTED,
                  "ascq_matmul_w8a8_packed: a is [m, k] and the weights are in the packed layout (no trans_a, no NZ)");
-    ASCQ_REQUIRE(d->activation != ASCQ_MM_ACT_SWIGLU, ASCQ_EUNSUPPORTED,
-                 "ascq_matmul_w8a8_packed: SwiGLU is not available on packed weights (use ascq_matmul_w8a8)");
     GemmParams p{};
     p.a = static_cast<const int8_t*>(a);
     p.b = static_cast<const int8_t*>(w_packed);
@@ -896,8 +904,8 @@ extern "C" int ascq_linear_w8a8_dynamic(const ascq_matmul_desc* d, int32_t x_dty
     if (rc != ASCQ_OK) {
         return rc;
     }
-    if ((x_dtype == ASCQ_F16 || x_dtype == ASCQ_BF16) && d->trans_b && d->b_format == ASCQ_MM_B_ND &&
-        d->activation != ASCQ_MM_ACT_SWIGLU && aligned16(x) && gemm_packed_dyn_fits(d->m, d->k)) {
+    if ((x_dtype == ASCQ_F16 || x_dtype == ASCQ_BF16) && d->trans_b && d->b_format == ASCQ_MM_B_ND && aligned16(x) &&
+        gemm_packed_dyn_fits(d->m, d->k)) {
         // decode on [n, k] weights: the quantisation happens inside the weight-streaming kernel (same bits, one launch)
         GemmParams p{};
         p.a = static_cast<const int8_t*>(x);  // only its alignment is looked at
@@ -934,9 +942,8 @@ extern "C" int ascq_linear_w8a8_dynamic_packed(const ascq_matmul_desc* d, int32_
                  "ascq_linear_w8a8_dynamic_packed: x dtype %d is not half / bfloat16 / float", x_dtype);
     ASCQ_REQUIRE(d->quant_mode != ASCQ_MM_QUANT_NONE && d->out_dtype != ASCQ_I8, ASCQ_EUNSUPPORTED,
                  "ascq_linear_w8a8_dynamic_packed: the token scales need a floating-point dequantising epilogue");
-    ASCQ_REQUIRE(!d->trans_a && d->b_format == ASCQ_MM_B_ND && d->activation != ASCQ_MM_ACT_SWIGLU, ASCQ_EUNSUPPORTED,
-                 "ascq_linear_w8a8_dynamic_packed: x is [m, k], the weights are in the packed layout, SwiGLU is not "
-                 "available on packed weights");
+    ASCQ_REQUIRE(!d->trans_a && d->b_format == ASCQ_MM_B_ND, ASCQ_EUNSUPPORTED,
+                 "ascq_linear_w8a8_dynamic_packed: x is [m, k] and the weights are in the packed layout (no trans_a, no NZ)");
     ASCQ_REQUIRE(d->k % 64u == 0, ASCQ_EUNSUPPORTED, "ascq_linear_w8a8_dynamic_packed: k = %u must be a multiple of 64", d->k);
     ascq_matmul_desc dd = *d;
     dd.has_tok_scale = 1;

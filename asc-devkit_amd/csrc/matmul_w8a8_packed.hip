@@ -191,7 +191,7 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_kernel(PackedParams
             sum += bias_pre;
             const uint32_t row = p.m0 + row_in_pass;
             const float tok = e.has_tok ? e.tok_scale[row] : 1.0f;
-            dispatch_out(e, [&](auto tag) { epilogue_store<decltype(tag)::value>(e, row, col, sum, q, tok, bp); });
+            epilogue_store_lanes(e, row, col, sum, q, tok, bp);
         }
     }
 }
@@ -410,10 +410,7 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_dyn_kernel(PackedPa
             const uint32_t row_in_pass = 4u * half + lq;
             if (row_in_pass < p.rows) {
                 const int32_t sum = OUT[s][row_in_pass][lc] + bias_pre;
-                const float tok = TOK[row_in_pass];
-                dispatch_out(e, [&](auto tag) {
-                    epilogue_store<decltype(tag)::value>(e, p.m0 + row_in_pass, col, sum, q, tok, bp);
-                });
+                epilogue_store_lanes(e, p.m0 + row_in_pass, col, sum, q, TOK[row_in_pass], bp);
             }
         }
     }
@@ -602,11 +599,17 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_ws_kernel(PackedParams p)
             const ChannelQ q = load_channel_q(e, col);
             const float bp = load_bias_post(e, col);
             const int32_t bias_pre = e.bias_kind == ASCQ_MM_BIAS_I32_PRE ? static_cast<const int32_t*>(e.bias)[col] : 0;
-            dispatch_out(e, [&](auto tag) {
+            if (e.activation == ASCQ_MM_ACT_SWIGLU) {  // uniform: column pairs through neighbouring lanes
                 for (uint32_t row = wave; row < brows; row += kPkWaves) {
-                    epilogue_store<decltype(tag)::value>(e, p.m0 + b0 + row, col, OUT[row][c] + bias_pre, q, TS[row], bp);
+                    epilogue_store_lanes(e, p.m0 + b0 + row, col, OUT[row][c] + bias_pre, q, TS[row], bp);
                 }
-            });
+            } else {
+                dispatch_out(e, [&](auto tag) {
+                    for (uint32_t row = wave; row < brows; row += kPkWaves) {
+                        epilogue_store<decltype(tag)::value>(e, p.m0 + b0 + row, col, OUT[row][c] + bias_pre, q, TS[row], bp);
+                    }
+                });
+            }
         }
         if (b0 + kWsRows < p.rows) {
             __syncthreads();  // the next block clears what this epilogue read

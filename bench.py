@@ -64,7 +64,7 @@ def main():
     ap.add_argument("--quick", action="store_true", help="headline + W4A16 GEMV only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="run a single workload: w8a8 | w4a16 | w4a16_per_weight | w4a16_per_weight_m4 | w4a16_per_weight_m16 | w4a16_nd | w4a16_m4 | w4a16_m16 | w4a16_nd_m4 | w4a16_nd_m16 | "
-                         "w8a8_zeros | w8a8_m1 | w8a8_m8 | w8a8_m16 | w8a8_m128 | w8a8_m512 | w8a8_m8192 | w8a8_packed_m1 | w8a8_packed_m8 | w8a8_packed_m16 | w8a8_packed_m32 | w8a8_packed_m64 | w8a8_packed_m128 | w8a8_nk_m32 | w8a8_nk_m64 | w8a8_m32 | w8a8_nk_m1 | w8a8_nk_m16 | w8a8_nk_m128 | w8a8_linear_nk_m1 | w8a8_linear_nk_m4 | w8a8_linear_nk_m16 | w8a8_linear_packed_m1 | w8a8_linear_packed_m4 | w8a16_m1 | w8a16_m16 | w8a16_nk_m1 | w8a16_nk_m4 | w8a16_nk_sum_m1 | w8a16_nk_sum_m4 | "
+                         "w8a8_zeros | w8a8_m1 | w8a8_m8 | w8a8_m16 | w8a8_m128 | w8a8_m512 | w8a8_m8192 | w8a8_packed_m1 | w8a8_packed_m8 | w8a8_packed_m16 | w8a8_packed_m32 | w8a8_packed_m64 | w8a8_packed_m128 | w8a8_nk_m32 | w8a8_nk_m64 | w8a8_m32 | w8a8_nk_m1 | w8a8_nk_m16 | w8a8_nk_m128 | w8a8_linear_nk_m1 | w8a8_linear_nk_m4 | w8a8_linear_nk_m16 | w8a8_linear_packed_m1 | w8a8_linear_packed_m4 | w8a8_linear_packed_swiglu_m1 | w8a8_linear_nk_swiglu_m1 | w8a16_m1 | w8a16_m16 | w8a16_nk_m1 | w8a16_nk_m4 | w8a16_nk_sum_m1 | w8a16_nk_sum_m4 | "
                          "w8a16_nk_m16 | w8a16_m2048 | w8a16_nk_m2048 | quant | dequant | antiquant | group | group_example | mx_fp4 | mx_fp4_e1m2 | mx_fp8 (a W4A16 name without _nd "
                          "is the packed-weight path, in the group-sum form unless it says per_weight; _nk: weights kept as [n, k])")
     ap.add_argument("--copy-probe", action="store_true",
@@ -223,7 +223,7 @@ def main():
                 "gemm_tops": flops / (kern_ms * 1e-3) / 1e12, "gemm_gbs": bytes_ / (kern_ms * 1e-3) / 1e9,
                 "ops": flops, "bytes": bytes_, "tensors": (x, w, cs)}
 
-    def w8a8_linear(M, steps, warmup, sets=7, packed=False):
+    def w8a8_linear(M, steps, warmup, sets=7, packed=False, swiglu=False):
         """The whole W8A8 linear as one call on weights kept as [n, k] (ascq_linear_w8a8_dynamic) or packed once
         (ascq_linear_w8a8_dynamic_packed): up to 8 rows the per-token quantisation happens inside the weight-streaming
         kernel, one launch per step."""
@@ -231,11 +231,12 @@ def main():
         x = torch.randn((M, K), device=dev, generator=gen).to(torch.bfloat16)
         ws = [rand_i8(N, K) for _ in range(sets)]
         cs = torch.rand(N, device=dev, generator=gen) * (1e-2 - 1e-4) + 1e-4
-        c = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+        act = abi.MM_ACT_SWIGLU if swiglu else abi.MM_ACT_NONE   # SwiGLU: column pairs -> [M, N / 2]
+        c = torch.empty((M, N // 2 if swiglu else N), dtype=torch.bfloat16, device=dev)
         if packed:
-            lins = [ops.DynamicLinear(M, K, ops.pack_weight_w8(w, K, N, True), cs, packed_n=N) for w in ws]
+            lins = [ops.DynamicLinear(M, K, ops.pack_weight_w8(w, K, N, True), cs, packed_n=N, activation=act) for w in ws]
         else:
-            lins = [ops.DynamicLinear(M, K, w, cs, trans_b=True) for w in ws]
+            lins = [ops.DynamicLinear(M, K, w, cs, trans_b=True, activation=act) for w in ws]
         ms, kern_ms = timed(lambda i, a, b: lins[i % sets](c, x), steps, warmup)
         bytes_ = 2 * M * K + K * N + 4 * N + 2 * M * N
         return {"ms_per_step": ms, "kernel_ms": kern_ms, "gbs": bytes_ / (kern_ms * 1e-3) / 1e9, "bytes": bytes_,
@@ -444,6 +445,8 @@ def main():
               "w8a8_linear_nk_m16": lambda: w8a8_linear(16, args.steps, args.warmup),
               "w8a8_linear_packed_m1": lambda: w8a8_linear(1, args.steps, args.warmup, packed=True),
               "w8a8_linear_packed_m4": lambda: w8a8_linear(4, args.steps, args.warmup, packed=True),
+              "w8a8_linear_packed_swiglu_m1": lambda: w8a8_linear(1, args.steps, args.warmup, packed=True, swiglu=True),
+              "w8a8_linear_nk_swiglu_m1": lambda: w8a8_linear(1, args.steps, args.warmup, swiglu=True),
               "w8a8_nk_m1": lambda: w8a8(1, args.steps, args.warmup, sets=7, b_nk=True),
               "w8a8_nk_m16": lambda: w8a8(16, args.steps, args.warmup, sets=7, b_nk=True),
               "w8a16_nk_m1": lambda: w8a16(1, args.steps, args.warmup, b_nk=True),

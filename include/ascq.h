@@ -373,8 +373,8 @@ int ascq_matmul_w8a8_workspace_size(const ascq_matmul_desc* desc, size_t* bytes)
  * into ascq_pack_weight_w8_size(k, n) bytes: slabs of 16 columns, each one contiguous run of tiles of 64 k (1 KiB: lane l
  * of a wavefront owns column l % 16 and the 16 consecutive bytes k 16 (l / 16) .. + 15); columns past n and k past the
  * end hold 0, and 16 tiles of zeros follow the last slab.
- * ascq_matmul_w8a8_packed computes exactly what ascq_matmul_w8a8 computes (same descriptor, epilogues and outputs;
- * desc.trans_b is ignored, desc.trans_a and ASCQ_MM_ACT_SWIGLU are not supported) in one launch with no workspace: a
+ * ascq_matmul_w8a8_packed computes exactly what ascq_matmul_w8a8 computes (same descriptor, epilogues - SwiGLU
+ * included - and outputs; desc.trans_b is ignored, desc.trans_a is not supported) in one launch with no workspace: a
  * workgroup owns whole columns, its wavefronts split k, and integer partial sums are exact in any order.  Up to 16
  * rows the activations stay in LDS and the weights stream past them once.  More rows with k up to 4096 turn the roles
  * round: a workgroup first fetches the weights of its columns into registers and then streams the activations past
@@ -460,7 +460,7 @@ int ascq_linear_w8a8_dynamic_workspace_size(const ascq_matmul_desc* desc, size_t
 
 /*
  * The same linear on weights packed once by ascq_pack_weight_w8 (see ascq_matmul_w8a8_packed for the layout and what
- * the descriptor may ask for: no trans_a, no NZ, no SwiGLU, k % 64 == 0; desc->trans_b is ignored).  Results are those
+ * the descriptor may ask for: no trans_a, no NZ, k % 64 == 0; desc->trans_b is ignored).  Results are those
  * of ascq_linear_w8a8_dynamic on the unpacked weights, bit for bit.  Up to 8 rows of half or bfloat16 x are one launch
  * (the packed decode kernel quantises x itself); otherwise the quantiser kernel runs first and
  * ascq_matmul_w8a8_packed after it, with q and the token scales in the workspace.  The workspace holds

@@ -426,7 +426,7 @@ def test_linear_dynamic_packed_argument_checks():
     assert call(d(), dt=abi.I8) == abi.EUNSUPPORTED and "x dtype" in err()
     assert call(d(k=100)) == abi.EUNSUPPORTED and "multiple of 64" in err()
     assert call(d(trans_a=1)) == abi.EUNSUPPORTED
-    assert call(d(activation=abi.MM_ACT_SWIGLU)) == abi.EUNSUPPORTED and "SwiGLU" in err()
+    assert call(d(activation=abi.MM_ACT_SWIGLU, n=63)) == abi.EINVAL and "must be even" in err()   # SwiGLU pairs columns
     assert call(d(quant_mode=abi.MM_QUANT_NONE)) == abi.EUNSUPPORTED
     assert call(d(out_dtype=abi.I8)) == abi.EUNSUPPORTED
     assert call(d(), ws=None) == abi.ENULL

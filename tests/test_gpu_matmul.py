@@ -1156,6 +1156,75 @@ def test_group_matmul_swiglu_and_dynamic_linear():
         swiglu_close(bits(c), orc.matmul_w8a8(d, q, wl, None, cs, tsn).view(np.uint16), "bf16")
 
 
+@pytest.mark.parametrize("m", [1, 5, 16, 17, 64, 130, 300])
+@pytest.mark.parametrize("n,k", [(22, 128), (1040, 2048), (528, 384), (96, 4096)])
+@pytest.mark.parametrize("out,bias", [(torch.bfloat16, None), (torch.float16, "f32"), (torch.float32, "bf16")])
+def test_matmul_swiglu_in_the_decode_kernels(m, n, k, out, bias):
+    """SwiGLU on [n, k] and on packed weights: the decode kernels (activations resident in LDS up to 16 rows, weights
+    held in registers beyond) pair the columns of a row through neighbouring lanes in their own epilogue - one launch,
+    no raw accumulators; [n, k] weights past 224 rows take the tile kernels.  Against the oracle."""
+    announce("swiglu decode", m, n, k, out, bias)
+    rng = np.random.default_rng(m * 5 + n + k)
+    a, b = rand_i8(rng, (m, k)), rand_i8(rng, (k, n))
+    cs = rng.uniform(1e-4, 4e-4, n).astype(np.float32)
+    ts = rng.uniform(0.5, 2.0, m).astype(np.float32)
+    bv = None
+    if bias == "f32":
+        bv = (rng.standard_normal(n).astype(np.float32), None)
+    elif bias == "bf16":
+        bv = (orc.f32_to_bf16_bits(rng.standard_normal(n).astype(np.float32)), "bf16")
+    beta = 1.0 if m % 2 else 1.702
+    want = None
+    for packed in (False, True):
+        mm = ops.Matmul(m, n, k, False, not packed)
+        mm.set_tensor_a(to_dev(a))
+        if packed:
+            mm.set_tensor_b_packed(ops.pack_weight_w8(to_dev(b), k, n))
+        else:
+            mm.set_tensor_b(to_dev(np.ascontiguousarray(b.T)))
+        mm.set_quant_vector(to_dev(cs))
+        mm.set_token_scale(to_dev(ts))
+        if bv is not None:
+            mm.set_bias(to_dev(bv[0], bv[1]))
+        mm.set_activation(abi.MM_ACT_SWIGLU, beta)
+        c = torch.zeros((m, n // 2), dtype=out, device=DEV)
+        mm.iterate_all(c)
+        if want is None:
+            d = abi.MatmulDesc(m=m, n=n, k=k, out_dtype=mm.desc.out_dtype, quant_mode=abi.MM_QUANT_VECTOR,
+                               scale_format=abi.MM_SCALE_F32, has_tok_scale=1, bias_kind=mm.desc.bias_kind,
+                               activation=abi.MM_ACT_SWIGLU, act_beta=beta)
+            want = oracle_mm(d, a, b, bv, cs, ts)
+        if out == torch.float32:
+            assert np.all(np.abs(c.cpu().numpy() - want) <= 4 * np.spacing(np.abs(want)) + 1e-30)
+        else:
+            swiglu_close(bits(c), want.view(np.uint16), "bf16" if out == torch.bfloat16 else "f16")
+
+
+@pytest.mark.parametrize("m", [1, 3, 8, 12, 40])
+def test_linear_dynamic_swiglu_in_one_launch(m):
+    """The gate / up projection of a decode step in one call: per-token quantisation, int8 matmul on [n, k] or packed
+    weights, SwiGLU of the column pairs (up to 8 rows inside one kernel).  Against the oracle of the steps."""
+    announce("linear dynamic swiglu", m)
+    rng = np.random.default_rng(0x5E + m)
+    k, n = 512, 736
+    xa = orc.f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32))
+    w = rand_i8(rng, (k, n))
+    cs = rng.uniform(1e-4, 4e-4, n).astype(np.float32)
+    q, tsn = orc.dynamic_quant_per_token(abi.BF16, xa)
+    d = abi.MatmulDesc(m=m, n=n, k=k, out_dtype=abi.BF16, quant_mode=abi.MM_QUANT_VECTOR, scale_format=abi.MM_SCALE_F32,
+                       has_tok_scale=1, activation=abi.MM_ACT_SWIGLU, act_beta=1.0)
+    want = orc.matmul_w8a8(d, q, w, None, cs, tsn).view(np.uint16)
+    c = torch.zeros((m, n // 2), dtype=torch.bfloat16, device=DEV)
+    ops.linear_w8a8_dynamic(c, to_dev(xa, "bf16"), to_dev(np.ascontiguousarray(w.T)), to_dev(cs), trans_b=True,
+                            activation=abi.MM_ACT_SWIGLU)
+    swiglu_close(bits(c), want, "bf16")
+    c2 = torch.zeros((m, n // 2), dtype=torch.bfloat16, device=DEV)
+    ops.linear_w8a8_dynamic_packed(c2, to_dev(xa, "bf16"), ops.pack_weight_w8(to_dev(w), k, n), n, to_dev(cs),
+                                   activation=abi.MM_ACT_SWIGLU)
+    swiglu_close(bits(c2), want, "bf16")
+    assert torch.equal(c, c2)
+
+
 # ------------------------------------------------------------------ workspace contract, determinism
 @pytest.mark.parametrize("m", [1, 5, 16, 19, 130])
 def test_workspaces_need_no_initialisation_and_results_repeat(m):
