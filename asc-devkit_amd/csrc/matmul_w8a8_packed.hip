@@ -33,7 +33,7 @@ constexpr uint32_t kPkPadTiles = 16;   // tiles of zeros behind the last slab (a
 constexpr uint32_t kPkWaves = 8, kPkBatch = 4, kPkMaxSlabs = 8, kPkMaxRows = 16;
 constexpr int kPkBuf = 2;              // register buffers: one batch in flight while the other is computed
 constexpr uint32_t kPkRowPad = 16;     // bytes added to a staged activation row: rows start 4 banks apart
-constexpr uint32_t kPkXBytes = 88 * 1024;  // LDS for the staged activations of a workgroup (the partial sums take 64 KiB)
+constexpr uint32_t kPkPool = 152 * 1024;  // LDS of a workgroup: the staged activations, then 8 KiB of partial sums per slab
 constexpr uint32_t kPkPastEnd = 0x7FFFFFF0u;
 constexpr int kPkNt = 2;               // cache policy of the weight loads: non-temporal (read once per call)
 
@@ -48,6 +48,8 @@ struct PackedParams {
     uint32_t slabs, ktiles;
     uint32_t tpw;          // tiles of k per wavefront
     uint32_t rows_magic;   // ceil(2^32 / rows)
+    uint32_t red_off;      // gemm_packed_kernel: bytes of LDS in front of the partial sums
+    uint32_t red_slabs;    // ... and the slabs a workgroup holds at most
     EpiParams epi;
 };
 
@@ -60,8 +62,11 @@ __device__ __forceinline__ uint32_t pk_xcd_order(uint32_t wg, uint32_t wgs)
 template <bool kNK>
 __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_kernel(PackedParams p)
 {
-    __shared__ __attribute__((aligned(16))) char XS[kPkXBytes];
-    __shared__ int32_t RED[kPkWaves][kPkMaxSlabs][4][64];
+    // the staged activations (rows x 8 wavefronts x pitch bytes), then the partial sums [wavefront][slab][4][64]
+    __shared__ __attribute__((aligned(16))) char POOL[kPkPool];
+    char* const XS = POOL;
+    int32_t* const red = reinterpret_cast<int32_t*>(POOL + p.red_off);
+    const uint32_t red_wave = p.red_slabs * 256u;  // words from a wavefront's sums to the next one's
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t lc = lane & 15u, lq = lane >> 4;
@@ -148,7 +153,7 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_kernel(PackedParams
         ++c_q;
         if (++c_b == nb) {  // the slab is done: register i of lane l is row 4 (l / 16) + i, column l % 16
 #pragma unroll
-            for (int i = 0; i < 4; ++i) RED[wave][c_slab][i][lane] = acc[i];
+            for (int i = 0; i < 4; ++i) red[wave * red_wave + c_slab * 256u + i * 64u + lane] = acc[i];
             acc = i32x4{0, 0, 0, 0};
             c_b = 0;
             ++c_slab;
@@ -164,7 +169,7 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_kernel(PackedParams
     if (batches == 0u) {  // a wavefront without tiles (k shorter than 8 tiles) contributes zeros
         for (uint32_t s = 0; s < nslabs; ++s) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) RED[wave][s][i][lane] = 0;
+            for (int i = 0; i < 4; ++i) red[wave * red_wave + s * 256u + i * 64u + lane] = 0;
         }
     }
     __syncthreads();
@@ -185,9 +190,10 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_kernel(PackedParams
             if (row_in_pass >= p.rows) {
                 continue;
             }
-            int32_t sum = RED[0][s][i][lane];
+            const int32_t* part = red + s * 256u + static_cast<uint32_t>(i) * 64u + lane;
+            int32_t sum = part[0];
 #pragma unroll
-            for (uint32_t wv = 1; wv < kPkWaves; ++wv) sum += RED[wv][s][i][lane];
+            for (uint32_t wv = 1; wv < kPkWaves; ++wv) sum += part[wv * red_wave];
             sum += bias_pre;
             const uint32_t row = p.m0 + row_in_pass;
             const float tok = e.has_tok ? e.tok_scale[row] : 1.0f;
@@ -688,10 +694,14 @@ int launch_gemm_packed(const GemmParams& p, hipStream_t st, bool b_nk)
     if ((q.slabs + grid - 1u) / grid > kPkMaxSlabs) {
         grid = (q.slabs + kPkMaxSlabs - 1u) / kPkMaxSlabs;
     }
-    // rows per pass: 16, fewer when k is so long that the staged activations of 16 rows would not fit the LDS
+    // rows per pass: 16, fewer when k is so long that the staged activations of 16 rows would not fit the LDS beside
+    // the partial sums (8 KiB per slab of a workgroup)
+    q.red_slabs = (q.slabs + grid - 1u) / grid;
+    const uint32_t red_bytes = q.red_slabs * kPkWaves * 1024u;
     const uint32_t row_bytes = kPkWaves * (q.tpw * kPkTileK + kPkRowPad);
-    uint32_t pass_rows = kPkXBytes / row_bytes;
+    uint32_t pass_rows = (kPkPool - red_bytes) / row_bytes;
     pass_rows = pass_rows > kPkMaxRows ? kPkMaxRows : pass_rows;
+    q.red_off = pass_rows * row_bytes;
     if (pass_rows == 0u) {
         return fail(ASCQ_EUNSUPPORTED, "ascq_matmul_w8a8_packed: k = %u is too long for the staged activations", p.k);
     }
@@ -701,7 +711,7 @@ int launch_gemm_packed(const GemmParams& p, hipStream_t st, bool b_nk)
         q.rows = left < pass_rows ? left : pass_rows;
         q.rows_magic = static_cast<uint32_t>(((1ull << 32) + q.rows - 1u) / q.rows);
         if (plan_note(ASCQ_MM_KERNEL_STREAM, 16, 16 * ((q.slabs + grid - 1u) / grid), kPkTileK, grid, 1,
-                      kPkXBytes + kPkWaves * kPkMaxSlabs * 1024u, 0)) {
+                      kPkPool, 0)) {
             return ASCQ_OK;
         }
         if (b_nk) {
