@@ -232,8 +232,10 @@ int launch_gemm_nk(const GemmParams& p, hipStream_t st);
 bool gemm_packed_supported(const GemmParams& p);
 bool gemm_packed_nk_supported(const GemmParams& p);
 int launch_gemm_packed(const GemmParams& p, hipStream_t st, bool b_nk = false);
-// More than 16 rows on packed weights (17 to 224 on [n, k] weights): the weights of a workgroup's columns held in
-// registers, the activations streamed past them, one launch (k up to 4096).
+// Rows of one pass of that kernel (16, fewer when k is long).
+uint32_t gemm_packed_pass_rows(const GemmParams& p);
+// More rows than one such pass takes (on [n, k] weights up to 224): the weights of a workgroup's columns held in
+// registers, the activations streamed past them, one launch (k up to 16384).
 bool gemm_ws_supported(const GemmParams& p, bool b_nk);
 int launch_gemm_ws(const GemmParams& p, hipStream_t st, bool b_nk);
 // The same kernel with the per-token quantisation of x (half or bfloat16, [m, k]) inside: m <= 8 rows that fit the LDS.

@@ -611,7 +611,7 @@ bool swiglu_in_decode_kernel(const ascq_matmul_desc* d, const GemmParams& p, con
     if (!d->trans_b || d->trans_a || d->b_format != ASCQ_MM_B_ND || !fast_path_ok(d, a, b)) {
         return false;
     }
-    return (d->m <= 16 && gemm_packed_nk_supported(p)) || gemm_ws_supported(p, true);
+    return (d->m <= gemm_packed_pass_rows(p) && gemm_packed_nk_supported(p)) || gemm_ws_supported(p, true);
 }
 
 inline size_t round256(size_t v) { return (v + 255u) & ~static_cast<size_t>(255u); }
@@ -657,7 +657,7 @@ extern "C" int ascq_matmul_w8a8_workspace_size(const ascq_matmul_desc* d, size_t
         *bytes = round256(inner) + static_cast<size_t>(d->m) * d->n * sizeof(int32_t);
         return ASCQ_OK;
     }
-    // 17 to 224 rows on [n, k] weights with k up to 4096 run with the weights held in registers: no scratch
+    // [n, k] weights held in registers (17 to 224 rows at k up to 4096, fewer at longer k): no scratch
     const bool ws_nk = d->trans_b && !d->trans_a && d->b_format == ASCQ_MM_B_ND && gemm_ws_supported(shape, true);
     if (ws_nk) {
         return ASCQ_OK;
@@ -755,9 +755,9 @@ extern "C" int ascq_matmul_w8a8(const ascq_matmul_desc* d, void* c, const void* 
         return launch_gemm_stream(p, workspace, st);
     }
     if (d->trans_b && !d->trans_a && gemm_ws_supported(p, true)) {
-        return launch_gemm_ws(p, st, true);  // 17 to 224 rows: the weights held in registers, the activations streamed
+        return launch_gemm_ws(p, st, true);  // the weights held in registers, the activations streamed
     }
-    if (d->m <= 16 && d->trans_b && !d->trans_a && gemm_packed_nk_supported(p)) {
+    if (d->m <= gemm_packed_pass_rows(p) && d->trans_b && !d->trans_a && gemm_packed_nk_supported(p)) {
         return launch_gemm_packed(p, st, true);  // activations resident in LDS, nothing but weights in the load queue
     }
     if (d->m <= 32 && d->trans_b && !d->trans_a && gemm_nk_supported(p)) {

@@ -422,26 +422,28 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_dyn_kernel(PackedPa
     }
 }
 
-// The weight-stationary form, for more than 16 activation rows.  Many rows do not fit the LDS, and activations that
-// are streamed beside the weights share the compute unit's in-order load queue with them (every L2 hit of an
-// activation load then waits behind the weights' trips to memory).  So the two are separated in time: a workgroup
-// first requests all the weights of its columns (up to 3 slabs x 64 tiles = 192 KiB, a wavefront holding its k range
-// of them in 96 registers as ready matrix operands) in one burst with nothing else in the queue, and then streams the
-// activations, 16 rows at a time, from the L2 through a two-slot LDS ring per wavefront: one matrix instruction per
-// slab and tile on operands that are already in registers.  A row tile's sums over the wavefronts' k ranges meet in
-// one LDS array (atomic adds of integers: exact in any order); the epilogue runs once at the end.
-constexpr uint32_t kWsSlabs = 3, kWsTpw = 8, kWsRows = 128;
+// The weight-stationary form, for more rows than the LDS can hold.  Activations that are streamed beside the weights
+// share the compute unit's in-order load queue with them (every L2 hit of an activation load then waits behind the
+// weights' trips to memory).  So the two are separated in time: a workgroup first requests all the weights of its
+// columns (kS slabs, a wavefront's k range of each in kC chunks of 8 tiles: 96 or 128 registers of ready matrix
+// operands per lane) in one burst with nothing else in the queue, and then streams the activations, 16 rows and one
+// chunk of k at a time, from the L2 through a two-slot LDS ring per wavefront: one matrix instruction per slab and
+// tile on operands that are already in registers.  A row tile's sums over the wavefronts' k ranges meet in one LDS
+// array (atomic adds of integers: exact in any order); the epilogue runs once per block of 128 rows.
+//   <3, 1>: k up to 4096, up to 3 slabs per workgroup      <2, 2>: k up to 8192, up to 2 slabs
+//   <1, 4>: k up to 16384, one slab per workgroup
+constexpr uint32_t kWsTpw = 8, kWsRows = 128, kWsMaxChunks = 4;
 constexpr uint32_t kWsNkMaxRows = 224;  // [n, k] weights: beyond this the tile kernels are level or ahead
-constexpr uint32_t kWsRowBytes = kWsTpw * kPkTileK;   // 512: a staged row (the wavefront's k range, padded)
+constexpr uint32_t kWsRowBytes = kWsTpw * kPkTileK;   // 512: a staged row (one chunk of the wavefront's k range)
 constexpr uint32_t kWsSlot = 16u * kWsRowBytes;       // 8 KiB: 16 rows
 constexpr int kWsDma = 8;                             // direct-to-LDS instructions per slot (two rows each)
 
-template <bool kNK>
+template <bool kNK, uint32_t kS, uint32_t kC>
 __global__ __launch_bounds__(kPkWaves * 64) void gemm_ws_kernel(PackedParams p)
 {
     __shared__ __attribute__((aligned(1024))) char R0[kPkWaves * kWsSlot];
     __shared__ __attribute__((aligned(1024))) char R1[kPkWaves * kWsSlot];
-    __shared__ int32_t OUT[kWsRows][kWsSlabs * kPkCols];
+    __shared__ int32_t OUT[kWsRows][kS * kPkCols];
     __shared__ float TS[kWsRows];
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -449,11 +451,13 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_ws_kernel(PackedParams p)
     const uint32_t wg = pk_xcd_order(blockIdx.x, gridDim.x);
     const uint32_t s0 = static_cast<uint32_t>(static_cast<uint64_t>(wg) * p.slabs / gridDim.x);
     const uint32_t s1 = static_cast<uint32_t>(static_cast<uint64_t>(wg + 1u) * p.slabs / gridDim.x);
-    const uint32_t nslabs = s1 - s0;  // at most kWsSlabs: the host has chosen the grid
-    const uint32_t ta = min(wave * p.tpw, p.ktiles), tb = min(ta + p.tpw, p.ktiles), cnt = tb - ta;  // at most kWsTpw
+    const uint32_t nslabs = s1 - s0;  // at most kS: the host has chosen the grid
+    // this wavefront's tiles of k: cnt of them, in nchunks chunks of kWsTpw (nchunks <= kC: the host has chosen kC)
+    const uint32_t ta = min(wave * p.tpw, p.ktiles), tb = min(ta + p.tpw, p.ktiles), cnt = tb - ta;
+    const uint32_t nchunks = (p.tpw + kWsTpw - 1u) / kWsTpw;
     // the sums of a block of kWsRows rows start at zero; the rows' token scales are kept for the epilogue
     auto begin_block = [&](uint32_t b0) __attribute__((always_inline)) {
-        for (uint32_t i = tid; i < kWsRows * kWsSlabs * kPkCols; i += kPkWaves * 64u) (&OUT[0][0])[i] = 0;
+        for (uint32_t i = tid; i < kWsRows * kS * kPkCols; i += kPkWaves * 64u) (&OUT[0][0])[i] = 0;
         if (tid < kWsRows) {
             TS[tid] = (p.epi.has_tok && b0 + tid < p.rows) ? p.epi.tok_scale[p.m0 + b0 + tid] : 1.0f;
         }
@@ -466,68 +470,122 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_ws_kernel(PackedParams p)
         const_cast<i32x4*>(p.wp), 0,
         static_cast<int>(kNK ? p.n * p.k : (p.slabs * p.ktiles + kPkPadTiles) * kPkTileBytes), 0x00020000);
     const uint32_t w_lane = kNK ? lc * p.k + lq * 16u : lane * 16u;
-    i32x4 wreg[kWsSlabs][kWsTpw];
+    i32x4 wreg[kC][kS][kWsTpw];
 #pragma unroll
-    for (uint32_t s = 0; s < kWsSlabs; ++s) {
+    for (uint32_t kc = 0; kc < kC; ++kc) {
 #pragma unroll
-        for (uint32_t t = 0; t < kWsTpw; ++t) {
-            // a tile this wavefront does not have is requested past the end of the buffer: no data moves, the
-            // instruction count stays what the waits below assume
-            const uint32_t off = (s < nslabs && t < cnt) ? w_lane : kPkPastEnd;
-            const uint32_t base = kNK ? (s0 + s) * kPkCols * p.k + (ta + t) * kPkTileK
-                                      : ((s0 + s) * p.ktiles + ta + t) * kPkTileBytes;  // scalar
-            wreg[s][t] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, off, base, kPkNt));
+        for (uint32_t s = 0; s < kS; ++s) {
+#pragma unroll
+            for (uint32_t t = 0; t < kWsTpw; ++t) {
+                // a tile this wavefront does not have is requested past the end of the buffer: no data moves, the
+                // instruction count stays what the waits below assume
+                const uint32_t tile = kc * kWsTpw + t;
+                const uint32_t off = (s < nslabs && tile < cnt) ? w_lane : kPkPastEnd;
+                const uint32_t base = kNK ? (s0 + s) * kPkCols * p.k + (ta + tile) * kPkTileK
+                                          : ((s0 + s) * p.ktiles + ta + tile) * kPkTileBytes;  // scalar
+                wreg[kc][s][t] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, off, base, kPkNt));
+            }
         }
     }
 
-    // ---- activations: slot position (row r, piece q) holds the row's piece q ^ r of this wavefront's k range (the
-    // reader's 16 rows then fall on 16 different bank groups); pieces past the range fetch piece 0 and are not read
+    // ---- activations: slot position (row r, piece q) holds piece q ^ r of the row's share of one chunk (the
+    // reader's 16 rows then fall on 16 different bank groups); pieces past the wavefront's range fetch the chunk's
+    // piece 0 and are not read
     char* const r0w = R0 + wave * kWsSlot;
     char* const r1w = R1 + wave * kWsSlot;
-    // A load's address is a wavefront-uniform base (the row tile) plus the lane's 32-bit offset, which the instruction
-    // adds itself; the last row tile, where rows past the end repeat the last row, has offsets of its own.
+    // A load's address is a wavefront-uniform base (row tile and chunk) plus the lane's 32-bit offset, which the
+    // instruction adds itself; the last row tile, where rows past the end repeat the last row, has offsets of its own.
     // (ntiles, the offsets of the last tile and the base belong to the block of rows being worked on)
-    uint32_t ntiles = 0;
-    uint32_t a_off[kWsDma], a_off_last[kWsDma], a_col[kWsDma];
+    const uint32_t l31 = lane & 31u, l5 = lane >> 5;
+    uint32_t ntiles = 0, last_row = 0;  // last_row: the last valid row of the block's last row tile, 0 .. 15
+    // instruction u of a slot brings rows 2 u and 2 u + 1: the lane's row is r = 2 u + lane / 32, its piece
+    // q = (lane % 32) ^ r, its offset from the base r k + 16 q + the start of the wavefront's k range.  The eight
+    // offsets of a full chunk in a full row tile are kept.  With one chunk per range (kC == 1) its partial filling
+    // is in them, and the block's last row tile has eight offsets of its own.  With more chunks those registers
+    // belong to the weights: a last row tile that is not full and a chunk that the range fills only partly redo
+    // these few operations per request (the asm statement there keeps the compiler from holding the offsets, or
+    // their parts, across the loop all the same).
+    const uint32_t a_lane = l5 * p.k + (cnt != 0u ? ta : 0u) * kPkTileK;  // (no tiles: any valid piece)
+    uint32_t a_off[kWsDma], a_off_last[kC == 1u ? kWsDma : 1];
 #pragma unroll
-    for (int u = 0; u < kWsDma; ++u) {
-        const uint32_t sidx = static_cast<uint32_t>(u) * 64u + lane;
-        const uint32_t r = sidx >> 5, q = (sidx & 31u) ^ r;
-        a_col[u] = (q < cnt * 4u ? q : 0u) * 16u + (cnt != 0u ? ta : 0u) * kPkTileK;  // (no tiles: any valid piece)
-        a_off[u] = r * p.k + a_col[u];
-        a_off_last[u] = a_off[u];
+    for (uint32_t u = 0; u < static_cast<uint32_t>(kWsDma); ++u) {
+        const uint32_t q = l31 ^ (2u * u + l5);
+        a_off[u] = a_lane + 2u * u * p.k + ((kC == 1u && q >= cnt * 4u) ? 0u : q * 16u);
     }
     const int8_t* a_base = p.a;
-    auto issue = [&](uint32_t rt, char* slot) __attribute__((always_inline)) {
-        // past the last row tile: the last one again (never read; keeps the count of loads in flight what the waits assume)
-        const uint32_t tile = rt < ntiles ? rt : ntiles - 1u;
-        const uint64_t bv = reinterpret_cast<uint64_t>(a_base + static_cast<size_t>(tile) * 16u * p.k);
-        uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bv));
-        uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bv >> 32));
-        asm volatile("" : "+s"(lo), "+s"(hi));
-        const int8_t* base = reinterpret_cast<const int8_t*>((static_cast<uint64_t>(hi) << 32) | lo);
-        if (tile + 1u == ntiles) {  // uniform
+    uint32_t i_rt = 0, i_kc = 0;  // the (row tile, chunk) the next request fetches
+    auto issue = [&](char* slot) __attribute__((always_inline)) {
+        // Past the last row tile the requests go on (the count of loads in flight stays what the waits assume) and
+        // fetch something valid that is never read.
+        auto base_of = [&](uint32_t tile, uint32_t col) __attribute__((always_inline)) {
+            const uint64_t bv = reinterpret_cast<uint64_t>(a_base + static_cast<size_t>(tile) * 16u * p.k + col);
+            uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bv));
+            uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bv >> 32));
+            asm volatile("" : "+s"(lo), "+s"(hi));
+            return reinterpret_cast<const int8_t*>((static_cast<uint64_t>(hi) << 32) | lo);
+        };
+        if constexpr (kC == 1u) {
+            const uint32_t tile = i_rt < ntiles ? i_rt : ntiles - 1u;  // (past the end: the last one again)
+            const int8_t* base = base_of(tile, 0u);
+            if (tile + 1u == ntiles) {  // uniform
 #pragma unroll
-            for (int u = 0; u < kWsDma; ++u) {
-                __builtin_amdgcn_global_load_lds((gptr_t)(base + a_off_last[u]), (lds_ptr_t)(slot + u * 1024), 16, 0, 0);
+                for (int u = 0; u < kWsDma; ++u) {
+                    __builtin_amdgcn_global_load_lds((gptr_t)(base + a_off_last[u]), (lds_ptr_t)(slot + u * 1024), 16, 0, 0);
+                }
+            } else {
+#pragma unroll
+                for (int u = 0; u < kWsDma; ++u) {
+                    __builtin_amdgcn_global_load_lds((gptr_t)(base + a_off[u]), (lds_ptr_t)(slot + u * 1024), 16, 0, 0);
+                }
             }
+            ++i_rt;
         } else {
+            const uint32_t t0 = i_kc * kWsTpw;
+            const uint32_t live = cnt > t0 ? min(kWsTpw, cnt - t0) : 0u;  // tiles of this chunk the wavefront has
+            if (i_rt >= ntiles) {  // uniform; past the end: every lane the first piece of the block's first row
+                const int8_t* base = base_of(0u, 0u);
+                uint32_t first = (cnt != 0u ? ta : 0u) * kPkTileK;
+                asm volatile("" : "+v"(first));
 #pragma unroll
-            for (int u = 0; u < kWsDma; ++u) {
-                __builtin_amdgcn_global_load_lds((gptr_t)(base + a_off[u]), (lds_ptr_t)(slot + u * 1024), 16, 0, 0);
+                for (int u = 0; u < kWsDma; ++u) {
+                    __builtin_amdgcn_global_load_lds((gptr_t)(base + first), (lds_ptr_t)(slot + u * 1024), 16, 0, 0);
+                }
+            } else {
+                const int8_t* base = base_of(i_rt, live != 0u ? t0 * kPkTileK : 0u);
+                const uint32_t row_max = i_rt + 1u == ntiles ? last_row : 15u;
+                if (live == kWsTpw && row_max == 15u) {  // uniform
+#pragma unroll
+                    for (int u = 0; u < kWsDma; ++u) {
+                        __builtin_amdgcn_global_load_lds((gptr_t)(base + a_off[u]), (lds_ptr_t)(slot + u * 1024), 16, 0, 0);
+                    }
+                } else {  // rows past the block's last one fetch the last one; pieces past the range fetch piece 0
+                    const uint32_t pieces = live * 4u;
+                    uint32_t x31 = l31, x5 = l5, xc = (cnt != 0u ? ta : 0u) * kPkTileK;
+                    asm volatile("" : "+v"(x31), "+v"(x5), "+v"(xc));
+#pragma unroll
+                    for (uint32_t u = 0; u < static_cast<uint32_t>(kWsDma); ++u) {
+                        const uint32_t r = 2u * u + x5, q = x31 ^ r;  // (both factors below 2^24: k is at most 16384)
+                        const uint32_t off = xc + __umul24(min(r, row_max), p.k) + (q < pieces ? q * 16u : 0u);
+                        __builtin_amdgcn_global_load_lds((gptr_t)(base + off), (lds_ptr_t)(slot + u * 1024), 16, 0, 0);
+                    }
+                }
+            }
+            if (++i_kc == nchunks) {
+                i_kc = 0;
+                ++i_rt;
             }
         }
     };
     // the lane's fragment of tile t: row lc, pieces 4 t + lq; its four sums of a row tile and slab: rows 4 lq + i
     const uint32_t frag = lc * kWsRowBytes;
     const uint32_t out_lane = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)&OUT[0][0])) +
-                              (4u * lq * kWsSlabs * kPkCols + lc) * 4u;
-    i32x4 acc[kWsSlabs];
+                              (4u * lq * kS * kPkCols + lc) * 4u;
+    i32x4 acc[kS];
 #pragma unroll
-    for (uint32_t s = 0; s < kWsSlabs; ++s) acc[s] = i32x4{0, 0, 0, 0};
-    auto compute = [&](uint32_t rt, char* slot) __attribute__((always_inline)) {
+    for (uint32_t s = 0; s < kS; ++s) acc[s] = i32x4{0, 0, 0, 0};
+    // a slot's fragments into registers (after which the slot can be refilled), then the arithmetic on them
+    auto fetch = [&](i32x4 (&a)[kWsTpw], char* slot) __attribute__((always_inline)) {
         const uint32_t sa = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)slot)) + frag;
-        i32x4 a[kWsTpw];
 #pragma unroll
         for (uint32_t t = 0; t < kWsTpw; ++t) {
             const uint32_t addr = sa + (((4u * t + lq) ^ lc) << 4);
@@ -535,31 +593,36 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_ws_kernel(PackedParams p)
         }
         asm volatile("s_waitcnt lgkmcnt(0)"
                      : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7]));
+    };
+    auto compute = [&](const i32x4 (&a)[kWsTpw], uint32_t kc, uint32_t rt) __attribute__((always_inline)) {
 #pragma unroll
         for (uint32_t t = 0; t < kWsTpw; ++t) {
-            if (t < cnt) {  // uniform
+            if (kc * kWsTpw + t < cnt) {  // uniform
 #pragma unroll
-                for (uint32_t s = 0; s < kWsSlabs; ++s) {
+                for (uint32_t s = 0; s < kS; ++s) {
                     if (s < nslabs) {  // uniform
-                        acc[s] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[t], wreg[s][t], acc[s], 0, 0, 0);
+                        acc[s] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[t], wreg[kc][s][t], acc[s], 0, 0, 0);
                     }
                 }
             }
         }
+        if (kc + 1u != nchunks) {  // uniform: the row tile's sums are complete after its last chunk
+            return;
+        }
         // Register i of lane l is row 4 (l / 16) + i of the row tile, column l % 16 of the slab.  Rows past the last
         // one (copies of it) are added to rows of OUT that nobody reads.  The additions are written as instructions:
         // an LDS atomic the compiler knows of makes it wait for every direct-to-LDS load in flight first.
-        const uint32_t oa = out_lane + rt * (16u * kWsSlabs * kPkCols * 4u);
+        const uint32_t oa = out_lane + rt * (16u * kS * kPkCols * 4u);
 #pragma unroll
-        for (uint32_t s = 0; s < kWsSlabs; ++s) {
+        for (uint32_t s = 0; s < kS; ++s) {
             if (s < nslabs) {  // uniform
                 asm volatile("ds_add_u32 %0, %1 offset:%5\n\tds_add_u32 %0, %2 offset:%6\n\t"
                              "ds_add_u32 %0, %3 offset:%7\n\tds_add_u32 %0, %4 offset:%8"
                              :
                              : "v"(oa), "v"(acc[s][0]), "v"(acc[s][1]), "v"(acc[s][2]), "v"(acc[s][3]),
-                               "i"(s * kPkCols * 4u), "i"(s * kPkCols * 4u + kWsSlabs * kPkCols * 4u),
-                               "i"(s * kPkCols * 4u + 2u * kWsSlabs * kPkCols * 4u),
-                               "i"(s * kPkCols * 4u + 3u * kWsSlabs * kPkCols * 4u)
+                               "i"(s * kPkCols * 4u), "i"(s * kPkCols * 4u + kS * kPkCols * 4u),
+                               "i"(s * kPkCols * 4u + 2u * kS * kPkCols * 4u),
+                               "i"(s * kPkCols * 4u + 3u * kS * kPkCols * 4u)
                              : "memory");
             }
             acc[s] = i32x4{0, 0, 0, 0};
@@ -570,30 +633,53 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_ws_kernel(PackedParams p)
     auto set_block = [&](uint32_t b0) __attribute__((always_inline)) {
         brows = min(kWsRows, p.rows - b0);
         ntiles = (brows + 15u) / 16u;
-        const uint32_t rows_last = brows - (ntiles - 1u) * 16u;  // rows of the block's last row tile, 1 .. 16
+        last_row = brows - (ntiles - 1u) * 16u - 1u;
+        if constexpr (kC == 1u) {
 #pragma unroll
-        for (int u = 0; u < kWsDma; ++u) {
-            const uint32_t r = (static_cast<uint32_t>(u) * 64u + lane) >> 5;
-            a_off_last[u] = min(r, rows_last - 1u) * p.k + a_col[u];
+            for (uint32_t u = 0; u < static_cast<uint32_t>(kWsDma); ++u) {
+                const uint32_t r = 2u * u + l5;
+                a_off_last[u] = a_off[u] - (r - min(r, last_row)) * p.k;
+            }
         }
         a_base = p.a + static_cast<size_t>(p.m0 + b0) * p.k;
+        i_rt = 0;
+        i_kc = 0;
     };
-    // the first block's first two row tiles are requested right behind the weights
+    // the first block's first two slots are requested right behind the weights
     set_block(0u);
-    issue(0u, r0w);
-    issue(1u, r1w);
+    issue(r0w);
+    issue(r1w);
     for (uint32_t b0 = 0; b0 < p.rows; b0 += kWsRows) {  // blocks of kWsRows rows: the weights stay where they are
         // Loads return in order: with at most the newest slot's kWsDma loads outstanding, everything older (the
         // weights, the slot about to be read) has arrived.  A slot is refilled as soon as its fragments are in
         // registers; past the last row tile the refills fetch the last tile again, so that the count never changes.
-        for (uint32_t rt = 0; rt < ntiles; rt += 2u) {
+        // (the wait for the LDS counter alone, which the compiler understands, keeps it from placing one of its own
+        // inside the loop for something that was pending in front of it)
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+        auto step = [&](uint32_t kc, uint32_t rt, char* slot) __attribute__((always_inline)) {
             __builtin_amdgcn_s_waitcnt((kWsDma & 15) | ((kWsDma >> 4) << 14) | (7 << 4) | (15 << 8));
-            compute(rt, r0w);
-            issue(rt + 2u, r0w);
-            if (rt + 1u < ntiles) {
-                __builtin_amdgcn_s_waitcnt((kWsDma & 15) | ((kWsDma >> 4) << 14) | (7 << 4) | (15 << 8));
-                compute(rt + 1u, r1w);
-                issue(rt + 3u, r1w);
+            i32x4 a[kWsTpw];
+            fetch(a, slot);
+            issue(slot);
+            compute(a, kc, rt);
+        };
+        if constexpr (kC == 1u) {
+            for (uint32_t rt = 0; rt < ntiles; rt += 2u) {
+                step(0u, rt, r0w);
+                if (rt + 1u < ntiles) {
+                    step(0u, rt + 1u, r1w);
+                }
+            }
+        } else {
+            uint32_t parity = 0;
+            for (uint32_t rt = 0; rt < ntiles; ++rt) {
+#pragma unroll
+                for (uint32_t kc = 0; kc < kC; ++kc) {
+                    if (kc < nchunks) {  // uniform
+                        step(kc, rt, parity != 0u ? r1w : r0w);
+                        parity ^= 1u;
+                    }
+                }
             }
         }
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // nothing lands in LDS after the barrier
@@ -621,8 +707,8 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_ws_kernel(PackedParams p)
             __syncthreads();  // the next block clears what this epilogue read
             begin_block(b0 + kWsRows);
             set_block(b0 + kWsRows);
-            issue(0u, r0w);
-            issue(1u, r1w);
+            issue(r0w);
+            issue(r1w);
         }
     }
 }
@@ -675,11 +761,37 @@ bool gemm_packed_supported(const GemmParams& p)
            (static_cast<uint64_t>((p.n + kPkCols - 1u) / kPkCols) * (p.k / kPkTileK) + kPkPadTiles) * kPkTileBytes < (1ull << 31);
 }
 
-// p.b: the packed weights, or with b_nk the plain [n, k] matrix.  Any m: up to 16 rows per pass over the weights
-// (the callers send more than 16 rows here only when k is too long for the weight-stationary form).
+namespace {
+
+// the grid of the resident form: one workgroup per compute unit when the slabs allow it, at most kPkMaxSlabs slabs each
+uint32_t packed_grid(uint32_t slabs)
+{
+    const uint32_t cus = device_compute_units();
+    uint32_t grid = slabs < cus ? slabs : cus;
+    if ((slabs + grid - 1u) / grid > kPkMaxSlabs) {
+        grid = (slabs + kPkMaxSlabs - 1u) / kPkMaxSlabs;
+    }
+    return grid;
+}
+
+}  // namespace
+
+// Rows the resident form takes per pass over the weights: 16, fewer when k is so long that the staged activations of
+// 16 rows would not fit the LDS beside the partial sums (8 KiB per slab of a workgroup); 0: k is too long altogether.
+uint32_t gemm_packed_pass_rows(const GemmParams& p)
+{
+    const uint32_t slabs = (p.n + kPkCols - 1u) / kPkCols;
+    const uint32_t grid = packed_grid(slabs);
+    const uint32_t tpw = (p.k / kPkTileK + kPkWaves - 1u) / kPkWaves;
+    const uint32_t red_bytes = (slabs + grid - 1u) / grid * kPkWaves * 1024u;
+    const uint32_t rows = (kPkPool - red_bytes) / (kPkWaves * (tpw * kPkTileK + kPkRowPad));
+    return rows > kPkMaxRows ? kPkMaxRows : rows;
+}
+
+// p.b: the packed weights, or with b_nk the plain [n, k] matrix.  Any m, gemm_packed_pass_rows() rows per pass over
+// the weights (the callers send more rows than one pass takes only when k is too long for the weight-stationary form).
 int launch_gemm_packed(const GemmParams& p, hipStream_t st, bool b_nk)
 {
-    const int cus = static_cast<int>(device_compute_units());
     PackedParams q{};
     q.wp = reinterpret_cast<const i32x4*>(p.b);
     q.a = p.a;
@@ -689,18 +801,10 @@ int launch_gemm_packed(const GemmParams& p, hipStream_t st, bool b_nk)
     q.ktiles = p.k / kPkTileK;
     q.tpw = (q.ktiles + kPkWaves - 1u) / kPkWaves;
     q.epi = p.epi;
-    // one workgroup per compute unit when the slabs allow it, at most kPkMaxSlabs slabs per workgroup
-    uint32_t grid = q.slabs < static_cast<uint32_t>(cus) ? q.slabs : static_cast<uint32_t>(cus);
-    if ((q.slabs + grid - 1u) / grid > kPkMaxSlabs) {
-        grid = (q.slabs + kPkMaxSlabs - 1u) / kPkMaxSlabs;
-    }
-    // rows per pass: 16, fewer when k is so long that the staged activations of 16 rows would not fit the LDS beside
-    // the partial sums (8 KiB per slab of a workgroup)
+    const uint32_t grid = packed_grid(q.slabs);
     q.red_slabs = (q.slabs + grid - 1u) / grid;
-    const uint32_t red_bytes = q.red_slabs * kPkWaves * 1024u;
     const uint32_t row_bytes = kPkWaves * (q.tpw * kPkTileK + kPkRowPad);
-    uint32_t pass_rows = (kPkPool - red_bytes) / row_bytes;
-    pass_rows = pass_rows > kPkMaxRows ? kPkMaxRows : pass_rows;
+    const uint32_t pass_rows = gemm_packed_pass_rows(p);
     q.red_off = pass_rows * row_bytes;
     if (pass_rows == 0u) {
         return fail(ASCQ_EUNSUPPORTED, "ascq_matmul_w8a8_packed: k = %u is too long for the staged activations", p.k);
@@ -723,21 +827,57 @@ int launch_gemm_packed(const GemmParams& p, hipStream_t st, bool b_nk)
     return launch_status(b_nk ? "ascq_matmul_w8a8 ([n, k] weight stream)" : "ascq_matmul_w8a8_packed");
 }
 
-// The weight-stationary form: more than 16 rows, k up to 4096 (a wavefront's k range of a slab fits 8 tile registers),
-// any number of rows in one launch (the sums and the epilogue go in blocks of 128 rows).  At k = 4096, n = 11008 it
-// costs 9.5 us (packed weights; 11.5 us for [n, k] weights, whose tiles arrive as 16 runs of 64 bytes) plus about 1 us
-// per 16 rows: every workgroup streams all of the activations, 128 MB through the L2s at 128 rows.  On packed weights it
-// is the path for every call of more than 16 rows; on [n, k] weights up to 128 rows, where it leads the K-split tiles
-// (22.3 against 24.4 us at 128 rows).
+// The weight-stationary form: any number of rows in one launch (the sums and the epilogue go in blocks of 128 rows), k
+// up to 16384 (a wavefront's k range of its slabs fits 96 or 128 tile registers).  At k = 4096, n = 11008 it costs
+// 9.5 us (packed weights; 11.5 us for [n, k] weights, whose tiles arrive as 16 runs of 64 bytes) plus about 1 us per
+// 16 rows: every workgroup streams all of the activations, 128 MB through the L2s at 128 rows.  It takes the calls
+// whose rows the resident form cannot hold in one pass: on packed weights all of them; on [n, k] weights those up to
+// 224 rows at k up to 4096, where it leads the K-split tiles (22.3 against 24.4 us at 128 rows), and at longer k
+// those up to 32 rows whose slabs one round of workgroups holds (k = 11008, n = 4096, 32 rows: 19 against 21 us;
+// the tile kernels lead from 64 rows on, and at once where the workgroups need a second round).
+namespace {
+
+// chunks of kWsTpw tiles in a wavefront's k range; the slabs a workgroup's registers hold then; the grid: one
+// workgroup per compute unit when that leaves it no more slabs than that, otherwise more workgroups
+uint32_t ws_chunks(uint32_t k)
+{
+    const uint32_t tpw = (k / kPkTileK + kPkWaves - 1u) / kPkWaves;
+    return (tpw + kWsTpw - 1u) / kWsTpw;
+}
+
+uint32_t ws_max_slabs(uint32_t nchunks) { return nchunks == 1u ? 3u : nchunks == 2u ? 2u : 1u; }
+
+uint32_t ws_grid(uint32_t slabs, uint32_t max_slabs)
+{
+    const uint32_t cus = device_compute_units();
+    uint32_t grid = slabs < cus ? slabs : cus;
+    if ((slabs + grid - 1u) / grid > max_slabs) {
+        grid = (slabs + max_slabs - 1u) / max_slabs;
+    }
+    return grid;
+}
+
+}  // namespace
+
 bool gemm_ws_supported(const GemmParams& p, bool b_nk)
 {
-    if (p.m <= kPkMaxRows || p.k % kPkTileK != 0 || p.k / kPkTileK > kPkWaves * kWsTpw) {
+    if (p.k % kPkTileK != 0 || p.k / kPkTileK > kPkWaves * kWsTpw * kWsMaxChunks) {
         return false;
     }
-    if (b_nk) {
-        return p.m <= kWsNkMaxRows && gemm_packed_nk_supported(p);  // more rows: the tile kernels
+    if (p.m <= gemm_packed_pass_rows(p)) {
+        return false;  // the activations fit the LDS: the resident form
     }
-    return gemm_packed_supported(p);
+    if (!b_nk) {
+        return gemm_packed_supported(p);
+    }
+    if (!gemm_packed_nk_supported(p)) {
+        return false;
+    }
+    const uint32_t nchunks = ws_chunks(p.k);
+    if (nchunks == 1u) {
+        return p.m <= kWsNkMaxRows;
+    }
+    return p.m <= 32u && ws_grid((p.n + kPkCols - 1u) / kPkCols, ws_max_slabs(nchunks)) <= device_compute_units();
 }
 
 int launch_gemm_ws(const GemmParams& p, hipStream_t st, bool b_nk)
@@ -753,21 +893,28 @@ int launch_gemm_ws(const GemmParams& p, hipStream_t st, bool b_nk)
     q.tpw = (q.ktiles + kPkWaves - 1u) / kPkWaves;
     q.epi = p.epi;
     q.rows_magic = 0;
-    // one workgroup per compute unit when that leaves it at most kWsSlabs slabs, otherwise more workgroups
-    uint32_t grid = q.slabs < cus ? q.slabs : cus;
-    if ((q.slabs + grid - 1u) / grid > kWsSlabs) {
-        grid = (q.slabs + kWsSlabs - 1u) / kWsSlabs;
-    }
+    const uint32_t nchunks = ws_chunks(p.k), max_slabs = ws_max_slabs(nchunks);
+    const uint32_t grid = ws_grid(q.slabs, max_slabs);
     q.m0 = 0;
     q.rows = p.m;
     if (plan_note(ASCQ_MM_KERNEL_STREAM, kWsRows, kPkCols * ((q.slabs + grid - 1u) / grid), kPkTileK, grid, 1,
-                  2u * kPkWaves * kWsSlot + kWsRows * kWsSlabs * kPkCols * 4u, 0)) {
+                  2u * kPkWaves * kWsSlot + kWsRows * max_slabs * kPkCols * 4u, 0)) {
         return ASCQ_OK;
     }
+    auto go = [&](auto nk) {
+        constexpr bool kNK = decltype(nk)::value;
+        if (nchunks == 1u) {
+            gemm_ws_kernel<kNK, 3, 1><<<grid, kPkWaves * 64u, 0, st>>>(q);
+        } else if (nchunks == 2u) {
+            gemm_ws_kernel<kNK, 2, 2><<<grid, kPkWaves * 64u, 0, st>>>(q);
+        } else {
+            gemm_ws_kernel<kNK, 1, 4><<<grid, kPkWaves * 64u, 0, st>>>(q);
+        }
+    };
     if (b_nk) {
-        gemm_ws_kernel<true><<<grid, kPkWaves * 64u, 0, st>>>(q);
+        go(std::true_type{});
     } else {
-        gemm_ws_kernel<false><<<grid, kPkWaves * 64u, 0, st>>>(q);
+        go(std::false_type{});
     }
     return launch_status(b_nk ? "ascq_matmul_w8a8 ([n, k] weights held in registers)"
                               : "ascq_matmul_w8a8_packed (weights held in registers)");

@@ -190,9 +190,8 @@ def test_pack_weight_w8_layout(k, n):
 def test_w8a8_packed_small(m, n, k):
     """The one-launch kernel on packed weights computes what ascq_matmul_w8a8 computes: int32 accumulators and the
     dequantising epilogues bit for bit against the oracle on the unpacked weights.  k of one tile (seven wavefronts
-    without work), column tails, more rows than a pass, k long enough for several batches per slab; more than 16 rows
-    with the weights held in registers where a wavefront's k range fits them (k up to 4096), in passes of 16 rows or
-    fewer where it does not."""
+    without work), column tails, more rows than a pass, k long enough for several batches per slab; more rows than a
+    pass holds with the weights held in registers (k up to 16384)."""
     announce("w8a8 packed", m, n, k)
     rng = np.random.default_rng(m * 31 + n + k)
     a, b = rand_i8(rng, (m, k)), rand_i8(rng, (k, n))
@@ -217,8 +216,8 @@ def test_w8a8_packed_small(m, n, k):
 @pytest.mark.parametrize("n,k", [(16, 64), (48, 128), (1040, 512), (272, 4096), (2064, 192), (13000, 256), (96, 4160)])
 def test_w8a8_weights_held_in_registers(m, n, k):
     """More than 16 rows on packed weights (17 to 224 on [n, k] weights): the weights of a workgroup's columns stay in
-    registers and the activations stream past them, the sums and the epilogue in blocks of 128 rows (k up to 4096;
-    longer k and, on [n, k] weights, more rows take the other kernels).  int32 accumulators against int64
+    registers and the activations stream past them, the sums and the epilogue in blocks of 128 rows (on [n, k]
+    weights, more rows take the other kernels).  int32 accumulators against int64
     arithmetic, the dequantising epilogue bit for bit against the oracle, both forms."""
     announce("w8a8 weights in registers", m, n, k)
     rng = np.random.default_rng(m * 37 + n + k)
@@ -251,6 +250,36 @@ def test_w8a8_weights_held_in_registers(m, n, k):
     assert np.array_equal(bits(c8), gold8)
     cg, dg = run_mm_packed(m, n, k, a, b, out=torch.float16, scalar=1e-3, act=abi.MM_ACT_FASTER_GELU)
     assert max_ulp(bits(cg), oracle_mm(dg, a, b).view(np.uint16), "f16") <= 1
+
+
+@pytest.mark.parametrize("m", [13, 16, 17, 64, 129, 300])
+@pytest.mark.parametrize("n,k", [(48, 11008), (272, 8192), (4112, 4160), (1040, 5632), (40, 16384), (96, 14336),
+                                 (528, 12352)])
+def test_w8a8_weights_held_in_registers_long_k(m, n, k):
+    """k beyond 4096 (up to 16384): a wavefront's k range of its slabs is held in chunks of 8 tiles, two slabs by two
+    chunks (k up to 8192; n = 4112 gives workgroups two slabs) or one slab by four, and the activations stream past
+    them a chunk at a time.  Also the calls of 13 to 16 rows whose staged activations no longer fit the LDS in one
+    pass.  int32 accumulators against exact double arithmetic, the dequantising epilogue bit for bit against the
+    oracle, packed and [n, k] weights."""
+    announce("w8a8 weights in registers, long k", m, n, k)
+    rng = np.random.default_rng(m * 41 + n + k)
+    a, b = rand_i8(rng, (m, k)), rand_i8(rng, (k, n))
+    bt = np.ascontiguousarray(b.T)
+    want = (a.astype(np.float64) @ b.astype(np.float64)).astype(np.int64)  # sums below 2^53: exact
+    c, _ = run_mm_packed(m, n, k, a, b, out=torch.int32)
+    assert np.array_equal(c.cpu().numpy(), want)
+    c, _ = run_mm(m, n, k, a, bt, out=torch.int32, trans_b=True)
+    assert np.array_equal(c.cpu().numpy(), want)
+    if n > 2064:
+        return
+    cs = rng.uniform(1e-4, 1e-2, n).astype(np.float32)
+    ts = rng.uniform(1e-2, 1e-1, m).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    c, desc = run_mm_packed(m, n, k, a, b, out=torch.bfloat16, bias=(bias, None), quant=cs, tok=ts)
+    gold = oracle_mm(desc, a, b, (bias, None), cs, ts)
+    assert np.array_equal(bits(c), gold)
+    c, desc = run_mm(m, n, k, a, bt, out=torch.bfloat16, bias=(bias, None), quant=cs, tok=ts, trans_b=True)
+    assert np.array_equal(bits(c), gold)
 
 
 @pytest.mark.parametrize("m", [1, 16, 32])
