@@ -64,7 +64,7 @@ def main():
     ap.add_argument("--quick", action="store_true", help="headline + W4A16 GEMV only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="run a single workload: w8a8 | w4a16 | w4a16_per_weight | w4a16_per_weight_m4 | w4a16_per_weight_m16 | w4a16_nd | w4a16_m4 | w4a16_m16 | w4a16_nd_m4 | w4a16_nd_m16 | "
-                         "w8a8_zeros | w8a8_m1 | w8a8_m8 | w8a8_m16 | w8a8_m128 | w8a8_m512 | w8a8_m8192 | w8a8_packed_m1 | w8a8_packed_m8 | w8a8_packed_m16 | w8a8_packed_m32 | w8a8_packed_m64 | w8a8_packed_m128 | w8a8_nk_m32 | w8a8_nk_m64 | w8a8_m32 | w8a8_nk_m1 | w8a8_nk_m16 | w8a8_nk_m128 | w8a8_linear_nk_m1 | w8a8_linear_nk_m4 | w8a8_linear_nk_m16 | w8a8_linear_packed_m1 | w8a8_linear_packed_m4 | w8a8_linear_packed_swiglu_m1 | w8a8_linear_nk_swiglu_m1 | w8a16_m1 | w8a16_m16 | w8a16_nk_m1 | w8a16_nk_m4 | w8a16_nk_sum_m1 | w8a16_nk_sum_m4 | "
+                         "w8a8_zeros | w8a8_m1 | w8a8_m8 | w8a8_m16 | w8a8_m128 | w8a8_m512 | w8a8_m8192 | w8a8_packed_m1 | w8a8_packed_m8 | w8a8_packed_m16 | w8a8_packed_m32 | w8a8_packed_m64 | w8a8_packed_m128 | w8a8_packed_down_m16 | w8a8_packed_down_m64 | w8a8_nk_down_m16 | w8a8_nk_m32 | w8a8_nk_m64 | w8a8_m32 | w8a8_nk_m1 | w8a8_nk_m16 | w8a8_nk_m128 | w8a8_linear_nk_m1 | w8a8_linear_nk_m4 | w8a8_linear_nk_m16 | w8a8_linear_packed_m1 | w8a8_linear_packed_m4 | w8a8_linear_packed_swiglu_m1 | w8a8_linear_nk_swiglu_m1 | w8a16_m1 | w8a16_m16 | w8a16_nk_m1 | w8a16_nk_m4 | w8a16_nk_sum_m1 | w8a16_nk_sum_m4 | "
                          "w8a16_nk_m16 | w8a16_m2048 | w8a16_nk_m2048 | quant | dequant | antiquant | group | group_example | mx_fp4 | mx_fp4_e1m2 | mx_fp8 (a W4A16 name without _nd "
                          "is the packed-weight path, in the group-sum form unless it says per_weight; _nk: weights kept as [n, k])")
     ap.add_argument("--copy-probe", action="store_true",
@@ -152,13 +152,15 @@ def main():
         torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------ W8A8 linear (config 3)
-    def w8a8(M, steps, warmup, sets=1, settle=None, zero=False, gauss=False, b_nk=False, packed=False):
+    def w8a8(M, steps, warmup, sets=1, settle=None, zero=False, gauss=False, b_nk=False, packed=False,
+             shape=(4096, 11008)):
         """`sets` > 1 rotates the weights over several copies (together larger than the Infinity Cache) so that the
         weight-bound small-M cases read them from HBM.  The weights are uniform over [-127, 127] unless `gauss`: then
         they are normal weights quantised per output channel by their absolute maximum, as a checkpoint's would be.
         b_nk: the weights are kept as [n, k] (isTransposeB).  packed: the weights in the layout of ascq_pack_weight_w8
-        (packed once, outside the timed region) and the one-launch kernel for few rows."""
-        K, N = 4096, 11008
+        (packed once, outside the timed region) and the one-launch kernel for few rows.  shape: (K, N), by default the
+        up projection's; (11008, 4096) is the down projection of the same layer."""
+        K, N = shape
         x = torch.randn((M, K), device=dev, generator=gen).to(torch.bfloat16)
         if gauss:
             ws = []
@@ -438,6 +440,9 @@ def main():
               "w8a8_packed_m64": lambda: w8a8(64, args.steps, args.warmup, sets=7, packed=True),
               "w8a8_packed_m128": lambda: w8a8(128, args.steps, args.warmup, sets=7, packed=True),
               "w8a8_nk_m64": lambda: w8a8(64, args.steps, args.warmup, sets=7, b_nk=True),
+              "w8a8_packed_down_m16": lambda: w8a8(16, args.steps, args.warmup, sets=7, packed=True, shape=(11008, 4096)),
+              "w8a8_packed_down_m64": lambda: w8a8(64, args.steps, args.warmup, sets=7, packed=True, shape=(11008, 4096)),
+              "w8a8_nk_down_m16": lambda: w8a8(16, args.steps, args.warmup, sets=7, b_nk=True, shape=(11008, 4096)),
               "w8a8_nk_m32": lambda: w8a8(32, args.steps, args.warmup, sets=7, b_nk=True),
               "w8a8_m32": lambda: w8a8(32, args.steps, args.warmup, sets=7),
               "w8a8_linear_nk_m1": lambda: w8a8_linear(1, args.steps, args.warmup),
@@ -565,6 +570,13 @@ def main():
                                            "hbm_frac": r["gemm_gbs"] / PEAK_HBM_GBS,
                                            "note": "weights pre-packed by ascq_pack_weight_w8 (outside the timed "
                                                    "region): one launch, no workspace"}
+            torch.cuda.empty_cache()
+        for M in (16, 64):
+            r = strip(w8a8(M, s2, w2, sets=7, packed=True, shape=(11008, 4096)))
+            others[f"w8a8_packed_down_m{M}"] = {"gemm_kernel_ms": r["gemm_kernel_ms"], "gemm_gbs": r["gemm_gbs"],
+                                                "hbm_frac": r["gemm_gbs"] / PEAK_HBM_GBS,
+                                                "note": "the down projection of the same layer (K=11008, N=4096) on "
+                                                        "packed weights: one launch, weights held in registers"}
             torch.cuda.empty_cache()
         r = strip(w8a8(8192, 40, 5, settle=40))
         others["w8a8_m8192"] = {"gemm_kernel_ms": r["gemm_kernel_ms"], "gemm_tops": r["gemm_tops"],
