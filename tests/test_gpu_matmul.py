@@ -1186,12 +1186,13 @@ def test_group_matmul_swiglu_and_dynamic_linear():
 
 
 @pytest.mark.parametrize("m", [1, 5, 16, 17, 64, 130, 300])
-@pytest.mark.parametrize("n,k", [(22, 128), (1040, 2048), (528, 384), (96, 4096)])
+@pytest.mark.parametrize("n,k", [(22, 128), (1040, 2048), (528, 384), (96, 4096), (64, 8192), (48, 11008)])
 @pytest.mark.parametrize("out,bias", [(torch.bfloat16, None), (torch.float16, "f32"), (torch.float32, "bf16")])
 def test_matmul_swiglu_in_the_decode_kernels(m, n, k, out, bias):
     """SwiGLU on [n, k] and on packed weights: the decode kernels (activations resident in LDS up to 16 rows, weights
-    held in registers beyond) pair the columns of a row through neighbouring lanes in their own epilogue - one launch,
-    no raw accumulators; [n, k] weights past 224 rows take the tile kernels.  Against the oracle."""
+    held in registers beyond, also in chunks of a longer k) pair the columns of a row through neighbouring lanes in
+    their own epilogue - one launch, no raw accumulators; [n, k] weights past 224 rows (32 at k above 4096) take the
+    tile kernels.  Against the oracle."""
     announce("swiglu decode", m, n, k, out, bias)
     rng = np.random.default_rng(m * 5 + n + k)
     a, b = rand_i8(rng, (m, k)), rand_i8(rng, (k, n))
