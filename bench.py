@@ -64,7 +64,7 @@ def main():
     ap.add_argument("--quick", action="store_true", help="headline + W4A16 GEMV only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="run a single workload: w8a8 | w4a16 | w4a16_per_weight | w4a16_per_weight_m4 | w4a16_per_weight_m16 | w4a16_nd | w4a16_m4 | w4a16_m16 | w4a16_nd_m4 | w4a16_nd_m16 | "
-                         "w8a8_zeros | w8a8_m1 | w8a8_m8 | w8a8_m16 | w8a8_m128 | w8a8_m512 | w8a8_m8192 | w8a8_packed_m1 | w8a8_packed_m8 | w8a8_packed_m16 | w8a8_packed_m32 | w8a8_packed_m64 | w8a8_packed_m128 | w8a8_packed_down_m16 | w8a8_packed_down_m64 | w8a8_nk_down_m16 | w8a8_nk_m32 | w8a8_nk_m64 | w8a8_m32 | w8a8_nk_m1 | w8a8_nk_m16 | w8a8_nk_m128 | w8a8_linear_nk_m1 | w8a8_linear_nk_m4 | w8a8_linear_nk_m16 | w8a8_linear_packed_m1 | w8a8_linear_packed_m4 | w8a8_linear_packed_swiglu_m1 | w8a8_linear_nk_swiglu_m1 | w8a16_m1 | w8a16_m16 | w8a16_nk_m1 | w8a16_nk_m4 | w8a16_nk_sum_m1 | w8a16_nk_sum_m4 | "
+                         "w8a8_zeros | w8a8_m1 | w8a8_m8 | w8a8_m16 | w8a8_m128 | w8a8_m512 | w8a8_m8192 | w8a8_packed_m1 | w8a8_packed_m8 | w8a8_packed_m16 | w8a8_packed_m32 | w8a8_packed_m64 | w8a8_packed_m128 | w8a8_packed_down_m16 | w8a8_packed_down_m64 | w8a8_nk_down_m16 | w8a8_nk_m32 | w8a8_nk_m64 | w8a8_m32 | w8a8_nk_m1 | w8a8_nk_m16 | w8a8_nk_m128 | w8a8_linear_nk_m1 | w8a8_linear_nk_m4 | w8a8_linear_nk_m16 | w8a8_linear_packed_m1 | w8a8_linear_packed_m4 | w8a8_linear_packed_swiglu_m1 | w8a8_linear_nk_swiglu_m1 | w8a8_decode_layer_packed_m1 | w8a8_decode_layer_packed_m4 | w8a8_decode_layer_packed_m16 | w8a8_decode_layer_nk_m1 | w8a16_m1 | w8a16_m16 | w8a16_nk_m1 | w8a16_nk_m4 | w8a16_nk_sum_m1 | w8a16_nk_sum_m4 | "
                          "w8a16_nk_m16 | w8a16_m2048 | w8a16_nk_m2048 | quant | dequant | antiquant | group | group_example | mx_fp4 | mx_fp4_e1m2 | mx_fp8 (a W4A16 name without _nd "
                          "is the packed-weight path, in the group-sum form unless it says per_weight; _nk: weights kept as [n, k])")
     ap.add_argument("--copy-probe", action="store_true",
@@ -243,6 +243,45 @@ def main():
         bytes_ = 2 * M * K + K * N + 4 * N + 2 * M * N
         return {"ms_per_step": ms, "kernel_ms": kern_ms, "gbs": bytes_ / (kern_ms * 1e-3) / 1e9, "bytes": bytes_,
                 "tops": 2.0 * M * K * N / (kern_ms * 1e-3) / 1e12, "tensors": (x, ws[0], cs)}
+
+    def w8a8_decode_layer(M, steps, warmup, sets=2, packed=True):
+        """The four W8A8 linears of one decoder layer (hidden 4096, feed-forward 11008) at M rows, one call each: QKV
+        (4096 -> 12288), attention output (4096 -> 4096), gate / up with SwiGLU (4096 -> 2 x 11008 -> 11008) and down
+        (11008 -> 4096), the last one on the output of the one before.  The attention between the first two is not part
+        of this library: its output is a fixed random tensor.  The 202 MB of weights rotate over `sets` copies."""
+        H, F = 4096, 11008
+        x = torch.randn((M, H), device=dev, generator=gen).to(torch.bfloat16)
+        attn = torch.randn((M, H), device=dev, generator=gen).to(torch.bfloat16)
+        qkv = torch.empty((M, 3 * H), dtype=torch.bfloat16, device=dev)
+        h = torch.empty((M, H), dtype=torch.bfloat16, device=dev)
+        g = torch.empty((M, F), dtype=torch.bfloat16, device=dev)
+        y = torch.empty((M, H), dtype=torch.bfloat16, device=dev)
+        plan = (("qkv", H, 3 * H, abi.MM_ACT_NONE), ("o", H, H, abi.MM_ACT_NONE), ("gate_up", H, 2 * F, abi.MM_ACT_SWIGLU),
+                ("down", F, H, abi.MM_ACT_NONE))
+        layers = []
+        for _ in range(sets):
+            lin = {}
+            for name, K, N, act in plan:
+                w = rand_i8(N, K)
+                cs = torch.rand(N, device=dev, generator=gen) * (2e-4 - 1e-4) + 1e-4
+                if packed:
+                    lin[name] = ops.DynamicLinear(M, K, ops.pack_weight_w8(w, K, N, True), cs, packed_n=N, activation=act)
+                    del w
+                else:
+                    lin[name] = ops.DynamicLinear(M, K, w, cs, trans_b=True, activation=act)
+            layers.append(lin)
+
+        def step(i, starts, stops):
+            lin = layers[i % sets]
+            lin["qkv"](qkv, x)
+            lin["o"](h, attn)
+            lin["gate_up"](g, h)
+            lin["down"](y, g)
+
+        ms, kern_ms = timed(step, steps, warmup)
+        bytes_ = sum(K * N + 4 * N + 2 * M * K + 2 * M * (N // 2 if act == abi.MM_ACT_SWIGLU else N) for _, K, N, act in plan)
+        return {"ms_per_step": ms, "kernel_ms": kern_ms, "gbs": bytes_ / (kern_ms * 1e-3) / 1e9, "bytes": bytes_,
+                "launches": 4 if M <= 8 else None, "tensors": (x, attn)}
 
     # ------------------------------------------------------------------ W4A16 decode (config 4)
     def w4a16(M, steps, warmup, sets=4, packed=False, mode=abi.W4A16_PER_WEIGHT):
@@ -452,6 +491,10 @@ def main():
               "w8a8_linear_packed_m4": lambda: w8a8_linear(4, args.steps, args.warmup, packed=True),
               "w8a8_linear_packed_swiglu_m1": lambda: w8a8_linear(1, args.steps, args.warmup, packed=True, swiglu=True),
               "w8a8_linear_nk_swiglu_m1": lambda: w8a8_linear(1, args.steps, args.warmup, swiglu=True),
+              "w8a8_decode_layer_packed_m1": lambda: w8a8_decode_layer(1, args.steps, args.warmup),
+              "w8a8_decode_layer_packed_m4": lambda: w8a8_decode_layer(4, args.steps, args.warmup),
+              "w8a8_decode_layer_packed_m16": lambda: w8a8_decode_layer(16, args.steps, args.warmup),
+              "w8a8_decode_layer_nk_m1": lambda: w8a8_decode_layer(1, args.steps, args.warmup, packed=False),
               "w8a8_nk_m1": lambda: w8a8(1, args.steps, args.warmup, sets=7, b_nk=True),
               "w8a8_nk_m16": lambda: w8a8(16, args.steps, args.warmup, sets=7, b_nk=True),
               "w8a16_nk_m1": lambda: w8a16(1, args.steps, args.warmup, b_nk=True),
@@ -604,6 +647,14 @@ def main():
                                                   "gbs": r["gbs"], "hbm_frac": r["gbs"] / PEAK_HBM_GBS,
                                                   "note": "ascq_linear_w8a8_dynamic_packed: the same one-launch "
                                                           "linear on weights packed by ascq_pack_weight_w8"}
+            torch.cuda.empty_cache()
+        for M in (1, 4):
+            r = strip(w8a8_decode_layer(M, s2, w2))
+            others[f"w8a8_decode_layer_packed_m{M}"] = {
+                "step_ms": r["ms_per_step"], "kernel_ms": r["kernel_ms"], "gbs": r["gbs"],
+                "hbm_frac": r["gbs"] / PEAK_HBM_GBS,
+                "note": "the four linears of a decoder layer (hidden 4096, feed-forward 11008: QKV, attention output, "
+                        "gate / up with SwiGLU, down) on packed weights, four launches per step, 202 MB of weights"}
             torch.cuda.empty_cache()
         for M in (4, 16):
             r = strip(w4a16(M, s2, w2))
