@@ -218,12 +218,13 @@ __device__ __forceinline__ float load_bias_post(const EpiParams& e, size_t col)
 // Large-M kernel built on direct-to-LDS loads and transposing LDS reads (matmul_w8a8_dma.hip).
 bool gemm_dma_supported(const GemmParams& p);
 // b_nk: B is [n][k] (the transposed operand of the plain matmul); not with grouped or fractal B
-int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st, bool b_nk = false);
+// b_layout: 0 B is [k, n] (or fractal), 1 [n, k], 2 the layout of ascq_pack_weight_w8
+int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st, int b_layout = 0);
 uint32_t gemm_dma_skinny_splits(uint32_t m, uint32_t n, uint32_t k);
 bool gemm_stream_supported(const GemmParams& p);
 size_t gemm_stream_workspace(uint32_t m, uint32_t n, uint32_t k);
 int launch_gemm_stream(const GemmParams& p, void* workspace, hipStream_t st);
-int launch_gemm_dma_skinny(GemmParams& p, void* workspace, size_t workspace_bytes, hipStream_t st, bool b_nk = false);
+int launch_gemm_dma_skinny(GemmParams& p, void* workspace, size_t workspace_bytes, hipStream_t st, int b_layout = 0);
 // Few rows, B as [n][k]: whole columns per workgroup, one launch, no workspace (matmul_w8a8_nk.hip).
 bool gemm_nk_supported(const GemmParams& p);
 int launch_gemm_nk(const GemmParams& p, hipStream_t st);
@@ -238,6 +239,7 @@ uint32_t gemm_packed_pass_rows(const GemmParams& p);
 // registers, the activations streamed past them, one launch (k up to 16384).
 bool gemm_ws_supported(const GemmParams& p, bool b_nk);
 int launch_gemm_ws(const GemmParams& p, hipStream_t st, bool b_nk);
+uint32_t gemm_ws_rounds(const GemmParams& p);
 // The same kernel with the per-token quantisation of x (half or bfloat16, [m, k]) inside: m <= 8 rows that fit the LDS.
 bool gemm_packed_dyn_fits(uint32_t m, uint32_t k);
 int launch_gemm_packed_dyn(const GemmParams& p, const void* x, bool x_bf16, hipStream_t st, bool b_nk);

@@ -559,6 +559,24 @@ bool fast_path_ok(const ascq_matmul_desc* d, const void* a, const void* b)
 
 // Up to this many rows the 128 x 128 direct-to-LDS kernel (K split over workgroups) is used when the shape allows.
 constexpr uint32_t kSkinnyMaxM = 512;
+
+// ascq_matmul_w8a8_packed between 129 and 512 rows: true when the 128 x 128 tiles (no K split: the call has no
+// workspace) are expected to beat the weights-in-registers form.  Both estimates are fits to measurements at
+// k = 4096, n = 11008 and k = 11008, n = 4096 (the crossovers there: 256 and about 380 rows).  Registers form: the
+// weights once (5 us + 1 us per 4.7 MB), then 0.95 us per 16 rows and 4096 of k, per round of workgroups.  Tiles:
+// 6.5 us per 1024 of k for up to one tile per compute unit, 1.45 times that with two (they share the unit), and in
+// proportion beyond.  Above 512 rows the 256-row tiles always lead.
+bool packed_tiles_faster(const GemmParams& p)
+{
+    const double kk = p.k / 4096.0;
+    const double ws_us = 5.0 + static_cast<double>(p.n) * p.k / 4.7e6 +
+                         0.95 * kk * ((p.m + 15u) / 16u) * gemm_ws_rounds(p);
+    const double tiles = static_cast<double>((p.m + 127u) / 128u) * ((p.n + 127u) / 128u);
+    const double cus = device_compute_units();
+    const double load = tiles <= cus ? 1.0 : tiles <= 2.0 * cus ? 1.0 + 0.45 * (tiles - cus) / cus : 1.45 * tiles / (2.0 * cus);
+    const double tiles_us = 4.0 + 26.0 * kk * load;
+    return tiles_us < ws_us;
+}
 // Up to this many rows the weight-stream kernel is preferred over those tiles.
 constexpr uint32_t kStreamMaxM = 8;
 
@@ -832,6 +850,15 @@ extern "C" int ascq_matmul_w8a8_packed(const ascq_matmul_desc* d, void* c, const
     ASCQ_REQUIRE(d->k % 64u == 0, ASCQ_EUNSUPPORTED, "ascq_matmul_w8a8_packed: k = %u must be a multiple of 64", d->k);
     ASCQ_REQUIRE(aligned16(a) && aligned16(w_packed), ASCQ_EALIGN, "ascq_matmul_w8a8_packed: a and w_packed must be 16-byte aligned");
     ASCQ_REQUIRE(gemm_packed_supported(p), ASCQ_EUNSUPPORTED, "ascq_matmul_w8a8_packed: the packed weights must stay below 2 GiB");
+    // Many rows: the direct-to-LDS tile kernels read the packed tiles as they lie (one tile per load instruction), so a
+    // caller that packed its weights for decode needs no second copy of them for prefill.  (SwiGLU in those kernels'
+    // epilogue exists for 16-bit outputs.)
+    const bool tiles_ok = gemm_dma_supported(p) &&
+                          (d->activation != ASCQ_MM_ACT_SWIGLU || d->out_dtype == ASCQ_F16 || d->out_dtype == ASCQ_BF16);
+    if (tiles_ok && (d->m > kSkinnyMaxM || (d->m > 128u && packed_tiles_faster(p)))) {
+        return d->m <= kSkinnyMaxM ? launch_gemm_dma_skinny(p, nullptr, 0, static_cast<hipStream_t>(stream), 2)
+                                   : launch_gemm_dma(p, false, static_cast<hipStream_t>(stream), 2);
+    }
     if (gemm_ws_supported(p, false)) {
         return launch_gemm_ws(p, static_cast<hipStream_t>(stream), false);
     }

@@ -88,10 +88,13 @@ struct TilePlace {
     size_t chan_off;
 };
 
-template <int BM, int BN, bool kSplitK, bool kGrouped, bool kBT = false>
+// kB: how B lies in memory.  0: [k, n] (or the fractal panels); 1: [n, k]; 2: the layout of ascq_pack_weight_w8
+// (slabs of 16 columns, each a run of 1 KiB tiles of 64 k: lane l of a tile owns column l % 16, k 16 (l / 16) .. + 15).
+template <int BM, int BN, bool kSplitK, bool kGrouped, int kB = 0>
 __device__ __forceinline__ void gemm_dma_tile_at(const GemmParams& p, const TilePlace& at, uint32_t bidy, char* A0,
                                                  char* B0, char* A1, char* B1, float* TS)
 {
+    constexpr bool kBT = kB == 1, kBP = kB == 2;
     constexpr int kWN = BN / 64;            // wavefronts along N
     constexpr int kWM = 8 / kWN;            // wavefronts along M
     constexpr int TI = BM / 32 / kWM;       // 32x32 blocks per wavefront along M
@@ -134,6 +137,15 @@ __device__ __forceinline__ void gemm_dma_tile_at(const GemmParams& p, const Tile
 #pragma unroll
     for (int u = 0; u < kBInstr; ++u) {
         const uint32_t s = (wave * kBInstr + u) * 64 + lane;
+        if constexpr (kBP) {
+            // one instruction = one packed tile: piece (slab j of the tile's BN / 16, k tile h of the step's two)
+            // lands in LDS as it lies in memory; slabs past the last one are never stored
+            const uint32_t piece = wave * kBInstr + u, j = piece >> 1, h = piece & 1u;
+            const uint32_t slab0 = n0 >> 4, last = (N + 15u) / 16u - 1u;
+            const uint32_t slab = slab0 + j < last ? slab0 + j : last;
+            boff[u] = (slab - slab0) * (K * 16u) + h * 1024u + lane * 16u;
+            continue;
+        }
         if constexpr (kBT) {
             const uint32_t r = s >> 3, c = (s & 7u) ^ ((r >> 1) & 7u);
             uint32_t col = n0 + r;
@@ -149,7 +161,7 @@ __device__ __forceinline__ void gemm_dma_tile_at(const GemmParams& p, const Tile
         // fractal B: panels of 32 columns, each a contiguous row-major [K][32] block
         boff[u] = p.b_nz ? ((col >> 5) * K + kb) * 32u + (col & 31u) : kb * N + (col - n0);
     }
-    const uint32_t ldb = kBT ? 1u : p.b_nz ? 32u : N;  // bytes from one k to the next
+    const uint32_t ldb = kBT ? 1u : kBP ? 16u : p.b_nz ? 32u : N;  // bytes from one k to the next
     // K range of this workgroup, in steps of BK
     uint32_t s_begin = 0, steps = K / BK;
     if constexpr (kSplitK) {
@@ -157,7 +169,8 @@ __device__ __forceinline__ void gemm_dma_tile_at(const GemmParams& p, const Tile
         steps = steps * (bidy + 1u) / p.k_splits - s_begin;
     }
     const int8_t* Abase = p.a + static_cast<size_t>(row0) * K + static_cast<size_t>(s_begin) * BK;
-    const int8_t* Bbase = Bmat + (kBT ? static_cast<size_t>(n0) * K : p.b_nz ? 0u : n0) + static_cast<size_t>(s_begin) * BK * ldb;
+    const int8_t* Bbase = Bmat + (kBT ? static_cast<size_t>(n0) * K : kBP ? static_cast<size_t>(n0 >> 4) * K * 16u : p.b_nz ? 0u : n0) +
+                          static_cast<size_t>(s_begin) * BK * ldb;
     // A wavefront-uniform address, pinned to scalar registers: a load's address is then this base plus the lane's
     // 32-bit offset, which the load instruction adds itself (otherwise the compiler widens the offsets to 64 bits
     // ahead of the loop and adds the base per load: twice the registers and an addition per load).
@@ -206,6 +219,11 @@ __device__ __forceinline__ void gemm_dma_tile_at(const GemmParams& p, const Tile
     for (int ks = 0; ks < 4; ++ks) {
         a_base[ks] = (wm * (TI * 32) + lrow) * 128 + (((2 * ks + g) ^ ((lrow >> 1) & 7u)) << 4);
         bt_base[ks] = (wn * (TJ * 32) + lrow) * 128 + (((2 * ks + g) ^ ((lrow >> 1) & 7u)) << 4);
+        if constexpr (kBP) {
+            // column block j of the wavefront: slabs 4 wn + 2 j + lrow / 16 (2 KiB each: the step's two k tiles); sub-step
+            // ks is k tile ks / 2, its 16-byte groups 2 (ks % 2) + g; inside a group the 16 columns lie side by side
+            bt_base[ks] = wn * 8192u + (lrow >> 4) * 2048u + (ks >> 1) * 1024u + ((ks & 1) * 2u + g) * 256u + (lrow & 15u) * 16u;
+        }
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
@@ -215,7 +233,7 @@ __device__ __forceinline__ void gemm_dma_tile_at(const GemmParams& p, const Tile
     // In the order the MFMAs of a sub-step want them (they run row block by row block): B0, A0, B1, A1, A2, ...
     auto load_frags = [&](const char* As, const char* Bs, int ks, i32x4 (&af)[TI], i32x4 (&bf)[TJ]) {
         auto load_b = [&](int j) {
-            if constexpr (kBT) {
+            if constexpr (kBT || kBP) {
                 bf[j] = *reinterpret_cast<const i32x4*>(Bs + bt_base[ks] + j * 4096);
             } else {
                 const i32x2_t lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2_t)(Bs + b_base[j] + ks * kKsB));
@@ -247,7 +265,7 @@ __device__ __forceinline__ void gemm_dma_tile_at(const GemmParams& p, const Tile
     // instructions of its second half run while the last reads are still on their way: the next sub-step starts by
     // waiting for all of them.
     auto interleave = [&]() __attribute__((always_inline)) {
-        constexpr int kReads = TI + (kBT ? TJ : 2 * TJ);
+        constexpr int kReads = TI + ((kBT || kBP) ? TJ : 2 * TJ);
         constexpr int kMfmas = TI * TJ;
         constexpr int kFront = (kMfmas + 1) / 2;
         constexpr int kPer = (kReads + kFront - 1) / kFront;
@@ -269,7 +287,7 @@ __device__ __forceinline__ void gemm_dma_tile_at(const GemmParams& p, const Tile
         for (int q = 0; q < 4; ++q) asm volatile("" : "+v"(a_base[q]));
 #pragma unroll
         for (int q = 0; q < 2; ++q) asm volatile("" : "+v"(b_base[q]));
-        if constexpr (kBT) {
+        if constexpr (kBT || kBP) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) asm volatile("" : "+v"(bt_base[q]));
         }
@@ -526,7 +544,7 @@ __device__ __forceinline__ void gemm_dma_tile_at(const GemmParams& p, const Tile
 
 // The plain matmul: tile number `bid` of the launch (before the XCD remapping), column tiles counted from col_begin,
 // row tiles innermost so that the tiles an XCD runs side by side share their B columns.
-template <int BM, int BN, bool kSplitK, bool kBT>
+template <int BM, int BN, bool kSplitK, int kB>
 __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_begin, uint32_t bid, uint32_t bidy,
                                               char* A0, char* B0, char* A1, char* B1, float* TS)
 {
@@ -540,7 +558,7 @@ __device__ __forceinline__ void gemm_dma_tile(const GemmParams& p, uint32_t col_
     uint32_t ms, tn;
     band_order(t, p.tiles_m, p.tiles_n, ms, tn);
     const TilePlace at{ms * BM, p.m, col_begin + tn * BN, p.b, 0};
-    gemm_dma_tile_at<BM, BN, kSplitK, false, kBT>(p, at, bidy, A0, B0, A1, B1, TS);
+    gemm_dma_tile_at<BM, BN, kSplitK, false, kB>(p, at, bidy, A0, B0, A1, B1, TS);
 }
 
 // Rows [off, end) of group g (clipped to m); false when the group owns none.  `off` is carried from group to group.
@@ -690,7 +708,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_dma_group_kernel(GemmParams 
     gemm_dma_group_phase<2>(p, PLAN, A0, B0, A1, B1, TS);
 }
 
-template <int BM, int BN, bool kSplitK, bool kBT = false>
+template <int BM, int BN, bool kSplitK, int kB = 0>
 __global__ __launch_bounds__(kThreads, (BM * BK + BK * BN) * 2 <= 65536 ? 2 : 1) void gemm_dma_kernel(
     GemmParams p, uint32_t col_begin)
 {
@@ -699,13 +717,13 @@ __global__ __launch_bounds__(kThreads, (BM * BK + BK * BN) * 2 <= 65536 ? 2 : 1)
     __shared__ __attribute__((aligned(1024))) char A1[BM * BK];
     __shared__ __attribute__((aligned(1024))) char B1[BK * BN];
     __shared__ __attribute__((aligned(16))) float TS[BM];  // token scales of the tile's rows (1.0f when there are none)
-    gemm_dma_tile<BM, BN, kSplitK, kBT>(p, col_begin, blockIdx.x, blockIdx.y, A0, B0, A1, B1, TS);
+    gemm_dma_tile<BM, BN, kSplitK, kB>(p, col_begin, blockIdx.x, blockIdx.y, A0, B0, A1, B1, TS);
 }
 
 // One launch for a matrix whose last round of 256 x 256 tiles would be mostly empty: workgroups [0, wide_wgs) run the
 // 256 x 256 tiles of the first `p.tiles_n` tile columns, the rest 256 x 128 tiles of the remaining columns.  A compute
 // unit that has finished its wide tile takes a narrow one at once, without the drain between two launches.
-template <bool kBT>
+template <int kB>
 __global__ __launch_bounds__(kThreads, 1) void gemm_dma_dual_kernel(GemmParams p, uint32_t wide_wgs,
                                                                     uint32_t narrow_tiles_n, uint32_t col_begin)
 {
@@ -715,11 +733,11 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_dma_dual_kernel(GemmParams p
     __shared__ __attribute__((aligned(1024))) char B1[BK * 256];
     __shared__ __attribute__((aligned(16))) float TS[256];
     if (blockIdx.x < wide_wgs) {
-        gemm_dma_tile<256, 256, false, kBT>(p, 0u, blockIdx.x, 0u, A0, B0, A1, B1, TS);
+        gemm_dma_tile<256, 256, false, kB>(p, 0u, blockIdx.x, 0u, A0, B0, A1, B1, TS);
     } else {
         GemmParams q = p;
         q.tiles_n = narrow_tiles_n;
-        gemm_dma_tile<256, 128, false, kBT>(q, col_begin, blockIdx.x - wide_wgs, 0u, A0, B0, A1, B1, TS);
+        gemm_dma_tile<256, 128, false, kB>(q, col_begin, blockIdx.x - wide_wgs, 0u, A0, B0, A1, B1, TS);
     }
 }
 
@@ -760,7 +778,24 @@ bool gemm_dma_supported(const GemmParams& p)
     return p.k % BK == 0 && p.n % 16 == 0 && p.n >= 16 && aligned16(p.a) && aligned16(p.b);
 }
 
-int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st, bool b_nk)
+namespace {
+
+// calls f with the B layout (0: [k, n], 1: [n, k], 2: packed by ascq_pack_weight_w8) as a compile-time constant
+template <class F>
+void with_b_layout(int b_layout, F&& f)
+{
+    if (b_layout == 2) {
+        f(std::integral_constant<int, 2>{});
+    } else if (b_layout == 1) {
+        f(std::integral_constant<int, 1>{});
+    } else {
+        f(std::integral_constant<int, 0>{});
+    }
+}
+
+}  // namespace
+
+int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st, int b_layout)
 {
     uint32_t tiles_n = (p.n + 255u) / 256u;
     if (grouped) {
@@ -823,11 +858,10 @@ int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st, bool b_nk)
         const uint32_t wide_wgs = (p.tiles_m * wide_cols + 7u) / 8u * 8u;
         const uint32_t narrow_wgs = (p.tiles_m * narrow_tiles_n + 7u) / 8u * 8u;
         p.tiles_n = wide_cols;
-        if (b_nk) {
-            gemm_dma_dual_kernel<true><<<wide_wgs + narrow_wgs, kThreads, 0, st>>>(p, wide_wgs, narrow_tiles_n, col_begin);
-        } else {
-            gemm_dma_dual_kernel<false><<<wide_wgs + narrow_wgs, kThreads, 0, st>>>(p, wide_wgs, narrow_tiles_n, col_begin);
-        }
+        with_b_layout(b_layout, [&](auto kb) {
+            gemm_dma_dual_kernel<decltype(kb)::value><<<wide_wgs + narrow_wgs, kThreads, 0, st>>>(p, wide_wgs, narrow_tiles_n,
+                                                                                                  col_begin);
+        });
         return launch_status("ascq_matmul_w8a8");
     }
     if (wide_cols) {
@@ -838,21 +872,17 @@ int launch_gemm_dma(GemmParams& p, bool grouped, hipStream_t st, bool b_nk)
         if (narrow_cols) {
             q.n = p.n;  // row pitch stays n; columns >= wide_cols * 256 are simply not assigned to any tile
         }
-        if (b_nk) {
-            gemm_dma_kernel<256, 256, false, true><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(q, 0u);
-        } else {
-            gemm_dma_kernel<256, 256, false><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(q, 0u);
-        }
+        with_b_layout(b_layout, [&](auto kb) {
+            gemm_dma_kernel<256, 256, false, decltype(kb)::value><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(q, 0u);
+        });
     }
     if (narrow_cols) {
         const uint32_t col_begin = wide_cols * 256u;
         p.tiles_n = (p.n - col_begin + 127u) / 128u;
         const uint32_t t = p.tiles_m * p.tiles_n;
-        if (b_nk) {
-            gemm_dma_kernel<256, 128, false, true><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(p, col_begin);
-        } else {
-            gemm_dma_kernel<256, 128, false><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(p, col_begin);
-        }
+        with_b_layout(b_layout, [&](auto kb) {
+            gemm_dma_kernel<256, 128, false, decltype(kb)::value><<<(t + 7u) / 8u * 8u, kThreads, 0, st>>>(p, col_begin);
+        });
     }
     return launch_status("ascq_matmul_w8a8");
 }
@@ -878,15 +908,16 @@ uint32_t gemm_dma_skinny_splits(uint32_t m, uint32_t n, uint32_t k)
 }
 
 // M up to a few hundred rows: 128 x 128 tiles, K split over blockIdx.y when a workspace of
-// splits * m * n * 4 bytes (16-byte aligned) is given.  b_nk: B is [n][k].
-int launch_gemm_dma_skinny(GemmParams& p, void* workspace, size_t workspace_bytes, hipStream_t st, bool b_nk)
+// splits * m * n * 4 bytes (16-byte aligned) is given.  b_layout: 0 [k, n], 1 [n, k], 2 packed (never split: its
+// entry point has no workspace).
+int launch_gemm_dma_skinny(GemmParams& p, void* workspace, size_t workspace_bytes, hipStream_t st, int b_layout)
 {
     p.tiles_m = (p.m + 127u) / 128u;
     p.tiles_n = (p.n + 127u) / 128u;
     const uint32_t t = (p.tiles_m * p.tiles_n + 7u) / 8u * 8u;
     uint32_t splits = gemm_dma_skinny_splits(p.m, p.n, p.k);
     const size_t need = static_cast<size_t>(splits) * p.m * p.n * sizeof(int32_t);
-    if (splits > 1 && (workspace == nullptr || workspace_bytes < need || !aligned16(workspace))) {
+    if (splits > 1 && (workspace == nullptr || workspace_bytes < need || !aligned16(workspace) || b_layout == 2)) {
         splits = 1;
     }
     if (plan_recording()) {
@@ -898,17 +929,15 @@ int launch_gemm_dma_skinny(GemmParams& p, void* workspace, size_t workspace_byte
         return ASCQ_OK;
     }
     if (splits == 1) {
-        if (b_nk) {
-            gemm_dma_kernel<128, 128, false, true><<<t, kThreads, 0, st>>>(p, 0u);
-        } else {
-            gemm_dma_kernel<128, 128, false><<<t, kThreads, 0, st>>>(p, 0u);
-        }
+        with_b_layout(b_layout, [&](auto kb) {
+            gemm_dma_kernel<128, 128, false, decltype(kb)::value><<<t, kThreads, 0, st>>>(p, 0u);
+        });
         return launch_status("ascq_matmul_w8a8");
     }
     p.k_splits = splits;
     p.partial = static_cast<int32_t*>(workspace);
-    if (b_nk) {
-        gemm_dma_kernel<128, 128, true, true><<<dim3(t, splits), kThreads, 0, st>>>(p, 0u);
+    if (b_layout == 1) {
+        gemm_dma_kernel<128, 128, true, 1><<<dim3(t, splits), kThreads, 0, st>>>(p, 0u);
     } else {
         gemm_dma_kernel<128, 128, true><<<dim3(t, splits), kThreads, 0, st>>>(p, 0u);
     }

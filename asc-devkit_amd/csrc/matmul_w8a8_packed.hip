@@ -880,9 +880,15 @@ bool gemm_ws_supported(const GemmParams& p, bool b_nk)
     return p.m <= 32u && ws_grid((p.n + kPkCols - 1u) / kPkCols, ws_max_slabs(nchunks)) <= device_compute_units();
 }
 
-int launch_gemm_ws(const GemmParams& p, hipStream_t st, bool b_nk)
+// Rounds of workgroups the weight-stationary form needs on this device (1: every workgroup is resident at once).
+uint32_t gemm_ws_rounds(const GemmParams& p)
 {
     const uint32_t cus = device_compute_units();
+    return (ws_grid((p.n + kPkCols - 1u) / kPkCols, ws_max_slabs(ws_chunks(p.k))) + cus - 1u) / cus;
+}
+
+int launch_gemm_ws(const GemmParams& p, hipStream_t st, bool b_nk)
+{
     PackedParams q{};
     q.wp = reinterpret_cast<const i32x4*>(p.b);
     q.a = p.a;

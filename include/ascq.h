@@ -378,10 +378,12 @@ int ascq_matmul_w8a8_workspace_size(const ascq_matmul_desc* desc, size_t* bytes)
  * workgroup owns whole columns, its wavefronts split k, and integer partial sums are exact in any order.  Up to 16
  * rows (fewer at long k: 12 at k = 11008, n = 4096) the activations stay in LDS and the weights stream past them
  * once.  More rows with k up to 16384 turn the roles round: a workgroup first fetches the weights of its columns into
- * registers and then streams the activations past them, still in one launch - every workgroup reads all of the
- * activations, so the call suits m up to about 300 (beyond that ascq_matmul_w8a8 on unpacked weights is faster).
- * With k above 16384 the rows that do not fit the LDS take one pass over the weights per group that does.  Requires
- * k % 64 == 0 and a, w_packed 16-byte aligned.
+ * registers and then streams the activations past them, still in one launch.  Every workgroup reads all of the
+ * activations there, so from a few hundred rows on (always above 512; between 129 and 512 by an estimate of both
+ * times) the call runs the tile kernels of ascq_matmul_w8a8 instead, which read the packed tiles as they lie (n % 16 ==
+ * 0 and k % 128 == 0; other shapes stay with the registers form): weights packed for decode serve prefill at the speed
+ * of unpacked ones, without a second copy.  With k above 16384 the rows that do not fit the LDS take one pass over the
+ * weights per group that does.  Requires k % 64 == 0 and a, w_packed 16-byte aligned.
  * ref: include/adv_api/matmul/matmul.h:175-185 (the Matmul object and its quant epilogue)
  */
 int ascq_pack_weight_w8_size(uint32_t k, uint32_t n, size_t* bytes);

@@ -282,6 +282,48 @@ def test_w8a8_weights_held_in_registers_long_k(m, n, k):
     assert np.array_equal(bits(c), gold)
 
 
+@pytest.mark.parametrize("m", [129, 200, 256, 300, 513, 700, 1100])
+@pytest.mark.parametrize("n,k", [(256, 128), (1040, 512), (272, 4096), (2064, 384), (4112 + 16, 256), (96, 1152)])
+def test_w8a8_packed_many_rows_on_the_tile_kernels(m, n, k):
+    """Many rows on packed weights (n a multiple of 16, k of 128): the direct-to-LDS tile kernels (128 x 128 tiles up to
+    512 rows, 256-row tiles beyond, with the narrow tiles of a partly filled last round) read the packed tiles as they
+    lie.  int32 accumulators against exact double arithmetic; the dequantising epilogue, the requantising one and
+    SwiGLU against the oracle."""
+    announce("w8a8 packed, tile kernels", m, n, k)
+    rng = np.random.default_rng(m * 43 + n + k)
+    a, b = rand_i8(rng, (m, k)), rand_i8(rng, (k, n))
+    want = (a.astype(np.float64) @ b.astype(np.float64)).astype(np.int64)
+    c, _ = run_mm_packed(m, n, k, a, b, out=torch.int32)
+    assert np.array_equal(c.cpu().numpy(), want)
+    if n > 2064:
+        return
+    cs = rng.uniform(1e-4, 1e-2, n).astype(np.float32)
+    ts = rng.uniform(1e-2, 1e-1, m).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    c, desc = run_mm_packed(m, n, k, a, np.ascontiguousarray(b.T), out=torch.bfloat16, bias=(bias, None), quant=cs, tok=ts,
+                            trans_b=True)
+    assert np.array_equal(bits(c), oracle_mm(desc, a, b, (bias, None), cs, ts))
+    words = (cs * 50).astype(np.float32).view(np.uint32).astype(np.uint64) | (np.uint64(1) << np.uint64(46))
+    words[n // 2] |= (np.uint64(1) << np.uint64(36)) | (np.uint64(3) << np.uint64(32))
+    bias_i = rng.integers(-1000, 1000, n).astype(np.int32)
+    c8, d8 = run_mm_packed(m, n, k, a, b, out=torch.int8, bias=(bias_i, None), quant=words)
+    assert np.array_equal(bits(c8), oracle_mm(d8, a, b, (bias_i, None), words))
+    # SwiGLU of the column pairs in the tile kernels' epilogue (16-bit outputs)
+    css = rng.uniform(1e-4, 4e-4, n).astype(np.float32)
+    tss = rng.uniform(0.5, 2.0, m).astype(np.float32)
+    mm = ops.Matmul(m, n, k, False, False)
+    mm.set_tensor_a(to_dev(a))
+    mm.set_tensor_b_packed(ops.pack_weight_w8(to_dev(b), k, n))
+    mm.set_quant_vector(to_dev(css))
+    mm.set_token_scale(to_dev(tss))
+    mm.set_activation(abi.MM_ACT_SWIGLU, 1.702)
+    cg = torch.zeros((m, n // 2), dtype=torch.bfloat16, device=DEV)
+    mm.iterate_all(cg)
+    d = abi.MatmulDesc(m=m, n=n, k=k, out_dtype=abi.BF16, quant_mode=abi.MM_QUANT_VECTOR, scale_format=abi.MM_SCALE_F32,
+                       has_tok_scale=1, activation=abi.MM_ACT_SWIGLU, act_beta=1.702)
+    swiglu_close(bits(cg), oracle_mm(d, a, b, None, css, tss).view(np.uint16), "bf16")
+
+
 @pytest.mark.parametrize("m", [1, 16, 32])
 def test_config3_w8a8_linear_packed(m):
     """Config 3's decode sizes on packed weights: per-token quantisation on the GPU, one launch for the matmul, bf16
