@@ -33,7 +33,7 @@ constexpr uint32_t kPkPadTiles = 16;   // tiles of zeros behind the last slab (a
 constexpr uint32_t kPkWaves = 8, kPkBatch = 4, kPkMaxSlabs = 8, kPkMaxRows = 16;
 constexpr int kPkBuf = 2;              // register buffers: one batch in flight while the other is computed
 constexpr uint32_t kPkRowPad = 16;     // bytes added to a staged activation row: rows start 4 banks apart
-constexpr uint32_t kPkPool = 152 * 1024;  // LDS of a workgroup: the staged activations, then 8 KiB of partial sums per slab
+constexpr uint32_t kPkPool = 158 * 1024;  // LDS of a workgroup (of 160 KiB): the staged activations, then 8 KiB of partial sums per slab
 constexpr uint32_t kPkPastEnd = 0x7FFFFFF0u;
 constexpr int kPkNt = 2;               // cache policy of the weight loads: non-temporal (read once per call)
 

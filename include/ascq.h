@@ -376,7 +376,7 @@ int ascq_matmul_w8a8_workspace_size(const ascq_matmul_desc* desc, size_t* bytes)
  * ascq_matmul_w8a8_packed computes exactly what ascq_matmul_w8a8 computes (same descriptor, epilogues - SwiGLU
  * included - and outputs; desc.trans_b is ignored, desc.trans_a is not supported) in one launch with no workspace: a
  * workgroup owns whole columns, its wavefronts split k, and integer partial sums are exact in any order.  Up to 16
- * rows (fewer at long k: 12 at k = 11008, n = 4096) the activations stay in LDS and the weights stream past them
+ * rows (fewer at long k: 13 at k = 11008, n = 4096) the activations stay in LDS and the weights stream past them
  * once.  More rows with k up to 16384 turn the roles round: a workgroup first fetches the weights of its columns into
  * registers and then streams the activations past them, still in one launch.  Every workgroup reads all of the
  * activations there, so from a few hundred rows on (always above 512; between 129 and 512 by an estimate of both
