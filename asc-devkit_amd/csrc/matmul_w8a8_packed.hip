@@ -202,6 +202,171 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_kernel(PackedParams
     }
 }
 
+// The same kernel for weights kept as [n, k] with the weights going through LDS: read straight into registers as matrix
+// operands, a tile of [n, k] weights is 16 runs of 64 bytes per load instruction, which the memory pipeline of a
+// compute unit takes at about half the rate of long runs.  Here a load instruction brings four columns' 256 bytes (the
+// four tiles of a batch) into a two-slot ring per wavefront, with the 16-byte pieces of column c stored at position
+// piece ^ c, so that the 16 lanes that read one piece of 16 different columns fall on 16 different bank groups.  The
+// loads are buffer loads (range-checked: a batch that reaches past the matrix reads zeros, and the requests past the
+// last batch move no data); the ring is an array of its own, so that the compiler does not make the reads of the
+// staged activations wait for the weights in flight, and its reads are written as instructions.
+constexpr uint32_t kNlSlot = kPkBatch * kPkCols * kPkTileK;   // 4 KiB: 16 columns x 256 bytes
+constexpr uint32_t kNlRing = kPkWaves * 2u * kNlSlot;         // 64 KiB
+
+__global__ __launch_bounds__(kPkWaves * 64) void gemm_nkl_kernel(PackedParams p)
+{
+    __shared__ __attribute__((aligned(1024))) char RING[kNlRing];
+    __shared__ __attribute__((aligned(16))) char POOL[kPkPool - kNlRing];  // staged activations, then the partial sums
+    char* const XS = POOL;
+    int32_t* const red = reinterpret_cast<int32_t*>(POOL + p.red_off);
+    const uint32_t red_wave = p.red_slabs * 256u;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t lc = lane & 15u, lq = lane >> 4;
+    const uint32_t wg = pk_xcd_order(blockIdx.x, gridDim.x);
+    const uint32_t s0 = static_cast<uint32_t>(static_cast<uint64_t>(wg) * p.slabs / gridDim.x);
+    const uint32_t s1 = static_cast<uint32_t>(static_cast<uint64_t>(wg + 1u) * p.slabs / gridDim.x);
+    const uint32_t nslabs = s1 - s0;
+    const uint32_t ta = min(wave * p.tpw, p.ktiles), tb = min(ta + p.tpw, p.ktiles), cnt = tb - ta;
+    const uint32_t pitch = p.tpw * kPkTileK + kPkRowPad;
+    char* const xs = XS + wave * (p.rows * pitch);
+    {
+        const uint32_t row_pieces = cnt * (kPkTileK / 16u);
+        for (uint32_t r = 0; r < p.rows; ++r) {
+            const int8_t* src = p.a + static_cast<size_t>(p.m0 + r) * p.k + ta * kPkTileK + lane * 16u;
+            for (uint32_t c0 = 0; c0 < row_pieces; c0 += 64u) {
+                if (c0 + lane < row_pieces) {
+                    __builtin_amdgcn_global_load_lds((gptr_t)(src + c0 * 16u), (lds_ptr_t)(xs + r * pitch + c0 * 16u), 16, 0, 0);
+                }
+            }
+        }
+    }
+    const __amdgpu_buffer_rsrc_t rw =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<i32x4*>(p.wp), 0, static_cast<int>(p.n * p.k), 0x00020000);
+    // instruction u of a batch: columns 4 u .. 4 u + 3 of the slab; the lane's column and its position in the column's
+    // 256 bytes; it fetches piece position ^ column
+    uint32_t w_off[kPkBatch];
+#pragma unroll
+    for (uint32_t u = 0; u < kPkBatch; ++u) {
+        const uint32_t col = 4u * u + lq, pos = lc;
+        w_off[u] = col * p.k + ((pos ^ col) << 4);
+    }
+    char* const ring = RING + wave * (2u * kNlSlot);
+    const uint32_t x_lane = (lc - __umulhi(lc, p.rows_magic) * p.rows) * pitch + lq * 16u;
+    const uint32_t nb = (cnt + kPkBatch - 1u) / kPkBatch;
+    const uint32_t batches = nb * nslabs;
+    uint32_t l_slab = s0, l_b = 0, l_q = 0;
+    bool l_done = batches == 0u;
+    auto load = [&](char* slot) __attribute__((always_inline)) {
+        const uint32_t base = l_slab * kPkCols * p.k + (ta + l_b * kPkBatch) * kPkTileK;  // scalar
+#pragma unroll
+        for (uint32_t u = 0; u < kPkBatch; ++u) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(slot + u * 1024u), 16, l_done ? kPkPastEnd : w_off[u], base,
+                                                     0, kPkNt);
+        }
+        if (l_q + 1u < batches) {  // uniform
+            ++l_q;
+            if (++l_b == nb) {
+                l_b = 0;
+                ++l_slab;
+            }
+        } else {
+            l_done = true;
+        }
+    };
+    load(ring);
+    load(ring + kNlSlot);
+    // loads return in order: with at most the two batches outstanding the activations have landed
+    __builtin_amdgcn_s_waitcnt(((2 * kPkBatch) & 15) | (((2 * kPkBatch) >> 4) << 14) | (7 << 4) | (15 << 8));
+    asm volatile("" ::: "memory");
+
+    // the lane's fragment of tile t of a slot: column lc, piece 4 t + lq, stored at position piece ^ lc
+    const uint32_t ring_lane = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)ring)) + lc * 256u;
+    const uint32_t xs_lane = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)xs)) + x_lane;
+    const uint32_t red_lane = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)red)) + (wave * red_wave + lane) * 4u;
+    i32x4 acc = {0, 0, 0, 0};
+    uint32_t c_slab = 0, c_b = 0, c_q = 0;
+    auto step = [&](uint32_t slot_off, char* slot) __attribute__((always_inline)) {
+        if (c_q >= batches) {
+            return;  // uniform
+        }
+        // everything but the newest batch has landed
+        __builtin_amdgcn_s_waitcnt((kPkBatch & 15) | ((kPkBatch >> 4) << 14) | (7 << 4) | (15 << 8));
+        // (every LDS access of the loop is written as an instruction: one the compiler knows of makes it wait for
+        // all the weights in flight first.  A batch's last tiles may lie past the wavefront's k range: their
+        // activations are whatever follows in LDS, and they are not computed.)
+        const uint32_t t0 = c_b * kPkBatch;
+        const uint32_t live = min(kPkBatch, cnt - t0);
+        const uint32_t xa = xs_lane + t0 * kPkTileK;
+        i32x4 w[kPkBatch], a[kPkBatch];
+#pragma unroll
+        for (uint32_t t = 0; t < kPkBatch; ++t) {
+            const uint32_t addr = ring_lane + slot_off + (((4u * t + lq) ^ lc) << 4);
+            asm volatile("ds_read_b128 %0, %1" : "=v"(w[t]) : "v"(addr) : "memory");
+            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(a[t]) : "v"(xa), "i"(t * kPkTileK) : "memory");
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(w[0]), "+v"(w[1]), "+v"(w[2]), "+v"(w[3]), "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]));
+        load(slot);  // the slot is free again
+#pragma unroll
+        for (uint32_t t = 0; t < kPkBatch; ++t) {
+            if (t < live) {  // uniform
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[t], w[t], acc, 0, 0, 0);
+            }
+        }
+        ++c_q;
+        if (++c_b == nb) {
+            const uint32_t ra = red_lane + c_slab * 1024u;
+            asm volatile("ds_write_b32 %0, %1\n\tds_write_b32 %0, %2 offset:256\n\t"
+                         "ds_write_b32 %0, %3 offset:512\n\tds_write_b32 %0, %4 offset:768"
+                         :
+                         : "v"(ra), "v"(acc[0]), "v"(acc[1]), "v"(acc[2]), "v"(acc[3])
+                         : "memory");
+            acc = i32x4{0, 0, 0, 0};
+            c_b = 0;
+            ++c_slab;
+        }
+    };
+    for (uint32_t q = 0; q < batches; q += 2u) {
+        step(0u, ring);
+        step(kNlSlot, ring + kNlSlot);
+    }
+    if (batches == 0u) {
+        for (uint32_t s = 0; s < nslabs; ++s) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) red[wave * red_wave + s * 256u + i * 64u + lane] = 0;
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // the requests past the last batch, the sums' stores
+    __syncthreads();
+
+    const EpiParams& e = p.epi;
+    for (uint32_t s = wave; s < nslabs; s += kPkWaves) {
+        const uint32_t col = (s0 + s) * kPkCols + lc;
+        if (col >= p.n) {
+            continue;
+        }
+        const ChannelQ q = load_channel_q(e, col);
+        const float bp = load_bias_post(e, col);
+        const int32_t bias_pre = e.bias_kind == ASCQ_MM_BIAS_I32_PRE ? static_cast<const int32_t*>(e.bias)[col] : 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t row_in_pass = 4u * lq + static_cast<uint32_t>(i);
+            if (row_in_pass >= p.rows) {
+                continue;
+            }
+            const int32_t* part = red + s * 256u + static_cast<uint32_t>(i) * 64u + lane;
+            int32_t sum = part[0];
+#pragma unroll
+            for (uint32_t wv = 1; wv < kPkWaves; ++wv) sum += part[wv * red_wave];
+            sum += bias_pre;
+            const uint32_t row = p.m0 + row_in_pass;
+            const float tok = e.has_tok ? e.tok_scale[row] : 1.0f;
+            epilogue_store_lanes(e, row, col, sum, q, tok, bp);
+        }
+    }
+}
+
 // The decode kernel with the per-token quantisation of the activations inside (up to 8 rows of half or bfloat16 x):
 // q = ascq_dynamic_quant_per_token(x); c = matmul(q, w, tok_scale) in one launch, with those two calls' results bit for
 // bit.  Every workgroup needs all of x anyway, so every workgroup quantises it: a wavefront stages its k range of
@@ -808,6 +973,19 @@ int launch_gemm_packed(const GemmParams& p, hipStream_t st, bool b_nk)
     q.red_off = pass_rows * row_bytes;
     if (pass_rows == 0u) {
         return fail(ASCQ_EUNSUPPORTED, "ascq_matmul_w8a8_packed: k = %u is too long for the staged activations", p.k);
+    }
+    // [n, k] weights whose rows' activations leave 64 KiB of the LDS free: the weights go through a ring there
+    const uint32_t red_bytes = q.red_slabs * kPkWaves * 1024u;
+    if (b_nk && static_cast<uint64_t>(p.m) * row_bytes + red_bytes + kNlRing <= kPkPool) {
+        q.m0 = 0;
+        q.rows = p.m;
+        q.rows_magic = static_cast<uint32_t>(((1ull << 32) + q.rows - 1u) / q.rows);
+        q.red_off = p.m * row_bytes;
+        if (plan_note(ASCQ_MM_KERNEL_STREAM, 16, 16 * q.red_slabs, kPkTileK, grid, 1, kPkPool, 0)) {
+            return ASCQ_OK;
+        }
+        gemm_nkl_kernel<<<grid, kPkWaves * 64u, 0, st>>>(q);
+        return launch_status("ascq_matmul_w8a8 ([n, k] weight stream through LDS)");
     }
     for (uint32_t m0 = 0; m0 < p.m; m0 += q.rows) {
         const uint32_t left = p.m - m0;
