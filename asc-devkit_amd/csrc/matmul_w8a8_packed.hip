@@ -395,11 +395,18 @@ __device__ __forceinline__ float pk_wave_max_nonneg(float v)
     return __int_as_float(__builtin_amdgcn_readlane(x, 63));
 }
 
-template <bool kNK, bool kBf16>
+// kRing ([n, k] weights): the weights go through the LDS ring of gemm_nkl_kernel, which takes 64 KiB from the staged
+// activations; every LDS read between the first request and the last arrival is then written as an instruction (one
+// the compiler knows of makes it wait for all the weights in flight).
+constexpr uint32_t kPkDynRingHBytes = 60 * 1024, kPkDynRingQBytes = 30 * 1024;
+
+template <bool kNK, bool kBf16, bool kRing = false>
 __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_dyn_kernel(PackedParams p, const uint16_t* __restrict__ x)
 {
-    __shared__ __attribute__((aligned(16))) char XH[kPkDynHBytes];
-    __shared__ __attribute__((aligned(16))) char XS[kPkDynQBytes];
+    static_assert(kNK || !kRing, "the ring is for [n, k] weights");
+    __shared__ __attribute__((aligned(1024))) char RING[kRing ? kNlRing : 1024u];
+    __shared__ __attribute__((aligned(16))) char XH[kRing ? kPkDynRingHBytes : kPkDynHBytes];
+    __shared__ __attribute__((aligned(16))) char XS[kRing ? kPkDynRingQBytes : kPkDynQBytes];
     __shared__ int32_t OUT[kPkMaxSlabs][kPkDynRows][16];  // [slab][row][column]
     __shared__ float ROWMAX[kPkWaves][kPkDynRows];
     __shared__ float TOK[kPkDynRows];
@@ -436,6 +443,14 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_dyn_kernel(PackedPa
     i32x4 wq[kPkBuf][kPkBatch];
     uint32_t l_slab = s0, l_b = 0, l_q = 0;
     bool l_done = batches == 0u;
+    // (ring) instruction u of a batch: the lane's column 4 u + lq, position lc in its 256 bytes, piece position ^ column
+    uint32_t w_off[kPkBatch];
+#pragma unroll
+    for (uint32_t u = 0; u < kPkBatch; ++u) {
+        const uint32_t col = 4u * u + lq;
+        w_off[u] = col * p.k + ((lc ^ col) << 4);
+    }
+    char* const ring = RING + (kRing ? wave * (2u * kNlSlot) : 0u);
     auto load = [&](int buf) __attribute__((always_inline)) {
         const uint32_t l_w = l_done ? kPkPastEnd : w_lane;
         constexpr uint32_t kStep = kNK ? kPkTileK : kPkTileBytes;
@@ -443,7 +458,12 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_dyn_kernel(PackedPa
                                   : (l_slab * p.ktiles + ta + l_b * kPkBatch) * kPkTileBytes;  // scalar
 #pragma unroll
         for (uint32_t t = 0; t < kPkBatch; ++t) {
-            wq[buf][t] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, l_w, base + t * kStep, kPkNt));
+            if constexpr (kRing) {
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(ring + buf * kNlSlot + t * 1024u), 16,
+                                                         l_done ? kPkPastEnd : w_off[t], base, 0, kPkNt);
+            } else {
+                wq[buf][t] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, l_w, base + t * kStep, kPkNt));
+            }
         }
         if (l_q + 1u < batches) {  // uniform
             ++l_q;
@@ -465,6 +485,18 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_dyn_kernel(PackedPa
     auto widen = [](uint32_t half_bits) __attribute__((always_inline)) {
         return kBf16 ? bf16_bits_to_f32(half_bits) : half_bits_to_f32(half_bits);
     };
+    auto lds_read16 = [](const char* ptr) __attribute__((always_inline)) {
+        if constexpr (kRing) {
+            u32x4 v;
+            asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)"
+                         : "=v"(v)
+                         : "v"(static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)ptr)))
+                         : "memory");
+            return v;
+        } else {
+            return *reinterpret_cast<const u32x4*>(ptr);
+        }
+    };
     for (uint32_t i = tid; i < kPkMaxSlabs * kPkDynRows * 16u; i += kPkWaves * 64u) (&OUT[0][0][0])[i] = 0;
 #pragma unroll
     for (uint32_t r = 0; r < kPkDynRows; ++r) {
@@ -472,7 +504,7 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_dyn_kernel(PackedPa
             float amax = 0.0f;
             for (uint32_t c0 = 0; c0 < row_pieces; c0 += 64u) {
                 if (c0 + lane < row_pieces) {
-                    const u32x4 v = *reinterpret_cast<const u32x4*>(xh + r * 2u * pitch + (c0 + lane) * 16u);
+                    const u32x4 v = lds_read16(xh + r * 2u * pitch + (c0 + lane) * 16u);
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         amax = fmaxf(amax, fabsf(widen(v[i] & 0xFFFFu)));
@@ -496,7 +528,18 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_dyn_kernel(PackedPa
         float amax = 0.0f;
         if (lane < p.rows) {
 #pragma unroll
-            for (uint32_t wv = 0; wv < kPkWaves; ++wv) amax = fmaxf(amax, ROWMAX[wv][lane]);
+            for (uint32_t wv = 0; wv < kPkWaves; ++wv) {
+                float other;
+                if constexpr (kRing) {
+                    asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)"
+                                 : "=v"(other)
+                                 : "v"(static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)&ROWMAX[wv][lane])))
+                                 : "memory");
+                } else {
+                    other = ROWMAX[wv][lane];
+                }
+                amax = fmaxf(amax, other);
+            }
         }
         const bool zero = !(amax > 0.0f);
         lane_inv = zero ? 0.0f : 127.0f / amax;
@@ -510,7 +553,7 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_dyn_kernel(PackedPa
             const float inv = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(lane_inv), static_cast<int>(r)));
             for (uint32_t c0 = 0; c0 < row_pieces; c0 += 64u) {
                 if (c0 + lane < row_pieces) {
-                    const u32x4 v = *reinterpret_cast<const u32x4*>(xh + r * 2u * pitch + (c0 + lane) * 16u);
+                    const u32x4 v = lds_read16(xh + r * 2u * pitch + (c0 + lane) * 16u);
                     uint32_t u[8];
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
@@ -559,12 +602,62 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_packed_dyn_kernel(PackedPa
             ++c_slab;
         }
     };
+    // (ring) a batch's fragments and the activations' from LDS, the slot refilled, then the arithmetic, as in
+    // gemm_nkl_kernel; the sums of a finished slab are added with atomic instructions
+    const uint32_t ring_lane = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)ring)) + lc * 256u;
+    const uint32_t xs_lane = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)xs)) + x_lane;
+    const uint32_t out_lane = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)&OUT[0][0][0])) + (4u * lq * 16u + lc) * 4u;
+    auto ring_step = [&](int buf) __attribute__((always_inline)) {
+        if (c_q >= batches) {
+            return;  // uniform
+        }
+        __builtin_amdgcn_s_waitcnt((kPkBatch & 15) | ((kPkBatch >> 4) << 14) | (7 << 4) | (15 << 8));
+        const uint32_t t0 = c_b * kPkBatch;
+        const uint32_t live = min(kPkBatch, cnt - t0);
+        const uint32_t xa = xs_lane + t0 * kPkTileK;
+        i32x4 w[kPkBatch], a[kPkBatch];
+#pragma unroll
+        for (uint32_t t = 0; t < kPkBatch; ++t) {
+            const uint32_t addr = ring_lane + buf * kNlSlot + (((4u * t + lq) ^ lc) << 4);
+            asm volatile("ds_read_b128 %0, %1" : "=v"(w[t]) : "v"(addr) : "memory");
+            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(a[t]) : "v"(xa), "i"(t * kPkTileK) : "memory");
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(w[0]), "+v"(w[1]), "+v"(w[2]), "+v"(w[3]), "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]));
+        load(buf);
+#pragma unroll
+        for (uint32_t t = 0; t < kPkBatch; ++t) {
+            if (t < live) {  // uniform
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[t], w[t], acc, 0, 0, 0);
+            }
+        }
+        ++c_q;
+        if (++c_b == nb) {
+            if (4u * lq < p.rows) {
+                asm volatile("ds_add_u32 %0, %1\n\tds_add_u32 %0, %2 offset:64\n\t"
+                             "ds_add_u32 %0, %3 offset:128\n\tds_add_u32 %0, %4 offset:192"
+                             :
+                             : "v"(out_lane + c_slab * (kPkDynRows * 16u * 4u)), "v"(acc[0]), "v"(acc[1]), "v"(acc[2]), "v"(acc[3])
+                             : "memory");
+            }
+            acc = i32x4{0, 0, 0, 0};
+            c_b = 0;
+            ++c_slab;
+        }
+    };
     for (uint32_t q = 0; q < batches; q += kPkBuf) {
 #pragma unroll
         for (int b = 0; b < kPkBuf; ++b) {
-            compute(b);
-            load(b);
+            if constexpr (kRing) {
+                ring_step(b);
+            } else {
+                compute(b);
+                load(b);
+            }
         }
+    }
+    if constexpr (kRing) {
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // the requests past the last batch, the additions
     }
     __syncthreads();
 
@@ -1135,7 +1228,15 @@ int launch_gemm_packed_dyn(const GemmParams& p, const void* x, bool x_bf16, hipS
         grid = (q.slabs + kPkMaxSlabs - 1u) / kPkMaxSlabs;
     }
     const uint16_t* xp = static_cast<const uint16_t*>(x);
-    if (b_nk) {
+    // [n, k] weights go through the LDS ring where the rows' int8 image leaves room for it
+    const bool ring = b_nk && p.m * kPkWaves * (q.tpw * kPkTileK + kPkRowPad) <= kPkDynRingQBytes;
+    if (ring) {
+        if (x_bf16) {
+            gemm_packed_dyn_kernel<true, true, true><<<grid, kPkWaves * 64u, 0, st>>>(q, xp);
+        } else {
+            gemm_packed_dyn_kernel<true, false, true><<<grid, kPkWaves * 64u, 0, st>>>(q, xp);
+        }
+    } else if (b_nk) {
         if (x_bf16) {
             gemm_packed_dyn_kernel<true, true><<<grid, kPkWaves * 64u, 0, st>>>(q, xp);
         } else {
