@@ -241,7 +241,7 @@ bool gemm_ws_supported(const GemmParams& p, bool b_nk);
 int launch_gemm_ws(const GemmParams& p, hipStream_t st, bool b_nk);
 uint32_t gemm_ws_rounds(const GemmParams& p);
 // The same kernel with the per-token quantisation of x (half or bfloat16, [m, k]) inside: m <= 8 rows that fit the LDS.
-bool gemm_packed_dyn_fits(uint32_t m, uint32_t k);
+bool gemm_packed_dyn_fits(uint32_t m, uint32_t k, bool b_nk);
 int launch_gemm_packed_dyn(const GemmParams& p, const void* x, bool x_bf16, hipStream_t st, bool b_nk);
 
 }  // namespace ascq

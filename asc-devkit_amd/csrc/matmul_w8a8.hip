@@ -932,7 +932,7 @@ extern "C" int ascq_linear_w8a8_dynamic(const ascq_matmul_desc* d, int32_t x_dty
         return rc;
     }
     if ((x_dtype == ASCQ_F16 || x_dtype == ASCQ_BF16) && d->trans_b && d->b_format == ASCQ_MM_B_ND && aligned16(x) &&
-        gemm_packed_dyn_fits(d->m, d->k)) {
+        gemm_packed_dyn_fits(d->m, d->k, true)) {
         // decode on [n, k] weights: the quantisation happens inside the weight-streaming kernel (same bits, one launch)
         GemmParams p{};
         p.a = static_cast<const int8_t*>(x);  // only its alignment is looked at
@@ -988,7 +988,7 @@ extern "C" int ascq_linear_w8a8_dynamic_packed(const ascq_matmul_desc* d, int32_
         return rc;
     }
     ASCQ_REQUIRE(aligned16(w_packed), ASCQ_EALIGN, "ascq_linear_w8a8_dynamic_packed: w_packed must be 16-byte aligned");
-    if ((x_dtype == ASCQ_F16 || x_dtype == ASCQ_BF16) && aligned16(x) && gemm_packed_dyn_fits(d->m, d->k)) {
+    if ((x_dtype == ASCQ_F16 || x_dtype == ASCQ_BF16) && aligned16(x) && gemm_packed_dyn_fits(d->m, d->k, false)) {
         GemmParams p{};
         p.a = static_cast<const int8_t*>(x);  // only its alignment is looked at
         p.b = static_cast<const int8_t*>(w_packed);

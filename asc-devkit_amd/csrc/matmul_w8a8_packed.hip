@@ -1199,13 +1199,16 @@ int launch_gemm_ws(const GemmParams& p, hipStream_t st, bool b_nk)
 
 // The fused form: x [m, k] of halves or bfloat16s is quantised per token inside the kernel (p.epi.has_tok must be set;
 // p.a and p.epi.tok_scale are not read).  False when the shape does not fit (the caller then runs the two kernels).
-bool gemm_packed_dyn_fits(uint32_t m, uint32_t k)
+// On [n, k] weights the form runs where the LDS ring for the weights fits beside the rows (7 rows at k = 4096, 4 at
+// 7168, 2 at 14848): without the ring the separate quantiser and the ring kernel for the matmul are level or ahead.
+bool gemm_packed_dyn_fits(uint32_t m, uint32_t k, bool b_nk)
 {
     if (m == 0u || m > kPkDynRows || k % kPkTileK != 0) {
         return false;
     }
     const uint32_t tpw = (k / kPkTileK + kPkWaves - 1u) / kPkWaves;
-    return m * kPkWaves * (tpw * kPkTileK + kPkRowPad) <= kPkDynQBytes;  // the staged rows take twice that, of twice the space
+    // (the staged rows take twice the int8 image's bytes, of twice the space)
+    return m * kPkWaves * (tpw * kPkTileK + kPkRowPad) <= (b_nk ? kPkDynRingQBytes : kPkDynQBytes);
 }
 
 int launch_gemm_packed_dyn(const GemmParams& p, const void* x, bool x_bf16, hipStream_t st, bool b_nk)
@@ -1228,19 +1231,14 @@ int launch_gemm_packed_dyn(const GemmParams& p, const void* x, bool x_bf16, hipS
         grid = (q.slabs + kPkMaxSlabs - 1u) / kPkMaxSlabs;
     }
     const uint16_t* xp = static_cast<const uint16_t*>(x);
-    // [n, k] weights go through the LDS ring where the rows' int8 image leaves room for it
-    const bool ring = b_nk && p.m * kPkWaves * (q.tpw * kPkTileK + kPkRowPad) <= kPkDynRingQBytes;
-    if (ring) {
+    if (!gemm_packed_dyn_fits(p.m, p.k, b_nk)) {
+        return fail(ASCQ_EUNSUPPORTED, "ascq_linear_w8a8_dynamic: %u rows of k = %u do not fit the fused decode kernel", p.m, p.k);
+    }
+    if (b_nk) {  // [n, k] weights go through the LDS ring
         if (x_bf16) {
             gemm_packed_dyn_kernel<true, true, true><<<grid, kPkWaves * 64u, 0, st>>>(q, xp);
         } else {
             gemm_packed_dyn_kernel<true, false, true><<<grid, kPkWaves * 64u, 0, st>>>(q, xp);
-        }
-    } else if (b_nk) {
-        if (x_bf16) {
-            gemm_packed_dyn_kernel<true, true><<<grid, kPkWaves * 64u, 0, st>>>(q, xp);
-        } else {
-            gemm_packed_dyn_kernel<true, false><<<grid, kPkWaves * 64u, 0, st>>>(q, xp);
         }
     } else if (x_bf16) {
         gemm_packed_dyn_kernel<false, true><<<grid, kPkWaves * 64u, 0, st>>>(q, xp);

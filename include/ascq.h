@@ -449,9 +449,9 @@ int ascq_matmul_w8a8_plan(const ascq_matmul_desc* desc, const void* c, const voi
  * with exactly those results.  x [m, k] of x_dtype (ASCQ_F16 | ASCQ_BF16 | ASCQ_F32); desc as for ascq_matmul_w8a8 with
  * a dequantising epilogue (quant_mode SCALAR or VECTOR, floating-point out_dtype); desc->has_tok_scale is ignored.
  * The two kernels run one after the other on the stream, with q and tok in the workspace (sized by
- * ascq_linear_w8a8_dynamic_workspace_size; always required, whatever kernel runs).  Decode calls - up to 8 rows of half
- * or bfloat16 x on weights kept as [n, k] (desc->trans_b), k a multiple of 64 up to 5632 at 8 rows, 11776 at 4 - are one
- * launch: the weight-streaming kernel quantises x itself on its way into LDS (the same bits; the workspace is not
+ * ascq_linear_w8a8_dynamic_workspace_size; always required, whatever kernel runs).  Decode calls - half or bfloat16 x
+ * on weights kept as [n, k] (desc->trans_b), k a multiple of 64, up to 7 rows at k = 4096, 4 at 7168, 2 at 14848 - are
+ * one launch: the weight-streaming kernel quantises x itself on its way into LDS (the same bits; the workspace is not
  * touched).  No single reference operator does this: the reference composes it from
  * ReduceMax / AscendQuant PER_TOKEN (ascend_quant_per_group_3510_impl.h:142-178) and Matmul (matmul.h:175-185).
  */
