@@ -16,7 +16,7 @@ import subprocess
 import sys
 
 # kernels built on the inline-assembly read pattern, by the name they have in the sources
-GUARDED = ("gemm_nkl_kernel", "w4a16_gemv_kernel", "w4a16_tile_kernel", "w8a16_tile_kernel", "gemm_stream_kernel", "gemm_dma_kernel",
+GUARDED = ("gemm_nkl_kernel", "w8a16_nk_stream_kernel", "w4a16_gemv_kernel", "w4a16_tile_kernel", "w8a16_tile_kernel", "gemm_stream_kernel", "gemm_dma_kernel",
            "gemm_dma_dual_kernel", "gemm_dma_group_kernel", "w4a16_packed_kernel", "w4a16_packed_rows_kernel",
            "gemm_packed_kernel", "gemm_packed_dyn_kernel", "gemm_ws_kernel", "mx_tile_kernel")
 

@@ -226,6 +226,16 @@ constexpr int kSkBuf = 2;
 constexpr uint32_t kSkRowPad = 32;             // bytes added to a staged row of x
 constexpr uint32_t kSkXBytes = 96 * 1024;      // LDS for the staged activations of a workgroup
 constexpr uint32_t kSkPastEnd = 0x7FFFFFF0u;
+// kRing: the weights go through LDS instead of straight into registers.  Read as matrix operands, a tile of [n, k]
+// weights is 16 runs of 64 bytes per load instruction, which a compute unit's load path takes at about half the rate
+// of long runs; through a two-slot ring per wavefront a load instruction brings four columns' 256 bytes (the four
+// tiles of a batch), the 16-byte pieces of column c stored at position piece ^ c so that the 16 lanes reading one
+// piece of 16 columns fall on 16 bank groups.  The loads are range-checked buffer loads to LDS; every LDS read of the
+// loop is written as an instruction (one the compiler knows of makes it wait for all the weights in flight).
+constexpr uint32_t kSkSlot = kSkBatch * 16u * kSkTileK;    // 4 KiB: 16 columns x 256 bytes
+constexpr uint32_t kSkRing = kWaves * 2u * kSkSlot;        // 64 KiB
+constexpr uint32_t kSkRingXBytes = 76 * 1024;              // what is left for the staged activations beside it
+typedef __attribute__((address_space(3))) void* sk_lds_t;
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef __attribute__((address_space(1))) const void* gptr_t;
@@ -247,10 +257,11 @@ __device__ __forceinline__ uint32_t sk_xcd_order(uint32_t wg, uint32_t wgs)
     return (wgs & 7u) == 0u ? (wg & 7u) * (wgs >> 3) + (wg >> 3) : wg;
 }
 
-template <bool kHasOffset, bool kSum>
+template <bool kHasOffset, bool kSum, bool kRing>
 __global__ __launch_bounds__(kWaves * 64) void w8a16_nk_stream_kernel(SkParams p)
 {
-    __shared__ __attribute__((aligned(16))) char XS[kSkXBytes];
+    __shared__ __attribute__((aligned(1024))) char RING[kRing ? kSkRing : 1024u];
+    __shared__ __attribute__((aligned(16))) char XS[kRing ? kSkRingXBytes : kSkXBytes];
     __shared__ float RED[kWaves][kSkMaxSlabs][4][16];
     __shared__ uint32_t PAR[kSkMaxSlabs][16];  // (scale | offset << 16) of the workgroup's columns
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
@@ -295,6 +306,7 @@ __global__ __launch_bounds__(kWaves * 64) void w8a16_nk_stream_kernel(SkParams p
     const uint32_t nb = (cnt + kSkBatch - 1u) / kSkBatch;
     const uint32_t batches = nb * nslabs;
     u32x4 wq[kSkBuf][kSkBatch];
+    char* const ring = RING + (kRing ? wave * (2u * kSkSlot) : 0u);
     uint32_t l_slab = s0, l_b = 0, l_q = 0;
     bool l_done = batches == 0u;
     auto load = [&](int buf) __attribute__((always_inline)) {
@@ -305,7 +317,13 @@ __global__ __launch_bounds__(kWaves * 64) void w8a16_nk_stream_kernel(SkParams p
         const uint32_t base = l_slab * 16u * p.k + (ta + l_b * kSkBatch) * kSkTileK;  // scalar
 #pragma unroll
         for (uint32_t t = 0; t < kSkBatch; ++t) {
-            wq[buf][t] = __builtin_amdgcn_raw_buffer_load_b128(rw, l_w, base + t * kSkTileK, 2);
+            if constexpr (kRing) {  // instruction t: the lane's column 4 t + lq, position lc, piece position ^ column
+                const uint32_t col = 4u * t + lq;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (sk_lds_t)(ring + buf * kSkSlot + t * 1024u), 16,
+                                                         l_done ? kSkPastEnd : col * p.k + ((lc ^ col) << 4), base, 0, 2);
+            } else {
+                wq[buf][t] = __builtin_amdgcn_raw_buffer_load_b128(rw, l_w, base + t * kSkTileK, 2);
+            }
         }
         if (l_q + 1u < batches) {  // uniform
             ++l_q;
@@ -326,7 +344,10 @@ __global__ __launch_bounds__(kWaves * 64) void w8a16_nk_stream_kernel(SkParams p
     if (tid < nslabs * 16u) {
         PAR[tid >> 4][tid & 15u] = my_par;
     }
-    __syncthreads();
+    // a plain barrier: the fence of __syncthreads() would also wait for the weight loads in flight
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
 
     f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f}, xsum = {0.0f, 0.0f, 0.0f, 0.0f};
     f16x2_t sc2 = {}, of2 = {};
@@ -339,8 +360,26 @@ __global__ __launch_bounds__(kWaves * 64) void w8a16_nk_stream_kernel(SkParams p
         if (c_q >= batches) {
             return;  // uniform
         }
+        if constexpr (kRing) {  // the batch's fragments out of the ring, the slot refilled at once
+            const uint32_t wa = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((sk_lds_t)ring)) + buf * kSkSlot + lc * 256u;
+#pragma unroll
+            for (uint32_t t = 0; t < kSkBatch; ++t) {
+                const uint32_t addr = wa + (((4u * t + lq) ^ lc) << 4);
+                asm volatile("ds_read_b128 %0, %1" : "=v"(wq[buf][t]) : "v"(addr) : "memory");
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(wq[buf][0]), "+v"(wq[buf][1]), "+v"(wq[buf][2]), "+v"(wq[buf][3]));
+            load(buf);
+        }
         if (c_b == 0u) {  // a new column group: the lane's column parameters
-            const uint32_t pr = PAR[c_slab][lc];
+            uint32_t pr;
+            if constexpr (kRing) {
+                asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)"
+                             : "=v"(pr)
+                             : "v"(static_cast<uint32_t>(reinterpret_cast<uintptr_t>((sk_lds_t)&PAR[c_slab][lc])))
+                             : "memory");
+            } else {
+                pr = PAR[c_slab][lc];
+            }
             sc2 = h2_from_bits((pr & 0xFFFFu) | (pr << 16));
             of2 = h2_from_bits((pr >> 16) | (pr & 0xFFFF0000u));
             corr = (kHasOffset ? static_cast<float>(of2[0]) : 0.0f) - 1152.0f;
@@ -351,8 +390,17 @@ __global__ __launch_bounds__(kWaves * 64) void w8a16_nk_stream_kernel(SkParams p
 #pragma unroll
         for (uint32_t t = 0; t < kSkBatch; ++t) {
             if (t < live) {  // uniform
-                const f16x8_t a0 = *reinterpret_cast<const f16x8_t*>(xa0 + t * (kSkTileK * 2u));
-                const f16x8_t a1 = *reinterpret_cast<const f16x8_t*>(xa0 + t * (kSkTileK * 2u) + 16u);
+                f16x8_t a0, a1;
+                if constexpr (kRing) {
+                    const uint32_t xa = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((sk_lds_t)xa0));
+                    asm volatile("ds_read_b128 %0, %2 offset:%3\n\tds_read_b128 %1, %2 offset:%4\n\ts_waitcnt lgkmcnt(0)"
+                                 : "=&v"(a0), "=&v"(a1)
+                                 : "v"(xa), "i"(t * (kSkTileK * 2u)), "i"(t * (kSkTileK * 2u) + 16u)
+                                 : "memory");
+                } else {
+                    a0 = *reinterpret_cast<const f16x8_t*>(xa0 + t * (kSkTileK * 2u));
+                    a1 = *reinterpret_cast<const f16x8_t*>(xa0 + t * (kSkTileK * 2u) + 16u);
+                }
                 uint32_t h[8];
 #pragma unroll
                 for (int d = 0; d < 4; ++d) {
@@ -393,8 +441,13 @@ __global__ __launch_bounds__(kWaves * 64) void w8a16_nk_stream_kernel(SkParams p
 #pragma unroll
         for (int b = 0; b < kSkBuf; ++b) {
             compute(b);
-            load(b);
+            if constexpr (!kRing) {
+                load(b);
+            }
         }
+    }
+    if constexpr (kRing) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the requests past the last batch
     }
     if (batches == 0u && lq == 0u) {  // a wavefront without tiles (k shorter than 8 tiles) contributes zeros
         for (uint32_t s = 0; s < nslabs; ++s) {
@@ -700,22 +753,25 @@ int launch_w8a16_nk(const void* x, const void* w, const void* scale, const void*
         q.out_f32 = out_f32 ? 1u : 0u;
         q.scale_bits = scale_bits;
         q.offset_bits = offset_bits;
-        if (kWaves * m * (q.tpw * kSkTileK * 2u + kSkRowPad) <= kSkXBytes) {
+        const uint32_t x_bytes = kWaves * m * (q.tpw * kSkTileK * 2u + kSkRowPad);
+        const bool ring = x_bytes <= kSkRingXBytes;
+        if (x_bytes <= kSkXBytes) {
             const uint32_t cus = device_compute_units();
             uint32_t grid = q.slabs < cus ? q.slabs : cus;
             if ((q.slabs + grid - 1u) / grid > kSkMaxSlabs) {
                 grid = (q.slabs + kSkMaxSlabs - 1u) / kSkMaxSlabs;
             }
+            auto go = [&](auto off, auto sum, auto rg) {
+                w8a16_nk_stream_kernel<decltype(off)::value, decltype(sum)::value, decltype(rg)::value>
+                    <<<grid, kWaves * 64u, 0, st>>>(q);
+            };
+            auto pick_ring = [&](auto off, auto sum) {
+                ring ? go(off, sum, std::true_type{}) : go(off, sum, std::false_type{});
+            };
             if (channel_sum) {
-                if (has_offset) {
-                    w8a16_nk_stream_kernel<true, true><<<grid, kWaves * 64u, 0, st>>>(q);
-                } else {
-                    w8a16_nk_stream_kernel<false, true><<<grid, kWaves * 64u, 0, st>>>(q);
-                }
-            } else if (has_offset) {
-                w8a16_nk_stream_kernel<true, false><<<grid, kWaves * 64u, 0, st>>>(q);
+                has_offset ? pick_ring(std::true_type{}, std::true_type{}) : pick_ring(std::false_type{}, std::true_type{});
             } else {
-                w8a16_nk_stream_kernel<false, false><<<grid, kWaves * 64u, 0, st>>>(q);
+                has_offset ? pick_ring(std::true_type{}, std::false_type{}) : pick_ring(std::false_type{}, std::false_type{});
             }
             return launch_status("ascq_matmul_w8a16");
         }
