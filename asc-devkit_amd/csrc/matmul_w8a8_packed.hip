@@ -727,21 +727,73 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_ws_kernel(PackedParams p)
     const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<i32x4*>(p.wp), 0,
         static_cast<int>(kNK ? p.n * p.k : (p.slabs * p.ktiles + kPkPadTiles) * kPkTileBytes), 0x00020000);
-    const uint32_t w_lane = kNK ? lc * p.k + lq * 16u : lane * 16u;
     i32x4 wreg[kC][kS][kWsTpw];
+    char* const r0w = R0 + wave * kWsSlot;
+    char* const r1w = R1 + wave * kWsSlot;
+    if constexpr (!kNK) {
+        const uint32_t w_lane = lane * 16u;
 #pragma unroll
-    for (uint32_t kc = 0; kc < kC; ++kc) {
+        for (uint32_t kc = 0; kc < kC; ++kc) {
 #pragma unroll
-        for (uint32_t s = 0; s < kS; ++s) {
+            for (uint32_t s = 0; s < kS; ++s) {
 #pragma unroll
-            for (uint32_t t = 0; t < kWsTpw; ++t) {
-                // a tile this wavefront does not have is requested past the end of the buffer: no data moves, the
-                // instruction count stays what the waits below assume
-                const uint32_t tile = kc * kWsTpw + t;
-                const uint32_t off = (s < nslabs && tile < cnt) ? w_lane : kPkPastEnd;
-                const uint32_t base = kNK ? (s0 + s) * kPkCols * p.k + (ta + tile) * kPkTileK
-                                          : ((s0 + s) * p.ktiles + ta + tile) * kPkTileBytes;  // scalar
-                wreg[kc][s][t] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, off, base, kPkNt));
+                for (uint32_t t = 0; t < kWsTpw; ++t) {
+                    // a tile this wavefront does not have is requested past the end of the buffer: no data moves, the
+                    // instruction count stays what the waits below assume
+                    const uint32_t tile = kc * kWsTpw + t;
+                    const uint32_t off = (s < nslabs && tile < cnt) ? w_lane : kPkPastEnd;
+                    const uint32_t base = ((s0 + s) * p.ktiles + ta + tile) * kPkTileBytes;  // scalar
+                    wreg[kc][s][t] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, off, base, kPkNt));
+                }
+            }
+        }
+    } else {
+        // [n, k] weights reach their registers through the (still idle) activation ring, as in gemm_nkl_kernel: a
+        // load instruction brings four columns' 256 bytes, the pieces of column c at position piece ^ c; four slots
+        // of a batch (four tiles of one slab) each, three batches in flight while one is read.
+        constexpr uint32_t kUnits = kC * kS * 2u;
+        uint32_t w_off[kPkBatch];
+#pragma unroll
+        for (uint32_t u = 0; u < kPkBatch; ++u) {
+            const uint32_t col = 4u * u + lq;
+            w_off[u] = col * p.k + ((lc ^ col) << 4);
+        }
+        auto slot_of = [&](uint32_t j) __attribute__((always_inline)) { return ((j & 2u) != 0u ? r1w : r0w) + (j & 1u) * kNlSlot; };
+        auto request = [&](uint32_t j) __attribute__((always_inline)) {  // j: compile-time after unrolling
+            const uint32_t kc = j / (kS * 2u), s = (j / 2u) % kS, t0 = kc * kWsTpw + (j % 2u) * kPkBatch;
+            const bool have = s < nslabs && t0 < cnt;  // uniform; a batch the wavefront lacks moves no data
+            const uint32_t base = have ? (s0 + s) * kPkCols * p.k + (ta + t0) * kPkTileK : 0u;
+            char* const slot = slot_of(j & 3u);
+#pragma unroll
+            for (uint32_t u = 0; u < kPkBatch; ++u) {
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(slot + u * 1024u), 16, have ? w_off[u] : kPkPastEnd, base, 0,
+                                                         kPkNt);
+            }
+        };
+#pragma unroll
+        for (uint32_t j = 0; j < (kUnits < 4u ? kUnits : 4u); ++j) request(j);
+#pragma unroll
+        for (uint32_t j = 0; j < kUnits; ++j) {
+            constexpr uint32_t kAll = kUnits;
+            const uint32_t behind = (kAll - 1u - j < 3u ? kAll - 1u - j : 3u) * kPkBatch;  // loads that may still be out
+            // (a constant after unrolling; the builtin wants an immediate)
+            switch (behind) {
+                case 12: __builtin_amdgcn_s_waitcnt((12 & 15) | (7 << 4) | (15 << 8)); break;
+                case 8: __builtin_amdgcn_s_waitcnt((8 & 15) | (7 << 4) | (15 << 8)); break;
+                case 4: __builtin_amdgcn_s_waitcnt((4 & 15) | (7 << 4) | (15 << 8)); break;
+                default: __builtin_amdgcn_s_waitcnt((0 & 15) | (7 << 4) | (15 << 8)); break;
+            }
+            const uint32_t kc = j / (kS * 2u), s = (j / 2u) % kS, h = (j % 2u) * kPkBatch;
+            const uint32_t sa = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)slot_of(j & 3u))) + lc * 256u;
+#pragma unroll
+            for (uint32_t t = 0; t < kPkBatch; ++t) {
+                const uint32_t addr = sa + (((4u * t + lq) ^ lc) << 4);
+                asm volatile("ds_read_b128 %0, %1" : "=v"(wreg[kc][s][h + t]) : "v"(addr) : "memory");
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)"
+                         : "+v"(wreg[kc][s][h]), "+v"(wreg[kc][s][h + 1u]), "+v"(wreg[kc][s][h + 2u]), "+v"(wreg[kc][s][h + 3u]));
+            if (j + 4u < kUnits) {
+                request(j + 4u);
             }
         }
     }
@@ -749,8 +801,6 @@ __global__ __launch_bounds__(kPkWaves * 64) void gemm_ws_kernel(PackedParams p)
     // ---- activations: slot position (row r, piece q) holds piece q ^ r of the row's share of one chunk (the
     // reader's 16 rows then fall on 16 different bank groups); pieces past the wavefront's range fetch the chunk's
     // piece 0 and are not read
-    char* const r0w = R0 + wave * kWsSlot;
-    char* const r1w = R1 + wave * kWsSlot;
     // A load's address is a wavefront-uniform base (row tile and chunk) plus the lane's 32-bit offset, which the
     // instruction adds itself; the last row tile, where rows past the end repeat the last row, has offsets of its own.
     // (ntiles, the offsets of the last tile and the base belong to the block of rows being worked on)
