@@ -1153,9 +1153,10 @@ int launch_gemm_packed(const GemmParams& p, hipStream_t st, bool b_nk)
 // 9.5 us (packed weights; 11.5 us for [n, k] weights, whose tiles arrive as 16 runs of 64 bytes) plus about 1 us per
 // 16 rows: every workgroup streams all of the activations, 128 MB through the L2s at 128 rows.  It takes the calls
 // whose rows the resident form cannot hold in one pass: on packed weights all of them; on [n, k] weights those up to
-// 224 rows at k up to 4096, where it leads the K-split tiles (22.3 against 24.4 us at 128 rows), and at longer k
-// those up to 32 rows whose slabs one round of workgroups holds (k = 11008, n = 4096, 32 rows: 19 against 21 us;
-// the tile kernels lead from 64 rows on, and at once where the workgroups need a second round).
+// 224 rows at k up to 4096, where it leads the K-split tiles (20.4 against 24.4 us at 128 rows), and at longer k
+// those up to 64 rows (k up to 8192; 48 beyond) whose slabs one round of workgroups holds (k = 8192, n = 8192, 64
+// rows: 21.2 against 23.9 us; k = 11008, n = 4096, 32 rows: 17.0 against 20.9 us; the tile kernels lead from there
+// on, and at once where the workgroups need a second round).
 namespace {
 
 // chunks of kWsTpw tiles in a wavefront's k range; the slabs a workgroup's registers hold then; the grid: one
@@ -1198,7 +1199,7 @@ bool gemm_ws_supported(const GemmParams& p, bool b_nk)
     if (nchunks == 1u) {
         return p.m <= kWsNkMaxRows;
     }
-    return p.m <= 32u && ws_grid((p.n + kPkCols - 1u) / kPkCols, ws_max_slabs(nchunks)) <= device_compute_units();
+    return p.m <= (nchunks == 2u ? 64u : 48u) && ws_grid((p.n + kPkCols - 1u) / kPkCols, ws_max_slabs(nchunks)) <= device_compute_units();
 }
 
 // Rounds of workgroups the weight-stationary form needs on this device (1: every workgroup is resident at once).

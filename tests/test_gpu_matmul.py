@@ -1233,7 +1233,7 @@ def test_group_matmul_swiglu_and_dynamic_linear():
 def test_matmul_swiglu_in_the_decode_kernels(m, n, k, out, bias):
     """SwiGLU on [n, k] and on packed weights: the decode kernels (activations resident in LDS up to 16 rows, weights
     held in registers beyond, also in chunks of a longer k) pair the columns of a row through neighbouring lanes in
-    their own epilogue - one launch, no raw accumulators; [n, k] weights past 224 rows (32 at k above 4096) take the
+    their own epilogue - one launch, no raw accumulators; [n, k] weights past 224 rows (64 or 48 at k above 4096) take the
     tile kernels.  Against the oracle."""
     announce("swiglu decode", m, n, k, out, bias)
     rng = np.random.default_rng(m * 5 + n + k)
