@@ -212,6 +212,32 @@ def test_w8a8_packed_small(m, n, k):
     assert max_ulp(bits(cg), oracle_mm(dg, a, b).view(np.uint16), "f16") <= 1
 
 
+@pytest.mark.parametrize("m", [1, 2, 3, 5, 8, 13, 16])
+@pytest.mark.parametrize("n,k", [(16, 64), (48, 128), (1040, 512), (272, 4096), (2064, 192), (100, 5632), (96, 8192),
+                                 (40, 11008), (4100, 256)])
+def test_w8a8_decode_on_n_k_weights_through_lds(m, n, k):
+    """Up to 16 rows on weights kept as [n, k]: where the staged activations leave 64 KiB of LDS free the weights go
+    through a ring there (four columns' 256 bytes per load, XOR-swizzled pieces), otherwise straight into registers
+    (long k with many rows).  k of one tile (seven wavefronts without work), column counts that are no multiple of 16
+    (the last slab's columns past n read as zeros), several slabs per workgroup, batches that end inside a wavefront's
+    range.  int32 accumulators exactly, the dequantising and the requantising epilogue against the oracle."""
+    announce("w8a8 [n, k] decode", m, n, k)
+    rng = np.random.default_rng(m * 47 + n + k)
+    a, b = rand_i8(rng, (m, k), -128, 127), rand_i8(rng, (k, n), -128, 127)
+    bt = np.ascontiguousarray(b.T)
+    c, _ = run_mm(m, n, k, a, bt, out=torch.int32, trans_b=True)
+    assert np.array_equal(c.cpu().numpy(), a.astype(np.int64) @ b.astype(np.int64))
+    cs = rng.uniform(1e-4, 1e-2, n).astype(np.float32)
+    ts = rng.uniform(1e-2, 1e-1, m).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    c, desc = run_mm(m, n, k, a, bt, out=torch.bfloat16, bias=(bias, None), quant=cs, tok=ts, trans_b=True)
+    assert np.array_equal(bits(c), oracle_mm(desc, a, bt, (bias, None), cs, ts))  # (the descriptor says [n, k])
+    words = (cs * 50).astype(np.float32).view(np.uint32).astype(np.uint64) | (np.uint64(1) << np.uint64(46))
+    bias_i = rng.integers(-1000, 1000, n).astype(np.int32)
+    c8, d8 = run_mm(m, n, k, a, bt, out=torch.int8, bias=(bias_i, None), quant=words, trans_b=True)
+    assert np.array_equal(bits(c8), oracle_mm(d8, a, bt, (bias_i, None), words))
+
+
 @pytest.mark.parametrize("m", [17, 33, 47, 64, 100, 128, 129, 224, 225, 300])
 @pytest.mark.parametrize("n,k", [(16, 64), (48, 128), (1040, 512), (272, 4096), (2064, 192), (13000, 256), (96, 4160)])
 def test_w8a8_weights_held_in_registers(m, n, k):
